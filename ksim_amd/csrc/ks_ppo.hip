@@ -1,0 +1,362 @@
+// GAE / returns scan, advantage normalisation, PPO loss and reward/termination
+// reduction for gfx950.  Streaming, HBM-bound kernels: every array is read or
+// written exactly once per launch, with 64 consecutive elements per wavefront.
+#include "ks_common.h"
+
+namespace ks {
+
+static thread_local char g_err[256] = "";
+char* err_buf() { return g_err; }
+
+// ---------------------------------------------------------------------------------------------
+// GAE, (B, T) layout.  One wavefront per env row; lanes run along time.  The
+// recurrences R_t = r'_t + g m_t R_{t+1} and A_t = d_t + g l m_t A_{t+1}
+// (ksim/task/ppo.py:66-75) are compositions of affine maps x -> d + c x, which are
+// associative, so a 64-wide reverse Kogge-Stone scan with wavefront shuffles handles one
+// 64-step chunk; chunks are chained from the end of the row through a scalar carry.
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void gae_bt_kernel(
+    int64_t B, int64_t T, const float* __restrict__ values, const float* __restrict__ rewards,
+    const uint8_t* __restrict__ dones, const uint8_t* __restrict__ successes, float gamma, float lam,
+    int mc, float* __restrict__ gae, float* __restrict__ returns, float* __restrict__ targets) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  if (row >= B) return;  // whole wavefront leaves together
+  const int64_t base = row * T;
+  const float v_last = values[base + T - 1];  // bootstrap = last value repeated, ppo.py:79
+  const float gl = gamma * lam;
+  const float omg = 1.0f - gamma;
+  float carry_r = 0.f, carry_a = 0.f, v_next_chunk = v_last;
+  const int64_t nchunk = (T + 63) >> 6;
+  for (int64_t c = nchunk - 1; c >= 0; --c) {
+    const int64_t t = (c << 6) + lane;
+    const bool valid = t < T;
+    float v = 0.f, r = 0.f;
+    bool dn = false, sc = false;
+    if (valid) {
+      v = values[base + t];
+      r = rewards[base + t];
+      dn = dones[base + t] != 0;
+      if (successes) sc = successes[base + t] != 0;
+    }
+    float v_up = __shfl_down(v, 1);
+    if (lane == 63) v_up = v_next_chunk;
+    if (t + 1 >= T) v_up = v_last;
+    const float mask = dn ? 0.f : 1.f;
+    const float rb = omg * r + gamma * v * (sc ? 1.f : 0.f);  // ppo.py:82-83
+    const float delta = rb + gamma * v_up * mask - v;          // ppo.py:86
+    float c_r = valid ? gamma * mask : 1.f, d_r = valid ? rb : 0.f;
+    float c_a = valid ? gl * mask : 1.f, d_a = valid ? delta : 0.f;
+#pragma unroll
+    for (int s = 1; s < 64; s <<= 1) {
+      const float pc_r = __shfl_down(c_r, s), pd_r = __shfl_down(d_r, s);
+      const float pc_a = __shfl_down(c_a, s), pd_a = __shfl_down(d_a, s);
+      if (lane + s < 64) {
+        d_r = d_r + c_r * pd_r;
+        c_r = c_r * pc_r;
+        d_a = d_a + c_a * pd_a;
+        c_a = c_a * pc_a;
+      }
+    }
+    const float R = d_r + c_r * carry_r;
+    const float A = d_a + c_a * carry_a;
+    if (valid) {
+      if (gae) gae[base + t] = A;
+      if (returns) returns[base + t] = R;
+      if (targets) targets[base + t] = mc ? R : A + v;  // ppo.py:107
+    }
+    carry_r = __shfl(R, 0);
+    carry_a = __shfl(A, 0);
+    v_next_chunk = __shfl(v, 0);
+  }
+}
+
+// GAE, (T, N) layout: one lane per env, walking back in time; a wavefront reads 64
+// consecutive envs per step (256 B), and the loads of the next steps do not depend on the
+// recurrence so the compiler can keep several in flight.
+__global__ __launch_bounds__(256) void gae_tn_kernel(
+    int64_t T, int64_t N, const float* __restrict__ values, const float* __restrict__ rewards,
+    const uint8_t* __restrict__ dones, const uint8_t* __restrict__ successes, float gamma, float lam,
+    int mc, float* __restrict__ gae, float* __restrict__ returns, float* __restrict__ targets) {
+  const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= N) return;
+  const float gl = gamma * lam, omg = 1.0f - gamma;
+  float R = 0.f, A = 0.f;
+  float v_up = values[(T - 1) * N + e];
+#pragma unroll 4
+  for (int64_t t = T - 1; t >= 0; --t) {
+    const int64_t i = t * N + e;
+    const float v = values[i], r = rewards[i];
+    const float mask = dones[i] ? 0.f : 1.f;
+    const float sc = (successes && successes[i]) ? 1.f : 0.f;
+    const float rb = omg * r + gamma * v * sc;
+    const float delta = rb + gamma * v_up * mask - v;
+    R = rb + gamma * mask * R;
+    A = delta + gl * mask * A;
+    if (gae) gae[i] = A;
+    if (returns) returns[i] = R;
+    if (targets) targets[i] = mc ? R : A + v;
+    v_up = v;
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Deterministic two-stage reductions (no atomics): stage 1 writes one partial per block,
+// stage 2 re-reads the <= 1024 partials in a fixed order.
+// ---------------------------------------------------------------------------------------------
+constexpr int kMaxPartials = 1024;
+
+__device__ inline double wave_sum(double x) {
+#pragma unroll
+  for (int s = 32; s > 0; s >>= 1) x += __shfl_down(x, s);
+  return x;
+}
+
+// Sum over a 256-thread block; result valid in thread 0.
+__device__ inline double block_sum(double x, double* lds4) {
+  x = wave_sum(x);
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) lds4[threadIdx.x >> 6] = x;
+  __syncthreads();
+  return lds4[0] + lds4[1] + lds4[2] + lds4[3];
+}
+
+__global__ __launch_bounds__(256) void moments_kernel(int64_t n, const float* __restrict__ x,
+                                                       double* __restrict__ partial) {
+  __shared__ double lds[4];
+  double s = 0.0, ss = 0.0;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
+    const double v = x[i];
+    s += v;
+    ss += v * v;
+  }
+  s = block_sum(s, lds);
+  ss = block_sum(ss, lds);
+  if (threadIdx.x == 0) {
+    partial[blockIdx.x] = s;
+    partial[kMaxPartials + blockIdx.x] = ss;
+  }
+}
+
+__global__ __launch_bounds__(256) void normalize_kernel(int64_t n, int nparts, const float* __restrict__ x,
+                                                         const double* __restrict__ partial,
+                                                         float* __restrict__ out) {
+  __shared__ double lds[4];
+  __shared__ float s_mean, s_inv;
+  double s = 0.0, ss = 0.0;
+  for (int i = threadIdx.x; i < nparts; i += blockDim.x) {
+    s += partial[i];
+    ss += partial[kMaxPartials + i];
+  }
+  s = block_sum(s, lds);
+  ss = block_sum(ss, lds);
+  if (threadIdx.x == 0) {
+    const double mean = s / (double)n;
+    double var = ss / (double)n - mean * mean;
+    if (var < 0.0) var = 0.0;
+    double sd = sqrt(var);
+    if (sd < 1e-6) sd = 1e-6;  // ppo.py:118
+    s_mean = (float)mean;
+    s_inv = (float)(1.0 / sd);
+  }
+  __syncthreads();
+  const float mean = s_mean, inv = s_inv;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
+    out[i] = (x[i] - mean) * inv;
+}
+
+// ---------------------------------------------------------------------------------------------
+// PPO loss (ppo.py:207-246).  One lane per (b, t) element; the A log-probs of an element are
+// contiguous, so a wavefront touches one contiguous 64*A*4-byte span per array.
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void ppo_loss_kernel(
+    int64_t n, int A, KsPpoLossParams p, const float* __restrict__ adv, const float* __restrict__ tgt,
+    const float* __restrict__ lp_on, const float* __restrict__ v_on, const float* __restrict__ lp_off,
+    const float* __restrict__ v_off, const float* __restrict__ ent, float* __restrict__ o_policy,
+    float* __restrict__ o_value, float* __restrict__ o_kl, float* __restrict__ o_ent,
+    double* __restrict__ partial) {
+  __shared__ double lds[4];
+  double acc = 0.0;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
+    float log_ratio = 0.f, kl = 0.f, es = 0.f;
+    const float* a_on = lp_on + i * A;
+    const float* a_off = lp_off + i * A;
+    for (int a = 0; a < A; ++a) {
+      const float on = a_on[a], off = a_off[a];
+      log_ratio += off - on;
+      kl += on - off;
+    }
+    if (ent) {
+      const float* e = ent + i * A;
+      for (int a = 0; a < A; ++a) es += e[a];
+    }
+    const float lr = fminf(fmaxf(log_ratio, -p.log_clip_value), p.log_clip_value);
+    const float ratio = expf(lr);
+    const float cr = fminf(fmaxf(ratio, 1.f - p.clip_param), 1.f + p.clip_param);
+    const float ad = adv[i];
+    const float policy = -fminf(ratio * ad, cr * ad);
+    const float von = v_on[i], voff = v_off[i], tg = tgt[i];
+    float vobj;
+    if (p.use_clipped_value_loss) {
+      const float vc = von + fminf(fmaxf(voff - von, -p.clip_param), p.clip_param);
+      const float ce = vc - tg, er = voff - tg;
+      vobj = 0.5f * fmaxf(er * er, ce * ce);
+    } else {
+      const float er = tg - voff;
+      vobj = 0.5f * er * er;
+    }
+    const float value = vobj * p.value_loss_coef;
+    const float klv = kl * p.kl_coef * p.kl_scale;
+    const float entv = ent ? -es * p.entropy_coef : 0.f;
+    if (o_policy) o_policy[i] = policy;
+    if (o_value) o_value[i] = value;
+    if (o_kl) o_kl[i] = klv;
+    if (o_ent && ent) o_ent[i] = entv;
+    acc += (double)(policy + value + klv + entv);
+  }
+  acc = block_sum(acc, lds);
+  if (threadIdx.x == 0) partial[blockIdx.x] = acc;
+}
+
+__global__ __launch_bounds__(256) void mean_finish_kernel(int nparts, int64_t n, const double* __restrict__ partial,
+                                                           float* __restrict__ out) {
+  __shared__ double lds[4];
+  double s = 0.0;
+  for (int i = threadIdx.x; i < nparts; i += blockDim.x) s += partial[i];
+  s = block_sum(s, lds);
+  if (threadIdx.x == 0) out[0] = (float)(s / (double)n);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Reward total (rl.py:219-239) and done/success (rl.py:1049-1050).
+// ---------------------------------------------------------------------------------------------
+struct RewardScales {
+  float s[KS_MAX_REWARD_TERMS];
+};
+
+__global__ __launch_bounds__(256) void reward_total_kernel(
+    int64_t n, int K, const float* __restrict__ comps, RewardScales sc, int use_min, float cmin, int use_max,
+    float cmax, float* __restrict__ total, int k, const int8_t* __restrict__ terms, uint8_t* __restrict__ done,
+    uint8_t* __restrict__ success) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  if (total) {
+    float t = 0.f;
+    for (int j = 0; j < K; ++j) {
+      const float term = comps[(int64_t)j * n + i] * sc.s[j];
+      t = (j == 0) ? term : t + term;  // insertion-order sum, rl.py:235
+    }
+    if (use_min) t = fmaxf(t, cmin);
+    if (use_max) t = fminf(t, cmax);
+    total[i] = t;
+  }
+  if (k > 0) {
+    bool d = false, s = true;
+    for (int j = 0; j < k; ++j) {
+      const int8_t t = terms[(int64_t)j * n + i];
+      d |= t != 0;
+      s &= t != -1;
+    }
+    if (done) done[i] = d ? 1 : 0;
+    if (success) success[i] = (s && d) ? 1 : 0;
+  }
+}
+
+static inline int grid_for(int64_t n, int block, int cap) {
+  int64_t g = (n + block - 1) / block;
+  if (g > cap) g = cap;
+  if (g < 1) g = 1;
+  return (int)g;
+}
+
+}  // namespace ks
+
+using namespace ks;
+
+extern "C" const char* ks_version(void) { return "ksim_hip 0.1 (gfx950)"; }
+extern "C" const char* ks_last_error(void) { return ks::err_buf(); }
+
+static int check_gae_args(int64_t n0, int64_t n1, const float* v, const float* r, const uint8_t* d) {
+  if (n0 < 0 || n1 < 0) return fail(KS_EINVAL, "ks_gae: negative size");
+  if (n0 > 0 && n1 > 0 && (!v || !r || !d)) return fail(KS_EINVAL, "ks_gae: null input");
+  if (n0 > (int64_t)1 << 40 || n1 > (int64_t)1 << 40) return fail(KS_ELIMIT, "ks_gae: size too large");
+  return KS_OK;
+}
+
+extern "C" int ks_gae_bt(ks_stream_t stream, int64_t B, int64_t T, const float* values, const float* rewards,
+                         const uint8_t* dones, const uint8_t* successes, float gamma, float lam,
+                         int monte_carlo_returns, float* gae, float* returns, float* targets) {
+  if (int rc = check_gae_args(B, T, values, rewards, dones)) return rc;
+  if (B == 0 || T == 0) return KS_OK;
+  const int rows_per_block = 4;
+  const int64_t grid = (B + rows_per_block - 1) / rows_per_block;
+  if (grid > 0x7fffffff) return fail(KS_ELIMIT, "ks_gae_bt: B too large");
+  hipLaunchKernelGGL(gae_bt_kernel, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, B, T, values, rewards,
+                     dones, successes, gamma, lam, monte_carlo_returns, gae, returns, targets);
+  return check_launch("ks_gae_bt");
+}
+
+extern "C" int ks_gae_tn(ks_stream_t stream, int64_t T, int64_t N, const float* values, const float* rewards,
+                         const uint8_t* dones, const uint8_t* successes, float gamma, float lam,
+                         int monte_carlo_returns, float* gae, float* returns, float* targets) {
+  if (int rc = check_gae_args(T, N, values, rewards, dones)) return rc;
+  if (N == 0 || T == 0) return KS_OK;
+  const int64_t grid = (N + 63) / 64;
+  if (grid > 0x7fffffff) return fail(KS_ELIMIT, "ks_gae_tn: N too large");
+  hipLaunchKernelGGL(gae_tn_kernel, dim3((unsigned)grid), dim3(64), 0, (hipStream_t)stream, T, N, values, rewards,
+                     dones, successes, gamma, lam, monte_carlo_returns, gae, returns, targets);
+  return check_launch("ks_gae_tn");
+}
+
+extern "C" int ks_normalize_advantages(ks_stream_t stream, int64_t n, const float* gae, float* advantages,
+                                       void* workspace) {
+  if (n < 0) return fail(KS_EINVAL, "ks_normalize_advantages: negative size");
+  if (n == 0) return KS_OK;
+  if (!gae || !advantages || !workspace) return fail(KS_EINVAL, "ks_normalize_advantages: null pointer");
+  const int g = grid_for(n, 256 * 4, kMaxPartials);
+  double* partial = (double*)workspace;
+  hipLaunchKernelGGL(moments_kernel, dim3(g), dim3(256), 0, (hipStream_t)stream, n, gae, partial);
+  hipLaunchKernelGGL(normalize_kernel, dim3(grid_for(n, 256, 4096)), dim3(256), 0, (hipStream_t)stream, n, g, gae,
+                     partial, advantages);
+  return check_launch("ks_normalize_advantages");
+}
+
+extern "C" int ks_ppo_loss(ks_stream_t stream, int64_t n, int32_t A, const KsPpoLossParams* params,
+                           const float* advantages, const float* value_targets, const float* on_log_probs,
+                           const float* on_values, const float* off_log_probs, const float* off_values,
+                           const float* off_entropy, float* policy_loss, float* value_loss, float* kl_loss,
+                           float* entropy_loss, float* loss_out, void* workspace) {
+  if (n < 0 || A < 1) return fail(KS_EINVAL, "ks_ppo_loss: bad size n=%lld A=%d", (long long)n, A);
+  if (!params) return fail(KS_EINVAL, "ks_ppo_loss: null params");
+  if (n == 0) return KS_OK;
+  if (!advantages || !value_targets || !on_log_probs || !on_values || !off_log_probs || !off_values || !workspace)
+    return fail(KS_EINVAL, "ks_ppo_loss: null pointer");
+  const int g = grid_for(n, 256, kMaxPartials);
+  double* partial = (double*)workspace;
+  hipLaunchKernelGGL(ppo_loss_kernel, dim3(g), dim3(256), 0, (hipStream_t)stream, n, (int)A, *params, advantages,
+                     value_targets, on_log_probs, on_values, off_log_probs, off_values, off_entropy, policy_loss,
+                     value_loss, kl_loss, entropy_loss, partial);
+  if (loss_out)
+    hipLaunchKernelGGL(mean_finish_kernel, dim3(1), dim3(256), 0, (hipStream_t)stream, g, n, partial, loss_out);
+  return check_launch("ks_ppo_loss");
+}
+
+extern "C" int ks_reward_total(ks_stream_t stream, int64_t n, int32_t K, const float* components,
+                               const float* scales, int32_t use_clip_min, float clip_min, int32_t use_clip_max,
+                               float clip_max, float* total, int32_t k, const int8_t* terminations, uint8_t* done,
+                               uint8_t* success) {
+  if (n < 0 || K < 0 || k < 0) return fail(KS_EINVAL, "ks_reward_total: negative size");
+  if (K > KS_MAX_REWARD_TERMS || k > KS_MAX_REWARD_TERMS)
+    return fail(KS_ELIMIT, "ks_reward_total: more than %d terms", KS_MAX_REWARD_TERMS);
+  if (n == 0) return KS_OK;
+  if (total && (K == 0 || !components || !scales)) return fail(KS_EINVAL, "ks_reward_total: total needs K>0 components");
+  if (k > 0 && !terminations) return fail(KS_EINVAL, "ks_reward_total: null terminations");
+  RewardScales sc{};
+  for (int j = 0; j < K && scales; ++j) sc.s[j] = scales[j];
+  const int64_t grid = (n + 255) / 256;
+  if (grid > 0x7fffffff) return fail(KS_ELIMIT, "ks_reward_total: n too large");
+  hipLaunchKernelGGL(reward_total_kernel, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, n, (int)K,
+                     components, sc, use_clip_min, clip_min, use_clip_max, clip_max, total, (int)k, terminations, done,
+                     success);
+  return check_launch("ks_reward_total");
+}

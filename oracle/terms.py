@@ -1,0 +1,207 @@
+"""numpy restatement of the reference's per-env terms (test infrastructure).
+
+Rewards follow ksim/rewards.py, terminations ksim/terminations.py, the PD
+actuator ksim/actuators.py:182-217, the latency blend ksim/engine.py:287-288,
+the done/success combination ksim/task/rl.py:1049-1050 and the reward total
+ksim/task/rl.py:219-239.  Shapes are per env, time leading, like the reference.
+"""
+
+from __future__ import annotations
+
+import numpy as np
+
+
+# --------------------------------------------------------------------------- quaternions (Hamilton, wxyz)
+def quat_mul(a, b):
+    aw, ax, ay, az = np.moveaxis(np.asarray(a), -1, 0)
+    bw, bx, by, bz = np.moveaxis(np.asarray(b), -1, 0)
+    return np.stack(
+        [
+            aw * bw - ax * bx - ay * by - az * bz,
+            aw * bx + ax * bw + ay * bz - az * by,
+            aw * by - ax * bz + ay * bw + az * bx,
+            aw * bz + ax * by - ay * bx + az * bw,
+        ],
+        axis=-1,
+    )
+
+
+def rotate_vector_by_quat(v, q, inverse: bool = False):
+    """v' = q v q* (inverse: q* v q); the quaternion is normalised first (xax convention assumed)."""
+    q = np.asarray(q, dtype=np.float64)
+    q = q / np.linalg.norm(q, axis=-1, keepdims=True)
+    if inverse:
+        q = q * np.array([1.0, -1.0, -1.0, -1.0])
+    v = np.asarray(v, dtype=np.float64)
+    qv = np.concatenate([np.zeros(v.shape[:-1] + (1,)), v], axis=-1)
+    qc = q * np.array([1.0, -1.0, -1.0, -1.0])
+    return quat_mul(quat_mul(q, qv), qc)[..., 1:]
+
+
+# --------------------------------------------------------------------------- norms / kernels
+def get_norm(x, norm: str):
+    """xax.get_norm as pinned by reference tests/test_rewards.py:95-98,120-123."""
+    if norm == "l1":
+        return np.abs(x)
+    if norm == "l2":
+        return np.square(x)
+    raise ValueError(norm)
+
+
+def exp_kernel(x, scale):  # rewards.py:72-73
+    return np.exp(-np.square(x) / (2 * scale**2))
+
+
+def exp_kernel_with_penalty(x, scale, sq_scale, abs_scale):  # rewards.py:84-88
+    return np.abs(x) * -abs_scale + np.square(x) * -sq_scale + np.exp(-np.square(x) / (2 * scale**2))
+
+
+# --------------------------------------------------------------------------- rewards
+def _edge_pad_front(x, n):
+    return np.concatenate([np.repeat(x[:1], n, axis=0), x], axis=0)
+
+
+def action_velocity_penalty(action_ta, done_t, norm="l2"):  # rewards.py:410-419
+    a = _edge_pad_front(np.asarray(action_ta, dtype=np.float64), 1)
+    done = _edge_pad_front(np.asarray(done_t).astype(bool), 1)[:-1, None]
+    vel = np.where(done, 0.0, a[1:] - a[:-1])
+    pen = get_norm(vel, norm).mean(axis=-1)
+    return np.where(np.arange(len(pen)) >= 1, pen, 0.0)
+
+
+def action_acceleration_penalty(action_ta, done_t, norm="l2"):  # rewards.py:428-440
+    a = _edge_pad_front(np.asarray(action_ta, dtype=np.float64), 2)
+    done = _edge_pad_front(np.asarray(done_t).astype(bool), 2)[:-1, None]
+    vel = np.where(done, 0.0, a[1:] - a[:-1])
+    acc = np.where(done[1:], 0.0, vel[1:] - vel[:-1])
+    pen = get_norm(acc, norm).mean(axis=-1)
+    return np.where(np.arange(len(pen)) >= 2, pen, 0.0)
+
+
+def action_jerk_penalty(action_ta, done_t, norm="l2"):  # rewards.py:449-460
+    a = _edge_pad_front(np.asarray(action_ta, dtype=np.float64), 3)
+    done = _edge_pad_front(np.asarray(done_t).astype(bool), 3)[:-1, None]
+    vel = np.where(done, 0.0, a[1:] - a[:-1])
+    acc = np.where(done[1:], 0.0, vel[1:] - vel[:-1])
+    jerk = np.where(done[2:], 0.0, acc[1:] - acc[:-1])
+    pen = get_norm(jerk, norm).mean(axis=-1)
+    return np.where(np.arange(len(pen)) >= 3, pen, 0.0)
+
+
+def stay_alive_reward(done_t, success_t, balance=100.0, success_reward=None):  # rewards.py:178-188
+    alive = 1.0 / balance
+    return np.where(done_t, np.where(success_t, alive if success_reward is None else success_reward, -1.0), alive)
+
+
+def base_height_reward(qpos_tq, height_target, kernel_scale=0.25):  # rewards.py:382-385
+    return exp_kernel(np.asarray(qpos_tq)[..., 2] - height_target, kernel_scale)
+
+
+def base_height_range_reward(qpos_tq, z_lower, z_upper, dropoff):  # rewards.py:396-401
+    z = np.asarray(qpos_tq)[..., 2]
+    return np.clip(1.0 - np.clip(np.maximum(z_lower - z, z - z_upper), 0.0, None) * dropoff, 0.0, None)
+
+
+def upright_reward(qpos_tq, qvel_tv, s=0.25, sq=0.1, ab=0.1):  # rewards.py:760-777 (defaults)
+    qpos = np.asarray(qpos_tq, dtype=np.float64)
+    qvel = np.asarray(qvel_tv, dtype=np.float64)
+    z_b = rotate_vector_by_quat(np.broadcast_to([0.0, 0.0, 1.0], qpos.shape[:-1] + (3,)), qpos[..., 3:7], inverse=True)
+    pitch = np.arctan2(z_b[..., 0], z_b[..., 2])
+    return {
+        "angvel": exp_kernel_with_penalty(qvel[..., 4], s, sq, ab),
+        "linvel": exp_kernel_with_penalty(qvel[..., 2], s, sq, ab),
+        "pose": exp_kernel_with_penalty(pitch, s, sq, ab),
+    }
+
+
+def total_reward(components, scales, is_penalty, clip_min=None, clip_max=None):
+    """rl.py:219-239: each term * (+/-)scale, summed in insertion order, optional clip."""
+    total = None
+    out = {}
+    for name, val in components.items():
+        s = -scales[name] if is_penalty[name] else scales[name]
+        out[name] = np.asarray(val) * s
+        total = out[name] if total is None else total + out[name]
+    if clip_min is not None:
+        total = np.maximum(total, clip_min)
+    if clip_max is not None:
+        total = np.minimum(total, clip_max)
+    return total, out
+
+
+# --------------------------------------------------------------------------- terminations (int32 in {-1, 0, +1})
+def minimum_height_termination(qpos, min_height):  # terminations.py:79-80
+    return np.where(np.asarray(qpos)[..., 2] < min_height, -1, 0).astype(np.int32)
+
+
+def bad_z_termination(qpos, min_z, max_z, level=0.0, final_min_z=None, final_max_z=None):  # terminations.py:140-146
+    z = np.asarray(qpos)[..., 2]
+    fmin = min_z if final_min_z is None else final_min_z
+    fmax = max_z if final_max_z is None else final_max_z
+    lo = (fmin - min_z) * level + min_z
+    hi = (fmax - max_z) * level + max_z
+    return np.where((z < lo) | (z > hi), -1, 0).astype(np.int32)
+
+
+def not_upright_termination(qpos, max_radians):  # terminations.py:66-70
+    qpos = np.asarray(qpos, dtype=np.float64)
+    g = rotate_vector_by_quat(np.broadcast_to([0.0, 0.0, 1.0], qpos.shape[:-1] + (3,)), qpos[..., 3:7], inverse=True)
+    return np.where(np.arccos(np.clip(g[..., 2], -1.0, 1.0)) > max_radians, -1, 0).astype(np.int32)
+
+
+def bad_velocity_termination(qvel, max_vel):  # terminations.py:155-157
+    return np.where(np.linalg.norm(np.asarray(qvel)[..., 0:3], axis=-1) > max_vel, -1, 0).astype(np.int32)
+
+
+def far_from_origin_termination(qpos, max_dist, pos_termination=True):  # terminations.py:170-172
+    val = 1 if pos_termination else -1
+    return np.where(np.linalg.norm(np.asarray(qpos)[..., :3], axis=-1) > max_dist, val, 0).astype(np.int32)
+
+
+def episode_length_termination(time, max_length_sec, pos_termination=True):  # terminations.py:186-192
+    val = 1 if pos_termination else -1
+    return np.where(np.asarray(time) > max_length_sec, val, 0).astype(np.int32)
+
+
+def illegal_contact_termination(ncon, geom1, geom2, dist, illegal_geom_idxs, contact_eps=-1e-3):  # terminations.py:90-99
+    if ncon == 0:
+        return np.int32(0)
+    bad = np.isin(geom1, illegal_geom_idxs) | np.isin(geom2, illegal_geom_idxs)
+    return np.int32(-1 if np.any(np.where(bad, np.asarray(dist) < contact_eps, False)) else 0)
+
+
+def combine_terminations(terms):
+    """rl.py:1049-1050: done = OR(t != 0); success = AND(t != -1) & done."""
+    terms = [np.asarray(t) for t in terms]
+    done = np.zeros(terms[0].shape, dtype=bool)
+    succ = np.ones(terms[0].shape, dtype=bool)
+    for t in terms:
+        done |= t != 0
+        succ &= t != -1
+    return done, succ & done
+
+
+# --------------------------------------------------------------------------- actuator / engine sub-step helpers
+def position_actuator_torque(
+    action, qpos_j, qvel_j, kp, kd, ctrl_clip,
+    action_scale=1.0, action_noise=0.0, action_bias=0.0, torque_noise=0.0, torque_bias=0.0,
+    kp_scale=1.0, kd_scale=1.0, torque_limit_scale=1.0,
+):
+    """actuators.py:198-217 with the noise draws passed in as explicit arrays."""
+    target = action * action_scale + action_noise + action_bias
+    ctrl = (kp * kp_scale) * (target - qpos_j) + (kd * kd_scale) * (0.0 - qvel_j)
+    ctrl = ctrl + torque_noise + torque_bias
+    lim = ctrl_clip * torque_limit_scale
+    return np.clip(ctrl, -lim, lim)
+
+
+def latency_blend(step_num, latency, last_ctrl, action, drop):
+    """engine.py:287-288."""
+    prct = np.clip(step_num - latency, 0.0, 1.0)
+    return np.where(drop, last_ctrl, last_ctrl * (1.0 - prct) + action * prct)
+
+
+def scrub_action(action, clip_max=1e3):
+    """rl.py:998-1001: NaN -> 0, then clip."""
+    a = np.where(np.isnan(action), 0.0, action)
+    return np.clip(a, -clip_max, clip_max)

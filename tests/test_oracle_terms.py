@@ -1,0 +1,90 @@
+"""Pins oracle/terms.py against the reference's own known-answer vectors (CPU only)."""
+import itertools
+import json
+import os
+
+import numpy as np
+import pytest
+
+from oracle import terms
+
+GOLD = os.path.join(os.path.dirname(__file__), "golden")
+REWARD_KATS = json.load(open(os.path.join(GOLD, "reward_kats.json")))
+TERM_KATS = json.load(open(os.path.join(GOLD, "termination_kats.json")))
+FN = {"velocity": terms.action_velocity_penalty, "acceleration": terms.action_acceleration_penalty,
+      "jerk": terms.action_jerk_penalty}
+
+
+@pytest.mark.parametrize("kat", REWARD_KATS, ids=[k["ref"] for k in REWARD_KATS])
+def test_reward_kats(kat):
+    a = np.array(kat["actions"], dtype=np.float64)
+    done = np.zeros(len(a), bool) if kat["done"] is None else np.array(kat["done"])
+    got = FN[kat["fn"]](a, done, kat["norm"])
+    np.testing.assert_allclose(got, kat["expected"], atol=kat["atol"], rtol=0)
+
+
+@pytest.mark.parametrize("kat", TERM_KATS, ids=[f'{k["fn"]}-{i}' for i, k in enumerate(TERM_KATS)])
+def test_termination_kats(kat):
+    if kat["fn"] == "not_upright":
+        got = terms.not_upright_termination(np.array(kat["qpos"]), kat["max_radians"])
+    elif kat["fn"] == "minimum_height":
+        got = terms.minimum_height_termination(np.array(kat["qpos"]), kat["min_height"])
+    else:
+        got = terms.illegal_contact_termination(kat["ncon"], np.array(kat["geom1"]), np.array(kat["geom2"]),
+                                                np.array(kat["dist"]), np.array(kat["illegal"]))
+    assert int(got) == kat["expected"]
+
+
+def test_done_success_truth_table():
+    for k in (1, 2, 3):
+        for combo in itertools.product([-1, 0, 1], repeat=k):
+            done, succ = terms.combine_terminations([np.array(c) for c in combo])
+            assert bool(done) == any(c != 0 for c in combo)
+            assert bool(succ) == (any(c != 0 for c in combo) and all(c != -1 for c in combo))
+
+
+def test_rotate_vector_by_quat_against_scipy():
+    from scipy.spatial.transform import Rotation
+
+    rng = np.random.default_rng(0)
+    q = rng.normal(size=(20, 4))
+    v = rng.normal(size=(20, 3))
+    R = Rotation.from_quat(q[:, [1, 2, 3, 0]])  # scipy is xyzw and normalises
+    np.testing.assert_allclose(terms.rotate_vector_by_quat(v, q), R.apply(v), atol=1e-12)
+    np.testing.assert_allclose(terms.rotate_vector_by_quat(v, q, inverse=True), R.inv().apply(v), atol=1e-12)
+
+
+def test_latency_blend_cases():
+    last, act = np.array([1.0, 2.0]), np.array([5.0, 6.0])
+    nodrop = np.array([False, False])
+    # latency 0: substep 0 still applies the previous ctrl, substep >= 1 the new action (engine.py:287-288)
+    np.testing.assert_array_equal(terms.latency_blend(0.0, 0.0, last, act, nodrop), last)
+    np.testing.assert_array_equal(terms.latency_blend(1.0, 0.0, last, act, nodrop), act)
+    # latency >= S: never switches; fractional latency blends linearly
+    for s in range(4):
+        np.testing.assert_array_equal(terms.latency_blend(float(s), 4.0, last, act, nodrop), last)
+    np.testing.assert_allclose(terms.latency_blend(1.0, 0.25, last, act, nodrop), last * 0.25 + act * 0.75)
+    np.testing.assert_array_equal(terms.latency_blend(3.0, 0.0, last, act, np.array([True, False])), [1.0, 6.0])
+
+
+def test_pd_actuator_and_scrub():
+    tau = terms.position_actuator_torque(np.array([0.5, -2.0]), np.array([0.1, 0.0]), np.array([1.0, -1.0]),
+                                         kp=np.array([20.0, 100.0]), kd=np.array([1.0, 2.0]), ctrl_clip=np.array([np.inf, 50.0]))
+    np.testing.assert_allclose(tau, [20 * 0.4 - 1.0, -50.0])
+    a = terms.scrub_action(np.array([np.nan, 2e3, -5.0, -1e9]))
+    np.testing.assert_array_equal(a, [0.0, 1e3, -5.0, -1e3])
+
+
+def test_simple_rewards():
+    done = np.array([False, True, True]); succ = np.array([False, False, True])
+    np.testing.assert_allclose(terms.stay_alive_reward(done, succ), [0.01, -1.0, 0.01])
+    np.testing.assert_allclose(terms.stay_alive_reward(done, succ, success_reward=3.0), [0.01, -1.0, 3.0])
+    q = np.zeros((2, 9)); q[:, 2] = [1.0, 1.5]; q[:, 3] = 1.0
+    np.testing.assert_allclose(terms.base_height_reward(q, 1.0), [1.0, np.exp(-0.25 / (2 * 0.0625))])
+    np.testing.assert_allclose(terms.base_height_range_reward(q, 0.8, 1.2, 2.0), [1.0, 0.4])
+    up = terms.upright_reward(q, np.zeros((2, 8)))
+    np.testing.assert_allclose(up["pose"], [1.0, 1.0])
+    tot, comps = terms.total_reward({"a_reward": np.array([1.0, 2.0]), "b_penalty": np.array([4.0, 0.5])},
+                                    {"a_reward": 2.0, "b_penalty": 0.5}, {"a_reward": False, "b_penalty": True},
+                                    clip_min=0.5)
+    np.testing.assert_allclose(tot, [0.5, 3.75])
