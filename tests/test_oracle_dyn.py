@@ -1,0 +1,296 @@
+"""Pins the C dynamics oracle against brute force, closed forms and invariants (CPU only, float64)."""
+import numpy as np
+import pytest
+from scipy.optimize import minimize
+from scipy.spatial.transform import Rotation
+
+from ksim_amd import model as km
+from oracle.dyn import Oracle
+
+
+def _random_state(m, rng, vel_scale=1.0):
+    qpos = m.qpos0.copy()
+    qvel = rng.normal(size=m.nv) * vel_scale
+    for b in range(1, m.nb):
+        qa = m.body_qadr[b]
+        if m.body_jtype[b] == km.JNT_FREE:
+            qpos[qa:qa + 3] += rng.normal(size=3) * 0.3
+            q = rng.normal(size=4)
+            qpos[qa + 3:qa + 7] = q / np.linalg.norm(q)
+        else:
+            qpos[qa] = rng.uniform(-1.0, 1.0)
+    return qpos, qvel
+
+
+def _integrate_pos(m, qpos, qvel, h):
+    """Independent position integration (scipy rotations) used for finite differences."""
+    out = qpos.copy()
+    for b in range(1, m.nb):
+        qa, da = m.body_qadr[b], m.body_dofadr[b]
+        if m.body_jtype[b] == km.JNT_FREE:
+            out[qa:qa + 3] += h * qvel[da:da + 3]
+            R = Rotation.from_quat(qpos[qa + 3:qa + 7][[1, 2, 3, 0]]) * Rotation.from_rotvec(h * qvel[da + 3:da + 6])
+            out[qa + 3:qa + 7] = R.as_quat()[[3, 0, 1, 2]]
+        else:
+            out[qa] += h * qvel[da]
+    return out
+
+
+
+def _sink_to_contact(m, qpos, depth=0.01):
+    """Moves a free-root model vertically so that its lowest contact sphere penetrates by ``depth``."""
+    kin = km.host_kinematics(m.arrays(), qpos)
+    low = min(kin["xpos"][b][2] + (kin["xmat"][b] @ p)[2] - r for b, p, r in zip(m.sph_body, m.sph_pos, m.sph_radius))
+    out = qpos.copy()
+    out[2] -= low + depth
+    return out
+
+
+MODELS = {
+    "chain": lambda: km.pendulum_chain_model(),
+    "humanoid": lambda: km.humanoid_model(),
+    "kbot": lambda: km.kbot_scale_model(),
+}
+
+
+@pytest.fixture(scope="module", params=list(MODELS))
+def model(request):
+    return MODELS[request.param]()
+
+
+def test_model_dimensions():
+    h, k, c = km.humanoid_model(), km.kbot_scale_model(), km.pendulum_chain_model()
+    assert (h.nq, h.nv, h.nu, h.nb, h.ns) == (28, 27, 21, 23, 4)
+    assert (k.nq, k.nv, k.nu, k.nb, k.ns) == (27, 26, 20, 22, 8)
+    assert (c.nq, c.nv, c.nu, c.nb, c.ns) == (3, 3, 3, 4, 0)
+
+
+def test_kinematics_against_brute_force_and_invariants(model):
+    rng = np.random.default_rng(0)
+    orc = Oracle(model.arrays())
+    for _ in range(3):
+        qpos, _ = _random_state(model, rng)
+        d = orc.data(qpos)
+        orc.position_stage(d)
+        kin = km.host_kinematics(model.arrays(), qpos)
+        for k in ("xpos", "xmat", "xipos", "ximat", "xanchor"):
+            np.testing.assert_allclose(getattr(d, k).reshape(model.nb, -1), kin[k].reshape(model.nb, -1), atol=1e-12)
+        np.testing.assert_allclose(np.linalg.norm(d.xquat, axis=1), 1.0, atol=1e-12)
+        R = d.xmat.reshape(-1, 3, 3)
+        np.testing.assert_allclose(np.einsum("bij,bkj->bik", R, R), np.broadcast_to(np.eye(3), R.shape), atol=1e-12)
+
+
+def test_planar_chain_closed_form():
+    m = km.pendulum_chain_model()
+    orc = Oracle(m.arrays())
+    q = np.array([0.3, -0.5, 0.9])
+    d = orc.data(q)
+    orc.position_stage(d)
+    # hinge about +y rotates the -z link towards -x: tip_k = sum_j L * (-sin(th_j), 0, -cos(th_j)), th_j cumulative
+    th = np.cumsum(q)
+    joints = np.concatenate([[np.zeros(3)], np.cumsum(0.5 * np.stack([-np.sin(th), 0 * th, -np.cos(th)], 1), 0)])
+    np.testing.assert_allclose(d.xpos[1:], joints[:3], atol=1e-12)
+    # textbook mass matrix entry: M[2,2] = I_yy + m (L/2)^2 for the last link about its own hinge
+    I = km.capsule_inertia(1.0, 0.05, 0.5)[0]
+    assert d.M[2, 2] == pytest.approx(I + 0.25**2, rel=1e-12)
+
+
+def test_mass_matrix_against_jacobian_sum(model):
+    rng = np.random.default_rng(1)
+    orc = Oracle(model.arrays())
+    for trial in range(3):
+        qpos, _ = _random_state(model, rng)
+        scale = rng.uniform(0.9, 1.1, size=model.nb) if trial else None
+        d = orc.data(qpos, mass_scale=scale)
+        orc.position_stage(d)
+        M = km.host_mass_matrix(model.arrays(), qpos, scale)
+        np.testing.assert_allclose(d.M, M, rtol=1e-10, atol=1e-11)
+        np.testing.assert_allclose(d.M, d.M.T, atol=0)
+        assert np.linalg.eigvalsh(d.M).min() > 0
+
+
+def _bias_projected_newton_euler(m, qpos, qvel, eps=1e-6):
+    """sum_b Jp^T m (Jp_dot qd - g) + Jr^T (I Jr_dot qd + w x I w): independent of the oracle's RNE."""
+    a = m.arrays()
+    kin0 = km.host_kinematics(a, qpos)
+    kin1 = km.host_kinematics(a, _integrate_pos(m, qpos, qvel, eps))
+    kinm = km.host_kinematics(a, _integrate_pos(m, qpos, qvel, -eps))
+    out = np.zeros(m.nv)
+    for b in range(1, m.nb):
+        jp, jr = km.host_jacobian(a, kin0, kin0["xipos"][b], b)
+        jp1, jr1 = km.host_jacobian(a, kin1, kin1["xipos"][b], b)
+        jpm, jrm = km.host_jacobian(a, kinm, kinm["xipos"][b], b)
+        acc = (jp1 - jpm) / (2 * eps) @ qvel
+        alpha = (jr1 - jrm) / (2 * eps) @ qvel
+        w = jr @ qvel
+        Iw = kin0["ximat"][b] @ np.diag(m.body_inertia[b]) @ kin0["ximat"][b].T
+        out += jp.T @ (m.body_mass[b] * (acc - m.gravity)) + jr.T @ (Iw @ alpha + np.cross(w, Iw @ w))
+    return out
+
+
+def test_bias_forces_against_projected_newton_euler(model):
+    rng = np.random.default_rng(2)
+    orc = Oracle(model.arrays())
+    for _ in range(3):
+        qpos, qvel = _random_state(model, rng)
+        d = orc.data(qpos, qvel)
+        orc.position_stage(d)
+        orc.velocity_stage(d)
+        want = _bias_projected_newton_euler(model, qpos, qvel)
+        np.testing.assert_allclose(d.qfrc_bias, want, rtol=1e-6, atol=1e-6 * np.abs(want).max())
+    # zero velocity: pure gravity torque = -dU/dq ... bias = dU/dq by finite differences of potential energy
+    qpos, _ = _random_state(model, rng)
+    d = orc.data(qpos, np.zeros(model.nv))
+    orc.position_stage(d)
+    orc.velocity_stage(d)
+
+    def U(q):
+        kin = km.host_kinematics(model.arrays(), q)
+        return -sum(model.body_mass[b] * model.gravity @ kin["xipos"][b] for b in range(1, model.nb))
+
+    g = np.zeros(model.nv)
+    for i in range(model.nv):
+        e = np.zeros(model.nv); e[i] = 1.0
+        g[i] = (U(_integrate_pos(model, qpos, e, 1e-6)) - U(_integrate_pos(model, qpos, e, -1e-6))) / 2e-6
+    np.testing.assert_allclose(d.qfrc_bias, g, rtol=1e-6, atol=1e-6)
+
+
+def test_energy_conservation_of_the_undamped_chain():
+    m = km.pendulum_chain_model(damping=0.0, dt=1e-4)
+    orc = Oracle(m.arrays())
+    d = orc.data(np.array([0.8, -0.4, 0.3]))
+
+    def energy():
+        orc.position_stage(d)
+        kin = km.host_kinematics(m.arrays(), np.array(d.qpos))
+        return 0.5 * d.qvel @ d.M @ d.qvel - sum(m.body_mass[b] * m.gravity @ kin["xipos"][b] for b in range(1, m.nb))
+
+    e0 = energy()
+    for _ in range(2000):
+        orc.step(d)
+    assert abs(energy() - e0) < 2e-3 * abs(e0) + 1e-3
+    assert d.time == pytest.approx(0.2)
+
+
+def _ball(radius=0.1, mass=2.0, z=0.5, **opts):
+    mb = km.ModelBuilder(**opts)
+    b = mb.add_body(0, (0, 0, z), joint="free", mass=mass, inertia=[0.4 * mass * radius**2] * 3, name="ball")
+    mb.add_contact_sphere(b, (0, 0, 0), radius)
+    return mb.build()
+
+
+def test_free_fall_closed_form_and_quaternion_integration():
+    m = _ball(z=10.0)
+    orc = Oracle(m.arrays())
+    w = np.array([0.3, -1.1, 0.7])
+    d = orc.data(qvel=np.concatenate([[0.5, 0, 0], w]))
+    z, v = 10.0, 0.0
+    for _ in range(50):
+        orc.step(d)
+        v -= 9.81 * m.dt
+        z += v * m.dt
+    assert d.qpos[2] == pytest.approx(z, abs=1e-12) and d.qvel[2] == pytest.approx(v, abs=1e-12)
+    assert d.qpos[0] == pytest.approx(0.5 * 50 * m.dt)
+    # a symmetric ball keeps its body-frame angular velocity: orientation = exp(w t)
+    np.testing.assert_allclose(d.qvel[3:6], w, atol=1e-12)
+    R = Rotation.from_rotvec(w * 50 * m.dt).as_quat()[[3, 0, 1, 2]]
+    got = np.array(d.qpos[3:7])
+    np.testing.assert_allclose(got * np.sign(got[0]), R * np.sign(R[0]), atol=1e-10)
+
+
+def test_contact_geometry_and_jacobian(model):
+    if model.ns == 0:
+        pytest.skip("no contacts")
+    rng = np.random.default_rng(3)
+    orc = Oracle(model.arrays())
+    qpos, qvel = _random_state(model, rng)
+    qpos = _sink_to_contact(model, qpos)
+    d = orc.data(qpos, qvel, friction=0.7)
+    orc.forward(d)
+    kin = km.host_kinematics(model.arrays(), qpos)
+    centres = np.array([kin["xpos"][b] + kin["xmat"][b] @ p for b, p in zip(model.sph_body, model.sph_pos)])
+    np.testing.assert_allclose(d.con_dist, centres[:, 2] - model.sph_radius, atol=1e-12)
+    active = np.where(np.array(d.con_dist) < 0)[0]
+    assert d.nefc == 4 * len(active) and len(active) > 0
+    mu = 0.7
+    for r, s in enumerate(active):
+        jp, _ = km.host_jacobian(model.arrays(), kin, np.array(d.con_pos[s]), model.sph_body[s])
+        rows = np.stack([jp[2] + mu * jp[1], jp[2] - mu * jp[1], jp[2] - mu * jp[0], jp[2] + mu * jp[0]])
+        np.testing.assert_allclose(d.efc_J[4 * r:4 * r + 4], rows, atol=1e-11)
+        assert np.all(np.array(d.efc_pos[4 * r:4 * r + 4]) == d.con_dist[s])
+    # velocity of the contact point by finite differences = J qvel (normal row of an un-tilted pyramid)
+    s = active[0]
+    b = model.sph_body[s]
+    local = kin["xmat"][b].T @ (np.array(d.con_pos[s]) - kin["xpos"][b])
+    k1 = km.host_kinematics(model.arrays(), _integrate_pos(model, qpos, qvel, 1e-7))
+    vel_fd = ((k1["xpos"][b] + k1["xmat"][b] @ local) - np.array(d.con_pos[s])) / 1e-7
+    jp, _ = km.host_jacobian(model.arrays(), kin, np.array(d.con_pos[s]), b)
+    np.testing.assert_allclose(jp @ qvel, vel_fd, atol=1e-5)
+
+
+def _cost(orc, d, a):
+    nv = len(a)
+    r = d.efc_J @ a - d.efc_aref
+    da = a - d.qacc_smooth
+    return 0.5 * da @ d.M @ da + 0.5 * np.sum(d.efc_D * np.minimum(r, 0.0) ** 2)
+
+
+def test_solver_fixed_point_kkt_and_scipy(model):
+    if model.ns == 0:
+        pytest.skip("no contacts")
+    rng = np.random.default_rng(4)
+    a = dict(model.arrays()); a["iterations"] = 100; a["ls_iterations"] = 50
+    orc = Oracle(a)
+    qpos, qvel = _random_state(model, rng, vel_scale=0.5)
+    qpos = _sink_to_contact(model, qpos)
+    d = orc.data(qpos, qvel)
+    d.ctrl = rng.normal(size=model.nu)
+    orc.forward(d)
+    assert d.nefc > 0
+    acc = np.array(d.qacc)
+    r = d.efc_J @ acc - d.efc_aref
+    f = np.where(r < 0, -d.efc_D * r, 0.0)
+    np.testing.assert_allclose(d.efc_force, f, rtol=1e-9, atol=1e-9)
+    resid = d.M @ (acc - d.qacc_smooth) - d.efc_J.T @ f
+    assert np.abs(resid).max() < 1e-7 * max(1.0, np.abs(d.M @ acc).max())
+    np.testing.assert_allclose(d.qfrc_constraint, d.efc_J.T @ f, atol=1e-8)
+    # an independent minimiser of the same convex cost cannot do better, and lands on the same point
+    res = minimize(lambda x: _cost(orc, d, x), np.array(d.qacc_smooth), method="BFGS", options=dict(gtol=1e-9, maxiter=5000))
+    assert _cost(orc, d, acc) <= res.fun + 1e-9 * max(1.0, abs(res.fun))
+    # smooth dynamics identity: M qacc_smooth = passive - bias + actuator
+    np.testing.assert_allclose(d.M @ d.qacc_smooth, d.qfrc_passive - d.qfrc_bias + d.qfrc_actuator, atol=1e-9)
+
+
+def test_ball_rests_at_the_depth_the_spring_damper_predicts():
+    m = _ball(z=0.1, friction=1.0)
+    orc = Oracle(m.arrays())
+    d = orc.data()
+    for _ in range(2000):
+        orc.step(d)
+    assert np.abs(d.qvel).max() < 1e-6
+    pos = d.qpos[2] - 0.1
+    assert pos < 0
+    # at rest: 4 pyramid rows, each carrying D * k * imp * |pos|; their normal components sum to m g
+    dmin, dmax, width, mid, power = m.solimp
+    tc = max(m.solref[0], 2 * m.dt)
+    k = 1 / (dmax**2 * tc**2 * m.solref[1] ** 2)
+    x = abs(pos) / width
+    y = (1 / mid ** (power - 1)) * x**power if x < mid else 1 - (1 / (1 - mid) ** (power - 1)) * (1 - x) ** power
+    imp = dmax if x > 1 else np.clip(dmin + y * (dmax - dmin), dmin, dmax)
+    t = 1 / 2.0  # translational inverse weight of a free 2 kg ball
+    R = (t + t) * 2 / 1.0 * (1 - imp) / imp
+    assert 4 * (1 / R) * k * imp * abs(pos) == pytest.approx(2.0 * 9.81, rel=1e-6)
+    assert m.body_invweight0[1, 0] == pytest.approx(t)
+
+
+def test_float_and_double_oracles_agree():
+    m = km.kbot_scale_model()
+    rng = np.random.default_rng(5)
+    qpos, qvel = _random_state(m, rng, vel_scale=0.3)
+    qpos = _sink_to_contact(m, qpos)
+    o64, o32 = Oracle(m.arrays(), np.float64), Oracle(m.arrays(), np.float32)
+    d64, d32 = o64.data(qpos, qvel), o32.data(qpos, qvel)
+    o64.forward(d64); o32.forward(d32)
+    assert d64.nefc == d32.nefc and d64.nefc > 0
+    scale = np.abs(d64.qacc).max()
+    assert np.abs(np.array(d32.qacc) - d64.qacc).max() < 2e-4 * scale
