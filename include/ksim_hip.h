@@ -91,6 +91,109 @@ int ks_reward_total(ks_stream_t stream, int64_t n, int32_t K, const float* compo
                     int32_t use_clip_max, float clip_max, float* total, int32_t k,
                     const int8_t* terminations, uint8_t* done, uint8_t* success);
 
+/* ------------------------------------------------------------------ physics model
+ * Replaces the mjx.Model produced by ksim/utils/mujoco.py:388-391 (mjx.put_model) for the
+ * model subset of the rollout configs: a kinematic tree whose bodies (depth-first order,
+ * body 0 = world) each carry one free or hinge joint, motor actuators (one per dof at
+ * most) and contact spheres against the ground plane z = 0 with pyramidal friction cones.
+ * ks_model_create copies the description to the current HIP device (the only call that
+ * allocates); the handle is immutable afterwards.
+ */
+#define KS_MAX_BODIES 32
+#define KS_MAX_QPOS 40
+#define KS_MAX_DOFS 32
+#define KS_MAX_ACTUATORS 32
+#define KS_MAX_SPHERES 16
+enum { KS_JNT_NONE = 0, KS_JNT_FREE = 1, KS_JNT_HINGE = 2 };
+
+typedef struct KsModelDesc {
+  int32_t nb, nq, nv, nu, ns;
+  int32_t iterations, ls_iterations; /* Newton / line-search limits (ksim/task/rl.py:717-748 sets opt.*) */
+  int32_t eulerdamp;                 /* must be 0: ksim disables EULERDAMP (rl.py:575-578,745-746) */
+  double dt, gravity[3], tolerance, ls_tolerance, impratio, meaninertia, friction;
+  double solref[2], solimp[5];
+  int32_t body_parent[KS_MAX_BODIES], body_jtype[KS_MAX_BODIES], body_qadr[KS_MAX_BODIES],
+      body_dofadr[KS_MAX_BODIES], body_subtree_end[KS_MAX_BODIES];
+  double body_pos[KS_MAX_BODIES][3], body_quat[KS_MAX_BODIES][4], body_mass[KS_MAX_BODIES],
+      body_ipos[KS_MAX_BODIES][3], body_iquat[KS_MAX_BODIES][4], body_inertia[KS_MAX_BODIES][3],
+      jnt_axis[KS_MAX_BODIES][3], jnt_pos[KS_MAX_BODIES][3], body_invweight0[KS_MAX_BODIES];
+  double qpos0[KS_MAX_QPOS];
+  int32_t dof_body[KS_MAX_DOFS], dof_parent[KS_MAX_DOFS];
+  double dof_damping[KS_MAX_DOFS], dof_armature[KS_MAX_DOFS];
+  int32_t act_dof[KS_MAX_ACTUATORS];
+  double act_gear[KS_MAX_ACTUATORS], act_lo[KS_MAX_ACTUATORS], act_hi[KS_MAX_ACTUATORS];
+  int32_t sph_body[KS_MAX_SPHERES];
+  double sph_pos[KS_MAX_SPHERES][3], sph_radius[KS_MAX_SPHERES];
+} KsModelDesc;
+
+typedef struct KsModel KsModel;
+int ks_model_create(const KsModelDesc* desc /*host*/, KsModel** out);
+int ks_model_destroy(KsModel* model);
+int ks_model_lds_bytes(const KsModel* model); /* LDS one env needs in the step kernel */
+
+/* ------------------------------------------------------------------ control step / forward
+ * ks_step replaces MjxEngine.step (ksim/engine.py:259-361): `substeps` physics steps of
+ * mjx.step (engine.py:257) with the latency blend (287-288), the actuator update every
+ * `actuator_period` substeps (290-318) and last_ctrl <- action (355), for N envs at once
+ * (the reference vmaps the per-env call, ksim/task/rl.py:1615).
+ * ks_forward replaces the mjx.forward of MjxEngine.reset (engine.py:213): derived fields
+ * and the warm start for the given qpos/qvel/ctrl_in, without integrating.
+ *
+ * All arrays are env-major rows: (N, dim) f32, like the reference's vmapped pytrees.
+ * Nullable inputs fall back to: latency 0, zero_offset 0, no drops, scales 1, no noise,
+ * no bias, model friction, mass scale 1.  Noise arrays are explicit pre-sampled draws,
+ * (substeps, N, nu), so that results can be compared on identical seeded inputs.
+ */
+enum { KS_ACT_TORQUE = 0, KS_ACT_POSITION = 1 }; /* actuators.py:70-87 / 98-238 */
+
+typedef struct KsStepIO {
+  int64_t N;
+  int32_t substeps;        /* EngineData.phys_steps_per_ctrl_steps, engine.py:150 */
+  int32_t actuator_period; /* EngineData.phys_steps_per_actuator_step, engine.py:151 */
+  int32_t actuator_type;
+  float action_scale;      /* PositionActuators.action_scale, actuators.py:107 */
+  /* state, in/out */
+  float* qpos;             /* (N, nq) */
+  float* qvel;             /* (N, nv) */
+  float* qacc_warmstart;   /* (N, nv) */
+  float* time;             /* (N) nullable */
+  float* last_ctrl;        /* (N, nu) PhysicsState.last_ctrl, ksim/types.py:33-43 */
+  /* inputs */
+  const float* action;      /* (N, nu) */
+  const float* ctrl_in;     /* (N, nu) ks_forward only: data.ctrl; nullable = 0 */
+  const float* latency;     /* (N) PhysicsState.action_latency in substeps */
+  const float* zero_offset; /* (N, nu) */
+  const uint8_t* drop;      /* (N, nu) drop_action mask, engine.py:277-278 */
+  const float* kp;          /* (nu) */
+  const float* kd;          /* (nu) */
+  const float* ctrl_clip;   /* (nu), +inf = unlimited */
+  const float* kp_scale;    /* (N) ActuatorState, actuators.py:90-95 */
+  const float* kd_scale;    /* (N) */
+  const float* torque_limit_scale; /* (N) */
+  const float* action_bias; /* (N, nu) */
+  const float* torque_bias; /* (N, nu) */
+  const float* action_noise; /* (substeps, N, nu) */
+  const float* torque_noise; /* (substeps, N, nu) */
+  const float* friction;    /* (N) per-env contact friction (FloorFrictionRandomizer, randomization.py:74-104) */
+  const float* mass_scale;  /* (N, nb) per-env body mass factor (randomization.py:207-222) */
+  /* outputs, each nullable */
+  float* qacc;              /* (N, nv) of the last substep */
+  float* ctrl_out;          /* (N, nu) torques applied in the last substep = data.ctrl */
+  float* xpos;              /* (N, nb*3) body positions at the start of the last substep */
+  float* xquat;             /* (N, nb*4) */
+  float* cvel;              /* (N, nb*6) com-based body velocities [angular; linear] */
+  int32_t* solver_niter;    /* (N) Newton iterations of the last substep */
+  int32_t* nefc;            /* (N) active constraint rows of the last substep */
+  /* intermediate quantities for parity tests, each nullable */
+  float* dbg_M;             /* (N, nv*nv) */
+  float* dbg_bias;          /* (N, nv) */
+  float* dbg_qacc_smooth;   /* (N, nv) */
+  float* dbg_con_dist;      /* (N, ns) */
+} KsStepIO;
+
+int ks_step(const KsModel* model, ks_stream_t stream, const KsStepIO* io /*host*/);
+int ks_forward(const KsModel* model, ks_stream_t stream, const KsStepIO* io /*host*/);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,25 @@
+// Kernel argument block of the fused control-step kernel (device pointers, passed by value).
+#pragma once
+#include <stdint.h>
+
+namespace ks {
+
+struct DevModel;
+
+struct StepArgs {
+  const DevModel* model;
+  int64_t N;
+  int substeps, actuator_period, actuator_type, forward_only;
+  float action_scale;
+  float *qpos, *qvel, *qacc_warmstart, *time, *last_ctrl;
+  const float *action, *ctrl_in, *latency, *zero_offset;
+  const uint8_t* drop;
+  const float *kp, *kd, *ctrl_clip, *kp_scale, *kd_scale, *torque_limit_scale;
+  const float *action_bias, *torque_bias, *action_noise, *torque_noise;
+  const float *friction, *mass_scale;
+  float *qacc, *ctrl_out, *xpos, *xquat, *cvel;
+  int32_t *solver_niter, *nefc;
+  float *dbg_M, *dbg_bias, *dbg_qacc_smooth, *dbg_con_dist;
+};
+
+}  // namespace ks

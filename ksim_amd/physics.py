@@ -1,0 +1,114 @@
+"""Device-resident physics model and the batched control-step call (thin layer over the C ABI).
+
+``DeviceModel`` plays the part of the ``mjx.Model`` that ``mjx.put_model`` returns
+(ksim/utils/mujoco.py:388-391); ``control_step`` / ``forward`` are the batched forms of
+``MjxEngine.step`` / the ``mjx.forward`` inside ``MjxEngine.reset`` (ksim/engine.py:205-361).
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Mapping
+
+import torch
+
+from . import _lib, _lib_dyn
+from .model import KinematicModel
+
+
+class DeviceModel:
+    """Handle of a model uploaded to the current GPU. Immutable; hashable by identity."""
+
+    def __init__(self, model: KinematicModel):
+        lib = _lib.load()
+        if not torch.cuda.is_available():
+            raise _lib.KsError("DeviceModel needs a GPU (there is no CPU path)")
+        torch.cuda.current_device()  # make sure a HIP context exists
+        torch.zeros(1, device="cuda")
+        self.model = model
+        self._lib = lib
+        self._handle = ctypes.c_void_p()
+        desc = _lib_dyn.model_desc(model)
+        _lib.check(lib.ks_model_create(ctypes.byref(desc), ctypes.byref(self._handle)))
+
+    @property
+    def handle(self) -> ctypes.c_void_p:
+        if not self._handle:
+            raise _lib.KsError("model handle was closed")
+        return self._handle
+
+    @property
+    def lds_bytes(self) -> int:
+        return int(self._lib.ks_model_lds_bytes(self.handle))
+
+    def close(self) -> None:
+        if self._handle:
+            self._lib.ks_model_destroy(self._handle)
+            self._handle = ctypes.c_void_p()
+
+    def __del__(self):  # pragma: no cover
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+_F32 = ("qpos", "qvel", "qacc_warmstart", "time", "last_ctrl", "action", "ctrl_in", "latency", "zero_offset", "kp",
+        "kd", "ctrl_clip", "kp_scale", "kd_scale", "torque_limit_scale", "action_bias", "torque_bias", "action_noise",
+        "torque_noise", "friction", "mass_scale", "qacc", "ctrl_out", "xpos", "xquat", "cvel", "dbg_M", "dbg_bias",
+        "dbg_qacc_smooth", "dbg_con_dist")
+_I32 = ("solver_niter", "nefc")
+
+
+def _expected_shapes(m: KinematicModel, N: int, S: int) -> dict:
+    nb, nq, nv, nu, ns = m.nb, m.nq, m.nv, m.nu, m.ns
+    return {
+        "qpos": (N, nq), "qvel": (N, nv), "qacc_warmstart": (N, nv), "time": (N,), "last_ctrl": (N, nu),
+        "action": (N, nu), "ctrl_in": (N, nu), "latency": (N,), "zero_offset": (N, nu), "drop": (N, nu),
+        "kp": (nu,), "kd": (nu,), "ctrl_clip": (nu,), "kp_scale": (N,), "kd_scale": (N,),
+        "torque_limit_scale": (N,), "action_bias": (N, nu), "torque_bias": (N, nu), "action_noise": (S, N, nu),
+        "torque_noise": (S, N, nu), "friction": (N,), "mass_scale": (N, nb), "qacc": (N, nv), "ctrl_out": (N, nu),
+        "xpos": (N, nb * 3), "xquat": (N, nb * 4), "cvel": (N, nb * 6), "solver_niter": (N,), "nefc": (N,),
+        "dbg_M": (N, nv * nv), "dbg_bias": (N, nv), "dbg_qacc_smooth": (N, nv), "dbg_con_dist": (N, ns),
+    }
+
+
+def _make_io(dm: DeviceModel, buffers: Mapping[str, torch.Tensor | None], substeps: int, actuator_period: int,
+             actuator_type: int, action_scale: float) -> _lib_dyn.KsStepIO:
+    """Checks every operand shape on the host against what the kernel's indexing assumes."""
+    m = dm.model
+    qpos = buffers.get("qpos")
+    if qpos is None or qpos.dim() != 2:
+        raise _lib.KsError("qpos (N, nq) is required")
+    N = qpos.shape[0]
+    shapes = _expected_shapes(m, N, max(substeps, 1))
+    io = _lib_dyn.KsStepIO()
+    io.N, io.substeps, io.actuator_period, io.actuator_type = N, substeps, actuator_period, actuator_type
+    io.action_scale = action_scale
+    for name, t in buffers.items():
+        if name not in shapes:
+            raise _lib.KsError(f"unknown step buffer {name!r}")
+        if t is None:
+            continue
+        want = torch.uint8 if name == "drop" else (torch.int32 if name in _I32 else torch.float32)
+        if name == "drop" and t.dtype == torch.bool:
+            t = t.view(torch.uint8)
+        _lib.require_cuda(t, dtype=want)
+        if tuple(t.shape) != shapes[name] and not (t.numel() == 0 and 0 in shapes[name]):
+            raise _lib.KsError(f"{name}: expected shape {shapes[name]}, got {tuple(t.shape)}")
+        if t.numel():
+            setattr(io, name, t.data_ptr())
+    return io
+
+
+def control_step(dm: DeviceModel, buffers: Mapping[str, torch.Tensor | None], *, substeps: int,
+                 actuator_period: int = 1, actuator_type: int = _lib_dyn.KS_ACT_POSITION,
+                 action_scale: float = 1.0) -> None:
+    """One control step of every env, in place on ``qpos, qvel, qacc_warmstart, time, last_ctrl``."""
+    io = _make_io(dm, buffers, substeps, actuator_period, actuator_type, action_scale)
+    _lib.check(dm._lib.ks_step(dm.handle, _lib.current_stream(), ctypes.byref(io)))
+
+
+def forward(dm: DeviceModel, buffers: Mapping[str, torch.Tensor | None]) -> None:
+    """Derived quantities (and the warm start) for the given state, without integrating."""
+    io = _make_io(dm, buffers, 0, 1, _lib_dyn.KS_ACT_TORQUE, 1.0)
+    _lib.check(dm._lib.ks_forward(dm.handle, _lib.current_stream(), ctypes.byref(io)))

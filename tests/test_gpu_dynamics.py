@@ -1,0 +1,233 @@
+"""Parity of the fused HIP control-step kernel against the CPU oracle (through the C ABI).
+
+Tolerances are BASELINE's: qacc and one-step state 1e-4 relative, 10-step trajectories 1e-3
+(fp32 kernel against the float64 oracle; "relative" = max abs error of an env's vector over
+that vector's max magnitude).
+"""
+import numpy as np
+import pytest
+import torch
+
+from dyn_common import oracle_forward, random_states, rel_err
+from ksim_amd import model as km
+from oracle import terms as oterms
+from oracle.dyn import Oracle
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+MODELS = {"chain": km.pendulum_chain_model, "humanoid": km.humanoid_model, "kbot": km.kbot_scale_model}
+ONE_STEP_TOL, TEN_STEP_TOL = 1e-4, 1e-3
+
+
+def t32(a):
+    return torch.tensor(np.asarray(a), dtype=torch.float32, device=DEV).contiguous()
+
+
+def zeros(*shape, dtype=torch.float32):
+    return torch.zeros(*shape, dtype=dtype, device=DEV)
+
+
+@pytest.fixture(scope="module", params=list(MODELS))
+def setup(request):
+    from ksim_amd import physics
+
+    m = MODELS[request.param]()
+    return request.param, m, physics.DeviceModel(m)
+
+
+def test_forward_quantities_match_oracle(setup):
+    from ksim_amd import physics
+
+    name, m, dm = setup
+    N = 48
+    qpos, qvel = random_states(m, N, seed=11)
+    rng = np.random.default_rng(12)
+    ctrl = rng.normal(size=(N, m.nu)) * 5
+    fr = rng.uniform(0.4, 1.2, size=N)
+    ms = rng.uniform(0.9, 1.1, size=(N, m.nb))
+    warm = rng.normal(size=(N, m.nv))
+    want = oracle_forward(m, qpos, qvel, ctrl, fr, ms, warm)
+    buf = dict(qpos=t32(qpos), qvel=t32(qvel), qacc_warmstart=t32(warm), ctrl_in=t32(ctrl), friction=t32(fr),
+               mass_scale=t32(ms), qacc=zeros(N, m.nv), xpos=zeros(N, m.nb * 3), xquat=zeros(N, m.nb * 4),
+               cvel=zeros(N, m.nb * 6), nefc=zeros(N, dtype=torch.int32), solver_niter=zeros(N, dtype=torch.int32),
+               dbg_M=zeros(N, m.nv * m.nv), dbg_bias=zeros(N, m.nv), dbg_qacc_smooth=zeros(N, m.nv),
+               dbg_con_dist=zeros(N, m.ns))
+    q0 = buf["qpos"].clone()
+    physics.forward(dm, buf)
+    g = {k: v.cpu().numpy() for k, v in buf.items()}
+    assert torch.equal(buf["qpos"], q0), "forward must not integrate"
+    for got, ref, tol in [("dbg_M", "M", 1e-5), ("dbg_bias", "qfrc_bias", 1e-5), ("xpos", "xpos", 1e-5),
+                          ("xquat", "xquat", 1e-5), ("cvel", "cvel", 1e-5), ("dbg_qacc_smooth", "qacc_smooth", 1e-4),
+                          ("qacc", "qacc", ONE_STEP_TOL), ("qacc_warmstart", "qacc", ONE_STEP_TOL)]:
+        err = rel_err(g[got], want[ref]).max()
+        assert err <= tol, f"{name}.{ref}: rel err {err:.2e} > {tol}"
+    if m.ns:
+        assert np.abs(g["dbg_con_dist"] - want["con_dist"]).max() < 1e-6
+        assert np.array_equal(g["nefc"], want["nefc"]), "active contact sets differ"  # integer: bit-exact
+        assert (want["nefc"] > 0).sum() >= N // 4
+
+
+@pytest.mark.parametrize("steps,tol", [(1, ONE_STEP_TOL), (10, TEN_STEP_TOL)])
+def test_torque_driven_trajectories(setup, steps, tol):
+    """`steps` physics steps (one substep per call, constant torque) against the oracle."""
+    from ksim_amd import physics
+    from ksim_amd._lib_dyn import KS_ACT_TORQUE
+
+    name, m, dm = setup
+    N = 32
+    qpos, qvel = random_states(m, N, seed=21, vel_scale=0.3)
+    rng = np.random.default_rng(22)
+    ctrl = rng.normal(size=(N, m.nu)) * 3
+    orc = Oracle(m.arrays())
+    wq, wv = [], []
+    for e in range(N):
+        d = orc.data(qpos[e], qvel[e])
+        d.ctrl = ctrl[e]
+        for _ in range(steps):
+            orc.step(d)
+        wq.append(np.array(d.qpos)); wv.append(np.array(d.qvel))
+    buf = dict(qpos=t32(qpos), qvel=t32(qvel), qacc_warmstart=zeros(N, m.nv), time=zeros(N), last_ctrl=t32(ctrl),
+               action=t32(ctrl))
+    for _ in range(steps):
+        physics.control_step(dm, buf, substeps=1, actuator_type=KS_ACT_TORQUE)
+    eq, ev = rel_err(buf["qpos"].cpu().numpy(), wq).max(), rel_err(buf["qvel"].cpu().numpy(), wv).max()
+    assert eq <= tol and ev <= tol, f"{name}: qpos {eq:.2e} qvel {ev:.2e} > {tol}"
+    np.testing.assert_allclose(buf["time"].cpu().numpy(), steps * m.dt, rtol=1e-5)
+
+
+def _oracle_control_steps(m, qpos, qvel, actions, kp, kd, clip, S, latency, friction, mass_scale, period=1):
+    """Python composition of the oracle's pieces: engine.py:287-320 + actuators.py:198-217 + the C step."""
+    orc = Oracle(m.arrays())
+    N = qpos.shape[0]
+    rq, rv = (7, 6) if m.has_free_root else (0, 0)
+    datas = [orc.data(qpos[e], qvel[e], friction=friction[e], mass_scale=mass_scale[e]) for e in range(N)]
+    last = np.zeros((N, m.nu))
+    for action in actions:
+        for e, d in enumerate(datas):
+            torque = np.zeros(m.nu)
+            for s in range(S):
+                c = oterms.latency_blend(float(s), latency[e], last[e], action[e], np.zeros(m.nu, bool))
+                if s % period == 0:
+                    torque = oterms.position_actuator_torque(c, np.array(d.qpos[rq:]), np.array(d.qvel[rv:]), kp, kd, clip)
+                d.ctrl = torque
+                orc.step(d)
+        last = action.copy()
+    return datas
+
+
+@pytest.mark.parametrize("name,S,T,period", [("chain", 1, 10, 1), ("kbot", 4, 2, 1), ("humanoid", 4, 2, 2)])
+def test_position_controlled_steps(name, S, T, period):
+    """Fused control step (latency blend + PD + S substeps) with per-env friction / mass scale."""
+    from ksim_amd import physics
+
+    m = MODELS[name]()
+    dm = physics.DeviceModel(m)
+    N = 24
+    qpos, qvel = random_states(m, N, seed=31, vel_scale=0.2, joint_range=0.3)
+    rng = np.random.default_rng(32)
+    actions = rng.uniform(-0.5, 0.5, size=(T, N, m.nu))
+    kp, kd = rng.uniform(20, 150, m.nu), rng.uniform(1, 5, m.nu)
+    clip = np.where(rng.random(m.nu) < 0.5, 40.0, np.inf)
+    latency = rng.uniform(0.0, 1.5, N)
+    fr, ms = rng.uniform(0.4, 1.2, N), rng.uniform(0.9, 1.1, (N, m.nb))
+    datas = _oracle_control_steps(m, qpos, qvel, actions, kp, kd, clip, S, latency, fr, ms, period)
+    buf = dict(qpos=t32(qpos), qvel=t32(qvel), qacc_warmstart=zeros(N, m.nv), time=zeros(N), last_ctrl=zeros(N, m.nu),
+               latency=t32(latency), kp=t32(kp), kd=t32(kd), ctrl_clip=t32(clip), friction=t32(fr), mass_scale=t32(ms),
+               ctrl_out=zeros(N, m.nu), xpos=zeros(N, m.nb * 3), xquat=zeros(N, m.nb * 4), qacc=zeros(N, m.nv))
+    for k in range(T):
+        buf["action"] = t32(actions[k])
+        physics.control_step(dm, buf, substeps=S, actuator_period=period)
+    tol = ONE_STEP_TOL if S * T == 1 else TEN_STEP_TOL
+    for field, ref in [("qpos", "qpos"), ("qvel", "qvel"), ("ctrl_out", "ctrl"), ("qacc", "qacc")]:
+        want = np.array([np.array(getattr(d, ref)) for d in datas])
+        err = rel_err(buf[field].cpu().numpy(), want).max()
+        assert err <= tol, f"{name}.{field}: {err:.2e} > {tol}"
+    # xpos / xquat are those of the start of the last substep (mjx.step runs kinematics before integrating)
+    want = np.array([np.array(d.xpos).reshape(-1) for d in datas])
+    assert rel_err(buf["xpos"].cpu().numpy(), want).max() <= tol
+    assert torch.equal(buf["last_ctrl"], buf["action"])  # engine.py:355
+
+
+def test_cfg1_chain_200_steps():
+    """BASELINE config 1: 128 envs, 200 steps, targets resampled every step; checked at steps 1, 10, 200."""
+    from ksim_amd import physics
+
+    m = km.pendulum_chain_model()
+    dm = physics.DeviceModel(m)
+    rng = np.random.default_rng(1001)
+    N, T = 128, 200
+    qpos = rng.uniform(-0.5, 0.5, (N, 3))
+    targets = rng.uniform(-1.0, 1.0, (T, N, 3))
+    kp, kd, clip = np.full(3, 20.0), np.full(3, 1.0), np.full(3, np.inf)
+    orc = Oracle(m.arrays())
+    datas = [orc.data(qpos[e]) for e in range(N)]
+    buf = dict(qpos=t32(qpos), qvel=zeros(N, 3), qacc_warmstart=zeros(N, 3), time=zeros(N), last_ctrl=zeros(N, 3),
+               kp=t32(kp), kd=t32(kd), ctrl_clip=t32(clip), qacc=zeros(N, 3))
+    # latency 1 substep back: the reference's blend applies the new target from substep 1 on, so with one substep
+    # per control step each step is driven by the previous target (engine.py:287-288)
+    last = np.zeros((N, 3))
+    for k in range(T):
+        buf["action"] = t32(targets[k])
+        physics.control_step(dm, buf, substeps=1)
+        for e, d in enumerate(datas):
+            d.ctrl = oterms.position_actuator_torque(last[e], np.array(d.qpos), np.array(d.qvel), kp, kd, clip)
+            orc.step(d)
+        last = targets[k]
+        if k + 1 in (1, 10, 200):
+            want_q = np.array([np.array(d.qpos) for d in datas])
+            want_v = np.array([np.array(d.qvel) for d in datas])
+            tol = ONE_STEP_TOL if k == 0 else (TEN_STEP_TOL if k == 9 else 5e-3)
+            eq = rel_err(buf["qpos"].cpu().numpy(), want_q).max()
+            ev = rel_err(buf["qvel"].cpu().numpy(), want_v).max()
+            assert eq <= tol and ev <= tol, f"step {k + 1}: qpos {eq:.2e} qvel {ev:.2e}"
+            if k == 0:
+                want_a = np.array([np.array(d.qacc) for d in datas])
+                assert rel_err(buf["qacc"].cpu().numpy(), want_a).max() <= ONE_STEP_TOL
+
+
+def test_step_is_deterministic_and_env_independent():
+    from ksim_amd import physics
+
+    m = km.kbot_scale_model()
+    dm = physics.DeviceModel(m)
+    N = 64
+    qpos, qvel = random_states(m, N, seed=41)
+    rng = np.random.default_rng(42)
+    act = rng.uniform(-0.3, 0.3, (N, m.nu))
+    kp, kd, clip = np.full(m.nu, 60.0), np.full(m.nu, 2.0), np.full(m.nu, 80.0)
+
+    def run(idx):
+        buf = dict(qpos=t32(qpos[idx]), qvel=t32(qvel[idx]), qacc_warmstart=zeros(len(idx), m.nv),
+                   last_ctrl=zeros(len(idx), m.nu), action=t32(act[idx]), kp=t32(kp), kd=t32(kd), ctrl_clip=t32(clip))
+        physics.control_step(dm, buf, substeps=4)
+        return buf["qpos"].clone(), buf["qvel"].clone()
+
+    a = run(np.arange(N))
+    b = run(np.arange(N))
+    assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
+    perm = np.random.default_rng(0).permutation(N)[:17]  # ragged subset in another order: same per-env bits
+    c = run(perm)
+    assert torch.equal(c[0], a[0][torch.from_numpy(perm).to(DEV)])
+
+
+def test_errors_are_reported():
+    from ksim_amd import _lib, physics
+
+    m = km.kbot_scale_model()
+    dm = physics.DeviceModel(m)
+    N = 4
+    good = dict(qpos=zeros(N, m.nq), qvel=zeros(N, m.nv), qacc_warmstart=zeros(N, m.nv), last_ctrl=zeros(N, m.nu),
+                action=zeros(N, m.nu), kp=zeros(m.nu), kd=zeros(m.nu), ctrl_clip=zeros(m.nu))
+    with pytest.raises(_lib.KsError):
+        physics.control_step(dm, dict(good, qvel=zeros(N, m.nv + 1)), substeps=4)
+    with pytest.raises(_lib.KsError):
+        physics.control_step(dm, dict(good, kp=None), substeps=4)
+    with pytest.raises(_lib.KsError):
+        physics.control_step(dm, good, substeps=0)
+    with pytest.raises(_lib.KsError):
+        physics.control_step(dm, dict(good, qpos=torch.zeros(N, m.nq)), substeps=4)
+    physics.control_step(dm, dict(qpos=zeros(0, m.nq), qvel=zeros(0, m.nv), last_ctrl=zeros(0, m.nu),
+                                  action=zeros(0, m.nu), kp=zeros(m.nu), kd=zeros(m.nu), ctrl_clip=zeros(m.nu)),
+                         substeps=4)  # empty batch is a no-op
+    with pytest.raises(ValueError):
+        km.ModelBuilder().add_body(0, (0, 0, 0), joint=None, mass=1.0, inertia=(1, 1, 1))
