@@ -176,12 +176,16 @@ typedef struct KsStepIO {
   const float* torque_noise; /* (substeps, N, nu) */
   const float* friction;    /* (N) per-env contact friction (FloorFrictionRandomizer, randomization.py:74-104) */
   const float* mass_scale;  /* (N, nb) per-env body mass factor (randomization.py:207-222) */
+  const uint8_t* env_mask;  /* (N) nullable: envs with 0 are skipped entirely (reset-under-cond, rl.py:1072-1080) */
   /* outputs, each nullable */
   float* qacc;              /* (N, nv) of the last substep */
   float* ctrl_out;          /* (N, nu) torques applied in the last substep = data.ctrl */
   float* xpos;              /* (N, nb*3) body positions at the start of the last substep */
   float* xquat;             /* (N, nb*4) */
   float* cvel;              /* (N, nb*6) com-based body velocities [angular; linear] */
+  float* traj_ctrl;         /* (N, nu)   second copies of ctrl_out / xpos / xquat for the transition record */
+  float* traj_xpos;         /* (N, nb*3) (Trajectory.ctrl/xpos/xquat, ksim/task/rl.py:1054-1070) */
+  float* traj_xquat;        /* (N, nb*4) */
   int32_t* solver_niter;    /* (N) Newton iterations of the last substep */
   int32_t* nefc;            /* (N) active constraint rows of the last substep */
   /* intermediate quantities for parity tests, each nullable */
@@ -193,6 +197,170 @@ typedef struct KsStepIO {
 
 int ks_step(const KsModel* model, ks_stream_t stream, const KsStepIO* io /*host*/);
 int ks_forward(const KsModel* model, ks_stream_t stream, const KsStepIO* io /*host*/);
+
+/* ------------------------------------------------------------------ per-env terms
+ * One spec holds the compiled tables of the task's observations, terminations and
+ * resets; ks_terms_create copies it to the device (allocates), after which
+ * ks_observe / ks_terminate_reset / ks_sample_action allocate nothing.
+ *
+ * Observations (replaces get_observation + Observation.observe/add_noise,
+ * ksim/task/rl.py:153-186, ksim/observation.py:89-145,184-257,300-352,705-713): every
+ * element k of the concatenated observation vector is described by one KsObsElem.
+ */
+enum { /* KsObsElem.src: which per-env array the element reads, all (N, dim) f32 */
+  KS_SRC_QPOS = 0, KS_SRC_QVEL = 1, KS_SRC_QACC = 2, KS_SRC_CTRL = 3, KS_SRC_LAST_ACTION = 4,
+  KS_SRC_COMMAND = 5, KS_SRC_TIME = 6, KS_SRC_XPOS = 7, KS_SRC_XQUAT = 8, KS_SRC_CVEL = 9,
+  KS_SRC_CONST = 10, KS_SRC_COUNT = 11
+};
+enum { /* KsObsElem.kind */
+  KS_OBS_COPY = 0,      /* src[index]                                  (observation.py:185-195,254-257,300-303,343-352) */
+  KS_OBS_JOINT_POS = 1, /* qpos[index] - zero_offset[index - 7]        (observation.py:220-225) */
+  KS_OBS_ROT_INV = 2    /* component `comp` of q^-1 v q, q = qpos[3:7], v = src[index..index+2] or (c0,c1,c2)
+                           (in_robot_frame velocities, observation.py:198-217; gravity in the body frame) */
+};
+enum { KS_NOISE_NONE = 0, KS_NOISE_ADD_GAUSSIAN = 1, KS_NOISE_ADD_UNIFORM = 2, KS_NOISE_MUL_GAUSSIAN = 3,
+       KS_NOISE_MUL_UNIFORM = 4 }; /* ksim/noise.py:184-213 */
+typedef struct KsObsElem {
+  int32_t kind, src, index, comp;
+  float c0, c1, c2;
+  int32_t noise_kind;
+  float noise_mean, noise_scale; /* std or mag, multiplied by the curriculum level (noise.py:86,102) */
+} KsObsElem;
+
+/* Terminations (replaces get_terminations + terms, rl.py:288-299, ksim/terminations.py:60-192). */
+enum { KS_TERM_MIN_HEIGHT = 0, KS_TERM_BAD_Z = 1, KS_TERM_NOT_UPRIGHT = 2, KS_TERM_BAD_VELOCITY = 3,
+       KS_TERM_FAR_FROM_ORIGIN = 4, KS_TERM_EPISODE_LENGTH = 5 };
+typedef struct KsTermDesc {
+  int32_t kind;
+  int32_t value; /* what a firing term reports: -1 or +1 */
+  float p0, p1, p2, p3; /* min_height | min_z,max_z,final_min_z,final_max_z | max_radians | max_vel | max_dist | max_sec,disable_level(<0: never) */
+} KsTermDesc;
+
+/* Resets (replaces the Reset list applied in MjxEngine.reset, engine.py:207-220, ksim/resets.py:122-189,
+ * 308-334): qpos[i] <- clip(base[i] + u*mag[i]*(level if by_level[i]), lo[i], hi[i]) with u ~ U(-1,1);
+ * optional heading: quat <- quat * yaw(U(-pi,pi)); qvel, time and last_ctrl <- 0. */
+#define KS_MAX_OBS 512
+#define KS_MAX_TERMS 16
+typedef struct KsTermsDesc {
+  int32_t nq, nv, nu, nb;
+  int32_t obs_dim, n_terms, command_dim, random_heading;
+  KsObsElem obs[KS_MAX_OBS];
+  KsTermDesc terms[KS_MAX_TERMS];
+  float reset_base[KS_MAX_QPOS], reset_mag[KS_MAX_QPOS], reset_lo[KS_MAX_QPOS], reset_hi[KS_MAX_QPOS];
+  int32_t reset_by_level[KS_MAX_QPOS];
+} KsTermsDesc;
+typedef struct KsTerms KsTerms;
+int ks_terms_create(const KsTermsDesc* desc /*host*/, KsTerms** out);
+int ks_terms_destroy(KsTerms* terms);
+
+/* Random draws: every entry point that needs randomness takes either explicit pre-sampled
+ * buffers (so both sides of a parity test see identical draws) or, when they are NULL, a
+ * counter-based Philox-4x32-10 stream keyed by (seed, env, step, purpose). */
+typedef struct KsRng {
+  uint64_t seed;
+  uint64_t step;
+} KsRng;
+
+typedef struct KsObserveIO {
+  int64_t N;
+  float level;               /* curriculum level */
+  const float* src[KS_SRC_COUNT]; /* indexed by KS_SRC_*; an unused source may be NULL */
+  const float* zero_offset;  /* (N, nu) nullable */
+  const float* bias;         /* (N, obs_dim) additive per-episode bias value, nullable */
+  const float* noise_normal; /* (N, obs_dim) standard normal draws, nullable -> Philox */
+  const float* noise_uniform;/* (N, obs_dim) U[0,1) draws, nullable -> Philox */
+  KsRng rng;
+  float* obs;                /* (N, obs_dim) clean, nullable */
+  float* noisy_obs;          /* (N, obs_dim) noisy copy, nullable (rl.py:181-184) */
+} KsObserveIO;
+int ks_observe(const KsTerms* terms, ks_stream_t stream, const KsObserveIO* io /*host*/);
+
+/* Terminations, trajectory record and reset predication for the post-step state
+ * (replaces RLTask._get_step_env_state, rl.py:1023-1136, for the physics part):
+ * writes done/success/components and the transition copies, then overwrites the state of
+ * finished envs with a fresh episode.  reset_mask marks them for a following ks_forward. */
+typedef struct KsTerminateIO {
+  int64_t N;
+  float level;
+  float* qpos; float* qvel; float* qacc_warmstart; float* time; float* last_ctrl; /* state, in/out */
+  int8_t* components;        /* (n_terms, N) int8 in {-1,0,1}, nullable */
+  uint8_t* done; uint8_t* success; /* (N) */
+  float* traj_qpos; float* traj_qvel; float* traj_time; /* transition copies of the pre-reset state, nullable */
+  uint8_t* reset_mask;       /* (N) = done, nullable */
+  int32_t* episode_length;   /* (N) control steps in the current episode, in/out, nullable */
+  const float* reset_uniform; /* (N, nq + 1) U(-1,1) draws (last one: heading), nullable -> Philox */
+  KsRng rng;
+  int32_t apply_reset;       /* 0: report terminations only; 1: reset finished envs; 2: reset every env (initial reset) */
+} KsTerminateIO;
+int ks_terminate_reset(const KsTerms* terms, ks_stream_t stream, const KsTerminateIO* io /*host*/);
+
+/* Action post-processing (replaces the sampling tail of RLTask._sample_action, rl.py:998-1001):
+ * action = mean + std * noise, NaN -> 0, clip to +-clip_max.  log_std (nu) nullable = deterministic. */
+int ks_sample_action(ks_stream_t stream, int64_t N, int32_t nu, const float* mean, const float* log_std,
+                     const float* noise_normal /*(N,nu) nullable -> Philox*/, KsRng rng, float clip_max,
+                     float* action);
+
+/* ------------------------------------------------------------------ policy / critic / discriminator MLP
+ * The dense contraction of the path: the network a task's sample_action calls
+ * (ksim/task/rl.py:892-926,986-996; plain MLP stacks as in examples/walking.py:40-208's
+ * heads) and the AMP discriminator forward (ksim/task/amp.py:327-358).
+ * y = W_L act(... act(W_1 x + b_1) ...) + b_L, weights (out, in) row-major like the
+ * reference's linear layers.  KS_MLP_BF16 rounds weights and activations to bf16 and
+ * accumulates in fp32 on the matrix cores; KS_MLP_F32 keeps fp32 throughout.
+ * ks_mlp_create uploads (allocates); ks_mlp_forward allocates nothing: the caller
+ * provides ks_mlp_workspace_bytes(mlp, M) bytes of device scratch.
+ */
+#define KS_MAX_LAYERS 8
+enum { KS_ACT_NONE = 0, KS_ACT_ELU = 1, KS_ACT_RELU = 2, KS_ACT_TANH = 3 };
+enum { KS_MLP_F32 = 0, KS_MLP_BF16 = 1 };
+typedef struct KsMlpDesc {
+  int32_t n_layers;
+  int32_t dims[KS_MAX_LAYERS + 1];  /* in, hidden..., out */
+  int32_t activation;               /* applied after every layer but the last */
+  int32_t dtype;
+  const float* weights[KS_MAX_LAYERS]; /* host, (dims[l+1], dims[l]) */
+  const float* biases[KS_MAX_LAYERS];  /* host, (dims[l+1]) */
+} KsMlpDesc;
+typedef struct KsMlp KsMlp;
+int ks_mlp_create(const KsMlpDesc* desc /*host*/, KsMlp** out);
+int ks_mlp_destroy(KsMlp* mlp);
+int64_t ks_mlp_workspace_bytes(const KsMlp* mlp, int64_t M);
+int ks_mlp_forward(const KsMlp* mlp, ks_stream_t stream, int64_t M, const float* x /*(M, in)*/,
+                   float* y /*(M, out)*/, void* workspace);
+
+/* ------------------------------------------------------------------ rewards over a rollout
+ * Replaces get_rewards + the stateless Reward.get_reward terms the configs name
+ * (ksim/task/rl.py:189-245; ksim/rewards.py:166-188 StayAlive, 374-401 BaseHeight / BaseHeightRange,
+ * 404-460 ActionVelocity / Acceleration / Jerk penalties, 746-777 Upright).
+ * Trajectory arrays are time-major (T, N, dim); outputs are (T, N).  Each descriptor yields one
+ * component scaled by `scale` (sign already folded for *Penalty classes, rl.py:219-221); the total is
+ * their sum in order, optionally clipped (rl.py:235-239).
+ */
+enum { KS_REW_STAY_ALIVE = 0, KS_REW_BASE_HEIGHT = 1, KS_REW_BASE_HEIGHT_RANGE = 2, KS_REW_ACTION_VEL = 3,
+       KS_REW_ACTION_ACC = 4, KS_REW_ACTION_JERK = 5, KS_REW_UPRIGHT_ANGVEL = 6, KS_REW_UPRIGHT_LINVEL = 7,
+       KS_REW_UPRIGHT_POSE = 8 };
+enum { KS_NORM_L1 = 0, KS_NORM_L2 = 1 }; /* xax.get_norm: l1 = |x|, l2 = x^2 (reference tests/test_rewards.py:95-98) */
+typedef struct KsRewardDesc {
+  int32_t kind;
+  int32_t norm;   /* action-difference penalties */
+  float scale;
+  float p0, p1, p2; /* balance,success_reward,has_success_reward | target,kernel_scale | lo,hi,dropoff | scale,sq,abs */
+} KsRewardDesc;
+typedef struct KsRewardIO {
+  int64_t T, N;
+  int32_t nq, nv, nu, n_rewards;
+  KsRewardDesc rewards[KS_MAX_REWARD_TERMS];
+  int32_t use_clip_min, use_clip_max;
+  float clip_min, clip_max;
+  const float* qpos;   /* (T, N, nq) */
+  const float* qvel;   /* (T, N, nv) */
+  const float* action; /* (T, N, nu) */
+  const uint8_t* done; /* (T, N) */
+  const uint8_t* success; /* (T, N) */
+  float* components;   /* (n_rewards, T, N) nullable */
+  float* total;        /* (T, N) */
+} KsRewardIO;
+int ks_rewards(ks_stream_t stream, const KsRewardIO* io /*host*/);
 
 #ifdef __cplusplus
 }

@@ -63,9 +63,10 @@ def load() -> ctypes.CDLL:
 
 
 def _bind_optional(lib) -> None:
-    from . import _lib_dyn  # noqa: PLC0415
+    from . import _lib_dyn, _lib_terms  # noqa: PLC0415
 
     _lib_dyn.bind(lib)
+    _lib_terms.bind(lib)
 
 
 def check(rc: int) -> None:

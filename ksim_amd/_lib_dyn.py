@@ -36,7 +36,8 @@ STEP_IO_POINTERS = (
     "qpos", "qvel", "qacc_warmstart", "time", "last_ctrl",
     "action", "ctrl_in", "latency", "zero_offset", "drop", "kp", "kd", "ctrl_clip", "kp_scale", "kd_scale",
     "torque_limit_scale", "action_bias", "torque_bias", "action_noise", "torque_noise", "friction", "mass_scale",
-    "qacc", "ctrl_out", "xpos", "xquat", "cvel", "solver_niter", "nefc",
+    "env_mask",
+    "qacc", "ctrl_out", "xpos", "xquat", "cvel", "traj_ctrl", "traj_xpos", "traj_xquat", "solver_niter", "nefc",
     "dbg_M", "dbg_bias", "dbg_qacc_smooth", "dbg_con_dist",
 )
 

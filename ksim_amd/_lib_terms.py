@@ -1,0 +1,96 @@
+"""ctypes signatures of the per-env-term and MLP entry points (include/ksim_hip.h)."""
+from __future__ import annotations
+
+import ctypes
+from ctypes import POINTER, c_float, c_int8, c_int32, c_int64, c_uint8, c_uint64, c_void_p
+
+KS_MAX_OBS, KS_MAX_TERMS, KS_MAX_QPOS, KS_MAX_LAYERS = 512, 16, 40, 8
+(SRC_QPOS, SRC_QVEL, SRC_QACC, SRC_CTRL, SRC_LAST_ACTION, SRC_COMMAND, SRC_TIME, SRC_XPOS, SRC_XQUAT, SRC_CVEL,
+ SRC_CONST, SRC_COUNT) = range(12)
+OBS_COPY, OBS_JOINT_POS, OBS_ROT_INV = 0, 1, 2
+NOISE_NONE, NOISE_ADD_GAUSSIAN, NOISE_ADD_UNIFORM, NOISE_MUL_GAUSSIAN, NOISE_MUL_UNIFORM = range(5)
+(TERM_MIN_HEIGHT, TERM_BAD_Z, TERM_NOT_UPRIGHT, TERM_BAD_VELOCITY, TERM_FAR_FROM_ORIGIN,
+ TERM_EPISODE_LENGTH) = range(6)
+ACT_NONE, ACT_ELU, ACT_RELU, ACT_TANH = range(4)
+MLP_F32, MLP_BF16 = 0, 1
+
+
+class KsObsElem(ctypes.Structure):
+    _fields_ = [("kind", c_int32), ("src", c_int32), ("index", c_int32), ("comp", c_int32), ("c0", c_float),
+                ("c1", c_float), ("c2", c_float), ("noise_kind", c_int32), ("noise_mean", c_float),
+                ("noise_scale", c_float)]
+
+
+class KsTermDesc(ctypes.Structure):
+    _fields_ = [("kind", c_int32), ("value", c_int32), ("p0", c_float), ("p1", c_float), ("p2", c_float),
+                ("p3", c_float)]
+
+
+class KsTermsDesc(ctypes.Structure):
+    _fields_ = [("nq", c_int32), ("nv", c_int32), ("nu", c_int32), ("nb", c_int32), ("obs_dim", c_int32),
+                ("n_terms", c_int32), ("command_dim", c_int32), ("random_heading", c_int32),
+                ("obs", KsObsElem * KS_MAX_OBS), ("terms", KsTermDesc * KS_MAX_TERMS),
+                ("reset_base", c_float * KS_MAX_QPOS), ("reset_mag", c_float * KS_MAX_QPOS),
+                ("reset_lo", c_float * KS_MAX_QPOS), ("reset_hi", c_float * KS_MAX_QPOS),
+                ("reset_by_level", c_int32 * KS_MAX_QPOS)]
+
+
+class KsRng(ctypes.Structure):
+    _fields_ = [("seed", c_uint64), ("step", c_uint64)]
+
+
+class KsObserveIO(ctypes.Structure):
+    _fields_ = [("N", c_int64), ("level", c_float), ("src", c_void_p * SRC_COUNT), ("zero_offset", c_void_p),
+                ("bias", c_void_p), ("noise_normal", c_void_p), ("noise_uniform", c_void_p), ("rng", KsRng),
+                ("obs", c_void_p), ("noisy_obs", c_void_p)]
+
+
+class KsTerminateIO(ctypes.Structure):
+    _fields_ = [("N", c_int64), ("level", c_float), ("qpos", c_void_p), ("qvel", c_void_p),
+                ("qacc_warmstart", c_void_p), ("time", c_void_p), ("last_ctrl", c_void_p), ("components", c_void_p),
+                ("done", c_void_p), ("success", c_void_p), ("traj_qpos", c_void_p), ("traj_qvel", c_void_p),
+                ("traj_time", c_void_p), ("reset_mask", c_void_p), ("episode_length", c_void_p),
+                ("reset_uniform", c_void_p), ("rng", KsRng), ("apply_reset", c_int32)]
+
+
+class KsMlpDesc(ctypes.Structure):
+    _fields_ = [("n_layers", c_int32), ("dims", c_int32 * (KS_MAX_LAYERS + 1)), ("activation", c_int32),
+                ("dtype", c_int32), ("weights", c_void_p * KS_MAX_LAYERS), ("biases", c_void_p * KS_MAX_LAYERS)]
+
+
+(REW_STAY_ALIVE, REW_BASE_HEIGHT, REW_BASE_HEIGHT_RANGE, REW_ACTION_VEL, REW_ACTION_ACC, REW_ACTION_JERK,
+ REW_UPRIGHT_ANGVEL, REW_UPRIGHT_LINVEL, REW_UPRIGHT_POSE) = range(9)
+NORM_L1, NORM_L2 = 0, 1
+KS_MAX_REWARD_TERMS = 32
+
+
+class KsRewardDesc(ctypes.Structure):
+    _fields_ = [("kind", c_int32), ("norm", c_int32), ("scale", c_float), ("p0", c_float), ("p1", c_float),
+                ("p2", c_float)]
+
+
+class KsRewardIO(ctypes.Structure):
+    _fields_ = [("T", c_int64), ("N", c_int64), ("nq", c_int32), ("nv", c_int32), ("nu", c_int32),
+                ("n_rewards", c_int32), ("rewards", KsRewardDesc * KS_MAX_REWARD_TERMS), ("use_clip_min", c_int32),
+                ("use_clip_max", c_int32), ("clip_min", c_float), ("clip_max", c_float), ("qpos", c_void_p),
+                ("qvel", c_void_p), ("action", c_void_p), ("done", c_void_p), ("success", c_void_p),
+                ("components", c_void_p), ("total", c_void_p)]
+
+
+def bind(lib) -> None:
+    lib.ks_rewards.argtypes = [c_void_p, POINTER(KsRewardIO)]
+    lib.ks_rewards.restype = c_int32
+    lib.ks_terms_create.argtypes = [POINTER(KsTermsDesc), POINTER(c_void_p)]
+    lib.ks_terms_destroy.argtypes = [c_void_p]
+    lib.ks_observe.argtypes = [c_void_p, c_void_p, POINTER(KsObserveIO)]
+    lib.ks_terminate_reset.argtypes = [c_void_p, c_void_p, POINTER(KsTerminateIO)]
+    lib.ks_sample_action.argtypes = [c_void_p, c_int64, c_int32, c_void_p, c_void_p, c_void_p, KsRng, c_float,
+                                     c_void_p]
+    lib.ks_mlp_create.argtypes = [POINTER(KsMlpDesc), POINTER(c_void_p)]
+    lib.ks_mlp_destroy.argtypes = [c_void_p]
+    lib.ks_mlp_workspace_bytes.argtypes = [c_void_p, c_int64]
+    lib.ks_mlp_workspace_bytes.restype = c_int64
+    lib.ks_mlp_forward.argtypes = [c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_void_p]
+    for name in ("ks_terms_create", "ks_terms_destroy", "ks_observe", "ks_terminate_reset", "ks_sample_action",
+                 "ks_mlp_create", "ks_mlp_destroy", "ks_mlp_forward"):
+        getattr(lib, name).restype = c_int32

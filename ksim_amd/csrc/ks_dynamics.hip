@@ -301,6 +301,7 @@ __global__ __launch_bounds__(64) void step_kernel(StepArgs a) {
   const DevModel& m = *a.model;
   const int lane = threadIdx.x;
   const int64_t env = blockIdx.x;
+  if (a.env_mask && !a.env_mask[env]) return;  // wave-uniform
   const int nb = m.nb, nq = m.nq, nv = m.nv, nu = m.nu, ns = m.ns, nvs = m.nvs;
   const Lds l = carve(lds_raw, m);
   const int rq = (nb > 1 && m.body_jtype[1] == kJntFree) ? 7 : 0;
@@ -619,6 +620,9 @@ __global__ __launch_bounds__(64) void step_kernel(StepArgs a) {
   if (a.xpos) for (int i = lane; i < nb * 3; i += 64) a.xpos[env * nb * 3 + i] = l.xpos[i];
   if (a.xquat) for (int i = lane; i < nb * 4; i += 64) a.xquat[env * nb * 4 + i] = l.xquat[i];
   if (a.cvel) for (int i = lane; i < nb * 6; i += 64) a.cvel[env * nb * 6 + i] = l.cvel[i];
+  if (a.traj_ctrl) for (int i = lane; i < nu; i += 64) a.traj_ctrl[env * nu + i] = l.tau[i];
+  if (a.traj_xpos) for (int i = lane; i < nb * 3; i += 64) a.traj_xpos[env * nb * 3 + i] = l.xpos[i];
+  if (a.traj_xquat) for (int i = lane; i < nb * 4; i += 64) a.traj_xquat[env * nb * 4 + i] = l.xquat[i];
   if (a.solver_niter && lane == 0) a.solver_niter[env] = niter_out;
   if (a.nefc && lane == 0) a.nefc[env] = nefc_out;
 }
@@ -756,8 +760,9 @@ static int launch_step(const KsModel* km, ks_stream_t stream, const KsStepIO* io
   a.N = io->N;
   a.forward_only = forward_only ? 1 : 0;
   a.qpos = io->qpos; a.qvel = io->qvel; a.qacc_warmstart = io->qacc_warmstart; a.time = io->time;
-  a.friction = io->friction; a.mass_scale = io->mass_scale;
+  a.friction = io->friction; a.mass_scale = io->mass_scale; a.env_mask = io->env_mask;
   a.qacc = io->qacc; a.ctrl_out = io->ctrl_out; a.xpos = io->xpos; a.xquat = io->xquat; a.cvel = io->cvel;
+  a.traj_ctrl = io->traj_ctrl; a.traj_xpos = io->traj_xpos; a.traj_xquat = io->traj_xquat;
   a.solver_niter = io->solver_niter; a.nefc = io->nefc;
   a.dbg_M = io->dbg_M; a.dbg_bias = io->dbg_bias; a.dbg_qacc_smooth = io->dbg_qacc_smooth;
   a.dbg_con_dist = io->dbg_con_dist;

@@ -17,7 +17,8 @@ struct StepArgs {
   const float *kp, *kd, *ctrl_clip, *kp_scale, *kd_scale, *torque_limit_scale;
   const float *action_bias, *torque_bias, *action_noise, *torque_noise;
   const float *friction, *mass_scale;
-  float *qacc, *ctrl_out, *xpos, *xquat, *cvel;
+  const uint8_t* env_mask;
+  float *qacc, *ctrl_out, *xpos, *xquat, *cvel, *traj_ctrl, *traj_xpos, *traj_xquat;
   int32_t *solver_niter, *nefc;
   float *dbg_M, *dbg_bias, *dbg_qacc_smooth, *dbg_con_dist;
 };

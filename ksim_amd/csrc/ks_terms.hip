@@ -1,0 +1,408 @@
+// Fused per-env terms: observation assembly + noise, terminations + trajectory record + reset
+// predication, and action sampling.  Streaming kernels over (N, dim) env-major rows.
+#include "ks_common.h"
+#include "ks_philox.h"
+
+#include <cstring>
+
+namespace ks {
+
+struct DevTerms {
+  KsTermsDesc d;
+};
+
+__device__ inline void rot_inv(const float* q4, float vx, float vy, float vz, float* out) {
+  // q^-1 v q for the (normalised) wxyz quaternion q
+  float w = q4[0], x = q4[1], y = q4[2], z = q4[3];
+  const float n = sqrtf(w * w + x * x + y * y + z * z);
+  const float inv = n > 0.f ? 1.0f / n : 0.f;
+  w *= inv; x = -x * inv; y = -y * inv; z = -z * inv;  // conjugate
+  // t = 2 * (qv x v); v' = v + w t + qv x t
+  const float tx = 2.f * (y * vz - z * vy), ty = 2.f * (z * vx - x * vz), tz = 2.f * (x * vy - y * vx);
+  out[0] = vx + w * tx + (y * tz - z * ty);
+  out[1] = vy + w * ty + (z * tx - x * tz);
+  out[2] = vz + w * tz + (x * ty - y * tx);
+}
+
+struct ObserveArgs {
+  const DevTerms* t;
+  int64_t N;
+  float level;
+  const float* src[KS_SRC_COUNT];
+  int src_dim[KS_SRC_COUNT];
+  const float *zero_offset, *bias, *noise_normal, *noise_uniform;
+  KsRng rng;
+  float *obs, *noisy;
+  int obs_dim, nq, nu;
+};
+
+__global__ __launch_bounds__(256) void observe_kernel(ObserveArgs a) {
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= a.N * a.obs_dim) return;
+  const int64_t e = idx / a.obs_dim;
+  const int k = (int)(idx - e * a.obs_dim);
+  const KsObsElem el = a.t->d.obs[k];
+  float v;
+  if (el.kind == KS_OBS_COPY) {
+    v = (el.src == KS_SRC_CONST) ? el.c0 : a.src[el.src][e * a.src_dim[el.src] + el.index];
+  } else if (el.kind == KS_OBS_JOINT_POS) {
+    v = a.src[KS_SRC_QPOS][e * a.nq + el.index] - (a.zero_offset ? a.zero_offset[e * a.nu + (el.index - 7)] : 0.f);
+  } else {
+    float vec[3] = {el.c0, el.c1, el.c2}, out[3];
+    if (el.src != KS_SRC_CONST) {
+      const float* p = a.src[el.src] + e * a.src_dim[el.src] + el.index;
+      vec[0] = p[0]; vec[1] = p[1]; vec[2] = p[2];
+    }
+    rot_inv(a.src[KS_SRC_QPOS] + e * a.nq + 3, vec[0], vec[1], vec[2], out);
+    v = out[el.comp];
+  }
+  if (a.obs) a.obs[idx] = v;
+  if (a.noisy) {
+    float nv = v;
+    if (el.noise_kind != KS_NOISE_NONE) {
+      float n01, u01v;
+      if (a.noise_normal && a.noise_uniform) {
+        n01 = a.noise_normal[idx];
+        u01v = a.noise_uniform[idx];
+      } else {
+        const Philox4 r = draw(a.rng.seed, a.rng.step, kRngObsNoise, (uint64_t)e, (uint32_t)k);
+        n01 = normal_from(r.x, r.y);
+        u01v = u01(r.z);
+      }
+      const float sc = el.noise_scale * a.level;
+      const bool gauss = el.noise_kind == KS_NOISE_ADD_GAUSSIAN || el.noise_kind == KS_NOISE_MUL_GAUSSIAN;
+      const float rv = gauss ? n01 * sc + el.noise_mean : (el.noise_mean - sc) + 2.f * sc * u01v;
+      nv = (el.noise_kind == KS_NOISE_ADD_GAUSSIAN || el.noise_kind == KS_NOISE_ADD_UNIFORM) ? v + rv : v * rv;
+    }
+    if (a.bias) nv += a.bias[idx];
+    a.noisy[idx] = nv;
+  }
+}
+
+struct TerminateArgs {
+  const DevTerms* t;
+  int64_t N;
+  float level;
+  float *qpos, *qvel, *warm, *time, *last_ctrl;
+  int8_t* components;
+  uint8_t *done, *success;
+  float *traj_qpos, *traj_qvel, *traj_time;
+  uint8_t* reset_mask;
+  int32_t* episode_length;
+  const float* reset_uniform;
+  KsRng rng;
+  int apply_reset, nq, nv, nu, n_terms, random_heading;
+};
+
+// One lane per env.  Termination comparisons are strict and done in fp32 on the stored state, so
+// the integer outputs are reproducible bit for bit.
+__global__ __launch_bounds__(256) void terminate_kernel(TerminateArgs a) {
+  const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= a.N) return;
+  const KsTermsDesc& d = a.t->d;
+  float* q = a.qpos + e * a.nq;
+  float* v = a.qvel + e * a.nv;
+  const float tm = a.time ? a.time[e] : 0.f;
+  bool done = false, succ = true;
+  for (int j = 0; j < a.n_terms; ++j) {
+    const KsTermDesc td = d.terms[j];
+    bool fire = false;
+    switch (td.kind) {
+      case KS_TERM_MIN_HEIGHT: fire = q[2] < td.p0; break;
+      case KS_TERM_BAD_Z: {
+        const float lo = (td.p2 - td.p0) * a.level + td.p0, hi = (td.p3 - td.p1) * a.level + td.p1;
+        fire = (q[2] < lo) || (q[2] > hi);
+      } break;
+      case KS_TERM_NOT_UPRIGHT: {
+        float out[3];
+        rot_inv(q + 3, 0.f, 0.f, 1.f, out);
+        fire = acosf(fminf(fmaxf(out[2], -1.f), 1.f)) > td.p0;
+      } break;
+      case KS_TERM_BAD_VELOCITY: fire = sqrtf(v[0] * v[0] + v[1] * v[1] + v[2] * v[2]) > td.p0; break;
+      case KS_TERM_FAR_FROM_ORIGIN: fire = sqrtf(q[0] * q[0] + q[1] * q[1] + q[2] * q[2]) > td.p0; break;
+      case KS_TERM_EPISODE_LENGTH: fire = (tm > td.p0) && !(td.p1 >= 0.f && a.level < td.p1); break;
+      default: break;
+    }
+    const int8_t val = fire ? (int8_t)td.value : (int8_t)0;
+    if (a.components) a.components[(int64_t)j * a.N + e] = val;
+    done |= val != 0;
+    succ &= val != -1;
+  }
+  succ = succ && done;
+  if (a.done) a.done[e] = done ? 1 : 0;
+  if (a.success) a.success[e] = succ ? 1 : 0;
+  if (a.traj_qpos) for (int i = 0; i < a.nq; ++i) a.traj_qpos[e * a.nq + i] = q[i];
+  if (a.traj_qvel) for (int i = 0; i < a.nv; ++i) a.traj_qvel[e * a.nv + i] = v[i];
+  if (a.traj_time) a.traj_time[e] = tm;
+  const bool do_reset = a.apply_reset == 2 || (done && a.apply_reset == 1);
+  if (a.reset_mask) a.reset_mask[e] = do_reset ? 1 : 0;
+  if (a.episode_length) a.episode_length[e] = do_reset ? 0 : a.episode_length[e] + 1;
+  if (!do_reset) return;
+  // ---- fresh episode (engine.py:207-246): qpos from the reset table, everything else zero
+  for (int i = 0; i < a.nq; ++i) {
+    float u;
+    if (a.reset_uniform) u = a.reset_uniform[e * (a.nq + 1) + i];
+    else u = 2.f * u01(draw(a.rng.seed, a.rng.step, kRngReset, (uint64_t)e, (uint32_t)i).x) - 1.f;
+    const float mag = d.reset_mag[i] * (d.reset_by_level[i] ? a.level : 1.f);
+    float x = d.reset_base[i] + u * mag;
+    x = fminf(fmaxf(x, d.reset_lo[i]), d.reset_hi[i]);
+    q[i] = x;
+  }
+  if (a.random_heading && a.nq >= 7) {
+    float u;
+    if (a.reset_uniform) u = a.reset_uniform[e * (a.nq + 1) + a.nq];
+    else u = 2.f * u01(draw(a.rng.seed, a.rng.step, kRngReset, (uint64_t)e, (uint32_t)a.nq).x) - 1.f;
+    const float h = 0.5f * 3.14159265358979323846f * u;  // yaw/2, yaw ~ U(-pi, pi)
+    const float cw = cosf(h), sz = sinf(h);
+    const float w = q[3], x = q[4], y = q[5], z = q[6];
+    q[3] = w * cw - z * sz; q[4] = x * cw + y * sz; q[5] = y * cw - x * sz; q[6] = z * cw + w * sz;
+  }
+  for (int i = 0; i < a.nv; ++i) v[i] = 0.f;
+  if (a.warm) for (int i = 0; i < a.nv; ++i) a.warm[e * a.nv + i] = 0.f;
+  if (a.time) a.time[e] = 0.f;
+  if (a.last_ctrl) for (int i = 0; i < a.nu; ++i) a.last_ctrl[e * a.nu + i] = 0.f;
+}
+
+__global__ __launch_bounds__(256) void sample_action_kernel(int64_t n, int nu, const float* __restrict__ mean,
+                                                            const float* __restrict__ log_std,
+                                                            const float* __restrict__ noise, KsRng rng, float clip_max,
+                                                            float* __restrict__ action) {
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= n) return;
+  const int64_t e = idx / nu;
+  const int u = (int)(idx - e * nu);
+  float a = mean[idx];
+  if (log_std) {
+    float z;
+    if (noise) z = noise[idx];
+    else {
+      const Philox4 r = draw(rng.seed, rng.step, kRngAction, (uint64_t)e, (uint32_t)u);
+      z = normal_from(r.x, r.y);
+    }
+    a += expf(log_std[u]) * z;
+  }
+  if (a != a) a = 0.f;                         // NaN -> 0, rl.py:999-1000
+  a = fminf(fmaxf(a, -clip_max), clip_max);    // rl.py:1001
+  action[idx] = a;
+}
+
+// ---------------------------------------------------------------------------------------------
+// Rewards over a time-major rollout.  One lane per (t, env).
+// Action differences follow rewards.py:410-460: v(t) = a[t]-a[t-1], A(t) = v(t)-v(t-1),
+// J(t) = A(t)-A(t-1), each zeroed when the step before it ended an episode, and the first
+// 1 / 2 / 3 steps of the rollout masked to zero.
+// ---------------------------------------------------------------------------------------------
+__device__ inline float kernel_with_penalty(float x, float scale, float sq, float ab) {
+  return fabsf(x) * -ab + x * x * -sq + expf(-(x * x) / (2.f * scale * scale));
+}
+
+__global__ __launch_bounds__(256) void rewards_kernel(KsRewardIO io) {
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t TN = io.T * io.N;
+  if (idx >= TN) return;
+  const int64_t t = idx / io.N;
+  const float* q = io.qpos ? io.qpos + idx * io.nq : nullptr;
+  const float* v = io.qvel ? io.qvel + idx * io.nv : nullptr;
+  const bool dn = io.done[idx] != 0, sc = io.success && io.success[idx] != 0;
+  const bool d1 = t >= 1 && io.done[idx - io.N] != 0;
+  const bool d2 = t >= 2 && io.done[idx - 2 * io.N] != 0;
+  const bool d3 = t >= 3 && io.done[idx - 3 * io.N] != 0;
+  float total = 0.f;
+  for (int j = 0; j < io.n_rewards; ++j) {
+    const KsRewardDesc r = io.rewards[j];
+    float val = 0.f;
+    switch (r.kind) {
+      case KS_REW_STAY_ALIVE: {
+        const float alive = 1.0f / r.p0;
+        val = dn ? (sc ? (r.p2 != 0.f ? r.p1 : alive) : -1.0f) : alive;
+      } break;
+      case KS_REW_BASE_HEIGHT: {
+        const float x = q[2] - r.p0;
+        val = expf(-(x * x) / (2.f * r.p1 * r.p1));
+      } break;
+      case KS_REW_BASE_HEIGHT_RANGE: {
+        const float z = q[2];
+        val = fmaxf(1.0f - fmaxf(fmaxf(r.p0 - z, z - r.p1), 0.f) * r.p2, 0.f);
+      } break;
+      case KS_REW_ACTION_VEL:
+      case KS_REW_ACTION_ACC:
+      case KS_REW_ACTION_JERK: {
+        const int order = r.kind - KS_REW_ACTION_VEL + 1;
+        float s = 0.f;
+        if (t >= order) {
+          const float* a0 = io.action + idx * io.nu;
+          for (int u = 0; u < io.nu; ++u) {
+            const float x0 = a0[u], x1 = a0[u - io.N * io.nu];
+            const float v0 = d1 ? 0.f : x0 - x1;
+            float x = v0;
+            if (order >= 2) {
+              const float x2 = a0[u - 2 * io.N * io.nu];
+              const float v1 = d2 ? 0.f : x1 - x2;
+              const float A0 = d1 ? 0.f : v0 - v1;
+              x = A0;
+              if (order == 3) {
+                const float x3 = a0[u - 3 * io.N * io.nu];
+                const float v2 = d3 ? 0.f : x2 - x3;
+                const float A1 = d2 ? 0.f : v1 - v2;
+                x = d1 ? 0.f : A0 - A1;
+              }
+            }
+            s += r.norm == KS_NORM_L1 ? fabsf(x) : x * x;
+          }
+          s /= (float)io.nu;
+        }
+        val = s;
+      } break;
+      case KS_REW_UPRIGHT_ANGVEL: val = kernel_with_penalty(v[4], r.p0, r.p1, r.p2); break;
+      case KS_REW_UPRIGHT_LINVEL: val = kernel_with_penalty(v[2], r.p0, r.p1, r.p2); break;
+      case KS_REW_UPRIGHT_POSE: {
+        float zb[3];
+        rot_inv(q + 3, 0.f, 0.f, 1.f, zb);
+        val = kernel_with_penalty(atan2f(zb[0], zb[2]), r.p0, r.p1, r.p2);
+      } break;
+      default: break;
+    }
+    val *= r.scale;
+    if (io.components) io.components[(int64_t)j * TN + idx] = val;
+    total = j == 0 ? val : total + val;
+  }
+  if (io.use_clip_min) total = fmaxf(total, io.clip_min);
+  if (io.use_clip_max) total = fminf(total, io.clip_max);
+  if (io.total) io.total[idx] = total;
+}
+
+}  // namespace ks
+
+using namespace ks;
+
+struct KsTerms {
+  KsTermsDesc host;
+  DevTerms* dev;
+};
+
+extern "C" int ks_terms_create(const KsTermsDesc* d, KsTerms** out) {
+  if (!d || !out) return fail(KS_EINVAL, "ks_terms_create: null argument");
+  if (d->obs_dim < 0 || d->obs_dim > KS_MAX_OBS) return fail(KS_ELIMIT, "ks_terms_create: obs_dim %d > %d", d->obs_dim, KS_MAX_OBS);
+  if (d->n_terms < 0 || d->n_terms > KS_MAX_TERMS) return fail(KS_ELIMIT, "ks_terms_create: %d terminations > %d", d->n_terms, KS_MAX_TERMS);
+  if (d->nq < 0 || d->nq > KS_MAX_QPOS || d->nv < 0 || d->nu < 0 || d->nb < 1) return fail(KS_EINVAL, "ks_terms_create: bad sizes");
+  const int src_dim[KS_SRC_COUNT] = {d->nq, d->nv, d->nv, d->nu, d->nu, d->command_dim, 1, d->nb * 3, d->nb * 4, d->nb * 6, 0};
+  for (int k = 0; k < d->obs_dim; ++k) {
+    const KsObsElem& el = d->obs[k];
+    if (el.src < 0 || el.src >= KS_SRC_COUNT) return fail(KS_EINVAL, "ks_terms_create: obs %d: bad source %d", k, el.src);
+    if (el.kind < KS_OBS_COPY || el.kind > KS_OBS_ROT_INV) return fail(KS_EINVAL, "ks_terms_create: obs %d: bad kind", k);
+    const int span = el.kind == KS_OBS_ROT_INV ? 3 : 1;
+    if (el.src != KS_SRC_CONST && (el.index < 0 || el.index + span > src_dim[el.src]))
+      return fail(KS_EINVAL, "ks_terms_create: obs %d reads [%d,%d) of a source with %d columns", k, el.index, el.index + span, src_dim[el.src]);
+    if (el.kind == KS_OBS_JOINT_POS && (el.src != KS_SRC_QPOS || el.index < 7 || el.index - 7 >= d->nu))
+      return fail(KS_EINVAL, "ks_terms_create: obs %d: joint position index %d out of range", k, el.index);
+    if (el.kind == KS_OBS_ROT_INV && (el.comp < 0 || el.comp > 2 || d->nq < 7))
+      return fail(KS_EINVAL, "ks_terms_create: obs %d: bad rotation component", k);
+    if (el.noise_kind < KS_NOISE_NONE || el.noise_kind > KS_NOISE_MUL_UNIFORM) return fail(KS_EINVAL, "ks_terms_create: obs %d: bad noise kind", k);
+  }
+  for (int j = 0; j < d->n_terms; ++j) {
+    const KsTermDesc& t = d->terms[j];
+    if (t.kind < KS_TERM_MIN_HEIGHT || t.kind > KS_TERM_EPISODE_LENGTH) return fail(KS_EINVAL, "ks_terms_create: termination %d: bad kind", j);
+    if (t.value != 1 && t.value != -1) return fail(KS_EINVAL, "ks_terms_create: termination %d must report +1 or -1", j);
+    if ((t.kind == KS_TERM_NOT_UPRIGHT) && d->nq < 7) return fail(KS_EINVAL, "ks_terms_create: termination %d needs a free root", j);
+    if (d->nq < 3 || d->nv < 3) return fail(KS_EINVAL, "ks_terms_create: terminations need a floating base");
+  }
+  KsTerms* t = new KsTerms();
+  t->host = *d;
+  if (hipMalloc((void**)&t->dev, sizeof(DevTerms)) != hipSuccess) { delete t; return fail(KS_ELAUNCH, "ks_terms_create: hipMalloc failed"); }
+  if (hipMemcpy(t->dev, d, sizeof(KsTermsDesc), hipMemcpyHostToDevice) != hipSuccess) {
+    (void)hipFree(t->dev); delete t; return fail(KS_ELAUNCH, "ks_terms_create: upload failed");
+  }
+  *out = t;
+  return KS_OK;
+}
+
+extern "C" int ks_terms_destroy(KsTerms* t) {
+  if (!t) return KS_OK;
+  (void)hipFree(t->dev);
+  delete t;
+  return KS_OK;
+}
+
+extern "C" int ks_observe(const KsTerms* t, ks_stream_t stream, const KsObserveIO* io) {
+  if (!t || !io) return fail(KS_EINVAL, "ks_observe: null argument");
+  const KsTermsDesc& d = t->host;
+  if (io->N < 0) return fail(KS_EINVAL, "ks_observe: negative env count");
+  if (io->N == 0 || d.obs_dim == 0) return KS_OK;
+  const int src_dim[KS_SRC_COUNT] = {d.nq, d.nv, d.nv, d.nu, d.nu, d.command_dim, 1, d.nb * 3, d.nb * 4, d.nb * 6, 0};
+  ObserveArgs a;
+  std::memset(&a, 0, sizeof(a));
+  bool needs_quat = false, needs_noise = false;
+  for (int k = 0; k < d.obs_dim; ++k) {
+    const KsObsElem& el = d.obs[k];
+    if (el.src != KS_SRC_CONST && !io->src[el.src]) return fail(KS_EINVAL, "ks_observe: observation %d reads source %d, which is NULL", k, el.src);
+    needs_quat |= el.kind == KS_OBS_ROT_INV;
+    needs_noise |= el.noise_kind != KS_NOISE_NONE;
+  }
+  if (needs_quat && !io->src[KS_SRC_QPOS]) return fail(KS_EINVAL, "ks_observe: qpos is required for body-frame observations");
+  if ((io->noise_normal == nullptr) != (io->noise_uniform == nullptr)) return fail(KS_EINVAL, "ks_observe: pass both explicit noise buffers or neither");
+  (void)needs_noise;
+  a.t = t->dev; a.N = io->N; a.level = io->level;
+  for (int s = 0; s < KS_SRC_COUNT; ++s) { a.src[s] = io->src[s]; a.src_dim[s] = src_dim[s]; }
+  a.zero_offset = io->zero_offset; a.bias = io->bias; a.noise_normal = io->noise_normal; a.noise_uniform = io->noise_uniform;
+  a.rng = io->rng; a.obs = io->obs; a.noisy = io->noisy_obs; a.obs_dim = d.obs_dim; a.nq = d.nq; a.nu = d.nu;
+  const int64_t n = io->N * d.obs_dim;
+  const int64_t grid = (n + 255) / 256;
+  if (grid > 0x7fffffff) return fail(KS_ELIMIT, "ks_observe: too many elements");
+  hipLaunchKernelGGL(observe_kernel, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, a);
+  return check_launch("ks_observe");
+}
+
+extern "C" int ks_terminate_reset(const KsTerms* t, ks_stream_t stream, const KsTerminateIO* io) {
+  if (!t || !io) return fail(KS_EINVAL, "ks_terminate_reset: null argument");
+  const KsTermsDesc& d = t->host;
+  if (io->N < 0) return fail(KS_EINVAL, "ks_terminate_reset: negative env count");
+  if (io->N == 0) return KS_OK;
+  if (!io->qpos || !io->qvel) return fail(KS_EINVAL, "ks_terminate_reset: qpos and qvel are required");
+  TerminateArgs a;
+  std::memset(&a, 0, sizeof(a));
+  a.t = t->dev; a.N = io->N; a.level = io->level;
+  a.qpos = io->qpos; a.qvel = io->qvel; a.warm = io->qacc_warmstart; a.time = io->time; a.last_ctrl = io->last_ctrl;
+  a.components = io->components; a.done = io->done; a.success = io->success;
+  a.traj_qpos = io->traj_qpos; a.traj_qvel = io->traj_qvel; a.traj_time = io->traj_time;
+  a.reset_mask = io->reset_mask; a.episode_length = io->episode_length; a.reset_uniform = io->reset_uniform;
+  a.rng = io->rng; a.apply_reset = io->apply_reset; a.nq = d.nq; a.nv = d.nv; a.nu = d.nu; a.n_terms = d.n_terms;
+  a.random_heading = d.random_heading;
+  const int64_t grid = (io->N + 255) / 256;
+  hipLaunchKernelGGL(terminate_kernel, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, a);
+  return check_launch("ks_terminate_reset");
+}
+
+extern "C" int ks_sample_action(ks_stream_t stream, int64_t N, int32_t nu, const float* mean, const float* log_std,
+                                const float* noise_normal, KsRng rng, float clip_max, float* action) {
+  if (N < 0 || nu < 0) return fail(KS_EINVAL, "ks_sample_action: negative size");
+  if (N == 0 || nu == 0) return KS_OK;
+  if (!mean || !action) return fail(KS_EINVAL, "ks_sample_action: null pointer");
+  const int64_t n = N * nu, grid = (n + 255) / 256;
+  if (grid > 0x7fffffff) return fail(KS_ELIMIT, "ks_sample_action: too many elements");
+  hipLaunchKernelGGL(sample_action_kernel, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, n, (int)nu, mean,
+                     log_std, noise_normal, rng, clip_max, action);
+  return check_launch("ks_sample_action");
+}
+
+extern "C" int ks_rewards(ks_stream_t stream, const KsRewardIO* io) {
+  if (!io) return fail(KS_EINVAL, "ks_rewards: null argument");
+  if (io->T < 0 || io->N < 0) return fail(KS_EINVAL, "ks_rewards: negative size");
+  if (io->n_rewards < 0 || io->n_rewards > KS_MAX_REWARD_TERMS) return fail(KS_ELIMIT, "ks_rewards: more than %d terms", KS_MAX_REWARD_TERMS);
+  if (io->T == 0 || io->N == 0) return KS_OK;
+  if (!io->done) return fail(KS_EINVAL, "ks_rewards: done is required");
+  for (int j = 0; j < io->n_rewards; ++j) {
+    const int k = io->rewards[j].kind;
+    if (k < KS_REW_STAY_ALIVE || k > KS_REW_UPRIGHT_POSE) return fail(KS_EINVAL, "ks_rewards: term %d: bad kind", j);
+    const bool needs_q = k == KS_REW_BASE_HEIGHT || k == KS_REW_BASE_HEIGHT_RANGE || k == KS_REW_UPRIGHT_POSE;
+    const bool needs_v = k == KS_REW_UPRIGHT_ANGVEL || k == KS_REW_UPRIGHT_LINVEL;
+    const bool needs_a = k >= KS_REW_ACTION_VEL && k <= KS_REW_ACTION_JERK;
+    if (needs_q && (!io->qpos || io->nq < 7)) return fail(KS_EINVAL, "ks_rewards: term %d needs qpos of a floating base", j);
+    if (needs_v && (!io->qvel || io->nv < 6)) return fail(KS_EINVAL, "ks_rewards: term %d needs qvel of a floating base", j);
+    if (needs_a && (!io->action || io->nu < 1)) return fail(KS_EINVAL, "ks_rewards: term %d needs actions", j);
+    if (k == KS_REW_STAY_ALIVE && !(io->rewards[j].p0 != 0.f)) return fail(KS_EINVAL, "ks_rewards: term %d: zero balance", j);
+  }
+  const int64_t n = io->T * io->N, grid = (n + 255) / 256;
+  if (grid > 0x7fffffff) return fail(KS_ELIMIT, "ks_rewards: too many elements");
+  hipLaunchKernelGGL(rewards_kernel, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, *io);
+  return check_launch("ks_rewards");
+}

@@ -1,0 +1,233 @@
+"""Physics engine behind the reference's PhysicsEngine interface (ksim/engine.py:48-523), batched.
+
+``HipEngine`` is the MI355X counterpart of ``MjxEngine`` (engine.py:202-361): ``reset`` and ``step`` keep
+the reference's argument meaning, but operate on all N envs at once (the reference vmaps the per-env call,
+ksim/task/rl.py:1615) and update the PhysicsState in place (the reference donates it, engine.py:259-263).
+"""
+from __future__ import annotations
+
+import logging
+from abc import ABC, abstractmethod
+from dataclasses import dataclass
+from typing import Literal, Mapping, Sequence
+
+import torch
+
+from . import _lib, physics
+from .actuators import Actuators, PositionActuators, TorqueActuators
+from .env_terms import EnvTerms
+from .noise import RandomVariable
+from .resets import Reset
+from .types import PhysicsData, PhysicsState
+
+logger = logging.getLogger(__name__)
+EngineType = Literal["hip"]
+MISSING = None
+
+
+@dataclass
+class EngineConfig:  # engine.py:48-139
+    action_latency_range: tuple[float, float] = (0.0, 0.0)
+    drop_action_prob: float = 0.0
+    zero_offset_std: float | None = None
+    zero_offset_mag: float | None = None
+    actuator_update_dt: float | None = None
+    ctrl_dt: float | None = MISSING
+    dt: float | None = MISSING
+
+    def __post_init__(self) -> None:
+        if self.dt is MISSING:
+            raise ValueError("`dt` is required")
+        if self.ctrl_dt is MISSING:
+            raise ValueError("`ctrl_dt` is required")
+        lo, hi = self.action_latency_range
+        if lo < 0:
+            raise ValueError("`min_action_latency` must be non-negative")
+        if lo > hi:
+            raise ValueError("`min_action_latency` must be less than or equal to `max_action_latency`")
+        if hi > self.ctrl_dt:
+            logger.warning("`max_action_latency=%f` is greater than `ctrl_dt=%f`", hi, self.ctrl_dt)
+        if (self.ctrl_dt - round(self.ctrl_dt / self.dt) * self.dt) > 1e-6:
+            logger.warning("`ctrl_dt=%f` is not a multiple of `dt=%f`", self.ctrl_dt, self.dt)
+        if self.drop_action_prob < 0 or self.drop_action_prob >= 1:
+            raise ValueError("`drop_action_prob` must be between 0 and 1")
+
+    @property
+    def min_action_latency_step(self) -> float:
+        return self.action_latency_range[0] / self.dt
+
+    @property
+    def max_action_latency_step(self) -> float:
+        return self.action_latency_range[1] / self.dt
+
+    @property
+    def phys_steps_per_ctrl_steps(self) -> int:
+        return round(self.ctrl_dt / self.dt)
+
+    @property
+    def phys_steps_per_actuator_step(self) -> int:
+        if self.actuator_update_dt is not None:
+            return max(1, round(self.actuator_update_dt / self.dt))
+        return 1
+
+    def zero_offset_random_variable(self) -> RandomVariable:  # engine.py:117-138
+        return RandomVariable(mean=0.0, std=self.zero_offset_std or 0.0, mag=self.zero_offset_mag or 0.0)
+
+
+@dataclass(frozen=True)
+class EngineData:  # engine.py:141-168
+    dt: float
+    ctrl_dt: float
+    drop_action_prob: float
+    actuator_update_dt: float | None
+    min_action_latency_step: float
+    max_action_latency_step: float
+    phys_steps_per_ctrl_steps: int
+    phys_steps_per_actuator_step: int
+    zero_offset: RandomVariable
+
+    @classmethod
+    def from_config(cls, config: EngineConfig) -> "EngineData":
+        return cls(dt=config.dt, ctrl_dt=config.ctrl_dt, drop_action_prob=config.drop_action_prob,
+                   actuator_update_dt=config.actuator_update_dt,
+                   min_action_latency_step=config.min_action_latency_step,
+                   max_action_latency_step=config.max_action_latency_step,
+                   phys_steps_per_ctrl_steps=config.phys_steps_per_ctrl_steps,
+                   phys_steps_per_actuator_step=config.phys_steps_per_actuator_step,
+                   zero_offset=config.zero_offset_random_variable())
+
+
+class PhysicsEngine(ABC):  # engine.py:171-199
+    actuators: Actuators
+    resets: tuple
+    events: Mapping
+    data: EngineData
+
+    @abstractmethod
+    def reset(self, physics_model, curriculum_level, rng, num_envs: int, randomization=None) -> PhysicsState:
+        """Reset the engine and return the physics state of `num_envs` fresh episodes."""
+
+    @abstractmethod
+    def step(self, action, physics_model, physics_state: PhysicsState, curriculum_level, rng,
+             randomization=None) -> PhysicsState:
+        """Step the engine and return the updated physics state."""
+
+
+def _generator(rng, device) -> torch.Generator:
+    if isinstance(rng, torch.Generator):
+        return rng
+    g = torch.Generator(device=device)
+    g.manual_seed(int(rng))
+    return g
+
+
+class HipEngine(PhysicsEngine):
+    """Engine for `physics.DeviceModel`s: every physics substep of a control step runs in one HIP kernel."""
+
+    def __init__(self, actuators: Actuators, resets: Sequence[Reset], events: Mapping | None, data: EngineData):
+        if events:
+            raise NotImplementedError("events inside the substep loop (ksim/events.py) are not compiled yet")
+        self.actuators, self.resets, self.events, self.data = actuators, tuple(resets), {}, data
+        self._terms: dict[int, EnvTerms] = {}
+
+    def __hash__(self) -> int:
+        return id(self)
+
+    def _reset_terms(self, physics_model: physics.DeviceModel) -> EnvTerms:
+        key = id(physics_model)
+        if key not in self._terms:
+            self._terms[key] = EnvTerms(physics_model.model, {}, {}, self.resets)
+        return self._terms[key]
+
+    def _check(self, physics_model) -> None:
+        m = physics_model.model
+        if abs(m.dt - self.data.dt) > 1e-9:
+            raise ValueError(f"model dt {m.dt} differs from the engine's dt {self.data.dt}")
+        if isinstance(self.actuators, PositionActuators) and len(self.actuators.kps) != m.nu:
+            raise ValueError("one kp / kd per actuator is required")
+
+    # -------------------------------------------------------------------------------------- reset (engine.py:205-246)
+    def reset(self, physics_model: physics.DeviceModel, curriculum_level, rng, num_envs: int,
+              randomization: Mapping[str, torch.Tensor] | None = None, reset_uniform=None) -> PhysicsState:
+        self._check(physics_model)
+        m, N, dev = physics_model.model, int(num_envs), torch.device("cuda")
+        gen = _generator(rng, dev)
+        z = lambda *s: torch.zeros(*s, dtype=torch.float32, device=dev)  # noqa: E731
+        data = PhysicsData(qpos=z(N, m.nq), qvel=z(N, m.nv), qacc=z(N, m.nv), qacc_warmstart=z(N, m.nv),
+                           ctrl=z(N, m.nu), time=z(N), xpos=z(N, m.nb * 3), xquat=z(N, m.nb * 4), cvel=z(N, m.nb * 6))
+        level = float(curriculum_level)
+        lo, hi = self.data.min_action_latency_step * level, self.data.max_action_latency_step * level
+        state = PhysicsState(
+            last_ctrl=z(N, m.nu), data=data, event_states={},
+            actuator_state=self.actuators.get_initial_state(N, gen) if isinstance(self.actuators, PositionActuators) else None,
+            action_latency=lo + (hi - lo) * torch.rand(N, generator=gen, device=dev),
+            zero_offset=self.data.zero_offset.sample((N, m.nu), gen, level),
+        )
+        seed = int(torch.randint(0, 2**31 - 1, (1,), generator=gen, device=dev).item())
+        self.reset_where(physics_model, state, None, curriculum_level, seed, 0, randomization, reset_uniform)
+        return state
+
+    def reset_where(self, physics_model, state: PhysicsState, mask, curriculum_level, seed: int, step: int,
+                    randomization=None, reset_uniform=None) -> None:
+        """Fresh episodes for the envs in `mask` (all when None): resets, then mjx.forward's counterpart."""
+        d = state.data
+        terms = self._reset_terms(physics_model)
+        st = dict(qpos=d.qpos, qvel=d.qvel, qacc_warmstart=d.qacc_warmstart, time=d.time, last_ctrl=state.last_ctrl)
+        if mask is None:
+            terms.terminate_reset(st, level=float(curriculum_level), seed=seed, step=step, apply_reset=2,
+                                  reset_uniform=reset_uniform)
+        self.forward(physics_model, state, mask, randomization)
+
+    def forward(self, physics_model, state: PhysicsState, mask=None, randomization=None) -> None:
+        d = state.data
+        rnd = randomization or {}
+        physics.forward(physics_model, dict(qpos=d.qpos, qvel=d.qvel, qacc_warmstart=d.qacc_warmstart, env_mask=mask,
+                                            friction=rnd.get("friction"), mass_scale=rnd.get("mass_scale"),
+                                            xpos=d.xpos, xquat=d.xquat, cvel=d.cvel))
+        # engine.py:217-220: qvel and qacc are zeroed after the forward pass (qvel is already zero here)
+
+    # -------------------------------------------------------------------------------------- step (engine.py:259-361)
+    def step(self, action: torch.Tensor, physics_model: physics.DeviceModel, physics_state: PhysicsState,
+             curriculum_level, rng, randomization: Mapping[str, torch.Tensor] | None = None,
+             noise: Mapping[str, torch.Tensor] | None = None,
+             record: Mapping[str, torch.Tensor] | None = None) -> PhysicsState:
+        m, d, s = physics_model.model, physics_state.data, physics_state
+        rnd, noise, record = randomization or {}, noise or {}, record or {}
+        drop = noise.get("drop")
+        p_drop = self.data.drop_action_prob * float(curriculum_level)
+        if drop is None and p_drop > 0:  # engine.py:277-278
+            gen = _generator(rng, action.device)
+            drop = (torch.rand(action.shape, generator=gen, device=action.device) < p_drop).to(torch.uint8)
+        buf = dict(qpos=d.qpos, qvel=d.qvel, qacc_warmstart=d.qacc_warmstart, time=d.time, last_ctrl=s.last_ctrl,
+                   action=action, latency=s.action_latency, zero_offset=s.zero_offset, drop=drop,
+                   friction=rnd.get("friction"), mass_scale=rnd.get("mass_scale"), qacc=d.qacc, ctrl_out=d.ctrl,
+                   xpos=d.xpos, xquat=d.xquat, cvel=d.cvel, action_noise=noise.get("action_noise"),
+                   torque_noise=noise.get("torque_noise"), traj_ctrl=record.get("ctrl"),
+                   traj_xpos=record.get("xpos"), traj_xquat=record.get("xquat"))
+        act = self.actuators
+        if isinstance(act, PositionActuators):
+            cache = getattr(self, "_gain_cache", None)
+            if cache is None or cache[0] is not act or cache[1].device != action.device:
+                t = lambda a: torch.tensor(a, dtype=torch.float32, device=action.device)  # noqa: E731
+                cache = (act, t(act.kps), t(act.kds), t(act.clip_array()))
+                self._gain_cache = cache
+            ast = s.actuator_state or {}
+            buf.update(kp=cache[1], kd=cache[2], ctrl_clip=cache[3], kp_scale=ast.get("kp_scale"),
+                       kd_scale=ast.get("kd_scale"), torque_limit_scale=ast.get("torque_limit_scale"),
+                       action_bias=ast.get("action"), torque_bias=ast.get("torque"))
+            physics.control_step(physics_model, buf, substeps=self.data.phys_steps_per_ctrl_steps,
+                                 actuator_period=self.data.phys_steps_per_actuator_step,
+                                 actuator_type=act.kind, action_scale=act.action_scale)
+        elif isinstance(act, TorqueActuators):
+            physics.control_step(physics_model, buf, substeps=self.data.phys_steps_per_ctrl_steps,
+                                 actuator_period=self.data.phys_steps_per_actuator_step, actuator_type=act.kind)
+        else:
+            raise ValueError(f"Unsupported actuators: {type(act).__name__}")
+        return physics_state
+
+
+def get_physics_engine(engine_type: str, resets, events, actuators: Actuators, config: EngineConfig) -> PhysicsEngine:
+    """Factory with the reference's signature (engine.py:488-515); the only engine type here is "hip"."""
+    if engine_type != "hip":
+        raise ValueError(f"Unsupported physics model type: {engine_type}")
+    return HipEngine(actuators=actuators, resets=resets, events=events, data=EngineData.from_config(config))

@@ -1,0 +1,159 @@
+"""Compiled per-env terms: observations, terminations, resets -> one device spec + the fused kernels.
+
+Covers get_observation (ksim/task/rl.py:153-186), get_terminations and the done/success combination
+(rl.py:288-299,1049-1050), the reset-under-cond of _get_step_env_state (rl.py:1072-1080) and the NaN
+scrub / clip of sampled actions (rl.py:998-1001).
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Mapping, Sequence
+
+import numpy as np
+import torch
+
+from . import _lib
+from . import _lib_terms as T
+from .model import KinematicModel
+from .observation import Observation
+from .resets import Reset, compile_resets
+from .terminations import Termination
+
+
+def _rng(seed: int, step: int) -> T.KsRng:
+    return T.KsRng(int(seed) & (2**64 - 1), int(step) & (2**64 - 1))
+
+
+class EnvTerms:
+    def __init__(self, model: KinematicModel, observations: Mapping[str, Observation],
+                 terminations: Mapping[str, Termination], resets: Sequence[Reset], command_dim: int = 0):
+        lib = _lib.load()
+        torch.zeros(1, device="cuda")
+        self.model, self._lib = model, lib
+        self.observations, self.terminations, self.resets = dict(observations), dict(terminations), tuple(resets)
+        self.command_dim = int(command_dim)
+        d = T.KsTermsDesc()
+        d.nq, d.nv, d.nu, d.nb, d.command_dim = model.nq, model.nv, model.nu, model.nb, self.command_dim
+        self.obs_slices: dict[str, slice] = {}
+        self.bias_std = []
+        k = 0
+        for name, obs in self.observations.items():
+            elems = obs.elements(model, self.command_dim)
+            noise = obs._noise()
+            if k + len(elems) > T.KS_MAX_OBS:
+                raise _lib.KsError(f"observation vector longer than {T.KS_MAX_OBS}")
+            for el in elems:
+                e = d.obs[k]
+                e.kind, e.src, e.index, e.comp = el.kind, el.src, el.index, el.comp
+                e.c0, e.c1, e.c2 = el.const
+                if noise is not None:
+                    e.noise_kind, e.noise_mean, e.noise_scale = noise.kind, noise.mean, noise.scale
+                self.bias_std.append(0.0 if obs.bias is None else float(obs.bias))
+                k += 1
+            self.obs_slices[name] = slice(k - len(elems), k)
+        d.obs_dim = self.obs_dim = k
+        if len(self.terminations) > T.KS_MAX_TERMS:
+            raise _lib.KsError("too many terminations")
+        for j, term in enumerate(self.terminations.values()):
+            t = d.terms[j]
+            t.kind, t.value, t.p0, t.p1, t.p2, t.p3 = term.desc()
+        d.n_terms = self.n_terms = len(self.terminations)
+        tab = compile_resets(self.resets, model)
+        big = 3.0e38
+        for i in range(model.nq):
+            d.reset_base[i], d.reset_mag[i] = tab["base"][i], tab["mag"][i]
+            d.reset_lo[i], d.reset_hi[i] = max(tab["lo"][i], -big), min(tab["hi"][i], big)
+            d.reset_by_level[i] = int(tab["by_level"][i])
+        d.random_heading = int(tab["heading"])
+        self.reset_table = tab
+        self._handle = ctypes.c_void_p()
+        _lib.check(lib.ks_terms_create(ctypes.byref(d), ctypes.byref(self._handle)))
+
+    # ------------------------------------------------------------------ observations
+    def observe(self, sources: Mapping[int, torch.Tensor | None], N: int, *, level: float = 1.0,
+                zero_offset=None, bias=None, noise_normal=None, noise_uniform=None, seed: int = 0, step: int = 0,
+                obs: torch.Tensor | None = None, noisy_obs: torch.Tensor | None = None):
+        m = self.model
+        dims = {T.SRC_QPOS: m.nq, T.SRC_QVEL: m.nv, T.SRC_QACC: m.nv, T.SRC_CTRL: m.nu, T.SRC_LAST_ACTION: m.nu,
+                T.SRC_COMMAND: self.command_dim, T.SRC_TIME: 1, T.SRC_XPOS: m.nb * 3, T.SRC_XQUAT: m.nb * 4,
+                T.SRC_CVEL: m.nb * 6}
+        io = T.KsObserveIO()
+        io.N, io.level = N, level
+        for s, t in sources.items():
+            if t is None:
+                continue
+            _lib.require_cuda(t, dtype=torch.float32)
+            if t.numel() != N * dims[s]:
+                raise _lib.KsError(f"observation source {s}: expected {N}x{dims[s]} elements, got {tuple(t.shape)}")
+            io.src[s] = t.data_ptr()
+        for name, t, shape in (("zero_offset", zero_offset, (N, m.nu)), ("bias", bias, (N, self.obs_dim)),
+                               ("noise_normal", noise_normal, (N, self.obs_dim)),
+                               ("noise_uniform", noise_uniform, (N, self.obs_dim)), ("obs", obs, (N, self.obs_dim)),
+                               ("noisy_obs", noisy_obs, (N, self.obs_dim))):
+            if t is None:
+                continue
+            _lib.require_cuda(t, dtype=torch.float32)
+            if tuple(t.shape) != shape:
+                raise _lib.KsError(f"{name}: expected {shape}, got {tuple(t.shape)}")
+            setattr(io, name, t.data_ptr())
+        io.rng = _rng(seed, step)
+        _lib.check(self._lib.ks_observe(self._handle, _lib.current_stream(), ctypes.byref(io)))
+        return obs, noisy_obs
+
+    # ------------------------------------------------------------------ terminations + reset predication
+    def terminate_reset(self, state: Mapping[str, torch.Tensor], *, level: float = 1.0, components=None, done=None,
+                        success=None, traj_qpos=None, traj_qvel=None, traj_time=None, reset_mask=None,
+                        episode_length=None, reset_uniform=None, seed: int = 0, step: int = 0,
+                        apply_reset: bool = True) -> None:
+        m = self.model
+        qpos = state["qpos"]
+        N = qpos.shape[0]
+        io = T.KsTerminateIO()
+        io.N, io.level, io.apply_reset = N, level, int(apply_reset)
+        spec = [("qpos", state.get("qpos"), (N, m.nq), torch.float32), ("qvel", state.get("qvel"), (N, m.nv), torch.float32),
+                ("qacc_warmstart", state.get("qacc_warmstart"), (N, m.nv), torch.float32),
+                ("time", state.get("time"), (N,), torch.float32), ("last_ctrl", state.get("last_ctrl"), (N, m.nu), torch.float32),
+                ("components", components, (self.n_terms, N), torch.int8), ("done", done, (N,), torch.uint8),
+                ("success", success, (N,), torch.uint8), ("traj_qpos", traj_qpos, (N, m.nq), torch.float32),
+                ("traj_qvel", traj_qvel, (N, m.nv), torch.float32), ("traj_time", traj_time, (N,), torch.float32),
+                ("reset_mask", reset_mask, (N,), torch.uint8), ("episode_length", episode_length, (N,), torch.int32),
+                ("reset_uniform", reset_uniform, (N, m.nq + 1), torch.float32)]
+        for name, t, shape, dt in spec:
+            if t is None:
+                continue
+            if t.dtype == torch.bool and dt == torch.uint8:
+                t = t.view(torch.uint8)
+            _lib.require_cuda(t, dtype=dt)
+            if tuple(t.shape) != shape:
+                raise _lib.KsError(f"{name}: expected {shape}, got {tuple(t.shape)}")
+            setattr(io, name, t.data_ptr())
+        io.rng = _rng(seed, step)
+        _lib.check(self._lib.ks_terminate_reset(self._handle, _lib.current_stream(), ctypes.byref(io)))
+
+    def close(self) -> None:
+        if self._handle:
+            self._lib.ks_terms_destroy(self._handle)
+            self._handle = ctypes.c_void_p()
+
+    def __del__(self):  # pragma: no cover
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+def sample_action(mean: torch.Tensor, log_std: torch.Tensor | None, *, noise: torch.Tensor | None = None,
+                  seed: int = 0, step: int = 0, clip_max: float = 1e3, out: torch.Tensor | None = None):
+    """action = mean + exp(log_std) * N(0,1); NaN -> 0; clip to +-clip_max (ksim/task/rl.py:998-1001)."""
+    lib = _lib.load()
+    _lib.require_cuda(mean, log_std, noise, out, dtype=torch.float32)
+    N, nu = mean.shape
+    if log_std is not None and tuple(log_std.shape) != (nu,):
+        raise _lib.KsError("log_std must have shape (nu,)")
+    if noise is not None and noise.shape != mean.shape:
+        raise _lib.KsError("noise must match the mean's shape")
+    if out is None:
+        out = torch.empty_like(mean)
+    _lib.check(lib.ks_sample_action(_lib.current_stream(), N, nu, _lib.ptr(mean), _lib.ptr(log_std), _lib.ptr(noise),
+                                    _rng(seed, step), float(clip_max), _lib.ptr(out)))
+    return out

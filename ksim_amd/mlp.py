@@ -1,0 +1,101 @@
+"""MLP forward on the matrix cores (policy / critic / discriminator networks of the rollout path).
+
+The reference leaves the network to the task (``sample_action``, ksim/task/rl.py:892-926); the configs here
+use plain MLP stacks.  Weights are given as (out, in) fp32 arrays, like the reference's linear layers.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Sequence
+
+import numpy as np
+import torch
+
+from . import _lib
+from . import _lib_terms as T
+
+_ACT = {None: T.ACT_NONE, "none": T.ACT_NONE, "elu": T.ACT_ELU, "relu": T.ACT_RELU, "tanh": T.ACT_TANH}
+
+
+class MLP:
+    def __init__(self, weights: Sequence, biases: Sequence, activation: str = "elu", dtype: str = "bf16"):
+        lib = _lib.load()
+        if len(weights) != len(biases) or not weights:
+            raise _lib.KsError("one bias per weight matrix is required")
+        if dtype not in ("bf16", "f32"):
+            raise _lib.KsError("dtype must be 'bf16' or 'f32'")
+        torch.zeros(1, device="cuda")  # make sure a HIP context exists before the library allocates
+        ws = [np.ascontiguousarray(w.detach().cpu().numpy() if isinstance(w, torch.Tensor) else w, dtype=np.float32)
+              for w in weights]
+        bs = [np.ascontiguousarray(b.detach().cpu().numpy() if isinstance(b, torch.Tensor) else b, dtype=np.float32)
+              for b in biases]
+        dims = [ws[0].shape[1]]
+        for w, b in zip(ws, bs):
+            if w.ndim != 2 or w.shape[1] != dims[-1] or b.shape != (w.shape[0],):
+                raise _lib.KsError("weight / bias shapes do not chain")
+            dims.append(w.shape[0])
+        d = T.KsMlpDesc()
+        d.n_layers, d.activation = len(ws), _ACT[activation]
+        d.dtype = T.MLP_BF16 if dtype == "bf16" else T.MLP_F32
+        for i, v in enumerate(dims):
+            d.dims[i] = v
+        for i, (w, b) in enumerate(zip(ws, bs)):
+            d.weights[i] = w.ctypes.data
+            d.biases[i] = b.ctypes.data
+        self.dims, self.dtype, self.activation = dims, dtype, activation
+        self._lib = lib
+        self._handle = ctypes.c_void_p()
+        _lib.check(lib.ks_mlp_create(ctypes.byref(d), ctypes.byref(self._handle)))
+        self._ws: torch.Tensor | None = None
+
+    @property
+    def in_dim(self) -> int:
+        return self.dims[0]
+
+    @property
+    def out_dim(self) -> int:
+        return self.dims[-1]
+
+    def flops_per_row(self) -> int:
+        return 2 * sum(a * b for a, b in zip(self.dims[:-1], self.dims[1:]))
+
+    def workspace(self, M: int, device) -> torch.Tensor:
+        need = int(self._lib.ks_mlp_workspace_bytes(self._handle, M))
+        if self._ws is None or self._ws.numel() < need or self._ws.device != torch.device(device):
+            self._ws = torch.empty(need, dtype=torch.uint8, device=device)
+        return self._ws
+
+    def __call__(self, x: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+        _lib.require_cuda(x, dtype=torch.float32)
+        if x.dim() != 2 or x.shape[1] != self.in_dim:
+            raise _lib.KsError(f"expected input (M, {self.in_dim}), got {tuple(x.shape)}")
+        M = x.shape[0]
+        if out is None:
+            out = torch.empty((M, self.out_dim), dtype=torch.float32, device=x.device)
+        else:
+            _lib.require_cuda(out, dtype=torch.float32)
+            if tuple(out.shape) != (M, self.out_dim):
+                raise _lib.KsError("output has the wrong shape")
+        ws = self.workspace(M, x.device)
+        _lib.check(self._lib.ks_mlp_forward(self._handle, _lib.current_stream(), M, _lib.ptr(x), _lib.ptr(out),
+                                            _lib.ptr(ws)))
+        return out
+
+    def close(self) -> None:
+        if self._handle:
+            self._lib.ks_mlp_destroy(self._handle)
+            self._handle = ctypes.c_void_p()
+
+    def __del__(self):  # pragma: no cover
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+def random_mlp(dims: Sequence[int], seed: int, activation: str = "elu", dtype: str = "bf16"):
+    """Random-init network: W ~ N(0, 1/fan_in), b = 0. Returns (MLP, weights, biases)."""
+    rng = np.random.default_rng(seed)
+    ws = [rng.normal(scale=1.0 / np.sqrt(i), size=(o, i)).astype(np.float32) for i, o in zip(dims[:-1], dims[1:])]
+    bs = [np.zeros(o, dtype=np.float32) for o in dims[1:]]
+    return MLP(ws, bs, activation=activation, dtype=dtype), ws, bs

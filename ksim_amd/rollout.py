@@ -1,0 +1,123 @@
+"""Batched rollout of N envs for T control steps (ksim/task/rl.py:1164-1211 step_engine, 1604-1665 _single_unroll).
+
+One control step launches, in order on the current stream: observation (+noise) -> actor MLP (and critic)
+-> action sampling / scrub / clip -> fused physics control step -> terminations + transition record + reset
+predication -> forward pass of the freshly reset envs.  Nothing synchronises the host inside the loop.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Mapping, Sequence
+
+import torch
+
+from . import _lib
+from . import _lib_terms as T
+from . import ppo as ppo_mod
+from .engine import HipEngine
+from .env_terms import EnvTerms, sample_action
+from .mlp import MLP
+from .physics import DeviceModel
+from .rewards import Reward, get_rewards
+from .types import PhysicsState, RewardState, Trajectory
+
+
+@dataclass
+class RolloutConstants:  # the static pieces, ksim/task/rl.py:138-150
+    physics_model: DeviceModel
+    engine: HipEngine
+    terms: EnvTerms
+    rewards: Mapping[str, Reward]
+    actor: MLP
+    critic: MLP | None
+    log_std: torch.Tensor | None
+    action_clip_max: float = 1e3  # RLConfig.action_clip_max, rl.py:589-592
+    reward_clip_min: float | None = None
+    reward_clip_max: float | None = None
+
+
+class RolloutEnvState:  # ksim/task/rl.py:110-123, batched
+    def __init__(self, physics_state: PhysicsState, randomization: Mapping[str, torch.Tensor], commands: torch.Tensor,
+                 obs_bias: torch.Tensor | None, seed: int):
+        self.physics_state = physics_state
+        self.randomization_dict = dict(randomization)
+        self.commands = commands
+        self.obs_bias = obs_bias
+        self.seed = int(seed)
+        self.step = 0
+        N = physics_state.data.qpos.shape[0]
+        self.episode_length = torch.zeros(N, dtype=torch.int32, device=physics_state.data.qpos.device)
+
+
+class Rollout:
+    """Owns the time-major trajectory buffers of one (T, N) rollout and runs it."""
+
+    def __init__(self, constants: RolloutConstants, num_envs: int, rollout_length: int):
+        c, m = constants, constants.physics_model.model
+        self.c, self.N, self.T = c, int(num_envs), int(rollout_length)
+        dev = torch.device("cuda")
+        N, Tn = self.N, self.T
+        f = lambda *s: torch.empty(*s, dtype=torch.float32, device=dev)  # noqa: E731
+        b = lambda *s: torch.zeros(*s, dtype=torch.uint8, device=dev)  # noqa: E731
+        self.obs, self.noisy_obs = f(Tn, N, c.terms.obs_dim), f(Tn, N, c.terms.obs_dim)
+        self.action, self.mean = f(Tn, N, m.nu), f(N, m.nu)
+        self.qpos, self.qvel = f(Tn, N, m.nq), f(Tn, N, m.nv)
+        self.xpos, self.xquat, self.ctrl = f(Tn, N, m.nb * 3), f(Tn, N, m.nb * 4), f(Tn, N, m.nu)
+        self.done, self.success, self.timestep = b(Tn, N), b(Tn, N), f(Tn, N)
+        self.components = torch.zeros(Tn, max(c.terms.n_terms, 1), N, dtype=torch.int8, device=dev)
+        self.values = f(Tn, N, 1) if c.critic is not None else None
+        self.reset_mask = b(N)
+        if c.actor.in_dim != c.terms.obs_dim or c.actor.out_dim != m.nu:
+            raise _lib.KsError("actor must map the observation vector to one mean per actuator")
+        if c.critic is not None and (c.critic.in_dim != c.terms.obs_dim or c.critic.out_dim != 1):
+            raise _lib.KsError("critic must map the observation vector to one value")
+
+    def step_engine(self, env: RolloutEnvState, t: int, level: float = 1.0, noise: Mapping | None = None) -> None:
+        """One control step of every env; the transition lands in slot t of the buffers."""
+        c, ps = self.c, env.physics_state
+        d, noise = ps.data, noise or {}
+        src = {T.SRC_QPOS: d.qpos, T.SRC_QVEL: d.qvel, T.SRC_QACC: d.qacc, T.SRC_CTRL: d.ctrl,
+               T.SRC_LAST_ACTION: ps.last_ctrl, T.SRC_COMMAND: env.commands, T.SRC_TIME: d.time, T.SRC_XPOS: d.xpos,
+               T.SRC_XQUAT: d.xquat, T.SRC_CVEL: d.cvel}
+        c.terms.observe(src, self.N, level=level, zero_offset=ps.zero_offset, bias=env.obs_bias,
+                        noise_normal=noise.get("obs_normal"), noise_uniform=noise.get("obs_uniform"), seed=env.seed,
+                        step=env.step, obs=self.obs[t], noisy_obs=self.noisy_obs[t])
+        c.actor(self.noisy_obs[t], out=self.mean)           # actor reads the noisy copy (walking.py:592-595)
+        if c.critic is not None:
+            c.critic(self.obs[t], out=self.values[t])       # critic reads the clean one (walking.py:626-638)
+        sample_action(self.mean, c.log_std, noise=noise.get("action_normal"), seed=env.seed, step=env.step,
+                      clip_max=c.action_clip_max, out=self.action[t])
+        # the step kernel also writes ctrl / xpos / xquat of the post-step data into the transition slot
+        c.engine.step(self.action[t], c.physics_model, ps, level, env.seed + env.step, env.randomization_dict,
+                      noise=noise.get("engine"), record=dict(ctrl=self.ctrl[t], xpos=self.xpos[t], xquat=self.xquat[t]))
+        st = dict(qpos=d.qpos, qvel=d.qvel, qacc_warmstart=d.qacc_warmstart, time=d.time, last_ctrl=ps.last_ctrl)
+        c.terms.terminate_reset(st, level=level, components=self.components[t][: c.terms.n_terms] if c.terms.n_terms else None,
+                                done=self.done[t], success=self.success[t], traj_qpos=self.qpos[t],
+                                traj_qvel=self.qvel[t], traj_time=self.timestep[t], reset_mask=self.reset_mask,
+                                episode_length=env.episode_length, reset_uniform=noise.get("reset_uniform"),
+                                seed=env.seed, step=env.step)
+        # refresh the derived fields and the warm start of the reset envs (engine.py:213)
+        c.engine.forward(c.physics_model, ps, self.reset_mask, env.randomization_dict)
+        env.step += 1
+
+    def unroll(self, env: RolloutEnvState, level: float = 1.0) -> tuple[Trajectory, RewardState]:
+        for t in range(self.T):
+            self.step_engine(env, t, level)
+        traj = self.trajectory()
+        rewards = get_rewards(traj, self.c.rewards, self.c.reward_clip_min, self.c.reward_clip_max,
+                              want_components=False)
+        return traj, rewards
+
+    def trajectory(self) -> Trajectory:
+        names = list(self.c.terms.terminations)
+        return Trajectory(qpos=self.qpos, qvel=self.qvel, xpos=self.xpos, xquat=self.xquat, ctrl=self.ctrl,
+                          obs={"obs": self.obs, "noisy_obs": self.noisy_obs}, command={}, event_state={},
+                          action=self.action, done=self.done, success=self.success, timestep=self.timestep,
+                          termination_components={n: self.components[:, j] for j, n in enumerate(names)})
+
+    def ppo_inputs(self, rewards: RewardState, gamma: float, lam: float, normalize_advantages: bool = True):
+        """GAE / returns over the rollout in its own (T, N) layout (ksim/task/ppo.py:54-121)."""
+        if self.values is None:
+            raise _lib.KsError("a critic is required for GAE")
+        return ppo_mod.compute_ppo_inputs(self.values.view(self.T, self.N), rewards.total, self.done, self.success,
+                                          gamma, lam, normalize_advantages=normalize_advantages, time_major=True)

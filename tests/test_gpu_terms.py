@@ -1,0 +1,251 @@
+"""Parity of the fused per-env term kernels (observations, terminations/resets, actions, rewards)."""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import terms as ot
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+GOLD = os.path.join(os.path.dirname(__file__), "golden")
+
+
+def t32(a):
+    return torch.tensor(np.asarray(a), dtype=torch.float32, device=DEV).contiguous()
+
+
+def _state(m, N, seed):
+    rng = np.random.default_rng(seed)
+    qpos = rng.normal(size=(N, m.nq))
+    qpos[:, 3:7] /= np.linalg.norm(qpos[:, 3:7], axis=1, keepdims=True)
+    return dict(qpos=qpos, qvel=rng.normal(size=(N, m.nv)), qacc=rng.normal(size=(N, m.nv)),
+                ctrl=rng.normal(size=(N, m.nu)), last=rng.normal(size=(N, m.nu)), cmd=rng.normal(size=(N, 2)),
+                time=rng.random(N) * 3, zero=rng.normal(size=(N, m.nu)) * 0.01, rng=rng)
+
+
+def test_observation_assembly_and_noise():
+    from ksim_amd import _lib_terms as T, model as km, noise, observation as ob
+    from ksim_amd.env_terms import EnvTerms
+
+    m = km.humanoid_model()
+    N = 37
+    s = _state(m, N, 0)
+    observations = {
+        "joint_position": ob.JointPositionObservation(noise=0.01),
+        "joint_velocity": ob.JointVelocityObservation(noise=noise.MultiplicativeUniformNoise(mag=0.1)),
+        "projected_gravity": ob.ProjectedGravityObservation(),
+        "base_angular_velocity": ob.BaseAngularVelocityObservation(in_robot_frame=True, noise=noise.AdditiveUniformNoise(mag=0.2, mean=0.1)),
+        "last_action": ob.LastActionObservation(),
+        "command": ob.CommandObservation(),
+        "base_linear_velocity": ob.BaseLinearVelocityObservation(noise=noise.MultiplicativeGaussianNoise(std=0.05)),
+        "timestep": ob.TimestepObservation(),
+        "actuator_force": ob.ActuatorForceObservation(bias=0.02),
+    }
+    terms = EnvTerms(m, observations, {}, [], command_dim=2)
+    assert terms.obs_dim == 21 + 21 + 3 + 3 + 21 + 2 + 3 + 1 + 21
+    assert terms.obs_dim - 25 == 71  # the first six are the 71-wide actor input of BASELINE config 3
+    K = terms.obs_dim
+    nn, uu = s["rng"].normal(size=(N, K)), s["rng"].random((N, K))
+    bias = s["rng"].normal(size=(N, K)) * 0.02
+    level = 0.7
+    src = {T.SRC_QPOS: t32(s["qpos"]), T.SRC_QVEL: t32(s["qvel"]), T.SRC_QACC: t32(s["qacc"]), T.SRC_CTRL: t32(s["ctrl"]),
+           T.SRC_LAST_ACTION: t32(s["last"]), T.SRC_COMMAND: t32(s["cmd"]), T.SRC_TIME: t32(s["time"])}
+    obs = torch.empty(N, K, device=DEV); noisy = torch.empty(N, K, device=DEV)
+    terms.observe(src, N, level=level, zero_offset=t32(s["zero"]), bias=t32(bias), noise_normal=t32(nn),
+                  noise_uniform=t32(uu), obs=obs, noisy_obs=noisy)
+    q, v = s["qpos"], s["qvel"]
+    g = ot.rotate_vector_by_quat(np.broadcast_to([0, 0, -9.81], (N, 3)), q[:, 3:7], inverse=True)
+    w = ot.rotate_vector_by_quat(v[:, 3:6], q[:, 3:7], inverse=True)
+    want = np.concatenate([q[:, 7:] - s["zero"], v[:, 6:], g, w, s["last"], s["cmd"], v[:, 0:3], s["time"][:, None],
+                           s["ctrl"]], axis=1)
+    np.testing.assert_allclose(obs.cpu().numpy(), want, rtol=2e-6, atol=2e-6)
+    sl = terms.obs_slices
+    wn = want.copy()
+    a = sl["joint_position"]; wn[:, a] = want[:, a] + nn[:, a] * 0.01 * level            # noise.py:102
+    a = sl["joint_velocity"]; wn[:, a] = want[:, a] * ((1.0 - 0.1 * level) + 2 * 0.1 * level * uu[:, a])  # noise.py:86
+    a = sl["base_angular_velocity"]; wn[:, a] = want[:, a] + (0.1 - 0.2 * level) + 2 * 0.2 * level * uu[:, a]
+    a = sl["base_linear_velocity"]; wn[:, a] = want[:, a] * (nn[:, a] * 0.05 * level + 1.0)
+    wn = wn + bias
+    np.testing.assert_allclose(noisy.cpu().numpy(), wn, rtol=3e-6, atol=3e-6)
+    # in-kernel Philox: deterministic for a (seed, step), different across steps, unit-variance normals
+    a1 = torch.empty(N, K, device=DEV); a2 = torch.empty(N, K, device=DEV); a3 = torch.empty(N, K, device=DEV)
+    terms.observe(src, N, seed=5, step=1, zero_offset=t32(s["zero"]), noisy_obs=a1)
+    terms.observe(src, N, seed=5, step=1, zero_offset=t32(s["zero"]), noisy_obs=a2)
+    terms.observe(src, N, seed=5, step=2, zero_offset=t32(s["zero"]), noisy_obs=a3)
+    assert torch.equal(a1, a2) and not torch.equal(a1, a3)
+    z = ((a1 - obs)[:, sl["joint_position"]] / 0.01).flatten()
+    assert abs(z.mean().item()) < 0.15 and abs(z.std().item() - 1.0) < 0.15
+
+
+def test_termination_kats_and_masks_bit_exact():
+    from ksim_amd import model as km, terminations as tm
+    from ksim_amd.env_terms import EnvTerms
+
+    m = km.kbot_scale_model()
+    # the reference's known answers (tests/test_terminations.py:66-99) on its dummy qpos
+    for kat in json.load(open(os.path.join(GOLD, "termination_kats.json"))):
+        if kat["fn"] == "illegal_contact":
+            continue
+        term = tm.NotUprightTermination(kat["max_radians"]) if kat["fn"] == "not_upright" else tm.MinimumHeightTermination(kat["min_height"])
+        terms = EnvTerms(m, {}, {"t": term}, [])
+        qpos = np.zeros((1, m.nq)); qpos[0, :9] = kat["qpos"]
+        comps = torch.zeros(1, 1, dtype=torch.int8, device=DEV)
+        done = torch.zeros(1, dtype=torch.uint8, device=DEV); succ = torch.zeros(1, dtype=torch.uint8, device=DEV)
+        terms.terminate_reset(dict(qpos=t32(qpos), qvel=torch.zeros(1, m.nv, device=DEV)), components=comps, done=done,
+                              success=succ, apply_reset=False)
+        assert comps.item() == kat["expected"] and done.item() == (kat["expected"] != 0) and succ.item() == 0
+    # all term kinds on random states, against the oracle, bit-exact
+    N = 500
+    s = _state(m, N, 3)
+    s["qpos"][:, :3] *= 2.0
+    term_objs = {
+        "min_height": tm.MinimumHeightTermination(0.5), "bad_z": tm.BadZTermination(-1.0, 2.0, -0.5, 1.5),
+        "not_upright": tm.NotUprightTermination(1.2), "bad_vel": tm.BadVelocityTermination(2.5),
+        "far": tm.FarFromOriginTermination(3.0), "length": tm.EpisodeLengthTermination(1.5),
+    }
+    terms = EnvTerms(m, {}, term_objs, [])
+    level = 0.4
+    comps = torch.zeros(6, N, dtype=torch.int8, device=DEV)
+    done = torch.zeros(N, dtype=torch.uint8, device=DEV); succ = torch.zeros(N, dtype=torch.uint8, device=DEV)
+    q32, v32, t32_ = s["qpos"].astype(np.float32), s["qvel"].astype(np.float32), s["time"].astype(np.float32)
+    terms.terminate_reset(dict(qpos=t32(q32), qvel=t32(v32), time=t32(t32_)), level=level, components=comps, done=done,
+                          success=succ, apply_reset=False)
+    want = [ot.minimum_height_termination(q32, np.float32(0.5)), ot.bad_z_termination(q32, -1.0, 2.0, np.float32(level), -0.5, 1.5),
+            ot.not_upright_termination(q32, 1.2), ot.bad_velocity_termination(v32, 2.5),
+            ot.far_from_origin_termination(q32, 3.0), ot.episode_length_termination(t32_, 1.5)]
+    got = comps.cpu().numpy()
+    # exclude the measure-zero band where fp32 and float64 evaluation of a norm/acos straddle the threshold
+    near = np.zeros(N, bool)
+    near |= np.abs(np.linalg.norm(v32[:, :3], axis=1) - 2.5) < 1e-5
+    near |= np.abs(np.linalg.norm(q32[:, :3], axis=1) - 3.0) < 1e-5
+    for j, w in enumerate(want):
+        assert np.array_equal(got[j][~near], w[~near]), list(term_objs)[j]
+    wd, ws = ot.combine_terminations([g for g in got])
+    assert np.array_equal(done.cpu().numpy().astype(bool), wd) and np.array_equal(succ.cpu().numpy().astype(bool), ws)
+    assert wd.sum() > 20 and ws.sum() > 5
+
+
+def test_reset_predication():
+    from ksim_amd import model as km, resets as rs, terminations as tm
+    from ksim_amd.env_terms import EnvTerms
+
+    m = km.kbot_scale_model()
+    N = 64
+    nj = m.nq - 7
+    zeros = tuple(np.linspace(-0.2, 0.2, nj))
+    resets = [rs.RandomJointPositionReset(scale=0.1, scale_by_curriculum=False, zeros=zeros, mins=(-0.25,) * nj, maxs=(0.25,) * nj),
+              rs.RandomJointVelocityReset(scale=0.5), rs.RandomHeightReset(range=(0.0, 0.2)), rs.RandomHeadingReset()]
+    terms = EnvTerms(m, {}, {"h": tm.MinimumHeightTermination(0.5)}, resets)
+    s = _state(m, N, 4)
+    s["qpos"][:, 2] = np.where(np.arange(N) % 3 == 0, 0.2, 0.9)
+    u = s["rng"].uniform(-1, 1, size=(N, m.nq + 1))
+    st = dict(qpos=t32(s["qpos"]), qvel=t32(s["qvel"]), qacc_warmstart=t32(s["qacc"]), time=t32(s["time"]), last_ctrl=t32(s["last"]))
+    before = {k: v.clone() for k, v in st.items()}
+    done = torch.zeros(N, dtype=torch.uint8, device=DEV); mask = torch.zeros(N, dtype=torch.uint8, device=DEV)
+    tq = torch.zeros(N, m.nq, device=DEV); ep = torch.full((N,), 7, dtype=torch.int32, device=DEV)
+    terms.terminate_reset(st, done=done, reset_mask=mask, traj_qpos=tq, episode_length=ep, reset_uniform=t32(u))
+    dn = np.arange(N) % 3 == 0
+    assert np.array_equal(done.cpu().numpy().astype(bool), dn) and torch.equal(done, mask)
+    assert torch.equal(tq, before["qpos"])  # the transition records the pre-reset state
+    keep = torch.from_numpy(~dn).to(DEV)
+    for k in st:
+        assert torch.equal(st[k][keep], before[k][keep]), k  # surviving envs are untouched, bit for bit
+    q = st["qpos"].cpu().numpy()[dn]
+    base = m.qpos0.copy(); base[2] += 0.1
+    np.testing.assert_allclose(q[:, :2], np.broadcast_to(base[:2], q[:, :2].shape), atol=1e-7)
+    np.testing.assert_allclose(q[:, 2], base[2] + 0.1 * u[dn, 2], atol=1e-6)
+    np.testing.assert_allclose(q[:, 7:], np.clip(np.array(zeros) + 0.1 * u[dn, 7:m.nq], -0.25, 0.25), atol=1e-6)
+    yaw = np.pi * u[dn, m.nq]
+    np.testing.assert_allclose(q[:, 3:7], np.stack([np.cos(yaw / 2), 0 * yaw, 0 * yaw, np.sin(yaw / 2)], 1), atol=1e-6)
+    for k in ("qvel", "qacc_warmstart", "time", "last_ctrl"):
+        assert st[k].cpu().numpy()[dn].any() == False  # noqa: E712
+    e = ep.cpu().numpy()
+    assert (e[dn] == 0).all() and (e[~dn] == 8).all()
+    # Philox draws: in range, reproducible
+    st2 = {k: v.clone() for k, v in before.items()}; st3 = {k: v.clone() for k, v in before.items()}
+    terms.terminate_reset(st2, seed=9, step=3); terms.terminate_reset(st3, seed=9, step=3)
+    assert torch.equal(st2["qpos"], st3["qpos"])
+    j = st2["qpos"].cpu().numpy()[dn][:, 7:]
+    assert (np.abs(j) <= 0.25 + 1e-6).all() and j.std() > 0.03
+
+
+def test_sample_action_scrub_and_clip():
+    from ksim_amd.env_terms import sample_action
+
+    N, nu = 33, 20
+    rng = np.random.default_rng(1)
+    mean = rng.normal(size=(N, nu)).astype(np.float32)
+    mean[0, 0], mean[1, 1], mean[2, 2] = np.nan, 1e9, -1e9
+    ls = rng.normal(size=nu).astype(np.float32) * 0.3
+    z = rng.normal(size=(N, nu)).astype(np.float32)
+    got = sample_action(t32(mean), t32(ls), noise=t32(z), clip_max=1e3).cpu().numpy()
+    want = ot.scrub_action(mean.astype(np.float64) + np.exp(ls.astype(np.float64)) * z, 1e3)
+    np.testing.assert_allclose(got, want, rtol=2e-6, atol=2e-6)
+    assert got[0, 0] == 0.0 and got[1, 1] == 1e3 and got[2, 2] == -1e3
+    det = sample_action(t32(mean), None).cpu().numpy()
+    np.testing.assert_array_equal(det, ot.scrub_action(mean, 1e3).astype(np.float32))
+    a = sample_action(t32(mean), t32(ls), seed=3, step=4); b = sample_action(t32(mean), t32(ls), seed=3, step=4)
+    assert torch.equal(a, b)
+
+
+def _traj(Tn, N, nq, nv, nu, seed, p_done=0.1):
+    rng = np.random.default_rng(seed)
+    q = rng.normal(size=(Tn, N, nq)); q[..., 3:7] /= np.linalg.norm(q[..., 3:7], axis=-1, keepdims=True)
+    done = rng.random((Tn, N)) < p_done
+    return dict(qpos=q, qvel=rng.normal(size=(Tn, N, nv)), action=rng.normal(size=(Tn, N, nu)), done=done,
+                success=done & (rng.random((Tn, N)) < 0.3))
+
+
+def test_reward_kats_through_the_kernel():
+    """The reference's own action-penalty vectors (tests/test_rewards.py:63-271), evaluated by the HIP kernel."""
+    from ksim_amd import rewards as rw
+    from ksim_amd.types import Trajectory
+
+    cls = {"velocity": rw.ActionVelocityPenalty, "acceleration": rw.ActionAccelerationPenalty, "jerk": rw.ActionJerkPenalty}
+    for kat in json.load(open(os.path.join(GOLD, "reward_kats.json"))):
+        a = np.array(kat["actions"])[:, None, :]  # (T, N=1, 3)
+        Tn = a.shape[0]
+        done = np.zeros((Tn, 1), bool) if kat["done"] is None else np.array(kat["done"])[:, None]
+        traj = Trajectory(qpos=None, qvel=None, xpos=None, xquat=None, ctrl=None, obs={}, command={}, event_state={},
+                          action=t32(a), done=torch.from_numpy(done).to(DEV), success=None, timestep=None)
+        out = rw.get_rewards(traj, {"p": cls[kat["fn"]](scale=1.0, norm=kat["norm"])})
+        # a *Penalty enters the total with a negative sign (rl.py:219-221); the KAT is the raw term
+        np.testing.assert_allclose(-out.total.cpu().numpy()[:, 0], kat["expected"], atol=kat["atol"], rtol=0)
+
+
+def test_rewards_against_oracle():
+    from ksim_amd import rewards as rw
+    from ksim_amd.types import Trajectory
+
+    Tn, N, nq, nv, nu = 40, 19, 27, 26, 20
+    tr = _traj(Tn, N, nq, nv, nu, 7)
+    rewards = {"stay_alive": rw.StayAliveReward(scale=1.0, success_reward=2.0), "height": rw.BaseHeightReward(scale=0.5, height_target=0.9),
+               "range": rw.BaseHeightRangeReward(scale=0.3, z_lower=-0.5, z_upper=0.5, dropoff=2.0),
+               "vel": rw.ActionVelocityPenalty(scale=0.01, norm="l1"), "acc": rw.ActionAccelerationPenalty(scale=0.02),
+               "jerk": rw.ActionJerkPenalty(scale=0.03), "upright": rw.UprightReward(scale=0.7)}
+    traj = Trajectory(qpos=t32(tr["qpos"]), qvel=t32(tr["qvel"]), xpos=None, xquat=None, ctrl=None, obs={}, command={},
+                      event_state={}, action=t32(tr["action"]), done=torch.from_numpy(tr["done"]).to(DEV),
+                      success=torch.from_numpy(tr["success"]).to(DEV), timestep=None)
+    out = rw.get_rewards(traj, rewards, clip_min=-0.5, clip_max=2.5)
+    comps = {}
+    for e in range(N):
+        a, dn, sc, q, v = tr["action"][:, e], tr["done"][:, e], tr["success"][:, e], tr["qpos"][:, e], tr["qvel"][:, e]
+        up = ot.upright_reward(q, v)
+        c = {"stay_alive": ot.stay_alive_reward(dn, sc, success_reward=2.0), "height": ot.base_height_reward(q, 0.9),
+             "range": ot.base_height_range_reward(q, -0.5, 0.5, 2.0), "vel": ot.action_velocity_penalty(a, dn, "l1"),
+             "acc": ot.action_acceleration_penalty(a, dn), "jerk": ot.action_jerk_penalty(a, dn),
+             "upright/angvel": up["angvel"], "upright/linvel": up["linvel"], "upright/pose": up["pose"]}
+        for k, val in c.items():
+            comps.setdefault(k, []).append(val)
+    scales = {"stay_alive": 1.0, "height": 0.5, "range": 0.3, "vel": 0.01, "acc": 0.02, "jerk": 0.03,
+              "upright/angvel": 0.7, "upright/linvel": 0.7, "upright/pose": 0.7}
+    pen = {k: k in ("vel", "acc", "jerk") for k in scales}
+    stacked = {k: np.stack(v, axis=1) for k, v in comps.items()}
+    total, scaled = ot.total_reward(stacked, scales, pen, clip_min=-0.5, clip_max=2.5)
+    assert list(out.components) == list(scales)
+    for k in scales:
+        np.testing.assert_allclose(out.components[k].cpu().numpy(), scaled[k], rtol=1e-5, atol=2e-5, err_msg=k)
+    np.testing.assert_allclose(out.total.cpu().numpy(), total, rtol=1e-5, atol=5e-5)
