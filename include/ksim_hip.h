@@ -244,6 +244,8 @@ typedef struct KsTermDesc {
 typedef struct KsTermsDesc {
   int32_t nq, nv, nu, nb;
   int32_t obs_dim, n_terms, command_dim, random_heading;
+  int32_t nonfinite_terminates; /* 1: an env whose qpos/qvel is not finite counts as failed (done, no success);
+                                   the reference has no such guard and would carry the NaNs forever */
   KsObsElem obs[KS_MAX_OBS];
   KsTermDesc terms[KS_MAX_TERMS];
   float reset_base[KS_MAX_QPOS], reset_mag[KS_MAX_QPOS], reset_lo[KS_MAX_QPOS], reset_hi[KS_MAX_QPOS];

@@ -91,7 +91,7 @@ struct TerminateArgs {
   int32_t* episode_length;
   const float* reset_uniform;
   KsRng rng;
-  int apply_reset, nq, nv, nu, n_terms, random_heading;
+  int apply_reset, nq, nv, nu, n_terms, random_heading, nonfinite_terminates;
 };
 
 // One lane per env.  Termination comparisons are strict and done in fp32 on the stored state, so
@@ -127,6 +127,12 @@ __global__ __launch_bounds__(256) void terminate_kernel(TerminateArgs a) {
     if (a.components) a.components[(int64_t)j * a.N + e] = val;
     done |= val != 0;
     succ &= val != -1;
+  }
+  if (a.nonfinite_terminates) {
+    bool finite = true;
+    for (int i = 0; i < a.nq; ++i) finite &= fabsf(q[i]) <= 3.0e38f;  // false for NaN and inf
+    for (int i = 0; i < a.nv; ++i) finite &= fabsf(v[i]) <= 3.0e38f;
+    if (!finite) { done = true; succ = false; }
   }
   succ = succ && done;
   if (a.done) a.done[e] = done ? 1 : 0;
@@ -366,7 +372,7 @@ extern "C" int ks_terminate_reset(const KsTerms* t, ks_stream_t stream, const Ks
   a.traj_qpos = io->traj_qpos; a.traj_qvel = io->traj_qvel; a.traj_time = io->traj_time;
   a.reset_mask = io->reset_mask; a.episode_length = io->episode_length; a.reset_uniform = io->reset_uniform;
   a.rng = io->rng; a.apply_reset = io->apply_reset; a.nq = d.nq; a.nv = d.nv; a.nu = d.nu; a.n_terms = d.n_terms;
-  a.random_heading = d.random_heading;
+  a.random_heading = d.random_heading; a.nonfinite_terminates = d.nonfinite_terminates;
   const int64_t grid = (io->N + 255) / 256;
   hipLaunchKernelGGL(terminate_kernel, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, a);
   return check_launch("ks_terminate_reset");

@@ -26,7 +26,8 @@ def _rng(seed: int, step: int) -> T.KsRng:
 
 class EnvTerms:
     def __init__(self, model: KinematicModel, observations: Mapping[str, Observation],
-                 terminations: Mapping[str, Termination], resets: Sequence[Reset], command_dim: int = 0):
+                 terminations: Mapping[str, Termination], resets: Sequence[Reset], command_dim: int = 0,
+                 terminate_on_nonfinite: bool = True):
         lib = _lib.load()
         torch.zeros(1, device="cuda")
         self.model, self._lib = model, lib
@@ -65,6 +66,7 @@ class EnvTerms:
             d.reset_lo[i], d.reset_hi[i] = max(tab["lo"][i], -big), min(tab["hi"][i], big)
             d.reset_by_level[i] = int(tab["by_level"][i])
         d.random_heading = int(tab["heading"])
+        d.nonfinite_terminates = int(terminate_on_nonfinite)
         self.reset_table = tab
         self._handle = ctypes.c_void_p()
         _lib.check(lib.ks_terms_create(ctypes.byref(d), ctypes.byref(self._handle)))

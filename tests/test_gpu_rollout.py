@@ -1,0 +1,171 @@
+"""End-to-end rollout (obs -> MLP -> action -> fused physics -> termination -> reset -> record) vs the oracle."""
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from dyn_common import rel_err
+from oracle import ppo as oppo
+from oracle import terms as ot
+from oracle.dyn import Oracle
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def t32(a):
+    return torch.tensor(np.asarray(a), dtype=torch.float32, device=DEV).contiguous()
+
+
+def build(N, T, seed=0, min_height=0.9):
+    from ksim_amd import actuators, engine, model as km, observation as ob, physics, randomization as rnd, resets as rs
+    from ksim_amd import rewards as rw, terminations as tm
+    from ksim_amd.env_terms import EnvTerms
+    from ksim_amd.mlp import MLP
+    from ksim_amd.rollout import Rollout, RolloutConstants, RolloutEnvState
+
+    m = km.kbot_scale_model()
+    rng = np.random.default_rng(seed)
+    # kd * dt / (armature + link inertia) must stay below 1 for the explicit damping term to be stable
+    kps, kds = rng.uniform(20, 150, m.nu), rng.uniform(0.5, 1.5, m.nu)
+    clip = np.tile([60.0, 40.0, 40.0, 60.0, 17.0], 4); clip[10:] = [17.0, 17.0, 14.0, 14.0, 5.0] * 2
+    act = actuators.PositionActuators(kps=tuple(kps), kds=tuple(kds), ctrl_clip=tuple(clip))
+    resets = [rs.RandomJointPositionReset(scale=0.1, scale_by_curriculum=False)]
+    cfg = engine.EngineConfig(dt=0.005, ctrl_dt=0.02)
+    eng = engine.get_physics_engine("hip", resets, {}, act, cfg)
+    observations = {"jp": ob.JointPositionObservation(noise=0.01), "jv": ob.JointVelocityObservation(noise=0.01),
+                    "g": ob.ProjectedGravityObservation(noise=0.01),
+                    "w": ob.BaseAngularVelocityObservation(in_robot_frame=True, noise=0.01),
+                    "a": ob.LastActionObservation(), "c": ob.CommandObservation()}
+    terms = EnvTerms(m, observations, {"min_height": tm.MinimumHeightTermination(min_height)}, resets, command_dim=2)
+    dims = (terms.obs_dim, 64, 64, m.nu)
+    ws = [rng.normal(scale=1 / np.sqrt(i), size=(o, i)).astype(np.float32) for i, o in zip(dims[:-1], dims[1:])]
+    ws[-1] *= 0.1  # small final layer: actions stay near the PD set point
+    bs = [np.zeros(o, np.float32) for o in dims[1:]]
+    cdims = (terms.obs_dim, 64, 1)
+    cws = [rng.normal(scale=1 / np.sqrt(i), size=(o, i)).astype(np.float32) for i, o in zip(cdims[:-1], cdims[1:])]
+    cbs = [np.zeros(o, np.float32) for o in cdims[1:]]
+    dm = physics.DeviceModel(m)
+    log_std = np.full(m.nu, -2.0, np.float32)
+    rewards = {"stay_alive": rw.StayAliveReward(scale=1.0), "height": rw.BaseHeightReward(scale=0.5, height_target=1.0),
+               "vel": rw.ActionVelocityPenalty(scale=0.01)}
+    consts = RolloutConstants(physics_model=dm, engine=eng, terms=terms, rewards=rewards,
+                              actor=MLP(ws, bs, dtype="f32"), critic=MLP(cws, cbs, dtype="f32"), log_std=t32(log_std))
+    gen = torch.Generator(device=DEV); gen.manual_seed(seed)
+    randomization = rnd.get_physics_randomizers(m, {"f": rnd.FloorFrictionRandomizer(0.4, 1.2),
+                                                    "m": rnd.AllBodiesMassMultiplicationRandomizer(0.9, 1.1)}, N, gen)
+    return m, consts, randomization, (ws, bs, cws, cbs, log_std, kps, kds, clip), Rollout(consts, N, T), RolloutEnvState
+
+
+def _mlp64(x, ws, bs):
+    h = torch.from_numpy(np.asarray(x, dtype=np.float64))
+    for i, (w, b) in enumerate(zip(ws, bs)):
+        h = F.linear(h, torch.from_numpy(w).double(), torch.from_numpy(b).double())
+        if i + 1 < len(ws):
+            h = F.elu(h)
+    return h.numpy()
+
+
+def test_rollout_matches_oracle_composition():
+    N, T = 12, 3
+    m, c, rnd_, (ws, bs, cws, cbs, log_std, kps, kds, clip), ro, EnvState = build(N, T, seed=5)
+    rng = np.random.default_rng(6)
+    K = c.terms.obs_dim
+    u0 = rng.uniform(-1, 1, (N, m.nq + 1))
+    ps = c.engine.reset(c.physics_model, 1.0, 0, N, rnd_, reset_uniform=t32(u0))
+    # a third of the envs start just below the termination height (feet touching), so they finish on the first step
+    low = np.arange(N) % 3 == 0
+    ps.data.qpos[torch.from_numpy(low).to(DEV), 2] = 0.87
+    cmd = rng.normal(size=(N, 2))
+    env = EnvState(ps, rnd_, t32(cmd), None, seed=1)
+    fr, ms = rnd_["friction"].cpu().numpy().astype(np.float64), rnd_["mass_scale"].cpu().numpy().astype(np.float64)
+    # ---- oracle side state
+    orc = Oracle(m.arrays())
+    q0 = ps.data.qpos.cpu().numpy().astype(np.float64)
+    want_q0 = np.tile(m.qpos0, (N, 1)); want_q0[:, 7:] += 0.1 * u0[:, 7:m.nq]
+    np.testing.assert_allclose(q0[~low], want_q0[~low], atol=1e-6)  # engine.reset applied the reset table
+    datas = [orc.data(q0[e], friction=fr[e], mass_scale=ms[e]) for e in range(N)]
+    for d in datas:
+        orc.forward(d)  # engine.py:213 — warm start of the fresh episode
+        d.qvel = 0.0
+    last = np.zeros((N, m.nu))
+    for t in range(T):
+        noise = dict(obs_normal=rng.normal(size=(N, K)), obs_uniform=rng.random((N, K)),
+                     action_normal=rng.normal(size=(N, m.nu)), reset_uniform=rng.uniform(-1, 1, (N, m.nq + 1)))
+        ro.step_engine(env, t, 1.0, {k: t32(v) for k, v in noise.items()})
+        # oracle: observation
+        q = np.array([np.array(d.qpos) for d in datas]); v = np.array([np.array(d.qvel) for d in datas])
+        g = ot.rotate_vector_by_quat(np.broadcast_to([0, 0, -9.81], (N, 3)), q[:, 3:7], inverse=True)
+        w = ot.rotate_vector_by_quat(v[:, 3:6], q[:, 3:7], inverse=True)
+        obs = np.concatenate([q[:, 7:], v[:, 6:], g, w, last, cmd], axis=1)
+        noisy = obs.copy(); noisy[:, : 2 * m.nu + 6] += 0.01 * noise["obs_normal"][:, : 2 * m.nu + 6]
+        np.testing.assert_allclose(ro.obs[t].cpu().numpy(), obs, rtol=1e-4, atol=2e-4)
+        mean = _mlp64(noisy, ws, bs)
+        action = ot.scrub_action(mean + np.exp(log_std.astype(np.float64)) * noise["action_normal"])
+        np.testing.assert_allclose(ro.action[t].cpu().numpy(), action, rtol=1e-3, atol=2e-3)
+        value = _mlp64(obs, cws, cbs)
+        np.testing.assert_allclose(ro.values[t].cpu().numpy(), value, rtol=1e-3, atol=2e-3)
+        # oracle: physics (4 substeps, blend + PD), termination, reset
+        for e, d in enumerate(datas):
+            tau = np.zeros(m.nu)
+            for s in range(4):
+                ctl = ot.latency_blend(float(s), 0.0, last[e], action[e], np.zeros(m.nu, bool))
+                tau = ot.position_actuator_torque(ctl, np.array(d.qpos[7:]), np.array(d.qvel[6:]), kps, kds, clip)
+                d.ctrl = tau
+                orc.step(d)
+        last = action.copy()
+        q = np.array([np.array(d.qpos) for d in datas]); v = np.array([np.array(d.qvel) for d in datas])
+        term = ot.minimum_height_termination(q, 0.9)
+        done, succ = ot.combine_terminations([term])
+        assert np.array_equal(ro.done[t].cpu().numpy().astype(bool), done), f"done mask differs at step {t}"
+        assert np.array_equal(ro.success[t].cpu().numpy().astype(bool), succ)
+        assert np.array_equal(ro.components[t][0].cpu().numpy(), term)
+        tol = 1e-4 if t == 0 else 1e-3
+        assert rel_err(ro.qpos[t].cpu().numpy(), q).max() <= tol, rel_err(ro.qpos[t].cpu().numpy(), q).max()
+        assert rel_err(ro.qvel[t].cpu().numpy(), v, floor=1e-2).max() <= tol
+        xp = np.array([np.array(d.xpos).reshape(-1) for d in datas])
+        assert rel_err(ro.xpos[t].cpu().numpy(), xp).max() <= tol
+        np.testing.assert_allclose(ro.timestep[t].cpu().numpy(), [d.time for d in datas], rtol=1e-5)
+        for e in np.where(done)[0]:
+            nq = m.qpos0.copy(); nq[7:] += 0.1 * noise["reset_uniform"][e, 7:m.nq]
+            datas[e] = orc.data(nq, friction=fr[e], mass_scale=ms[e])
+            orc.forward(datas[e])
+            last[e] = 0.0
+        if t == 0:
+            assert done.sum() == low.sum()
+    # live state after the rollout: reset envs restarted, others continued
+    q = np.array([np.array(d.qpos) for d in datas])
+    assert rel_err(ps.data.qpos.cpu().numpy(), q).max() <= 1e-3
+    # rewards + GAE over the recorded rollout, against the oracle on the recorded arrays
+    traj = ro.trajectory()
+    from ksim_amd.rewards import get_rewards
+    rew = get_rewards(traj, c.rewards)
+    a_, dn, sc, qq = (x.cpu().numpy() for x in (ro.action, ro.done, ro.success, ro.qpos))
+    tot = np.stack([ot.stay_alive_reward(dn[:, e].astype(bool), sc[:, e].astype(bool)) + 0.5 * ot.base_height_reward(qq[:, e], 1.0)
+                    - 0.01 * ot.action_velocity_penalty(a_[:, e], dn[:, e].astype(bool)) for e in range(N)], axis=1)
+    np.testing.assert_allclose(rew.total.cpu().numpy(), tot, rtol=1e-5, atol=1e-5)
+    inp = ro.ppo_inputs(rew, 0.99, 0.95, normalize_advantages=False)
+    vals = ro.values.view(T, N).cpu().numpy()
+    want = oppo.compute_ppo_inputs(vals.T, rew.total.cpu().numpy().T, dn.T, sc.T, 0.99, 0.95)
+    np.testing.assert_allclose(inp.gae_bt.cpu().numpy(), want["gae"].T, rtol=1e-5, atol=1e-5)
+    np.testing.assert_allclose(inp.returns_bt.cpu().numpy(), want["returns"].T, rtol=1e-5, atol=1e-5)
+
+
+def test_long_rollout_with_resets_stays_finite_and_reproducible():
+    """Philox mode: 200 control steps with resets; two runs with one seed are bit-identical."""
+    N, T = 256, 8
+    outs = []
+    for _ in range(2):
+        m, c, rnd_, _, ro, EnvState = build(N, T, seed=11, min_height=0.7)
+        ps = c.engine.reset(c.physics_model, 1.0, 3, N, rnd_)
+        env = EnvState(ps, rnd_, torch.zeros(N, 2, device=DEV), None, seed=77)
+        ndone = 0
+        for _ in range(25):
+            traj, rew = ro.unroll(env)
+            ndone += int(traj.done.sum().item())
+            assert torch.isfinite(traj.qpos).all() and torch.isfinite(rew.total).all()
+        outs.append((ps.data.qpos.clone(), ndone, env.episode_length.clone()))
+    assert outs[0][1] > 0, "no env ever terminated: the reset path was not exercised"
+    assert torch.equal(outs[0][0], outs[1][0]) and outs[0][1] == outs[1][1]
+    assert torch.equal(outs[0][2], outs[1][2])
+    assert (outs[0][0][:, 2] > 0.5).all()  # every env sits above the termination height after its reset
