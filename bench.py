@@ -1,0 +1,202 @@
+"""Headline benchmark: env-steps/sec of the 8192-env K-Bot-scale rollout on one MI355X.
+
+A "step" is one control step of every env: observation (+noise) -> actor and critic MLPs (bf16 MFMA) -> action
+sampling -> fused physics (4 substeps) -> termination + transition record + reset -> forward pass of the reset
+envs; every `--rollout` steps the rewards and GAE kernels run over the recorded rollout.  Inputs are synthetic,
+seeded, resident in HBM before the timed region.  Prints ONE JSON line.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
+BF16_PEAK_TFLOPS = 2500.0  # dense MFMA bf16
+FP32_VALU_PEAK_TFLOPS = 157.3
+
+
+def cpu_baseline(target_seconds: float = 12.0):
+    """The oracle's C restatement of the control step (float32, OpenMP over envs) on this host's cores."""
+    import numpy as np
+
+    from ksim_amd import model as km
+    from ksim_amd.configs import KBOT_TORQUE_LIMITS
+    from oracle.dyn import Oracle
+
+    m = km.kbot_scale_model(seed=1004)
+    orc = Oracle(m.arrays(), np.float32)
+    cores = min(16, os.cpu_count() or 1)
+    N = 2048
+    rng = np.random.default_rng(1004)
+    block = orc.batch(N)
+    for e in range(N):
+        d = block[e]
+        q = m.qpos0.copy()
+        q[7:] += rng.uniform(-0.1, 0.1, m.nu)
+        for i, v in enumerate(q):
+            d.qpos[i] = v
+        for b in range(m.nb):
+            d.mass_scale[b] = rng.uniform(0.9, 1.1)
+        d.friction = rng.uniform(0.4, 1.2)
+    last = np.zeros((N, m.nu), dtype=np.float32)
+    kp = np.tile(rng.uniform(20, 150, m.nu), (N, 1))
+    kd = np.tile(rng.uniform(0.5, 1.5, m.nu), (N, 1))
+    lat = np.zeros(N)
+
+    def run(k):
+        t0 = time.perf_counter()
+        for _ in range(k):
+            act = rng.normal(scale=0.1, size=(N, m.nu))
+            orc.ctrl_step_batch(block, 4, 1, act, last, lat, None, kp, kd, KBOT_TORQUE_LIMITS, nthreads=cores)
+        return time.perf_counter() - t0
+
+    run(10)  # let the robots land on their feet so contacts are active, as in the GPU run
+    t1 = run(2)
+    k = max(2, int(target_seconds / max(t1 / 2, 1e-3)))
+    t = run(k)
+    return {"value": N * k / t, "unit": "env-steps/s", "cores": cores, "kind": "port",
+            "sample": f"physics control step only (PD + 4 substeps), {N} envs x {k} steps, float32 C restatement "
+                      f"of the MJX path (not MJX), OpenMP over envs"}
+
+
+def main() -> None:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=40)
+    ap.add_argument("--envs", type=int, default=8192)
+    ap.add_argument("--rollout", type=int, default=32)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    from ksim_amd import _lib, ppo
+    from ksim_amd.configs import kbot_rollout, step_algorithmic_bytes
+    from ksim_amd.rewards import get_rewards
+
+    _lib.load()
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    N, T = args.envs, args.rollout
+    consts, env, ro, _ = kbot_rollout(num_envs=N, rollout_length=T)
+    m = consts.physics_model.model
+
+    # time the dominant kernel (the fused physics control step) with events on the launch stream
+    step_events: list = []
+    orig_step = consts.engine.step
+
+    def timed_step(*a, **kw):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        out = orig_step(*a, **kw)
+        e1.record()
+        step_events.append((e0, e1))
+        return out
+
+    def one_step(k: int) -> None:
+        t = k % T
+        ro.step_engine(env, t)
+        if t == T - 1:
+            rew = get_rewards(ro.trajectory(), consts.rewards, want_components=False)
+            ro.ppo_inputs(rew, 0.99, 0.95, normalize_advantages=True)
+
+    for k in range(args.warmup):
+        one_step(k)
+    consts.engine.step = timed_step
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for k in range(args.warmup, args.warmup + args.steps):
+        one_step(k)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    consts.engine.step = orig_step
+    kernel_ms = sum(a.elapsed_time(b) for a, b in step_events) / len(step_events)
+    ndone = int(ro.done.sum().item())
+    assert torch.isfinite(env.physics_state.data.qpos).all(), "non-finite state after the benchmark"
+
+    # GAE on rotating cfg-2 sized buffers (T=128, N=4096): larger than the caches in total
+    gae = gae_bandwidth(torch, ppo)
+    mlp = mlp_rate(torch, consts)
+
+    obs_dim = consts.terms.obs_dim
+    bytes_per_env = step_algorithmic_bytes(m, obs_dim, 1 + m.nb)
+    achieved = bytes_per_env * N / (kernel_ms * 1e-3) / 1e9
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "step_kernel_traffic.json")
+    if os.path.exists(tpath):
+        traffic = json.load(open(tpath)).get("hbm_bytes_per_launch")
+    line = {
+        "metric": "env-steps/sec, 8192-env humanoid rollout (1 GPU)", "value": N * args.steps / elapsed,
+        "unit": "env-steps/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": elapsed / args.steps * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "cfg4: K-Bot-scale biped (free root + 20 hinges, 8 foot spheres), per-env friction/mass "
+                               "randomisation, obs noise 0.01, reset on z<0.5, actor+critic 3x512 bf16 MLP, "
+                               "dt=0.005 x 4 substeps", "num_envs": N, "rollout_length": T, "substeps": 4,
+                   "obs_dim": obs_dim, "episodes_finished_in_last_rollout": ndone},
+        "roofline": {"bound": "hbm", "kernel": "step_kernel (fused control step)", "achieved": achieved,
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
+                     "algorithmic_bytes_per_env_step": bytes_per_env, "kernel_ms": kernel_ms,
+                     "note": "the fused step is fp32-VALU/LDS-bound (~1e3 flop/byte); the HBM fraction is reported "
+                             "against the bytes the engine contract obliges a step to move"},
+        "gae": gae, "policy_mlp": mlp,
+    }
+    if not args.no_cpu_baseline:
+        line["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(line))
+
+
+def gae_bandwidth(torch, ppo, T=128, N=4096, sets=32, reps=4):
+    dev = "cuda"
+    g = torch.Generator(device=dev)
+    g.manual_seed(1002)
+    bufs = [(torch.randn(N, T, device=dev, generator=g), torch.randn(N, T, device=dev, generator=g),
+             (torch.rand(N, T, device=dev, generator=g) < 0.01)) for _ in range(sets)]
+    for v, r, d in bufs[:2]:
+        ppo.compute_ppo_inputs(v, r, d, None, 0.99, 0.95)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        for v, r, d in bufs:
+            ppo.compute_ppo_inputs(v, r, d, None, 0.99, 0.95)
+    e1.record()
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / (reps * sets)
+    nbytes = T * N * 21
+    return {"workload": "cfg2: T=128, N=4096 fp32, (B,T) layout, 32 rotating buffer sets", "ms_per_call": ms,
+            "achieved_GBps": nbytes / (ms * 1e-3) / 1e9, "frac_of_hbm_peak": nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+            "algorithmic_bytes": nbytes}
+
+
+def mlp_rate(torch, consts, reps=20):
+    out = {}
+    for M in (8192, 524288):
+        x = torch.randn(M, consts.actor.in_dim, device="cuda")
+        y = torch.empty(M, consts.actor.out_dim, device="cuda")
+        consts.actor(x, out=y)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            consts.actor(x, out=y)
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / reps
+        tf = consts.actor.flops_per_row() * M / (ms * 1e-3) / 1e12
+        out[f"rows_{M}"] = {"ms": ms, "TFLOPs": tf, "mfma_utilisation": tf / BF16_PEAK_TFLOPS}
+    out["net"] = "actor " + "x".join(str(d) for d in consts.actor.dims) + " bf16, fp32 accumulate"
+    return out
+
+
+if __name__ == "__main__":
+    main()

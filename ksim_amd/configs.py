@@ -1,0 +1,67 @@
+"""The benchmark workloads as ready-to-run rollouts (seeded, synthetic, random-init networks)."""
+from __future__ import annotations
+
+import numpy as np
+import torch
+
+from . import actuators, engine, model as km, observation as ob, physics, randomization as rnd, resets as rs
+from . import rewards as rw, terminations as tm
+from .env_terms import EnvTerms
+from .mlp import MLP
+from .rollout import Rollout, RolloutConstants, RolloutEnvState
+
+# soft torque limits by joint class (N m): legs (hip pitch/roll/yaw, knee, ankle), arms (shoulder x3, elbow, wrist)
+KBOT_TORQUE_LIMITS = np.array([60.0, 40.0, 40.0, 60.0, 17.0] * 2 + [17.0, 17.0, 14.0, 14.0, 5.0] * 2)
+
+
+def _net(dims, rng, last_scale=1.0, dtype="bf16"):
+    ws = [rng.normal(scale=1.0 / np.sqrt(i), size=(o, i)).astype(np.float32) for i, o in zip(dims[:-1], dims[1:])]
+    ws[-1] *= last_scale
+    bs = [np.zeros(o, dtype=np.float32) for o in dims[1:]]
+    return MLP(ws, bs, activation="elu", dtype=dtype)
+
+
+def kbot_rollout(num_envs: int = 8192, rollout_length: int = 32, seed: int = 1004, hidden: int = 512,
+                 dtype: str = "bf16", min_height: float = 0.5):
+    """K-Bot-scale biped rollout: free root + 20 hinges, 8 foot spheres, per-env friction ~U(0.4,1.2) and
+    mass scale ~U(0.9,1.1), observation noise N(0,0.01), reset on base height < `min_height`, actor and critic
+    3 x `hidden` MLPs, dt 0.005 with 4 physics substeps per control step."""
+    m = km.kbot_scale_model(seed=seed)
+    rng = np.random.default_rng(seed)
+    kps = rng.uniform(20.0, 150.0, m.nu)
+    kds = rng.uniform(0.5, 1.5, m.nu)
+    act = actuators.PositionActuators(kps=tuple(kps), kds=tuple(kds), ctrl_clip=tuple(KBOT_TORQUE_LIMITS))
+    resets = [rs.RandomJointPositionReset(scale=0.1, scale_by_curriculum=False)]
+    eng = engine.get_physics_engine("hip", resets, {}, act, engine.EngineConfig(dt=0.005, ctrl_dt=0.02))
+    noise = 0.01
+    observations = {
+        "joint_position": ob.JointPositionObservation(noise=noise),
+        "joint_velocity": ob.JointVelocityObservation(noise=noise),
+        "projected_gravity": ob.ProjectedGravityObservation(noise=noise),
+        "base_angular_velocity": ob.BaseAngularVelocityObservation(in_robot_frame=True, noise=noise),
+        "last_action": ob.LastActionObservation(),
+        "command": ob.CommandObservation(),
+    }
+    terms = EnvTerms(m, observations, {"minimum_height": tm.MinimumHeightTermination(min_height)}, resets,
+                     command_dim=2)
+    dm = physics.DeviceModel(m)
+    dev = torch.device("cuda")
+    actor = _net((terms.obs_dim, hidden, hidden, hidden, m.nu), rng, last_scale=0.1, dtype=dtype)
+    critic = _net((terms.obs_dim, hidden, hidden, hidden, 1), rng, dtype=dtype)
+    rewards = {"stay_alive": rw.StayAliveReward(scale=1.0), "base_height": rw.BaseHeightReward(scale=0.5, height_target=0.87),
+               "upright": rw.UprightReward(scale=0.2), "action_velocity": rw.ActionVelocityPenalty(scale=0.01)}
+    consts = RolloutConstants(physics_model=dm, engine=eng, terms=terms, rewards=rewards, actor=actor, critic=critic,
+                              log_std=torch.full((m.nu,), -2.0, device=dev))
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(seed)
+    randomization = rnd.get_physics_randomizers(
+        m, {"floor_friction": rnd.FloorFrictionRandomizer(0.4, 1.2),
+            "mass": rnd.AllBodiesMassMultiplicationRandomizer(0.9, 1.1)}, num_envs, gen)
+    ps = eng.reset(dm, 1.0, gen, num_envs, randomization)
+    env = RolloutEnvState(ps, randomization, torch.zeros(num_envs, 2, device=dev), None, seed=seed)
+    return consts, env, Rollout(consts, num_envs, rollout_length), dict(kps=kps, kds=kds, clip=KBOT_TORQUE_LIMITS)
+
+
+def step_algorithmic_bytes(m, obs_dim: int, per_env_params: int) -> int:
+    """Bytes one fused control step is obliged to move per env: state in/out, transition record, observation."""
+    return 4 * (2 * m.nq + 4 * m.nv + 3 * m.nu + 1 + 7 * m.nb + obs_dim + per_env_params) + 2

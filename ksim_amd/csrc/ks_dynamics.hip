@@ -296,6 +296,9 @@ __device__ __forceinline__ bool in_bracket(const LsPoint& x, const LsPoint& y) {
 }
 
 // ------------------------------------------------------------------------------------------- the fused kernel
+// FWD = true is the forward-only variant (derived fields + warm start of a given state, no actuation, no
+// integration) that replaces the mjx.forward of a reset.
+template <bool FWD>
 __global__ __launch_bounds__(64) void step_kernel(StepArgs a) {
   extern __shared__ float lds_raw[];
   const DevModel& m = *a.model;
@@ -325,10 +328,10 @@ __global__ __launch_bounds__(64) void step_kernel(StepArgs a) {
   float my_qacc = 0.f;
   KS_SYNC();
 
-  const int nsub = a.forward_only ? 1 : a.substeps;
+  const int nsub = FWD ? 1 : a.substeps;
   for (int sub = 0; sub < nsub; ++sub) {
     // ---- actuators (ksim/engine.py:287-320, ksim/actuators.py:198-217)
-    if (!a.forward_only && (sub % a.actuator_period) == 0 && lane < nu) {
+    if (!FWD && (sub % a.actuator_period) == 0 && lane < nu) {
       const int u = lane;
       const int64_t eu = env * nu + u;
       float prct = (float)sub - latency;
@@ -582,7 +585,7 @@ __global__ __launch_bounds__(64) void step_kernel(StepArgs a) {
     if (lane < nv) { l.warm[lane] = qacc; l.qacc[lane] = qacc; }
 
     // ---- semi-implicit Euler
-    if (!a.forward_only) {
+    if (!FWD) {
       if (lane < nv) l.qvel[lane] = my_qvel + m.dt * qacc;
       KS_SYNC();
       if (lane > 0 && lane < nb) {
@@ -608,7 +611,7 @@ __global__ __launch_bounds__(64) void step_kernel(StepArgs a) {
   }
 
   // ---- write back
-  if (!a.forward_only) {
+  if (!FWD) {
     for (int i = lane; i < nq; i += 64) a.qpos[env * nq + i] = l.qpos[i];
     for (int i = lane; i < nv; i += 64) a.qvel[env * nv + i] = l.qvel[i];
     if (a.time && lane == 0) a.time[env] = time;
@@ -758,7 +761,6 @@ static int launch_step(const KsModel* km, ks_stream_t stream, const KsStepIO* io
   std::memset(&a, 0, sizeof(a));
   a.model = km->dev;
   a.N = io->N;
-  a.forward_only = forward_only ? 1 : 0;
   a.qpos = io->qpos; a.qvel = io->qvel; a.qacc_warmstart = io->qacc_warmstart; a.time = io->time;
   a.friction = io->friction; a.mass_scale = io->mass_scale; a.env_mask = io->env_mask;
   a.qacc = io->qacc; a.ctrl_out = io->ctrl_out; a.xpos = io->xpos; a.xquat = io->xquat; a.cvel = io->cvel;
@@ -787,11 +789,13 @@ static int launch_step(const KsModel* km, ks_stream_t stream, const KsStepIO* io
   }
   const int bytes = lds_floats(m.nb, m.nq, m.nv, m.nu, m.ns) * 4;
   if (bytes > 160 * 1024) return fail(KS_ELIMIT, "ks_step: model needs %d bytes of LDS", bytes);
+  const void* fn = forward_only ? (const void*)step_kernel<true> : (const void*)step_kernel<false>;
   if (bytes > 64 * 1024) {
-    hipError_t e = hipFuncSetAttribute((const void*)step_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
     if (e != hipSuccess) return fail(KS_ELAUNCH, "ks_step: cannot raise the LDS limit: %s", hipGetErrorString(e));
   }
-  hipLaunchKernelGGL(step_kernel, dim3((unsigned)io->N), dim3(64), bytes, (hipStream_t)stream, a);
+  if (forward_only) hipLaunchKernelGGL(step_kernel<true>, dim3((unsigned)io->N), dim3(64), bytes, (hipStream_t)stream, a);
+  else hipLaunchKernelGGL(step_kernel<false>, dim3((unsigned)io->N), dim3(64), bytes, (hipStream_t)stream, a);
   return check_launch("ks_step");
 }
 

@@ -9,7 +9,7 @@ struct DevModel;
 struct StepArgs {
   const DevModel* model;
   int64_t N;
-  int substeps, actuator_period, actuator_type, forward_only;
+  int substeps, actuator_period, actuator_type;
   float action_scale;
   float *qpos, *qvel, *qacc_warmstart, *time, *last_ctrl;
   const float *action, *ctrl_in, *latency, *zero_offset;
