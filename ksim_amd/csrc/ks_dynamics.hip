@@ -1,13 +1,18 @@
-// Fused control-step kernel: S physics substeps of one env per wavefront, state resident in LDS.
+// Fused control-step kernel: S physics substeps of one env per wavefront.
 //
-// One 64-lane wavefront owns one env.  Lanes map to bodies, dofs, constraint rows or matrix
-// entries depending on the phase; all cross-lane traffic goes through LDS or DPP reductions and
-// every branch on solver progress (Newton iterations, line-search refinements, contact count) is
-// wave-uniform, so a converged env stops iterating.  Phases of one substep:
-//   kinematics (per-body chain walk) -> centre of mass -> com-based inertias and motion axes ->
-//   composite inertias -> dense mass matrix -> body velocities + RNE bias -> smooth forces ->
-//   sphere/plane contacts and pyramidal constraint rows -> Cholesky of M -> Newton solver with
-//   exact line search -> semi-implicit Euler.
+// One 64-lane wavefront owns one env (64-thread workgroups, so a workgroup barrier is a wave barrier).
+// Where the data lives:
+//   registers  row i of the mass matrix, of the Newton Hessian / its Cholesky factor and (for lanes that are
+//              constraint rows) of the constraint Jacobian; the lane's own body / dof / sphere constants;
+//              all per-dof and per-row solver vectors
+//   LDS        state (qpos, qvel, warm start, torques), body poses, com-based inertias and motion axes,
+//              a staging copy of M and of J (column access), one broadcast vector
+//   HBM        touched once at the start and once at the end of the control step
+// Cross-lane traffic is v_readlane broadcasts (Cholesky, triangular solves), DPP reductions and LDS
+// broadcasts; every branch on solver progress is wave-uniform, so a converged env stops iterating.
+// Phases of one substep: level-wise kinematics -> centre of mass -> com-based inertias / motion axes ->
+// composite inertias -> mass matrix -> level-wise velocities + RNE bias -> smooth forces -> sphere/plane
+// contacts, pyramidal rows -> Cholesky of M -> Newton with exact line search -> semi-implicit Euler.
 // The arithmetic follows the MuJoCo model that ksim/engine.py:257 invokes through mjx.step.
 #include "ks_common.h"
 #include "ks_model.h"
@@ -18,273 +23,148 @@
 namespace ks {
 
 #define KS_SYNC() __syncthreads()
+// Phase timers for kernel tuning: compiled in only with -DKS_PROFILE, which reuses the dbg_M buffer for cycle counts.
+#ifdef KS_PROFILE
+#define KS_TICK(k) { const long long t_now = clock64(); prof[k] += (float)(t_now - t_last); t_last = t_now; }
+#else
+#define KS_TICK(k)
+#endif
+constexpr int NP = 32;  // register rows are padded to 32 columns
 
 struct Lds {
-  float *qpos, *qvel, *warm, *tau, *sc, *bmass;
-  float *xpos, *xquat, *xmat, *xipos, *ximat, *xanchor, *xaxis;
-  float *cinert, *crb, *cdof, *cvel, *cfrc, *fsub, *buf;
-  float *M, *H, *J;
-  float *vbuf, *fbuf, *wbuf, *qfs, *qacc;
+  float *qpos, *qvel, *warm, *tau;
+  float *xpos, *xquat, *xmat, *xanchor, *xaxis;
+  float *cinert, *crb, *cdof, *buf, *cvel, *cacc, *cfrc, *fsub;
+  float *M, *J, *vbuf;
   float *con_off, *con_D, *con_kip;
-  int* con_body;
+  int *con_body, *sub_end;
+  unsigned* con_mask;
 };
 
+__host__ __device__ inline int up4(int n) { return (n + 3) & ~3; }
+
 __host__ __device__ inline int lds_floats(int nb, int nq, int nv, int nu, int ns) {
-  const int nvs = nv | 1;
+  const int nvs = nv | 1, js = up4(nv) % 32 == 0 ? up4(nv) + 4 : up4(nv);
   int n = 0;
-  n += nq + nv + nv + nu + 2 * nq + nb;                   // qpos qvel warm tau sc bmass
-  n += nb * (3 + 4 + 9 + 3 + 9 + 3 + 3);                  // xpos xquat xmat xipos ximat xanchor xaxis
-  n += nb * 10 * 2 + nv * 6 + nb * 6 * 3 + nv * 6;        // cinert crb cdof cvel cfrc fsub buf
-  n += nv * nvs * 2 + 4 * ns * nvs;                       // M H J
-  n += nv + 4 * ns + 4 * ns + nv + nv;                    // vbuf fbuf wbuf qfs qacc
-  n += ns * 3 + ns + ns + ns;                             // con_off con_D con_kip con_body
+  n += up4(nq) + 32 + up4(nv) + up4(nu);                             // qpos qvel(32) warm tau
+  n += up4(nb * 3) + up4(nb * 4) + up4(nb * 9) + 2 * up4(nb * 3);      // xpos xquat xmat xanchor xaxis
+  n += up4(nv * 6) + up4(nb * 6);                                    // cdof cvel
+  const int scratch = 2 * up4(nb * 10) + up4(nv * 6) + 3 * up4(nb * 6);  // cinert crb buf cacc cfrc fsub
+  const int jsz = up4(4 * ns * js + 32);                             // J overlays that scratch once it is dead
+  n += scratch > jsz ? scratch : jsz;
+  n += up4(nv * nvs) + 32;                                           // M vbuf
+  n += up4(ns * 3) + 4 * up4(ns) + up4(nb);                          // con_off con_D con_kip con_body con_mask sub_end
   return n + 8;
 }
 
 __device__ inline Lds carve(float* p, const DevModel& m) {
-  const int nb = m.nb, nq = m.nq, nv = m.nv, nu = m.nu, ns = m.ns, nvs = m.nvs;
+  const int nb = m.nb, nq = m.nq, nv = m.nv, nu = m.nu, ns = m.ns, nvs = m.nvs, js = m.js;
   Lds l;
   auto take = [&](int n) {
     float* r = p;
-    p += n;
+    p += up4(n);
     return r;
   };
-  l.qpos = take(nq); l.qvel = take(nv); l.warm = take(nv); l.tau = take(nu); l.sc = take(2 * nq); l.bmass = take(nb);
-  l.xpos = take(nb * 3); l.xquat = take(nb * 4); l.xmat = take(nb * 9); l.xipos = take(nb * 3);
-  l.ximat = take(nb * 9); l.xanchor = take(nb * 3); l.xaxis = take(nb * 3);
-  l.cinert = take(nb * 10); l.crb = take(nb * 10); l.cdof = take(nv * 6); l.cvel = take(nb * 6);
-  l.cfrc = take(nb * 6); l.fsub = take(nb * 6); l.buf = take(nv * 6);
-  l.M = take(nv * nvs); l.H = take(nv * nvs); l.J = take(4 * ns * nvs);
-  l.vbuf = take(nv); l.fbuf = take(4 * ns); l.wbuf = take(4 * ns); l.qfs = take(nv); l.qacc = take(nv);
+  l.qpos = take(nq); l.qvel = take(32); l.warm = take(nv); l.tau = take(nu);
+  l.xpos = take(nb * 3); l.xquat = take(nb * 4); l.xmat = take(nb * 9); l.xanchor = take(nb * 3); l.xaxis = take(nb * 3);
+  l.cdof = take(nv * 6); l.cvel = take(nb * 6);
+  {
+    float* base = p;
+    l.cinert = take(nb * 10); l.crb = take(nb * 10); l.buf = take(nv * 6);
+    l.cacc = take(nb * 6); l.cfrc = take(nb * 6); l.fsub = take(nb * 6);
+    float* end = p;
+    l.J = base;  // written only after the bias forces are out of fsub
+    float* jend = base + up4(4 * ns * js + 32);
+    p = end > jend ? end : jend;
+  }
+  l.M = take(nv * nvs); l.vbuf = take(32);
   l.con_off = take(ns * 3); l.con_D = take(ns); l.con_kip = take(ns);
   l.con_body = reinterpret_cast<int*>(take(ns));
+  l.con_mask = reinterpret_cast<unsigned*>(take(ns));
+  l.sub_end = reinterpret_cast<int*>(take(nb));
   return l;
 }
 
-// ------------------------------------------------------------------------------------------- position stage
-__device__ inline void kinematics(const DevModel& m, const Lds& l, int lane) {
-  // half-angle sines/cosines of every hinge coordinate
-  for (int i = lane; i < m.nq; i += 64) {
-    const float h = 0.5f * (l.qpos[i] - m.qpos0[i]);
-    l.sc[2 * i] = sinf(h);
-    l.sc[2 * i + 1] = cosf(h);
-  }
-  KS_SYNC();
-  if (lane == 0) {
-    for (int k = 0; k < 3; ++k) { l.xpos[k] = 0.f; l.xipos[k] = 0.f; l.xanchor[k] = 0.f; l.xaxis[k] = 0.f; }
-    l.xquat[0] = 1.f; l.xquat[1] = l.xquat[2] = l.xquat[3] = 0.f;
-    for (int k = 0; k < 9; ++k) { l.xmat[k] = (k % 4 == 0) ? 1.f : 0.f; l.ximat[k] = l.xmat[k]; }
-  } else if (lane < m.nb) {
-    const int b = lane;
-    V3 pos = {0.f, 0.f, 0.f}, anchor = {0.f, 0.f, 0.f}, axis = {0.f, 0.f, 1.f};
-    Quat quat = {1.f, 0.f, 0.f, 0.f};
-    Mat3 R = q2mat(quat);
-    const int depth = m.body_depth[b];
-    for (int d = 0; d < depth; ++d) {
-      const int c = m.body_chain[b][d];
-      const int jt = m.body_jtype[c];
-      if (jt == kJntFree) {
-        const int qa = m.body_qadr[c];
-        pos = ld3(l.qpos + qa);
-        quat = qnormalize({l.qpos[qa + 3], l.qpos[qa + 4], l.qpos[qa + 5], l.qpos[qa + 6]});
-        anchor = pos;
-        axis = {0.f, 0.f, 1.f};
-      } else {
-        V3 npos = pos + mul(R, ld3(m.body_pos[c]));
-        Quat nq = qmul(quat, {m.body_quat[c][0], m.body_quat[c][1], m.body_quat[c][2], m.body_quat[c][3]});
-        if (jt == kJntHinge) {
-          const V3 jpos = ld3(m.jnt_pos[c]), jax = ld3(m.jnt_axis[c]);
-          const Mat3 Rn = q2mat(nq);
-          anchor = npos + mul(Rn, jpos);
-          axis = mul(Rn, jax);
-          const float s = l.sc[2 * m.body_qadr[c]], co = l.sc[2 * m.body_qadr[c] + 1];
-          nq = qmul(nq, {co, jax.x * s, jax.y * s, jax.z * s});
-          npos = anchor - mul(q2mat(nq), jpos);
-        }
-        quat = qnormalize(nq);
-        pos = npos;
-      }
-      R = q2mat(quat);
-    }
-    st3(l.xpos + 3 * b, pos);
-    l.xquat[4 * b] = quat.w; l.xquat[4 * b + 1] = quat.x; l.xquat[4 * b + 2] = quat.y; l.xquat[4 * b + 3] = quat.z;
-    for (int k = 0; k < 9; ++k) l.xmat[9 * b + k] = R.m[k];
-    st3(l.xanchor + 3 * b, anchor);
-    st3(l.xaxis + 3 * b, axis);
-    st3(l.xipos + 3 * b, pos + mul(R, ld3(m.body_ipos[b])));
-    const Mat3 Ri = q2mat(qnormalize(
-        qmul(quat, {m.body_iquat[b][0], m.body_iquat[b][1], m.body_iquat[b][2], m.body_iquat[b][3]})));
-    for (int k = 0; k < 9; ++k) l.ximat[9 * b + k] = Ri.m[k];
-  }
-  KS_SYNC();
-}
-
-// centre of mass of the tree (wave-uniform result), com-based inertias, motion axes
-__device__ inline V3 com_pos(const DevModel& m, const Lds& l, int lane, const float* mass_scale) {
-  float mass = 0.f;
-  V3 mp = {0.f, 0.f, 0.f};
-  if (lane > 0 && lane < m.nb) {
-    mass = m.body_mass[lane] * (mass_scale ? mass_scale[lane] : 1.f);
-    mp = ld3(l.xipos + 3 * lane) * mass;
-    l.bmass[lane] = mass;
-  }
-  const float mt = wave_sum(mass);
-  const float inv = mt > 1e-15f ? 1.0f / mt : 0.f;
-  const V3 com = {wave_sum(mp.x) * inv, wave_sum(mp.y) * inv, wave_sum(mp.z) * inv};
-  if (lane == 0) {
-    for (int k = 0; k < 10; ++k) l.cinert[k] = 0.f;
-  } else if (lane < m.nb) {
-    const int b = lane;
-    const float* R = l.ximat + 9 * b;
-    const float I0 = m.body_inertia[b][0], I1 = m.body_inertia[b][1], I2 = m.body_inertia[b][2];
-    const V3 d = ld3(l.xipos + 3 * b) - com;
-    const float xx = R[0] * I0 * R[0] + R[1] * I1 * R[1] + R[2] * I2 * R[2];
-    const float yy = R[3] * I0 * R[3] + R[4] * I1 * R[4] + R[5] * I2 * R[5];
-    const float zz = R[6] * I0 * R[6] + R[7] * I1 * R[7] + R[8] * I2 * R[8];
-    const float xy = R[0] * I0 * R[3] + R[1] * I1 * R[4] + R[2] * I2 * R[5];
-    const float xz = R[0] * I0 * R[6] + R[1] * I1 * R[7] + R[2] * I2 * R[8];
-    const float yz = R[3] * I0 * R[6] + R[4] * I1 * R[7] + R[5] * I2 * R[8];
-    const float d2 = dot(d, d);
-    float* ci = l.cinert + 10 * b;
-    ci[0] = xx + mass * (d2 - d.x * d.x);
-    ci[1] = yy + mass * (d2 - d.y * d.y);
-    ci[2] = zz + mass * (d2 - d.z * d.z);
-    ci[3] = xy - mass * d.x * d.y;
-    ci[4] = xz - mass * d.x * d.z;
-    ci[5] = yz - mass * d.y * d.z;
-    ci[6] = mass * d.x; ci[7] = mass * d.y; ci[8] = mass * d.z;
-    ci[9] = mass;
-  }
-  if (lane < m.nv) {
-    const int j = lane, b = m.dof_body[j];
-    const V3 off = com - ld3(l.xanchor + 3 * b);
-    Sp cd;
-    if (m.body_jtype[b] == kJntFree) {
-      const int k = j - m.body_dofadr[b];
-      if (k < 3) {
-        cd.a = {0.f, 0.f, 0.f};
-        cd.l = {k == 0 ? 1.f : 0.f, k == 1 ? 1.f : 0.f, k == 2 ? 1.f : 0.f};
-      } else {
-        const float* R = l.xmat + 9 * b;
-        const V3 ax = {R[k - 3], R[3 + k - 3], R[6 + k - 3]};
-        cd.a = ax;
-        cd.l = cross(ax, off);
-      }
-    } else {
-      const V3 ax = ld3(l.xaxis + 3 * b);
-      cd.a = ax;
-      cd.l = cross(ax, off);
-    }
-    st6(l.cdof + 6 * j, cd);
-  }
-  KS_SYNC();
-  return com;
-}
-
-// composite inertias (subtree sums over the depth-first body order) and the dense mass matrix
-__device__ inline void crb_mass_matrix(const DevModel& m, const Lds& l, int lane) {
-  for (int idx = lane; idx < m.nb * 10; idx += 64) {
-    const int b = idx / 10, k = idx - 10 * b;
-    float s = 0.f;
-    if (b > 0) {
-      const int e = m.body_subtree_end[b];
-      for (int c = b; c < e; ++c) s += l.cinert[10 * c + k];
-    }
-    l.crb[idx] = s;
-  }
-  for (int idx = lane; idx < m.nv * m.nvs; idx += 64) l.M[idx] = 0.f;
-  KS_SYNC();
-  if (lane < m.nv) st6(l.buf + 6 * lane, inert_mul(l.crb + 10 * m.dof_body[lane], ld6(l.cdof + 6 * lane)));
-  KS_SYNC();
-  for (int p = lane; p < m.npairs; p += 64) {
-    const int i = m.pair_i[p], j = m.pair_j[p];
-    float v = dot(ld6(l.cdof + 6 * j), ld6(l.buf + 6 * i));
-    if (i == j) v += m.dof_armature[i];
-    l.M[i * m.nvs + j] = v;
-    l.M[j * m.nvs + i] = v;
-  }
-  KS_SYNC();
-}
-
-// ------------------------------------------------------------------------------------------- velocity stage
-// body velocities, axis derivatives and RNE with zero joint acceleration; leaves qfrc_bias in l.vbuf
-__device__ inline void velocity_and_bias(const DevModel& m, const Lds& l, int lane) {
-  if (lane == 0) {
-    for (int k = 0; k < 6; ++k) { l.cvel[k] = 0.f; l.cfrc[k] = 0.f; }
-  } else if (lane < m.nb) {
-    const int b = lane;
-    Sp v = {{0.f, 0.f, 0.f}, {0.f, 0.f, 0.f}};
-    Sp acc = {{0.f, 0.f, 0.f}, {-m.gravity[0], -m.gravity[1], -m.gravity[2]}};
-    const int depth = m.body_depth[b];
-    for (int d = 0; d < depth; ++d) {
-      const int c = m.body_chain[b][d];
-      const int da = m.body_dofadr[c];
-      if (m.body_jtype[c] == kJntFree) {
-        for (int k = 0; k < 3; ++k) v = v + ld6(l.cdof + 6 * (da + k)) * l.qvel[da + k];
-        Sp dv = {{0.f, 0.f, 0.f}, {0.f, 0.f, 0.f}};
-        for (int k = 3; k < 6; ++k) {
-          const Sp cd = ld6(l.cdof + 6 * (da + k));
-          acc = acc + cross_motion(v, cd) * l.qvel[da + k];
-          dv = dv + cd * l.qvel[da + k];
-        }
-        v = v + dv;
-      } else if (m.body_jtype[c] == kJntHinge) {
-        const Sp cd = ld6(l.cdof + 6 * da);
-        acc = acc + cross_motion(v, cd) * l.qvel[da];
-        v = v + cd * l.qvel[da];
-      }
-    }
-    st6(l.cvel + 6 * b, v);
-    const float* ci = l.cinert + 10 * b;
-    st6(l.cfrc + 6 * b, inert_mul(ci, acc) + cross_force(v, inert_mul(ci, v)));
-  }
-  KS_SYNC();
-  for (int idx = lane; idx < m.nb * 6; idx += 64) {
-    const int b = idx / 6, k = idx - 6 * b;
-    float s = 0.f;
-    if (b > 0) {
-      const int e = m.body_subtree_end[b];
-      for (int c = b; c < e; ++c) s += l.cfrc[6 * c + k];
-    }
-    l.fsub[idx] = s;
-  }
-  KS_SYNC();
-}
-
-// ------------------------------------------------------------------------------------------- dense linear algebra in LDS
-// In-place Cholesky of the lower triangle of A (row stride nvs): lane i owns row i.
-__device__ inline void cholesky_inplace(float* A, int n, int nvs, int lane) {
-  for (int j = 0; j < n; ++j) {
-    float s = 0.f;
-    if (lane >= j && lane < n) {
-      const float* ri = A + lane * nvs;
-      const float* rj = A + j * nvs;
-      s = ri[j];
-      for (int k = 0; k < j; ++k) s -= ri[k] * rj[k];
-    }
-    const float piv = lane_bcast(s, j);
-    const float d = sqrtf(fmaxf(piv, 1e-30f));
-    const float inv = 1.0f / d;
-    if (lane == j) A[j * nvs + j] = d;
-    else if (lane > j && lane < n) A[lane * nvs + j] = s * inv;
-    KS_SYNC();
+// 32 consecutive floats from a 16-byte aligned LDS address, the same address in every lane (broadcast)
+__device__ __forceinline__ void load32(const float* p, float (&v)[NP]) {
+  const float4* q = reinterpret_cast<const float4*>(p);
+#pragma unroll
+  for (int k = 0; k < NP / 4; ++k) {
+    const float4 t = q[k];
+    v[4 * k] = t.x; v[4 * k + 1] = t.y; v[4 * k + 2] = t.z; v[4 * k + 3] = t.w;
   }
 }
 
-// x = (L L^T)^-1 b with lane i holding b_i / x_i in a register
-__device__ inline float cholesky_solve(const float* L, int n, int nvs, int lane, float b) {
+__device__ __forceinline__ float rsqrt_refined(float x) {
+  float y = __builtin_amdgcn_rsqf(x);
+  y = y * (1.5f - 0.5f * x * y * y);  // one Newton step: full fp32 accuracy
+  return y;
+}
+
+// In-register Cholesky: lane i holds row i of the symmetric matrix in R[0..n); on return R holds row i of L
+// (zeros above the diagonal) and invd[j] = 1 / L[j][j] (wave-uniform).  Row k of L is fetched from lane k
+// with v_readlane, so there is no LDS traffic and no barrier.
+__device__ __forceinline__ void chol_regs(float (&R)[NP], float (&invd)[NP], int n, int lane) {
+#pragma unroll
+  for (int j = 0; j < NP; ++j) {
+    if (j < n) {
+      float s = R[j];
+#pragma unroll
+      for (int k = 0; k < j; ++k) s -= R[k] * lane_bcast(R[k], j);
+      const float piv = fmaxf(lane_bcast(s, j), 1e-30f);
+      const float inv = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, rsqrt_refined(piv))));
+      invd[j] = inv;
+      R[j] = lane > j ? s * inv : (lane == j ? piv * inv : 0.f);
+    }
+  }
+}
+
+// x = (L L^T)^-1 b, lane i holding b_i and returning x_i
+__device__ __forceinline__ float solve_regs(const float (&R)[NP], const float (&invd)[NP], int n, int lane, float b) {
   float r = b;
-  for (int j = 0; j < n; ++j) {
-    const float xj = lane_bcast(r, j) / L[j * nvs + j];
-    if (lane == j) r = xj;
-    else if (lane > j && lane < n) r -= L[lane * nvs + j] * xj;
+#pragma unroll
+  for (int j = 0; j < NP; ++j) {
+    if (j < n) {
+      const float xj = lane_bcast(r, j) * invd[j];
+      r = lane == j ? xj : r - R[j] * xj;  // R[j] is zero in lanes < j and >= n
+    }
   }
-  for (int j = n - 1; j >= 0; --j) {
-    const float xj = lane_bcast(r, j) / L[j * nvs + j];
-    if (lane == j) r = xj;
-    else if (lane < j) r -= L[j * nvs + lane] * xj;
+#pragma unroll
+  for (int j = NP - 1; j >= 0; --j) {
+    if (j < n) {
+      const float s = wave_sum(lane > j ? R[j] * r : 0.f);
+      if (lane == j) r = (r - s) * invd[j];
+    }
   }
   return r;
+}
+
+
+// dot product of an LDS row (per-lane address, odd stride between lanes) with a broadcast register vector
+__device__ __forceinline__ float row_dot(const float* row, int n, const float (&vv)[NP]) {
+  float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+  for (int j = 0; j < NP; j += 2) {
+    if (j < n) s0 += row[j] * vv[j];
+    if (j + 1 < n) s1 += row[j + 1] * vv[j + 1];
+  }
+  return s0 + s1;
+}
+
+// Row r of the constraint Jacobian (LDS, 16-byte aligned rows) times a vector in LDS.  Lane r starts at column
+// r mod n and walks cyclically, which spreads the lanes over the LDS banks although the row stride is a multiple of 4.
+__device__ __forceinline__ float jrow_dot(const float* row, int n, const float* v, int lane) {
+  int c = lane;
+  while (c >= n) c -= n;
+  float s0 = 0.f, s1 = 0.f;
+  for (int j = 0; j + 1 < n; j += 2) {
+    const int c1 = c + 1 == n ? 0 : c + 1;
+    s0 += row[c] * v[c];
+    s1 += row[c1] * v[c1];
+    c = c1 + 1 == n ? 0 : c1 + 1;
+  }
+  if (n & 1) s0 += row[c] * v[c];
+  return s0 + s1;
 }
 
 struct LsPoint {
@@ -295,29 +175,45 @@ __device__ __forceinline__ bool in_bracket(const LsPoint& x, const LsPoint& y) {
   return ((x.d0 < y.d0) && (y.d0 < 0.f)) || ((x.d0 > y.d0) && (y.d0 > 0.f));
 }
 
+// sum of one component over a contiguous subtree range of an array with `w` floats per body
+__device__ __forceinline__ float range_sum(const float* base, int w, int b, int e) {
+  float s0 = 0.f, s1 = 0.f;
+  int c = b;
+  for (; c + 1 < e; c += 2) {
+    s0 += base[w * c];
+    s1 += base[w * (c + 1)];
+  }
+  if (c < e) s0 += base[w * c];
+  return s0 + s1;
+}
+
 // ------------------------------------------------------------------------------------------- the fused kernel
 // FWD = true is the forward-only variant (derived fields + warm start of a given state, no actuation, no
 // integration) that replaces the mjx.forward of a reset.
 template <bool FWD>
 __global__ __launch_bounds__(64) void step_kernel(StepArgs a) {
-  extern __shared__ float lds_raw[];
+  extern __shared__ __attribute__((aligned(16))) float lds_raw[];
   const DevModel& m = *a.model;
   const int lane = threadIdx.x;
   const int64_t env = blockIdx.x;
   if (a.env_mask && !a.env_mask[env]) return;  // wave-uniform
-  const int nb = m.nb, nq = m.nq, nv = m.nv, nu = m.nu, ns = m.ns, nvs = m.nvs;
+  const int nb = m.nb, nq = m.nq, nv = m.nv, nu = m.nu, ns = m.ns, nvs = m.nvs, js = m.js;
   const Lds l = carve(lds_raw, m);
   const int rq = (nb > 1 && m.body_jtype[1] == kJntFree) ? 7 : 0;
   const int rv = rq ? 6 : 0;
 
   for (int i = lane; i < nq; i += 64) l.qpos[i] = a.qpos[env * nq + i];
-  for (int i = lane; i < nv; i += 64) {
-    l.qvel[i] = a.qvel[env * nv + i];
-    l.warm[i] = a.qacc_warmstart ? a.qacc_warmstart[env * nv + i] : 0.f;
-  }
+  if (lane < 32) l.qvel[lane] = lane < nv ? a.qvel[env * nv + lane] : 0.f;
+  if (lane < nv) l.warm[lane] = a.qacc_warmstart ? a.qacc_warmstart[env * nv + lane] : 0.f;
   for (int i = lane; i < nu; i += 64) l.tau[i] = a.ctrl_in ? a.ctrl_in[env * nu + i] : 0.f;
+  for (int i = lane; i < nb; i += 64) l.sub_end[i] = m.body_subtree_end[i];
+  if (lane == 0) {  // world body
+    for (int k = 0; k < 3; ++k) { l.xpos[k] = 0.f; l.xanchor[k] = 0.f; l.xaxis[k] = 0.f; }
+    l.xquat[0] = 1.f; l.xquat[1] = l.xquat[2] = l.xquat[3] = 0.f;
+    for (int k = 0; k < 9; ++k) l.xmat[k] = (k % 4 == 0) ? 1.f : 0.f;
+    for (int k = 0; k < 6; ++k) l.cvel[k] = 0.f;
+  }
   const float mu = a.friction ? a.friction[env] : m.friction;
-  const float* mass_scale = a.mass_scale ? a.mass_scale + env * nb : nullptr;
   float time = a.time ? a.time[env] : 0.f;
   const float latency = a.latency ? a.latency[env] : 0.f;
   const float kp_scale = a.kp_scale ? a.kp_scale[env] : 1.f;
@@ -326,85 +222,275 @@ __global__ __launch_bounds__(64) void step_kernel(StepArgs a) {
   const float scale = 1.0f / (m.meaninertia * (float)(nv > 1 ? nv : 1));
   int niter_out = 0, nefc_out = 0;
   float my_qacc = 0.f;
+  // actuator inputs of this control step (lane = actuator), read once
+  float u_last = 0.f, u_act = 0.f, u_kp = 0.f, u_kd = 0.f, u_lim = 0.f, u_zero = 0.f, u_abias = 0.f, u_tbias = 0.f;
+  bool u_drop = false;
+  if (!FWD && lane < nu) {
+    const int64_t eu = env * nu + lane;
+    u_last = a.last_ctrl[eu];
+    u_act = a.action[eu];
+    u_drop = a.drop && a.drop[eu];
+    u_zero = a.zero_offset ? a.zero_offset[eu] : 0.f;
+    if (a.actuator_type == KS_ACT_POSITION) {
+      u_kp = a.kp[lane] * kp_scale;
+      u_kd = a.kd[lane] * kd_scale;
+      u_lim = a.ctrl_clip[lane] * lim_scale;
+      u_abias = a.action_bias ? a.action_bias[eu] : 0.f;
+      u_tbias = a.torque_bias ? a.torque_bias[eu] : 0.f;
+    }
+  }
   KS_SYNC();
+#ifdef KS_PROFILE
+  float prof[16];
+  for (int k = 0; k < 16; ++k) prof[k] = 0.f;
+  long long t_last = clock64();
+#endif
 
   const int nsub = FWD ? 1 : a.substeps;
   for (int sub = 0; sub < nsub; ++sub) {
+    // The lane id is re-materialised per substep so that per-lane LDS addresses are recomputed inside the loop
+    // instead of being hoisted out of it into ~130 long-lived registers (which would halve the occupancy).
+    int lane_v = threadIdx.x;
+    asm volatile("" : "+v"(lane_v));
+    const int lane = lane_v;
+      // ---- per-lane model constants: re-read every substep (they hit the vector L1) so that they do not stay live
+      // across the solver, whose register rows set the occupancy
+    const bool is_body = lane > 0 && lane < nb;
+    const int bl = is_body ? lane : 0;
+    const int b_parent = m.body_parent[bl], b_jtype = m.body_jtype[bl], b_qadr = m.body_qadr[bl],
+              b_dofadr = m.body_dofadr[bl], b_depth = is_body ? m.body_depth[bl] : -1;
+    const V3 b_pos = ld3(m.body_pos[bl]), b_ipos = ld3(m.body_ipos[bl]), b_inertia = ld3(m.body_inertia[bl]),
+             b_jaxis = ld3(m.jnt_axis[bl]), b_jpos = ld3(m.jnt_pos[bl]);
+    const Quat b_quat = {m.body_quat[bl][0], m.body_quat[bl][1], m.body_quat[bl][2], m.body_quat[bl][3]};
+    const Quat b_iquat = {m.body_iquat[bl][0], m.body_iquat[bl][1], m.body_iquat[bl][2], m.body_iquat[bl][3]};
+    const float b_q0 = (is_body && b_jtype == kJntHinge) ? m.qpos0[b_qadr] : 0.f;
+    const float b_mass = is_body ? m.body_mass[bl] * (a.mass_scale ? a.mass_scale[env * nb + bl] : 1.f) : 0.f;
+    const bool is_dof = lane < nv;
+    const int dl = is_dof ? lane : 0;
+    const int d_body = m.dof_body[dl], d_act = is_dof ? m.dof_act[dl] : -1;
+    const int d_jtype = m.body_jtype[d_body], d_k = dl - m.body_dofadr[d_body];
+    const float d_damping = m.dof_damping[dl], d_armature = m.dof_armature[dl];
+    const int ua = d_act >= 0 ? d_act : 0;
+    const float d_gear = m.act_gear[ua], d_lo = m.act_lo[ua], d_hi = m.act_hi[ua];
+    const bool is_sph = lane < ns;
+    const int sl = is_sph ? lane : 0;
+    const int s_body = m.sph_body[sl];
+    const V3 s_pos = ld3(m.sph_pos[sl]);
+    const float s_rad = m.sph_radius[sl], s_invw = m.body_invweight0[s_body];
+    const unsigned s_mask = m.body_dofmask[s_body];
+    int pk[kMaxPairs / 64 + 1];
+  #pragma unroll
+    for (int k = 0; k < kMaxPairs / 64 + 1; ++k) {
+      const int p = lane + 64 * k;
+      pk[k] = p < m.npairs ? ((int)m.pair_i[p] << 8) | (int)m.pair_j[p] : -1;
+    }
+
     // ---- actuators (ksim/engine.py:287-320, ksim/actuators.py:198-217)
     if (!FWD && (sub % a.actuator_period) == 0 && lane < nu) {
       const int u = lane;
-      const int64_t eu = env * nu + u;
       float prct = (float)sub - latency;
       prct = fminf(fmaxf(prct, 0.f), 1.f);
-      const float last = a.last_ctrl[eu], act = a.action[eu];
-      const bool drop = a.drop && a.drop[eu];
-      const float c = drop ? last : last * (1.0f - prct) + act * prct;
+      const float c = u_drop ? u_last : u_last * (1.0f - prct) + u_act * prct;
       const int64_t su = ((int64_t)sub * a.N + env) * nu + u;
       float t;
       if (a.actuator_type == KS_ACT_TORQUE) {
         t = c + (a.torque_noise ? a.torque_noise[su] : 0.f);
       } else {
-        const float target = c * a.action_scale + (a.action_noise ? a.action_noise[su] : 0.f) +
-                             (a.action_bias ? a.action_bias[eu] : 0.f);
-        const float q = l.qpos[rq + u] - (a.zero_offset ? a.zero_offset[eu] : 0.f);
-        t = (a.kp[u] * kp_scale) * (target - q) + (a.kd[u] * kd_scale) * (0.f - l.qvel[rv + u]);
-        t = t + (a.torque_noise ? a.torque_noise[su] : 0.f) + (a.torque_bias ? a.torque_bias[eu] : 0.f);
-        const float lim = a.ctrl_clip[u] * lim_scale;
-        t = fminf(fmaxf(t, -lim), lim);
+        const float target = c * a.action_scale + (a.action_noise ? a.action_noise[su] : 0.f) + u_abias;
+        const float q = l.qpos[rq + u] - u_zero;
+        t = u_kp * (target - q) + u_kd * (0.f - l.qvel[rv + u]);
+        t = t + (a.torque_noise ? a.torque_noise[su] : 0.f) + u_tbias;
+        t = fminf(fmaxf(t, -u_lim), u_lim);
       }
       l.tau[u] = t;
     }
-    KS_SYNC();
 
-    // ---- position and velocity stages
-    kinematics(m, l, lane);
-    const V3 com = com_pos(m, l, lane, mass_scale);
-    crb_mass_matrix(m, l, lane);
-    velocity_and_bias(m, l, lane);
-
-    // smooth forces: passive - bias + actuator
-    float qfs = 0.f, my_qvel = 0.f;
-    if (lane < nv) {
-      const int j = lane;
-      my_qvel = l.qvel[j];
-      const float bias = dot(ld6(l.cdof + 6 * j), ld6(l.fsub + 6 * m.dof_body[j]));
-      float f = -m.dof_damping[j] * my_qvel - bias;
-      const int u = m.dof_act[j];
-      if (u >= 0) {
-        const float c = fminf(fmaxf(l.tau[u], m.act_lo[u]), m.act_hi[u]);
-        f += m.act_gear[u] * c;
+    KS_TICK(0)
+    // ---- kinematics, one tree level per pass (parents are complete before their children read them)
+    V3 xipos = {0.f, 0.f, 0.f};
+    Mat3 ximat;
+#pragma unroll
+    for (int k = 0; k < 9; ++k) ximat.m[k] = 0.f;
+    float hs = 0.f, hc = 1.f;
+    if (is_body && b_jtype == kJntHinge) sincosf(0.5f * (l.qpos[b_qadr] - b_q0), &hs, &hc);
+    for (int lev = 1; lev <= m.max_depth; ++lev) {
+      if (b_depth == lev) {
+        const int b = lane;
+        V3 pos, anchor, axis = {0.f, 0.f, 1.f};
+        Quat quat;
+        if (b_jtype == kJntFree) {
+          pos = ld3(l.qpos + b_qadr);
+          quat = qnormalize({l.qpos[b_qadr + 3], l.qpos[b_qadr + 4], l.qpos[b_qadr + 5], l.qpos[b_qadr + 6]});
+          anchor = pos;
+        } else {
+          const Quat pq = {l.xquat[4 * b_parent], l.xquat[4 * b_parent + 1], l.xquat[4 * b_parent + 2],
+                           l.xquat[4 * b_parent + 3]};
+          pos = ld3(l.xpos + 3 * b_parent) + mul(q2mat(pq), b_pos);
+          Quat nq_ = qmul(pq, b_quat);
+          anchor = pos;
+          if (b_jtype == kJntHinge) {
+            const Mat3 Rn = q2mat(nq_);
+            anchor = pos + mul(Rn, b_jpos);
+            axis = mul(Rn, b_jaxis);
+            nq_ = qmul(nq_, {hc, b_jaxis.x * hs, b_jaxis.y * hs, b_jaxis.z * hs});
+            pos = anchor - mul(q2mat(nq_), b_jpos);
+          }
+          quat = qnormalize(nq_);
+        }
+        const Mat3 R = q2mat(quat);
+        st3(l.xpos + 3 * b, pos);
+        l.xquat[4 * b] = quat.w; l.xquat[4 * b + 1] = quat.x; l.xquat[4 * b + 2] = quat.y; l.xquat[4 * b + 3] = quat.z;
+#pragma unroll
+        for (int k = 0; k < 9; ++k) l.xmat[9 * b + k] = R.m[k];
+        st3(l.xanchor + 3 * b, anchor);
+        st3(l.xaxis + 3 * b, axis);
+        xipos = pos + mul(R, b_ipos);
+        ximat = q2mat(qnormalize(qmul(quat, b_iquat)));
       }
-      qfs = f;
-      l.qfs[j] = f;
-      if (a.dbg_bias) a.dbg_bias[env * nv + j] = bias;
+      KS_SYNC();
     }
 
+    KS_TICK(1)
+    // ---- centre of mass of the tree (wave-uniform), com-based inertias and motion axes
+    const float mt = wave_sum(b_mass);
+    const float minv = mt > 1e-15f ? 1.0f / mt : 0.f;
+    const V3 com = {wave_sum(b_mass * xipos.x) * minv, wave_sum(b_mass * xipos.y) * minv,
+                    wave_sum(b_mass * xipos.z) * minv};
+    if (lane == 0) {  // world body entries of the per-substep scratch (the scratch is reused by J later)
+      for (int k = 0; k < 10; ++k) l.cinert[k] = 0.f;
+      for (int k = 0; k < 6; ++k) { l.cfrc[k] = 0.f; l.cacc[k] = k < 3 ? 0.f : -m.gravity[k - 3]; }
+    }
+    float ci[10];
+    {
+      const float* R = ximat.m;
+      const float I0 = b_inertia.x, I1 = b_inertia.y, I2 = b_inertia.z;
+      const V3 d = xipos - com;
+      const float d2 = dot(d, d);
+      ci[0] = R[0] * I0 * R[0] + R[1] * I1 * R[1] + R[2] * I2 * R[2] + b_mass * (d2 - d.x * d.x);
+      ci[1] = R[3] * I0 * R[3] + R[4] * I1 * R[4] + R[5] * I2 * R[5] + b_mass * (d2 - d.y * d.y);
+      ci[2] = R[6] * I0 * R[6] + R[7] * I1 * R[7] + R[8] * I2 * R[8] + b_mass * (d2 - d.z * d.z);
+      ci[3] = R[0] * I0 * R[3] + R[1] * I1 * R[4] + R[2] * I2 * R[5] - b_mass * d.x * d.y;
+      ci[4] = R[0] * I0 * R[6] + R[1] * I1 * R[7] + R[2] * I2 * R[8] - b_mass * d.x * d.z;
+      ci[5] = R[3] * I0 * R[6] + R[4] * I1 * R[7] + R[5] * I2 * R[8] - b_mass * d.y * d.z;
+      ci[6] = b_mass * d.x; ci[7] = b_mass * d.y; ci[8] = b_mass * d.z;
+      ci[9] = b_mass;
+      if (is_body) {
+#pragma unroll
+        for (int k = 0; k < 10; ++k) l.cinert[10 * lane + k] = ci[k];
+      }
+    }
+    Sp my_cdof = {{0.f, 0.f, 0.f}, {0.f, 0.f, 0.f}};
+    if (is_dof) {
+      const V3 off = com - ld3(l.xanchor + 3 * d_body);
+      if (d_jtype == kJntFree) {
+        if (d_k < 3) {
+          my_cdof.l = {d_k == 0 ? 1.f : 0.f, d_k == 1 ? 1.f : 0.f, d_k == 2 ? 1.f : 0.f};
+        } else {
+          const float* R = l.xmat + 9 * d_body;
+          const V3 ax = {R[d_k - 3], R[3 + d_k - 3], R[6 + d_k - 3]};
+          my_cdof = {ax, cross(ax, off)};
+        }
+      } else {
+        const V3 ax = ld3(l.xaxis + 3 * d_body);
+        my_cdof = {ax, cross(ax, off)};
+      }
+      st6(l.cdof + 6 * lane, my_cdof);
+    }
+    KS_SYNC();
+
+    KS_TICK(2)
+    // ---- composite inertias (subtree = contiguous body range) and the mass matrix
+    for (int idx = lane; idx < nb * 10; idx += 64) {
+      const int b = idx / 10, k = idx - 10 * b;
+      l.crb[idx] = b > 0 ? range_sum(l.cinert + k, 10, b, l.sub_end[b]) : 0.f;
+    }
+    for (int idx = lane; idx < nv * nvs; idx += 64) l.M[idx] = 0.f;
+    KS_SYNC();
+    if (is_dof) st6(l.buf + 6 * lane, inert_mul(l.crb + 10 * d_body, my_cdof));
+    KS_SYNC();
+#pragma unroll
+    for (int k = 0; k < kMaxPairs / 64 + 1; ++k) {
+      if (pk[k] >= 0) {
+        const int i = pk[k] >> 8, j = pk[k] & 0xff;
+        float v = dot(ld6(l.cdof + 6 * j), ld6(l.buf + 6 * i));
+        if (i == j) v += m.dof_armature[i];
+        l.M[i * nvs + j] = v;
+        l.M[j * nvs + i] = v;
+      }
+    }
+
+    KS_TICK(3)
+    // ---- body velocities, axis derivatives, RNE forces: one tree level per pass
+    for (int lev = 1; lev <= m.max_depth; ++lev) {
+      if (b_depth == lev) {
+        Sp v = ld6(l.cvel + 6 * b_parent), acc = ld6(l.cacc + 6 * b_parent);
+        if (b_jtype == kJntFree) {
+          for (int k = 0; k < 3; ++k) v = v + ld6(l.cdof + 6 * (b_dofadr + k)) * l.qvel[b_dofadr + k];
+          Sp dv = {{0.f, 0.f, 0.f}, {0.f, 0.f, 0.f}};
+          for (int k = 3; k < 6; ++k) {
+            const Sp cd = ld6(l.cdof + 6 * (b_dofadr + k));
+            const float qd = l.qvel[b_dofadr + k];
+            acc = acc + cross_motion(v, cd) * qd;
+            dv = dv + cd * qd;
+          }
+          v = v + dv;
+        } else if (b_jtype == kJntHinge) {
+          const Sp cd = ld6(l.cdof + 6 * b_dofadr);
+          const float qd = l.qvel[b_dofadr];
+          acc = acc + cross_motion(v, cd) * qd;
+          v = v + cd * qd;
+        }
+        st6(l.cvel + 6 * lane, v);
+        st6(l.cacc + 6 * lane, acc);
+        st6(l.cfrc + 6 * lane, inert_mul(ci, acc) + cross_force(v, inert_mul(ci, v)));
+      }
+      KS_SYNC();
+    }
+    for (int idx = lane; idx < nb * 6; idx += 64) {
+      const int b = idx / 6, k = idx - 6 * b;
+      l.fsub[idx] = b > 0 ? range_sum(l.cfrc + k, 6, b, l.sub_end[b]) : 0.f;
+    }
+    KS_SYNC();
+
+    KS_TICK(4)
+    // ---- mass-matrix row into registers; smooth forces: passive - bias + actuator
+    const float* Mrow = l.M + (is_dof ? lane : 0) * nvs;  // row stride is odd: conflict-free across lanes
+    float qfs = 0.f, my_qvel = 0.f;
+    if (is_dof) {
+      my_qvel = l.qvel[lane];
+      const float bias = dot(my_cdof, ld6(l.fsub + 6 * d_body));
+      float f = -d_damping * my_qvel - bias;
+      if (d_act >= 0) f += d_gear * fminf(fmaxf(l.tau[d_act], d_lo), d_hi);
+      qfs = f;
+      if (a.dbg_bias) a.dbg_bias[env * nv + lane] = bias;
+#ifndef KS_PROFILE
+      if (a.dbg_M) for (int j = 0; j < nv; ++j) a.dbg_M[env * nv * nv + lane * nv + j] = l.M[lane * nvs + j];
+#endif
+    }
+
+    KS_TICK(5)
     // ---- contacts: sphere vs plane z = 0, compacted to the penetrating ones
     float dist = 1.f;
     V3 cpos = {0.f, 0.f, 0.f};
-    if (lane < ns) {
-      const int b = m.sph_body[lane];
-      const float* R = l.xmat + 9 * b;
-      const V3 lp = ld3(m.sph_pos[lane]);
-      const V3 c = ld3(l.xpos + 3 * b) + V3{R[0] * lp.x + R[1] * lp.y + R[2] * lp.z,
-                                           R[3] * lp.x + R[4] * lp.y + R[5] * lp.z,
-                                           R[6] * lp.x + R[7] * lp.y + R[8] * lp.z};
-      const float r = m.sph_radius[lane];
-      dist = c.z - r;
-      cpos = {c.x, c.y, c.z - r - 0.5f * dist};
+    if (is_sph) {
+      const float* R = l.xmat + 9 * s_body;
+      const V3 c = ld3(l.xpos + 3 * s_body) + V3{R[0] * s_pos.x + R[1] * s_pos.y + R[2] * s_pos.z,
+                                                R[3] * s_pos.x + R[4] * s_pos.y + R[5] * s_pos.z,
+                                                R[6] * s_pos.x + R[7] * s_pos.y + R[8] * s_pos.z};
+      dist = c.z - s_rad;
+      cpos = {c.x, c.y, c.z - s_rad - 0.5f * dist};
       if (a.dbg_con_dist) a.dbg_con_dist[env * ns + lane] = dist;
     }
-    const bool touching = (lane < ns) && (dist < 0.f);
+    const bool touching = is_sph && (dist < 0.f);
     const unsigned long long cmask = __ballot(touching);
     const int ncon = __popcll(cmask);
     const int nefc = 4 * ncon;
     if (touching) {
       const int c = __popcll(cmask & ((1ull << lane) - 1ull));
-      const int b = m.sph_body[lane];
-      l.con_body[c] = b;
+      l.con_body[c] = s_body;
+      l.con_mask[c] = s_mask;
       st3(l.con_off + 3 * c, cpos - com);
-      const float t = m.body_invweight0[b];
-      const float invweight = (t + mu * mu * t) * 2.f * mu * mu / m.impratio;
+      const float invweight = (s_invw + mu * mu * s_invw) * 2.f * mu * mu / m.impratio;
       const float ix = fabsf(dist) / m.width;
       const float ia = (1.0f / powf(m.mid, m.power - 1.f)) * powf(ix, m.power);
       const float ib = 1.f - (1.0f / powf(1.f - m.mid, m.power - 1.f)) * powf(1.f - ix, m.power);
@@ -412,126 +498,158 @@ __global__ __launch_bounds__(64) void step_kernel(StepArgs a) {
       float imp = m.dmin + iy * (m.dmax - m.dmin);
       imp = fminf(fmaxf(imp, m.dmin), m.dmax);
       if (ix > 1.f) imp = m.dmax;
-      float Rr = invweight * (1.f - imp) / imp;
-      Rr = fmaxf(Rr, 1e-15f);
+      const float Rr = fmaxf(invweight * (1.f - imp) / imp, 1e-15f);
       l.con_D[c] = 1.0f / Rr;
       l.con_kip[c] = m.con_k * imp * dist;
     }
     KS_SYNC();
-    for (int idx = lane; idx < nefc * nv; idx += 64) {
-      const int r = idx / nv, j = idx - r * nv;
-      const int c = r >> 2, q = r & 3;
-      const int b = l.con_body[c];
-      float val = 0.f;
-      if ((m.body_dofmask[b] >> j) & 1u) {
-        const Sp cd = ld6(l.cdof + 6 * j);
-        const V3 jac = cd.l + cross(cd.a, ld3(l.con_off + 3 * c));
-        const float tang = (q < 2) ? jac.y : -jac.x;
-        val = jac.z + ((q & 1) ? -mu : mu) * tang;
-      }
-      l.J[r * nvs + j] = val;
-    }
-    // ---- factor M (into H) and the unconstrained acceleration
-    for (int idx = lane; idx < nv * nvs; idx += 64) l.H[idx] = l.M[idx];
-    if (a.dbg_M) for (int idx = lane; idx < nv * nv; idx += 64) a.dbg_M[env * nv * nv + idx] = l.M[(idx / nv) * nvs + idx % nv];
-    KS_SYNC();
-    cholesky_inplace(l.H, nv, nvs, lane);
-    const float qas = cholesky_solve(l.H, nv, nvs, lane, qfs);
-    if (a.dbg_qacc_smooth && lane < nv) a.dbg_qacc_smooth[env * nv + lane] = qas;
 
-    // ---- constraint rows: reference acceleration and regulariser (lane = row)
-    float aref = 0.f, D = 0.f;
-    if (lane < nefc) {
-      const float* Jr = l.J + lane * nvs;
-      float vel = 0.f;
-      for (int j = 0; j < nv; ++j) vel += Jr[j] * l.qvel[j];
-      aref = -m.con_b * vel - l.con_kip[lane >> 2];
-      D = l.con_D[lane >> 2];
-    }
+    KS_TICK(6)
+    // ---- Cholesky of M and the unconstrained acceleration (registers only)
+    float R[NP], invd[NP];
+#pragma unroll
+    for (int j = 0; j < NP; ++j) { R[j] = (is_dof && j < nv) ? Mrow[j] : 0.f; invd[j] = 0.f; }
+    chol_regs(R, invd, nv, lane);
+    const float qas = solve_regs(R, invd, nv, lane, qfs);
+    if (a.dbg_qacc_smooth && is_dof) a.dbg_qacc_smooth[env * nv + lane] = qas;
 
-    // ---- Newton solver (wave-uniform control flow)
+    KS_TICK(7)
     float qacc = qas;
     int niter = 0;
     if (nefc > 0) {
-      const float warm = (lane < nv) ? l.warm[lane] : 0.f;
-      // cost of the warm start and of the unconstrained acceleration
+      // ---- constraint rows: lane r builds row r of J in registers and mirrors it to LDS for column access
+      const bool is_row = lane < nefc;
+      float aref = 0.f, D = 0.f;
+      {
+        const int c = is_row ? lane >> 2 : 0, q = lane & 3;
+        const unsigned cm = is_row ? l.con_mask[c] : 0u;
+        const V3 off = ld3(l.con_off + 3 * c);
+        const float smu = (q & 1) ? -mu : mu;
+        unsigned um = 0;  // union of the dof masks of the active contacts (wave-uniform)
+        for (int k = 0; k < ncon; ++k) um |= l.con_mask[k];
+        float vv[NP];
+        load32(l.qvel, vv);
+        float vel = 0.f;
+#pragma unroll
+        for (int j = 0; j < NP; ++j) {
+          float val = 0.f;
+          if (j < nv && ((um >> j) & 1u)) {
+            const Sp cd = ld6(l.cdof + 6 * j);
+            const V3 jac = cd.l + cross(cd.a, off);
+            const float tang = (q < 2) ? jac.y : -jac.x;
+            val = ((cm >> j) & 1u) ? jac.z + smu * tang : 0.f;
+          }
+          vel += val * vv[j];
+          if (is_row && j < nv) l.J[lane * js + j] = val;
+        }
+        if (is_row) {
+          aref = -m.con_b * vel - l.con_kip[c];
+          D = l.con_D[c];
+        }
+      }
+      const float warm = is_dof ? l.warm[lane] : 0.f;
+      KS_SYNC();
+      KS_TICK(8)
+
+      // cost of the warm start and of the unconstrained acceleration; start from the cheaper one
       float Ma_w = 0.f, Ma_s = 0.f, Jar_w = 0.f, Jar_s = 0.f;
-      KS_SYNC();
-      if (lane < nv) l.vbuf[lane] = warm;
-      KS_SYNC();
-      if (lane < nv) { const float* Mr = l.M + lane * nvs; for (int j = 0; j < nv; ++j) Ma_w += Mr[j] * l.vbuf[j]; }
-      if (lane < nefc) { const float* Jr = l.J + lane * nvs; for (int j = 0; j < nv; ++j) Jar_w += Jr[j] * l.vbuf[j]; Jar_w -= aref; }
-      KS_SYNC();
-      if (lane < nv) l.vbuf[lane] = qas;
-      KS_SYNC();
-      if (lane < nv) { const float* Mr = l.M + lane * nvs; for (int j = 0; j < nv; ++j) Ma_s += Mr[j] * l.vbuf[j]; }
-      if (lane < nefc) { const float* Jr = l.J + lane * nvs; for (int j = 0; j < nv; ++j) Jar_s += Jr[j] * l.vbuf[j]; Jar_s -= aref; }
-      const float cost_w = wave_sum((lane < nefc && Jar_w < 0.f) ? 0.5f * D * Jar_w * Jar_w : 0.f) +
-                           0.5f * wave_sum((lane < nv) ? (Ma_w - qfs) * (warm - qas) : 0.f);
-      const float cost_s = wave_sum((lane < nefc && Jar_s < 0.f) ? 0.5f * D * Jar_s * Jar_s : 0.f) +
-                           0.5f * wave_sum((lane < nv) ? (Ma_s - qfs) * (qas - qas) : 0.f);
+      {
+        float vv[NP];
+        if (lane < 32) l.vbuf[lane] = warm;
+        KS_SYNC();
+        load32(l.vbuf, vv);
+        if (is_dof) Ma_w = row_dot(Mrow, nv, vv);
+        if (is_row) Jar_w = jrow_dot(l.J + lane * js, nv, l.vbuf, lane) - aref;
+        KS_SYNC();
+        if (lane < 32) l.vbuf[lane] = qas;
+        KS_SYNC();
+        load32(l.vbuf, vv);
+        if (is_dof) Ma_s = row_dot(Mrow, nv, vv);
+        if (is_row) Jar_s = jrow_dot(l.J + lane * js, nv, l.vbuf, lane) - aref;
+      }
+      const float cost_w = wave_sum((is_row && Jar_w < 0.f) ? 0.5f * D * Jar_w * Jar_w : 0.f) +
+                           0.5f * wave_sum(is_dof ? (Ma_w - qfs) * (warm - qas) : 0.f);
+      const float cost_s = wave_sum((is_row && Jar_s < 0.f) ? 0.5f * D * Jar_s * Jar_s : 0.f);
       const bool use_warm = cost_w < cost_s;
       qacc = use_warm ? warm : qas;
       float Ma = use_warm ? Ma_w : Ma_s;
       float Jaref = use_warm ? Jar_w : Jar_s;
       float cost = use_warm ? cost_w : cost_s;
       float prev_cost = INFINITY;
-      float gauss = 0.f, grad = 0.f, search = 0.f, qfc = 0.f;
-      bool active = false;
+      bool first = true;
+      KS_TICK(9)
 
-      auto update_constraint_and_gradient = [&](bool first) {
-        active = (lane < nefc) && (Jaref < 0.f);
+      while (true) {
+        // ---- constraint update: active set, forces, cost
+        const bool active = is_row && (Jaref < 0.f);
         const float force = active ? -D * Jaref : 0.f;
-        KS_SYNC();
-        if (lane < nefc) { l.fbuf[lane] = force; l.wbuf[lane] = active ? D : 0.f; }
-        KS_SYNC();
-        qfc = 0.f;
-        if (lane < nv) for (int r = 0; r < nefc; ++r) qfc += l.J[r * nvs + lane] * l.fbuf[r];
-        gauss = 0.5f * wave_sum((lane < nv) ? (Ma - qfs) * (qacc - qas) : 0.f);
+        unsigned long long am = __ballot(active);
+        float qfc = 0.f;
+        for (unsigned long long t = am; t; t &= t - 1) {
+          const int r = __builtin_ctzll(t);
+          qfc += l.J[r * js + (lane < nv ? lane : 0)] * lane_bcast(force, r);
+        }
+        if (!is_dof) qfc = 0.f;
+        const float gauss = 0.5f * wave_sum(is_dof ? (Ma - qfs) * (qacc - qas) : 0.f);
         if (!first) {
           prev_cost = cost;
           cost = wave_sum(active ? 0.5f * D * Jaref * Jaref : 0.f) + gauss;
         }
-        grad = (lane < nv) ? Ma - qfs - qfc : 0.f;
-        // H = M + J^T diag(D active) J  (lower triangle), then factor and solve
-        for (int idx = lane; idx < nv * nv; idx += 64) {
-          const int i = idx / nv, j = idx - i * nv;
-          if (j <= i) {
-            float h = l.M[i * nvs + j];
-            for (int r = 0; r < nefc; ++r) h += l.wbuf[r] * l.J[r * nvs + i] * l.J[r * nvs + j];
-            l.H[i * nvs + j] = h;
-          }
-        }
-        KS_SYNC();
-        cholesky_inplace(l.H, nv, nvs, lane);
-        const float mgrad = cholesky_solve(l.H, nv, nvs, lane, grad);
-        search = -mgrad;
-      };
-      update_constraint_and_gradient(true);
-
-      while (true) {
+        first = false;
+        // ---- gradient; stop before paying for another Hessian when the solver is done
+        const float grad = is_dof ? Ma - qfs - qfc : 0.f;
         const float improvement = scale * (prev_cost - cost);
         const float gradient = scale * sqrtf(wave_sum(grad * grad));
         bool done = niter >= m.iterations;
         done |= improvement < m.tolerance;
         done |= gradient < m.tolerance;
         if (done && !(m.iterations == 1 && niter == 0)) break;
+        KS_TICK(10)
+        // ---- Newton direction: H = M + J^T diag(D active) J, row per lane, in registers
+#pragma unroll
+        for (int j = 0; j < NP; ++j) R[j] = (is_dof && j < nv) ? Mrow[j] : 0.f;
+        {
+          unsigned long long t = am;
+          while (t) {  // two constraint rows per pass so that the LDS loads of one overlap the FMAs of the other
+            const int r0 = __builtin_ctzll(t);
+            t &= t - 1;
+            const bool two = t != 0;
+            const int r1 = two ? __builtin_ctzll(t) : r0;
+            if (two) t &= t - 1;
+            const float c0 = is_dof ? lane_bcast(D, r0) * l.J[r0 * js + lane] : 0.f;
+            const float c1 = (is_dof && two) ? lane_bcast(D, r1) * l.J[r1 * js + lane] : 0.f;
+            float j0[NP], j1[NP];
+            load32(l.J + r0 * js, j0);
+            load32(l.J + r1 * js, j1);
+#pragma unroll
+            for (int j = 0; j < NP; ++j)
+              if (j < nv) R[j] += c0 * j0[j] + c1 * j1[j];
+          }
+        }
+        KS_TICK(11)
+        chol_regs(R, invd, nv, lane);
+        const float search = -solve_regs(R, invd, nv, lane, grad);
+        KS_TICK(12)
 
         // ---- exact line search along `search`
-        KS_SYNC();
-        if (lane < nv) l.vbuf[lane] = search;
-        KS_SYNC();
         float mv = 0.f, jv = 0.f;
-        if (lane < nv) { const float* Mr = l.M + lane * nvs; for (int j = 0; j < nv; ++j) mv += Mr[j] * l.vbuf[j]; }
-        if (lane < nefc) { const float* Jr = l.J + lane * nvs; for (int j = 0; j < nv; ++j) jv += Jr[j] * l.vbuf[j]; }
+        {
+          float vv[NP];
+          KS_SYNC();
+          if (lane < 32) l.vbuf[lane] = search;
+          KS_SYNC();
+          load32(l.vbuf, vv);
+          if (is_dof) mv = row_dot(Mrow, nv, vv);
+          if (is_row) jv = jrow_dot(l.J + lane * js, nv, l.vbuf, lane);
+        }
         const float smag = sqrtf(wave_sum(search * search)) * m.meaninertia * (float)(nv > 1 ? nv : 1);
         const float gtol = m.tolerance * m.ls_tolerance * smag;
         const float q0r = 0.5f * Jaref * Jaref * D, q1r = jv * Jaref * D, q2r = 0.5f * jv * jv * D;
         const float g0 = gauss;
-        const float g1 = wave_sum((lane < nv) ? search * (Ma - qfs) : 0.f);
-        const float g2 = 0.5f * wave_sum((lane < nv) ? search * mv : 0.f);
+        const float g1 = wave_sum(is_dof ? search * (Ma - qfs) : 0.f);
+        const float g2 = 0.5f * wave_sum(is_dof ? search * mv : 0.f);
         auto point = [&](float alpha) {
-          const bool on = (lane < nefc) && (Jaref + alpha * jv < 0.f);
+          const bool on = is_row && (Jaref + alpha * jv < 0.f);
           const float q0 = g0 + wave_sum(on ? q0r : 0.f);
           const float q1 = g1 + wave_sum(on ? q1r : 0.f);
           const float q2 = g2 + wave_sum(on ? q2r : 0.f);
@@ -574,23 +692,24 @@ __global__ __launch_bounds__(64) void step_kernel(StepArgs a) {
         qacc += alpha * search;
         Ma += alpha * mv;
         Jaref += alpha * jv;
-        update_constraint_and_gradient(false);
         ++niter;
+        KS_TICK(13)
       }
     }
     niter_out = niter;
     nefc_out = nefc;
     my_qacc = qacc;
     KS_SYNC();
-    if (lane < nv) { l.warm[lane] = qacc; l.qacc[lane] = qacc; }
+    if (is_dof) l.warm[lane] = qacc;
 
+    KS_TICK(14)
     // ---- semi-implicit Euler
     if (!FWD) {
-      if (lane < nv) l.qvel[lane] = my_qvel + m.dt * qacc;
+      if (is_dof) l.qvel[lane] = my_qvel + m.dt * qacc;
       KS_SYNC();
-      if (lane > 0 && lane < nb) {
-        const int b = lane, qa = m.body_qadr[b], da = m.body_dofadr[b];
-        if (m.body_jtype[b] == kJntFree) {
+      if (is_body) {
+        const int qa = b_qadr, da = b_dofadr;
+        if (b_jtype == kJntFree) {
           for (int k = 0; k < 3; ++k) l.qpos[qa + k] += m.dt * l.qvel[da + k];
           const V3 w = ld3(l.qvel + da + 3);
           const float n = sqrtf(dot(w, w));
@@ -601,7 +720,7 @@ __global__ __launch_bounds__(64) void step_kernel(StepArgs a) {
           }
           q = qnormalize(q);
           l.qpos[qa + 3] = q.w; l.qpos[qa + 4] = q.x; l.qpos[qa + 5] = q.y; l.qpos[qa + 6] = q.z;
-        } else if (m.body_jtype[b] == kJntHinge) {
+        } else if (b_jtype == kJntHinge) {
           l.qpos[qa] += m.dt * l.qvel[da];
         }
       }
@@ -610,14 +729,18 @@ __global__ __launch_bounds__(64) void step_kernel(StepArgs a) {
     KS_SYNC();
   }
 
+  KS_TICK(15)
+#ifdef KS_PROFILE
+  if (a.dbg_M && lane == 0) for (int k = 0; k < 16; ++k) a.dbg_M[env * nv * nv + k] = prof[k];
+#endif
   // ---- write back
   if (!FWD) {
     for (int i = lane; i < nq; i += 64) a.qpos[env * nq + i] = l.qpos[i];
-    for (int i = lane; i < nv; i += 64) a.qvel[env * nv + i] = l.qvel[i];
+    if (lane < nv) a.qvel[env * nv + lane] = l.qvel[lane];
     if (a.time && lane == 0) a.time[env] = time;
-    if (a.last_ctrl) for (int i = lane; i < nu; i += 64) a.last_ctrl[env * nu + i] = a.action[env * nu + i];
+    if (a.last_ctrl && lane < nu) a.last_ctrl[env * nu + lane] = u_act;
   }
-  if (a.qacc_warmstart) for (int i = lane; i < nv; i += 64) a.qacc_warmstart[env * nv + i] = l.warm[i];
+  if (a.qacc_warmstart && lane < nv) a.qacc_warmstart[env * nv + lane] = l.warm[lane];
   if (a.qacc && lane < nv) a.qacc[env * nv + lane] = my_qacc;
   if (a.ctrl_out) for (int i = lane; i < nu; i += 64) a.ctrl_out[env * nu + i] = l.tau[i];
   if (a.xpos) for (int i = lane; i < nb * 3; i += 64) a.xpos[env * nb * 3 + i] = l.xpos[i];
@@ -658,6 +781,7 @@ extern "C" int ks_model_create(const KsModelDesc* d, KsModel** out) {
   m.nb = d->nb; m.nq = d->nq; m.nv = d->nv; m.nu = d->nu; m.ns = d->ns;
   m.iterations = d->iterations; m.ls_iterations = d->ls_iterations; m.eulerdamp = d->eulerdamp;
   m.nvs = d->nv | 1;
+  m.js = up4(d->nv) % 32 == 0 ? up4(d->nv) + 4 : up4(d->nv);
   m.dt = (float)d->dt;
   for (int k = 0; k < 3; ++k) m.gravity[k] = (float)d->gravity[k];
   m.tolerance = (float)d->tolerance; m.ls_tolerance = (float)d->ls_tolerance;
@@ -694,6 +818,7 @@ extern "C" int ks_model_create(const KsModelDesc* d, KsModel** out) {
     for (int c = b; c > 0; c = d->body_parent[c]) chain[n++] = c;
     if (n > kMaxDepth) { delete km; return fail(KS_ELIMIT, "ks_model_create: tree deeper than %d", kMaxDepth); }
     m.body_depth[b] = n;
+    if (n > m.max_depth) m.max_depth = n;
     for (int k = 0; k < n; ++k) m.body_chain[b][k] = chain[n - 1 - k];
   }
   for (int q = 0; q < d->nq; ++q) m.qpos0[q] = (float)d->qpos0[q];
