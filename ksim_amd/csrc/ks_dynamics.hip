@@ -108,9 +108,14 @@ __device__ __forceinline__ void chol_regs(float (&R)[NP], float (&invd)[NP], int
 #pragma unroll
   for (int j = 0; j < NP; ++j) {
     if (j < n) {
-      float s = R[j];
+      float s = R[j], s2 = 0.f;  // two chains halve the dependent-FMA latency of a column
 #pragma unroll
-      for (int k = 0; k < j; ++k) s -= R[k] * lane_bcast(R[k], j);
+      for (int k = 0; k + 1 < j; k += 2) {
+        s -= R[k] * lane_bcast(R[k], j);
+        s2 -= R[k + 1] * lane_bcast(R[k + 1], j);
+      }
+      if (j & 1) s -= R[j - 1] * lane_bcast(R[j - 1], j);
+      s += s2;
       const float piv = fmaxf(lane_bcast(s, j), 1e-30f);
       const float inv = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, rsqrt_refined(piv))));
       invd[j] = inv;
@@ -129,11 +134,23 @@ __device__ __forceinline__ float solve_regs(const float (&R)[NP], const float (&
       r = lane == j ? xj : r - R[j] * xj;  // R[j] is zero in lanes < j and >= n
     }
   }
+  // Backward substitution, four columns per batch: the four cross-lane sums over the already solved rows are
+  // independent (their DPP chains interleave); the 4x4 triangle inside the batch is resolved with lane reads.
 #pragma unroll
-  for (int j = NP - 1; j >= 0; --j) {
-    if (j < n) {
-      const float s = wave_sum(lane > j ? R[j] * r : 0.f);
-      if (lane == j) r = (r - s) * invd[j];
+  for (int jb = NP - 4; jb >= 0; jb -= 4) {
+    if (jb < n) {
+      float s[4], x[4];
+#pragma unroll
+      for (int c = 0; c < 4; ++c) s[c] = wave_sum(lane > jb + 3 ? R[jb + c] * r : 0.f);
+#pragma unroll
+      for (int c = 3; c >= 0; --c) {
+        const int j = jb + c;
+        float acc = lane_bcast(r, j) - s[c];
+#pragma unroll
+        for (int d = c + 1; d < 4; ++d) acc -= lane_bcast(R[j], jb + d) * x[d];  // L[jb+d][j] lives in lane jb+d
+        x[c] = (j < n) ? acc * invd[j] : 0.f;
+        if (lane == j) r = x[c];
+      }
     }
   }
   return r;
@@ -157,6 +174,7 @@ __device__ __forceinline__ float jrow_dot(const float* row, int n, const float* 
   int c = lane;
   while (c >= n) c -= n;
   float s0 = 0.f, s1 = 0.f;
+#pragma unroll 4
   for (int j = 0; j + 1 < n; j += 2) {
     const int c1 = c + 1 == n ? 0 : c + 1;
     s0 += row[c] * v[c];
