@@ -16,12 +16,15 @@ namespace ks {
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(4))) unsigned u32x4;  // a 16-byte register vector (plain vector type, so arrays of it stay in registers)
 
-constexpr int kBM = 128, kBN = 128;
+constexpr int kBM = 128, kBN = 128;  // kBM: the largest row tile
 
-template <int ACT>
+// FAST: the result is rounded to bf16 right away, so the hardware exponential (abs. error ~1e-7 near zero) is
+// exact enough; the fp32 path keeps expm1f.
+template <int ACT, bool FAST>
 __device__ __forceinline__ float activate(float x) {
-  if (ACT == KS_ACT_ELU) return x > 0.f ? x : expm1f(x);
+  if (ACT == KS_ACT_ELU) return x > 0.f ? x : (FAST ? __expf(x) - 1.0f : expm1f(x));
   if (ACT == KS_ACT_RELU) return fmaxf(x, 0.f);
   if (ACT == KS_ACT_TANH) return tanhf(x);
   return x;
@@ -29,114 +32,165 @@ __device__ __forceinline__ float activate(float x) {
 
 __device__ __forceinline__ __bf16 to_bf16(float x) { return (__bf16)x; }
 
+
+// First layer: VEC consecutive fp32 inputs of row m starting at column k (zero beyond the real width or batch),
+// converted to T and packed into one 16-byte register vector.
+template <typename T, int VEC>
+__device__ __forceinline__ u32x4 load_first(const float* __restrict__ x, int64_t m, int64_t M, int64_t ldx, int k,
+                                            int Kreal) {
+  float f[VEC];
+  if (m < M && (ldx & 3) == 0 && k + VEC <= Kreal) {  // whole vector inside a 16-byte aligned row: wide loads
+    const float4* p4 = reinterpret_cast<const float4*>(x + m * ldx + k);
+#pragma unroll
+    for (int e = 0; e < VEC / 4; ++e) {
+      const float4 t = p4[e];
+      f[4 * e] = t.x; f[4 * e + 1] = t.y; f[4 * e + 2] = t.z; f[4 * e + 3] = t.w;
+    }
+  } else {
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) f[e] = (m < M && k + e < Kreal) ? x[m * ldx + k + e] : 0.f;
+  }
+  u32x4 out;
+  if constexpr (sizeof(T) == 2) {
+    unsigned w[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const unsigned lo = __builtin_bit_cast(unsigned short, (__bf16)f[2 * e]);
+      const unsigned hi = __builtin_bit_cast(unsigned short, (__bf16)f[2 * e + 1]);
+      w[e] = lo | (hi << 16);
+    }
+    out = u32x4{w[0], w[1], w[2], w[3]};
+  } else {
+    out = u32x4{__builtin_bit_cast(unsigned, f[0]), __builtin_bit_cast(unsigned, f[1]),
+                __builtin_bit_cast(unsigned, f[2]), __builtin_bit_cast(unsigned, f[3])};
+  }
+  return out;
+}
+
 // T = math/storage type of activations and weights (__bf16 or float).
 // FIRST: x is the caller's unpadded fp32 input (row stride ldx = in_dim).
 // LAST: y is the caller's unpadded fp32 output (row stride ldy = out_dim).
-template <typename T, bool FIRST, bool LAST, int ACT>
-__global__ __launch_bounds__(256) void mlp_layer_kernel(int64_t M, int K /*padded*/, int Kreal, int Nreal,
+// BM: rows per workgroup (128, or 64 for small batches so that the grid still covers every CU twice).
+// The K loop is software-pipelined: the global loads of slice k+1 are issued into registers before the MFMAs
+// of slice k run out of LDS, so HBM/L2 latency overlaps the matrix-core work.
+template <typename T, bool FIRST, bool LAST, int ACT, int BM, int BN, int WAVES_M, int WAVES_N>
+__global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void mlp_layer_kernel(int64_t M, int K /*padded to BK*/, int Kreal, int Nreal,
                                                         const void* __restrict__ xin, int64_t ldx,
                                                         const T* __restrict__ W /*(Np, K)*/,
                                                         const float* __restrict__ bias /*(Np)*/,
                                                         void* __restrict__ yout, int64_t ldy) {
   constexpr bool BF = sizeof(T) == 2;
-  constexpr int BK = BF ? 32 : 16;
-  constexpr int PAD = BF ? 8 : 4;  // keeps 16-byte alignment of rows and spreads LDS banks
-  __shared__ __attribute__((aligned(16))) T As[kBM][BK + PAD];
-  __shared__ __attribute__((aligned(16))) T Bs[kBN][BK + PAD];
+  constexpr int BK = BF ? 64 : 32;       // elements of K per slice
+  constexpr int PAD = BF ? 8 : 4;        // keeps 16-byte row alignment and spreads LDS banks
+  constexpr int VEC = 16 / sizeof(T);    // elements per 16-byte load
+  constexpr int NT = 64 * WAVES_M * WAVES_N;    // threads per workgroup
+  constexpr int A_VECS = BM * BK / VEC / NT;    // 16-byte loads per thread for the A slice
+  constexpr int B_VECS = BN * BK / VEC / NT;
+  constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;  // output block of one wavefront
+  constexpr int MI = WM / 32, NI = WN / 32;     // 32 x 32 MFMA tiles per wavefront
+  static_assert(A_VECS >= 1 && B_VECS >= 1 && MI >= 1 && NI >= 1, "tile too small for the workgroup");
+  extern __shared__ __attribute__((aligned(16))) unsigned char mlp_lds[];
+  T (*As)[BK + PAD] = reinterpret_cast<T (*)[BK + PAD]>(mlp_lds);
+  T (*Bs)[BK + PAD] = reinterpret_cast<T (*)[BK + PAD]>(mlp_lds + sizeof(T) * BM * (BK + PAD));
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int wm = wave >> 1, wn = wave & 1;
-  const int64_t m0 = (int64_t)blockIdx.x * kBM;
-  const int n0 = blockIdx.y * kBN;
-  f32x16 acc[2][2];
+  const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+  const int64_t m0 = (int64_t)blockIdx.x * BM;
+  const int n0 = blockIdx.y * BN;
+  f32x16 acc[MI][NI];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < MI; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < NI; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-  const int lrow = tid >> 1;               // 0..127
-  const int lcol = (tid & 1) * (BK / 2);   // each thread stages BK/2 elements of one row
+  constexpr int VPR = BK / VEC;  // 16-byte vectors per tile row
+  u32x4 ra[A_VECS], rb[B_VECS];
+  // global -> registers for the K slice starting at KS_K0 (kept as a macro so the register arrays never have
+  // their address taken)
+#define KS_FETCH(KS_K0)                                                                                        \
+  {                                                                                                            \
+    _Pragma("unroll") for (int c = 0; c < A_VECS; ++c) {                                                       \
+      const int v = tid + NT * c, row = v / VPR, col = (v % VPR) * VEC;                                        \
+      const int64_t m = m0 + row;                                                                              \
+      if constexpr (FIRST) {                                                                                   \
+        ra[c] = load_first<T, VEC>((const float*)xin, m, M, ldx, (KS_K0) + col, Kreal);                        \
+      } else {                                                                                                 \
+        ra[c] = (m < M) ? *reinterpret_cast<const u32x4*>((const T*)xin + m * ldx + (KS_K0) + col)             \
+                        : u32x4{0u, 0u, 0u, 0u};                                                              \
+      }                                                                                                        \
+    }                                                                                                          \
+    _Pragma("unroll") for (int c = 0; c < B_VECS; ++c) {                                                       \
+      const int v = tid + NT * c, row = v / VPR, col = (v % VPR) * VEC;                                        \
+      rb[c] = *reinterpret_cast<const u32x4*>(W + (int64_t)(n0 + row) * K + (KS_K0) + col);                    \
+    }                                                                                                          \
+  }
+
+  KS_FETCH(0)
   for (int k0 = 0; k0 < K; k0 += BK) {
-    // ---- stage A (activations)
-    {
-      const int64_t m = m0 + lrow;
-      T* dst = &As[lrow][lcol];
-      if (FIRST) {
-        const float* x = (const float*)xin;
 #pragma unroll
-        for (int c = 0; c < BK / 2; ++c) {
-          const int k = k0 + lcol + c;
-          const float v = (m < M && k < Kreal) ? x[m * ldx + k] : 0.f;
-          dst[c] = BF ? (T)to_bf16(v) : (T)v;
-        }
-      } else {
-        const T* x = (const T*)xin;
-        if (m < M) {
-          const uint4* src = (const uint4*)(x + m * ldx + k0 + lcol);
-#pragma unroll
-          for (int c = 0; c < (BK / 2) * (int)sizeof(T) / 16; ++c) ((uint4*)dst)[c] = src[c];
-        } else {
-#pragma unroll
-          for (int c = 0; c < (BK / 2) * (int)sizeof(T) / 16; ++c) ((uint4*)dst)[c] = make_uint4(0, 0, 0, 0);
-        }
-      }
+    for (int c = 0; c < A_VECS; ++c) {
+      const int v = tid + NT * c, row = v / VPR, col = (v % VPR) * VEC;
+      *reinterpret_cast<u32x4*>(&As[row][col]) = ra[c];
     }
-    // ---- stage B (weights, padded so no guards are needed)
-    {
-      const uint4* src = (const uint4*)(W + (int64_t)(n0 + lrow) * K + k0 + lcol);
-      uint4* dst = (uint4*)&Bs[lrow][lcol];
 #pragma unroll
-      for (int c = 0; c < (BK / 2) * (int)sizeof(T) / 16; ++c) dst[c] = src[c];
+    for (int c = 0; c < B_VECS; ++c) {
+      const int v = tid + NT * c, row = v / VPR, col = (v % VPR) * VEC;
+      *reinterpret_cast<u32x4*>(&Bs[row][col]) = rb[c];
     }
     __syncthreads();
+    // Next slice in flight while the matrix cores work on this one.  The fetch is unconditional (the last pass
+    // re-reads its own slice) so that the register arrays are plain loop-carried values.
+    const int kn = k0 + BK < K ? k0 + BK : k0;
+    KS_FETCH(kn)
     if constexpr (BF) {
 #pragma unroll
       for (int kk = 0; kk < BK; kk += 16) {
-        bf16x8 af[2], bfr[2];
+        bf16x8 af[MI], bfr[NI];
 #pragma unroll
-        for (int i = 0; i < 2; ++i) af[i] = *(const bf16x8*)&As[wm * 64 + i * 32 + (lane & 31)][kk + (lane >> 5) * 8];
+        for (int i = 0; i < MI; ++i) af[i] = *(const bf16x8*)&As[wm * WM + i * 32 + (lane & 31)][kk + (lane >> 5) * 8];
 #pragma unroll
-        for (int j = 0; j < 2; ++j) bfr[j] = *(const bf16x8*)&Bs[wn * 64 + j * 32 + (lane & 31)][kk + (lane >> 5) * 8];
+        for (int j = 0; j < NI; ++j) bfr[j] = *(const bf16x8*)&Bs[wn * WN + j * 32 + (lane & 31)][kk + (lane >> 5) * 8];
 #pragma unroll
-        for (int i = 0; i < 2; ++i)
+        for (int i = 0; i < MI; ++i)
 #pragma unroll
-          for (int j = 0; j < 2; ++j)
+          for (int j = 0; j < NI; ++j)
             acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);
       }
     } else {
 #pragma unroll
       for (int kk = 0; kk < BK; kk += 2) {
-        float af[2], bfr[2];
+        float af[MI], bfr[NI];
 #pragma unroll
-        for (int i = 0; i < 2; ++i) af[i] = (float)As[wm * 64 + i * 32 + (lane & 31)][kk + (lane >> 5)];
+        for (int i = 0; i < MI; ++i) af[i] = (float)As[wm * WM + i * 32 + (lane & 31)][kk + (lane >> 5)];
 #pragma unroll
-        for (int j = 0; j < 2; ++j) bfr[j] = (float)Bs[wn * 64 + j * 32 + (lane & 31)][kk + (lane >> 5)];
+        for (int j = 0; j < NI; ++j) bfr[j] = (float)Bs[wn * WN + j * 32 + (lane & 31)][kk + (lane >> 5)];
 #pragma unroll
-        for (int i = 0; i < 2; ++i)
+        for (int i = 0; i < MI; ++i)
 #pragma unroll
-          for (int j = 0; j < 2; ++j)
+          for (int j = 0; j < NI; ++j)
             acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i], bfr[j], acc[i][j], 0, 0, 0);
       }
     }
     __syncthreads();
   }
+#undef KS_FETCH
   // ---- epilogue: bias + activation + store
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < MI; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int col = n0 + wn * 64 + j * 32 + (lane & 31);
+    for (int j = 0; j < NI; ++j) {
+      const int col = n0 + wn * WN + j * 32 + (lane & 31);
       const float b = bias[col];
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        const int64_t row = m0 + wm * 64 + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+        const int64_t row = m0 + wm * WM + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
         if (row >= M) continue;
         const float v = acc[i][j][r] + b;
         if (LAST) {
           if (col < Nreal) ((float*)yout)[row * ldy + col] = v;
         } else {
-          const float h = activate<ACT>(v);
+          const float h = activate<ACT, BF>(v);
           ((T*)yout)[row * ldy + col] = BF ? (T)to_bf16(h) : (T)h;
         }
       }
@@ -162,20 +216,44 @@ static uint16_t f32_to_bf16_rne(float f) {
   return (uint16_t)(u >> 16);
 }
 
-template <typename T, bool FIRST, bool LAST>
-static void launch_layer(int act, dim3 grid, hipStream_t s, int64_t M, int K, int Kreal, int Nreal, const void* x,
-                         int64_t ldx, const void* W, const float* b, void* y, int64_t ldy) {
-#define KS_LAUNCH(A)                                                                                             \
-  hipLaunchKernelGGL((mlp_layer_kernel<T, FIRST, LAST, A>), grid, dim3(256), 0, s, M, K, Kreal, Nreal, x, ldx, \
-                     (const T*)W, b, y, ldy)
-  if (LAST) { KS_LAUNCH(KS_ACT_NONE); return; }
+template <typename T, bool FIRST, bool LAST, int BM, int BN, int WAVES_M, int WAVES_N>
+static int launch_layer_tile(int act, hipStream_t s, int64_t M, int npad, int K, int Kreal, int Nreal, const void* x,
+                             int64_t ldx, const void* W, const float* b, void* y, int64_t ldy) {
+  constexpr int BK = sizeof(T) == 2 ? 64 : 32, PAD = sizeof(T) == 2 ? 8 : 4;
+  constexpr int lds = (int)sizeof(T) * (BM + BN) * (BK + PAD);
+  const dim3 grid((unsigned)((M + BM - 1) / BM), (unsigned)(npad / BN));
+  const dim3 block(64 * WAVES_M * WAVES_N);
+#define KS_LAUNCH(A)                                                                                           \
+  {                                                                                                            \
+    auto kfn = mlp_layer_kernel<T, FIRST, LAST, A, BM, BN, WAVES_M, WAVES_N>;                                  \
+    if (lds > 64 * 1024 &&                                                                                     \
+        hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)  \
+      return fail(KS_ELAUNCH, "ks_mlp_forward: cannot raise the LDS limit to %d bytes", lds);                  \
+    hipLaunchKernelGGL(kfn, grid, block, lds, s, M, K, Kreal, Nreal, x, ldx, (const T*)W, b, y, ldy);          \
+  }
+  if (LAST) { KS_LAUNCH(KS_ACT_NONE) return KS_OK; }
   switch (act) {
-    case KS_ACT_ELU: KS_LAUNCH(KS_ACT_ELU); break;
-    case KS_ACT_RELU: KS_LAUNCH(KS_ACT_RELU); break;
-    case KS_ACT_TANH: KS_LAUNCH(KS_ACT_TANH); break;
-    default: KS_LAUNCH(KS_ACT_NONE); break;
+    case KS_ACT_ELU: KS_LAUNCH(KS_ACT_ELU) break;
+    case KS_ACT_RELU: KS_LAUNCH(KS_ACT_RELU) break;
+    case KS_ACT_TANH: KS_LAUNCH(KS_ACT_TANH) break;
+    default: KS_LAUNCH(KS_ACT_NONE) break;
   }
 #undef KS_LAUNCH
+  return KS_OK;
+}
+
+// Tile choice.  Large batches take the whole layer width per workgroup (BN = 512 or 256) so that the activations
+// are read from HBM once per layer; small (rollout-sized) batches take 64 x 128 tiles so that the grid still
+// covers the 256 CUs more than once.
+template <typename T, bool FIRST, bool LAST>
+static int launch_layer(int act, hipStream_t s, int64_t M, int npad, int K, int Kreal, int Nreal, const void* x,
+                        int64_t ldx, const void* W, const float* b, void* y, int64_t ldy) {
+#define KS_ARGS act, s, M, npad, K, Kreal, Nreal, x, ldx, W, b, y, ldy
+  if (M >= 32768 && npad % 512 == 0 && sizeof(T) == 2) return launch_layer_tile<T, FIRST, LAST, 128, 512, 2, 4>(KS_ARGS);
+  if (M >= 32768 && npad % 256 == 0) return launch_layer_tile<T, FIRST, LAST, 128, 256, 2, 2>(KS_ARGS);
+  if (M * (npad / kBN) <= 128 * 512) return launch_layer_tile<T, FIRST, LAST, 64, 128, 2, 2>(KS_ARGS);
+  return launch_layer_tile<T, FIRST, LAST, 128, 128, 2, 2>(KS_ARGS);
+#undef KS_ARGS
 }
 
 }  // namespace ks
@@ -197,7 +275,7 @@ extern "C" int ks_mlp_create(const KsMlpDesc* d, KsMlp** out) {
   DevMlp& m = h->m;
   std::memset(&m, 0, sizeof(m));
   m.n_layers = d->n_layers; m.activation = d->activation; m.dtype = d->dtype;
-  const int bk = d->dtype == KS_MLP_BF16 ? 32 : 16;
+  const int bk = d->dtype == KS_MLP_BF16 ? 64 : 32;
   const size_t esz = d->dtype == KS_MLP_BF16 ? 2 : 4;
   for (int l = 0; l <= d->n_layers; ++l) m.dims[l] = d->dims[l];
   for (int l = 0; l < d->n_layers; ++l) {
@@ -263,14 +341,15 @@ extern "C" int ks_mlp_forward(const KsMlp* h, ks_stream_t stream, int64_t M, con
     const bool first = l == 0, last = l == m.n_layers - 1;
     void* outp = last ? (void*)y : (void*)buf[l & 1];
     const int64_t ldo = last ? m.dims[l + 1] : m.npad[l];
-    const dim3 grid((unsigned)((M + kBM - 1) / kBM), (unsigned)(m.npad[l] / kBN));
-#define KS_GO(T)                                                                                                 \
-  if (first && last) launch_layer<T, true, true>(m.activation, grid, s, M, m.kpad[l], m.dims[l], m.dims[l + 1], in, ldin, m.W[l], m.b[l], outp, ldo); \
-  else if (first) launch_layer<T, true, false>(m.activation, grid, s, M, m.kpad[l], m.dims[l], m.dims[l + 1], in, ldin, m.W[l], m.b[l], outp, ldo);   \
-  else if (last) launch_layer<T, false, true>(m.activation, grid, s, M, m.kpad[l], m.dims[l], m.dims[l + 1], in, ldin, m.W[l], m.b[l], outp, ldo);    \
-  else launch_layer<T, false, false>(m.activation, grid, s, M, m.kpad[l], m.dims[l], m.dims[l + 1], in, ldin, m.W[l], m.b[l], outp, ldo);
+#define KS_GO(T)                                                                                                      \
+  if (first && last) rc = launch_layer<T, true, true>(m.activation, s, M, m.npad[l], m.kpad[l], m.dims[l], m.dims[l + 1], in, ldin, m.W[l], m.b[l], outp, ldo); \
+  else if (first) rc = launch_layer<T, true, false>(m.activation, s, M, m.npad[l], m.kpad[l], m.dims[l], m.dims[l + 1], in, ldin, m.W[l], m.b[l], outp, ldo);   \
+  else if (last) rc = launch_layer<T, false, true>(m.activation, s, M, m.npad[l], m.kpad[l], m.dims[l], m.dims[l + 1], in, ldin, m.W[l], m.b[l], outp, ldo);    \
+  else rc = launch_layer<T, false, false>(m.activation, s, M, m.npad[l], m.kpad[l], m.dims[l], m.dims[l + 1], in, ldin, m.W[l], m.b[l], outp, ldo);
+    int rc = KS_OK;
     if (m.dtype == KS_MLP_BF16) { KS_GO(__bf16) } else { KS_GO(float) }
 #undef KS_GO
+    if (rc != KS_OK) return rc;
     in = outp;
     ldin = ldo;
   }
