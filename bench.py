@@ -155,27 +155,40 @@ def main() -> None:
     print(json.dumps(line))
 
 
-def gae_bandwidth(torch, ppo, T=128, N=4096, sets=32, reps=4):
-    dev = "cuda"
-    g = torch.Generator(device=dev)
-    g.manual_seed(1002)
-    bufs = [(torch.randn(N, T, device=dev, generator=g), torch.randn(N, T, device=dev, generator=g),
-             (torch.rand(N, T, device=dev, generator=g) < 0.01)) for _ in range(sets)]
-    for v, r, d in bufs[:2]:
-        ppo.compute_ppo_inputs(v, r, d, None, 0.99, 0.95)
-    torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record()
-    for _ in range(reps):
-        for v, r, d in bufs:
-            ppo.compute_ppo_inputs(v, r, d, None, 0.99, 0.95)
-    e1.record()
-    torch.cuda.synchronize()
-    ms = e0.elapsed_time(e1) / (reps * sets)
-    nbytes = T * N * 21
-    return {"workload": "cfg2: T=128, N=4096 fp32, (B,T) layout, 32 rotating buffer sets", "ms_per_call": ms,
-            "achieved_GBps": nbytes / (ms * 1e-3) / 1e9, "frac_of_hbm_peak": nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
-            "algorithmic_bytes": nbytes}
+def gae_bandwidth(torch, ppo, reps=8):
+    """GAE GB/s through the C ABI on rotating buffer sets (larger in total than the caches), outputs preallocated."""
+    from ksim_amd import _lib
+
+    lib = _lib.load()
+    out = {}
+    for name, N, T, sets in (("cfg2_T128_N4096", 4096, 128, 32), ("large_T128_N65536", 65536, 128, 4)):
+        g = torch.Generator(device="cuda")
+        g.manual_seed(1002)
+        bufs = [(torch.randn(N, T, device="cuda", generator=g), torch.randn(N, T, device="cuda", generator=g),
+                 (torch.rand(N, T, device="cuda", generator=g) < 0.01).view(torch.uint8)) for _ in range(sets)]
+        res = [torch.empty(N, T, device="cuda") for _ in range(3)]
+        st = _lib.current_stream()
+
+        def run(v, r, d):
+            _lib.check(lib.ks_gae_bt(st, N, T, _lib.ptr(v), _lib.ptr(r), _lib.ptr(d), None, 0.99, 0.95, 0,
+                                     _lib.ptr(res[0]), _lib.ptr(res[1]), _lib.ptr(res[2])))
+
+        for b in bufs[:2]:
+            run(*b)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            for b in bufs:
+                run(*b)
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / (reps * sets)
+        nbytes = T * N * 21
+        out[name] = {"layout": "(B,T) fp32, dones int8", "ms_per_call": ms, "achieved_GBps": nbytes / (ms * 1e-3) / 1e9,
+                     "frac_of_hbm_peak": nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "algorithmic_bytes": nbytes,
+                     "buffer_sets": sets}
+    return out
 
 
 def mlp_rate(torch, consts, reps=20):

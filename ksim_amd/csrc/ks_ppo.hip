@@ -9,12 +9,43 @@ static thread_local char g_err[256] = "";
 char* err_buf() { return g_err; }
 
 // ---------------------------------------------------------------------------------------------
-// GAE, (B, T) layout.  One wavefront per env row; lanes run along time.  The
-// recurrences R_t = r'_t + g m_t R_{t+1} and A_t = d_t + g l m_t A_{t+1}
-// (ksim/task/ppo.py:66-75) are compositions of affine maps x -> d + c x, which are
-// associative, so a 64-wide reverse Kogge-Stone scan with wavefront shuffles handles one
-// 64-step chunk; chunks are chained from the end of the row through a scalar carry.
+// GAE, (B, T) layout.  One wavefront per env row.  The recurrences R_t = r'_t + g m_t R_{t+1} and
+// A_t = d_t + g l m_t A_{t+1} (ksim/task/ppo.py:66-75) are compositions of affine maps x -> d + c x, which are
+// associative.  Lanes hold time in DESCENDING order (lane i of a 64-step chunk holds t = chunk_end - i), so the
+// reverse scan over time is a forward scan over lanes: four DPP row_shr steps inside 16-lane rows, then
+// row_bcast:15 and row_bcast:31 to chain the rows; no LDS traffic.  Chunks are chained from the end of the row
+// through a wave-uniform carry read from lane 63.
 // ---------------------------------------------------------------------------------------------
+template <int kCtrl, int kRowMask>
+__device__ __forceinline__ float dpp_take(float old, float x) {  // lanes without a valid source keep `old`
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, old), __builtin_bit_cast(int, x),
+                                                                kCtrl, kRowMask, 0xf, false));
+}
+
+// one scan step: (c, d) <- (c, d) o (c, d)[source lane]; identity where there is no source
+template <int kCtrl, int kRowMask>
+__device__ __forceinline__ void scan_step(float& c, float& d) {
+  const float pc = dpp_take<kCtrl, kRowMask>(1.0f, c);
+  const float pd = dpp_take<kCtrl, kRowMask>(0.0f, d);
+  d = d + c * pd;
+  c = c * pc;
+}
+
+__device__ __forceinline__ void affine_scan64(float& c, float& d) {
+  scan_step<0x111, 0xf>(c, d);  // row_shr:1
+  scan_step<0x112, 0xf>(c, d);  // row_shr:2
+  scan_step<0x114, 0xf>(c, d);  // row_shr:4
+  scan_step<0x118, 0xf>(c, d);  // row_shr:8
+  scan_step<0x142, 0xa>(c, d);  // row_bcast:15 -> rows 1 and 3
+  scan_step<0x143, 0xc>(c, d);  // row_bcast:31 -> rows 2 and 3
+}
+
+__device__ __forceinline__ float lane63(float x) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), 63));
+}
+
+constexpr int kGaeMaxChunks = 4;  // rows of up to 256 steps keep every load in flight at once
+
 __global__ __launch_bounds__(256) void gae_bt_kernel(
     int64_t B, int64_t T, const float* __restrict__ values, const float* __restrict__ rewards,
     const uint8_t* __restrict__ dones, const uint8_t* __restrict__ successes, float gamma, float lam,
@@ -26,48 +57,49 @@ __global__ __launch_bounds__(256) void gae_bt_kernel(
   const float v_last = values[base + T - 1];  // bootstrap = last value repeated, ppo.py:79
   const float gl = gamma * lam;
   const float omg = 1.0f - gamma;
-  float carry_r = 0.f, carry_a = 0.f, v_next_chunk = v_last;
+  float carry_r = 0.f, carry_a = 0.f, v_after = v_last;  // v_after: value at the first step after the chunk
   const int64_t nchunk = (T + 63) >> 6;
-  for (int64_t c = nchunk - 1; c >= 0; --c) {
-    const int64_t t = (c << 6) + lane;
-    const bool valid = t < T;
-    float v = 0.f, r = 0.f;
-    bool dn = false, sc = false;
-    if (valid) {
-      v = values[base + t];
-      r = rewards[base + t];
-      dn = dones[base + t] != 0;
-      if (successes) sc = successes[base + t] != 0;
-    }
-    float v_up = __shfl_down(v, 1);
-    if (lane == 63) v_up = v_next_chunk;
-    if (t + 1 >= T) v_up = v_last;
-    const float mask = dn ? 0.f : 1.f;
-    const float rb = omg * r + gamma * v * (sc ? 1.f : 0.f);  // ppo.py:82-83
-    const float delta = rb + gamma * v_up * mask - v;          // ppo.py:86
-    float c_r = valid ? gamma * mask : 1.f, d_r = valid ? rb : 0.f;
-    float c_a = valid ? gl * mask : 1.f, d_a = valid ? delta : 0.f;
+  for (int64_t c0 = nchunk - 1; c0 >= 0; c0 -= kGaeMaxChunks) {
+    // issue the loads of up to kGaeMaxChunks chunks before any of them is scanned
+    float v[kGaeMaxChunks], r[kGaeMaxChunks];
+    uint8_t dn[kGaeMaxChunks], sc[kGaeMaxChunks];
 #pragma unroll
-    for (int s = 1; s < 64; s <<= 1) {
-      const float pc_r = __shfl_down(c_r, s), pd_r = __shfl_down(d_r, s);
-      const float pc_a = __shfl_down(c_a, s), pd_a = __shfl_down(d_a, s);
-      if (lane + s < 64) {
-        d_r = d_r + c_r * pd_r;
-        c_r = c_r * pc_r;
-        d_a = d_a + c_a * pd_a;
-        c_a = c_a * pc_a;
+    for (int k = 0; k < kGaeMaxChunks; ++k) {
+      const int64_t c = c0 - k;
+      const int64_t t = (c << 6) + 63 - lane;  // descending time across lanes
+      const bool valid = c >= 0 && t < T;
+      v[k] = valid ? values[base + t] : 0.f;
+      r[k] = valid ? rewards[base + t] : 0.f;
+      dn[k] = valid ? dones[base + t] : (uint8_t)0;
+      sc[k] = (valid && successes) ? successes[base + t] : (uint8_t)0;
+    }
+#pragma unroll
+    for (int k = 0; k < kGaeMaxChunks; ++k) {
+      const int64_t c = c0 - k;
+      if (c < 0) break;
+      const int64_t t = (c << 6) + 63 - lane;
+      const bool valid = t < T;
+      // V(s_{t+1}) sits one lane down; lane 0 takes the first value after the chunk (wave_shr:1 keeps `old` there)
+      float v_up = dpp_take<0x138, 0xf>(v_after, v[k]);
+      if (t + 1 >= T) v_up = v_last;
+      const float mask = dn[k] ? 0.f : 1.f;
+      const float rb = omg * r[k] + gamma * v[k] * (sc[k] ? 1.f : 0.f);  // ppo.py:82-83
+      const float delta = rb + gamma * v_up * mask - v[k];                // ppo.py:86
+      float c_r = valid ? gamma * mask : 1.f, d_r = valid ? rb : 0.f;
+      float c_a = valid ? gl * mask : 1.f, d_a = valid ? delta : 0.f;
+      affine_scan64(c_r, d_r);
+      affine_scan64(c_a, d_a);
+      const float R = d_r + c_r * carry_r;
+      const float A = d_a + c_a * carry_a;
+      if (valid) {
+        if (gae) gae[base + t] = A;
+        if (returns) returns[base + t] = R;
+        if (targets) targets[base + t] = mc ? R : A + v[k];  // ppo.py:107
       }
+      carry_r = lane63(R);
+      carry_a = lane63(A);
+      v_after = lane63(v[k]);
     }
-    const float R = d_r + c_r * carry_r;
-    const float A = d_a + c_a * carry_a;
-    if (valid) {
-      if (gae) gae[base + t] = A;
-      if (returns) returns[base + t] = R;
-      if (targets) targets[base + t] = mc ? R : A + v;  // ppo.py:107
-    }
-    carry_r = __shfl(R, 0);
-    carry_a = __shfl(A, 0);
-    v_next_chunk = __shfl(v, 0);
   }
 }
 
