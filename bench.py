@@ -73,6 +73,8 @@ def main() -> None:
     ap.add_argument("--envs", type=int, default=8192)
     ap.add_argument("--rollout", type=int, default=32)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--traffic-probe", action="store_true",
+                    help="also launch ks_copy_f32 on 64 Mi floats once: the known-size kernel for counter calibration")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -123,6 +125,12 @@ def main() -> None:
     ndone = int(ro.done.sum().item())
     assert torch.isfinite(env.physics_state.data.qpos).all(), "non-finite state after the benchmark"
 
+    if args.traffic_probe:
+        n = 64 * 1024 * 1024
+        src, dst = torch.ones(n, device="cuda"), torch.empty(n, device="cuda")
+        _lib.check(_lib.load().ks_copy_f32(_lib.current_stream(), n, _lib.ptr(src), _lib.ptr(dst)))
+        torch.cuda.synchronize()
+
     # GAE on rotating cfg-2 sized buffers (T=128, N=4096): larger than the caches in total
     gae = gae_bandwidth(torch, ppo)
     mlp = mlp_rate(torch, consts)
@@ -131,9 +139,11 @@ def main() -> None:
     bytes_per_env = step_algorithmic_bytes(m, obs_dim, 1 + m.nb)
     achieved = bytes_per_env * N / (kernel_ms * 1e-3) / 1e9
     traffic = None
-    tpath = os.path.join(ROOT, "profiles", "step_kernel_traffic.json")
-    if os.path.exists(tpath):
-        traffic = json.load(open(tpath)).get("hbm_bytes_per_launch")
+    tpath = os.path.join(ROOT, "profiles", "step_kernel_cfg4_hbm_traffic.txt")
+    if os.path.exists(tpath):  # measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, see that file
+        for ln in open(tpath):
+            if ln.startswith("hbm_bytes_per_launch="):
+                traffic = float(ln.split("=", 1)[1])
     line = {
         "metric": "env-steps/sec, 8192-env humanoid rollout (1 GPU)", "value": N * args.steps / elapsed,
         "unit": "env-steps/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,

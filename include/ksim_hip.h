@@ -364,6 +364,11 @@ typedef struct KsRewardIO {
 } KsRewardIO;
 int ks_rewards(ks_stream_t stream, const KsRewardIO* io /*host*/);
 
+/* ------------------------------------------------------------------ measurement aid
+ * A plain f32 copy of n elements (reads 4n bytes, writes 4n bytes): the known-size kernel that hardware
+ * traffic counters are calibrated against.  No counterpart in the reference. */
+int ks_copy_f32(ks_stream_t stream, int64_t n, const float* src, float* dst);
+
 #ifdef __cplusplus
 }
 #endif

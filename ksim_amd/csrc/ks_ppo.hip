@@ -294,6 +294,10 @@ __global__ __launch_bounds__(256) void reward_total_kernel(
   }
 }
 
+__global__ __launch_bounds__(256) void copy_f32_kernel(int64_t n, const float* __restrict__ src, float* __restrict__ dst) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) dst[i] = src[i];
+}
+
 static inline int grid_for(int64_t n, int block, int cap) {
   int64_t g = (n + block - 1) / block;
   if (g > cap) g = cap;
@@ -391,4 +395,12 @@ extern "C" int ks_reward_total(ks_stream_t stream, int64_t n, int32_t K, const f
                      components, sc, use_clip_min, clip_min, use_clip_max, clip_max, total, (int)k, terminations, done,
                      success);
   return check_launch("ks_reward_total");
+}
+
+extern "C" int ks_copy_f32(ks_stream_t stream, int64_t n, const float* src, float* dst) {
+  if (n < 0) return fail(KS_EINVAL, "ks_copy_f32: negative size");
+  if (n == 0) return KS_OK;
+  if (!src || !dst) return fail(KS_EINVAL, "ks_copy_f32: null pointer");
+  hipLaunchKernelGGL(copy_f32_kernel, dim3(grid_for(n, 256, 65536)), dim3(256), 0, (hipStream_t)stream, n, src, dst);
+  return check_launch("ks_copy_f32");
 }

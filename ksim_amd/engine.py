@@ -190,7 +190,7 @@ class HipEngine(PhysicsEngine):
     def step(self, action: torch.Tensor, physics_model: physics.DeviceModel, physics_state: PhysicsState,
              curriculum_level, rng, randomization: Mapping[str, torch.Tensor] | None = None,
              noise: Mapping[str, torch.Tensor] | None = None,
-             record: Mapping[str, torch.Tensor] | None = None) -> PhysicsState:
+             record: Mapping[str, torch.Tensor] | None = None, want_cvel: bool = True) -> PhysicsState:
         m, d, s = physics_model.model, physics_state.data, physics_state
         rnd, noise, record = randomization or {}, noise or {}, record or {}
         drop = noise.get("drop")
@@ -201,7 +201,8 @@ class HipEngine(PhysicsEngine):
         buf = dict(qpos=d.qpos, qvel=d.qvel, qacc_warmstart=d.qacc_warmstart, time=d.time, last_ctrl=s.last_ctrl,
                    action=action, latency=s.action_latency, zero_offset=s.zero_offset, drop=drop,
                    friction=rnd.get("friction"), mass_scale=rnd.get("mass_scale"), qacc=d.qacc, ctrl_out=d.ctrl,
-                   xpos=d.xpos, xquat=d.xquat, cvel=d.cvel, action_noise=noise.get("action_noise"),
+                   xpos=d.xpos, xquat=d.xquat, cvel=d.cvel if want_cvel else None,
+                   action_noise=noise.get("action_noise"),
                    torque_noise=noise.get("torque_noise"), traj_ctrl=record.get("ctrl"),
                    traj_xpos=record.get("xpos"), traj_xquat=record.get("xquat"))
         act = self.actuators

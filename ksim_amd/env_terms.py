@@ -36,6 +36,7 @@ class EnvTerms:
         d = T.KsTermsDesc()
         d.nq, d.nv, d.nu, d.nb, d.command_dim = model.nq, model.nv, model.nu, model.nb, self.command_dim
         self.obs_slices: dict[str, slice] = {}
+        self.sources_used: set[int] = set()
         self.bias_std = []
         k = 0
         for name, obs in self.observations.items():
@@ -47,6 +48,7 @@ class EnvTerms:
                 e = d.obs[k]
                 e.kind, e.src, e.index, e.comp = el.kind, el.src, el.index, el.comp
                 e.c0, e.c1, e.c2 = el.const
+                self.sources_used.add(el.src)
                 if noise is not None:
                     e.noise_kind, e.noise_mean, e.noise_scale = noise.kind, noise.mean, noise.scale
                 self.bias_std.append(0.0 if obs.bias is None else float(obs.bias))

@@ -89,7 +89,8 @@ class Rollout:
                       clip_max=c.action_clip_max, out=self.action[t])
         # the step kernel also writes ctrl / xpos / xquat of the post-step data into the transition slot
         c.engine.step(self.action[t], c.physics_model, ps, level, env.seed + env.step, env.randomization_dict,
-                      noise=noise.get("engine"), record=dict(ctrl=self.ctrl[t], xpos=self.xpos[t], xquat=self.xquat[t]))
+                      noise=noise.get("engine"), record=dict(ctrl=self.ctrl[t], xpos=self.xpos[t], xquat=self.xquat[t]),
+                      want_cvel=T.SRC_CVEL in c.terms.sources_used)
         st = dict(qpos=d.qpos, qvel=d.qvel, qacc_warmstart=d.qacc_warmstart, time=d.time, last_ctrl=ps.last_ctrl)
         c.terms.terminate_reset(st, level=level, components=self.components[t][: c.terms.n_terms] if c.terms.n_terms else None,
                                 done=self.done[t], success=self.success[t], traj_qpos=self.qpos[t],
