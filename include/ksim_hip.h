@@ -30,6 +30,10 @@ enum {
 /* Library identity / error text (host). */
 const char* ks_version(void);
 const char* ks_last_error(void);
+/* sizeof() of a public struct as this library was compiled, for binding self-checks:
+ * 0 KsPpoLossParams, 1 KsModelDesc, 2 KsStepIO, 3 KsTermsDesc, 4 KsObserveIO, 5 KsTerminateIO, 6 KsMlpDesc,
+ * 7 KsRewardIO, 8 KsObsElem, 9 KsTermDesc, 10 KsRewardDesc, 11 KsRng; -1 for anything else. */
+int64_t ks_abi_sizeof(int32_t which);
 
 /* ------------------------------------------------------------------ GAE / returns
  * Replaces compute_ppo_inputs, ksim/task/ppo.py:54-121.

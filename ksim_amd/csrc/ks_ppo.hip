@@ -311,6 +311,23 @@ using namespace ks;
 
 extern "C" const char* ks_version(void) { return "ksim_hip 0.1 (gfx950)"; }
 extern "C" const char* ks_last_error(void) { return ks::err_buf(); }
+extern "C" int64_t ks_abi_sizeof(int32_t which) {
+  switch (which) {
+    case 0: return sizeof(KsPpoLossParams);
+    case 1: return sizeof(KsModelDesc);
+    case 2: return sizeof(KsStepIO);
+    case 3: return sizeof(KsTermsDesc);
+    case 4: return sizeof(KsObserveIO);
+    case 5: return sizeof(KsTerminateIO);
+    case 6: return sizeof(KsMlpDesc);
+    case 7: return sizeof(KsRewardIO);
+    case 8: return sizeof(KsObsElem);
+    case 9: return sizeof(KsTermDesc);
+    case 10: return sizeof(KsRewardDesc);
+    case 11: return sizeof(KsRng);
+    default: return -1;
+  }
+}
 
 static int check_gae_args(int64_t n0, int64_t n1, const float* v, const float* r, const uint8_t* d) {
   if (n0 < 0 || n1 < 0) return fail(KS_EINVAL, "ks_gae: negative size");

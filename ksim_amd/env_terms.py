@@ -24,6 +24,51 @@ def _rng(seed: int, step: int) -> T.KsRng:
     return T.KsRng(int(seed) & (2**64 - 1), int(step) & (2**64 - 1))
 
 
+def compile_terms(model: KinematicModel, observations: Mapping[str, Observation],
+                  terminations: Mapping[str, Termination], resets: Sequence[Reset], command_dim: int = 0,
+                  terminate_on_nonfinite: bool = True):
+    """Host-side compilation of the task's terms into the flat tables of KsTermsDesc (no GPU involved).
+
+    Returns (desc, obs_slices, sources_used, bias_std, reset_table)."""
+    d = T.KsTermsDesc()
+    d.nq, d.nv, d.nu, d.nb, d.command_dim = model.nq, model.nv, model.nu, model.nb, int(command_dim)
+    obs_slices: dict[str, slice] = {}
+    sources_used: set[int] = set()
+    bias_std: list[float] = []
+    k = 0
+    for name, obs in observations.items():
+        elems = obs.elements(model, int(command_dim))
+        noise = obs._noise()
+        if k + len(elems) > T.KS_MAX_OBS:
+            raise _lib.KsError(f"observation vector longer than {T.KS_MAX_OBS}")
+        for el in elems:
+            e = d.obs[k]
+            e.kind, e.src, e.index, e.comp = el.kind, el.src, el.index, el.comp
+            e.c0, e.c1, e.c2 = el.const
+            sources_used.add(el.src)
+            if noise is not None:
+                e.noise_kind, e.noise_mean, e.noise_scale = noise.kind, noise.mean, noise.scale
+            bias_std.append(0.0 if obs.bias is None else float(obs.bias))
+            k += 1
+        obs_slices[name] = slice(k - len(elems), k)
+    d.obs_dim = k
+    if len(terminations) > T.KS_MAX_TERMS:
+        raise _lib.KsError("too many terminations")
+    for j, term in enumerate(terminations.values()):
+        t = d.terms[j]
+        t.kind, t.value, t.p0, t.p1, t.p2, t.p3 = term.desc()
+    d.n_terms = len(terminations)
+    tab = compile_resets(resets, model)
+    big = 3.0e38
+    for i in range(model.nq):
+        d.reset_base[i], d.reset_mag[i] = tab["base"][i], tab["mag"][i]
+        d.reset_lo[i], d.reset_hi[i] = max(tab["lo"][i], -big), min(tab["hi"][i], big)
+        d.reset_by_level[i] = int(tab["by_level"][i])
+    d.random_heading = int(tab["heading"])
+    d.nonfinite_terminates = int(terminate_on_nonfinite)
+    return d, obs_slices, sources_used, bias_std, tab
+
+
 class EnvTerms:
     def __init__(self, model: KinematicModel, observations: Mapping[str, Observation],
                  terminations: Mapping[str, Termination], resets: Sequence[Reset], command_dim: int = 0,
@@ -33,43 +78,9 @@ class EnvTerms:
         self.model, self._lib = model, lib
         self.observations, self.terminations, self.resets = dict(observations), dict(terminations), tuple(resets)
         self.command_dim = int(command_dim)
-        d = T.KsTermsDesc()
-        d.nq, d.nv, d.nu, d.nb, d.command_dim = model.nq, model.nv, model.nu, model.nb, self.command_dim
-        self.obs_slices: dict[str, slice] = {}
-        self.sources_used: set[int] = set()
-        self.bias_std = []
-        k = 0
-        for name, obs in self.observations.items():
-            elems = obs.elements(model, self.command_dim)
-            noise = obs._noise()
-            if k + len(elems) > T.KS_MAX_OBS:
-                raise _lib.KsError(f"observation vector longer than {T.KS_MAX_OBS}")
-            for el in elems:
-                e = d.obs[k]
-                e.kind, e.src, e.index, e.comp = el.kind, el.src, el.index, el.comp
-                e.c0, e.c1, e.c2 = el.const
-                self.sources_used.add(el.src)
-                if noise is not None:
-                    e.noise_kind, e.noise_mean, e.noise_scale = noise.kind, noise.mean, noise.scale
-                self.bias_std.append(0.0 if obs.bias is None else float(obs.bias))
-                k += 1
-            self.obs_slices[name] = slice(k - len(elems), k)
-        d.obs_dim = self.obs_dim = k
-        if len(self.terminations) > T.KS_MAX_TERMS:
-            raise _lib.KsError("too many terminations")
-        for j, term in enumerate(self.terminations.values()):
-            t = d.terms[j]
-            t.kind, t.value, t.p0, t.p1, t.p2, t.p3 = term.desc()
-        d.n_terms = self.n_terms = len(self.terminations)
-        tab = compile_resets(self.resets, model)
-        big = 3.0e38
-        for i in range(model.nq):
-            d.reset_base[i], d.reset_mag[i] = tab["base"][i], tab["mag"][i]
-            d.reset_lo[i], d.reset_hi[i] = max(tab["lo"][i], -big), min(tab["hi"][i], big)
-            d.reset_by_level[i] = int(tab["by_level"][i])
-        d.random_heading = int(tab["heading"])
-        d.nonfinite_terminates = int(terminate_on_nonfinite)
-        self.reset_table = tab
+        d, self.obs_slices, self.sources_used, self.bias_std, self.reset_table = compile_terms(
+            model, self.observations, self.terminations, self.resets, self.command_dim, terminate_on_nonfinite)
+        self.obs_dim, self.n_terms = int(d.obs_dim), int(d.n_terms)
         self._handle = ctypes.c_void_p()
         _lib.check(lib.ks_terms_create(ctypes.byref(d), ctypes.byref(self._handle)))
 

@@ -1,0 +1,116 @@
+"""Host-side logic that needs no GPU: config validation, table compilation, struct layouts, model builder."""
+import ctypes
+
+import numpy as np
+import pytest
+
+from ksim_amd import _lib, _lib_dyn, _lib_terms as T
+from ksim_amd import actuators, engine, model as km, noise, observation as ob, resets as rs, rewards as rw
+from ksim_amd import terminations as tm
+from ksim_amd.env_terms import compile_terms
+
+
+def test_struct_layouts_match_the_library():
+    lib = ctypes.CDLL(_lib.LIB_PATH)
+    lib.ks_abi_sizeof.restype = ctypes.c_int64
+    lib.ks_abi_sizeof.argtypes = [ctypes.c_int32]
+    structs = [_lib.KsPpoLossParams, _lib_dyn.KsModelDesc, _lib_dyn.KsStepIO, T.KsTermsDesc, T.KsObserveIO,
+               T.KsTerminateIO, T.KsMlpDesc, T.KsRewardIO, T.KsObsElem, T.KsTermDesc, T.KsRewardDesc, T.KsRng]
+    for i, st in enumerate(structs):
+        assert lib.ks_abi_sizeof(i) == ctypes.sizeof(st), st.__name__
+    assert lib.ks_abi_sizeof(99) == -1
+
+
+def test_engine_config_validation_matches_reference_rules():
+    with pytest.raises(ValueError, match="`dt` is required"):
+        engine.EngineConfig(ctrl_dt=0.02)
+    with pytest.raises(ValueError, match="`ctrl_dt` is required"):
+        engine.EngineConfig(dt=0.005)
+    with pytest.raises(ValueError, match="non-negative"):
+        engine.EngineConfig(dt=0.005, ctrl_dt=0.02, action_latency_range=(-0.1, 0.0))
+    with pytest.raises(ValueError, match="less than or equal"):
+        engine.EngineConfig(dt=0.005, ctrl_dt=0.02, action_latency_range=(0.02, 0.01))
+    with pytest.raises(ValueError, match="drop_action_prob"):
+        engine.EngineConfig(dt=0.005, ctrl_dt=0.02, drop_action_prob=1.0)
+    cfg = engine.EngineConfig(dt=0.004, ctrl_dt=0.02, action_latency_range=(0.0, 0.008), actuator_update_dt=0.008)
+    data = engine.EngineData.from_config(cfg)
+    assert data.phys_steps_per_ctrl_steps == 5 and data.phys_steps_per_actuator_step == 2
+    assert data.max_action_latency_step == pytest.approx(2.0) and data.min_action_latency_step == 0.0
+    assert engine.EngineConfig(dt=0.005, ctrl_dt=0.02).phys_steps_per_actuator_step == 1
+    with pytest.raises(ValueError, match="Unsupported physics model type"):
+        engine.get_physics_engine("mjx", [], {}, actuators.TorqueActuators(), cfg)
+    eng = engine.get_physics_engine("hip", [], {}, actuators.TorqueActuators(), cfg)
+    hash(eng)  # engines must stay hashable (reference tests/test_resets.py:82-84 checks the same of resets)
+    with pytest.raises(NotImplementedError):
+        engine.HipEngine(actuators.TorqueActuators(), [], {"push": object()}, data)
+
+
+def test_actuator_and_term_validation():
+    with pytest.raises(ValueError, match="negative"):
+        actuators.PositionActuators(kps=(1.0, -1.0), kds=(1.0, 1.0))
+    with pytest.raises(ValueError):
+        actuators.PositionActuators(kps=(1.0,), kds=(1.0, 1.0))
+    with pytest.raises(ValueError):
+        actuators.PositionActuators(kps=(1.0,), kds=(1.0,), ctrl_clip=(-5.0,))
+    assert np.isinf(actuators.PositionActuators(kps=(1.0, 2.0), kds=(0.1, 0.1)).clip_array()).all()
+    with pytest.raises(ValueError):
+        tm.MinimumHeightTermination(0.0)
+    with pytest.raises(ValueError):
+        tm.NotUprightTermination(-1.0)
+    assert tm.MinimumHeightTermination(0.5).termination_name == "minimum_height_termination"
+    assert tm.FarFromOriginTermination(3.0).desc()[1] == 1 and tm.FarFromOriginTermination(3.0, False).desc()[1] == -1
+    assert rw.ActionVelocityPenalty().is_penalty and not rw.StayAliveReward().is_penalty
+    with pytest.raises(ValueError, match="Invalid norm"):
+        rw.ActionJerkPenalty(norm="l3").descs()
+
+    class Odd(rw.Reward):
+        pass
+
+    with pytest.raises(ValueError, match="does not end with"):
+        Odd().is_penalty
+    assert noise.convert_to_noise(0.01).kind == T.NOISE_ADD_GAUSSIAN and noise.convert_to_noise(None) is None
+    with pytest.raises(ValueError):
+        noise.convert_to_noise("x")
+
+
+def test_term_tables_compile():
+    m = km.humanoid_model()
+    observations = {"jp": ob.JointPositionObservation(noise=0.01), "jv": ob.JointVelocityObservation(),
+                    "g": ob.ProjectedGravityObservation(), "w": ob.BaseAngularVelocityObservation(in_robot_frame=True),
+                    "a": ob.LastActionObservation(), "c": ob.CommandObservation()}
+    resets = [rs.RandomJointPositionReset(scale=0.1, scale_by_curriculum=False), rs.RandomHeightReset(range=(0.0, 0.1)),
+              rs.RandomHeadingReset(), rs.RandomJointVelocityReset()]
+    d, slices, used, bias, tab = compile_terms(m, observations, {"h": tm.MinimumHeightTermination(0.5)}, resets, 2)
+    assert d.obs_dim == 71 and slices["g"] == slice(42, 45) and slices["c"] == slice(69, 71)  # BASELINE config 3: 71
+    assert d.obs[0].kind == T.OBS_JOINT_POS and d.obs[0].index == 7 and d.obs[0].noise_kind == T.NOISE_ADD_GAUSSIAN
+    assert d.obs[42].kind == T.OBS_ROT_INV and d.obs[44].comp == 2 and d.obs[44].c2 == pytest.approx(-9.81)
+    assert T.SRC_CVEL not in used and T.SRC_QPOS in used
+    assert d.n_terms == 1 and d.terms[0].kind == T.TERM_MIN_HEIGHT and d.terms[0].value == -1
+    assert d.random_heading == 1 and d.reset_by_level[7] == 0 and d.reset_mag[7] == pytest.approx(0.1)
+    assert d.reset_base[2] == pytest.approx(m.qpos0[2] + 0.05) and d.reset_mag[2] == pytest.approx(0.05)
+    assert d.reset_mag[0] == 0.0 and d.nonfinite_terminates == 1
+
+
+def test_model_builder_rules_and_constants():
+    mb = km.ModelBuilder()
+    a = mb.add_body(0, (0, 0, 1), joint="free", mass=1.0, inertia=(0.1, 0.1, 0.1))
+    b = mb.add_body(a, (0, 0, -0.2), mass=0.5, inertia=(0.01, 0.01, 0.01))
+    c = mb.add_body(b, (0, 0, -0.2), mass=0.5, inertia=(0.01, 0.01, 0.01))
+    mb.add_body(a, (0, 0.1, 0), mass=0.5, inertia=(0.01, 0.01, 0.01))  # back up to an ancestor: still depth-first
+    with pytest.raises(ValueError, match="depth-first"):
+        mb.add_body(c, (0, 0, -0.2), mass=0.5, inertia=(0.01, 0.01, 0.01))  # c's subtree was already closed
+    with pytest.raises(ValueError, match="attach to the world"):
+        mb.add_body(a, (0, 0, 0), joint="free", mass=1.0, inertia=(1, 1, 1))
+    with pytest.raises(ValueError, match="hinge"):
+        mb.add_actuator(a)
+    m = mb.build()
+    assert (m.nq, m.nv, m.nb) == (10, 9, 5)
+    assert list(m.dof_parent) == [-1, 0, 1, 2, 3, 4, 5, 6, 5] and list(m.body_subtree_end) == [5, 5, 4, 4, 5]
+    M = km.host_mass_matrix(m.arrays(), m.qpos0)
+    assert m.meaninertia == pytest.approx(np.trace(M) / m.nv)
+    assert m.body_invweight0[1, 0] > 0 and m.body_invweight0[0, 0] == 0
+    desc = _lib_dyn.model_desc(m)
+    assert desc.nb == 5 and desc.body_parent[3] == 2 and desc.act_lo[0] == 0.0
+    h = km.humanoid_model()
+    assert h.max_depth == 6 and km.humanoid_model(seed=1).body_mass[3] != h.body_mass[3]
+    assert np.allclose(km.capsule_inertia(1.0, 1e-9, 1.0)[:2], 1.0 / 12.0, rtol=1e-6)  # thin rod limit
