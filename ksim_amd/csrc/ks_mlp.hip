@@ -197,6 +197,145 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void mlp_layer_kernel(int64
     }
 }
 
+
+// ---------------------------------------------------------------- whole network in one kernel (bf16)
+// A 512-thread workgroup keeps a BM-row tile of activations in LDS as bf16 for the whole network and walks the
+// layers in place; only the network input and output touch HBM.  The product is computed transposed,
+// C^T = W * A^T: the weights are the MFMA "A" operand (32 output features x 16 k), the activations the "B"
+// operand (16 k x 32 batch rows), so that a lane's accumulators hold 4 consecutive features of one batch row
+// and the epilogue writes them back with one 8-byte LDS store.  Wavefront w owns output tiles w and w + 8 and
+// all BM rows; its weight fragments stream from global memory (L2-resident, pre-ordered so that a fragment is
+// one contiguous 1 KB read) through a register ring kPF steps deep; activation fragments come from LDS.
+constexpr int kFusedMaxWidth = 512;
+constexpr int kFusedWaves = 8;
+constexpr int kPF = 4;
+
+struct FusedArgs {
+  int64_t M;
+  int n_layers, in_dim, out_dim, lda;
+  int fk[KS_MAX_LAYERS], fn[KS_MAX_LAYERS];
+  const u32x4* Wp[KS_MAX_LAYERS];
+  const float* bp[KS_MAX_LAYERS];
+  const float* x;
+  float* y;
+};
+
+template <int NT, int MI>
+__device__ __forceinline__ void fused_layer_mma(f32x16 (&acc)[2][MI], const u32x4* __restrict__ w0,
+                                                const u32x4* __restrict__ w1, int nk, const __bf16* __restrict__ act,
+                                                int lda, int lane) {
+  u32x4 rw[kPF][NT];
+#pragma unroll
+  for (int u = 0; u < kPF; ++u) {
+    const int st = u < nk ? u : nk - 1;
+    rw[u][0] = w0[(int64_t)st * 64];
+    if (NT > 1) rw[u][NT - 1] = w1[(int64_t)st * 64];
+  }
+  const __bf16* arow = act + (lane & 31) * lda + (lane >> 5) * 8;
+  for (int s = 0; s < nk; s += kPF) {
+#pragma unroll
+    for (int u = 0; u < kPF; ++u) {
+      if (s + u < nk) {
+        bf16x8 bfr[MI];
+#pragma unroll
+        for (int i = 0; i < MI; ++i) bfr[i] = *(const bf16x8*)(arow + i * 32 * lda + (s + u) * 16);
+        bf16x8 wf[NT];
+#pragma unroll
+        for (int t = 0; t < NT; ++t) wf[t] = __builtin_bit_cast(bf16x8, rw[u][t]);
+        const int nx = s + u + kPF < nk ? s + u + kPF : nk - 1;
+        rw[u][0] = w0[(int64_t)nx * 64];
+        if (NT > 1) rw[u][NT - 1] = w1[(int64_t)nx * 64];
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+#pragma unroll
+          for (int i = 0; i < MI; ++i)
+            acc[t][i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[t], bfr[i], acc[t][i], 0, 0, 0);
+      }
+    }
+  }
+}
+
+template <int ACT, int BM>
+__global__ __launch_bounds__(64 * kFusedWaves) void mlp_fused_kernel(const FusedArgs a) {
+  constexpr int MI = BM / 32;
+  constexpr int NTHR = 64 * kFusedWaves;
+  extern __shared__ __attribute__((aligned(16))) unsigned char mlp_lds[];
+  __bf16* act = reinterpret_cast<__bf16*>(mlp_lds);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int64_t m0 = (int64_t)blockIdx.x * BM;
+  const int lda = a.lda;
+  {  // network input -> bf16 tile, zero beyond the batch and in the K padding of the first layer
+    const int K0 = a.fk[0] * 16;
+    const int64_t rows_left = a.M - m0;
+    const int rows = rows_left < BM ? (int)rows_left : BM;
+    const float* src = a.x + m0 * a.in_dim;
+    const int total = rows * a.in_dim;
+    for (int idx = tid; idx < BM * K0; idx += NTHR) {
+      const int r = idx / K0, c = idx - r * K0;
+      if (r >= rows || c >= a.in_dim) act[r * lda + c] = (__bf16)0.0f;
+    }
+    for (int idx = tid; idx < total; idx += NTHR) {
+      const int r = idx / a.in_dim, c = idx - r * a.in_dim;
+      act[r * lda + c] = (__bf16)src[idx];
+    }
+  }
+  __syncthreads();
+  for (int l = 0; l < a.n_layers; ++l) {
+    const int nk = a.fk[l], nt = a.fn[l];
+    const int mine = wave < nt ? (wave + kFusedWaves < nt ? 2 : 1) : 0;
+    const bool last = l == a.n_layers - 1;
+    f32x16 acc[2][MI];
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int i = 0; i < MI; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[t][i][r] = 0.f;
+    const u32x4* w0 = a.Wp[l] + (int64_t)wave * nk * 64 + lane;
+    const u32x4* w1 = a.Wp[l] + (int64_t)(wave + kFusedWaves) * nk * 64 + lane;
+    if (mine == 2) fused_layer_mma<2, MI>(acc, w0, w1, nk, act, lda, lane);
+    else if (mine == 1) fused_layer_mma<1, MI>(acc, w0, w0, nk, act, lda, lane);
+    __syncthreads();  // every wavefront has read this layer's input; the tile can be overwritten
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      if (t < mine) {
+        const int j = wave + kFusedWaves * t;
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const int f0 = j * 32 + 8 * g + 4 * (lane >> 5);
+          const float4 b = *reinterpret_cast<const float4*>(a.bp[l] + f0);
+#pragma unroll
+          for (int i = 0; i < MI; ++i) {
+            const int row = i * 32 + (lane & 31);
+            float v[4] = {acc[t][i][4 * g] + b.x, acc[t][i][4 * g + 1] + b.y, acc[t][i][4 * g + 2] + b.z,
+                          acc[t][i][4 * g + 3] + b.w};
+            if (last) {
+              const int64_t m = m0 + row;
+              if (m < a.M) {
+                float* dst = a.y + m * a.out_dim + f0;
+                if ((a.out_dim & 3) == 0 && f0 + 4 <= a.out_dim) {
+                  *reinterpret_cast<float4*>(dst) = float4{v[0], v[1], v[2], v[3]};
+                } else {
+#pragma unroll
+                  for (int e = 0; e < 4; ++e)
+                    if (f0 + e < a.out_dim) dst[e] = v[e];
+                }
+              }
+            } else {
+              unsigned short hb[4];
+#pragma unroll
+              for (int e = 0; e < 4; ++e) hb[e] = __builtin_bit_cast(unsigned short, (__bf16)activate<ACT, true>(v[e]));
+              const uint2 packed = {(unsigned)hb[0] | ((unsigned)hb[1] << 16), (unsigned)hb[2] | ((unsigned)hb[3] << 16)};
+              *reinterpret_cast<uint2*>(act + row * lda + f0) = packed;
+            }
+          }
+        }
+      }
+    }
+    __syncthreads();
+  }
+}
+
 struct DevMlp {
   int n_layers, activation, dtype;
   int dims[KS_MAX_LAYERS + 1];
@@ -204,6 +343,13 @@ struct DevMlp {
   int npad[KS_MAX_LAYERS];  // padded output width of layer l
   void* W[KS_MAX_LAYERS];
   float* b[KS_MAX_LAYERS];
+  // whole-network kernel (bf16, every padded width <= kFusedMaxWidth): weights re-ordered into MFMA fragments
+  int fused;                    // 1 when the tables below are valid
+  int fk[KS_MAX_LAYERS];        // K steps of 16 per layer
+  int fn[KS_MAX_LAYERS];        // 32-wide output tiles per layer
+  int lda;                      // LDS row stride of the activation tile, in bf16 elements
+  void* Wp[KS_MAX_LAYERS];      // [tile][k step][lane] x 16 bytes
+  float* bp[KS_MAX_LAYERS];     // bias padded to 32 * fn
 };
 
 static inline int round_up(int x, int m) { return (x + m - 1) / m * m; }
@@ -300,6 +446,39 @@ extern "C" int ks_mlp_create(const KsMlpDesc* d, KsMlp** out) {
       return fail(KS_ELAUNCH, "ks_mlp_create: upload of layer %d failed", l);
     }
   }
+  // fragment-ordered copy for the whole-network kernel
+  bool fusable = d->dtype == KS_MLP_BF16;
+  for (int l = 0; l <= d->n_layers && fusable; ++l)
+    if (round_up(d->dims[l], 32) > kFusedMaxWidth) fusable = false;
+  if (fusable) {
+    int kmax = 0;
+    for (int l = 0; l < d->n_layers; ++l) {
+      m.fn[l] = round_up(d->dims[l + 1], 32) / 32;
+      m.fk[l] = (l == 0 ? round_up(d->dims[0], 16) : m.fn[l - 1] * 32) / 16;
+      kmax = m.fk[l] * 16 > kmax ? m.fk[l] * 16 : kmax;
+      if (l + 1 < d->n_layers && m.fn[l] * 32 > kmax) kmax = m.fn[l] * 32;
+      const size_t n = (size_t)m.fn[l] * m.fk[l] * 64 * 8;
+      std::vector<uint16_t> w(n, 0);
+      for (int j = 0; j < m.fn[l]; ++j)
+        for (int st = 0; st < m.fk[l]; ++st)
+          for (int lane = 0; lane < 64; ++lane)
+            for (int e = 0; e < 8; ++e) {
+              const int o = j * 32 + (lane & 31), i = st * 16 + (lane >> 5) * 8 + e;
+              if (o < d->dims[l + 1] && i < d->dims[l])
+                w[(((size_t)j * m.fk[l] + st) * 64 + lane) * 8 + e] = f32_to_bf16_rne(d->weights[l][(size_t)o * d->dims[l] + i]);
+            }
+      std::vector<float> b(m.fn[l] * 32, 0.f);
+      for (int o = 0; o < d->dims[l + 1]; ++o) b[o] = d->biases[l][o];
+      if (hipMalloc(&m.Wp[l], n * 2) != hipSuccess || hipMalloc((void**)&m.bp[l], b.size() * 4) != hipSuccess ||
+          hipMemcpy(m.Wp[l], w.data(), n * 2, hipMemcpyHostToDevice) != hipSuccess ||
+          hipMemcpy(m.bp[l], b.data(), b.size() * 4, hipMemcpyHostToDevice) != hipSuccess) {
+        ks_mlp_destroy(h);
+        return fail(KS_ELAUNCH, "ks_mlp_create: upload of layer %d failed", l);
+      }
+    }
+    m.lda = kmax + 8;  // +16 bytes per row: 16-byte aligned rows that start 4 banks apart
+    m.fused = 1;
+  }
   *out = h;
   return KS_OK;
 }
@@ -309,13 +488,55 @@ extern "C" int ks_mlp_destroy(KsMlp* h) {
   for (int l = 0; l < KS_MAX_LAYERS; ++l) {
     if (h->m.W[l]) (void)hipFree(h->m.W[l]);
     if (h->m.b[l]) (void)hipFree(h->m.b[l]);
+    if (h->m.Wp[l]) (void)hipFree(h->m.Wp[l]);
+    if (h->m.bp[l]) (void)hipFree(h->m.bp[l]);
   }
   delete h;
   return KS_OK;
 }
 
+template <int BM>
+static int launch_fused_tile(const DevMlp& m, hipStream_t s, int64_t M, const float* x, float* y) {
+  FusedArgs a;
+  std::memset(&a, 0, sizeof(a));
+  a.M = M; a.n_layers = m.n_layers; a.in_dim = m.dims[0]; a.out_dim = m.dims[m.n_layers]; a.lda = m.lda;
+  for (int l = 0; l < m.n_layers; ++l) {
+    a.fk[l] = m.fk[l]; a.fn[l] = m.fn[l];
+    a.Wp[l] = (const u32x4*)m.Wp[l]; a.bp[l] = m.bp[l];
+  }
+  a.x = x; a.y = y;
+  const int lds = BM * m.lda * 2;
+  const int64_t blocks = (M + BM - 1) / BM;
+  if (blocks > 0x7fffffff) return fail(KS_ELIMIT, "ks_mlp_forward: too many rows");
+#define KS_LAUNCH(A)                                                                                           \
+  {                                                                                                            \
+    auto kfn = mlp_fused_kernel<A, BM>;                                                                        \
+    if (lds > 64 * 1024 &&                                                                                     \
+        hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)  \
+      return fail(KS_ELAUNCH, "ks_mlp_forward: cannot raise the LDS limit to %d bytes", lds);                  \
+    hipLaunchKernelGGL(kfn, dim3((unsigned)blocks), dim3(64 * kFusedWaves), lds, s, a);                        \
+  }
+  switch (m.activation) {
+    case KS_ACT_ELU: KS_LAUNCH(KS_ACT_ELU) break;
+    case KS_ACT_RELU: KS_LAUNCH(KS_ACT_RELU) break;
+    case KS_ACT_TANH: KS_LAUNCH(KS_ACT_TANH) break;
+    default: KS_LAUNCH(KS_ACT_NONE) break;
+  }
+#undef KS_LAUNCH
+  return check_launch("ks_mlp_forward");
+}
+
+// Row tile: 128 rows amortise each weight fragment over four MFMAs; smaller batches take smaller tiles so that
+// the grid still reaches every CU.
+static int launch_fused(const DevMlp& m, hipStream_t s, int64_t M, const float* x, float* y) {
+  if (M >= 128 * 256) return launch_fused_tile<128>(m, s, M, x, y);
+  if (M >= 64 * 256) return launch_fused_tile<64>(m, s, M, x, y);
+  return launch_fused_tile<32>(m, s, M, x, y);
+}
+
 extern "C" int64_t ks_mlp_workspace_bytes(const KsMlp* h, int64_t M) {
   if (!h || M < 0) return 0;
+  if (h->m.fused) return 0;
   int widest = 0;
   for (int l = 0; l + 1 < h->m.n_layers; ++l) widest = h->m.npad[l] > widest ? h->m.npad[l] : widest;
   const int64_t esz = h->m.dtype == KS_MLP_BF16 ? 2 : 4;
@@ -328,6 +549,7 @@ extern "C" int ks_mlp_forward(const KsMlp* h, ks_stream_t stream, int64_t M, con
   if (M == 0) return KS_OK;
   if (!x || !y) return fail(KS_EINVAL, "ks_mlp_forward: null pointer");
   const DevMlp& m = h->m;
+  if (m.fused) return launch_fused(m, (hipStream_t)stream, M, x, y);
   if (m.n_layers > 1 && !workspace) return fail(KS_EINVAL, "ks_mlp_forward: workspace required");
   if ((M + kBM - 1) / kBM > 0x7fffffff) return fail(KS_ELIMIT, "ks_mlp_forward: too many rows");
   const int64_t esz = m.dtype == KS_MLP_BF16 ? 2 : 4;
