@@ -10,6 +10,7 @@
 
 #include <cmath>
 #include <cstring>
+#include <cstdlib>
 #include <vector>
 
 namespace ks {
@@ -218,45 +219,171 @@ struct FusedArgs {
   const float* bp[KS_MAX_LAYERS];
   const float* x;
   float* y;
+  long long* prof;  // phase time stamps of wavefront 0, written only by -DKS_PROFILE builds
 };
 
+#ifdef KS_PROFILE
+#define KS_MLP_STAMP(k) if (a.prof && tid == 0) a.prof[(int64_t)blockIdx.x * 32 + (k)] = wall_clock64();
+#else
+#define KS_MLP_STAMP(k)
+#endif
+
+typedef __attribute__((ext_vector_type(2))) float f32x2;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+
+__device__ __forceinline__ unsigned pack_bf16(float lo, float hi) {
+  return __builtin_bit_cast(unsigned, __builtin_convertvector(f32x2{lo, hi}, bf16x2));
+}
+
+// One layer's MFMA work of one wavefront: NT output tiles (weights w[t]) times MI row tiles.  `arow` points at
+// this lane's activation fragment of K step 0 (row lane % 32 of the first row tile, k half lane / 32).
+// Weight fragments sit in a register ring kPF steps ahead; activation fragments are read one step ahead.
 template <int NT, int MI>
 __device__ __forceinline__ void fused_layer_mma(f32x16 (&acc)[2][MI], const u32x4* __restrict__ w0,
-                                                const u32x4* __restrict__ w1, int nk, const __bf16* __restrict__ act,
-                                                int lda, int lane) {
+                                                const u32x4* __restrict__ w1, int nk, const __bf16* __restrict__ arow,
+                                                int lda) {
+  static_assert(kPF % 2 == 0, "the activation double buffer relies on an even ring depth");
   u32x4 rw[kPF][NT];
 #pragma unroll
   for (int u = 0; u < kPF; ++u) {
     const int st = u < nk ? u : nk - 1;
-    rw[u][0] = w0[(int64_t)st * 64];
-    if (NT > 1) rw[u][NT - 1] = w1[(int64_t)st * 64];
+    rw[u][0] = w0[st * 64];
+    if (NT > 1) rw[u][NT - 1] = w1[st * 64];
   }
-  const __bf16* arow = act + (lane & 31) * lda + (lane >> 5) * 8;
-  for (int s = 0; s < nk; s += kPF) {
+  bf16x8 bq[2][MI];
+#pragma unroll
+  for (int i = 0; i < MI; ++i) bq[0][i] = *(const bf16x8*)(arow + i * 32 * lda);
+  int s = 0;
+  for (; s + kPF <= nk; s += kPF) {
 #pragma unroll
     for (int u = 0; u < kPF; ++u) {
-      if (s + u < nk) {
-        bf16x8 bfr[MI];
+      const int step = s + u;
+      const int nstep = step + 1 < nk ? step + 1 : step;
 #pragma unroll
-        for (int i = 0; i < MI; ++i) bfr[i] = *(const bf16x8*)(arow + i * 32 * lda + (s + u) * 16);
-        bf16x8 wf[NT];
+      for (int i = 0; i < MI; ++i) bq[(u + 1) & 1][i] = *(const bf16x8*)(arow + i * 32 * lda + nstep * 16);
+      bf16x8 wf[NT];
 #pragma unroll
-        for (int t = 0; t < NT; ++t) wf[t] = __builtin_bit_cast(bf16x8, rw[u][t]);
-        const int nx = s + u + kPF < nk ? s + u + kPF : nk - 1;
-        rw[u][0] = w0[(int64_t)nx * 64];
-        if (NT > 1) rw[u][NT - 1] = w1[(int64_t)nx * 64];
+      for (int t = 0; t < NT; ++t) wf[t] = __builtin_bit_cast(bf16x8, rw[u][t]);
+      const int nx = step + kPF < nk ? step + kPF : nk - 1;
+      rw[u][0] = w0[nx * 64];
+      if (NT > 1) rw[u][NT - 1] = w1[nx * 64];
 #pragma unroll
-        for (int t = 0; t < NT; ++t)
+      for (int t = 0; t < NT; ++t)
 #pragma unroll
-          for (int i = 0; i < MI; ++i)
-            acc[t][i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[t], bfr[i], acc[t][i], 0, 0, 0);
-      }
+        for (int i = 0; i < MI; ++i)
+          acc[t][i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[t], bq[u & 1][i], acc[t][i], 0, 0, 0);
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < kPF - 1; ++u) {
+    if (s + u < nk) {
+      const int step = s + u;
+      const int nstep = step + 1 < nk ? step + 1 : step;
+#pragma unroll
+      for (int i = 0; i < MI; ++i) bq[(u + 1) & 1][i] = *(const bf16x8*)(arow + i * 32 * lda + nstep * 16);
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int i = 0; i < MI; ++i)
+          acc[t][i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, rw[u][t]), bq[u & 1][i],
+                                                              acc[t][i], 0, 0, 0);
     }
   }
 }
 
+// Accumulator tile layout: lane l, register r -> feature 32 j + 8 (r / 4) + 4 (l / 32) + r % 4 of batch row l % 32.
+__device__ __forceinline__ void fused_bias_init(f32x16& acc, const float* __restrict__ bias, int j, int lane) {
+#pragma unroll
+  for (int g = 0; g < 4; ++g) {
+    const float4 b = *reinterpret_cast<const float4*>(bias + j * 32 + 8 * g + 4 * (lane >> 5));
+    acc[4 * g] = b.x; acc[4 * g + 1] = b.y; acc[4 * g + 2] = b.z; acc[4 * g + 3] = b.w;
+  }
+}
+
+// Hidden layer: activation, round to bf16, back into the tile (4 consecutive features = one 8-byte LDS store).
+template <int ACT>
+__device__ __forceinline__ void fused_store_hidden(const f32x16& acc, __bf16* __restrict__ act, int lda, int j,
+                                                   int row, int lane) {
+#pragma unroll
+  for (int g = 0; g < 4; ++g) {
+    const int f0 = j * 32 + 8 * g + 4 * (lane >> 5);
+    const uint2 packed = {pack_bf16(activate<ACT, true>(acc[4 * g]), activate<ACT, true>(acc[4 * g + 1])),
+                          pack_bf16(activate<ACT, true>(acc[4 * g + 2]), activate<ACT, true>(acc[4 * g + 3]))};
+    *reinterpret_cast<uint2*>(act + row * lda + f0) = packed;
+  }
+}
+
+// Output layer: fp32 rows of the caller's (M, out_dim) matrix.
+__device__ __forceinline__ void fused_store_output(const f32x16& acc, float* __restrict__ y, int64_t M, int out_dim,
+                                                   int j, int64_t m, int lane) {
+  if (m >= M) return;
+#pragma unroll
+  for (int g = 0; g < 4; ++g) {
+    const int f0 = j * 32 + 8 * g + 4 * (lane >> 5);
+    float* dst = y + m * out_dim + f0;
+    if ((out_dim & 3) == 0 && f0 + 4 <= out_dim) {
+      *reinterpret_cast<float4*>(dst) = float4{acc[4 * g], acc[4 * g + 1], acc[4 * g + 2], acc[4 * g + 3]};
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        if (f0 + e < out_dim) dst[e] = acc[4 * g + e];
+    }
+  }
+}
+
+// One layer of the whole-network kernel for one wavefront: MFMA work, barrier, epilogue, barrier.
+template <int ACT, int MI, bool LAST>
+__device__ __forceinline__ void fused_layer(const FusedArgs& a, int l, __bf16* __restrict__ act, int64_t m0, int lane,
+                                            int wave) {
+  const int nk = a.fk[l], nt = a.fn[l], lda = a.lda;
+  const __bf16* arow = act + (lane & 31) * lda + (lane >> 5) * 8;
+  const int row = lane & 31;
+  if (nt * MI <= kFusedWaves) {  // few tiles: one (feature tile, row tile) pair per wavefront
+    const bool busy = wave < nt * MI;
+    const int j = busy ? wave / MI : 0, i = busy ? wave % MI : 0;
+    f32x16 acc[2][1];
+    fused_bias_init(acc[0][0], a.bp[l], j, lane);
+    acc[1][0] = acc[0][0];
+    const u32x4* w0 = a.Wp[l] + (int64_t)j * nk * 64 + lane;
+    if (busy) fused_layer_mma<1, 1>(acc, w0, w0, nk, arow + i * 32 * lda, lda);
+    __syncthreads();  // every wavefront has read this layer's input; the tile can be overwritten
+    if (busy) {
+      if (LAST) fused_store_output(acc[0][0], a.y, a.M, a.out_dim, j, m0 + i * 32 + row, lane);
+      else fused_store_hidden<ACT>(acc[0][0], act, lda, j, i * 32 + row, lane);
+    }
+  } else {
+    const int mine = wave < nt ? (wave + kFusedWaves < nt ? 2 : 1) : 0;
+    const int j0 = wave < nt ? wave : 0, j1 = wave + kFusedWaves < nt ? wave + kFusedWaves : j0;
+    f32x16 acc[2][MI];
+    fused_bias_init(acc[0][0], a.bp[l], j0, lane);
+    fused_bias_init(acc[1][0], a.bp[l], j1, lane);
+#pragma unroll
+    for (int i = 1; i < MI; ++i) {
+      acc[0][i] = acc[0][0];
+      acc[1][i] = acc[1][0];
+    }
+    const u32x4* w0 = a.Wp[l] + (int64_t)j0 * nk * 64 + lane;
+    const u32x4* w1 = a.Wp[l] + (int64_t)j1 * nk * 64 + lane;
+    if (mine == 2) fused_layer_mma<2, MI>(acc, w0, w1, nk, arow, lda);
+    else if (mine == 1) fused_layer_mma<1, MI>(acc, w0, w0, nk, arow, lda);
+    __syncthreads();
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+      if (t < mine) {
+        const int j = t == 0 ? j0 : j1;
+#pragma unroll
+        for (int i = 0; i < MI; ++i) {
+          if (LAST) fused_store_output(acc[t][i], a.y, a.M, a.out_dim, j, m0 + i * 32 + row, lane);
+          else fused_store_hidden<ACT>(acc[t][i], act, lda, j, i * 32 + row, lane);
+        }
+      }
+  }
+  __syncthreads();
+}
+
 template <int ACT, int BM>
-__global__ __launch_bounds__(64 * kFusedWaves) void mlp_fused_kernel(const FusedArgs a) {
+__global__ __launch_bounds__(64 * kFusedWaves) __attribute__((amdgpu_waves_per_eu(BM <= 64 ? 4 : 2, BM <= 64 ? 4 : 2)))
+void mlp_fused_kernel(const FusedArgs a) {
   constexpr int MI = BM / 32;
   constexpr int NTHR = 64 * kFusedWaves;
   extern __shared__ __attribute__((aligned(16))) unsigned char mlp_lds[];
@@ -264,76 +391,68 @@ __global__ __launch_bounds__(64 * kFusedWaves) void mlp_fused_kernel(const Fused
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int64_t m0 = (int64_t)blockIdx.x * BM;
   const int lda = a.lda;
-  {  // network input -> bf16 tile, zero beyond the batch and in the K padding of the first layer
-    const int K0 = a.fk[0] * 16;
+  KS_MLP_STAMP(0)
+  {  // network input -> bf16 tile; zero beyond the batch and in the K padding of the first layer
+    const int K0 = a.fk[0] * 16, in_dim = a.in_dim;
     const int64_t rows_left = a.M - m0;
     const int rows = rows_left < BM ? (int)rows_left : BM;
-    const float* src = a.x + m0 * a.in_dim;
-    const int total = rows * a.in_dim;
-    for (int idx = tid; idx < BM * K0; idx += NTHR) {
-      const int r = idx / K0, c = idx - r * K0;
-      if (r >= rows || c >= a.in_dim) act[r * lda + c] = (__bf16)0.0f;
+    const float* src = a.x + m0 * in_dim;
+    const int padw = K0 - in_dim;
+    for (int idx = tid; idx < BM * padw; idx += NTHR) {
+      const int r = idx / padw, c = idx - r * padw;
+      act[r * lda + in_dim + c] = (__bf16)0.0f;
     }
-    for (int idx = tid; idx < total; idx += NTHR) {
-      const int r = idx / a.in_dim, c = idx - r * a.in_dim;
-      act[r * lda + c] = (__bf16)src[idx];
+    for (int idx = rows * in_dim + tid; idx < BM * in_dim; idx += NTHR) {
+      const int r = idx / in_dim, c = idx - r * in_dim;
+      act[r * lda + c] = (__bf16)0.0f;
     }
-  }
-  __syncthreads();
-  for (int l = 0; l < a.n_layers; ++l) {
-    const int nk = a.fk[l], nt = a.fn[l];
-    const int mine = wave < nt ? (wave + kFusedWaves < nt ? 2 : 1) : 0;
-    const bool last = l == a.n_layers - 1;
-    f32x16 acc[2][MI];
+    if ((in_dim & 3) == 0) {  // rows are 16-byte aligned: four wide loads in flight per thread
+      const float4* src4 = reinterpret_cast<const float4*>(src);
+      const int total4 = rows * in_dim / 4;
+      for (int base = tid; base < total4; base += NTHR * 4) {
+        float4 v[4];
 #pragma unroll
-    for (int t = 0; t < 2; ++t)
+        for (int q = 0; q < 4; ++q) {
+          const int idx = base + q * NTHR;
+          v[q] = idx < total4 ? src4[idx] : float4{0.f, 0.f, 0.f, 0.f};
+        }
 #pragma unroll
-      for (int i = 0; i < MI; ++i)
+        for (int q = 0; q < 4; ++q) {
+          const int idx = base + q * NTHR;
+          if (idx < total4) {
+            const int r = idx * 4 / in_dim, c = idx * 4 - r * in_dim;
+            *reinterpret_cast<uint2*>(act + r * lda + c) = uint2{pack_bf16(v[q].x, v[q].y), pack_bf16(v[q].z, v[q].w)};
+          }
+        }
+      }
+    } else {
+      const int total = rows * in_dim;
+      for (int base = tid; base < total; base += NTHR * 4) {
+        float v[4];
 #pragma unroll
-        for (int r = 0; r < 16; ++r) acc[t][i][r] = 0.f;
-    const u32x4* w0 = a.Wp[l] + (int64_t)wave * nk * 64 + lane;
-    const u32x4* w1 = a.Wp[l] + (int64_t)(wave + kFusedWaves) * nk * 64 + lane;
-    if (mine == 2) fused_layer_mma<2, MI>(acc, w0, w1, nk, act, lda, lane);
-    else if (mine == 1) fused_layer_mma<1, MI>(acc, w0, w0, nk, act, lda, lane);
-    __syncthreads();  // every wavefront has read this layer's input; the tile can be overwritten
+        for (int q = 0; q < 4; ++q) {
+          const int idx = base + q * NTHR;
+          v[q] = idx < total ? src[idx] : 0.f;
+        }
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
-      if (t < mine) {
-        const int j = wave + kFusedWaves * t;
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          const int f0 = j * 32 + 8 * g + 4 * (lane >> 5);
-          const float4 b = *reinterpret_cast<const float4*>(a.bp[l] + f0);
-#pragma unroll
-          for (int i = 0; i < MI; ++i) {
-            const int row = i * 32 + (lane & 31);
-            float v[4] = {acc[t][i][4 * g] + b.x, acc[t][i][4 * g + 1] + b.y, acc[t][i][4 * g + 2] + b.z,
-                          acc[t][i][4 * g + 3] + b.w};
-            if (last) {
-              const int64_t m = m0 + row;
-              if (m < a.M) {
-                float* dst = a.y + m * a.out_dim + f0;
-                if ((a.out_dim & 3) == 0 && f0 + 4 <= a.out_dim) {
-                  *reinterpret_cast<float4*>(dst) = float4{v[0], v[1], v[2], v[3]};
-                } else {
-#pragma unroll
-                  for (int e = 0; e < 4; ++e)
-                    if (f0 + e < a.out_dim) dst[e] = v[e];
-                }
-              }
-            } else {
-              unsigned short hb[4];
-#pragma unroll
-              for (int e = 0; e < 4; ++e) hb[e] = __builtin_bit_cast(unsigned short, (__bf16)activate<ACT, true>(v[e]));
-              const uint2 packed = {(unsigned)hb[0] | ((unsigned)hb[1] << 16), (unsigned)hb[2] | ((unsigned)hb[3] << 16)};
-              *reinterpret_cast<uint2*>(act + row * lda + f0) = packed;
-            }
+        for (int q = 0; q < 4; ++q) {
+          const int idx = base + q * NTHR;
+          if (idx < total) {
+            const int r = idx / in_dim, c = idx - r * in_dim;
+            act[r * lda + c] = (__bf16)v[q];
           }
         }
       }
     }
-    __syncthreads();
   }
+  __syncthreads();
+  KS_MLP_STAMP(1)
+  for (int l = 0; l + 1 < a.n_layers; ++l) {
+    fused_layer<ACT, MI, false>(a, l, act, m0, lane, wave);
+    KS_MLP_STAMP(2 + l)
+  }
+  fused_layer<ACT, MI, true>(a, a.n_layers - 1, act, m0, lane, wave);
+  KS_MLP_STAMP(2 + a.n_layers - 1)
 }
 
 struct DevMlp {
@@ -505,6 +624,9 @@ static int launch_fused_tile(const DevMlp& m, hipStream_t s, int64_t M, const fl
     a.Wp[l] = (const u32x4*)m.Wp[l]; a.bp[l] = m.bp[l];
   }
   a.x = x; a.y = y;
+#ifdef KS_PROFILE
+  if (const char* e = getenv("KS_MLP_PROF_PTR")) a.prof = (long long*)strtoull(e, nullptr, 16);
+#endif
   const int lds = BM * m.lda * 2;
   const int64_t blocks = (M + BM - 1) / BM;
   if (blocks > 0x7fffffff) return fail(KS_ELIMIT, "ks_mlp_forward: too many rows");
@@ -529,6 +651,12 @@ static int launch_fused_tile(const DevMlp& m, hipStream_t s, int64_t M, const fl
 // Row tile: 128 rows amortise each weight fragment over four MFMAs; smaller batches take smaller tiles so that
 // the grid still reaches every CU.
 static int launch_fused(const DevMlp& m, hipStream_t s, int64_t M, const float* x, float* y) {
+  if (const char* e = getenv("KS_MLP_BM")) {
+    const int bm = atoi(e);
+    if (bm == 128) return launch_fused_tile<128>(m, s, M, x, y);
+    if (bm == 64) return launch_fused_tile<64>(m, s, M, x, y);
+    if (bm == 32) return launch_fused_tile<32>(m, s, M, x, y);
+  }
   if (M >= 128 * 256) return launch_fused_tile<128>(m, s, M, x, y);
   if (M >= 64 * 256) return launch_fused_tile<64>(m, s, M, x, y);
   return launch_fused_tile<32>(m, s, M, x, y);
