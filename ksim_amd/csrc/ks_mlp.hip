@@ -224,8 +224,10 @@ struct FusedArgs {
 
 #ifdef KS_PROFILE
 #define KS_MLP_STAMP(k) if (a.prof && tid == 0) a.prof[(int64_t)blockIdx.x * 32 + (k)] = wall_clock64();
+#define KS_MLP_STAMP2(k) if (a.prof && threadIdx.x == 0) a.prof[(int64_t)blockIdx.x * 32 + (k)] = wall_clock64();
 #else
 #define KS_MLP_STAMP(k)
+#define KS_MLP_STAMP2(k)
 #endif
 
 typedef __attribute__((ext_vector_type(2))) float f32x2;
@@ -346,7 +348,9 @@ __device__ __forceinline__ void fused_layer(const FusedArgs& a, int l, __bf16* _
     acc[1][0] = acc[0][0];
     const u32x4* w0 = a.Wp[l] + (int64_t)j * nk * 64 + lane;
     if (busy) fused_layer_mma<1, 1>(acc, w0, w0, nk, arow + i * 32 * lda, lda);
+    KS_MLP_STAMP2(2 + 3 * l)
     __syncthreads();  // every wavefront has read this layer's input; the tile can be overwritten
+    KS_MLP_STAMP2(3 + 3 * l)
     if (busy) {
       if (LAST) fused_store_output(acc[0][0], a.y, a.M, a.out_dim, j, m0 + i * 32 + row, lane);
       else fused_store_hidden<ACT>(acc[0][0], act, lda, j, i * 32 + row, lane);
@@ -366,7 +370,9 @@ __device__ __forceinline__ void fused_layer(const FusedArgs& a, int l, __bf16* _
     const u32x4* w1 = a.Wp[l] + (int64_t)j1 * nk * 64 + lane;
     if (mine == 2) fused_layer_mma<2, MI>(acc, w0, w1, nk, arow, lda);
     else if (mine == 1) fused_layer_mma<1, MI>(acc, w0, w0, nk, arow, lda);
+    KS_MLP_STAMP2(2 + 3 * l)
     __syncthreads();
+    KS_MLP_STAMP2(3 + 3 * l)
 #pragma unroll
     for (int t = 0; t < 2; ++t)
       if (t < mine) {
@@ -379,6 +385,7 @@ __device__ __forceinline__ void fused_layer(const FusedArgs& a, int l, __bf16* _
       }
   }
   __syncthreads();
+  KS_MLP_STAMP2(4 + 3 * l)
 }
 
 template <int ACT, int BM>
@@ -449,10 +456,8 @@ void mlp_fused_kernel(const FusedArgs a) {
   KS_MLP_STAMP(1)
   for (int l = 0; l + 1 < a.n_layers; ++l) {
     fused_layer<ACT, MI, false>(a, l, act, m0, lane, wave);
-    KS_MLP_STAMP(2 + l)
   }
   fused_layer<ACT, MI, true>(a, a.n_layers - 1, act, m0, lane, wave);
-  KS_MLP_STAMP(2 + a.n_layers - 1)
 }
 
 struct DevMlp {
@@ -651,12 +656,14 @@ static int launch_fused_tile(const DevMlp& m, hipStream_t s, int64_t M, const fl
 // Row tile: 128 rows amortise each weight fragment over four MFMAs; smaller batches take smaller tiles so that
 // the grid still reaches every CU.
 static int launch_fused(const DevMlp& m, hipStream_t s, int64_t M, const float* x, float* y) {
+#ifdef KS_PROFILE
   if (const char* e = getenv("KS_MLP_BM")) {
     const int bm = atoi(e);
     if (bm == 128) return launch_fused_tile<128>(m, s, M, x, y);
     if (bm == 64) return launch_fused_tile<64>(m, s, M, x, y);
     if (bm == 32) return launch_fused_tile<32>(m, s, M, x, y);
   }
+#endif
   if (M >= 128 * 256) return launch_fused_tile<128>(m, s, M, x, y);
   if (M >= 64 * 256) return launch_fused_tile<64>(m, s, M, x, y);
   return launch_fused_tile<32>(m, s, M, x, y);

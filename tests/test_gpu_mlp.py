@@ -12,7 +12,7 @@ def reference(x, ws, bs, act, bf16):
     """float64 library reference; for the bf16 path weights and layer inputs are rounded to bf16 first."""
     rnd = (lambda t: t.to(torch.bfloat16).to(torch.float64)) if bf16 else (lambda t: t.to(torch.float64))
     h = torch.from_numpy(x)
-    fn = {"elu": F.elu, "relu": F.relu, "tanh": torch.tanh, None: lambda t: t}[act]
+    fn = {"elu": F.elu, "relu": F.relu, "tanh": torch.tanh, None: lambda t: t, "none": lambda t: t}[act]
     for i, (w, b) in enumerate(zip(ws, bs)):
         h = F.linear(rnd(h.to(torch.float32)), rnd(torch.from_numpy(w)), torch.from_numpy(b).to(torch.float64))
         if i + 1 < len(ws):
@@ -26,6 +26,11 @@ def reference(x, ws, bs, act, bf16):
     ((68, 512, 512, 512, 1), "bf16", "elu", 129),      # config 4 critic, ragged tile
     ((71, 256, 256, 1), "bf16", "relu", 64),           # config 5 discriminator shape
     ((5, 3), "f32", None, 7), ((40, 100, 9), "f32", "tanh", 1), ((33, 130, 130, 2), "bf16", "tanh", 257),
+    ((68, 512, 512, 512, 20), "bf16", "elu", 16384 + 45),   # 64-row tiles of the whole-network kernel
+    ((68, 512, 512, 512, 20), "bf16", "elu", 32768 + 77),   # 128-row tiles
+    ((71, 256, 256, 1), "bf16", "relu", 40000),             # 128-row tiles, one output tile per wavefront
+    ((64, 1024, 8), "bf16", "elu", 500),                    # wider than the whole-network kernel takes: per-layer path
+    ((600, 64, 3), "bf16", "none", 100),
 ])
 def test_mlp_matches_reference(dims, dtype, act, M):
     from ksim_amd.mlp import MLP
@@ -34,7 +39,7 @@ def test_mlp_matches_reference(dims, dtype, act, M):
     ws = [rng.normal(scale=1 / np.sqrt(i), size=(o, i)).astype(np.float32) for i, o in zip(dims[:-1], dims[1:])]
     bs = [rng.normal(scale=0.1, size=o).astype(np.float32) for o in dims[1:]]
     x = rng.normal(size=(M, dims[0])).astype(np.float32)
-    net = MLP(ws, bs, activation=act or "none", dtype=dtype)
+    net = MLP(ws, bs, activation=act if act not in (None, "none") else "none", dtype=dtype)
     y = net(torch.from_numpy(x).to(DEV)).cpu().numpy()
     want = reference(x, ws, bs, act, dtype == "bf16")
     scale = np.abs(want).max()
@@ -54,6 +59,8 @@ def test_mlp_rows_are_independent_and_errors():
     y = net(x)
     y2 = net(x[123:460].contiguous())
     assert torch.equal(y[123:460], y2)
+    big = torch.randn(33000, 68, device=DEV)  # another row tile size, same bits per row
+    assert torch.equal(net(big)[5000:5700], net(big[5000:5700].contiguous()))
     with pytest.raises(_lib.KsError):
         net(torch.randn(4, 67, device=DEV))
     with pytest.raises(_lib.KsError):
