@@ -23,13 +23,21 @@
 namespace ks {
 
 #define KS_SYNC() __syncthreads()
+#ifndef KS_STEP_WAVES
+#define KS_STEP_WAVES 3  // wavefronts per SIMD the register allocation aims at
+#endif
 // Phase timers for kernel tuning: compiled in only with -DKS_PROFILE, which reuses the dbg_M buffer for cycle counts.
 #ifdef KS_PROFILE
 #define KS_TICK(k) { const long long t_now = clock64(); prof[k] += (float)(t_now - t_last); t_last = t_now; }
 #else
 #define KS_TICK(k)
 #endif
-constexpr int NP = 32;  // register rows are padded to 32 columns
+// Register rows (mass matrix, Hessian, Jacobian) are padded from nv to a compile-time width NP, one kernel
+// instantiation per width: the padding rows are unit rows and the padding columns zero, so the factorisation,
+// the triangular solves and the row products run without any bound checks.
+__host__ __device__ inline int padded_nv(int nv) { return nv <= 8 ? 8 : nv <= 16 ? 16 : nv <= 24 ? 24 : nv <= 28 ? 28 : 32; }
+__host__ __device__ inline int m_stride(int nv) { return padded_nv(nv) | 1; }  // odd: conflict-free across lanes
+__host__ __device__ inline int j_stride(int nv) { return padded_nv(nv) % 32 == 0 ? padded_nv(nv) + 4 : padded_nv(nv); }
 
 struct Lds {
   float *qpos, *qvel, *warm, *tau;
@@ -44,7 +52,7 @@ struct Lds {
 __host__ __device__ inline int up4(int n) { return (n + 3) & ~3; }
 
 __host__ __device__ inline int lds_floats(int nb, int nq, int nv, int nu, int ns) {
-  const int nvs = nv | 1, js = up4(nv) % 32 == 0 ? up4(nv) + 4 : up4(nv);
+  const int nvs = m_stride(nv), js = j_stride(nv);
   int n = 0;
   n += up4(nq) + 32 + up4(nv) + up4(nu);                             // qpos qvel(32) warm tau
   n += up4(nb * 3) + up4(nb * 4) + up4(nb * 9) + 2 * up4(nb * 3);      // xpos xquat xmat xanchor xaxis
@@ -85,8 +93,9 @@ __device__ inline Lds carve(float* p, const DevModel& m) {
   return l;
 }
 
-// 32 consecutive floats from a 16-byte aligned LDS address, the same address in every lane (broadcast)
-__device__ __forceinline__ void load32(const float* p, float (&v)[NP]) {
+// NP consecutive floats from a 16-byte aligned LDS address, the same address in every lane (broadcast)
+template <int NP>
+__device__ __forceinline__ void load_row(const float* p, float (&v)[NP]) {
   const float4* q = reinterpret_cast<const float4*>(p);
 #pragma unroll
   for (int k = 0; k < NP / 4; ++k) {
@@ -104,53 +113,49 @@ __device__ __forceinline__ float rsqrt_refined(float x) {
 // In-register Cholesky: lane i holds row i of the symmetric matrix in R[0..n); on return R holds row i of L
 // (zeros above the diagonal) and invd[j] = 1 / L[j][j] (wave-uniform).  Row k of L is fetched from lane k
 // with v_readlane, so there is no LDS traffic and no barrier.
-__device__ __forceinline__ void chol_regs(float (&R)[NP], float (&invd)[NP], int n, int lane) {
+template <int NP>
+__device__ __forceinline__ void chol_regs(float (&R)[NP], float (&invd)[NP], int lane) {
 #pragma unroll
   for (int j = 0; j < NP; ++j) {
-    if (j < n) {
-      float s = R[j], s2 = 0.f;  // two chains halve the dependent-FMA latency of a column
+    float s = R[j], s2 = 0.f;  // two chains halve the dependent-FMA latency of a column
 #pragma unroll
-      for (int k = 0; k + 1 < j; k += 2) {
-        s -= R[k] * lane_bcast(R[k], j);
-        s2 -= R[k + 1] * lane_bcast(R[k + 1], j);
-      }
-      if (j & 1) s -= R[j - 1] * lane_bcast(R[j - 1], j);
-      s += s2;
-      const float piv = fmaxf(lane_bcast(s, j), 1e-30f);
-      const float inv = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, rsqrt_refined(piv))));
-      invd[j] = inv;
-      R[j] = lane > j ? s * inv : (lane == j ? piv * inv : 0.f);
+    for (int k = 0; k + 1 < j; k += 2) {
+      s -= R[k] * lane_bcast(R[k], j);
+      s2 -= R[k + 1] * lane_bcast(R[k + 1], j);
     }
+    if (j & 1) s -= R[j - 1] * lane_bcast(R[j - 1], j);
+    s += s2;
+    const float piv = fmaxf(lane_bcast(s, j), 1e-30f);
+    const float inv = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, rsqrt_refined(piv))));
+    invd[j] = inv;
+    R[j] = lane > j ? s * inv : (lane == j ? piv * inv : 0.f);
   }
 }
 
 // x = (L L^T)^-1 b, lane i holding b_i and returning x_i
-__device__ __forceinline__ float solve_regs(const float (&R)[NP], const float (&invd)[NP], int n, int lane, float b) {
+template <int NP>
+__device__ __forceinline__ float solve_regs(const float (&R)[NP], const float (&invd)[NP], int lane, float b) {
   float r = b;
 #pragma unroll
   for (int j = 0; j < NP; ++j) {
-    if (j < n) {
-      const float xj = lane_bcast(r, j) * invd[j];
-      r = lane == j ? xj : r - R[j] * xj;  // R[j] is zero in lanes < j and >= n
-    }
+    const float xj = lane_bcast(r, j) * invd[j];
+    r = lane == j ? xj : r - R[j] * xj;  // R[j] is zero in lanes < j and in lanes that hold no row
   }
   // Backward substitution, four columns per batch: the four cross-lane sums over the already solved rows are
   // independent (their DPP chains interleave); the 4x4 triangle inside the batch is resolved with lane reads.
 #pragma unroll
   for (int jb = NP - 4; jb >= 0; jb -= 4) {
-    if (jb < n) {
-      float s[4], x[4];
+    float s[4], x[4];
 #pragma unroll
-      for (int c = 0; c < 4; ++c) s[c] = wave_sum(lane > jb + 3 ? R[jb + c] * r : 0.f);
+    for (int c = 0; c < 4; ++c) s[c] = jb + 4 < NP ? wave_sum(lane > jb + 3 ? R[jb + c] * r : 0.f) : 0.f;
 #pragma unroll
-      for (int c = 3; c >= 0; --c) {
-        const int j = jb + c;
-        float acc = lane_bcast(r, j) - s[c];
+    for (int c = 3; c >= 0; --c) {
+      const int j = jb + c;
+      float acc = lane_bcast(r, j) - s[c];
 #pragma unroll
-        for (int d = c + 1; d < 4; ++d) acc -= lane_bcast(R[j], jb + d) * x[d];  // L[jb+d][j] lives in lane jb+d
-        x[c] = (j < n) ? acc * invd[j] : 0.f;
-        if (lane == j) r = x[c];
-      }
+      for (int d = c + 1; d < 4; ++d) acc -= lane_bcast(R[j], jb + d) * x[d];  // L[jb+d][j] lives in lane jb+d
+      x[c] = acc * invd[j];
+      if (lane == j) r = x[c];
     }
   }
   return r;
@@ -158,30 +163,30 @@ __device__ __forceinline__ float solve_regs(const float (&R)[NP], const float (&
 
 
 // dot product of an LDS row (per-lane address, odd stride between lanes) with a broadcast register vector
-__device__ __forceinline__ float row_dot(const float* row, int n, const float (&vv)[NP]) {
+template <int NP>
+__device__ __forceinline__ float row_dot(const float* row, const float (&vv)[NP]) {
   float s0 = 0.f, s1 = 0.f;
 #pragma unroll
   for (int j = 0; j < NP; j += 2) {
-    if (j < n) s0 += row[j] * vv[j];
-    if (j + 1 < n) s1 += row[j + 1] * vv[j + 1];
+    s0 += row[j] * vv[j];
+    s1 += row[j + 1] * vv[j + 1];
   }
   return s0 + s1;
 }
 
 // Row r of the constraint Jacobian (LDS, 16-byte aligned rows) times a vector in LDS.  Lane r starts at column
-// r mod n and walks cyclically, which spreads the lanes over the LDS banks although the row stride is a multiple of 4.
-__device__ __forceinline__ float jrow_dot(const float* row, int n, const float* v, int lane) {
-  int c = lane;
-  while (c >= n) c -= n;
+// r mod NP and walks cyclically, which spreads the lanes over the LDS banks although the row stride is a multiple of 4.
+template <int NP>
+__device__ __forceinline__ float jrow_dot(const float* row, const float* v, int lane) {
+  int c = lane % NP;
   float s0 = 0.f, s1 = 0.f;
-#pragma unroll 4
-  for (int j = 0; j + 1 < n; j += 2) {
-    const int c1 = c + 1 == n ? 0 : c + 1;
+#pragma unroll
+  for (int j = 0; j < NP; j += 2) {
+    const int c1 = c + 1 == NP ? 0 : c + 1;
     s0 += row[c] * v[c];
     s1 += row[c1] * v[c1];
-    c = c1 + 1 == n ? 0 : c1 + 1;
+    c = c1 + 1 == NP ? 0 : c1 + 1;
   }
-  if (n & 1) s0 += row[c] * v[c];
   return s0 + s1;
 }
 
@@ -208,8 +213,9 @@ __device__ __forceinline__ float range_sum(const float* base, int w, int b, int 
 // ------------------------------------------------------------------------------------------- the fused kernel
 // FWD = true is the forward-only variant (derived fields + warm start of a given state, no actuation, no
 // integration) that replaces the mjx.forward of a reset.
-template <bool FWD>
-__global__ __launch_bounds__(64) void step_kernel(StepArgs a) {
+template <bool FWD, int NP>
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(KS_STEP_WAVES, KS_STEP_WAVES)))
+void step_kernel(StepArgs a) {
   extern __shared__ __attribute__((aligned(16))) float lds_raw[];
   const DevModel& m = *a.model;
   const int lane = threadIdx.x;
@@ -526,9 +532,9 @@ __global__ __launch_bounds__(64) void step_kernel(StepArgs a) {
     // ---- Cholesky of M and the unconstrained acceleration (registers only)
     float R[NP], invd[NP];
 #pragma unroll
-    for (int j = 0; j < NP; ++j) { R[j] = (is_dof && j < nv) ? Mrow[j] : 0.f; invd[j] = 0.f; }
-    chol_regs(R, invd, nv, lane);
-    const float qas = solve_regs(R, invd, nv, lane, qfs);
+    for (int j = 0; j < NP; ++j) { R[j] = is_dof ? Mrow[j] : (lane == j ? 1.f : 0.f); invd[j] = 0.f; }
+    chol_regs<NP>(R, invd, lane);
+    const float qas = solve_regs<NP>(R, invd, lane, qfs);
     if (a.dbg_qacc_smooth && is_dof) a.dbg_qacc_smooth[env * nv + lane] = qas;
 
     KS_TICK(7)
@@ -546,19 +552,19 @@ __global__ __launch_bounds__(64) void step_kernel(StepArgs a) {
         unsigned um = 0;  // union of the dof masks of the active contacts (wave-uniform)
         for (int k = 0; k < ncon; ++k) um |= l.con_mask[k];
         float vv[NP];
-        load32(l.qvel, vv);
+        load_row<NP>(l.qvel, vv);
         float vel = 0.f;
 #pragma unroll
         for (int j = 0; j < NP; ++j) {
           float val = 0.f;
-          if (j < nv && ((um >> j) & 1u)) {
+          if ((um >> j) & 1u) {
             const Sp cd = ld6(l.cdof + 6 * j);
             const V3 jac = cd.l + cross(cd.a, off);
             const float tang = (q < 2) ? jac.y : -jac.x;
             val = ((cm >> j) & 1u) ? jac.z + smu * tang : 0.f;
           }
           vel += val * vv[j];
-          if (is_row && j < nv) l.J[lane * js + j] = val;
+          if (is_row) l.J[lane * js + j] = val;
         }
         if (is_row) {
           aref = -m.con_b * vel - l.con_kip[c];
@@ -575,15 +581,15 @@ __global__ __launch_bounds__(64) void step_kernel(StepArgs a) {
         float vv[NP];
         if (lane < 32) l.vbuf[lane] = warm;
         KS_SYNC();
-        load32(l.vbuf, vv);
-        if (is_dof) Ma_w = row_dot(Mrow, nv, vv);
-        if (is_row) Jar_w = jrow_dot(l.J + lane * js, nv, l.vbuf, lane) - aref;
+        load_row<NP>(l.vbuf, vv);
+        if (is_dof) Ma_w = row_dot<NP>(Mrow, vv);
+        if (is_row) Jar_w = jrow_dot<NP>(l.J + lane * js, l.vbuf, lane) - aref;
         KS_SYNC();
         if (lane < 32) l.vbuf[lane] = qas;
         KS_SYNC();
-        load32(l.vbuf, vv);
-        if (is_dof) Ma_s = row_dot(Mrow, nv, vv);
-        if (is_row) Jar_s = jrow_dot(l.J + lane * js, nv, l.vbuf, lane) - aref;
+        load_row<NP>(l.vbuf, vv);
+        if (is_dof) Ma_s = row_dot<NP>(Mrow, vv);
+        if (is_row) Jar_s = jrow_dot<NP>(l.J + lane * js, l.vbuf, lane) - aref;
       }
       const float cost_w = wave_sum((is_row && Jar_w < 0.f) ? 0.5f * D * Jar_w * Jar_w : 0.f) +
                            0.5f * wave_sum(is_dof ? (Ma_w - qfs) * (warm - qas) : 0.f);
@@ -625,7 +631,7 @@ __global__ __launch_bounds__(64) void step_kernel(StepArgs a) {
         KS_TICK(10)
         // ---- Newton direction: H = M + J^T diag(D active) J, row per lane, in registers
 #pragma unroll
-        for (int j = 0; j < NP; ++j) R[j] = (is_dof && j < nv) ? Mrow[j] : 0.f;
+        for (int j = 0; j < NP; ++j) R[j] = is_dof ? Mrow[j] : (lane == j ? 1.f : 0.f);
         {
           unsigned long long t = am;
           while (t) {  // two constraint rows per pass so that the LDS loads of one overlap the FMAs of the other
@@ -637,16 +643,15 @@ __global__ __launch_bounds__(64) void step_kernel(StepArgs a) {
             const float c0 = is_dof ? lane_bcast(D, r0) * l.J[r0 * js + lane] : 0.f;
             const float c1 = (is_dof && two) ? lane_bcast(D, r1) * l.J[r1 * js + lane] : 0.f;
             float j0[NP], j1[NP];
-            load32(l.J + r0 * js, j0);
-            load32(l.J + r1 * js, j1);
+            load_row<NP>(l.J + r0 * js, j0);
+            load_row<NP>(l.J + r1 * js, j1);
 #pragma unroll
-            for (int j = 0; j < NP; ++j)
-              if (j < nv) R[j] += c0 * j0[j] + c1 * j1[j];
+            for (int j = 0; j < NP; ++j) R[j] += c0 * j0[j] + c1 * j1[j];
           }
         }
         KS_TICK(11)
-        chol_regs(R, invd, nv, lane);
-        const float search = -solve_regs(R, invd, nv, lane, grad);
+        chol_regs<NP>(R, invd, lane);
+        const float search = -solve_regs<NP>(R, invd, lane, grad);
         KS_TICK(12)
 
         // ---- exact line search along `search`
@@ -656,9 +661,9 @@ __global__ __launch_bounds__(64) void step_kernel(StepArgs a) {
           KS_SYNC();
           if (lane < 32) l.vbuf[lane] = search;
           KS_SYNC();
-          load32(l.vbuf, vv);
-          if (is_dof) mv = row_dot(Mrow, nv, vv);
-          if (is_row) jv = jrow_dot(l.J + lane * js, nv, l.vbuf, lane);
+          load_row<NP>(l.vbuf, vv);
+          if (is_dof) mv = row_dot<NP>(Mrow, vv);
+          if (is_row) jv = jrow_dot<NP>(l.J + lane * js, l.vbuf, lane);
         }
         const float smag = sqrtf(wave_sum(search * search)) * m.meaninertia * (float)(nv > 1 ? nv : 1);
         const float gtol = m.tolerance * m.ls_tolerance * smag;
@@ -798,8 +803,8 @@ extern "C" int ks_model_create(const KsModelDesc* d, KsModel** out) {
   std::memset(&m, 0, sizeof(m));
   m.nb = d->nb; m.nq = d->nq; m.nv = d->nv; m.nu = d->nu; m.ns = d->ns;
   m.iterations = d->iterations; m.ls_iterations = d->ls_iterations; m.eulerdamp = d->eulerdamp;
-  m.nvs = d->nv | 1;
-  m.js = up4(d->nv) % 32 == 0 ? up4(d->nv) + 4 : up4(d->nv);
+  m.nvs = m_stride(d->nv);
+  m.js = j_stride(d->nv);
   m.dt = (float)d->dt;
   for (int k = 0; k < 3; ++k) m.gravity[k] = (float)d->gravity[k];
   m.tolerance = (float)d->tolerance; m.ls_tolerance = (float)d->ls_tolerance;
@@ -932,13 +937,18 @@ static int launch_step(const KsModel* km, ks_stream_t stream, const KsStepIO* io
   }
   const int bytes = lds_floats(m.nb, m.nq, m.nv, m.nu, m.ns) * 4;
   if (bytes > 160 * 1024) return fail(KS_ELIMIT, "ks_step: model needs %d bytes of LDS", bytes);
-  const void* fn = forward_only ? (const void*)step_kernel<true> : (const void*)step_kernel<false>;
+  void (*fn)(StepArgs) = nullptr;
+  switch (padded_nv(m.nv)) {
+#define KS_CASE(W) case W: fn = forward_only ? step_kernel<true, W> : step_kernel<false, W>; break;
+    KS_CASE(8) KS_CASE(16) KS_CASE(24) KS_CASE(28) KS_CASE(32)
+#undef KS_CASE
+    default: return fail(KS_ELIMIT, "ks_step: no kernel for %d dofs", m.nv);
+  }
   if (bytes > 64 * 1024) {
-    hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    hipError_t e = hipFuncSetAttribute((const void*)fn, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
     if (e != hipSuccess) return fail(KS_ELAUNCH, "ks_step: cannot raise the LDS limit: %s", hipGetErrorString(e));
   }
-  if (forward_only) hipLaunchKernelGGL(step_kernel<true>, dim3((unsigned)io->N), dim3(64), bytes, (hipStream_t)stream, a);
-  else hipLaunchKernelGGL(step_kernel<false>, dim3((unsigned)io->N), dim3(64), bytes, (hipStream_t)stream, a);
+  hipLaunchKernelGGL(fn, dim3((unsigned)io->N), dim3(64), bytes, (hipStream_t)stream, a);
   return check_launch("ks_step");
 }
 
