@@ -110,57 +110,47 @@ __device__ __forceinline__ float rsqrt_refined(float x) {
   return y;
 }
 
-// In-register Cholesky: lane i holds row i of the symmetric matrix in R[0..n); on return R holds row i of L
-// (zeros above the diagonal) and invd[j] = 1 / L[j][j] (wave-uniform).  Row k of L is fetched from lane k
-// with v_readlane, so there is no LDS traffic and no barrier.
+// In-register Cholesky, right-looking on the full symmetric rows: lane i holds row i of the matrix in R[0..NP).
+// Step j scales column j below the diagonal into L and subtracts the rank-1 term from every later row, all
+// NP-1-j updates of a step being independent FMAs.  Row j of the running Schur complement is fetched from lane
+// j with v_readlane, so there is no LDS traffic and no barrier.  On return, in lane i:
+//   R[j], j < i : L[i][j]                       (row i of L, for the forward substitution)
+//   R[k], k > i : L[k][i] * L[i][i]             (column i of L times its pivot root, for the backward one)
+// invd[j] = 1 / L[j][j] is wave-uniform and myinv = invd[i].  Keeping both triangles makes both substitutions
+// column-oriented: one lane read and one FMA per column, no cross-lane sums.
 template <int NP>
-__device__ __forceinline__ void chol_regs(float (&R)[NP], float (&invd)[NP], int lane) {
+__device__ __forceinline__ void chol_regs(float (&R)[NP], float (&invd)[NP], float& myinv, int lane) {
+  myinv = 1.f;
 #pragma unroll
   for (int j = 0; j < NP; ++j) {
-    float s = R[j], s2 = 0.f;  // two chains halve the dependent-FMA latency of a column
-#pragma unroll
-    for (int k = 0; k + 1 < j; k += 2) {
-      s -= R[k] * lane_bcast(R[k], j);
-      s2 -= R[k + 1] * lane_bcast(R[k + 1], j);
-    }
-    if (j & 1) s -= R[j - 1] * lane_bcast(R[j - 1], j);
-    s += s2;
-    const float piv = fmaxf(lane_bcast(s, j), 1e-30f);
+    const float piv = fmaxf(lane_bcast(R[j], j), 1e-30f);
     const float inv = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, rsqrt_refined(piv))));
     invd[j] = inv;
-    R[j] = lane > j ? s * inv : (lane == j ? piv * inv : 0.f);
+    const bool below = lane > j;
+    myinv = lane == j ? inv : myinv;
+    const float w = below ? R[j] * (inv * inv) : 0.f;
+    R[j] = below ? R[j] * inv : R[j];
+#pragma unroll
+    for (int k = j + 1; k < NP; ++k) R[k] -= w * lane_bcast(R[k], j);
   }
 }
 
 // x = (L L^T)^-1 b, lane i holding b_i and returning x_i
 template <int NP>
-__device__ __forceinline__ float solve_regs(const float (&R)[NP], const float (&invd)[NP], int lane, float b) {
+__device__ __forceinline__ float solve_regs(const float (&R)[NP], const float (&invd)[NP], float myinv, int lane, float b) {
   float r = b;
 #pragma unroll
-  for (int j = 0; j < NP; ++j) {
-    const float xj = lane_bcast(r, j) * invd[j];
-    r = lane == j ? xj : r - R[j] * xj;  // R[j] is zero in lanes < j and in lanes that hold no row
+  for (int j = 0; j < NP; ++j) {  // L y = b; lane j keeps r_j = y_j * L[j][j]
+    const float yj = lane_bcast(r, j) * invd[j];
+    r = lane > j ? r - R[j] * yj : r;
   }
-  // Backward substitution, four columns per batch: the four cross-lane sums over the already solved rows are
-  // independent (their DPP chains interleave); the 4x4 triangle inside the batch is resolved with lane reads.
 #pragma unroll
-  for (int jb = NP - 4; jb >= 0; jb -= 4) {
-    float s[4], x[4];
-#pragma unroll
-    for (int c = 0; c < 4; ++c) s[c] = jb + 4 < NP ? wave_sum(lane > jb + 3 ? R[jb + c] * r : 0.f) : 0.f;
-#pragma unroll
-    for (int c = 3; c >= 0; --c) {
-      const int j = jb + c;
-      float acc = lane_bcast(r, j) - s[c];
-#pragma unroll
-      for (int d = c + 1; d < 4; ++d) acc -= lane_bcast(R[j], jb + d) * x[d];  // L[jb+d][j] lives in lane jb+d
-      x[c] = acc * invd[j];
-      if (lane == j) r = x[c];
-    }
+  for (int k = NP - 1; k >= 0; --k) {  // L^T x = y in the scaled form  sum_{k>i} R[k] x_k + L[i][i]^2 x_i = r_i
+    const float xk = lane_bcast(r, k) * (invd[k] * invd[k]);
+    r = lane < k ? r - R[k] * xk : r;
   }
-  return r;
+  return r * (myinv * myinv);
 }
-
 
 // dot product of an LDS row (per-lane address, odd stride between lanes) with a broadcast register vector
 template <int NP>
@@ -533,8 +523,9 @@ void step_kernel(StepArgs a) {
     float R[NP], invd[NP];
 #pragma unroll
     for (int j = 0; j < NP; ++j) { R[j] = is_dof ? Mrow[j] : (lane == j ? 1.f : 0.f); invd[j] = 0.f; }
-    chol_regs<NP>(R, invd, lane);
-    const float qas = solve_regs<NP>(R, invd, lane, qfs);
+    float myinv;
+    chol_regs<NP>(R, invd, myinv, lane);
+    const float qas = solve_regs<NP>(R, invd, myinv, lane, qfs);
     if (a.dbg_qacc_smooth && is_dof) a.dbg_qacc_smooth[env * nv + lane] = qas;
 
     KS_TICK(7)
@@ -650,8 +641,8 @@ void step_kernel(StepArgs a) {
           }
         }
         KS_TICK(11)
-        chol_regs<NP>(R, invd, lane);
-        const float search = -solve_regs<NP>(R, invd, lane, grad);
+        chol_regs<NP>(R, invd, myinv, lane);
+        const float search = -solve_regs<NP>(R, invd, myinv, lane, grad);
         KS_TICK(12)
 
         // ---- exact line search along `search`
