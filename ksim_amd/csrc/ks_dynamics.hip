@@ -22,6 +22,8 @@
 
 namespace ks {
 
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+
 #define KS_SYNC() __syncthreads()
 #ifndef KS_STEP_WAVES
 #define KS_STEP_WAVES 3  // wavefronts per SIMD the register allocation aims at
@@ -43,7 +45,7 @@ struct Lds {
   float *qpos, *qvel, *warm, *tau;
   float *xpos, *xquat, *xmat, *xanchor, *xaxis;
   float *cinert, *crb, *cdof, *buf, *cvel, *cacc, *cfrc, *fsub;
-  float *M, *J, *vbuf;
+  float *M, *J, *vbuf, *drow;
   float *con_off, *con_D, *con_kip;
   int *con_body, *sub_end;
   unsigned* con_mask;
@@ -60,7 +62,7 @@ __host__ __device__ inline int lds_floats(int nb, int nq, int nv, int nu, int ns
   const int scratch = 2 * up4(nb * 10) + up4(nv * 6) + 3 * up4(nb * 6);  // cinert crb buf cacc cfrc fsub
   const int jsz = up4(4 * ns * js + 32);                             // J overlays that scratch once it is dead
   n += scratch > jsz ? scratch : jsz;
-  n += up4(nv * nvs) + 32;                                           // M vbuf
+  n += up4(nv * nvs) + 32 + 64;                                      // M vbuf drow
   n += up4(ns * 3) + 4 * up4(ns) + up4(nb);                          // con_off con_D con_kip con_body con_mask sub_end
   return n + 8;
 }
@@ -85,7 +87,7 @@ __device__ inline Lds carve(float* p, const DevModel& m) {
     float* jend = base + up4(4 * ns * js + 32);
     p = end > jend ? end : jend;
   }
-  l.M = take(nv * nvs); l.vbuf = take(32);
+  l.M = take(nv * nvs); l.vbuf = take(32); l.drow = take(64);
   l.con_off = take(ns * 3); l.con_D = take(ns); l.con_kip = take(ns);
   l.con_body = reinterpret_cast<int*>(take(ns));
   l.con_mask = reinterpret_cast<unsigned*>(take(ns));
@@ -620,25 +622,33 @@ void step_kernel(StepArgs a) {
         done |= gradient < m.tolerance;
         if (done && !(m.iterations == 1 && niter == 0)) break;
         KS_TICK(10)
-        // ---- Newton direction: H = M + J^T diag(D active) J, row per lane, in registers
-#pragma unroll
-        for (int j = 0; j < NP; ++j) R[j] = is_dof ? Mrow[j] : (lane == j ? 1.f : 0.f);
+        // ---- Newton direction: H = M + J^T diag(D active) J.  The rank-nefc term runs on the matrix cores: one
+        // 32x32x2 fp32 MFMA per pair of constraint rows, operands straight from the LDS copy of J (lane = column,
+        // lane half = row of the pair).  The accumulator tile holds, in lane c, rows {8g + 4 (lane / 32) + e} of
+        // column c, which by symmetry is row c: the upper lane half hands its 16 entries to the lower one and
+        // lane i < 32 ends up with row i of H in registers, as the factorisation wants it.
+        l.drow[lane] = active ? D : 0.f;
+        KS_SYNC();
         {
-          unsigned long long t = am;
-          while (t) {  // two constraint rows per pass so that the LDS loads of one overlap the FMAs of the other
-            const int r0 = __builtin_ctzll(t);
-            t &= t - 1;
-            const bool two = t != 0;
-            const int r1 = two ? __builtin_ctzll(t) : r0;
-            if (two) t &= t - 1;
-            const float c0 = is_dof ? lane_bcast(D, r0) * l.J[r0 * js + lane] : 0.f;
-            const float c1 = (is_dof && two) ? lane_bcast(D, r1) * l.J[r1 * js + lane] : 0.f;
-            float j0[NP], j1[NP];
-            load_row<NP>(l.J + r0 * js, j0);
-            load_row<NP>(l.J + r1 * js, j1);
+          f32x16 hc;
 #pragma unroll
-            for (int j = 0; j < NP; ++j) R[j] += c0 * j0[j] + c1 * j1[j];
+          for (int q = 0; q < 16; ++q) hc[q] = 0.f;
+          const int col = lane & 31, half = lane >> 5;
+          const bool col_ok = NP == 32 || col < NP;
+          for (int r0 = 0; r0 < nefc; r0 += 2) {
+            const int r = r0 + half;
+            const float jv = (col_ok && r < nefc) ? l.J[r * js + col] : 0.f;
+            hc = __builtin_amdgcn_mfma_f32_32x32x2f32(l.drow[r] * jv, jv, hc, 0, 0, 0);
           }
+#pragma unroll
+          for (int g = 0; g < 4; ++g)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const float other = __shfl_xor(hc[4 * g + e], 32);
+              const int jlo = 8 * g + e, jhi = 8 * g + 4 + e;
+              if (jlo < NP) R[jlo] = is_dof ? Mrow[jlo] + hc[4 * g + e] : (lane == jlo ? 1.f : 0.f);
+              if (jhi < NP) R[jhi] = is_dof ? Mrow[jhi] + other : (lane == jhi ? 1.f : 0.f);
+            }
         }
         KS_TICK(11)
         chol_regs<NP>(R, invd, myinv, lane);
