@@ -38,8 +38,11 @@ typedef __attribute__((ext_vector_type(16))) float f32x16;
 // instantiation per width: the padding rows are unit rows and the padding columns zero, so the factorisation,
 // the triangular solves and the row products run without any bound checks.
 __host__ __device__ inline int padded_nv(int nv) { return nv <= 8 ? 8 : nv <= 16 ? 16 : nv <= 24 ? 24 : nv <= 28 ? 28 : 32; }
-__host__ __device__ inline int m_stride(int nv) { return padded_nv(nv) | 1; }  // odd: conflict-free across lanes
-__host__ __device__ inline int j_stride(int nv) { return padded_nv(nv) % 32 == 0 ? padded_nv(nv) + 4 : padded_nv(nv); }
+// Row stride of M and J in LDS: rows are 16-byte aligned (read with ds_read_b128, one row per lane) and the
+// stride in 16-byte units is odd, which spreads 16 consecutive rows over all 64 banks.
+__host__ __device__ inline int row_stride(int nv) { return (padded_nv(nv) / 4) % 2 ? padded_nv(nv) : padded_nv(nv) + 4; }
+__host__ __device__ inline int m_stride(int nv) { return row_stride(nv); }
+__host__ __device__ inline int j_stride(int nv) { return row_stride(nv); }
 
 struct Lds {
   float *qpos, *qvel, *warm, *tau;
@@ -95,7 +98,7 @@ __device__ inline Lds carve(float* p, const DevModel& m) {
   return l;
 }
 
-// NP consecutive floats from a 16-byte aligned LDS address, the same address in every lane (broadcast)
+// NP consecutive floats from a 16-byte aligned LDS address
 template <int NP>
 __device__ __forceinline__ void load_row(const float* p, float (&v)[NP]) {
   const float4* q = reinterpret_cast<const float4*>(p);
@@ -154,30 +157,16 @@ __device__ __forceinline__ float solve_regs(const float (&R)[NP], const float (&
   return r * (myinv * myinv);
 }
 
-// dot product of an LDS row (per-lane address, odd stride between lanes) with a broadcast register vector
+// dot product of an LDS row (per-lane address, 16-byte aligned) with a broadcast register vector
 template <int NP>
 __device__ __forceinline__ float row_dot(const float* row, const float (&vv)[NP]) {
+  const float4* q = reinterpret_cast<const float4*>(row);
   float s0 = 0.f, s1 = 0.f;
 #pragma unroll
-  for (int j = 0; j < NP; j += 2) {
-    s0 += row[j] * vv[j];
-    s1 += row[j + 1] * vv[j + 1];
-  }
-  return s0 + s1;
-}
-
-// Row r of the constraint Jacobian (LDS, 16-byte aligned rows) times a vector in LDS.  Lane r starts at column
-// r mod NP and walks cyclically, which spreads the lanes over the LDS banks although the row stride is a multiple of 4.
-template <int NP>
-__device__ __forceinline__ float jrow_dot(const float* row, const float* v, int lane) {
-  int c = lane % NP;
-  float s0 = 0.f, s1 = 0.f;
-#pragma unroll
-  for (int j = 0; j < NP; j += 2) {
-    const int c1 = c + 1 == NP ? 0 : c + 1;
-    s0 += row[c] * v[c];
-    s1 += row[c1] * v[c1];
-    c = c1 + 1 == NP ? 0 : c1 + 1;
+  for (int k = 0; k < NP / 4; ++k) {
+    const float4 t = q[k];
+    s0 += t.x * vv[4 * k] + t.z * vv[4 * k + 2];
+    s1 += t.y * vv[4 * k + 1] + t.w * vv[4 * k + 3];
   }
   return s0 + s1;
 }
@@ -470,7 +459,7 @@ void step_kernel(StepArgs a) {
 
     KS_TICK(4)
     // ---- mass-matrix row into registers; smooth forces: passive - bias + actuator
-    const float* Mrow = l.M + (is_dof ? lane : 0) * nvs;  // row stride is odd: conflict-free across lanes
+    const float* Mrow = l.M + (is_dof ? lane : 0) * nvs;
     float qfs = 0.f, my_qvel = 0.f;
     if (is_dof) {
       my_qvel = l.qvel[lane];
@@ -523,8 +512,9 @@ void step_kernel(StepArgs a) {
     KS_TICK(6)
     // ---- Cholesky of M and the unconstrained acceleration (registers only)
     float R[NP], invd[NP];
+    load_row<NP>(Mrow, R);
 #pragma unroll
-    for (int j = 0; j < NP; ++j) { R[j] = is_dof ? Mrow[j] : (lane == j ? 1.f : 0.f); invd[j] = 0.f; }
+    for (int j = 0; j < NP; ++j) { R[j] = is_dof ? R[j] : (lane == j ? 1.f : 0.f); invd[j] = 0.f; }
     float myinv;
     chol_regs<NP>(R, invd, myinv, lane);
     const float qas = solve_regs<NP>(R, invd, myinv, lane, qfs);
@@ -576,13 +566,13 @@ void step_kernel(StepArgs a) {
         KS_SYNC();
         load_row<NP>(l.vbuf, vv);
         if (is_dof) Ma_w = row_dot<NP>(Mrow, vv);
-        if (is_row) Jar_w = jrow_dot<NP>(l.J + lane * js, l.vbuf, lane) - aref;
+        if (is_row) Jar_w = row_dot<NP>(l.J + (is_row ? lane : 0) * js, vv) - aref;
         KS_SYNC();
         if (lane < 32) l.vbuf[lane] = qas;
         KS_SYNC();
         load_row<NP>(l.vbuf, vv);
         if (is_dof) Ma_s = row_dot<NP>(Mrow, vv);
-        if (is_row) Jar_s = jrow_dot<NP>(l.J + lane * js, l.vbuf, lane) - aref;
+        if (is_row) Jar_s = row_dot<NP>(l.J + (is_row ? lane : 0) * js, vv) - aref;
       }
       const float cost_w = wave_sum((is_row && Jar_w < 0.f) ? 0.5f * D * Jar_w * Jar_w : 0.f) +
                            0.5f * wave_sum(is_dof ? (Ma_w - qfs) * (warm - qas) : 0.f);
@@ -633,6 +623,8 @@ void step_kernel(StepArgs a) {
           f32x16 hc;
 #pragma unroll
           for (int q = 0; q < 16; ++q) hc[q] = 0.f;
+          float mr[NP];
+          load_row<NP>(Mrow, mr);
           const int col = lane & 31, half = lane >> 5;
           const bool col_ok = NP == 32 || col < NP;
           for (int r0 = 0; r0 < nefc; r0 += 2) {
@@ -646,8 +638,8 @@ void step_kernel(StepArgs a) {
             for (int e = 0; e < 4; ++e) {
               const float other = __shfl_xor(hc[4 * g + e], 32);
               const int jlo = 8 * g + e, jhi = 8 * g + 4 + e;
-              if (jlo < NP) R[jlo] = is_dof ? Mrow[jlo] + hc[4 * g + e] : (lane == jlo ? 1.f : 0.f);
-              if (jhi < NP) R[jhi] = is_dof ? Mrow[jhi] + other : (lane == jhi ? 1.f : 0.f);
+              if (jlo < NP) R[jlo] = is_dof ? mr[jlo] + hc[4 * g + e] : (lane == jlo ? 1.f : 0.f);
+              if (jhi < NP) R[jhi] = is_dof ? mr[jhi] + other : (lane == jhi ? 1.f : 0.f);
             }
         }
         KS_TICK(11)
@@ -664,7 +656,7 @@ void step_kernel(StepArgs a) {
           KS_SYNC();
           load_row<NP>(l.vbuf, vv);
           if (is_dof) mv = row_dot<NP>(Mrow, vv);
-          if (is_row) jv = jrow_dot<NP>(l.J + lane * js, l.vbuf, lane);
+          if (is_row) jv = row_dot<NP>(l.J + (is_row ? lane : 0) * js, vv);
         }
         const float smag = sqrtf(wave_sum(search * search)) * m.meaninertia * (float)(nv > 1 ? nv : 1);
         const float gtol = m.tolerance * m.ls_tolerance * smag;

@@ -19,7 +19,7 @@ enum { kJntNone = 0, kJntFree = 1, kJntHinge = 2 };
 // Immutable after ks_model_create(); lives in device global memory and is read through the
 // vector L1 / scalar cache (it is ~10 KB and shared by every wavefront).
 struct DevModel {
-  int nb, nq, nv, nu, ns, iterations, ls_iterations, eulerdamp, npairs, nvs /* odd row stride */, max_depth,
+  int nb, nq, nv, nu, ns, iterations, ls_iterations, eulerdamp, npairs, nvs /* row stride of the mass matrix in LDS, a multiple of 4 */, max_depth,
       js /* row stride of the constraint Jacobian in LDS, a multiple of 4 */;
   float dt, gravity[3], tolerance, ls_tolerance, meaninertia, friction, impratio;
   // contact impedance constants, already clamped the way the constraint builder wants them
