@@ -121,16 +121,16 @@ __device__ __forceinline__ float rsqrt_refined(float x) {
 // j with v_readlane, so there is no LDS traffic and no barrier.  On return, in lane i:
 //   R[j], j < i : L[i][j]                       (row i of L, for the forward substitution)
 //   R[k], k > i : L[k][i] * L[i][i]             (column i of L times its pivot root, for the backward one)
-// invd[j] = 1 / L[j][j] is wave-uniform and myinv = invd[i].  Keeping both triangles makes both substitutions
-// column-oriented: one lane read and one FMA per column, no cross-lane sums.
+// and myinv = 1 / L[i][i] (kept per lane rather than as NP wave-uniform values, which would sit in scalar
+// registers the kernel is short of).  Keeping both triangles makes both substitutions column-oriented: one lane
+// read and one FMA per column, no cross-lane sums.
 template <int NP>
-__device__ __forceinline__ void chol_regs(float (&R)[NP], float (&invd)[NP], float& myinv, int lane) {
+__device__ __forceinline__ void chol_regs(float (&R)[NP], float& myinv, int lane) {
   myinv = 1.f;
 #pragma unroll
   for (int j = 0; j < NP; ++j) {
     const float piv = fmaxf(lane_bcast(R[j], j), 1e-30f);
     const float inv = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, rsqrt_refined(piv))));
-    invd[j] = inv;
     const bool below = lane > j;
     myinv = lane == j ? inv : myinv;
     const float w = below ? R[j] * (inv * inv) : 0.f;
@@ -142,19 +142,20 @@ __device__ __forceinline__ void chol_regs(float (&R)[NP], float (&invd)[NP], flo
 
 // x = (L L^T)^-1 b, lane i holding b_i and returning x_i
 template <int NP>
-__device__ __forceinline__ float solve_regs(const float (&R)[NP], const float (&invd)[NP], float myinv, int lane, float b) {
+__device__ __forceinline__ float solve_regs(const float (&R)[NP], float myinv, int lane, float b) {
   float r = b;
 #pragma unroll
   for (int j = 0; j < NP; ++j) {  // L y = b; lane j keeps r_j = y_j * L[j][j]
-    const float yj = lane_bcast(r, j) * invd[j];
+    const float yj = lane_bcast(r * myinv, j);
     r = lane > j ? r - R[j] * yj : r;
   }
+  const float myinv2 = myinv * myinv;
 #pragma unroll
   for (int k = NP - 1; k >= 0; --k) {  // L^T x = y in the scaled form  sum_{k>i} R[k] x_k + L[i][i]^2 x_i = r_i
-    const float xk = lane_bcast(r, k) * (invd[k] * invd[k]);
+    const float xk = lane_bcast(r * myinv2, k);
     r = lane < k ? r - R[k] * xk : r;
   }
-  return r * (myinv * myinv);
+  return r * myinv2;
 }
 
 // dot product of an LDS row (per-lane address, 16-byte aligned) with a broadcast register vector
@@ -511,13 +512,13 @@ void step_kernel(StepArgs a) {
 
     KS_TICK(6)
     // ---- Cholesky of M and the unconstrained acceleration (registers only)
-    float R[NP], invd[NP];
+    float R[NP];
     load_row<NP>(Mrow, R);
 #pragma unroll
-    for (int j = 0; j < NP; ++j) { R[j] = is_dof ? R[j] : (lane == j ? 1.f : 0.f); invd[j] = 0.f; }
+    for (int j = 0; j < NP; ++j) R[j] = is_dof ? R[j] : (lane == j ? 1.f : 0.f);
     float myinv;
-    chol_regs<NP>(R, invd, myinv, lane);
-    const float qas = solve_regs<NP>(R, invd, myinv, lane, qfs);
+    chol_regs<NP>(R, myinv, lane);
+    const float qas = solve_regs<NP>(R, myinv, lane, qfs);
     if (a.dbg_qacc_smooth && is_dof) a.dbg_qacc_smooth[env * nv + lane] = qas;
 
     KS_TICK(7)
@@ -643,8 +644,8 @@ void step_kernel(StepArgs a) {
             }
         }
         KS_TICK(11)
-        chol_regs<NP>(R, invd, myinv, lane);
-        const float search = -solve_regs<NP>(R, invd, myinv, lane, grad);
+        chol_regs<NP>(R, myinv, lane);
+        const float search = -solve_regs<NP>(R, myinv, lane, grad);
         KS_TICK(12)
 
         // ---- exact line search along `search`
