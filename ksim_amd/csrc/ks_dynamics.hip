@@ -26,7 +26,7 @@ typedef __attribute__((ext_vector_type(16))) float f32x16;
 
 #define KS_SYNC() __syncthreads()
 #ifndef KS_STEP_WAVES
-#define KS_STEP_WAVES 3  // wavefronts per SIMD the register allocation aims at
+#define KS_STEP_WAVES 4  // wavefronts per SIMD the register allocation aims at
 #endif
 // Phase timers for kernel tuning: compiled in only with -DKS_PROFILE, which reuses the dbg_M buffer for cycle counts.
 #ifdef KS_PROFILE
@@ -46,7 +46,7 @@ __host__ __device__ inline int j_stride(int nv) { return row_stride(nv); }
 
 struct Lds {
   float *qpos, *qvel, *warm, *tau;
-  float *xpos, *xquat, *xmat, *xanchor, *xaxis;
+  float *xpos, *xquat, *xanchor, *xaxis;
   float *cinert, *crb, *cdof, *buf, *cvel, *cacc, *cfrc, *fsub;
   float *M, *J, *vbuf, *drow;
   float *con_off, *con_D, *con_kip;
@@ -60,9 +60,9 @@ __host__ __device__ inline int lds_floats(int nb, int nq, int nv, int nu, int ns
   const int nvs = m_stride(nv), js = j_stride(nv);
   int n = 0;
   n += up4(nq) + 32 + up4(nv) + up4(nu);                             // qpos qvel(32) warm tau
-  n += up4(nb * 3) + up4(nb * 4) + up4(nb * 9) + 2 * up4(nb * 3);      // xpos xquat xmat xanchor xaxis
+  n += up4(nb * 3) + up4(nb * 4) + 2 * up4(nb * 3);                    // xpos xquat xanchor xaxis
   n += up4(nv * 6) + up4(nb * 6);                                    // cdof cvel
-  const int scratch = 2 * up4(nb * 10) + up4(nv * 6) + 3 * up4(nb * 6);  // cinert crb buf cacc cfrc fsub
+  const int scratch = 2 * up4(nb * 10) + up4(nv * 6) + 2 * up4(nb * 6);  // cinert crb buf cacc(=fsub) cfrc
   const int jsz = up4(4 * ns * js + 32);                             // J overlays that scratch once it is dead
   n += scratch > jsz ? scratch : jsz;
   n += up4(nv * nvs) + 32 + 64;                                      // M vbuf drow
@@ -79,12 +79,13 @@ __device__ inline Lds carve(float* p, const DevModel& m) {
     return r;
   };
   l.qpos = take(nq); l.qvel = take(32); l.warm = take(nv); l.tau = take(nu);
-  l.xpos = take(nb * 3); l.xquat = take(nb * 4); l.xmat = take(nb * 9); l.xanchor = take(nb * 3); l.xaxis = take(nb * 3);
+  l.xpos = take(nb * 3); l.xquat = take(nb * 4); l.xanchor = take(nb * 3); l.xaxis = take(nb * 3);
   l.cdof = take(nv * 6); l.cvel = take(nb * 6);
   {
     float* base = p;
     l.cinert = take(nb * 10); l.crb = take(nb * 10); l.buf = take(nv * 6);
-    l.cacc = take(nb * 6); l.cfrc = take(nb * 6); l.fsub = take(nb * 6);
+    l.cacc = take(nb * 6); l.cfrc = take(nb * 6);
+    l.fsub = l.cacc;  // the subtree force sums replace the accelerations once the level passes are done
     float* end = p;
     l.J = base;  // written only after the bias forces are out of fsub
     float* jend = base + up4(4 * ns * js + 32);
@@ -216,7 +217,6 @@ void step_kernel(StepArgs a) {
   if (lane == 0) {  // world body
     for (int k = 0; k < 3; ++k) { l.xpos[k] = 0.f; l.xanchor[k] = 0.f; l.xaxis[k] = 0.f; }
     l.xquat[0] = 1.f; l.xquat[1] = l.xquat[2] = l.xquat[3] = 0.f;
-    for (int k = 0; k < 9; ++k) l.xmat[k] = (k % 4 == 0) ? 1.f : 0.f;
     for (int k = 0; k < 6; ++k) l.cvel[k] = 0.f;
   }
   const float mu = a.friction ? a.friction[env] : m.friction;
@@ -346,8 +346,6 @@ void step_kernel(StepArgs a) {
         const Mat3 R = q2mat(quat);
         st3(l.xpos + 3 * b, pos);
         l.xquat[4 * b] = quat.w; l.xquat[4 * b + 1] = quat.x; l.xquat[4 * b + 2] = quat.y; l.xquat[4 * b + 3] = quat.z;
-#pragma unroll
-        for (int k = 0; k < 9; ++k) l.xmat[9 * b + k] = R.m[k];
         st3(l.xanchor + 3 * b, anchor);
         st3(l.xaxis + 3 * b, axis);
         xipos = pos + mul(R, b_ipos);
@@ -392,7 +390,8 @@ void step_kernel(StepArgs a) {
         if (d_k < 3) {
           my_cdof.l = {d_k == 0 ? 1.f : 0.f, d_k == 1 ? 1.f : 0.f, d_k == 2 ? 1.f : 0.f};
         } else {
-          const float* R = l.xmat + 9 * d_body;
+          const Mat3 Rb = q2mat({l.xquat[4 * d_body], l.xquat[4 * d_body + 1], l.xquat[4 * d_body + 2], l.xquat[4 * d_body + 3]});
+          const float* R = Rb.m;
           const V3 ax = {R[d_k - 3], R[3 + d_k - 3], R[6 + d_k - 3]};
           my_cdof = {ax, cross(ax, off)};
         }
@@ -479,7 +478,8 @@ void step_kernel(StepArgs a) {
     float dist = 1.f;
     V3 cpos = {0.f, 0.f, 0.f};
     if (is_sph) {
-      const float* R = l.xmat + 9 * s_body;
+      const Mat3 Rb = q2mat({l.xquat[4 * s_body], l.xquat[4 * s_body + 1], l.xquat[4 * s_body + 2], l.xquat[4 * s_body + 3]});
+      const float* R = Rb.m;
       const V3 c = ld3(l.xpos + 3 * s_body) + V3{R[0] * s_pos.x + R[1] * s_pos.y + R[2] * s_pos.z,
                                                 R[3] * s_pos.x + R[4] * s_pos.y + R[5] * s_pos.z,
                                                 R[6] * s_pos.x + R[7] * s_pos.y + R[8] * s_pos.z};
