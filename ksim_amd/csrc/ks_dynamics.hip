@@ -110,11 +110,6 @@ __device__ __forceinline__ void load_row(const float* p, float (&v)[NP]) {
   }
 }
 
-__device__ __forceinline__ float rsqrt_refined(float x) {
-  float y = __builtin_amdgcn_rsqf(x);
-  y = y * (1.5f - 0.5f * x * y * y);  // one Newton step: full fp32 accuracy
-  return y;
-}
 
 // In-register Cholesky, right-looking on the full symmetric rows: lane i holds row i of the matrix in R[0..NP).
 // Step j scales column j below the diagonal into L and subtracts the rank-1 term from every later row, all
@@ -130,12 +125,14 @@ __device__ __forceinline__ void chol_regs(float (&R)[NP], float& myinv, int lane
   myinv = 1.f;
 #pragma unroll
   for (int j = 0; j < NP; ++j) {
+    // every lane computes the same 1 / sqrt(pivot) from the broadcast pivot (v_rsq_f32 is accurate to 1 ulp)
     const float piv = fmaxf(lane_bcast(R[j], j), 1e-30f);
-    const float inv = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, rsqrt_refined(piv))));
+    const float inv = __builtin_amdgcn_rsqf(piv);
     const bool below = lane > j;
     myinv = lane == j ? inv : myinv;
-    const float w = below ? R[j] * (inv * inv) : 0.f;
-    R[j] = below ? R[j] * inv : R[j];
+    const float t = R[j] * inv;
+    const float w = below ? t * inv : 0.f;
+    R[j] = below ? t : R[j];
 #pragma unroll
     for (int k = j + 1; k < NP; ++k) R[k] -= w * lane_bcast(R[k], j);
   }
