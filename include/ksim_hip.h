@@ -265,6 +265,8 @@ int ks_terms_destroy(KsTerms* terms);
 typedef struct KsRng {
   uint64_t seed;
   uint64_t step;
+  const uint64_t* step_base; /* device, nullable: added to `step` when the kernel runs, so that a captured
+                                HIP graph of a rollout draws fresh numbers on every replay */
 } KsRng;
 
 typedef struct KsObserveIO {
@@ -344,7 +346,8 @@ int ks_mlp_forward(const KsMlp* mlp, ks_stream_t stream, int64_t M, const float*
  */
 enum { KS_REW_STAY_ALIVE = 0, KS_REW_BASE_HEIGHT = 1, KS_REW_BASE_HEIGHT_RANGE = 2, KS_REW_ACTION_VEL = 3,
        KS_REW_ACTION_ACC = 4, KS_REW_ACTION_JERK = 5, KS_REW_UPRIGHT_ANGVEL = 6, KS_REW_UPRIGHT_LINVEL = 7,
-       KS_REW_UPRIGHT_POSE = 8 };
+       KS_REW_UPRIGHT_POSE = 8,
+       KS_REW_AMP = 9 /* max(0, 1 - 0.25 (logit - 1)^2) of the discriminator logits, ksim/task/amp.py:99-112 */ };
 enum { KS_NORM_L1 = 0, KS_NORM_L2 = 1 }; /* xax.get_norm: l1 = |x|, l2 = x^2 (reference tests/test_rewards.py:95-98) */
 typedef struct KsRewardDesc {
   int32_t kind;
@@ -363,6 +366,7 @@ typedef struct KsRewardIO {
   const float* action; /* (T, N, nu) */
   const uint8_t* done; /* (T, N) */
   const uint8_t* success; /* (T, N) */
+  const float* disc_logits; /* (T, N) discriminator output per frame (ks_mlp_forward on the motion frames), KS_REW_AMP only */
   float* components;   /* (n_rewards, T, N) nullable */
   float* total;        /* (T, N) */
 } KsRewardIO;

@@ -37,7 +37,7 @@ class KsTermsDesc(ctypes.Structure):
 
 
 class KsRng(ctypes.Structure):
-    _fields_ = [("seed", c_uint64), ("step", c_uint64)]
+    _fields_ = [("seed", c_uint64), ("step", c_uint64), ("step_base", c_void_p)]
 
 
 class KsObserveIO(ctypes.Structure):
@@ -60,7 +60,7 @@ class KsMlpDesc(ctypes.Structure):
 
 
 (REW_STAY_ALIVE, REW_BASE_HEIGHT, REW_BASE_HEIGHT_RANGE, REW_ACTION_VEL, REW_ACTION_ACC, REW_ACTION_JERK,
- REW_UPRIGHT_ANGVEL, REW_UPRIGHT_LINVEL, REW_UPRIGHT_POSE) = range(9)
+ REW_UPRIGHT_ANGVEL, REW_UPRIGHT_LINVEL, REW_UPRIGHT_POSE, REW_AMP) = range(10)
 NORM_L1, NORM_L2 = 0, 1
 KS_MAX_REWARD_TERMS = 32
 
@@ -75,7 +75,7 @@ class KsRewardIO(ctypes.Structure):
                 ("n_rewards", c_int32), ("rewards", KsRewardDesc * KS_MAX_REWARD_TERMS), ("use_clip_min", c_int32),
                 ("use_clip_max", c_int32), ("clip_min", c_float), ("clip_max", c_float), ("qpos", c_void_p),
                 ("qvel", c_void_p), ("action", c_void_p), ("done", c_void_p), ("success", c_void_p),
-                ("components", c_void_p), ("total", c_void_p)]
+                ("disc_logits", c_void_p), ("components", c_void_p), ("total", c_void_p)]
 
 
 def bind(lib) -> None:

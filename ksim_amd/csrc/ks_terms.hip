@@ -65,7 +65,7 @@ __global__ __launch_bounds__(256) void observe_kernel(ObserveArgs a) {
         n01 = a.noise_normal[idx];
         u01v = a.noise_uniform[idx];
       } else {
-        const Philox4 r = draw(a.rng.seed, a.rng.step, kRngObsNoise, (uint64_t)e, (uint32_t)k);
+        const Philox4 r = draw(a.rng.seed, a.rng.step + (a.rng.step_base ? *a.rng.step_base : 0ull), kRngObsNoise, (uint64_t)e, (uint32_t)k);
         n01 = normal_from(r.x, r.y);
         u01v = u01(r.z);
       }
@@ -148,7 +148,7 @@ __global__ __launch_bounds__(256) void terminate_kernel(TerminateArgs a) {
   for (int i = 0; i < a.nq; ++i) {
     float u;
     if (a.reset_uniform) u = a.reset_uniform[e * (a.nq + 1) + i];
-    else u = 2.f * u01(draw(a.rng.seed, a.rng.step, kRngReset, (uint64_t)e, (uint32_t)i).x) - 1.f;
+    else u = 2.f * u01(draw(a.rng.seed, a.rng.step + (a.rng.step_base ? *a.rng.step_base : 0ull), kRngReset, (uint64_t)e, (uint32_t)i).x) - 1.f;
     const float mag = d.reset_mag[i] * (d.reset_by_level[i] ? a.level : 1.f);
     float x = d.reset_base[i] + u * mag;
     x = fminf(fmaxf(x, d.reset_lo[i]), d.reset_hi[i]);
@@ -157,7 +157,7 @@ __global__ __launch_bounds__(256) void terminate_kernel(TerminateArgs a) {
   if (a.random_heading && a.nq >= 7) {
     float u;
     if (a.reset_uniform) u = a.reset_uniform[e * (a.nq + 1) + a.nq];
-    else u = 2.f * u01(draw(a.rng.seed, a.rng.step, kRngReset, (uint64_t)e, (uint32_t)a.nq).x) - 1.f;
+    else u = 2.f * u01(draw(a.rng.seed, a.rng.step + (a.rng.step_base ? *a.rng.step_base : 0ull), kRngReset, (uint64_t)e, (uint32_t)a.nq).x) - 1.f;
     const float h = 0.5f * 3.14159265358979323846f * u;  // yaw/2, yaw ~ U(-pi, pi)
     const float cw = cosf(h), sz = sinf(h);
     const float w = q[3], x = q[4], y = q[5], z = q[6];
@@ -182,7 +182,7 @@ __global__ __launch_bounds__(256) void sample_action_kernel(int64_t n, int nu, c
     float z;
     if (noise) z = noise[idx];
     else {
-      const Philox4 r = draw(rng.seed, rng.step, kRngAction, (uint64_t)e, (uint32_t)u);
+      const Philox4 r = draw(rng.seed, rng.step + (rng.step_base ? *rng.step_base : 0ull), kRngAction, (uint64_t)e, (uint32_t)u);
       z = normal_from(r.x, r.y);
     }
     a += expf(log_std[u]) * z;
@@ -265,6 +265,10 @@ __global__ __launch_bounds__(256) void rewards_kernel(KsRewardIO io) {
         float zb[3];
         rot_inv(q + 3, 0.f, 0.f, 1.f, zb);
         val = kernel_with_penalty(atan2f(zb[0], zb[2]), r.p0, r.p1, r.p2);
+      } break;
+      case KS_REW_AMP: {
+        const float d = io.disc_logits[idx] - 1.0f;
+        val = fmaxf(0.f, 1.0f - 0.25f * d * d);
       } break;
       default: break;
     }
@@ -398,13 +402,14 @@ extern "C" int ks_rewards(ks_stream_t stream, const KsRewardIO* io) {
   if (!io->done) return fail(KS_EINVAL, "ks_rewards: done is required");
   for (int j = 0; j < io->n_rewards; ++j) {
     const int k = io->rewards[j].kind;
-    if (k < KS_REW_STAY_ALIVE || k > KS_REW_UPRIGHT_POSE) return fail(KS_EINVAL, "ks_rewards: term %d: bad kind", j);
+    if (k < KS_REW_STAY_ALIVE || k > KS_REW_AMP) return fail(KS_EINVAL, "ks_rewards: term %d: bad kind", j);
     const bool needs_q = k == KS_REW_BASE_HEIGHT || k == KS_REW_BASE_HEIGHT_RANGE || k == KS_REW_UPRIGHT_POSE;
     const bool needs_v = k == KS_REW_UPRIGHT_ANGVEL || k == KS_REW_UPRIGHT_LINVEL;
     const bool needs_a = k >= KS_REW_ACTION_VEL && k <= KS_REW_ACTION_JERK;
     if (needs_q && (!io->qpos || io->nq < 7)) return fail(KS_EINVAL, "ks_rewards: term %d needs qpos of a floating base", j);
     if (needs_v && (!io->qvel || io->nv < 6)) return fail(KS_EINVAL, "ks_rewards: term %d needs qvel of a floating base", j);
     if (needs_a && (!io->action || io->nu < 1)) return fail(KS_EINVAL, "ks_rewards: term %d needs actions", j);
+    if (k == KS_REW_AMP && !io->disc_logits) return fail(KS_EINVAL, "ks_rewards: term %d needs the discriminator logits", j);
     if (k == KS_REW_STAY_ALIVE && !(io->rewards[j].p0 != 0.f)) return fail(KS_EINVAL, "ks_rewards: term %d: zero balance", j);
   }
   const int64_t n = io->T * io->N, grid = (n + 255) / 256;

@@ -186,6 +186,19 @@ class HipEngine(PhysicsEngine):
                                             xpos=d.xpos, xquat=d.xquat, cvel=d.cvel))
         # engine.py:217-220: qvel and qacc are zeroed after the forward pass (qvel is already zero here)
 
+    def prepare(self, device):
+        """Uploads the actuator gain tables (once per device); call before capturing `step` into a HIP graph,
+        where host-to-device copies are not allowed."""
+        act = self.actuators
+        if not isinstance(act, PositionActuators):
+            return None
+        cache = getattr(self, "_gain_cache", None)
+        if cache is None or cache[0] is not act or cache[1].device != torch.device(device):
+            t = lambda a: torch.tensor(a, dtype=torch.float32, device=device)  # noqa: E731
+            cache = (act, t(act.kps), t(act.kds), t(act.clip_array()))
+            object.__setattr__(self, "_gain_cache", cache)
+        return cache
+
     # -------------------------------------------------------------------------------------- step (engine.py:259-361)
     def step(self, action: torch.Tensor, physics_model: physics.DeviceModel, physics_state: PhysicsState,
              curriculum_level, rng, randomization: Mapping[str, torch.Tensor] | None = None,
@@ -207,11 +220,7 @@ class HipEngine(PhysicsEngine):
                    traj_xpos=record.get("xpos"), traj_xquat=record.get("xquat"))
         act = self.actuators
         if isinstance(act, PositionActuators):
-            cache = getattr(self, "_gain_cache", None)
-            if cache is None or cache[0] is not act or cache[1].device != action.device:
-                t = lambda a: torch.tensor(a, dtype=torch.float32, device=action.device)  # noqa: E731
-                cache = (act, t(act.kps), t(act.kds), t(act.clip_array()))
-                self._gain_cache = cache
+            cache = self.prepare(action.device)
             ast = s.actuator_state or {}
             buf.update(kp=cache[1], kd=cache[2], ctrl_clip=cache[3], kp_scale=ast.get("kp_scale"),
                        kd_scale=ast.get("kd_scale"), torque_limit_scale=ast.get("torque_limit_scale"),

@@ -20,8 +20,11 @@ from .resets import Reset, compile_resets
 from .terminations import Termination
 
 
-def _rng(seed: int, step: int) -> T.KsRng:
-    return T.KsRng(int(seed) & (2**64 - 1), int(step) & (2**64 - 1))
+def _rng(seed: int, step: int, step_base: torch.Tensor | None = None) -> T.KsRng:
+    """Philox key; `step_base` (one int64 on the device) is added to `step` when the kernel runs."""
+    if step_base is not None:
+        _lib.require_cuda(step_base, dtype=torch.int64)
+    return T.KsRng(int(seed) & (2**64 - 1), int(step) & (2**64 - 1), _lib.ptr(step_base).value)
 
 
 def compile_terms(model: KinematicModel, observations: Mapping[str, Observation],
@@ -87,6 +90,7 @@ class EnvTerms:
     # ------------------------------------------------------------------ observations
     def observe(self, sources: Mapping[int, torch.Tensor | None], N: int, *, level: float = 1.0,
                 zero_offset=None, bias=None, noise_normal=None, noise_uniform=None, seed: int = 0, step: int = 0,
+                step_base=None,
                 obs: torch.Tensor | None = None, noisy_obs: torch.Tensor | None = None):
         m = self.model
         dims = {T.SRC_QPOS: m.nq, T.SRC_QVEL: m.nv, T.SRC_QACC: m.nv, T.SRC_CTRL: m.nu, T.SRC_LAST_ACTION: m.nu,
@@ -111,14 +115,14 @@ class EnvTerms:
             if tuple(t.shape) != shape:
                 raise _lib.KsError(f"{name}: expected {shape}, got {tuple(t.shape)}")
             setattr(io, name, t.data_ptr())
-        io.rng = _rng(seed, step)
+        io.rng = _rng(seed, step, step_base)
         _lib.check(self._lib.ks_observe(self._handle, _lib.current_stream(), ctypes.byref(io)))
         return obs, noisy_obs
 
     # ------------------------------------------------------------------ terminations + reset predication
     def terminate_reset(self, state: Mapping[str, torch.Tensor], *, level: float = 1.0, components=None, done=None,
                         success=None, traj_qpos=None, traj_qvel=None, traj_time=None, reset_mask=None,
-                        episode_length=None, reset_uniform=None, seed: int = 0, step: int = 0,
+                        episode_length=None, reset_uniform=None, seed: int = 0, step: int = 0, step_base=None,
                         apply_reset: bool = True) -> None:
         m = self.model
         qpos = state["qpos"]
@@ -142,7 +146,7 @@ class EnvTerms:
             if tuple(t.shape) != shape:
                 raise _lib.KsError(f"{name}: expected {shape}, got {tuple(t.shape)}")
             setattr(io, name, t.data_ptr())
-        io.rng = _rng(seed, step)
+        io.rng = _rng(seed, step, step_base)
         _lib.check(self._lib.ks_terminate_reset(self._handle, _lib.current_stream(), ctypes.byref(io)))
 
     def close(self) -> None:
@@ -158,7 +162,8 @@ class EnvTerms:
 
 
 def sample_action(mean: torch.Tensor, log_std: torch.Tensor | None, *, noise: torch.Tensor | None = None,
-                  seed: int = 0, step: int = 0, clip_max: float = 1e3, out: torch.Tensor | None = None):
+                  seed: int = 0, step: int = 0, step_base=None, clip_max: float = 1e3,
+                  out: torch.Tensor | None = None):
     """action = mean + exp(log_std) * N(0,1); NaN -> 0; clip to +-clip_max (ksim/task/rl.py:998-1001)."""
     lib = _lib.load()
     _lib.require_cuda(mean, log_std, noise, out, dtype=torch.float32)
@@ -170,5 +175,5 @@ def sample_action(mean: torch.Tensor, log_std: torch.Tensor | None, *, noise: to
     if out is None:
         out = torch.empty_like(mean)
     _lib.check(lib.ks_sample_action(_lib.current_stream(), N, nu, _lib.ptr(mean), _lib.ptr(log_std), _lib.ptr(noise),
-                                    _rng(seed, step), float(clip_max), _lib.ptr(out)))
+                                    _rng(seed, step, step_base), float(clip_max), _lib.ptr(out)))
     return out

@@ -111,6 +111,17 @@ class UprightReward(Reward):  # rewards.py:746-777 — a mapping of three compon
                 ("pose", T.REW_UPRIGHT_POSE, 0, self.pose_scale, self.pose_sq_scale, self.pose_abs_scale)]
 
 
+DISCRIMINATOR_OUTPUT_KEY = "_discriminator_output"  # ksim/task/amp.py:47
+
+
+@dataclass(frozen=True)
+class AMPReward(Reward):  # ksim/task/amp.py:99-112
+    """max(0, 1 - 0.25 (logit - 1)^2) of the discriminator logits found in `trajectory.aux_outputs`."""
+
+    def descs(self):
+        return [(None, T.REW_AMP, 0, 0.0, 0.0, 0.0)]
+
+
 def get_rewards(trajectory: Trajectory, rewards: Mapping[str, Reward], clip_min: float | None = None,
                 clip_max: float | None = None, want_components: bool = True) -> RewardState:
     """Reward total and components over a (T, N) rollout (ksim/task/rl.py:189-245)."""
@@ -149,6 +160,12 @@ def get_rewards(trajectory: Trajectory, rewards: Mapping[str, Reward], clip_min:
     action = tensor(trajectory.action, torch.float32, None if trajectory.action is None else trajectory.action.shape[-1])
     done_t = tensor(done, torch.uint8, None)
     succ_t = tensor(trajectory.success, torch.uint8, None)
+    logits = None
+    if any(io.rewards[j].kind == T.REW_AMP for j in range(len(names))):
+        if DISCRIMINATOR_OUTPUT_KEY not in trajectory.aux_outputs:  # same failure as amp.py:103-107
+            raise ValueError("AMPReward auxiliary output is missing! Make sure you are using it within the context of "
+                             "an AMP task, which populates the auxiliary output for you.")
+        logits = tensor(trajectory.aux_outputs[DISCRIMINATOR_OUTPUT_KEY], torch.float32, None)
     io.nq = 0 if qpos is None else qpos.shape[-1]
     io.nv = 0 if qvel is None else qvel.shape[-1]
     io.nu = 0 if action is None else action.shape[-1]
@@ -158,6 +175,7 @@ def get_rewards(trajectory: Trajectory, rewards: Mapping[str, Reward], clip_min:
     comps = torch.empty((len(names), Tn, N), dtype=torch.float32, device=done.device) if want_components else None
     io.qpos, io.qvel, io.action = _lib.ptr(qpos).value, _lib.ptr(qvel).value, _lib.ptr(action).value
     io.done, io.success = _lib.ptr(done_t).value, _lib.ptr(succ_t).value
+    io.disc_logits = _lib.ptr(logits).value
     io.components, io.total = _lib.ptr(comps).value, _lib.ptr(total).value
     _lib.check(lib.ks_rewards(_lib.current_stream(), ctypes.byref(io)))
     components = {} if comps is None else {n: comps[j] for j, n in enumerate(names)}

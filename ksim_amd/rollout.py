@@ -2,7 +2,9 @@
 
 One control step launches, in order on the current stream: observation (+noise) -> actor MLP (and critic)
 -> action sampling / scrub / clip -> fused physics control step -> terminations + transition record + reset
-predication -> forward pass of the freshly reset envs.  Nothing synchronises the host inside the loop.
+predication -> forward pass of the freshly reset envs.  Nothing synchronises the host inside the loop, so a
+whole rollout (T steps and the reward pass) can be captured once as a HIP graph and replayed, which takes the
+per-launch host cost out of the loop (`Rollout.unroll(..., graph=True)`).
 """
 from __future__ import annotations
 
@@ -67,26 +69,32 @@ class Rollout:
         self.components = torch.zeros(Tn, max(c.terms.n_terms, 1), N, dtype=torch.int8, device=dev)
         self.values = f(Tn, N, 1) if c.critic is not None else None
         self.reset_mask = b(N)
+        # Philox step counter of graph replays: kernels add it to the step baked into the captured launch
+        self.step_base = torch.zeros(1, dtype=torch.int64, device=dev)
+        self._graph = None
         if c.actor.in_dim != c.terms.obs_dim or c.actor.out_dim != m.nu:
             raise _lib.KsError("actor must map the observation vector to one mean per actuator")
         if c.critic is not None and (c.critic.in_dim != c.terms.obs_dim or c.critic.out_dim != 1):
             raise _lib.KsError("critic must map the observation vector to one value")
 
-    def step_engine(self, env: RolloutEnvState, t: int, level: float = 1.0, noise: Mapping | None = None) -> None:
+    def step_engine(self, env: RolloutEnvState, t: int, level: float = 1.0, noise: Mapping | None = None,
+                    _relative_step: bool = False) -> None:
         """One control step of every env; the transition lands in slot t of the buffers."""
         c, ps = self.c, env.physics_state
         d, noise = ps.data, noise or {}
+        # under graph capture the random-number step is (device counter + t) instead of the host counter
+        step, step_base = (t, self.step_base) if _relative_step else (env.step, None)
         src = {T.SRC_QPOS: d.qpos, T.SRC_QVEL: d.qvel, T.SRC_QACC: d.qacc, T.SRC_CTRL: d.ctrl,
                T.SRC_LAST_ACTION: ps.last_ctrl, T.SRC_COMMAND: env.commands, T.SRC_TIME: d.time, T.SRC_XPOS: d.xpos,
                T.SRC_XQUAT: d.xquat, T.SRC_CVEL: d.cvel}
         c.terms.observe(src, self.N, level=level, zero_offset=ps.zero_offset, bias=env.obs_bias,
                         noise_normal=noise.get("obs_normal"), noise_uniform=noise.get("obs_uniform"), seed=env.seed,
-                        step=env.step, obs=self.obs[t], noisy_obs=self.noisy_obs[t])
+                        step=step, step_base=step_base, obs=self.obs[t], noisy_obs=self.noisy_obs[t])
         c.actor(self.noisy_obs[t], out=self.mean)           # actor reads the noisy copy (walking.py:592-595)
         if c.critic is not None:
             c.critic(self.obs[t], out=self.values[t])       # critic reads the clean one (walking.py:626-638)
-        sample_action(self.mean, c.log_std, noise=noise.get("action_normal"), seed=env.seed, step=env.step,
-                      clip_max=c.action_clip_max, out=self.action[t])
+        sample_action(self.mean, c.log_std, noise=noise.get("action_normal"), seed=env.seed, step=step,
+                      step_base=step_base, clip_max=c.action_clip_max, out=self.action[t])
         # the step kernel also writes ctrl / xpos / xquat of the post-step data into the transition slot
         c.engine.step(self.action[t], c.physics_model, ps, level, env.seed + env.step, env.randomization_dict,
                       noise=noise.get("engine"), record=dict(ctrl=self.ctrl[t], xpos=self.xpos[t], xquat=self.xquat[t]),
@@ -96,17 +104,47 @@ class Rollout:
                                 done=self.done[t], success=self.success[t], traj_qpos=self.qpos[t],
                                 traj_qvel=self.qvel[t], traj_time=self.timestep[t], reset_mask=self.reset_mask,
                                 episode_length=env.episode_length, reset_uniform=noise.get("reset_uniform"),
-                                seed=env.seed, step=env.step)
+                                seed=env.seed, step=step, step_base=step_base)
         # refresh the derived fields and the warm start of the reset envs (engine.py:213)
         c.engine.forward(c.physics_model, ps, self.reset_mask, env.randomization_dict)
-        env.step += 1
+        if not _relative_step:
+            env.step += 1
 
-    def unroll(self, env: RolloutEnvState, level: float = 1.0) -> tuple[Trajectory, RewardState]:
+    def unroll(self, env: RolloutEnvState, level: float = 1.0, graph: bool = False) -> tuple[Trajectory, RewardState]:
+        """T control steps and the reward pass.  With `graph=True` the launches are captured once as a HIP graph
+        (per env state object and curriculum level) and replayed on later calls; the results are the same bits."""
+        if graph:
+            return self._unroll_graph(env, level)
         for t in range(self.T):
             self.step_engine(env, t, level)
         traj = self.trajectory()
         rewards = get_rewards(traj, self.c.rewards, self.c.reward_clip_min, self.c.reward_clip_max,
                               want_components=False)
+        return traj, rewards
+
+    def _unroll_graph(self, env: RolloutEnvState, level: float) -> tuple[Trajectory, RewardState]:
+        if self.c.engine.data.drop_action_prob * float(level) > 0:
+            raise _lib.KsError("graph replay needs drop_action_prob == 0 (the drop mask is sampled on the host side)")
+        key = (id(env), float(level))
+        if self._graph is None or self._graph[0] != key:
+            self.step_base.fill_(env.step)
+            self.c.engine.prepare(self.step_base.device)
+            torch.cuda.synchronize()
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                for t in range(self.T):
+                    self.step_engine(env, t, level, _relative_step=True)
+                traj = self.trajectory()
+                rewards = get_rewards(traj, self.c.rewards, self.c.reward_clip_min, self.c.reward_clip_max,
+                                      want_components=False)
+                self.step_base += self.T
+            self._graph = (key, g, traj, rewards)
+        elif int(env.step) != self._graph_step:
+            self.step_base.fill_(env.step)  # the eager path ran in between
+        _, g, traj, rewards = self._graph
+        g.replay()
+        env.step += self.T
+        self._graph_step = int(env.step)
         return traj, rewards
 
     def trajectory(self) -> Trajectory:

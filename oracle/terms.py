@@ -102,6 +102,11 @@ def base_height_range_reward(qpos_tq, z_lower, z_upper, dropoff):  # rewards.py:
     return np.clip(1.0 - np.clip(np.maximum(z_lower - z, z - z_upper), 0.0, None) * dropoff, 0.0, None)
 
 
+def amp_reward(discriminator_logits):  # ksim/task/amp.py:109-111
+    d = np.asarray(discriminator_logits, dtype=np.float64)
+    return np.maximum(0.0, 1.0 - 0.25 * np.square(d - 1.0))
+
+
 def upright_reward(qpos_tq, qvel_tv, s=0.25, sq=0.1, ab=0.1):  # rewards.py:760-777 (defaults)
     qpos = np.asarray(qpos_tq, dtype=np.float64)
     qvel = np.asarray(qvel_tv, dtype=np.float64)

@@ -169,3 +169,28 @@ def test_long_rollout_with_resets_stays_finite_and_reproducible():
     assert torch.equal(outs[0][0], outs[1][0]) and outs[0][1] == outs[1][1]
     assert torch.equal(outs[0][2], outs[1][2])
     assert (outs[0][0][:, 2] > 0.5).all()  # every env sits above the termination height after its reset
+
+
+def test_graph_replay_equals_eager_rollout():
+    """A captured rollout graph, replayed several times with eager work and synchronisations in between, gives
+    the same bits as the eager loop on every replay (same Philox keys: device step counter + baked step)."""
+    N, T, iters = 192, 8, 10
+    runs = []
+    for use_graph in (False, True):
+        m, c, rnd_, _, ro, EnvState = build(N, T, seed=5, min_height=0.8)
+        ps = c.engine.reset(c.physics_model, 1.0, 3, N, rnd_)
+        env = EnvState(ps, rnd_, torch.zeros(N, 2, device=DEV), None, seed=123)
+        snaps = []
+        for it in range(iters):
+            traj, rew = ro.unroll(env, graph=use_graph)
+            torch.cuda.synchronize()
+            snaps.append((traj.qpos.clone(), traj.action.clone(), traj.done.clone(), rew.total.clone(),
+                          ps.data.qpos.clone(), env.episode_length.clone()))
+            junk = torch.randn(512, 512, device=DEV)  # unrelated eager work between replays
+            (junk @ junk).sum().item()
+        assert env.step == iters * T
+        runs.append(snaps)
+    assert sum(int(s[2].sum().item()) for s in runs[0]) > 0, "no resets happened: the reset path was not replayed"
+    for it, (a, b) in enumerate(zip(*runs)):
+        for x, y, name in zip(a, b, ("qpos", "action", "done", "reward", "state", "episode_length")):
+            assert torch.equal(x, y), f"replay {it}: {name} differs from the eager rollout"

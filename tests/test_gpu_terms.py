@@ -249,3 +249,39 @@ def test_rewards_against_oracle():
     for k in scales:
         np.testing.assert_allclose(out.components[k].cpu().numpy(), scaled[k], rtol=1e-5, atol=2e-5, err_msg=k)
     np.testing.assert_allclose(out.total.cpu().numpy(), total, rtol=1e-5, atol=5e-5)
+
+
+def test_amp_reward_from_discriminator_logits():
+    """Discriminator forward (BASELINE config 5 shape, 71 -> 256 -> 256 -> 1) and the AMP reward on its logits."""
+    import torch.nn.functional as F
+    from ksim_amd import rewards as rw
+    from ksim_amd.mlp import MLP
+    from ksim_amd.types import Trajectory
+
+    Tn, N, dim = 32, 50, 71
+    rng = np.random.default_rng(1005)
+    dims = (dim, 256, 256, 1)
+    ws = [rng.normal(scale=1 / np.sqrt(i), size=(o, i)).astype(np.float32) for i, o in zip(dims[:-1], dims[1:])]
+    bs = [rng.normal(scale=0.1, size=o).astype(np.float32) for o in dims[1:]]
+    frames = rng.normal(size=(Tn, N, dim)).astype(np.float32)
+    disc = MLP(ws, bs, activation="relu", dtype="f32")
+    logits = disc(t32(frames.reshape(Tn * N, dim))).reshape(Tn, N)
+    h = torch.from_numpy(frames.reshape(-1, dim)).double()
+    for i, (w, b) in enumerate(zip(ws, bs)):
+        h = F.linear(h, torch.from_numpy(w).double(), torch.from_numpy(b).double())
+        if i + 1 < len(ws):
+            h = F.relu(h)
+    want_logits = h.numpy().reshape(Tn, N)
+    np.testing.assert_allclose(logits.cpu().numpy(), want_logits, rtol=0, atol=2e-5 * np.abs(want_logits).max())
+    done = torch.zeros(Tn, N, dtype=torch.bool, device=DEV)
+    traj = Trajectory(qpos=None, qvel=None, xpos=None, xquat=None, ctrl=None, obs={}, command={}, event_state={},
+                      action=None, done=done, success=done.clone(), timestep=None,
+                      aux_outputs={rw.DISCRIMINATOR_OUTPUT_KEY: logits})
+    out = rw.get_rewards(traj, {"amp_reward": rw.AMPReward(scale=0.5)})
+    got_logits = logits.cpu().numpy().astype(np.float64)
+    np.testing.assert_allclose(out.total.cpu().numpy(), 0.5 * ot.amp_reward(got_logits), rtol=1e-5, atol=1e-6)
+    assert list(out.components) == ["amp_reward"]
+    traj_missing = Trajectory(qpos=None, qvel=None, xpos=None, xquat=None, ctrl=None, obs={}, command={}, event_state={},
+                              action=None, done=done, success=done.clone(), timestep=None)
+    with pytest.raises(ValueError, match="auxiliary output is missing"):
+        rw.get_rewards(traj_missing, {"amp_reward": rw.AMPReward(scale=0.5)})

@@ -88,3 +88,11 @@ def test_simple_rewards():
                                     {"a_reward": 2.0, "b_penalty": 0.5}, {"a_reward": False, "b_penalty": True},
                                     clip_min=0.5)
     np.testing.assert_allclose(tot, [0.5, 3.75])
+
+
+def test_amp_reward_closed_form():
+    # ksim/task/amp.py:111: a parabola with its apex (1) at logit 1, zero at logits -1 and 3, clamped outside
+    np.testing.assert_allclose(terms.amp_reward([1.0, 3.0, -1.0, 5.0, -7.0, 0.0, 2.0]), [1.0, 0.0, 0.0, 0.0, 0.0, 0.75, 0.75])
+    x = np.linspace(-4, 6, 101)
+    np.testing.assert_allclose(terms.amp_reward(x), terms.amp_reward(2.0 - x))  # symmetric about logit 1
+    assert (terms.amp_reward(x) >= 0).all() and terms.amp_reward(x).max() == 1.0
