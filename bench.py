@@ -125,6 +125,24 @@ def main() -> None:
     ndone = int(ro.done.sum().item())
     assert torch.isfinite(env.physics_state.data.qpos).all(), "non-finite state after the benchmark"
 
+    # The same rollout captured once as a HIP graph and replayed: the launches leave the host out of the loop.
+    # Reported beside the headline (whose timed region keeps per-launch events for the roofline figure).
+    graph = None
+    if not args.traffic_probe:
+        reps = max(1, args.steps // T)
+        ro.unroll(env, graph=True)  # capture + first replay
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            rew = ro.unroll(env, graph=True)[1]
+            ro.ppo_inputs(rew, 0.99, 0.95, normalize_advantages=True)
+        torch.cuda.synchronize()
+        g_elapsed = time.perf_counter() - t0
+        assert torch.isfinite(env.physics_state.data.qpos).all(), "non-finite state after the graph replays"
+        graph = {"value": N * reps * T / g_elapsed, "unit": "env-steps/s", "steps": reps * T,
+                 "ms_per_step": g_elapsed / (reps * T) * 1e3,
+                 "what": "the same control steps, rewards and GAE with each T-step rollout replayed from one HIP graph"}
+
     if args.traffic_probe:
         n = 64 * 1024 * 1024
         src, dst = torch.ones(n, device="cuda"), torch.empty(n, device="cuda")
@@ -158,7 +176,7 @@ def main() -> None:
                      "algorithmic_bytes_per_env_step": bytes_per_env, "kernel_ms": kernel_ms,
                      "note": "the fused step is fp32-VALU/LDS-bound (~1e3 flop/byte); the HBM fraction is reported "
                              "against the bytes the engine contract obliges a step to move"},
-        "gae": gae, "policy_mlp": mlp,
+        "gae": gae, "policy_mlp": mlp, "graph_replay": graph,
     }
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline()

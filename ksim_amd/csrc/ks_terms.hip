@@ -94,79 +94,115 @@ struct TerminateArgs {
   int apply_reset, nq, nv, nu, n_terms, random_heading, nonfinite_terminates;
 };
 
-// One lane per env.  Termination comparisons are strict and done in fp32 on the stored state, so
-// the integer outputs are reproducible bit for bit.
+// A 256-thread workgroup owns kTermEnvs consecutive envs.  The state rows of those envs are contiguous in memory,
+// so the transition copies, the finiteness check and the reset writes all walk them as flat, coalesced
+// arrays; the per-env decisions (one lane per env, a handful of scalars each) sit between the flat passes.
+// Termination comparisons are strict and done in fp32 on the stored state, so the integer outputs are
+// reproducible bit for bit.
+constexpr int kTermEnvs = 32;
+
 __global__ __launch_bounds__(256) void terminate_kernel(TerminateArgs a) {
-  const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (e >= a.N) return;
+  __shared__ int s_bad[kTermEnvs];    // non-finite state seen
+  __shared__ int s_reset[kTermEnvs];  // env starts a fresh episode
   const KsTermsDesc& d = a.t->d;
-  float* q = a.qpos + e * a.nq;
-  float* v = a.qvel + e * a.nv;
-  const float tm = a.time ? a.time[e] : 0.f;
-  bool done = false, succ = true;
-  for (int j = 0; j < a.n_terms; ++j) {
-    const KsTermDesc td = d.terms[j];
-    bool fire = false;
-    switch (td.kind) {
-      case KS_TERM_MIN_HEIGHT: fire = q[2] < td.p0; break;
-      case KS_TERM_BAD_Z: {
-        const float lo = (td.p2 - td.p0) * a.level + td.p0, hi = (td.p3 - td.p1) * a.level + td.p1;
-        fire = (q[2] < lo) || (q[2] > hi);
-      } break;
-      case KS_TERM_NOT_UPRIGHT: {
-        float out[3];
-        rot_inv(q + 3, 0.f, 0.f, 1.f, out);
-        fire = acosf(fminf(fmaxf(out[2], -1.f), 1.f)) > td.p0;
-      } break;
-      case KS_TERM_BAD_VELOCITY: fire = sqrtf(v[0] * v[0] + v[1] * v[1] + v[2] * v[2]) > td.p0; break;
-      case KS_TERM_FAR_FROM_ORIGIN: fire = sqrtf(q[0] * q[0] + q[1] * q[1] + q[2] * q[2]) > td.p0; break;
-      case KS_TERM_EPISODE_LENGTH: fire = (tm > td.p0) && !(td.p1 >= 0.f && a.level < td.p1); break;
-      default: break;
+  const int tid = threadIdx.x;
+  const int64_t e0 = (int64_t)blockIdx.x * kTermEnvs;
+  const int ne = a.N - e0 < kTermEnvs ? (int)(a.N - e0) : kTermEnvs;
+  const int nq = a.nq, nv = a.nv, nu = a.nu;
+  if (tid < kTermEnvs) s_bad[tid] = 0;
+  __syncthreads();
+  // ---- flat pass 1: transition record (post-step state) and finiteness
+  float* qb = a.qpos + e0 * nq;
+  float* vb = a.qvel + e0 * nv;
+  for (int idx = tid; idx < ne * nq; idx += 256) {
+    const float x = qb[idx];
+    if (a.traj_qpos) a.traj_qpos[e0 * nq + idx] = x;
+    if (a.nonfinite_terminates && !(fabsf(x) <= 3.0e38f)) s_bad[idx / nq] = 1;  // true for NaN and inf
+  }
+  for (int idx = tid; idx < ne * nv; idx += 256) {
+    const float x = vb[idx];
+    if (a.traj_qvel) a.traj_qvel[e0 * nv + idx] = x;
+    if (a.nonfinite_terminates && !(fabsf(x) <= 3.0e38f)) s_bad[idx / nv] = 1;
+  }
+  __syncthreads();
+  // ---- one lane per env: terminations, done / success, reset decision
+  if (tid < ne) {
+    const int64_t e = e0 + tid;
+    const float* q = qb + tid * nq;
+    const float* v = vb + tid * nv;
+    const float tm = a.time ? a.time[e] : 0.f;
+    bool done = false, succ = true;
+    for (int j = 0; j < a.n_terms; ++j) {
+      const KsTermDesc td = d.terms[j];
+      bool fire = false;
+      switch (td.kind) {
+        case KS_TERM_MIN_HEIGHT: fire = q[2] < td.p0; break;
+        case KS_TERM_BAD_Z: {
+          const float lo = (td.p2 - td.p0) * a.level + td.p0, hi = (td.p3 - td.p1) * a.level + td.p1;
+          fire = (q[2] < lo) || (q[2] > hi);
+        } break;
+        case KS_TERM_NOT_UPRIGHT: {
+          float out[3];
+          rot_inv(q + 3, 0.f, 0.f, 1.f, out);
+          fire = acosf(fminf(fmaxf(out[2], -1.f), 1.f)) > td.p0;
+        } break;
+        case KS_TERM_BAD_VELOCITY: fire = sqrtf(v[0] * v[0] + v[1] * v[1] + v[2] * v[2]) > td.p0; break;
+        case KS_TERM_FAR_FROM_ORIGIN: fire = sqrtf(q[0] * q[0] + q[1] * q[1] + q[2] * q[2]) > td.p0; break;
+        case KS_TERM_EPISODE_LENGTH: fire = (tm > td.p0) && !(td.p1 >= 0.f && a.level < td.p1); break;
+        default: break;
+      }
+      const int8_t val = fire ? (int8_t)td.value : (int8_t)0;
+      if (a.components) a.components[(int64_t)j * a.N + e] = val;
+      done |= val != 0;
+      succ &= val != -1;
     }
-    const int8_t val = fire ? (int8_t)td.value : (int8_t)0;
-    if (a.components) a.components[(int64_t)j * a.N + e] = val;
-    done |= val != 0;
-    succ &= val != -1;
+    if (s_bad[tid]) { done = true; succ = false; }
+    succ = succ && done;
+    if (a.done) a.done[e] = done ? 1 : 0;
+    if (a.success) a.success[e] = succ ? 1 : 0;
+    if (a.traj_time) a.traj_time[e] = tm;
+    const bool do_reset = a.apply_reset == 2 || (done && a.apply_reset == 1);
+    s_reset[tid] = do_reset ? 1 : 0;
+    if (a.reset_mask) a.reset_mask[e] = do_reset ? 1 : 0;
+    if (a.episode_length) a.episode_length[e] = do_reset ? 0 : a.episode_length[e] + 1;
+    if (do_reset && a.time) a.time[e] = 0.f;
   }
-  if (a.nonfinite_terminates) {
-    bool finite = true;
-    for (int i = 0; i < a.nq; ++i) finite &= fabsf(q[i]) <= 3.0e38f;  // false for NaN and inf
-    for (int i = 0; i < a.nv; ++i) finite &= fabsf(v[i]) <= 3.0e38f;
-    if (!finite) { done = true; succ = false; }
-  }
-  succ = succ && done;
-  if (a.done) a.done[e] = done ? 1 : 0;
-  if (a.success) a.success[e] = succ ? 1 : 0;
-  if (a.traj_qpos) for (int i = 0; i < a.nq; ++i) a.traj_qpos[e * a.nq + i] = q[i];
-  if (a.traj_qvel) for (int i = 0; i < a.nv; ++i) a.traj_qvel[e * a.nv + i] = v[i];
-  if (a.traj_time) a.traj_time[e] = tm;
-  const bool do_reset = a.apply_reset == 2 || (done && a.apply_reset == 1);
-  if (a.reset_mask) a.reset_mask[e] = do_reset ? 1 : 0;
-  if (a.episode_length) a.episode_length[e] = do_reset ? 0 : a.episode_length[e] + 1;
-  if (!do_reset) return;
-  // ---- fresh episode (engine.py:207-246): qpos from the reset table, everything else zero
-  for (int i = 0; i < a.nq; ++i) {
+  __syncthreads();
+  // ---- flat pass 2: fresh episodes (engine.py:207-246): qpos from the reset table, everything else zero
+  const uint64_t step = a.rng.step + (a.rng.step_base ? *a.rng.step_base : 0ull);
+  for (int idx = tid; idx < ne * nq; idx += 256) {
+    const int le = idx / nq, i = idx - le * nq;
+    if (!s_reset[le]) continue;
+    const int64_t e = e0 + le;
     float u;
-    if (a.reset_uniform) u = a.reset_uniform[e * (a.nq + 1) + i];
-    else u = 2.f * u01(draw(a.rng.seed, a.rng.step + (a.rng.step_base ? *a.rng.step_base : 0ull), kRngReset, (uint64_t)e, (uint32_t)i).x) - 1.f;
+    if (a.reset_uniform) u = a.reset_uniform[e * (nq + 1) + i];
+    else u = 2.f * u01(draw(a.rng.seed, step, kRngReset, (uint64_t)e, (uint32_t)i).x) - 1.f;
     const float mag = d.reset_mag[i] * (d.reset_by_level[i] ? a.level : 1.f);
-    float x = d.reset_base[i] + u * mag;
-    x = fminf(fmaxf(x, d.reset_lo[i]), d.reset_hi[i]);
-    q[i] = x;
+    const float x = d.reset_base[i] + u * mag;
+    qb[idx] = fminf(fmaxf(x, d.reset_lo[i]), d.reset_hi[i]);
   }
-  if (a.random_heading && a.nq >= 7) {
-    float u;
-    if (a.reset_uniform) u = a.reset_uniform[e * (a.nq + 1) + a.nq];
-    else u = 2.f * u01(draw(a.rng.seed, a.rng.step + (a.rng.step_base ? *a.rng.step_base : 0ull), kRngReset, (uint64_t)e, (uint32_t)a.nq).x) - 1.f;
-    const float h = 0.5f * 3.14159265358979323846f * u;  // yaw/2, yaw ~ U(-pi, pi)
-    const float cw = cosf(h), sz = sinf(h);
-    const float w = q[3], x = q[4], y = q[5], z = q[6];
-    q[3] = w * cw - z * sz; q[4] = x * cw + y * sz; q[5] = y * cw - x * sz; q[6] = z * cw + w * sz;
+  for (int idx = tid; idx < ne * nv; idx += 256) {
+    if (!s_reset[idx / nv]) continue;
+    vb[idx] = 0.f;
+    if (a.warm) a.warm[e0 * nv + idx] = 0.f;
   }
-  for (int i = 0; i < a.nv; ++i) v[i] = 0.f;
-  if (a.warm) for (int i = 0; i < a.nv; ++i) a.warm[e * a.nv + i] = 0.f;
-  if (a.time) a.time[e] = 0.f;
-  if (a.last_ctrl) for (int i = 0; i < a.nu; ++i) a.last_ctrl[e * a.nu + i] = 0.f;
+  if (a.last_ctrl)
+    for (int idx = tid; idx < ne * nu; idx += 256)
+      if (s_reset[idx / nu]) a.last_ctrl[e0 * nu + idx] = 0.f;
+  if (a.random_heading && nq >= 7) {
+    __syncthreads();  // the base orientation written above is read back by the env's own lane
+    if (tid < ne && s_reset[tid]) {
+      const int64_t e = e0 + tid;
+      float* q = qb + tid * nq;
+      float u;
+      if (a.reset_uniform) u = a.reset_uniform[e * (nq + 1) + nq];
+      else u = 2.f * u01(draw(a.rng.seed, step, kRngReset, (uint64_t)e, (uint32_t)nq).x) - 1.f;
+      const float h = 0.5f * 3.14159265358979323846f * u;  // yaw/2, yaw ~ U(-pi, pi)
+      const float cw = cosf(h), sz = sinf(h);
+      const float w = q[3], x = q[4], y = q[5], z = q[6];
+      q[3] = w * cw - z * sz; q[4] = x * cw + y * sz; q[5] = y * cw - x * sz; q[6] = z * cw + w * sz;
+    }
+  }
 }
 
 __global__ __launch_bounds__(256) void sample_action_kernel(int64_t n, int nu, const float* __restrict__ mean,
@@ -377,7 +413,8 @@ extern "C" int ks_terminate_reset(const KsTerms* t, ks_stream_t stream, const Ks
   a.reset_mask = io->reset_mask; a.episode_length = io->episode_length; a.reset_uniform = io->reset_uniform;
   a.rng = io->rng; a.apply_reset = io->apply_reset; a.nq = d.nq; a.nv = d.nv; a.nu = d.nu; a.n_terms = d.n_terms;
   a.random_heading = d.random_heading; a.nonfinite_terminates = d.nonfinite_terminates;
-  const int64_t grid = (io->N + 255) / 256;
+  const int64_t grid = (io->N + kTermEnvs - 1) / kTermEnvs;
+  if (grid > 0x7fffffff) return fail(KS_ELIMIT, "ks_terminate_reset: too many envs");
   hipLaunchKernelGGL(terminate_kernel, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, a);
   return check_launch("ks_terminate_reset");
 }
