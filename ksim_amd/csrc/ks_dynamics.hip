@@ -47,7 +47,7 @@ __host__ __device__ inline int j_stride(int nv) { return row_stride(nv); }
 struct Lds {
   float *qpos, *qvel, *warm, *tau;
   float *xpos, *xquat, *xanchor, *xaxis;
-  float *cinert, *crb, *cdof, *buf, *cvel, *cacc, *cfrc, *fsub;
+  float *cinert, *crb, *cdof, *buf, *cvel, *cfrc, *fsub;
   float *M, *J, *vbuf, *drow;
   float *con_off, *con_D, *con_kip;
   int *con_body, *sub_end;
@@ -62,7 +62,7 @@ __host__ __device__ inline int lds_floats(int nb, int nq, int nv, int nu, int ns
   n += up4(nq) + 32 + up4(nv) + up4(nu);                             // qpos qvel(32) warm tau
   n += up4(nb * 3) + up4(nb * 4) + 2 * up4(nb * 3);                    // xpos xquat xanchor xaxis
   n += up4(nv * 6) + up4(nb * 6);                                    // cdof cvel
-  const int scratch = 2 * up4(nb * 10) + up4(nv * 6) + 2 * up4(nb * 6);  // cinert crb buf cacc(=fsub) cfrc
+  const int scratch = 2 * up4(nb * 10) + up4(nv * 6) + 2 * up4(nb * 6);  // cinert crb buf fsub cfrc
   const int jsz = up4(4 * ns * js + 32);                             // J overlays that scratch once it is dead
   n += scratch > jsz ? scratch : jsz;
   n += up4(nv * nvs) + 32 + 64;                                      // M vbuf drow
@@ -84,8 +84,7 @@ __device__ inline Lds carve(float* p, const DevModel& m) {
   {
     float* base = p;
     l.cinert = take(nb * 10); l.crb = take(nb * 10); l.buf = take(nv * 6);
-    l.cacc = take(nb * 6); l.cfrc = take(nb * 6);
-    l.fsub = l.cacc;  // the subtree force sums replace the accelerations once the level passes are done
+    l.fsub = take(nb * 6); l.cfrc = take(nb * 6);
     float* end = p;
     l.J = base;  // written only after the bias forces are out of fsub
     float* jend = base + up4(4 * ns * js + 32);
@@ -309,47 +308,66 @@ void step_kernel(StepArgs a) {
     }
 
     KS_TICK(0)
-    // ---- kinematics, one tree level per pass (parents are complete before their children read them)
+    // ---- kinematics.  Every body first writes its pose relative to its parent (joint rotation included) to
+    // LDS, then composes the poses along its own chain of ancestors from the root down: max_depth short
+    // steps shared by all bodies instead of one full pass per tree level.
     V3 xipos = {0.f, 0.f, 0.f};
     Mat3 ximat;
 #pragma unroll
     for (int k = 0; k < 9; ++k) ximat.m[k] = 0.f;
-    float hs = 0.f, hc = 1.f;
-    if (is_body && b_jtype == kJntHinge) sincosf(0.5f * (l.qpos[b_qadr] - b_q0), &hs, &hc);
-    for (int lev = 1; lev <= m.max_depth; ++lev) {
-      if (b_depth == lev) {
-        const int b = lane;
-        V3 pos, anchor, axis = {0.f, 0.f, 1.f};
-        Quat quat;
-        if (b_jtype == kJntFree) {
-          pos = ld3(l.qpos + b_qadr);
-          quat = qnormalize({l.qpos[b_qadr + 3], l.qpos[b_qadr + 4], l.qpos[b_qadr + 5], l.qpos[b_qadr + 6]});
-          anchor = pos;
-        } else {
-          const Quat pq = {l.xquat[4 * b_parent], l.xquat[4 * b_parent + 1], l.xquat[4 * b_parent + 2],
-                           l.xquat[4 * b_parent + 3]};
-          pos = ld3(l.xpos + 3 * b_parent) + mul(q2mat(pq), b_pos);
-          Quat nq_ = qmul(pq, b_quat);
-          anchor = pos;
-          if (b_jtype == kJntHinge) {
-            const Mat3 Rn = q2mat(nq_);
-            anchor = pos + mul(Rn, b_jpos);
-            axis = mul(Rn, b_jaxis);
-            nq_ = qmul(nq_, {hc, b_jaxis.x * hs, b_jaxis.y * hs, b_jaxis.z * hs});
-            pos = anchor - mul(q2mat(nq_), b_jpos);
-          }
-          quat = qnormalize(nq_);
+    float* lpose = l.cinert;  // 7 floats per body; the inertia scratch is not in use yet
+    if (is_body) {
+      V3 tl;
+      Quat ql;
+      if (b_jtype == kJntFree) {
+        tl = ld3(l.qpos + b_qadr);
+        ql = qnormalize({l.qpos[b_qadr + 3], l.qpos[b_qadr + 4], l.qpos[b_qadr + 5], l.qpos[b_qadr + 6]});
+      } else {
+        tl = b_pos;
+        ql = b_quat;
+        if (b_jtype == kJntHinge) {
+          float hs, hc;
+          sincosf(0.5f * (l.qpos[b_qadr] - b_q0), &hs, &hc);
+          const Quat jr = {hc, b_jaxis.x * hs, b_jaxis.y * hs, b_jaxis.z * hs};
+          // rotation about the joint anchor: p + R_b (a - R_j a) with a the anchor in the body frame
+          const V3 ra = mul(q2mat(jr), b_jpos);
+          tl = b_pos + mul(q2mat(b_quat), b_jpos - ra);
+          ql = qmul(b_quat, jr);
         }
+      }
+      st3(lpose + 7 * lane, tl);
+      lpose[7 * lane + 3] = ql.w; lpose[7 * lane + 4] = ql.x; lpose[7 * lane + 5] = ql.y; lpose[7 * lane + 6] = ql.z;
+    }
+    KS_SYNC();
+    {
+      V3 pos = {0.f, 0.f, 0.f};
+      Quat quat = {1.f, 0.f, 0.f, 0.f};
+      for (int k = 0; k < m.max_depth; ++k) {
+        if (k < b_depth) {
+          const int cb = m.body_chain[bl][k];
+          const V3 tl = ld3(lpose + 7 * cb);
+          const Quat ql = {lpose[7 * cb + 3], lpose[7 * cb + 4], lpose[7 * cb + 5], lpose[7 * cb + 6]};
+          pos = pos + mul(q2mat(quat), tl);
+          quat = qmul(quat, ql);
+        }
+      }
+      if (is_body) {
+        quat = qnormalize(quat);
         const Mat3 R = q2mat(quat);
-        st3(l.xpos + 3 * b, pos);
-        l.xquat[4 * b] = quat.w; l.xquat[4 * b + 1] = quat.x; l.xquat[4 * b + 2] = quat.y; l.xquat[4 * b + 3] = quat.z;
-        st3(l.xanchor + 3 * b, anchor);
-        st3(l.xaxis + 3 * b, axis);
+        V3 anchor = pos, axis = {0.f, 0.f, 1.f};
+        if (b_jtype == kJntHinge) {
+          anchor = pos + mul(R, b_jpos);
+          axis = mul(R, b_jaxis);
+        }
+        st3(l.xpos + 3 * lane, pos);
+        l.xquat[4 * lane] = quat.w; l.xquat[4 * lane + 1] = quat.x; l.xquat[4 * lane + 2] = quat.y; l.xquat[4 * lane + 3] = quat.z;
+        st3(l.xanchor + 3 * lane, anchor);
+        st3(l.xaxis + 3 * lane, axis);
         xipos = pos + mul(R, b_ipos);
         ximat = q2mat(qnormalize(qmul(quat, b_iquat)));
       }
-      KS_SYNC();
     }
+    KS_SYNC();
 
     KS_TICK(1)
     // ---- centre of mass of the tree (wave-uniform), com-based inertias and motion axes
@@ -359,7 +377,7 @@ void step_kernel(StepArgs a) {
                     wave_sum(b_mass * xipos.z) * minv};
     if (lane == 0) {  // world body entries of the per-substep scratch (the scratch is reused by J later)
       for (int k = 0; k < 10; ++k) l.cinert[k] = 0.f;
-      for (int k = 0; k < 6; ++k) { l.cfrc[k] = 0.f; l.cacc[k] = k < 3 ? 0.f : -m.gravity[k - 3]; }
+      for (int k = 0; k < 6; ++k) l.cfrc[k] = 0.f;
     }
     float ci[10];
     {
@@ -422,32 +440,39 @@ void step_kernel(StepArgs a) {
     }
 
     KS_TICK(3)
-    // ---- body velocities, axis derivatives, RNE forces: one tree level per pass
-    for (int lev = 1; lev <= m.max_depth; ++lev) {
-      if (b_depth == lev) {
-        Sp v = ld6(l.cvel + 6 * b_parent), acc = ld6(l.cacc + 6 * b_parent);
-        if (b_jtype == kJntFree) {
-          for (int k = 0; k < 3; ++k) v = v + ld6(l.cdof + 6 * (b_dofadr + k)) * l.qvel[b_dofadr + k];
-          Sp dv = {{0.f, 0.f, 0.f}, {0.f, 0.f, 0.f}};
-          for (int k = 3; k < 6; ++k) {
-            const Sp cd = ld6(l.cdof + 6 * (b_dofadr + k));
-            const float qd = l.qvel[b_dofadr + k];
+    // ---- body velocities and bias accelerations: the motion axes are all expressed in one frame, so every
+    // body accumulates them over the dofs of its own ancestor chain, root first (no pass per tree level)
+    {
+      Sp v = {{0.f, 0.f, 0.f}, {0.f, 0.f, 0.f}};
+      Sp acc = {{0.f, 0.f, 0.f}, {-m.gravity[0], -m.gravity[1], -m.gravity[2]}};
+      for (int k = 0; k < m.max_depth; ++k) {
+        if (k < b_depth) {
+          const int cb = m.body_chain[bl][k];
+          const int jt = m.body_jtype[cb], da = m.body_dofadr[cb];
+          if (jt == kJntFree) {
+            for (int c = 0; c < 3; ++c) v = v + ld6(l.cdof + 6 * (da + c)) * l.qvel[da + c];
+            Sp dv = {{0.f, 0.f, 0.f}, {0.f, 0.f, 0.f}};
+            for (int c = 3; c < 6; ++c) {
+              const Sp cd = ld6(l.cdof + 6 * (da + c));
+              const float qd = l.qvel[da + c];
+              acc = acc + cross_motion(v, cd) * qd;
+              dv = dv + cd * qd;
+            }
+            v = v + dv;
+          } else if (jt == kJntHinge) {
+            const Sp cd = ld6(l.cdof + 6 * da);
+            const float qd = l.qvel[da];
             acc = acc + cross_motion(v, cd) * qd;
-            dv = dv + cd * qd;
+            v = v + cd * qd;
           }
-          v = v + dv;
-        } else if (b_jtype == kJntHinge) {
-          const Sp cd = ld6(l.cdof + 6 * b_dofadr);
-          const float qd = l.qvel[b_dofadr];
-          acc = acc + cross_motion(v, cd) * qd;
-          v = v + cd * qd;
         }
+      }
+      if (is_body) {
         st6(l.cvel + 6 * lane, v);
-        st6(l.cacc + 6 * lane, acc);
         st6(l.cfrc + 6 * lane, inert_mul(ci, acc) + cross_force(v, inert_mul(ci, v)));
       }
-      KS_SYNC();
     }
+    KS_SYNC();
     for (int idx = lane; idx < nb * 6; idx += 64) {
       const int b = idx / 6, k = idx - 6 * b;
       l.fsub[idx] = b > 0 ? range_sum(l.cfrc + k, 6, b, l.sub_end[b]) : 0.f;
