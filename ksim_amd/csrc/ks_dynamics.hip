@@ -2,14 +2,14 @@
 //
 // One 64-lane wavefront owns one env (64-thread workgroups, so a workgroup barrier is a wave barrier).
 // Where the data lives:
-//   registers  row i of the mass matrix, of the Newton Hessian / its Cholesky factor and (for lanes that are
-//              constraint rows) of the constraint Jacobian; the lane's own body / dof / sphere constants;
-//              all per-dof and per-row solver vectors
+//   registers  the mass matrix / Newton Hessian as a 32x32 matrix-core accumulator tile while it is assembled and
+//              factored, then row i of the factor for the substitutions; the lane's own body / dof / sphere
+//              constants; all per-dof and per-row solver vectors
 //   LDS        state (qpos, qvel, warm start, torques), body poses, com-based inertias and motion axes,
 //              a staging copy of M and of J (column access), one broadcast vector
 //   HBM        touched once at the start and once at the end of the control step
-// Cross-lane traffic is v_readlane broadcasts (Cholesky, triangular solves), DPP reductions and LDS
-// broadcasts; every branch on solver progress is wave-uniform, so a converged env stops iterating.
+// Cross-lane traffic is v_readlane broadcasts (pivots, triangular solves), DPP reductions and LDS
+// broadcasts; the rank updates of the Hessian and of its factorisation run as 32x32x2 fp32 MFMAs; every branch on solver progress is wave-uniform, so a converged env stops iterating.
 // Phases of one substep: level-wise kinematics -> centre of mass -> com-based inertias / motion axes ->
 // composite inertias -> mass matrix -> level-wise velocities + RNE bias -> smooth forces -> sphere/plane
 // contacts, pyramidal rows -> Cholesky of M -> Newton with exact line search -> semi-implicit Euler.
@@ -110,30 +110,56 @@ __device__ __forceinline__ void load_row(const float* p, float (&v)[NP]) {
 }
 
 
-// In-register Cholesky, right-looking on the full symmetric rows: lane i holds row i of the matrix in R[0..NP).
-// Step j scales column j below the diagonal into L and subtracts the rank-1 term from every later row, all
-// NP-1-j updates of a step being independent FMAs.  Row j of the running Schur complement is fetched from lane
-// j with v_readlane, so there is no LDS traffic and no barrier.  On return, in lane i:
-//   R[j], j < i : L[i][j]                       (row i of L, for the forward substitution)
-//   R[k], k > i : L[k][i] * L[i][i]             (column i of L times its pivot root, for the backward one)
-// and myinv = 1 / L[i][i] (kept per lane rather than as NP wave-uniform values, which would sit in scalar
-// registers the kernel is short of).  Keeping both triangles makes both substitutions column-oriented: one lane
-// read and one FMA per column, no cross-lane sums.
+// Right-looking Cholesky of a symmetric matrix of up to 32 rows with the rank-1 updates on the matrix cores.
+// The matrix sits in the accumulator layout of the 32x32x2 fp32 MFMA: lane c + 32 h holds, in register
+// 4 g + e, the entry (row 8 g + 4 h + e, column c).  Step j reads the pivot from the lane that owns column j, scales row j (one register of the 32 lanes of one
+// half) and feeds that scaled row to one MFMA as both operands, -l l^T, which updates every entry right of and
+// below the pivot at once; the other lane half contributes zeros.  A step costs about eight vector instructions
+// instead of two per updated column.  Column j below the diagonal is left as it was when the pivot was reached
+// (L[k][j] * L[j][j]) and row j right of the diagonal holds L[k][j]: read down a lane, that is row c of L to the
+// left of the diagonal and the scaled column c below it, exactly what the column-oriented substitutions take,
+// once the upper lane half has handed its 16 registers to the lower one.  On return, in lane i < NP:
+//   R[j], j < i : L[i][j]              R[k], k > i : L[k][i] * L[i][i]              myinv = 1 / L[i][i]
 template <int NP>
-__device__ __forceinline__ void chol_regs(float (&R)[NP], float& myinv, int lane) {
+__device__ __forceinline__ void chol_tile(f32x16& T, float (&R)[NP], float& myinv, int lane) {
+  const int c = lane & 31, half = lane >> 5;
   myinv = 1.f;
 #pragma unroll
   for (int j = 0; j < NP; ++j) {
-    // every lane computes the same 1 / sqrt(pivot) from the broadcast pivot (v_rsq_f32 is accurate to 1 ulp)
-    const float piv = fmaxf(lane_bcast(R[j], j), 1e-30f);
+    const int hj = (j >> 2) & 1, rho = 4 * (j >> 3) + (j & 3);
+    const float piv = fmaxf(lane_bcast(T[rho], j + 32 * hj), 1e-30f);
     const float inv = __builtin_amdgcn_rsqf(piv);
-    const bool below = lane > j;
     myinv = lane == j ? inv : myinv;
-    const float t = R[j] * inv;
-    const float w = below ? t * inv : 0.f;
-    R[j] = below ? t : R[j];
+    const bool sel = half == hj && c > j;
+    const float t = T[rho] * inv;
+    const float a = sel ? t : 0.f;
+    T[rho] = sel ? t : T[rho];
+    if (j + 1 < NP) T = __builtin_amdgcn_mfma_f32_32x32x2f32(-a, a, T, 0, 0, 0);
+  }
 #pragma unroll
-    for (int k = j + 1; k < NP; ++k) R[k] -= w * lane_bcast(R[k], j);
+  for (int g = 0; g < 4; ++g)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int jlo = 8 * g + e, jhi = 8 * g + 4 + e;
+      if (jlo < NP) R[jlo] = T[4 * g + e];
+      if (jhi < NP) R[jhi] = __shfl_xor(T[4 * g + e], 32);
+    }
+}
+
+// Mass matrix (LDS, rows of `stride` floats, zero beyond nv) into the accumulator layout, unit diagonal on the padding.
+__device__ __forceinline__ void load_mtile(f32x16& T, const float* __restrict__ M, int stride, int nv, int np, int lane) {
+  const int c = lane & 31, half = lane >> 5;
+  const bool real = c < nv;
+  const float* row = M + (real ? c : 0) * stride;
+#pragma unroll
+  for (int g = 0; g < 4; ++g) {
+    const int r0 = 8 * g + 4 * half;
+    const bool inside = r0 + 4 <= np;
+    const float4 v = *reinterpret_cast<const float4*>(row + (inside ? r0 : 0));
+    T[4 * g] = (real && inside) ? v.x : (r0 == c ? 1.f : 0.f);
+    T[4 * g + 1] = (real && inside) ? v.y : (r0 + 1 == c ? 1.f : 0.f);
+    T[4 * g + 2] = (real && inside) ? v.z : (r0 + 2 == c ? 1.f : 0.f);
+    T[4 * g + 3] = (real && inside) ? v.w : (r0 + 3 == c ? 1.f : 0.f);
   }
 }
 
@@ -535,12 +561,14 @@ void step_kernel(StepArgs a) {
     KS_TICK(6)
     // ---- Cholesky of M and the unconstrained acceleration (registers only)
     float R[NP];
-    load_row<NP>(Mrow, R);
-#pragma unroll
-    for (int j = 0; j < NP; ++j) R[j] = is_dof ? R[j] : (lane == j ? 1.f : 0.f);
     float myinv;
-    chol_regs<NP>(R, myinv, lane);
-    const float qas = solve_regs<NP>(R, myinv, lane, qfs);
+    {
+      f32x16 T;
+      load_mtile(T, l.M, nvs, nv, NP, lane);
+      chol_tile<NP>(T, R, myinv, lane);
+    }
+    const float qas_all = solve_regs<NP>(R, myinv, lane, qfs);
+    const float qas = is_dof ? qas_all : 0.f;  // lanes that hold no row carry meaningless numbers
     if (a.dbg_qacc_smooth && is_dof) a.dbg_qacc_smooth[env * nv + lane] = qas;
 
     KS_TICK(7)
@@ -644,10 +672,7 @@ void step_kernel(StepArgs a) {
         KS_SYNC();
         {
           f32x16 hc;
-#pragma unroll
-          for (int q = 0; q < 16; ++q) hc[q] = 0.f;
-          float mr[NP];
-          load_row<NP>(Mrow, mr);
+          load_mtile(hc, l.M, nvs, nv, NP, lane);
           const int col = lane & 31, half = lane >> 5;
           const bool col_ok = NP == 32 || col < NP;
           for (int r0 = 0; r0 < nefc; r0 += 2) {
@@ -655,19 +680,11 @@ void step_kernel(StepArgs a) {
             const float jv = (col_ok && r < nefc) ? l.J[r * js + col] : 0.f;
             hc = __builtin_amdgcn_mfma_f32_32x32x2f32(l.drow[r] * jv, jv, hc, 0, 0, 0);
           }
-#pragma unroll
-          for (int g = 0; g < 4; ++g)
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              const float other = __shfl_xor(hc[4 * g + e], 32);
-              const int jlo = 8 * g + e, jhi = 8 * g + 4 + e;
-              if (jlo < NP) R[jlo] = is_dof ? mr[jlo] + hc[4 * g + e] : (lane == jlo ? 1.f : 0.f);
-              if (jhi < NP) R[jhi] = is_dof ? mr[jhi] + other : (lane == jhi ? 1.f : 0.f);
-            }
+          KS_TICK(11)
+          chol_tile<NP>(hc, R, myinv, lane);
         }
-        KS_TICK(11)
-        chol_regs<NP>(R, myinv, lane);
-        const float search = -solve_regs<NP>(R, myinv, lane, grad);
+        const float search_all = -solve_regs<NP>(R, myinv, lane, grad);
+        const float search = is_dof ? search_all : 0.f;
         KS_TICK(12)
 
         // ---- exact line search along `search`
