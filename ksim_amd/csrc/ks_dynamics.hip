@@ -18,6 +18,7 @@
 #include "ks_model.h"
 #include "ks_step_args.h"
 
+#include <cmath>
 #include <cstring>
 
 namespace ks {
@@ -546,8 +547,12 @@ void step_kernel(StepArgs a) {
       st3(l.con_off + 3 * c, cpos - com);
       const float invweight = (s_invw + mu * mu * s_invw) * 2.f * mu * mu / m.impratio;
       const float ix = fabsf(dist) / m.width;
-      const float ia = (1.0f / powf(m.mid, m.power - 1.f)) * powf(ix, m.power);
-      const float ib = 1.f - (1.0f / powf(1.f - m.mid, m.power - 1.f)) * powf(1.f - ix, m.power);
+      // x^power: the default power of 2 (and 1) without the general power function
+      const float ox = 1.f - ix;
+      const float px = m.power == 2.f ? ix * ix : (m.power == 1.f ? ix : powf(ix, m.power));
+      const float po = m.power == 2.f ? ox * ox : (m.power == 1.f ? ox : powf(ox, m.power));
+      const float ia = m.imp_a * px;
+      const float ib = 1.f - m.imp_b * po;
       const float iy = ix < m.mid ? ia : ib;
       float imp = m.dmin + iy * (m.dmax - m.dmin);
       imp = fminf(fmaxf(imp, m.dmin), m.dmax);
@@ -854,6 +859,7 @@ extern "C" int ks_model_create(const KsModelDesc* d, KsModel** out) {
     if (d->solref[1] <= 0) b = -d->solref[1] / dmax;
     m.con_k = (float)k; m.con_b = (float)b; m.dmin = (float)dmin; m.dmax = (float)dmax; m.width = (float)width;
     m.mid = (float)mid; m.power = (float)power;
+    m.imp_a = (float)(1.0 / std::pow(mid, power - 1.0)); m.imp_b = (float)(1.0 / std::pow(1.0 - mid, power - 1.0));
   }
   for (int b = 0; b < d->nb; ++b) {
     m.body_parent[b] = d->body_parent[b]; m.body_jtype[b] = d->body_jtype[b]; m.body_qadr[b] = d->body_qadr[b];

@@ -24,6 +24,7 @@ struct DevModel {
   float dt, gravity[3], tolerance, ls_tolerance, meaninertia, friction, impratio;
   // contact impedance constants, already clamped the way the constraint builder wants them
   float con_k, con_b, dmin, dmax, width, mid, power;
+  float imp_a, imp_b;  // 1 / mid^(power-1) and 1 / (1-mid)^(power-1), the constant factors of the impedance curve
   int body_parent[kMaxB], body_jtype[kMaxB], body_qadr[kMaxB], body_dofadr[kMaxB], body_subtree_end[kMaxB],
       body_depth[kMaxB];
   int body_chain[kMaxB][kMaxDepth];  // ancestors from the tree root down to the body itself
