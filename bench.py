@@ -162,6 +162,13 @@ def main() -> None:
         for ln in open(tpath):
             if ln.startswith("hbm_bytes_per_launch="):
                 traffic = float(ln.split("=", 1)[1])
+    valu = {}
+    vpath = os.path.join(ROOT, "profiles", "step_kernel_cfg4_instruction_mix.txt")
+    if os.path.exists(vpath):  # rocprofv3 --pmc SQ_* summary, see that file
+        for ln in open(vpath):
+            if ln.startswith("valu_"):
+                k, v = ln.strip().split("=", 1)
+                valu[k] = float(v)
     line = {
         "metric": "env-steps/sec, 8192-env humanoid rollout (1 GPU)", "value": N * args.steps / elapsed,
         "unit": "env-steps/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -174,7 +181,10 @@ def main() -> None:
         "roofline": {"bound": "hbm", "kernel": "step_kernel (fused control step)", "achieved": achieved,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
                      "algorithmic_bytes_per_env_step": bytes_per_env, "kernel_ms": kernel_ms,
-                     "note": "the fused step is fp32-VALU/LDS-bound (~1e3 flop/byte); the HBM fraction is reported "
+                     "valu_issue_fraction_profiled": valu.get("valu_issue_fraction"),
+                     "valu_insts_per_env_step_profiled": valu.get("valu_insts_per_env_step"),
+                     "note": "the fused step is bound by fp32 vector-ALU issue (~1e3 flop/byte; the profiled share of "
+                             "cycles with a VALU instruction issuing is given beside); the HBM fraction is reported "
                              "against the bytes the engine contract obliges a step to move"},
         "gae": gae, "policy_mlp": mlp, "graph_replay": graph,
     }

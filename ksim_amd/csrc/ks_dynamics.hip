@@ -9,10 +9,11 @@
 //              a staging copy of M and of J (column access), one broadcast vector
 //   HBM        touched once at the start and once at the end of the control step
 // Cross-lane traffic is v_readlane broadcasts (pivots, triangular solves), DPP reductions and LDS
-// broadcasts; the rank updates of the Hessian and of its factorisation run as 32x32x2 fp32 MFMAs; every branch on solver progress is wave-uniform, so a converged env stops iterating.
-// Phases of one substep: level-wise kinematics -> centre of mass -> com-based inertias / motion axes ->
-// composite inertias -> mass matrix -> level-wise velocities + RNE bias -> smooth forces -> sphere/plane
-// contacts, pyramidal rows -> Cholesky of M -> Newton with exact line search -> semi-implicit Euler.
+// broadcasts; the rank updates of the Hessian and of its factorisation run as 32x32x2 fp32 MFMAs; every
+// branch on solver progress is wave-uniform, so a converged env stops iterating.
+// Phases of one substep: kinematics along ancestor chains -> centre of mass -> com-based inertias / motion
+// axes -> composite inertias -> mass matrix -> velocities + RNE bias along ancestor chains -> smooth forces ->
+// sphere/plane contacts, pyramidal rows -> Cholesky of M -> Newton with exact line search -> semi-implicit Euler.
 // The arithmetic follows the MuJoCo model that ksim/engine.py:257 invokes through mjx.step.
 #include "ks_common.h"
 #include "ks_model.h"
