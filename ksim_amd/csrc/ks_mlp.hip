@@ -209,6 +209,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void mlp_layer_kernel(int64
 // one contiguous 1 KB read) through a register ring kPF steps deep; activation fragments come from LDS.
 constexpr int kFusedMaxWidth = 512;
 constexpr int kFusedWaves = 8;
+// ring depth: 4 steps, 2 for the 64-row tile (two workgroups per CU, 128 registers each)
 constexpr int kPF = 4;
 
 struct FusedArgs {
@@ -240,7 +241,7 @@ __device__ __forceinline__ unsigned pack_bf16(float lo, float hi) {
 // One layer's MFMA work of one wavefront: NT output tiles (weights w[t]) times MI row tiles.  `arow` points at
 // this lane's activation fragment of K step 0 (row lane % 32 of the first row tile, k half lane / 32).
 // Weight fragments sit in a register ring kPF steps ahead; activation fragments are read one step ahead.
-template <int NT, int MI>
+template <int NT, int MI, int kPF>
 __device__ __forceinline__ void fused_layer_mma(f32x16 (&acc)[2][MI], const u32x4* __restrict__ w0,
                                                 const u32x4* __restrict__ w1, int nk, const __bf16* __restrict__ arow,
                                                 int lda) {
@@ -347,7 +348,7 @@ __device__ __forceinline__ void fused_layer(const FusedArgs& a, int l, __bf16* _
     fused_bias_init(acc[0][0], a.bp[l], j, lane);
     acc[1][0] = acc[0][0];
     const u32x4* w0 = a.Wp[l] + (int64_t)j * nk * 64 + lane;
-    if (busy) fused_layer_mma<1, 1>(acc, w0, w0, nk, arow + i * 32 * lda, lda);
+    if (busy) fused_layer_mma<1, 1, (MI == 2 ? 2 : kPF)>(acc, w0, w0, nk, arow + i * 32 * lda, lda);
     KS_MLP_STAMP2(2 + 3 * l)
     __syncthreads();  // every wavefront has read this layer's input; the tile can be overwritten
     KS_MLP_STAMP2(3 + 3 * l)
@@ -368,8 +369,8 @@ __device__ __forceinline__ void fused_layer(const FusedArgs& a, int l, __bf16* _
     }
     const u32x4* w0 = a.Wp[l] + (int64_t)j0 * nk * 64 + lane;
     const u32x4* w1 = a.Wp[l] + (int64_t)j1 * nk * 64 + lane;
-    if (mine == 2) fused_layer_mma<2, MI>(acc, w0, w1, nk, arow, lda);
-    else if (mine == 1) fused_layer_mma<1, MI>(acc, w0, w0, nk, arow, lda);
+    if (mine == 2) fused_layer_mma<2, MI, (MI == 2 ? 2 : kPF)>(acc, w0, w1, nk, arow, lda);
+    else if (mine == 1) fused_layer_mma<1, MI, (MI == 2 ? 2 : kPF)>(acc, w0, w0, nk, arow, lda);
     KS_MLP_STAMP2(2 + 3 * l)
     __syncthreads();
     KS_MLP_STAMP2(3 + 3 * l)
