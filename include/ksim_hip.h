@@ -32,7 +32,7 @@ const char* ks_version(void);
 const char* ks_last_error(void);
 /* sizeof() of a public struct as this library was compiled, for binding self-checks:
  * 0 KsPpoLossParams, 1 KsModelDesc, 2 KsStepIO, 3 KsTermsDesc, 4 KsObserveIO, 5 KsTerminateIO, 6 KsMlpDesc,
- * 7 KsRewardIO, 8 KsObsElem, 9 KsTermDesc, 10 KsRewardDesc, 11 KsRng; -1 for anything else. */
+ * 7 KsRewardIO, 8 KsObsElem, 9 KsTermDesc, 10 KsRewardDesc, 11 KsRng, 12 KsAdamParams; -1 for anything else. */
 int64_t ks_abi_sizeof(int32_t which);
 
 /* ------------------------------------------------------------------ GAE / returns
@@ -335,6 +335,54 @@ int ks_mlp_destroy(KsMlp* mlp);
 int64_t ks_mlp_workspace_bytes(const KsMlp* mlp, int64_t M);
 int ks_mlp_forward(const KsMlp* mlp, ks_stream_t stream, int64_t M, const float* x /*(M, in)*/,
                    float* y /*(M, out)*/, void* workspace);
+
+/* ------------------------------------------------------------------ policy update: gradients and optimiser
+ * The native pieces of PPOTask._single_step / update_model (ksim/task/ppo.py:495-565, 572-694) for an
+ * MLP actor / critic with a Gaussian head: the backward pass that jax.grad performs through
+ * _get_ppo_loss_and_metrics (ppo.py:412-492) and the optax chain of the examples' get_optimizer
+ * (examples/walking.py:373-387: zero_nans, clip_by_global_norm, add_decayed_weights, scale_by_adam,
+ * learning rate, -1).  ks_mlp_train_init keeps fp32 master weights, gradients and Adam moments beside
+ * the working-precision copies that ks_mlp_forward reads; after ks_mlp_adam_step every copy is refreshed.
+ *   ks_mlp_train_forward  y = net(x), hidden activations kept in `workspace` for the backward pass
+ *   ks_mlp_train_backward gradients of sum(dy * y) w.r.t. every weight and bias, into the handle
+ *   ks_grad_sqnorm        adds the squared norm of n floats (NaNs skipped) to *acc (device double)
+ *   ks_mlp_grad_sqnorm    the same over all gradients of a network
+ *   ks_mlp_adam_step      one optimiser step with `sqnorm` = squared global gradient norm over everything
+ *                         that is optimised together (NULL or max_grad_norm <= 0: no clipping)
+ *   ks_adam_step          the same chain on a bare parameter vector (e.g. the log standard deviations) */
+typedef struct KsAdamParams {
+  float lr, b1, b2, eps, weight_decay, max_grad_norm;
+  int64_t step; /* 1 for the first update (bias correction) */
+} KsAdamParams;
+int ks_mlp_train_init(KsMlp* mlp);
+int64_t ks_mlp_train_workspace_bytes(const KsMlp* mlp, int64_t M);
+int ks_mlp_train_forward(KsMlp* mlp, ks_stream_t stream, int64_t M, const float* x, float* y, void* workspace);
+int ks_mlp_train_backward(KsMlp* mlp, ks_stream_t stream, int64_t M, const float* x, const float* dy /*(M, out)*/,
+                          void* workspace);
+int ks_grad_sqnorm(ks_stream_t stream, int64_t n, const float* g, double* acc);
+int ks_mlp_grad_sqnorm(const KsMlp* mlp, ks_stream_t stream, double* acc);
+int ks_mlp_adam_step(KsMlp* mlp, ks_stream_t stream, const KsAdamParams* params /*host*/, const double* sqnorm);
+int ks_adam_step(ks_stream_t stream, int64_t n, float* param, const float* grad, float* m1, float* m2,
+                 const KsAdamParams* params /*host*/, const double* sqnorm);
+/* Copies of the parameters and gradients in the caller's (out, in) layout, for checks and checkpoints. */
+int ks_mlp_get_params(const KsMlp* mlp, ks_stream_t stream, int32_t layer, float* weight /*(out,in) dev*/, float* bias /*(out) dev*/,
+                      int32_t gradients /*0: parameters, 1: gradients*/);
+
+/* Gaussian policy head and the gradient of the PPO objective (ppo.py:149-246, total 473-486):
+ *   ks_gaussian_log_prob: per action dimension log N(action; mean, exp(log_std)) and entropy
+ *   ks_ppo_loss_grad: d(total loss)/d(mean), d/d(value), d/d(log_std) for the mean over the M rows of
+ *   policy + value + kl + entropy terms, with the new log-probabilities taken from (mean, log_std, action).
+ *   d_log_std is overwritten; workspace >= KS_PPO_GRAD_WORKSPACE_BYTES(nu). */
+int ks_gaussian_log_prob(ks_stream_t stream, int64_t M, int32_t nu, const float* mean, const float* log_std,
+                         const float* action, float* log_prob /*(M,nu)*/, float* entropy /*(M,nu) nullable*/);
+#define KS_MAX_ACTIONS 32
+#define KS_PPO_GRAD_BLOCKS 256
+#define KS_PPO_GRAD_WORKSPACE_BYTES(nu) ((size_t)KS_PPO_GRAD_BLOCKS * (nu) * 4)
+int ks_ppo_loss_grad(ks_stream_t stream, int64_t M, int32_t nu, const KsPpoLossParams* params /*host*/,
+                     const float* mean, const float* log_std, const float* action, const float* on_log_probs /*(M,nu)*/,
+                     const float* advantages, const float* value_targets, const float* on_values,
+                     const float* values, float* d_mean /*(M,nu)*/, float* d_value /*(M)*/, float* d_log_std /*(nu)*/,
+                     void* workspace);
 
 /* ------------------------------------------------------------------ rewards over a rollout
  * Replaces get_rewards + the stateless Reward.get_reward terms the configs name

@@ -56,6 +56,8 @@ def load() -> ctypes.CDLL:
     lib.ks_reward_total.argtypes = [p, c_int64, c_int32, p, POINTER(c_float), c_int32, c_float, c_int32, c_float, p,
                                     c_int32, p, p, p]
     lib.ks_copy_f32.argtypes = [p, c_int64, p, p]
+    lib.ks_ppo_loss_grad.argtypes = [p, c_int64, c_int32, POINTER(KsPpoLossParams)] + [p] * 12
+    lib.ks_ppo_loss_grad.restype = c_int32
     for name in ("ks_gae_bt", "ks_gae_tn", "ks_normalize_advantages", "ks_ppo_loss", "ks_reward_total", "ks_copy_f32"):
         getattr(lib, name).restype = c_int32
     _bind_optional(lib)

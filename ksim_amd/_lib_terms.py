@@ -78,6 +78,11 @@ class KsRewardIO(ctypes.Structure):
                 ("disc_logits", c_void_p), ("components", c_void_p), ("total", c_void_p)]
 
 
+class KsAdamParams(ctypes.Structure):
+    _fields_ = [("lr", c_float), ("b1", c_float), ("b2", c_float), ("eps", c_float), ("weight_decay", c_float),
+                ("max_grad_norm", c_float), ("step", c_int64)]
+
+
 def bind(lib) -> None:
     lib.ks_rewards.argtypes = [c_void_p, POINTER(KsRewardIO)]
     lib.ks_rewards.restype = c_int32
@@ -92,6 +97,20 @@ def bind(lib) -> None:
     lib.ks_mlp_workspace_bytes.argtypes = [c_void_p, c_int64]
     lib.ks_mlp_workspace_bytes.restype = c_int64
     lib.ks_mlp_forward.argtypes = [c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_void_p]
+    lib.ks_mlp_train_init.argtypes = [c_void_p]
+    lib.ks_mlp_train_workspace_bytes.argtypes = [c_void_p, c_int64]
+    lib.ks_mlp_train_workspace_bytes.restype = c_int64
+    lib.ks_mlp_train_forward.argtypes = [c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_void_p]
+    lib.ks_mlp_train_backward.argtypes = [c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_void_p]
+    lib.ks_grad_sqnorm.argtypes = [c_void_p, c_int64, c_void_p, c_void_p]
+    lib.ks_mlp_grad_sqnorm.argtypes = [c_void_p, c_void_p, c_void_p]
+    lib.ks_mlp_adam_step.argtypes = [c_void_p, c_void_p, POINTER(KsAdamParams), c_void_p]
+    lib.ks_adam_step.argtypes = [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, POINTER(KsAdamParams), c_void_p]
+    lib.ks_mlp_get_params.argtypes = [c_void_p, c_void_p, c_int32, c_void_p, c_void_p, c_int32]
+    lib.ks_gaussian_log_prob.argtypes = [c_void_p, c_int64, c_int32, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]
+    for name in ("ks_mlp_train_init", "ks_mlp_train_forward", "ks_mlp_train_backward", "ks_grad_sqnorm",
+                 "ks_mlp_grad_sqnorm", "ks_mlp_adam_step", "ks_adam_step", "ks_mlp_get_params", "ks_gaussian_log_prob"):
+        getattr(lib, name).restype = c_int32
     for name in ("ks_terms_create", "ks_terms_destroy", "ks_observe", "ks_terminate_reset", "ks_sample_action",
                  "ks_mlp_create", "ks_mlp_destroy", "ks_mlp_forward"):
         getattr(lib, name).restype = c_int32

@@ -475,7 +475,143 @@ struct DevMlp {
   int lda;                      // LDS row stride of the activation tile, in bf16 elements
   void* Wp[KS_MAX_LAYERS];      // [tile][k step][lane] x 16 bytes
   float* bp[KS_MAX_LAYERS];     // bias padded to 32 * fn
+  // training state (ks_mlp_train_init): fp32 master weights in the padded (npad, kpad) layout, their gradients
+  // and Adam moments, and the transposed working copy that the input-gradient GEMM reads
+  int train;
+  float *mW[KS_MAX_LAYERS], *mb[KS_MAX_LAYERS];
+  float *gW[KS_MAX_LAYERS], *gb[KS_MAX_LAYERS];
+  float *m1W[KS_MAX_LAYERS], *m2W[KS_MAX_LAYERS], *m1b[KS_MAX_LAYERS], *m2b[KS_MAX_LAYERS];
+  void* Wt[KS_MAX_LAYERS];      // (kpad, npad) working-precision transpose, layers >= 1
+  float* zero_bias;             // zeros, as wide as the widest GEMM output
 };
+
+
+// ---------------------------------------------------------------- training: the small kernels around the GEMMs
+// The three matrix products of a layer's backward pass reuse mlp_layer_kernel (Y = X W^T):
+//   input gradient   dY_prev = dZ W        : X = dZ (M, npad),      "W" = W^T (kpad, npad)
+//   weight gradient  dW = dZ^T Y_prev      : X = dZ^T (npad, Mp),   "W" = Y_prev^T (kpad, Mp), fp32 output
+// so what is left are transposes, the activation derivative, column sums and the optimiser.
+template <typename T>
+__device__ __forceinline__ float to_f32(T v) { return (float)v; }
+template <typename T>
+__device__ __forceinline__ T from_f32(float v) { return (T)v; }
+
+// fp32 (M, n) -> T (M, ld), zero in the padding columns
+template <typename T>
+__global__ __launch_bounds__(256) void cast_pad_kernel(int64_t M, int n, int ld, const float* __restrict__ src, T* __restrict__ dst) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= M * ld) return;
+  const int64_t m = idx / ld;
+  const int c = (int)(idx - m * ld);
+  dst[idx] = from_f32<T>(c < n ? src[m * n + c] : 0.f);
+}
+
+// (M, ld_src) with C meaningful columns -> (Cpad, Mp) transposed, zero outside (C, M).  S is float or T.
+template <typename S, typename T>
+__global__ __launch_bounds__(256) void transpose_kernel(int64_t M, int C, int64_t ld_src, const S* __restrict__ src, int Cpad, int64_t Mp,
+                                                        T* __restrict__ dst) {
+  __shared__ float tile[32][33];
+  const int64_t m0 = (int64_t)blockIdx.x * 32;
+  const int c0 = blockIdx.y * 32;
+  const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;  // 32 x 8
+  for (int r = ty; r < 32; r += 8) {
+    const int64_t m = m0 + r;
+    const int c = c0 + tx;
+    tile[r][tx] = (m < M && c < C) ? (float)src[m * ld_src + c] : 0.f;
+  }
+  __syncthreads();
+  for (int r = ty; r < 32; r += 8) {
+    const int c = c0 + r;
+    const int64_t m = m0 + tx;
+    if (c < Cpad && m < Mp) dst[(int64_t)c * Mp + m] = from_f32<T>(tile[tx][r]);
+  }
+}
+
+// dZ = dY * act'(Z), written over dY; act' is expressed through the stored activation output Y.
+template <typename T, int ACT>
+__global__ __launch_bounds__(256) void act_backward_kernel(int64_t n, const T* __restrict__ y, T* __restrict__ dy) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= n) return;
+  const float yv = to_f32(y[idx]);
+  float d = 1.f;
+  if (ACT == KS_ACT_ELU) d = yv > 0.f ? 1.f : yv + 1.f;  // elu'(z) = exp(z) = elu(z) + 1 for z <= 0
+  if (ACT == KS_ACT_RELU) d = yv > 0.f ? 1.f : 0.f;
+  if (ACT == KS_ACT_TANH) d = 1.f - yv * yv;
+  dy[idx] = from_f32<T>(to_f32(dy[idx]) * d);
+}
+
+// column sums of a (M, ld) matrix: one workgroup per 64 columns, rows in a fixed order (deterministic)
+template <typename T>
+__global__ __launch_bounds__(256) void colsum_kernel(int64_t M, int ld, const T* __restrict__ a, float* __restrict__ out) {
+  __shared__ float part[4][64];
+  const int c = blockIdx.x * 64 + (threadIdx.x & 63), g = threadIdx.x >> 6;
+  float s = 0.f;
+  if (c < ld)
+    for (int64_t m = g; m < M; m += 4) s += to_f32(a[m * ld + c]);
+  part[g][threadIdx.x & 63] = s;
+  __syncthreads();
+  if (g == 0 && c < ld) out[c] = (part[0][threadIdx.x] + part[1][threadIdx.x]) + (part[2][threadIdx.x] + part[3][threadIdx.x]);
+}
+
+// sum of squares of a buffer, NaNs counted as zero (the optimiser zeroes them first), added to *acc in double
+__global__ __launch_bounds__(256) void sqnorm_kernel(int64_t n, const float* __restrict__ g, double* __restrict__ acc) {
+  __shared__ double red[256];
+  double s = 0.0;
+  for (int64_t i = threadIdx.x; i < n; i += 256) {
+    const float v = g[i];
+    if (v == v) s += (double)v * (double)v;
+  }
+  red[threadIdx.x] = s;
+  __syncthreads();
+  for (int w = 128; w > 0; w >>= 1) {
+    if ((int)threadIdx.x < w) red[threadIdx.x] += red[threadIdx.x + w];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) *acc += red[0];  // launches are ordered on one stream: no atomics needed
+}
+
+// optax.chain(zero_nans, clip_by_global_norm, add_decayed_weights, scale_by_adam, scale(lr), scale(-1)) on one tensor
+__global__ __launch_bounds__(256) void adam_kernel(int64_t n, float* __restrict__ p, const float* __restrict__ g,
+                                                  float* __restrict__ m1, float* __restrict__ m2, KsAdamParams a,
+                                                  const double* __restrict__ sqnorm) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n) return;
+  float gv = g[i];
+  if (!(gv == gv)) gv = 0.f;                                       // zero_nans
+  if (a.max_grad_norm > 0.f && sqnorm) {                           // clip_by_global_norm
+    const float norm = (float)sqrt(*sqnorm);
+    if (norm > a.max_grad_norm) gv = gv / norm * a.max_grad_norm;
+  }
+  gv += a.weight_decay * p[i];                                     // add_decayed_weights
+  const float nm1 = a.b1 * m1[i] + (1.f - a.b1) * gv;              // scale_by_adam
+  const float nm2 = a.b2 * m2[i] + (1.f - a.b2) * gv * gv;
+  m1[i] = nm1;
+  m2[i] = nm2;
+  const float mhat = nm1 / (1.f - powf(a.b1, (float)a.step));
+  const float vhat = nm2 / (1.f - powf(a.b2, (float)a.step));
+  p[i] -= a.lr * mhat / (sqrtf(vhat) + a.eps);
+}
+
+// fp32 master (npad, kpad) -> working copies: W (npad, kpad), W^T (kpad, npad) and, for the whole-network kernel,
+// the fragment-ordered copy [tile][k step][lane][8]
+template <typename T>
+__global__ __launch_bounds__(256) void refresh_kernel(int npad, int kpad, const float* __restrict__ mW, T* __restrict__ W,
+                                                      T* __restrict__ Wt, __bf16* __restrict__ Wp, int fk, int fn) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx < (int64_t)npad * kpad) {
+    const int o = (int)(idx / kpad), i = (int)(idx - (int64_t)o * kpad);
+    const float v = mW[idx];
+    W[idx] = from_f32<T>(v);
+    if (Wt) Wt[(int64_t)i * npad + o] = from_f32<T>(v);
+  }
+  if (Wp && idx < (int64_t)fn * fk * 64 * 8) {
+    const int e = (int)(idx & 7), lane = (int)((idx >> 3) & 63);
+    const int64_t js = idx >> 9;
+    const int st = (int)(js % fk), j = (int)(js / fk);
+    const int o = j * 32 + (lane & 31), i = st * 16 + (lane >> 5) * 8 + e;
+    Wp[idx] = (__bf16)((o < npad && i < kpad) ? mW[(int64_t)o * kpad + i] : 0.f);
+  }
+}
 
 static inline int round_up(int x, int m) { return (x + m - 1) / m * m; }
 
@@ -533,6 +669,7 @@ using namespace ks;
 
 struct KsMlp {
   DevMlp m;
+  std::vector<float> host_w[KS_MAX_LAYERS], host_b[KS_MAX_LAYERS];  // the caller's fp32 parameters, for ks_mlp_train_init
 };
 
 extern "C" int ks_mlp_create(const KsMlpDesc* d, KsMlp** out) {
@@ -551,6 +688,8 @@ extern "C" int ks_mlp_create(const KsMlpDesc* d, KsMlp** out) {
   for (int l = 0; l <= d->n_layers; ++l) m.dims[l] = d->dims[l];
   for (int l = 0; l < d->n_layers; ++l) {
     if (!d->weights[l] || !d->biases[l]) { ks_mlp_destroy(h); return fail(KS_EINVAL, "ks_mlp_create: layer %d has no weights", l); }
+    h->host_w[l].assign(d->weights[l], d->weights[l] + (size_t)d->dims[l + 1] * d->dims[l]);
+    h->host_b[l].assign(d->biases[l], d->biases[l] + d->dims[l + 1]);
     m.npad[l] = round_up(d->dims[l + 1], kBN);
     // hidden activations are stored with the producer's padded width, so the consumer's K equals it
     m.kpad[l] = l == 0 ? round_up(d->dims[0], bk) : m.npad[l - 1];
@@ -615,7 +754,12 @@ extern "C" int ks_mlp_destroy(KsMlp* h) {
     if (h->m.b[l]) (void)hipFree(h->m.b[l]);
     if (h->m.Wp[l]) (void)hipFree(h->m.Wp[l]);
     if (h->m.bp[l]) (void)hipFree(h->m.bp[l]);
+    float* t[] = {h->m.mW[l], h->m.mb[l], h->m.gW[l], h->m.gb[l], h->m.m1W[l], h->m.m2W[l], h->m.m1b[l], h->m.m2b[l]};
+    for (float* q : t)
+      if (q) (void)hipFree(q);
+    if (h->m.Wt[l]) (void)hipFree(h->m.Wt[l]);
   }
+  if (h->m.zero_bias) (void)hipFree(h->m.zero_bias);
   delete h;
   return KS_OK;
 }
@@ -712,4 +856,255 @@ extern "C" int ks_mlp_forward(const KsMlp* h, ks_stream_t stream, int64_t M, con
     ldin = ldo;
   }
   return check_launch("ks_mlp_forward");
+}
+
+// ---------------------------------------------------------------------------------------------
+// training entry points
+// ---------------------------------------------------------------------------------------------
+static int widest_pad(const DevMlp& m) {
+  int w = 0;
+  for (int l = 0; l < m.n_layers; ++l) {
+    w = m.npad[l] > w ? m.npad[l] : w;
+    w = round_up(m.kpad[l], kBN) > w ? round_up(m.kpad[l], kBN) : w;
+  }
+  return w;
+}
+
+template <typename T>
+static void refresh_layers(DevMlp& m, hipStream_t s);
+
+extern "C" int ks_mlp_train_init(KsMlp* h) {
+  if (!h) return fail(KS_EINVAL, "ks_mlp_train_init: null handle");
+  DevMlp& m = h->m;
+  if (m.train) return KS_OK;
+  const size_t esz = m.dtype == KS_MLP_BF16 ? 2 : 4;
+  for (int l = 0; l < m.n_layers; ++l) {
+    const size_t n = (size_t)m.npad[l] * m.kpad[l], nb = m.npad[l];
+    std::vector<float> w(n, 0.f), b(nb, 0.f);
+    for (int o = 0; o < m.dims[l + 1]; ++o) {
+      for (int i = 0; i < m.dims[l]; ++i) w[(size_t)o * m.kpad[l] + i] = h->host_w[l][(size_t)o * m.dims[l] + i];
+      b[o] = h->host_b[l][o];
+    }
+    float** wbufs[] = {&m.mW[l], &m.gW[l], &m.m1W[l], &m.m2W[l]};
+    float** bbufs[] = {&m.mb[l], &m.gb[l], &m.m1b[l], &m.m2b[l]};
+    for (float** q : wbufs)
+      if (hipMalloc((void**)q, n * 4) != hipSuccess || hipMemset(*q, 0, n * 4) != hipSuccess) return fail(KS_ELAUNCH, "ks_mlp_train_init: allocation failed");
+    for (float** q : bbufs)
+      if (hipMalloc((void**)q, nb * 4) != hipSuccess || hipMemset(*q, 0, nb * 4) != hipSuccess) return fail(KS_ELAUNCH, "ks_mlp_train_init: allocation failed");
+    if (hipMemcpy(m.mW[l], w.data(), n * 4, hipMemcpyHostToDevice) != hipSuccess ||
+        hipMemcpy(m.mb[l], b.data(), nb * 4, hipMemcpyHostToDevice) != hipSuccess)
+      return fail(KS_ELAUNCH, "ks_mlp_train_init: upload failed");
+    if (l > 0 && hipMalloc(&m.Wt[l], n * esz) != hipSuccess) return fail(KS_ELAUNCH, "ks_mlp_train_init: allocation failed");
+  }
+  const int wz = widest_pad(m);
+  if (hipMalloc((void**)&m.zero_bias, (size_t)wz * 4) != hipSuccess || hipMemset(m.zero_bias, 0, (size_t)wz * 4) != hipSuccess)
+    return fail(KS_ELAUNCH, "ks_mlp_train_init: allocation failed");
+  m.train = 1;
+  // working copies (among them the transposes, which did not exist yet) from the master weights
+  if (m.dtype == KS_MLP_BF16) refresh_layers<__bf16>(m, (hipStream_t)0);
+  else refresh_layers<float>(m, (hipStream_t)0);
+  if (hipStreamSynchronize((hipStream_t)0) != hipSuccess) return fail(KS_ELAUNCH, "ks_mlp_train_init: refresh failed");
+  return KS_OK;
+}
+
+template <typename T>
+static void refresh_layers(DevMlp& m, hipStream_t s) {
+  for (int l = 0; l < m.n_layers; ++l) {
+    const int64_t n = (int64_t)m.npad[l] * m.kpad[l];
+    const int64_t np = m.fused ? (int64_t)m.fn[l] * m.fk[l] * 512 : 0;
+    const int64_t tot = n > np ? n : np;
+    hipLaunchKernelGGL(refresh_kernel<T>, dim3((unsigned)((tot + 255) / 256)), dim3(256), 0, s, m.npad[l], m.kpad[l], m.mW[l],
+                       (T*)m.W[l], (T*)m.Wt[l], m.fused ? (__bf16*)m.Wp[l] : (__bf16*)nullptr, m.fk[l], m.fn[l]);
+    (void)hipMemcpyAsync(m.b[l], m.mb[l], (size_t)m.npad[l] * 4, hipMemcpyDeviceToDevice, s);
+    if (m.fused) (void)hipMemcpyAsync(m.bp[l], m.mb[l], (size_t)m.fn[l] * 32 * 4, hipMemcpyDeviceToDevice, s);
+  }
+}
+
+// workspace: hidden activations of every layer, two (M, widest) gradient buffers, two transposes (widest, Mp)
+struct TrainWs {
+  char* act[KS_MAX_LAYERS];
+  char *d0, *d1, *t0, *t1;
+  int64_t Mp;
+};
+static int64_t carve_train(const DevMlp& m, int64_t M, char* base, TrainWs* ws) {
+  const int64_t esz = m.dtype == KS_MLP_BF16 ? 2 : 4;
+  const int64_t Mp = (M + 63) / 64 * 64;
+  const int wz = widest_pad(m);
+  int64_t off = 0;
+  auto take = [&](int64_t bytes) {
+    char* p = base ? base + off : nullptr;
+    off += (bytes + 255) / 256 * 256;
+    return p;
+  };
+  TrainWs w;
+  std::memset(&w, 0, sizeof(w));
+  for (int l = 0; l + 1 < m.n_layers; ++l) w.act[l] = take(M * m.npad[l] * esz);
+  w.d0 = take(M * wz * esz);
+  w.d1 = take(M * wz * esz);
+  w.t0 = take((int64_t)wz * Mp * esz);
+  w.t1 = take((int64_t)wz * Mp * esz);
+  w.Mp = Mp;
+  if (ws) *ws = w;
+  return off;
+}
+
+extern "C" int64_t ks_mlp_train_workspace_bytes(const KsMlp* h, int64_t M) {
+  if (!h || M < 0) return 0;
+  return carve_train(h->m, M, nullptr, nullptr) + 256;
+}
+
+template <typename T>
+static int train_forward(DevMlp& m, hipStream_t s, int64_t M, const float* x, float* y, const TrainWs& ws) {
+  const void* in = x;
+  int64_t ldin = m.dims[0];
+  for (int l = 0; l < m.n_layers; ++l) {
+    const bool first = l == 0, last = l == m.n_layers - 1;
+    void* outp = last ? (void*)y : (void*)ws.act[l];
+    const int64_t ldo = last ? m.dims[l + 1] : m.npad[l];
+    int rc;
+    if (first && last) rc = launch_layer<T, true, true>(m.activation, s, M, m.npad[l], m.kpad[l], m.dims[l], m.dims[l + 1], in, ldin, m.W[l], m.b[l], outp, ldo);
+    else if (first) rc = launch_layer<T, true, false>(m.activation, s, M, m.npad[l], m.kpad[l], m.dims[l], m.dims[l + 1], in, ldin, m.W[l], m.b[l], outp, ldo);
+    else if (last) rc = launch_layer<T, false, true>(m.activation, s, M, m.npad[l], m.kpad[l], m.dims[l], m.dims[l + 1], in, ldin, m.W[l], m.b[l], outp, ldo);
+    else rc = launch_layer<T, false, false>(m.activation, s, M, m.npad[l], m.kpad[l], m.dims[l], m.dims[l + 1], in, ldin, m.W[l], m.b[l], outp, ldo);
+    if (rc != KS_OK) return rc;
+    in = outp;
+    ldin = ldo;
+  }
+  return KS_OK;
+}
+
+extern "C" int ks_mlp_train_forward(KsMlp* h, ks_stream_t stream, int64_t M, const float* x, float* y, void* workspace) {
+  if (!h || !h->m.train) return fail(KS_EINVAL, "ks_mlp_train_forward: call ks_mlp_train_init first");
+  if (M <= 0 || !x || !y || !workspace) return fail(KS_EINVAL, "ks_mlp_train_forward: bad argument");
+  if ((M + kBM - 1) / kBM > 0x7fffffff) return fail(KS_ELIMIT, "ks_mlp_train_forward: too many rows");
+  TrainWs ws;
+  carve_train(h->m, M, (char*)workspace, &ws);
+  const int rc = h->m.dtype == KS_MLP_BF16 ? train_forward<__bf16>(h->m, (hipStream_t)stream, M, x, y, ws)
+                                           : train_forward<float>(h->m, (hipStream_t)stream, M, x, y, ws);
+  return rc != KS_OK ? rc : check_launch("ks_mlp_train_forward");
+}
+
+template <typename T>
+static int train_backward(DevMlp& m, hipStream_t s, int64_t M, const float* x, const float* dy, const TrainWs& ws) {
+  const int L = m.n_layers;
+  const int64_t Mp = ws.Mp;
+  T* dz = (T*)ws.d0;
+  T* dnext = (T*)ws.d1;
+  {  // the output gradient in working precision, padded to the last layer's width
+    const int64_t n = M * m.npad[L - 1];
+    hipLaunchKernelGGL(cast_pad_kernel<T>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, M, m.dims[L], m.npad[L - 1], dy, dz);
+  }
+  for (int l = L - 1; l >= 0; --l) {
+    const int np = m.npad[l], kp = m.kpad[l], kp128 = round_up(kp, kBN);
+    // bias gradient
+    hipLaunchKernelGGL(colsum_kernel<T>, dim3((unsigned)((np + 63) / 64)), dim3(256), 0, s, M, np, dz, m.gb[l]);
+    // weight gradient: dZ^T (np, Mp) times Y_prev^T (kp128, Mp)^T
+    hipLaunchKernelGGL((transpose_kernel<T, T>), dim3((unsigned)((Mp + 31) / 32), (unsigned)((np + 31) / 32)), dim3(256), 0, s, M, np,
+                       (int64_t)np, dz, np, Mp, (T*)ws.t0);
+    if (l == 0)
+      hipLaunchKernelGGL((transpose_kernel<float, T>), dim3((unsigned)((Mp + 31) / 32), (unsigned)((kp128 + 31) / 32)), dim3(256), 0, s, M,
+                         m.dims[0], (int64_t)m.dims[0], x, kp128, Mp, (T*)ws.t1);
+    else
+      hipLaunchKernelGGL((transpose_kernel<T, T>), dim3((unsigned)((Mp + 31) / 32), (unsigned)((kp128 + 31) / 32)), dim3(256), 0, s, M,
+                         m.npad[l - 1], (int64_t)m.npad[l - 1], (const T*)ws.act[l - 1], kp128, Mp, (T*)ws.t1);
+    int rc = launch_layer<T, false, true>(KS_ACT_NONE, s, np, kp128, (int)Mp, (int)Mp, kp, ws.t0, Mp, ws.t1, m.zero_bias, m.gW[l], kp);
+    if (rc != KS_OK) return rc;
+    if (l == 0) break;
+    // input gradient, then through the activation of the layer below
+    rc = launch_layer<T, false, false>(KS_ACT_NONE, s, M, kp, np, np, kp, dz, np, m.Wt[l], m.zero_bias, dnext, kp);
+    if (rc != KS_OK) return rc;
+    const int64_t n = M * kp;
+#define KS_ACTB(A) hipLaunchKernelGGL((act_backward_kernel<T, A>), dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, n, (const T*)ws.act[l - 1], dnext)
+    switch (m.activation) {
+      case KS_ACT_ELU: KS_ACTB(KS_ACT_ELU); break;
+      case KS_ACT_RELU: KS_ACTB(KS_ACT_RELU); break;
+      case KS_ACT_TANH: KS_ACTB(KS_ACT_TANH); break;
+      default: break;
+    }
+#undef KS_ACTB
+    T* tmp = dz; dz = dnext; dnext = tmp;
+  }
+  return KS_OK;
+}
+
+extern "C" int ks_mlp_train_backward(KsMlp* h, ks_stream_t stream, int64_t M, const float* x, const float* dy, void* workspace) {
+  if (!h || !h->m.train) return fail(KS_EINVAL, "ks_mlp_train_backward: call ks_mlp_train_init first");
+  if (M <= 0 || !x || !dy || !workspace) return fail(KS_EINVAL, "ks_mlp_train_backward: bad argument");
+  if (M > (1 << 30)) return fail(KS_ELIMIT, "ks_mlp_train_backward: too many rows");
+  TrainWs ws;
+  carve_train(h->m, M, (char*)workspace, &ws);
+  const int rc = h->m.dtype == KS_MLP_BF16 ? train_backward<__bf16>(h->m, (hipStream_t)stream, M, x, dy, ws)
+                                           : train_backward<float>(h->m, (hipStream_t)stream, M, x, dy, ws);
+  return rc != KS_OK ? rc : check_launch("ks_mlp_train_backward");
+}
+
+extern "C" int ks_grad_sqnorm(ks_stream_t stream, int64_t n, const float* g, double* acc) {
+  if (n < 0 || !acc || (n > 0 && !g)) return fail(KS_EINVAL, "ks_grad_sqnorm: bad argument");
+  if (n == 0) return KS_OK;
+  hipLaunchKernelGGL(sqnorm_kernel, dim3(1), dim3(256), 0, (hipStream_t)stream, n, g, acc);
+  return check_launch("ks_grad_sqnorm");
+}
+
+extern "C" int ks_mlp_grad_sqnorm(const KsMlp* h, ks_stream_t stream, double* acc) {
+  if (!h || !h->m.train || !acc) return fail(KS_EINVAL, "ks_mlp_grad_sqnorm: bad argument");
+  for (int l = 0; l < h->m.n_layers; ++l) {
+    hipLaunchKernelGGL(sqnorm_kernel, dim3(1), dim3(256), 0, (hipStream_t)stream, (int64_t)h->m.npad[l] * h->m.kpad[l], h->m.gW[l], acc);
+    hipLaunchKernelGGL(sqnorm_kernel, dim3(1), dim3(256), 0, (hipStream_t)stream, (int64_t)h->m.npad[l], h->m.gb[l], acc);
+  }
+  return check_launch("ks_mlp_grad_sqnorm");
+}
+
+static int check_adam(const KsAdamParams* p, const char* who) {
+  if (!p) return fail(KS_EINVAL, "%s: null parameters", who);
+  if (p->step < 1) return fail(KS_EINVAL, "%s: step starts at 1", who);
+  if (!(p->b1 >= 0.f && p->b1 < 1.f && p->b2 >= 0.f && p->b2 < 1.f)) return fail(KS_EINVAL, "%s: betas must be in [0, 1)", who);
+  return KS_OK;
+}
+
+extern "C" int ks_adam_step(ks_stream_t stream, int64_t n, float* param, const float* grad, float* m1, float* m2,
+                            const KsAdamParams* p, const double* sqnorm) {
+  const int rc = check_adam(p, "ks_adam_step");
+  if (rc != KS_OK) return rc;
+  if (n < 0 || (n > 0 && (!param || !grad || !m1 || !m2))) return fail(KS_EINVAL, "ks_adam_step: bad argument");
+  if (n == 0) return KS_OK;
+  hipLaunchKernelGGL(adam_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream, n, param, grad, m1, m2, *p, sqnorm);
+  return check_launch("ks_adam_step");
+}
+
+extern "C" int ks_mlp_adam_step(KsMlp* h, ks_stream_t stream, const KsAdamParams* p, const double* sqnorm) {
+  if (!h || !h->m.train) return fail(KS_EINVAL, "ks_mlp_adam_step: call ks_mlp_train_init first");
+  const int rc = check_adam(p, "ks_mlp_adam_step");
+  if (rc != KS_OK) return rc;
+  DevMlp& m = h->m;
+  hipStream_t s = (hipStream_t)stream;
+  for (int l = 0; l < m.n_layers; ++l) {
+    const int64_t n = (int64_t)m.npad[l] * m.kpad[l], nb = m.npad[l];
+    hipLaunchKernelGGL(adam_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, n, m.mW[l], m.gW[l], m.m1W[l], m.m2W[l], *p, sqnorm);
+    hipLaunchKernelGGL(adam_kernel, dim3((unsigned)((nb + 255) / 256)), dim3(256), 0, s, nb, m.mb[l], m.gb[l], m.m1b[l], m.m2b[l], *p, sqnorm);
+  }
+  if (m.dtype == KS_MLP_BF16) refresh_layers<__bf16>(m, s);
+  else refresh_layers<float>(m, s);
+  return check_launch("ks_mlp_adam_step");
+}
+
+// strided copy of the meaningful (out, in) block of a padded (npad, kpad) matrix
+__global__ __launch_bounds__(256) void unpad_kernel(int rows, int cols, int ld, const float* __restrict__ src, float* __restrict__ dst) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= (int64_t)rows * cols) return;
+  const int r = (int)(idx / cols), c = (int)(idx - (int64_t)r * cols);
+  dst[idx] = src[(int64_t)r * ld + c];
+}
+
+extern "C" int ks_mlp_get_params(const KsMlp* h, ks_stream_t stream, int32_t l, float* weight, float* bias, int32_t gradients) {
+  if (!h || !h->m.train) return fail(KS_EINVAL, "ks_mlp_get_params: call ks_mlp_train_init first");
+  const DevMlp& m = h->m;
+  if (l < 0 || l >= m.n_layers) return fail(KS_EINVAL, "ks_mlp_get_params: layer %d out of range", l);
+  const int out = m.dims[l + 1], in = m.dims[l];
+  if (weight)
+    hipLaunchKernelGGL(unpad_kernel, dim3((unsigned)(((int64_t)out * in + 255) / 256)), dim3(256), 0, (hipStream_t)stream, out, in,
+                       m.kpad[l], gradients ? m.gW[l] : m.mW[l], weight);
+  if (bias)
+    hipLaunchKernelGGL(unpad_kernel, dim3((unsigned)((out + 255) / 256)), dim3(256), 0, (hipStream_t)stream, 1, out, out,
+                       gradients ? m.gb[l] : m.mb[l], bias);
+  return check_launch("ks_mlp_get_params");
 }

@@ -325,6 +325,7 @@ extern "C" int64_t ks_abi_sizeof(int32_t which) {
     case 9: return sizeof(KsTermDesc);
     case 10: return sizeof(KsRewardDesc);
     case 11: return sizeof(KsRng);
+    case 12: return sizeof(KsAdamParams);
     default: return -1;
   }
 }
@@ -420,4 +421,131 @@ extern "C" int ks_copy_f32(ks_stream_t stream, int64_t n, const float* src, floa
   if (!src || !dst) return fail(KS_EINVAL, "ks_copy_f32: null pointer");
   hipLaunchKernelGGL(copy_f32_kernel, dim3(grid_for(n, 256, 65536)), dim3(256), 0, (hipStream_t)stream, n, src, dst);
   return check_launch("ks_copy_f32");
+}
+
+// ---------------------------------------------------------------------------------------------
+// Gaussian policy head and the gradient of the PPO objective
+// ---------------------------------------------------------------------------------------------
+namespace ks {
+
+constexpr float kHalfLog2Pi = 0.91893853320467274178f;
+
+__global__ __launch_bounds__(256) void gaussian_log_prob_kernel(int64_t n, int nu, const float* __restrict__ mean,
+                                                               const float* __restrict__ log_std,
+                                                               const float* __restrict__ action, float* __restrict__ lp,
+                                                               float* __restrict__ ent) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= n) return;
+  const int a = (int)(idx % nu);
+  const float ls = log_std[a];
+  const float z = (action[idx] - mean[idx]) * __expf(-ls);
+  lp[idx] = -0.5f * z * z - ls - kHalfLog2Pi;
+  if (ent) ent[idx] = 0.5f + kHalfLog2Pi + ls;
+}
+
+// One thread per row m; every workgroup also accumulates the log-std gradient of its rows, reduced in a fixed
+// order (block partials, then ppo_grad_finish_kernel), so the result does not depend on scheduling.
+__global__ __launch_bounds__(256) void ppo_loss_grad_kernel(int64_t M, int nu, KsPpoLossParams p, const float* __restrict__ mean,
+                                                           const float* __restrict__ log_std, const float* __restrict__ action,
+                                                           const float* __restrict__ on_lp, const float* __restrict__ adv,
+                                                           const float* __restrict__ tgt, const float* __restrict__ on_v,
+                                                           const float* __restrict__ v, float* __restrict__ d_mean,
+                                                           float* __restrict__ d_value, float* __restrict__ partial) {
+  __shared__ float red[256];
+  float dls[KS_MAX_ACTIONS];
+#pragma unroll
+  for (int a = 0; a < KS_MAX_ACTIONS; ++a) dls[a] = 0.f;
+  const float inv_m = 1.0f / (float)M;
+  for (int64_t m = (int64_t)blockIdx.x * 256 + threadIdx.x; m < M; m += (int64_t)gridDim.x * 256) {
+    // new log-probabilities and the log ratio
+    float logr = 0.f;
+    for (int a = 0; a < nu; ++a) {
+      const float ls = log_std[a];
+      const float z = (action[m * nu + a] - mean[m * nu + a]) * __expf(-ls);
+      logr += (-0.5f * z * z - ls - kHalfLog2Pi) - on_lp[m * nu + a];
+    }
+    const bool log_inside = logr > -p.log_clip_value && logr < p.log_clip_value;
+    const float ratio = __expf(fminf(fmaxf(logr, -p.log_clip_value), p.log_clip_value));
+    const float A = adv[m];
+    const float lo = 1.f - p.clip_param, hi = 1.f + p.clip_param;
+    const float s1 = ratio * A, s2 = fminf(fmaxf(ratio, lo), hi) * A;
+    // d(-min(s1, s2)) / d(log ratio); inside the clip range both surrogates coincide
+    const bool ratio_inside = ratio > lo && ratio < hi;
+    float g_logr = 0.f;
+    if (log_inside) {
+      if (s1 < s2 || ratio_inside) g_logr = -A * ratio;   // the unclipped surrogate is active (or both are the same)
+    }
+    // kl term: (on_lp - lp) * kl_coef * kl_scale per action
+    const float g_lp = (g_logr - p.kl_coef * p.kl_scale) * inv_m;
+    const float g_ent = -p.entropy_coef * inv_m;
+    for (int a = 0; a < nu; ++a) {
+      const float ls = log_std[a];
+      const float is = __expf(-ls);
+      const float z = (action[m * nu + a] - mean[m * nu + a]) * is;
+      d_mean[m * nu + a] = g_lp * z * is;
+      dls[a] += g_lp * (z * z - 1.f) + g_ent;
+    }
+    // value term
+    const float vv = v[m], vo = on_v[m], t = tgt[m];
+    float gv;
+    if (p.use_clipped_value_loss) {
+      const float dvv = vv - vo;
+      const float vc = vo + fminf(fmaxf(dvv, -p.clip_param), p.clip_param);
+      const float e = vv - t, ec = vc - t;
+      if (e * e >= ec * ec) gv = e;
+      else gv = (dvv > -p.clip_param && dvv < p.clip_param) ? ec : 0.f;
+    } else {
+      gv = vv - t;
+    }
+    d_value[m] = p.value_loss_coef * gv * inv_m;
+  }
+  for (int a = 0; a < nu; ++a) {
+    red[threadIdx.x] = dls[a];
+    __syncthreads();
+    for (int w = 128; w > 0; w >>= 1) {
+      if ((int)threadIdx.x < w) red[threadIdx.x] += red[threadIdx.x + w];
+      __syncthreads();
+    }
+    if (threadIdx.x == 0) partial[(int64_t)blockIdx.x * nu + a] = red[0];
+    __syncthreads();
+  }
+}
+
+__global__ void ppo_grad_finish_kernel(int nblocks, int nu, const float* __restrict__ partial, float* __restrict__ d_log_std) {
+  const int a = threadIdx.x;
+  if (a >= nu) return;
+  float s = 0.f;
+  for (int b = 0; b < nblocks; ++b) s += partial[(int64_t)b * nu + a];
+  d_log_std[a] = s;
+}
+
+}  // namespace ks
+
+extern "C" int ks_gaussian_log_prob(ks_stream_t stream, int64_t M, int32_t nu, const float* mean, const float* log_std,
+                                    const float* action, float* log_prob, float* entropy) {
+  if (M < 0 || nu < 1) return ks::fail(KS_EINVAL, "ks_gaussian_log_prob: bad shape");
+  if (M == 0) return KS_OK;
+  if (!mean || !log_std || !action || !log_prob) return ks::fail(KS_EINVAL, "ks_gaussian_log_prob: null pointer");
+  const int64_t n = M * nu;
+  hipLaunchKernelGGL(ks::gaussian_log_prob_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream, n, nu, mean,
+                     log_std, action, log_prob, entropy);
+  return ks::check_launch("ks_gaussian_log_prob");
+}
+
+extern "C" int ks_ppo_loss_grad(ks_stream_t stream, int64_t M, int32_t nu, const KsPpoLossParams* params, const float* mean,
+                                const float* log_std, const float* action, const float* on_log_probs,
+                                const float* advantages, const float* value_targets, const float* on_values,
+                                const float* values, float* d_mean, float* d_value, float* d_log_std, void* workspace) {
+  if (!params) return ks::fail(KS_EINVAL, "ks_ppo_loss_grad: null parameters");
+  if (M < 1 || nu < 1 || nu > KS_MAX_ACTIONS) return ks::fail(KS_EINVAL, "ks_ppo_loss_grad: bad shape (1..%d actions)", KS_MAX_ACTIONS);
+  if (!mean || !log_std || !action || !on_log_probs || !advantages || !value_targets || !on_values || !values || !d_mean ||
+      !d_value || !d_log_std || !workspace)
+    return ks::fail(KS_EINVAL, "ks_ppo_loss_grad: null pointer");
+  const int64_t want = (M + 255) / 256;
+  const int blocks = (int)(want < KS_PPO_GRAD_BLOCKS ? want : KS_PPO_GRAD_BLOCKS);
+  hipLaunchKernelGGL(ks::ppo_loss_grad_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream, M, nu, *params, mean, log_std, action,
+                     on_log_probs, advantages, value_targets, on_values, values, d_mean, d_value, (float*)workspace);
+  hipLaunchKernelGGL(ks::ppo_grad_finish_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, blocks, nu, (const float*)workspace,
+                     d_log_std);
+  return ks::check_launch("ks_ppo_loss_grad");
 }

@@ -81,6 +81,58 @@ class MLP:
                                             _lib.ptr(ws)))
         return out
 
+    # ------------------------------------------------------------------ training (ksim/task/ppo.py:495-565)
+    def train_init(self) -> None:
+        """fp32 master weights, gradients and Adam moments beside the working copies."""
+        _lib.check(self._lib.ks_mlp_train_init(self._handle))
+        self._training = True
+
+    def _train_ws(self, M: int, device) -> torch.Tensor:
+        need = int(self._lib.ks_mlp_train_workspace_bytes(self._handle, M))
+        ws = getattr(self, "_tws", None)
+        if ws is None or ws.numel() < need or ws.device != torch.device(device):
+            ws = torch.empty(need, dtype=torch.uint8, device=device)
+            self._tws = ws
+        return ws
+
+    def train_forward(self, x: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+        """Forward pass that keeps the hidden activations for `backward` (same rows, called next)."""
+        _lib.require_cuda(x, dtype=torch.float32)
+        if x.dim() != 2 or x.shape[1] != self.in_dim:
+            raise _lib.KsError(f"expected input (M, {self.in_dim}), got {tuple(x.shape)}")
+        M = x.shape[0]
+        if out is None:
+            out = torch.empty((M, self.out_dim), dtype=torch.float32, device=x.device)
+        _lib.check(self._lib.ks_mlp_train_forward(self._handle, _lib.current_stream(), M, _lib.ptr(x), _lib.ptr(out),
+                                                  _lib.ptr(self._train_ws(M, x.device))))
+        return out
+
+    def backward(self, x: torch.Tensor, dy: torch.Tensor) -> None:
+        """Gradients of sum(dy * net(x)) into the handle; `x` is the input of the preceding `train_forward`."""
+        _lib.require_cuda(x, dy, dtype=torch.float32)
+        if tuple(dy.shape) != (x.shape[0], self.out_dim):
+            raise _lib.KsError("dy must have the shape of the network output")
+        _lib.check(self._lib.ks_mlp_train_backward(self._handle, _lib.current_stream(), x.shape[0], _lib.ptr(x),
+                                                   _lib.ptr(dy), _lib.ptr(self._train_ws(x.shape[0], x.device))))
+
+    def grad_sqnorm(self, acc: torch.Tensor) -> None:
+        _lib.require_cuda(acc, dtype=torch.float64)
+        _lib.check(self._lib.ks_mlp_grad_sqnorm(self._handle, _lib.current_stream(), _lib.ptr(acc)))
+
+    def adam_step(self, params: "T.KsAdamParams", sqnorm: torch.Tensor | None) -> None:
+        _lib.check(self._lib.ks_mlp_adam_step(self._handle, _lib.current_stream(), ctypes.byref(params), _lib.ptr(sqnorm)))
+
+    def parameters(self, gradients: bool = False) -> list[tuple[torch.Tensor, torch.Tensor]]:
+        """[(weight (out, in), bias (out))] copies of the fp32 master parameters, or of their gradients."""
+        out = []
+        for l, (i, o) in enumerate(zip(self.dims[:-1], self.dims[1:])):
+            w = torch.empty((o, i), dtype=torch.float32, device="cuda")
+            b = torch.empty((o,), dtype=torch.float32, device="cuda")
+            _lib.check(self._lib.ks_mlp_get_params(self._handle, _lib.current_stream(), l, _lib.ptr(w), _lib.ptr(b),
+                                                   int(gradients)))
+            out.append((w, b))
+        return out
+
     def close(self) -> None:
         if self._handle:
             self._lib.ks_mlp_destroy(self._handle)

@@ -1,0 +1,159 @@
+"""Policy update of a PPO iteration (ksim/task/ppo.py:495-565 `_single_step`, 572-694 `update_model`) for an MLP
+actor / critic with a state-independent Gaussian head.
+
+The reference differentiates `_get_ppo_loss_and_metrics` (ppo.py:412-492) with `jax.grad` and applies the task's
+optax chain; here the same gradient is written out: the loss gradient w.r.t. the policy outputs
+(`ks_ppo_loss_grad`), the networks' backward passes (`ks_mlp_train_backward`, three MFMA GEMMs per layer) and the
+optimiser chain of the examples (`ks_mlp_adam_step`).  As in the reference, GAE is recomputed from the current
+value estimates at every minibatch step and enters the loss as a constant.
+Trajectories are time-major (T, N, ...), the rollout buffers' own layout; a minibatch is a set of env columns.
+"""
+from __future__ import annotations
+
+import ctypes
+from dataclasses import dataclass, field
+
+import torch
+
+from . import _lib
+from . import _lib_terms as T
+from . import ppo as ppo_mod
+from .mlp import MLP
+
+
+@dataclass
+class PPOUpdateConfig:  # ksim/task/ppo.py:254-311 defaults, examples/walking.py:373-387 optimiser
+    gamma: float = 0.99
+    lam: float = 0.95
+    normalize_advantages: bool = True
+    monte_carlo_returns: bool = False
+    clip_param: float = 0.2
+    value_loss_coef: float = 0.5
+    entropy_coef: float = 0.008
+    kl_coef: float = 1e-3
+    log_clip_value: float = 5.0
+    use_clipped_value_loss: bool = True
+    adaptive_kl: bool = False
+    desired_kl: float = 0.01
+    num_passes: int = 1
+    batch_size: int = 256          # envs per minibatch
+    learning_rate: float = 3e-4
+    adam_b1: float = 0.9
+    adam_b2: float = 0.999
+    adam_eps: float = 1e-8
+    adam_weight_decay: float = 0.0
+    grad_clip: float = 2.0
+
+
+@dataclass
+class GaussianMlpPolicy:
+    """Actor (obs -> action means), critic (obs -> value) and one log standard deviation per action."""
+    actor: MLP
+    critic: MLP
+    log_std: torch.Tensor
+    opt_step: int = 0
+    kl_coef: float | None = None
+    _m1: torch.Tensor | None = field(default=None, repr=False)
+    _m2: torch.Tensor | None = field(default=None, repr=False)
+
+    def train_init(self) -> None:
+        self.actor.train_init()
+        self.critic.train_init()
+        self._m1, self._m2 = torch.zeros_like(self.log_std), torch.zeros_like(self.log_std)
+
+
+def get_ppo_variables(policy: GaussianMlpPolicy, actor_obs: torch.Tensor, critic_obs: torch.Tensor,
+                      action: torch.Tensor, train: bool = False):
+    """log-probabilities (rows, nu), values (rows), entropy (rows, nu) and the means, for flattened rows."""
+    lib = _lib.load()
+    mean = policy.actor.train_forward(actor_obs) if train else policy.actor(actor_obs)
+    value = (policy.critic.train_forward(critic_obs) if train else policy.critic(critic_obs)).reshape(-1)
+    lp, ent = torch.empty_like(mean), torch.empty_like(mean)
+    _lib.check(lib.ks_gaussian_log_prob(_lib.current_stream(), mean.shape[0], mean.shape[1], _lib.ptr(mean),
+                                        _lib.ptr(policy.log_std), _lib.ptr(action), _lib.ptr(lp), _lib.ptr(ent)))
+    return lp, value, ent, mean
+
+
+def _adam(cfg: PPOUpdateConfig, step: int) -> T.KsAdamParams:
+    return T.KsAdamParams(cfg.learning_rate, cfg.adam_b1, cfg.adam_b2, cfg.adam_eps, cfg.adam_weight_decay,
+                          cfg.grad_clip, step)
+
+
+def single_step(policy: GaussianMlpPolicy, cfg: PPOUpdateConfig, actor_obs, critic_obs, action, rewards, done, success,
+                on_log_probs, on_values) -> dict:
+    """One minibatch step (ppo.py:495-565): arrays are (T, b, ...) time-major slices of the rollout."""
+    lib = _lib.load()
+    Tn, b = done.shape
+    rows = Tn * b
+    nu = action.shape[-1]
+    a_obs, c_obs, act = actor_obs.reshape(rows, -1), critic_obs.reshape(rows, -1), action.reshape(rows, nu)
+    lp, value, ent, mean = get_ppo_variables(policy, a_obs, c_obs, act, train=True)
+    inputs = ppo_mod.compute_ppo_inputs(value.view(Tn, b), rewards, done, success, cfg.gamma, cfg.lam,
+                                        normalize_advantages=cfg.normalize_advantages,
+                                        monte_carlo_returns=cfg.monte_carlo_returns, time_major=True)
+    kl_coef_now = policy.kl_coef if (cfg.adaptive_kl and policy.kl_coef is not None) else cfg.kl_coef
+    p = _lib.KsPpoLossParams(cfg.clip_param, cfg.value_loss_coef, cfg.entropy_coef, cfg.kl_coef, cfg.log_clip_value,
+                             kl_coef_now / cfg.kl_coef, int(cfg.use_clipped_value_loss))
+    d_mean = torch.empty_like(mean)
+    d_value = torch.empty(rows, 1, dtype=torch.float32, device=mean.device)
+    d_log_std = torch.empty_like(policy.log_std)
+    ws = torch.empty(256 * nu, dtype=torch.float32, device=mean.device)
+    on_lp, on_v = on_log_probs.reshape(rows, nu), on_values.reshape(rows)
+    _lib.check(lib.ks_ppo_loss_grad(_lib.current_stream(), rows, nu, ctypes.byref(p), _lib.ptr(mean),
+                                    _lib.ptr(policy.log_std), _lib.ptr(act), _lib.ptr(on_lp),
+                                    _lib.ptr(inputs.advantages_bt), _lib.ptr(inputs.value_targets_bt), _lib.ptr(on_v),
+                                    _lib.ptr(value), _lib.ptr(d_mean), _lib.ptr(d_value), _lib.ptr(d_log_std), _lib.ptr(ws)))
+    policy.actor.backward(a_obs, d_mean)
+    policy.critic.backward(c_obs, d_value)
+    # optimiser chain over every parameter together: global norm first
+    sq = torch.zeros(1, dtype=torch.float64, device=mean.device)
+    policy.actor.grad_sqnorm(sq)
+    policy.critic.grad_sqnorm(sq)
+    _lib.check(lib.ks_grad_sqnorm(_lib.current_stream(), nu, _lib.ptr(d_log_std), _lib.ptr(sq)))
+    policy.opt_step += 1
+    ap = _adam(cfg, policy.opt_step)
+    policy.actor.adam_step(ap, sq)
+    policy.critic.adam_step(ap, sq)
+    _lib.check(lib.ks_adam_step(_lib.current_stream(), nu, _lib.ptr(policy.log_std), _lib.ptr(d_log_std),
+                                _lib.ptr(policy._m1), _lib.ptr(policy._m2), ctypes.byref(ap), _lib.ptr(sq)))
+    metrics = {"grad_norm": sq.sqrt(), "d_mean": d_mean, "d_value": d_value, "d_log_std": d_log_std,
+               "log_probs": lp, "values": value, "advantages": inputs.advantages_bt}
+    if cfg.adaptive_kl:  # ppo.py:548-563
+        kl_mean = float((on_lp - lp).sum(-1).mean().item()) * kl_coef_now
+        new = kl_coef_now
+        if kl_mean > cfg.desired_kl * 1.5:
+            new = kl_coef_now * 1.5
+        if kl_mean < cfg.desired_kl / 1.5:
+            new = new / 1.5
+        policy.kl_coef = min(max(new, 1e-8), 1e2)
+    return metrics
+
+
+def update_model(policy: GaussianMlpPolicy, cfg: PPOUpdateConfig, actor_obs, critic_obs, action, rewards, done, success,
+                 permutations: list[torch.Tensor] | None = None, seed: int = 0) -> list[dict]:
+    """num_passes x (N / batch_size) minibatch steps over a (T, N) rollout (ppo.py:572-694).
+
+    `permutations` (one index vector per pass) replaces the reference's `jax.random.permutation`."""
+    Tn, N = done.shape
+    if policy._m1 is None:
+        policy.train_init()
+    if cfg.adaptive_kl and policy.kl_coef is None:
+        policy.kl_coef = cfg.kl_coef
+    nu = action.shape[-1]
+    # on-policy variables of the whole rollout with the pre-update parameters (ppo.py:603-607)
+    on_lp, on_v, _, _ = get_ppo_variables(policy, actor_obs.reshape(Tn * N, -1), critic_obs.reshape(Tn * N, -1),
+                                          action.reshape(Tn * N, nu))
+    on_lp, on_v = on_lp.view(Tn, N, nu).clone(), on_v.view(Tn, N).clone()
+    bs = min(cfg.batch_size, N)
+    if N % bs:
+        raise _lib.KsError("the env count must be a multiple of the batch size (ppo.py:647 reshapes the permutation)")
+    gen = torch.Generator(device=done.device)
+    gen.manual_seed(seed)
+    out = []
+    for k in range(cfg.num_passes):
+        perm = permutations[k] if permutations is not None else torch.randperm(N, generator=gen, device=done.device)
+        for idx in perm.view(-1, bs):
+            sel = lambda t: t.index_select(1, idx).contiguous()  # noqa: E731
+            out.append(single_step(policy, cfg, sel(actor_obs), sel(critic_obs), sel(action), sel(rewards), sel(done),
+                                   sel(success), sel(on_lp), sel(on_v)))
+    return out

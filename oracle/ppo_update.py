@@ -1,0 +1,138 @@
+"""TEST INFRASTRUCTURE: float64 restatement of the PPO policy update for an MLP actor / critic with a Gaussian head.
+
+Follows ksim/task/ppo.py:412-492 (`_get_ppo_loss_and_metrics`: forward, GAE as a constant, loss, mean),
+495-565 (`_single_step`: gradient, optimiser, adaptive KL), 572-694 (`update_model`: on-policy variables once,
+passes x minibatches) and the optax chain of examples/walking.py:373-387.  The gradient is taken by torch's
+CPU autograd in float64 (the library routine the hand-written backward pass is checked against); the loss written
+here in torch is pinned against the numpy restatement in oracle/ppo.py by tests/test_oracle_ppo_update.py.
+Distribution formulas (xax.Normal, not in the reference tree): log N(a; mu, sigma) per action and the Gaussian
+entropy 0.5 + 0.5 log(2 pi) + log sigma.  Only tests may import this module.
+"""
+from __future__ import annotations
+
+import math
+
+import numpy as np
+import torch
+import torch.nn.functional as F
+
+from . import ppo as oppo
+
+_ACT = {"elu": F.elu, "relu": F.relu, "tanh": torch.tanh, "none": lambda t: t}
+
+
+def mlp(x, ws, bs, act="elu"):
+    h = x
+    for i, (w, b) in enumerate(zip(ws, bs)):
+        h = F.linear(h, w, b)
+        if i + 1 < len(ws):
+            h = _ACT[act](h)
+    return h
+
+
+def gaussian(mean, log_std, action):
+    z = (action - mean) * torch.exp(-log_std)
+    lp = -0.5 * z * z - log_std - 0.5 * math.log(2 * math.pi)
+    ent = (0.5 + 0.5 * math.log(2 * math.pi) + log_std).expand_as(mean)
+    return lp, ent
+
+
+def ppo_loss_torch(adv, tgt, on_lp, on_v, lp, v, ent, cfg, kl_scale=1.0):
+    """ppo.py:207-246 per element and 485-486 total, in torch so that autograd can differentiate it."""
+    log_ratio = (lp - on_lp).sum(-1)
+    ratio = torch.exp(torch.clamp(log_ratio, -cfg["log_clip_value"], cfg["log_clip_value"]))
+    clipped = torch.clamp(ratio, 1 - cfg["clip_param"], 1 + cfg["clip_param"])
+    policy = -torch.minimum(ratio * adv, clipped * adv)
+    if cfg["use_clipped_value_loss"]:
+        vc = on_v + torch.clamp(v - on_v, -cfg["clip_param"], cfg["clip_param"])
+        value = 0.5 * torch.maximum((v - tgt) ** 2, (vc - tgt) ** 2)
+    else:
+        value = 0.5 * (tgt - v) ** 2
+    value = value * cfg["value_loss_coef"]
+    kl = (on_lp - lp).sum(-1) * cfg["kl_coef"] * kl_scale
+    entropy = -ent.sum(-1) * cfg["entropy_coef"]
+    return (policy + value + kl + entropy).mean(), {"policy": policy, "value": value, "kl": kl, "entropy": entropy}
+
+
+def loss_and_grads(params, batch, cfg, kl_scale=1.0, act="elu"):
+    """params: dict(actor_w, actor_b, critic_w, critic_b: lists of float64 arrays; log_std).  batch: (T, b, ...) arrays.
+    Returns (loss, grads with the structure of params, aux)."""
+    tp = {k: ([torch.tensor(np.asarray(a, dtype=np.float64), requires_grad=True) for a in v] if isinstance(v, list)
+              else torch.tensor(np.asarray(v, dtype=np.float64), requires_grad=True)) for k, v in params.items()}
+    t64 = lambda a: torch.tensor(np.asarray(a, dtype=np.float64))  # noqa: E731
+    Tn, b = batch["done"].shape
+    mean = mlp(t64(batch["actor_obs"]), tp["actor_w"], tp["actor_b"], act)
+    v = mlp(t64(batch["critic_obs"]), tp["critic_w"], tp["critic_b"], act)[..., 0]
+    lp, ent = gaussian(mean, tp["log_std"], t64(batch["action"]))
+    # GAE on (B, T) arrays with the current values, as a constant (ppo.py:121 stop_gradient)
+    gi = oppo.compute_ppo_inputs(v.detach().numpy().T, np.asarray(batch["rewards"], np.float64).T, np.asarray(batch["done"]).T,
+                                 np.asarray(batch["success"]).T, cfg["gamma"], cfg["lam"], cfg["normalize_advantages"],
+                                 cfg["monte_carlo_returns"], np.float64)
+    adv, tgt = t64(gi["advantages"].T), t64(gi["value_targets"].T)
+    loss, terms = ppo_loss_torch(adv, tgt, t64(batch["on_log_probs"]), t64(batch["on_values"]), lp, v, ent, cfg, kl_scale)
+    loss.backward()
+    grads = {k: ([a.grad.numpy() for a in v] if isinstance(v, list) else v.grad.numpy()) for k, v in tp.items()}
+    aux = {"mean": mean.detach().numpy(), "values": v.detach().numpy(), "log_probs": lp.detach().numpy(),
+           "advantages": adv.numpy(), "value_targets": tgt.numpy(), "terms": {k: t.detach().numpy() for k, t in terms.items()}}
+    return float(loss.detach()), grads, aux
+
+
+def flat(tree):
+    out = []
+    for k in ("actor_w", "actor_b", "critic_w", "critic_b"):
+        out += list(tree[k])
+    return out + [tree["log_std"]]
+
+
+def optax_chain_step(params, grads, m1, m2, step, cfg):
+    """zero_nans -> clip_by_global_norm -> add_decayed_weights -> scale_by_adam -> lr -> -1 (examples/walking.py:380-387;
+    optax: clip scales by max_norm / norm when norm > max_norm; Adam with bias correction, eps outside the root)."""
+    g = [np.nan_to_num(np.asarray(x, np.float64), nan=0.0, posinf=np.inf, neginf=-np.inf) for x in grads]
+    norm = math.sqrt(sum(float((x * x).sum()) for x in g))
+    if cfg["grad_clip"] > 0 and norm > cfg["grad_clip"]:
+        g = [x / norm * cfg["grad_clip"] for x in g]
+    new_p, new_m1, new_m2 = [], [], []
+    for p, x, a, b in zip(params, g, m1, m2):
+        x = x + cfg["adam_weight_decay"] * p
+        a = cfg["adam_b1"] * a + (1 - cfg["adam_b1"]) * x
+        b = cfg["adam_b2"] * b + (1 - cfg["adam_b2"]) * x * x
+        ah, bh = a / (1 - cfg["adam_b1"] ** step), b / (1 - cfg["adam_b2"] ** step)
+        new_p.append(p - cfg["learning_rate"] * ah / (np.sqrt(bh) + cfg["adam_eps"]))
+        new_m1.append(a)
+        new_m2.append(b)
+    return new_p, new_m1, new_m2, norm
+
+
+def unflat(vals, like):
+    it = iter(vals)
+    out = {}
+    for k in ("actor_w", "actor_b", "critic_w", "critic_b"):
+        out[k] = [next(it) for _ in like[k]]
+    out["log_std"] = next(it)
+    return out
+
+
+def update_model(params, rollout, cfg, permutations, act="elu"):
+    """ppo.py:572-694 with explicit minibatch permutations.  rollout arrays are (T, N, ...)."""
+    params = {k: ([np.asarray(a, np.float64) for a in v] if isinstance(v, list) else np.asarray(v, np.float64)) for k, v in params.items()}
+    t64 = lambda a: torch.tensor(np.asarray(a, dtype=np.float64))  # noqa: E731
+    with torch.no_grad():
+        tw = lambda k: [t64(a) for a in params[k]]  # noqa: E731
+        mean = mlp(t64(rollout["actor_obs"]), tw("actor_w"), tw("actor_b"), act)
+        on_v = mlp(t64(rollout["critic_obs"]), tw("critic_w"), tw("critic_b"), act)[..., 0].numpy()
+        on_lp = gaussian(mean, t64(params["log_std"]), t64(rollout["action"]))[0].numpy()
+    m1 = [np.zeros_like(x) for x in flat(params)]
+    m2 = [np.zeros_like(x) for x in flat(params)]
+    step, losses = 0, []
+    N = rollout["done"].shape[1]
+    bs = min(cfg["batch_size"], N)
+    for perm in permutations:
+        for idx in np.asarray(perm).reshape(-1, bs):
+            batch = {k: np.asarray(v)[:, idx] for k, v in rollout.items()}
+            batch["on_log_probs"], batch["on_values"] = on_lp[:, idx], on_v[:, idx]
+            loss, grads, _ = loss_and_grads(params, batch, cfg, 1.0, act)
+            step += 1
+            new_p, m1, m2, _ = optax_chain_step(flat(params), flat(grads), m1, m2, step, cfg)
+            params = unflat(new_p, params)
+            losses.append(loss)
+    return params, losses

@@ -1,0 +1,184 @@
+"""Policy update (gradients through the Gaussian head, the PPO loss and the MLPs; optimiser chain; minibatch loop)
+through the C ABI against the float64 autograd oracle."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import ppo_update as ou
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+CFG = dict(gamma=0.99, lam=0.95, normalize_advantages=True, monte_carlo_returns=False, clip_param=0.2, value_loss_coef=0.5,
+           entropy_coef=0.008, kl_coef=1e-3, log_clip_value=5.0, use_clipped_value_loss=True, learning_rate=3e-4,
+           adam_b1=0.9, adam_b2=0.999, adam_eps=1e-8, adam_weight_decay=0.01, grad_clip=2.0, batch_size=8, num_passes=2)
+
+
+def t32(a):
+    return torch.tensor(np.asarray(a), dtype=torch.float32, device=DEV).contiguous()
+
+
+def rel(got, want):
+    want = np.asarray(want, np.float64)
+    return np.abs(np.asarray(got, np.float64) - want).max() / max(np.abs(want).max(), 1e-30)
+
+
+@pytest.mark.parametrize("dims,dtype,act,M,tol", [
+    ((71, 256, 256, 21), "f32", "elu", 300, 2e-4),     # fp32 path: accumulation-order error only
+    ((68, 512, 512, 512, 20), "bf16", "elu", 1000, 3e-2),  # bf16 operands, fp32 accumulate
+    ((33, 130, 2), "f32", "tanh", 77, 2e-4), ((40, 64, 64, 1), "f32", "relu", 129, 2e-4),
+])
+def test_mlp_backward_matches_autograd(dims, dtype, act, M, tol):
+    from ksim_amd.mlp import MLP
+
+    rng = np.random.default_rng(sum(dims))
+    ws = [rng.normal(scale=1 / np.sqrt(i), size=(o, i)).astype(np.float32) for i, o in zip(dims[:-1], dims[1:])]
+    bs = [rng.normal(scale=0.1, size=o).astype(np.float32) for o in dims[1:]]
+    x = rng.normal(size=(M, dims[0])).astype(np.float32)
+    dy = rng.normal(size=(M, dims[-1])).astype(np.float32)
+    net = MLP(ws, bs, activation=act, dtype=dtype)
+    net.train_init()
+    xd = t32(x)
+    y = net.train_forward(xd)
+    net.backward(xd, t32(dy))
+    tw = [torch.tensor(w, dtype=torch.float64, requires_grad=True) for w in ws]
+    tb = [torch.tensor(b, dtype=torch.float64, requires_grad=True) for b in bs]
+    yo = ou.mlp(torch.tensor(x, dtype=torch.float64), tw, tb, act)
+    (yo * torch.tensor(dy, dtype=torch.float64)).sum().backward()
+    assert rel(y.cpu().numpy(), yo.detach().numpy()) < (2e-5 if dtype == "f32" else 1e-2)
+    for (gw, gb), w, b in zip(net.parameters(gradients=True), tw, tb):
+        assert rel(gw.cpu().numpy(), w.grad.numpy()) < tol
+        assert rel(gb.cpu().numpy(), b.grad.numpy()) < tol
+    for (pw, pb), w, b in zip(net.parameters(), ws, bs):  # master copy is the caller's fp32 parameters, bit for bit
+        assert np.array_equal(pw.cpu().numpy(), w) and np.array_equal(pb.cpu().numpy(), b)
+    y2 = net(xd)  # the inference path still reads the same weights
+    assert rel(y2.cpu().numpy(), yo.detach().numpy()) < (2e-5 if dtype == "f32" else 1e-2)
+
+
+def test_ppo_loss_gradient_kernel_matches_autograd():
+    from ksim_amd import _lib
+
+    lib = _lib.load()
+    rng = np.random.default_rng(3)
+    M, A = 5000, 20
+    mean, ls, act = rng.normal(size=(M, A)), rng.normal(size=A) * 0.2 - 1.0, rng.normal(size=(M, A))
+    act = mean + np.exp(ls) * act                        # actions the policy plausibly took
+    on_lp = ou.gaussian(torch.tensor(mean + rng.normal(size=(M, A)) * 0.02), torch.tensor(ls), torch.tensor(act))[0].numpy()
+    adv, tgt, on_v, v = rng.normal(size=M), rng.normal(size=M), rng.normal(size=M), rng.normal(size=M)
+    v = on_v + rng.normal(size=M) * 0.3                  # both sides of the value clip
+    tm = torch.tensor(mean, requires_grad=True); tl = torch.tensor(ls, requires_grad=True); tv = torch.tensor(v, requires_grad=True)
+    lp, ent = ou.gaussian(tm, tl, torch.tensor(act))
+    loss, _ = ou.ppo_loss_torch(torch.tensor(adv), torch.tensor(tgt), torch.tensor(on_lp), torch.tensor(on_v), lp, tv, ent, CFG, 1.3)
+    loss.backward()
+    p = _lib.KsPpoLossParams(0.2, 0.5, 0.008, 1e-3, 5.0, 1.3, 1)
+    d_mean, d_value, d_ls = torch.empty(M, A, device=DEV), torch.empty(M, device=DEV), torch.empty(A, device=DEV)
+    ws = torch.empty(256 * A, device=DEV)
+    args = [t32(a) for a in (mean, ls, act, on_lp, adv, tgt, on_v, v)]
+    _lib.check(lib.ks_ppo_loss_grad(_lib.current_stream(), M, A, ctypes.byref(p), *[_lib.ptr(a) for a in args],
+                                    _lib.ptr(d_mean), _lib.ptr(d_value), _lib.ptr(d_ls), _lib.ptr(ws)))
+    assert rel(d_mean.cpu().numpy(), tm.grad.numpy()) < 1e-4
+    assert rel(d_value.cpu().numpy(), tv.grad.numpy()) < 1e-5
+    assert rel(d_ls.cpu().numpy(), tl.grad.numpy()) < 1e-4
+    lp_k, ent_k = torch.empty(M, A, device=DEV), torch.empty(M, A, device=DEV)
+    _lib.check(lib.ks_gaussian_log_prob(_lib.current_stream(), M, A, _lib.ptr(args[0]), _lib.ptr(args[1]), _lib.ptr(args[2]),
+                                        _lib.ptr(lp_k), _lib.ptr(ent_k)))
+    np.testing.assert_allclose(lp_k.cpu().numpy(), lp.detach().numpy(), rtol=1e-5, atol=1e-5)   # GAE/returns class tolerance
+    np.testing.assert_allclose(ent_k.cpu().numpy(), ent.detach().numpy(), rtol=1e-6, atol=1e-6)
+
+
+def test_adam_chain_kernel_matches_optax_restatement():
+    from ksim_amd import _lib, _lib_terms as T
+
+    lib = _lib.load()
+    rng = np.random.default_rng(4)
+    n = 3000
+    p0, g = rng.normal(size=n), rng.normal(size=n) * 0.1
+    g[5] = np.nan
+    p, m1, m2 = t32(p0), torch.zeros(n, device=DEV), torch.zeros(n, device=DEV)
+    po, o1, o2 = [p0.astype(np.float32).astype(np.float64)], [np.zeros(n)], [np.zeros(n)]
+    for step in (1, 2, 3):
+        gs = g * step
+        sq = torch.zeros(1, dtype=torch.float64, device=DEV)
+        gd = t32(gs)
+        _lib.check(lib.ks_grad_sqnorm(_lib.current_stream(), n, _lib.ptr(gd), _lib.ptr(sq)))
+        ap = T.KsAdamParams(3e-4, 0.9, 0.999, 1e-8, 0.01, 2.0, step)
+        _lib.check(lib.ks_adam_step(_lib.current_stream(), n, _lib.ptr(p), _lib.ptr(gd), _lib.ptr(m1), _lib.ptr(m2),
+                                    ctypes.byref(ap), _lib.ptr(sq)))
+        po, o1, o2, norm = ou.optax_chain_step(po, [gs.astype(np.float32).astype(np.float64)], o1, o2, step, CFG)
+        assert abs(float(sq.sqrt().item()) - norm) < 1e-5 * norm
+    np.testing.assert_allclose(p.cpu().numpy(), po[0], rtol=0, atol=2e-6)
+    np.testing.assert_allclose(m1.cpu().numpy(), o1[0], rtol=1e-5, atol=1e-8)
+
+
+def _setup(seed, Tn, N, od, A, hidden):
+    from ksim_amd.mlp import MLP
+    from ksim_amd.ppo_update import GaussianMlpPolicy
+
+    rng = np.random.default_rng(seed)
+    ad, cd = (od, hidden, hidden, A), (od, hidden, 1)
+    mk = lambda dims: ([rng.normal(scale=1 / np.sqrt(i), size=(o, i)).astype(np.float32) for i, o in zip(dims[:-1], dims[1:])],  # noqa: E731
+                       [rng.normal(scale=0.05, size=o).astype(np.float32) for o in dims[1:]])
+    (aw, ab), (cw, cb) = mk(ad), mk(cd)
+    ls = (rng.normal(size=A) * 0.1 - 0.7).astype(np.float32)
+    rollout = dict(actor_obs=rng.normal(size=(Tn, N, od)).astype(np.float32), critic_obs=rng.normal(size=(Tn, N, od)).astype(np.float32),
+                   rewards=rng.normal(size=(Tn, N)).astype(np.float32), done=rng.random((Tn, N)) < 0.05,
+                   success=np.zeros((Tn, N), bool))
+    mean = ou.mlp(torch.tensor(rollout["actor_obs"], dtype=torch.float64), [torch.tensor(w, dtype=torch.float64) for w in aw],
+                  [torch.tensor(b, dtype=torch.float64) for b in ab]).numpy()
+    rollout["action"] = (mean + np.exp(ls) * rng.normal(size=mean.shape)).astype(np.float32)
+    pol = GaussianMlpPolicy(actor=MLP(aw, ab, dtype="f32"), critic=MLP(cw, cb, dtype="f32"), log_std=t32(ls))
+    params = dict(actor_w=aw, actor_b=ab, critic_w=cw, critic_b=cb, log_std=ls)
+    return pol, params, rollout, rng
+
+
+def test_single_step_gradients_match_oracle():
+    from ksim_amd.ppo_update import PPOUpdateConfig, get_ppo_variables, single_step
+
+    Tn, N, od, A = 16, 8, 30, 6
+    pol, params, ro, rng = _setup(7, Tn, N, od, A, 64)
+    pol.train_init()
+    cfg = PPOUpdateConfig(**{k: v for k, v in CFG.items() if k != "adam_weight_decay"}, adam_weight_decay=0.01)
+    d = {k: (torch.tensor(v, device=DEV) if v.dtype == bool else t32(v)) for k, v in ro.items()}
+    rows = Tn * N
+    on_lp, on_v, _, _ = get_ppo_variables(pol, d["actor_obs"].reshape(rows, od), d["critic_obs"].reshape(rows, od), d["action"].reshape(rows, A))
+    on_lp, on_v = on_lp.view(Tn, N, A).clone() - 0.05, on_v.view(Tn, N).clone() + 0.1   # a previous policy, slightly off
+    batch = dict(ro, on_log_probs=on_lp.cpu().numpy(), on_values=on_v.cpu().numpy())
+    loss, grads, aux = ou.loss_and_grads(params, batch, CFG)
+    met = single_step(pol, cfg, d["actor_obs"], d["critic_obs"], d["action"], d["rewards"], d["done"], d["success"], on_lp, on_v)
+    assert rel(met["advantages"].cpu().numpy(), aux["advantages"]) < 1e-4
+    for (gw, gb), w, b in zip(pol.actor.parameters(gradients=True), grads["actor_w"], grads["actor_b"]):
+        assert rel(gw.cpu().numpy(), w) < 5e-4 and rel(gb.cpu().numpy(), b) < 5e-4
+    for (gw, gb), w, b in zip(pol.critic.parameters(gradients=True), grads["critic_w"], grads["critic_b"]):
+        assert rel(gw.cpu().numpy(), w) < 5e-4 and rel(gb.cpu().numpy(), b) < 5e-4
+    assert rel(met["d_log_std"].cpu().numpy(), grads["log_std"]) < 5e-4
+    norm = np.sqrt(sum(float((np.asarray(g) ** 2).sum()) for g in ou.flat(grads)))
+    assert abs(float(met["grad_norm"].item()) - norm) < 1e-3 * norm
+
+
+def test_update_model_tracks_oracle():
+    from ksim_amd.ppo_update import PPOUpdateConfig, update_model
+
+    Tn, N, od, A = 12, 16, 24, 4
+    pol, params, ro, rng = _setup(9, Tn, N, od, A, 64)
+    cfg = PPOUpdateConfig(**CFG)
+    perms = [rng.permutation(N) for _ in range(cfg.num_passes)]
+    want, losses = ou.update_model(params, ro, CFG, perms)
+    d = {k: (torch.tensor(v, device=DEV) if v.dtype == bool else t32(v)) for k, v in ro.items()}
+    mets = update_model(pol, cfg, d["actor_obs"], d["critic_obs"], d["action"], d["rewards"], d["done"], d["success"],
+                        permutations=[torch.tensor(p, device=DEV) for p in perms])
+    steps = cfg.num_passes * (N // cfg.batch_size)
+    assert len(mets) == steps and pol.opt_step == steps
+    # Adam's first steps move a coordinate by about lr whatever the size of its gradient, so a coordinate whose
+    # gradient is at rounding level may go the other way: the bound is a few lr, the typical error far below
+    bound = 2.5 * cfg.learning_rate * steps
+    errs = []
+    for (pw, pb), w, b in zip(pol.actor.parameters() + pol.critic.parameters(), want["actor_w"] + want["critic_w"], want["actor_b"] + want["critic_b"]):
+        for got, ref in ((pw, w), (pb, b)):
+            e = np.abs(got.cpu().numpy() - ref)
+            assert e.max() <= bound
+            errs.append(e.ravel())
+    assert np.abs(pol.log_std.cpu().numpy() - want["log_std"]).max() <= bound
+    assert np.median(np.concatenate(errs)) < 2e-6, "typical parameter error after the update"
+    moved = np.abs(pol.actor.parameters()[0][0].cpu().numpy() - params["actor_w"][0]).max()
+    assert moved > 0.5 * cfg.learning_rate, "the update did not move the parameters"
