@@ -127,8 +127,12 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void mlp_layer_kernel(int64
     }                                                                                                          \
   }
 
-  KS_FETCH(0)
-  for (int k0 = 0; k0 < K; k0 += BK) {
+  // gridDim.z > 1: this workgroup reduces only its slice of K and writes partial sums to its own copy of the
+  // output (LAST outputs only; the caller adds the copies up in a fixed order)
+  const int kslice = K / (int)gridDim.z;
+  const int kbeg = (int)blockIdx.z * kslice, kend = kbeg + kslice;
+  KS_FETCH(kbeg)
+  for (int k0 = kbeg; k0 < kend; k0 += BK) {
 #pragma unroll
     for (int c = 0; c < A_VECS; ++c) {
       const int v = tid + NT * c, row = v / VPR, col = (v % VPR) * VEC;
@@ -142,7 +146,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void mlp_layer_kernel(int64
     __syncthreads();
     // Next slice in flight while the matrix cores work on this one.  The fetch is unconditional (the last pass
     // re-reads its own slice) so that the register arrays are plain loop-carried values.
-    const int kn = k0 + BK < K ? k0 + BK : k0;
+    const int kn = k0 + BK < kend ? k0 + BK : k0;
     KS_FETCH(kn)
     if constexpr (BF) {
 #pragma unroll
@@ -182,14 +186,14 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void mlp_layer_kernel(int64
 #pragma unroll
     for (int j = 0; j < NI; ++j) {
       const int col = n0 + wn * WN + j * 32 + (lane & 31);
-      const float b = bias[col];
+      const float b = blockIdx.z == 0 ? bias[col] : 0.f;
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int64_t row = m0 + wm * WM + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
         if (row >= M) continue;
         const float v = acc[i][j][r] + b;
         if (LAST) {
-          if (col < Nreal) ((float*)yout)[row * ldy + col] = v;
+          if (col < Nreal) ((float*)yout)[(int64_t)blockIdx.z * M * ldy + row * ldy + col] = v;
         } else {
           const float h = activate<ACT, BF>(v);
           ((T*)yout)[row * ldy + col] = BF ? (T)to_bf16(h) : (T)h;
@@ -540,24 +544,37 @@ __global__ __launch_bounds__(256) void act_backward_kernel(int64_t n, const T* _
   dy[idx] = from_f32<T>(to_f32(dy[idx]) * d);
 }
 
-// column sums of a (M, ld) matrix: one workgroup per 64 columns, rows in a fixed order (deterministic)
+// column sums of a (M, ld) matrix in two deterministic stages: gridDim.y row slices write partial sums, which
+// sum_parts_kernel adds up in a fixed order
+constexpr int kColsumSlices = 64;
 template <typename T>
-__global__ __launch_bounds__(256) void colsum_kernel(int64_t M, int ld, const T* __restrict__ a, float* __restrict__ out) {
-  __shared__ float part[4][64];
+__global__ __launch_bounds__(256) void colsum_kernel(int64_t M, int ld, const T* __restrict__ a, float* __restrict__ part) {
+  __shared__ float red[4][64];
   const int c = blockIdx.x * 64 + (threadIdx.x & 63), g = threadIdx.x >> 6;
   float s = 0.f;
   if (c < ld)
-    for (int64_t m = g; m < M; m += 4) s += to_f32(a[m * ld + c]);
-  part[g][threadIdx.x & 63] = s;
+    for (int64_t m = (int64_t)blockIdx.y * 4 + g; m < M; m += 4 * kColsumSlices) s += to_f32(a[m * ld + c]);
+  red[g][threadIdx.x & 63] = s;
   __syncthreads();
-  if (g == 0 && c < ld) out[c] = (part[0][threadIdx.x] + part[1][threadIdx.x]) + (part[2][threadIdx.x] + part[3][threadIdx.x]);
+  if (g == 0 && c < ld)
+    part[(int64_t)blockIdx.y * ld + c] = (red[0][threadIdx.x] + red[1][threadIdx.x]) + (red[2][threadIdx.x] + red[3][threadIdx.x]);
 }
 
-// sum of squares of a buffer, NaNs counted as zero (the optimiser zeroes them first), added to *acc in double
+// out[i] = sum over z of part[z][i], z ascending
+__global__ __launch_bounds__(256) void sum_parts_kernel(int64_t n, int nz, const float* __restrict__ part, float* __restrict__ out) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n) return;
+  float s = 0.f;
+  for (int z = 0; z < nz; ++z) s += part[(int64_t)z * n + i];
+  out[i] = s;
+}
+
+// sum of squares of a buffer, NaNs counted as zero (the optimiser zeroes them first), added to *acc in double.
+// One atomic per workgroup: the order of the additions can differ between runs in the last bit of the double.
 __global__ __launch_bounds__(256) void sqnorm_kernel(int64_t n, const float* __restrict__ g, double* __restrict__ acc) {
   __shared__ double red[256];
   double s = 0.0;
-  for (int64_t i = threadIdx.x; i < n; i += 256) {
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
     const float v = g[i];
     if (v == v) s += (double)v * (double)v;
   }
@@ -567,7 +584,7 @@ __global__ __launch_bounds__(256) void sqnorm_kernel(int64_t n, const float* __r
     if ((int)threadIdx.x < w) red[threadIdx.x] += red[threadIdx.x + w];
     __syncthreads();
   }
-  if (threadIdx.x == 0) *acc += red[0];  // launches are ordered on one stream: no atomics needed
+  if (threadIdx.x == 0) atomicAdd(acc, red[0]);
 }
 
 // optax.chain(zero_nans, clip_by_global_norm, add_decayed_weights, scale_by_adam, scale(lr), scale(-1)) on one tensor
@@ -625,10 +642,10 @@ static uint16_t f32_to_bf16_rne(float f) {
 
 template <typename T, bool FIRST, bool LAST, int BM, int BN, int WAVES_M, int WAVES_N>
 static int launch_layer_tile(int act, hipStream_t s, int64_t M, int npad, int K, int Kreal, int Nreal, const void* x,
-                             int64_t ldx, const void* W, const float* b, void* y, int64_t ldy) {
+                             int64_t ldx, const void* W, const float* b, void* y, int64_t ldy, int ksplit = 1) {
   constexpr int BK = sizeof(T) == 2 ? 64 : 32, PAD = sizeof(T) == 2 ? 8 : 4;
   constexpr int lds = (int)sizeof(T) * (BM + BN) * (BK + PAD);
-  const dim3 grid((unsigned)((M + BM - 1) / BM), (unsigned)(npad / BN));
+  const dim3 grid((unsigned)((M + BM - 1) / BM), (unsigned)(npad / BN), (unsigned)ksplit);
   const dim3 block(64 * WAVES_M * WAVES_N);
 #define KS_LAUNCH(A)                                                                                           \
   {                                                                                                            \
@@ -920,10 +937,13 @@ static void refresh_layers(DevMlp& m, hipStream_t s) {
   }
 }
 
+constexpr int kDwSplit = 16;  // most slices the weight-gradient reduction over the rows is cut into
+
 // workspace: hidden activations of every layer, two (M, widest) gradient buffers, two transposes (widest, Mp)
 struct TrainWs {
   char* act[KS_MAX_LAYERS];
   char *d0, *d1, *t0, *t1;
+  float* part;  // partial sums of the split reductions
   int64_t Mp;
 };
 static int64_t carve_train(const DevMlp& m, int64_t M, char* base, TrainWs* ws) {
@@ -943,6 +963,10 @@ static int64_t carve_train(const DevMlp& m, int64_t M, char* base, TrainWs* ws) 
   w.d1 = take(M * wz * esz);
   w.t0 = take((int64_t)wz * Mp * esz);
   w.t1 = take((int64_t)wz * Mp * esz);
+  int64_t maxw = 0;
+  for (int l = 0; l < m.n_layers; ++l) maxw = (int64_t)m.npad[l] * m.kpad[l] > maxw ? (int64_t)m.npad[l] * m.kpad[l] : maxw;
+  const int64_t nparts = kDwSplit * maxw > (int64_t)kColsumSlices * wz ? kDwSplit * maxw : (int64_t)kColsumSlices * wz;
+  w.part = (float*)take(nparts * 4);
   w.Mp = Mp;
   if (ws) *ws = w;
   return off;
@@ -997,7 +1021,8 @@ static int train_backward(DevMlp& m, hipStream_t s, int64_t M, const float* x, c
   for (int l = L - 1; l >= 0; --l) {
     const int np = m.npad[l], kp = m.kpad[l], kp128 = round_up(kp, kBN);
     // bias gradient
-    hipLaunchKernelGGL(colsum_kernel<T>, dim3((unsigned)((np + 63) / 64)), dim3(256), 0, s, M, np, dz, m.gb[l]);
+    hipLaunchKernelGGL(colsum_kernel<T>, dim3((unsigned)((np + 63) / 64), kColsumSlices), dim3(256), 0, s, M, np, dz, ws.part);
+    hipLaunchKernelGGL(sum_parts_kernel, dim3((unsigned)((np + 255) / 256)), dim3(256), 0, s, (int64_t)np, kColsumSlices, ws.part, m.gb[l]);
     // weight gradient: dZ^T (np, Mp) times Y_prev^T (kp128, Mp)^T
     hipLaunchKernelGGL((transpose_kernel<T, T>), dim3((unsigned)((Mp + 31) / 32), (unsigned)((np + 31) / 32)), dim3(256), 0, s, M, np,
                        (int64_t)np, dz, np, Mp, (T*)ws.t0);
@@ -1007,8 +1032,16 @@ static int train_backward(DevMlp& m, hipStream_t s, int64_t M, const float* x, c
     else
       hipLaunchKernelGGL((transpose_kernel<T, T>), dim3((unsigned)((Mp + 31) / 32), (unsigned)((kp128 + 31) / 32)), dim3(256), 0, s, M,
                          m.npad[l - 1], (int64_t)m.npad[l - 1], (const T*)ws.act[l - 1], kp128, Mp, (T*)ws.t1);
-    int rc = launch_layer<T, false, true>(KS_ACT_NONE, s, np, kp128, (int)Mp, (int)Mp, kp, ws.t0, Mp, ws.t1, m.zero_bias, m.gW[l], kp);
+    // the reduction runs over the rows: cut it into slices so that the grid covers the chip, then add the slices up
+    int ksplit = kDwSplit;
+    while (ksplit > 1 && (Mp / 64) % ksplit != 0) ksplit >>= 1;
+    int rc = launch_layer_tile<T, false, true, 64, 128, 2, 2>(KS_ACT_NONE, s, np, kp128, (int)Mp, (int)Mp, kp, ws.t0, Mp, ws.t1,
+                                                               m.zero_bias, ksplit > 1 ? (void*)ws.part : (void*)m.gW[l], kp, ksplit);
     if (rc != KS_OK) return rc;
+    if (ksplit > 1) {
+      const int64_t n = (int64_t)np * kp;
+      hipLaunchKernelGGL(sum_parts_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, n, ksplit, ws.part, m.gW[l]);
+    }
     if (l == 0) break;
     // input gradient, then through the activation of the layer below
     rc = launch_layer<T, false, false>(KS_ACT_NONE, s, M, kp, np, np, kp, dz, np, m.Wt[l], m.zero_bias, dnext, kp);
@@ -1041,14 +1074,14 @@ extern "C" int ks_mlp_train_backward(KsMlp* h, ks_stream_t stream, int64_t M, co
 extern "C" int ks_grad_sqnorm(ks_stream_t stream, int64_t n, const float* g, double* acc) {
   if (n < 0 || !acc || (n > 0 && !g)) return fail(KS_EINVAL, "ks_grad_sqnorm: bad argument");
   if (n == 0) return KS_OK;
-  hipLaunchKernelGGL(sqnorm_kernel, dim3(1), dim3(256), 0, (hipStream_t)stream, n, g, acc);
+  hipLaunchKernelGGL(sqnorm_kernel, dim3((unsigned)(n >= 65536 ? 64 : 1)), dim3(256), 0, (hipStream_t)stream, n, g, acc);
   return check_launch("ks_grad_sqnorm");
 }
 
 extern "C" int ks_mlp_grad_sqnorm(const KsMlp* h, ks_stream_t stream, double* acc) {
   if (!h || !h->m.train || !acc) return fail(KS_EINVAL, "ks_mlp_grad_sqnorm: bad argument");
   for (int l = 0; l < h->m.n_layers; ++l) {
-    hipLaunchKernelGGL(sqnorm_kernel, dim3(1), dim3(256), 0, (hipStream_t)stream, (int64_t)h->m.npad[l] * h->m.kpad[l], h->m.gW[l], acc);
+    hipLaunchKernelGGL(sqnorm_kernel, dim3(64), dim3(256), 0, (hipStream_t)stream, (int64_t)h->m.npad[l] * h->m.kpad[l], h->m.gW[l], acc);
     hipLaunchKernelGGL(sqnorm_kernel, dim3(1), dim3(256), 0, (hipStream_t)stream, (int64_t)h->m.npad[l], h->m.gb[l], acc);
   }
   return check_launch("ks_mlp_grad_sqnorm");
