@@ -152,6 +152,7 @@ def main() -> None:
     # GAE on rotating cfg-2 sized buffers (T=128, N=4096): larger than the caches in total
     gae = gae_bandwidth(torch, ppo)
     mlp = mlp_rate(torch, consts)
+    upd = ppo_update_rate(torch)
 
     obs_dim = consts.terms.obs_dim
     bytes_per_env = step_algorithmic_bytes(m, obs_dim, 1 + m.nb)
@@ -186,7 +187,7 @@ def main() -> None:
                      "note": "the fused step is bound by fp32 vector-ALU issue (~1e3 flop/byte; the profiled share of "
                              "cycles with a VALU instruction issuing is given beside); the HBM fraction is reported "
                              "against the bytes the engine contract obliges a step to move"},
-        "gae": gae, "policy_mlp": mlp, "graph_replay": graph,
+        "gae": gae, "policy_mlp": mlp, "ppo_update": upd, "graph_replay": graph,
     }
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline()
@@ -227,6 +228,43 @@ def gae_bandwidth(torch, ppo, reps=8):
                      "frac_of_hbm_peak": nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "algorithmic_bytes": nbytes,
                      "buffer_sets": sets}
     return out
+
+
+def ppo_update_rate(torch, reps=6):
+    """One minibatch step of the policy update at BASELINE config 5's shape: 2048 envs x T=32 rows through actor and
+    critic (3x512 bf16), GAE, loss gradient, backward GEMMs, optimiser chain."""
+    from ksim_amd.mlp import random_mlp
+    from ksim_amd.ppo_update import GaussianMlpPolicy, PPOUpdateConfig, get_ppo_variables, single_step
+
+    Tn, b, od, A = 32, 2048, 68, 20
+    actor, _, _ = random_mlp((od, 512, 512, 512, A), 0)
+    critic, _, _ = random_mlp((od, 512, 512, 512, 1), 1)
+    pol = GaussianMlpPolicy(actor=actor, critic=critic, log_std=torch.full((A,), -1.0, device="cuda"))
+    pol.train_init()
+    cfg = PPOUpdateConfig()
+    g = torch.Generator(device="cuda")
+    g.manual_seed(0)
+    obs = torch.randn(Tn, b, od, device="cuda", generator=g)
+    act = torch.randn(Tn, b, A, device="cuda", generator=g) * 0.3
+    rew = torch.randn(Tn, b, device="cuda", generator=g)
+    done = torch.rand(Tn, b, device="cuda", generator=g) < 0.02
+    succ = torch.zeros_like(done)
+    on_lp, on_v, _, _ = get_ppo_variables(pol, obs.reshape(-1, od), obs.reshape(-1, od), act.reshape(-1, A))
+    on_lp, on_v = on_lp.view(Tn, b, A).clone(), on_v.view(Tn, b).clone()
+    for _ in range(2):
+        single_step(pol, cfg, obs, obs, act, rew, done, succ, on_lp, on_v)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        single_step(pol, cfg, obs, obs, act, rew, done, succ, on_lp, on_v)
+    e1.record()
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / reps
+    flops = 3 * (actor.flops_per_row() + critic.flops_per_row()) * Tn * b
+    return {"rows": Tn * b, "ms_per_minibatch_step": ms, "TFLOPs": flops / ms / 1e9,
+            "mfma_utilisation": flops / ms / 1e9 / (BF16_PEAK_TFLOPS),
+            "what": "forward + backward (3x the forward flops) of actor and critic 68-3x512-{20,1} bf16, GAE, loss "
+                    "gradient and optimiser chain on 2048 envs x 32 steps"}
 
 
 def mlp_rate(torch, consts, reps=20):
