@@ -710,11 +710,35 @@ void step_kernel(StepArgs a) {
         const float g0 = gauss;
         const float g1 = wave_sum(is_dof ? search * (Ma - qfs) : 0.f);
         const float g2 = 0.5f * wave_sum(is_dof ? search * mv : 0.f);
+        // With at most 16 constraint rows the three sums of a cost evaluation share one reduction: the 16-lane
+        // groups 0, 1, 2 hold copies of the rows with the constant, linear and quadratic coefficient, and one
+        // DPP reduction within the groups yields all three totals.
+        const bool packed = nefc <= 16;
+        float pk_j = 0.f, pk_jv = 0.f, pk_q = 0.f;
+        if (packed) {
+          const int r = lane & 15, grp = lane >> 4;
+          pk_j = __shfl(Jaref, r);
+          pk_jv = __shfl(jv, r);
+          const float c0 = __shfl(q0r, r), c1 = __shfl(q1r, r), c2 = __shfl(q2r, r);
+          pk_q = grp == 0 ? c0 : (grp == 1 ? c1 : (grp == 2 ? c2 : 0.f));
+        }
         auto point = [&](float alpha) {
-          const bool on = is_row && (Jaref + alpha * jv < 0.f);
-          const float q0 = g0 + wave_sum(on ? q0r : 0.f);
-          const float q1 = g1 + wave_sum(on ? q1r : 0.f);
-          const float q2 = g2 + wave_sum(on ? q2r : 0.f);
+          float q0, q1, q2;
+          if (packed) {
+            float x = (pk_j + alpha * pk_jv < 0.f) ? pk_q : 0.f;  // rows beyond nefc carry zeros
+            x += dpp_shift<0x111, 0xf>(x);
+            x += dpp_shift<0x112, 0xf>(x);
+            x += dpp_shift<0x114, 0xf>(x);
+            x += dpp_shift<0x118, 0xf>(x);  // lane 15 of each 16-lane group holds the group's total
+            q0 = g0 + lane_bcast(x, 15);
+            q1 = g1 + lane_bcast(x, 31);
+            q2 = g2 + lane_bcast(x, 47);
+          } else {
+            const bool on = is_row && (Jaref + alpha * jv < 0.f);
+            q0 = g0 + wave_sum(on ? q0r : 0.f);
+            q1 = g1 + wave_sum(on ? q1r : 0.f);
+            q2 = g2 + wave_sum(on ? q2r : 0.f);
+          }
           LsPoint p;
           p.alpha = alpha;
           p.cost = alpha * alpha * q2 + alpha * q1 + q0;
