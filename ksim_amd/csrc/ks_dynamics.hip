@@ -197,6 +197,26 @@ __device__ __forceinline__ float row_dot(const float* row, const float (&vv)[NP]
   return s0 + s1;
 }
 
+// Per-lane constants of one substep, as stored in DevModel::lane_rec (64 dwords, filled by ks_model_create):
+// lane L's body (L < nb), dof (L < nv), contact sphere (L < ns) and its share of the (i, ancestor j) dof pairs.
+// Lanes beyond a range carry the entries of index 0 (or -1 / zero where the kernel tests for that).
+struct LaneRec {
+  int b_parent, b_jtype, b_qadr, b_dofadr;
+  int b_depth;
+  float b_q0, b_mass, pad0;
+  float b_pos[3], b_ipos[3], b_inertia[3], b_jaxis[3], b_jpos[3], pad1;
+  float b_quat[4], b_iquat[4];
+  int d_body, d_act, d_jtype, d_k;
+  float d_damping, d_armature, d_gear, d_lo, d_hi;
+  int s_body;
+  float s_rad, s_invw;
+  float s_pos[3];
+  unsigned s_mask;
+  int pk[kMaxPairs / 64 + 1];
+  int pad2[64 - 48 - (kMaxPairs / 64 + 1)];
+};
+static_assert(sizeof(LaneRec) == 256, "LaneRec must fill the 64-dword record");
+
 struct LsPoint {
   float alpha, cost, d0, d1;
 };
@@ -287,33 +307,35 @@ void step_kernel(StepArgs a) {
       // across the solver, whose register rows set the occupancy
     const bool is_body = lane > 0 && lane < nb;
     const int bl = is_body ? lane : 0;
-    const int b_parent = m.body_parent[bl], b_jtype = m.body_jtype[bl], b_qadr = m.body_qadr[bl],
-              b_dofadr = m.body_dofadr[bl], b_depth = is_body ? m.body_depth[bl] : -1;
-    const V3 b_pos = ld3(m.body_pos[bl]), b_ipos = ld3(m.body_ipos[bl]), b_inertia = ld3(m.body_inertia[bl]),
-             b_jaxis = ld3(m.jnt_axis[bl]), b_jpos = ld3(m.jnt_pos[bl]);
-    const Quat b_quat = {m.body_quat[bl][0], m.body_quat[bl][1], m.body_quat[bl][2], m.body_quat[bl][3]};
-    const Quat b_iquat = {m.body_iquat[bl][0], m.body_iquat[bl][1], m.body_iquat[bl][2], m.body_iquat[bl][3]};
-    const float b_q0 = (is_body && b_jtype == kJntHinge) ? m.qpos0[b_qadr] : 0.f;
-    const float b_mass = is_body ? m.body_mass[bl] * (a.mass_scale ? a.mass_scale[env * nb + bl] : 1.f) : 0.f;
     const bool is_dof = lane < nv;
-    const int dl = is_dof ? lane : 0;
-    const int d_body = m.dof_body[dl], d_act = is_dof ? m.dof_act[dl] : -1;
-    const int d_jtype = m.body_jtype[d_body], d_k = dl - m.body_dofadr[d_body];
-    const float d_damping = m.dof_damping[dl], d_armature = m.dof_armature[dl];
-    const int ua = d_act >= 0 ? d_act : 0;
-    const float d_gear = m.act_gear[ua], d_lo = m.act_lo[ua], d_hi = m.act_hi[ua];
     const bool is_sph = lane < ns;
-    const int sl = is_sph ? lane : 0;
-    const int s_body = m.sph_body[sl];
-    const V3 s_pos = ld3(m.sph_pos[sl]);
-    const float s_rad = m.sph_radius[sl], s_invw = m.body_invweight0[s_body];
-    const unsigned s_mask = m.body_dofmask[s_body];
-    int pk[kMaxPairs / 64 + 1];
-  #pragma unroll
-    for (int k = 0; k < kMaxPairs / 64 + 1; ++k) {
-      const int p = lane + 64 * k;
-      pk[k] = p < m.npairs ? ((int)m.pair_i[p] << 8) | (int)m.pair_j[p] : -1;
+    LaneRec rec;
+    {
+      const uint4* src = reinterpret_cast<const uint4*>(m.lane_rec[lane]);
+      uint4* dst = reinterpret_cast<uint4*>(&rec);
+#pragma unroll
+      for (int k = 0; k < 16; ++k) dst[k] = src[k];
     }
+    const int b_parent = rec.b_parent, b_jtype = rec.b_jtype, b_qadr = rec.b_qadr, b_dofadr = rec.b_dofadr,
+              b_depth = rec.b_depth;
+    (void)b_parent;
+    const V3 b_pos = {rec.b_pos[0], rec.b_pos[1], rec.b_pos[2]}, b_ipos = {rec.b_ipos[0], rec.b_ipos[1], rec.b_ipos[2]},
+             b_inertia = {rec.b_inertia[0], rec.b_inertia[1], rec.b_inertia[2]},
+             b_jaxis = {rec.b_jaxis[0], rec.b_jaxis[1], rec.b_jaxis[2]}, b_jpos = {rec.b_jpos[0], rec.b_jpos[1], rec.b_jpos[2]};
+    const Quat b_quat = {rec.b_quat[0], rec.b_quat[1], rec.b_quat[2], rec.b_quat[3]};
+    const Quat b_iquat = {rec.b_iquat[0], rec.b_iquat[1], rec.b_iquat[2], rec.b_iquat[3]};
+    const float b_q0 = rec.b_q0;
+    const float b_mass = is_body ? rec.b_mass * (a.mass_scale ? a.mass_scale[env * nb + bl] : 1.f) : 0.f;
+    const int d_body = rec.d_body, d_act = rec.d_act, d_jtype = rec.d_jtype, d_k = rec.d_k;
+    const float d_damping = rec.d_damping, d_armature = rec.d_armature, d_gear = rec.d_gear, d_lo = rec.d_lo, d_hi = rec.d_hi;
+    (void)d_armature;
+    const int s_body = rec.s_body;
+    const V3 s_pos = {rec.s_pos[0], rec.s_pos[1], rec.s_pos[2]};
+    const float s_rad = rec.s_rad, s_invw = rec.s_invw;
+    const unsigned s_mask = rec.s_mask;
+    int pk[kMaxPairs / 64 + 1];
+#pragma unroll
+    for (int k = 0; k < kMaxPairs / 64 + 1; ++k) pk[k] = rec.pk[k];
 
     // ---- actuators (ksim/engine.py:287-320, ksim/actuators.py:198-217)
     if (!FWD && (sub % a.actuator_period) == 0 && lane < nu) {
@@ -940,6 +962,39 @@ extern "C" int ks_model_create(const KsModelDesc* d, KsModel** out) {
         if (c == d->dof_body[j]) { mask |= 1u << j; break; }
     }
     m.body_dofmask[b] = mask;
+  }
+  for (int L = 0; L < 64; ++L) {
+    LaneRec r;
+    std::memset(&r, 0, sizeof(r));
+    const bool is_body = L > 0 && L < d->nb;
+    const int bl = is_body ? L : 0;
+    r.b_parent = m.body_parent[bl]; r.b_jtype = m.body_jtype[bl]; r.b_qadr = m.body_qadr[bl]; r.b_dofadr = m.body_dofadr[bl];
+    r.b_depth = is_body ? m.body_depth[bl] : -1;
+    r.b_q0 = (is_body && r.b_jtype == kJntHinge) ? m.qpos0[r.b_qadr] : 0.f;
+    r.b_mass = m.body_mass[bl];
+    for (int k = 0; k < 3; ++k) {
+      r.b_pos[k] = m.body_pos[bl][k]; r.b_ipos[k] = m.body_ipos[bl][k]; r.b_inertia[k] = m.body_inertia[bl][k];
+      r.b_jaxis[k] = m.jnt_axis[bl][k]; r.b_jpos[k] = m.jnt_pos[bl][k];
+    }
+    for (int k = 0; k < 4; ++k) { r.b_quat[k] = m.body_quat[bl][k]; r.b_iquat[k] = m.body_iquat[bl][k]; }
+    const bool is_dof = L < d->nv;
+    const int dl = is_dof ? L : 0;
+    r.d_body = d->nv > 0 ? m.dof_body[dl] : 0;
+    r.d_act = is_dof ? m.dof_act[dl] : -1;
+    r.d_jtype = m.body_jtype[r.d_body];
+    r.d_k = dl - m.body_dofadr[r.d_body];
+    r.d_damping = m.dof_damping[dl]; r.d_armature = m.dof_armature[dl];
+    const int ua = r.d_act >= 0 ? r.d_act : 0;
+    r.d_gear = m.act_gear[ua]; r.d_lo = m.act_lo[ua]; r.d_hi = m.act_hi[ua];
+    const int sl = L < d->ns ? L : 0;
+    r.s_body = m.sph_body[sl]; r.s_rad = m.sph_radius[sl]; r.s_invw = m.body_invweight0[r.s_body];
+    for (int k = 0; k < 3; ++k) r.s_pos[k] = m.sph_pos[sl][k];
+    r.s_mask = m.body_dofmask[r.s_body];
+    for (int k = 0; k < kMaxPairs / 64 + 1; ++k) {
+      const int p = L + 64 * k;
+      r.pk[k] = p < m.npairs ? ((int)m.pair_i[p] << 8) | (int)m.pair_j[p] : -1;
+    }
+    std::memcpy(m.lane_rec[L], &r, sizeof(r));
   }
   if (hipGetDevice(&km->device) != hipSuccess) { delete km; return fail(KS_ELAUNCH, "ks_model_create: no HIP device"); }
   if (hipMalloc((void**)&km->dev, sizeof(DevModel)) != hipSuccess) { delete km; return fail(KS_ELAUNCH, "ks_model_create: hipMalloc failed"); }

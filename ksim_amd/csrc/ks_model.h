@@ -39,6 +39,9 @@ struct DevModel {
   int sph_body[kMaxS];
   float sph_pos[kMaxS][3], sph_radius[kMaxS];
   short pair_i[kMaxPairs], pair_j[kMaxPairs];  // (i, j): j is i or an ancestor dof of i
+  // What lane L reads at the top of every substep, gathered into one 64-dword record so that it arrives in
+  // sixteen 16-byte loads from one base address (layout: LaneRec in ks_dynamics.hip).
+  unsigned lane_rec[64][64];
 };
 
 // ---------------------------------------------------------------- wavefront reductions (DPP, no LDS)
