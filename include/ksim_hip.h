@@ -32,7 +32,8 @@ const char* ks_version(void);
 const char* ks_last_error(void);
 /* sizeof() of a public struct as this library was compiled, for binding self-checks:
  * 0 KsPpoLossParams, 1 KsModelDesc, 2 KsStepIO, 3 KsTermsDesc, 4 KsObserveIO, 5 KsTerminateIO, 6 KsMlpDesc,
- * 7 KsRewardIO, 8 KsObsElem, 9 KsTermDesc, 10 KsRewardDesc, 11 KsRng, 12 KsAdamParams; -1 for anything else. */
+ * 7 KsRewardIO, 8 KsObsElem, 9 KsTermDesc, 10 KsRewardDesc, 11 KsRng, 12 KsAdamParams, 13 KsEventDesc;
+ * -1 for anything else. */
 int64_t ks_abi_sizeof(int32_t which);
 
 /* ------------------------------------------------------------------ GAE / returns
@@ -135,6 +136,34 @@ int ks_model_create(const KsModelDesc* desc /*host*/, KsModel** out);
 int ks_model_destroy(KsModel* model);
 int ks_model_lds_bytes(const KsModel* model); /* LDS one env needs in the step kernel */
 
+/* Random draws: every entry point that needs randomness takes either explicit pre-sampled
+ * buffers (so both sides of a parity test see identical draws) or, when they are NULL, a
+ * counter-based Philox-4x32-10 stream keyed by (seed, env, step, purpose). */
+typedef struct KsRng {
+  uint64_t seed;
+  uint64_t step;
+  const uint64_t* step_base; /* device, nullable: added to `step` when the kernel runs, so that a captured
+                                HIP graph of a rollout draws fresh numbers on every replay */
+} KsRng;
+
+/* Velocity events inside the substep loop (ksim/events.py:58-237, called per physics step at
+ * ksim/engine.py:322-333): every substep the time remaining of an event is decremented by dt; when it reaches
+ * zero the root velocity gets an impulse and a new interval is drawn.
+ *   linear push : qvel[0:3] += (cos t, sin t, 0) * (lo + u1 (hi - lo)) * mag * level_scale, t = 2 pi u0
+ *   angular push: qvel[5]   += +-(lo + u1 (hi - lo)) * mag * level_scale, minus when u0 < 0.5
+ *   jump        : qvel[0:3] += sqrt(2 * -gravity * (lo + u0 (hi - lo)) * level_scale)
+ *   all         : time remaining = interval_lo + u2 (interval_hi - interval_lo)
+ * The continuous-force event (ForcePushEvent, events.py:240-365) is not built. */
+#define KS_MAX_EVENTS 4
+enum { KS_EVENT_LINEAR_PUSH = 0, KS_EVENT_ANGULAR_PUSH = 1, KS_EVENT_JUMP = 2 };
+typedef struct KsEventDesc {
+  int32_t kind;
+  float mag;          /* linvel | angvel | unused */
+  float lo, hi;       /* vel_range | jump_height_range */
+  float interval_lo, interval_hi;
+  float level_scale;  /* event.scale.get_scale(curriculum_level) */
+} KsEventDesc;
+
 /* ------------------------------------------------------------------ control step / forward
  * ks_step replaces MjxEngine.step (ksim/engine.py:259-361): `substeps` physics steps of
  * mjx.step (engine.py:257) with the latency blend (287-288), the actuator update every
@@ -197,6 +226,12 @@ typedef struct KsStepIO {
   float* dbg_bias;          /* (N, nv) */
   float* dbg_qacc_smooth;   /* (N, nv) */
   float* dbg_con_dist;      /* (N, ns) */
+  /* events (ks_step only) */
+  int32_t n_events;
+  KsEventDesc events[KS_MAX_EVENTS];
+  float* event_state;          /* (n_events, N) time remaining, in/out */
+  const float* event_uniform;  /* (substeps, N, n_events, 3) U[0,1) draws, nullable -> Philox */
+  KsRng event_rng;
 } KsStepIO;
 
 int ks_step(const KsModel* model, ks_stream_t stream, const KsStepIO* io /*host*/);
@@ -259,16 +294,6 @@ typedef struct KsTerms KsTerms;
 int ks_terms_create(const KsTermsDesc* desc /*host*/, KsTerms** out);
 int ks_terms_destroy(KsTerms* terms);
 
-/* Random draws: every entry point that needs randomness takes either explicit pre-sampled
- * buffers (so both sides of a parity test see identical draws) or, when they are NULL, a
- * counter-based Philox-4x32-10 stream keyed by (seed, env, step, purpose). */
-typedef struct KsRng {
-  uint64_t seed;
-  uint64_t step;
-  const uint64_t* step_base; /* device, nullable: added to `step` when the kernel runs, so that a captured
-                                HIP graph of a rollout draws fresh numbers on every replay */
-} KsRng;
-
 typedef struct KsObserveIO {
   int64_t N;
   float level;               /* curriculum level */
@@ -299,6 +324,11 @@ typedef struct KsTerminateIO {
   const float* reset_uniform; /* (N, nq + 1) U(-1,1) draws (last one: heading), nullable -> Philox */
   KsRng rng;
   int32_t apply_reset;       /* 0: report terminations only; 1: reset finished envs; 2: reset every env (initial reset) */
+  /* event timers of the envs that start a fresh episode: a new interval each (engine.py:226-232) */
+  int32_t n_events;
+  float event_interval[KS_MAX_EVENTS][2];
+  float* event_state;               /* (n_events, N), nullable when n_events == 0 */
+  const float* event_reset_uniform; /* (N, n_events) U[0,1) draws, nullable -> Philox */
 } KsTerminateIO;
 int ks_terminate_reset(const KsTerms* terms, ks_stream_t stream, const KsTerminateIO* io /*host*/);
 

@@ -31,6 +31,8 @@ class KsModelDesc(ctypes.Structure):
     ]
 
 
+from . import _lib_terms as _T  # noqa: E402  (event and random-number structs)
+
 _P = c_void_p
 STEP_IO_POINTERS = (
     "qpos", "qvel", "qacc_warmstart", "time", "last_ctrl",
@@ -44,7 +46,9 @@ STEP_IO_POINTERS = (
 
 class KsStepIO(ctypes.Structure):
     _fields_ = [("N", c_int64), ("substeps", c_int32), ("actuator_period", c_int32), ("actuator_type", c_int32),
-                ("action_scale", c_float)] + [(name, _P) for name in STEP_IO_POINTERS]
+                ("action_scale", c_float)] + [(name, _P) for name in STEP_IO_POINTERS] + [
+                    ("n_events", c_int32), ("events", _T.KsEventDesc * _T.KS_MAX_EVENTS), ("event_state", _P),
+                    ("event_uniform", _P), ("event_rng", _T.KsRng)]
 
 
 def model_desc(m) -> KsModelDesc:

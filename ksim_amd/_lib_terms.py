@@ -40,6 +40,15 @@ class KsRng(ctypes.Structure):
     _fields_ = [("seed", c_uint64), ("step", c_uint64), ("step_base", c_void_p)]
 
 
+KS_MAX_EVENTS = 4
+EVENT_LINEAR_PUSH, EVENT_ANGULAR_PUSH, EVENT_JUMP = range(3)
+
+
+class KsEventDesc(ctypes.Structure):
+    _fields_ = [("kind", c_int32), ("mag", c_float), ("lo", c_float), ("hi", c_float), ("interval_lo", c_float),
+                ("interval_hi", c_float), ("level_scale", c_float)]
+
+
 class KsObserveIO(ctypes.Structure):
     _fields_ = [("N", c_int64), ("level", c_float), ("src", c_void_p * SRC_COUNT), ("zero_offset", c_void_p),
                 ("bias", c_void_p), ("noise_normal", c_void_p), ("noise_uniform", c_void_p), ("rng", KsRng),
@@ -51,7 +60,9 @@ class KsTerminateIO(ctypes.Structure):
                 ("qacc_warmstart", c_void_p), ("time", c_void_p), ("last_ctrl", c_void_p), ("components", c_void_p),
                 ("done", c_void_p), ("success", c_void_p), ("traj_qpos", c_void_p), ("traj_qvel", c_void_p),
                 ("traj_time", c_void_p), ("reset_mask", c_void_p), ("episode_length", c_void_p),
-                ("reset_uniform", c_void_p), ("rng", KsRng), ("apply_reset", c_int32)]
+                ("reset_uniform", c_void_p), ("rng", KsRng), ("apply_reset", c_int32), ("n_events", c_int32),
+                ("event_interval", (c_float * 2) * KS_MAX_EVENTS), ("event_state", c_void_p),
+                ("event_reset_uniform", c_void_p)]
 
 
 class KsMlpDesc(ctypes.Structure):

@@ -17,6 +17,7 @@
 // The arithmetic follows the MuJoCo model that ksim/engine.py:257 invokes through mjx.step.
 #include "ks_common.h"
 #include "ks_model.h"
+#include "ks_philox.h"
 #include "ks_step_args.h"
 
 #include <cmath>
@@ -272,6 +273,10 @@ void step_kernel(StepArgs a) {
   const float scale = 1.0f / (m.meaninertia * (float)(nv > 1 ? nv : 1));
   int niter_out = 0, nefc_out = 0;
   float my_qacc = 0.f;
+  // time remaining of every velocity event (wave-uniform), kept in registers for the whole control step
+  float ev_left[KS_MAX_EVENTS];
+#pragma unroll
+  for (int e = 0; e < KS_MAX_EVENTS; ++e) ev_left[e] = (!FWD && e < a.n_events) ? a.event_state[(int64_t)e * a.N + env] : 0.f;
   // actuator inputs of this control step (lane = actuator), read once
   float u_last = 0.f, u_act = 0.f, u_kp = 0.f, u_kd = 0.f, u_lim = 0.f, u_zero = 0.f, u_abias = 0.f, u_tbias = 0.f;
   bool u_drop = false;
@@ -355,6 +360,44 @@ void step_kernel(StepArgs a) {
         t = fminf(fmaxf(t, -u_lim), u_lim);
       }
       l.tau[u] = t;
+    }
+
+    // ---- events (ksim/engine.py:322-333, ksim/events.py): impulses on the root velocity when an interval runs out
+    if (!FWD && a.n_events > 0) {
+      const uint64_t ev_step = a.event_rng.step + (a.event_rng.step_base ? *a.event_rng.step_base : 0ull);
+#pragma unroll
+      for (int e = 0; e < KS_MAX_EVENTS; ++e) {
+        if (e < a.n_events) {
+          const KsEventDesc ev = a.events[e];
+          float left = ev_left[e] - m.dt;
+          if (left <= 0.f) {  // wave-uniform
+            float u0, u1, u2;
+            if (a.event_uniform) {
+              const float* u = a.event_uniform + (((int64_t)sub * a.N + env) * a.n_events + e) * 3;
+              u0 = u[0]; u1 = u[1]; u2 = u[2];
+            } else {
+              const Philox4 r = draw(a.event_rng.seed, ev_step, kRngEvent, (uint64_t)env, (uint32_t)(sub * KS_MAX_EVENTS + e));
+              u0 = u01(r.x); u1 = u01(r.y); u2 = u01(r.z);
+            }
+            if (lane == 0) {
+              if (ev.kind == KS_EVENT_LINEAR_PUSH) {
+                const float th = 6.28318530717958647692f * u0, mag = (ev.lo + u1 * (ev.hi - ev.lo)) * ev.mag * ev.level_scale;
+                l.qvel[0] += cosf(th) * mag;
+                l.qvel[1] += sinf(th) * mag;
+              } else if (ev.kind == KS_EVENT_ANGULAR_PUSH) {
+                const float mag = (ev.lo + u1 * (ev.hi - ev.lo)) * ev.mag;
+                l.qvel[5] += (u0 < 0.5f ? -mag : mag) * ev.level_scale;
+              } else if (ev.kind == KS_EVENT_JUMP) {
+                const float h = (ev.lo + u0 * (ev.hi - ev.lo)) * ev.level_scale;
+                for (int k = 0; k < 3; ++k) l.qvel[k] += sqrtf(2.f * -m.gravity[k] * h);
+              }
+            }
+            left = ev.interval_lo + u2 * (ev.interval_hi - ev.interval_lo);
+          }
+          ev_left[e] = left;
+        }
+      }
+      KS_SYNC();
     }
 
     KS_TICK(0)
@@ -857,6 +900,8 @@ void step_kernel(StepArgs a) {
   if (a.traj_ctrl) for (int i = lane; i < nu; i += 64) a.traj_ctrl[env * nu + i] = l.tau[i];
   if (a.traj_xpos) for (int i = lane; i < nb * 3; i += 64) a.traj_xpos[env * nb * 3 + i] = l.xpos[i];
   if (a.traj_xquat) for (int i = lane; i < nb * 4; i += 64) a.traj_xquat[env * nb * 4 + i] = l.xquat[i];
+  if (!FWD && lane == 0)
+    for (int e = 0; e < a.n_events; ++e) a.event_state[(int64_t)e * a.N + env] = ev_left[e];
   if (a.solver_niter && lane == 0) a.solver_niter[env] = niter_out;
   if (a.nefc && lane == 0) a.nefc[env] = nefc_out;
 }
@@ -1053,6 +1098,17 @@ static int launch_step(const KsModel* km, ks_stream_t stream, const KsStepIO* io
     a.action_scale = io->action_scale;
     a.action_noise = io->action_noise; a.torque_noise = io->torque_noise; a.action_bias = io->action_bias;
     a.torque_bias = io->torque_bias;
+    if (io->n_events < 0 || io->n_events > KS_MAX_EVENTS) return fail(KS_ELIMIT, "ks_step: %d events (0..%d)", io->n_events, KS_MAX_EVENTS);
+    if (io->n_events > 0) {
+      if (!io->event_state) return fail(KS_EINVAL, "ks_step: events need event_state");
+      if (m.nv < 6 || m.body_jtype[1] != kJntFree) return fail(KS_EINVAL, "ks_step: events push a floating base");
+      for (int e = 0; e < io->n_events; ++e)
+        if (io->events[e].kind < KS_EVENT_LINEAR_PUSH || io->events[e].kind > KS_EVENT_JUMP)
+          return fail(KS_EINVAL, "ks_step: event %d: unknown kind %d", e, io->events[e].kind);
+      a.n_events = io->n_events;
+      for (int e = 0; e < io->n_events; ++e) a.events[e] = io->events[e];
+      a.event_state = io->event_state; a.event_uniform = io->event_uniform; a.event_rng = io->event_rng;
+    }
   }
   const int bytes = lds_floats(m.nb, m.nq, m.nv, m.nu, m.ns) * 4;
   if (bytes > 160 * 1024) return fail(KS_ELIMIT, "ks_step: model needs %d bytes of LDS", bytes);

@@ -326,6 +326,7 @@ extern "C" int64_t ks_abi_sizeof(int32_t which) {
     case 10: return sizeof(KsRewardDesc);
     case 11: return sizeof(KsRng);
     case 12: return sizeof(KsAdamParams);
+    case 13: return sizeof(KsEventDesc);
     default: return -1;
   }
 }

@@ -2,6 +2,8 @@
 #pragma once
 #include <stdint.h>
 
+#include "../../include/ksim_hip.h"
+
 namespace ks {
 
 struct DevModel;
@@ -21,6 +23,11 @@ struct StepArgs {
   float *qacc, *ctrl_out, *xpos, *xquat, *cvel, *traj_ctrl, *traj_xpos, *traj_xquat;
   int32_t *solver_niter, *nefc;
   float *dbg_M, *dbg_bias, *dbg_qacc_smooth, *dbg_con_dist;
+  int n_events;
+  KsEventDesc events[KS_MAX_EVENTS];
+  float* event_state;
+  const float* event_uniform;
+  KsRng event_rng;
 };
 
 }  // namespace ks

@@ -92,6 +92,10 @@ struct TerminateArgs {
   const float* reset_uniform;
   KsRng rng;
   int apply_reset, nq, nv, nu, n_terms, random_heading, nonfinite_terminates;
+  int n_events;
+  float event_interval[KS_MAX_EVENTS][2];
+  float* event_state;
+  const float* event_reset_uniform;
 };
 
 // A 256-thread workgroup owns kTermEnvs consecutive envs.  The state rows of those envs are contiguous in memory,
@@ -166,6 +170,13 @@ __global__ __launch_bounds__(256) void terminate_kernel(TerminateArgs a) {
     if (a.reset_mask) a.reset_mask[e] = do_reset ? 1 : 0;
     if (a.episode_length) a.episode_length[e] = do_reset ? 0 : a.episode_length[e] + 1;
     if (do_reset && a.time) a.time[e] = 0.f;
+    if (do_reset)
+      for (int k = 0; k < a.n_events; ++k) {
+        float u;
+        if (a.event_reset_uniform) u = a.event_reset_uniform[e * a.n_events + k];
+        else u = u01(draw(a.rng.seed, a.rng.step + (a.rng.step_base ? *a.rng.step_base : 0ull), kRngEvent, (uint64_t)e, 0x10000u + k).x);
+        a.event_state[(int64_t)k * a.N + e] = a.event_interval[k][0] + u * (a.event_interval[k][1] - a.event_interval[k][0]);
+      }
   }
   __syncthreads();
   // ---- flat pass 2: fresh episodes (engine.py:207-246): qpos from the reset table, everything else zero
@@ -413,6 +424,10 @@ extern "C" int ks_terminate_reset(const KsTerms* t, ks_stream_t stream, const Ks
   a.reset_mask = io->reset_mask; a.episode_length = io->episode_length; a.reset_uniform = io->reset_uniform;
   a.rng = io->rng; a.apply_reset = io->apply_reset; a.nq = d.nq; a.nv = d.nv; a.nu = d.nu; a.n_terms = d.n_terms;
   a.random_heading = d.random_heading; a.nonfinite_terminates = d.nonfinite_terminates;
+  if (io->n_events < 0 || io->n_events > KS_MAX_EVENTS) return fail(KS_ELIMIT, "ks_terminate_reset: %d events (0..%d)", io->n_events, KS_MAX_EVENTS);
+  if (io->n_events > 0 && !io->event_state) return fail(KS_EINVAL, "ks_terminate_reset: events need event_state");
+  a.n_events = io->n_events; a.event_state = io->event_state; a.event_reset_uniform = io->event_reset_uniform;
+  for (int k = 0; k < io->n_events; ++k) { a.event_interval[k][0] = io->event_interval[k][0]; a.event_interval[k][1] = io->event_interval[k][1]; }
   const int64_t grid = (io->N + kTermEnvs - 1) / kTermEnvs;
   if (grid > 0x7fffffff) return fail(KS_ELIMIT, "ks_terminate_reset: too many envs");
   hipLaunchKernelGGL(terminate_kernel, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, a);

@@ -14,6 +14,7 @@ from typing import Literal, Mapping, Sequence
 import torch
 
 from . import _lib, physics
+from . import _lib_terms as T
 from .actuators import Actuators, PositionActuators, TorqueActuators
 from .env_terms import EnvTerms
 from .noise import RandomVariable
@@ -125,9 +126,14 @@ class HipEngine(PhysicsEngine):
     """Engine for `physics.DeviceModel`s: every physics substep of a control step runs in one HIP kernel."""
 
     def __init__(self, actuators: Actuators, resets: Sequence[Reset], events: Mapping | None, data: EngineData):
-        if events:
-            raise NotImplementedError("events inside the substep loop (ksim/events.py) are not compiled yet")
-        self.actuators, self.resets, self.events, self.data = actuators, tuple(resets), {}, data
+        from .events import Event  # noqa: PLC0415
+        events = dict(events or {})
+        for name, ev in events.items():
+            if not isinstance(ev, Event):
+                raise NotImplementedError(f"event {name!r} ({type(ev).__name__}) is not one of the compiled velocity events")
+        if len(events) > T.KS_MAX_EVENTS:
+            raise ValueError(f"at most {T.KS_MAX_EVENTS} events")
+        self.actuators, self.resets, self.events, self.data = actuators, tuple(resets), events, data
         self._terms: dict[int, EnvTerms] = {}
 
     def __hash__(self) -> int:
@@ -158,7 +164,7 @@ class HipEngine(PhysicsEngine):
         level = float(curriculum_level)
         lo, hi = self.data.min_action_latency_step * level, self.data.max_action_latency_step * level
         state = PhysicsState(
-            last_ctrl=z(N, m.nu), data=data, event_states={},
+            last_ctrl=z(N, m.nu), data=data, event_states=self._initial_event_states(N, gen, dev),
             actuator_state=self.actuators.get_initial_state(N, gen) if isinstance(self.actuators, PositionActuators) else None,
             action_latency=lo + (hi - lo) * torch.rand(N, generator=gen, device=dev),
             zero_offset=self.data.zero_offset.sample((N, m.nu), gen, level),
@@ -166,6 +172,23 @@ class HipEngine(PhysicsEngine):
         seed = int(torch.randint(0, 2**31 - 1, (1,), generator=gen, device=dev).item())
         self.reset_where(physics_model, state, None, curriculum_level, seed, 0, randomization, reset_uniform)
         return state
+
+    def _initial_event_states(self, N: int, gen, dev) -> dict:
+        """One timer per event and env (engine.py:226-232); rows of one (n_events, N) buffer, which the kernels take."""
+        if not self.events:
+            return {}
+        buf = torch.stack([ev.get_initial_event_state(N, gen, dev) for ev in self.events.values()]).contiguous()
+        out = {name: buf[j] for j, name in enumerate(self.events)}
+        out["_buffer"] = buf
+        return out
+
+    def event_args(self, physics_state: PhysicsState, curriculum_level, seed: int, step: int, step_base=None, uniform=None):
+        """(descs, state, draws, rng) for `physics.control_step`, or None when the engine has no events."""
+        if not self.events:
+            return None
+        descs = [ev.desc(float(curriculum_level)) for ev in self.events.values()]
+        rng = T.KsRng(int(seed) & (2**64 - 1), int(step) & (2**64 - 1), _lib.ptr(step_base).value)
+        return descs, physics_state.event_states["_buffer"], uniform, rng
 
     def reset_where(self, physics_model, state: PhysicsState, mask, curriculum_level, seed: int, step: int,
                     randomization=None, reset_uniform=None) -> None:
@@ -203,7 +226,8 @@ class HipEngine(PhysicsEngine):
     def step(self, action: torch.Tensor, physics_model: physics.DeviceModel, physics_state: PhysicsState,
              curriculum_level, rng, randomization: Mapping[str, torch.Tensor] | None = None,
              noise: Mapping[str, torch.Tensor] | None = None,
-             record: Mapping[str, torch.Tensor] | None = None, want_cvel: bool = True) -> PhysicsState:
+             record: Mapping[str, torch.Tensor] | None = None, want_cvel: bool = True,
+             step: int = 0, step_base=None, event_seed: int = 0) -> PhysicsState:
         m, d, s = physics_model.model, physics_state.data, physics_state
         rnd, noise, record = randomization or {}, noise or {}, record or {}
         drop = noise.get("drop")
@@ -219,6 +243,7 @@ class HipEngine(PhysicsEngine):
                    torque_noise=noise.get("torque_noise"), traj_ctrl=record.get("ctrl"),
                    traj_xpos=record.get("xpos"), traj_xquat=record.get("xquat"))
         act = self.actuators
+        ev = self.event_args(s, curriculum_level, event_seed, step, step_base, noise.get("event_uniform"))
         if isinstance(act, PositionActuators):
             cache = self.prepare(action.device)
             ast = s.actuator_state or {}
@@ -227,10 +252,10 @@ class HipEngine(PhysicsEngine):
                        action_bias=ast.get("action"), torque_bias=ast.get("torque"))
             physics.control_step(physics_model, buf, substeps=self.data.phys_steps_per_ctrl_steps,
                                  actuator_period=self.data.phys_steps_per_actuator_step,
-                                 actuator_type=act.kind, action_scale=act.action_scale)
+                                 actuator_type=act.kind, action_scale=act.action_scale, events=ev)
         elif isinstance(act, TorqueActuators):
             physics.control_step(physics_model, buf, substeps=self.data.phys_steps_per_ctrl_steps,
-                                 actuator_period=self.data.phys_steps_per_actuator_step, actuator_type=act.kind)
+                                 actuator_period=self.data.phys_steps_per_actuator_step, actuator_type=act.kind, events=ev)
         else:
             raise ValueError(f"Unsupported actuators: {type(act).__name__}")
         return physics_state

@@ -123,6 +123,7 @@ class EnvTerms:
     def terminate_reset(self, state: Mapping[str, torch.Tensor], *, level: float = 1.0, components=None, done=None,
                         success=None, traj_qpos=None, traj_qvel=None, traj_time=None, reset_mask=None,
                         episode_length=None, reset_uniform=None, seed: int = 0, step: int = 0, step_base=None,
+                        event_state=None, event_intervals=(), event_reset_uniform=None,
                         apply_reset: bool = True) -> None:
         m = self.model
         qpos = state["qpos"]
@@ -147,6 +148,18 @@ class EnvTerms:
                 raise _lib.KsError(f"{name}: expected {shape}, got {tuple(t.shape)}")
             setattr(io, name, t.data_ptr())
         io.rng = _rng(seed, step, step_base)
+        if event_state is not None:  # timers of the events, re-drawn for the envs that start a fresh episode
+            _lib.require_cuda(event_state, dtype=torch.float32)
+            if tuple(event_state.shape) != (len(event_intervals), N):
+                raise _lib.KsError("event state must be (n_events, N)")
+            io.n_events, io.event_state = len(event_intervals), event_state.data_ptr()
+            for j, (lo, hi) in enumerate(event_intervals):
+                io.event_interval[j][0], io.event_interval[j][1] = float(lo), float(hi)
+            if event_reset_uniform is not None:
+                _lib.require_cuda(event_reset_uniform, dtype=torch.float32)
+                if tuple(event_reset_uniform.shape) != (N, len(event_intervals)):
+                    raise _lib.KsError("event reset draws must be (N, n_events)")
+                io.event_reset_uniform = event_reset_uniform.data_ptr()
         _lib.check(self._lib.ks_terminate_reset(self._handle, _lib.current_stream(), ctypes.byref(io)))
 
     def close(self) -> None:

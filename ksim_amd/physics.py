@@ -103,9 +103,29 @@ def _make_io(dm: DeviceModel, buffers: Mapping[str, torch.Tensor | None], subste
 
 def control_step(dm: DeviceModel, buffers: Mapping[str, torch.Tensor | None], *, substeps: int,
                  actuator_period: int = 1, actuator_type: int = _lib_dyn.KS_ACT_POSITION,
-                 action_scale: float = 1.0) -> None:
-    """One control step of every env, in place on ``qpos, qvel, qacc_warmstart, time, last_ctrl``."""
+                 action_scale: float = 1.0, events=None) -> None:
+    """One control step of every env, in place on ``qpos, qvel, qacc_warmstart, time, last_ctrl``.
+
+    `events`: (descs, state (n_events, N), uniform (substeps, N, n_events, 3) or None, KsRng) for velocity events."""
     io = _make_io(dm, buffers, substeps, actuator_period, actuator_type, action_scale)
+    if events is not None:
+        descs, state, uniform, rng = events
+        N = int(io.N)
+        if len(descs) > _lib_dyn._T.KS_MAX_EVENTS:
+            raise _lib.KsError(f"at most {_lib_dyn._T.KS_MAX_EVENTS} events")
+        _lib.require_cuda(state, dtype=torch.float32)
+        if tuple(state.shape) != (len(descs), N):
+            raise _lib.KsError(f"event state: expected shape {(len(descs), N)}, got {tuple(state.shape)}")
+        if uniform is not None:
+            _lib.require_cuda(uniform, dtype=torch.float32)
+            if tuple(uniform.shape) != (substeps, N, len(descs), 3):
+                raise _lib.KsError(f"event draws: expected shape {(substeps, N, len(descs), 3)}, got {tuple(uniform.shape)}")
+        io.n_events = len(descs)
+        for j, dsc in enumerate(descs):
+            io.events[j] = dsc
+        io.event_state, io.event_uniform = state.data_ptr(), _lib.ptr(uniform).value
+        if rng is not None:
+            io.event_rng = rng
     _lib.check(dm._lib.ks_step(dm.handle, _lib.current_stream(), ctypes.byref(io)))
 
 

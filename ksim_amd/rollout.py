@@ -98,13 +98,16 @@ class Rollout:
         # the step kernel also writes ctrl / xpos / xquat of the post-step data into the transition slot
         c.engine.step(self.action[t], c.physics_model, ps, level, env.seed + env.step, env.randomization_dict,
                       noise=noise.get("engine"), record=dict(ctrl=self.ctrl[t], xpos=self.xpos[t], xquat=self.xquat[t]),
-                      want_cvel=T.SRC_CVEL in c.terms.sources_used)
+                      want_cvel=T.SRC_CVEL in c.terms.sources_used, step=step, step_base=step_base, event_seed=env.seed)
+        ev_buf = ps.event_states.get("_buffer") if ps.event_states else None
         st = dict(qpos=d.qpos, qvel=d.qvel, qacc_warmstart=d.qacc_warmstart, time=d.time, last_ctrl=ps.last_ctrl)
         c.terms.terminate_reset(st, level=level, components=self.components[t][: c.terms.n_terms] if c.terms.n_terms else None,
                                 done=self.done[t], success=self.success[t], traj_qpos=self.qpos[t],
                                 traj_qvel=self.qvel[t], traj_time=self.timestep[t], reset_mask=self.reset_mask,
                                 episode_length=env.episode_length, reset_uniform=noise.get("reset_uniform"),
-                                seed=env.seed, step=step, step_base=step_base)
+                                seed=env.seed, step=step, step_base=step_base, event_state=ev_buf,
+                                event_intervals=[ev.interval_range for ev in c.engine.events.values()],
+                                event_reset_uniform=noise.get("event_reset_uniform"))
         # refresh the derived fields and the warm start of the reset envs (engine.py:213)
         c.engine.forward(c.physics_model, ps, self.reset_mask, env.randomization_dict)
         if not _relative_step:

@@ -188,14 +188,14 @@ class Oracle:
         return (self.Data * N)()
 
     def ctrl_step_batch(self, block, S, actuator_period, action, last_ctrl, latency, zero_offset, kp, kd, ctrl_clip,
-                        nthreads=1):
+                        nthreads=1, qvel_impulse=None):
         N = len(block)
         dt = self.dtype
         c = lambda x: None if x is None else np.ascontiguousarray(x, dtype=dt)  # noqa: E731
-        action, latency, zero_offset, kp, kd, ctrl_clip = map(c, (action, latency, zero_offset, kp, kd, ctrl_clip))
+        action, latency, zero_offset, kp, kd, ctrl_clip, qvel_impulse = map(c, (action, latency, zero_offset, kp, kd, ctrl_clip, qvel_impulse))
         assert last_ctrl.dtype == dt and last_ctrl.flags.c_contiguous
         p = lambda x: None if x is None else x.ctypes.data_as(ctypes.c_void_p)  # noqa: E731
         f = self.fn("ksor_ctrl_step_batch")
-        f.argtypes = [ctypes.c_void_p, c_int, c_int, c_int, ctypes.c_void_p] + [ctypes.c_void_p] * 7 + [c_int]
+        f.argtypes = [ctypes.c_void_p, c_int, c_int, c_int, ctypes.c_void_p] + [ctypes.c_void_p] * 7 + [c_int, ctypes.c_void_p]
         f(ctypes.byref(self.model), N, S, actuator_period, ctypes.byref(block), p(action), p(last_ctrl), p(latency),
-          p(zero_offset), p(kp), p(kd), p(ctrl_clip), nthreads)
+          p(zero_offset), p(kp), p(kd), p(ctrl_clip), nthreads, p(qvel_impulse))

@@ -664,7 +664,8 @@ void FN(ksor_step)(const KsorModel* m, Data* d) {
 void FN(ksor_ctrl_step_batch)(const KsorModel* m, int N, int S, int actuator_period, Data* data /*N*/,
                               const REAL* action /*N,nu*/, REAL* last_ctrl /*N,nu*/, const REAL* latency /*N*/,
                               const REAL* zero_offset /*N,nu or NULL*/, const REAL* kp /*N,nu*/,
-                              const REAL* kd /*N,nu*/, const REAL* ctrl_clip /*nu*/, int nthreads) {
+                              const REAL* kd /*N,nu*/, const REAL* ctrl_clip /*nu*/, int nthreads,
+                              const REAL* qvel_impulse /*S,N,nv or NULL: events, ksim/engine.py:322-333*/) {
   const int nu = m->nu;
   const int rq = (m->nb > 1 && m->body_jtype[1] == KSOR_JNT_FREE) ? 7 : 0;
   const int rv = rq ? 6 : 0;
@@ -687,6 +688,8 @@ void FN(ksor_ctrl_step_batch)(const KsorModel* m, int N, int S, int actuator_per
         }
       }
       for (int u = 0; u < nu; ++u) d->ctrl[u] = torque[u];
+      if (qvel_impulse)
+        for (int j = 0; j < m->nv; ++j) d->qvel[j] += qvel_impulse[((size_t)s * N + e) * m->nv + j];
       FN(ksor_step)(m, d);
     }
     for (int u = 0; u < nu; ++u) last_ctrl[e * nu + u] = action[e * nu + u];

@@ -210,3 +210,30 @@ def scrub_action(action, clip_max=1e3):
     """rl.py:998-1001: NaN -> 0, then clip."""
     a = np.where(np.isnan(action), 0.0, action)
     return np.clip(a, -clip_max, clip_max)
+
+
+def velocity_event(kind, params, time_remaining, dt, u, level_scale, gravity=(0.0, 0.0, -9.81)):
+    """One physics substep of a velocity event for one env (ksim/events.py:58-237): returns (impulse on qvel[0:6],
+    new time remaining).  `u` = three U[0,1) draws (direction / sign / height, magnitude, next interval).
+    kind: "linear" (linvel, vel_range), "angular" (angvel, vel_range), "jump" (jump_height_range)."""
+    f32 = np.float32
+    left = f32(time_remaining) - f32(dt)  # events.py:77-78: float32 timestep
+    imp = np.zeros(6)
+    if left > 0.0:
+        return imp, float(left)
+    u0, u1, u2 = (float(x) for x in u)
+    if kind == "linear":  # events.py:153-171
+        theta = 2.0 * np.pi * u0
+        mag = (params["vel_range"][0] + u1 * (params["vel_range"][1] - params["vel_range"][0])) * params["linvel"]
+        imp[:3] = np.array([np.cos(theta), np.sin(theta), 0.0]) * mag * level_scale
+    elif kind == "angular":  # events.py:92-108: flipped when the Bernoulli(0.5) draw is true
+        mag = (params["vel_range"][0] + u1 * (params["vel_range"][1] - params["vel_range"][0])) * params["angvel"]
+        imp[5] = (-mag if u0 < 0.5 else mag) * level_scale
+    elif kind == "jump":  # events.py:204-231
+        lo, hi = params["jump_height_range"]
+        h = (lo + u0 * (hi - lo)) * level_scale
+        imp[:3] = np.sqrt(2.0 * -np.asarray(gravity, dtype=np.float64) * h)
+    else:
+        raise ValueError(kind)
+    lo, hi = params["interval_range"]
+    return imp, lo + u2 * (hi - lo)

@@ -231,3 +231,68 @@ def test_errors_are_reported():
                          substeps=4)  # empty batch is a no-op
     with pytest.raises(ValueError):
         km.ModelBuilder().add_body(0, (0, 0, 0), joint=None, mass=1.0, inertia=(1, 1, 1))
+
+
+def test_velocity_events_inside_the_substep_loop():
+    """Linear / angular push and jump events (ksim/events.py) fired from explicit draws: the fused step against
+    the oracle with the same impulses applied before each physics substep, and the timers bit for bit."""
+    from ksim_amd import events as kev, physics
+
+    m = MODELS["kbot"]()
+    dm = physics.DeviceModel(m)
+    N, S, T = 16, 4, 3
+    qpos, qvel = random_states(m, N, seed=41, vel_scale=0.1, joint_range=0.2)
+    rng = np.random.default_rng(42)
+    actions = rng.uniform(-0.3, 0.3, size=(T, N, m.nu))
+    kp, kd, clip = rng.uniform(20, 150, m.nu), rng.uniform(1, 3, m.nu), np.full(m.nu, 40.0)
+    evs = [kev.LinearPushEvent(linvel=1.0, vel_range=(0.2, 0.8), interval_range=(0.004, 0.03), scale=0.5),
+           kev.AngularPushEvent(angvel=2.0, vel_range=(0.0, 1.0), interval_range=(0.01, 0.05)),
+           kev.JumpEvent(jump_height_range=(0.02, 0.1), interval_range=(0.02, 0.06))]
+    kinds = [("linear", dict(linvel=1.0, vel_range=(0.2, 0.8), interval_range=(0.004, 0.03)), 0.5),
+             ("angular", dict(angvel=2.0, vel_range=(0.0, 1.0), interval_range=(0.01, 0.05)), 1.0),
+             ("jump", dict(jump_height_range=(0.02, 0.1), interval_range=(0.02, 0.06)), 1.0)]
+    u = rng.random(size=(T, S, N, 3, 3)).astype(np.float32)
+    left0 = rng.uniform(0.0, 0.03, size=(3, N)).astype(np.float32)
+    # oracle: per env, per substep: PD torque from the pre-event state, events, physics step (engine.py:290-335)
+    orc = Oracle(m.arrays())
+    datas = [orc.data(qpos[e], qvel[e]) for e in range(N)]
+    left = left0.astype(np.float64).copy()
+    last = np.zeros((N, m.nu))
+    fired = 0
+    for k in range(T):
+        for e, d in enumerate(datas):
+            for s in range(S):
+                c = oterms.latency_blend(float(s), 0.0, last[e], actions[k, e], np.zeros(m.nu, bool))
+                d.ctrl = oterms.position_actuator_torque(c, np.array(d.qpos[7:]), np.array(d.qvel[6:]), kp, kd, clip)
+                for j, (kind, prm, scale) in enumerate(kinds):
+                    imp, left[j, e] = oterms.velocity_event(kind, prm, left[j, e], m.dt, u[k, s, e, j], scale)
+                    left[j, e] = float(np.float32(left[j, e]))
+                    fired += bool(imp.any())
+                    for i in range(6):
+                        d.qvel[i] += imp[i]
+                orc.step(d)
+        last = actions[k].copy()
+    assert fired >= 20, "the draws did not fire enough events to test anything"
+    buf = dict(qpos=t32(qpos), qvel=t32(qvel), qacc_warmstart=zeros(N, m.nv), time=zeros(N), last_ctrl=zeros(N, m.nu),
+               kp=t32(kp), kd=t32(kd), ctrl_clip=t32(clip))
+    state = t32(left0)
+    descs = [ev.desc(1.0) for ev in evs]
+    for k in range(T):
+        buf["action"] = t32(actions[k])
+        physics.control_step(dm, buf, substeps=S, events=(descs, state, t32(u[k]), None))
+    for field in ("qpos", "qvel"):
+        want = np.array([np.array(getattr(d, field)) for d in datas])
+        assert rel_err(buf[field].cpu().numpy(), want).max() <= TEN_STEP_TOL, field
+    np.testing.assert_allclose(state.cpu().numpy(), left, rtol=0, atol=1e-6)  # timers: float32 arithmetic on both sides
+    # without draws the kernel's own counter-based stream is used: reproducible, and the timers stay inside their ranges
+    outs = []
+    for _ in range(2):
+        b2 = {k: v.clone() for k, v in buf.items()}
+        st = t32(left0)
+        from ksim_amd import _lib_terms as T_
+        for k in range(20):
+            physics.control_step(dm, b2, substeps=S, events=(descs, st, None, T_.KsRng(7, k, None)))
+        outs.append((b2["qvel"].clone(), st.clone()))
+    assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])
+    hi = torch.tensor([0.03, 0.05, 0.06], device=DEV)[:, None]
+    assert (outs[0][1] <= hi).all() and (outs[0][1] > -0.006).all()

@@ -17,7 +17,7 @@ def t32(a):
     return torch.tensor(np.asarray(a), dtype=torch.float32, device=DEV).contiguous()
 
 
-def build(N, T, seed=0, min_height=0.9):
+def build(N, T, seed=0, min_height=0.9, events=None):
     from ksim_amd import actuators, engine, model as km, observation as ob, physics, randomization as rnd, resets as rs
     from ksim_amd import rewards as rw, terminations as tm
     from ksim_amd.env_terms import EnvTerms
@@ -32,7 +32,7 @@ def build(N, T, seed=0, min_height=0.9):
     act = actuators.PositionActuators(kps=tuple(kps), kds=tuple(kds), ctrl_clip=tuple(clip))
     resets = [rs.RandomJointPositionReset(scale=0.1, scale_by_curriculum=False)]
     cfg = engine.EngineConfig(dt=0.005, ctrl_dt=0.02)
-    eng = engine.get_physics_engine("hip", resets, {}, act, cfg)
+    eng = engine.get_physics_engine("hip", resets, events or {}, act, cfg)
     observations = {"jp": ob.JointPositionObservation(noise=0.01), "jv": ob.JointVelocityObservation(noise=0.01),
                     "g": ob.ProjectedGravityObservation(noise=0.01),
                     "w": ob.BaseAngularVelocityObservation(in_robot_frame=True, noise=0.01),
@@ -171,13 +171,21 @@ def test_long_rollout_with_resets_stays_finite_and_reproducible():
     assert (outs[0][0][:, 2] > 0.5).all()  # every env sits above the termination height after its reset
 
 
-def test_graph_replay_equals_eager_rollout():
+def _push_events():
+    from ksim_amd import events as kev
+    return {"push": kev.LinearPushEvent(linvel=0.5, interval_range=(0.05, 0.3)),
+            "spin": kev.AngularPushEvent(angvel=0.5, interval_range=(0.1, 0.4)),
+            "jump": kev.JumpEvent(jump_height_range=(0.01, 0.05), interval_range=(0.2, 0.6))}
+
+
+@pytest.mark.parametrize("with_events", [False, True])
+def test_graph_replay_equals_eager_rollout(with_events):
     """A captured rollout graph, replayed several times with eager work and synchronisations in between, gives
     the same bits as the eager loop on every replay (same Philox keys: device step counter + baked step)."""
     N, T, iters = 192, 8, 10
     runs = []
     for use_graph in (False, True):
-        m, c, rnd_, _, ro, EnvState = build(N, T, seed=5, min_height=0.8)
+        m, c, rnd_, _, ro, EnvState = build(N, T, seed=5, min_height=0.8, events=_push_events() if with_events else None)
         ps = c.engine.reset(c.physics_model, 1.0, 3, N, rnd_)
         env = EnvState(ps, rnd_, torch.zeros(N, 2, device=DEV), None, seed=123)
         snaps = []
@@ -194,3 +202,55 @@ def test_graph_replay_equals_eager_rollout():
     for it, (a, b) in enumerate(zip(*runs)):
         for x, y, name in zip(a, b, ("qpos", "action", "done", "reward", "state", "episode_length")):
             assert torch.equal(x, y), f"replay {it}: {name} differs from the eager rollout"
+
+
+def test_events_in_the_rollout_fire_and_restart_with_the_episode():
+    """Event timers through the environment loop: explicit draws, one control step; envs that continue carry
+    the kernel's timers (fired ones re-armed from the draw), envs that finish get fresh timers from the reset draw
+    (ksim/engine.py:226-232), and the pushes change the state relative to a run without events."""
+    N, T = 12, 2
+    evs = _push_events()
+    m, c, rnd_, _, ro, EnvState = build(N, T, seed=5, events=evs)
+    _, c0, rnd0, _, ro0, _ = build(N, T, seed=5)
+    rng = np.random.default_rng(8)
+    u0 = t32(rng.uniform(-1, 1, (N, m.nq + 1)))
+    ps = c.engine.reset(c.physics_model, 1.0, 0, N, rnd_, reset_uniform=u0)
+    ps0 = c0.engine.reset(c0.physics_model, 1.0, 0, N, rnd0, reset_uniform=u0)
+    names = list(evs)
+    assert set(ps.event_states) == set(names) | {"_buffer"}
+    for j, n in enumerate(names):  # initial timers inside the interval range (events.py get_initial_event_state)
+        lo, hi = evs[n].interval_range
+        assert ((ps.event_states[n] >= lo) & (ps.event_states[n] <= hi)).all()
+    low = np.arange(N) % 3 == 0
+    for p in (ps, ps0):
+        p.data.qpos[torch.from_numpy(low).to(DEV), 2] = 0.87
+    left0 = rng.uniform(0.0, 0.05, (len(names), N)).astype(np.float32)  # some timers run out within the 4 substeps
+    ps.event_states["_buffer"].copy_(t32(left0))
+    K = c.terms.obs_dim
+    noise = dict(obs_normal=rng.normal(size=(N, K)), obs_uniform=rng.random((N, K)), action_normal=rng.normal(size=(N, m.nu)),
+                 reset_uniform=rng.uniform(-1, 1, (N, m.nq + 1)), event_reset_uniform=rng.random((N, len(names))))
+    ev_u = rng.random((4, N, len(names), 3)).astype(np.float32)
+    noise_t = {k: t32(v) for k, v in noise.items()}
+    env = EnvState(ps, rnd_, torch.zeros(N, 2, device=DEV), None, seed=1)
+    env0 = EnvState(ps0, rnd0, torch.zeros(N, 2, device=DEV), None, seed=1)
+    ro.step_engine(env, 0, 1.0, dict(noise_t, engine=dict(event_uniform=t32(ev_u))))
+    ro0.step_engine(env0, 0, 1.0, {k: v for k, v in noise_t.items() if k != "event_reset_uniform"})
+    done = ro.done[0].cpu().numpy().astype(bool)
+    assert np.array_equal(done, low)
+    kinds = {"push": ("linear", dict(linvel=0.5, vel_range=(0.0, 1.0), interval_range=(0.05, 0.3))),
+             "spin": ("angular", dict(angvel=0.5, vel_range=(0.0, 1.0), interval_range=(0.1, 0.4))),
+             "jump": ("jump", dict(jump_height_range=(0.01, 0.05), interval_range=(0.2, 0.6)))}
+    want = left0.astype(np.float64).copy()
+    fired = np.zeros(N, bool)
+    for j, n in enumerate(names):
+        for e in range(N):
+            for s in range(4):
+                imp, want[j, e] = ot.velocity_event(kinds[n][0], kinds[n][1], want[j, e], m.dt, ev_u[s, e, j], 1.0)
+                want[j, e] = float(np.float32(want[j, e]))
+                fired[e] |= bool(imp.any())
+        lo, hi = evs[n].interval_range
+        want[j, done] = lo + noise["event_reset_uniform"][done, j] * (hi - lo)
+    np.testing.assert_allclose(ps.event_states["_buffer"].cpu().numpy(), want, rtol=0, atol=1e-6)
+    assert torch.equal(ps.event_states["push"], ps.event_states["_buffer"][0])  # named views of the one buffer
+    moved = (ro.qvel[0] - ro0.qvel[0]).abs().amax(dim=1).cpu().numpy() > 1e-4
+    assert fired.any() and np.array_equal(moved, fired), "exactly the envs whose events fired differ from the run without events"

@@ -114,3 +114,37 @@ def test_model_builder_rules_and_constants():
     h = km.humanoid_model()
     assert h.max_depth == 6 and km.humanoid_model(seed=1).body_mass[3] != h.body_mass[3]
     assert np.allclose(km.capsule_inertia(1.0, 1e-9, 1.0)[:2], 1.0 / 12.0, rtol=1e-6)  # thin rod limit
+
+
+def test_scales_and_event_descriptors():
+    """Curriculum scales (ksim/scales.py) and the event records the step kernel reads (ksim/events.py)."""
+    from ksim_amd import _lib_terms as T, events as kev, scales as sc
+
+    assert sc.convert_to_scale(2).get_scale(0.3) == 2.0
+    assert sc.LinearScale.from_endpoints(0.5, 1.5).get_scale(0.5) == pytest.approx(1.0)
+    assert sc.QuadraticScale(scale=2.0, bias=1.0).get_scale(0.5) == pytest.approx(1.5)
+    assert sc.SquareRootScale(scale=2.0).get_scale(0.25) == pytest.approx(1.0)
+    nz = sc.NonZeroScale(scale=3.0, bias=0.5)
+    assert (nz.get_scale(0.0), nz.get_scale(0.1)) == (0.5, 3.0)
+    for bad in (lambda: sc.ConstantScale(scale=-1.0), lambda: sc.LinearScale(scale=-2.0, bias=1.0),
+                lambda: sc.LinearScale(scale=1.0, bias=-0.1), lambda: sc.convert_to_scale("x")):
+        with pytest.raises(ValueError):
+            bad()
+    d = kev.LinearPushEvent(linvel=2.0, vel_range=(0.1, 0.9), interval_range=(1.0, 3.0),
+                            scale=sc.LinearScale(scale=1.0, bias=0.5)).desc(0.25)
+    assert (d.kind, d.mag, d.lo, d.hi, d.interval_lo, d.interval_hi) == (T.EVENT_LINEAR_PUSH, 2.0, pytest.approx(0.1),
+                                                                        pytest.approx(0.9), 1.0, 3.0)
+    assert d.level_scale == pytest.approx(0.75)
+    j = kev.JumpEvent(jump_height_range=(0.1, 0.2), interval_range=(2.0, 4.0)).desc(1.0)
+    assert (j.kind, j.lo, j.hi, j.level_scale) == (T.EVENT_JUMP, pytest.approx(0.1), pytest.approx(0.2), 1.0)
+    a = kev.AngularPushEvent(angvel=1.5, interval_range=(0.5, 1.0)).desc(1.0)
+    assert (a.kind, a.mag, a.lo, a.hi) == (T.EVENT_ANGULAR_PUSH, 1.5, 0.0, 1.0)
+    # the engine refuses events that are not compiled into the step kernel, and more than the kernel holds
+    from ksim_amd import actuators, engine
+    act = actuators.TorqueActuators()
+    cfg = engine.EngineConfig(dt=0.005, ctrl_dt=0.02)
+    with pytest.raises(NotImplementedError):
+        engine.get_physics_engine("hip", [], {"x": object()}, act, cfg)
+    many = {f"e{i}": kev.JumpEvent(interval_range=(1.0, 2.0)) for i in range(T.KS_MAX_EVENTS + 1)}
+    with pytest.raises(ValueError):
+        engine.get_physics_engine("hip", [], many, act, cfg)

@@ -96,3 +96,24 @@ def test_amp_reward_closed_form():
     x = np.linspace(-4, 6, 101)
     np.testing.assert_allclose(terms.amp_reward(x), terms.amp_reward(2.0 - x))  # symmetric about logit 1
     assert (terms.amp_reward(x) >= 0).all() and terms.amp_reward(x).max() == 1.0
+
+
+def test_velocity_events_closed_forms():
+    # timer above dt: nothing happens, the timer runs down by the float32 timestep (events.py:77-78)
+    imp, left = terms.velocity_event("linear", dict(linvel=1.0, vel_range=(0.0, 1.0), interval_range=(1.0, 2.0)), 0.5, 0.005, (0.1, 0.2, 0.3), 1.0)
+    assert not imp.any() and left == float(np.float32(0.5) - np.float32(0.005))
+    # firing: direction theta = 2 pi u0, magnitude linear in u1, next interval linear in u2, curriculum scale on top
+    p = dict(linvel=2.0, vel_range=(0.5, 1.5), interval_range=(1.0, 3.0))
+    imp, left = terms.velocity_event("linear", p, 0.004, 0.005, (0.25, 0.5, 0.75), 0.5)
+    np.testing.assert_allclose(imp, [0.0, 2.0 * 1.0 * 0.5, 0.0, 0.0, 0.0, 0.0], atol=1e-15)   # theta = pi/2
+    assert left == 2.5
+    # angular push acts on qvel[5] only and is flipped when the Bernoulli(0.5) draw comes out true (u0 < 0.5)
+    pa = dict(angvel=3.0, vel_range=(0.0, 1.0), interval_range=(0.0, 1.0))
+    assert terms.velocity_event("angular", pa, 0.0, 0.005, (0.4, 1.0, 0.0), 1.0)[0][5] == -3.0
+    assert terms.velocity_event("angular", pa, 0.0, 0.005, (0.6, 1.0, 0.0), 1.0)[0][5] == 3.0
+    # jump: the impulse that reaches the height, v = sqrt(2 g h)
+    pj = dict(jump_height_range=(0.1, 0.3), interval_range=(2.0, 2.0))
+    imp, left = terms.velocity_event("jump", pj, 0.001, 0.005, (0.5, 0.0, 0.9), 1.0)
+    np.testing.assert_allclose(imp[:3], [0.0, 0.0, np.sqrt(2 * 9.81 * 0.2)])
+    v = imp[2]
+    assert abs(v * v / (2 * 9.81) - 0.2) < 1e-12 and left == 2.0
