@@ -153,15 +153,30 @@ typedef struct KsRng {
  *   angular push: qvel[5]   += +-(lo + u1 (hi - lo)) * mag * level_scale, minus when u0 < 0.5
  *   jump        : qvel[0:3] += sqrt(2 * -gravity * (lo + u0 (hi - lo)) * level_scale)
  *   all         : time remaining = interval_lo + u2 (interval_hi - interval_lo)
- * The continuous-force event (ForcePushEvent, events.py:240-365) is not built. */
+ * The force push (ForcePushEvent, events.py:240-365) holds a Cartesian force and torque on one body, applied at
+ * its centre of mass in the world frame like MuJoCo's xfrc_applied, for a drawn duration.  Per env it carries,
+ * besides the time remaining, KS_EVENT_FORCE_STATE floats: [force duration left, force(3), torque(3), unused].
+ * Every substep: both timers lose dt; the stored wrench is multiplied by level_scale (events.py:296 rescales the
+ * carried value itself); while the duration is positive the body receives stored * level_scale (events.py:297-299);
+ * when the interval runs out a new wrench is drawn (events.py:320-358):
+ *   force  = dir(u0,u1,u2) * s * mag,  torque = dir(u4,u5,u6) * s * mag2,  dir(.) = unit vector of 2u - 1,
+ *   s = lo + u3 (hi - lo);  case floor(3 u7): 0 force only, 1 torque only, 2 both;
+ *   time remaining = interval_lo + u8 (interval_hi - interval_lo);  duration = duration_lo + u9 (duration_hi - duration_lo).
+ * As in the reference, each force push first clears the applied forces of all bodies, so with several of them only
+ * the last one in the list acts. */
 #define KS_MAX_EVENTS 4
-enum { KS_EVENT_LINEAR_PUSH = 0, KS_EVENT_ANGULAR_PUSH = 1, KS_EVENT_JUMP = 2 };
+#define KS_EVENT_DRAWS 12      /* uniforms per (substep, env, event) in an explicit draw buffer */
+#define KS_EVENT_FORCE_STATE 8 /* floats per (event, env) of force-push state */
+enum { KS_EVENT_LINEAR_PUSH = 0, KS_EVENT_ANGULAR_PUSH = 1, KS_EVENT_JUMP = 2, KS_EVENT_FORCE_PUSH = 3 };
 typedef struct KsEventDesc {
   int32_t kind;
-  float mag;          /* linvel | angvel | unused */
-  float lo, hi;       /* vel_range | jump_height_range */
+  float mag;          /* linvel | angvel | unused | max_force */
+  float lo, hi;       /* vel_range | jump_height_range | force_range */
   float interval_lo, interval_hi;
   float level_scale;  /* event.scale.get_scale(curriculum_level) */
+  float mag2;         /* force push: max_torque */
+  float duration_lo, duration_hi; /* force push: duration_range */
+  int32_t body;       /* force push: body index (0 = world) */
 } KsEventDesc;
 
 /* ------------------------------------------------------------------ control step / forward
@@ -230,8 +245,9 @@ typedef struct KsStepIO {
   int32_t n_events;
   KsEventDesc events[KS_MAX_EVENTS];
   float* event_state;          /* (n_events, N) time remaining, in/out */
-  const float* event_uniform;  /* (substeps, N, n_events, 3) U[0,1) draws, nullable -> Philox */
+  const float* event_uniform;  /* (substeps, N, n_events, KS_EVENT_DRAWS) U[0,1) draws, nullable -> Philox */
   KsRng event_rng;
+  float* event_force;          /* (n_events, N, KS_EVENT_FORCE_STATE) in/out; required when a force push is listed */
 } KsStepIO;
 
 int ks_step(const KsModel* model, ks_stream_t stream, const KsStepIO* io /*host*/);
@@ -329,6 +345,7 @@ typedef struct KsTerminateIO {
   float event_interval[KS_MAX_EVENTS][2];
   float* event_state;               /* (n_events, N), nullable when n_events == 0 */
   const float* event_reset_uniform; /* (N, n_events) U[0,1) draws, nullable -> Philox */
+  float* event_force;               /* (n_events, N, KS_EVENT_FORCE_STATE), nullable: zeroed for the reset envs */
 } KsTerminateIO;
 int ks_terminate_reset(const KsTerms* terms, ks_stream_t stream, const KsTerminateIO* io /*host*/);
 

@@ -41,12 +41,14 @@ class KsRng(ctypes.Structure):
 
 
 KS_MAX_EVENTS = 4
-EVENT_LINEAR_PUSH, EVENT_ANGULAR_PUSH, EVENT_JUMP = range(3)
+KS_EVENT_DRAWS, KS_EVENT_FORCE_STATE = 12, 8
+EVENT_LINEAR_PUSH, EVENT_ANGULAR_PUSH, EVENT_JUMP, EVENT_FORCE_PUSH = range(4)
 
 
 class KsEventDesc(ctypes.Structure):
     _fields_ = [("kind", c_int32), ("mag", c_float), ("lo", c_float), ("hi", c_float), ("interval_lo", c_float),
-                ("interval_hi", c_float), ("level_scale", c_float)]
+                ("interval_hi", c_float), ("level_scale", c_float), ("mag2", c_float), ("duration_lo", c_float),
+                ("duration_hi", c_float), ("body", c_int32)]
 
 
 class KsObserveIO(ctypes.Structure):
@@ -62,7 +64,7 @@ class KsTerminateIO(ctypes.Structure):
                 ("traj_time", c_void_p), ("reset_mask", c_void_p), ("episode_length", c_void_p),
                 ("reset_uniform", c_void_p), ("rng", KsRng), ("apply_reset", c_int32), ("n_events", c_int32),
                 ("event_interval", (c_float * 2) * KS_MAX_EVENTS), ("event_state", c_void_p),
-                ("event_reset_uniform", c_void_p)]
+                ("event_reset_uniform", c_void_p), ("event_force", c_void_p)]
 
 
 class KsMlpDesc(ctypes.Structure):

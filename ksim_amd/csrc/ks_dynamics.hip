@@ -367,13 +367,13 @@ void step_kernel(StepArgs a) {
       const uint64_t ev_step = a.event_rng.step + (a.event_rng.step_base ? *a.event_rng.step_base : 0ull);
 #pragma unroll
       for (int e = 0; e < KS_MAX_EVENTS; ++e) {
-        if (e < a.n_events) {
+        if (e < a.n_events && a.events[e].kind != KS_EVENT_FORCE_PUSH) {
           const KsEventDesc ev = a.events[e];
           float left = ev_left[e] - m.dt;
           if (left <= 0.f) {  // wave-uniform
             float u0, u1, u2;
             if (a.event_uniform) {
-              const float* u = a.event_uniform + (((int64_t)sub * a.N + env) * a.n_events + e) * 3;
+              const float* u = a.event_uniform + (((int64_t)sub * a.N + env) * a.n_events + e) * KS_EVENT_DRAWS;
               u0 = u[0]; u1 = u[1]; u2 = u[2];
             } else {
               const Philox4 r = draw(a.event_rng.seed, ev_step, kRngEvent, (uint64_t)env, (uint32_t)(sub * KS_MAX_EVENTS + e));
@@ -500,7 +500,7 @@ void step_kernel(StepArgs a) {
         } else {
           const Mat3 Rb = q2mat({l.xquat[4 * d_body], l.xquat[4 * d_body + 1], l.xquat[4 * d_body + 2], l.xquat[4 * d_body + 3]});
           const float* R = Rb.m;
-          const V3 ax = {R[d_k - 3], R[3 + d_k - 3], R[6 + d_k - 3]};
+          const V3 ax = d_k == 3 ? V3{R[0], R[3], R[6]} : d_k == 4 ? V3{R[1], R[4], R[7]} : V3{R[2], R[5], R[8]};
           my_cdof = {ax, cross(ax, off)};
         }
       } else {
@@ -560,9 +560,65 @@ void step_kernel(StepArgs a) {
           }
         }
       }
+      Sp cf = inert_mul(ci, acc) + cross_force(v, inert_mul(ci, v));
+      // ---- force pushes (ksim/events.py:240-365): a wrench held on one body enters the Newton-Euler pass as an
+      // external force on that body, so the subtree sums and the projection on the motion axes below turn it into
+      // the generalised force J^T f.  Lane 0 owns the state in memory; the other lanes get it by broadcast.
+      if (!FWD && a.n_force_events > 0) {
+        const uint64_t ev_step = a.event_rng.step + (a.event_rng.step_base ? *a.event_rng.step_base : 0ull);
+        Sp ext = {{0.f, 0.f, 0.f}, {0.f, 0.f, 0.f}};
+        for (int e = 0; e < a.n_events; ++e) {
+          if (a.events[e].kind != KS_EVENT_FORCE_PUSH) continue;
+          const KsEventDesc ev = a.events[e];
+          float* st = a.event_force + ((int64_t)e * a.N + env) * KS_EVENT_FORCE_STATE;
+          float* tleft = a.event_state + (int64_t)e * a.N + env;
+          float s7[7];
+#pragma unroll
+          for (int k = 0; k < 7; ++k) s7[k] = lane_bcast(lane == 0 ? st[k] : 0.f, 0);
+          float dur = s7[0] - m.dt, left = lane_bcast(lane == 0 ? *tleft : 0.f, 0) - m.dt;
+#pragma unroll
+          for (int k = 0; k < 6; ++k) s7[1 + k] *= ev.level_scale;   // events.py:296: the carried wrench itself is rescaled
+          const bool on = dur > 0.f && lane == ev.body;                // events.py:297-299, 302-307
+          const V3 f = {s7[1] * ev.level_scale, s7[2] * ev.level_scale, s7[3] * ev.level_scale};
+          const V3 tq = {s7[4] * ev.level_scale, s7[5] * ev.level_scale, s7[6] * ev.level_scale};
+          const V3 mom = tq + cross(xipos - com, f);                    // moment about the centre of mass of the tree
+          ext = {{on ? mom.x : 0.f, on ? mom.y : 0.f, on ? mom.z : 0.f}, {on ? f.x : 0.f, on ? f.y : 0.f, on ? f.z : 0.f}};
+          if (left <= 0.f) {  // wave-uniform: a new wrench (events.py:320-358)
+            float u[10];
+            if (a.event_uniform) {
+              const float* up = a.event_uniform + (((int64_t)sub * a.N + env) * a.n_events + e) * KS_EVENT_DRAWS;
+#pragma unroll
+              for (int k = 0; k < 10; ++k) u[k] = up[k];
+            } else {
+#pragma unroll
+              for (int q = 0; q < 3; ++q) {
+                const Philox4 r = draw(a.event_rng.seed, ev_step, kRngEvent, (uint64_t)env, (uint32_t)((sub * KS_MAX_EVENTS + e) * 4 + 1 + q));
+                u[4 * q] = u01(r.x); u[4 * q + 1] = u01(r.y);
+                if (q < 2) { u[4 * q + 2] = u01(r.z); u[4 * q + 3] = u01(r.w); }
+              }
+            }
+            const V3 d0 = {2.f * u[0] - 1.f, 2.f * u[1] - 1.f, 2.f * u[2] - 1.f}, d1 = {2.f * u[4] - 1.f, 2.f * u[5] - 1.f, 2.f * u[6] - 1.f};
+            const float sc = ev.lo + u[3] * (ev.hi - ev.lo);
+            const float kf = sc * ev.mag / sqrtf(dot(d0, d0)), kt = sc * ev.mag2 / sqrtf(dot(d1, d1));
+            const int which = min(2, (int)(3.f * u[7]));
+            const float wf = which == 1 ? 0.f : kf, wt = which == 0 ? 0.f : kt;
+            s7[1] = d0.x * wf; s7[2] = d0.y * wf; s7[3] = d0.z * wf;
+            s7[4] = d1.x * wt; s7[5] = d1.y * wt; s7[6] = d1.z * wt;
+            left = ev.interval_lo + u[8] * (ev.interval_hi - ev.interval_lo);
+            dur = ev.duration_lo + u[9] * (ev.duration_hi - ev.duration_lo);
+          }
+          if (lane == 0) {
+            *tleft = left;
+            st[0] = dur;
+#pragma unroll
+            for (int k = 1; k < 7; ++k) st[k] = s7[k];
+          }
+        }
+        cf = {cf.a - ext.a, cf.l - ext.l};
+      }
       if (is_body) {
         st6(l.cvel + 6 * lane, v);
-        st6(l.cfrc + 6 * lane, inert_mul(ci, acc) + cross_force(v, inert_mul(ci, v)));
+        st6(l.cfrc + 6 * lane, cf);
       }
     }
     KS_SYNC();
@@ -901,7 +957,9 @@ void step_kernel(StepArgs a) {
   if (a.traj_xpos) for (int i = lane; i < nb * 3; i += 64) a.traj_xpos[env * nb * 3 + i] = l.xpos[i];
   if (a.traj_xquat) for (int i = lane; i < nb * 4; i += 64) a.traj_xquat[env * nb * 4 + i] = l.xquat[i];
   if (!FWD && lane == 0)
-    for (int e = 0; e < a.n_events; ++e) a.event_state[(int64_t)e * a.N + env] = ev_left[e];
+#pragma unroll
+    for (int e = 0; e < KS_MAX_EVENTS; ++e)  // the force pushes keep their timers in memory
+      if (e < a.n_events && a.events[e].kind != KS_EVENT_FORCE_PUSH) a.event_state[(int64_t)e * a.N + env] = ev_left[e];
   if (a.solver_niter && lane == 0) a.solver_niter[env] = niter_out;
   if (a.nefc && lane == 0) a.nefc[env] = nefc_out;
 }
@@ -1101,10 +1159,19 @@ static int launch_step(const KsModel* km, ks_stream_t stream, const KsStepIO* io
     if (io->n_events < 0 || io->n_events > KS_MAX_EVENTS) return fail(KS_ELIMIT, "ks_step: %d events (0..%d)", io->n_events, KS_MAX_EVENTS);
     if (io->n_events > 0) {
       if (!io->event_state) return fail(KS_EINVAL, "ks_step: events need event_state");
-      if (m.nv < 6 || m.body_jtype[1] != kJntFree) return fail(KS_EINVAL, "ks_step: events push a floating base");
-      for (int e = 0; e < io->n_events; ++e)
-        if (io->events[e].kind < KS_EVENT_LINEAR_PUSH || io->events[e].kind > KS_EVENT_JUMP)
-          return fail(KS_EINVAL, "ks_step: event %d: unknown kind %d", e, io->events[e].kind);
+      for (int e = 0; e < io->n_events; ++e) {
+        const KsEventDesc& ev = io->events[e];
+        if (ev.kind < KS_EVENT_LINEAR_PUSH || ev.kind > KS_EVENT_FORCE_PUSH)
+          return fail(KS_EINVAL, "ks_step: event %d: unknown kind %d", e, ev.kind);
+        if (ev.kind == KS_EVENT_FORCE_PUSH) {
+          if (ev.body < 1 || ev.body >= m.nb) return fail(KS_EINVAL, "ks_step: event %d: body %d outside 1..%d", e, ev.body, m.nb - 1);
+          if (!io->event_force) return fail(KS_EINVAL, "ks_step: a force push needs event_force");
+          ++a.n_force_events;
+        } else if (m.nv < 6 || m.body_jtype[1] != kJntFree) {
+          return fail(KS_EINVAL, "ks_step: velocity events push a floating base");
+        }
+      }
+      a.event_force = io->event_force;
       a.n_events = io->n_events;
       for (int e = 0; e < io->n_events; ++e) a.events[e] = io->events[e];
       a.event_state = io->event_state; a.event_uniform = io->event_uniform; a.event_rng = io->event_rng;

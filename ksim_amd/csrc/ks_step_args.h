@@ -28,6 +28,8 @@ struct StepArgs {
   float* event_state;
   const float* event_uniform;
   KsRng event_rng;
+  float* event_force;
+  int n_force_events;
 };
 
 }  // namespace ks

@@ -96,6 +96,7 @@ struct TerminateArgs {
   float event_interval[KS_MAX_EVENTS][2];
   float* event_state;
   const float* event_reset_uniform;
+  float* event_force;
 };
 
 // A 256-thread workgroup owns kTermEnvs consecutive envs.  The state rows of those envs are contiguous in memory,
@@ -176,6 +177,8 @@ __global__ __launch_bounds__(256) void terminate_kernel(TerminateArgs a) {
         if (a.event_reset_uniform) u = a.event_reset_uniform[e * a.n_events + k];
         else u = u01(draw(a.rng.seed, a.rng.step + (a.rng.step_base ? *a.rng.step_base : 0ull), kRngEvent, (uint64_t)e, 0x10000u + k).x);
         a.event_state[(int64_t)k * a.N + e] = a.event_interval[k][0] + u * (a.event_interval[k][1] - a.event_interval[k][0]);
+        if (a.event_force)  // no force held at the start of an episode (events.py:360-365)
+          for (int j = 0; j < KS_EVENT_FORCE_STATE; ++j) a.event_force[((int64_t)k * a.N + e) * KS_EVENT_FORCE_STATE + j] = 0.f;
       }
   }
   __syncthreads();
@@ -426,7 +429,7 @@ extern "C" int ks_terminate_reset(const KsTerms* t, ks_stream_t stream, const Ks
   a.random_heading = d.random_heading; a.nonfinite_terminates = d.nonfinite_terminates;
   if (io->n_events < 0 || io->n_events > KS_MAX_EVENTS) return fail(KS_ELIMIT, "ks_terminate_reset: %d events (0..%d)", io->n_events, KS_MAX_EVENTS);
   if (io->n_events > 0 && !io->event_state) return fail(KS_EINVAL, "ks_terminate_reset: events need event_state");
-  a.n_events = io->n_events; a.event_state = io->event_state; a.event_reset_uniform = io->event_reset_uniform;
+  a.n_events = io->n_events; a.event_state = io->event_state; a.event_reset_uniform = io->event_reset_uniform; a.event_force = io->event_force;
   for (int k = 0; k < io->n_events; ++k) { a.event_interval[k][0] = io->event_interval[k][0]; a.event_interval[k][1] = io->event_interval[k][1]; }
   const int64_t grid = (io->N + kTermEnvs - 1) / kTermEnvs;
   if (grid > 0x7fffffff) return fail(KS_ELIMIT, "ks_terminate_reset: too many envs");

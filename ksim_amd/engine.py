@@ -130,7 +130,7 @@ class HipEngine(PhysicsEngine):
         events = dict(events or {})
         for name, ev in events.items():
             if not isinstance(ev, Event):
-                raise NotImplementedError(f"event {name!r} ({type(ev).__name__}) is not one of the compiled velocity events")
+                raise NotImplementedError(f"event {name!r} ({type(ev).__name__}) is not one of the compiled events")
         if len(events) > T.KS_MAX_EVENTS:
             raise ValueError(f"at most {T.KS_MAX_EVENTS} events")
         self.actuators, self.resets, self.events, self.data = actuators, tuple(resets), events, data
@@ -177,9 +177,18 @@ class HipEngine(PhysicsEngine):
         """One timer per event and env (engine.py:226-232); rows of one (n_events, N) buffer, which the kernels take."""
         if not self.events:
             return {}
+        from .events import ForcePushEvent  # noqa: PLC0415
         buf = torch.stack([ev.get_initial_event_state(N, gen, dev) for ev in self.events.values()]).contiguous()
         out = {name: buf[j] for j, name in enumerate(self.events)}
         out["_buffer"] = buf
+        if any(isinstance(ev, ForcePushEvent) for ev in self.events.values()):
+            # force pushes also carry (duration left, force, torque) per env, zero at the start (events.py:360-365);
+            # their state reads (time remaining, duration left, wrench) like the reference's tuple
+            force = torch.zeros(len(self.events), N, T.KS_EVENT_FORCE_STATE, dtype=torch.float32, device=dev)
+            out["_force_buffer"] = force
+            for j, (name, ev) in enumerate(self.events.items()):
+                if isinstance(ev, ForcePushEvent):
+                    out[name] = (buf[j], force[j, :, 0], force[j, :, 1:7])
         return out
 
     def event_args(self, physics_state: PhysicsState, curriculum_level, seed: int, step: int, step_base=None, uniform=None):
@@ -188,7 +197,7 @@ class HipEngine(PhysicsEngine):
             return None
         descs = [ev.desc(float(curriculum_level)) for ev in self.events.values()]
         rng = T.KsRng(int(seed) & (2**64 - 1), int(step) & (2**64 - 1), _lib.ptr(step_base).value)
-        return descs, physics_state.event_states["_buffer"], uniform, rng
+        return descs, physics_state.event_states["_buffer"], uniform, rng, physics_state.event_states.get("_force_buffer")
 
     def reset_where(self, physics_model, state: PhysicsState, mask, curriculum_level, seed: int, step: int,
                     randomization=None, reset_uniform=None) -> None:

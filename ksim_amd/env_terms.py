@@ -123,7 +123,7 @@ class EnvTerms:
     def terminate_reset(self, state: Mapping[str, torch.Tensor], *, level: float = 1.0, components=None, done=None,
                         success=None, traj_qpos=None, traj_qvel=None, traj_time=None, reset_mask=None,
                         episode_length=None, reset_uniform=None, seed: int = 0, step: int = 0, step_base=None,
-                        event_state=None, event_intervals=(), event_reset_uniform=None,
+                        event_state=None, event_intervals=(), event_reset_uniform=None, event_force=None,
                         apply_reset: bool = True) -> None:
         m = self.model
         qpos = state["qpos"]
@@ -160,6 +160,11 @@ class EnvTerms:
                 if tuple(event_reset_uniform.shape) != (N, len(event_intervals)):
                     raise _lib.KsError("event reset draws must be (N, n_events)")
                 io.event_reset_uniform = event_reset_uniform.data_ptr()
+            if event_force is not None:
+                _lib.require_cuda(event_force, dtype=torch.float32)
+                if tuple(event_force.shape) != (len(event_intervals), N, T.KS_EVENT_FORCE_STATE):
+                    raise _lib.KsError("force-push state must be (n_events, N, KS_EVENT_FORCE_STATE)")
+                io.event_force = event_force.data_ptr()
         _lib.check(self._lib.ks_terminate_reset(self._handle, _lib.current_stream(), ctypes.byref(io)))
 
     def close(self) -> None:

@@ -106,11 +106,13 @@ def control_step(dm: DeviceModel, buffers: Mapping[str, torch.Tensor | None], *,
                  action_scale: float = 1.0, events=None) -> None:
     """One control step of every env, in place on ``qpos, qvel, qacc_warmstart, time, last_ctrl``.
 
-    `events`: (descs, state (n_events, N), uniform (substeps, N, n_events, 3) or None, KsRng) for velocity events."""
+    `events`: (descs, state (n_events, N), uniform (substeps, N, n_events, KS_EVENT_DRAWS) or None, KsRng[, force
+    state (n_events, N, KS_EVENT_FORCE_STATE)]); the last entry is needed when a force push is among the events."""
     io = _make_io(dm, buffers, substeps, actuator_period, actuator_type, action_scale)
     if events is not None:
-        descs, state, uniform, rng = events
-        N = int(io.N)
+        descs, state, uniform, rng, *rest = events
+        force = rest[0] if rest else None
+        N, draws = int(io.N), _lib_dyn._T.KS_EVENT_DRAWS
         if len(descs) > _lib_dyn._T.KS_MAX_EVENTS:
             raise _lib.KsError(f"at most {_lib_dyn._T.KS_MAX_EVENTS} events")
         _lib.require_cuda(state, dtype=torch.float32)
@@ -118,8 +120,13 @@ def control_step(dm: DeviceModel, buffers: Mapping[str, torch.Tensor | None], *,
             raise _lib.KsError(f"event state: expected shape {(len(descs), N)}, got {tuple(state.shape)}")
         if uniform is not None:
             _lib.require_cuda(uniform, dtype=torch.float32)
-            if tuple(uniform.shape) != (substeps, N, len(descs), 3):
-                raise _lib.KsError(f"event draws: expected shape {(substeps, N, len(descs), 3)}, got {tuple(uniform.shape)}")
+            if tuple(uniform.shape) != (substeps, N, len(descs), draws):
+                raise _lib.KsError(f"event draws: expected shape {(substeps, N, len(descs), draws)}, got {tuple(uniform.shape)}")
+        if force is not None:
+            _lib.require_cuda(force, dtype=torch.float32)
+            if tuple(force.shape) != (len(descs), N, _lib_dyn._T.KS_EVENT_FORCE_STATE):
+                raise _lib.KsError(f"force-push state: expected shape {(len(descs), N, _lib_dyn._T.KS_EVENT_FORCE_STATE)}")
+            io.event_force = force.data_ptr()
         io.n_events = len(descs)
         for j, dsc in enumerate(descs):
             io.events[j] = dsc

@@ -107,7 +107,8 @@ class Rollout:
                                 episode_length=env.episode_length, reset_uniform=noise.get("reset_uniform"),
                                 seed=env.seed, step=step, step_base=step_base, event_state=ev_buf,
                                 event_intervals=[ev.interval_range for ev in c.engine.events.values()],
-                                event_reset_uniform=noise.get("event_reset_uniform"))
+                                event_reset_uniform=noise.get("event_reset_uniform"),
+                                event_force=ps.event_states.get("_force_buffer") if ps.event_states else None)
         # refresh the derived fields and the warm start of the reset envs (engine.py:213)
         c.engine.forward(c.physics_model, ps, self.reset_mask, env.randomization_dict)
         if not _relative_step:

@@ -49,7 +49,7 @@ def _data_struct(real):
         _fields_ = [
             ("qpos", real * MAXQ), ("qvel", real * MAXV), ("ctrl", real * MAXU), ("qacc_warmstart", real * MAXV),
             ("time", real),
-            ("mass_scale", real * MAXB), ("friction", real),
+            ("mass_scale", real * MAXB), ("friction", real), ("xfrc_applied", real * 6 * MAXB),
             ("xpos", real * 3 * MAXB), ("xquat", real * 4 * MAXB), ("xmat", real * 9 * MAXB),
             ("xipos", real * 3 * MAXB), ("ximat", real * 9 * MAXB), ("xanchor", real * 3 * MAXB),
             ("xaxis", real * 3 * MAXB), ("com", real * 3),
@@ -117,7 +117,7 @@ class DataView:
             return v
         arr = np.ctypeslib.as_array(v)
         nb, nq, nv, nu, ns = a["nb"], a["nq"], a["nv"], a["nu"], a["ns"]
-        trim = {"qpos": nq, "qvel": nv, "ctrl": nu, "qacc_warmstart": nv, "mass_scale": nb, "xpos": nb, "xquat": nb,
+        trim = {"qpos": nq, "qvel": nv, "ctrl": nu, "qacc_warmstart": nv, "mass_scale": nb, "xfrc_applied": nb, "xpos": nb, "xquat": nb,
                 "xmat": nb, "xipos": nb, "ximat": nb, "xanchor": nb, "xaxis": nb, "cinert": nb, "crb": nb, "cdof": nv,
                 "cvel": nb, "cdof_dot": nv, "qfrc_bias": nv, "qfrc_passive": nv, "qfrc_actuator": nv,
                 "actuator_force": nu, "qfrc_smooth": nv, "qacc_smooth": nv, "con_dist": ns, "con_pos": ns,

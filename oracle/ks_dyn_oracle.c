@@ -26,6 +26,9 @@ typedef struct FN(KsorData) {
   REAL qpos[KSOR_MAXQ], qvel[KSOR_MAXV], ctrl[KSOR_MAXU], qacc_warmstart[KSOR_MAXV], time;
   /* per-env parameters */
   REAL mass_scale[KSOR_MAXB], friction;
+  /* Cartesian force (3) and torque (3) per body, world frame, acting at the body's centre of mass: MuJoCo's
+   * xfrc_applied, which ForcePushEvent writes (ksim/events.py:302-307) */
+  REAL xfrc_applied[KSOR_MAXB][6];
   /* position-dependent */
   REAL xpos[KSOR_MAXB][3], xquat[KSOR_MAXB][4], xmat[KSOR_MAXB][9], xipos[KSOR_MAXB][3], ximat[KSOR_MAXB][9],
       xanchor[KSOR_MAXB][3], xaxis[KSOR_MAXB][3], com[3];
@@ -609,6 +612,25 @@ void FN(ksor_forward)(const KsorModel* m, Data* d) {
     d->qfrc_actuator[m->act_dof[u]] += d->actuator_force[u];
   }
   for (int i = 0; i < nv; ++i) d->qfrc_smooth[i] = d->qfrc_passive[i] - d->qfrc_bias[i] + d->qfrc_actuator[i];
+  /* applied Cartesian forces: qfrc += Jp(xipos)^T f + Jr^T t over the dofs of the body's ancestor chain */
+  for (int b = 1; b < m->nb; ++b) {
+    const REAL* w = d->xfrc_applied[b];
+    int any = 0;
+    for (int k = 0; k < 6; ++k) any |= w[k] != 0;
+    if (!any) continue;
+    REAL jacp[3 * KSOR_MAXV];
+    jac_point(m, d, jacp, d->xipos[b], b);
+    int j = -1;
+    for (int bb = b; bb > 0 && j < 0; bb = m->body_parent[bb]) {
+      if (m->body_jtype[bb] == KSOR_JNT_FREE) j = m->body_dofadr[bb] + 5;
+      else if (m->body_jtype[bb] == KSOR_JNT_HINGE) j = m->body_dofadr[bb];
+    }
+    for (; j >= 0; j = m->dof_parent[j]) {
+      REAL q = 0;
+      for (int k = 0; k < 3; ++k) q += jacp[k * nv + j] * w[k] + d->cdof[j][k] * w[3 + k];
+      d->qfrc_smooth[j] += q;
+    }
+  }
   chol_solve(d->qacc_smooth, d->L, d->qfrc_smooth, nv);
   FN(ksor_solve)(m, d);
 }

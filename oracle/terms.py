@@ -214,14 +214,14 @@ def scrub_action(action, clip_max=1e3):
 
 def velocity_event(kind, params, time_remaining, dt, u, level_scale, gravity=(0.0, 0.0, -9.81)):
     """One physics substep of a velocity event for one env (ksim/events.py:58-237): returns (impulse on qvel[0:6],
-    new time remaining).  `u` = three U[0,1) draws (direction / sign / height, magnitude, next interval).
+    new time remaining).  `u` = U[0,1) draws, the first three used (direction / sign / height, magnitude, next interval).
     kind: "linear" (linvel, vel_range), "angular" (angvel, vel_range), "jump" (jump_height_range)."""
     f32 = np.float32
     left = f32(time_remaining) - f32(dt)  # events.py:77-78: float32 timestep
     imp = np.zeros(6)
     if left > 0.0:
         return imp, float(left)
-    u0, u1, u2 = (float(x) for x in u)
+    u0, u1, u2 = (float(x) for x in u[:3])
     if kind == "linear":  # events.py:153-171
         theta = 2.0 * np.pi * u0
         mag = (params["vel_range"][0] + u1 * (params["vel_range"][1] - params["vel_range"][0])) * params["linvel"]
@@ -237,3 +237,26 @@ def velocity_event(kind, params, time_remaining, dt, u, level_scale, gravity=(0.
         raise ValueError(kind)
     lo, hi = params["interval_range"]
     return imp, lo + u2 * (hi - lo)
+
+
+def force_push_event(params, state, dt, u, level_scale):
+    """One physics substep of ForcePushEvent for one env (ksim/events.py:279-365).  `state` = (time remaining,
+    force duration left, wrench(6) = force then torque); `u` = ten U[0,1) draws (force direction 3, magnitude,
+    torque direction 3, case, interval, duration).  Returns (wrench applied to the body this substep, new state).
+    Float32 timers like the reference (events.py:293-295)."""
+    f32 = np.float32
+    left, dur, wrench = state
+    left, dur = f32(left) - f32(dt), f32(dur) - f32(dt)           # events.py:293-295
+    wrench = np.asarray(wrench, dtype=np.float64) * level_scale   # events.py:296: rebinds the carried value
+    applied = wrench * level_scale if dur > 0.0 else np.zeros(6)  # events.py:297-299
+    if left <= 0.0:                                                # events.py:310-315 -> _sample_force 320-358
+        u = [float(x) for x in u]
+        d0, d1 = 2.0 * np.array(u[0:3]) - 1.0, 2.0 * np.array(u[4:7]) - 1.0
+        s = params["force_range"][0] + u[3] * (params["force_range"][1] - params["force_range"][0])
+        force = d0 / np.linalg.norm(d0) * s * params["max_force"]
+        torque = d1 / np.linalg.norm(d1) * s * params["max_torque"]
+        which = min(2, int(3.0 * u[7]))                            # randint(0, 3)
+        wrench = np.concatenate([force if which != 1 else np.zeros(3), torque if which != 0 else np.zeros(3)])
+        left = params["interval_range"][0] + u[8] * (params["interval_range"][1] - params["interval_range"][0])
+        dur = params["duration_range"][0] + u[9] * (params["duration_range"][1] - params["duration_range"][0])
+    return applied, (float(left), float(dur), wrench)

@@ -251,7 +251,7 @@ def test_velocity_events_inside_the_substep_loop():
     kinds = [("linear", dict(linvel=1.0, vel_range=(0.2, 0.8), interval_range=(0.004, 0.03)), 0.5),
              ("angular", dict(angvel=2.0, vel_range=(0.0, 1.0), interval_range=(0.01, 0.05)), 1.0),
              ("jump", dict(jump_height_range=(0.02, 0.1), interval_range=(0.02, 0.06)), 1.0)]
-    u = rng.random(size=(T, S, N, 3, 3)).astype(np.float32)
+    u = rng.random(size=(T, S, N, 3, 12)).astype(np.float32)  # the velocity events use the first three draws
     left0 = rng.uniform(0.0, 0.03, size=(3, N)).astype(np.float32)
     # oracle: per env, per substep: PD torque from the pre-event state, events, physics step (engine.py:290-335)
     orc = Oracle(m.arrays())
@@ -296,3 +296,82 @@ def test_velocity_events_inside_the_substep_loop():
     assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])
     hi = torch.tensor([0.03, 0.05, 0.06], device=DEV)[:, None]
     assert (outs[0][1] <= hi).all() and (outs[0][1] > -0.006).all()
+
+
+def test_force_push_event_holds_a_wrench_on_one_body():
+    """ForcePushEvent (ksim/events.py:240-365) from explicit draws, on a foot and on the torso of the biped, together with a
+    linear push: state machine and trajectories against the oracle, which applies the same wrench as xfrc_applied."""
+    from ksim_amd import events as kev, physics
+
+    m = MODELS["kbot"]()
+    dm = physics.DeviceModel(m)
+    N, S, T = 16, 4, 4
+    qpos, qvel = random_states(m, N, seed=51, vel_scale=0.1, joint_range=0.2)
+    rng = np.random.default_rng(52)
+    actions = rng.uniform(-0.3, 0.3, size=(T, N, m.nu))
+    kp, kd, clip = rng.uniform(20, 150, m.nu), rng.uniform(1, 3, m.nu), np.full(m.nu, 40.0)
+    foot = m.nb - 1
+    prm = [dict(max_force=80.0, max_torque=10.0, force_range=(0.3, 1.0), duration_range=(0.01, 0.04), interval_range=(0.02, 0.06)),
+           None,
+           dict(max_force=30.0, max_torque=4.0, force_range=(0.5, 1.0), duration_range=(0.005, 0.03), interval_range=(0.01, 0.05))]
+    push = dict(linvel=1.0, vel_range=(0.2, 0.8), interval_range=(0.004, 0.03))
+    scales = [0.9, 1.0, 1.0]
+    # only the last force push in the list acts (each clears the applied forces of all bodies, events.py:302), so the
+    # first one is listed to check exactly that: its state advances, its wrench never reaches the body
+    evs = [kev.ForcePushEvent(body_id=1, scale=scales[0], **prm[0]), kev.LinearPushEvent(**push),
+           kev.ForcePushEvent(body_id=foot, scale=scales[2], **prm[2])]
+    bodies = [1, None, foot]
+    u = rng.random(size=(T, S, N, 3, 12)).astype(np.float32)
+    left0 = rng.uniform(0.0, 0.03, size=(3, N)).astype(np.float32)
+    force0 = np.zeros((3, N, 8), np.float32)
+    force0[0, :, 0] = rng.uniform(0.0, 0.02, N); force0[0, :, 1:7] = rng.normal(size=(N, 6)) * 5   # a push already under way
+    force0[2, :, 0] = rng.uniform(0.0, 0.02, N); force0[2, :, 1:7] = rng.normal(size=(N, 6)) * 5
+    orc = Oracle(m.arrays())
+    datas = [orc.data(qpos[e], qvel[e]) for e in range(N)]
+    left = left0.astype(np.float64).copy()
+    fstate = [[(float(left0[j, e]), float(force0[j, e, 0]), force0[j, e, 1:7].astype(np.float64)) for e in range(N)] for j in range(3)]
+    last = np.zeros((N, m.nu))
+    applied_steps = 0
+    for k in range(T):
+        for e, d in enumerate(datas):
+            for s in range(S):
+                c = oterms.latency_blend(float(s), 0.0, last[e], actions[k, e], np.zeros(m.nu, bool))
+                d.ctrl = oterms.position_actuator_torque(c, np.array(d.qpos[7:]), np.array(d.qvel[6:]), kp, kd, clip)
+                d.xfrc_applied = 0.0
+                for j in range(3):
+                    if prm[j] is None:
+                        imp, left[j, e] = oterms.velocity_event("linear", push, left[j, e], m.dt, u[k, s, e, j], 1.0)
+                        left[j, e] = float(np.float32(left[j, e]))
+                        for i in range(6):
+                            d.qvel[i] += imp[i]
+                    else:
+                        ap, st = oterms.force_push_event(prm[j], fstate[j][e], m.dt, u[k, s, e, j], scales[j])
+                        fstate[j][e] = (float(np.float32(st[0])), float(np.float32(st[1])), st[2].astype(np.float32).astype(np.float64))
+                        d.xfrc_applied = 0.0           # events.py:302: every force push clears all bodies first
+                        d.xfrc_applied[bodies[j]] = ap
+                        applied_steps += bool(ap.any()) and j == 2
+                orc.step(d)
+        last = actions[k].copy()
+    assert applied_steps >= 40, "the draws did not hold a force long enough to test anything"
+    buf = dict(qpos=t32(qpos), qvel=t32(qvel), qacc_warmstart=zeros(N, m.nv), time=zeros(N), last_ctrl=zeros(N, m.nu),
+               kp=t32(kp), kd=t32(kd), ctrl_clip=t32(clip))
+    state, force = t32(left0), t32(force0)
+    descs = [ev.desc(1.0) for ev in evs]
+    with pytest.raises(Exception, match="event_force"):
+        physics.control_step(dm, dict(buf, action=t32(actions[0])), substeps=S, events=(descs, state, t32(u[0]), None))
+    for k in range(T):
+        buf["action"] = t32(actions[k])
+        physics.control_step(dm, buf, substeps=S, events=(descs, state, t32(u[k]), None, force))
+    for field in ("qpos", "qvel"):
+        want = np.array([np.array(getattr(d, field)) for d in datas])
+        assert rel_err(buf[field].cpu().numpy(), want).max() <= TEN_STEP_TOL, field
+    got_t, got_f = state.cpu().numpy(), force.cpu().numpy()
+    np.testing.assert_allclose(got_t[1], left[1], rtol=0, atol=1e-6)
+    for j in (0, 2):
+        np.testing.assert_allclose(got_t[j], [fstate[j][e][0] for e in range(N)], rtol=0, atol=1e-6)
+        np.testing.assert_allclose(got_f[j, :, 0], [fstate[j][e][1] for e in range(N)], rtol=0, atol=1e-6)
+        np.testing.assert_allclose(got_f[j, :, 1:7], [fstate[j][e][2] for e in range(N)], rtol=1e-5, atol=1e-5)
+    # a bad body index is refused before any launch
+    bad = [kev.ForcePushEvent(body_id=m.nb, **prm[0]).desc(1.0)]
+    with pytest.raises(Exception, match="body"):
+        physics.control_step(dm, buf, substeps=S, events=(bad, t32(left0[:1]), None, None, t32(force0[:1])))

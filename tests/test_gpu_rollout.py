@@ -171,11 +171,15 @@ def test_long_rollout_with_resets_stays_finite_and_reproducible():
     assert (outs[0][0][:, 2] > 0.5).all()  # every env sits above the termination height after its reset
 
 
-def _push_events():
+def _push_events(force=False):
     from ksim_amd import events as kev
-    return {"push": kev.LinearPushEvent(linvel=0.5, interval_range=(0.05, 0.3)),
-            "spin": kev.AngularPushEvent(angvel=0.5, interval_range=(0.1, 0.4)),
-            "jump": kev.JumpEvent(jump_height_range=(0.01, 0.05), interval_range=(0.2, 0.6))}
+    evs = {"push": kev.LinearPushEvent(linvel=0.5, interval_range=(0.05, 0.3)),
+           "spin": kev.AngularPushEvent(angvel=0.5, interval_range=(0.1, 0.4)),
+           "jump": kev.JumpEvent(jump_height_range=(0.01, 0.05), interval_range=(0.2, 0.6))}
+    if force:
+        evs["shove"] = kev.ForcePushEvent(max_force=60.0, max_torque=5.0, duration_range=(0.05, 0.2),
+                                          interval_range=(0.1, 0.5), body_id=1)
+    return evs
 
 
 @pytest.mark.parametrize("with_events", [False, True])
@@ -185,22 +189,28 @@ def test_graph_replay_equals_eager_rollout(with_events):
     N, T, iters = 192, 8, 10
     runs = []
     for use_graph in (False, True):
-        m, c, rnd_, _, ro, EnvState = build(N, T, seed=5, min_height=0.8, events=_push_events() if with_events else None)
+        m, c, rnd_, _, ro, EnvState = build(N, T, seed=5, min_height=0.8, events=_push_events(force=True) if with_events else None)
         ps = c.engine.reset(c.physics_model, 1.0, 3, N, rnd_)
         env = EnvState(ps, rnd_, torch.zeros(N, 2, device=DEV), None, seed=123)
-        snaps = []
+        snaps, pushed = [], False
         for it in range(iters):
             traj, rew = ro.unroll(env, graph=use_graph)
             torch.cuda.synchronize()
             snaps.append((traj.qpos.clone(), traj.action.clone(), traj.done.clone(), rew.total.clone(),
                           ps.data.qpos.clone(), env.episode_length.clone()))
+            if with_events:
+                shove = ps.event_states["shove"]  # (time remaining, duration left, wrench) like the reference's tuple
+                snaps[-1] += (ps.event_states["_buffer"].clone(), shove[1].clone(), shove[2].clone())
+                pushed |= bool((shove[2].abs().amax(dim=1) > 0).any())
             junk = torch.randn(512, 512, device=DEV)  # unrelated eager work between replays
             (junk @ junk).sum().item()
         assert env.step == iters * T
+        assert pushed or not with_events, "no force push was ever drawn"
         runs.append(snaps)
     assert sum(int(s[2].sum().item()) for s in runs[0]) > 0, "no resets happened: the reset path was not replayed"
     for it, (a, b) in enumerate(zip(*runs)):
-        for x, y, name in zip(a, b, ("qpos", "action", "done", "reward", "state", "episode_length")):
+        for x, y, name in zip(a, b, ("qpos", "action", "done", "reward", "state", "episode_length", "event timers",
+                                     "force duration", "held wrench")):
             assert torch.equal(x, y), f"replay {it}: {name} differs from the eager rollout"
 
 
@@ -229,7 +239,7 @@ def test_events_in_the_rollout_fire_and_restart_with_the_episode():
     K = c.terms.obs_dim
     noise = dict(obs_normal=rng.normal(size=(N, K)), obs_uniform=rng.random((N, K)), action_normal=rng.normal(size=(N, m.nu)),
                  reset_uniform=rng.uniform(-1, 1, (N, m.nq + 1)), event_reset_uniform=rng.random((N, len(names))))
-    ev_u = rng.random((4, N, len(names), 3)).astype(np.float32)
+    ev_u = rng.random((4, N, len(names), 12)).astype(np.float32)
     noise_t = {k: t32(v) for k, v in noise.items()}
     env = EnvState(ps, rnd_, torch.zeros(N, 2, device=DEV), None, seed=1)
     env0 = EnvState(ps0, rnd0, torch.zeros(N, 2, device=DEV), None, seed=1)

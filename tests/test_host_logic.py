@@ -139,6 +139,17 @@ def test_scales_and_event_descriptors():
     assert (j.kind, j.lo, j.hi, j.level_scale) == (T.EVENT_JUMP, pytest.approx(0.1), pytest.approx(0.2), 1.0)
     a = kev.AngularPushEvent(angvel=1.5, interval_range=(0.5, 1.0)).desc(1.0)
     assert (a.kind, a.mag, a.lo, a.hi) == (T.EVENT_ANGULAR_PUSH, 1.5, 0.0, 1.0)
+    from ksim_amd import model as km
+    mdl = km.kbot_scale_model()
+    name = mdl.body_names[3]
+    fp = kev.ForcePushEvent.from_body_name(mdl, name, max_force=50.0, max_torque=5.0, duration_range=(0.1, 0.3),
+                                           interval_range=(1.0, 2.0), scale=0.5)
+    fd = fp.desc(1.0)
+    assert (fd.kind, fd.mag, fd.mag2, fd.body, fd.level_scale) == (T.EVENT_FORCE_PUSH, 50.0, 5.0, 3, 0.5)
+    assert (fd.lo, fd.hi, fd.duration_lo, fd.duration_hi) == (0.0, 1.0, pytest.approx(0.1), pytest.approx(0.3))
+    with pytest.raises(ValueError, match="not found"):
+        kev.ForcePushEvent.from_body_name(mdl, "no such body", max_force=1.0, max_torque=1.0, duration_range=(0.1, 0.2),
+                                          interval_range=(1.0, 2.0))
     # the engine refuses events that are not compiled into the step kernel, and more than the kernel holds
     from ksim_amd import actuators, engine
     act = actuators.TorqueActuators()

@@ -294,3 +294,35 @@ def test_float_and_double_oracles_agree():
     assert d64.nefc == d32.nefc and d64.nefc > 0
     scale = np.abs(d64.qacc).max()
     assert np.abs(np.array(d32.qacc) - d64.qacc).max() < 2e-4 * scale
+
+
+def test_applied_cartesian_force_closed_form_and_virtual_work(model):
+    """xfrc_applied (MuJoCo: force and torque on a body at its centre of mass, world frame).  A free ball accelerates
+    by f/m and I^-1 t; on the articulated models the generalised force does the same work as the wrench on the
+    body's finite-difference displacement, for random virtual velocities."""
+    ball = _ball(z=10.0)
+    orc = Oracle(ball.arrays())
+    d = orc.data()
+    f, t = np.array([1.0, -2.0, 3.0]), np.array([0.02, 0.01, -0.03])
+    d.xfrc_applied[1] = np.concatenate([f, t])
+    orc.forward(d)
+    np.testing.assert_allclose(d.qacc[:3], f / 2.0 + [0, 0, -9.81], atol=1e-12)
+    np.testing.assert_allclose(d.qacc[3:6], t / (0.4 * 2.0 * 0.1**2), atol=1e-9)
+    rng = np.random.default_rng(9)
+    orc = Oracle(model.arrays())
+    a = model.arrays()
+    for trial in range(4):
+        qpos, qvel = _random_state(model, rng)
+        b = int(rng.integers(1, model.nb))
+        w = rng.normal(size=6)
+        d0, d1 = orc.data(qpos, qvel), orc.data(qpos, qvel)
+        d1.xfrc_applied[b] = w
+        orc.forward(d0); orc.forward(d1)
+        Q = np.array(d1.qfrc_smooth) - np.array(d0.qfrc_smooth)
+        for _ in range(3):
+            dq, eps = rng.normal(size=model.nv), 1e-6
+            kp, km_ = (km.host_kinematics(a, _integrate_pos(model, qpos, dq, s * eps)) for s in (1, -1))
+            dx = (kp["xipos"][b] - km_["xipos"][b]) / (2 * eps)
+            S = kp["xmat"][b] @ km_["xmat"][b].T
+            om = np.array([S[2, 1] - S[1, 2], S[0, 2] - S[2, 0], S[1, 0] - S[0, 1]]) / 2 / (2 * eps)
+            assert Q @ dq == pytest.approx(w[:3] @ dx + w[3:] @ om, rel=1e-6, abs=1e-7)

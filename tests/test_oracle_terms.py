@@ -117,3 +117,33 @@ def test_velocity_events_closed_forms():
     np.testing.assert_allclose(imp[:3], [0.0, 0.0, np.sqrt(2 * 9.81 * 0.2)])
     v = imp[2]
     assert abs(v * v / (2 * 9.81) - 0.2) < 1e-12 and left == 2.0
+
+
+def test_force_push_event_state_machine():
+    """ForcePushEvent (ksim/events.py:240-365) step by step on hand-computed cases."""
+    p = dict(max_force=10.0, max_torque=2.0, force_range=(0.5, 1.0), duration_range=(0.1, 0.3), interval_range=(1.0, 2.0))
+    zero = np.zeros(6)
+    # nothing held, interval not over: no force, both timers lose dt
+    ap, (left, dur, w) = terms.force_push_event(p, (0.5, 0.0, zero), 0.005, np.zeros(10), 1.0)
+    assert not ap.any() and not w.any() and left == float(np.float32(0.5) - np.float32(0.005)) and dur == float(-np.float32(0.005))
+    # interval over: a new wrench is drawn but not yet applied in this substep; "both" case, unit directions
+    u = np.array([1.0, 0.5, 0.5, 1.0, 0.5, 0.5, 0.0, 0.99, 0.5, 0.5])
+    ap, (left, dur, w) = terms.force_push_event(p, (0.004, 0.0, zero), 0.005, u, 1.0)
+    assert not ap.any()
+    np.testing.assert_allclose(w, [10.0, 0, 0, 0, 0, -2.0], atol=1e-12)
+    assert (left, dur) == (1.5, pytest.approx(0.2))
+    # while the duration lasts the body gets the wrench; the magnitude is the drawn scale times the maximum
+    ap, st = terms.force_push_event(p, (left, dur, w), 0.005, np.zeros(10), 1.0)
+    np.testing.assert_allclose(ap, w)
+    ap, _ = terms.force_push_event(p, (1.0, 0.004, w), 0.005, np.zeros(10), 1.0)
+    assert not ap.any()  # duration ran out
+    # force-only / torque-only cases and the scale of the magnitude
+    for u7, keep in ((0.1, slice(0, 3)), (0.5, slice(3, 6))):
+        u = np.array([0.9, 0.2, 0.6, 0.0, 0.3, 0.8, 0.1, u7, 0.0, 0.0])
+        _, (_, _, w) = terms.force_push_event(p, (0.0, 0.0, zero), 0.005, u, 1.0)
+        other = slice(3, 6) if keep == slice(0, 3) else slice(0, 3)
+        assert not w[other].any()
+        assert np.linalg.norm(w[keep]) == pytest.approx(0.5 * (10.0 if keep == slice(0, 3) else 2.0))
+    # the curriculum scale multiplies the carried wrench every substep and once more when it is applied
+    ap, (_, _, w2) = terms.force_push_event(p, (1.0, 0.1, np.ones(6)), 0.005, np.zeros(10), 0.5)
+    np.testing.assert_allclose(w2, 0.5 * np.ones(6)); np.testing.assert_allclose(ap, 0.25 * np.ones(6))
