@@ -32,7 +32,8 @@ const char* ks_version(void);
 const char* ks_last_error(void);
 /* sizeof() of a public struct as this library was compiled, for binding self-checks:
  * 0 KsPpoLossParams, 1 KsModelDesc, 2 KsStepIO, 3 KsTermsDesc, 4 KsObserveIO, 5 KsTerminateIO, 6 KsMlpDesc,
- * 7 KsRewardIO, 8 KsObsElem, 9 KsTermDesc, 10 KsRewardDesc, 11 KsRng, 12 KsAdamParams, 13 KsEventDesc;
+ * 7 KsRewardIO, 8 KsObsElem, 9 KsTermDesc, 10 KsRewardDesc, 11 KsRng, 12 KsAdamParams, 13 KsEventDesc,
+ * 14 KsRewardScanIO, 15 KsRewardScanDesc;
  * -1 for anything else. */
 int64_t ks_abi_sizeof(int32_t which);
 
@@ -240,7 +241,8 @@ typedef struct KsStepIO {
   float* dbg_M;             /* (N, nv*nv) */
   float* dbg_bias;          /* (N, nv) */
   float* dbg_qacc_smooth;   /* (N, nv) */
-  float* dbg_con_dist;      /* (N, ns) */
+  float* contact_dist;      /* (N, ns) signed distance sphere - floor of the last substep's collision pass (negative =
+                               touching): the data.contact.dist that contact observations read (ksim/utils/mujoco.py:175-217) */
   /* events (ks_step only) */
   int32_t n_events;
   KsEventDesc events[KS_MAX_EVENTS];
@@ -265,13 +267,23 @@ int ks_forward(const KsModel* model, ks_stream_t stream, const KsStepIO* io /*ho
 enum { /* KsObsElem.src: which per-env array the element reads, all (N, dim) f32 */
   KS_SRC_QPOS = 0, KS_SRC_QVEL = 1, KS_SRC_QACC = 2, KS_SRC_CTRL = 3, KS_SRC_LAST_ACTION = 4,
   KS_SRC_COMMAND = 5, KS_SRC_TIME = 6, KS_SRC_XPOS = 7, KS_SRC_XQUAT = 8, KS_SRC_CVEL = 9,
-  KS_SRC_CONST = 10, KS_SRC_COUNT = 11
+  KS_SRC_CONST = 10, KS_SRC_CONTACT_DIST = 11 /* (N, ns) KsStepIO.contact_dist */, KS_SRC_COUNT = 12
 };
 enum { /* KsObsElem.kind */
   KS_OBS_COPY = 0,      /* src[index]                                  (observation.py:185-195,254-257,300-303,343-352) */
   KS_OBS_JOINT_POS = 1, /* qpos[index] - zero_offset[index - 7]        (observation.py:220-225) */
-  KS_OBS_ROT_INV = 2    /* component `comp` of q^-1 v q, q = qpos[3:7], v = src[index..index+2] or (c0,c1,c2)
+  KS_OBS_ROT_INV = 2,   /* component `comp` of q^-1 v q, q = qpos[3:7], v = src[index..index+2] or (c0,c1,c2)
                            (in_robot_frame velocities, observation.py:198-217; gravity in the body frame) */
+  KS_OBS_CONTACT = 3,   /* 1 when src[index] < 0 else 0: geoms_colliding of one sphere with the floor
+                           (observation.py:481-521, utils/mujoco.py:175-217) */
+  KS_OBS_DELAYED = 4,   /* the value `comp` control steps ago (observation.py:228-252,260-283): the element owns the
+                           column carry[carry + d * stride], d = 0..comp-1, oldest first; it emits slot 0 (minus
+                           zero_offset when src is qpos), shifts the column down and appends src[index].  A fresh
+                           episode fills the column with the current value. */
+  KS_OBS_GRAVITY_EMA = 5 /* component `comp` of the lagged, biased gravity reading (observation.py:355-442):
+                           p = R(euler bias) (q^-1 (c0,c1,c2) q), x <- x lag + p (1 - lag), emits x.
+                           carry[carry .. carry+6] = x(3), lag, bias(3); a fresh episode sets x = 0,
+                           lag ~ U(q0, q1), bias ~ U(-q2, q2)^3 from four draws. */
 };
 enum { KS_NOISE_NONE = 0, KS_NOISE_ADD_GAUSSIAN = 1, KS_NOISE_ADD_UNIFORM = 2, KS_NOISE_MUL_GAUSSIAN = 3,
        KS_NOISE_MUL_UNIFORM = 4 }; /* ksim/noise.py:184-213 */
@@ -280,6 +292,8 @@ typedef struct KsObsElem {
   float c0, c1, c2;
   int32_t noise_kind;
   float noise_mean, noise_scale; /* std or mag, multiplied by the curriculum level (noise.py:86,102) */
+  int32_t carry, stride;         /* stateful kinds: offset into the env's carry row, distance between delay slots */
+  float q0, q1, q2;              /* KS_OBS_GRAVITY_EMA: min_lag, max_lag, imu_bias */
 } KsObsElem;
 
 /* Terminations (replaces get_terminations + terms, rl.py:288-299, ksim/terminations.py:60-192). */
@@ -299,6 +313,8 @@ typedef struct KsTermDesc {
 typedef struct KsTermsDesc {
   int32_t nq, nv, nu, nb;
   int32_t obs_dim, n_terms, command_dim, random_heading;
+  int32_t ns;        /* contact spheres of the model (width of KS_SRC_CONTACT_DIST) */
+  int32_t carry_dim; /* floats of observation carry per env (0: no stateful observation) */
   int32_t nonfinite_terminates; /* 1: an env whose qpos/qvel is not finite counts as failed (done, no success);
                                    the reference has no such guard and would carry the NaNs forever */
   KsObsElem obs[KS_MAX_OBS];
@@ -321,6 +337,11 @@ typedef struct KsObserveIO {
   KsRng rng;
   float* obs;                /* (N, obs_dim) clean, nullable */
   float* noisy_obs;          /* (N, obs_dim) noisy copy, nullable (rl.py:181-184) */
+  /* stateful observations (rl.py:166-176: observe_stateful with the carry of the previous control step) */
+  float* carry;               /* (N, carry_dim) in/out; required when carry_dim > 0 */
+  const uint8_t* fresh;       /* (N) nullable: non-zero = the env starts an episode, its carries are initialised from the
+                                 current state before observing (initial_carry, rl.py:1034-1080); NULL = none */
+  const float* carry_uniform; /* (N, carry_dim) U[0,1) draws for the initial carries, nullable -> Philox */
 } KsObserveIO;
 int ks_observe(const KsTerms* terms, ks_stream_t stream, const KsObserveIO* io /*host*/);
 
@@ -442,7 +463,8 @@ int ks_ppo_loss_grad(ks_stream_t stream, int64_t M, int32_t nu, const KsPpoLossP
 enum { KS_REW_STAY_ALIVE = 0, KS_REW_BASE_HEIGHT = 1, KS_REW_BASE_HEIGHT_RANGE = 2, KS_REW_ACTION_VEL = 3,
        KS_REW_ACTION_ACC = 4, KS_REW_ACTION_JERK = 5, KS_REW_UPRIGHT_ANGVEL = 6, KS_REW_UPRIGHT_LINVEL = 7,
        KS_REW_UPRIGHT_POSE = 8,
-       KS_REW_AMP = 9 /* max(0, 1 - 0.25 (logit - 1)^2) of the discriminator logits, ksim/task/amp.py:99-112 */ };
+       KS_REW_AMP = 9, /* max(0, 1 - 0.25 (logit - 1)^2) of the discriminator logits, ksim/task/amp.py:99-112 */
+       KS_REW_STATEFUL = 10 /* a value ks_reward_scan computed: stateful[norm] (norm = slot index) */ };
 enum { KS_NORM_L1 = 0, KS_NORM_L2 = 1 }; /* xax.get_norm: l1 = |x|, l2 = x^2 (reference tests/test_rewards.py:95-98) */
 typedef struct KsRewardDesc {
   int32_t kind;
@@ -464,8 +486,48 @@ typedef struct KsRewardIO {
   const float* disc_logits; /* (T, N) discriminator output per frame (ks_mlp_forward on the motion frames), KS_REW_AMP only */
   float* components;   /* (n_rewards, T, N) nullable */
   float* total;        /* (T, N) */
+  const float* stateful; /* (n_slots, T, N) output of ks_reward_scan, KS_REW_STATEFUL only */
 } KsRewardIO;
 int ks_rewards(ks_stream_t stream, const KsRewardIO* io /*host*/);
+
+/* Stateful rewards (StatefulReward.get_reward_stateful, ksim/rewards.py:127-163): sequential scans over the T steps of
+ * a rollout with a per-env carry that persists between rollouts.  One lane walks one env forward in time.  As in
+ * get_rewards (rl.py:206-214) the carry an env starts from is the initial one when the LAST step of this rollout is
+ * done.  Outputs are unscaled; KS_REW_STATEFUL terms of ks_rewards pick them up in dict order.
+ *   KS_SCAN_FEET_AIR_TIME (rewards.py:992-1085): carry = 3 n counters (air, ground, stationary ground; whole numbers
+ *     kept as f32), three output slots (air, gnd, stationary_gnd).
+ *   KS_SCAN_SPARSE_TARGET_HEIGHT (rewards.py:1148-1192): carry = n running maximum heights, one output slot.
+ * Contact flags are the (n_contact, n) block of 0/1 values at obs[contact_index...] (any over n_contact, > 0.5);
+ * positions the (n, 3) block at obs[position_index...]. */
+#define KS_MAX_REWARD_SCANS 4
+#define KS_MAX_SCAN_BODIES 8
+enum { KS_SCAN_FEET_AIR_TIME = 0, KS_SCAN_SPARSE_TARGET_HEIGHT = 1 };
+typedef struct KsRewardScanDesc {
+  int32_t kind;
+  int32_t n;               /* feet / bodies */
+  int32_t n_contact;       /* contact geoms per foot */
+  int32_t contact_index, position_index;
+  int32_t slot;            /* first output slot */
+  int32_t carry_index;     /* offset into the env's carry row */
+  int32_t linvel_cmd_index, angvel_cmd_index; /* feet air time: index into the command vector whose |value| decides
+                                                 "moving", or -1 to use |qvel[0:2]| and qvel[5] (rewards.py:1020-1037) */
+  float air_steps, gnd_steps; /* round(gait_period * air_time_percent / ctrl_dt), round(gait_period * (1 - pct) / ctrl_dt) */
+  float bias, ground_penalty;
+  float linvel_threshold, angvel_threshold;
+  float height;            /* sparse target height: the reward is clipped at it */
+} KsRewardScanDesc;
+typedef struct KsRewardScanIO {
+  int64_t T, N;
+  int32_t obs_dim, nv, command_dim, n_scans, carry_dim, n_slots;
+  KsRewardScanDesc scans[KS_MAX_REWARD_SCANS];
+  const float* obs;      /* (T, N, obs_dim) */
+  const float* qvel;     /* (T, N, nv) */
+  const float* command;  /* (T, N, command_dim) nullable unless a *_cmd_index is set */
+  const uint8_t* done;   /* (T, N) */
+  float* carry;          /* (N, carry_dim) in/out */
+  float* out;            /* (n_slots, T, N) */
+} KsRewardScanIO;
+int ks_reward_scan(ks_stream_t stream, const KsRewardScanIO* io /*host*/);
 
 /* ------------------------------------------------------------------ measurement aid
  * A plain f32 copy of n elements (reads 4n bytes, writes 4n bytes): the known-size kernel that hardware

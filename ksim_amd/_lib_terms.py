@@ -6,8 +6,8 @@ from ctypes import POINTER, c_float, c_int8, c_int32, c_int64, c_uint8, c_uint64
 
 KS_MAX_OBS, KS_MAX_TERMS, KS_MAX_QPOS, KS_MAX_LAYERS = 512, 16, 40, 8
 (SRC_QPOS, SRC_QVEL, SRC_QACC, SRC_CTRL, SRC_LAST_ACTION, SRC_COMMAND, SRC_TIME, SRC_XPOS, SRC_XQUAT, SRC_CVEL,
- SRC_CONST, SRC_COUNT) = range(12)
-OBS_COPY, OBS_JOINT_POS, OBS_ROT_INV = 0, 1, 2
+ SRC_CONST, SRC_CONTACT_DIST, SRC_COUNT) = range(13)
+OBS_COPY, OBS_JOINT_POS, OBS_ROT_INV, OBS_CONTACT, OBS_DELAYED, OBS_GRAVITY_EMA = range(6)
 NOISE_NONE, NOISE_ADD_GAUSSIAN, NOISE_ADD_UNIFORM, NOISE_MUL_GAUSSIAN, NOISE_MUL_UNIFORM = range(5)
 (TERM_MIN_HEIGHT, TERM_BAD_Z, TERM_NOT_UPRIGHT, TERM_BAD_VELOCITY, TERM_FAR_FROM_ORIGIN,
  TERM_EPISODE_LENGTH) = range(6)
@@ -18,7 +18,8 @@ MLP_F32, MLP_BF16 = 0, 1
 class KsObsElem(ctypes.Structure):
     _fields_ = [("kind", c_int32), ("src", c_int32), ("index", c_int32), ("comp", c_int32), ("c0", c_float),
                 ("c1", c_float), ("c2", c_float), ("noise_kind", c_int32), ("noise_mean", c_float),
-                ("noise_scale", c_float)]
+                ("noise_scale", c_float), ("carry", c_int32), ("stride", c_int32), ("q0", c_float), ("q1", c_float),
+                ("q2", c_float)]
 
 
 class KsTermDesc(ctypes.Structure):
@@ -29,7 +30,7 @@ class KsTermDesc(ctypes.Structure):
 class KsTermsDesc(ctypes.Structure):
     _fields_ = [("nq", c_int32), ("nv", c_int32), ("nu", c_int32), ("nb", c_int32), ("obs_dim", c_int32),
                 ("n_terms", c_int32), ("command_dim", c_int32), ("random_heading", c_int32),
-                ("nonfinite_terminates", c_int32),
+                ("ns", c_int32), ("carry_dim", c_int32), ("nonfinite_terminates", c_int32),
                 ("obs", KsObsElem * KS_MAX_OBS), ("terms", KsTermDesc * KS_MAX_TERMS),
                 ("reset_base", c_float * KS_MAX_QPOS), ("reset_mag", c_float * KS_MAX_QPOS),
                 ("reset_lo", c_float * KS_MAX_QPOS), ("reset_hi", c_float * KS_MAX_QPOS),
@@ -54,7 +55,8 @@ class KsEventDesc(ctypes.Structure):
 class KsObserveIO(ctypes.Structure):
     _fields_ = [("N", c_int64), ("level", c_float), ("src", c_void_p * SRC_COUNT), ("zero_offset", c_void_p),
                 ("bias", c_void_p), ("noise_normal", c_void_p), ("noise_uniform", c_void_p), ("rng", KsRng),
-                ("obs", c_void_p), ("noisy_obs", c_void_p)]
+                ("obs", c_void_p), ("noisy_obs", c_void_p), ("carry", c_void_p), ("fresh", c_void_p),
+                ("carry_uniform", c_void_p)]
 
 
 class KsTerminateIO(ctypes.Structure):
@@ -73,7 +75,9 @@ class KsMlpDesc(ctypes.Structure):
 
 
 (REW_STAY_ALIVE, REW_BASE_HEIGHT, REW_BASE_HEIGHT_RANGE, REW_ACTION_VEL, REW_ACTION_ACC, REW_ACTION_JERK,
- REW_UPRIGHT_ANGVEL, REW_UPRIGHT_LINVEL, REW_UPRIGHT_POSE, REW_AMP) = range(10)
+ REW_UPRIGHT_ANGVEL, REW_UPRIGHT_LINVEL, REW_UPRIGHT_POSE, REW_AMP, REW_STATEFUL) = range(11)
+KS_MAX_REWARD_SCANS, KS_MAX_SCAN_BODIES = 4, 8
+SCAN_FEET_AIR_TIME, SCAN_SPARSE_TARGET_HEIGHT = 0, 1
 NORM_L1, NORM_L2 = 0, 1
 KS_MAX_REWARD_TERMS = 32
 
@@ -88,7 +92,22 @@ class KsRewardIO(ctypes.Structure):
                 ("n_rewards", c_int32), ("rewards", KsRewardDesc * KS_MAX_REWARD_TERMS), ("use_clip_min", c_int32),
                 ("use_clip_max", c_int32), ("clip_min", c_float), ("clip_max", c_float), ("qpos", c_void_p),
                 ("qvel", c_void_p), ("action", c_void_p), ("done", c_void_p), ("success", c_void_p),
-                ("disc_logits", c_void_p), ("components", c_void_p), ("total", c_void_p)]
+                ("disc_logits", c_void_p), ("components", c_void_p), ("total", c_void_p), ("stateful", c_void_p)]
+
+
+class KsRewardScanDesc(ctypes.Structure):
+    _fields_ = [("kind", c_int32), ("n", c_int32), ("n_contact", c_int32), ("contact_index", c_int32),
+                ("position_index", c_int32), ("slot", c_int32), ("carry_index", c_int32),
+                ("linvel_cmd_index", c_int32), ("angvel_cmd_index", c_int32), ("air_steps", c_float),
+                ("gnd_steps", c_float), ("bias", c_float), ("ground_penalty", c_float), ("linvel_threshold", c_float),
+                ("angvel_threshold", c_float), ("height", c_float)]
+
+
+class KsRewardScanIO(ctypes.Structure):
+    _fields_ = [("T", c_int64), ("N", c_int64), ("obs_dim", c_int32), ("nv", c_int32), ("command_dim", c_int32),
+                ("n_scans", c_int32), ("carry_dim", c_int32), ("n_slots", c_int32),
+                ("scans", KsRewardScanDesc * KS_MAX_REWARD_SCANS), ("obs", c_void_p), ("qvel", c_void_p),
+                ("command", c_void_p), ("done", c_void_p), ("carry", c_void_p), ("out", c_void_p)]
 
 
 class KsAdamParams(ctypes.Structure):
@@ -99,6 +118,8 @@ class KsAdamParams(ctypes.Structure):
 def bind(lib) -> None:
     lib.ks_rewards.argtypes = [c_void_p, POINTER(KsRewardIO)]
     lib.ks_rewards.restype = c_int32
+    lib.ks_reward_scan.argtypes = [c_void_p, POINTER(KsRewardScanIO)]
+    lib.ks_reward_scan.restype = c_int32
     lib.ks_terms_create.argtypes = [POINTER(KsTermsDesc), POINTER(c_void_p)]
     lib.ks_terms_destroy.argtypes = [c_void_p]
     lib.ks_observe.argtypes = [c_void_p, c_void_p, POINTER(KsObserveIO)]

@@ -656,7 +656,7 @@ void step_kernel(StepArgs a) {
                                                 R[6] * s_pos.x + R[7] * s_pos.y + R[8] * s_pos.z};
       dist = c.z - s_rad;
       cpos = {c.x, c.y, c.z - s_rad - 0.5f * dist};
-      if (a.dbg_con_dist) a.dbg_con_dist[env * ns + lane] = dist;
+      if (a.contact_dist) a.contact_dist[env * ns + lane] = dist;
     }
     const bool touching = is_sph && (dist < 0.f);
     const unsigned long long cmask = __ballot(touching);
@@ -1137,7 +1137,7 @@ static int launch_step(const KsModel* km, ks_stream_t stream, const KsStepIO* io
   a.traj_ctrl = io->traj_ctrl; a.traj_xpos = io->traj_xpos; a.traj_xquat = io->traj_xquat;
   a.solver_niter = io->solver_niter; a.nefc = io->nefc;
   a.dbg_M = io->dbg_M; a.dbg_bias = io->dbg_bias; a.dbg_qacc_smooth = io->dbg_qacc_smooth;
-  a.dbg_con_dist = io->dbg_con_dist;
+  a.contact_dist = io->contact_dist;
   a.ctrl_in = io->ctrl_in;
   if (!forward_only) {
     if (io->substeps < 1 || io->substeps > 64) return fail(KS_EINVAL, "ks_step: substeps must be in 1..64");

@@ -327,6 +327,8 @@ extern "C" int64_t ks_abi_sizeof(int32_t which) {
     case 11: return sizeof(KsRng);
     case 12: return sizeof(KsAdamParams);
     case 13: return sizeof(KsEventDesc);
+    case 14: return sizeof(KsRewardScanIO);
+    case 15: return sizeof(KsRewardScanDesc);
     default: return -1;
   }
 }

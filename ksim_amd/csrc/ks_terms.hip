@@ -34,7 +34,20 @@ struct ObserveArgs {
   KsRng rng;
   float *obs, *noisy;
   int obs_dim, nq, nu;
+  float* carry;
+  const uint8_t* fresh;
+  const float* carry_uniform;
+  int carry_dim;
 };
+
+// v rotated by the (normalised) wxyz quaternion q
+__device__ inline void rot_fwd(const float* q4, const float* v, float* out) {
+  const float w = q4[0], x = q4[1], y = q4[2], z = q4[3];
+  const float tx = 2.f * (y * v[2] - z * v[1]), ty = 2.f * (z * v[0] - x * v[2]), tz = 2.f * (x * v[1] - y * v[0]);
+  out[0] = v[0] + w * tx + (y * tz - z * ty);
+  out[1] = v[1] + w * ty + (z * tx - x * tz);
+  out[2] = v[2] + w * tz + (x * ty - y * tx);
+}
 
 __global__ __launch_bounds__(256) void observe_kernel(ObserveArgs a) {
   const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -47,6 +60,44 @@ __global__ __launch_bounds__(256) void observe_kernel(ObserveArgs a) {
     v = (el.src == KS_SRC_CONST) ? el.c0 : a.src[el.src][e * a.src_dim[el.src] + el.index];
   } else if (el.kind == KS_OBS_JOINT_POS) {
     v = a.src[KS_SRC_QPOS][e * a.nq + el.index] - (a.zero_offset ? a.zero_offset[e * a.nu + (el.index - 7)] : 0.f);
+  } else if (el.kind == KS_OBS_CONTACT) {
+    v = a.src[el.src][e * a.src_dim[el.src] + el.index] < 0.f ? 1.f : 0.f;
+  } else if (el.kind == KS_OBS_DELAYED) {
+    // this thread owns one column of the delay buffer: nobody else reads or writes it
+    float* col = a.carry + e * a.carry_dim + el.carry;
+    const float cur = a.src[el.src][e * a.src_dim[el.src] + el.index];
+    const bool fresh = a.fresh && a.fresh[e];
+    v = fresh ? cur : col[0];
+    for (int d = 0; d + 1 < el.comp; ++d) col[d * el.stride] = fresh ? cur : col[(d + 1) * el.stride];
+    col[(el.comp - 1) * el.stride] = cur;
+    if (el.src == KS_SRC_QPOS && a.zero_offset) v -= a.zero_offset[e * a.nu + (el.index - 7)];
+  } else if (el.kind == KS_OBS_GRAVITY_EMA) {
+    // the three components of one reading run in three threads; each recomputes the vector and owns x[comp]
+    float* c = a.carry + e * a.carry_dim + el.carry;
+    float x = c[el.comp], lag = c[3], b[3] = {c[4], c[5], c[6]};
+    if (a.fresh && a.fresh[e]) {
+      float u[4];
+      if (a.carry_uniform) {
+        for (int j = 0; j < 4; ++j) u[j] = a.carry_uniform[e * a.carry_dim + el.carry + 3 + j];
+      } else {
+        const Philox4 r = draw(a.rng.seed, a.rng.step + (a.rng.step_base ? *a.rng.step_base : 0ull), kRngObsCarry, (uint64_t)e, (uint32_t)el.carry);
+        u[0] = u01(r.x); u[1] = u01(r.y); u[2] = u01(r.z); u[3] = u01(r.w);
+      }
+      x = 0.f;
+      lag = el.q0 + u[0] * (el.q1 - el.q0);
+      for (int j = 0; j < 3; ++j) b[j] = -el.q2 + u[1 + j] * (2.f * el.q2);
+      if (el.comp == 0) { c[3] = lag; c[4] = b[0]; c[5] = b[1]; c[6] = b[2]; }
+    }
+    float g[3], p[3];
+    rot_inv(a.src[KS_SRC_QPOS] + e * a.nq + 3, el.c0, el.c1, el.c2, g);
+    // roll-pitch-yaw (x, y, z angles; z applied last) to a quaternion
+    const float cr = cosf(0.5f * b[0]), sr = sinf(0.5f * b[0]), cp = cosf(0.5f * b[1]), sp = sinf(0.5f * b[1]);
+    const float cy = cosf(0.5f * b[2]), sy = sinf(0.5f * b[2]);
+    const float bq[4] = {cr * cp * cy + sr * sp * sy, sr * cp * cy - cr * sp * sy, cr * sp * cy + sr * cp * sy, cr * cp * sy - sr * sp * cy};
+    rot_fwd(bq, g, p);
+    x = x * lag + p[el.comp] * (1.f - lag);
+    c[el.comp] = x;
+    v = x;
   } else {
     float vec[3] = {el.c0, el.c1, el.c2}, out[3];
     if (el.src != KS_SRC_CONST) {
@@ -320,6 +371,7 @@ __global__ __launch_bounds__(256) void rewards_kernel(KsRewardIO io) {
         const float d = io.disc_logits[idx] - 1.0f;
         val = fmaxf(0.f, 1.0f - 0.25f * d * d);
       } break;
+      case KS_REW_STATEFUL: val = io.stateful[(int64_t)r.norm * TN + idx]; break;
       default: break;
     }
     val *= r.scale;
@@ -329,6 +381,74 @@ __global__ __launch_bounds__(256) void rewards_kernel(KsRewardIO io) {
   if (io.use_clip_min) total = fmaxf(total, io.clip_min);
   if (io.use_clip_max) total = fminf(total, io.clip_max);
   if (io.total) io.total[idx] = total;
+}
+
+// One lane walks one env through the T steps of the rollout; every load of a step is coalesced over envs for the
+// (T, N) arrays and strided by the row length for the (T, N, dim) ones.
+__global__ __launch_bounds__(256) void reward_scan_kernel(KsRewardScanIO io) {
+  const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= io.N) return;
+  const int64_t TN = io.T * io.N;
+  const bool restart = io.done[(io.T - 1) * io.N + e] != 0;  // ksim/task/rl.py:206-214
+  for (int sidx = 0; sidx < io.n_scans; ++sidx) {
+    const KsRewardScanDesc s = io.scans[sidx];
+    float* cr = io.carry + e * io.carry_dim + s.carry_index;
+    float c[3 * KS_MAX_SCAN_BODIES];  // counter k of body f at c[k * KS_MAX_SCAN_BODIES + f]; packed as k * n + f in memory
+    const int nk = s.kind == KS_SCAN_FEET_AIR_TIME ? 3 : 1;
+    for (int k = 0; k < 3; ++k)
+      for (int f = 0; f < KS_MAX_SCAN_BODIES; ++f)
+        c[k * KS_MAX_SCAN_BODIES + f] = (k < nk && f < s.n && !restart) ? cr[k * s.n + f] : 0.f;
+    for (int64_t t = 0; t < io.T; ++t) {
+      const int64_t idx = t * io.N + e;
+      const float* ob = io.obs + idx * io.obs_dim;
+      const float* qv = io.qvel + idx * io.nv;
+      const bool dn = io.done[idx] != 0;
+      if (s.kind == KS_SCAN_FEET_AIR_TIME) {
+        const float* cmd = io.command ? io.command + idx * io.command_dim : nullptr;
+        const bool lin = s.linvel_cmd_index >= 0 ? fabsf(cmd[s.linvel_cmd_index]) > s.linvel_threshold
+                                                 : sqrtf(qv[0] * qv[0] + qv[1] * qv[1]) > s.linvel_threshold;
+        const bool ang = s.angvel_cmd_index >= 0 ? fabsf(cmd[s.angvel_cmd_index]) > s.angvel_threshold
+                                                 : qv[5] > s.angvel_threshold;
+        const bool moving = (lin || ang) && !dn;
+        float air = -INFINITY, gnd = -INFINITY, stat = -INFINITY;
+        for (int f = 0; f < KS_MAX_SCAN_BODIES; ++f) {
+          if (f >= s.n) break;
+          bool contact = false;
+          for (int g = 0; g < s.n_contact; ++g) contact |= ob[s.contact_index + g * s.n + f] > 0.5f;
+          const float a_ = (!contact && moving) ? c[f] + 1.f : 0.f;
+          const float g_ = (contact && moving) ? c[KS_MAX_SCAN_BODIES + f] + 1.f : 0.f;
+          const float s_ = (contact && !moving) ? c[2 * KS_MAX_SCAN_BODIES + f] + 1.f : 0.f;
+          c[f] = a_; c[KS_MAX_SCAN_BODIES + f] = g_; c[2 * KS_MAX_SCAN_BODIES + f] = s_;
+          air = fmaxf(air, a_ < s.air_steps ? a_ / s.air_steps + s.bias : 0.f);
+          gnd = fmaxf(gnd, g_ < s.gnd_steps ? g_ / s.gnd_steps + s.bias : -s.ground_penalty);
+          stat = fmaxf(stat, fminf(fmaxf(s_ / s.gnd_steps, 0.f), 1.f) + s.bias);
+        }
+        io.out[(int64_t)s.slot * TN + idx] = air;
+        io.out[(int64_t)(s.slot + 1) * TN + idx] = gnd;
+        io.out[(int64_t)(s.slot + 2) * TN + idx] = stat;
+      } else {
+        const bool still = (sqrtf(qv[0] * qv[0] + qv[1] * qv[1]) < s.linvel_threshold && qv[5] < s.angvel_threshold) || dn;
+        float best = -INFINITY;
+        for (int f = 0; f < KS_MAX_SCAN_BODIES; ++f) {
+          if (f >= s.n) break;
+          bool contact = false;
+          for (int g = 0; g < s.n_contact; ++g) contact |= ob[s.contact_index + g * s.n + f] > 0.5f;
+          const float h = ob[s.position_index + 3 * f + 2];
+          best = fmaxf(best, fminf(contact ? c[f] : 0.f, s.height));
+          c[f] = (still || contact) ? 0.f : fmaxf(c[f], h);
+        }
+        io.out[(int64_t)s.slot * TN + idx] = best;
+      }
+    }
+    if (s.kind == KS_SCAN_FEET_AIR_TIME) {
+      for (int k = 0; k < 3; ++k)
+        for (int f = 0; f < KS_MAX_SCAN_BODIES; ++f)
+          if (f < s.n) cr[k * s.n + f] = c[k * KS_MAX_SCAN_BODIES + f];
+    } else {
+      for (int f = 0; f < KS_MAX_SCAN_BODIES; ++f)
+        if (f < s.n) cr[f] = c[f];
+    }
+  }
 }
 
 }  // namespace ks
@@ -345,11 +465,23 @@ extern "C" int ks_terms_create(const KsTermsDesc* d, KsTerms** out) {
   if (d->obs_dim < 0 || d->obs_dim > KS_MAX_OBS) return fail(KS_ELIMIT, "ks_terms_create: obs_dim %d > %d", d->obs_dim, KS_MAX_OBS);
   if (d->n_terms < 0 || d->n_terms > KS_MAX_TERMS) return fail(KS_ELIMIT, "ks_terms_create: %d terminations > %d", d->n_terms, KS_MAX_TERMS);
   if (d->nq < 0 || d->nq > KS_MAX_QPOS || d->nv < 0 || d->nu < 0 || d->nb < 1) return fail(KS_EINVAL, "ks_terms_create: bad sizes");
-  const int src_dim[KS_SRC_COUNT] = {d->nq, d->nv, d->nv, d->nu, d->nu, d->command_dim, 1, d->nb * 3, d->nb * 4, d->nb * 6, 0};
+  const int src_dim[KS_SRC_COUNT] = {d->nq, d->nv, d->nv, d->nu, d->nu, d->command_dim, 1, d->nb * 3, d->nb * 4, d->nb * 6, 0, d->ns};
+  if (d->ns < 0 || d->carry_dim < 0) return fail(KS_EINVAL, "ks_terms_create: negative sphere count or carry size");
   for (int k = 0; k < d->obs_dim; ++k) {
     const KsObsElem& el = d->obs[k];
     if (el.src < 0 || el.src >= KS_SRC_COUNT) return fail(KS_EINVAL, "ks_terms_create: obs %d: bad source %d", k, el.src);
-    if (el.kind < KS_OBS_COPY || el.kind > KS_OBS_ROT_INV) return fail(KS_EINVAL, "ks_terms_create: obs %d: bad kind", k);
+    if (el.kind < KS_OBS_COPY || el.kind > KS_OBS_GRAVITY_EMA) return fail(KS_EINVAL, "ks_terms_create: obs %d: bad kind", k);
+    if (el.kind == KS_OBS_DELAYED) {
+      if (el.comp < 1 || el.stride < 1 || el.carry < 0 || el.carry + (el.comp - 1) * el.stride >= d->carry_dim)
+        return fail(KS_EINVAL, "ks_terms_create: obs %d: delay buffer outside the carry row", k);
+      if (el.src == KS_SRC_CONST) return fail(KS_EINVAL, "ks_terms_create: obs %d: a delayed constant", k);
+      if (el.src == KS_SRC_QPOS && (el.index < 7 || el.index - 7 >= d->nu)) return fail(KS_EINVAL, "ks_terms_create: obs %d: delayed joint position index %d out of range", k, el.index);
+    }
+    if (el.kind == KS_OBS_GRAVITY_EMA) {
+      if (el.comp < 0 || el.comp > 2 || d->nq < 7 || el.src != KS_SRC_CONST) return fail(KS_EINVAL, "ks_terms_create: obs %d: bad gravity reading", k);
+      if (el.carry < 0 || el.carry + 7 > d->carry_dim) return fail(KS_EINVAL, "ks_terms_create: obs %d: carry outside the carry row", k);
+      if (!(el.q0 >= 0.f && el.q0 < 1.f && el.q1 >= 0.f && el.q1 < 1.f && el.q2 >= 0.f)) return fail(KS_EINVAL, "ks_terms_create: obs %d: lag outside [0, 1) or negative bias", k);
+    }
     const int span = el.kind == KS_OBS_ROT_INV ? 3 : 1;
     if (el.src != KS_SRC_CONST && (el.index < 0 || el.index + span > src_dim[el.src]))
       return fail(KS_EINVAL, "ks_terms_create: obs %d reads [%d,%d) of a source with %d columns", k, el.index, el.index + span, src_dim[el.src]);
@@ -388,14 +520,15 @@ extern "C" int ks_observe(const KsTerms* t, ks_stream_t stream, const KsObserveI
   const KsTermsDesc& d = t->host;
   if (io->N < 0) return fail(KS_EINVAL, "ks_observe: negative env count");
   if (io->N == 0 || d.obs_dim == 0) return KS_OK;
-  const int src_dim[KS_SRC_COUNT] = {d.nq, d.nv, d.nv, d.nu, d.nu, d.command_dim, 1, d.nb * 3, d.nb * 4, d.nb * 6, 0};
+  const int src_dim[KS_SRC_COUNT] = {d.nq, d.nv, d.nv, d.nu, d.nu, d.command_dim, 1, d.nb * 3, d.nb * 4, d.nb * 6, 0, d.ns};
+  if (d.carry_dim > 0 && !io->carry) return fail(KS_EINVAL, "ks_observe: the stateful observations need a carry buffer");
   ObserveArgs a;
   std::memset(&a, 0, sizeof(a));
   bool needs_quat = false, needs_noise = false;
   for (int k = 0; k < d.obs_dim; ++k) {
     const KsObsElem& el = d.obs[k];
     if (el.src != KS_SRC_CONST && !io->src[el.src]) return fail(KS_EINVAL, "ks_observe: observation %d reads source %d, which is NULL", k, el.src);
-    needs_quat |= el.kind == KS_OBS_ROT_INV;
+    needs_quat |= el.kind == KS_OBS_ROT_INV || el.kind == KS_OBS_GRAVITY_EMA;
     needs_noise |= el.noise_kind != KS_NOISE_NONE;
   }
   if (needs_quat && !io->src[KS_SRC_QPOS]) return fail(KS_EINVAL, "ks_observe: qpos is required for body-frame observations");
@@ -405,6 +538,7 @@ extern "C" int ks_observe(const KsTerms* t, ks_stream_t stream, const KsObserveI
   for (int s = 0; s < KS_SRC_COUNT; ++s) { a.src[s] = io->src[s]; a.src_dim[s] = src_dim[s]; }
   a.zero_offset = io->zero_offset; a.bias = io->bias; a.noise_normal = io->noise_normal; a.noise_uniform = io->noise_uniform;
   a.rng = io->rng; a.obs = io->obs; a.noisy = io->noisy_obs; a.obs_dim = d.obs_dim; a.nq = d.nq; a.nu = d.nu;
+  a.carry = io->carry; a.fresh = io->fresh; a.carry_uniform = io->carry_uniform; a.carry_dim = d.carry_dim;
   const int64_t n = io->N * d.obs_dim;
   const int64_t grid = (n + 255) / 256;
   if (grid > 0x7fffffff) return fail(KS_ELIMIT, "ks_observe: too many elements");
@@ -457,7 +591,8 @@ extern "C" int ks_rewards(ks_stream_t stream, const KsRewardIO* io) {
   if (!io->done) return fail(KS_EINVAL, "ks_rewards: done is required");
   for (int j = 0; j < io->n_rewards; ++j) {
     const int k = io->rewards[j].kind;
-    if (k < KS_REW_STAY_ALIVE || k > KS_REW_AMP) return fail(KS_EINVAL, "ks_rewards: term %d: bad kind", j);
+    if (k < KS_REW_STAY_ALIVE || k > KS_REW_STATEFUL) return fail(KS_EINVAL, "ks_rewards: term %d: bad kind", j);
+    if (k == KS_REW_STATEFUL && (!io->stateful || io->rewards[j].norm < 0)) return fail(KS_EINVAL, "ks_rewards: term %d needs the scanned values", j);
     const bool needs_q = k == KS_REW_BASE_HEIGHT || k == KS_REW_BASE_HEIGHT_RANGE || k == KS_REW_UPRIGHT_POSE;
     const bool needs_v = k == KS_REW_UPRIGHT_ANGVEL || k == KS_REW_UPRIGHT_LINVEL;
     const bool needs_a = k >= KS_REW_ACTION_VEL && k <= KS_REW_ACTION_JERK;
@@ -471,4 +606,33 @@ extern "C" int ks_rewards(ks_stream_t stream, const KsRewardIO* io) {
   if (grid > 0x7fffffff) return fail(KS_ELIMIT, "ks_rewards: too many elements");
   hipLaunchKernelGGL(rewards_kernel, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, *io);
   return check_launch("ks_rewards");
+}
+
+extern "C" int ks_reward_scan(ks_stream_t stream, const KsRewardScanIO* io) {
+  using namespace ks;
+  if (!io) return fail(KS_EINVAL, "ks_reward_scan: null argument");
+  if (io->T < 0 || io->N < 0) return fail(KS_EINVAL, "ks_reward_scan: negative size");
+  if (io->n_scans < 0 || io->n_scans > KS_MAX_REWARD_SCANS) return fail(KS_ELIMIT, "ks_reward_scan: more than %d scans", KS_MAX_REWARD_SCANS);
+  if (io->T == 0 || io->N == 0 || io->n_scans == 0) return KS_OK;
+  if (!io->obs || !io->qvel || !io->done || !io->carry || !io->out) return fail(KS_EINVAL, "ks_reward_scan: obs, qvel, done, carry and out are required");
+  if (io->nv < 6) return fail(KS_EINVAL, "ks_reward_scan: the rewards read the velocity of a floating base");
+  for (int j = 0; j < io->n_scans; ++j) {
+    const KsRewardScanDesc& s = io->scans[j];
+    if (s.kind != KS_SCAN_FEET_AIR_TIME && s.kind != KS_SCAN_SPARSE_TARGET_HEIGHT) return fail(KS_EINVAL, "ks_reward_scan: scan %d: bad kind", j);
+    const bool feet = s.kind == KS_SCAN_FEET_AIR_TIME;
+    if (s.n < 1 || s.n > KS_MAX_SCAN_BODIES || s.n_contact < 1) return fail(KS_ELIMIT, "ks_reward_scan: scan %d: %d bodies (1..%d), %d contact rows", j, s.n, KS_MAX_SCAN_BODIES, s.n_contact);
+    if (s.contact_index < 0 || s.contact_index + s.n_contact * s.n > io->obs_dim) return fail(KS_EINVAL, "ks_reward_scan: scan %d: contact block outside the observation", j);
+    if (!feet && (s.position_index < 0 || s.position_index + 3 * s.n > io->obs_dim)) return fail(KS_EINVAL, "ks_reward_scan: scan %d: position block outside the observation", j);
+    if (s.slot < 0 || s.slot + (feet ? 3 : 1) > io->n_slots) return fail(KS_EINVAL, "ks_reward_scan: scan %d: output slot outside n_slots", j);
+    if (s.carry_index < 0 || s.carry_index + (feet ? 3 : 1) * s.n > io->carry_dim) return fail(KS_EINVAL, "ks_reward_scan: scan %d: carry outside the carry row", j);
+    if (feet) {
+      for (int idx : {s.linvel_cmd_index, s.angvel_cmd_index})
+        if (idx >= 0 && (!io->command || idx >= io->command_dim)) return fail(KS_EINVAL, "ks_reward_scan: scan %d: command index %d without such a command", j, idx);
+      if (!(s.air_steps > 0.f) || !(s.gnd_steps > 0.f)) return fail(KS_EINVAL, "ks_reward_scan: scan %d: the gait needs at least one step in the air and one on the ground", j);
+    }
+  }
+  const int64_t grid = (io->N + 255) / 256;
+  if (grid > 0x7fffffff) return fail(KS_ELIMIT, "ks_reward_scan: too many envs");
+  hipLaunchKernelGGL(reward_scan_kernel, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, *io);
+  return check_launch("ks_reward_scan");
 }

@@ -32,9 +32,12 @@ def compile_terms(model: KinematicModel, observations: Mapping[str, Observation]
                   terminate_on_nonfinite: bool = True):
     """Host-side compilation of the task's terms into the flat tables of KsTermsDesc (no GPU involved).
 
-    Returns (desc, obs_slices, sources_used, bias_std, reset_table)."""
+    Returns (desc, obs_slices, sources_used, bias_std, reset_table); `desc.carry_dim` is the length of the per-env
+    carry row of the stateful observations, laid out in dict order."""
     d = T.KsTermsDesc()
     d.nq, d.nv, d.nu, d.nb, d.command_dim = model.nq, model.nv, model.nu, model.nb, int(command_dim)
+    d.ns = model.ns
+    carry_at = 0
     obs_slices: dict[str, slice] = {}
     sources_used: set[int] = set()
     bias_std: list[float] = []
@@ -48,13 +51,18 @@ def compile_terms(model: KinematicModel, observations: Mapping[str, Observation]
             e = d.obs[k]
             e.kind, e.src, e.index, e.comp = el.kind, el.src, el.index, el.comp
             e.c0, e.c1, e.c2 = el.const
+            e.carry, e.stride = carry_at + el.carry, el.stride
+            e.q0, e.q1, e.q2 = el.q
             sources_used.add(el.src)
+            if el.kind == T.OBS_GRAVITY_EMA:
+                sources_used.add(T.SRC_QPOS)
             if noise is not None:
                 e.noise_kind, e.noise_mean, e.noise_scale = noise.kind, noise.mean, noise.scale
             bias_std.append(0.0 if obs.bias is None else float(obs.bias))
             k += 1
         obs_slices[name] = slice(k - len(elems), k)
-    d.obs_dim = k
+        carry_at += obs.carry_size(model)
+    d.obs_dim, d.carry_dim = k, carry_at
     if len(terminations) > T.KS_MAX_TERMS:
         raise _lib.KsError("too many terminations")
     for j, term in enumerate(terminations.values()):
@@ -83,19 +91,21 @@ class EnvTerms:
         self.command_dim = int(command_dim)
         d, self.obs_slices, self.sources_used, self.bias_std, self.reset_table = compile_terms(
             model, self.observations, self.terminations, self.resets, self.command_dim, terminate_on_nonfinite)
-        self.obs_dim, self.n_terms = int(d.obs_dim), int(d.n_terms)
+        self.obs_dim, self.n_terms, self.carry_dim = int(d.obs_dim), int(d.n_terms), int(d.carry_dim)
         self._handle = ctypes.c_void_p()
         _lib.check(lib.ks_terms_create(ctypes.byref(d), ctypes.byref(self._handle)))
 
     # ------------------------------------------------------------------ observations
     def observe(self, sources: Mapping[int, torch.Tensor | None], N: int, *, level: float = 1.0,
                 zero_offset=None, bias=None, noise_normal=None, noise_uniform=None, seed: int = 0, step: int = 0,
-                step_base=None,
+                step_base=None, carry=None, fresh=None, carry_uniform=None,
                 obs: torch.Tensor | None = None, noisy_obs: torch.Tensor | None = None):
+        """`carry` (N, carry_dim) is advanced in place; `fresh` (N) uint8 marks the envs whose carries are initialised
+        from the current state first (those that were just reset)."""
         m = self.model
         dims = {T.SRC_QPOS: m.nq, T.SRC_QVEL: m.nv, T.SRC_QACC: m.nv, T.SRC_CTRL: m.nu, T.SRC_LAST_ACTION: m.nu,
                 T.SRC_COMMAND: self.command_dim, T.SRC_TIME: 1, T.SRC_XPOS: m.nb * 3, T.SRC_XQUAT: m.nb * 4,
-                T.SRC_CVEL: m.nb * 6}
+                T.SRC_CVEL: m.nb * 6, T.SRC_CONTACT_DIST: m.ns}
         io = T.KsObserveIO()
         io.N, io.level = N, level
         for s, t in sources.items():
@@ -108,13 +118,19 @@ class EnvTerms:
         for name, t, shape in (("zero_offset", zero_offset, (N, m.nu)), ("bias", bias, (N, self.obs_dim)),
                                ("noise_normal", noise_normal, (N, self.obs_dim)),
                                ("noise_uniform", noise_uniform, (N, self.obs_dim)), ("obs", obs, (N, self.obs_dim)),
-                               ("noisy_obs", noisy_obs, (N, self.obs_dim))):
+                               ("noisy_obs", noisy_obs, (N, self.obs_dim)), ("carry", carry, (N, self.carry_dim)),
+                               ("carry_uniform", carry_uniform, (N, self.carry_dim))):
             if t is None:
                 continue
             _lib.require_cuda(t, dtype=torch.float32)
             if tuple(t.shape) != shape:
                 raise _lib.KsError(f"{name}: expected {shape}, got {tuple(t.shape)}")
             setattr(io, name, t.data_ptr())
+        if fresh is not None:
+            _lib.require_cuda(fresh, dtype=torch.uint8)
+            if tuple(fresh.shape) != (N,):
+                raise _lib.KsError(f"fresh: expected ({N},), got {tuple(fresh.shape)}")
+            io.fresh = fresh.data_ptr()
         io.rng = _rng(seed, step, step_base)
         _lib.check(self._lib.ks_observe(self._handle, _lib.current_stream(), ctypes.byref(io)))
         return obs, noisy_obs

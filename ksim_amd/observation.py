@@ -2,8 +2,9 @@
 
 Each class compiles to per-element descriptors that the fused observation kernel evaluates
 (`ks_observe`); ``noise`` / ``bias`` follow ksim/observation.py:89-145 (a float noise is additive
-Gaussian).  Stateful observations (delay buffers, the IMU-lag filter of ProjectedGravityObservation,
-contact observations) are not compiled here.
+Gaussian).  Stateful observations (delay buffers, the lag filter and bias of ProjectedGravityObservation) own a
+slice of a per-env carry row (`carry_size`); the kernel advances it in place every control step and initialises
+it for the envs that start an episode.
 """
 from __future__ import annotations
 
@@ -21,6 +22,9 @@ class ObsElem:
     index: int = 0
     comp: int = 0
     const: tuple = (0.0, 0.0, 0.0)
+    carry: int = 0      # offset inside the observation's own carry block
+    stride: int = 0
+    q: tuple = (0.0, 0.0, 0.0)
 
 
 @dataclass(frozen=True)
@@ -30,6 +34,10 @@ class Observation:
 
     def elements(self, model: KinematicModel, command_dim: int) -> list[ObsElem]:  # pragma: no cover
         raise NotImplementedError
+
+    def carry_size(self, model: KinematicModel) -> int:
+        """Floats of per-env carry (StatefulObservation.initial_carry, observation.py:148-181); 0 when stateless."""
+        return 0
 
     def get_name(self) -> str:
         name = type(self).__name__
@@ -146,11 +154,98 @@ class TimestepObservation(Observation):  # observation.py:705-713
 
 @dataclass(frozen=True)
 class ProjectedGravityObservation(Observation):
-    """Gravity in the base frame, rot(q_base)^-1 g: the stateless core of observation.py:355-442 (lag 0, no IMU bias)."""
+    """Gravity in the base frame, rot(q_base)^-1 g (observation.py:355-442; the base quaternion stands for the
+    framequat sensor).  With a lag range or an IMU bias the reading is the exponential average
+    x <- x lag + g_body (1 - lag) of the biased vector, lag and bias drawn per episode; without them it is stateless."""
     gravity: tuple = (0.0, 0.0, -9.81)
+    min_lag: float = 0.0
+    max_lag: float = 0.0
+    imu_bias: float = 0.0
+
+    def __post_init__(self):
+        for name in ("min_lag", "max_lag"):  # observation.py:372-373
+            if not 0.0 <= getattr(self, name) < 1.0:
+                raise ValueError(f"{name} must be in [0, 1)")
+        if self.imu_bias < 0.0:
+            raise ValueError("imu_bias must be non-negative")
+
+    @property
+    def stateful(self) -> bool:
+        return self.min_lag > 0.0 or self.max_lag > 0.0 or self.imu_bias > 0.0
+
+    def carry_size(self, m):
+        return 7 if self.stateful else 0  # x(3), lag, bias(3): ProjectedGravityCarry
 
     def elements(self, m, command_dim):
-        return _rot(T.SRC_CONST, 0, tuple(float(g) for g in self.gravity))
+        g = tuple(float(x) for x in self.gravity)
+        if not self.stateful:
+            return _rot(T.SRC_CONST, 0, g)
+        return [ObsElem(T.OBS_GRAVITY_EMA, T.SRC_CONST, 0, c, g, 0, 0, (self.min_lag, self.max_lag, self.imu_bias))
+                for c in range(3)]
+
+
+@dataclass(frozen=True)
+class _Delayed(Observation):
+    delay_steps: int = 1
+
+    def __post_init__(self):
+        if self.delay_steps < 1:  # observation.py:230
+            raise ValueError("delay_steps must be >= 1")
+
+    def _source(self, m):  # pragma: no cover
+        raise NotImplementedError
+
+    def carry_size(self, m):
+        return self.delay_steps * self._source(m)[2]
+
+    def elements(self, m, command_dim):
+        src, start, n = self._source(m)
+        return [ObsElem(T.OBS_DELAYED, src, start + i, self.delay_steps, carry=i, stride=n) for i in range(n)]
+
+
+@dataclass(frozen=True)
+class DelayedJointPositionObservation(_Delayed):  # observation.py:228-252 (minus zero_offset, like the live one)
+    def _source(self, m):
+        return T.SRC_QPOS, 7, m.nq - 7
+
+
+@dataclass(frozen=True)
+class DelayedJointVelocityObservation(_Delayed):  # observation.py:260-283
+    def _source(self, m):
+        return T.SRC_QVEL, 6, m.nv - 6
+
+
+@dataclass(frozen=True)
+class FeetContactObservation(Observation):
+    """1.0 where a foot's contact sphere touches the floor (observation.py:481-521 over geoms_colliding,
+    utils/mujoco.py:175-217).  `foot_left` / `foot_right` list contact-sphere indices of the model, equally many;
+    the output is the (n_spheres_per_foot, 2) block the reference emits, row-major."""
+    foot_left: tuple = ()
+    foot_right: tuple = ()
+
+    def __post_init__(self):
+        if len(self.foot_left) != len(self.foot_right) or not self.foot_left:
+            raise ValueError("foot_left and foot_right need the same, non-zero number of contact spheres")
+
+    @classmethod
+    def create(cls, *, physics_model, foot_left_body_names, foot_right_body_names, noise=None):
+        """Feet given by body name: every contact sphere attached to the named bodies."""
+        def spheres(names):
+            names = [names] if isinstance(names, str) else list(names)
+            ids = []
+            for n in names:
+                if n not in physics_model.body_names:
+                    raise ValueError(f"Body name {n} not found in model")
+                b = list(physics_model.body_names).index(n)
+                ids += [i for i, sb in enumerate(physics_model.sph_body) if int(sb) == b]
+            return tuple(ids)
+        return cls(foot_left=spheres(foot_left_body_names), foot_right=spheres(foot_right_body_names), noise=noise)
+
+    def elements(self, m, command_dim):
+        out = []
+        for l_, r_ in zip(self.foot_left, self.foot_right):
+            out += [ObsElem(T.OBS_CONTACT, T.SRC_CONTACT_DIST, int(l_)), ObsElem(T.OBS_CONTACT, T.SRC_CONTACT_DIST, int(r_))]
+        return out
 
 
 @dataclass(frozen=True)

@@ -55,7 +55,7 @@ class DeviceModel:
 _F32 = ("qpos", "qvel", "qacc_warmstart", "time", "last_ctrl", "action", "ctrl_in", "latency", "zero_offset", "kp",
         "kd", "ctrl_clip", "kp_scale", "kd_scale", "torque_limit_scale", "action_bias", "torque_bias", "action_noise",
         "torque_noise", "friction", "mass_scale", "qacc", "ctrl_out", "xpos", "xquat", "cvel", "dbg_M", "dbg_bias",
-        "dbg_qacc_smooth", "dbg_con_dist")
+        "dbg_qacc_smooth", "contact_dist")
 _I32 = ("solver_niter", "nefc")
 
 
@@ -69,7 +69,7 @@ def _expected_shapes(m: KinematicModel, N: int, S: int) -> dict:
         "torque_noise": (S, N, nu), "friction": (N,), "mass_scale": (N, nb), "env_mask": (N,), "qacc": (N, nv), "ctrl_out": (N, nu),
         "xpos": (N, nb * 3), "xquat": (N, nb * 4), "cvel": (N, nb * 6), "traj_ctrl": (N, nu),
         "traj_xpos": (N, nb * 3), "traj_xquat": (N, nb * 4), "solver_niter": (N,), "nefc": (N,),
-        "dbg_M": (N, nv * nv), "dbg_bias": (N, nv), "dbg_qacc_smooth": (N, nv), "dbg_con_dist": (N, ns),
+        "dbg_M": (N, nv * nv), "dbg_bias": (N, nv), "dbg_qacc_smooth": (N, nv), "contact_dist": (N, ns),
     }
 
 

@@ -7,19 +7,27 @@ time-major (T, N, ...) tensors.
 from __future__ import annotations
 
 import ctypes
+import math
 from dataclasses import dataclass
 from typing import Mapping
 
+import numpy as np
 import torch
 
 from . import _lib
 from . import _lib_terms as T
+from .scales import convert_to_scale
 from .types import RewardState, Trajectory
+
+
+def _reward_scale(rew, level: float) -> float:
+    """reward.scale.get_scale(curriculum_level) (rl.py:217): a float is a constant scale."""
+    return float(convert_to_scale(rew.scale).get_scale(level))
 
 
 @dataclass(frozen=True)
 class Reward:
-    scale: float = 1.0
+    scale: object = 1.0  # a float or a curriculum scale (ksim/scales.py)
 
     def descs(self) -> list[tuple]:  # [(suffix | None, kind, norm, p0, p1, p2)]  # pragma: no cover
         raise NotImplementedError
@@ -122,23 +130,188 @@ class AMPReward(Reward):  # ksim/task/amp.py:99-112
         return [(None, T.REW_AMP, 0, 0.0, 0.0, 0.0)]
 
 
+@dataclass(frozen=True)
+class StatefulReward(Reward):
+    """Rewards that scan the rollout with a per-env carry (rewards.py:127-163); evaluated by `ks_reward_scan`."""
+
+    def carry_size(self) -> int:  # pragma: no cover
+        raise NotImplementedError
+
+    def n_slots(self) -> int:  # pragma: no cover
+        raise NotImplementedError
+
+    def suffixes(self) -> tuple:
+        return (None,)
+
+    def scan_desc(self, obs_slices: Mapping[str, slice], command_slices: Mapping[str, slice], level: float) -> T.KsRewardScanDesc:
+        raise NotImplementedError  # pragma: no cover
+
+
+def _block(obs_slices, name, what):
+    if name not in obs_slices:
+        raise KeyError(f"{what} observation {name!r} is not among the observations: {sorted(obs_slices)}")
+    return obs_slices[name]
+
+
+@dataclass(frozen=True)
+class FeetAirTimeReward(StatefulReward):  # rewards.py:992-1085
+    gait_period: object = 1.0   # a float or a curriculum scale
+    air_time_percent: float = 0.5
+    ctrl_dt: float = 0.02
+    contact_obs: str = ""
+    num_feet: int = 2
+    bias: float = 0.0
+    alpha: float = 0.1
+    ground_penalty: float = 0.1
+    linvel_moving_threshold: float = 0.1
+    angvel_moving_threshold: float = math.radians(10)
+    linvel_cmd: str | None = None
+    angvel_cmd: str | None = None
+
+    def carry_size(self):
+        return 3 * self.num_feet  # air, ground and stationary-ground step counters per foot
+
+    def n_slots(self):
+        return 3
+
+    def suffixes(self):
+        return ("air", "gnd", "stationary_gnd")
+
+    def scan_desc(self, obs_slices, command_slices, level):
+        sl = _block(obs_slices, self.contact_obs, "contact")
+        width = sl.stop - sl.start
+        if width % self.num_feet:
+            raise ValueError(f"contact observation has {width} entries, not a multiple of {self.num_feet} feet")
+        f32 = np.float32
+        period = f32(convert_to_scale(self.gait_period).get_scale(level))
+        d = T.KsRewardScanDesc()
+        d.kind, d.n, d.n_contact, d.contact_index = T.SCAN_FEET_AIR_TIME, self.num_feet, width // self.num_feet, sl.start
+        # rewards.py:1049-1050, in float32 like the reference; numpy rounds half to even like jnp.round
+        d.air_steps = float(np.round(period * f32(self.air_time_percent) / f32(self.ctrl_dt)))
+        d.gnd_steps = float(np.round(period * f32(1.0 - self.air_time_percent) / f32(self.ctrl_dt)))
+        d.bias, d.ground_penalty = self.bias, self.ground_penalty
+        d.linvel_threshold, d.angvel_threshold = self.linvel_moving_threshold, self.angvel_moving_threshold
+        for field_, cmd in (("linvel_cmd_index", self.linvel_cmd), ("angvel_cmd_index", self.angvel_cmd)):
+            if cmd is None:
+                setattr(d, field_, -1)
+            else:
+                if cmd not in command_slices:
+                    raise KeyError(f"command {cmd!r} is not among the commands: {sorted(command_slices)}")
+                setattr(d, field_, command_slices[cmd].start)
+        return d
+
+
+@dataclass(frozen=True)
+class SparseTargetHeightReward(StatefulReward):  # rewards.py:1148-1192
+    contact_obs: str = ""
+    position_obs: str = ""
+    height: float = 0.0
+    num_bodies: int = 2
+    linvel_moving_threshold: float = 0.5
+    angvel_moving_threshold: float = math.radians(30)
+
+    def carry_size(self):
+        return self.num_bodies  # highest point of each body since it last touched down
+
+    def n_slots(self):
+        return 1
+
+    def scan_desc(self, obs_slices, command_slices, level):
+        sl, ps = _block(obs_slices, self.contact_obs, "contact"), _block(obs_slices, self.position_obs, "position")
+        width = sl.stop - sl.start
+        if width % self.num_bodies or ps.stop - ps.start != 3 * self.num_bodies:
+            raise ValueError("contact / position observations do not match num_bodies")
+        d = T.KsRewardScanDesc()
+        d.kind, d.n, d.n_contact = T.SCAN_SPARSE_TARGET_HEIGHT, self.num_bodies, width // self.num_bodies
+        d.contact_index, d.position_index, d.height = sl.start, ps.start, self.height
+        d.linvel_threshold, d.angvel_threshold = self.linvel_moving_threshold, self.angvel_moving_threshold
+        d.linvel_cmd_index = d.angvel_cmd_index = -1
+        return d
+
+
+def reward_carry_size(rewards: Mapping[str, Reward]) -> int:
+    return sum(r.carry_size() for r in rewards.values() if isinstance(r, StatefulReward))
+
+
+def _scan_stateful(trajectory, rewards, rewards_carry, obs_slices, command_slices, obs_key, level, Tn, N):
+    """Runs `ks_reward_scan` over the stateful terms; returns (values (n_slots, T, N), first slot per reward name)."""
+    stateful = {n: r for n, r in rewards.items() if isinstance(r, StatefulReward)}
+    if len(stateful) > T.KS_MAX_REWARD_SCANS:
+        raise _lib.KsError(f"at most {T.KS_MAX_REWARD_SCANS} stateful rewards")
+    if obs_slices is None:
+        raise _lib.KsError("stateful rewards read named observations: pass obs_slices (EnvTerms.obs_slices)")
+    obs = trajectory.obs[obs_key]
+    _lib.require_cuda(obs, dtype=torch.float32)
+    if obs.dim() != 3 or tuple(obs.shape[:2]) != (Tn, N):
+        raise _lib.KsError(f"observation leaf has shape {tuple(obs.shape)}, expected ({Tn}, {N}, obs_dim)")
+    io = T.KsRewardScanIO()
+    io.T, io.N, io.obs_dim, io.nv = Tn, N, obs.shape[-1], trajectory.qvel.shape[-1]
+    slots, carry_at, first = 0, 0, {}
+    for j, (name, r) in enumerate(stateful.items()):
+        d = r.scan_desc(obs_slices, command_slices or {}, level)
+        d.slot, d.carry_index = slots, carry_at
+        io.scans[j] = d
+        first[name] = slots
+        slots += r.n_slots()
+        carry_at += r.carry_size()
+    io.n_scans, io.n_slots, io.carry_dim = len(stateful), slots, carry_at
+    if rewards_carry is None:
+        rewards_carry = torch.zeros((N, carry_at), dtype=torch.float32, device=obs.device)  # initial_carry: zeros
+    _lib.require_cuda(rewards_carry, dtype=torch.float32)
+    if tuple(rewards_carry.shape) != (N, carry_at):
+        raise _lib.KsError(f"reward carry has shape {tuple(rewards_carry.shape)}, expected {(N, carry_at)}")
+    cmd = trajectory.command.get("_buffer") if trajectory.command else None
+    if cmd is not None:
+        _lib.require_cuda(cmd, dtype=torch.float32)
+        if cmd.dim() != 3 or tuple(cmd.shape[:2]) != (Tn, N):
+            raise _lib.KsError(f"command leaf has shape {tuple(cmd.shape)}, expected ({Tn}, {N}, command_dim)")
+        io.command_dim, io.command = cmd.shape[-1], cmd.data_ptr()
+    out = torch.empty((slots, Tn, N), dtype=torch.float32, device=obs.device)
+    done = trajectory.done.view(torch.uint8) if trajectory.done.dtype == torch.bool else trajectory.done
+    io.obs, io.qvel, io.done = obs.data_ptr(), trajectory.qvel.data_ptr(), done.data_ptr()
+    io.carry, io.out = rewards_carry.data_ptr(), out.data_ptr()
+    _lib.check(_lib.load().ks_reward_scan(_lib.current_stream(), ctypes.byref(io)))
+    return out, first, rewards_carry
+
+
 def get_rewards(trajectory: Trajectory, rewards: Mapping[str, Reward], clip_min: float | None = None,
-                clip_max: float | None = None, want_components: bool = True) -> RewardState:
-    """Reward total and components over a (T, N) rollout (ksim/task/rl.py:189-245)."""
+                clip_max: float | None = None, want_components: bool = True, *, rewards_carry: torch.Tensor | None = None,
+                obs_slices: Mapping[str, slice] | None = None, command_slices: Mapping[str, slice] | None = None,
+                obs_key: str = "obs", level: float = 1.0) -> RewardState:
+    """Reward total and components over a (T, N) rollout (ksim/task/rl.py:189-245).
+
+    Stateful rewards read their observations by name out of the concatenated vector `trajectory.obs[obs_key]`
+    (`obs_slices` maps names to columns) and advance `rewards_carry` (N, reward_carry_size(rewards)) in place; the
+    returned state holds it under `carry["_buffer"]`.  Commands for them come as `trajectory.command["_buffer"]`
+    (T, N, command_dim) with `command_slices`."""
     lib = _lib.load()
     done = trajectory.done
     Tn, N = done.shape
     io = T.KsRewardIO()
     io.T, io.N = Tn, N
     names = []
+    scanned, first_slot = None, {}
+    if any(isinstance(r, StatefulReward) for r in rewards.values()):
+        scanned, first_slot, rewards_carry = _scan_stateful(trajectory, rewards, rewards_carry, obs_slices, command_slices,
+                                                           obs_key, float(level), Tn, N)
+        io.stateful = scanned.data_ptr()
     for name, rew in rewards.items():
         sign = -1.0 if rew.is_penalty else 1.0
+        if isinstance(rew, StatefulReward):
+            for k, suffix in enumerate(rew.suffixes()):
+                j = len(names)
+                if j >= T.KS_MAX_REWARD_TERMS:
+                    raise _lib.KsError("too many reward terms")
+                d = io.rewards[j]
+                d.kind, d.norm, d.scale = T.REW_STATEFUL, first_slot[name] + k, sign * _reward_scale(rew, level)
+                names.append(name if suffix is None else f"{name}/{suffix}")
+            continue
         for suffix, kind, norm, p0, p1, p2 in rew.descs():
             j = len(names)
             if j >= T.KS_MAX_REWARD_TERMS:
                 raise _lib.KsError("too many reward terms")
             d = io.rewards[j]
-            d.kind, d.norm, d.scale, d.p0, d.p1, d.p2 = kind, norm, sign * float(rew.scale), p0, p1, p2
+            d.kind, d.norm, d.scale, d.p0, d.p1, d.p2 = kind, norm, sign * _reward_scale(rew, level), p0, p1, p2
             names.append(name if suffix is None else f"{name}/{suffix}")  # rl.py:223-226
     io.n_rewards = len(names)
     if not names:
@@ -179,4 +352,4 @@ def get_rewards(trajectory: Trajectory, rewards: Mapping[str, Reward], clip_min:
     io.components, io.total = _lib.ptr(comps).value, _lib.ptr(total).value
     _lib.check(lib.ks_rewards(_lib.current_stream(), ctypes.byref(io)))
     components = {} if comps is None else {n: comps[j] for j, n in enumerate(names)}
-    return RewardState(total=total, components=components, carry={})
+    return RewardState(total=total, components=components, carry={} if rewards_carry is None else {"_buffer": rewards_carry})

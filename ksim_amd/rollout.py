@@ -20,7 +20,7 @@ from .engine import HipEngine
 from .env_terms import EnvTerms, sample_action
 from .mlp import MLP
 from .physics import DeviceModel
-from .rewards import Reward, get_rewards
+from .rewards import Reward, get_rewards, reward_carry_size
 from .types import PhysicsState, RewardState, Trajectory
 
 
@@ -47,6 +47,8 @@ class RolloutEnvState:  # ksim/task/rl.py:110-123, batched
         self.obs_bias = obs_bias
         self.seed = int(seed)
         self.step = 0
+        self.obs_carry = None     # (N, carry_dim) carries of the stateful observations (rl.py:118), made on first use
+        self.reward_carry = None  # (N, reward carry size) carries of the stateful rewards (rl.py:119)
         N = physics_state.data.qpos.shape[0]
         self.episode_length = torch.zeros(N, dtype=torch.int32, device=physics_state.data.qpos.device)
 
@@ -86,10 +88,14 @@ class Rollout:
         step, step_base = (t, self.step_base) if _relative_step else (env.step, None)
         src = {T.SRC_QPOS: d.qpos, T.SRC_QVEL: d.qvel, T.SRC_QACC: d.qacc, T.SRC_CTRL: d.ctrl,
                T.SRC_LAST_ACTION: ps.last_ctrl, T.SRC_COMMAND: env.commands, T.SRC_TIME: d.time, T.SRC_XPOS: d.xpos,
-               T.SRC_XQUAT: d.xquat, T.SRC_CVEL: d.cvel}
+               T.SRC_XQUAT: d.xquat, T.SRC_CVEL: d.cvel, T.SRC_CONTACT_DIST: d.contact_dist}
+        self._prepare_env(env)
+        # the reset mask still holds the envs that the previous control step reset: their carries start afresh
         c.terms.observe(src, self.N, level=level, zero_offset=ps.zero_offset, bias=env.obs_bias,
                         noise_normal=noise.get("obs_normal"), noise_uniform=noise.get("obs_uniform"), seed=env.seed,
-                        step=step, step_base=step_base, obs=self.obs[t], noisy_obs=self.noisy_obs[t])
+                        step=step, step_base=step_base, obs=self.obs[t], noisy_obs=self.noisy_obs[t],
+                        carry=env.obs_carry, fresh=self.reset_mask if c.terms.carry_dim else None,
+                        carry_uniform=noise.get("obs_carry_uniform"))
         c.actor(self.noisy_obs[t], out=self.mean)           # actor reads the noisy copy (walking.py:592-595)
         if c.critic is not None:
             c.critic(self.obs[t], out=self.values[t])       # critic reads the clean one (walking.py:626-638)
@@ -122,9 +128,7 @@ class Rollout:
         for t in range(self.T):
             self.step_engine(env, t, level)
         traj = self.trajectory()
-        rewards = get_rewards(traj, self.c.rewards, self.c.reward_clip_min, self.c.reward_clip_max,
-                              want_components=False)
-        return traj, rewards
+        return traj, self._rewards(traj, env, level)
 
     def _unroll_graph(self, env: RolloutEnvState, level: float) -> tuple[Trajectory, RewardState]:
         if self.c.engine.data.drop_action_prob * float(level) > 0:
@@ -133,14 +137,14 @@ class Rollout:
         if self._graph is None or self._graph[0] != key:
             self.step_base.fill_(env.step)
             self.c.engine.prepare(self.step_base.device)
+            self._prepare_env(env)
             torch.cuda.synchronize()
             g = torch.cuda.CUDAGraph()
             with torch.cuda.graph(g):
                 for t in range(self.T):
                     self.step_engine(env, t, level, _relative_step=True)
                 traj = self.trajectory()
-                rewards = get_rewards(traj, self.c.rewards, self.c.reward_clip_min, self.c.reward_clip_max,
-                                      want_components=False)
+                rewards = self._rewards(traj, env, level)
                 self.step_base += self.T
             self._graph = (key, g, traj, rewards)
         elif int(env.step) != self._graph_step:
@@ -150,6 +154,23 @@ class Rollout:
         env.step += self.T
         self._graph_step = int(env.step)
         return traj, rewards
+
+    def _prepare_env(self, env: RolloutEnvState) -> None:
+        """Carry buffers of an env state seen for the first time (never inside a graph capture: `_unroll_graph`
+        calls this before it starts capturing)."""
+        if self.c.terms.carry_dim and env.obs_carry is None:
+            env.obs_carry = torch.zeros(self.N, self.c.terms.carry_dim, dtype=torch.float32, device=self.done.device)
+            self.reset_mask.fill_(1)  # every env starts an episode: the first observation initialises all carries
+        n = reward_carry_size(self.c.rewards)
+        if n and env.reward_carry is None:
+            env.reward_carry = torch.zeros(self.N, n, dtype=torch.float32, device=self.done.device)
+
+    def _rewards(self, traj: Trajectory, env: RolloutEnvState, level: float, want_components: bool = False) -> RewardState:
+        """get_rewards over the recorded rollout; the carries of stateful rewards live in the env state (rl.py:1640-1650)."""
+        self._prepare_env(env)
+        return get_rewards(traj, self.c.rewards, self.c.reward_clip_min, self.c.reward_clip_max,
+                           want_components=want_components, rewards_carry=env.reward_carry,
+                           obs_slices=self.c.terms.obs_slices, level=level)
 
     def trajectory(self) -> Trajectory:
         names = list(self.c.terms.terminations)

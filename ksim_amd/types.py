@@ -23,6 +23,7 @@ class PhysicsData:
     xpos: torch.Tensor            # (N, nb*3)
     xquat: torch.Tensor           # (N, nb*4)
     cvel: torch.Tensor            # (N, nb*6)
+    contact_dist: torch.Tensor | None = None  # (N, ns) sphere-floor distance of the last collision pass (contact.dist)
 
 
 @dataclass

@@ -260,3 +260,76 @@ def force_push_event(params, state, dt, u, level_scale):
         left = params["interval_range"][0] + u[8] * (params["interval_range"][1] - params["interval_range"][0])
         dur = params["duration_range"][0] + u[9] * (params["duration_range"][1] - params["duration_range"][0])
     return applied, (float(left), float(dur), wrench)
+
+
+# ------------------------------------------------------------------ stateful observations, contact observations
+def feet_contact_observation(contact_dist, foot_left, foot_right):
+    """FeetContactObservation (ksim/observation.py:481-521) on sphere-floor contacts: geoms_colliding
+    (ksim/utils/mujoco.py:175-217) is "a contact of the pair exists with negative distance".  Returns (c, 2)."""
+    d = np.asarray(contact_dist)
+    return np.stack([d[list(foot_left)] < 0.0, d[list(foot_right)] < 0.0], axis=-1).astype(np.float64)
+
+
+def delayed_observation(carry, current, zero_offset=None):
+    """Delayed joint observation (observation.py:228-283): emits the oldest slot, rolls, appends the current value.
+    carry (delay, n).  The initial carry is the current value tiled (observation.py:231-236)."""
+    carry = np.asarray(carry, dtype=np.float64)
+    out = carry[0] - (0.0 if zero_offset is None else np.asarray(zero_offset))
+    new = np.roll(carry, -1, axis=0)
+    new[-1] = current
+    return out, new
+
+
+def euler_to_quat(rpy):
+    """Roll-pitch-yaw to a wxyz quaternion, yaw applied last (R = Rz Ry Rx)."""
+    r, p, y = (0.5 * float(a) for a in rpy)
+    cr, sr, cp, sp, cy, sy = np.cos(r), np.sin(r), np.cos(p), np.sin(p), np.cos(y), np.sin(y)
+    return np.array([cr * cp * cy + sr * sp * sy, sr * cp * cy - cr * sp * sy, cr * sp * cy + sr * cp * sy,
+                     cr * cp * sy - sr * sp * cy])
+
+
+def projected_gravity_ema(x, lag, bias, quat, gravity=(0.0, 0.0, -9.81)):
+    """ProjectedGravityObservation.observe_stateful (observation.py:421-442): gravity in the sensor frame, rotated by
+    the bias quaternion, averaged exponentially."""
+    g = rotate_vector_by_quat(np.asarray(gravity, dtype=np.float64)[None], np.asarray(quat, dtype=np.float64)[None], inverse=True)
+    g = rotate_vector_by_quat(g, euler_to_quat(bias)[None])[0]
+    return np.asarray(x) * lag + g * (1.0 - lag)
+
+
+# ------------------------------------------------------------------ stateful rewards
+def feet_air_time_reward(contact_tcn, qvel_t, done_t, carry, *, air_steps, gnd_steps, bias=0.0, ground_penalty=0.1,
+                         linvel_threshold=0.1, angvel_threshold=np.radians(10), lin_cmd_t=None, ang_cmd_t=None):
+    """FeetAirTimeReward.get_reward_stateful for one env (ksim/rewards.py:1020-1085).  contact (T, c, n) of 0/1 values,
+    carry = (air, gnd, stationary) integer counters per foot.  Returns ({air, gnd, stationary_gnd}: (T,), carry)."""
+    contact_tn = (np.asarray(contact_tcn) > 0.5).any(axis=-2)
+    T_ = contact_tn.shape[0]
+    lin = (np.linalg.norm(qvel_t[:, :2], axis=-1) > linvel_threshold) if lin_cmd_t is None else np.abs(lin_cmd_t) > linvel_threshold
+    ang = (qvel_t[:, 5] > angvel_threshold) if ang_cmd_t is None else np.abs(ang_cmd_t) > angvel_threshold
+    moving = (lin | ang) & ~np.asarray(done_t, dtype=bool)
+    air, gnd, sta = (np.asarray(c, dtype=np.int64).copy() for c in carry)
+    out = {"air": np.zeros(T_), "gnd": np.zeros(T_), "stationary_gnd": np.zeros(T_)}
+    for t in range(T_):
+        c, mv = contact_tn[t], moving[t]
+        air = np.where(~c & mv, air + 1, 0)
+        gnd = np.where(c & mv, gnd + 1, 0)
+        sta = np.where(c & ~mv, sta + 1, 0)
+        out["air"][t] = np.where(air < air_steps, air / air_steps + bias, 0.0).max()
+        out["gnd"][t] = np.where(gnd < gnd_steps, gnd / gnd_steps + bias, -ground_penalty).max()
+        out["stationary_gnd"][t] = (np.clip(sta / gnd_steps, 0.0, 1.0) + bias).max()
+    return out, (air, gnd, sta)
+
+
+def sparse_target_height_reward(contact_tcn, position_tn3, qvel_t, done_t, carry, *, height, linvel_threshold=0.5,
+                                angvel_threshold=np.radians(30)):
+    """SparseTargetHeightReward.get_reward_stateful for one env (ksim/rewards.py:1160-1192): on touch-down a body earns
+    the greatest height it reached since its last contact, capped at `height`."""
+    contact_tn = (np.asarray(contact_tcn) > 0.5).any(axis=-2)
+    still = ((np.linalg.norm(qvel_t[:, :2], axis=-1) < linvel_threshold) & (qvel_t[:, 5] < angvel_threshold)) | np.asarray(done_t, dtype=bool)
+    best = np.asarray(carry, dtype=np.float64).copy()
+    out = np.zeros(contact_tn.shape[0])
+    for t in range(contact_tn.shape[0]):
+        rew = np.minimum(np.where(contact_tn[t], best, 0.0), height)
+        best = np.maximum(best, position_tn3[t][:, 2])
+        best = np.where(still[t] | contact_tn[t], 0.0, best)
+        out[t] = rew.max()
+    return out, best

@@ -51,7 +51,7 @@ def test_forward_quantities_match_oracle(setup):
                mass_scale=t32(ms), qacc=zeros(N, m.nv), xpos=zeros(N, m.nb * 3), xquat=zeros(N, m.nb * 4),
                cvel=zeros(N, m.nb * 6), nefc=zeros(N, dtype=torch.int32), solver_niter=zeros(N, dtype=torch.int32),
                dbg_M=zeros(N, m.nv * m.nv), dbg_bias=zeros(N, m.nv), dbg_qacc_smooth=zeros(N, m.nv),
-               dbg_con_dist=zeros(N, m.ns))
+               contact_dist=zeros(N, m.ns))
     q0 = buf["qpos"].clone()
     physics.forward(dm, buf)
     g = {k: v.cpu().numpy() for k, v in buf.items()}
@@ -62,7 +62,7 @@ def test_forward_quantities_match_oracle(setup):
         err = rel_err(g[got], want[ref]).max()
         assert err <= tol, f"{name}.{ref}: rel err {err:.2e} > {tol}"
     if m.ns:
-        assert np.abs(g["dbg_con_dist"] - want["con_dist"]).max() < 1e-6
+        assert np.abs(g["contact_dist"] - want["con_dist"]).max() < 1e-6
         assert np.array_equal(g["nefc"], want["nefc"]), "active contact sets differ"  # integer: bit-exact
         assert (want["nefc"] > 0).sum() >= N // 4
 

@@ -17,7 +17,7 @@ def t32(a):
     return torch.tensor(np.asarray(a), dtype=torch.float32, device=DEV).contiguous()
 
 
-def build(N, T, seed=0, min_height=0.9, events=None):
+def build(N, T, seed=0, min_height=0.9, events=None, gait=False):
     from ksim_amd import actuators, engine, model as km, observation as ob, physics, randomization as rnd, resets as rs
     from ksim_amd import rewards as rw, terminations as tm
     from ksim_amd.env_terms import EnvTerms
@@ -37,6 +37,14 @@ def build(N, T, seed=0, min_height=0.9, events=None):
                     "g": ob.ProjectedGravityObservation(noise=0.01),
                     "w": ob.BaseAngularVelocityObservation(in_robot_frame=True, noise=0.01),
                     "a": ob.LastActionObservation(), "c": ob.CommandObservation()}
+    if gait:  # what a walking task adds: contact flags, foot positions, sensor lag, and the gait rewards over them
+        feet = [b for b in range(m.nb) if any(int(sb) == b for sb in m.sph_body)]
+        left = tuple(i for i, sb in enumerate(m.sph_body) if int(sb) == feet[0])
+        right = tuple(i for i, sb in enumerate(m.sph_body) if int(sb) == feet[1])
+        observations.update({"contact": ob.FeetContactObservation(foot_left=left, foot_right=right),
+                             "feet_pos": ob.BodyPositionObservation(body_ids=tuple(feet)),
+                             "old_jp": ob.DelayedJointPositionObservation(delay_steps=2),
+                             "imu_g": ob.ProjectedGravityObservation(min_lag=0.2, max_lag=0.6, imu_bias=0.02)})
     terms = EnvTerms(m, observations, {"min_height": tm.MinimumHeightTermination(min_height)}, resets, command_dim=2)
     dims = (terms.obs_dim, 64, 64, m.nu)
     ws = [rng.normal(scale=1 / np.sqrt(i), size=(o, i)).astype(np.float32) for i, o in zip(dims[:-1], dims[1:])]
@@ -49,6 +57,11 @@ def build(N, T, seed=0, min_height=0.9, events=None):
     log_std = np.full(m.nu, -2.0, np.float32)
     rewards = {"stay_alive": rw.StayAliveReward(scale=1.0), "height": rw.BaseHeightReward(scale=0.5, height_target=1.0),
                "vel": rw.ActionVelocityPenalty(scale=0.01)}
+    if gait:
+        rewards.update({"air_time": rw.FeetAirTimeReward(scale=1.0, gait_period=0.2, air_time_percent=0.5, ctrl_dt=0.02,
+                                                         contact_obs="contact", linvel_moving_threshold=0.05),
+                        "step_height": rw.SparseTargetHeightReward(scale=2.0, contact_obs="contact", position_obs="feet_pos",
+                                                                   height=0.1, linvel_moving_threshold=0.02)})
     consts = RolloutConstants(physics_model=dm, engine=eng, terms=terms, rewards=rewards,
                               actor=MLP(ws, bs, dtype="f32"), critic=MLP(cws, cbs, dtype="f32"), log_std=t32(log_std))
     gen = torch.Generator(device=DEV); gen.manual_seed(seed)
@@ -133,6 +146,10 @@ def test_rollout_matches_oracle_composition():
             last[e] = 0.0
         if t == 0:
             assert done.sum() == low.sum()
+        # sphere-floor distances of the last collision pass (data.contact.dist): of the last substep for the envs that go
+        # on, of the forward pass over the fresh state for the envs that were reset
+        cd = np.array([np.array(d.con_dist) for d in datas])
+        np.testing.assert_allclose(ps.data.contact_dist.cpu().numpy(), cd, rtol=0, atol=2e-5)
     # live state after the rollout: reset envs restarted, others continued
     q = np.array([np.array(d.qpos) for d in datas])
     assert rel_err(ps.data.qpos.cpu().numpy(), q).max() <= 1e-3
@@ -264,3 +281,57 @@ def test_events_in_the_rollout_fire_and_restart_with_the_episode():
     assert torch.equal(ps.event_states["push"], ps.event_states["_buffer"][0])  # named views of the one buffer
     moved = (ro.qvel[0] - ro0.qvel[0]).abs().amax(dim=1).cpu().numpy() > 1e-4
     assert fired.any() and np.array_equal(moved, fired), "exactly the envs whose events fired differ from the run without events"
+
+
+def test_gait_terms_in_the_rollout_and_under_graph_replay():
+    """Contact flags, delayed and lagged observations and the stateful gait rewards inside the environment loop: the
+    rewards recomputed by the oracle from the recorded rollout, carried over three rollouts, and the graph replay
+    equal to the eager loop bit for bit."""
+    N, T = 64, 8
+    runs = []
+    for use_graph in (False, True):
+        m, c, rnd_, _, ro, EnvState = build(N, T, seed=7, min_height=0.8, gait=True)
+        ps = c.engine.reset(c.physics_model, 1.0, 3, N, rnd_)
+        env = EnvState(ps, rnd_, torch.zeros(N, 2, device=DEV), None, seed=9)
+        sl = c.terms.obs_slices
+        carries = [((np.zeros(2, int),) * 3, np.zeros(2)) for _ in range(N)]
+        snaps = []
+        for it in range(4):
+            traj, rew = ro.unroll(env, graph=use_graph)
+            torch.cuda.synchronize()
+            snaps.append((traj.obs["obs"].clone(), rew.total.clone(), env.obs_carry.clone(), env.reward_carry.clone()))
+            if use_graph:
+                continue
+            obs, qvel, done = traj.obs["obs"].cpu().numpy(), traj.qvel.cpu().numpy(), traj.done.cpu().numpy().astype(bool)
+            from ksim_amd.rewards import get_rewards
+            full = get_rewards(traj, c.rewards, want_components=True, obs_slices=sl) if it == 0 else None  # from a zero carry
+            xpos = traj.xpos.cpu().numpy().reshape(T, N, m.nb, 3)
+            feet = [b for b in range(m.nb) if any(int(sb) == b for sb in m.sph_body)]
+            # the recorded observation is taken before the step, the recorded xpos after it: row t+1 of the former
+            # shows the bodies of row t of the latter, unless the env was reset in between
+            for t in range(T - 1):
+                keep = ~done[t]
+                np.testing.assert_allclose(obs[t + 1][keep][:, sl["feet_pos"]].reshape(-1, 2, 3), xpos[t][keep][:, feet], atol=1e-6)
+            assert set(np.unique(obs[..., sl["contact"]])) <= {0.0, 1.0}
+            touched = obs[..., sl["contact"]].mean() if it == 0 else max(touched, obs[..., sl["contact"]].mean())
+            want = np.zeros((T, N))
+            for e in range(N):
+                a0, h0 = carries[e] if not done[-1, e] else ((np.zeros(2, int),) * 3, np.zeros(2))
+                con = obs[:, e, sl["contact"]].reshape(T, -1, 2)
+                a, a1 = ot.feet_air_time_reward(con, qvel[:, e], done[:, e], a0, air_steps=5.0, gnd_steps=5.0, linvel_threshold=0.05)
+                h, h1 = ot.sparse_target_height_reward(con, obs[:, e, sl["feet_pos"]].reshape(T, 2, 3), qvel[:, e], done[:, e], h0,
+                                                       height=0.1, linvel_threshold=0.02)
+                carries[e] = (a1, h1)
+                want[:, e] = a["air"] + a["gnd"] + a["stationary_gnd"] + 2.0 * h
+            if full is not None:
+                got = sum(v for k, v in full.components.items() if k.startswith(("air_time", "step_height"))).cpu().numpy()
+                np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-5)
+            else:  # later rollouts: the carried counters enter; check through the carry buffer
+                cr = env.reward_carry.cpu().numpy()
+                np.testing.assert_allclose(cr[:, :6], [np.concatenate(cv[0]) for cv in carries])
+                np.testing.assert_allclose(cr[:, 6:8], [cv[1] for cv in carries], rtol=1e-6, atol=1e-7)
+        assert use_graph or 0.05 < touched < 1.0, "the feet never touched the floor: the contact terms were not exercised"
+        runs.append(snaps)
+    for it, (a, b) in enumerate(zip(*runs)):
+        for x, y, name in zip(a, b, ("observations", "reward", "observation carry", "reward carry")):
+            assert torch.equal(x, y), f"replay {it}: {name} differs from the eager rollout"

@@ -285,3 +285,142 @@ def test_amp_reward_from_discriminator_logits():
                               action=None, done=done, success=done.clone(), timestep=None)
     with pytest.raises(ValueError, match="auxiliary output is missing"):
         rw.get_rewards(traj_missing, {"amp_reward": rw.AMPReward(scale=0.5)})
+
+
+def test_stateful_and_contact_observations():
+    """Delay lines, the lagged and biased gravity reading and feet contact flags over several control steps, with
+    some envs restarting in between (their carries are initialised from the state they restart in)."""
+    from ksim_amd import _lib_terms as T, model as km, observation as ob
+    from ksim_amd.env_terms import EnvTerms
+
+    m = km.kbot_scale_model()
+    N, steps = 19, 7
+    rng = np.random.default_rng(3)
+    observations = {
+        "joint_position": ob.JointPositionObservation(),
+        "delayed_position": ob.DelayedJointPositionObservation(delay_steps=3, noise=0.01),
+        "gravity": ob.ProjectedGravityObservation(min_lag=0.3, max_lag=0.8, imu_bias=0.05),
+        "contact": ob.FeetContactObservation(foot_left=(0, 1, 2, 3), foot_right=(4, 5, 6, 7)),
+        "delayed_velocity": ob.DelayedJointVelocityObservation(delay_steps=1),
+    }
+    terms = EnvTerms(m, observations, {}, [])
+    nj = m.nu
+    assert terms.carry_dim == 3 * nj + 7 + nj and terms.obs_dim == nj + nj + 3 + 8 + nj
+    K, C = terms.obs_dim, terms.carry_dim
+    zero = rng.normal(size=(N, nj)) * 0.01
+    carry = torch.full((N, C), float("nan"), device=DEV)  # never read before it is initialised
+    # oracle-side carries
+    dpos, dvel = [None] * N, [None] * N
+    gx, glag, gbias = np.zeros((N, 3)), np.zeros(N), np.zeros((N, 3))
+    sl = terms.obs_slices
+    for k in range(steps):
+        s = _state(m, N, 100 + k)
+        dist = rng.normal(size=(N, m.ns)) * 0.01
+        fresh = np.ones(N, bool) if k == 0 else (rng.random(N) < 0.3 if k in (3, 4) else np.zeros(N, bool))
+        cu = rng.random((N, C))
+        src = {T.SRC_QPOS: t32(s["qpos"]), T.SRC_QVEL: t32(s["qvel"]), T.SRC_CONTACT_DIST: t32(dist)}
+        obs = torch.empty(N, K, device=DEV)
+        terms.observe(src, N, zero_offset=t32(zero), carry=carry, fresh=torch.from_numpy(fresh.astype(np.uint8)).to(DEV),
+                      carry_uniform=t32(cu), obs=obs)
+        got = obs.cpu().numpy()
+        g0 = 3 * nj  # the gravity carry follows the position delay line: x(3), lag, bias(3)
+        for e in range(N):
+            q, v = s["qpos"][e], s["qvel"][e]
+            if fresh[e]:
+                dpos[e], dvel[e] = np.tile(q[7:], (3, 1)), np.tile(v[6:], (1, 1))
+                gx[e] = 0.0
+                glag[e] = 0.3 + cu[e, g0 + 3] * 0.5
+                gbias[e] = -0.05 + cu[e, g0 + 4:g0 + 7] * 0.1
+            want_dp, dpos[e] = ot.delayed_observation(dpos[e], q[7:], zero[e])
+            want_dv, dvel[e] = ot.delayed_observation(dvel[e], v[6:])
+            gx[e] = ot.projected_gravity_ema(gx[e], glag[e], gbias[e], q[3:7])
+            np.testing.assert_allclose(got[e, sl["delayed_position"]], want_dp, rtol=1e-6, atol=1e-6)
+            np.testing.assert_allclose(got[e, sl["delayed_velocity"]], want_dv, rtol=1e-6, atol=1e-6)
+            np.testing.assert_allclose(got[e, sl["gravity"]], gx[e], rtol=1e-5, atol=1e-5)
+            want_c = ot.feet_contact_observation(dist[e].astype(np.float32), (0, 1, 2, 3), (4, 5, 6, 7))
+            assert np.array_equal(got[e, sl["contact"]].reshape(4, 2), want_c)
+            np.testing.assert_allclose(got[e, sl["joint_position"]], q[7:] - zero[e], rtol=1e-6, atol=1e-6)
+    # the carry row holds what the reference keeps: delay slots oldest first, then x, lag, bias
+    cr = carry.cpu().numpy()
+    np.testing.assert_allclose(cr[:, :3 * nj].reshape(N, 3, nj), np.array(dpos), rtol=1e-6, atol=1e-6)
+    np.testing.assert_allclose(cr[:, g0 + 3], glag, rtol=1e-6)
+    # Philox initial carries: lag and bias inside their ranges, reproducible for a seed
+    c1, c2 = torch.zeros(N, C, device=DEV), torch.zeros(N, C, device=DEV)
+    ones = torch.ones(N, dtype=torch.uint8, device=DEV)
+    terms.observe(src, N, carry=c1, fresh=ones, seed=3, step=5, obs=obs)
+    terms.observe(src, N, carry=c2, fresh=ones, seed=3, step=5, obs=obs)
+    assert torch.equal(c1, c2)
+    lag, bias = c1[:, g0 + 3], c1[:, g0 + 4:g0 + 7]
+    assert ((lag >= 0.3) & (lag <= 0.8)).all() and (bias.abs() <= 0.05).all() and lag.std() > 0.05
+    with pytest.raises(Exception, match="carry"):
+        terms.observe(src, N, obs=obs)
+
+
+def test_stateful_rewards_scan_against_oracle():
+    """FeetAirTimeReward and SparseTargetHeightReward over two consecutive rollouts (the carry continues, and restarts
+    for the envs whose rollout ends finished), mixed with stateless terms, total and components."""
+    from ksim_amd import rewards as rw
+    from ksim_amd.scales import LinearScale
+    from ksim_amd.types import Trajectory
+
+    Tn, N, nq, nv, nu = 24, 33, 27, 26, 20
+    rng = np.random.default_rng(12)
+    obs_slices = {"pad": slice(0, 5), "contact": slice(5, 9), "feet_pos": slice(9, 15), "tail": slice(15, 17)}
+    rewards = {
+        "alive": rw.StayAliveReward(scale=0.5),
+        "air_time": rw.FeetAirTimeReward(scale=2.0, gait_period=LinearScale(scale=0.2, bias=0.1), air_time_percent=0.4,
+                                         ctrl_dt=0.02, contact_obs="contact", bias=0.05, ground_penalty=0.2),
+        "vel": rw.ActionVelocityPenalty(scale=0.01),
+        "height": rw.SparseTargetHeightReward(scale=3.0, contact_obs="contact", position_obs="feet_pos", height=0.12),
+        "cmd_air": rw.FeetAirTimeReward(scale=1.0, gait_period=0.25, air_time_percent=0.5, ctrl_dt=0.02, contact_obs="contact",
+                                        linvel_cmd="lin", angvel_cmd="ang", linvel_moving_threshold=0.3),
+    }
+    level = 0.5
+    period = np.float32(0.2 * level + 0.1)
+    air1 = float(np.round(period * np.float32(0.4) / np.float32(0.02))); gnd1 = float(np.round(period * np.float32(0.6) / np.float32(0.02)))
+    air2 = float(np.round(np.float32(0.25) * np.float32(0.5) / np.float32(0.02))); gnd2 = air2
+    assert (air1, gnd1, air2) == (4.0, 6.0, 6.0)
+    carry = None
+    ocarry = [dict(a=(np.zeros(2, int),) * 3, h=np.zeros(2), c=(np.zeros(2, int),) * 3) for _ in range(N)]
+    for rollout in range(2):
+        obs = rng.normal(size=(Tn, N, 17)).astype(np.float32)
+        obs[..., 5:9] = (rng.random((Tn, N, 4)) < 0.6)            # (c=2, n=2) contact flags, long stance phases
+        obs[..., 9:15] = np.abs(rng.normal(size=(Tn, N, 6))) * 0.1
+        qvel = rng.normal(size=(Tn, N, nv)).astype(np.float32) * 0.3
+        cmd = rng.normal(size=(Tn, N, 3)).astype(np.float32) * 0.4
+        done = rng.random((Tn, N)) < 0.05
+        action = rng.normal(size=(Tn, N, nu)).astype(np.float32)
+        traj = Trajectory(qpos=t32(rng.normal(size=(Tn, N, nq))), qvel=t32(qvel), xpos=None, xquat=None, ctrl=None,
+                          obs={"obs": t32(obs)}, command={"_buffer": t32(cmd)}, event_state={}, action=t32(action),
+                          done=torch.from_numpy(done).to(DEV), success=None, timestep=None)
+        st = rw.get_rewards(traj, rewards, clip_max=5.0, rewards_carry=carry, obs_slices=obs_slices,
+                            command_slices={"lin": slice(0, 1), "ang": slice(2, 3)}, level=level)
+        carry = st.carry["_buffer"]
+        assert list(st.components) == ["alive", "air_time/air", "air_time/gnd", "air_time/stationary_gnd", "vel", "height",
+                                       "cmd_air/air", "cmd_air/gnd", "cmd_air/stationary_gnd"]
+        comp = {k: v.cpu().numpy() for k, v in st.components.items()}
+        total = st.total.cpu().numpy()
+        for e in range(N):
+            oc = ocarry[e]
+            if done[-1, e]:  # ksim/task/rl.py:206-214: the carry this rollout starts from is the initial one
+                oc = dict(a=(np.zeros(2, int),) * 3, h=np.zeros(2), c=(np.zeros(2, int),) * 3)
+            con = obs[:, e, 5:9].reshape(Tn, 2, 2)
+            a, oc["a"] = ot.feet_air_time_reward(con, qvel[:, e], done[:, e], oc["a"], air_steps=air1, gnd_steps=gnd1, bias=0.05,
+                                                 ground_penalty=0.2)
+            h, oc["h"] = ot.sparse_target_height_reward(con, obs[:, e, 9:15].reshape(Tn, 2, 3), qvel[:, e], done[:, e], oc["h"],
+                                                        height=0.12)
+            c, oc["c"] = ot.feet_air_time_reward(con, qvel[:, e], done[:, e], oc["c"], air_steps=air2, gnd_steps=gnd2,
+                                                 linvel_threshold=0.3, lin_cmd_t=cmd[:, e, 0], ang_cmd_t=cmd[:, e, 2])
+            ocarry[e] = oc
+            for k in ("air", "gnd", "stationary_gnd"):
+                np.testing.assert_allclose(comp[f"air_time/{k}"][:, e], 2.0 * a[k], rtol=1e-6, atol=1e-6)
+                np.testing.assert_allclose(comp[f"cmd_air/{k}"][:, e], c[k], rtol=1e-6, atol=1e-6)
+            np.testing.assert_allclose(comp["height"][:, e], 3.0 * h, rtol=1e-6, atol=1e-6)
+        want_total = np.minimum(sum(comp.values()), 5.0)
+        np.testing.assert_allclose(total, want_total, rtol=1e-5, atol=1e-5)
+        cr = carry.cpu().numpy()
+        np.testing.assert_allclose(cr[:, 0:6], [np.concatenate(o["a"]) for o in ocarry])
+        np.testing.assert_allclose(cr[:, 6:8], [o["h"] for o in ocarry], rtol=1e-6)
+        np.testing.assert_allclose(cr[:, 8:14], [np.concatenate(o["c"]) for o in ocarry])
+    with pytest.raises(KeyError, match="contact"):
+        rw.get_rewards(traj, rewards, obs_slices={"feet_pos": slice(0, 6)}, command_slices={"lin": slice(0, 1), "ang": slice(2, 3)})

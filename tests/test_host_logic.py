@@ -15,7 +15,8 @@ def test_struct_layouts_match_the_library():
     lib.ks_abi_sizeof.restype = ctypes.c_int64
     lib.ks_abi_sizeof.argtypes = [ctypes.c_int32]
     structs = [_lib.KsPpoLossParams, _lib_dyn.KsModelDesc, _lib_dyn.KsStepIO, T.KsTermsDesc, T.KsObserveIO,
-               T.KsTerminateIO, T.KsMlpDesc, T.KsRewardIO, T.KsObsElem, T.KsTermDesc, T.KsRewardDesc, T.KsRng]
+               T.KsTerminateIO, T.KsMlpDesc, T.KsRewardIO, T.KsObsElem, T.KsTermDesc, T.KsRewardDesc, T.KsRng,
+               T.KsAdamParams, T.KsEventDesc, T.KsRewardScanIO, T.KsRewardScanDesc]
     for i, st in enumerate(structs):
         assert lib.ks_abi_sizeof(i) == ctypes.sizeof(st), st.__name__
     assert lib.ks_abi_sizeof(99) == -1
@@ -159,3 +160,46 @@ def test_scales_and_event_descriptors():
     many = {f"e{i}": kev.JumpEvent(interval_range=(1.0, 2.0)) for i in range(T.KS_MAX_EVENTS + 1)}
     with pytest.raises(ValueError):
         engine.get_physics_engine("hip", [], many, act, cfg)
+
+
+def test_stateful_terms_compile_to_carry_layouts():
+    """Stateful observations get consecutive slices of the carry row in dict order; stateful rewards validate the
+    observations they name (no GPU involved)."""
+    m = km.kbot_scale_model()
+    observations = {"jp": ob.JointPositionObservation(),
+                    "old": ob.DelayedJointPositionObservation(delay_steps=3),
+                    "g": ob.ProjectedGravityObservation(min_lag=0.1, max_lag=0.5),
+                    "oldv": ob.DelayedJointVelocityObservation(delay_steps=2),
+                    "plain_g": ob.ProjectedGravityObservation(),
+                    "contact": ob.FeetContactObservation(foot_left=(0, 1), foot_right=(4, 5))}
+    d, slices, used, _, _ = compile_terms(m, observations, {}, [])
+    nj = m.nu
+    assert d.carry_dim == 3 * nj + 7 + 2 * nj and d.ns == m.ns
+    old, g, oldv = d.obs[slices["old"].start], d.obs[slices["g"].start + 2], d.obs[slices["oldv"].start + 1]
+    assert (old.kind, old.comp, old.carry, old.stride, old.index) == (T.OBS_DELAYED, 3, 0, nj, 7)
+    assert (g.kind, g.comp, g.carry) == (T.OBS_GRAVITY_EMA, 2, 3 * nj) and (g.q0, g.q1) == (pytest.approx(0.1), 0.5)
+    assert (oldv.carry, oldv.stride, oldv.src, oldv.index) == (3 * nj + 7 + 1, nj, T.SRC_QVEL, 7)
+    assert d.obs[slices["plain_g"].start].kind == T.OBS_ROT_INV
+    c = [d.obs[k] for k in range(slices["contact"].start, slices["contact"].stop)]
+    assert [e.index for e in c] == [0, 4, 1, 5] and all(e.kind == T.OBS_CONTACT and e.src == T.SRC_CONTACT_DIST for e in c)
+    assert T.SRC_CONTACT_DIST in used and T.SRC_QPOS in used
+    for bad in (lambda: ob.DelayedJointPositionObservation(delay_steps=0), lambda: ob.ProjectedGravityObservation(max_lag=1.0),
+                lambda: ob.ProjectedGravityObservation(imu_bias=-0.1), lambda: ob.FeetContactObservation(foot_left=(0,), foot_right=())):
+        with pytest.raises(ValueError):
+            bad()
+    fc = ob.FeetContactObservation.create(physics_model=m, foot_left_body_names=m.body_names[int(m.sph_body[0])],
+                                          foot_right_body_names=[m.body_names[int(m.sph_body[-1])]])
+    assert len(fc.foot_left) == len(fc.foot_right) == 4 and set(fc.foot_left).isdisjoint(fc.foot_right)
+    from ksim_amd.scales import LinearScale
+    air = rw.FeetAirTimeReward(scale=1.0, gait_period=LinearScale(scale=0.2, bias=0.3), air_time_percent=0.25, ctrl_dt=0.02,
+                               contact_obs="contact")
+    sd = air.scan_desc(slices, {}, 1.0)
+    assert (sd.kind, sd.n, sd.n_contact, sd.contact_index) == (T.SCAN_FEET_AIR_TIME, 2, 2, slices["contact"].start)
+    assert (sd.air_steps, sd.gnd_steps, sd.linvel_cmd_index) == (6.0, 19.0, -1)  # round(0.5*0.25/0.02), round(0.5*0.75/0.02)
+    assert rw.reward_carry_size({"a": air, "b": rw.StayAliveReward(), "c": rw.SparseTargetHeightReward(contact_obs="contact")}) == 8
+    with pytest.raises(KeyError):
+        rw.FeetAirTimeReward(contact_obs="nope").scan_desc(slices, {}, 1.0)
+    with pytest.raises(KeyError):
+        rw.FeetAirTimeReward(contact_obs="contact", linvel_cmd="v").scan_desc(slices, {}, 1.0)
+    with pytest.raises(ValueError):
+        rw.SparseTargetHeightReward(contact_obs="contact", position_obs="jp", num_bodies=2).scan_desc(slices, {}, 1.0)

@@ -147,3 +147,80 @@ def test_force_push_event_state_machine():
     # the curriculum scale multiplies the carried wrench every substep and once more when it is applied
     ap, (_, _, w2) = terms.force_push_event(p, (1.0, 0.1, np.ones(6)), 0.005, np.zeros(10), 0.5)
     np.testing.assert_allclose(w2, 0.5 * np.ones(6)); np.testing.assert_allclose(ap, 0.25 * np.ones(6))
+
+
+def test_stateful_observations_closed_forms():
+    from scipy.spatial.transform import Rotation
+    # contact flags: negative distance = touching; block is (spheres per foot, 2 feet)
+    c = terms.feet_contact_observation([-0.01, 0.2, 0.0, -1e-6], foot_left=(0, 1), foot_right=(2, 3))
+    assert c.tolist() == [[1.0, 0.0], [0.0, 1.0]]
+    # delay line: after the fill the output at step k is the input at step k - delay
+    rng = np.random.default_rng(0)
+    xs = rng.normal(size=(9, 4))
+    carry = np.tile(xs[0], (3, 1))
+    outs = []
+    for k in range(1, 9):
+        out, carry = terms.delayed_observation(carry, xs[k], zero_offset=np.full(4, 0.5))
+        outs.append(out)
+    np.testing.assert_allclose(outs[:3], np.tile(xs[0] - 0.5, (3, 1)))
+    np.testing.assert_allclose(outs[3:], xs[1:6] - 0.5)
+    # roll-pitch-yaw quaternion against scipy's extrinsic xyz composition
+    for rpy in rng.uniform(-1, 1, size=(5, 3)):
+        q = terms.euler_to_quat(rpy)
+        want = Rotation.from_euler("xyz", rpy).as_quat()[[3, 0, 1, 2]]
+        np.testing.assert_allclose(q * np.sign(q[0]), want * np.sign(want[0]), atol=1e-12)
+    # exponential average of a constant reading: x_k = p (1 - lag^k); p = R_bias R_q^-1 g
+    quat = Rotation.from_euler("xyz", [0.3, -0.2, 0.9]).as_quat()[[3, 0, 1, 2]]
+    bias = np.array([0.05, -0.02, 0.01])
+    p = Rotation.from_euler("xyz", bias).apply(Rotation.from_quat(quat[[1, 2, 3, 0]]).inv().apply([0, 0, -9.81]))
+    x = np.zeros(3)
+    for k in range(1, 6):
+        x = terms.projected_gravity_ema(x, 0.7, bias, quat)
+        np.testing.assert_allclose(x, p * (1 - 0.7**k), atol=1e-12)
+    np.testing.assert_allclose(terms.projected_gravity_ema(np.ones(3), 0.0, np.zeros(3), [1, 0, 0, 0]), [0, 0, -9.81])
+
+
+def test_feet_air_time_reward_hand_computed():
+    """Two feet, one contact sphere each, air and ground phases of 2 and 3 steps; counters and rewards by hand."""
+    #            t:  0  1  2  3  4  5  6
+    left = np.array([1, 0, 0, 0, 1, 1, 1])    # left foot: down, three steps up, down
+    right = np.ones(7, dtype=int)               # right foot always down
+    contact = np.stack([left, right], axis=-1)[:, None, :].astype(float)
+    qvel = np.zeros((7, 6)); qvel[:, 0] = 1.0   # moving
+    qvel[5, 0] = 0.0                            # standing at t = 5
+    done = np.zeros(7, bool); done[6] = True    # a finished step never counts as moving
+    zero = (np.zeros(2, int),) * 3
+    out, (air, gnd, sta) = terms.feet_air_time_reward(contact, qvel, done, zero, air_steps=2.0, gnd_steps=3.0, bias=0.1,
+                                                     ground_penalty=0.25)
+    # left air counter 0 1 2 3 0 0 0 -> reward cnt/2 + bias while cnt < 2, else 0; right foot never in the air: bias
+    np.testing.assert_allclose(out["air"], [0.1, 0.6, 0.1, 0.1, 0.1, 0.1, 0.1])
+    # ground counters: left 1 0 0 0 1 0 0, right 1 2 3 4 5 0 0; cnt/3 + bias while cnt < 3 else -penalty; max over feet
+    np.testing.assert_allclose(out["gnd"], [1 / 3 + 0.1, 2 / 3 + 0.1, 0.1, 0.1, 1 / 3 + 0.1, 0.1, 0.1])
+    # stationary counters only run while in contact and not moving: t=5 -> 1, t=6 (done) -> 2
+    np.testing.assert_allclose(out["stationary_gnd"], [0.1, 0.1, 0.1, 0.1, 0.1, 1 / 3 + 0.1, 2 / 3 + 0.1])
+    assert air.tolist() == [0, 0] and gnd.tolist() == [0, 0] and sta.tolist() == [2, 2]
+    # the carry continues the count across rollouts; yaw rate alone counts as moving only when positive
+    qv = np.zeros((1, 6)); qv[0, 5] = -1.0
+    out2, (_, _, sta2) = terms.feet_air_time_reward(contact[:1], qv, np.zeros(1, bool), (air, gnd, sta), air_steps=2.0, gnd_steps=3.0)
+    assert sta2.tolist() == [3, 3] and out2["stationary_gnd"][0] == 1.0
+    # commands replace the measured velocity when named
+    out3, (_, gnd3, _) = terms.feet_air_time_reward(contact[:1], qv, np.zeros(1, bool), zero, air_steps=2.0, gnd_steps=3.0,
+                                                    lin_cmd_t=np.array([-0.5]), ang_cmd_t=np.array([0.0]))
+    assert gnd3.tolist() == [1, 1]
+
+
+def test_sparse_target_height_reward_hand_computed():
+    #              t:  0    1    2    3    4    5
+    z = np.array([0.0, 0.1, 0.3, 0.2, 0.0, 0.5])
+    contact = np.array([1, 0, 0, 0, 1, 0])[:, None, None].astype(float)
+    pos = np.zeros((6, 1, 3)); pos[:, 0, 2] = z
+    qvel = np.zeros((6, 6)); qvel[:, 0] = 1.0
+    out, best = terms.sparse_target_height_reward(contact, pos, qvel, np.zeros(6, bool), np.array([0.15]), height=0.25)
+    # t=0: touching with a carried maximum of 0.15 -> reward 0.15, maximum reset; t=4: touch-down after a swing that
+    # peaked at 0.3 -> capped at 0.25; t=5: in the air again, the maximum restarts from this height
+    np.testing.assert_allclose(out, [0.15, 0, 0, 0, 0.25, 0])
+    np.testing.assert_allclose(best, [0.5])
+    # a robot that is not moving loses the running maximum
+    qvel[3, 0] = 0.0
+    out, _ = terms.sparse_target_height_reward(contact, pos, qvel, np.zeros(6, bool), np.array([0.0]), height=0.25)
+    np.testing.assert_allclose(out, [0, 0, 0, 0, 0.0, 0])
