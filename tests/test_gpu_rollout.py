@@ -335,3 +335,25 @@ def test_gait_terms_in_the_rollout_and_under_graph_replay():
     for it, (a, b) in enumerate(zip(*runs)):
         for x, y, name in zip(a, b, ("observations", "reward", "observation carry", "reward carry")):
             assert torch.equal(x, y), f"replay {it}: {name} differs from the eager rollout"
+
+
+def test_rollout_written_to_the_dataset_format_and_read_back(tmp_path):
+    """collect_dataset's data path (ksim/task/rl.py:2315-2411): a device rollout goes to the float32 memory map one env per
+    sample and comes back equal."""
+    from ksim_amd.dataset import TrajectoryDataset
+
+    N, T = 16, 8
+    m, c, rnd_, _, ro, EnvState = build(N, T, seed=3)
+    ps = c.engine.reset(c.physics_model, 1.0, 3, N, rnd_)
+    env = EnvState(ps, rnd_, torch.zeros(N, 2, device=DEV), None, seed=4)
+    traj, _ = ro.unroll(env)
+    rew = ro._rewards(traj, env, 1.0, want_components=True)
+    path = tmp_path / "rollouts.bin"
+    with TrajectoryDataset.writer(path, num_samples=N) as w:
+        assert w.write_batch(traj, rew) == N
+    ds = TrajectoryDataset(path, device=DEV)
+    for e in (0, 7, 15):
+        t, r = ds.get(e)
+        assert torch.equal(t.qpos, traj.qpos[:, e]) and torch.equal(t.obs["noisy_obs"], traj.obs["noisy_obs"][:, e])
+        assert torch.equal(t.xquat, traj.xquat[:, e]) and torch.equal(t.done, traj.done[:, e].float())
+        assert torch.equal(r.total, rew.total[:, e]) and torch.equal(r.components["height"], rew.components["height"][:, e])
