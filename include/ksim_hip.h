@@ -33,7 +33,7 @@ const char* ks_last_error(void);
 /* sizeof() of a public struct as this library was compiled, for binding self-checks:
  * 0 KsPpoLossParams, 1 KsModelDesc, 2 KsStepIO, 3 KsTermsDesc, 4 KsObserveIO, 5 KsTerminateIO, 6 KsMlpDesc,
  * 7 KsRewardIO, 8 KsObsElem, 9 KsTermDesc, 10 KsRewardDesc, 11 KsRng, 12 KsAdamParams, 13 KsEventDesc,
- * 14 KsRewardScanIO, 15 KsRewardScanDesc;
+ * 14 KsRewardScanIO, 15 KsRewardScanDesc, 16 KsGruDesc;
  * -1 for anything else. */
 int64_t ks_abi_sizeof(int32_t which);
 
@@ -387,7 +387,8 @@ int ks_sample_action(ks_stream_t stream, int64_t N, int32_t nu, const float* mea
  * provides ks_mlp_workspace_bytes(mlp, M) bytes of device scratch.
  */
 #define KS_MAX_LAYERS 8
-enum { KS_ACT_NONE = 0, KS_ACT_ELU = 1, KS_ACT_RELU = 2, KS_ACT_TANH = 3 };
+enum { KS_ACT_NONE = 0, KS_ACT_ELU = 1, KS_ACT_RELU = 2, KS_ACT_TANH = 3,
+       KS_ACT_GELU = 4 /* tanh form, jax.nn.gelu's default (examples/walking.py:103); forward only */ };
 enum { KS_MLP_F32 = 0, KS_MLP_BF16 = 1 };
 typedef struct KsMlpDesc {
   int32_t n_layers;
@@ -403,6 +404,28 @@ int ks_mlp_destroy(KsMlp* mlp);
 int64_t ks_mlp_workspace_bytes(const KsMlp* mlp, int64_t M);
 int ks_mlp_forward(const KsMlp* mlp, ks_stream_t stream, int64_t M, const float* x /*(M, in)*/,
                    float* y /*(M, out)*/, void* workspace);
+
+/* ------------------------------------------------------------------ GRU cell (recurrent policies, forward)
+ * The recurrent actors / critics of the shipped examples (examples/walking.py:40-208: input projection, a stack of
+ * eqx.nn.GRUCell, output MLP) step once per control step inside the rollout (ksim/task/rl.py:892-926).  One cell:
+ *   gi = W_ih x + bias, gh = W_hh h;  r = sigmoid(gi_r + gh_r), z = sigmoid(gi_z + gh_z),
+ *   n = tanh(gi_n + r (gh_n + bias_n)),  h' = n + z (h - n)        (gate order r | z | n along the 3H rows)
+ * `fresh` marks envs that start an episode: their carry is taken as zero (get_initial_model_carry after a reset,
+ * rl.py:1072-1080).  h_out may alias h_in.  Forward only: backpropagation through time is not built. */
+typedef struct KsGruDesc {
+  int32_t input_size, hidden_size, dtype; /* dtype: KS_MLP_F32 | KS_MLP_BF16 for the two projections */
+  const float* weight_ih; /* host (3H, input_size) */
+  const float* weight_hh; /* host (3H, H) */
+  const float* bias;      /* host (3H), nullable */
+  const float* bias_n;    /* host (H), nullable */
+} KsGruDesc;
+typedef struct KsGru KsGru;
+int ks_gru_create(const KsGruDesc* desc /*host*/, KsGru** out);
+int ks_gru_destroy(KsGru* gru);
+int64_t ks_gru_workspace_bytes(const KsGru* gru, int64_t M);
+int ks_gru_forward(const KsGru* gru, ks_stream_t stream, int64_t M, const float* x /*(M, input_size)*/,
+                   const float* h_in /*(M, H)*/, const uint8_t* fresh /*(M) nullable*/, float* h_out /*(M, H)*/,
+                   void* workspace);
 
 /* ------------------------------------------------------------------ policy update: gradients and optimiser
  * The native pieces of PPOTask._single_step / update_model (ksim/task/ppo.py:495-565, 572-694) for an

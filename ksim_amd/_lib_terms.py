@@ -11,7 +11,7 @@ OBS_COPY, OBS_JOINT_POS, OBS_ROT_INV, OBS_CONTACT, OBS_DELAYED, OBS_GRAVITY_EMA 
 NOISE_NONE, NOISE_ADD_GAUSSIAN, NOISE_ADD_UNIFORM, NOISE_MUL_GAUSSIAN, NOISE_MUL_UNIFORM = range(5)
 (TERM_MIN_HEIGHT, TERM_BAD_Z, TERM_NOT_UPRIGHT, TERM_BAD_VELOCITY, TERM_FAR_FROM_ORIGIN,
  TERM_EPISODE_LENGTH) = range(6)
-ACT_NONE, ACT_ELU, ACT_RELU, ACT_TANH = range(4)
+ACT_NONE, ACT_ELU, ACT_RELU, ACT_TANH, ACT_GELU = range(5)
 MLP_F32, MLP_BF16 = 0, 1
 
 
@@ -110,6 +110,11 @@ class KsRewardScanIO(ctypes.Structure):
                 ("command", c_void_p), ("done", c_void_p), ("carry", c_void_p), ("out", c_void_p)]
 
 
+class KsGruDesc(ctypes.Structure):
+    _fields_ = [("input_size", c_int32), ("hidden_size", c_int32), ("dtype", c_int32), ("weight_ih", c_void_p),
+                ("weight_hh", c_void_p), ("bias", c_void_p), ("bias_n", c_void_p)]
+
+
 class KsAdamParams(ctypes.Structure):
     _fields_ = [("lr", c_float), ("b1", c_float), ("b2", c_float), ("eps", c_float), ("weight_decay", c_float),
                 ("max_grad_norm", c_float), ("step", c_int64)]
@@ -118,6 +123,13 @@ class KsAdamParams(ctypes.Structure):
 def bind(lib) -> None:
     lib.ks_rewards.argtypes = [c_void_p, POINTER(KsRewardIO)]
     lib.ks_rewards.restype = c_int32
+    lib.ks_gru_create.argtypes = [POINTER(KsGruDesc), POINTER(c_void_p)]
+    lib.ks_gru_destroy.argtypes = [c_void_p]
+    lib.ks_gru_workspace_bytes.argtypes = [c_void_p, c_int64]
+    lib.ks_gru_workspace_bytes.restype = c_int64
+    lib.ks_gru_forward.argtypes = [c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]
+    for name in ("ks_gru_create", "ks_gru_destroy", "ks_gru_forward"):
+        getattr(lib, name).restype = c_int32
     lib.ks_reward_scan.argtypes = [c_void_p, POINTER(KsRewardScanIO)]
     lib.ks_reward_scan.restype = c_int32
     lib.ks_terms_create.argtypes = [POINTER(KsTermsDesc), POINTER(c_void_p)]

@@ -28,6 +28,12 @@ __device__ __forceinline__ float activate(float x) {
   if (ACT == KS_ACT_ELU) return x > 0.f ? x : (FAST ? __expf(x) - 1.0f : expm1f(x));
   if (ACT == KS_ACT_RELU) return fmaxf(x, 0.f);
   if (ACT == KS_ACT_TANH) return tanhf(x);
+  if (ACT == KS_ACT_GELU) {  // tanh form (jax.nn.gelu's default): 0.5 x (1 + tanh(sqrt(2/pi) (x + 0.044715 x^3)))
+    const float u = 0.7978845608028654f * (x + 0.044715f * x * x * x);
+    // tanh(u) = 1 - 2 / (exp(2u) + 1); the hardware exponential is exact enough when the result is rounded to bf16
+    const float t = FAST ? 1.f - 2.f / (__expf(2.f * u) + 1.f) : tanhf(u);
+    return 0.5f * x * (1.f + t);
+  }
   return x;
 }
 
@@ -660,6 +666,7 @@ static int launch_layer_tile(int act, hipStream_t s, int64_t M, int npad, int K,
     case KS_ACT_ELU: KS_LAUNCH(KS_ACT_ELU) break;
     case KS_ACT_RELU: KS_LAUNCH(KS_ACT_RELU) break;
     case KS_ACT_TANH: KS_LAUNCH(KS_ACT_TANH) break;
+    case KS_ACT_GELU: KS_LAUNCH(KS_ACT_GELU) break;
     default: KS_LAUNCH(KS_ACT_NONE) break;
   }
 #undef KS_LAUNCH
@@ -693,7 +700,7 @@ extern "C" int ks_mlp_create(const KsMlpDesc* d, KsMlp** out) {
   if (!d || !out) return fail(KS_EINVAL, "ks_mlp_create: null argument");
   if (d->n_layers < 1 || d->n_layers > KS_MAX_LAYERS) return fail(KS_ELIMIT, "ks_mlp_create: %d layers (1..%d)", d->n_layers, KS_MAX_LAYERS);
   if (d->dtype != KS_MLP_F32 && d->dtype != KS_MLP_BF16) return fail(KS_EINVAL, "ks_mlp_create: unknown dtype");
-  if (d->activation < KS_ACT_NONE || d->activation > KS_ACT_TANH) return fail(KS_EINVAL, "ks_mlp_create: unknown activation");
+  if (d->activation < KS_ACT_NONE || d->activation > KS_ACT_GELU) return fail(KS_EINVAL, "ks_mlp_create: unknown activation");
   for (int l = 0; l <= d->n_layers; ++l)
     if (d->dims[l] < 1 || d->dims[l] > 65536) return fail(KS_EINVAL, "ks_mlp_create: bad width %d", d->dims[l]);
   KsMlp* h = new KsMlp();
@@ -809,6 +816,7 @@ static int launch_fused_tile(const DevMlp& m, hipStream_t s, int64_t M, const fl
     case KS_ACT_ELU: KS_LAUNCH(KS_ACT_ELU) break;
     case KS_ACT_RELU: KS_LAUNCH(KS_ACT_RELU) break;
     case KS_ACT_TANH: KS_LAUNCH(KS_ACT_TANH) break;
+    case KS_ACT_GELU: KS_LAUNCH(KS_ACT_GELU) break;
     default: KS_LAUNCH(KS_ACT_NONE) break;
   }
 #undef KS_LAUNCH
@@ -892,6 +900,7 @@ static void refresh_layers(DevMlp& m, hipStream_t s);
 
 extern "C" int ks_mlp_train_init(KsMlp* h) {
   if (!h) return fail(KS_EINVAL, "ks_mlp_train_init: null handle");
+  if (h->m.activation == KS_ACT_GELU) return fail(KS_EINVAL, "ks_mlp_train_init: the backward pass keeps activations, not pre-activations, and GELU cannot be differentiated from its output");
   DevMlp& m = h->m;
   if (m.train) return KS_OK;
   const size_t esz = m.dtype == KS_MLP_BF16 ? 2 : 4;

@@ -329,6 +329,7 @@ extern "C" int64_t ks_abi_sizeof(int32_t which) {
     case 13: return sizeof(KsEventDesc);
     case 14: return sizeof(KsRewardScanIO);
     case 15: return sizeof(KsRewardScanDesc);
+    case 16: return sizeof(KsGruDesc);
     default: return -1;
   }
 }

@@ -14,7 +14,8 @@ import torch
 from . import _lib
 from . import _lib_terms as T
 
-_ACT = {None: T.ACT_NONE, "none": T.ACT_NONE, "elu": T.ACT_ELU, "relu": T.ACT_RELU, "tanh": T.ACT_TANH}
+_ACT = {None: T.ACT_NONE, "none": T.ACT_NONE, "elu": T.ACT_ELU, "relu": T.ACT_RELU, "tanh": T.ACT_TANH,
+        "gelu": T.ACT_GELU}
 
 
 class MLP:

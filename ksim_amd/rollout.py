@@ -20,6 +20,7 @@ from .engine import HipEngine
 from .env_terms import EnvTerms, sample_action
 from .mlp import MLP
 from .physics import DeviceModel
+from .recurrent import RecurrentNetwork
 from .rewards import Reward, get_rewards, reward_carry_size
 from .types import PhysicsState, RewardState, Trajectory
 
@@ -30,8 +31,8 @@ class RolloutConstants:  # the static pieces, ksim/task/rl.py:138-150
     engine: HipEngine
     terms: EnvTerms
     rewards: Mapping[str, Reward]
-    actor: MLP
-    critic: MLP | None
+    actor: MLP | RecurrentNetwork
+    critic: MLP | RecurrentNetwork | None
     log_std: torch.Tensor | None
     action_clip_max: float = 1e3  # RLConfig.action_clip_max, rl.py:589-592
     reward_clip_min: float | None = None
@@ -49,6 +50,8 @@ class RolloutEnvState:  # ksim/task/rl.py:110-123, batched
         self.step = 0
         self.obs_carry = None     # (N, carry_dim) carries of the stateful observations (rl.py:118), made on first use
         self.reward_carry = None  # (N, reward carry size) carries of the stateful rewards (rl.py:119)
+        self.actor_carry = None   # (depth, N, hidden) carries of recurrent networks (rl.py:117)
+        self.critic_carry = None
         N = physics_state.data.qpos.shape[0]
         self.episode_length = torch.zeros(N, dtype=torch.int32, device=physics_state.data.qpos.device)
 
@@ -96,9 +99,16 @@ class Rollout:
                         step=step, step_base=step_base, obs=self.obs[t], noisy_obs=self.noisy_obs[t],
                         carry=env.obs_carry, fresh=self.reset_mask if c.terms.carry_dim else None,
                         carry_uniform=noise.get("obs_carry_uniform"))
-        c.actor(self.noisy_obs[t], out=self.mean)           # actor reads the noisy copy (walking.py:592-595)
-        if c.critic is not None:
-            c.critic(self.obs[t], out=self.values[t])       # critic reads the clean one (walking.py:626-638)
+        # actor reads the noisy copy (walking.py:592-595), critic the clean one (walking.py:626-638); recurrent networks
+        # advance their carries, which restart from zero for the envs the previous control step reset
+        if isinstance(c.actor, RecurrentNetwork):
+            c.actor(self.noisy_obs[t], env.actor_carry, fresh=self.reset_mask, out=self.mean)
+        else:
+            c.actor(self.noisy_obs[t], out=self.mean)
+        if isinstance(c.critic, RecurrentNetwork):
+            c.critic(self.obs[t], env.critic_carry, fresh=self.reset_mask, out=self.values[t])
+        elif c.critic is not None:
+            c.critic(self.obs[t], out=self.values[t])
         sample_action(self.mean, c.log_std, noise=noise.get("action_normal"), seed=env.seed, step=step,
                       step_base=step_base, clip_max=c.action_clip_max, out=self.action[t])
         # the step kernel also writes ctrl / xpos / xquat of the post-step data into the transition slot
@@ -161,6 +171,9 @@ class Rollout:
         if self.c.terms.carry_dim and env.obs_carry is None:
             env.obs_carry = torch.zeros(self.N, self.c.terms.carry_dim, dtype=torch.float32, device=self.done.device)
             self.reset_mask.fill_(1)  # every env starts an episode: the first observation initialises all carries
+        for net, name in ((self.c.actor, "actor_carry"), (self.c.critic, "critic_carry")):
+            if isinstance(net, RecurrentNetwork) and getattr(env, name) is None:
+                setattr(env, name, net.initial_carry(self.N, self.done.device))
         n = reward_carry_size(self.c.rewards)
         if n and env.reward_carry is None:
             env.reward_carry = torch.zeros(self.N, n, dtype=torch.float32, device=self.done.device)

@@ -1,0 +1,50 @@
+"""TEST INFRASTRUCTURE: float64 restatement of the recurrent networks of the reference's examples
+(examples/walking.py:40-208).  The GRU cell follows eqx.nn.GRUCell's equations (equinox is a third-party dependency
+that is not in the reference tree): gi = W_ih x + b, gh = W_hh h, r = s(gi_r + gh_r), z = s(gi_z + gh_z),
+n = tanh(gi_n + r (gh_n + b_n)), h' = n + z (h - n).  Pinned by torch.nn.GRUCell, which computes the same cell when its
+hidden bias is (0, 0, b_n), and by hand-checkable limits (tests/test_oracle_recurrent.py).  GELU is the tanh form,
+jax.nn.gelu's default."""
+import numpy as np
+
+
+def sigmoid(x):
+    return 1.0 / (1.0 + np.exp(-x))
+
+
+def gru_cell(x, h, weight_ih, weight_hh, bias=None, bias_n=None):
+    """x (N, I), h (N, H) -> h' (N, H)."""
+    x, h = np.asarray(x, dtype=np.float64), np.asarray(h, dtype=np.float64)
+    H = h.shape[-1]
+    gi = x @ np.asarray(weight_ih, dtype=np.float64).T + (0.0 if bias is None else np.asarray(bias, dtype=np.float64))
+    gh = h @ np.asarray(weight_hh, dtype=np.float64).T
+    bn = 0.0 if bias_n is None else np.asarray(bias_n, dtype=np.float64)
+    r = sigmoid(gi[:, :H] + gh[:, :H])
+    z = sigmoid(gi[:, H:2 * H] + gh[:, H:2 * H])
+    n = np.tanh(gi[:, 2 * H:] + r * (gh[:, 2 * H:] + bn))
+    return n + z * (h - n)
+
+
+def gelu(x):
+    x = np.asarray(x, dtype=np.float64)
+    return 0.5 * x * (1.0 + np.tanh(np.sqrt(2.0 / np.pi) * (x + 0.044715 * x**3)))
+
+
+def mlp(x, weights, biases, act):
+    h = np.asarray(x, dtype=np.float64)
+    for i, (w, b) in enumerate(zip(weights, biases)):
+        h = h @ np.asarray(w, dtype=np.float64).T + np.asarray(b, dtype=np.float64)
+        if i + 1 < len(weights):
+            h = act(h)
+    return h
+
+
+def recurrent_network(obs, carry, fresh, input_proj, cells, out_weights, out_biases, act=gelu):
+    """One control step (examples/walking.py:124-150): returns (output, new carry (depth, N, H)); envs marked fresh
+    start from a zero carry."""
+    carry = np.where(np.asarray(fresh, dtype=bool)[None, :, None], 0.0, np.asarray(carry, dtype=np.float64))
+    x = np.asarray(obs, dtype=np.float64) @ np.asarray(input_proj[0], dtype=np.float64).T + input_proj[1]
+    new = []
+    for c, h in zip(cells, carry):
+        x = gru_cell(x, h, *c)
+        new.append(x)
+    return mlp(x, out_weights, out_biases, act), np.stack(new)

@@ -17,7 +17,7 @@ def t32(a):
     return torch.tensor(np.asarray(a), dtype=torch.float32, device=DEV).contiguous()
 
 
-def build(N, T, seed=0, min_height=0.9, events=None, gait=False):
+def build(N, T, seed=0, min_height=0.9, events=None, gait=False, recurrent=False):
     from ksim_amd import actuators, engine, model as km, observation as ob, physics, randomization as rnd, resets as rs
     from ksim_amd import rewards as rw, terminations as tm
     from ksim_amd.env_terms import EnvTerms
@@ -62,8 +62,23 @@ def build(N, T, seed=0, min_height=0.9, events=None, gait=False):
                                                          contact_obs="contact", linvel_moving_threshold=0.05),
                         "step_height": rw.SparseTargetHeightReward(scale=2.0, contact_obs="contact", position_obs="feet_pos",
                                                                    height=0.1, linvel_moving_threshold=0.02)})
+    actor, critic = MLP(ws, bs, dtype="f32"), MLP(cws, cbs, dtype="f32")
+    if recurrent:  # the shape of the shipped examples' networks: projection, GRU stack, GELU / ELU output MLP
+        from ksim_amd.recurrent import GRUCell, RecurrentNetwork
+        H = 32
+        def cell():
+            s_ = 1 / np.sqrt(H)
+            return (rng.uniform(-s_, s_, (3 * H, H)), rng.uniform(-s_, s_, (3 * H, H)), rng.uniform(-s_, s_, 3 * H), rng.uniform(-s_, s_, H))
+        def net(out, act):
+            proj = (rng.normal(size=(H, terms.obs_dim)) / np.sqrt(terms.obs_dim), np.zeros(H))
+            cells = [cell() for _ in range(2)]
+            ow, ob_ = [rng.normal(size=(H, H)) / np.sqrt(H), 0.1 * rng.normal(size=(out, H)) / np.sqrt(H)], [np.zeros(H), np.zeros(out)]
+            n = RecurrentNetwork(proj, [GRUCell(*c_, dtype="f32") for c_ in cells], MLP(ow, ob_, activation=act, dtype="f32"), dtype="f32")
+            n.params = (proj, cells, ow, ob_)
+            return n
+        actor, critic = net(m.nu, "gelu"), net(1, "elu")
     consts = RolloutConstants(physics_model=dm, engine=eng, terms=terms, rewards=rewards,
-                              actor=MLP(ws, bs, dtype="f32"), critic=MLP(cws, cbs, dtype="f32"), log_std=t32(log_std))
+                              actor=actor, critic=critic, log_std=t32(log_std))
     gen = torch.Generator(device=DEV); gen.manual_seed(seed)
     randomization = rnd.get_physics_randomizers(m, {"f": rnd.FloorFrictionRandomizer(0.4, 1.2),
                                                     "m": rnd.AllBodiesMassMultiplicationRandomizer(0.9, 1.1)}, N, gen)
@@ -357,3 +372,40 @@ def test_rollout_written_to_the_dataset_format_and_read_back(tmp_path):
         assert torch.equal(t.qpos, traj.qpos[:, e]) and torch.equal(t.obs["noisy_obs"], traj.obs["noisy_obs"][:, e])
         assert torch.equal(t.xquat, traj.xquat[:, e]) and torch.equal(t.done, traj.done[:, e].float())
         assert torch.equal(r.total, rew.total[:, e]) and torch.equal(r.components["height"], rew.components["height"][:, e])
+
+
+def test_recurrent_actor_and_critic_in_the_rollout():
+    """GRU actor and critic inside the environment loop: the carries replayed by the oracle from the recorded
+    observations and done flags (a finished env continues from a zero carry), and the graph replay equal to eager."""
+    from oracle import recurrent as orec
+
+    N, T = 24, 8
+    runs = []
+    for use_graph in (False, True):
+        m, c, rnd_, _, ro, EnvState = build(N, T, seed=13, min_height=0.8, recurrent=True)
+        ps = c.engine.reset(c.physics_model, 1.0, 3, N, rnd_)
+        env = EnvState(ps, rnd_, torch.zeros(N, 2, device=DEV), None, seed=21)
+        want = {"actor": np.zeros((2, N, 32)), "critic": np.zeros((2, N, 32))}
+        fresh = np.zeros(N, bool)
+        snaps, finished = [], 0
+        for it in range(5):
+            traj, rew = ro.unroll(env, graph=use_graph)
+            torch.cuda.synchronize()
+            finished += int(traj.done.sum().item())
+            snaps.append((traj.action.clone(), ro.values.clone(), env.actor_carry.clone(), env.critic_carry.clone()))
+            if use_graph:
+                continue
+            obs, noisy, done = (x.cpu().numpy() for x in (traj.obs["obs"], traj.obs["noisy_obs"], traj.done))
+            for t in range(T):
+                proj, cells, ow, ob_ = c.critic.params
+                v, want["critic"] = orec.recurrent_network(obs[t], want["critic"], fresh, proj, cells, ow, ob_, act=lambda x: np.where(x > 0, x, np.expm1(x)))
+                proj, cells, ow, ob_ = c.actor.params
+                _, want["actor"] = orec.recurrent_network(noisy[t], want["actor"], fresh, proj, cells, ow, ob_)
+                np.testing.assert_allclose(ro.values[t].cpu().numpy(), v, rtol=2e-4, atol=2e-4)
+                fresh = done[t].astype(bool)
+            np.testing.assert_allclose(env.actor_carry.cpu().numpy(), want["actor"], rtol=2e-4, atol=2e-4)
+        runs.append(snaps)
+        assert use_graph or finished > 0, "no env finished: the carry restart was not exercised"
+    for it, (a, b) in enumerate(zip(*runs)):
+        for x, y, name in zip(a, b, ("action", "values", "actor carry", "critic carry")):
+            assert torch.equal(x, y), f"replay {it}: {name} differs from the eager rollout"
