@@ -29,7 +29,7 @@ def cpu_baseline(target_seconds: float = 12.0):
     from ksim_amd.configs import KBOT_TORQUE_LIMITS
     from oracle.dyn import Oracle
 
-    m = km.kbot_scale_model(seed=1004)
+    m = km.kbot_scale_model(seed=1004, integrator="implicitfast")  # the integrator ksim selects (ksim/task/rl.py:555-578)
     orc = Oracle(m.arrays(), np.float32)
     cores = min(16, os.cpu_count() or 1)
     N = 2048
@@ -177,7 +177,7 @@ def main() -> None:
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": "cfg4: K-Bot-scale biped (free root + 20 hinges, 8 foot spheres), per-env friction/mass "
                                "randomisation, obs noise 0.01, reset on z<0.5, actor+critic 3x512 bf16 MLP, "
-                               "dt=0.005 x 4 substeps", "num_envs": N, "rollout_length": T, "substeps": 4,
+                               "dt=0.005 x 4 substeps, Newton 8/8, implicitfast (damping-implicit) integration", "num_envs": N, "rollout_length": T, "substeps": 4,
                    "obs_dim": obs_dim, "episodes_finished_in_last_rollout": ndone},
         "roofline": {"bound": "hbm", "kernel": "step_kernel (fused control step)", "achieved": achieved,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,

@@ -115,7 +115,10 @@ enum { KS_JNT_NONE = 0, KS_JNT_FREE = 1, KS_JNT_HINGE = 2 };
 typedef struct KsModelDesc {
   int32_t nb, nq, nv, nu, ns;
   int32_t iterations, ls_iterations; /* Newton / line-search limits (ksim/task/rl.py:717-748 sets opt.*) */
-  int32_t eulerdamp;                 /* must be 0: ksim disables EULERDAMP (rl.py:575-578,745-746) */
+  int32_t eulerdamp;                 /* 1: the velocity update is implicit in joint damping, (M + dt diag(damping)) a = M qacc.
+                                        That is MuJoCo's Euler step with EULERDAMP and also, for models whose smooth forces
+                                        depend on velocity only through joint damping (torque motors), its implicitfast
+                                        integrator, which ksim selects (rl.py:555-578,730-748).  0: plain semi-implicit Euler */
   double dt, gravity[3], tolerance, ls_tolerance, impratio, meaninertia, friction;
   double solref[2], solimp[5];
   int32_t body_parent[KS_MAX_BODIES], body_jtype[KS_MAX_BODIES], body_qadr[KS_MAX_BODIES],

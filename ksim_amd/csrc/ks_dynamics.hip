@@ -700,6 +700,7 @@ void step_kernel(StepArgs a) {
 
     KS_TICK(7)
     float qacc = qas;
+    float Mqacc = qfs;  // M qacc = smooth + constraint force: what the implicit integration step solves against
     int niter = 0;
     if (nefc > 0) {
       // ---- constraint rows: lane r builds row r of J in registers and mirrors it to LDS for column access
@@ -902,6 +903,7 @@ void step_kernel(StepArgs a) {
         ++niter;
         KS_TICK(13)
       }
+      Mqacc = Ma;
     }
     niter_out = niter;
     nefc_out = nefc;
@@ -912,7 +914,25 @@ void step_kernel(StepArgs a) {
     KS_TICK(14)
     // ---- semi-implicit Euler
     if (!FWD) {
-      if (is_dof) l.qvel[lane] = my_qvel + m.dt * qacc;
+      float qacc_int = qacc;
+      if (m.eulerdamp) {
+        // implicit in the joint damping: (M + dt diag(damping)) a = M qacc.  For torque motors, whose force does
+        // not depend on velocity, this is MuJoCo's implicitfast step; qacc itself (warm start, output) is unchanged.
+        f32x16 T;
+        load_mtile(T, l.M, nvs, nv, NP, lane);
+        const int c = lane & 31, half = lane >> 5;
+        const float hd = m.dt * __shfl(is_dof ? d_damping : 0.f, c);
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) T[4 * g + e] += (8 * g + 4 * half + e == c) ? hd : 0.f;
+        float R2[NP];
+        float inv2;
+        chol_tile<NP>(T, R2, inv2, lane);
+        const float sol = solve_regs<NP>(R2, inv2, lane, is_dof ? Mqacc : 0.f);
+        qacc_int = is_dof ? sol : 0.f;
+      }
+      if (is_dof) l.qvel[lane] = my_qvel + m.dt * qacc_int;
       KS_SYNC();
       if (is_body) {
         const int qa = b_qadr, da = b_dofadr;
@@ -984,7 +1004,6 @@ extern "C" int ks_model_create(const KsModelDesc* d, KsModel** out) {
     return fail(KS_ELIMIT, "ks_model_create: sizes nb=%d nq=%d nv=%d nu=%d ns=%d exceed %d/%d/%d/%d/%d", d->nb, d->nq,
                 d->nv, d->nu, d->ns, kMaxB, kMaxQ, kMaxV, kMaxU, kMaxS);
   if (d->nv > 64 || 4 * d->ns > 64) return fail(KS_ELIMIT, "ks_model_create: more than 64 dofs or constraint rows");
-  if (d->eulerdamp) return fail(KS_EINVAL, "ks_model_create: the implicit-damping Euler variant is not implemented");
   if (!(d->dt > 0.0)) return fail(KS_EINVAL, "ks_model_create: dt must be positive");
   KsModel* km = new KsModel();
   DevModel& m = km->host;

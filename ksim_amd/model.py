@@ -156,7 +156,13 @@ class ModelBuilder:
 
     def __init__(self, dt=0.005, gravity=(0.0, 0.0, -9.81), iterations=8, ls_iterations=8, tolerance=1e-10,
                  ls_tolerance=0.01, impratio=1.0, eulerdamp=False, solref=(0.02, 1.0),
-                 solimp=(0.9, 0.95, 0.001, 0.5, 2.0), friction=1.0):
+                 solimp=(0.9, 0.95, 0.001, 0.5, 2.0), friction=1.0, integrator=None):
+        # integrator: "euler" (explicit joint damping unless `eulerdamp`) or "implicitfast", the one ksim sets
+        # (ksim/task/rl.py:555-578).  With torque motors the only velocity-dependent smooth force is joint damping, so
+        # implicitfast is the damping-implicit velocity update, (M + dt diag(damping)) a = M qacc.
+        if integrator not in (None, "euler", "implicitfast"):
+            raise ValueError(f"unknown integrator {integrator!r}")
+        eulerdamp = bool(eulerdamp) or integrator == "implicitfast"
         self.opt = dict(dt=float(dt), gravity=np.array(gravity, dtype=np.float64), iterations=int(iterations),
                         ls_iterations=int(ls_iterations), tolerance=float(tolerance),
                         ls_tolerance=float(ls_tolerance), impratio=float(impratio), eulerdamp=bool(eulerdamp),

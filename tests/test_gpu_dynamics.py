@@ -15,7 +15,11 @@ from oracle.dyn import Oracle
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
-MODELS = {"chain": km.pendulum_chain_model, "humanoid": km.humanoid_model, "kbot": km.kbot_scale_model}
+MODELS = {"chain": km.pendulum_chain_model, "humanoid": km.humanoid_model, "kbot": km.kbot_scale_model,
+          # the integrator ksim selects: velocity update implicit in joint damping
+          "chain-implicit": lambda: km.pendulum_chain_model(integrator="implicitfast", damping=0.5),
+          "kbot-implicit": lambda: km.kbot_scale_model(integrator="implicitfast"),
+          "humanoid-implicit": lambda: km.humanoid_model(integrator="implicitfast")}
 ONE_STEP_TOL, TEN_STEP_TOL = 1e-4, 1e-3
 
 
@@ -115,7 +119,9 @@ def _oracle_control_steps(m, qpos, qvel, actions, kp, kd, clip, S, latency, fric
     return datas
 
 
-@pytest.mark.parametrize("name,S,T,period", [("chain", 1, 10, 1), ("kbot", 4, 2, 1), ("humanoid", 4, 2, 2)])
+@pytest.mark.parametrize("name,S,T,period", [("chain", 1, 10, 1), ("kbot", 4, 2, 1), ("humanoid", 4, 2, 2),
+                                             ("chain-implicit", 1, 10, 1), ("kbot-implicit", 4, 2, 1),
+                                             ("kbot-implicit", 1, 1, 1), ("humanoid-implicit", 4, 2, 2)])
 def test_position_controlled_steps(name, S, T, period):
     """Fused control step (latency blend + PD + S substeps) with per-env friction / mass scale."""
     from ksim_amd import physics

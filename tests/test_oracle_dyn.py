@@ -47,9 +47,9 @@ def _sink_to_contact(m, qpos, depth=0.01):
 
 
 MODELS = {
-    "chain": lambda: km.pendulum_chain_model(),
-    "humanoid": lambda: km.humanoid_model(),
-    "kbot": lambda: km.kbot_scale_model(),
+    "chain": lambda **o: km.pendulum_chain_model(**o),
+    "humanoid": lambda **o: km.humanoid_model(**o),
+    "kbot": lambda **o: km.kbot_scale_model(**o),
 }
 
 
@@ -326,3 +326,33 @@ def test_applied_cartesian_force_closed_form_and_virtual_work(model):
             S = kp["xmat"][b] @ km_["xmat"][b].T
             om = np.array([S[2, 1] - S[1, 2], S[0, 2] - S[2, 0], S[1, 0] - S[0, 1]]) / 2 / (2 * eps)
             assert Q @ dq == pytest.approx(w[:3] @ dx + w[3:] @ om, rel=1e-6, abs=1e-7)
+
+
+def test_damping_implicit_velocity_update():
+    """implicitfast with torque motors = Euler implicit in joint damping: (M + h D) a = M qacc.  One damped hinge without
+    gravity decays as v_k = v_0 (I / (I + h d))^k; on the articulated models the step equals a dense solve done here."""
+    m = km.pendulum_chain_model(n_links=1, damping=0.7, gravity=(0.0, 0.0, 0.0), integrator="implicitfast")
+    orc = Oracle(m.arrays())
+    d = orc.data(qvel=np.array([2.0]))
+    orc.forward(d)
+    inertia = float(d.M[0, 0])
+    v = 2.0
+    for _ in range(20):
+        orc.step(d)
+        v *= inertia / (inertia + m.dt * 0.7)
+        assert d.qvel[0] == pytest.approx(v, rel=1e-12)
+    rng = np.random.default_rng(4)
+    for name in ("kbot", "humanoid"):
+        mi = MODELS[name](integrator="implicitfast")
+        me = MODELS[name]()
+        assert mi.eulerdamp and not me.eulerdamp and np.any(mi.dof_damping > 0)
+        qpos, qvel = _random_state(mi, rng, vel_scale=0.5)
+        qpos = _sink_to_contact(mi, qpos)
+        oi, oe = Oracle(mi.arrays()), Oracle(me.arrays())
+        di, de = oi.data(qpos, qvel), oe.data(qpos, qvel)
+        oi.step(di); oe.forward(de)
+        np.testing.assert_allclose(di.qacc, de.qacc, rtol=1e-12, atol=1e-12)  # the solve before integration is the same
+        M, qacc = np.array(de.M), np.array(de.qacc)
+        a = np.linalg.solve(M + mi.dt * np.diag(mi.dof_damping), M @ qacc)
+        np.testing.assert_allclose(di.qvel, qvel + mi.dt * a, rtol=1e-9, atol=1e-10)
+        assert np.abs(np.array(di.qvel) - (qvel + mi.dt * qacc)).max() > 1e-6  # and differs from the explicit update
