@@ -265,35 +265,8 @@ void step_kernel(StepArgs a) {
     for (int k = 0; k < 6; ++k) l.cvel[k] = 0.f;
   }
   const float mu = a.friction ? a.friction[env] : m.friction;
-  float time = a.time ? a.time[env] : 0.f;
   const float latency = a.latency ? a.latency[env] : 0.f;
-  const float kp_scale = a.kp_scale ? a.kp_scale[env] : 1.f;
-  const float kd_scale = a.kd_scale ? a.kd_scale[env] : 1.f;
-  const float lim_scale = a.torque_limit_scale ? a.torque_limit_scale[env] : 1.f;
   const float scale = 1.0f / (m.meaninertia * (float)(nv > 1 ? nv : 1));
-  int niter_out = 0, nefc_out = 0;
-  float my_qacc = 0.f;
-  // time remaining of every velocity event (wave-uniform), kept in registers for the whole control step
-  float ev_left[KS_MAX_EVENTS];
-#pragma unroll
-  for (int e = 0; e < KS_MAX_EVENTS; ++e) ev_left[e] = (!FWD && e < a.n_events) ? a.event_state[(int64_t)e * a.N + env] : 0.f;
-  // actuator inputs of this control step (lane = actuator), read once
-  float u_last = 0.f, u_act = 0.f, u_kp = 0.f, u_kd = 0.f, u_lim = 0.f, u_zero = 0.f, u_abias = 0.f, u_tbias = 0.f;
-  bool u_drop = false;
-  if (!FWD && lane < nu) {
-    const int64_t eu = env * nu + lane;
-    u_last = a.last_ctrl[eu];
-    u_act = a.action[eu];
-    u_drop = a.drop && a.drop[eu];
-    u_zero = a.zero_offset ? a.zero_offset[eu] : 0.f;
-    if (a.actuator_type == KS_ACT_POSITION) {
-      u_kp = a.kp[lane] * kp_scale;
-      u_kd = a.kd[lane] * kd_scale;
-      u_lim = a.ctrl_clip[lane] * lim_scale;
-      u_abias = a.action_bias ? a.action_bias[eu] : 0.f;
-      u_tbias = a.torque_bias ? a.torque_bias[eu] : 0.f;
-    }
-  }
   KS_SYNC();
 #ifdef KS_PROFILE
   float prof[16];
@@ -345,6 +318,20 @@ void step_kernel(StepArgs a) {
     // ---- actuators (ksim/engine.py:287-320, ksim/actuators.py:198-217)
     if (!FWD && (sub % a.actuator_period) == 0 && lane < nu) {
       const int u = lane;
+      // the actuator inputs of this control step are read again at every actuator update (they stay in the caches):
+      // held in registers they would be live across the solver of every substep
+      const int64_t eu = env * nu + lane;
+      const float u_last = a.last_ctrl[eu], u_act = a.action[eu];
+      const bool u_drop = a.drop && a.drop[eu];
+      const float u_zero = a.zero_offset ? a.zero_offset[eu] : 0.f;
+      float u_kp = 0.f, u_kd = 0.f, u_lim = 0.f, u_abias = 0.f, u_tbias = 0.f;
+      if (a.actuator_type == KS_ACT_POSITION) {
+        u_kp = a.kp[lane] * (a.kp_scale ? a.kp_scale[env] : 1.f);
+        u_kd = a.kd[lane] * (a.kd_scale ? a.kd_scale[env] : 1.f);
+        u_lim = a.ctrl_clip[lane] * (a.torque_limit_scale ? a.torque_limit_scale[env] : 1.f);
+        u_abias = a.action_bias ? a.action_bias[eu] : 0.f;
+        u_tbias = a.torque_bias ? a.torque_bias[eu] : 0.f;
+      }
       float prct = (float)sub - latency;
       prct = fminf(fmaxf(prct, 0.f), 1.f);
       const float c = u_drop ? u_last : u_last * (1.0f - prct) + u_act * prct;
@@ -365,11 +352,13 @@ void step_kernel(StepArgs a) {
     // ---- events (ksim/engine.py:322-333, ksim/events.py): impulses on the root velocity when an interval runs out
     if (!FWD && a.n_events > 0) {
       const uint64_t ev_step = a.event_rng.step + (a.event_rng.step_base ? *a.event_rng.step_base : 0ull);
-#pragma unroll
-      for (int e = 0; e < KS_MAX_EVENTS; ++e) {
-        if (e < a.n_events && a.events[e].kind != KS_EVENT_FORCE_PUSH) {
+#pragma nounroll
+      for (int e = 0; e < a.n_events; ++e) {  // a rolled loop: nothing of the event records is kept across the substeps
+        if (a.events[e].kind != KS_EVENT_FORCE_PUSH) {
           const KsEventDesc ev = a.events[e];
-          float left = ev_left[e] - m.dt;
+          // the timer stays in memory between substeps (lane 0 owns it) so that it costs no register over the solver
+          float* tleft = a.event_state + (int64_t)e * a.N + env;
+          float left = lane_bcast(lane == 0 ? *tleft : 0.f, 0) - m.dt;
           if (left <= 0.f) {  // wave-uniform
             float u0, u1, u2;
             if (a.event_uniform) {
@@ -394,7 +383,7 @@ void step_kernel(StepArgs a) {
             }
             left = ev.interval_lo + u2 * (ev.interval_hi - ev.interval_lo);
           }
-          ev_left[e] = left;
+          if (lane == 0) *tleft = left;
         }
       }
       KS_SYNC();
@@ -567,6 +556,7 @@ void step_kernel(StepArgs a) {
       if (!FWD && a.n_force_events > 0) {
         const uint64_t ev_step = a.event_rng.step + (a.event_rng.step_base ? *a.event_rng.step_base : 0ull);
         Sp ext = {{0.f, 0.f, 0.f}, {0.f, 0.f, 0.f}};
+#pragma nounroll
         for (int e = 0; e < a.n_events; ++e) {
           if (a.events[e].kind != KS_EVENT_FORCE_PUSH) continue;
           const KsEventDesc ev = a.events[e];
@@ -905,9 +895,11 @@ void step_kernel(StepArgs a) {
       }
       Mqacc = Ma;
     }
-    niter_out = niter;
-    nefc_out = nefc;
-    my_qacc = qacc;
+    if (sub == nsub - 1) {  // outputs of the last substep go out here: nothing of them stays live to the end
+      if (a.qacc && lane < nv) a.qacc[env * nv + lane] = qacc;
+      if (a.solver_niter && lane == 0) a.solver_niter[env] = niter;
+      if (a.nefc && lane == 0) a.nefc[env] = nefc;
+    }
     KS_SYNC();
     if (is_dof) l.warm[lane] = qacc;
 
@@ -951,7 +943,6 @@ void step_kernel(StepArgs a) {
           l.qpos[qa] += m.dt * l.qvel[da];
         }
       }
-      time += m.dt;
     }
     KS_SYNC();
   }
@@ -964,11 +955,14 @@ void step_kernel(StepArgs a) {
   if (!FWD) {
     for (int i = lane; i < nq; i += 64) a.qpos[env * nq + i] = l.qpos[i];
     if (lane < nv) a.qvel[env * nv + lane] = l.qvel[lane];
-    if (a.time && lane == 0) a.time[env] = time;
-    if (a.last_ctrl && lane < nu) a.last_ctrl[env * nu + lane] = u_act;
+    if (a.time && lane == 0) {  // dt added once per substep in fp32, like the reference's accumulation
+      float time = a.time[env];
+      for (int k = 0; k < nsub; ++k) time += m.dt;
+      a.time[env] = time;
+    }
+    if (a.last_ctrl && lane < nu) a.last_ctrl[env * nu + lane] = a.action[env * nu + lane];
   }
   if (a.qacc_warmstart && lane < nv) a.qacc_warmstart[env * nv + lane] = l.warm[lane];
-  if (a.qacc && lane < nv) a.qacc[env * nv + lane] = my_qacc;
   if (a.ctrl_out) for (int i = lane; i < nu; i += 64) a.ctrl_out[env * nu + i] = l.tau[i];
   if (a.xpos) for (int i = lane; i < nb * 3; i += 64) a.xpos[env * nb * 3 + i] = l.xpos[i];
   if (a.xquat) for (int i = lane; i < nb * 4; i += 64) a.xquat[env * nb * 4 + i] = l.xquat[i];
@@ -976,12 +970,6 @@ void step_kernel(StepArgs a) {
   if (a.traj_ctrl) for (int i = lane; i < nu; i += 64) a.traj_ctrl[env * nu + i] = l.tau[i];
   if (a.traj_xpos) for (int i = lane; i < nb * 3; i += 64) a.traj_xpos[env * nb * 3 + i] = l.xpos[i];
   if (a.traj_xquat) for (int i = lane; i < nb * 4; i += 64) a.traj_xquat[env * nb * 4 + i] = l.xquat[i];
-  if (!FWD && lane == 0)
-#pragma unroll
-    for (int e = 0; e < KS_MAX_EVENTS; ++e)  // the force pushes keep their timers in memory
-      if (e < a.n_events && a.events[e].kind != KS_EVENT_FORCE_PUSH) a.event_state[(int64_t)e * a.N + env] = ev_left[e];
-  if (a.solver_niter && lane == 0) a.solver_niter[env] = niter_out;
-  if (a.nefc && lane == 0) a.nefc[env] = nefc_out;
 }
 
 }  // namespace ks

@@ -382,7 +382,7 @@ def test_recurrent_actor_and_critic_in_the_rollout():
     N, T = 24, 8
     runs = []
     for use_graph in (False, True):
-        m, c, rnd_, _, ro, EnvState = build(N, T, seed=13, min_height=0.8, recurrent=True)
+        m, c, rnd_, _, ro, EnvState = build(N, T, seed=13, min_height=0.95, recurrent=True)
         ps = c.engine.reset(c.physics_model, 1.0, 3, N, rnd_)
         env = EnvState(ps, rnd_, torch.zeros(N, 2, device=DEV), None, seed=21)
         want = {"actor": np.zeros((2, N, 32)), "critic": np.zeros((2, N, 32))}
