@@ -33,7 +33,7 @@ const char* ks_last_error(void);
 /* sizeof() of a public struct as this library was compiled, for binding self-checks:
  * 0 KsPpoLossParams, 1 KsModelDesc, 2 KsStepIO, 3 KsTermsDesc, 4 KsObserveIO, 5 KsTerminateIO, 6 KsMlpDesc,
  * 7 KsRewardIO, 8 KsObsElem, 9 KsTermDesc, 10 KsRewardDesc, 11 KsRng, 12 KsAdamParams, 13 KsEventDesc,
- * 14 KsRewardScanIO, 15 KsRewardScanDesc, 16 KsGruDesc;
+ * 14 KsRewardScanIO, 15 KsRewardScanDesc, 16 KsGruDesc, 17 KsLstmDesc, 18 KsGaussianHead;
  * -1 for anything else. */
 int64_t ks_abi_sizeof(int32_t which);
 
@@ -379,6 +379,21 @@ int ks_sample_action(ks_stream_t stream, int64_t N, int32_t nu, const float* mea
                      const float* noise_normal /*(N,nu) nullable -> Philox*/, KsRng rng, float clip_max,
                      float* action);
 
+/* The same tail for a network that also emits the standard deviation (examples/kbot/train.py:915-932): raw is
+ * (N, 2 nu) = means then raw deviations; mean = raw_mean + mean_bias, std = min((softplus(raw_std) + min_std) * var_scale,
+ * max_std), action = mean + std * noise.  Optionally returns mean, std and the per-dimension log-probability of the sample
+ * before the NaN scrub and clip, which is what the task stores as the old policy's log-probability.  The example's low-pass
+ * filter on the mean and its command-dependent bias are task code and stay outside. */
+typedef struct KsGaussianHead {
+  float min_std, max_std, var_scale;
+  int32_t deterministic;   /* 1: action = mean (argmax_action) */
+  const float* mean_bias;  /* device (nu), nullable */
+} KsGaussianHead;
+int ks_sample_action_head(ks_stream_t stream, int64_t N, int32_t nu, const float* raw /*(N, 2 nu)*/,
+                          const KsGaussianHead* head /*host*/, const float* noise_normal /*(N,nu) nullable -> Philox*/,
+                          KsRng rng, float clip_max, float* action /*(N,nu)*/, float* mean_out /*nullable*/,
+                          float* std_out /*nullable*/, float* log_prob_out /*(N,nu) nullable*/);
+
 /* ------------------------------------------------------------------ policy / critic / discriminator MLP
  * The dense contraction of the path: the network a task's sample_action calls
  * (ksim/task/rl.py:892-926,986-996; plain MLP stacks as in examples/walking.py:40-208's
@@ -429,6 +444,23 @@ int64_t ks_gru_workspace_bytes(const KsGru* gru, int64_t M);
 int ks_gru_forward(const KsGru* gru, ks_stream_t stream, int64_t M, const float* x /*(M, input_size)*/,
                    const float* h_in /*(M, H)*/, const uint8_t* fresh /*(M) nullable*/, float* h_out /*(M, H)*/,
                    void* workspace);
+
+/* LSTM cell (eqx.nn.LSTMCell, the recurrent layer of examples/kbot/train.py:837-995): g = W_ih x + W_hh h + bias with the
+ * 4H rows in gate order input | forget | cell | output; c' = sigmoid(f) c + sigmoid(i) tanh(g), h' = sigmoid(o) tanh(c').
+ * Envs marked fresh start from h = c = 0.  h_out / c_out may alias h_in / c_in.  Forward only. */
+typedef struct KsLstmDesc {
+  int32_t input_size, hidden_size, dtype;
+  const float* weight_ih; /* host (4H, input_size) */
+  const float* weight_hh; /* host (4H, H) */
+  const float* bias;      /* host (4H), nullable */
+} KsLstmDesc;
+typedef struct KsLstm KsLstm;
+int ks_lstm_create(const KsLstmDesc* desc /*host*/, KsLstm** out);
+int ks_lstm_destroy(KsLstm* lstm);
+int64_t ks_lstm_workspace_bytes(const KsLstm* lstm, int64_t M);
+int ks_lstm_forward(const KsLstm* lstm, ks_stream_t stream, int64_t M, const float* x /*(M, input_size)*/,
+                    const float* h_in /*(M, H)*/, const float* c_in /*(M, H)*/, const uint8_t* fresh /*(M) nullable*/,
+                    float* h_out, float* c_out, void* workspace);
 
 /* ------------------------------------------------------------------ policy update: gradients and optimiser
  * The native pieces of PPOTask._single_step / update_model (ksim/task/ppo.py:495-565, 572-694) for an

@@ -115,6 +115,16 @@ class KsGruDesc(ctypes.Structure):
                 ("weight_hh", c_void_p), ("bias", c_void_p), ("bias_n", c_void_p)]
 
 
+class KsGaussianHead(ctypes.Structure):
+    _fields_ = [("min_std", c_float), ("max_std", c_float), ("var_scale", c_float), ("deterministic", c_int32),
+                ("mean_bias", c_void_p)]
+
+
+class KsLstmDesc(ctypes.Structure):
+    _fields_ = [("input_size", c_int32), ("hidden_size", c_int32), ("dtype", c_int32), ("weight_ih", c_void_p),
+                ("weight_hh", c_void_p), ("bias", c_void_p)]
+
+
 class KsAdamParams(ctypes.Structure):
     _fields_ = [("lr", c_float), ("b1", c_float), ("b2", c_float), ("eps", c_float), ("weight_decay", c_float),
                 ("max_grad_norm", c_float), ("step", c_int64)]
@@ -128,7 +138,12 @@ def bind(lib) -> None:
     lib.ks_gru_workspace_bytes.argtypes = [c_void_p, c_int64]
     lib.ks_gru_workspace_bytes.restype = c_int64
     lib.ks_gru_forward.argtypes = [c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]
-    for name in ("ks_gru_create", "ks_gru_destroy", "ks_gru_forward"):
+    lib.ks_lstm_create.argtypes = [POINTER(KsLstmDesc), POINTER(c_void_p)]
+    lib.ks_lstm_destroy.argtypes = [c_void_p]
+    lib.ks_lstm_workspace_bytes.argtypes = [c_void_p, c_int64]
+    lib.ks_lstm_workspace_bytes.restype = c_int64
+    lib.ks_lstm_forward.argtypes = [c_void_p, c_void_p, c_int64] + [c_void_p] * 7
+    for name in ("ks_gru_create", "ks_gru_destroy", "ks_gru_forward", "ks_lstm_create", "ks_lstm_destroy", "ks_lstm_forward"):
         getattr(lib, name).restype = c_int32
     lib.ks_reward_scan.argtypes = [c_void_p, POINTER(KsRewardScanIO)]
     lib.ks_reward_scan.restype = c_int32
@@ -138,6 +153,9 @@ def bind(lib) -> None:
     lib.ks_terminate_reset.argtypes = [c_void_p, c_void_p, POINTER(KsTerminateIO)]
     lib.ks_sample_action.argtypes = [c_void_p, c_int64, c_int32, c_void_p, c_void_p, c_void_p, KsRng, c_float,
                                      c_void_p]
+    lib.ks_sample_action_head.argtypes = [c_void_p, c_int64, c_int32, c_void_p, POINTER(KsGaussianHead), c_void_p, KsRng,
+                                          c_float, c_void_p, c_void_p, c_void_p, c_void_p]
+    lib.ks_sample_action_head.restype = c_int32
     lib.ks_mlp_create.argtypes = [POINTER(KsMlpDesc), POINTER(c_void_p)]
     lib.ks_mlp_destroy.argtypes = [c_void_p]
     lib.ks_mlp_workspace_bytes.argtypes = [c_void_p, c_int64]

@@ -330,6 +330,8 @@ extern "C" int64_t ks_abi_sizeof(int32_t which) {
     case 14: return sizeof(KsRewardScanIO);
     case 15: return sizeof(KsRewardScanDesc);
     case 16: return sizeof(KsGruDesc);
+    case 17: return sizeof(KsLstmDesc);
+    case 18: return sizeof(KsGaussianHead);
     default: return -1;
   }
 }

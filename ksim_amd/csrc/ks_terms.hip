@@ -293,6 +293,37 @@ __global__ __launch_bounds__(256) void sample_action_kernel(int64_t n, int nu, c
   action[idx] = a;
 }
 
+// Gaussian head with a state-dependent standard deviation: the network emits (mean, raw std) per actuator.
+__global__ __launch_bounds__(256) void sample_action_head_kernel(int64_t n, int nu, const float* __restrict__ raw,
+                                                                 KsGaussianHead hd, const float* __restrict__ noise,
+                                                                 KsRng rng, float clip_max, float* __restrict__ action,
+                                                                 float* __restrict__ mean_out, float* __restrict__ std_out,
+                                                                 float* __restrict__ logp_out) {
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= n) return;
+  const int64_t e = idx / nu;
+  const int u = (int)(idx - e * nu);
+  const float mean = raw[e * 2 * nu + u] + (hd.mean_bias ? hd.mean_bias[u] : 0.f);
+  const float r = raw[e * 2 * nu + nu + u];
+  const float sp = r > 20.f ? r : log1pf(expf(r));  // softplus, linear where exp would overflow
+  const float sd = fminf((sp + hd.min_std) * hd.var_scale, hd.max_std);
+  float z = 0.f;
+  if (!hd.deterministic) {
+    if (noise) z = noise[idx];
+    else {
+      const Philox4 p = draw(rng.seed, rng.step + (rng.step_base ? *rng.step_base : 0ull), kRngAction, (uint64_t)e, (uint32_t)u);
+      z = normal_from(p.x, p.y);
+    }
+  }
+  float a = mean + sd * z;
+  if (logp_out) logp_out[idx] = -0.5f * z * z - logf(sd) - 0.91893853320467274178f;  // log N(a; mean, sd), (a - mean) / sd = z
+  if (mean_out) mean_out[idx] = mean;
+  if (std_out) std_out[idx] = sd;
+  if (a != a) a = 0.f;                         // NaN -> 0, rl.py:999-1000
+  a = fminf(fmaxf(a, -clip_max), clip_max);    // rl.py:1001
+  action[idx] = a;
+}
+
 // ---------------------------------------------------------------------------------------------
 // Rewards over a time-major rollout.  One lane per (t, env).
 // Action differences follow rewards.py:410-460: v(t) = a[t]-a[t-1], A(t) = v(t)-v(t-1),
@@ -581,6 +612,21 @@ extern "C" int ks_sample_action(ks_stream_t stream, int64_t N, int32_t nu, const
   hipLaunchKernelGGL(sample_action_kernel, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, n, (int)nu, mean,
                      log_std, noise_normal, rng, clip_max, action);
   return check_launch("ks_sample_action");
+}
+
+extern "C" int ks_sample_action_head(ks_stream_t stream, int64_t N, int32_t nu, const float* raw, const KsGaussianHead* head,
+                                     const float* noise_normal, KsRng rng, float clip_max, float* action, float* mean_out,
+                                     float* std_out, float* log_prob_out) {
+  if (N < 0 || nu < 1) return fail(KS_EINVAL, "ks_sample_action_head: bad sizes");
+  if (N == 0) return KS_OK;
+  if (!raw || !head || !action) return fail(KS_EINVAL, "ks_sample_action_head: raw, head and action are required");
+  if (!(head->max_std > 0.f) || head->min_std < 0.f || !(head->var_scale > 0.f)) return fail(KS_EINVAL, "ks_sample_action_head: standard deviation limits must be positive");
+  if (!(clip_max > 0.f)) return fail(KS_EINVAL, "ks_sample_action_head: clip_max must be positive");
+  const int64_t n = N * nu, grid = (n + 255) / 256;
+  if (grid > 0x7fffffff) return fail(KS_ELIMIT, "ks_sample_action_head: too many elements");
+  hipLaunchKernelGGL(sample_action_head_kernel, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, n, (int)nu, raw, *head,
+                     noise_normal, rng, clip_max, action, mean_out, std_out, log_prob_out);
+  return check_launch("ks_sample_action_head");
 }
 
 extern "C" int ks_rewards(ks_stream_t stream, const KsRewardIO* io) {

@@ -211,3 +211,30 @@ def sample_action(mean: torch.Tensor, log_std: torch.Tensor | None, *, noise: to
     _lib.check(lib.ks_sample_action(_lib.current_stream(), N, nu, _lib.ptr(mean), _lib.ptr(log_std), _lib.ptr(noise),
                                     _rng(seed, step, step_base), float(clip_max), _lib.ptr(out)))
     return out
+
+
+def sample_action_head(raw: torch.Tensor, *, min_std: float, max_std: float, var_scale: float = 1.0,
+                       mean_bias: torch.Tensor | None = None, noise: torch.Tensor | None = None, deterministic: bool = False,
+                       seed: int = 0, step: int = 0, step_base=None, clip_max: float = 1e3, out: torch.Tensor | None = None,
+                       want_stats: bool = False):
+    """Sampling tail for a network that emits means and raw deviations, `raw` (N, 2 nu) (examples/kbot/train.py:915-932):
+    std = min((softplus(raw_std) + min_std) * var_scale, max_std); action = mean + std * N(0,1), scrubbed and clipped
+    (ksim/task/rl.py:998-1001).  With `want_stats` also returns (mean, std, per-dimension log-probability)."""
+    lib = _lib.load()
+    _lib.require_cuda(raw, mean_bias, noise, out, dtype=torch.float32)
+    if raw.dim() != 2 or raw.shape[1] % 2:
+        raise _lib.KsError("raw must be (N, 2 nu)")
+    N, nu = raw.shape[0], raw.shape[1] // 2
+    if mean_bias is not None and tuple(mean_bias.shape) != (nu,):
+        raise _lib.KsError("mean_bias must have shape (nu,)")
+    if noise is not None and tuple(noise.shape) != (N, nu):
+        raise _lib.KsError("noise must be (N, nu)")
+    if out is None:
+        out = torch.empty((N, nu), dtype=torch.float32, device=raw.device)
+    elif tuple(out.shape) != (N, nu):
+        raise _lib.KsError("out must be (N, nu)")
+    stats = tuple(torch.empty((N, nu), dtype=torch.float32, device=raw.device) for _ in range(3)) if want_stats else (None,) * 3
+    head = T.KsGaussianHead(float(min_std), float(max_std), float(var_scale), int(bool(deterministic)), _lib.ptr(mean_bias).value)
+    _lib.check(lib.ks_sample_action_head(_lib.current_stream(), N, nu, _lib.ptr(raw), ctypes.byref(head), _lib.ptr(noise),
+                                         _rng(seed, step, step_base), float(clip_max), _lib.ptr(out), *(_lib.ptr(t) for t in stats)))
+    return (out, *stats) if want_stats else out

@@ -2,7 +2,8 @@
 (examples/walking.py:40-208).  The GRU cell follows eqx.nn.GRUCell's equations (equinox is a third-party dependency
 that is not in the reference tree): gi = W_ih x + b, gh = W_hh h, r = s(gi_r + gh_r), z = s(gi_z + gh_z),
 n = tanh(gi_n + r (gh_n + b_n)), h' = n + z (h - n).  Pinned by torch.nn.GRUCell, which computes the same cell when its
-hidden bias is (0, 0, b_n), and by hand-checkable limits (tests/test_oracle_recurrent.py).  GELU is the tanh form,
+hidden bias is (0, 0, b_n), and by hand-checkable limits (tests/test_oracle_recurrent.py).  The LSTM cell
+(eqx.nn.LSTMCell, gate order input | forget | cell | output) is pinned by torch.nn.LSTMCell.  GELU is the tanh form,
 jax.nn.gelu's default."""
 import numpy as np
 
@@ -24,6 +25,18 @@ def gru_cell(x, h, weight_ih, weight_hh, bias=None, bias_n=None):
     return n + z * (h - n)
 
 
+def lstm_cell(x, h, c, weight_ih, weight_hh, bias=None):
+    """eqx.nn.LSTMCell's equations (gate rows input | forget | cell | output): returns (h', c')."""
+    x, h, c = (np.asarray(v, dtype=np.float64) for v in (x, h, c))
+    H = h.shape[-1]
+    g = x @ np.asarray(weight_ih, dtype=np.float64).T + h @ np.asarray(weight_hh, dtype=np.float64).T
+    if bias is not None:
+        g = g + np.asarray(bias, dtype=np.float64)
+    i, f, gg, o = sigmoid(g[:, :H]), sigmoid(g[:, H:2 * H]), np.tanh(g[:, 2 * H:3 * H]), sigmoid(g[:, 3 * H:])
+    cn = f * c + i * gg
+    return o * np.tanh(cn), cn
+
+
 def gelu(x):
     x = np.asarray(x, dtype=np.float64)
     return 0.5 * x * (1.0 + np.tanh(np.sqrt(2.0 / np.pi) * (x + 0.044715 * x**3)))
@@ -41,10 +54,17 @@ def mlp(x, weights, biases, act):
 def recurrent_network(obs, carry, fresh, input_proj, cells, out_weights, out_biases, act=gelu):
     """One control step (examples/walking.py:124-150): returns (output, new carry (depth, N, H)); envs marked fresh
     start from a zero carry."""
-    carry = np.where(np.asarray(fresh, dtype=bool)[None, :, None], 0.0, np.asarray(carry, dtype=np.float64))
+    carry = np.asarray(carry, dtype=np.float64)
+    lstm = carry.ndim == 4  # (depth, 2, N, H): hidden then cell state (examples/kbot/train.py:910-913)
+    keep = ~np.asarray(fresh, dtype=bool)
+    carry = carry * (keep[None, None, :, None] if lstm else keep[None, :, None])
     x = np.asarray(obs, dtype=np.float64) @ np.asarray(input_proj[0], dtype=np.float64).T + input_proj[1]
     new = []
     for c, h in zip(cells, carry):
-        x = gru_cell(x, h, *c)
-        new.append(x)
+        if lstm:
+            x, cn = lstm_cell(x, h[0], h[1], *c)
+            new.append(np.stack([x, cn]))
+        else:
+            x = gru_cell(x, h, *c)
+            new.append(x)
     return mlp(x, out_weights, out_biases, act), np.stack(new)

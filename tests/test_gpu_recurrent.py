@@ -98,3 +98,41 @@ def test_gelu_mlp_bf16():
     m = MLP(ws, bs, activation="gelu", dtype="f32")
     with pytest.raises(Exception, match="GELU"):
         m.train_init()
+
+
+@pytest.mark.parametrize("N,I,H", [(40, 12, 16), (4096, 128, 128)])
+def test_lstm_cell_and_network(N, I, H):
+    from ksim_amd.mlp import MLP
+    from ksim_amd.recurrent import LSTMCell, RecurrentNetwork
+
+    rng = np.random.default_rng(N + 1)
+    s = 1.0 / np.sqrt(H)
+    def params(i):
+        return (rng.uniform(-s, s, (4 * H, i)), rng.uniform(-s, s, (4 * H, H)), rng.uniform(-s, s, 4 * H))
+    wi, wh, b = params(I)
+    x, h, c = rng.normal(size=(N, I)), rng.normal(size=(N, H)) * 0.5, rng.normal(size=(N, H))
+    fresh = rng.random(N) < 0.25
+    keep = ~fresh[:, None]
+    hw, cw = orec.lstm_cell(x, h * keep, c * keep, wi, wh, b)
+    mask = torch.from_numpy(fresh.astype(np.uint8)).to(DEV)
+    hg, cg = LSTMCell(wi, wh, b, dtype="f32")(t32(x), t32(h), t32(c), mask)
+    np.testing.assert_allclose(hg.cpu().numpy(), hw, rtol=2e-5, atol=2e-5)
+    np.testing.assert_allclose(cg.cpu().numpy(), cw, rtol=2e-5, atol=2e-5)
+    hg, cg = LSTMCell(wi, wh, b, dtype="bf16")(t32(x), t32(h), t32(c), mask)
+    assert np.abs(hg.cpu().numpy() - hw).max() < 3e-2 and np.abs(cg.cpu().numpy() - cw).max() < 5e-2
+    # the K-Bot actor's shape: projection, two LSTM layers, ELU output MLP; carry (depth, 2, N, H) advanced in place
+    proj = (rng.normal(size=(H, I)) / np.sqrt(I), rng.normal(size=H) * 0.1)
+    cells = [params(H) for _ in range(2)]
+    ow, ob_ = [rng.normal(size=(H, H)) / np.sqrt(H), rng.normal(size=(40, H)) / np.sqrt(H)], [rng.normal(size=H) * 0.1, np.zeros(40)]
+    net = RecurrentNetwork(proj, [LSTMCell(*p, dtype="f32") for p in cells], MLP(ow, ob_, activation="elu", dtype="f32"), dtype="f32")
+    carry = net.initial_carry(N, DEV)
+    assert tuple(carry.shape) == (2, 2, N, H)
+    want_carry = np.zeros((2, 2, N, H))
+    elu = lambda v: np.where(v > 0, v, np.expm1(v))  # noqa: E731
+    for k in range(6):
+        obs = rng.normal(size=(N, I))
+        fr = rng.random(N) < (0.0 if k == 0 else 0.2)
+        out = net(t32(obs), carry, torch.from_numpy(fr.astype(np.uint8)).to(DEV))
+        want, want_carry = orec.recurrent_network(obs, want_carry, fr, proj, cells, ow, ob_, act=elu)
+        np.testing.assert_allclose(out.cpu().numpy(), want, rtol=2e-4, atol=2e-4)
+        np.testing.assert_allclose(carry.cpu().numpy(), want_carry, rtol=2e-4, atol=2e-4)

@@ -424,3 +424,43 @@ def test_stateful_rewards_scan_against_oracle():
         np.testing.assert_allclose(cr[:, 8:14], [np.concatenate(o["c"]) for o in ocarry])
     with pytest.raises(KeyError, match="contact"):
         rw.get_rewards(traj, rewards, obs_slices={"feet_pos": slice(0, 6)}, command_slices={"lin": slice(0, 1), "ang": slice(2, 3)})
+
+
+def test_gaussian_head_with_state_dependent_deviation():
+    """mean | raw deviation head (examples/kbot/train.py:915-932): softplus, floor, scale and cap of the deviation, the
+    sample, its log-density against scipy, scrub and clip."""
+    from scipy.stats import norm
+    from ksim_amd.env_terms import sample_action_head
+
+    rng = np.random.default_rng(8)
+    N, nu = 77, 20
+    raw = rng.normal(size=(N, 2 * nu)) * 2.0
+    raw[0, nu] = 50.0        # softplus in its linear range -> capped by max_std
+    raw[1, nu + 1] = -40.0   # softplus underflows -> the floor min_std
+    raw[2, 3] = np.nan       # a NaN mean is scrubbed to 0 after sampling
+    bias = rng.normal(size=nu) * 0.1
+    z = rng.normal(size=(N, nu))
+    out, mean, std, logp = sample_action_head(t32(raw), min_std=0.01, max_std=1.5, var_scale=0.5, mean_bias=t32(bias),
+                                              noise=t32(z), clip_max=2.0, want_stats=True)
+    w_mean = raw[:, :nu] + bias
+    w_std = np.minimum((np.logaddexp(0.0, raw[:, nu:]) + 0.01) * 0.5, 1.5)
+    assert std[0, 0].item() == 1.5 and abs(std[1, 1].item() - 0.005) < 1e-7
+    np.testing.assert_allclose(std.cpu().numpy(), w_std, rtol=2e-6)
+    ok = ~np.isnan(w_mean)
+    np.testing.assert_allclose(mean.cpu().numpy()[ok], w_mean[ok], rtol=1e-6, atol=1e-6)
+    sample = w_mean + w_std * z
+    want = np.clip(np.where(np.isnan(sample), 0.0, sample), -2.0, 2.0)
+    np.testing.assert_allclose(out.cpu().numpy(), want, rtol=1e-5, atol=1e-5)
+    assert out[2, 3].item() == 0.0 and (np.abs(sample[ok]) > 2.0).any()
+    np.testing.assert_allclose(logp.cpu().numpy()[ok], norm.logpdf(sample[ok], w_mean[ok], w_std[ok]), rtol=1e-4, atol=1e-4)
+    det = sample_action_head(t32(raw), min_std=0.01, max_std=1.5, var_scale=0.5, mean_bias=t32(bias), deterministic=True, clip_max=10.0)
+    np.testing.assert_allclose(det.cpu().numpy()[ok], w_mean[ok], rtol=1e-6, atol=1e-6)
+    # Philox: reproducible per (seed, step), standard normal scores
+    a1 = sample_action_head(t32(raw), min_std=0.01, max_std=1.5, seed=4, step=9, clip_max=1e3, want_stats=True)
+    a2 = sample_action_head(t32(raw), min_std=0.01, max_std=1.5, seed=4, step=9, clip_max=1e3)
+    a3 = sample_action_head(t32(raw), min_std=0.01, max_std=1.5, seed=4, step=10, clip_max=1e3)
+    assert torch.equal(a1[0], a2) and not torch.equal(a2, a3)
+    zs = ((a1[0] - a1[1]) / a1[2]).cpu().numpy()[ok]
+    assert abs(zs.mean()) < 0.1 and abs(zs.std() - 1.0) < 0.1
+    with pytest.raises(Exception, match="2 nu"):
+        sample_action_head(t32(raw[:, :-1]), min_std=0.01, max_std=1.0)

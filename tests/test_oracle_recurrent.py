@@ -43,3 +43,23 @@ def test_gelu_and_network_composition():
     h0 = orec.gru_cell(x0, c0[0], *cells[0]); h1 = orec.gru_cell(h0, c0[1], *cells[1])
     np.testing.assert_allclose(new, np.stack([h0, h1]))
     np.testing.assert_allclose(out, orec.gelu(h1 @ ow[0].T + ob_[0]) @ ow[1].T)
+
+
+def test_lstm_cell_matches_the_library_cell():
+    rng = np.random.default_rng(2)
+    N, I, H = 5, 7, 6
+    wi, wh, b = rng.normal(size=(4 * H, I)), rng.normal(size=(4 * H, H)), rng.normal(size=4 * H)
+    x, h, c = rng.normal(size=(N, I)), rng.normal(size=(N, H)), rng.normal(size=(N, H))
+    cell = torch.nn.LSTMCell(I, H).double()
+    with torch.no_grad():
+        cell.weight_ih.copy_(torch.from_numpy(wi)); cell.weight_hh.copy_(torch.from_numpy(wh))
+        cell.bias_ih.copy_(torch.from_numpy(b)); cell.bias_hh.zero_()
+        hw, cw = cell(torch.from_numpy(x), (torch.from_numpy(h), torch.from_numpy(c)))
+    hn, cn = orec.lstm_cell(x, h, c, wi, wh, b)
+    np.testing.assert_allclose(hn, hw.numpy(), rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(cn, cw.numpy(), rtol=1e-12, atol=1e-12)
+    # forget gate saturated open, input gate shut: the cell state is kept and h = sigmoid(o) tanh(c)
+    big = np.zeros(4 * H); big[:H] = -50.0; big[H:2 * H] = 50.0
+    hn, cn = orec.lstm_cell(x, h, c, 0 * wi, 0 * wh, big)
+    np.testing.assert_allclose(cn, c, atol=1e-12)
+    np.testing.assert_allclose(hn, 0.5 * np.tanh(c), atol=1e-12)
