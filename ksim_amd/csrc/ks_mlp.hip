@@ -550,6 +550,70 @@ __global__ __launch_bounds__(256) void act_backward_kernel(int64_t n, const T* _
   dy[idx] = from_f32<T>(to_f32(dy[idx]) * d);
 }
 
+// One pass over the gradient that a layer hands down, fusing what the backward step of the layer below needs:
+//   dZ = dY * act'(Y) (in place), its transpose (for the weight-gradient product), the transpose of the stored
+//   activation Y (the other operand of the weight-gradient product of the layer above) and the column sums of dZ
+//   (the bias gradient, as kColsumSlices partial rows that sum_parts_kernel adds in a fixed order).
+// A workgroup owns 64 columns and every kColsumSlices-th tile of 64 rows; tiles go through LDS so that both the
+// row-major and the transposed accesses are 16-byte vectors.  Needs C % 64 == 0 and Mp % 64 == 0.
+template <typename T, int ACT>
+__global__ __launch_bounds__(256) void bwd_prep_kernel(int64_t M, int64_t Mp, int C, const T* __restrict__ y, T* __restrict__ dy,
+                                                       T* __restrict__ dzT, T* __restrict__ yT, float* __restrict__ part) {
+  constexpr int kPad = sizeof(T) == 2 ? 2 : 1;
+  constexpr int kVec = 16 / sizeof(T);        // elements per 16-byte vector
+  constexpr int kNv = 16 / kVec;              // vectors per thread and tile (16 elements)
+  __shared__ T sdz[64][64 + kPad];
+  __shared__ T sy[64][64 + kPad];
+  const int t = threadIdx.x;
+  const int c0 = blockIdx.x * 64;
+  const int r = t >> 2, seg = (t & 3) * 16;
+  float acc = 0.f;
+  for (int64_t tile = blockIdx.y; tile < Mp / 64; tile += gridDim.y) {
+    const int64_t m0 = tile * 64, m = m0 + r;
+    T vy[16], vd[16];
+    if (m < M) {
+#pragma unroll
+      for (int k = 0; k < kNv; ++k) {
+        reinterpret_cast<uint4*>(vy)[k] = reinterpret_cast<const uint4*>(y + m * C + c0 + seg)[k];
+        reinterpret_cast<uint4*>(vd)[k] = reinterpret_cast<const uint4*>(dy + m * C + c0 + seg)[k];
+      }
+#pragma unroll
+      for (int k = 0; k < 16; ++k) {
+        const float yv = to_f32(vy[k]);
+        float d = 1.f;
+        if (ACT == KS_ACT_ELU) d = yv > 0.f ? 1.f : yv + 1.f;
+        if (ACT == KS_ACT_RELU) d = yv > 0.f ? 1.f : 0.f;
+        if (ACT == KS_ACT_TANH) d = 1.f - yv * yv;
+        vd[k] = from_f32<T>(to_f32(vd[k]) * d);
+      }
+#pragma unroll
+      for (int k = 0; k < kNv; ++k) reinterpret_cast<uint4*>(dy + m * C + c0 + seg)[k] = reinterpret_cast<uint4*>(vd)[k];
+    } else {
+#pragma unroll
+      for (int k = 0; k < 16; ++k) { vy[k] = from_f32<T>(0.f); vd[k] = from_f32<T>(0.f); }
+    }
+    __syncthreads();  // the previous tile's readers are done
+#pragma unroll
+    for (int k = 0; k < 16; ++k) { sdz[r][seg + k] = vd[k]; sy[r][seg + k] = vy[k]; }
+    __syncthreads();
+    if (t < 64) {
+      float s0 = 0.f;
+      for (int rr = 0; rr < 64; ++rr) s0 += to_f32(sdz[rr][t]);
+      acc += s0;
+    }
+    // transposed: this thread writes 16 consecutive rows of column c0 + r
+    T od[16], oy[16];
+#pragma unroll
+    for (int k = 0; k < 16; ++k) { od[k] = sdz[seg + k][r]; oy[k] = sy[seg + k][r]; }
+#pragma unroll
+    for (int k = 0; k < kNv; ++k) {
+      reinterpret_cast<uint4*>(dzT + (int64_t)(c0 + r) * Mp + m0 + seg)[k] = reinterpret_cast<uint4*>(od)[k];
+      reinterpret_cast<uint4*>(yT + (int64_t)(c0 + r) * Mp + m0 + seg)[k] = reinterpret_cast<uint4*>(oy)[k];
+    }
+  }
+  if (t < 64) part[(int64_t)blockIdx.y * C + c0 + t] = acc;
+}
+
 // column sums of a (M, ld) matrix in two deterministic stages: gridDim.y row slices write partial sums, which
 // sum_parts_kernel adds up in a fixed order
 constexpr int kColsumSlices = 64;
@@ -951,7 +1015,7 @@ constexpr int kDwSplit = 16;  // most slices the weight-gradient reduction over 
 // workspace: hidden activations of every layer, two (M, widest) gradient buffers, two transposes (widest, Mp)
 struct TrainWs {
   char* act[KS_MAX_LAYERS];
-  char *d0, *d1, *t0, *t1;
+  char *d0, *d1, *t0, *t1, *t2;
   float* part;  // partial sums of the split reductions
   int64_t Mp;
 };
@@ -972,6 +1036,7 @@ static int64_t carve_train(const DevMlp& m, int64_t M, char* base, TrainWs* ws) 
   w.d1 = take(M * wz * esz);
   w.t0 = take((int64_t)wz * Mp * esz);
   w.t1 = take((int64_t)wz * Mp * esz);
+  w.t2 = take((int64_t)wz * Mp * esz);
   int64_t maxw = 0;
   for (int l = 0; l < m.n_layers; ++l) maxw = (int64_t)m.npad[l] * m.kpad[l] > maxw ? (int64_t)m.npad[l] * m.kpad[l] : maxw;
   const int64_t nparts = kDwSplit * maxw > (int64_t)kColsumSlices * wz ? kDwSplit * maxw : (int64_t)kColsumSlices * wz;
@@ -1027,44 +1092,75 @@ static int train_backward(DevMlp& m, hipStream_t s, int64_t M, const float* x, c
     const int64_t n = M * m.npad[L - 1];
     hipLaunchKernelGGL(cast_pad_kernel<T>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, M, m.dims[L], m.npad[L - 1], dy, dz);
   }
+  // The layer-l step needs dZ_l (row-major, for the input gradient), dZ_l^T and Y_{l-1}^T (for the weight gradient) and
+  // the column sums of dZ_l.  For hidden layers of a width that is a multiple of 64 one fused pass (bwd_prep_kernel)
+  // turns the input gradient of the layer above into all four; otherwise separate kernels do.
+  T* dzT = (T*)ws.t0;    // dZ_l^T
+  T* dzT_next = (T*)ws.t2;
+  bool have_dzT = false, have_bias = false;
   for (int l = L - 1; l >= 0; --l) {
     const int np = m.npad[l], kp = m.kpad[l], kp128 = round_up(kp, kBN);
-    // bias gradient
-    hipLaunchKernelGGL(colsum_kernel<T>, dim3((unsigned)((np + 63) / 64), kColsumSlices), dim3(256), 0, s, M, np, dz, ws.part);
-    hipLaunchKernelGGL(sum_parts_kernel, dim3((unsigned)((np + 255) / 256)), dim3(256), 0, s, (int64_t)np, kColsumSlices, ws.part, m.gb[l]);
+    if (!have_bias) {
+      hipLaunchKernelGGL(colsum_kernel<T>, dim3((unsigned)((np + 63) / 64), kColsumSlices), dim3(256), 0, s, M, np, dz, ws.part);
+      hipLaunchKernelGGL(sum_parts_kernel, dim3((unsigned)((np + 255) / 256)), dim3(256), 0, s, (int64_t)np, kColsumSlices, ws.part, m.gb[l]);
+    }
+    if (!have_dzT)
+      hipLaunchKernelGGL((transpose_kernel<T, T>), dim3((unsigned)((Mp + 31) / 32), (unsigned)((np + 31) / 32)), dim3(256), 0, s, M, np,
+                         (int64_t)np, dz, np, Mp, dzT);
+    have_dzT = have_bias = false;
+    bool have_yT = false;
+    int rc;
+    if (l > 0) {
+      // input gradient, then through the activation of the layer below
+      rc = launch_layer<T, false, false>(KS_ACT_NONE, s, M, kp, np, np, kp, dz, np, m.Wt[l], m.zero_bias, dnext, kp);
+      if (rc != KS_OK) return rc;
+      const bool fused = kp % 64 == 0 && kp == kp128 && kp == m.npad[l - 1];
+      if (fused) {
+#define KS_PREP(A) hipLaunchKernelGGL((bwd_prep_kernel<T, A>), dim3((unsigned)(kp / 64), kColsumSlices), dim3(256), 0, s, M, Mp, kp, \
+                                      (const T*)ws.act[l - 1], dnext, dzT_next, (T*)ws.t1, ws.part)
+        switch (m.activation) {
+          case KS_ACT_ELU: KS_PREP(KS_ACT_ELU); break;
+          case KS_ACT_RELU: KS_PREP(KS_ACT_RELU); break;
+          case KS_ACT_TANH: KS_PREP(KS_ACT_TANH); break;
+          default: KS_PREP(KS_ACT_NONE); break;
+        }
+#undef KS_PREP
+        hipLaunchKernelGGL(sum_parts_kernel, dim3((unsigned)((kp + 255) / 256)), dim3(256), 0, s, (int64_t)kp, kColsumSlices, ws.part, m.gb[l - 1]);
+        have_yT = have_dzT = have_bias = true;
+      } else {
+        const int64_t n = M * kp;
+#define KS_ACTB(A) hipLaunchKernelGGL((act_backward_kernel<T, A>), dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, n, (const T*)ws.act[l - 1], dnext)
+        switch (m.activation) {
+          case KS_ACT_ELU: KS_ACTB(KS_ACT_ELU); break;
+          case KS_ACT_RELU: KS_ACTB(KS_ACT_RELU); break;
+          case KS_ACT_TANH: KS_ACTB(KS_ACT_TANH); break;
+          default: break;
+        }
+#undef KS_ACTB
+      }
+    }
     // weight gradient: dZ^T (np, Mp) times Y_prev^T (kp128, Mp)^T
-    hipLaunchKernelGGL((transpose_kernel<T, T>), dim3((unsigned)((Mp + 31) / 32), (unsigned)((np + 31) / 32)), dim3(256), 0, s, M, np,
-                       (int64_t)np, dz, np, Mp, (T*)ws.t0);
-    if (l == 0)
-      hipLaunchKernelGGL((transpose_kernel<float, T>), dim3((unsigned)((Mp + 31) / 32), (unsigned)((kp128 + 31) / 32)), dim3(256), 0, s, M,
-                         m.dims[0], (int64_t)m.dims[0], x, kp128, Mp, (T*)ws.t1);
-    else
-      hipLaunchKernelGGL((transpose_kernel<T, T>), dim3((unsigned)((Mp + 31) / 32), (unsigned)((kp128 + 31) / 32)), dim3(256), 0, s, M,
-                         m.npad[l - 1], (int64_t)m.npad[l - 1], (const T*)ws.act[l - 1], kp128, Mp, (T*)ws.t1);
+    if (!have_yT) {
+      if (l == 0)
+        hipLaunchKernelGGL((transpose_kernel<float, T>), dim3((unsigned)((Mp + 31) / 32), (unsigned)((kp128 + 31) / 32)), dim3(256), 0, s, M,
+                           m.dims[0], (int64_t)m.dims[0], x, kp128, Mp, (T*)ws.t1);
+      else
+        hipLaunchKernelGGL((transpose_kernel<T, T>), dim3((unsigned)((Mp + 31) / 32), (unsigned)((kp128 + 31) / 32)), dim3(256), 0, s, M,
+                           m.npad[l - 1], (int64_t)m.npad[l - 1], (const T*)ws.act[l - 1], kp128, Mp, (T*)ws.t1);
+    }
     // the reduction runs over the rows: cut it into slices so that the grid covers the chip, then add the slices up
     int ksplit = kDwSplit;
     while (ksplit > 1 && (Mp / 64) % ksplit != 0) ksplit >>= 1;
-    int rc = launch_layer_tile<T, false, true, 64, 128, 2, 2>(KS_ACT_NONE, s, np, kp128, (int)Mp, (int)Mp, kp, ws.t0, Mp, ws.t1,
-                                                               m.zero_bias, ksplit > 1 ? (void*)ws.part : (void*)m.gW[l], kp, ksplit);
+    rc = launch_layer_tile<T, false, true, 64, 128, 2, 2>(KS_ACT_NONE, s, np, kp128, (int)Mp, (int)Mp, kp, dzT, Mp, ws.t1,
+                                                           m.zero_bias, ksplit > 1 ? (void*)ws.part : (void*)m.gW[l], kp, ksplit);
     if (rc != KS_OK) return rc;
     if (ksplit > 1) {
       const int64_t n = (int64_t)np * kp;
       hipLaunchKernelGGL(sum_parts_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, n, ksplit, ws.part, m.gW[l]);
     }
     if (l == 0) break;
-    // input gradient, then through the activation of the layer below
-    rc = launch_layer<T, false, false>(KS_ACT_NONE, s, M, kp, np, np, kp, dz, np, m.Wt[l], m.zero_bias, dnext, kp);
-    if (rc != KS_OK) return rc;
-    const int64_t n = M * kp;
-#define KS_ACTB(A) hipLaunchKernelGGL((act_backward_kernel<T, A>), dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, n, (const T*)ws.act[l - 1], dnext)
-    switch (m.activation) {
-      case KS_ACT_ELU: KS_ACTB(KS_ACT_ELU); break;
-      case KS_ACT_RELU: KS_ACTB(KS_ACT_RELU); break;
-      case KS_ACT_TANH: KS_ACTB(KS_ACT_TANH); break;
-      default: break;
-    }
-#undef KS_ACTB
     T* tmp = dz; dz = dnext; dnext = tmp;
+    tmp = dzT; dzT = dzT_next; dzT_next = tmp;
   }
   return KS_OK;
 }
