@@ -246,6 +246,9 @@ typedef struct KsStepIO {
   float* dbg_qacc_smooth;   /* (N, nv) */
   float* contact_dist;      /* (N, ns) signed distance sphere - floor of the last substep's collision pass (negative =
                                touching): the data.contact.dist that contact observations read (ksim/utils/mujoco.py:175-217) */
+  float* cinert;            /* (N, nb*10) com-based body inertias of the last substep, mjData.cinert's layout: the six
+                               entries of the symmetric inertia about the tree's centre of mass (xx yy zz xy xz yz), mass times
+                               the offset of the body's centre (3), mass (ksim/observation.py:285-290); nullable */
   /* events (ks_step only) */
   int32_t n_events;
   KsEventDesc events[KS_MAX_EVENTS];
@@ -270,7 +273,8 @@ int ks_forward(const KsModel* model, ks_stream_t stream, const KsStepIO* io /*ho
 enum { /* KsObsElem.src: which per-env array the element reads, all (N, dim) f32 */
   KS_SRC_QPOS = 0, KS_SRC_QVEL = 1, KS_SRC_QACC = 2, KS_SRC_CTRL = 3, KS_SRC_LAST_ACTION = 4,
   KS_SRC_COMMAND = 5, KS_SRC_TIME = 6, KS_SRC_XPOS = 7, KS_SRC_XQUAT = 8, KS_SRC_CVEL = 9,
-  KS_SRC_CONST = 10, KS_SRC_CONTACT_DIST = 11 /* (N, ns) KsStepIO.contact_dist */, KS_SRC_COUNT = 12
+  KS_SRC_CONST = 10, KS_SRC_CONTACT_DIST = 11 /* (N, ns) KsStepIO.contact_dist */,
+  KS_SRC_CINERT = 12 /* (N, nb*10) KsStepIO.cinert */, KS_SRC_COUNT = 13
 };
 enum { /* KsObsElem.kind */
   KS_OBS_COPY = 0,      /* src[index]                                  (observation.py:185-195,254-257,300-303,343-352) */

@@ -6,7 +6,7 @@ from ctypes import POINTER, c_float, c_int8, c_int32, c_int64, c_uint8, c_uint64
 
 KS_MAX_OBS, KS_MAX_TERMS, KS_MAX_QPOS, KS_MAX_LAYERS = 512, 16, 40, 8
 (SRC_QPOS, SRC_QVEL, SRC_QACC, SRC_CTRL, SRC_LAST_ACTION, SRC_COMMAND, SRC_TIME, SRC_XPOS, SRC_XQUAT, SRC_CVEL,
- SRC_CONST, SRC_CONTACT_DIST, SRC_COUNT) = range(13)
+ SRC_CONST, SRC_CONTACT_DIST, SRC_CINERT, SRC_COUNT) = range(14)
 OBS_COPY, OBS_JOINT_POS, OBS_ROT_INV, OBS_CONTACT, OBS_DELAYED, OBS_GRAVITY_EMA = range(6)
 NOISE_NONE, NOISE_ADD_GAUSSIAN, NOISE_ADD_UNIFORM, NOISE_MUL_GAUSSIAN, NOISE_MUL_UNIFORM = range(5)
 (TERM_MIN_HEIGHT, TERM_BAD_Z, TERM_NOT_UPRIGHT, TERM_BAD_VELOCITY, TERM_FAR_FROM_ORIGIN,

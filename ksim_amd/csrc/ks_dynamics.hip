@@ -478,7 +478,13 @@ void step_kernel(StepArgs a) {
       if (is_body) {
 #pragma unroll
         for (int k = 0; k < 10; ++k) l.cinert[10 * lane + k] = ci[k];
+        if (a.cinert && sub == nsub - 1) {  // the LDS copy is scratch that the constraint rows reuse: export it here
+#pragma unroll
+          for (int k = 0; k < 10; ++k) a.cinert[((int64_t)env * nb + lane) * 10 + k] = ci[k];
+        }
       }
+      if (a.cinert && sub == nsub - 1 && lane == 0)
+        for (int k = 0; k < 10; ++k) a.cinert[(int64_t)env * nb * 10 + k] = 0.f;  // world body
     }
     Sp my_cdof = {{0.f, 0.f, 0.f}, {0.f, 0.f, 0.f}};
     if (is_dof) {
@@ -1144,7 +1150,7 @@ static int launch_step(const KsModel* km, ks_stream_t stream, const KsStepIO* io
   a.traj_ctrl = io->traj_ctrl; a.traj_xpos = io->traj_xpos; a.traj_xquat = io->traj_xquat;
   a.solver_niter = io->solver_niter; a.nefc = io->nefc;
   a.dbg_M = io->dbg_M; a.dbg_bias = io->dbg_bias; a.dbg_qacc_smooth = io->dbg_qacc_smooth;
-  a.contact_dist = io->contact_dist;
+  a.contact_dist = io->contact_dist; a.cinert = io->cinert;
   a.ctrl_in = io->ctrl_in;
   if (!forward_only) {
     if (io->substeps < 1 || io->substeps > 64) return fail(KS_EINVAL, "ks_step: substeps must be in 1..64");

@@ -496,7 +496,7 @@ extern "C" int ks_terms_create(const KsTermsDesc* d, KsTerms** out) {
   if (d->obs_dim < 0 || d->obs_dim > KS_MAX_OBS) return fail(KS_ELIMIT, "ks_terms_create: obs_dim %d > %d", d->obs_dim, KS_MAX_OBS);
   if (d->n_terms < 0 || d->n_terms > KS_MAX_TERMS) return fail(KS_ELIMIT, "ks_terms_create: %d terminations > %d", d->n_terms, KS_MAX_TERMS);
   if (d->nq < 0 || d->nq > KS_MAX_QPOS || d->nv < 0 || d->nu < 0 || d->nb < 1) return fail(KS_EINVAL, "ks_terms_create: bad sizes");
-  const int src_dim[KS_SRC_COUNT] = {d->nq, d->nv, d->nv, d->nu, d->nu, d->command_dim, 1, d->nb * 3, d->nb * 4, d->nb * 6, 0, d->ns};
+  const int src_dim[KS_SRC_COUNT] = {d->nq, d->nv, d->nv, d->nu, d->nu, d->command_dim, 1, d->nb * 3, d->nb * 4, d->nb * 6, 0, d->ns, d->nb * 10};
   if (d->ns < 0 || d->carry_dim < 0) return fail(KS_EINVAL, "ks_terms_create: negative sphere count or carry size");
   for (int k = 0; k < d->obs_dim; ++k) {
     const KsObsElem& el = d->obs[k];
@@ -551,7 +551,7 @@ extern "C" int ks_observe(const KsTerms* t, ks_stream_t stream, const KsObserveI
   const KsTermsDesc& d = t->host;
   if (io->N < 0) return fail(KS_EINVAL, "ks_observe: negative env count");
   if (io->N == 0 || d.obs_dim == 0) return KS_OK;
-  const int src_dim[KS_SRC_COUNT] = {d.nq, d.nv, d.nv, d.nu, d.nu, d.command_dim, 1, d.nb * 3, d.nb * 4, d.nb * 6, 0, d.ns};
+  const int src_dim[KS_SRC_COUNT] = {d.nq, d.nv, d.nv, d.nu, d.nu, d.command_dim, 1, d.nb * 3, d.nb * 4, d.nb * 6, 0, d.ns, d.nb * 10};
   if (d.carry_dim > 0 && !io->carry) return fail(KS_EINVAL, "ks_observe: the stateful observations need a carry buffer");
   ObserveArgs a;
   std::memset(&a, 0, sizeof(a));

@@ -131,6 +131,29 @@ class CenterOfMassVelocityObservation(Observation):  # observation.py:293-297 (c
 
 
 @dataclass(frozen=True)
+class CenterOfMassInertiaObservation(Observation):  # observation.py:285-290 (cinert[1:].ravel())
+    def elements(self, m, command_dim):
+        return _copy(T.SRC_CINERT, 10, (m.nb - 1) * 10)
+
+
+@dataclass(frozen=True)
+class BodyVelocityObservation(Observation):  # observation.py:544-560 (cvel of chosen bodies: angular, then linear)
+    body_idxs: tuple = ()
+
+    def elements(self, m, command_dim):
+        return [e for b in self.body_idxs for e in _copy(T.SRC_CVEL, 6 * b, 6)]
+
+
+@dataclass(frozen=True)
+class ActPosObservation(Observation):  # observation.py:717-750: (last action, joint position) of one joint, for debugging
+    ctrl_idx: int = 0
+    qpos_idx: int = 7
+
+    def elements(self, m, command_dim):
+        return _copy(T.SRC_LAST_ACTION, self.ctrl_idx, 1) + _copy(T.SRC_QPOS, self.qpos_idx, 1)
+
+
+@dataclass(frozen=True)
 class BodyPositionObservation(Observation):  # observation.py:524-559 (xpos of chosen bodies)
     body_ids: tuple = ()
 
@@ -144,6 +167,13 @@ class BodyOrientationObservation(Observation):  # observation.py:618-641
 
     def elements(self, m, command_dim):
         return [e for b in self.body_ids for e in _copy(T.SRC_XQUAT, 4 * b, 4)]
+
+
+@dataclass(frozen=True)
+class FeetOrientationObservation(BodyOrientationObservation):  # observation.py:672-703: exactly the two feet
+    def __post_init__(self):
+        if len(self.body_ids) != 2:
+            raise ValueError("FeetOrientationObservation expects exactly two bodies (left and right foot).")
 
 
 @dataclass(frozen=True)

@@ -24,6 +24,7 @@ class PhysicsData:
     xquat: torch.Tensor           # (N, nb*4)
     cvel: torch.Tensor            # (N, nb*6)
     contact_dist: torch.Tensor | None = None  # (N, ns) sphere-floor distance of the last collision pass (contact.dist)
+    cinert: torch.Tensor | None = None        # (N, nb*10) com-based body inertias (mjData.cinert)
 
 
 @dataclass

@@ -464,3 +464,28 @@ def test_gaussian_head_with_state_dependent_deviation():
     assert abs(zs.mean()) < 0.1 and abs(zs.std() - 1.0) < 0.1
     with pytest.raises(Exception, match="2 nu"):
         sample_action_head(t32(raw[:, :-1]), min_std=0.01, max_std=1.0)
+
+
+def test_body_velocity_inertia_and_debug_observations():
+    """Observations over the step kernel's extra outputs (cvel, cinert) and the small gather classes."""
+    from ksim_amd import _lib_terms as T, model as km, observation as ob
+    from ksim_amd.env_terms import EnvTerms
+
+    m = km.kbot_scale_model()
+    N = 9
+    s = _state(m, N, 21)
+    rng = s["rng"]
+    cvel, cinert, xquat = rng.normal(size=(N, m.nb * 6)), rng.normal(size=(N, m.nb * 10)), rng.normal(size=(N, m.nb * 4))
+    observations = {"inertia": ob.CenterOfMassInertiaObservation(), "body_vel": ob.BodyVelocityObservation(body_idxs=(3, 1)),
+                    "feet_quat": ob.FeetOrientationObservation(body_ids=(5, 9)), "act_pos": ob.ActPosObservation(ctrl_idx=4, qpos_idx=11)}
+    terms = EnvTerms(m, observations, {}, [])
+    assert terms.obs_dim == (m.nb - 1) * 10 + 12 + 8 + 2 and T.SRC_CINERT in terms.sources_used
+    src = {T.SRC_QPOS: t32(s["qpos"]), T.SRC_CVEL: t32(cvel), T.SRC_CINERT: t32(cinert), T.SRC_XQUAT: t32(xquat),
+           T.SRC_LAST_ACTION: t32(s["last"])}
+    obs = torch.empty(N, terms.obs_dim, device=DEV)
+    terms.observe(src, N, obs=obs)
+    want = np.concatenate([cinert[:, 10:], cvel[:, 18:24], cvel[:, 6:12], xquat[:, 20:24], xquat[:, 36:40],
+                           s["last"][:, 4:5], s["qpos"][:, 11:12]], axis=1)
+    np.testing.assert_allclose(obs.cpu().numpy(), want.astype(np.float32), rtol=0, atol=0)
+    with pytest.raises(ValueError):
+        ob.FeetOrientationObservation(body_ids=(1, 2, 3))

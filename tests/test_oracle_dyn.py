@@ -356,3 +356,27 @@ def test_damping_implicit_velocity_update():
         a = np.linalg.solve(M + mi.dt * np.diag(mi.dof_damping), M @ qacc)
         np.testing.assert_allclose(di.qvel, qvel + mi.dt * a, rtol=1e-9, atol=1e-10)
         assert np.abs(np.array(di.qvel) - (qvel + mi.dt * qacc)).max() > 1e-6  # and differs from the explicit update
+
+
+def test_com_based_inertia_closed_form(model):
+    """cinert = (inertia about the tree's centre of mass: xx yy zz xy xz yz, m d, m) with d = body centre - tree centre:
+    parallel-axis theorem on the rotated principal inertia, stated here with plain numpy.  The per-env mass scale
+    multiplies the masses only, like the randomizer it models (ksim/randomization.py:207-222)."""
+    rng = np.random.default_rng(17)
+    qpos, _ = _random_state(model, rng)
+    scale = rng.uniform(0.9, 1.1, size=model.nb)
+    orc = Oracle(model.arrays())
+    d = orc.data(qpos, mass_scale=scale)
+    orc.position_stage(d)
+    a = model.arrays()
+    kin = km.host_kinematics(a, qpos)
+    mass = np.asarray(a["body_mass"]) * scale
+    com = (mass[:, None] * kin["xipos"]).sum(0) / mass.sum()
+    np.testing.assert_allclose(d.com, com, atol=1e-12)
+    got = np.array(d.cinert)
+    for b in range(1, model.nb):
+        R = kin["ximat"][b]
+        off = kin["xipos"][b] - com
+        I = R @ np.diag(np.asarray(a["body_inertia"])[b]) @ R.T + mass[b] * (off @ off * np.eye(3) - np.outer(off, off))
+        want = [I[0, 0], I[1, 1], I[2, 2], I[0, 1], I[0, 2], I[1, 2], *(mass[b] * off), mass[b]]
+        np.testing.assert_allclose(got[b], want, rtol=1e-10, atol=1e-12)
