@@ -249,6 +249,9 @@ typedef struct KsStepIO {
   float* cinert;            /* (N, nb*10) com-based body inertias of the last substep, mjData.cinert's layout: the six
                                entries of the symmetric inertia about the tree's centre of mass (xx yy zz xy xz yz), mass times
                                the offset of the body's centre (3), mass (ksim/observation.py:285-290); nullable */
+  float* cfrc_ext;          /* (N, nb*6) contact force on each body of the last substep as a spatial force about the tree's
+                               centre of mass, world axes, torque then force: mjData.cfrc_ext, which the feet force / torque
+                               observations read (ksim/observation.py:563-616); nullable */
   /* events (ks_step only) */
   int32_t n_events;
   KsEventDesc events[KS_MAX_EVENTS];
@@ -274,7 +277,8 @@ enum { /* KsObsElem.src: which per-env array the element reads, all (N, dim) f32
   KS_SRC_QPOS = 0, KS_SRC_QVEL = 1, KS_SRC_QACC = 2, KS_SRC_CTRL = 3, KS_SRC_LAST_ACTION = 4,
   KS_SRC_COMMAND = 5, KS_SRC_TIME = 6, KS_SRC_XPOS = 7, KS_SRC_XQUAT = 8, KS_SRC_CVEL = 9,
   KS_SRC_CONST = 10, KS_SRC_CONTACT_DIST = 11 /* (N, ns) KsStepIO.contact_dist */,
-  KS_SRC_CINERT = 12 /* (N, nb*10) KsStepIO.cinert */, KS_SRC_COUNT = 13
+  KS_SRC_CINERT = 12 /* (N, nb*10) KsStepIO.cinert */,
+  KS_SRC_CFRC_EXT = 13 /* (N, nb*6) KsStepIO.cfrc_ext */, KS_SRC_COUNT = 14
 };
 enum { /* KsObsElem.kind */
   KS_OBS_COPY = 0,      /* src[index]                                  (observation.py:185-195,254-257,300-303,343-352) */
@@ -526,13 +530,26 @@ enum { KS_REW_STAY_ALIVE = 0, KS_REW_BASE_HEIGHT = 1, KS_REW_BASE_HEIGHT_RANGE =
        KS_REW_ACTION_ACC = 4, KS_REW_ACTION_JERK = 5, KS_REW_UPRIGHT_ANGVEL = 6, KS_REW_UPRIGHT_LINVEL = 7,
        KS_REW_UPRIGHT_POSE = 8,
        KS_REW_AMP = 9, /* max(0, 1 - 0.25 (logit - 1)^2) of the discriminator logits, ksim/task/amp.py:99-112 */
-       KS_REW_STATEFUL = 10 /* a value ks_reward_scan computed: stateful[norm] (norm = slot index) */ };
+       KS_REW_STATEFUL = 10, /* a value ks_reward_scan computed: stateful[norm] (norm = slot index) */
+       /* command tracking (ksim/rewards.py:84-88,236-372).  k(x) = -abs |x| - sq x^2 + exp(-x^2 / (2 scale^2)), p0 = scale,
+        * p1 = sq, p2 = abs, p3 = zero_threshold; the command entries sit at command[index ...]. */
+       KS_REW_LINVEL_CMD = 11, /* base velocity in the robot frame against a LinearVelocityCommandValue (vel, yaw, xvel,
+                                  yvel at index + 0..3); norm picks the component: 0 vel = k(|v_xy| - vel), 1 yaw =
+                                  k(atan2(v_y, v_x) - yaw), 2 x = k(v_x - xvel), 3 y = k(v_y - yvel); components 1-3 are
+                                  zero while |vel command| < p3 */
+       KS_REW_ANGVEL_CMD = 12, /* yaw rate qvel[5] against command[index]: norm 0 mag = k(w - cmd); norm 1 dir = +1 when
+                                  the signs (zero inside +-p3) agree, else -1 */
+       KS_REW_OFF_AXIS = 13,   /* exp(-v^2 / (2 p0^2)) of v = qvel[2] (norm 0), qvel[4] (norm 1), qvel[5] (norm 2) */
+       KS_REW_MOTIONLESS = 14, /* |qvel[6:]| while |qvel[0:2]| < p0 and qvel[5] < p1, else 0 (rewards.py:1206-1221) */
+       KS_REW_FORCE = 15       /* max over `norm` bodies of (max(|obs[index + 3 b .. +3]| - p1, 0) / p0)^2 (rewards.py:1224-1240) */ };
 enum { KS_NORM_L1 = 0, KS_NORM_L2 = 1 }; /* xax.get_norm: l1 = |x|, l2 = x^2 (reference tests/test_rewards.py:95-98) */
 typedef struct KsRewardDesc {
   int32_t kind;
   int32_t norm;   /* action-difference penalties */
   float scale;
   float p0, p1, p2; /* balance,success_reward,has_success_reward | target,kernel_scale | lo,hi,dropoff | scale,sq,abs */
+  float p3;
+  int32_t index;    /* offset into the command or observation vector, for the kinds that read one */
 } KsRewardDesc;
 typedef struct KsRewardIO {
   int64_t T, N;
@@ -549,6 +566,9 @@ typedef struct KsRewardIO {
   float* components;   /* (n_rewards, T, N) nullable */
   float* total;        /* (T, N) */
   const float* stateful; /* (n_slots, T, N) output of ks_reward_scan, KS_REW_STATEFUL only */
+  int32_t command_dim, obs_dim;
+  const float* command;  /* (T, N, command_dim), command-tracking kinds only */
+  const float* obs;      /* (T, N, obs_dim), KS_REW_FORCE only */
 } KsRewardIO;
 int ks_rewards(ks_stream_t stream, const KsRewardIO* io /*host*/);
 

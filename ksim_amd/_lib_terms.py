@@ -6,7 +6,7 @@ from ctypes import POINTER, c_float, c_int8, c_int32, c_int64, c_uint8, c_uint64
 
 KS_MAX_OBS, KS_MAX_TERMS, KS_MAX_QPOS, KS_MAX_LAYERS = 512, 16, 40, 8
 (SRC_QPOS, SRC_QVEL, SRC_QACC, SRC_CTRL, SRC_LAST_ACTION, SRC_COMMAND, SRC_TIME, SRC_XPOS, SRC_XQUAT, SRC_CVEL,
- SRC_CONST, SRC_CONTACT_DIST, SRC_CINERT, SRC_COUNT) = range(14)
+ SRC_CONST, SRC_CONTACT_DIST, SRC_CINERT, SRC_CFRC_EXT, SRC_COUNT) = range(15)
 OBS_COPY, OBS_JOINT_POS, OBS_ROT_INV, OBS_CONTACT, OBS_DELAYED, OBS_GRAVITY_EMA = range(6)
 NOISE_NONE, NOISE_ADD_GAUSSIAN, NOISE_ADD_UNIFORM, NOISE_MUL_GAUSSIAN, NOISE_MUL_UNIFORM = range(5)
 (TERM_MIN_HEIGHT, TERM_BAD_Z, TERM_NOT_UPRIGHT, TERM_BAD_VELOCITY, TERM_FAR_FROM_ORIGIN,
@@ -75,7 +75,8 @@ class KsMlpDesc(ctypes.Structure):
 
 
 (REW_STAY_ALIVE, REW_BASE_HEIGHT, REW_BASE_HEIGHT_RANGE, REW_ACTION_VEL, REW_ACTION_ACC, REW_ACTION_JERK,
- REW_UPRIGHT_ANGVEL, REW_UPRIGHT_LINVEL, REW_UPRIGHT_POSE, REW_AMP, REW_STATEFUL) = range(11)
+ REW_UPRIGHT_ANGVEL, REW_UPRIGHT_LINVEL, REW_UPRIGHT_POSE, REW_AMP, REW_STATEFUL, REW_LINVEL_CMD, REW_ANGVEL_CMD,
+ REW_OFF_AXIS, REW_MOTIONLESS, REW_FORCE) = range(16)
 KS_MAX_REWARD_SCANS, KS_MAX_SCAN_BODIES = 4, 8
 SCAN_FEET_AIR_TIME, SCAN_SPARSE_TARGET_HEIGHT = 0, 1
 NORM_L1, NORM_L2 = 0, 1
@@ -84,7 +85,7 @@ KS_MAX_REWARD_TERMS = 32
 
 class KsRewardDesc(ctypes.Structure):
     _fields_ = [("kind", c_int32), ("norm", c_int32), ("scale", c_float), ("p0", c_float), ("p1", c_float),
-                ("p2", c_float)]
+                ("p2", c_float), ("p3", c_float), ("index", c_int32)]
 
 
 class KsRewardIO(ctypes.Structure):
@@ -92,7 +93,8 @@ class KsRewardIO(ctypes.Structure):
                 ("n_rewards", c_int32), ("rewards", KsRewardDesc * KS_MAX_REWARD_TERMS), ("use_clip_min", c_int32),
                 ("use_clip_max", c_int32), ("clip_min", c_float), ("clip_max", c_float), ("qpos", c_void_p),
                 ("qvel", c_void_p), ("action", c_void_p), ("done", c_void_p), ("success", c_void_p),
-                ("disc_logits", c_void_p), ("components", c_void_p), ("total", c_void_p), ("stateful", c_void_p)]
+                ("disc_logits", c_void_p), ("components", c_void_p), ("total", c_void_p), ("stateful", c_void_p),
+                ("command_dim", c_int32), ("obs_dim", c_int32), ("command", c_void_p), ("obs", c_void_p)]
 
 
 class KsRewardScanDesc(ctypes.Structure):

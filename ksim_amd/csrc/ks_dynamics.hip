@@ -900,6 +900,33 @@ void step_kernel(StepArgs a) {
         KS_TICK(13)
       }
       Mqacc = Ma;
+      // ---- Cartesian contact forces on the bodies (mjData.cfrc_ext), only when asked for: a pyramid row with force f
+      // pushes along normal +- mu tangent (rows of a contact: z + mu y, z - mu y, z - mu x, z + mu x)
+      if (a.cfrc_ext && sub == nsub - 1) {
+        const float f = (is_row && Jaref < 0.f) ? -D * Jaref : 0.f;
+        const int q = lane & 3;
+        float fx = q == 3 ? mu * f : (q == 2 ? -mu * f : 0.f);
+        float fy = q == 0 ? mu * f : (q == 1 ? -mu * f : 0.f);
+        float fz = f;
+        fx += __shfl_xor(fx, 1); fy += __shfl_xor(fy, 1); fz += __shfl_xor(fz, 1);
+        fx += __shfl_xor(fx, 2); fy += __shfl_xor(fy, 2); fz += __shfl_xor(fz, 2);
+        KS_SYNC();  // the line search is done with drow
+        if (is_row && q == 0) { l.drow[3 * (lane >> 2)] = fx; l.drow[3 * (lane >> 2) + 1] = fy; l.drow[3 * (lane >> 2) + 2] = fz; }
+        KS_SYNC();
+        if (lane < nb) {
+          Sp w = {{0.f, 0.f, 0.f}, {0.f, 0.f, 0.f}};
+          for (int k = 0; k < ncon; ++k)
+            if (l.con_body[k] == lane) {
+              const V3 F = ld3(l.drow + 3 * k);
+              w.a = w.a + cross(ld3(l.con_off + 3 * k), F);
+              w.l = w.l + F;
+            }
+          float* dst = a.cfrc_ext + ((int64_t)env * nb + lane) * 6;
+          dst[0] = w.a.x; dst[1] = w.a.y; dst[2] = w.a.z; dst[3] = w.l.x; dst[4] = w.l.y; dst[5] = w.l.z;
+        }
+      }
+    } else if (a.cfrc_ext && sub == nsub - 1) {
+      for (int i = lane; i < nb * 6; i += 64) a.cfrc_ext[(int64_t)env * nb * 6 + i] = 0.f;
     }
     if (sub == nsub - 1) {  // outputs of the last substep go out here: nothing of them stays live to the end
       if (a.qacc && lane < nv) a.qacc[env * nv + lane] = qacc;
@@ -1150,7 +1177,7 @@ static int launch_step(const KsModel* km, ks_stream_t stream, const KsStepIO* io
   a.traj_ctrl = io->traj_ctrl; a.traj_xpos = io->traj_xpos; a.traj_xquat = io->traj_xquat;
   a.solver_niter = io->solver_niter; a.nefc = io->nefc;
   a.dbg_M = io->dbg_M; a.dbg_bias = io->dbg_bias; a.dbg_qacc_smooth = io->dbg_qacc_smooth;
-  a.contact_dist = io->contact_dist; a.cinert = io->cinert;
+  a.contact_dist = io->contact_dist; a.cinert = io->cinert; a.cfrc_ext = io->cfrc_ext;
   a.ctrl_in = io->ctrl_in;
   if (!forward_only) {
     if (io->substeps < 1 || io->substeps > 64) return fail(KS_EINVAL, "ks_step: substeps must be in 1..64");

@@ -22,7 +22,7 @@ struct StepArgs {
   const uint8_t* env_mask;
   float *qacc, *ctrl_out, *xpos, *xquat, *cvel, *traj_ctrl, *traj_xpos, *traj_xquat;
   int32_t *solver_niter, *nefc;
-  float *dbg_M, *dbg_bias, *dbg_qacc_smooth, *contact_dist, *cinert;
+  float *dbg_M, *dbg_bias, *dbg_qacc_smooth, *contact_dist, *cinert, *cfrc_ext;
   int n_events;
   KsEventDesc events[KS_MAX_EVENTS];
   float* event_state;

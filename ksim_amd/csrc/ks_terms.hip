@@ -403,6 +403,48 @@ __global__ __launch_bounds__(256) void rewards_kernel(KsRewardIO io) {
         val = fmaxf(0.f, 1.0f - 0.25f * d * d);
       } break;
       case KS_REW_STATEFUL: val = io.stateful[(int64_t)r.norm * TN + idx]; break;
+      case KS_REW_LINVEL_CMD: {
+        const float* cmd = io.command + idx * io.command_dim + r.index;
+        float lv[3];
+        rot_inv(q + 3, v[0], v[1], v[2], lv);
+        float x;
+        if (r.norm == 0) x = sqrtf(lv[0] * lv[0] + lv[1] * lv[1]) - cmd[0];
+        else if (r.norm == 1) x = atan2f(lv[1], lv[0]) - cmd[1];
+        else if (r.norm == 2) x = lv[0] - cmd[2];
+        else x = lv[1] - cmd[3];
+        val = kernel_with_penalty(x, r.p0, r.p1, r.p2);
+        if (r.norm != 0 && fabsf(cmd[0]) < r.p3) val = 0.f;
+      } break;
+      case KS_REW_ANGVEL_CMD: {
+        const float c = io.command[idx * io.command_dim + r.index], w = v[5];
+        if (r.norm == 0) {
+          val = kernel_with_penalty(w - c, r.p0, r.p1, r.p2);
+        } else {
+          const float sw = fabsf(w) < r.p3 ? 0.f : (w > 0.f ? 1.f : -1.f);
+          const float sc2 = fabsf(c) < r.p3 ? 0.f : (c > 0.f ? 1.f : -1.f);
+          val = sw == sc2 ? 1.f : -1.f;
+        }
+      } break;
+      case KS_REW_OFF_AXIS: {
+        const float x = v[r.norm == 0 ? 2 : (r.norm == 1 ? 4 : 5)];
+        val = expf(-(x * x) / (2.f * r.p0 * r.p0));
+      } break;
+      case KS_REW_MOTIONLESS: {
+        const bool still = sqrtf(v[0] * v[0] + v[1] * v[1]) < r.p0 && v[5] < r.p1;
+        float s2 = 0.f;
+        for (int j = 6; j < io.nv; ++j) s2 += v[j] * v[j];
+        val = still ? sqrtf(s2) : 0.f;
+      } break;
+      case KS_REW_FORCE: {
+        const float* ob = io.obs + idx * io.obs_dim + r.index;
+        float best = 0.f;
+        for (int b = 0; b < r.norm; ++b) {
+          const float n = sqrtf(ob[3 * b] * ob[3 * b] + ob[3 * b + 1] * ob[3 * b + 1] + ob[3 * b + 2] * ob[3 * b + 2]);
+          const float e = fmaxf(n - r.p1, 0.f) / r.p0;
+          best = b == 0 ? e * e : fmaxf(best, e * e);
+        }
+        val = best;
+      } break;
       default: break;
     }
     val *= r.scale;
@@ -496,7 +538,7 @@ extern "C" int ks_terms_create(const KsTermsDesc* d, KsTerms** out) {
   if (d->obs_dim < 0 || d->obs_dim > KS_MAX_OBS) return fail(KS_ELIMIT, "ks_terms_create: obs_dim %d > %d", d->obs_dim, KS_MAX_OBS);
   if (d->n_terms < 0 || d->n_terms > KS_MAX_TERMS) return fail(KS_ELIMIT, "ks_terms_create: %d terminations > %d", d->n_terms, KS_MAX_TERMS);
   if (d->nq < 0 || d->nq > KS_MAX_QPOS || d->nv < 0 || d->nu < 0 || d->nb < 1) return fail(KS_EINVAL, "ks_terms_create: bad sizes");
-  const int src_dim[KS_SRC_COUNT] = {d->nq, d->nv, d->nv, d->nu, d->nu, d->command_dim, 1, d->nb * 3, d->nb * 4, d->nb * 6, 0, d->ns, d->nb * 10};
+  const int src_dim[KS_SRC_COUNT] = {d->nq, d->nv, d->nv, d->nu, d->nu, d->command_dim, 1, d->nb * 3, d->nb * 4, d->nb * 6, 0, d->ns, d->nb * 10, d->nb * 6};
   if (d->ns < 0 || d->carry_dim < 0) return fail(KS_EINVAL, "ks_terms_create: negative sphere count or carry size");
   for (int k = 0; k < d->obs_dim; ++k) {
     const KsObsElem& el = d->obs[k];
@@ -551,7 +593,7 @@ extern "C" int ks_observe(const KsTerms* t, ks_stream_t stream, const KsObserveI
   const KsTermsDesc& d = t->host;
   if (io->N < 0) return fail(KS_EINVAL, "ks_observe: negative env count");
   if (io->N == 0 || d.obs_dim == 0) return KS_OK;
-  const int src_dim[KS_SRC_COUNT] = {d.nq, d.nv, d.nv, d.nu, d.nu, d.command_dim, 1, d.nb * 3, d.nb * 4, d.nb * 6, 0, d.ns, d.nb * 10};
+  const int src_dim[KS_SRC_COUNT] = {d.nq, d.nv, d.nv, d.nu, d.nu, d.command_dim, 1, d.nb * 3, d.nb * 4, d.nb * 6, 0, d.ns, d.nb * 10, d.nb * 6};
   if (d.carry_dim > 0 && !io->carry) return fail(KS_EINVAL, "ks_observe: the stateful observations need a carry buffer");
   ObserveArgs a;
   std::memset(&a, 0, sizeof(a));
@@ -637,10 +679,19 @@ extern "C" int ks_rewards(ks_stream_t stream, const KsRewardIO* io) {
   if (!io->done) return fail(KS_EINVAL, "ks_rewards: done is required");
   for (int j = 0; j < io->n_rewards; ++j) {
     const int k = io->rewards[j].kind;
-    if (k < KS_REW_STAY_ALIVE || k > KS_REW_STATEFUL) return fail(KS_EINVAL, "ks_rewards: term %d: bad kind", j);
+    if (k < KS_REW_STAY_ALIVE || k > KS_REW_FORCE) return fail(KS_EINVAL, "ks_rewards: term %d: bad kind", j);
+    const KsRewardDesc& rd = io->rewards[j];
+    if (k == KS_REW_LINVEL_CMD || k == KS_REW_ANGVEL_CMD) {
+      const int span = k == KS_REW_LINVEL_CMD ? 4 : 1;
+      if (!io->command || rd.index < 0 || rd.index + span > io->command_dim) return fail(KS_EINVAL, "ks_rewards: term %d reads command[%d..%d) of %d entries", j, rd.index, rd.index + span, io->command_dim);
+      if (rd.norm < 0 || rd.norm >= (k == KS_REW_LINVEL_CMD ? 4 : 2) || !(rd.p0 > 0.f)) return fail(KS_EINVAL, "ks_rewards: term %d: bad component or length scale", j);
+    }
+    if (k == KS_REW_OFF_AXIS && (rd.norm < 0 || rd.norm > 2 || !(rd.p0 > 0.f))) return fail(KS_EINVAL, "ks_rewards: term %d: bad component or length scale", j);
+    if (k == KS_REW_FORCE && (!io->obs || rd.norm < 1 || rd.index < 0 || rd.index + 3 * rd.norm > io->obs_dim || !(rd.p0 > 0.f)))
+      return fail(KS_EINVAL, "ks_rewards: term %d: force block outside the observation or zero expected weight", j);
     if (k == KS_REW_STATEFUL && (!io->stateful || io->rewards[j].norm < 0)) return fail(KS_EINVAL, "ks_rewards: term %d needs the scanned values", j);
-    const bool needs_q = k == KS_REW_BASE_HEIGHT || k == KS_REW_BASE_HEIGHT_RANGE || k == KS_REW_UPRIGHT_POSE;
-    const bool needs_v = k == KS_REW_UPRIGHT_ANGVEL || k == KS_REW_UPRIGHT_LINVEL;
+    const bool needs_q = k == KS_REW_BASE_HEIGHT || k == KS_REW_BASE_HEIGHT_RANGE || k == KS_REW_UPRIGHT_POSE || k == KS_REW_LINVEL_CMD;
+    const bool needs_v = k == KS_REW_UPRIGHT_ANGVEL || k == KS_REW_UPRIGHT_LINVEL || (k >= KS_REW_LINVEL_CMD && k <= KS_REW_MOTIONLESS);
     const bool needs_a = k >= KS_REW_ACTION_VEL && k <= KS_REW_ACTION_JERK;
     if (needs_q && (!io->qpos || io->nq < 7)) return fail(KS_EINVAL, "ks_rewards: term %d needs qpos of a floating base", j);
     if (needs_v && (!io->qvel || io->nv < 6)) return fail(KS_EINVAL, "ks_rewards: term %d needs qvel of a floating base", j);

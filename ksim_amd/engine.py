@@ -161,7 +161,7 @@ class HipEngine(PhysicsEngine):
         z = lambda *s: torch.zeros(*s, dtype=torch.float32, device=dev)  # noqa: E731
         data = PhysicsData(qpos=z(N, m.nq), qvel=z(N, m.nv), qacc=z(N, m.nv), qacc_warmstart=z(N, m.nv),
                            ctrl=z(N, m.nu), time=z(N), xpos=z(N, m.nb * 3), xquat=z(N, m.nb * 4), cvel=z(N, m.nb * 6),
-                           contact_dist=z(N, m.ns) if m.ns else None, cinert=z(N, m.nb * 10))
+                           contact_dist=z(N, m.ns) if m.ns else None, cinert=z(N, m.nb * 10), cfrc_ext=z(N, m.nb * 6))
         level = float(curriculum_level)
         lo, hi = self.data.min_action_latency_step * level, self.data.max_action_latency_step * level
         state = PhysicsState(
@@ -217,7 +217,7 @@ class HipEngine(PhysicsEngine):
         physics.forward(physics_model, dict(qpos=d.qpos, qvel=d.qvel, qacc_warmstart=d.qacc_warmstart, env_mask=mask,
                                             friction=rnd.get("friction"), mass_scale=rnd.get("mass_scale"),
                                             xpos=d.xpos, xquat=d.xquat, cvel=d.cvel, contact_dist=d.contact_dist,
-                                            cinert=d.cinert))
+                                            cinert=d.cinert, cfrc_ext=d.cfrc_ext))
         # engine.py:217-220: qvel and qacc are zeroed after the forward pass (qvel is already zero here)
 
     def prepare(self, device):
@@ -238,6 +238,7 @@ class HipEngine(PhysicsEngine):
              curriculum_level, rng, randomization: Mapping[str, torch.Tensor] | None = None,
              noise: Mapping[str, torch.Tensor] | None = None,
              record: Mapping[str, torch.Tensor] | None = None, want_cvel: bool = True, want_cinert: bool = False,
+             want_cfrc_ext: bool = False,
              step: int = 0, step_base=None, event_seed: int = 0) -> PhysicsState:
         m, d, s = physics_model.model, physics_state.data, physics_state
         rnd, noise, record = randomization or {}, noise or {}, record or {}
@@ -250,7 +251,7 @@ class HipEngine(PhysicsEngine):
                    action=action, latency=s.action_latency, zero_offset=s.zero_offset, drop=drop,
                    friction=rnd.get("friction"), mass_scale=rnd.get("mass_scale"), qacc=d.qacc, ctrl_out=d.ctrl,
                    xpos=d.xpos, xquat=d.xquat, cvel=d.cvel if want_cvel else None, contact_dist=d.contact_dist,
-                   cinert=d.cinert if want_cinert else None,
+                   cinert=d.cinert if want_cinert else None, cfrc_ext=d.cfrc_ext if want_cfrc_ext else None,
                    action_noise=noise.get("action_noise"),
                    torque_noise=noise.get("torque_noise"), traj_ctrl=record.get("ctrl"),
                    traj_xpos=record.get("xpos"), traj_xquat=record.get("xquat"))

@@ -105,7 +105,7 @@ class EnvTerms:
         m = self.model
         dims = {T.SRC_QPOS: m.nq, T.SRC_QVEL: m.nv, T.SRC_QACC: m.nv, T.SRC_CTRL: m.nu, T.SRC_LAST_ACTION: m.nu,
                 T.SRC_COMMAND: self.command_dim, T.SRC_TIME: 1, T.SRC_XPOS: m.nb * 3, T.SRC_XQUAT: m.nb * 4,
-                T.SRC_CVEL: m.nb * 6, T.SRC_CONTACT_DIST: m.ns, T.SRC_CINERT: m.nb * 10}
+                T.SRC_CVEL: m.nb * 6, T.SRC_CONTACT_DIST: m.ns, T.SRC_CINERT: m.nb * 10, T.SRC_CFRC_EXT: m.nb * 6}
         io = T.KsObserveIO()
         io.N, io.level = N, level
         for s, t in sources.items():

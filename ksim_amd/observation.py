@@ -145,6 +145,28 @@ class BodyVelocityObservation(Observation):  # observation.py:544-560 (cvel of c
 
 
 @dataclass(frozen=True)
+class FeetForceObservation(Observation):
+    """cfrc_ext[foot][:3] of the left and right foot, stacked (2, 3) (observation.py:563-588).  MuJoCo orders cfrc_ext
+    torque first, so these three numbers are the contact torque about the tree's centre of mass; the reference's class
+    name notwithstanding, the slice is kept as it is there."""
+    foot_left: int = 0
+    foot_right: int = 0
+
+    def elements(self, m, command_dim):
+        return _copy(T.SRC_CFRC_EXT, 6 * self.foot_left, 3) + _copy(T.SRC_CFRC_EXT, 6 * self.foot_right, 3)
+
+
+@dataclass(frozen=True)
+class FeetTorqueObservation(Observation):
+    """cfrc_ext[foot][3:] of both feet, (2, 3) (observation.py:591-616): the linear contact force, see FeetForceObservation."""
+    foot_left: int = 0
+    foot_right: int = 0
+
+    def elements(self, m, command_dim):
+        return _copy(T.SRC_CFRC_EXT, 6 * self.foot_left + 3, 3) + _copy(T.SRC_CFRC_EXT, 6 * self.foot_right + 3, 3)
+
+
+@dataclass(frozen=True)
 class ActPosObservation(Observation):  # observation.py:717-750: (last action, joint position) of one joint, for debugging
     ctrl_idx: int = 0
     qpos_idx: int = 7

@@ -29,8 +29,12 @@ def _reward_scale(rew, level: float) -> float:
 class Reward:
     scale: object = 1.0  # a float or a curriculum scale (ksim/scales.py)
 
-    def descs(self) -> list[tuple]:  # [(suffix | None, kind, norm, p0, p1, p2)]  # pragma: no cover
+    def descs(self) -> list[tuple]:  # [(suffix | None, kind, norm, p0, p1, p2[, p3, index])]  # pragma: no cover
         raise NotImplementedError
+
+    def descs_in(self, obs_slices: Mapping[str, slice], command_slices: Mapping[str, slice]) -> list[tuple]:
+        """Descriptors for rewards that read a named command or observation; the others ignore the maps."""
+        return self.descs()
 
     @property
     def is_penalty(self) -> bool:  # rewards.py:117-124
@@ -128,6 +132,89 @@ class AMPReward(Reward):  # ksim/task/amp.py:99-112
 
     def descs(self):
         return [(None, T.REW_AMP, 0, 0.0, 0.0, 0.0)]
+
+
+def _named(slices, name, what):
+    if name not in slices:
+        raise KeyError(f"{what} {name!r} is not among {sorted(slices)}")
+    return slices[name]
+
+
+@dataclass(frozen=True)
+class LinearVelocityReward(Reward):
+    """Tracks a planar velocity command in the robot frame (rewards.py:236-275): components vel, yaw, x, y.  The command is
+    the LinearVelocityCommandValue laid out as (vel, yaw, xvel, yvel, ...) at `command_slices[cmd]`."""
+    cmd: str = ""
+    vel_length_scale: float = 0.25
+    yaw_length_scale: float = 0.25
+    zero_threshold: float = 0.01
+    sq_scale: float = 0.1
+    abs_scale: float = 0.1
+
+    def __post_init__(self):
+        if not (self.sq_scale > 0.0 and self.abs_scale > 0.0):
+            raise ValueError("sq_scale and abs_scale must be positive")
+
+    def descs_in(self, obs_slices, command_slices):
+        sl = _named(command_slices, self.cmd, "command")
+        if sl.stop - sl.start < 4:
+            raise ValueError("a linear velocity command has at least (vel, yaw, xvel, yvel)")
+        return [(name, T.REW_LINVEL_CMD, k, self.yaw_length_scale if k == 1 else self.vel_length_scale, self.sq_scale,
+                 self.abs_scale, self.zero_threshold, sl.start) for k, name in enumerate(("vel", "yaw", "x", "y"))]
+
+
+@dataclass(frozen=True)
+class AngularVelocityReward(Reward):
+    """Tracks a yaw-rate command (rewards.py:321-350): components mag and dir."""
+    cmd: str = ""
+    angvel_length_scale: float = 0.25
+    sq_scale: float = 0.1
+    abs_scale: float = 0.1
+    zero_threshold: float = math.radians(5.0)
+
+    def __post_init__(self):
+        if not (self.sq_scale > 0.0 and self.abs_scale > 0.0):
+            raise ValueError("sq_scale and abs_scale must be positive")
+
+    def descs_in(self, obs_slices, command_slices):
+        sl = _named(command_slices, self.cmd, "command")
+        return [(name, T.REW_ANGVEL_CMD, k, self.angvel_length_scale, self.sq_scale, self.abs_scale, self.zero_threshold, sl.start)
+                for k, name in enumerate(("mag", "dir"))]
+
+
+@dataclass(frozen=True)
+class OffAxisVelocityReward(Reward):  # rewards.py:353-372: components linz, angx, angy (qvel[2], qvel[4], qvel[5])
+    lin_length_scale: float = 0.25
+    ang_length_scale: float = 0.25
+
+    def descs(self):
+        return [("linz", T.REW_OFF_AXIS, 0, self.lin_length_scale, 0.0, 0.0), ("angx", T.REW_OFF_AXIS, 1, self.ang_length_scale, 0.0, 0.0),
+                ("angy", T.REW_OFF_AXIS, 2, self.ang_length_scale, 0.0, 0.0)]
+
+
+@dataclass(frozen=True)
+class MotionlessAtRestPenalty(Reward):  # rewards.py:1206-1221: joint speed while the base is not moving
+    linvel_moving_threshold: float = 0.5
+    angvel_moving_threshold: float = math.radians(30)
+
+    def descs(self):
+        return [(None, T.REW_MOTIONLESS, 0, self.linvel_moving_threshold, self.angvel_moving_threshold, 0.0)]
+
+
+@dataclass(frozen=True)
+class ForcePenalty(Reward):
+    """Squared contact force over the expected weight, worst body (rewards.py:1224-1240); `force_obs` names an (n, 3)
+    observation such as FeetForceObservation."""
+    force_obs: str = ""
+    ctrl_dt: float = 0.02
+    expected_weight: float = 1.0
+    bias: float = 0.0
+
+    def descs_in(self, obs_slices, command_slices):
+        sl = _named(obs_slices, self.force_obs, "observation")
+        if (sl.stop - sl.start) % 3:
+            raise ValueError("the force observation must be (n, 3)")
+        return [(None, T.REW_FORCE, (sl.stop - sl.start) // 3, self.expected_weight, self.bias, 0.0, 0.0, sl.start)]
 
 
 @dataclass(frozen=True)
@@ -306,12 +393,14 @@ def get_rewards(trajectory: Trajectory, rewards: Mapping[str, Reward], clip_min:
                 d.kind, d.norm, d.scale = T.REW_STATEFUL, first_slot[name] + k, sign * _reward_scale(rew, level)
                 names.append(name if suffix is None else f"{name}/{suffix}")
             continue
-        for suffix, kind, norm, p0, p1, p2 in rew.descs():
+        for suffix, kind, norm, p0, p1, p2, *more in rew.descs_in(obs_slices or {}, command_slices or {}):
             j = len(names)
             if j >= T.KS_MAX_REWARD_TERMS:
                 raise _lib.KsError("too many reward terms")
             d = io.rewards[j]
             d.kind, d.norm, d.scale, d.p0, d.p1, d.p2 = kind, norm, sign * _reward_scale(rew, level), p0, p1, p2
+            if more:
+                d.p3, d.index = float(more[0]), int(more[1])
             names.append(name if suffix is None else f"{name}/{suffix}")  # rl.py:223-226
     io.n_rewards = len(names)
     if not names:
@@ -339,6 +428,17 @@ def get_rewards(trajectory: Trajectory, rewards: Mapping[str, Reward], clip_min:
             raise ValueError("AMPReward auxiliary output is missing! Make sure you are using it within the context of "
                              "an AMP task, which populates the auxiliary output for you.")
         logits = tensor(trajectory.aux_outputs[DISCRIMINATOR_OUTPUT_KEY], torch.float32, None)
+    kinds = {io.rewards[j].kind for j in range(len(names))}
+    if kinds & {T.REW_LINVEL_CMD, T.REW_ANGVEL_CMD}:
+        cmd = trajectory.command.get("_buffer") if trajectory.command else None
+        if cmd is None:
+            raise KeyError('command-tracking rewards read trajectory.command["_buffer"] (T, N, command_dim)')
+        cmd = tensor(cmd, torch.float32, cmd.shape[-1])
+        io.command, io.command_dim = cmd.data_ptr(), cmd.shape[-1]
+    if T.REW_FORCE in kinds:
+        ob_ = trajectory.obs[obs_key]
+        ob_ = tensor(ob_, torch.float32, ob_.shape[-1])
+        io.obs, io.obs_dim = ob_.data_ptr(), ob_.shape[-1]
     io.nq = 0 if qpos is None else qpos.shape[-1]
     io.nv = 0 if qvel is None else qvel.shape[-1]
     io.nu = 0 if action is None else action.shape[-1]

@@ -91,7 +91,8 @@ class Rollout:
         step, step_base = (t, self.step_base) if _relative_step else (env.step, None)
         src = {T.SRC_QPOS: d.qpos, T.SRC_QVEL: d.qvel, T.SRC_QACC: d.qacc, T.SRC_CTRL: d.ctrl,
                T.SRC_LAST_ACTION: ps.last_ctrl, T.SRC_COMMAND: env.commands, T.SRC_TIME: d.time, T.SRC_XPOS: d.xpos,
-               T.SRC_XQUAT: d.xquat, T.SRC_CVEL: d.cvel, T.SRC_CONTACT_DIST: d.contact_dist, T.SRC_CINERT: d.cinert}
+               T.SRC_XQUAT: d.xquat, T.SRC_CVEL: d.cvel, T.SRC_CONTACT_DIST: d.contact_dist, T.SRC_CINERT: d.cinert,
+               T.SRC_CFRC_EXT: d.cfrc_ext}
         self._prepare_env(env)
         # the reset mask still holds the envs that the previous control step reset: their carries start afresh
         c.terms.observe(src, self.N, level=level, zero_offset=ps.zero_offset, bias=env.obs_bias,
@@ -114,7 +115,8 @@ class Rollout:
         # the step kernel also writes ctrl / xpos / xquat of the post-step data into the transition slot
         c.engine.step(self.action[t], c.physics_model, ps, level, env.seed + env.step, env.randomization_dict,
                       noise=noise.get("engine"), record=dict(ctrl=self.ctrl[t], xpos=self.xpos[t], xquat=self.xquat[t]),
-                      want_cvel=T.SRC_CVEL in c.terms.sources_used, want_cinert=T.SRC_CINERT in c.terms.sources_used, step=step, step_base=step_base, event_seed=env.seed)
+                      want_cvel=T.SRC_CVEL in c.terms.sources_used, want_cinert=T.SRC_CINERT in c.terms.sources_used,
+                      want_cfrc_ext=T.SRC_CFRC_EXT in c.terms.sources_used, step=step, step_base=step_base, event_seed=env.seed)
         ev_buf = ps.event_states.get("_buffer") if ps.event_states else None
         st = dict(qpos=d.qpos, qvel=d.qvel, qacc_warmstart=d.qacc_warmstart, time=d.time, last_ctrl=ps.last_ctrl)
         c.terms.terminate_reset(st, level=level, components=self.components[t][: c.terms.n_terms] if c.terms.n_terms else None,

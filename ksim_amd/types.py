@@ -25,6 +25,7 @@ class PhysicsData:
     cvel: torch.Tensor            # (N, nb*6)
     contact_dist: torch.Tensor | None = None  # (N, ns) sphere-floor distance of the last collision pass (contact.dist)
     cinert: torch.Tensor | None = None        # (N, nb*10) com-based body inertias (mjData.cinert)
+    cfrc_ext: torch.Tensor | None = None      # (N, nb*6) contact force on each body, torque then force (mjData.cfrc_ext)
 
 
 @dataclass

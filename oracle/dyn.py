@@ -62,7 +62,7 @@ def _data_struct(real):
             ("con_dist", real * MAXS), ("con_pos", real * 3 * MAXS),
             ("efc_J", real * (MAXR * MAXV)), ("efc_pos", real * MAXR), ("efc_aref", real * MAXR),
             ("efc_D", real * MAXR), ("efc_force", real * MAXR),
-            ("qfrc_constraint", real * MAXV), ("qacc", real * MAXV),
+            ("qfrc_constraint", real * MAXV), ("qacc", real * MAXV), ("cfrc_ext", real * 6 * MAXB),
         ]
 
     return KsorData
@@ -117,7 +117,7 @@ class DataView:
             return v
         arr = np.ctypeslib.as_array(v)
         nb, nq, nv, nu, ns = a["nb"], a["nq"], a["nv"], a["nu"], a["ns"]
-        trim = {"qpos": nq, "qvel": nv, "ctrl": nu, "qacc_warmstart": nv, "mass_scale": nb, "xfrc_applied": nb, "xpos": nb, "xquat": nb,
+        trim = {"qpos": nq, "qvel": nv, "ctrl": nu, "qacc_warmstart": nv, "mass_scale": nb, "xfrc_applied": nb, "cfrc_ext": nb, "xpos": nb, "xquat": nb,
                 "xmat": nb, "xipos": nb, "ximat": nb, "xanchor": nb, "xaxis": nb, "cinert": nb, "crb": nb, "cdof": nv,
                 "cvel": nb, "cdof_dot": nv, "qfrc_bias": nv, "qfrc_passive": nv, "qfrc_actuator": nv,
                 "actuator_force": nu, "qfrc_smooth": nv, "qacc_smooth": nv, "con_dist": ns, "con_pos": ns,

@@ -44,6 +44,9 @@ typedef struct FN(KsorData) {
   REAL efc_J[KSOR_MAXR * KSOR_MAXV], efc_pos[KSOR_MAXR], efc_aref[KSOR_MAXR], efc_D[KSOR_MAXR],
       efc_force[KSOR_MAXR];
   REAL qfrc_constraint[KSOR_MAXV], qacc[KSOR_MAXV];
+  /* contact forces on each body as a spatial force about the tree's centre of mass, world axes, torque then force
+   * (MuJoCo's cfrc_ext, which FeetForceObservation / FeetTorqueObservation read, ksim/observation.py:563-616) */
+  REAL cfrc_ext[KSOR_MAXB][6];
 } FN(KsorData);
 typedef FN(KsorData) Data;
 
@@ -633,6 +636,25 @@ void FN(ksor_forward)(const KsorModel* m, Data* d) {
   }
   chol_solve(d->qacc_smooth, d->L, d->qfrc_smooth, nv);
   FN(ksor_solve)(m, d);
+  /* Cartesian contact forces: a pyramid row with force f pushes along normal +- mu tangent, so a contact's force is
+   * the sum of its four edge forces; it acts on the sphere's body at the contact point */
+  memset(d->cfrc_ext, 0, sizeof(d->cfrc_ext));
+  int row = 0;
+  for (int s = 0; s < m->ns; ++s) {
+    if (!(d->con_dist[s] < 0)) continue;
+    REAL F[3] = {0, 0, 0};
+    for (int q = 0; q < 4; ++q) {
+      const REAL f = d->efc_force[row + q], smu = (q & 1) ? -d->friction : d->friction;
+      F[2] += f;
+      if (q < 2) F[1] += smu * f; else F[0] -= smu * f;
+    }
+    row += 4;
+    REAL off[3], tq[3];
+    for (int k = 0; k < 3; ++k) off[k] = d->con_pos[s][k] - d->com[k];
+    cross3(tq, off, F);
+    const int b = m->sph_body[s];
+    for (int k = 0; k < 3; ++k) { d->cfrc_ext[b][k] += tq[k]; d->cfrc_ext[b][3 + k] += F[k]; }
+  }
 }
 
 void FN(ksor_euler)(const KsorModel* m, Data* d) {

@@ -333,3 +333,44 @@ def sparse_target_height_reward(contact_tcn, position_tn3, qvel_t, done_t, carry
         best = np.where(still[t] | contact_tn[t], 0.0, best)
         out[t] = rew.max()
     return out, best
+
+
+# ------------------------------------------------------------------ command tracking and rest / force penalties
+def linear_velocity_reward(qpos_tq, qvel_tv, cmd_t4, vel_length_scale=0.25, yaw_length_scale=0.25, zero_threshold=0.01,
+                           sq_scale=0.1, abs_scale=0.1):
+    """LinearVelocityReward (ksim/rewards.py:248-272); cmd columns = (vel, yaw, xvel, yvel)."""
+    lin = rotate_vector_by_quat(qvel_tv[..., :3], qpos_tq[..., 3:7], inverse=True)
+    x, y = lin[..., 0], lin[..., 1]
+    vel, yaw = np.hypot(x, y), np.arctan2(y, x)
+    zero = np.abs(cmd_t4[..., 0]) < zero_threshold
+    k = lambda d, s: exp_kernel_with_penalty(d, s, sq_scale, abs_scale)  # noqa: E731
+    return {"vel": k(vel - cmd_t4[..., 0], vel_length_scale),
+            "yaw": np.where(zero, 0.0, k(yaw - cmd_t4[..., 1], yaw_length_scale)),
+            "x": np.where(zero, 0.0, k(x - cmd_t4[..., 2], vel_length_scale)),
+            "y": np.where(zero, 0.0, k(y - cmd_t4[..., 3], vel_length_scale))}
+
+
+def angular_velocity_reward(qvel_tv, cmd_t, angvel_length_scale=0.25, sq_scale=0.1, abs_scale=0.1,
+                            zero_threshold=np.radians(5.0)):
+    """AngularVelocityReward (rewards.py:332-347)."""
+    w = qvel_tv[..., 5]
+    real = np.where(np.abs(w) < zero_threshold, 0.0, np.sign(w))
+    want = np.where(np.abs(cmd_t) < zero_threshold, 0.0, np.sign(cmd_t))
+    return {"mag": exp_kernel_with_penalty(w - cmd_t, angvel_length_scale, sq_scale, abs_scale),
+            "dir": np.where(real == want, 1.0, -1.0)}
+
+
+def off_axis_velocity_reward(qvel_tv, lin_length_scale=0.25, ang_length_scale=0.25):  # rewards.py:360-372
+    g = lambda v, s: np.exp(-np.square(v) / (2 * s**2))  # noqa: E731
+    return {"linz": g(qvel_tv[..., 2], lin_length_scale), "angx": g(qvel_tv[..., 4], ang_length_scale),
+            "angy": g(qvel_tv[..., 5], ang_length_scale)}
+
+
+def motionless_at_rest_penalty(qvel_tv, linvel_moving_threshold=0.5, angvel_moving_threshold=np.radians(30)):  # rewards.py:1213-1221
+    still = (np.linalg.norm(qvel_tv[..., :2], axis=-1) < linvel_moving_threshold) & (qvel_tv[..., 5] < angvel_moving_threshold)
+    return np.where(still, np.linalg.norm(qvel_tv[..., 6:], axis=-1), 0.0)
+
+
+def force_penalty(force_tn3, expected_weight, bias=0.0):  # rewards.py:1237-1240
+    obs = np.clip(np.linalg.norm(force_tn3, axis=-1) - bias, 0.0, None)
+    return np.square(obs / expected_weight).max(axis=-1)

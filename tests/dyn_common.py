@@ -33,7 +33,7 @@ def oracle_forward(m, qpos, qvel, ctrl=None, friction=None, mass_scale=None, war
     orc = Oracle(m.arrays(), dtype)
     N = qpos.shape[0]
     keys = ("qpos", "qvel", "qacc", "qacc_smooth", "qfrc_bias", "M", "con_dist", "xpos", "xquat", "cvel",
-            "qacc_warmstart", "cinert")
+            "qacc_warmstart", "cinert", "cfrc_ext")
     out = {k: [] for k in keys}
     out["nefc"], out["niter"] = [], []
     for e in range(N):

@@ -489,3 +489,53 @@ def test_body_velocity_inertia_and_debug_observations():
     np.testing.assert_allclose(obs.cpu().numpy(), want.astype(np.float32), rtol=0, atol=0)
     with pytest.raises(ValueError):
         ob.FeetOrientationObservation(body_ids=(1, 2, 3))
+
+
+def test_command_tracking_rest_and_force_rewards():
+    """The rewards of the shipped walking tasks that read commands and contact forces, against the oracle."""
+    from ksim_amd import rewards as rw
+    from ksim_amd.types import Trajectory
+
+    Tn, N, nq, nv = 16, 29, 27, 26
+    rng = np.random.default_rng(31)
+    qpos = rng.normal(size=(Tn, N, nq)); qpos[..., 3:7] /= np.linalg.norm(qpos[..., 3:7], axis=-1, keepdims=True)
+    qvel = rng.normal(size=(Tn, N, nv)) * 0.5
+    cmd = rng.normal(size=(Tn, N, 8)) * 0.5
+    cmd[::3, :, 1] = 0.003            # some zero linear commands
+    cmd[1::4, :, 7] = 0.01            # some yaw commands inside the dead band
+    obs = rng.normal(size=(Tn, N, 12)) * 30
+    done = rng.random((Tn, N)) < 0.05
+    rewards = {"lin": rw.LinearVelocityReward(scale=1.5, cmd="lin_cmd", vel_length_scale=0.3, yaw_length_scale=0.5),
+               "ang": rw.AngularVelocityReward(scale=0.7, cmd="ang_cmd"),
+               "off": rw.OffAxisVelocityReward(scale=0.2, ang_length_scale=0.4),
+               "rest": rw.MotionlessAtRestPenalty(scale=0.1),
+               "force": rw.ForcePenalty(scale=0.05, force_obs="feet_force", expected_weight=40.0, bias=5.0),
+               "alive": rw.StayAliveReward(scale=1.0)}
+    traj = Trajectory(qpos=t32(qpos), qvel=t32(qvel), xpos=None, xquat=None, ctrl=None, obs={"obs": t32(obs)},
+                      command={"_buffer": t32(cmd)}, event_state={}, action=None, done=torch.from_numpy(done).to(DEV), success=None,
+                      timestep=None)
+    st = rw.get_rewards(traj, rewards, obs_slices={"x": slice(0, 4), "feet_force": slice(4, 10)},
+                        command_slices={"lin_cmd": slice(1, 7), "ang_cmd": slice(7, 8)})
+    f32 = lambda a: a.astype(np.float32).astype(np.float64)  # noqa: E731
+    q, v, c, o = f32(qpos), f32(qvel), f32(cmd), f32(obs)
+    lin = ot.linear_velocity_reward(q, v, c[..., 1:5], vel_length_scale=0.3, yaw_length_scale=0.5)
+    ang = ot.angular_velocity_reward(v, c[..., 7])
+    off = ot.off_axis_velocity_reward(v, ang_length_scale=0.4)
+    want = {**{f"lin/{k}": 1.5 * x for k, x in lin.items()}, **{f"ang/{k}": 0.7 * x for k, x in ang.items()},
+            **{f"off/{k}": 0.2 * x for k, x in off.items()}, "rest": -0.1 * ot.motionless_at_rest_penalty(v),
+            "force": -0.05 * ot.force_penalty(o[..., 4:10].reshape(Tn, N, 2, 3), 40.0, 5.0)}
+    assert list(st.components)[:-1] == list(want)
+    for k, w in want.items():
+        got = st.components[k].cpu().numpy()
+        if k == "lin/yaw":  # atan2 near the branch cut +-pi can land on the other side in fp32
+            close = np.abs(got - w) < 2e-4
+            assert close.mean() > 0.995
+        else:
+            np.testing.assert_allclose(got, w, rtol=2e-5, atol=2e-5, err_msg=k)
+    assert (st.components["lin/x"][::3] == 0).all() and (st.components["ang/dir"].abs() == 0.7).all()
+    total = sum(st.components[k] for k in st.components)
+    np.testing.assert_allclose(st.total.cpu().numpy(), total.cpu().numpy(), rtol=1e-5, atol=1e-5)
+    with pytest.raises(KeyError, match="nope"):
+        rw.get_rewards(traj, {"lin": rw.LinearVelocityReward(cmd="nope")}, command_slices={"lin_cmd": slice(0, 4)})
+    with pytest.raises(Exception, match="command"):
+        rw.get_rewards(traj, {"ang": rw.AngularVelocityReward(cmd="a")}, command_slices={"a": slice(8, 9)})

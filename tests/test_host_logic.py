@@ -203,3 +203,12 @@ def test_stateful_terms_compile_to_carry_layouts():
         rw.FeetAirTimeReward(contact_obs="contact", linvel_cmd="v").scan_desc(slices, {}, 1.0)
     with pytest.raises(ValueError):
         rw.SparseTargetHeightReward(contact_obs="contact", position_obs="jp", num_bodies=2).scan_desc(slices, {}, 1.0)
+
+
+def test_feet_force_observations_read_the_contact_force_rows():
+    m = km.kbot_scale_model()
+    d, slices, used, _, _ = compile_terms(m, {"f": ob.FeetForceObservation(foot_left=11, foot_right=6),
+                                              "t": ob.FeetTorqueObservation(foot_left=11, foot_right=6)}, {}, [])
+    idx = [d.obs[k].index for k in range(d.obs_dim)]
+    assert idx == [66, 67, 68, 36, 37, 38, 69, 70, 71, 39, 40, 41] and used == {T.SRC_CFRC_EXT}
+    assert all(d.obs[k].kind == T.OBS_COPY and d.obs[k].src == T.SRC_CFRC_EXT for k in range(d.obs_dim))

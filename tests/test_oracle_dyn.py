@@ -380,3 +380,43 @@ def test_com_based_inertia_closed_form(model):
         I = R @ np.diag(np.asarray(a["body_inertia"])[b]) @ R.T + mass[b] * (off @ off * np.eye(3) - np.outer(off, off))
         want = [I[0, 0], I[1, 1], I[2, 2], I[0, 1], I[0, 2], I[1, 2], *(mass[b] * off), mass[b]]
         np.testing.assert_allclose(got[b], want, rtol=1e-10, atol=1e-12)
+
+
+def test_contact_forces_on_bodies(model):
+    """cfrc_ext: projected on the motion axes of every ancestor dof the body forces reproduce the generalised constraint
+    force J^T f exactly; a ball at rest is carried by its weight."""
+    if model.ns == 0:
+        pytest.skip("no contacts in this model")
+    rng = np.random.default_rng(23)
+    orc = Oracle(model.arrays())
+    hits = 0
+    for _ in range(4):
+        qpos, qvel = _random_state(model, rng, vel_scale=0.3)
+        qpos = _sink_to_contact(model, qpos, depth=0.02)
+        d = orc.data(qpos, qvel, friction=0.8)
+        orc.forward(d)
+        if d.nefc == 0:
+            continue
+        hits += 1
+        cf, cdof = np.array(d.cfrc_ext), np.array(d.cdof)
+        assert np.abs(cf).max() > 0 and not cf[0].any()
+        want = np.zeros(model.nv)
+        for j in range(model.nv):
+            for b in range(1, model.nb):
+                anc = b
+                while anc > 0 and anc != model.dof_body[j]:
+                    anc = model.body_parent[anc]
+                if anc == model.dof_body[j]:
+                    want[j] += cdof[j] @ cf[b]
+        np.testing.assert_allclose(want, d.qfrc_constraint, rtol=1e-9, atol=1e-9)
+        assert (cf[:, 5] >= 0).all()  # the floor only pushes
+    assert hits >= 2
+    ball = _ball()
+    ob_ = Oracle(ball.arrays())
+    db = ob_.data()
+    db.qpos[2] = 0.0995
+    for _ in range(400):
+        ob_.step(db)
+    ob_.forward(db)
+    np.testing.assert_allclose(np.array(db.cfrc_ext)[1, 3:], [0, 0, 2.0 * 9.81], atol=2e-3)
+    np.testing.assert_allclose(np.array(db.cfrc_ext)[1, :3], 0, atol=1e-9)  # the contact point lies under the centre

@@ -224,3 +224,32 @@ def test_sparse_target_height_reward_hand_computed():
     qvel[3, 0] = 0.0
     out, _ = terms.sparse_target_height_reward(contact, pos, qvel, np.zeros(6, bool), np.array([0.0]), height=0.25)
     np.testing.assert_allclose(out, [0, 0, 0, 0, 0.0, 0])
+
+
+def test_command_tracking_and_rest_rewards_hand_computed():
+    k = lambda d, s=0.25, sq=0.1, ab=0.1: -ab * abs(d) - sq * d * d + np.exp(-d * d / (2 * s * s))  # noqa: E731
+    # base yawed by 90 degrees: a world velocity of (0, 2, 0) is 2 m/s straight ahead in the robot frame
+    q = np.zeros((1, 7)); q[0, 3:7] = [np.cos(np.pi / 4), 0, 0, np.sin(np.pi / 4)]
+    v = np.zeros((1, 8)); v[0, :3] = [0.0, 2.0, 0.0]
+    out = terms.linear_velocity_reward(q, v, np.array([[1.5, 0.1, 1.5, 0.0]]))
+    assert out["vel"][0] == pytest.approx(k(0.5)) and out["x"][0] == pytest.approx(k(0.5))
+    assert out["yaw"][0] == pytest.approx(k(-0.1)) and out["y"][0] == pytest.approx(k(0.0), abs=1e-12)
+    out = terms.linear_velocity_reward(q, v, np.array([[0.005, 0.1, 1.5, 0.0]]))  # a zero command mutes all but "vel"
+    assert (out["yaw"][0], out["x"][0], out["y"][0]) == (0.0, 0.0, 0.0) and out["vel"][0] == pytest.approx(k(1.995))
+    v[0, 5] = 0.3
+    a = terms.angular_velocity_reward(v, np.array([0.5]))
+    assert a["mag"][0] == pytest.approx(k(-0.2)) and a["dir"][0] == 1.0
+    assert terms.angular_velocity_reward(v, np.array([-0.5]))["dir"][0] == -1.0
+    assert terms.angular_velocity_reward(v, np.array([0.01]))["dir"][0] == -1.0   # command inside the dead band, robot turning
+    v[0, 5] = 0.01
+    assert terms.angular_velocity_reward(v, np.array([0.02]))["dir"][0] == 1.0    # both inside the dead band
+    v[0, 2], v[0, 4], v[0, 5] = 0.25, 0.5, 0.0
+    o = terms.off_axis_velocity_reward(v)
+    assert o["linz"][0] == pytest.approx(np.exp(-0.5)) and o["angx"][0] == pytest.approx(np.exp(-2.0)) and o["angy"][0] == 1.0
+    v[0, :3] = [0.3, 0.0, 0.0]; v[0, 6:] = [3.0, 4.0]
+    assert terms.motionless_at_rest_penalty(v)[0] == 5.0
+    v[0, 0] = 0.6
+    assert terms.motionless_at_rest_penalty(v)[0] == 0.0
+    f = np.array([[[3.0, 4.0, 0.0], [0.0, 0.0, 12.0]]])
+    assert terms.force_penalty(f, expected_weight=5.0, bias=2.0)[0] == pytest.approx(4.0)   # ((12 - 2) / 5)^2
+    assert terms.force_penalty(f * 0.1, expected_weight=5.0, bias=2.0)[0] == 0.0
