@@ -33,7 +33,7 @@ const char* ks_last_error(void);
 /* sizeof() of a public struct as this library was compiled, for binding self-checks:
  * 0 KsPpoLossParams, 1 KsModelDesc, 2 KsStepIO, 3 KsTermsDesc, 4 KsObserveIO, 5 KsTerminateIO, 6 KsMlpDesc,
  * 7 KsRewardIO, 8 KsObsElem, 9 KsTermDesc, 10 KsRewardDesc, 11 KsRng, 12 KsAdamParams, 13 KsEventDesc,
- * 14 KsRewardScanIO, 15 KsRewardScanDesc, 16 KsGruDesc, 17 KsLstmDesc, 18 KsGaussianHead;
+ * 14 KsRewardScanIO, 15 KsRewardScanDesc, 16 KsGruDesc, 17 KsLstmDesc, 18 KsGaussianHead, 19 KsCommandIO;
  * -1 for anything else. */
 int64_t ks_abi_sizeof(int32_t which);
 
@@ -380,6 +380,40 @@ typedef struct KsTerminateIO {
   float* event_force;               /* (n_events, N, KS_EVENT_FORCE_STATE), nullable: zeroed for the reset envs */
 } KsTerminateIO;
 int ks_terminate_reset(const KsTerms* terms, ks_stream_t stream, const KsTerminateIO* io /*host*/);
+
+/* Commands (replaces get_commands / get_initial_commands, ksim/task/rl.py:302-332, called per control step at
+ * rl.py:1082-1098, for the velocity commands of the shipped tasks, ksim/commands.py:281-391,451-507).  The env's command
+ * vector is the concatenation of the commands' values:
+ *   linear velocity : vel, yaw, xvel, yvel, target_vel, target_yaw     angular velocity : vel, target_vel
+ *   constant        : `dim` floats that are left alone
+ * Per step and command, in this order: an env that starts an episode (fresh) draws its initial command from its
+ * (reset) state: targets at random, current values measured (base speed and heading in the robot frame; yaw rate).
+ * Otherwise, with probability switch_prob new targets are drawn and the current values stay; else the current
+ * values move towards the targets by at most accel * ctrl_dt.  Draws u0..: linear = target speed, target yaw, zero,
+ * backward, switch; angular = target speed, flip, zero, switch. */
+#define KS_MAX_COMMANDS 8
+#define KS_COMMAND_DRAWS 8
+enum { KS_CMD_CONST = 0, KS_CMD_LINEAR_VELOCITY = 1, KS_CMD_ANGULAR_VELOCITY = 2 };
+typedef struct KsCommandDesc {
+  int32_t kind, index, dim;    /* offset and length inside the command vector */
+  float min_vel, max_vel, max_yaw, zero_prob, backward_prob, switch_prob; /* scales already evaluated at the curriculum level */
+  float ctrl_dt, linear_accel, angular_accel;
+} KsCommandDesc;
+typedef struct KsCommandIO {
+  int64_t N;
+  int32_t command_dim, n_commands, nq, nv;
+  KsCommandDesc commands[KS_MAX_COMMANDS];
+  float* command;            /* (N, command_dim) in/out */
+  float* traj_command;       /* (N, command_dim) nullable: receives the incoming commands, i.e. the ones the step that is
+                                being recorded was taken under (Trajectory.command, rl.py:1113-1128) */
+  const float* qpos;         /* (N, nq) */
+  const float* qvel;         /* (N, nv) */
+  const uint8_t* fresh;      /* (N) nullable: envs that start an episode */
+  int32_t all_fresh;         /* 1: every env draws an initial command (first step of a task) */
+  const float* uniform;      /* (N, n_commands, KS_COMMAND_DRAWS) U[0,1) draws, nullable -> Philox */
+  KsRng rng;
+} KsCommandIO;
+int ks_commands(ks_stream_t stream, const KsCommandIO* io /*host*/);
 
 /* Action post-processing (replaces the sampling tail of RLTask._sample_action, rl.py:998-1001):
  * action = mean + std * noise, NaN -> 0, clip to +-clip_max.  log_std (nu) nullable = deterministic. */

@@ -117,6 +117,23 @@ class KsGruDesc(ctypes.Structure):
                 ("weight_hh", c_void_p), ("bias", c_void_p), ("bias_n", c_void_p)]
 
 
+KS_MAX_COMMANDS, KS_COMMAND_DRAWS = 8, 8
+CMD_CONST, CMD_LINEAR_VELOCITY, CMD_ANGULAR_VELOCITY = range(3)
+
+
+class KsCommandDesc(ctypes.Structure):
+    _fields_ = [("kind", c_int32), ("index", c_int32), ("dim", c_int32), ("min_vel", c_float), ("max_vel", c_float),
+                ("max_yaw", c_float), ("zero_prob", c_float), ("backward_prob", c_float), ("switch_prob", c_float),
+                ("ctrl_dt", c_float), ("linear_accel", c_float), ("angular_accel", c_float)]
+
+
+class KsCommandIO(ctypes.Structure):
+    _fields_ = [("N", c_int64), ("command_dim", c_int32), ("n_commands", c_int32), ("nq", c_int32), ("nv", c_int32),
+                ("commands", KsCommandDesc * KS_MAX_COMMANDS), ("command", c_void_p), ("traj_command", c_void_p),
+                ("qpos", c_void_p), ("qvel", c_void_p), ("fresh", c_void_p), ("all_fresh", c_int32), ("uniform", c_void_p),
+                ("rng", KsRng)]
+
+
 class KsGaussianHead(ctypes.Structure):
     _fields_ = [("min_std", c_float), ("max_std", c_float), ("var_scale", c_float), ("deterministic", c_int32),
                 ("mean_bias", c_void_p)]
@@ -155,6 +172,8 @@ def bind(lib) -> None:
     lib.ks_terminate_reset.argtypes = [c_void_p, c_void_p, POINTER(KsTerminateIO)]
     lib.ks_sample_action.argtypes = [c_void_p, c_int64, c_int32, c_void_p, c_void_p, c_void_p, KsRng, c_float,
                                      c_void_p]
+    lib.ks_commands.argtypes = [c_void_p, POINTER(KsCommandIO)]
+    lib.ks_commands.restype = c_int32
     lib.ks_sample_action_head.argtypes = [c_void_p, c_int64, c_int32, c_void_p, POINTER(KsGaussianHead), c_void_p, KsRng,
                                           c_float, c_void_p, c_void_p, c_void_p, c_void_p]
     lib.ks_sample_action_head.restype = c_int32

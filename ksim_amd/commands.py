@@ -1,0 +1,140 @@
+"""Commands with the reference's class names (ksim/commands.py), advanced once per control step on the device.
+
+`CommandSet` lays the commands' values out in one `(N, command_dim)` vector per env (`slices[name]` says where) and
+replaces get_initial_commands / get_commands (ksim/task/rl.py:302-332): an env that starts an episode draws an initial
+command from its reset state, the others are updated.  A velocity command's value is the reference's dataclass flattened:
+`LinearVelocityCommandValue` = (vel, yaw, xvel, yvel, target_vel, target_yaw), `AngularVelocityCommandValue` = (vel, target_vel).
+"""
+from __future__ import annotations
+
+import ctypes
+from dataclasses import dataclass
+from typing import Mapping
+
+import torch
+
+from . import _lib
+from . import _lib_terms as T
+from .scales import convert_to_scale
+
+
+@dataclass(frozen=True)
+class Command:
+    def dim(self) -> int:  # pragma: no cover
+        raise NotImplementedError
+
+    def desc(self, level: float) -> T.KsCommandDesc:  # pragma: no cover
+        raise NotImplementedError
+
+
+def _s(scale, level: float) -> float:
+    return float(convert_to_scale(scale).get_scale(level))
+
+
+@dataclass(frozen=True)
+class LinearVelocityCommand(Command):  # commands.py:281-391
+    min_vel: object = 0.0
+    max_vel: object = 0.0
+    ctrl_dt: float = 0.02
+    linear_accel: float = 1.0
+    angular_accel: float = 1.0
+    max_yaw: object = 0.0
+    zero_prob: object = 0.0
+    backward_prob: object = 0.0
+    switch_prob: object = 0.0
+
+    def dim(self):
+        return 6
+
+    def desc(self, level):
+        d = T.KsCommandDesc()
+        d.kind, d.dim = T.CMD_LINEAR_VELOCITY, 6
+        d.min_vel, d.max_vel, d.max_yaw = _s(self.min_vel, level), _s(self.max_vel, level), _s(self.max_yaw, level)
+        d.zero_prob, d.backward_prob, d.switch_prob = _s(self.zero_prob, level), _s(self.backward_prob, level), _s(self.switch_prob, level)
+        d.ctrl_dt, d.linear_accel, d.angular_accel = self.ctrl_dt, self.linear_accel, self.angular_accel
+        return d
+
+
+@dataclass(frozen=True)
+class AngularVelocityCommand(Command):  # commands.py:451-507
+    max_vel: object = 0.0
+    ctrl_dt: float = 0.02
+    angular_accel: float = 1.0
+    min_vel: object = 0.0
+    zero_prob: object = 0.0
+    switch_prob: object = 0.0
+
+    def dim(self):
+        return 2
+
+    def desc(self, level):
+        d = T.KsCommandDesc()
+        d.kind, d.dim = T.CMD_ANGULAR_VELOCITY, 2
+        d.min_vel, d.max_vel = _s(self.min_vel, level), _s(self.max_vel, level)
+        d.zero_prob, d.switch_prob = _s(self.zero_prob, level), _s(self.switch_prob, level)
+        d.ctrl_dt, d.angular_accel = self.ctrl_dt, self.angular_accel
+        return d
+
+
+@dataclass(frozen=True)
+class ConstantCommand(Command):
+    """`size` floats that the task sets itself and that no step changes."""
+    size: int = 1
+
+    def dim(self):
+        return int(self.size)
+
+    def desc(self, level):
+        d = T.KsCommandDesc()
+        d.kind, d.dim = T.CMD_CONST, int(self.size)
+        return d
+
+
+class CommandSet:
+    def __init__(self, commands: Mapping[str, Command]):
+        if len(commands) > T.KS_MAX_COMMANDS:
+            raise ValueError(f"at most {T.KS_MAX_COMMANDS} commands")
+        self.commands = dict(commands)
+        self.slices: dict[str, slice] = {}
+        at = 0
+        for name, c in self.commands.items():
+            self.slices[name] = slice(at, at + c.dim())
+            at += c.dim()
+        self.command_dim = at
+        self._lib = _lib.load()
+
+    def initial(self, num_envs: int, device="cuda") -> torch.Tensor:
+        """A zeroed command vector; the first `update(..., all_fresh=True)` draws the initial commands."""
+        return torch.zeros(num_envs, self.command_dim, dtype=torch.float32, device=device)
+
+    def update(self, command: torch.Tensor, qpos: torch.Tensor, qvel: torch.Tensor, *, level: float = 1.0,
+               fresh: torch.Tensor | None = None, all_fresh: bool = False, record: torch.Tensor | None = None,
+               uniform: torch.Tensor | None = None, seed: int = 0, step: int = 0, step_base=None) -> torch.Tensor:
+        """Advances every env's commands in place; `record` (N, command_dim) receives the incoming values."""
+        N = command.shape[0]
+        _lib.require_cuda(command, qpos, qvel, record, uniform, dtype=torch.float32)
+        if tuple(command.shape) != (N, self.command_dim) or qpos.shape[0] != N or qvel.shape[0] != N:
+            raise _lib.KsError(f"command must be (N, {self.command_dim}) and the state must have N rows")
+        if record is not None and tuple(record.shape) != tuple(command.shape):
+            raise _lib.KsError("record must have the command's shape")
+        if uniform is not None and tuple(uniform.shape) != (N, len(self.commands), T.KS_COMMAND_DRAWS):
+            raise _lib.KsError(f"uniform must be (N, {len(self.commands)}, {T.KS_COMMAND_DRAWS})")
+        io = T.KsCommandIO()
+        io.N, io.command_dim, io.n_commands, io.nq, io.nv = N, self.command_dim, len(self.commands), qpos.shape[1], qvel.shape[1]
+        for k, (name, c) in enumerate(self.commands.items()):
+            d = c.desc(float(level))
+            d.index = self.slices[name].start
+            io.commands[k] = d
+        io.command, io.traj_command = command.data_ptr(), _lib.ptr(record).value
+        io.qpos, io.qvel = qpos.data_ptr(), qvel.data_ptr()
+        if fresh is not None:
+            _lib.require_cuda(fresh, dtype=torch.uint8)
+            if tuple(fresh.shape) != (N,):
+                raise _lib.KsError("fresh must be (N,) uint8")
+            io.fresh = fresh.data_ptr()
+        io.all_fresh, io.uniform = int(bool(all_fresh)), _lib.ptr(uniform).value
+        if step_base is not None:
+            _lib.require_cuda(step_base, dtype=torch.int64)
+        io.rng = T.KsRng(int(seed) & (2**64 - 1), int(step) & (2**64 - 1), _lib.ptr(step_base).value)
+        _lib.check(self._lib.ks_commands(_lib.current_stream(), ctypes.byref(io)))
+        return command

@@ -332,6 +332,7 @@ extern "C" int64_t ks_abi_sizeof(int32_t which) {
     case 16: return sizeof(KsGruDesc);
     case 17: return sizeof(KsLstmDesc);
     case 18: return sizeof(KsGaussianHead);
+    case 19: return sizeof(KsCommandIO);
     default: return -1;
   }
 }

@@ -524,6 +524,66 @@ __global__ __launch_bounds__(256) void reward_scan_kernel(KsRewardScanIO io) {
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Commands: one thread per (env, command).
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void command_kernel(KsCommandIO io) {
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= io.N * io.n_commands) return;
+  const int64_t e = idx / io.n_commands;
+  const int k = (int)(idx - e * io.n_commands);
+  const KsCommandDesc c = io.commands[k];
+  float* cmd = io.command + e * io.command_dim + c.index;
+  if (io.traj_command)
+    for (int j = 0; j < c.dim; ++j) io.traj_command[e * io.command_dim + c.index + j] = cmd[j];
+  if (c.kind == KS_CMD_CONST) return;
+  float u[KS_COMMAND_DRAWS];
+  if (io.uniform) {
+    for (int j = 0; j < KS_COMMAND_DRAWS; ++j) u[j] = io.uniform[idx * KS_COMMAND_DRAWS + j];
+  } else {
+    const uint64_t step = io.rng.step + (io.rng.step_base ? *io.rng.step_base : 0ull);
+    const Philox4 a = draw(io.rng.seed, step, kRngCommand, (uint64_t)e, (uint32_t)(2 * k));
+    const Philox4 b = draw(io.rng.seed, step, kRngCommand, (uint64_t)e, (uint32_t)(2 * k + 1));
+    u[0] = u01(a.x); u[1] = u01(a.y); u[2] = u01(a.z); u[3] = u01(a.w);
+    u[4] = u01(b.x); u[5] = u01(b.y); u[6] = u01(b.z); u[7] = u01(b.w);
+  }
+  const bool fresh = io.all_fresh || (io.fresh && io.fresh[e]);
+  const float* qv = io.qvel + e * io.nv;
+  if (c.kind == KS_CMD_LINEAR_VELOCITY) {
+    float vel = cmd[0], yaw = cmd[1], tv = cmd[4], ty = cmd[5];
+    const bool redraw = fresh || u[4] < c.switch_prob;
+    if (fresh) {  // measured speed and heading in the robot frame (commands.py:316-323)
+      float lv[3];
+      rot_inv(io.qpos + e * io.nq + 3, qv[0], qv[1], qv[2], lv);
+      vel = sqrtf(lv[0] * lv[0] + lv[1] * lv[1]);
+      yaw = atan2f(lv[1], lv[0]);
+    }
+    if (redraw) {  // commands.py:328-335
+      tv = c.min_vel + u[0] * (c.max_vel - c.min_vel);
+      ty = -c.max_yaw + u[1] * (2.f * c.max_yaw);
+      const bool zero = u[2] < c.zero_prob, back = u[3] < c.backward_prob;
+      tv = zero ? 0.f : (back ? -tv : tv);
+      ty = zero ? 0.f : ty;
+    } else {       // commands.py:349-357
+      vel += fminf(fmaxf(tv - vel, -c.linear_accel), c.linear_accel) * c.ctrl_dt;
+      yaw += fminf(fmaxf(ty - yaw, -c.angular_accel), c.angular_accel) * c.ctrl_dt;
+    }
+    cmd[0] = vel; cmd[1] = yaw; cmd[2] = vel * cosf(yaw); cmd[3] = vel * sinf(yaw); cmd[4] = tv; cmd[5] = ty;
+  } else {
+    float vel = cmd[0], tv = cmd[1];
+    const bool redraw = fresh || u[3] < c.switch_prob;
+    if (redraw) {  // commands.py:470-478: on a switch the current value is re-read from the state as well
+      tv = c.min_vel + u[0] * (c.max_vel - c.min_vel);
+      tv = u[1] < 0.5f ? -tv : tv;
+      tv = u[2] < c.zero_prob ? 0.f : tv;
+      vel = qv[5];
+    } else {
+      vel += fminf(fmaxf(tv - vel, -c.angular_accel), c.angular_accel) * c.ctrl_dt;
+    }
+    cmd[0] = vel; cmd[1] = tv;
+  }
+}
+
 }  // namespace ks
 
 using namespace ks;
@@ -732,4 +792,23 @@ extern "C" int ks_reward_scan(ks_stream_t stream, const KsRewardScanIO* io) {
   if (grid > 0x7fffffff) return fail(KS_ELIMIT, "ks_reward_scan: too many envs");
   hipLaunchKernelGGL(reward_scan_kernel, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, *io);
   return check_launch("ks_reward_scan");
+}
+
+extern "C" int ks_commands(ks_stream_t stream, const KsCommandIO* io) {
+  using namespace ks;
+  if (!io) return fail(KS_EINVAL, "ks_commands: null argument");
+  if (io->N < 0 || io->n_commands < 0 || io->n_commands > KS_MAX_COMMANDS) return fail(KS_ELIMIT, "ks_commands: %d commands (0..%d)", io->n_commands, KS_MAX_COMMANDS);
+  if (io->N == 0 || io->n_commands == 0) return KS_OK;
+  if (!io->command) return fail(KS_EINVAL, "ks_commands: the command buffer is required");
+  for (int k = 0; k < io->n_commands; ++k) {
+    const KsCommandDesc& c = io->commands[k];
+    const int need = c.kind == KS_CMD_LINEAR_VELOCITY ? 6 : (c.kind == KS_CMD_ANGULAR_VELOCITY ? 2 : c.dim);
+    if (c.kind < KS_CMD_CONST || c.kind > KS_CMD_ANGULAR_VELOCITY) return fail(KS_EINVAL, "ks_commands: command %d: bad kind", k);
+    if (c.dim != need || c.dim < 1 || c.index < 0 || c.index + c.dim > io->command_dim) return fail(KS_EINVAL, "ks_commands: command %d: [%d,%d) outside the %d-wide command vector or of the wrong length", k, c.index, c.index + c.dim, io->command_dim);
+    if (c.kind != KS_CMD_CONST && (!io->qpos || !io->qvel || io->nq < 7 || io->nv < 6)) return fail(KS_EINVAL, "ks_commands: velocity commands read the state of a floating base");
+  }
+  const int64_t n = io->N * io->n_commands, grid = (n + 255) / 256;
+  if (grid > 0x7fffffff) return fail(KS_ELIMIT, "ks_commands: too many elements");
+  hipLaunchKernelGGL(command_kernel, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, *io);
+  return check_launch("ks_commands");
 }

@@ -16,6 +16,7 @@ import torch
 from . import _lib
 from . import _lib_terms as T
 from . import ppo as ppo_mod
+from .commands import CommandSet
 from .engine import HipEngine
 from .env_terms import EnvTerms, sample_action
 from .mlp import MLP
@@ -37,6 +38,7 @@ class RolloutConstants:  # the static pieces, ksim/task/rl.py:138-150
     action_clip_max: float = 1e3  # RLConfig.action_clip_max, rl.py:589-592
     reward_clip_min: float | None = None
     reward_clip_max: float | None = None
+    commands: CommandSet | None = None  # commands advanced once per control step (rl.py:1082-1098); None: constant
 
 
 class RolloutEnvState:  # ksim/task/rl.py:110-123, batched
@@ -50,6 +52,7 @@ class RolloutEnvState:  # ksim/task/rl.py:110-123, batched
         self.step = 0
         self.obs_carry = None     # (N, carry_dim) carries of the stateful observations (rl.py:118), made on first use
         self.reward_carry = None  # (N, reward carry size) carries of the stateful rewards (rl.py:119)
+        self.commands_drawn = False  # whether the command set has drawn this env state's initial commands
         self.actor_carry = None   # (depth, N, hidden) carries of recurrent networks (rl.py:117)
         self.critic_carry = None
         N = physics_state.data.qpos.shape[0]
@@ -74,6 +77,9 @@ class Rollout:
         self.components = torch.zeros(Tn, max(c.terms.n_terms, 1), N, dtype=torch.int8, device=dev)
         self.values = f(Tn, N, 1) if c.critic is not None else None
         self.reset_mask = b(N)
+        self.command = f(Tn, N, c.commands.command_dim) if c.commands is not None else None
+        if c.commands is not None and c.commands.command_dim != c.terms.command_dim:
+            raise _lib.KsError("the command set and the observation terms disagree about the width of the command vector")
         # Philox step counter of graph replays: kernels add it to the step baked into the captured launch
         self.step_base = torch.zeros(1, dtype=torch.int64, device=dev)
         self._graph = None
@@ -129,6 +135,9 @@ class Rollout:
                                 event_force=ps.event_states.get("_force_buffer") if ps.event_states else None)
         # refresh the derived fields and the warm start of the reset envs (engine.py:213)
         c.engine.forward(c.physics_model, ps, self.reset_mask, env.randomization_dict)
+        if c.commands is not None:  # record the commands this step ran under, then advance them (rl.py:1082-1098)
+            c.commands.update(env.commands, d.qpos, d.qvel, level=level, fresh=self.reset_mask, record=self.command[t],
+                              uniform=noise.get("command_uniform"), seed=env.seed, step=step, step_base=step_base)
         if not _relative_step:
             env.step += 1
 
@@ -173,6 +182,10 @@ class Rollout:
         if self.c.terms.carry_dim and env.obs_carry is None:
             env.obs_carry = torch.zeros(self.N, self.c.terms.carry_dim, dtype=torch.float32, device=self.done.device)
             self.reset_mask.fill_(1)  # every env starts an episode: the first observation initialises all carries
+        if self.c.commands is not None and not env.commands_drawn:  # get_initial_commands on the reset state (rl.py:319-332)
+            d = env.physics_state.data
+            self.c.commands.update(env.commands, d.qpos, d.qvel, all_fresh=True, seed=env.seed, step=(1 << 62) + env.step)
+            env.commands_drawn = True
         for net, name in ((self.c.actor, "actor_carry"), (self.c.critic, "critic_carry")):
             if isinstance(net, RecurrentNetwork) and getattr(env, name) is None:
                 setattr(env, name, net.initial_carry(self.N, self.done.device))
@@ -185,12 +198,20 @@ class Rollout:
         self._prepare_env(env)
         return get_rewards(traj, self.c.rewards, self.c.reward_clip_min, self.c.reward_clip_max,
                            want_components=want_components, rewards_carry=env.reward_carry,
-                           obs_slices=self.c.terms.obs_slices, level=level)
+                           obs_slices=self.c.terms.obs_slices, level=level,
+                           command_slices=self.c.commands.slices if self.c.commands is not None else None)
+
+    def _command_leaves(self) -> dict:
+        if self.command is None:
+            return {}
+        out = {name: self.command[..., sl] for name, sl in self.c.commands.slices.items()}
+        out["_buffer"] = self.command
+        return out
 
     def trajectory(self) -> Trajectory:
         names = list(self.c.terms.terminations)
         return Trajectory(qpos=self.qpos, qvel=self.qvel, xpos=self.xpos, xquat=self.xquat, ctrl=self.ctrl,
-                          obs={"obs": self.obs, "noisy_obs": self.noisy_obs}, command={}, event_state={},
+                          obs={"obs": self.obs, "noisy_obs": self.noisy_obs}, command=self._command_leaves(), event_state={},
                           action=self.action, done=self.done, success=self.success, timestep=self.timestep,
                           termination_components={n: self.components[:, j] for j, n in enumerate(names)})
 

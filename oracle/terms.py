@@ -374,3 +374,40 @@ def motionless_at_rest_penalty(qvel_tv, linvel_moving_threshold=0.5, angvel_movi
 def force_penalty(force_tn3, expected_weight, bias=0.0):  # rewards.py:1237-1240
     obs = np.clip(np.linalg.norm(force_tn3, axis=-1) - bias, 0.0, None)
     return np.square(obs / expected_weight).max(axis=-1)
+
+
+# ------------------------------------------------------------------ commands
+def linear_velocity_command(prev, qpos, qvel, u, fresh, *, min_vel, max_vel, max_yaw=0.0, zero_prob=0.0, backward_prob=0.0,
+                            switch_prob=0.0, ctrl_dt, linear_accel, angular_accel):
+    """One control step of LinearVelocityCommand for one env (ksim/commands.py:301-391).  prev / result =
+    (vel, yaw, xvel, yvel, target_vel, target_yaw); u = draws (target speed, target yaw, zero, backward, switch);
+    `fresh` = the env starts an episode (initial_command without a previous command)."""
+    vel, yaw, _, _, tv, ty = (float(x) for x in prev)
+    redraw = fresh or u[4] < switch_prob
+    if fresh:
+        lv = rotate_vector_by_quat(np.asarray(qvel[:3], dtype=np.float64)[None], np.asarray(qpos[3:7], dtype=np.float64)[None], inverse=True)[0]
+        vel, yaw = float(np.hypot(lv[0], lv[1])), float(np.arctan2(lv[1], lv[0]))
+    if redraw:
+        tv = min_vel + u[0] * (max_vel - min_vel)
+        ty = -max_yaw + u[1] * (2.0 * max_yaw)
+        zero, back = u[2] < zero_prob, u[3] < backward_prob
+        tv = 0.0 if zero else (-tv if back else tv)
+        ty = 0.0 if zero else ty
+    else:
+        vel = vel + float(np.clip(tv - vel, -linear_accel, linear_accel)) * ctrl_dt
+        yaw = yaw + float(np.clip(ty - yaw, -angular_accel, angular_accel)) * ctrl_dt
+    return np.array([vel, yaw, vel * np.cos(yaw), vel * np.sin(yaw), tv, ty])
+
+
+def angular_velocity_command(prev, qvel, u, fresh, *, max_vel, min_vel=0.0, zero_prob=0.0, switch_prob=0.0, ctrl_dt, angular_accel):
+    """One control step of AngularVelocityCommand for one env (commands.py:460-507); prev / result = (vel, target_vel);
+    u = draws (target speed, flip, zero, switch)."""
+    vel, tv = float(prev[0]), float(prev[1])
+    if fresh or u[3] < switch_prob:
+        tv = min_vel + u[0] * (max_vel - min_vel)
+        tv = -tv if u[1] < 0.5 else tv
+        tv = 0.0 if u[2] < zero_prob else tv
+        vel = float(qvel[5])
+    else:
+        vel = vel + float(np.clip(tv - vel, -angular_accel, angular_accel)) * ctrl_dt
+    return np.array([vel, tv])

@@ -45,7 +45,15 @@ def build(N, T, seed=0, min_height=0.9, events=None, gait=False, recurrent=False
                              "feet_pos": ob.BodyPositionObservation(body_ids=tuple(feet)),
                              "old_jp": ob.DelayedJointPositionObservation(delay_steps=2),
                              "imu_g": ob.ProjectedGravityObservation(min_lag=0.2, max_lag=0.6, imu_bias=0.02)})
-    terms = EnvTerms(m, observations, {"min_height": tm.MinimumHeightTermination(min_height)}, resets, command_dim=2)
+    commands = None
+    if gait:  # the walking tasks' commands: 6 + 2 floats instead of the two constants
+        from ksim_amd.commands import AngularVelocityCommand, CommandSet, LinearVelocityCommand
+        commands = CommandSet({"lin": LinearVelocityCommand(min_vel=0.2, max_vel=1.0, max_yaw=0.3, zero_prob=0.1, backward_prob=0.2,
+                                                            switch_prob=0.05, ctrl_dt=0.02, linear_accel=1.0, angular_accel=1.0),
+                               "ang": AngularVelocityCommand(max_vel=0.5, zero_prob=0.2, switch_prob=0.05, ctrl_dt=0.02, angular_accel=1.0)})
+        observations["feet_force"] = ob.FeetTorqueObservation(foot_left=feet[0], foot_right=feet[1])
+    terms = EnvTerms(m, observations, {"min_height": tm.MinimumHeightTermination(min_height)}, resets,
+                     command_dim=commands.command_dim if commands else 2)
     dims = (terms.obs_dim, 64, 64, m.nu)
     ws = [rng.normal(scale=1 / np.sqrt(i), size=(o, i)).astype(np.float32) for i, o in zip(dims[:-1], dims[1:])]
     ws[-1] *= 0.1  # small final layer: actions stay near the PD set point
@@ -61,7 +69,11 @@ def build(N, T, seed=0, min_height=0.9, events=None, gait=False, recurrent=False
         rewards.update({"air_time": rw.FeetAirTimeReward(scale=1.0, gait_period=0.2, air_time_percent=0.5, ctrl_dt=0.02,
                                                          contact_obs="contact", linvel_moving_threshold=0.05),
                         "step_height": rw.SparseTargetHeightReward(scale=2.0, contact_obs="contact", position_obs="feet_pos",
-                                                                   height=0.1, linvel_moving_threshold=0.02)})
+                                                                   height=0.1, linvel_moving_threshold=0.02),
+                        "track_lin": rw.LinearVelocityReward(scale=0.5, cmd="lin"),
+                        "track_ang": rw.AngularVelocityReward(scale=0.25, cmd="ang"),
+                        "rest": rw.MotionlessAtRestPenalty(scale=0.01),
+                        "force": rw.ForcePenalty(scale=0.01, force_obs="feet_force", expected_weight=200.0)})
     actor, critic = MLP(ws, bs, dtype="f32"), MLP(cws, cbs, dtype="f32")
     if recurrent:  # the shape of the shipped examples' networks: projection, GRU stack, GELU / ELU output MLP
         from ksim_amd.recurrent import GRUCell, RecurrentNetwork
@@ -78,7 +90,7 @@ def build(N, T, seed=0, min_height=0.9, events=None, gait=False, recurrent=False
             return n
         actor, critic = net(m.nu, "gelu"), net(1, "elu")
     consts = RolloutConstants(physics_model=dm, engine=eng, terms=terms, rewards=rewards,
-                              actor=actor, critic=critic, log_std=t32(log_std))
+                              actor=actor, critic=critic, log_std=t32(log_std), commands=commands)
     gen = torch.Generator(device=DEV); gen.manual_seed(seed)
     randomization = rnd.get_physics_randomizers(m, {"f": rnd.FloorFrictionRandomizer(0.4, 1.2),
                                                     "m": rnd.AllBodiesMassMultiplicationRandomizer(0.9, 1.1)}, N, gen)
@@ -307,7 +319,7 @@ def test_gait_terms_in_the_rollout_and_under_graph_replay():
     for use_graph in (False, True):
         m, c, rnd_, _, ro, EnvState = build(N, T, seed=7, min_height=0.8, gait=True)
         ps = c.engine.reset(c.physics_model, 1.0, 3, N, rnd_)
-        env = EnvState(ps, rnd_, torch.zeros(N, 2, device=DEV), None, seed=9)
+        env = EnvState(ps, rnd_, c.commands.initial(N, DEV), None, seed=9)
         sl = c.terms.obs_slices
         carries = [((np.zeros(2, int),) * 3, np.zeros(2)) for _ in range(N)]
         snaps = []
@@ -315,11 +327,17 @@ def test_gait_terms_in_the_rollout_and_under_graph_replay():
             traj, rew = ro.unroll(env, graph=use_graph)
             torch.cuda.synchronize()
             snaps.append((traj.obs["obs"].clone(), rew.total.clone(), env.obs_carry.clone(), env.reward_carry.clone()))
+            snaps[-1] += (traj.command["_buffer"].clone(), env.commands.clone())
             if use_graph:
                 continue
+            cm = traj.command["_buffer"].cpu().numpy()
+            # recorded commands: step t+1 shows the update of step t; a finished env drew a fresh command instead
+            lin, ang = cm[..., c.commands.slices["lin"]], cm[..., c.commands.slices["ang"]]
+            np.testing.assert_allclose(lin[..., 2], lin[..., 0] * np.cos(lin[..., 1]), atol=1e-6)
+            assert (np.abs(lin[..., 4]) <= 1.0).all() and (np.abs(ang[..., 1]) <= 0.5).all() and np.abs(lin[..., 4]).max() > 0.2
             obs, qvel, done = traj.obs["obs"].cpu().numpy(), traj.qvel.cpu().numpy(), traj.done.cpu().numpy().astype(bool)
             from ksim_amd.rewards import get_rewards
-            full = get_rewards(traj, c.rewards, want_components=True, obs_slices=sl) if it == 0 else None  # from a zero carry
+            full = get_rewards(traj, c.rewards, want_components=True, obs_slices=sl, command_slices=c.commands.slices) if it == 0 else None  # zero carry
             xpos = traj.xpos.cpu().numpy().reshape(T, N, m.nb, 3)
             feet = [b for b in range(m.nb) if any(int(sb) == b for sb in m.sph_body)]
             # the recorded observation is taken before the step, the recorded xpos after it: row t+1 of the former
@@ -348,7 +366,7 @@ def test_gait_terms_in_the_rollout_and_under_graph_replay():
         assert use_graph or 0.05 < touched < 1.0, "the feet never touched the floor: the contact terms were not exercised"
         runs.append(snaps)
     for it, (a, b) in enumerate(zip(*runs)):
-        for x, y, name in zip(a, b, ("observations", "reward", "observation carry", "reward carry")):
+        for x, y, name in zip(a, b, ("observations", "reward", "observation carry", "reward carry", "recorded commands", "commands")):
             assert torch.equal(x, y), f"replay {it}: {name} differs from the eager rollout"
 
 

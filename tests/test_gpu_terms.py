@@ -539,3 +539,45 @@ def test_command_tracking_rest_and_force_rewards():
         rw.get_rewards(traj, {"lin": rw.LinearVelocityReward(cmd="nope")}, command_slices={"lin_cmd": slice(0, 4)})
     with pytest.raises(Exception, match="command"):
         rw.get_rewards(traj, {"ang": rw.AngularVelocityReward(cmd="a")}, command_slices={"a": slice(8, 9)})
+
+
+def test_velocity_commands_against_oracle():
+    """LinearVelocityCommand / AngularVelocityCommand over several control steps with explicit draws: episode starts,
+    slewing, switches, zero and backward targets; the recorded copy is the incoming command."""
+    from ksim_amd import _lib_terms as T
+    from ksim_amd.commands import AngularVelocityCommand, CommandSet, ConstantCommand, LinearVelocityCommand
+    from ksim_amd.scales import LinearScale
+
+    N, steps, level = 41, 12, 0.5
+    rng = np.random.default_rng(41)
+    lp = dict(min_vel=0.3, max_vel=LinearScale(scale=2.0, bias=0.5), max_yaw=0.4, zero_prob=0.2, backward_prob=0.3, switch_prob=0.15,
+              ctrl_dt=0.02, linear_accel=3.0, angular_accel=2.0)
+    ap = dict(max_vel=1.0, min_vel=0.1, zero_prob=0.25, switch_prob=0.2, ctrl_dt=0.02, angular_accel=1.5)
+    cs = CommandSet({"pad": ConstantCommand(size=3), "lin": LinearVelocityCommand(**lp), "ang": AngularVelocityCommand(**ap)})
+    assert cs.command_dim == 11 and cs.slices["lin"] == slice(3, 9)
+    lpo = dict(lp, max_vel=2.0 * level + 0.5)
+    cmd = cs.initial(N, DEV)
+    cmd[:, :3] = 7.0
+    want = np.zeros((N, 11)); want[:, :3] = 7.0
+    for k in range(steps):
+        qpos = rng.normal(size=(N, 27)); qpos[:, 3:7] /= np.linalg.norm(qpos[:, 3:7], axis=1, keepdims=True)
+        qvel = rng.normal(size=(N, 26))
+        u = rng.random((N, 3, T.KS_COMMAND_DRAWS)).astype(np.float32)
+        fresh = np.ones(N, bool) if k == 0 else rng.random(N) < 0.1
+        rec = torch.empty(N, 11, device=DEV)
+        cs.update(cmd, t32(qpos), t32(qvel), level=level, fresh=torch.from_numpy(fresh.astype(np.uint8)).to(DEV), record=rec, uniform=t32(u))
+        np.testing.assert_allclose(rec.cpu().numpy(), want, rtol=1e-5, atol=1e-6)
+        q32, v32 = qpos.astype(np.float32).astype(np.float64), qvel.astype(np.float32).astype(np.float64)
+        for e in range(N):
+            want[e, 3:9] = ot.linear_velocity_command(want[e, 3:9], q32[e], v32[e], u[e, 1].astype(np.float64), bool(fresh[e]), **lpo)
+            want[e, 9:11] = ot.angular_velocity_command(want[e, 9:11], v32[e], u[e, 2].astype(np.float64), bool(fresh[e]), **ap)
+        got = cmd.cpu().numpy()
+        # heading measured at an episode start sits on atan2's branch cut for a robot moving straight backwards
+        np.testing.assert_allclose(got, want, rtol=2e-5, atol=2e-5)
+    assert (want[:, 7] == 0).any() and (want[:, 7] < 0).any() and (cmd[:, :3] == 7.0).all()
+    # Philox: reproducible, targets inside the ranges
+    a, b = cs.initial(N, DEV), cs.initial(N, DEV)
+    cs.update(a, t32(qpos), t32(qvel), all_fresh=True, seed=3, step=1); cs.update(b, t32(qpos), t32(qvel), all_fresh=True, seed=3, step=1)
+    assert torch.equal(a, b) and (a[:, 7].abs() <= 2.5).all() and (a[:, 10].abs() <= 1.0).all() and a[:, 7].std() > 0.1
+    with pytest.raises(Exception, match="uniform"):
+        cs.update(a, t32(qpos), t32(qvel), uniform=t32(u[:, :2]))

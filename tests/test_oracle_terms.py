@@ -253,3 +253,33 @@ def test_command_tracking_and_rest_rewards_hand_computed():
     f = np.array([[[3.0, 4.0, 0.0], [0.0, 0.0, 12.0]]])
     assert terms.force_penalty(f, expected_weight=5.0, bias=2.0)[0] == pytest.approx(4.0)   # ((12 - 2) / 5)^2
     assert terms.force_penalty(f * 0.1, expected_weight=5.0, bias=2.0)[0] == 0.0
+
+
+def test_velocity_commands_hand_computed():
+    p = dict(min_vel=0.5, max_vel=1.5, max_yaw=0.4, zero_prob=0.2, backward_prob=0.3, switch_prob=0.1, ctrl_dt=0.02,
+             linear_accel=2.0, angular_accel=1.0)
+    q = np.zeros(7); q[3:7] = [np.cos(np.pi / 4), 0, 0, np.sin(np.pi / 4)]   # yawed by 90 degrees
+    v = np.zeros(8); v[:3] = [0.0, 2.0, 0.0]                                 # 2 m/s straight ahead in the robot frame
+    # episode start: measured speed / heading, fresh targets
+    c = terms.linear_velocity_command(np.zeros(6), q, v, [0.75, 0.25, 0.9, 0.9, 0.9], True, **p)
+    np.testing.assert_allclose(c, [2.0, 0.0, 2.0, 0.0, 1.25, -0.2], atol=1e-12)
+    # ordinary step: the current values slew towards the targets, limited by the accelerations
+    c2 = terms.linear_velocity_command(c, q, v, [0.0, 0.0, 0.9, 0.9, 0.9], False, **p)
+    np.testing.assert_allclose(c2[:2], [2.0 - 0.75 * 0.02, -0.2 * 0.02], atol=1e-12)
+    np.testing.assert_allclose(c2[2:4], [c2[0] * np.cos(c2[1]), c2[0] * np.sin(c2[1])])
+    assert tuple(c2[4:]) == (1.25, -0.2)
+    big = terms.linear_velocity_command([0.0, 0.0, 0.0, 0.0, 9.0, -9.0], q, v, [0, 0, 0, 0, 0.9], False, **p)
+    np.testing.assert_allclose(big[:2], [2.0 * 0.02, -1.0 * 0.02])           # clipped slew
+    # switch: new targets, current values kept (not measured, not slewed); zero and backward draws
+    c3 = terms.linear_velocity_command(c2, q, v, [0.5, 0.5, 0.9, 0.1, 0.05], False, **p)
+    np.testing.assert_allclose(c3, [c2[0], c2[1], c2[2], c2[3], -1.0, 0.0], atol=1e-12)
+    c4 = terms.linear_velocity_command(c2, q, v, [0.5, 0.9, 0.1, 0.1, 0.05], False, **p)
+    assert tuple(c4[4:]) == (0.0, 0.0)
+    pa = dict(max_vel=1.0, min_vel=0.2, zero_prob=0.1, switch_prob=0.3, ctrl_dt=0.02, angular_accel=0.5)
+    v[5] = 0.3
+    a = terms.angular_velocity_command([0.0, 0.0], v, [0.5, 0.4, 0.9, 0.9], True, **pa)
+    np.testing.assert_allclose(a, [0.3, -0.6])
+    a2 = terms.angular_velocity_command(a, v, [0, 0, 0, 0.9], False, **pa)
+    np.testing.assert_allclose(a2, [0.3 - 0.5 * 0.02, -0.6])
+    a3 = terms.angular_velocity_command(a2, v, [0.5, 0.6, 0.05, 0.1], False, **pa)   # switch: re-measured, zeroed target
+    np.testing.assert_allclose(a3, [0.3, 0.0])
