@@ -309,7 +309,9 @@ typedef struct KsObsElem {
 
 /* Terminations (replaces get_terminations + terms, rl.py:288-299, ksim/terminations.py:60-192). */
 enum { KS_TERM_MIN_HEIGHT = 0, KS_TERM_BAD_Z = 1, KS_TERM_NOT_UPRIGHT = 2, KS_TERM_BAD_VELOCITY = 3,
-       KS_TERM_FAR_FROM_ORIGIN = 4, KS_TERM_EPISODE_LENGTH = 5 };
+       KS_TERM_FAR_FROM_ORIGIN = 4, KS_TERM_EPISODE_LENGTH = 5,
+       KS_TERM_ILLEGAL_CONTACT = 6 /* a listed contact sphere is deeper than contact_eps into the floor: some
+                                      contact_dist[s] < p0 with bit s of the sphere mask (int)p1 set (terminations.py:84-99) */ };
 typedef struct KsTermDesc {
   int32_t kind;
   int32_t value; /* what a firing term reports: -1 or +1 */
@@ -378,6 +380,7 @@ typedef struct KsTerminateIO {
   float* event_state;               /* (n_events, N), nullable when n_events == 0 */
   const float* event_reset_uniform; /* (N, n_events) U[0,1) draws, nullable -> Philox */
   float* event_force;               /* (n_events, N, KS_EVENT_FORCE_STATE), nullable: zeroed for the reset envs */
+  const float* contact_dist;        /* (N, ns) KsStepIO.contact_dist of the step just taken; KS_TERM_ILLEGAL_CONTACT only */
 } KsTerminateIO;
 int ks_terminate_reset(const KsTerms* terms, ks_stream_t stream, const KsTerminateIO* io /*host*/);
 

@@ -10,7 +10,7 @@ KS_MAX_OBS, KS_MAX_TERMS, KS_MAX_QPOS, KS_MAX_LAYERS = 512, 16, 40, 8
 OBS_COPY, OBS_JOINT_POS, OBS_ROT_INV, OBS_CONTACT, OBS_DELAYED, OBS_GRAVITY_EMA = range(6)
 NOISE_NONE, NOISE_ADD_GAUSSIAN, NOISE_ADD_UNIFORM, NOISE_MUL_GAUSSIAN, NOISE_MUL_UNIFORM = range(5)
 (TERM_MIN_HEIGHT, TERM_BAD_Z, TERM_NOT_UPRIGHT, TERM_BAD_VELOCITY, TERM_FAR_FROM_ORIGIN,
- TERM_EPISODE_LENGTH) = range(6)
+ TERM_EPISODE_LENGTH, TERM_ILLEGAL_CONTACT) = range(7)
 ACT_NONE, ACT_ELU, ACT_RELU, ACT_TANH, ACT_GELU = range(5)
 MLP_F32, MLP_BF16 = 0, 1
 
@@ -66,7 +66,7 @@ class KsTerminateIO(ctypes.Structure):
                 ("traj_time", c_void_p), ("reset_mask", c_void_p), ("episode_length", c_void_p),
                 ("reset_uniform", c_void_p), ("rng", KsRng), ("apply_reset", c_int32), ("n_events", c_int32),
                 ("event_interval", (c_float * 2) * KS_MAX_EVENTS), ("event_state", c_void_p),
-                ("event_reset_uniform", c_void_p), ("event_force", c_void_p)]
+                ("event_reset_uniform", c_void_p), ("event_force", c_void_p), ("contact_dist", c_void_p)]
 
 
 class KsMlpDesc(ctypes.Structure):

@@ -148,6 +148,8 @@ struct TerminateArgs {
   float* event_state;
   const float* event_reset_uniform;
   float* event_force;
+  const float* contact_dist;
+  int ns;
 };
 
 // A 256-thread workgroup owns kTermEnvs consecutive envs.  The state rows of those envs are contiguous in memory,
@@ -205,6 +207,11 @@ __global__ __launch_bounds__(256) void terminate_kernel(TerminateArgs a) {
         case KS_TERM_BAD_VELOCITY: fire = sqrtf(v[0] * v[0] + v[1] * v[1] + v[2] * v[2]) > td.p0; break;
         case KS_TERM_FAR_FROM_ORIGIN: fire = sqrtf(q[0] * q[0] + q[1] * q[1] + q[2] * q[2]) > td.p0; break;
         case KS_TERM_EPISODE_LENGTH: fire = (tm > td.p0) && !(td.p1 >= 0.f && a.level < td.p1); break;
+        case KS_TERM_ILLEGAL_CONTACT: {
+          const unsigned mask = (unsigned)td.p1;
+          for (int sidx = 0; sidx < a.ns; ++sidx)
+            fire |= ((mask >> sidx) & 1u) && a.contact_dist[e * a.ns + sidx] < td.p0;
+        } break;
         default: break;
       }
       const int8_t val = fire ? (int8_t)td.value : (int8_t)0;
@@ -626,7 +633,9 @@ extern "C" int ks_terms_create(const KsTermsDesc* d, KsTerms** out) {
   }
   for (int j = 0; j < d->n_terms; ++j) {
     const KsTermDesc& t = d->terms[j];
-    if (t.kind < KS_TERM_MIN_HEIGHT || t.kind > KS_TERM_EPISODE_LENGTH) return fail(KS_EINVAL, "ks_terms_create: termination %d: bad kind", j);
+    if (t.kind < KS_TERM_MIN_HEIGHT || t.kind > KS_TERM_ILLEGAL_CONTACT) return fail(KS_EINVAL, "ks_terms_create: termination %d: bad kind", j);
+    if (t.kind == KS_TERM_ILLEGAL_CONTACT && (d->ns < 1 || d->ns > 24 || t.p1 < 0.f || t.p1 >= (float)(1u << d->ns)))
+      return fail(KS_EINVAL, "ks_terms_create: termination %d: sphere mask outside the model's %d spheres", j, d->ns);
     if (t.value != 1 && t.value != -1) return fail(KS_EINVAL, "ks_terms_create: termination %d must report +1 or -1", j);
     if ((t.kind == KS_TERM_NOT_UPRIGHT) && d->nq < 7) return fail(KS_EINVAL, "ks_terms_create: termination %d needs a free root", j);
     if (d->nq < 3 || d->nv < 3) return fail(KS_EINVAL, "ks_terms_create: terminations need a floating base");
@@ -696,6 +705,9 @@ extern "C" int ks_terminate_reset(const KsTerms* t, ks_stream_t stream, const Ks
   a.random_heading = d.random_heading; a.nonfinite_terminates = d.nonfinite_terminates;
   if (io->n_events < 0 || io->n_events > KS_MAX_EVENTS) return fail(KS_ELIMIT, "ks_terminate_reset: %d events (0..%d)", io->n_events, KS_MAX_EVENTS);
   if (io->n_events > 0 && !io->event_state) return fail(KS_EINVAL, "ks_terminate_reset: events need event_state");
+  a.contact_dist = io->contact_dist; a.ns = d.ns;
+  for (int j = 0; j < d.n_terms; ++j)
+    if (d.terms[j].kind == KS_TERM_ILLEGAL_CONTACT && !io->contact_dist) return fail(KS_EINVAL, "ks_terminate_reset: termination %d reads contact_dist", j);
   a.n_events = io->n_events; a.event_state = io->event_state; a.event_reset_uniform = io->event_reset_uniform; a.event_force = io->event_force;
   for (int k = 0; k < io->n_events; ++k) { a.event_interval[k][0] = io->event_interval[k][0]; a.event_interval[k][1] = io->event_interval[k][1]; }
   const int64_t grid = (io->N + kTermEnvs - 1) / kTermEnvs;

@@ -140,7 +140,7 @@ class EnvTerms:
                         success=None, traj_qpos=None, traj_qvel=None, traj_time=None, reset_mask=None,
                         episode_length=None, reset_uniform=None, seed: int = 0, step: int = 0, step_base=None,
                         event_state=None, event_intervals=(), event_reset_uniform=None, event_force=None,
-                        apply_reset: bool = True) -> None:
+                        contact_dist=None, apply_reset: bool = True) -> None:
         m = self.model
         qpos = state["qpos"]
         N = qpos.shape[0]
@@ -164,6 +164,11 @@ class EnvTerms:
                 raise _lib.KsError(f"{name}: expected {shape}, got {tuple(t.shape)}")
             setattr(io, name, t.data_ptr())
         io.rng = _rng(seed, step, step_base)
+        if contact_dist is not None:  # for IllegalContactTermination
+            _lib.require_cuda(contact_dist, dtype=torch.float32)
+            if tuple(contact_dist.shape) != (N, m.ns):
+                raise _lib.KsError(f"contact_dist must be ({N}, {m.ns})")
+            io.contact_dist = contact_dist.data_ptr()
         if event_state is not None:  # timers of the events, re-drawn for the envs that start a fresh episode
             _lib.require_cuda(event_state, dtype=torch.float32)
             if tuple(event_state.shape) != (len(event_intervals), N):

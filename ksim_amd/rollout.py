@@ -132,7 +132,8 @@ class Rollout:
                                 seed=env.seed, step=step, step_base=step_base, event_state=ev_buf,
                                 event_intervals=[ev.interval_range for ev in c.engine.events.values()],
                                 event_reset_uniform=noise.get("event_reset_uniform"),
-                                event_force=ps.event_states.get("_force_buffer") if ps.event_states else None)
+                                event_force=ps.event_states.get("_force_buffer") if ps.event_states else None,
+                                contact_dist=d.contact_dist)
         # refresh the derived fields and the warm start of the reset envs (engine.py:213)
         c.engine.forward(c.physics_model, ps, self.reset_mask, env.randomization_dict)
         if c.commands is not None:  # record the commands this step ran under, then advance them (rl.py:1082-1098)

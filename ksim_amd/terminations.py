@@ -83,3 +83,34 @@ class EpisodeLengthTermination(Termination):  # terminations.py:175-192
     def desc(self):
         lvl = -1.0 if self.disable_at_curriculum_level is None else float(self.disable_at_curriculum_level)
         return (T.TERM_EPISODE_LENGTH, 1 if self.pos_termination else -1, self.max_length_sec, lvl, 0.0, 0.0)
+
+
+@dataclass(frozen=True)
+class IllegalContactTermination(Termination):
+    """Fails the episode when one of the listed contact spheres is more than `-contact_eps` deep in the floor
+    (terminations.py:84-99; every contact of this model pairs a sphere with the floor, so "a contact involving an illegal
+    geom with dist < contact_eps" is a statement about the listed spheres)."""
+    illegal_sphere_idxs: tuple = ()
+    contact_eps: float = -0.001
+
+    @classmethod
+    def create(cls, physics_model, body_names, contact_eps: float = -1e-3) -> "IllegalContactTermination":
+        """Spheres given by the names of the bodies they are attached to (terminations.py:104-127)."""
+        names = set(body_names)
+        idxs = []
+        for s_, b in enumerate(physics_model.sph_body):
+            n = physics_model.body_names[int(b)]
+            if n in body_names:
+                idxs.append(s_)
+                names.discard(n)
+        if names:
+            raise ValueError(f"Bodies {names} carry no contact sphere. Choices are: {sorted(set(physics_model.body_names[int(b)] for b in physics_model.sph_body))}")
+        return cls(illegal_sphere_idxs=tuple(idxs), contact_eps=contact_eps)
+
+    def desc(self):
+        mask = 0
+        for s_ in self.illegal_sphere_idxs:
+            if not 0 <= int(s_) < 24:
+                raise ValueError("sphere index out of range")
+            mask |= 1 << int(s_)
+        return (T.TERM_ILLEGAL_CONTACT, -1, float(self.contact_eps), float(mask), 0.0, 0.0)

@@ -88,6 +88,17 @@ def test_termination_kats_and_masks_bit_exact():
     # the reference's known answers (tests/test_terminations.py:66-99) on its dummy qpos
     for kat in json.load(open(os.path.join(GOLD, "termination_kats.json"))):
         if kat["fn"] == "illegal_contact":
+            # contact k of the known answer becomes sphere k of the model: its distance, and illegal when either of its
+            # two geoms is in the illegal set
+            dist = np.full((1, m.ns), 1.0); dist[0, :kat["ncon"]] = kat["dist"][:kat["ncon"]]
+            bad = tuple(k for k in range(kat["ncon"]) if kat["geom1"][k] in kat["illegal"] or kat["geom2"][k] in kat["illegal"])
+            terms = EnvTerms(m, {}, {"t": tm.IllegalContactTermination(illegal_sphere_idxs=bad)}, [])
+            comps = torch.zeros(1, 1, dtype=torch.int8, device=DEV)
+            done = torch.zeros(1, dtype=torch.uint8, device=DEV); succ = torch.ones(1, dtype=torch.uint8, device=DEV)
+            qpos = np.zeros((1, m.nq)); qpos[0, 3] = 1.0
+            terms.terminate_reset(dict(qpos=t32(qpos), qvel=torch.zeros(1, m.nv, device=DEV)), components=comps, done=done, success=succ,
+                                  contact_dist=t32(dist), apply_reset=False)
+            assert comps.item() == kat["expected"] and done.item() == (kat["expected"] != 0) and succ.item() == 0
             continue
         term = tm.NotUprightTermination(kat["max_radians"]) if kat["fn"] == "not_upright" else tm.MinimumHeightTermination(kat["min_height"])
         terms = EnvTerms(m, {}, {"t": term}, [])
