@@ -252,6 +252,10 @@ typedef struct KsStepIO {
   float* cfrc_ext;          /* (N, nb*6) contact force on each body of the last substep as a spatial force about the tree's
                                centre of mass, world axes, torque then force: mjData.cfrc_ext, which the feet force / torque
                                observations read (ksim/observation.py:563-616); nullable */
+  /* more per-env model parameters (inputs, nullable = 1): factors on the joints' armature and damping
+     (ArmatureRandomizer, JointDampingRandomizer, ksim/randomization.py:108-123,226-243; the root's six dofs keep 1) */
+  const float* armature_scale; /* (N, nv) */
+  const float* damping_scale;  /* (N, nv) */
   /* events (ks_step only) */
   int32_t n_events;
   KsEventDesc events[KS_MAX_EVENTS];

@@ -40,7 +40,7 @@ STEP_IO_POINTERS = (
     "torque_limit_scale", "action_bias", "torque_bias", "action_noise", "torque_noise", "friction", "mass_scale",
     "env_mask",
     "qacc", "ctrl_out", "xpos", "xquat", "cvel", "traj_ctrl", "traj_xpos", "traj_xquat", "solver_niter", "nefc",
-    "dbg_M", "dbg_bias", "dbg_qacc_smooth", "contact_dist", "cinert", "cfrc_ext",
+    "dbg_M", "dbg_bias", "dbg_qacc_smooth", "contact_dist", "cinert", "cfrc_ext", "armature_scale", "damping_scale",
 )
 
 

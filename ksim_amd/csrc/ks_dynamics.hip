@@ -305,7 +305,8 @@ void step_kernel(StepArgs a) {
     const float b_q0 = rec.b_q0;
     const float b_mass = is_body ? rec.b_mass * (a.mass_scale ? a.mass_scale[env * nb + bl] : 1.f) : 0.f;
     const int d_body = rec.d_body, d_act = rec.d_act, d_jtype = rec.d_jtype, d_k = rec.d_k;
-    const float d_damping = rec.d_damping, d_armature = rec.d_armature, d_gear = rec.d_gear, d_lo = rec.d_lo, d_hi = rec.d_hi;
+    const float d_damping = rec.d_damping * ((a.damping_scale && is_dof) ? a.damping_scale[env * nv + lane] : 1.f);
+    const float d_armature = rec.d_armature, d_gear = rec.d_gear, d_lo = rec.d_lo, d_hi = rec.d_hi;
     (void)d_armature;
     const int s_body = rec.s_body;
     const V3 s_pos = {rec.s_pos[0], rec.s_pos[1], rec.s_pos[2]};
@@ -521,7 +522,7 @@ void step_kernel(StepArgs a) {
       if (pk[k] >= 0) {
         const int i = pk[k] >> 8, j = pk[k] & 0xff;
         float v = dot(ld6(l.cdof + 6 * j), ld6(l.buf + 6 * i));
-        if (i == j) v += m.dof_armature[i];
+        if (i == j) v += m.dof_armature[i] * (a.armature_scale ? a.armature_scale[env * nv + i] : 1.f);
         l.M[i * nvs + j] = v;
         l.M[j * nvs + i] = v;
       }
@@ -1178,6 +1179,7 @@ static int launch_step(const KsModel* km, ks_stream_t stream, const KsStepIO* io
   a.solver_niter = io->solver_niter; a.nefc = io->nefc;
   a.dbg_M = io->dbg_M; a.dbg_bias = io->dbg_bias; a.dbg_qacc_smooth = io->dbg_qacc_smooth;
   a.contact_dist = io->contact_dist; a.cinert = io->cinert; a.cfrc_ext = io->cfrc_ext;
+  a.armature_scale = io->armature_scale; a.damping_scale = io->damping_scale;
   a.ctrl_in = io->ctrl_in;
   if (!forward_only) {
     if (io->substeps < 1 || io->substeps > 64) return fail(KS_EINVAL, "ks_step: substeps must be in 1..64");

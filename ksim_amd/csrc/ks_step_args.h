@@ -23,6 +23,7 @@ struct StepArgs {
   float *qacc, *ctrl_out, *xpos, *xquat, *cvel, *traj_ctrl, *traj_xpos, *traj_xquat;
   int32_t *solver_niter, *nefc;
   float *dbg_M, *dbg_bias, *dbg_qacc_smooth, *contact_dist, *cinert, *cfrc_ext;
+  const float *armature_scale, *damping_scale;
   int n_events;
   KsEventDesc events[KS_MAX_EVENTS];
   float* event_state;

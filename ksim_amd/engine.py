@@ -216,6 +216,7 @@ class HipEngine(PhysicsEngine):
         rnd = randomization or {}
         physics.forward(physics_model, dict(qpos=d.qpos, qvel=d.qvel, qacc_warmstart=d.qacc_warmstart, env_mask=mask,
                                             friction=rnd.get("friction"), mass_scale=rnd.get("mass_scale"),
+                                            armature_scale=rnd.get("armature_scale"), damping_scale=rnd.get("damping_scale"),
                                             xpos=d.xpos, xquat=d.xquat, cvel=d.cvel, contact_dist=d.contact_dist,
                                             cinert=d.cinert, cfrc_ext=d.cfrc_ext))
         # engine.py:217-220: qvel and qacc are zeroed after the forward pass (qvel is already zero here)
@@ -249,7 +250,8 @@ class HipEngine(PhysicsEngine):
             drop = (torch.rand(action.shape, generator=gen, device=action.device) < p_drop).to(torch.uint8)
         buf = dict(qpos=d.qpos, qvel=d.qvel, qacc_warmstart=d.qacc_warmstart, time=d.time, last_ctrl=s.last_ctrl,
                    action=action, latency=s.action_latency, zero_offset=s.zero_offset, drop=drop,
-                   friction=rnd.get("friction"), mass_scale=rnd.get("mass_scale"), qacc=d.qacc, ctrl_out=d.ctrl,
+                   friction=rnd.get("friction"), mass_scale=rnd.get("mass_scale"), armature_scale=rnd.get("armature_scale"),
+                   damping_scale=rnd.get("damping_scale"), qacc=d.qacc, ctrl_out=d.ctrl,
                    xpos=d.xpos, xquat=d.xquat, cvel=d.cvel if want_cvel else None, contact_dist=d.contact_dist,
                    cinert=d.cinert if want_cinert else None, cfrc_ext=d.cfrc_ext if want_cfrc_ext else None,
                    action_noise=noise.get("action_noise"),

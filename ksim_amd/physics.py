@@ -55,7 +55,7 @@ class DeviceModel:
 _F32 = ("qpos", "qvel", "qacc_warmstart", "time", "last_ctrl", "action", "ctrl_in", "latency", "zero_offset", "kp",
         "kd", "ctrl_clip", "kp_scale", "kd_scale", "torque_limit_scale", "action_bias", "torque_bias", "action_noise",
         "torque_noise", "friction", "mass_scale", "qacc", "ctrl_out", "xpos", "xquat", "cvel", "dbg_M", "dbg_bias",
-        "dbg_qacc_smooth", "contact_dist", "cinert", "cfrc_ext")
+        "dbg_qacc_smooth", "contact_dist", "cinert", "cfrc_ext", "armature_scale", "damping_scale")
 _I32 = ("solver_niter", "nefc")
 
 
@@ -70,7 +70,7 @@ def _expected_shapes(m: KinematicModel, N: int, S: int) -> dict:
         "xpos": (N, nb * 3), "xquat": (N, nb * 4), "cvel": (N, nb * 6), "traj_ctrl": (N, nu),
         "traj_xpos": (N, nb * 3), "traj_xquat": (N, nb * 4), "solver_niter": (N,), "nefc": (N,),
         "dbg_M": (N, nv * nv), "dbg_bias": (N, nv), "dbg_qacc_smooth": (N, nv), "contact_dist": (N, ns),
-        "cinert": (N, nb * 10), "cfrc_ext": (N, nb * 6),
+        "cinert": (N, nb * 10), "cfrc_ext": (N, nb * 6), "armature_scale": (N, nv), "damping_scale": (N, nv),
     }
 
 

@@ -49,7 +49,8 @@ def _data_struct(real):
         _fields_ = [
             ("qpos", real * MAXQ), ("qvel", real * MAXV), ("ctrl", real * MAXU), ("qacc_warmstart", real * MAXV),
             ("time", real),
-            ("mass_scale", real * MAXB), ("friction", real), ("xfrc_applied", real * 6 * MAXB),
+            ("mass_scale", real * MAXB), ("friction", real), ("armature_scale", real * MAXV),
+            ("damping_scale", real * MAXV), ("xfrc_applied", real * 6 * MAXB),
             ("xpos", real * 3 * MAXB), ("xquat", real * 4 * MAXB), ("xmat", real * 9 * MAXB),
             ("xipos", real * 3 * MAXB), ("ximat", real * 9 * MAXB), ("xanchor", real * 3 * MAXB),
             ("xaxis", real * 3 * MAXB), ("com", real * 3),
@@ -117,7 +118,7 @@ class DataView:
             return v
         arr = np.ctypeslib.as_array(v)
         nb, nq, nv, nu, ns = a["nb"], a["nq"], a["nv"], a["nu"], a["ns"]
-        trim = {"qpos": nq, "qvel": nv, "ctrl": nu, "qacc_warmstart": nv, "mass_scale": nb, "xfrc_applied": nb, "cfrc_ext": nb, "xpos": nb, "xquat": nb,
+        trim = {"qpos": nq, "qvel": nv, "ctrl": nu, "qacc_warmstart": nv, "mass_scale": nb, "armature_scale": nv, "damping_scale": nv, "xfrc_applied": nb, "cfrc_ext": nb, "xpos": nb, "xquat": nb,
                 "xmat": nb, "xipos": nb, "ximat": nb, "xanchor": nb, "xaxis": nb, "cinert": nb, "crb": nb, "cdof": nv,
                 "cvel": nb, "cdof_dot": nv, "qfrc_bias": nv, "qfrc_passive": nv, "qfrc_actuator": nv,
                 "actuator_force": nu, "qfrc_smooth": nv, "qacc_smooth": nv, "con_dist": ns, "con_pos": ns,
@@ -156,13 +157,19 @@ class Oracle:
         f.restype = None
         return f
 
-    def data(self, qpos=None, qvel=None, friction=None, mass_scale=None) -> DataView:
+    def data(self, qpos=None, qvel=None, friction=None, mass_scale=None, armature_scale=None, damping_scale=None) -> DataView:
         raw = self.Data()
         d = DataView(raw, self.a)
         d.qpos = self.a["qpos0"] if qpos is None else qpos
         if qvel is not None:
             d.qvel = qvel
         d.mass_scale = 1.0 if mass_scale is None else mass_scale
+        d.raw.armature_scale[:] = [1.0] * MAXV
+        d.raw.damping_scale[:] = [1.0] * MAXV
+        if armature_scale is not None:
+            d.armature_scale = armature_scale
+        if damping_scale is not None:
+            d.damping_scale = damping_scale
         d.friction = self.a["friction"] if friction is None else friction
         return d
 
@@ -185,7 +192,12 @@ class Oracle:
 
     # ---- batched control step (N envs, env-major arrays) used by parity tests and the CPU baseline
     def batch(self, N: int):
-        return (self.Data * N)()
+        block = (self.Data * N)()
+        ones = [1.0] * MAXV
+        for e in range(N):  # neutral per-env parameters; the caller sets state, mass scales and friction
+            block[e].armature_scale[:] = ones
+            block[e].damping_scale[:] = ones
+        return block
 
     def ctrl_step_batch(self, block, S, actuator_period, action, last_ctrl, latency, zero_offset, kp, kd, ctrl_clip,
                         nthreads=1, qvel_impulse=None):

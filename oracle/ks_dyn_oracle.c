@@ -26,6 +26,7 @@ typedef struct FN(KsorData) {
   REAL qpos[KSOR_MAXQ], qvel[KSOR_MAXV], ctrl[KSOR_MAXU], qacc_warmstart[KSOR_MAXV], time;
   /* per-env parameters */
   REAL mass_scale[KSOR_MAXB], friction;
+  REAL armature_scale[KSOR_MAXV], damping_scale[KSOR_MAXV]; /* ksim/randomization.py:108-123, 226-243 */
   /* Cartesian force (3) and torque (3) per body, world frame, acting at the body's centre of mass: MuJoCo's
    * xfrc_applied, which ForcePushEvent writes (ksim/events.py:302-307) */
   REAL xfrc_applied[KSOR_MAXB][6];
@@ -237,7 +238,7 @@ void FN(ksor_crb)(const KsorModel* m, Data* d) {
       d->M[i * nv + j] = s;
       d->M[j * nv + i] = s;
     }
-    d->M[i * nv + i] += (REAL)m->dof_armature[i];
+    d->M[i * nv + i] += (REAL)m->dof_armature[i] * d->armature_scale[i];
   }
 }
 
@@ -606,7 +607,7 @@ void FN(ksor_forward)(const KsorModel* m, Data* d) {
   FN(ksor_make_constraint)(m, d); /* uses qvel for aref, like make_constraint after fwd_position in MJX */
   FN(ksor_com_vel)(m, d);
   FN(ksor_rne)(m, d);
-  for (int i = 0; i < nv; ++i) { d->qfrc_passive[i] = -(REAL)m->dof_damping[i] * d->qvel[i]; d->qfrc_actuator[i] = 0; }
+  for (int i = 0; i < nv; ++i) { d->qfrc_passive[i] = -(REAL)m->dof_damping[i] * d->damping_scale[i] * d->qvel[i]; d->qfrc_actuator[i] = 0; }
   for (int u = 0; u < m->nu; ++u) {
     REAL c = d->ctrl[u];
     if (c < (REAL)m->act_lo[u]) c = (REAL)m->act_lo[u];
@@ -666,7 +667,7 @@ void FN(ksor_euler)(const KsorModel* m, Data* d) {
     /* implicit in joint damping: (M + dt diag(damping)) qacc' = qfrc_smooth + qfrc_constraint */
     REAL H[KSOR_MAXV * KSOR_MAXV], Lh[KSOR_MAXV * KSOR_MAXV], rhs[KSOR_MAXV];
     for (int i = 0; i < nv * nv; ++i) H[i] = d->M[i];
-    for (int i = 0; i < nv; ++i) H[i * nv + i] += dt * (REAL)m->dof_damping[i];
+    for (int i = 0; i < nv; ++i) H[i * nv + i] += dt * (REAL)m->dof_damping[i] * d->damping_scale[i];
     for (int i = 0; i < nv; ++i) rhs[i] = d->qfrc_smooth[i] + d->qfrc_constraint[i];
     chol(Lh, H, nv);
     chol_solve(qacc, Lh, rhs, nv);

@@ -102,12 +102,13 @@ def test_torque_driven_trajectories(setup, steps, tol):
     np.testing.assert_allclose(buf["time"].cpu().numpy(), steps * m.dt, rtol=1e-5)
 
 
-def _oracle_control_steps(m, qpos, qvel, actions, kp, kd, clip, S, latency, friction, mass_scale, period=1):
+def _oracle_control_steps(m, qpos, qvel, actions, kp, kd, clip, S, latency, friction, mass_scale, period=1, arm=None, damp=None):
     """Python composition of the oracle's pieces: engine.py:287-320 + actuators.py:198-217 + the C step."""
     orc = Oracle(m.arrays())
     N = qpos.shape[0]
     rq, rv = (7, 6) if m.has_free_root else (0, 0)
-    datas = [orc.data(qpos[e], qvel[e], friction=friction[e], mass_scale=mass_scale[e]) for e in range(N)]
+    datas = [orc.data(qpos[e], qvel[e], friction=friction[e], mass_scale=mass_scale[e],
+                      armature_scale=None if arm is None else arm[e], damping_scale=None if damp is None else damp[e]) for e in range(N)]
     last = np.zeros((N, m.nu))
     for action in actions:
         for e, d in enumerate(datas):
@@ -139,8 +140,12 @@ def test_position_controlled_steps(name, S, T, period):
     clip = np.where(rng.random(m.nu) < 0.5, 40.0, np.inf)
     latency = rng.uniform(0.0, 1.5, N)
     fr, ms = rng.uniform(0.4, 1.2, N), rng.uniform(0.9, 1.1, (N, m.nb))
-    datas = _oracle_control_steps(m, qpos, qvel, actions, kp, kd, clip, S, latency, fr, ms, period)
+    # per-env armature and damping factors (ArmatureRandomizer, JointDampingRandomizer) on the implicit models
+    arm = rng.uniform(0.8, 1.2, (N, m.nv)) if "implicit" in name else None
+    damp = rng.uniform(0.5, 1.5, (N, m.nv)) if "implicit" in name else None
+    datas = _oracle_control_steps(m, qpos, qvel, actions, kp, kd, clip, S, latency, fr, ms, period, arm, damp)
     buf = dict(qpos=t32(qpos), qvel=t32(qvel), qacc_warmstart=zeros(N, m.nv), time=zeros(N), last_ctrl=zeros(N, m.nu),
+               armature_scale=None if arm is None else t32(arm), damping_scale=None if damp is None else t32(damp),
                latency=t32(latency), kp=t32(kp), kd=t32(kd), ctrl_clip=t32(clip), friction=t32(fr), mass_scale=t32(ms),
                ctrl_out=zeros(N, m.nu), xpos=zeros(N, m.nb * 3), xquat=zeros(N, m.nb * 4), qacc=zeros(N, m.nv))
     for k in range(T):

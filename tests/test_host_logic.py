@@ -212,3 +212,23 @@ def test_feet_force_observations_read_the_contact_force_rows():
     idx = [d.obs[k].index for k in range(d.obs_dim)]
     assert idx == [66, 67, 68, 36, 37, 38, 69, 70, 71, 39, 40, 41] and used == {T.SRC_CFRC_EXT}
     assert all(d.obs[k].kind == T.OBS_COPY and d.obs[k].src == T.SRC_CFRC_EXT for k in range(d.obs_dim))
+
+
+def test_joint_randomizers_leave_the_floating_base_alone():
+    import torch
+    from ksim_amd import randomization as rnd
+
+    m = km.kbot_scale_model()
+    gen = torch.Generator().manual_seed(0)
+    out = rnd.get_physics_randomizers(m, {"a": rnd.ArmatureRandomizer(0.9, 1.1), "d": rnd.JointDampingRandomizer(0.5, 2.0),
+                                          "m": rnd.MassMultiplicationRandomizer.from_body_name(m, m.body_names[2], 0.5, 0.6)}, 64, gen)
+    a, d, ms = out["armature_scale"], out["damping_scale"], out["mass_scale"]
+    assert tuple(a.shape) == (64, m.nv) and (a[:, :6] == 1).all() and (d[:, :6] == 1).all()
+    assert ((a[:, 6:] >= 0.9) & (a[:, 6:] <= 1.1)).all() and ((d[:, 6:] >= 0.5) & (d[:, 6:] <= 2.0)).all() and d[:, 6:].std() > 0.2
+    assert (ms[:, [0, 1, 3]] == 1).all() and ((ms[:, 2] >= 0.5) & (ms[:, 2] <= 0.6)).all()
+    add = rnd.MassAdditionRandomizer(body_id=1, scale_lower=1.0, scale_upper=1.0)(m, 4, gen)["mass_scale"]
+    assert torch.allclose(add[:, 1], torch.full((4,), (float(m.body_mass[1]) + 1.0) / float(m.body_mass[1])))
+    with pytest.raises(ValueError, match="duplicate"):
+        rnd.get_physics_randomizers(m, {"a": rnd.MassMultiplicationRandomizer(body_id=1), "b": rnd.AllBodiesMassMultiplicationRandomizer()}, 4, gen)
+    with pytest.raises(ValueError, match="not found"):
+        rnd.MassMultiplicationRandomizer.from_body_name(m, "nope")
