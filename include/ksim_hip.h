@@ -400,11 +400,17 @@ int ks_terminate_reset(const KsTerms* terms, ks_stream_t stream, const KsTermina
  * backward, switch; angular = target speed, flip, zero, switch. */
 #define KS_MAX_COMMANDS 8
 #define KS_COMMAND_DRAWS 8
-enum { KS_CMD_CONST = 0, KS_CMD_LINEAR_VELOCITY = 1, KS_CMD_ANGULAR_VELOCITY = 2 };
+#define KS_MAX_VECTOR_COMMAND 6
+enum { KS_CMD_CONST = 0, KS_CMD_LINEAR_VELOCITY = 1, KS_CMD_ANGULAR_VELOCITY = 2,
+       /* FloatVectorCommand / IntVectorCommand (commands.py:97-170): `dim` <= KS_MAX_VECTOR_COMMAND scalars, each uniform in
+          [lo, hi] (integers: lo..hi inclusive), all zero with probability zero_prob; redrawn at an episode start and with
+          probability switch_prob per step, otherwise kept.  Draws: u0 switch, u1 zero, u2.. one per scalar. */
+       KS_CMD_FLOAT_VECTOR = 3, KS_CMD_INT_VECTOR = 4 };
 typedef struct KsCommandDesc {
   int32_t kind, index, dim;    /* offset and length inside the command vector */
   float min_vel, max_vel, max_yaw, zero_prob, backward_prob, switch_prob; /* scales already evaluated at the curriculum level */
   float ctrl_dt, linear_accel, angular_accel;
+  float lo[KS_MAX_VECTOR_COMMAND], hi[KS_MAX_VECTOR_COMMAND]; /* vector commands: the ranges */
 } KsCommandDesc;
 typedef struct KsCommandIO {
   int64_t N;

@@ -118,13 +118,15 @@ class KsGruDesc(ctypes.Structure):
 
 
 KS_MAX_COMMANDS, KS_COMMAND_DRAWS = 8, 8
-CMD_CONST, CMD_LINEAR_VELOCITY, CMD_ANGULAR_VELOCITY = range(3)
+KS_MAX_VECTOR_COMMAND = 6
+CMD_CONST, CMD_LINEAR_VELOCITY, CMD_ANGULAR_VELOCITY, CMD_FLOAT_VECTOR, CMD_INT_VECTOR = range(5)
 
 
 class KsCommandDesc(ctypes.Structure):
     _fields_ = [("kind", c_int32), ("index", c_int32), ("dim", c_int32), ("min_vel", c_float), ("max_vel", c_float),
                 ("max_yaw", c_float), ("zero_prob", c_float), ("backward_prob", c_float), ("switch_prob", c_float),
-                ("ctrl_dt", c_float), ("linear_accel", c_float), ("angular_accel", c_float)]
+                ("ctrl_dt", c_float), ("linear_accel", c_float), ("angular_accel", c_float),
+                ("lo", c_float * KS_MAX_VECTOR_COMMAND), ("hi", c_float * KS_MAX_VECTOR_COMMAND)]
 
 
 class KsCommandIO(ctypes.Structure):

@@ -90,6 +90,33 @@ class ConstantCommand(Command):
         return d
 
 
+@dataclass(frozen=True)
+class FloatVectorCommand(Command):  # commands.py:97-133
+    ranges: tuple = ()
+    switch_prob: float = 0.0
+    zero_prob: float = 0.0
+    _kind = T.CMD_FLOAT_VECTOR
+
+    def __post_init__(self):
+        if not 1 <= len(self.ranges) <= T.KS_MAX_VECTOR_COMMAND:
+            raise ValueError(f"a vector command has 1..{T.KS_MAX_VECTOR_COMMAND} scalars")
+
+    def dim(self):
+        return len(self.ranges)
+
+    def desc(self, level):
+        d = T.KsCommandDesc()
+        d.kind, d.dim, d.switch_prob, d.zero_prob = self._kind, len(self.ranges), float(self.switch_prob), float(self.zero_prob)
+        for j, (lo, hi) in enumerate(self.ranges):
+            d.lo[j], d.hi[j] = float(lo), float(hi)
+        return d
+
+
+@dataclass(frozen=True)
+class IntVectorCommand(FloatVectorCommand):  # commands.py:136-170: integers lo..hi inclusive, stored as floats
+    _kind = T.CMD_INT_VECTOR
+
+
 class CommandSet:
     def __init__(self, commands: Mapping[str, Command]):
         if len(commands) > T.KS_MAX_COMMANDS:
@@ -113,7 +140,7 @@ class CommandSet:
         """Advances every env's commands in place; `record` (N, command_dim) receives the incoming values."""
         N = command.shape[0]
         _lib.require_cuda(command, qpos, qvel, record, uniform, dtype=torch.float32)
-        if tuple(command.shape) != (N, self.command_dim) or qpos.shape[0] != N or qvel.shape[0] != N:
+        if qpos.dim() != 2 or qvel.dim() != 2 or tuple(command.shape) != (N, self.command_dim) or qpos.shape[0] != N or qvel.shape[0] != N:
             raise _lib.KsError(f"command must be (N, {self.command_dim}) and the state must have N rows")
         if record is not None and tuple(record.shape) != tuple(command.shape):
             raise _lib.KsError("record must have the command's shape")

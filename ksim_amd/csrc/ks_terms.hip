@@ -576,6 +576,16 @@ __global__ __launch_bounds__(256) void command_kernel(KsCommandIO io) {
       yaw += fminf(fmaxf(ty - yaw, -c.angular_accel), c.angular_accel) * c.ctrl_dt;
     }
     cmd[0] = vel; cmd[1] = yaw; cmd[2] = vel * cosf(yaw); cmd[3] = vel * sinf(yaw); cmd[4] = tv; cmd[5] = ty;
+  } else if (c.kind == KS_CMD_FLOAT_VECTOR || c.kind == KS_CMD_INT_VECTOR) {
+    if (fresh || u[0] < c.switch_prob) {
+      const bool zero = u[1] < c.zero_prob;
+      for (int j = 0; j < c.dim; ++j) {
+        float val;
+        if (c.kind == KS_CMD_INT_VECTOR) val = fminf(floorf(c.lo[j] + u[2 + j] * (c.hi[j] + 1.f - c.lo[j])), c.hi[j]);
+        else val = c.lo[j] + u[2 + j] * (c.hi[j] - c.lo[j]);
+        cmd[j] = zero ? 0.f : val;
+      }
+    }
   } else {
     float vel = cmd[0], tv = cmd[1];
     const bool redraw = fresh || u[3] < c.switch_prob;
@@ -815,9 +825,11 @@ extern "C" int ks_commands(ks_stream_t stream, const KsCommandIO* io) {
   for (int k = 0; k < io->n_commands; ++k) {
     const KsCommandDesc& c = io->commands[k];
     const int need = c.kind == KS_CMD_LINEAR_VELOCITY ? 6 : (c.kind == KS_CMD_ANGULAR_VELOCITY ? 2 : c.dim);
-    if (c.kind < KS_CMD_CONST || c.kind > KS_CMD_ANGULAR_VELOCITY) return fail(KS_EINVAL, "ks_commands: command %d: bad kind", k);
+    if (c.kind < KS_CMD_CONST || c.kind > KS_CMD_INT_VECTOR) return fail(KS_EINVAL, "ks_commands: command %d: bad kind", k);
+    if (c.kind >= KS_CMD_FLOAT_VECTOR && c.dim > KS_MAX_VECTOR_COMMAND) return fail(KS_ELIMIT, "ks_commands: command %d: %d scalars (at most %d)", k, c.dim, KS_MAX_VECTOR_COMMAND);
     if (c.dim != need || c.dim < 1 || c.index < 0 || c.index + c.dim > io->command_dim) return fail(KS_EINVAL, "ks_commands: command %d: [%d,%d) outside the %d-wide command vector or of the wrong length", k, c.index, c.index + c.dim, io->command_dim);
-    if (c.kind != KS_CMD_CONST && (!io->qpos || !io->qvel || io->nq < 7 || io->nv < 6)) return fail(KS_EINVAL, "ks_commands: velocity commands read the state of a floating base");
+    if ((c.kind == KS_CMD_LINEAR_VELOCITY || c.kind == KS_CMD_ANGULAR_VELOCITY) && (!io->qpos || !io->qvel || io->nq < 7 || io->nv < 6))
+      return fail(KS_EINVAL, "ks_commands: velocity commands read the state of a floating base");
   }
   const int64_t n = io->N * io->n_commands, grid = (n + 255) / 256;
   if (grid > 0x7fffffff) return fail(KS_ELIMIT, "ks_commands: too many elements");

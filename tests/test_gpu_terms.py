@@ -592,3 +592,33 @@ def test_velocity_commands_against_oracle():
     assert torch.equal(a, b) and (a[:, 7].abs() <= 2.5).all() and (a[:, 10].abs() <= 1.0).all() and a[:, 7].std() > 0.1
     with pytest.raises(Exception, match="uniform"):
         cs.update(a, t32(qpos), t32(qvel), uniform=t32(u[:, :2]))
+
+
+def test_vector_commands():
+    """FloatVectorCommand / IntVectorCommand: the properties the reference's own tests check (shape, bounds, a command
+    that never switches stays what it was, reference tests/test_commands.py:64-96) and the draw arithmetic."""
+    from ksim_amd import _lib_terms as T
+    from ksim_amd.commands import CommandSet, FloatVectorCommand, IntVectorCommand
+
+    N = 500
+    cs = CommandSet({"f": FloatVectorCommand(ranges=((0.0, 2.0), (-1.0, 1.0))), "i": IntVectorCommand(ranges=((2, 5),), switch_prob=0.3, zero_prob=0.1)})
+    assert cs.command_dim == 3
+    q, v = torch.zeros(N, 7, device=DEV), torch.zeros(N, 6, device=DEV)
+    cmd = cs.initial(N, DEV)
+    cs.update(cmd, q, v, all_fresh=True, seed=1, step=0)
+    first = cmd.clone()
+    assert ((cmd[:, 0] >= 0) & (cmd[:, 0] <= 2) & (cmd[:, 1] >= -1) & (cmd[:, 1] <= 1)).all() and cmd[:, 0].std() > 0.3
+    ints = cmd[:, 2]
+    assert (ints == ints.round()).all() and set(ints.unique().tolist()) <= {0.0, 2.0, 3.0, 4.0, 5.0} and (ints == 5).any() and (ints == 2).any()
+    for k in range(5):
+        cs.update(cmd, q, v, seed=1, step=1 + k)
+    assert torch.equal(cmd[:, :2], first[:, :2])          # switch_prob 0: unchanged
+    assert (cmd[:, 2] != first[:, 2]).float().mean() > 0.3  # switch_prob 0.3 over five steps
+    # explicit draws: u0 switch, u1 zero, u2.. values
+    u = torch.zeros(N, 2, T.KS_COMMAND_DRAWS, device=DEV)
+    u[:, 1, 0] = 0.2; u[:, 1, 1] = 0.5; u[:, 1, 2] = 0.999
+    u[0, 1, 1] = 0.05  # env 0 draws the zero command
+    cs.update(cmd, q, v, uniform=u)
+    assert (cmd[1:, 2] == 5).all() and cmd[0, 2] == 0 and torch.equal(cmd[:, :2], first[:, :2])
+    with pytest.raises(ValueError):
+        FloatVectorCommand(ranges=())
