@@ -196,7 +196,11 @@ typedef struct KsEventDesc {
  * no bias, model friction, mass scale 1.  Noise arrays are explicit pre-sampled draws,
  * (substeps, N, nu), so that results can be compared on identical seeded inputs.
  */
-enum { KS_ACT_TORQUE = 0, KS_ACT_POSITION = 1 }; /* actuators.py:70-87 / 98-238 */
+enum { KS_ACT_TORQUE = 0, KS_ACT_POSITION = 1, /* actuators.py:70-87 / 98-238 */
+       KS_ACT_POSITION_VELOCITY = 2 /* actuators.py:241-293: the action is (position targets, velocity targets), 2 nu wide;
+                                       tau = kp (target_pos - q) + kd (target_vel - qd), noise, clipped.  action, last_ctrl,
+                                       drop and action_noise are then 2 nu wide (the second half of action_noise is the
+                                       velocity-target noise) */ };
 
 typedef struct KsStepIO {
   int64_t N;
@@ -332,6 +336,8 @@ typedef struct KsTermsDesc {
   int32_t obs_dim, n_terms, command_dim, random_heading;
   int32_t ns;        /* contact spheres of the model (width of KS_SRC_CONTACT_DIST) */
   int32_t carry_dim; /* floats of observation carry per env (0: no stateful observation) */
+  int32_t action_dim; /* width of the action vector = of last_ctrl and of KS_SRC_LAST_ACTION; 0 means nu
+                         (2 nu for position-velocity actuators) */
   int32_t nonfinite_terminates; /* 1: an env whose qpos/qvel is not finite counts as failed (done, no success);
                                    the reference has no such guard and would carry the NaNs forever */
   KsObsElem obs[KS_MAX_OBS];

@@ -7,7 +7,7 @@ from ctypes import POINTER, c_double, c_float, c_int32, c_int64, c_void_p
 import numpy as np
 
 MAXB, MAXQ, MAXV, MAXU, MAXS = 32, 40, 32, 32, 16
-KS_ACT_TORQUE, KS_ACT_POSITION = 0, 1
+KS_ACT_TORQUE, KS_ACT_POSITION, KS_ACT_POSITION_VELOCITY = 0, 1, 2
 
 
 class KsModelDesc(ctypes.Structure):

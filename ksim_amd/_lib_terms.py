@@ -30,7 +30,7 @@ class KsTermDesc(ctypes.Structure):
 class KsTermsDesc(ctypes.Structure):
     _fields_ = [("nq", c_int32), ("nv", c_int32), ("nu", c_int32), ("nb", c_int32), ("obs_dim", c_int32),
                 ("n_terms", c_int32), ("command_dim", c_int32), ("random_heading", c_int32),
-                ("ns", c_int32), ("carry_dim", c_int32), ("nonfinite_terminates", c_int32),
+                ("ns", c_int32), ("carry_dim", c_int32), ("action_dim", c_int32), ("nonfinite_terminates", c_int32),
                 ("obs", KsObsElem * KS_MAX_OBS), ("terms", KsTermDesc * KS_MAX_TERMS),
                 ("reset_base", c_float * KS_MAX_QPOS), ("reset_mag", c_float * KS_MAX_QPOS),
                 ("reset_lo", c_float * KS_MAX_QPOS), ("reset_hi", c_float * KS_MAX_QPOS),

@@ -5,13 +5,17 @@ from dataclasses import dataclass, field
 
 import numpy as np
 
-from ._lib_dyn import KS_ACT_POSITION, KS_ACT_TORQUE
+from ._lib_dyn import KS_ACT_POSITION, KS_ACT_POSITION_VELOCITY, KS_ACT_TORQUE
 from .noise import Noise, RandomVariable
 
 
 @dataclass(frozen=True, eq=False)
 class Actuators:
     kind: int = KS_ACT_TORQUE
+
+    def action_dim(self, nu: int) -> int:
+        """Width of the action vector (and of `PhysicsState.last_ctrl`) for a model with `nu` actuators."""
+        return nu
 
 
 @dataclass(frozen=True, eq=False)
@@ -72,3 +76,15 @@ class PositionActuators(Actuators):  # actuators.py:98-238
             "torque_limit_scale": rv(self.torque_limit_scale).sample((num_envs,), gen)
             if self.torque_limit_scale is not None else ones(num_envs),
         }
+
+
+@dataclass(frozen=True, eq=False)
+class PositionVelocityActuator(PositionActuators):  # actuators.py:241-293
+    """PD on position and velocity targets: the action is (position targets, velocity targets), 2 nu wide, and
+    tau = kp (target_pos - q) + kd (target_vel - qd); `action_noise` acts on the position half, `vel_action_noise` on the
+    velocity half."""
+    vel_action_noise: Noise | None = None
+    kind: int = KS_ACT_POSITION_VELOCITY
+
+    def action_dim(self, nu: int) -> int:
+        return 2 * nu

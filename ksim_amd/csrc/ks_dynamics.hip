@@ -321,12 +321,14 @@ void step_kernel(StepArgs a) {
       const int u = lane;
       // the actuator inputs of this control step are read again at every actuator update (they stay in the caches):
       // held in registers they would be live across the solver of every substep
-      const int64_t eu = env * nu + lane;
-      const float u_last = a.last_ctrl[eu], u_act = a.action[eu];
-      const bool u_drop = a.drop && a.drop[eu];
+      const bool posvel = a.actuator_type == KS_ACT_POSITION_VELOCITY;
+      const int na = posvel ? 2 * nu : nu;  // width of the action vector
+      const int64_t ea = env * na + lane, eu = env * nu + lane;
+      const float u_last = a.last_ctrl[ea], u_act = a.action[ea];
+      const bool u_drop = a.drop && a.drop[ea];
       const float u_zero = a.zero_offset ? a.zero_offset[eu] : 0.f;
       float u_kp = 0.f, u_kd = 0.f, u_lim = 0.f, u_abias = 0.f, u_tbias = 0.f;
-      if (a.actuator_type == KS_ACT_POSITION) {
+      if (a.actuator_type != KS_ACT_TORQUE) {
         u_kp = a.kp[lane] * (a.kp_scale ? a.kp_scale[env] : 1.f);
         u_kd = a.kd[lane] * (a.kd_scale ? a.kd_scale[env] : 1.f);
         u_lim = a.ctrl_clip[lane] * (a.torque_limit_scale ? a.torque_limit_scale[env] : 1.f);
@@ -336,14 +338,20 @@ void step_kernel(StepArgs a) {
       float prct = (float)sub - latency;
       prct = fminf(fmaxf(prct, 0.f), 1.f);
       const float c = u_drop ? u_last : u_last * (1.0f - prct) + u_act * prct;
-      const int64_t su = ((int64_t)sub * a.N + env) * nu + u;
+      const int64_t su = ((int64_t)sub * a.N + env) * nu + u, sa = ((int64_t)sub * a.N + env) * na + u;
       float t;
       if (a.actuator_type == KS_ACT_TORQUE) {
         t = c + (a.torque_noise ? a.torque_noise[su] : 0.f);
       } else {
-        const float target = c * a.action_scale + (a.action_noise ? a.action_noise[su] : 0.f) + u_abias;
+        float target_vel = 0.f;
+        if (posvel) {  // the velocity targets ride in the second half of the action vector
+          const float v_last = a.last_ctrl[ea + nu], v_act = a.action[ea + nu];
+          const bool v_drop = a.drop && a.drop[ea + nu];
+          target_vel = (v_drop ? v_last : v_last * (1.0f - prct) + v_act * prct) + (a.action_noise ? a.action_noise[sa + nu] : 0.f);
+        }
+        const float target = c * a.action_scale + (a.action_noise ? a.action_noise[sa] : 0.f) + u_abias;
         const float q = l.qpos[rq + u] - u_zero;
-        t = u_kp * (target - q) + u_kd * (0.f - l.qvel[rv + u]);
+        t = u_kp * (target - q) + u_kd * (target_vel - l.qvel[rv + u]);
         t = t + (a.torque_noise ? a.torque_noise[su] : 0.f) + u_tbias;
         t = fminf(fmaxf(t, -u_lim), u_lim);
       }
@@ -994,7 +1002,10 @@ void step_kernel(StepArgs a) {
       for (int k = 0; k < nsub; ++k) time += m.dt;
       a.time[env] = time;
     }
-    if (a.last_ctrl && lane < nu) a.last_ctrl[env * nu + lane] = a.action[env * nu + lane];
+    if (a.last_ctrl) {
+      const int na = a.actuator_type == KS_ACT_POSITION_VELOCITY ? 2 * nu : nu;
+      for (int i = lane; i < na; i += 64) a.last_ctrl[env * na + i] = a.action[env * na + i];
+    }
   }
   if (a.qacc_warmstart && lane < nv) a.qacc_warmstart[env * nv + lane] = l.warm[lane];
   if (a.ctrl_out) for (int i = lane; i < nu; i += 64) a.ctrl_out[env * nu + i] = l.tau[i];
@@ -1185,11 +1196,11 @@ static int launch_step(const KsModel* km, ks_stream_t stream, const KsStepIO* io
     if (io->substeps < 1 || io->substeps > 64) return fail(KS_EINVAL, "ks_step: substeps must be in 1..64");
     if (io->actuator_period < 1) return fail(KS_EINVAL, "ks_step: actuator_period must be >= 1");
     if (m.nu > 0 && (!io->action || !io->last_ctrl)) return fail(KS_EINVAL, "ks_step: action and last_ctrl are required");
-    if (io->actuator_type != KS_ACT_TORQUE && io->actuator_type != KS_ACT_POSITION)
+    if (io->actuator_type < KS_ACT_TORQUE || io->actuator_type > KS_ACT_POSITION_VELOCITY)
       return fail(KS_EINVAL, "ks_step: unknown actuator type %d", io->actuator_type);
-    if (io->actuator_type == KS_ACT_POSITION && m.nu > 0 && (!io->kp || !io->kd || !io->ctrl_clip))
+    if (io->actuator_type != KS_ACT_TORQUE && m.nu > 0 && (!io->kp || !io->kd || !io->ctrl_clip))
       return fail(KS_EINVAL, "ks_step: position actuators need kp, kd and ctrl_clip");
-    if (io->actuator_type == KS_ACT_POSITION && m.nu + (m.body_jtype[1] == kJntFree ? 7 : 0) > m.nq)
+    if (io->actuator_type != KS_ACT_TORQUE && m.nu + (m.body_jtype[1] == kJntFree ? 7 : 0) > m.nq)
       return fail(KS_EINVAL, "ks_step: position actuators assume one actuator per joint after the root");
     a.substeps = io->substeps; a.actuator_period = io->actuator_period; a.actuator_type = io->actuator_type;
     a.action = io->action; a.last_ctrl = io->last_ctrl; a.latency = io->latency; a.zero_offset = io->zero_offset;

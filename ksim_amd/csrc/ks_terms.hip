@@ -149,7 +149,7 @@ struct TerminateArgs {
   const float* event_reset_uniform;
   float* event_force;
   const float* contact_dist;
-  int ns;
+  int ns, na;
 };
 
 // A 256-thread workgroup owns kTermEnvs consecutive envs.  The state rows of those envs are contiguous in memory,
@@ -259,8 +259,8 @@ __global__ __launch_bounds__(256) void terminate_kernel(TerminateArgs a) {
     if (a.warm) a.warm[e0 * nv + idx] = 0.f;
   }
   if (a.last_ctrl)
-    for (int idx = tid; idx < ne * nu; idx += 256)
-      if (s_reset[idx / nu]) a.last_ctrl[e0 * nu + idx] = 0.f;
+    for (int idx = tid; idx < ne * a.na; idx += 256)
+      if (s_reset[idx / a.na]) a.last_ctrl[e0 * a.na + idx] = 0.f;
   if (a.random_heading && nq >= 7) {
     __syncthreads();  // the base orientation written above is read back by the env's own lane
     if (tid < ne && s_reset[tid]) {
@@ -615,7 +615,7 @@ extern "C" int ks_terms_create(const KsTermsDesc* d, KsTerms** out) {
   if (d->obs_dim < 0 || d->obs_dim > KS_MAX_OBS) return fail(KS_ELIMIT, "ks_terms_create: obs_dim %d > %d", d->obs_dim, KS_MAX_OBS);
   if (d->n_terms < 0 || d->n_terms > KS_MAX_TERMS) return fail(KS_ELIMIT, "ks_terms_create: %d terminations > %d", d->n_terms, KS_MAX_TERMS);
   if (d->nq < 0 || d->nq > KS_MAX_QPOS || d->nv < 0 || d->nu < 0 || d->nb < 1) return fail(KS_EINVAL, "ks_terms_create: bad sizes");
-  const int src_dim[KS_SRC_COUNT] = {d->nq, d->nv, d->nv, d->nu, d->nu, d->command_dim, 1, d->nb * 3, d->nb * 4, d->nb * 6, 0, d->ns, d->nb * 10, d->nb * 6};
+  const int src_dim[KS_SRC_COUNT] = {d->nq, d->nv, d->nv, d->nu, d->action_dim > 0 ? d->action_dim : d->nu, d->command_dim, 1, d->nb * 3, d->nb * 4, d->nb * 6, 0, d->ns, d->nb * 10, d->nb * 6};
   if (d->ns < 0 || d->carry_dim < 0) return fail(KS_EINVAL, "ks_terms_create: negative sphere count or carry size");
   for (int k = 0; k < d->obs_dim; ++k) {
     const KsObsElem& el = d->obs[k];
@@ -672,7 +672,7 @@ extern "C" int ks_observe(const KsTerms* t, ks_stream_t stream, const KsObserveI
   const KsTermsDesc& d = t->host;
   if (io->N < 0) return fail(KS_EINVAL, "ks_observe: negative env count");
   if (io->N == 0 || d.obs_dim == 0) return KS_OK;
-  const int src_dim[KS_SRC_COUNT] = {d.nq, d.nv, d.nv, d.nu, d.nu, d.command_dim, 1, d.nb * 3, d.nb * 4, d.nb * 6, 0, d.ns, d.nb * 10, d.nb * 6};
+  const int src_dim[KS_SRC_COUNT] = {d.nq, d.nv, d.nv, d.nu, d.action_dim > 0 ? d.action_dim : d.nu, d.command_dim, 1, d.nb * 3, d.nb * 4, d.nb * 6, 0, d.ns, d.nb * 10, d.nb * 6};
   if (d.carry_dim > 0 && !io->carry) return fail(KS_EINVAL, "ks_observe: the stateful observations need a carry buffer");
   ObserveArgs a;
   std::memset(&a, 0, sizeof(a));
@@ -715,7 +715,7 @@ extern "C" int ks_terminate_reset(const KsTerms* t, ks_stream_t stream, const Ks
   a.random_heading = d.random_heading; a.nonfinite_terminates = d.nonfinite_terminates;
   if (io->n_events < 0 || io->n_events > KS_MAX_EVENTS) return fail(KS_ELIMIT, "ks_terminate_reset: %d events (0..%d)", io->n_events, KS_MAX_EVENTS);
   if (io->n_events > 0 && !io->event_state) return fail(KS_EINVAL, "ks_terminate_reset: events need event_state");
-  a.contact_dist = io->contact_dist; a.ns = d.ns;
+  a.contact_dist = io->contact_dist; a.ns = d.ns; a.na = d.action_dim > 0 ? d.action_dim : d.nu;
   for (int j = 0; j < d.n_terms; ++j)
     if (d.terms[j].kind == KS_TERM_ILLEGAL_CONTACT && !io->contact_dist) return fail(KS_EINVAL, "ks_terminate_reset: termination %d reads contact_dist", j);
   a.n_events = io->n_events; a.event_state = io->event_state; a.event_reset_uniform = io->event_reset_uniform; a.event_force = io->event_force;

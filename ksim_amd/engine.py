@@ -142,7 +142,8 @@ class HipEngine(PhysicsEngine):
     def _reset_terms(self, physics_model: physics.DeviceModel) -> EnvTerms:
         key = id(physics_model)
         if key not in self._terms:
-            self._terms[key] = EnvTerms(physics_model.model, {}, {}, self.resets)
+            self._terms[key] = EnvTerms(physics_model.model, {}, {}, self.resets,
+                                        action_dim=self.actuators.action_dim(physics_model.model.nu))
         return self._terms[key]
 
     def _check(self, physics_model) -> None:
@@ -165,7 +166,7 @@ class HipEngine(PhysicsEngine):
         level = float(curriculum_level)
         lo, hi = self.data.min_action_latency_step * level, self.data.max_action_latency_step * level
         state = PhysicsState(
-            last_ctrl=z(N, m.nu), data=data, event_states=self._initial_event_states(N, gen, dev),
+            last_ctrl=z(N, self.actuators.action_dim(m.nu)), data=data, event_states=self._initial_event_states(N, gen, dev),
             actuator_state=self.actuators.get_initial_state(N, gen) if isinstance(self.actuators, PositionActuators) else None,
             action_latency=lo + (hi - lo) * torch.rand(N, generator=gen, device=dev),
             zero_offset=self.data.zero_offset.sample((N, m.nu), gen, level),
@@ -267,7 +268,7 @@ class HipEngine(PhysicsEngine):
                        action_bias=ast.get("action"), torque_bias=ast.get("torque"))
             physics.control_step(physics_model, buf, substeps=self.data.phys_steps_per_ctrl_steps,
                                  actuator_period=self.data.phys_steps_per_actuator_step,
-                                 actuator_type=act.kind, action_scale=act.action_scale, events=ev)
+                                 actuator_type=act.kind, action_scale=act.action_scale, events=ev)  # incl. position-velocity
         elif isinstance(act, TorqueActuators):
             physics.control_step(physics_model, buf, substeps=self.data.phys_steps_per_ctrl_steps,
                                  actuator_period=self.data.phys_steps_per_actuator_step, actuator_type=act.kind, events=ev)

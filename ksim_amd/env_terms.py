@@ -29,7 +29,7 @@ def _rng(seed: int, step: int, step_base: torch.Tensor | None = None) -> T.KsRng
 
 def compile_terms(model: KinematicModel, observations: Mapping[str, Observation],
                   terminations: Mapping[str, Termination], resets: Sequence[Reset], command_dim: int = 0,
-                  terminate_on_nonfinite: bool = True):
+                  terminate_on_nonfinite: bool = True, action_dim: int | None = None):
     """Host-side compilation of the task's terms into the flat tables of KsTermsDesc (no GPU involved).
 
     Returns (desc, obs_slices, sources_used, bias_std, reset_table); `desc.carry_dim` is the length of the per-env
@@ -37,6 +37,7 @@ def compile_terms(model: KinematicModel, observations: Mapping[str, Observation]
     d = T.KsTermsDesc()
     d.nq, d.nv, d.nu, d.nb, d.command_dim = model.nq, model.nv, model.nu, model.nb, int(command_dim)
     d.ns = model.ns
+    d.action_dim = model.nu if action_dim is None else int(action_dim)
     carry_at = 0
     obs_slices: dict[str, slice] = {}
     sources_used: set[int] = set()
@@ -83,14 +84,15 @@ def compile_terms(model: KinematicModel, observations: Mapping[str, Observation]
 class EnvTerms:
     def __init__(self, model: KinematicModel, observations: Mapping[str, Observation],
                  terminations: Mapping[str, Termination], resets: Sequence[Reset], command_dim: int = 0,
-                 terminate_on_nonfinite: bool = True):
+                 terminate_on_nonfinite: bool = True, action_dim: int | None = None):
         lib = _lib.load()
         torch.zeros(1, device="cuda")
         self.model, self._lib = model, lib
         self.observations, self.terminations, self.resets = dict(observations), dict(terminations), tuple(resets)
         self.command_dim = int(command_dim)
         d, self.obs_slices, self.sources_used, self.bias_std, self.reset_table = compile_terms(
-            model, self.observations, self.terminations, self.resets, self.command_dim, terminate_on_nonfinite)
+            model, self.observations, self.terminations, self.resets, self.command_dim, terminate_on_nonfinite, action_dim)
+        self.action_dim = int(d.action_dim)
         self.obs_dim, self.n_terms, self.carry_dim = int(d.obs_dim), int(d.n_terms), int(d.carry_dim)
         self._handle = ctypes.c_void_p()
         _lib.check(lib.ks_terms_create(ctypes.byref(d), ctypes.byref(self._handle)))
@@ -103,7 +105,7 @@ class EnvTerms:
         """`carry` (N, carry_dim) is advanced in place; `fresh` (N) uint8 marks the envs whose carries are initialised
         from the current state first (those that were just reset)."""
         m = self.model
-        dims = {T.SRC_QPOS: m.nq, T.SRC_QVEL: m.nv, T.SRC_QACC: m.nv, T.SRC_CTRL: m.nu, T.SRC_LAST_ACTION: m.nu,
+        dims = {T.SRC_QPOS: m.nq, T.SRC_QVEL: m.nv, T.SRC_QACC: m.nv, T.SRC_CTRL: m.nu, T.SRC_LAST_ACTION: self.action_dim,
                 T.SRC_COMMAND: self.command_dim, T.SRC_TIME: 1, T.SRC_XPOS: m.nb * 3, T.SRC_XQUAT: m.nb * 4,
                 T.SRC_CVEL: m.nb * 6, T.SRC_CONTACT_DIST: m.ns, T.SRC_CINERT: m.nb * 10, T.SRC_CFRC_EXT: m.nb * 6}
         io = T.KsObserveIO()
@@ -148,7 +150,7 @@ class EnvTerms:
         io.N, io.level, io.apply_reset = N, level, int(apply_reset)
         spec = [("qpos", state.get("qpos"), (N, m.nq), torch.float32), ("qvel", state.get("qvel"), (N, m.nv), torch.float32),
                 ("qacc_warmstart", state.get("qacc_warmstart"), (N, m.nv), torch.float32),
-                ("time", state.get("time"), (N,), torch.float32), ("last_ctrl", state.get("last_ctrl"), (N, m.nu), torch.float32),
+                ("time", state.get("time"), (N,), torch.float32), ("last_ctrl", state.get("last_ctrl"), (N, self.action_dim), torch.float32),
                 ("components", components, (self.n_terms, N), torch.int8), ("done", done, (N,), torch.uint8),
                 ("success", success, (N,), torch.uint8), ("traj_qpos", traj_qpos, (N, m.nq), torch.float32),
                 ("traj_qvel", traj_qvel, (N, m.nv), torch.float32), ("traj_time", traj_time, (N,), torch.float32),

@@ -304,8 +304,10 @@ class FeetContactObservation(Observation):
 class LastActionObservation(Observation):
     """The previous control step's action (PhysicsState.last_ctrl, ksim/types.py:33-43)."""
 
+    action_dim: int | None = None  # 2 nu for position-velocity actuators; None = nu
+
     def elements(self, m, command_dim):
-        return _copy(T.SRC_LAST_ACTION, 0, m.nu)
+        return _copy(T.SRC_LAST_ACTION, 0, m.nu if self.action_dim is None else int(self.action_dim))
 
 
 @dataclass(frozen=True)

@@ -59,13 +59,14 @@ _F32 = ("qpos", "qvel", "qacc_warmstart", "time", "last_ctrl", "action", "ctrl_i
 _I32 = ("solver_niter", "nefc")
 
 
-def _expected_shapes(m: KinematicModel, N: int, S: int) -> dict:
+def _expected_shapes(m: KinematicModel, N: int, S: int, actuator_type: int = _lib_dyn.KS_ACT_POSITION) -> dict:
     nb, nq, nv, nu, ns = m.nb, m.nq, m.nv, m.nu, m.ns
+    na = 2 * nu if actuator_type == _lib_dyn.KS_ACT_POSITION_VELOCITY else nu  # width of the action vector
     return {
-        "qpos": (N, nq), "qvel": (N, nv), "qacc_warmstart": (N, nv), "time": (N,), "last_ctrl": (N, nu),
-        "action": (N, nu), "ctrl_in": (N, nu), "latency": (N,), "zero_offset": (N, nu), "drop": (N, nu),
+        "qpos": (N, nq), "qvel": (N, nv), "qacc_warmstart": (N, nv), "time": (N,), "last_ctrl": (N, na),
+        "action": (N, na), "ctrl_in": (N, nu), "latency": (N,), "zero_offset": (N, nu), "drop": (N, na),
         "kp": (nu,), "kd": (nu,), "ctrl_clip": (nu,), "kp_scale": (N,), "kd_scale": (N,),
-        "torque_limit_scale": (N,), "action_bias": (N, nu), "torque_bias": (N, nu), "action_noise": (S, N, nu),
+        "torque_limit_scale": (N,), "action_bias": (N, nu), "torque_bias": (N, nu), "action_noise": (S, N, na),
         "torque_noise": (S, N, nu), "friction": (N,), "mass_scale": (N, nb), "env_mask": (N,), "qacc": (N, nv), "ctrl_out": (N, nu),
         "xpos": (N, nb * 3), "xquat": (N, nb * 4), "cvel": (N, nb * 6), "traj_ctrl": (N, nu),
         "traj_xpos": (N, nb * 3), "traj_xquat": (N, nb * 4), "solver_niter": (N,), "nefc": (N,),
@@ -82,7 +83,7 @@ def _make_io(dm: DeviceModel, buffers: Mapping[str, torch.Tensor | None], subste
     if qpos is None or qpos.dim() != 2:
         raise _lib.KsError("qpos (N, nq) is required")
     N = qpos.shape[0]
-    shapes = _expected_shapes(m, N, max(substeps, 1))
+    shapes = _expected_shapes(m, N, max(substeps, 1), actuator_type)
     io = _lib_dyn.KsStepIO()
     io.N, io.substeps, io.actuator_period, io.actuator_type = N, substeps, actuator_period, actuator_type
     io.action_scale = action_scale

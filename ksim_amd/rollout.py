@@ -70,7 +70,8 @@ class Rollout:
         f = lambda *s: torch.empty(*s, dtype=torch.float32, device=dev)  # noqa: E731
         b = lambda *s: torch.zeros(*s, dtype=torch.uint8, device=dev)  # noqa: E731
         self.obs, self.noisy_obs = f(Tn, N, c.terms.obs_dim), f(Tn, N, c.terms.obs_dim)
-        self.action, self.mean = f(Tn, N, m.nu), f(N, m.nu)
+        na = c.engine.actuators.action_dim(m.nu)  # 2 nu for position-velocity actuators
+        self.action, self.mean = f(Tn, N, na), f(N, na)
         self.qpos, self.qvel = f(Tn, N, m.nq), f(Tn, N, m.nv)
         self.xpos, self.xquat, self.ctrl = f(Tn, N, m.nb * 3), f(Tn, N, m.nb * 4), f(Tn, N, m.nu)
         self.done, self.success, self.timestep = b(Tn, N), b(Tn, N), f(Tn, N)
@@ -83,8 +84,8 @@ class Rollout:
         # Philox step counter of graph replays: kernels add it to the step baked into the captured launch
         self.step_base = torch.zeros(1, dtype=torch.int64, device=dev)
         self._graph = None
-        if c.actor.in_dim != c.terms.obs_dim or c.actor.out_dim != m.nu:
-            raise _lib.KsError("actor must map the observation vector to one mean per actuator")
+        if c.actor.in_dim != c.terms.obs_dim or c.actor.out_dim != na:
+            raise _lib.KsError("actor must map the observation vector to one mean per action entry")
         if c.critic is not None and (c.critic.in_dim != c.terms.obs_dim or c.critic.out_dim != 1):
             raise _lib.KsError("critic must map the observation vector to one value")
 

@@ -411,3 +411,12 @@ def angular_velocity_command(prev, qvel, u, fresh, *, max_vel, min_vel=0.0, zero
     else:
         vel = vel + float(np.clip(tv - vel, -angular_accel, angular_accel)) * ctrl_dt
     return np.array([vel, tv])
+
+
+def position_velocity_actuator_torque(action, qpos, qvel, kp, kd, ctrl_clip, pos_noise=0.0, vel_noise=0.0, torque_noise=0.0):
+    """PositionVelocityActuator.get_ctrl (ksim/actuators.py:261-293): action = (position targets, velocity targets)."""
+    n = len(qpos)
+    action = np.asarray(action, dtype=np.float64)
+    target_pos, target_vel = action[:n] + pos_noise, action[n:] + vel_noise
+    ctrl = np.asarray(kp) * (target_pos - qpos) + np.asarray(kd) * (target_vel - qvel)
+    return np.clip(ctrl + torque_noise, -np.asarray(ctrl_clip), np.asarray(ctrl_clip))

@@ -389,3 +389,47 @@ def test_force_push_event_holds_a_wrench_on_one_body():
     bad = [kev.ForcePushEvent(body_id=m.nb, **prm[0]).desc(1.0)]
     with pytest.raises(Exception, match="body"):
         physics.control_step(dm, buf, substeps=S, events=(bad, t32(left0[:1]), None, None, t32(force0[:1])))
+
+
+def test_position_velocity_actuator_steps():
+    """PositionVelocityActuator (ksim/actuators.py:241-293): a 2 nu wide action of position and velocity targets, blended
+    with the previous action under latency, with noise on both halves and dropped entries."""
+    from ksim_amd import physics
+    from ksim_amd._lib_dyn import KS_ACT_POSITION_VELOCITY
+
+    m = MODELS["kbot-implicit"]()
+    dm = physics.DeviceModel(m)
+    N, S, T = 20, 4, 3
+    nu = m.nu
+    qpos, qvel = random_states(m, N, seed=61, vel_scale=0.2, joint_range=0.3)
+    rng = np.random.default_rng(62)
+    actions = np.concatenate([rng.uniform(-0.4, 0.4, size=(T, N, nu)), rng.uniform(-1.0, 1.0, size=(T, N, nu))], axis=-1)
+    kp, kd, clip = rng.uniform(20, 150, nu), rng.uniform(1, 4, nu), np.full(nu, 45.0)
+    latency = rng.uniform(0.0, 1.5, N)
+    zero = rng.normal(size=(N, nu)) * 0.02
+    an = rng.normal(size=(T, S, N, 2 * nu)) * 0.01
+    tn = rng.normal(size=(T, S, N, nu)) * 0.1
+    drop = rng.random((T, N, 2 * nu)) < 0.1
+    orc = Oracle(m.arrays())
+    datas = [orc.data(qpos[e], qvel[e]) for e in range(N)]
+    last = np.zeros((N, 2 * nu))
+    for k in range(T):
+        for e, d in enumerate(datas):
+            for s in range(S):
+                c = oterms.latency_blend(float(s), latency[e], last[e], actions[k, e], drop[k, e])
+                d.ctrl = oterms.position_velocity_actuator_torque(c, np.array(d.qpos[7:]) - zero[e], np.array(d.qvel[6:]), kp, kd, clip,
+                                                                  pos_noise=an[k, s, e, :nu], vel_noise=an[k, s, e, nu:], torque_noise=tn[k, s, e])
+                orc.step(d)
+        last = actions[k].copy()
+    buf = dict(qpos=t32(qpos), qvel=t32(qvel), qacc_warmstart=zeros(N, m.nv), time=zeros(N), last_ctrl=zeros(N, 2 * nu),
+               latency=t32(latency), zero_offset=t32(zero), kp=t32(kp), kd=t32(kd), ctrl_clip=t32(clip), ctrl_out=zeros(N, nu))
+    for k in range(T):
+        buf.update(action=t32(actions[k]), action_noise=t32(an[k]), torque_noise=t32(tn[k]),
+                   drop=torch.from_numpy(drop[k].astype(np.uint8)).to(DEV))
+        physics.control_step(dm, buf, substeps=S, actuator_type=KS_ACT_POSITION_VELOCITY)
+    for field, ref in [("qpos", "qpos"), ("qvel", "qvel"), ("ctrl_out", "ctrl")]:
+        want = np.array([np.array(getattr(d, ref)) for d in datas])
+        assert rel_err(buf[field].cpu().numpy(), want).max() <= TEN_STEP_TOL, field
+    assert torch.equal(buf["last_ctrl"], buf["action"])
+    with pytest.raises(Exception, match="last_ctrl"):
+        physics.control_step(dm, dict(buf, last_ctrl=zeros(N, nu)), substeps=S, actuator_type=KS_ACT_POSITION_VELOCITY)

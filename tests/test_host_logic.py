@@ -232,3 +232,11 @@ def test_joint_randomizers_leave_the_floating_base_alone():
         rnd.get_physics_randomizers(m, {"a": rnd.MassMultiplicationRandomizer(body_id=1), "b": rnd.AllBodiesMassMultiplicationRandomizer()}, 4, gen)
     with pytest.raises(ValueError, match="not found"):
         rnd.MassMultiplicationRandomizer.from_body_name(m, "nope")
+
+
+def test_position_velocity_actuator_widths():
+    act = actuators.PositionVelocityActuator(kps=(10.0, 20.0), kds=(1.0, 2.0))
+    assert act.action_dim(2) == 4 and actuators.PositionActuators(kps=(1.0,), kds=(1.0,)).action_dim(1) == 1
+    m = km.kbot_scale_model()
+    d, slices, _, _, _ = compile_terms(m, {"a": ob.LastActionObservation(action_dim=2 * m.nu)}, {}, [], action_dim=2 * m.nu)
+    assert d.action_dim == 2 * m.nu and d.obs_dim == 2 * m.nu

@@ -283,3 +283,13 @@ def test_velocity_commands_hand_computed():
     np.testing.assert_allclose(a2, [0.3 - 0.5 * 0.02, -0.6])
     a3 = terms.angular_velocity_command(a2, v, [0.5, 0.6, 0.05, 0.1], False, **pa)   # switch: re-measured, zeroed target
     np.testing.assert_allclose(a3, [0.3, 0.0])
+
+
+def test_position_velocity_actuator_hand_computed():
+    tau = terms.position_velocity_actuator_torque([0.5, -0.2, 1.0, 0.0], np.array([0.1, 0.1]), np.array([0.5, -1.0]),
+                                                  kp=[10.0, 20.0], kd=[2.0, 1.0], ctrl_clip=[100.0, 5.5])
+    np.testing.assert_allclose(tau, [10 * 0.4 + 2 * 0.5, np.clip(20 * -0.3 + 1 * 1.0, -5.5, 5.5)])
+    # zero velocity targets reduce it to the position actuator
+    a = terms.position_velocity_actuator_torque([0.5, -0.2, 0.0, 0.0], np.array([0.1, 0.1]), np.array([0.5, -1.0]), [10.0, 20.0], [2.0, 1.0], [100.0, 100.0])
+    b = terms.position_actuator_torque(np.array([0.5, -0.2]), np.array([0.1, 0.1]), np.array([0.5, -1.0]), np.array([10.0, 20.0]), np.array([2.0, 1.0]), np.array([100.0, 100.0]))
+    np.testing.assert_allclose(a, b)
