@@ -260,6 +260,13 @@ typedef struct KsStepIO {
      (ArmatureRandomizer, JointDampingRandomizer, ksim/randomization.py:108-123,226-243; the root's six dofs keep 1) */
   const float* armature_scale; /* (N, nv) */
   const float* damping_scale;  /* (N, nv) */
+  /* launch order (no counterpart in the reference: its vmapped solver runs all envs in lock step).  Envs differ a lot in
+     cost (contacts, Newton iterations), and with only a few wavefronts per hardware slot the launch ends with the last heavy
+     env.  `work` returns an estimate of each env's cost in this step; ks_work_order turns it into a heaviest-first
+     permutation that the next step takes as `env_order`, so the heavy envs start first and the light ones fill the gaps.
+     Results do not depend on the order. */
+  const int32_t* env_order;    /* (N) a permutation of 0..N-1: workgroup i steps env env_order[i]; nullable = identity */
+  int32_t* work;               /* (N) nullable */
   /* events (ks_step only) */
   int32_t n_events;
   KsEventDesc events[KS_MAX_EVENTS];
@@ -270,6 +277,8 @@ typedef struct KsStepIO {
 } KsStepIO;
 
 int ks_step(const KsModel* model, ks_stream_t stream, const KsStepIO* io /*host*/);
+/* order = the envs sorted by work, heaviest first (a counting sort in one workgroup; ties in arbitrary order). */
+int ks_work_order(ks_stream_t stream, int64_t N, const int32_t* work, int32_t* order);
 int ks_forward(const KsModel* model, ks_stream_t stream, const KsStepIO* io /*host*/);
 
 /* ------------------------------------------------------------------ per-env terms

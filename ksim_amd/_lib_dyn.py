@@ -40,7 +40,7 @@ STEP_IO_POINTERS = (
     "torque_limit_scale", "action_bias", "torque_bias", "action_noise", "torque_noise", "friction", "mass_scale",
     "env_mask",
     "qacc", "ctrl_out", "xpos", "xquat", "cvel", "traj_ctrl", "traj_xpos", "traj_xquat", "solver_niter", "nefc",
-    "dbg_M", "dbg_bias", "dbg_qacc_smooth", "contact_dist", "cinert", "cfrc_ext", "armature_scale", "damping_scale",
+    "dbg_M", "dbg_bias", "dbg_qacc_smooth", "contact_dist", "cinert", "cfrc_ext", "armature_scale", "damping_scale", "env_order", "work",
 )
 
 
@@ -87,5 +87,6 @@ def bind(lib) -> None:
     lib.ks_model_lds_bytes.argtypes = [c_void_p]
     lib.ks_step.argtypes = [c_void_p, c_void_p, POINTER(KsStepIO)]
     lib.ks_forward.argtypes = [c_void_p, c_void_p, POINTER(KsStepIO)]
-    for name in ("ks_model_create", "ks_model_destroy", "ks_model_lds_bytes", "ks_step", "ks_forward"):
+    lib.ks_work_order.argtypes = [c_void_p, c_int64, c_void_p, c_void_p]
+    for name in ("ks_model_create", "ks_model_destroy", "ks_model_lds_bytes", "ks_step", "ks_forward", "ks_work_order"):
         getattr(lib, name).restype = c_int32

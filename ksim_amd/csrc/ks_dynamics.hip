@@ -247,8 +247,9 @@ void step_kernel(StepArgs a) {
   extern __shared__ __attribute__((aligned(16))) float lds_raw[];
   const DevModel& m = *a.model;
   const int lane = threadIdx.x;
-  const int64_t env = blockIdx.x;
+  const int64_t env = a.env_order ? a.env_order[blockIdx.x] : blockIdx.x;  // heaviest envs first when an order is given
   if (a.env_mask && !a.env_mask[env]) return;  // wave-uniform
+  int work = 0;  // wave-uniform cost estimate of this control step
   const int nb = m.nb, nq = m.nq, nv = m.nv, nu = m.nu, ns = m.ns, nvs = m.nvs, js = m.js;
   const Lds l = carve(lds_raw, m);
   const int rq = (nb > 1 && m.body_jtype[1] == kJntFree) ? 7 : 0;
@@ -667,6 +668,12 @@ void step_kernel(StepArgs a) {
     const unsigned long long cmask = __ballot(touching);
     const int ncon = __popcll(cmask);
     const int nefc = 4 * ncon;
+    // A launch ends with its slowest wavefront, and an env with many contacts runs several times longer than an airborne
+    // one: waves with more constraint rows get a higher issue priority on their SIMD, which shortens exactly those.
+    if (nefc >= 20) __builtin_amdgcn_s_setprio(3);
+    else if (nefc >= 12) __builtin_amdgcn_s_setprio(2);
+    else if (nefc > 0) __builtin_amdgcn_s_setprio(1);
+    else __builtin_amdgcn_s_setprio(0);
     if (touching) {
       const int c = __popcll(cmask & ((1ull << lane) - 1ull));
       l.con_body[c] = s_body;
@@ -770,6 +777,8 @@ void step_kernel(StepArgs a) {
       bool first = true;
       KS_TICK(9)
 
+      unsigned long long am_factored = 0ull;  // active set that R currently factors
+      bool have_factor = false;               // none yet: R holds the factor of M
       while (true) {
         // ---- constraint update: active set, forces, cost
         const bool active = is_row && (Jaref < 0.f);
@@ -801,9 +810,11 @@ void step_kernel(StepArgs a) {
         // lane half = row of the pair).  The accumulator tile holds, in lane c, rows {8g + 4 (lane / 32) + e} of
         // column c, which by symmetry is row c: the upper lane half hands its 16 entries to the lower one and
         // lane i < 32 ends up with row i of H in registers, as the factorisation wants it.
-        l.drow[lane] = active ? D : 0.f;
-        KS_SYNC();
-        {
+        // H depends on the iterate only through the active set: while that stays the same (the usual case once the
+        // solver closes in) the factor of the previous iteration is still the factor of H and is kept.
+        if (!have_factor || am != am_factored) {
+          l.drow[lane] = active ? D : 0.f;
+          KS_SYNC();
           f32x16 hc;
           load_mtile(hc, l.M, nvs, nv, NP, lane);
           const int col = lane & 31, half = lane >> 5;
@@ -815,6 +826,8 @@ void step_kernel(StepArgs a) {
           }
           KS_TICK(11)
           chol_tile<NP>(hc, R, myinv, lane);
+          am_factored = am;
+          have_factor = true;
         }
         const float search_all = -solve_regs<NP>(R, myinv, lane, grad);
         const float search = is_dof ? search_all : 0.f;
@@ -937,6 +950,7 @@ void step_kernel(StepArgs a) {
     } else if (a.cfrc_ext && sub == nsub - 1) {
       for (int i = lane; i < nb * 6; i += 64) a.cfrc_ext[(int64_t)env * nb * 6 + i] = 0.f;
     }
+    work += (1 + niter) * (16 + nefc);
     if (sub == nsub - 1) {  // outputs of the last substep go out here: nothing of them stays live to the end
       if (a.qacc && lane < nv) a.qacc[env * nv + lane] = qacc;
       if (a.solver_niter && lane == 0) a.solver_niter[env] = niter;
@@ -997,6 +1011,7 @@ void step_kernel(StepArgs a) {
   if (!FWD) {
     for (int i = lane; i < nq; i += 64) a.qpos[env * nq + i] = l.qpos[i];
     if (lane < nv) a.qvel[env * nv + lane] = l.qvel[lane];
+    if (a.work && lane == 0) a.work[env] = work;
     if (a.time && lane == 0) {  // dt added once per substep in fp32, like the reference's accumulation
       float time = a.time[env];
       for (int k = 0; k < nsub; ++k) time += m.dt;
@@ -1191,6 +1206,7 @@ static int launch_step(const KsModel* km, ks_stream_t stream, const KsStepIO* io
   a.dbg_M = io->dbg_M; a.dbg_bias = io->dbg_bias; a.dbg_qacc_smooth = io->dbg_qacc_smooth;
   a.contact_dist = io->contact_dist; a.cinert = io->cinert; a.cfrc_ext = io->cfrc_ext;
   a.armature_scale = io->armature_scale; a.damping_scale = io->damping_scale;
+  a.env_order = forward_only ? nullptr : io->env_order; a.work = io->work;
   a.ctrl_in = io->ctrl_in;
   if (!forward_only) {
     if (io->substeps < 1 || io->substeps > 64) return fail(KS_EINVAL, "ks_step: substeps must be in 1..64");
@@ -1253,4 +1269,47 @@ extern "C" int ks_step(const KsModel* model, ks_stream_t stream, const KsStepIO*
 
 extern "C" int ks_forward(const KsModel* model, ks_stream_t stream, const KsStepIO* io) {
   return launch_step(model, stream, io, true);
+}
+
+namespace ks {
+constexpr int kWorkBuckets = 2048;
+// Counting sort of the envs by descending work in one workgroup: histogram, suffix sums, scatter.
+__global__ __launch_bounds__(1024) void work_order_kernel(int64_t N, const int32_t* __restrict__ work, int32_t* __restrict__ order) {
+  __shared__ int hist[kWorkBuckets];
+  __shared__ int scan[kWorkBuckets];
+  const int t = threadIdx.x;
+  for (int b = t; b < kWorkBuckets; b += 1024) hist[b] = 0;
+  __syncthreads();
+  for (int64_t i = t; i < N; i += 1024) atomicAdd(&hist[min(max(work[i], 0), kWorkBuckets - 1)], 1);
+  __syncthreads();
+  // inclusive suffix sums (heaviest bucket first) by doubling
+  for (int b = t; b < kWorkBuckets; b += 1024) scan[b] = hist[b];
+  __syncthreads();
+  for (int off = 1; off < kWorkBuckets; off <<= 1) {
+    int v[kWorkBuckets / 1024];
+    for (int k = 0; k < kWorkBuckets / 1024; ++k) {
+      const int b = t + 1024 * k;
+      v[k] = scan[b] + (b + off < kWorkBuckets ? scan[b + off] : 0);
+    }
+    __syncthreads();
+    for (int k = 0; k < kWorkBuckets / 1024; ++k) scan[t + 1024 * k] = v[k];
+    __syncthreads();
+  }
+  // bucket b starts after all heavier buckets: scan[b] - hist[b]
+  for (int b = t; b < kWorkBuckets; b += 1024) hist[b] = scan[b] - hist[b];
+  __syncthreads();
+  for (int64_t i = t; i < N; i += 1024) {
+    const int pos = atomicAdd(&hist[min(max(work[i], 0), kWorkBuckets - 1)], 1);
+    order[pos] = (int32_t)i;
+  }
+}
+}  // namespace ks
+
+extern "C" int ks_work_order(ks_stream_t stream, int64_t N, const int32_t* work, int32_t* order) {
+  using namespace ks;
+  if (N < 0 || N > 0x7fffffff) return fail(KS_EINVAL, "ks_work_order: bad env count");
+  if (N == 0) return KS_OK;
+  if (!work || !order) return fail(KS_EINVAL, "ks_work_order: null argument");
+  hipLaunchKernelGGL(work_order_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, N, work, order);
+  return check_launch("ks_work_order");
 }

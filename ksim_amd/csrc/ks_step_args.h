@@ -24,6 +24,8 @@ struct StepArgs {
   int32_t *solver_niter, *nefc;
   float *dbg_M, *dbg_bias, *dbg_qacc_smooth, *contact_dist, *cinert, *cfrc_ext;
   const float *armature_scale, *damping_scale;
+  const int32_t* env_order;
+  int32_t* work;
   int n_events;
   KsEventDesc events[KS_MAX_EVENTS];
   float* event_state;

@@ -35,6 +35,8 @@ class EngineConfig:  # engine.py:48-139
     actuator_update_dt: float | None = None
     ctrl_dt: float | None = MISSING
     dt: float | None = MISSING
+    # not in the reference: launch the envs heaviest first, ordered by the previous step's cost (see KsStepIO.env_order)
+    balance_launch_order: bool = True
 
     def __post_init__(self) -> None:
         if self.dt is MISSING:
@@ -86,6 +88,7 @@ class EngineData:  # engine.py:141-168
     phys_steps_per_ctrl_steps: int
     phys_steps_per_actuator_step: int
     zero_offset: RandomVariable
+    balance_launch_order: bool = True
 
     @classmethod
     def from_config(cls, config: EngineConfig) -> "EngineData":
@@ -95,7 +98,7 @@ class EngineData:  # engine.py:141-168
                    max_action_latency_step=config.max_action_latency_step,
                    phys_steps_per_ctrl_steps=config.phys_steps_per_ctrl_steps,
                    phys_steps_per_actuator_step=config.phys_steps_per_actuator_step,
-                   zero_offset=config.zero_offset_random_variable())
+                   zero_offset=config.zero_offset_random_variable(), balance_launch_order=config.balance_launch_order)
 
 
 class PhysicsEngine(ABC):  # engine.py:171-199
@@ -222,6 +225,16 @@ class HipEngine(PhysicsEngine):
                                             cinert=d.cinert, cfrc_ext=d.cfrc_ext))
         # engine.py:217-220: qvel and qacc are zeroed after the forward pass (qvel is already zero here)
 
+    def prepare_state(self, state: PhysicsState):
+        """The (order, work) buffers of the heaviest-first launch order, made on first use; call before capturing
+        `step` into a HIP graph so that their initialisation is not part of the graph."""
+        sched = getattr(state, "_schedule", None)
+        if sched is None and self.data.balance_launch_order:
+            n, dev = state.data.qpos.shape[0], state.data.qpos.device
+            sched = (torch.arange(n, dtype=torch.int32, device=dev), torch.zeros(n, dtype=torch.int32, device=dev))
+            state._schedule = sched
+        return sched
+
     def prepare(self, device):
         """Uploads the actuator gain tables (once per device); call before capturing `step` into a HIP graph,
         where host-to-device copies are not allowed."""
@@ -258,6 +271,10 @@ class HipEngine(PhysicsEngine):
                    action_noise=noise.get("action_noise"),
                    torque_noise=noise.get("torque_noise"), traj_ctrl=record.get("ctrl"),
                    traj_xpos=record.get("xpos"), traj_xquat=record.get("xquat"))
+        # heaviest-first launch order from the previous step's cost estimates (kept on the state object)
+        sched = self.prepare_state(s)
+        if sched is not None:
+            buf.update(env_order=sched[0], work=sched[1])
         act = self.actuators
         ev = self.event_args(s, curriculum_level, event_seed, step, step_base, noise.get("event_uniform"))
         if isinstance(act, PositionActuators):
@@ -274,6 +291,8 @@ class HipEngine(PhysicsEngine):
                                  actuator_period=self.data.phys_steps_per_actuator_step, actuator_type=act.kind, events=ev)
         else:
             raise ValueError(f"Unsupported actuators: {type(act).__name__}")
+        if sched is not None:
+            physics.work_order(physics_model, sched[1], sched[0])
         return physics_state
 
 

@@ -56,7 +56,7 @@ _F32 = ("qpos", "qvel", "qacc_warmstart", "time", "last_ctrl", "action", "ctrl_i
         "kd", "ctrl_clip", "kp_scale", "kd_scale", "torque_limit_scale", "action_bias", "torque_bias", "action_noise",
         "torque_noise", "friction", "mass_scale", "qacc", "ctrl_out", "xpos", "xquat", "cvel", "dbg_M", "dbg_bias",
         "dbg_qacc_smooth", "contact_dist", "cinert", "cfrc_ext", "armature_scale", "damping_scale")
-_I32 = ("solver_niter", "nefc")
+_I32 = ("solver_niter", "nefc", "env_order", "work")
 
 
 def _expected_shapes(m: KinematicModel, N: int, S: int, actuator_type: int = _lib_dyn.KS_ACT_POSITION) -> dict:
@@ -71,7 +71,7 @@ def _expected_shapes(m: KinematicModel, N: int, S: int, actuator_type: int = _li
         "xpos": (N, nb * 3), "xquat": (N, nb * 4), "cvel": (N, nb * 6), "traj_ctrl": (N, nu),
         "traj_xpos": (N, nb * 3), "traj_xquat": (N, nb * 4), "solver_niter": (N,), "nefc": (N,),
         "dbg_M": (N, nv * nv), "dbg_bias": (N, nv), "dbg_qacc_smooth": (N, nv), "contact_dist": (N, ns),
-        "cinert": (N, nb * 10), "cfrc_ext": (N, nb * 6), "armature_scale": (N, nv), "damping_scale": (N, nv),
+        "cinert": (N, nb * 10), "cfrc_ext": (N, nb * 6), "armature_scale": (N, nv), "damping_scale": (N, nv), "env_order": (N,), "work": (N,),
     }
 
 
@@ -136,6 +136,16 @@ def control_step(dm: DeviceModel, buffers: Mapping[str, torch.Tensor | None], *,
         if rng is not None:
             io.event_rng = rng
     _lib.check(dm._lib.ks_step(dm.handle, _lib.current_stream(), ctypes.byref(io)))
+
+
+def work_order(dm: DeviceModel, work: torch.Tensor, order: torch.Tensor) -> torch.Tensor:
+    """`order` <- the envs sorted by `work` (the step kernel's cost estimate), heaviest first: the launch order of the
+    next control step."""
+    _lib.require_cuda(work, order, dtype=torch.int32)
+    if work.dim() != 1 or tuple(order.shape) != tuple(work.shape):
+        raise _lib.KsError("work and order must be (N,) int32")
+    _lib.check(dm._lib.ks_work_order(_lib.current_stream(), work.shape[0], work.data_ptr(), order.data_ptr()))
+    return order
 
 
 def forward(dm: DeviceModel, buffers: Mapping[str, torch.Tensor | None]) -> None:

@@ -181,6 +181,7 @@ class Rollout:
     def _prepare_env(self, env: RolloutEnvState) -> None:
         """Carry buffers of an env state seen for the first time (never inside a graph capture: `_unroll_graph`
         calls this before it starts capturing)."""
+        self.c.engine.prepare_state(env.physics_state)
         if self.c.terms.carry_dim and env.obs_carry is None:
             env.obs_carry = torch.zeros(self.N, self.c.terms.carry_dim, dtype=torch.float32, device=self.done.device)
             self.reset_mask.fill_(1)  # every env starts an episode: the first observation initialises all carries

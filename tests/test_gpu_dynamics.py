@@ -433,3 +433,35 @@ def test_position_velocity_actuator_steps():
     assert torch.equal(buf["last_ctrl"], buf["action"])
     with pytest.raises(Exception, match="last_ctrl"):
         physics.control_step(dm, dict(buf, last_ctrl=zeros(N, nu)), substeps=S, actuator_type=KS_ACT_POSITION_VELOCITY)
+
+
+def test_launch_order_does_not_change_results_and_sorts_heaviest_first():
+    """Stepping the envs in a heaviest-first order gives the same bits as the natural order; the order kernel sorts."""
+    from ksim_amd import physics
+
+    m = MODELS["kbot-implicit"]()
+    dm = physics.DeviceModel(m)
+    N, S = 300, 4
+    qpos, qvel = random_states(m, N, seed=71, vel_scale=0.2, joint_range=0.3)
+    rng = np.random.default_rng(72)
+    kp, kd, clip = rng.uniform(20, 150, m.nu), rng.uniform(1, 3, m.nu), np.full(m.nu, 40.0)
+    act = rng.uniform(-0.3, 0.3, size=(N, m.nu))
+    def run(order):
+        buf = dict(qpos=t32(qpos), qvel=t32(qvel), qacc_warmstart=zeros(N, m.nv), time=zeros(N), last_ctrl=zeros(N, m.nu),
+                   action=t32(act), kp=t32(kp), kd=t32(kd), ctrl_clip=t32(clip), work=zeros(N, dtype=torch.int32),
+                   nefc=zeros(N, dtype=torch.int32), solver_niter=zeros(N, dtype=torch.int32), env_order=order)
+        for _ in range(3):
+            physics.control_step(dm, buf, substeps=S)
+        return buf
+    a = run(None)
+    work = a["work"]
+    assert (work >= 4 * 16).all() and work.max() > work.min()          # airborne envs cost the floor, contacts more
+    order = torch.empty(N, dtype=torch.int32, device=DEV)
+    physics.work_order(dm, work, order)
+    o = order.cpu().numpy(); w = work.cpu().numpy()
+    assert sorted(o.tolist()) == list(range(N)) and (np.diff(w[o]) <= 0).all()
+    b = run(order)
+    for k in ("qpos", "qvel", "qacc_warmstart", "work", "nefc", "solver_niter"):
+        assert torch.equal(a[k], b[k]), k
+    rev = torch.from_numpy(np.ascontiguousarray(o[::-1])).to(DEV)
+    assert torch.equal(run(rev)["qpos"], a["qpos"])
