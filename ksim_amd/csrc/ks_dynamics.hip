@@ -853,19 +853,27 @@ void step_kernel(StepArgs a) {
         // With at most 16 constraint rows the three sums of a cost evaluation share one reduction: the 16-lane
         // groups 0, 1, 2 hold copies of the rows with the constant, linear and quadratic coefficient, and one
         // DPP reduction within the groups yields all three totals.
-        const bool packed = nefc <= 16;
-        float pk_j = 0.f, pk_jv = 0.f, pk_q = 0.f;
+        // Rows 16..31 ride along as a second copy in the same lanes, so up to 32 rows need no more reduction steps.
+        const bool packed = nefc <= 32, two = nefc > 16;
+        float pk_j = 0.f, pk_jv = 0.f, pk_q = 0.f, pk_j2 = 0.f, pk_jv2 = 0.f, pk_q2 = 0.f;
         if (packed) {
           const int r = lane & 15, grp = lane >> 4;
           pk_j = __shfl(Jaref, r);
           pk_jv = __shfl(jv, r);
           const float c0 = __shfl(q0r, r), c1 = __shfl(q1r, r), c2 = __shfl(q2r, r);
           pk_q = grp == 0 ? c0 : (grp == 1 ? c1 : (grp == 2 ? c2 : 0.f));
+          if (two) {
+            pk_j2 = __shfl(Jaref, 16 + r);
+            pk_jv2 = __shfl(jv, 16 + r);
+            const float e0 = __shfl(q0r, 16 + r), e1 = __shfl(q1r, 16 + r), e2 = __shfl(q2r, 16 + r);
+            pk_q2 = grp == 0 ? e0 : (grp == 1 ? e1 : (grp == 2 ? e2 : 0.f));
+          }
         }
         auto point = [&](float alpha) {
           float q0, q1, q2;
           if (packed) {
             float x = (pk_j + alpha * pk_jv < 0.f) ? pk_q : 0.f;  // rows beyond nefc carry zeros
+            if (two) x += (pk_j2 + alpha * pk_jv2 < 0.f) ? pk_q2 : 0.f;
             x += dpp_shift<0x111, 0xf>(x);
             x += dpp_shift<0x112, 0xf>(x);
             x += dpp_shift<0x114, 0xf>(x);
