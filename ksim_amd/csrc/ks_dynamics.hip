@@ -151,6 +151,9 @@ __device__ __forceinline__ void chol_tile(f32x16& T, float (&R)[NP], float& myin
 
 // Mass matrix (LDS, rows of `stride` floats, zero beyond nv) into the accumulator layout, unit diagonal on the padding.
 __device__ __forceinline__ void load_mtile(f32x16& T, const float* __restrict__ M, int stride, int nv, int np, int lane) {
+  // The lane id is made opaque here: otherwise the sixteen unit-diagonal constants below are computed once, shared by
+  // all the call sites of a substep and kept (spilled) across the whole solver instead of being rebuilt in a few cycles.
+  asm volatile("" : "+v"(lane));
   const int c = lane & 31, half = lane >> 5;
   const bool real = c < nv;
   const float* row = M + (real ? c : 0) * stride;
@@ -970,6 +973,14 @@ void step_kernel(StepArgs a) {
     KS_TICK(14)
     // ---- semi-implicit Euler
     if (!FWD) {
+      // What this stage needs of the lane's constants is read again here (through an opaque lane id, so that the loads
+      // are not merged with those at the top of the substep): nothing of it stays live across the solver.
+      int lane_e = threadIdx.x;
+      asm volatile("" : "+v"(lane_e));
+      const LaneRec* rec_e = reinterpret_cast<const LaneRec*>(m.lane_rec[lane_e]);
+      const int b_jtype = rec_e->b_jtype, b_qadr = rec_e->b_qadr, b_dofadr = rec_e->b_dofadr;
+      const float d_damping = rec_e->d_damping * ((a.damping_scale && lane_e < nv) ? a.damping_scale[env * nv + lane_e] : 1.f);
+      const float my_qvel = lane_e < nv ? l.qvel[lane_e] : 0.f;
       float qacc_int = qacc;
       if (m.eulerdamp) {
         // implicit in the joint damping: (M + dt diag(damping)) a = M qacc.  For torque motors, whose force does
