@@ -133,6 +133,13 @@ typedef struct KsModelDesc {
   double act_gear[KS_MAX_ACTUATORS], act_lo[KS_MAX_ACTUATORS], act_hi[KS_MAX_ACTUATORS];
   int32_t sph_body[KS_MAX_SPHERES];
   double sph_pos[KS_MAX_SPHERES][3], sph_radius[KS_MAX_SPHERES];
+  /* Joint limits of hinges, by body (MuJoCo jnt_limited / jnt_range; the real K-Bot limits every joint,
+   * examples/kbot/robot/kbot-headless/robot.mjcf:66-217), and dry joint friction (dof_frictionloss, robot.mjcf:5-18).
+   * A violated limit is one constraint row J = +-e_j, friction one row J = e_j whose force saturates at
+   * +-frictionloss; both are regularised with dof_invweight0[j], the diagonal of the inverse mass matrix at qpos0,
+   * and use the model's solref / solimp.  All zero: neither. */
+  int32_t jnt_limited[KS_MAX_BODIES];
+  double jnt_range[KS_MAX_BODIES][2], dof_invweight0[KS_MAX_DOFS], dof_frictionloss[KS_MAX_DOFS];
 } KsModelDesc;
 
 typedef struct KsModel KsModel;

@@ -28,6 +28,8 @@ class KsModelDesc(ctypes.Structure):
         ("act_dof", c_int32 * MAXU), ("act_gear", c_double * MAXU), ("act_lo", c_double * MAXU),
         ("act_hi", c_double * MAXU),
         ("sph_body", c_int32 * MAXS), ("sph_pos", c_double * 3 * MAXS), ("sph_radius", c_double * MAXS),
+        ("jnt_limited", c_int32 * MAXB), ("jnt_range", c_double * 2 * MAXB), ("dof_invweight0", c_double * MAXV),
+        ("dof_frictionloss", c_double * MAXV),
     ]
 
 
@@ -73,7 +75,8 @@ def model_desc(m) -> KsModelDesc:
     for k in ("gravity", "solref", "solimp", "body_parent", "body_jtype", "body_qadr", "body_dofadr",
               "body_subtree_end", "body_pos", "body_quat", "body_mass", "body_ipos", "body_iquat", "body_inertia",
               "jnt_axis", "jnt_pos", "qpos0", "dof_body", "dof_parent", "dof_damping", "dof_armature", "act_dof",
-              "act_gear", "sph_body", "sph_pos", "sph_radius"):
+              "act_gear", "sph_body", "sph_pos", "sph_radius", "jnt_limited", "jnt_range", "dof_invweight0",
+              "dof_frictionloss"):
         fill(k, getattr(m, k))
     fill("body_invweight0", m.body_invweight0[:, 0])
     fill("act_lo", m.act_ctrlrange.reshape(-1, 2)[:, 0])

@@ -217,13 +217,72 @@ struct LaneRec {
   float s_pos[3];
   unsigned s_mask;
   int pk[kMaxPairs / 64 + 1];
-  int pad2[64 - 48 - (kMaxPairs / 64 + 1)];
+  // rows that live on the dof's own lane: hinge limit (range, inverse weight, address of the joint angle) and dry
+  // friction (level and the constant stiffness 1 / R of its row)
+  int d_limited, d_qadr;
+  float d_rlo, d_rhi, d_invw, d_floss, d_frD;
 };
 static_assert(sizeof(LaneRec) == 256, "LaneRec must fill the 64-dword record");
 
 struct LsPoint {
   float alpha, cost, d0, d1;
 };
+
+// constraint impedance d(|pos|) of the model's solimp
+__device__ __forceinline__ float impedance(const DevModel& m, float pos) {
+  const float ix = fabsf(pos) / m.width;
+  // x^power: the default power of 2 (and 1) without the general power function
+  const float ox = 1.f - ix;
+  const float px = m.power == 2.f ? ix * ix : (m.power == 1.f ? ix : powf(ix, m.power));
+  const float po = m.power == 2.f ? ox * ox : (m.power == 1.f ? ox : powf(ox, m.power));
+  const float ia = m.imp_a * px;
+  const float ib = 1.f - m.imp_b * po;
+  const float iy = ix < m.mid ? ia : ib;
+  float imp = m.dmin + iy * (m.dmax - m.dmin);
+  imp = fminf(fmaxf(imp, m.dmin), m.dmax);
+  if (ix > 1.f) imp = m.dmax;
+  return imp;
+}
+
+// The rows a dof lane carries itself: the violated limit of its hinge (J = lim_s e_j, lim_s = +-1, 0 when none) and its
+// dry friction (J = e_j, force clipped at +-fr_fl, 0 when none).  All zero on lanes that hold no dof.
+struct DofRows {
+  float lim_s, lim_aref, lim_D, fr_fl, fr_aref, fr_D;
+};
+
+// Cost of the lane's rows at acceleration qa; their force on the dof, their Hessian diagonal and which of them are in
+// their quadratic zone (bit 0 limit, bit 1 friction).
+__device__ __forceinline__ float dofrow_eval(const DofRows& r, float qa, float& force, float& hdiag, int& zone) {
+  float cost = 0.f;
+  force = 0.f; hdiag = 0.f; zone = 0;
+  const float xl = r.lim_s * qa - r.lim_aref;
+  if (r.lim_s != 0.f && xl < 0.f) {
+    cost = 0.5f * r.lim_D * xl * xl; force = -r.lim_D * xl * r.lim_s; hdiag = r.lim_D; zone = 1;
+  }
+  if (r.fr_fl > 0.f) {
+    const float xf = qa - r.fr_aref, rf = r.fr_fl / r.fr_D;
+    if (xf <= -rf) { cost += r.fr_fl * (-0.5f * rf - xf); force += r.fr_fl; }
+    else if (xf >= rf) { cost += r.fr_fl * (-0.5f * rf + xf); force -= r.fr_fl; }
+    else { cost += 0.5f * r.fr_D * xf * xf; force -= r.fr_D * xf; hdiag += r.fr_D; zone |= 2; }
+  }
+  return cost;
+}
+
+// Coefficients of the rows' cost along qa + alpha s, in the zones the rows are in at that alpha.
+__device__ __forceinline__ void dofrow_quad(const DofRows& r, float qa, float sdir, float alpha, float& t0, float& t1,
+                                            float& t2) {
+  t0 = 0.f; t1 = 0.f; t2 = 0.f;
+  const float x0 = r.lim_s * qa - r.lim_aref, jv = r.lim_s * sdir;
+  if (r.lim_s != 0.f && x0 + alpha * jv < 0.f) {
+    t0 = 0.5f * x0 * x0 * r.lim_D; t1 = jv * x0 * r.lim_D; t2 = 0.5f * jv * jv * r.lim_D;
+  }
+  if (r.fr_fl > 0.f) {
+    const float f0 = qa - r.fr_aref, rf = r.fr_fl / r.fr_D, x = f0 + alpha * sdir;
+    if (x <= -rf) { t0 += r.fr_fl * (-0.5f * rf - f0); t1 -= r.fr_fl * sdir; }
+    else if (x >= rf) { t0 += r.fr_fl * (-0.5f * rf + f0); t1 += r.fr_fl * sdir; }
+    else { t0 += 0.5f * f0 * f0 * r.fr_D; t1 += sdir * f0 * r.fr_D; t2 += 0.5f * sdir * sdir * r.fr_D; }
+  }
+}
 
 __device__ __forceinline__ bool in_bracket(const LsPoint& x, const LsPoint& y) {
   return ((x.d0 < y.d0) && (y.d0 < 0.f)) || ((x.d0 > y.d0) && (y.d0 > 0.f));
@@ -244,7 +303,7 @@ __device__ __forceinline__ float range_sum(const float* base, int w, int b, int 
 // ------------------------------------------------------------------------------------------- the fused kernel
 // FWD = true is the forward-only variant (derived fields + warm start of a given state, no actuation, no
 // integration) that replaces the mjx.forward of a reset.
-template <bool FWD, int NP>
+template <bool FWD, int NP, bool DR>
 __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(KS_STEP_WAVES, KS_STEP_WAVES)))
 void step_kernel(StepArgs a) {
   extern __shared__ __attribute__((aligned(16))) float lds_raw[];
@@ -683,17 +742,7 @@ void step_kernel(StepArgs a) {
       l.con_mask[c] = s_mask;
       st3(l.con_off + 3 * c, cpos - com);
       const float invweight = (s_invw + mu * mu * s_invw) * 2.f * mu * mu / m.impratio;
-      const float ix = fabsf(dist) / m.width;
-      // x^power: the default power of 2 (and 1) without the general power function
-      const float ox = 1.f - ix;
-      const float px = m.power == 2.f ? ix * ix : (m.power == 1.f ? ix : powf(ix, m.power));
-      const float po = m.power == 2.f ? ox * ox : (m.power == 1.f ? ox : powf(ox, m.power));
-      const float ia = m.imp_a * px;
-      const float ib = 1.f - m.imp_b * po;
-      const float iy = ix < m.mid ? ia : ib;
-      float imp = m.dmin + iy * (m.dmax - m.dmin);
-      imp = fminf(fmaxf(imp, m.dmin), m.dmax);
-      if (ix > 1.f) imp = m.dmax;
+      const float imp = impedance(m, dist);
       const float Rr = fmaxf(invweight * (1.f - imp) / imp, 1e-15f);
       l.con_D[c] = 1.0f / Rr;
       l.con_kip[c] = m.con_k * imp * dist;
@@ -717,7 +766,33 @@ void step_kernel(StepArgs a) {
     float qacc = qas;
     float Mqacc = qfs;  // M qacc = smooth + constraint force: what the implicit integration step solves against
     int niter = 0;
-    if (nefc > 0) {
+    // ---- rows on the dof lanes (models with joint limits or dry friction only).  Their Jacobians are unit vectors, so
+    // nothing of them is stored: lane j derives J a - aref of its rows from its own qacc wherever the solver needs it.
+    DofRows dr = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    int ndr = 0;
+    if (DR) {
+      int lane_r = threadIdx.x;
+      asm volatile("" : "+v"(lane_r));
+      const LaneRec* rr = reinterpret_cast<const LaneRec*>(m.lane_rec[lane_r]);
+      if (is_dof) {
+        if (rr->d_limited) {
+          const float q = l.qpos[rr->d_qadr];
+          const float dlo = q - rr->d_rlo, dhi = rr->d_rhi - q;
+          const float pos = fminf(dlo, dhi);
+          if (pos < 0.f) {  // the nearer side, once violated
+            dr.lim_s = dlo < dhi ? 1.f : -1.f;
+            const float imp = impedance(m, pos);
+            dr.lim_D = 1.f / fmaxf(rr->d_invw * (1.f - imp) / imp, 1e-15f);
+            dr.lim_aref = -m.con_b * dr.lim_s * my_qvel - m.con_k * imp * pos;
+          }
+        }
+        dr.fr_fl = rr->d_floss;
+        dr.fr_D = rr->d_frD;
+        dr.fr_aref = -m.con_b * my_qvel;
+      }
+      ndr = __popcll(__ballot(dr.lim_s != 0.f)) + m.nfriction;
+    }
+    if (nefc > 0 || (DR && ndr > 0)) {
       // ---- constraint rows: lane r builds row r of J in registers and mirrors it to LDS for column access
       const bool is_row = lane < nefc;
       float aref = 0.f, D = 0.f;
@@ -768,9 +843,16 @@ void step_kernel(StepArgs a) {
         if (is_dof) Ma_s = row_dot<NP>(Mrow, vv);
         if (is_row) Jar_s = row_dot<NP>(l.J + (is_row ? lane : 0) * js, vv) - aref;
       }
-      const float cost_w = wave_sum((is_row && Jar_w < 0.f) ? 0.5f * D * Jar_w * Jar_w : 0.f) +
+      float drc_w = 0.f, drc_s = 0.f;
+      if (DR) {
+        float f_, h_;
+        int z_;
+        drc_w = dofrow_eval(dr, warm, f_, h_, z_);
+        drc_s = dofrow_eval(dr, qas, f_, h_, z_);
+      }
+      const float cost_w = wave_sum(((is_row && Jar_w < 0.f) ? 0.5f * D * Jar_w * Jar_w : 0.f) + drc_w) +
                            0.5f * wave_sum(is_dof ? (Ma_w - qfs) * (warm - qas) : 0.f);
-      const float cost_s = wave_sum((is_row && Jar_s < 0.f) ? 0.5f * D * Jar_s * Jar_s : 0.f);
+      const float cost_s = wave_sum(((is_row && Jar_s < 0.f) ? 0.5f * D * Jar_s * Jar_s : 0.f) + drc_s);
       const bool use_warm = cost_w < cost_s;
       qacc = use_warm ? warm : qas;
       float Ma = use_warm ? Ma_w : Ma_s;
@@ -781,6 +863,7 @@ void step_kernel(StepArgs a) {
       KS_TICK(9)
 
       unsigned long long am_factored = 0ull;  // active set that R currently factors
+      unsigned long long amd_factored = 0ull; // and the quadratic zones of the dof-lane rows
       bool have_factor = false;               // none yet: R holds the factor of M
       while (true) {
         // ---- constraint update: active set, forces, cost
@@ -792,11 +875,19 @@ void step_kernel(StepArgs a) {
           const int r = __builtin_ctzll(t);
           qfc += l.J[r * js + (lane < nv ? lane : 0)] * lane_bcast(force, r);
         }
+        float dr_cost = 0.f, dr_force = 0.f, dr_h = 0.f;
+        unsigned long long amd = 0ull;
+        if (DR) {
+          int zone;
+          dr_cost = dofrow_eval(dr, qacc, dr_force, dr_h, zone);
+          qfc += dr_force;
+          amd = (__ballot(zone & 1) & 0xffffffffull) | (__ballot(zone & 2) << 32);
+        }
         if (!is_dof) qfc = 0.f;
         const float gauss = 0.5f * wave_sum(is_dof ? (Ma - qfs) * (qacc - qas) : 0.f);
         if (!first) {
           prev_cost = cost;
-          cost = wave_sum(active ? 0.5f * D * Jaref * Jaref : 0.f) + gauss;
+          cost = wave_sum((active ? 0.5f * D * Jaref * Jaref : 0.f) + dr_cost) + gauss;
         }
         first = false;
         // ---- gradient; stop before paying for another Hessian when the solver is done
@@ -815,7 +906,7 @@ void step_kernel(StepArgs a) {
         // lane i < 32 ends up with row i of H in registers, as the factorisation wants it.
         // H depends on the iterate only through the active set: while that stays the same (the usual case once the
         // solver closes in) the factor of the previous iteration is still the factor of H and is kept.
-        if (!have_factor || am != am_factored) {
+        if (!have_factor || am != am_factored || (DR && amd != amd_factored)) {
           l.drow[lane] = active ? D : 0.f;
           KS_SYNC();
           f32x16 hc;
@@ -827,9 +918,17 @@ void step_kernel(StepArgs a) {
             const float jv = (col_ok && r < nefc) ? l.J[r * js + col] : 0.f;
             hc = __builtin_amdgcn_mfma_f32_32x32x2f32(l.drow[r] * jv, jv, hc, 0, 0, 0);
           }
+          if (DR) {  // unit-vector rows add their stiffness to the diagonal
+            const float hd = __shfl(dr_h, col);
+#pragma unroll
+            for (int g = 0; g < 4; ++g)
+#pragma unroll
+              for (int e = 0; e < 4; ++e) hc[4 * g + e] += (8 * g + 4 * half + e == col) ? hd : 0.f;
+          }
           KS_TICK(11)
           chol_tile<NP>(hc, R, myinv, lane);
           am_factored = am;
+          amd_factored = amd;
           have_factor = true;
         }
         const float search_all = -solve_regs<NP>(R, myinv, lane, grad);
@@ -889,6 +988,13 @@ void step_kernel(StepArgs a) {
             q0 = g0 + wave_sum(on ? q0r : 0.f);
             q1 = g1 + wave_sum(on ? q1r : 0.f);
             q2 = g2 + wave_sum(on ? q2r : 0.f);
+          }
+          if (DR && ndr > 0) {
+            float t0, t1, t2;
+            dofrow_quad(dr, qacc, search, alpha, t0, t1, t2);
+            q0 += wave_sum(t0);
+            q1 += wave_sum(t1);
+            q2 += wave_sum(t2);
           }
           LsPoint p;
           p.alpha = alpha;
@@ -961,11 +1067,11 @@ void step_kernel(StepArgs a) {
     } else if (a.cfrc_ext && sub == nsub - 1) {
       for (int i = lane; i < nb * 6; i += 64) a.cfrc_ext[(int64_t)env * nb * 6 + i] = 0.f;
     }
-    work += (1 + niter) * (16 + nefc);
+    work += (1 + niter) * (16 + nefc + ndr);
     if (sub == nsub - 1) {  // outputs of the last substep go out here: nothing of them stays live to the end
       if (a.qacc && lane < nv) a.qacc[env * nv + lane] = qacc;
       if (a.solver_niter && lane == 0) a.solver_niter[env] = niter;
-      if (a.nefc && lane == 0) a.nefc[env] = nefc;
+      if (a.nefc && lane == 0) a.nefc[env] = nefc + ndr;
     }
     KS_SYNC();
     if (is_dof) l.warm[lane] = qacc;
@@ -1125,6 +1231,20 @@ extern "C" int ks_model_create(const KsModelDesc* d, KsModel** out) {
     m.dof_damping[j] = (float)d->dof_damping[j]; m.dof_armature[j] = (float)d->dof_armature[j];
     if (d->dof_parent[j] >= j || d->dof_body[j] < 1 || d->dof_body[j] >= d->nb) { delete km; return fail(KS_EINVAL, "ks_model_create: bad dof %d", j); }
   }
+  for (int b = 1; b < d->nb; ++b) {
+    if (!d->jnt_limited[b]) continue;
+    if (d->body_jtype[b] != kJntHinge) { delete km; return fail(KS_EINVAL, "ks_model_create: body %d: only hinges can be limited", b); }
+    if (!(d->jnt_range[b][0] < d->jnt_range[b][1])) { delete km; return fail(KS_EINVAL, "ks_model_create: body %d: empty joint range", b); }
+    if (!(d->dof_invweight0[d->body_dofadr[b]] > 0.0)) { delete km; return fail(KS_EINVAL, "ks_model_create: body %d: a limited joint needs dof_invweight0 > 0", b); }
+    m.dofrows = 1;
+  }
+  for (int j = 0; j < d->nv; ++j) {
+    if (d->dof_frictionloss[j] == 0.0) continue;
+    if (!(d->dof_frictionloss[j] > 0.0) || d->body_jtype[d->dof_body[j]] != kJntHinge) { delete km; return fail(KS_EINVAL, "ks_model_create: dof %d: frictionloss must be positive and on a hinge", j); }
+    if (!(d->dof_invweight0[j] > 0.0)) { delete km; return fail(KS_EINVAL, "ks_model_create: dof %d: dry friction needs dof_invweight0 > 0", j); }
+    m.dofrows = 1;
+    ++m.nfriction;
+  }
   for (int u = 0; u < d->nu; ++u) {
     const int j = d->act_dof[u];
     if (j < 0 || j >= d->nv) { delete km; return fail(KS_EINVAL, "ks_model_create: actuator %d drives dof %d", u, j); }
@@ -1175,6 +1295,16 @@ extern "C" int ks_model_create(const KsModelDesc* d, KsModel** out) {
     r.d_damping = m.dof_damping[dl]; r.d_armature = m.dof_armature[dl];
     const int ua = r.d_act >= 0 ? r.d_act : 0;
     r.d_gear = m.act_gear[ua]; r.d_lo = m.act_lo[ua]; r.d_hi = m.act_hi[ua];
+    r.d_limited = 0; r.d_qadr = 0; r.d_rlo = 0.f; r.d_rhi = 0.f; r.d_invw = 0.f; r.d_floss = 0.f; r.d_frD = 0.f;
+    if (is_dof && r.d_jtype == kJntHinge) {
+      r.d_limited = d->jnt_limited[r.d_body] != 0;
+      r.d_qadr = m.body_qadr[r.d_body];
+      r.d_rlo = (float)d->jnt_range[r.d_body][0]; r.d_rhi = (float)d->jnt_range[r.d_body][1];
+      r.d_invw = (float)d->dof_invweight0[dl];
+      r.d_floss = (float)d->dof_frictionloss[dl];
+      const double imp0 = m.dmin;  // impedance at pos = 0
+      r.d_frD = (float)(1.0 / std::max(d->dof_invweight0[dl] * (1.0 - imp0) / imp0, 1e-15));
+    }
     const int sl = L < d->ns ? L : 0;
     r.s_body = m.sph_body[sl]; r.s_rad = m.sph_radius[sl]; r.s_invw = m.body_invweight0[r.s_body];
     for (int k = 0; k < 3; ++k) r.s_pos[k] = m.sph_pos[sl][k];
@@ -1269,7 +1399,11 @@ static int launch_step(const KsModel* km, ks_stream_t stream, const KsStepIO* io
   if (bytes > 160 * 1024) return fail(KS_ELIMIT, "ks_step: model needs %d bytes of LDS", bytes);
   void (*fn)(StepArgs) = nullptr;
   switch (padded_nv(m.nv)) {
-#define KS_CASE(W) case W: fn = forward_only ? step_kernel<true, W> : step_kernel<false, W>; break;
+#define KS_CASE(W)                                                                                       \
+  case W:                                                                                                \
+    fn = m.dofrows ? (forward_only ? step_kernel<true, W, true> : step_kernel<false, W, true>)           \
+                   : (forward_only ? step_kernel<true, W, false> : step_kernel<false, W, false>);        \
+    break;
     KS_CASE(8) KS_CASE(16) KS_CASE(24) KS_CASE(28) KS_CASE(32)
 #undef KS_CASE
     default: return fail(KS_ELIMIT, "ks_step: no kernel for %d dofs", m.nv);

@@ -20,7 +20,8 @@ enum { kJntNone = 0, kJntFree = 1, kJntHinge = 2 };
 // vector L1 / scalar cache (it is ~10 KB and shared by every wavefront).
 struct DevModel {
   int nb, nq, nv, nu, ns, iterations, ls_iterations, eulerdamp, npairs, nvs /* row stride of the mass matrix in LDS, a multiple of 4 */, max_depth,
-      js /* row stride of the constraint Jacobian in LDS, a multiple of 4 */;
+      js /* row stride of the constraint Jacobian in LDS, a multiple of 4 */,
+      dofrows /* 1 when a joint is limited or has dry friction */, nfriction /* dofs with dry friction */;
   float dt, gravity[3], tolerance, ls_tolerance, meaninertia, friction, impratio;
   // contact impedance constants, already clamped the way the constraint builder wants them
   float con_k, con_b, dmin, dmax, width, mid, power;

@@ -118,6 +118,10 @@ class KinematicModel:
     dof_parent: np.ndarray
     dof_damping: np.ndarray
     dof_armature: np.ndarray
+    # joint limits of hinges, by body (MuJoCo jnt_limited / jnt_range), and dry joint friction (dof_frictionloss)
+    jnt_limited: np.ndarray
+    jnt_range: np.ndarray
+    dof_frictionloss: np.ndarray
     # actuators (motors: force = gear * clip(ctrl, ctrlrange))
     act_dof: np.ndarray
     act_gear: np.ndarray
@@ -171,13 +175,14 @@ class ModelBuilder:
         self.bodies = [dict(parent=-1, jtype=JNT_NONE, pos=np.zeros(3), quat=np.array([1.0, 0, 0, 0]), mass=0.0,
                             ipos=np.zeros(3), iquat=np.array([1.0, 0, 0, 0]), inertia=np.zeros(3),
                             axis=np.array([0.0, 0, 1]), jpos=np.zeros(3), damping=0.0, armature=0.0, qpos0=0.0,
-                            name="world")]
+                            range=None, frictionloss=0.0, name="world")]
         self.actuators: list[dict] = []
         self.spheres: list[dict] = []
 
     def add_body(self, parent: int, pos, *, joint: str | None = "hinge", axis=(0.0, 1.0, 0.0),
                  joint_pos=(0.0, 0.0, 0.0), quat=(1.0, 0.0, 0.0, 0.0), mass: float, ipos=(0.0, 0.0, 0.0),
-                 iquat=(1.0, 0.0, 0.0, 0.0), inertia, damping=0.0, armature=0.0, name: str | None = None) -> int:
+                 iquat=(1.0, 0.0, 0.0, 0.0), inertia, damping=0.0, armature=0.0, range=None, frictionloss=0.0,
+                 name: str | None = None) -> int:
         b = len(self.bodies)
         if not (0 <= parent < b):
             raise ValueError(f"parent {parent} does not exist")
@@ -192,6 +197,14 @@ class ModelBuilder:
             raise ValueError("a free joint must attach to the world")
         if jtype == JNT_NONE:
             raise ValueError("every body needs a free or hinge joint in this model subset")
+        if range is not None:
+            if jtype != JNT_HINGE:
+                raise ValueError("joint limits apply to hinge joints")
+            if not (float(range[0]) < float(range[1])):
+                raise ValueError(f"joint range {range} is empty")
+            range = (float(range[0]), float(range[1]))
+        if frictionloss < 0 or (frictionloss > 0 and jtype != JNT_HINGE):
+            raise ValueError("frictionloss is a non-negative property of hinge joints")
         ax = np.array(axis, dtype=np.float64)
         ax /= np.linalg.norm(ax)
         q = np.array(quat, dtype=np.float64)
@@ -200,7 +213,8 @@ class ModelBuilder:
                                 quat=q / np.linalg.norm(q), mass=float(mass), ipos=np.array(ipos, dtype=np.float64),
                                 iquat=iq / np.linalg.norm(iq), inertia=np.array(inertia, dtype=np.float64), axis=ax,
                                 jpos=np.array(joint_pos, dtype=np.float64), damping=float(damping),
-                                armature=float(armature), qpos0=0.0, name=name or f"body{b}"))
+                                armature=float(armature), qpos0=0.0, range=range, frictionloss=float(frictionloss),
+                                name=name or f"body{b}"))
         return b
 
     def add_capsule_body(self, parent: int, pos, direction, length: float, radius: float, mass: float, **kw) -> int:
@@ -240,7 +254,8 @@ class ModelBuilder:
         for b in range(nb - 1, 0, -1):
             subtree_end[parent[b]] = max(subtree_end[parent[b]], subtree_end[b])
         dof_body, dof_parent = np.zeros(nv, np.int32), np.full(nv, -1, np.int32)
-        damping, armature = np.zeros(nv), np.zeros(nv)
+        damping, armature, frictionloss = np.zeros(nv), np.zeros(nv), np.zeros(nv)
+        limited, jrange = np.zeros(nb, np.int32), np.zeros((nb, 2))
 
         def last_dof_of(body: int) -> int:
             while body > 0:
@@ -263,6 +278,9 @@ class ModelBuilder:
                 dof_body[i] = b
                 dof_parent[i] = last_dof_of(int(parent[b]))
                 damping[i], armature[i] = body["damping"], body["armature"]
+                frictionloss[i] = body["frictionloss"]
+                if body["range"] is not None:
+                    limited[b], jrange[b] = 1, body["range"]
         qpos0 = np.zeros(nq)
         for b, body in enumerate(self.bodies):
             if body["jtype"] == JNT_FREE:
@@ -278,6 +296,7 @@ class ModelBuilder:
             body_mass=stack("mass"), body_ipos=stack("ipos"), body_iquat=stack("iquat"),
             body_inertia=stack("inertia"), jnt_axis=stack("axis"), jnt_pos=stack("jpos"), qpos0=qpos0,
             dof_body=dof_body, dof_parent=dof_parent, dof_damping=damping, dof_armature=armature,
+            jnt_limited=limited, jnt_range=jrange, dof_frictionloss=frictionloss,
             act_dof=np.array([dofadr[a["body"]] for a in self.actuators], np.int32).reshape(nu),
             act_gear=np.array([a["gear"] for a in self.actuators], np.float64).reshape(nu),
             act_ctrlrange=np.array([[a["lo"], a["hi"]] for a in self.actuators], np.float64).reshape(nu, 2),
@@ -380,27 +399,31 @@ def _compile_constants(m: dict):
 
 # --------------------------------------------------------------------------- procedural models of the benchmark configs
 def pendulum_chain_model(n_links: int = 3, length: float = 0.5, radius: float = 0.05, mass: float = 1.0,
-                         damping: float = 0.1, dt: float = 0.005, **opts) -> KinematicModel:
+                         damping: float = 0.1, dt: float = 0.005, joint_range=None, frictionloss: float = 0.0,
+                         **opts) -> KinematicModel:
     """Planar hinge chain hanging from the world origin along -z, hinge axes along y, no contacts."""
     mb = ModelBuilder(dt=dt, **opts)
     parent = 0
     for i in range(n_links):
         pos = (0.0, 0.0, 0.0) if i == 0 else (0.0, 0.0, -length)
         parent = mb.add_capsule_body(parent, pos, (0.0, 0.0, -1.0), length, radius, mass, joint="hinge",
-                                     axis=(0.0, 1.0, 0.0), damping=damping, name=f"link{i}")
+                                     axis=(0.0, 1.0, 0.0), damping=damping, range=joint_range,
+                                     frictionloss=frictionloss, name=f"link{i}")
         mb.add_actuator(parent)
     return mb.build()
 
 
 def _limb(mb: ModelBuilder, rng, parent: int, attach, axes: Sequence, direction, seg_len: Sequence[float],
-          radius: float, mass_range, damping: float, armature_range, name: str) -> list[int]:
+          radius: float, mass_range, damping: float, armature_range, name: str, joint_range=None,
+          frictionloss: float = 0.0) -> list[int]:
     ids = []
     pos = np.array(attach, dtype=np.float64)
     for k, (axis, ln) in enumerate(zip(axes, seg_len)):
         ln = float(ln * rng.uniform(0.9, 1.1))
         arm = float(rng.uniform(*armature_range)) if armature_range else 0.0
         b = mb.add_capsule_body(parent, pos, direction, ln, radius, float(rng.uniform(*mass_range)), joint="hinge",
-                                axis=axis, damping=damping, armature=arm, name=f"{name}{k}")
+                                axis=axis, damping=damping, armature=arm, range=joint_range, frictionloss=frictionloss,
+                                name=f"{name}{k}")
         mb.add_actuator(b)
         ids.append(b)
         parent = b
@@ -408,9 +431,14 @@ def _limb(mb: ModelBuilder, rng, parent: int, attach, axes: Sequence, direction,
     return ids
 
 
-def humanoid_model(seed: int = 1003, dt: float = 0.005, friction: float = 1.0, **opts) -> KinematicModel:
-    """Free root + 21 hinges in a seeded 5-limb tree (4+4+4+4+5), 4 foot spheres, 21 motors."""
+def humanoid_model(seed: int = 1003, dt: float = 0.005, friction: float = 1.0, joint_range=None,
+                   frictionloss: float = 0.0, **opts) -> KinematicModel:
+    """Free root + 21 hinges in a seeded 5-limb tree (4+4+4+4+5), 4 foot spheres, 21 motors.
+
+    ``joint_range`` limits every hinge to that interval and ``frictionloss`` gives every hinge that much dry friction
+    (both off by default)."""
     rng = np.random.default_rng(seed)
+    jl = dict(joint_range=joint_range, frictionloss=frictionloss)
     mb = ModelBuilder(dt=dt, friction=friction, **opts)
     mr = (0.5, 5.0)
     root = mb.add_capsule_body(0, (0.0, 0.0, 1.3), (0.0, 0.0, 1.0), 0.3, 0.1, float(rng.uniform(*mr)), joint="free",
@@ -419,13 +447,13 @@ def humanoid_model(seed: int = 1003, dt: float = 0.005, friction: float = 1.0, *
     feet = []
     for side, sy in (("l", 0.1), ("r", -0.1)):
         ids = _limb(mb, rng, root, (0.0, sy, -0.05), [X, Y, Y, Y], (0.0, 0.0, -1.0), [0.06, 0.4, 0.4, 0.06], 0.05, mr,
-                    0.2, (0.01, 0.01), f"leg_{side}")
+                    0.2, (0.01, 0.01), f"leg_{side}", **jl)
         feet.append(ids[-1])
     for side, sy in (("l", 0.2), ("r", -0.2)):
         _limb(mb, rng, root, (0.0, sy, 0.3), [X, Y, Y, X], (0.0, float(np.sign(sy)) * 0.3, -1.0),
-              [0.05, 0.28, 0.25, 0.05], 0.04, mr, 0.2, (0.01, 0.01), f"arm_{side}")
+              [0.05, 0.28, 0.25, 0.05], 0.04, mr, 0.2, (0.01, 0.01), f"arm_{side}", **jl)
     _limb(mb, rng, root, (0.0, 0.0, 0.32), [Z, Y, X, Y, Z], (0.0, 0.0, 1.0), [0.05, 0.1, 0.15, 0.05, 0.12], 0.07, mr,
-          0.2, (0.01, 0.01), "spine")
+          0.2, (0.01, 0.01), "spine", **jl)
     for f in feet:
         tip = mb.bodies[f]["ipos"] * 2
         mb.add_contact_sphere(f, tip + np.array([0.08, 0.0, 0.0]), 0.04)
@@ -433,9 +461,14 @@ def humanoid_model(seed: int = 1003, dt: float = 0.005, friction: float = 1.0, *
     return mb.build()
 
 
-def kbot_scale_model(seed: int = 1004, dt: float = 0.005, **opts) -> KinematicModel:
-    """K-Bot-scale biped: free root + 20 hinges (legs 5+5, arms 5+5), 8 foot spheres, armature ~U(0.01,0.05)."""
+def kbot_scale_model(seed: int = 1004, dt: float = 0.005, joint_range=None, frictionloss: float = 0.0,
+                     **opts) -> KinematicModel:
+    """K-Bot-scale biped: free root + 20 hinges (legs 5+5, arms 5+5), 8 foot spheres, armature ~U(0.01,0.05).
+
+    ``joint_range`` / ``frictionloss``: limits and dry friction on every hinge, as the real K-Bot's joints have
+    (examples/kbot/robot/kbot-headless/robot.mjcf:5-18); off by default."""
     rng = np.random.default_rng(seed)
+    jl = dict(joint_range=joint_range, frictionloss=frictionloss)
     mb = ModelBuilder(dt=dt, **opts)
     root = mb.add_capsule_body(0, (0.0, 0.0, 1.05), (0.0, 0.0, 1.0), 0.35, 0.1, 12.0, joint="free", name="torso")
     X, Y, Z = (1.0, 0, 0), (0, 1.0, 0), (0, 0, 1.0)
@@ -443,11 +476,11 @@ def kbot_scale_model(seed: int = 1004, dt: float = 0.005, **opts) -> KinematicMo
     feet = []
     for side, sy in (("l", 0.09), ("r", -0.09)):
         ids = _limb(mb, rng, root, (0.0, sy, -0.02), [Y, X, Z, Y, Y], (0.0, 0.0, -1.0),
-                    [0.05, 0.05, 0.35, 0.35, 0.05], 0.04, (0.8, 3.0), 0.2, arm_r, f"leg_{side}")
+                    [0.05, 0.05, 0.35, 0.35, 0.05], 0.04, (0.8, 3.0), 0.2, arm_r, f"leg_{side}", **jl)
         feet.append(ids[-1])
     for side, sy in (("l", 0.18), ("r", -0.18)):
         _limb(mb, rng, root, (0.0, sy, 0.33), [Y, X, Z, Y, X], (0.0, float(np.sign(sy)) * 0.15, -1.0),
-              [0.04, 0.04, 0.22, 0.2, 0.06], 0.03, (0.3, 1.2), 0.2, arm_r, f"arm_{side}")
+              [0.04, 0.04, 0.22, 0.2, 0.06], 0.03, (0.3, 1.2), 0.2, arm_r, f"arm_{side}", **jl)
     for f in feet:
         tip = mb.bodies[f]["ipos"] * 2
         for dx in (0.1, -0.06):

@@ -14,7 +14,7 @@ import numpy as np
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB = os.path.join(HERE, "libksoracle.so")
-MAXB, MAXQ, MAXV, MAXU, MAXS, MAXR = 32, 40, 32, 32, 16, 64
+MAXB, MAXQ, MAXV, MAXU, MAXS, MAXR = 32, 40, 32, 32, 16, 128
 
 
 def build(force: bool = False) -> str:
@@ -38,6 +38,8 @@ class KsorModel(ctypes.Structure):
         ("qpos0", c_double * MAXQ),
         ("dof_body", c_int * MAXV), ("dof_parent", c_int * MAXV), ("dof_damping", c_double * MAXV),
         ("dof_armature", c_double * MAXV),
+        ("jnt_limited", c_int * MAXB), ("jnt_range", c_double * 2 * MAXB), ("dof_invweight0", c_double * MAXV),
+        ("dof_frictionloss", c_double * MAXV),
         ("act_dof", c_int * MAXU), ("act_gear", c_double * MAXU), ("act_lo", c_double * MAXU),
         ("act_hi", c_double * MAXU),
         ("sph_body", c_int * MAXS), ("sph_pos", c_double * 3 * MAXS), ("sph_radius", c_double * MAXS),
@@ -62,7 +64,7 @@ def _data_struct(real):
             ("nefc", c_int), ("solver_niter", c_int),
             ("con_dist", real * MAXS), ("con_pos", real * 3 * MAXS),
             ("efc_J", real * (MAXR * MAXV)), ("efc_pos", real * MAXR), ("efc_aref", real * MAXR),
-            ("efc_D", real * MAXR), ("efc_force", real * MAXR),
+            ("efc_D", real * MAXR), ("efc_force", real * MAXR), ("efc_floss", real * MAXR),
             ("qfrc_constraint", real * MAXV), ("qacc", real * MAXV), ("cfrc_ext", real * 6 * MAXB),
         ]
 
@@ -99,6 +101,9 @@ def make_model(a: dict) -> KsorModel:
     for k in ("body_pos", "body_quat", "body_ipos", "body_iquat", "body_inertia", "jnt_axis", "jnt_pos", "sph_pos"):
         fill(k, a[k])
     fill("body_invweight0", np.asarray(a["body_invweight0"])[:, 0])
+    for k in ("jnt_limited", "jnt_range", "dof_invweight0", "dof_frictionloss"):
+        if k in a:  # absent: no limits, no dry friction
+            fill(k, a[k])
     fill("act_lo", np.asarray(a["act_ctrlrange"]).reshape(-1, 2)[:, 0])
     fill("act_hi", np.asarray(a["act_ctrlrange"]).reshape(-1, 2)[:, 1])
     return m
@@ -127,7 +132,7 @@ class DataView:
             return arr[: nv * nv].reshape(nv, nv)
         if name == "efc_J":
             return arr[: raw.nefc * nv].reshape(raw.nefc, nv)
-        if name in ("efc_pos", "efc_aref", "efc_D", "efc_force"):
+        if name in ("efc_pos", "efc_aref", "efc_D", "efc_force", "efc_floss"):
             return arr[: raw.nefc]
         if name in trim:
             return arr[: trim[name]]

@@ -43,7 +43,7 @@ typedef struct FN(KsorData) {
   int nefc, solver_niter;
   REAL con_dist[KSOR_MAXS], con_pos[KSOR_MAXS][3];
   REAL efc_J[KSOR_MAXR * KSOR_MAXV], efc_pos[KSOR_MAXR], efc_aref[KSOR_MAXR], efc_D[KSOR_MAXR],
-      efc_force[KSOR_MAXR];
+      efc_force[KSOR_MAXR], efc_floss[KSOR_MAXR]; /* efc_floss > 0 marks a dry-friction row */
   REAL qfrc_constraint[KSOR_MAXV], qacc[KSOR_MAXV];
   /* contact forces on each body as a spatial force about the tree's centre of mass, world axes, torque then force
    * (MuJoCo's cfrc_ext, which FeetForceObservation / FeetTorqueObservation read, ksim/observation.py:563-616) */
@@ -344,6 +344,20 @@ static void jac_point(const KsorModel* m, const Data* d, REAL* jacp, const REAL*
   }
 }
 
+/* constraint impedance d(|pos|) of MuJoCo's solimp = (dmin, dmax, width, midpoint, power) */
+static REAL impedance(REAL pos, REAL dmin, REAL dmax, REAL width, REAL mid, REAL power) {
+  const REAL ix = (REAL)fabs(pos) / width;
+  const REAL ia = (1 / (REAL)pow(mid, power - 1)) * (REAL)pow(ix, power);
+  const REAL ib = 1 - (1 / (REAL)pow(1 - mid, power - 1)) * (REAL)pow(1 - ix, power);
+  const REAL iy = ix < mid ? ia : ib;
+  REAL imp = dmin + iy * (dmax - dmin);
+  imp = imp < dmin ? dmin : (imp > dmax ? dmax : imp);
+  if (ix > 1) imp = dmax;
+  return imp;
+}
+
+/* Rows in the order contacts, joint limits, dry friction (MuJoCo orders them friction, limits, contacts; the order
+ * only changes the order of summation). */
 void FN(ksor_make_constraint)(const KsorModel* m, Data* d) {
   const int nv = m->nv;
   int nefc = 0;
@@ -381,15 +395,8 @@ void FN(ksor_make_constraint)(const KsorModel* m, Data* d) {
     const REAL* Jx = jacp;
     const REAL t = (REAL)m->body_invweight0[b];
     const REAL invweight = (t + mu * mu * t) * 2 * mu * mu / (REAL)m->impratio;
-    /* impedance */
     const REAL pos = dist;
-    const REAL ix = (REAL)fabs(pos) / width;
-    const REAL ia = (1 / (REAL)pow(mid, power - 1)) * (REAL)pow(ix, power);
-    const REAL ib = 1 - (1 / (REAL)pow(1 - mid, power - 1)) * (REAL)pow(1 - ix, power);
-    REAL iy = ix < mid ? ia : ib;
-    REAL imp = dmin + iy * (dmax - dmin);
-    imp = imp < dmin ? dmin : (imp > dmax ? dmax : imp);
-    if (ix > 1) imp = dmax;
+    const REAL imp = impedance(pos, dmin, dmax, width, mid, power);
     REAL R = invweight * (1 - imp) / imp;
     if (R < MINVAL) R = MINVAL;
     for (int q = 0; q < 4; ++q) {
@@ -403,8 +410,47 @@ void FN(ksor_make_constraint)(const KsorModel* m, Data* d) {
       d->efc_pos[nefc + q] = pos;
       d->efc_aref[nefc + q] = -bb * vel - kk * imp * pos;
       d->efc_D[nefc + q] = 1 / R;
+      d->efc_floss[nefc + q] = 0;
     }
     nefc += 4;
+  }
+  /* joint limits of hinges: one row for the nearer side once it is violated (margin 0), J = +1 on the lower side and
+   * -1 on the upper side, regularised with the dof's inverse weight */
+  for (int b = 1; b < m->nb; ++b) {
+    if (m->body_jtype[b] != KSOR_JNT_HINGE || !m->jnt_limited[b]) continue;
+    const int j = m->body_dofadr[b];
+    const REAL q = d->qpos[m->body_qadr[b]];
+    const REAL dlo = q - (REAL)m->jnt_range[b][0], dhi = (REAL)m->jnt_range[b][1] - q;
+    const REAL pos = dlo < dhi ? dlo : dhi;
+    if (!(pos < 0)) continue;
+    const REAL side = dlo < dhi ? 1 : -1;
+    REAL* row = d->efc_J + nefc * nv;
+    for (int i = 0; i < nv; ++i) row[i] = 0;
+    row[j] = side;
+    const REAL imp = impedance(pos, dmin, dmax, width, mid, power);
+    REAL R = (REAL)m->dof_invweight0[j] * (1 - imp) / imp;
+    if (R < MINVAL) R = MINVAL;
+    d->efc_pos[nefc] = pos;
+    d->efc_aref[nefc] = -bb * side * d->qvel[j] - kk * imp * pos;
+    d->efc_D[nefc] = 1 / R;
+    d->efc_floss[nefc] = 0;
+    ++nefc;
+  }
+  /* dry joint friction: a row J = e_j at pos = 0 whose force saturates at +-frictionloss */
+  for (int j = 0; j < nv; ++j) {
+    const REAL fl = (REAL)m->dof_frictionloss[j];
+    if (!(fl > 0)) continue;
+    REAL* row = d->efc_J + nefc * nv;
+    for (int i = 0; i < nv; ++i) row[i] = 0;
+    row[j] = 1;
+    const REAL imp = impedance(0, dmin, dmax, width, mid, power);
+    REAL R = (REAL)m->dof_invweight0[j] * (1 - imp) / imp;
+    if (R < MINVAL) R = MINVAL;
+    d->efc_pos[nefc] = 0;
+    d->efc_aref[nefc] = -bb * d->qvel[j];
+    d->efc_D[nefc] = 1 / R;
+    d->efc_floss[nefc] = fl;
+    ++nefc;
   }
   d->nefc = nefc;
 }
@@ -431,9 +477,18 @@ static void update_constraint(const KsorModel* m, const Data* d, Ctx* c) {
   REAL cost = 0;
   for (int i = 0; i < nv; ++i) c->qfrc_constraint[i] = 0;
   for (int r = 0; r < ne; ++r) {
-    c->active[r] = c->Jaref[r] < 0;
-    c->efc_force[r] = c->active[r] ? -d->efc_D[r] * c->Jaref[r] : 0;
-    if (c->active[r]) cost += (REAL)0.5 * d->efc_D[r] * c->Jaref[r] * c->Jaref[r];
+    const REAL fl = d->efc_floss[r], x = c->Jaref[r];
+    if (fl > 0) {
+      /* dry friction: quadratic inside |x| < R f, linear (constant force -+f) outside */
+      const REAL rf = fl / d->efc_D[r];
+      if (x <= -rf) { c->active[r] = 0; c->efc_force[r] = fl; cost += fl * (-(REAL)0.5 * rf - x); }
+      else if (x >= rf) { c->active[r] = 0; c->efc_force[r] = -fl; cost += fl * (-(REAL)0.5 * rf + x); }
+      else { c->active[r] = 1; c->efc_force[r] = -d->efc_D[r] * x; cost += (REAL)0.5 * d->efc_D[r] * x * x; }
+    } else {
+      c->active[r] = x < 0;
+      c->efc_force[r] = c->active[r] ? -d->efc_D[r] * x : 0;
+      if (c->active[r]) cost += (REAL)0.5 * d->efc_D[r] * x * x;
+    }
     for (int j = 0; j < nv; ++j) c->qfrc_constraint[j] += d->efc_J[r * nv + j] * c->efc_force[r];
   }
   REAL g = 0;
@@ -487,7 +542,13 @@ static LSPoint ls_point(const Data* d, const Ctx* c, REAL alpha, const REAL* jv,
   REAL q0 = quad_gauss[0], q1 = quad_gauss[1], q2 = quad_gauss[2];
   for (int r = 0; r < d->nefc; ++r) {
     const REAL x = c->Jaref[r] + alpha * jv[r];
-    if (x < 0) { q0 += quad[r][0]; q1 += quad[r][1]; q2 += quad[r][2]; }
+    const REAL fl = d->efc_floss[r];
+    if (fl > 0) {
+      const REAL rf = fl / d->efc_D[r];
+      if (x <= -rf) { q0 += fl * (-(REAL)0.5 * rf - c->Jaref[r]); q1 += -fl * jv[r]; }
+      else if (x >= rf) { q0 += fl * (-(REAL)0.5 * rf + c->Jaref[r]); q1 += fl * jv[r]; }
+      else { q0 += quad[r][0]; q1 += quad[r][1]; q2 += quad[r][2]; }
+    } else if (x < 0) { q0 += quad[r][0]; q1 += quad[r][1]; q2 += quad[r][2]; }
   }
   LSPoint p;
   p.alpha = alpha;

@@ -2,7 +2,8 @@
  *
  * Restates, in plain scalar C, what `mjx.step` computes at ksim/engine.py:257 for the
  * model subset the rollout configs use (kinematic tree of free/hinge joints, motor
- * actuators, sphere-plane contacts with pyramidal cones, Newton solver, Euler).
+ * actuators, sphere-plane contacts with pyramidal cones, joint limits, dry joint friction,
+ * Newton solver, Euler).
  * MJX itself is third-party and not vendored in the reference (ksim/requirements.txt:20-21,
  * unpinned); the algorithm follows the public MuJoCo "Computation" documentation.
  * Parity with MJX of the Newton iterates, impedance details and pyramidal regulariser
@@ -19,7 +20,7 @@
 #define KSOR_MAXV 32
 #define KSOR_MAXU 32
 #define KSOR_MAXS 16  /* contact spheres */
-#define KSOR_MAXR 64  /* constraint rows = 4 per sphere */
+#define KSOR_MAXR 128 /* constraint rows: 4 per sphere, one per limited joint at its limit, one per dof with dry friction */
 
 enum { KSOR_JNT_NONE = 0, KSOR_JNT_FREE = 1, KSOR_JNT_HINGE = 2 };
 
@@ -37,6 +38,10 @@ typedef struct KsorModel {
   double qpos0[KSOR_MAXQ];
   int dof_body[KSOR_MAXV], dof_parent[KSOR_MAXV];
   double dof_damping[KSOR_MAXV], dof_armature[KSOR_MAXV];
+  /* joint limits of hinges (MuJoCo jnt_limited / jnt_range, by body) and dry joint friction (dof_frictionloss);
+   * dof_invweight0 is the diagonal of the inverse mass matrix at qpos0, which scales their regularisation */
+  int jnt_limited[KSOR_MAXB];
+  double jnt_range[KSOR_MAXB][2], dof_invweight0[KSOR_MAXV], dof_frictionloss[KSOR_MAXV];
   int act_dof[KSOR_MAXU];
   double act_gear[KSOR_MAXU], act_lo[KSOR_MAXU], act_hi[KSOR_MAXU];
   int sph_body[KSOR_MAXS];

@@ -19,7 +19,13 @@ MODELS = {"chain": km.pendulum_chain_model, "humanoid": km.humanoid_model, "kbot
           # the integrator ksim selects: velocity update implicit in joint damping
           "chain-implicit": lambda: km.pendulum_chain_model(integrator="implicitfast", damping=0.5),
           "kbot-implicit": lambda: km.kbot_scale_model(integrator="implicitfast"),
-          "humanoid-implicit": lambda: km.humanoid_model(integrator="implicitfast")}
+          "humanoid-implicit": lambda: km.humanoid_model(integrator="implicitfast"),
+          # joint limits and dry joint friction (rows carried by the dof lanes), alone and together with contacts.  The test
+          # states draw hinge angles from U(-0.6, 0.6), so about a fifth of the joints start up to 0.15 rad beyond a limit
+          # (much deeper violations make the cost so large that its fp32 rounding hides the last Newton improvements).
+          "chain-friction": lambda: km.pendulum_chain_model(integrator="implicitfast", frictionloss=0.3),
+          "humanoid-limits": lambda: km.humanoid_model(joint_range=(-0.45, 0.5)),
+          "kbot-limits": lambda: km.kbot_scale_model(integrator="implicitfast", joint_range=(-0.45, 0.5), frictionloss=0.2)}
 ONE_STEP_TOL, TEN_STEP_TOL = 1e-4, 1e-3
 
 
@@ -125,7 +131,8 @@ def _oracle_control_steps(m, qpos, qvel, actions, kp, kd, clip, S, latency, fric
 
 @pytest.mark.parametrize("name,S,T,period", [("chain", 1, 10, 1), ("kbot", 4, 2, 1), ("humanoid", 4, 2, 2),
                                              ("chain-implicit", 1, 10, 1), ("kbot-implicit", 4, 2, 1),
-                                             ("kbot-implicit", 1, 1, 1), ("humanoid-implicit", 4, 2, 2)])
+                                             ("kbot-implicit", 1, 1, 1), ("humanoid-implicit", 4, 2, 2),
+                                             ("kbot-limits", 4, 2, 1), ("chain-friction", 1, 10, 1)])
 def test_position_controlled_steps(name, S, T, period):
     """Fused control step (latency blend + PD + S substeps) with per-env friction / mass scale."""
     from ksim_amd import physics
@@ -465,3 +472,45 @@ def test_launch_order_does_not_change_results_and_sorts_heaviest_first():
         assert torch.equal(a[k], b[k]), k
     rev = torch.from_numpy(np.ascontiguousarray(o[::-1])).to(DEV)
     assert torch.equal(run(rev)["qpos"], a["qpos"])
+
+
+def test_joint_limit_and_dry_friction_closed_forms():
+    """The kernel itself against the closed forms that pin the oracle's limit and friction rows."""
+    from ksim_amd import physics
+    from ksim_amd._lib_dyn import KS_ACT_TORQUE
+
+    # dry friction f on a hinge without gravity or damping: a fast joint decelerates at f / I per unit time
+    f = 0.4
+    m = km.pendulum_chain_model(n_links=1, damping=0.0, frictionloss=f, gravity=(0.0, 0.0, 0.0))
+    inertia = float(km.host_mass_matrix(m.arrays(), m.qpos0)[0, 0])
+    dm = physics.DeviceModel(m)
+    buf = dict(qpos=zeros(2, 1), qvel=t32([[2.0], [-2.0]]), qacc_warmstart=zeros(2, 1), time=zeros(2),
+               last_ctrl=zeros(2, 1), action=zeros(2, 1))
+    physics.control_step(dm, buf, substeps=10, actuator_type=KS_ACT_TORQUE)
+    want = 2.0 - 10 * m.dt * f / inertia
+    np.testing.assert_allclose(buf["qvel"].cpu().numpy()[:, 0], [want, -want], rtol=1e-5)
+    for _ in range(60):
+        physics.control_step(dm, buf, substeps=50, actuator_type=KS_ACT_TORQUE)
+    assert buf["qvel"].abs().max().item() < 1e-6  # stopped, and stays stopped
+
+    # a link on a horizontal hinge limited to (0.3, 1.0) settles just below 0.3, where the limit force
+    # D k imp |pos| balances the gravity torque m g (L / 2) sin q
+    L, mass = 0.5, 1.0
+    m = km.pendulum_chain_model(n_links=1, length=L, mass=mass, damping=0.5, joint_range=(0.3, 1.0))
+    dm = physics.DeviceModel(m)
+    buf = dict(qpos=t32([[0.6]]), qvel=zeros(1, 1), qacc_warmstart=zeros(1, 1), time=zeros(1), last_ctrl=zeros(1, 1),
+               action=zeros(1, 1))
+    for _ in range(80):
+        physics.control_step(dm, buf, substeps=50, actuator_type=KS_ACT_TORQUE)
+    q = buf["qpos"].item()
+    pos = q - 0.3
+    assert abs(buf["qvel"].item()) < 1e-5 and -0.01 < pos < 0
+    dmin, dmax, width, mid, power = m.solimp
+    x = abs(pos) / width
+    y = (1 / mid ** (power - 1)) * x**power if x < mid else 1 - (1 / (1 - mid) ** (power - 1)) * (1 - x) ** power
+    imp = dmax if x > 1 else float(np.clip(dmin + y * (dmax - dmin), dmin, dmax))
+    k = 1 / (dmax**2 * max(m.solref[0], 2 * m.dt) ** 2 * m.solref[1] ** 2)
+    inertia = float(km.host_mass_matrix(m.arrays(), m.qpos0)[0, 0])
+    R = (1 / inertia) * (1 - imp) / imp
+    # fp32 state: the penetration is ~1e-4 rad on an angle of 0.3, so it is resolved to about three digits
+    assert (1 / R) * k * imp * abs(pos) == pytest.approx(mass * 9.81 * (L / 2) * np.sin(q), rel=5e-3)

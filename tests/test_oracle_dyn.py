@@ -420,3 +420,123 @@ def test_contact_forces_on_bodies(model):
     ob_.forward(db)
     np.testing.assert_allclose(np.array(db.cfrc_ext)[1, 3:], [0, 0, 2.0 * 9.81], atol=2e-3)
     np.testing.assert_allclose(np.array(db.cfrc_ext)[1, :3], 0, atol=1e-9)  # the contact point lies under the centre
+
+
+# --------------------------------------------------------------------------- joint limits and dry joint friction
+def _impedance(m, pos):
+    dmin, dmax, width, mid, power = m.solimp
+    x = abs(pos) / width
+    y = (1 / mid ** (power - 1)) * x**power if x < mid else 1 - (1 / (1 - mid) ** (power - 1)) * (1 - x) ** power
+    return dmax if x > 1 else float(np.clip(dmin + y * (dmax - dmin), dmin, dmax))
+
+
+def _cost_rows(d, a):
+    """The convex cost whose minimiser the solver returns, with the saturating (Huber) term of friction rows."""
+    x = d.efc_J @ a - d.efc_aref
+    da = a - d.qacc_smooth
+    fl, D = np.array(d.efc_floss), np.array(d.efc_D)
+    rf = np.where(fl > 0, fl / D, 0.0)
+    quad = 0.5 * D * x**2
+    s = np.where(fl > 0, np.where(x <= -rf, fl * (-0.5 * rf - x), np.where(x >= rf, fl * (-0.5 * rf + x), quad)),
+                 np.where(x < 0, quad, 0.0))
+    return 0.5 * da @ d.M @ da + s.sum()
+
+
+@pytest.mark.parametrize("name", ["humanoid", "kbot"])
+def test_limit_and_friction_rows_fixed_point_and_scipy(name):
+    """Rows of violated joint limits (J = +-e_j) and of dry friction (J = e_j, force clipped at +-frictionloss) next to
+    the contact rows: the solver's point satisfies the stationarity condition of the cost and no independent minimiser
+    of that cost does better."""
+    m = MODELS[name](joint_range=(-0.4, 0.6), frictionloss=0.3)
+    rng = np.random.default_rng(12)
+    a = dict(m.arrays()); a["iterations"] = 100; a["ls_iterations"] = 50
+    orc = Oracle(a)
+    qpos, qvel = _random_state(m, rng, vel_scale=0.5)  # hinges ~U(-1, 1): many beyond (-0.4, 0.6)
+    qpos = _sink_to_contact(m, qpos)
+    d = orc.data(qpos, qvel)
+    d.ctrl = rng.normal(size=m.nu)
+    orc.forward(d)
+    nh = m.nv - 6
+    hinge_q = qpos[7:]
+    n_lim = int(((hinge_q < -0.4) | (hinge_q > 0.6)).sum())
+    n_con = int((np.array(d.con_dist) < 0).sum())
+    assert n_lim > 3 and n_con > 0
+    assert d.nefc == 4 * n_con + n_lim + nh
+    # limit rows: one entry, +1 below the range and -1 above it, pos = the violation
+    for r in range(4 * n_con, 4 * n_con + n_lim):
+        row = d.efc_J[r]
+        j = int(np.flatnonzero(row)[0])
+        assert np.count_nonzero(row) == 1
+        q = qpos[7 + j - 6]
+        assert (row[j], d.efc_pos[r]) == ((1.0, pytest.approx(q + 0.4)) if q < -0.4 else (-1.0, pytest.approx(0.6 - q)))
+        imp = _impedance(m, d.efc_pos[r])
+        assert d.efc_D[r] == pytest.approx(imp / (m.dof_invweight0[j] * (1 - imp)), rel=1e-12)
+    acc = np.array(d.qacc)
+    x = d.efc_J @ acc - d.efc_aref
+    fl, D = np.array(d.efc_floss), np.array(d.efc_D)
+    f = np.where(fl > 0, np.clip(-D * x, -fl, fl), np.where(x < 0, -D * x, 0.0))
+    np.testing.assert_allclose(d.efc_force, f, rtol=1e-9, atol=1e-9)
+    assert (np.abs(f[fl > 0]) <= 0.3 + 1e-12).all() and np.isclose(np.abs(f[fl > 0]), 0.3, rtol=1e-12).any()
+    resid = d.M @ (acc - d.qacc_smooth) - d.efc_J.T @ f
+    assert np.abs(resid).max() < 1e-7 * max(1.0, np.abs(d.M @ acc).max())
+    res = minimize(lambda v: _cost_rows(d, v), np.array(d.qacc_smooth), method="BFGS", options=dict(gtol=1e-9, maxiter=20000))
+    assert _cost_rows(d, acc) <= res.fun + 1e-9 * max(1.0, abs(res.fun))
+
+
+def test_pendulum_rests_on_its_limit_where_the_spring_predicts():
+    """One link on a horizontal hinge, range (0.3, 1.0): gravity pulls it towards 0 and it settles just below 0.3,
+    where the limit force D k imp |pos| balances the gravity torque m g (L/2) sin q."""
+    L, mass = 0.5, 1.0
+    m = km.pendulum_chain_model(n_links=1, length=L, mass=mass, damping=0.5, joint_range=(0.3, 1.0))
+    orc = Oracle(m.arrays())
+    d = orc.data(np.array([0.6]), np.zeros(1))
+    for _ in range(4000):
+        orc.step(d)
+    assert abs(d.qvel[0]) < 1e-7
+    q = float(d.qpos[0])
+    pos = q - 0.3
+    assert -0.01 < pos < 0
+    tc = max(m.solref[0], 2 * m.dt)
+    k = 1 / (m.solimp[1] ** 2 * tc**2 * m.solref[1] ** 2)
+    imp = _impedance(m, pos)
+    inertia = float(d.M[0, 0])  # the hinge's inertia, pinned against the Jacobian sum elsewhere
+    assert m.dof_invweight0[0] == pytest.approx(1 / inertia)
+    R = (1 / inertia) * (1 - imp) / imp
+    assert (1 / R) * k * imp * abs(pos) == pytest.approx(mass * 9.81 * (L / 2) * np.sin(q), rel=1e-6)
+    # inside the range the limit does nothing
+    free = km.pendulum_chain_model(n_links=1, length=L, mass=mass, damping=0.5)
+    a, b = orc.data(np.array([0.7]), np.array([0.1])), Oracle(free.arrays()).data(np.array([0.7]), np.array([0.1]))
+    orc.forward(a); Oracle(free.arrays()).forward(b)
+    assert a.nefc == 0 and a.qacc[0] == b.qacc[0]
+
+
+def test_dry_friction_closed_forms():
+    """A hinge without gravity or damping and frictionloss f.  Moving fast it decelerates at exactly f / I; pushed
+    from rest by a torque below f it (almost) sticks: a = tau / (I + D) with the row's stiffness D = 1 / R."""
+    f = 0.4
+    m = km.pendulum_chain_model(n_links=1, damping=0.0, frictionloss=f, gravity=(0.0, 0.0, 0.0))
+    orc = Oracle(m.arrays())
+    d = orc.data(np.zeros(1), np.array([2.0]))
+    orc.forward(d)
+    inertia = float(d.M[0, 0])
+    assert d.nefc == 1 and d.efc_force[0] == pytest.approx(-f)
+    assert d.qacc[0] == pytest.approx(-f / inertia, rel=1e-9)
+    v = [2.0]
+    for _ in range(10):
+        orc.step(d); v.append(float(d.qvel[0]))
+    np.testing.assert_allclose(np.diff(v), -m.dt * f / inertia, rtol=1e-9)
+    for _ in range(3000):
+        orc.step(d)
+    assert abs(d.qvel[0]) < 1e-9  # it stops and stays stopped
+    # opposite direction: the force flips
+    d2 = orc.data(np.zeros(1), np.array([-2.0])); orc.forward(d2)
+    assert d2.qacc[0] == pytest.approx(f / inertia, rel=1e-9)
+    # stiction: torque below the friction level
+    d3 = orc.data(np.zeros(1), np.zeros(1)); d3.ctrl = np.array([0.25]); orc.forward(d3)
+    imp = _impedance(m, 0.0)
+    D = 1 / ((1 / inertia) * (1 - imp) / imp)
+    assert d3.qacc[0] == pytest.approx(0.25 / (inertia + D), rel=1e-8)
+    assert abs(d3.efc_force[0]) < f
+    # above it the joint accelerates with the excess
+    d4 = orc.data(np.zeros(1), np.zeros(1)); d4.ctrl = np.array([1.0]); orc.forward(d4)
+    assert d4.qacc[0] == pytest.approx((1.0 - f) / inertia, rel=1e-8)
