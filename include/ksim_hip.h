@@ -499,6 +499,12 @@ int ks_mlp_destroy(KsMlp* mlp);
 int64_t ks_mlp_workspace_bytes(const KsMlp* mlp, int64_t M);
 int ks_mlp_forward(const KsMlp* mlp, ks_stream_t stream, int64_t M, const float* x /*(M, in)*/,
                    float* y /*(M, out)*/, void* workspace);
+/* Two networks over the same M rows, e.g. the actor on the noisy observations and the critic on the clean ones
+ * (ksim/task/rl.py:892-926 and the value call of examples/walking.py:626-638, which XLA schedules side by side).  Same
+ * results as two ks_mlp_forward calls; when both networks run as whole-network kernels with one activation and M is
+ * below 16384 they share a single launch, so the second network's workgroups overlap the first one's. */
+int ks_mlp_forward_pair(const KsMlp* mlp0, const KsMlp* mlp1, ks_stream_t stream, int64_t M, const float* x0,
+                        float* y0, const float* x1, float* y1, void* workspace0, void* workspace1);
 
 /* ------------------------------------------------------------------ GRU cell (recurrent policies, forward)
  * The recurrent actors / critics of the shipped examples (examples/walking.py:40-208: input projection, a stack of

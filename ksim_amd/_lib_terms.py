@@ -184,6 +184,8 @@ def bind(lib) -> None:
     lib.ks_mlp_workspace_bytes.argtypes = [c_void_p, c_int64]
     lib.ks_mlp_workspace_bytes.restype = c_int64
     lib.ks_mlp_forward.argtypes = [c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_void_p]
+    lib.ks_mlp_forward_pair.argtypes = [c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p,
+                                        c_void_p, c_void_p]
     lib.ks_mlp_train_init.argtypes = [c_void_p]
     lib.ks_mlp_train_workspace_bytes.argtypes = [c_void_p, c_int64]
     lib.ks_mlp_train_workspace_bytes.restype = c_int64
@@ -199,5 +201,5 @@ def bind(lib) -> None:
                  "ks_mlp_grad_sqnorm", "ks_mlp_adam_step", "ks_adam_step", "ks_mlp_get_params", "ks_gaussian_log_prob"):
         getattr(lib, name).restype = c_int32
     for name in ("ks_terms_create", "ks_terms_destroy", "ks_observe", "ks_terminate_reset", "ks_sample_action",
-                 "ks_mlp_create", "ks_mlp_destroy", "ks_mlp_forward"):
+                 "ks_mlp_create", "ks_mlp_destroy", "ks_mlp_forward", "ks_mlp_forward_pair"):
         getattr(lib, name).restype = c_int32

@@ -400,8 +400,7 @@ __device__ __forceinline__ void fused_layer(const FusedArgs& a, int l, __bf16* _
 }
 
 template <int ACT, int BM>
-__global__ __launch_bounds__(64 * kFusedWaves) __attribute__((amdgpu_waves_per_eu(BM <= 64 ? 4 : 2, BM <= 64 ? 4 : 2)))
-void mlp_fused_kernel(const FusedArgs a) {
+__device__ __forceinline__ void mlp_fused_body(const FusedArgs& a) {
   constexpr int MI = BM / 32;
   constexpr int NTHR = 64 * kFusedWaves;
   extern __shared__ __attribute__((aligned(16))) unsigned char mlp_lds[];
@@ -469,6 +468,21 @@ void mlp_fused_kernel(const FusedArgs a) {
     fused_layer<ACT, MI, false>(a, l, act, m0, lane, wave);
   }
   fused_layer<ACT, MI, true>(a, a.n_layers - 1, act, m0, lane, wave);
+}
+
+template <int ACT, int BM>
+__global__ __launch_bounds__(64 * kFusedWaves) __attribute__((amdgpu_waves_per_eu(BM <= 64 ? 4 : 2, BM <= 64 ? 4 : 2)))
+void mlp_fused_kernel(const FusedArgs a) {
+  mlp_fused_body<ACT, BM>(a);
+}
+
+// Two networks over the same rows in one launch (actor and critic of a control step): blockIdx.y picks the network, so
+// the second network's workgroups fill the CUs next to the first one's instead of waiting for their launch to drain.
+template <int ACT, int BM>
+__global__ __launch_bounds__(64 * kFusedWaves) __attribute__((amdgpu_waves_per_eu(BM <= 64 ? 4 : 2, BM <= 64 ? 4 : 2)))
+void mlp_fused_pair_kernel(const FusedArgs a, const FusedArgs b) {
+  if (blockIdx.y == 0) mlp_fused_body<ACT, BM>(a);
+  else mlp_fused_body<ACT, BM>(b);
 }
 
 struct DevMlp {
@@ -852,8 +866,7 @@ extern "C" int ks_mlp_destroy(KsMlp* h) {
   return KS_OK;
 }
 
-template <int BM>
-static int launch_fused_tile(const DevMlp& m, hipStream_t s, int64_t M, const float* x, float* y) {
+static FusedArgs fused_args(const DevMlp& m, int64_t M, const float* x, float* y) {
   FusedArgs a;
   std::memset(&a, 0, sizeof(a));
   a.M = M; a.n_layers = m.n_layers; a.in_dim = m.dims[0]; a.out_dim = m.dims[m.n_layers]; a.lda = m.lda;
@@ -862,6 +875,12 @@ static int launch_fused_tile(const DevMlp& m, hipStream_t s, int64_t M, const fl
     a.Wp[l] = (const u32x4*)m.Wp[l]; a.bp[l] = m.bp[l];
   }
   a.x = x; a.y = y;
+  return a;
+}
+
+template <int BM>
+static int launch_fused_tile(const DevMlp& m, hipStream_t s, int64_t M, const float* x, float* y) {
+  FusedArgs a = fused_args(m, M, x, y);
 #ifdef KS_PROFILE
   if (const char* e = getenv("KS_MLP_PROF_PTR")) a.prof = (long long*)strtoull(e, nullptr, 16);
 #endif
@@ -901,6 +920,48 @@ static int launch_fused(const DevMlp& m, hipStream_t s, int64_t M, const float* 
   if (M >= 128 * 256) return launch_fused_tile<128>(m, s, M, x, y);
   if (M >= 64 * 256) return launch_fused_tile<64>(m, s, M, x, y);
   return launch_fused_tile<32>(m, s, M, x, y);
+}
+
+template <int BM>
+static int launch_fused_pair_tile(const DevMlp& m0, const DevMlp& m1, hipStream_t s, int64_t M, const float* x0, float* y0,
+                                  const float* x1, float* y1) {
+  const FusedArgs a = fused_args(m0, M, x0, y0), b = fused_args(m1, M, x1, y1);
+  const int lds = BM * (m0.lda > m1.lda ? m0.lda : m1.lda) * 2;
+  const int64_t blocks = (M + BM - 1) / BM;
+  if (blocks > 0x7fffffff) return fail(KS_ELIMIT, "ks_mlp_forward_pair: too many rows");
+#define KS_LAUNCH(A)                                                                                           \
+  {                                                                                                            \
+    auto kfn = mlp_fused_pair_kernel<A, BM>;                                                                   \
+    if (lds > 64 * 1024 &&                                                                                     \
+        hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)  \
+      return fail(KS_ELAUNCH, "ks_mlp_forward_pair: cannot raise the LDS limit to %d bytes", lds);             \
+    hipLaunchKernelGGL(kfn, dim3((unsigned)blocks, 2), dim3(64 * kFusedWaves), lds, s, a, b);                  \
+  }
+  switch (m0.activation) {
+    case KS_ACT_ELU: KS_LAUNCH(KS_ACT_ELU) break;
+    case KS_ACT_RELU: KS_LAUNCH(KS_ACT_RELU) break;
+    case KS_ACT_TANH: KS_LAUNCH(KS_ACT_TANH) break;
+    case KS_ACT_GELU: KS_LAUNCH(KS_ACT_GELU) break;
+    default: KS_LAUNCH(KS_ACT_NONE) break;
+  }
+#undef KS_LAUNCH
+  return check_launch("ks_mlp_forward_pair");
+}
+
+extern "C" int ks_mlp_forward_pair(const KsMlp* h0, const KsMlp* h1, ks_stream_t stream, int64_t M, const float* x0,
+                                   float* y0, const float* x1, float* y1, void* workspace0, void* workspace1) {
+  if (!h0 || !h1) return fail(KS_EINVAL, "ks_mlp_forward_pair: null handle");
+  if (M < 0) return fail(KS_EINVAL, "ks_mlp_forward_pair: negative row count");
+  if (M == 0) return KS_OK;
+  if (!x0 || !y0 || !x1 || !y1) return fail(KS_EINVAL, "ks_mlp_forward_pair: null pointer");
+  if (y0 == y1) return fail(KS_EINVAL, "ks_mlp_forward_pair: the two outputs must differ");
+  hipStream_t s = (hipStream_t)stream;
+  // one launch when both networks run as whole-network kernels with the same activation and row tile; else one each
+  if (h0->m.fused && h1->m.fused && h0->m.activation == h1->m.activation && M < 64 * 256)
+    return launch_fused_pair_tile<32>(h0->m, h1->m, s, M, x0, y0, x1, y1);
+  const int rc = ks_mlp_forward(h0, stream, M, x0, y0, workspace0);
+  if (rc != KS_OK) return rc;
+  return ks_mlp_forward(h1, stream, M, x1, y1, workspace1);
 }
 
 extern "C" int64_t ks_mlp_workspace_bytes(const KsMlp* h, int64_t M) {

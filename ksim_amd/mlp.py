@@ -82,6 +82,20 @@ class MLP:
                                             _lib.ptr(ws)))
         return out
 
+    def forward_pair(self, x: torch.Tensor, out: torch.Tensor, other: "MLP", x_other: torch.Tensor,
+                     out_other: torch.Tensor) -> None:
+        """This network on ``x`` and ``other`` on ``x_other`` (same row count), in one launch when the library can."""
+        M = x.shape[0]
+        for net, a, o in ((self, x, out), (other, x_other, out_other)):
+            _lib.require_cuda(a, dtype=torch.float32)
+            _lib.require_cuda(o, dtype=torch.float32)
+            if tuple(a.shape) != (M, net.in_dim) or tuple(o.shape) != (M, net.out_dim):
+                raise _lib.KsError(f"expected input (M, {net.in_dim}) and output (M, {net.out_dim})")
+        _lib.check(self._lib.ks_mlp_forward_pair(self._handle, other._handle, _lib.current_stream(), M, _lib.ptr(x),
+                                                 _lib.ptr(out), _lib.ptr(x_other), _lib.ptr(out_other),
+                                                 _lib.ptr(self.workspace(M, x.device)),
+                                                 _lib.ptr(other.workspace(M, x.device))))
+
     # ------------------------------------------------------------------ training (ksim/task/ppo.py:495-565)
     def train_init(self) -> None:
         """fp32 master weights, gradients and Adam moments beside the working copies."""

@@ -109,14 +109,18 @@ class Rollout:
                         carry_uniform=noise.get("obs_carry_uniform"))
         # actor reads the noisy copy (walking.py:592-595), critic the clean one (walking.py:626-638); recurrent networks
         # advance their carries, which restart from zero for the envs the previous control step reset
-        if isinstance(c.actor, RecurrentNetwork):
-            c.actor(self.noisy_obs[t], env.actor_carry, fresh=self.reset_mask, out=self.mean)
+        if isinstance(c.actor, MLP) and isinstance(c.critic, MLP):
+            # two plain MLPs over the same rows share one launch
+            c.actor.forward_pair(self.noisy_obs[t], self.mean, c.critic, self.obs[t], self.values[t])
         else:
-            c.actor(self.noisy_obs[t], out=self.mean)
-        if isinstance(c.critic, RecurrentNetwork):
-            c.critic(self.obs[t], env.critic_carry, fresh=self.reset_mask, out=self.values[t])
-        elif c.critic is not None:
-            c.critic(self.obs[t], out=self.values[t])
+            if isinstance(c.actor, RecurrentNetwork):
+                c.actor(self.noisy_obs[t], env.actor_carry, fresh=self.reset_mask, out=self.mean)
+            else:
+                c.actor(self.noisy_obs[t], out=self.mean)
+            if isinstance(c.critic, RecurrentNetwork):
+                c.critic(self.obs[t], env.critic_carry, fresh=self.reset_mask, out=self.values[t])
+            elif c.critic is not None:
+                c.critic(self.obs[t], out=self.values[t])
         sample_action(self.mean, c.log_std, noise=noise.get("action_normal"), seed=env.seed, step=step,
                       step_base=step_base, clip_max=c.action_clip_max, out=self.action[t])
         # the step kernel also writes ctrl / xpos / xquat of the post-step data into the transition slot

@@ -66,3 +66,24 @@ def test_mlp_rows_are_independent_and_errors():
     with pytest.raises(_lib.KsError):
         net(torch.randn(4, 68))
     assert net(torch.empty(0, 68, device=DEV)).shape == (0, 20)
+
+
+@pytest.mark.parametrize("M", [8192, 777, 20000])
+def test_paired_forward_equals_two_single_forwards(M):
+    """Actor and critic over the same rows in one launch (below 16384 rows) or two: bit-identical to separate calls,
+    also for networks of different widths and for a pair that cannot share a launch."""
+    from ksim_amd import _lib
+    from ksim_amd.mlp import random_mlp
+
+    actor, _, _ = random_mlp((68, 512, 512, 512, 20), seed=5)
+    critic, _, _ = random_mlp((68, 512, 512, 512, 1), seed=6)
+    narrow, _, _ = random_mlp((68, 256, 256, 1), seed=7)
+    wide, _, _ = random_mlp((68, 1024, 1), seed=8)  # per-layer path: the pair falls back to two launches
+    x0, x1 = torch.randn(M, 68, device=DEV), torch.randn(M, 68, device=DEV)
+    for other in (critic, narrow, wide):
+        y0 = torch.full((M, 20), 7.0, device=DEV)
+        y1 = torch.full((M, 1), 7.0, device=DEV)
+        actor.forward_pair(x0, y0, other, x1, y1)
+        assert torch.equal(y0, actor(x0)) and torch.equal(y1, other(x1))
+    with pytest.raises(_lib.KsError):
+        actor.forward_pair(x0, torch.empty(M, 20, device=DEV), critic, x1[:-1], torch.empty(M - 1, 1, device=DEV))
