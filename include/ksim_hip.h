@@ -33,7 +33,8 @@ const char* ks_last_error(void);
 /* sizeof() of a public struct as this library was compiled, for binding self-checks:
  * 0 KsPpoLossParams, 1 KsModelDesc, 2 KsStepIO, 3 KsTermsDesc, 4 KsObserveIO, 5 KsTerminateIO, 6 KsMlpDesc,
  * 7 KsRewardIO, 8 KsObsElem, 9 KsTermDesc, 10 KsRewardDesc, 11 KsRng, 12 KsAdamParams, 13 KsEventDesc,
- * 14 KsRewardScanIO, 15 KsRewardScanDesc, 16 KsGruDesc, 17 KsLstmDesc, 18 KsGaussianHead, 19 KsCommandIO;
+ * 14 KsRewardScanIO, 15 KsRewardScanDesc, 16 KsGruDesc, 17 KsLstmDesc, 18 KsGaussianHead, 19 KsCommandIO,
+ * 20 KsMixtureHead;
  * -1 for anything else. */
 int64_t ks_abi_sizeof(int32_t which);
 
@@ -470,6 +471,29 @@ int ks_sample_action_head(ks_stream_t stream, int64_t N, int32_t nu, const float
                           const KsGaussianHead* head /*host*/, const float* noise_normal /*(N,nu) nullable -> Philox*/,
                           KsRng rng, float clip_max, float* action /*(N,nu)*/, float* mean_out /*nullable*/,
                           float* std_out /*nullable*/, float* log_prob_out /*(N,nu) nullable*/);
+
+/* Mixture-of-Gaussians head of the walking example's actor (examples/walking.py:127-144): raw is (N, 3 nu K) = component
+ * means (nu, K), raw deviations (nu, K), logits (nu, K) per env.  mean = clip(raw_mean + mean_bias, clip_lo, clip_hi)
+ * (zero bias and ClipPositions, walking.py:138-142), std = min((softplus(raw_std) + min_std) * var_scale, max_std).  Per
+ * action dimension one component is drawn from softmax(logits) with the uniform draw u (first k whose cumulative
+ * probability exceeds u), then action = mean_k + std_k * z; log_prob = logsumexp_k(log softmax(logits)_k + log N(action;
+ * mean_k, std_k)) of the sample before the NaN scrub and clip.  deterministic: the mean of the most probable component.
+ * The distribution itself (xax.MixtureOfGaussians) is a third-party class that is not part of the reference tree; this
+ * is the textbook mixture. */
+#define KS_MAX_MIXTURES 8
+typedef struct KsMixtureHead {
+  int32_t num_mixtures;   /* K in 1..KS_MAX_MIXTURES */
+  float min_std, max_std, var_scale;
+  int32_t deterministic;
+  const float* mean_bias; /* device (nu), nullable */
+  const float* clip_lo;   /* device (nu), nullable (then clip_hi must be NULL too) */
+  const float* clip_hi;
+} KsMixtureHead;
+int ks_sample_action_mixture(ks_stream_t stream, int64_t N, int32_t nu, const float* raw /*(N, 3 nu K)*/,
+                             const KsMixtureHead* head /*host*/, const float* uniform /*(N,nu) nullable -> Philox*/,
+                             const float* noise_normal /*(N,nu) nullable -> Philox*/, KsRng rng, float clip_max,
+                             float* action /*(N,nu)*/, float* log_prob_out /*(N,nu) nullable*/,
+                             int32_t* component_out /*(N,nu) nullable*/);
 
 /* ------------------------------------------------------------------ policy / critic / discriminator MLP
  * The dense contraction of the path: the network a task's sample_action calls

@@ -141,6 +141,11 @@ class KsGaussianHead(ctypes.Structure):
                 ("mean_bias", c_void_p)]
 
 
+class KsMixtureHead(ctypes.Structure):
+    _fields_ = [("num_mixtures", c_int32), ("min_std", c_float), ("max_std", c_float), ("var_scale", c_float),
+                ("deterministic", c_int32), ("mean_bias", c_void_p), ("clip_lo", c_void_p), ("clip_hi", c_void_p)]
+
+
 class KsLstmDesc(ctypes.Structure):
     _fields_ = [("input_size", c_int32), ("hidden_size", c_int32), ("dtype", c_int32), ("weight_ih", c_void_p),
                 ("weight_hh", c_void_p), ("bias", c_void_p)]
@@ -179,6 +184,9 @@ def bind(lib) -> None:
     lib.ks_sample_action_head.argtypes = [c_void_p, c_int64, c_int32, c_void_p, POINTER(KsGaussianHead), c_void_p, KsRng,
                                           c_float, c_void_p, c_void_p, c_void_p, c_void_p]
     lib.ks_sample_action_head.restype = c_int32
+    lib.ks_sample_action_mixture.argtypes = [c_void_p, c_int64, c_int32, c_void_p, POINTER(KsMixtureHead), c_void_p, c_void_p,
+                                             KsRng, c_float, c_void_p, c_void_p, c_void_p]
+    lib.ks_sample_action_mixture.restype = c_int32
     lib.ks_mlp_create.argtypes = [POINTER(KsMlpDesc), POINTER(c_void_p)]
     lib.ks_mlp_destroy.argtypes = [c_void_p]
     lib.ks_mlp_workspace_bytes.argtypes = [c_void_p, c_int64]

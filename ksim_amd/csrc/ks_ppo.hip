@@ -333,6 +333,7 @@ extern "C" int64_t ks_abi_sizeof(int32_t which) {
     case 17: return sizeof(KsLstmDesc);
     case 18: return sizeof(KsGaussianHead);
     case 19: return sizeof(KsCommandIO);
+    case 20: return sizeof(KsMixtureHead);
     default: return -1;
   }
 }

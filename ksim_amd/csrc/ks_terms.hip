@@ -331,6 +331,88 @@ __global__ __launch_bounds__(256) void sample_action_head_kernel(int64_t n, int 
   action[idx] = a;
 }
 
+// Mixture-of-Gaussians head: one lane per (env, action dimension) walks its K components three times (softmax
+// normaliser, component pick by inverse CDF, log-density of the sample), all in registers.
+__global__ __launch_bounds__(256) void sample_action_mixture_kernel(int64_t n, int nu, const float* __restrict__ raw,
+                                                                    KsMixtureHead hd, const float* __restrict__ uniform,
+                                                                    const float* __restrict__ noise, KsRng rng,
+                                                                    float clip_max, float* __restrict__ action,
+                                                                    float* __restrict__ logp_out, int* __restrict__ comp_out) {
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= n) return;
+  const int64_t e = idx / nu;
+  const int u = (int)(idx - e * nu);
+  const int K = hd.num_mixtures;
+  const float* rm = raw + e * 3 * nu * K + (int64_t)u * K;
+  const float* rs = rm + (int64_t)nu * K;
+  const float* rl = rs + (int64_t)nu * K;
+  const float bias = hd.mean_bias ? hd.mean_bias[u] : 0.f;
+  const float lo = hd.clip_lo ? hd.clip_lo[u] : -INFINITY, hi = hd.clip_hi ? hd.clip_hi[u] : INFINITY;
+  float mean[KS_MAX_MIXTURES], sd[KS_MAX_MIXTURES], lg[KS_MAX_MIXTURES];
+  float lmax = -INFINITY;
+  int best = 0;
+#pragma unroll
+  for (int k = 0; k < KS_MAX_MIXTURES; ++k) {
+    if (k < K) {
+      mean[k] = fminf(fmaxf(rm[k] + bias, lo), hi);
+      const float r = rs[k];
+      const float sp = r > 20.f ? r : log1pf(expf(r));
+      sd[k] = fminf((sp + hd.min_std) * hd.var_scale, hd.max_std);
+      lg[k] = rl[k];
+      if (lg[k] > lmax) { lmax = lg[k]; best = k; }
+    } else {
+      mean[k] = 0.f; sd[k] = 1.f; lg[k] = -INFINITY;
+    }
+  }
+  float zsum = 0.f;
+#pragma unroll
+  for (int k = 0; k < KS_MAX_MIXTURES; ++k) zsum += k < K ? expf(lg[k] - lmax) : 0.f;
+  const float lse = lmax + logf(zsum);  // log of the softmax normaliser
+  float uu = 0.f, z = 0.f;
+  int pick = best;
+  if (!hd.deterministic) {
+    if (uniform && noise) { uu = uniform[idx]; z = noise[idx]; }
+    else {
+      const Philox4 p = draw(rng.seed, rng.step + (rng.step_base ? *rng.step_base : 0ull), kRngAction, (uint64_t)e, (uint32_t)u);
+      z = noise ? noise[idx] : normal_from(p.x, p.y);
+      uu = uniform ? uniform[idx] : u01(p.z);
+    }
+    // inverse CDF: the first component whose cumulative probability exceeds the draw (the last one on rounding)
+    float cum = 0.f;
+    pick = K - 1;
+    bool found = false;
+#pragma unroll
+    for (int k = 0; k < KS_MAX_MIXTURES; ++k) {
+      if (k < K) {
+        cum += expf(lg[k] - lse);
+        if (!found && cum > uu) { pick = k; found = true; }
+      }
+    }
+  }
+  float pm = 0.f, ps = 1.f;
+#pragma unroll
+  for (int k = 0; k < KS_MAX_MIXTURES; ++k)
+    if (k == pick) { pm = mean[k]; ps = sd[k]; }
+  float a = hd.deterministic ? pm : pm + ps * z;
+  if (logp_out) {
+    float t[KS_MAX_MIXTURES], tmax = -INFINITY;
+#pragma unroll
+    for (int k = 0; k < KS_MAX_MIXTURES; ++k) {
+      const float d = (a - mean[k]) / sd[k];
+      t[k] = k < K ? (lg[k] - lse) - 0.5f * d * d - logf(sd[k]) - 0.91893853320467274178f : -INFINITY;
+      tmax = fmaxf(tmax, t[k]);
+    }
+    float acc = 0.f;
+#pragma unroll
+    for (int k = 0; k < KS_MAX_MIXTURES; ++k) acc += k < K ? expf(t[k] - tmax) : 0.f;
+    logp_out[idx] = tmax + logf(acc);
+  }
+  if (comp_out) comp_out[idx] = pick;
+  if (a != a) a = 0.f;
+  a = fminf(fmaxf(a, -clip_max), clip_max);
+  action[idx] = a;
+}
+
 // ---------------------------------------------------------------------------------------------
 // Rewards over a time-major rollout.  One lane per (t, env).
 // Action differences follow rewards.py:410-460: v(t) = a[t]-a[t-1], A(t) = v(t)-v(t-1),
@@ -751,6 +833,26 @@ extern "C" int ks_sample_action_head(ks_stream_t stream, int64_t N, int32_t nu, 
   hipLaunchKernelGGL(sample_action_head_kernel, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, n, (int)nu, raw, *head,
                      noise_normal, rng, clip_max, action, mean_out, std_out, log_prob_out);
   return check_launch("ks_sample_action_head");
+}
+
+extern "C" int ks_sample_action_mixture(ks_stream_t stream, int64_t N, int32_t nu, const float* raw, const KsMixtureHead* head,
+                                        const float* uniform, const float* noise_normal, KsRng rng, float clip_max,
+                                        float* action, float* log_prob_out, int32_t* component_out) {
+  using namespace ks;
+  if (N < 0 || nu < 1) return fail(KS_EINVAL, "ks_sample_action_mixture: bad sizes");
+  if (N == 0) return KS_OK;
+  if (!raw || !head || !action) return fail(KS_EINVAL, "ks_sample_action_mixture: null pointer");
+  if (head->num_mixtures < 1 || head->num_mixtures > KS_MAX_MIXTURES)
+    return fail(KS_ELIMIT, "ks_sample_action_mixture: %d components, 1..%d are built", head->num_mixtures, KS_MAX_MIXTURES);
+  if (!(head->max_std > 0.f) || head->min_std < 0.f || !(head->var_scale > 0.f))
+    return fail(KS_EINVAL, "ks_sample_action_mixture: bad deviation bounds");
+  if ((head->clip_lo == nullptr) != (head->clip_hi == nullptr)) return fail(KS_EINVAL, "ks_sample_action_mixture: clip_lo and clip_hi come together");
+  if (!(clip_max > 0.f)) return fail(KS_EINVAL, "ks_sample_action_mixture: clip_max must be positive");
+  const int64_t n = N * nu, grid = (n + 255) / 256;
+  if (grid > 0x7fffffff) return fail(KS_ELIMIT, "ks_sample_action_mixture: too many elements");
+  hipLaunchKernelGGL(sample_action_mixture_kernel, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, n, (int)nu, raw, *head,
+                     uniform, noise_normal, rng, clip_max, action, log_prob_out, component_out);
+  return check_launch("ks_sample_action_mixture");
 }
 
 extern "C" int ks_rewards(ks_stream_t stream, const KsRewardIO* io) {

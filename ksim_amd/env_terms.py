@@ -245,3 +245,36 @@ def sample_action_head(raw: torch.Tensor, *, min_std: float, max_std: float, var
     _lib.check(lib.ks_sample_action_head(_lib.current_stream(), N, nu, _lib.ptr(raw), ctypes.byref(head), _lib.ptr(noise),
                                          _rng(seed, step, step_base), float(clip_max), _lib.ptr(out), *(_lib.ptr(t) for t in stats)))
     return (out, *stats) if want_stats else out
+
+
+def sample_action_mixture(raw: torch.Tensor, num_mixtures: int, *, min_std: float, max_std: float, var_scale: float = 1.0,
+                          mean_bias: torch.Tensor | None = None, clip_lo: torch.Tensor | None = None,
+                          clip_hi: torch.Tensor | None = None, uniform: torch.Tensor | None = None,
+                          noise: torch.Tensor | None = None, deterministic: bool = False, seed: int = 0, step: int = 0,
+                          step_base=None, clip_max: float = 1e3, out: torch.Tensor | None = None, want_stats: bool = False):
+    """Sampling tail of the walking example's actor (examples/walking.py:127-144): `raw` (N, 3 nu K) holds component means,
+    raw deviations and logits, each (nu, K).  One component per action dimension is drawn from softmax(logits), the action
+    from that component's Gaussian; scrub and clip as ksim/task/rl.py:998-1001.  With `want_stats` also returns the
+    per-dimension log-probability of the sample under the mixture and the component drawn."""
+    lib = _lib.load()
+    _lib.require_cuda(raw, mean_bias, clip_lo, clip_hi, uniform, noise, out, dtype=torch.float32)
+    K = int(num_mixtures)
+    if raw.dim() != 2 or K < 1 or raw.shape[1] % (3 * K):
+        raise _lib.KsError("raw must be (N, 3 nu K)")
+    N, nu = raw.shape[0], raw.shape[1] // (3 * K)
+    for name, t, shape in (("mean_bias", mean_bias, (nu,)), ("clip_lo", clip_lo, (nu,)), ("clip_hi", clip_hi, (nu,)),
+                           ("uniform", uniform, (N, nu)), ("noise", noise, (N, nu))):
+        if t is not None and tuple(t.shape) != shape:
+            raise _lib.KsError(f"{name} must have shape {shape}")
+    if out is None:
+        out = torch.empty((N, nu), dtype=torch.float32, device=raw.device)
+    elif tuple(out.shape) != (N, nu):
+        raise _lib.KsError("out must be (N, nu)")
+    logp = torch.empty((N, nu), dtype=torch.float32, device=raw.device) if want_stats else None
+    comp = torch.empty((N, nu), dtype=torch.int32, device=raw.device) if want_stats else None
+    head = T.KsMixtureHead(K, float(min_std), float(max_std), float(var_scale), int(bool(deterministic)),
+                           _lib.ptr(mean_bias).value, _lib.ptr(clip_lo).value, _lib.ptr(clip_hi).value)
+    _lib.check(lib.ks_sample_action_mixture(_lib.current_stream(), N, nu, _lib.ptr(raw), ctypes.byref(head), _lib.ptr(uniform),
+                                            _lib.ptr(noise), _rng(seed, step, step_base), float(clip_max), _lib.ptr(out),
+                                            _lib.ptr(logp), _lib.ptr(comp)))
+    return (out, logp, comp) if want_stats else out

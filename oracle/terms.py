@@ -420,3 +420,38 @@ def position_velocity_actuator_torque(action, qpos, qvel, kp, kd, ctrl_clip, pos
     target_pos, target_vel = action[:n] + pos_noise, action[n:] + vel_noise
     ctrl = np.asarray(kp) * (target_pos - qpos) + np.asarray(kd) * (target_vel - qvel)
     return np.clip(ctrl + torque_noise, -np.asarray(ctrl_clip), np.asarray(ctrl_clip))
+
+
+def mixture_head(raw, num_mixtures, *, min_std, max_std, var_scale=1.0, mean_bias=None, clip_lo=None, clip_hi=None,
+                 uniform=None, normal=None, deterministic=False, clip_max=1e3):
+    """Mixture-of-Gaussians actor head (examples/walking.py:127-144): raw (N, 3 nu K) -> component means (zero bias, joint
+    range clip), deviations (softplus, floor, scale, cap) and logits, each (N, nu, K).  One component per action dimension
+    by inverse CDF of softmax(logits) at the uniform draw, action = mean_k + std_k z; log-probability of the sample under
+    the mixture; NaN scrub and clip (ksim/task/rl.py:998-1001).  xax.MixtureOfGaussians is third-party and absent: this is
+    the textbook mixture, pinned by scipy (logsumexp of norm.logpdf), unit mass and the K = 1 reduction to a Gaussian.
+    Returns (action, log_prob, component)."""
+    raw = np.asarray(raw, np.float64)
+    K = int(num_mixtures)
+    N, nu = raw.shape[0], raw.shape[1] // (3 * K)
+    mean = raw[:, : nu * K].reshape(N, nu, K)
+    rstd = raw[:, nu * K: 2 * nu * K].reshape(N, nu, K)
+    logit = raw[:, 2 * nu * K:].reshape(N, nu, K)
+    if mean_bias is not None:
+        mean = mean + np.asarray(mean_bias, np.float64)[None, :, None]
+    if clip_lo is not None:
+        mean = np.clip(mean, np.asarray(clip_lo, np.float64)[None, :, None], np.asarray(clip_hi, np.float64)[None, :, None])
+    std = np.minimum((np.logaddexp(0.0, rstd) + min_std) * var_scale, max_std)
+    logw = logit - np.logaddexp.reduce(logit, axis=-1, keepdims=True)
+    if deterministic:
+        comp = np.argmax(logit, axis=-1)
+        action = np.take_along_axis(mean, comp[..., None], -1)[..., 0]
+    else:
+        cum = np.cumsum(np.exp(logw), axis=-1)
+        comp = np.minimum((cum <= np.asarray(uniform, np.float64)[..., None]).sum(-1), K - 1)
+        pm = np.take_along_axis(mean, comp[..., None], -1)[..., 0]
+        ps = np.take_along_axis(std, comp[..., None], -1)[..., 0]
+        action = pm + ps * np.asarray(normal, np.float64)
+    d = (action[..., None] - mean) / std
+    logp = np.logaddexp.reduce(logw - 0.5 * d * d - np.log(std) - 0.5 * np.log(2 * np.pi), axis=-1)
+    action = np.clip(np.where(np.isnan(action), 0.0, action), -clip_max, clip_max)
+    return action, logp, comp

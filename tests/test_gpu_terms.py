@@ -622,3 +622,49 @@ def test_vector_commands():
     assert (cmd[1:, 2] == 5).all() and cmd[0, 2] == 0 and torch.equal(cmd[:, :2], first[:, :2])
     with pytest.raises(ValueError):
         FloatVectorCommand(ranges=())
+
+
+def test_mixture_of_gaussians_head():
+    """ks_sample_action_mixture against the oracle on the same draws: component (bit-exact), sample, log-density;
+    deterministic mode; Philox reproducibility and component frequencies."""
+    from ksim_amd.env_terms import sample_action_mixture
+
+    rng = np.random.default_rng(33)
+    N, nu, K = 300, 20, 5
+    raw = rng.normal(size=(N, 3 * nu * K)) * 1.5
+    raw[0, nu * K] = 60.0       # softplus in its linear range -> capped
+    raw[1, nu * K + 1] = -50.0  # softplus underflows -> floor
+    raw[2, 2 * nu * K: 2 * nu * K + K] = [30.0, -30.0, 0.0, 1.0, -5.0]  # one component takes (almost) all the weight
+    bias = rng.normal(size=nu) * 0.2
+    lo, hi = -np.ones(nu) * 0.9, np.ones(nu) * 1.2
+    u, z = rng.random((N, nu)), rng.normal(size=(N, nu))
+    # keep the draws away from the cumulative weights, where fp32 and float64 may pick neighbouring components
+    kw = dict(min_std=0.01, max_std=1.0, var_scale=0.5)
+    w_act, w_logp, w_comp = ot.mixture_head(raw, K, uniform=u, normal=z, mean_bias=bias, clip_lo=lo, clip_hi=hi, clip_max=2.0, **kw)
+    logit = raw[:, 2 * nu * K:].reshape(N, nu, K)
+    cum = np.cumsum(np.exp(logit - np.logaddexp.reduce(logit, -1, keepdims=True)), -1)
+    safe = np.abs(cum - u[..., None]).min(-1) > 1e-5
+    assert safe.mean() > 0.99
+    out, logp, comp = sample_action_mixture(t32(raw), K, mean_bias=t32(bias), clip_lo=t32(lo), clip_hi=t32(hi), uniform=t32(u),
+                                            noise=t32(z), clip_max=2.0, want_stats=True, **kw)
+    assert np.array_equal(comp.cpu().numpy()[safe], w_comp[safe])
+    np.testing.assert_allclose(out.cpu().numpy()[safe], w_act[safe], rtol=1e-5, atol=1e-5)
+    np.testing.assert_allclose(logp.cpu().numpy()[safe], w_logp[safe], rtol=2e-4, atol=2e-4)
+    assert comp[2, 0].item() == 0
+    det = sample_action_mixture(t32(raw), K, mean_bias=t32(bias), clip_lo=t32(lo), clip_hi=t32(hi), deterministic=True, **kw)
+    w_det, _, _ = ot.mixture_head(raw, K, mean_bias=bias, clip_lo=lo, clip_hi=hi, deterministic=True, **kw)
+    np.testing.assert_allclose(det.cpu().numpy(), w_det, rtol=1e-6, atol=1e-6)
+    # in-kernel draws: reproducible per (seed, step); components follow the weights
+    big = t32(np.tile(raw[5:6], (20000, 1)))
+    a1 = sample_action_mixture(big, K, seed=3, step=7, want_stats=True, **kw)
+    a2 = sample_action_mixture(big, K, seed=3, step=7, **kw)
+    a3 = sample_action_mixture(big, K, seed=3, step=8, **kw)
+    assert torch.equal(a1[0], a2) and not torch.equal(a2, a3)
+    cb = a1[2].cpu().numpy()
+    w5 = np.exp(logit[5] - np.logaddexp.reduce(logit[5], -1, keepdims=True))
+    freq = np.stack([(cb == k).mean(0) for k in range(K)], -1)
+    assert np.abs(freq - w5).max() < 0.015
+    with pytest.raises(Exception, match="3 nu K"):
+        sample_action_mixture(t32(raw), 7, **kw)
+    with pytest.raises(Exception, match="components"):
+        sample_action_mixture(t32(raw[:, :54]), 9, **kw)

@@ -16,7 +16,7 @@ def test_struct_layouts_match_the_library():
     lib.ks_abi_sizeof.argtypes = [ctypes.c_int32]
     structs = [_lib.KsPpoLossParams, _lib_dyn.KsModelDesc, _lib_dyn.KsStepIO, T.KsTermsDesc, T.KsObserveIO,
                T.KsTerminateIO, T.KsMlpDesc, T.KsRewardIO, T.KsObsElem, T.KsTermDesc, T.KsRewardDesc, T.KsRng,
-               T.KsAdamParams, T.KsEventDesc, T.KsRewardScanIO, T.KsRewardScanDesc, T.KsGruDesc, T.KsLstmDesc, T.KsGaussianHead, T.KsCommandIO]
+               T.KsAdamParams, T.KsEventDesc, T.KsRewardScanIO, T.KsRewardScanDesc, T.KsGruDesc, T.KsLstmDesc, T.KsGaussianHead, T.KsCommandIO, T.KsMixtureHead]
     for i, st in enumerate(structs):
         assert lib.ks_abi_sizeof(i) == ctypes.sizeof(st), st.__name__
     assert lib.ks_abi_sizeof(99) == -1

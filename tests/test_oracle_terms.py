@@ -293,3 +293,54 @@ def test_position_velocity_actuator_hand_computed():
     a = terms.position_velocity_actuator_torque([0.5, -0.2, 0.0, 0.0], np.array([0.1, 0.1]), np.array([0.5, -1.0]), [10.0, 20.0], [2.0, 1.0], [100.0, 100.0])
     b = terms.position_actuator_torque(np.array([0.5, -0.2]), np.array([0.1, 0.1]), np.array([0.5, -1.0]), np.array([10.0, 20.0]), np.array([2.0, 1.0]), np.array([100.0, 100.0]))
     np.testing.assert_allclose(a, b)
+
+
+def test_mixture_head_against_scipy_and_special_cases():
+    """The mixture-of-Gaussians head: log-density against scipy, unit mass, component frequencies of the inverse CDF, the
+    K = 1 reduction to the Gaussian head, the most probable component when deterministic."""
+    from scipy.special import logsumexp, softmax
+    from scipy.stats import norm
+
+    rng = np.random.default_rng(31)
+    N, nu, K = 40, 5, 3
+    raw = rng.normal(size=(N, 3 * nu * K)) * 1.5
+    bias = rng.normal(size=nu) * 0.2
+    lo, hi = -np.ones(nu) * 0.8, np.ones(nu) * 1.1
+    u, z = rng.random((N, nu)), rng.normal(size=(N, nu))
+    kw = dict(min_std=0.01, max_std=1.0, var_scale=0.5, mean_bias=bias, clip_lo=lo, clip_hi=hi)
+    act, logp, comp = terms.mixture_head(raw, K, uniform=u, normal=z, **kw)
+    mean = np.clip(raw[:, :nu * K].reshape(N, nu, K) + bias[None, :, None], lo[None, :, None], hi[None, :, None])
+    std = np.minimum((np.log1p(np.exp(raw[:, nu * K:2 * nu * K].reshape(N, nu, K))) + 0.01) * 0.5, 1.0)
+    w = softmax(raw[:, 2 * nu * K:].reshape(N, nu, K), axis=-1)
+    # component: the interval of the cumulative weights that holds the draw
+    cum = np.cumsum(w, -1)
+    for e, j in itertools.product(range(N), range(nu)):
+        k = int(np.searchsorted(cum[e, j], u[e, j], side="right"))
+        assert comp[e, j] == min(k, K - 1)
+    sample = np.take_along_axis(mean, comp[..., None], -1)[..., 0] + np.take_along_axis(std, comp[..., None], -1)[..., 0] * z
+    np.testing.assert_allclose(act, sample, rtol=1e-12)
+    want = logsumexp(np.log(w) + norm.logpdf(sample[..., None], mean, std), axis=-1)
+    np.testing.assert_allclose(logp, want, rtol=1e-10, atol=1e-10)
+    # the density integrates to one (one env, one joint, fine grid)
+    xs = np.linspace(-8, 8, 40001)
+    dens = (w[0, 0][None] * norm.pdf(xs[:, None], mean[0, 0][None], std[0, 0][None])).sum(-1)
+    assert np.sum(dens) * (xs[1] - xs[0]) == pytest.approx(1.0, abs=1e-6)
+    # K = 1: a Gaussian with that mean and deviation, whatever the logit
+    raw1 = rng.normal(size=(N, 3 * nu))
+    a1, l1, c1 = terms.mixture_head(raw1, 1, uniform=u, normal=z, min_std=0.02, max_std=50.0)
+    s1 = np.log1p(np.exp(raw1[:, nu:2 * nu])) + 0.02
+    np.testing.assert_allclose(a1, raw1[:, :nu] + s1 * z, rtol=1e-12)
+    np.testing.assert_allclose(l1, norm.logpdf(a1, raw1[:, :nu], s1), rtol=1e-10)
+    assert (c1 == 0).all()
+    # deterministic: the mean of the heaviest component; scrub and clip
+    ad, _, cd = terms.mixture_head(raw, K, deterministic=True, **kw)
+    assert (cd == np.argmax(w, -1)).all()
+    np.testing.assert_allclose(ad, np.take_along_axis(mean, cd[..., None], -1)[..., 0])
+    rawn = raw.copy(); rawn[0, 0:K] = np.nan
+    an, _, _ = terms.mixture_head(rawn, K, uniform=u, normal=z, clip_max=0.5, **kw)
+    assert an[0, 0] == 0.0 and np.abs(an).max() <= 0.5
+    # frequencies: many draws pick component k with probability w_k
+    big = np.tile(raw[:1], (20000, 1))
+    _, _, cb = terms.mixture_head(big, K, uniform=rng.random((20000, nu)), normal=np.zeros((20000, nu)), **kw)
+    freq = np.stack([(cb == k).mean(0) for k in range(K)], -1)
+    assert np.abs(freq - w[0]).max() < 0.015
