@@ -4,6 +4,10 @@ Rewards follow ksim/rewards.py, terminations ksim/terminations.py, the PD
 actuator ksim/actuators.py:182-217, the latency blend ksim/engine.py:287-288,
 the done/success combination ksim/task/rl.py:1049-1050 and the reward total
 ksim/task/rl.py:219-239.  Shapes are per env, time leading, like the reference.
+
+Parity unpinned (third-party xax, absent from the reference tree and from this image): the quaternion conventions of
+rotate_vector_by_quat / euler_to_quat (Hamilton wxyz assumed) and mixture_head against xax.MixtureOfGaussians (the
+textbook mixture is restated and pinned by scipy).
 """
 
 from __future__ import annotations
