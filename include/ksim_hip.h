@@ -592,6 +592,14 @@ int64_t ks_mlp_train_workspace_bytes(const KsMlp* mlp, int64_t M);
 int ks_mlp_train_forward(KsMlp* mlp, ks_stream_t stream, int64_t M, const float* x, float* y, void* workspace);
 int ks_mlp_train_backward(KsMlp* mlp, ks_stream_t stream, int64_t M, const float* x, const float* dy /*(M, out)*/,
                           void* workspace);
+/* ks_mlp_train_backward that also returns dx (M, in), the gradient with respect to the network input (added to dx when
+ * accumulate_dx, rows flagged in zero_rows written as zero); weight_gradients = 0 skips the weight and bias gradients
+ * (then x may be NULL).  For a one-layer network no preceding ks_mlp_train_forward is needed. */
+int ks_mlp_train_backward_dx(KsMlp* mlp, ks_stream_t stream, int64_t M, const float* x, const float* dy, float* dx,
+                             int32_t weight_gradients, int32_t accumulate_dx, const uint8_t* zero_rows /*(M) nullable*/,
+                             void* workspace);
+/* The first `count` bias entries of a layer are constants: the optimiser and the gradient norm skip them. */
+int ks_mlp_freeze_bias_prefix(KsMlp* mlp, int32_t layer, int32_t count);
 int ks_grad_sqnorm(ks_stream_t stream, int64_t n, const float* g, double* acc);
 int ks_mlp_grad_sqnorm(const KsMlp* mlp, ks_stream_t stream, double* acc);
 int ks_mlp_adam_step(KsMlp* mlp, ks_stream_t stream, const KsAdamParams* params /*host*/, const double* sqnorm);
@@ -600,6 +608,24 @@ int ks_adam_step(ks_stream_t stream, int64_t n, float* param, const float* grad,
 /* Copies of the parameters and gradients in the caller's (out, in) layout, for checks and checkpoints. */
 int ks_mlp_get_params(const KsMlp* mlp, ks_stream_t stream, int32_t layer, float* weight /*(out,in) dev*/, float* bias /*(out) dev*/,
                       int32_t gradients /*0: parameters, 1: gradients*/);
+
+/* Backward pass through time of a GRU stack (the jax.grad through the lax.scan over the trajectory in
+ * PPOTask._single_step, ksim/task/ppo.py:572-694, for the recurrent actors and critics of examples/walking.py:40-208).
+ * Forward over the trajectory with ks_gru_train_forward, which keeps per step saved (M, 5H) = r | z | n | hn | h.  Then per
+ * step, last to first, ks_gru_backward_step takes dh_out (M, H) = gradient from the layer above at that step + dh_in of
+ * the step after it, and returns d_gi, d_gh (M, 3H), the gradients of the two projections' outputs, and dh_in (M, H), the
+ * gradient of the step's incoming hidden state (zero for an env that started an episode there).  With d_gi, d_gh and
+ * saved[..., 4H:] stacked over all steps, one ks_mlp_train_backward_dx per projection (ks_gru_projections hands them
+ * out) yields the weight gradients and the gradient of the layer's inputs.  ks_gru_adam_step updates both. */
+int ks_gru_train_init(KsGru* gru);
+int ks_gru_projections(KsGru* gru, KsMlp** input_projection, KsMlp** hidden_projection);
+int ks_gru_train_forward(const KsGru* gru, ks_stream_t stream, int64_t M, const float* x, const float* h_in,
+                         const uint8_t* fresh, float* h_out, float* saved /*(M, 5H)*/, void* workspace /*ks_gru_workspace_bytes*/);
+int64_t ks_gru_backward_workspace_bytes(const KsGru* gru, int64_t M);
+int ks_gru_backward_step(KsGru* gru, ks_stream_t stream, int64_t M, const float* dh_out, const float* saved,
+                         const uint8_t* fresh, float* d_gi, float* d_gh, float* dh_in, void* workspace);
+int ks_gru_grad_sqnorm(const KsGru* gru, ks_stream_t stream, double* acc);
+int ks_gru_adam_step(KsGru* gru, ks_stream_t stream, const KsAdamParams* params /*host*/, const double* sqnorm);
 
 /* Gaussian policy head and the gradient of the PPO objective (ppo.py:149-246, total 473-486):
  *   ks_gaussian_log_prob: per action dimension log N(action; mean, exp(log_std)) and entropy

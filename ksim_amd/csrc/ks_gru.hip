@@ -1,4 +1,4 @@
-// GRU and LSTM cells for recurrent policies in the rollout (forward only).  The two gate projections are plain linear
+// GRU and LSTM cells for recurrent policies in the rollout, and the GRU's backward pass through time.  The two gate projections are plain linear
 // layers and run through the MLP entry points (matrix cores for bf16); one streaming kernel then combines the gates.
 #include "ks_common.h"
 
@@ -27,6 +27,55 @@ __global__ __launch_bounds__(256) void gru_gate_kernel(int64_t M, int H, const f
   const float z = 1.f / (1.f + expf(-(a[H + j] + hz)));
   const float n = tanhf(a[2 * H + j] + r * hn);
   h_out[idx] = n + z * (h - n);
+}
+
+// The same cell for training: also keeps what the backward pass needs, saved (M, 5H) = r | z | n | hn | h, where hn is the
+// hidden part of the candidate (what r multiplies) and h the hidden state the cell actually used (zero for a fresh env).
+__global__ __launch_bounds__(256) void gru_gate_train_kernel(int64_t M, int H, const float* __restrict__ gi,
+                                                             const float* __restrict__ gh, const float* __restrict__ h_in,
+                                                             const float* __restrict__ bias_n, const uint8_t* __restrict__ fresh,
+                                                             float* __restrict__ h_out, float* __restrict__ saved) {
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= M * H) return;
+  const int64_t m = idx / H;
+  const int j = (int)(idx - m * H);
+  const bool f = fresh && fresh[m];
+  const float* a = gi + m * 3 * H;
+  const float* b = gh + m * 3 * H;
+  const float hr = f ? 0.f : b[j], hz = f ? 0.f : b[H + j], hn = f ? bias_n[j] : b[2 * H + j];
+  const float h = f ? 0.f : h_in[idx];
+  const float r = 1.f / (1.f + expf(-(a[j] + hr)));
+  const float z = 1.f / (1.f + expf(-(a[H + j] + hz)));
+  const float n = tanhf(a[2 * H + j] + r * hn);
+  h_out[idx] = n + z * (h - n);
+  float* sv = saved + m * 5 * H;
+  sv[j] = r; sv[H + j] = z; sv[2 * H + j] = n; sv[3 * H + j] = hn; sv[4 * H + j] = h;
+}
+
+// Backward through the gates of one step.  dh_out is the gradient reaching h' (from the layer above at this step plus
+// from the next step).  d_gi (M, 3H) is the gradient of the input projection's output, d_gh (M, 3H) that of the hidden
+// projection's output (its n part is also the gradient of bias_n, fresh rows included); dh_in = dh_out * z is the direct
+// path to the previous hidden state, zero for a fresh env (the hidden projection adds its share afterwards).
+__global__ __launch_bounds__(256) void gru_gate_backward_kernel(int64_t M, int H, const float* __restrict__ dh_out,
+                                                                const float* __restrict__ saved, const uint8_t* __restrict__ fresh,
+                                                                float* __restrict__ d_gi, float* __restrict__ d_gh,
+                                                                float* __restrict__ dh_in) {
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= M * H) return;
+  const int64_t m = idx / H;
+  const int j = (int)(idx - m * H);
+  const bool f = fresh && fresh[m];
+  const float* sv = saved + m * 5 * H;
+  const float r = sv[j], z = sv[H + j], n = sv[2 * H + j], hn = sv[3 * H + j], h = sv[4 * H + j];
+  const float d = dh_out[idx];
+  const float dn_pre = d * (1.f - z) * (1.f - n * n);
+  const float dz_pre = d * (h - n) * z * (1.f - z);
+  const float dr_pre = dn_pre * hn * r * (1.f - r);
+  float* a = d_gi + m * 3 * H;
+  float* b = d_gh + m * 3 * H;
+  a[j] = dr_pre; a[H + j] = dz_pre; a[2 * H + j] = dn_pre;
+  b[j] = dr_pre; b[H + j] = dz_pre; b[2 * H + j] = dn_pre * r;
+  dh_in[idx] = f ? 0.f : d * z;
 }
 
 // LSTM: g = W_ih x + W_hh h + b (M, 4H) in gate order input | forget | cell | output:
@@ -60,7 +109,8 @@ using namespace ks;
 struct KsGru {
   int I, H;
   KsMlp *proj_i, *proj_h;
-  float* bias_n;  // device (H)
+  float* bias_n;    // device (H)
+  float* bias_tmp;  // device (3H), training only
 };
 
 extern "C" int ks_gru_create(const KsGruDesc* d, KsGru** out) {
@@ -70,7 +120,7 @@ extern "C" int ks_gru_create(const KsGruDesc* d, KsGru** out) {
   const int H = d->hidden_size, I = d->input_size;
   std::vector<float> zero(3 * (size_t)H, 0.f), bh(3 * (size_t)H, 0.f);
   if (d->bias_n) for (int j = 0; j < H; ++j) bh[2 * (size_t)H + j] = d->bias_n[j];
-  KsGru* g = new KsGru{I, H, nullptr, nullptr, nullptr};
+  KsGru* g = new KsGru{I, H, nullptr, nullptr, nullptr, nullptr};
   KsMlpDesc md = {};
   md.n_layers = 1; md.activation = KS_ACT_NONE; md.dtype = d->dtype;
   md.dims[0] = I; md.dims[1] = 3 * H; md.weights[0] = d->weight_ih; md.biases[0] = d->bias ? d->bias : zero.data();
@@ -92,6 +142,7 @@ extern "C" int ks_gru_destroy(KsGru* g) {
   ks_mlp_destroy(g->proj_i);
   ks_mlp_destroy(g->proj_h);
   if (g->bias_n) (void)hipFree(g->bias_n);
+  if (g->bias_tmp) (void)hipFree(g->bias_tmp);
   delete g;
   return KS_OK;
 }
@@ -125,6 +176,85 @@ extern "C" int ks_gru_forward(const KsGru* g, ks_stream_t stream, int64_t M, con
   hipLaunchKernelGGL(gru_gate_kernel, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, M, g->H, gi, gh, h_in,
                      g->bias_n, fresh, h_out);
   return check_launch("ks_gru_forward");
+}
+
+extern "C" int ks_gru_train_init(KsGru* g) {
+  if (!g) return fail(KS_EINVAL, "ks_gru_train_init: null handle");
+  int rc = ks_mlp_train_init(g->proj_i);
+  if (rc == KS_OK) rc = ks_mlp_train_init(g->proj_h);
+  // the hidden projection's bias is (0, 0, b_n): only its candidate part is a parameter of the cell
+  if (rc == KS_OK) rc = ks_mlp_freeze_bias_prefix(g->proj_h, 0, 2 * g->H);
+  if (rc == KS_OK && !g->bias_tmp && hipMalloc((void**)&g->bias_tmp, 3 * (size_t)g->H * 4) != hipSuccess)
+    rc = fail(KS_ELAUNCH, "ks_gru_train_init: allocation failed");
+  return rc;
+}
+
+extern "C" int ks_gru_projections(KsGru* g, KsMlp** input_projection, KsMlp** hidden_projection) {
+  if (!g || !input_projection || !hidden_projection) return fail(KS_EINVAL, "ks_gru_projections: null argument");
+  *input_projection = g->proj_i;
+  *hidden_projection = g->proj_h;
+  return KS_OK;
+}
+
+extern "C" int ks_gru_grad_sqnorm(const KsGru* g, ks_stream_t stream, double* acc) {
+  if (!g || !acc) return fail(KS_EINVAL, "ks_gru_grad_sqnorm: null argument");
+  const int rc = ks_mlp_grad_sqnorm(g->proj_i, stream, acc);
+  return rc != KS_OK ? rc : ks_mlp_grad_sqnorm(g->proj_h, stream, acc);
+}
+
+extern "C" int ks_gru_adam_step(KsGru* g, ks_stream_t stream, const KsAdamParams* params, const double* sqnorm) {
+  if (!g || !g->bias_tmp) return fail(KS_EINVAL, "ks_gru_adam_step: call ks_gru_train_init first");
+  int rc = ks_mlp_adam_step(g->proj_i, stream, params, sqnorm);
+  if (rc == KS_OK) rc = ks_mlp_adam_step(g->proj_h, stream, params, sqnorm);
+  // the gate kernel's own copy of b_n (used for envs that start an episode) follows the hidden projection's bias
+  if (rc == KS_OK) rc = ks_mlp_get_params(g->proj_h, stream, 0, nullptr, g->bias_tmp, 0);
+  if (rc == KS_OK && hipMemcpyAsync(g->bias_n, g->bias_tmp + 2 * (size_t)g->H, (size_t)g->H * 4, hipMemcpyDeviceToDevice,
+                                    (hipStream_t)stream) != hipSuccess)
+    rc = fail(KS_ELAUNCH, "ks_gru_adam_step: bias copy failed");
+  return rc;
+}
+
+extern "C" int ks_gru_train_forward(const KsGru* g, ks_stream_t stream, int64_t M, const float* x, const float* h_in,
+                                    const uint8_t* fresh, float* h_out, float* saved, void* workspace) {
+  if (!g || !x || !h_in || !h_out || !saved) return fail(KS_EINVAL, "ks_gru_train_forward: null argument");
+  if (M < 0) return fail(KS_EINVAL, "ks_gru_train_forward: negative row count");
+  if (M == 0) return KS_OK;
+  if (!workspace) return fail(KS_EINVAL, "ks_gru_train_forward: workspace is required");
+  const int64_t gates = up256(M * 3 * g->H * 4);
+  char* w = (char*)workspace;
+  float* gi = (float*)w;
+  float* gh = (float*)(w + gates);
+  void* wi = w + 2 * gates;
+  void* wh = w + 2 * gates + up256(ks_mlp_workspace_bytes(g->proj_i, M));
+  int rc = ks_mlp_forward(g->proj_i, stream, M, x, gi, wi);
+  if (rc != KS_OK) return rc;
+  rc = ks_mlp_forward(g->proj_h, stream, M, h_in, gh, wh);
+  if (rc != KS_OK) return rc;
+  const int64_t n = M * g->H, grid = (n + 255) / 256;
+  if (grid > 0x7fffffff) return fail(KS_ELIMIT, "ks_gru_train_forward: too many elements");
+  hipLaunchKernelGGL(gru_gate_train_kernel, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, M, g->H, gi, gh, h_in,
+                     g->bias_n, fresh, h_out, saved);
+  return check_launch("ks_gru_train_forward");
+}
+
+extern "C" int64_t ks_gru_backward_workspace_bytes(const KsGru* g, int64_t M) {
+  if (!g || M < 0) return -1;
+  return ks_mlp_train_workspace_bytes(g->proj_h, M);
+}
+
+extern "C" int ks_gru_backward_step(KsGru* g, ks_stream_t stream, int64_t M, const float* dh_out, const float* saved,
+                                    const uint8_t* fresh, float* d_gi, float* d_gh, float* dh_in, void* workspace) {
+  if (!g || !dh_out || !saved || !d_gi || !d_gh || !dh_in || !workspace) return fail(KS_EINVAL, "ks_gru_backward_step: null argument");
+  if (M < 0) return fail(KS_EINVAL, "ks_gru_backward_step: negative row count");
+  if (M == 0) return KS_OK;
+  const int64_t n = M * g->H, grid = (n + 255) / 256;
+  if (grid > 0x7fffffff) return fail(KS_ELIMIT, "ks_gru_backward_step: too many elements");
+  hipLaunchKernelGGL(gru_gate_backward_kernel, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, M, g->H, dh_out, saved, fresh,
+                     d_gi, d_gh, dh_in);
+  int rc = check_launch("ks_gru_backward_step");
+  if (rc != KS_OK) return rc;
+  // dh_in += d_gh W_hh, except across an episode boundary
+  return ks_mlp_train_backward_dx(g->proj_h, stream, M, nullptr, d_gh, dh_in, 0, 1, fresh, workspace);
 }
 
 struct KsLstm {

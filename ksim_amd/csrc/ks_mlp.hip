@@ -505,7 +505,8 @@ struct DevMlp {
   float *mW[KS_MAX_LAYERS], *mb[KS_MAX_LAYERS];
   float *gW[KS_MAX_LAYERS], *gb[KS_MAX_LAYERS];
   float *m1W[KS_MAX_LAYERS], *m2W[KS_MAX_LAYERS], *m1b[KS_MAX_LAYERS], *m2b[KS_MAX_LAYERS];
-  void* Wt[KS_MAX_LAYERS];      // (kpad, npad) working-precision transpose, layers >= 1
+  void* Wt[KS_MAX_LAYERS];      // (kpad, npad) working-precision transpose
+  int bias_frozen[KS_MAX_LAYERS];  // leading bias entries of the layer that the optimiser leaves alone
   float* zero_bias;             // zeros, as wide as the widest GEMM output
 };
 
@@ -528,6 +529,20 @@ __global__ __launch_bounds__(256) void cast_pad_kernel(int64_t M, int n, int ld,
   const int64_t m = idx / ld;
   const int c = (int)(idx - m * ld);
   dst[idx] = from_f32<T>(c < n ? src[m * n + c] : 0.f);
+}
+
+// T (M, ld) -> fp32 (M, n): the input gradient in the caller's layout; optionally added to what is there, and rows
+// flagged in zero_rows come out as zero (an episode boundary stops the gradient)
+template <typename T>
+__global__ __launch_bounds__(256) void unpad_cast_kernel(int64_t M, int n, int ld, const T* __restrict__ src, float* __restrict__ dst,
+                                                         int accumulate, const uint8_t* __restrict__ zero_rows) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= M * n) return;
+  const int64_t m = idx / n;
+  const int c = (int)(idx - m * n);
+  if (zero_rows && zero_rows[m]) { dst[idx] = 0.f; return; }
+  const float v = to_f32(src[m * ld + c]);
+  dst[idx] = accumulate ? dst[idx] + v : v;
 }
 
 // (M, ld_src) with C meaningful columns -> (Cpad, Mp) transposed, zero outside (C, M).  S is float or T.
@@ -1045,7 +1060,10 @@ extern "C" int ks_mlp_train_init(KsMlp* h) {
     if (hipMemcpy(m.mW[l], w.data(), n * 4, hipMemcpyHostToDevice) != hipSuccess ||
         hipMemcpy(m.mb[l], b.data(), nb * 4, hipMemcpyHostToDevice) != hipSuccess)
       return fail(KS_ELAUNCH, "ks_mlp_train_init: upload failed");
-    if (l > 0 && hipMalloc(&m.Wt[l], n * esz) != hipSuccess) return fail(KS_ELAUNCH, "ks_mlp_train_init: allocation failed");
+    // the first layer's transpose is padded to whole output tiles of the input-gradient product; the padding stays zero
+    const size_t nt = l == 0 ? (size_t)round_up(m.kpad[0], kBN) * m.npad[0] : n;
+    if (hipMalloc(&m.Wt[l], nt * esz) != hipSuccess || hipMemset(m.Wt[l], 0, nt * esz) != hipSuccess)
+      return fail(KS_ELAUNCH, "ks_mlp_train_init: allocation failed");
   }
   const int wz = widest_pad(m);
   if (hipMalloc((void**)&m.zero_bias, (size_t)wz * 4) != hipSuccess || hipMemset(m.zero_bias, 0, (size_t)wz * 4) != hipSuccess)
@@ -1144,7 +1162,8 @@ extern "C" int ks_mlp_train_forward(KsMlp* h, ks_stream_t stream, int64_t M, con
 }
 
 template <typename T>
-static int train_backward(DevMlp& m, hipStream_t s, int64_t M, const float* x, const float* dy, const TrainWs& ws) {
+static int train_backward(DevMlp& m, hipStream_t s, int64_t M, const float* x, const float* dy, const TrainWs& ws,
+                          float* dx = nullptr, bool want_w = true, bool accumulate_dx = false, const uint8_t* zero_rows = nullptr) {
   const int L = m.n_layers;
   const int64_t Mp = ws.Mp;
   T* dz = (T*)ws.d0;
@@ -1161,11 +1180,19 @@ static int train_backward(DevMlp& m, hipStream_t s, int64_t M, const float* x, c
   bool have_dzT = false, have_bias = false;
   for (int l = L - 1; l >= 0; --l) {
     const int np = m.npad[l], kp = m.kpad[l], kp128 = round_up(kp, kBN);
-    if (!have_bias) {
+    if (l == 0 && dx) {  // gradient with respect to the network input
+      const int rc0 = launch_layer<T, false, false>(KS_ACT_NONE, s, M, kp128, np, np, kp128, dz, np, m.Wt[0], m.zero_bias, dnext, kp128);
+      if (rc0 != KS_OK) return rc0;
+      const int64_t n = M * m.dims[0];
+      hipLaunchKernelGGL(unpad_cast_kernel<T>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, M, m.dims[0], kp128, (const T*)dnext, dx,
+                         accumulate_dx ? 1 : 0, zero_rows);
+    }
+    if (!want_w && l == 0) break;
+    if (want_w && !have_bias) {
       hipLaunchKernelGGL(colsum_kernel<T>, dim3((unsigned)((np + 63) / 64), kColsumSlices), dim3(256), 0, s, M, np, dz, ws.part);
       hipLaunchKernelGGL(sum_parts_kernel, dim3((unsigned)((np + 255) / 256)), dim3(256), 0, s, (int64_t)np, kColsumSlices, ws.part, m.gb[l]);
     }
-    if (!have_dzT)
+    if (want_w && !have_dzT)
       hipLaunchKernelGGL((transpose_kernel<T, T>), dim3((unsigned)((Mp + 31) / 32), (unsigned)((np + 31) / 32)), dim3(256), 0, s, M, np,
                          (int64_t)np, dz, np, Mp, dzT);
     have_dzT = have_bias = false;
@@ -1175,7 +1202,7 @@ static int train_backward(DevMlp& m, hipStream_t s, int64_t M, const float* x, c
       // input gradient, then through the activation of the layer below
       rc = launch_layer<T, false, false>(KS_ACT_NONE, s, M, kp, np, np, kp, dz, np, m.Wt[l], m.zero_bias, dnext, kp);
       if (rc != KS_OK) return rc;
-      const bool fused = kp % 64 == 0 && kp == kp128 && kp == m.npad[l - 1];
+      const bool fused = want_w && kp % 64 == 0 && kp == kp128 && kp == m.npad[l - 1];
       if (fused) {
 #define KS_PREP(A) hipLaunchKernelGGL((bwd_prep_kernel<T, A>), dim3((unsigned)(kp / 64), kColsumSlices), dim3(256), 0, s, M, Mp, kp, \
                                       (const T*)ws.act[l - 1], dnext, dzT_next, (T*)ws.t1, ws.part)
@@ -1199,6 +1226,10 @@ static int train_backward(DevMlp& m, hipStream_t s, int64_t M, const float* x, c
         }
 #undef KS_ACTB
       }
+    }
+    if (!want_w) {
+      T* tmp = dz; dz = dnext; dnext = tmp;
+      continue;
     }
     // weight gradient: dZ^T (np, Mp) times Y_prev^T (kp128, Mp)^T
     if (!have_yT) {
@@ -1237,6 +1268,27 @@ extern "C" int ks_mlp_train_backward(KsMlp* h, ks_stream_t stream, int64_t M, co
   return rc != KS_OK ? rc : check_launch("ks_mlp_train_backward");
 }
 
+extern "C" int ks_mlp_train_backward_dx(KsMlp* h, ks_stream_t stream, int64_t M, const float* x, const float* dy, float* dx,
+                                        int32_t weight_gradients, int32_t accumulate_dx, const uint8_t* zero_rows, void* workspace) {
+  if (!h || !h->m.train) return fail(KS_EINVAL, "ks_mlp_train_backward_dx: call ks_mlp_train_init first");
+  if (M <= 0 || !dy || !dx || !workspace || (weight_gradients && !x)) return fail(KS_EINVAL, "ks_mlp_train_backward_dx: bad argument");
+  if (M > (1 << 30)) return fail(KS_ELIMIT, "ks_mlp_train_backward_dx: too many rows");
+  TrainWs ws;
+  carve_train(h->m, M, (char*)workspace, &ws);
+  const bool w = weight_gradients != 0, acc = accumulate_dx != 0;
+  const int rc = h->m.dtype == KS_MLP_BF16 ? train_backward<__bf16>(h->m, (hipStream_t)stream, M, x, dy, ws, dx, w, acc, zero_rows)
+                                           : train_backward<float>(h->m, (hipStream_t)stream, M, x, dy, ws, dx, w, acc, zero_rows);
+  return rc != KS_OK ? rc : check_launch("ks_mlp_train_backward_dx");
+}
+
+extern "C" int ks_mlp_freeze_bias_prefix(KsMlp* h, int32_t layer, int32_t count) {
+  if (!h) return fail(KS_EINVAL, "ks_mlp_freeze_bias_prefix: null handle");
+  if (layer < 0 || layer >= h->m.n_layers || count < 0 || count > h->m.dims[layer + 1])
+    return fail(KS_EINVAL, "ks_mlp_freeze_bias_prefix: layer %d, count %d out of range", layer, count);
+  h->m.bias_frozen[layer] = count;
+  return KS_OK;
+}
+
 extern "C" int ks_grad_sqnorm(ks_stream_t stream, int64_t n, const float* g, double* acc) {
   if (n < 0 || !acc || (n > 0 && !g)) return fail(KS_EINVAL, "ks_grad_sqnorm: bad argument");
   if (n == 0) return KS_OK;
@@ -1248,7 +1300,9 @@ extern "C" int ks_mlp_grad_sqnorm(const KsMlp* h, ks_stream_t stream, double* ac
   if (!h || !h->m.train || !acc) return fail(KS_EINVAL, "ks_mlp_grad_sqnorm: bad argument");
   for (int l = 0; l < h->m.n_layers; ++l) {
     hipLaunchKernelGGL(sqnorm_kernel, dim3(64), dim3(256), 0, (hipStream_t)stream, (int64_t)h->m.npad[l] * h->m.kpad[l], h->m.gW[l], acc);
-    hipLaunchKernelGGL(sqnorm_kernel, dim3(1), dim3(256), 0, (hipStream_t)stream, (int64_t)h->m.npad[l], h->m.gb[l], acc);
+    const int fz = h->m.bias_frozen[l];
+    if (h->m.npad[l] > fz)
+      hipLaunchKernelGGL(sqnorm_kernel, dim3(1), dim3(256), 0, (hipStream_t)stream, (int64_t)h->m.npad[l] - fz, h->m.gb[l] + fz, acc);
   }
   return check_launch("ks_mlp_grad_sqnorm");
 }
@@ -1279,7 +1333,10 @@ extern "C" int ks_mlp_adam_step(KsMlp* h, ks_stream_t stream, const KsAdamParams
   for (int l = 0; l < m.n_layers; ++l) {
     const int64_t n = (int64_t)m.npad[l] * m.kpad[l], nb = m.npad[l];
     hipLaunchKernelGGL(adam_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, n, m.mW[l], m.gW[l], m.m1W[l], m.m2W[l], *p, sqnorm);
-    hipLaunchKernelGGL(adam_kernel, dim3((unsigned)((nb + 255) / 256)), dim3(256), 0, s, nb, m.mb[l], m.gb[l], m.m1b[l], m.m2b[l], *p, sqnorm);
+    const int fz = m.bias_frozen[l];
+    if (nb > fz)
+      hipLaunchKernelGGL(adam_kernel, dim3((unsigned)((nb - fz + 255) / 256)), dim3(256), 0, s, nb - fz, m.mb[l] + fz, m.gb[l] + fz,
+                         m.m1b[l] + fz, m.m2b[l] + fz, *p, sqnorm);
   }
   if (m.dtype == KS_MLP_BF16) refresh_layers<__bf16>(m, s);
   else refresh_layers<float>(m, s);

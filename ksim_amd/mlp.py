@@ -130,6 +130,34 @@ class MLP:
         _lib.check(self._lib.ks_mlp_train_backward(self._handle, _lib.current_stream(), x.shape[0], _lib.ptr(x),
                                                    _lib.ptr(dy), _lib.ptr(self._train_ws(x.shape[0], x.device))))
 
+    def backward_dx(self, x: torch.Tensor | None, dy: torch.Tensor, dx: torch.Tensor, *, weight_gradients: bool = True,
+                    accumulate: bool = False, zero_rows: torch.Tensor | None = None) -> torch.Tensor:
+        """`backward` that also writes (or adds) the gradient with respect to the network input into `dx`; without
+        `weight_gradients` only that.  Rows flagged in `zero_rows` (uint8) get a zero input gradient."""
+        _lib.require_cuda(x, dy, dx, dtype=torch.float32)
+        M = dy.shape[0]
+        if tuple(dy.shape) != (M, self.out_dim) or tuple(dx.shape) != (M, self.in_dim) or (x is not None and tuple(x.shape) != (M, self.in_dim)):
+            raise _lib.KsError("x and dx must be (M, in), dy (M, out)")
+        if x is None and weight_gradients:
+            raise _lib.KsError("the weight gradients need the input")
+        if zero_rows is not None:
+            _lib.require_cuda(zero_rows, dtype=torch.uint8)
+            if tuple(zero_rows.shape) != (M,):
+                raise _lib.KsError("zero_rows must be (M,) uint8")
+        _lib.check(self._lib.ks_mlp_train_backward_dx(self._handle, _lib.current_stream(), M, _lib.ptr(x), _lib.ptr(dy),
+                                                      _lib.ptr(dx), int(weight_gradients), int(accumulate),
+                                                      _lib.ptr(zero_rows), _lib.ptr(self._train_ws(M, dy.device))))
+        return dx
+
+    @classmethod
+    def _borrow(cls, lib, handle, dims, dtype: str) -> "MLP":
+        """A view of a network that another object owns (the projections inside a GRU cell): never destroyed here."""
+        self = cls.__new__(cls)
+        self._lib, self._handle, self.dims, self.dtype, self.activation = lib, handle, list(dims), dtype, "none"
+        self._ws = None
+        self._borrowed = True
+        return self
+
     def grad_sqnorm(self, acc: torch.Tensor) -> None:
         _lib.require_cuda(acc, dtype=torch.float64)
         _lib.check(self._lib.ks_mlp_grad_sqnorm(self._handle, _lib.current_stream(), _lib.ptr(acc)))
@@ -149,6 +177,8 @@ class MLP:
         return out
 
     def close(self) -> None:
+        if getattr(self, "_borrowed", False):
+            return
         if self._handle:
             self._lib.ks_mlp_destroy(self._handle)
             self._handle = ctypes.c_void_p()

@@ -1,4 +1,4 @@
-"""Recurrent policy / critic networks for the rollout (forward only).
+"""Recurrent policy / critic networks for the rollout, and the backward pass through time of the GRU stack.
 
 The shipped examples build their actor and critic as an input projection, a stack of GRU cells and an output MLP
 (examples/walking.py:40-208); the carry `(depth, N, hidden)` travels with the env state and is zeroed for envs that
@@ -77,6 +77,54 @@ class GRUCell:
         _lib.check(self._lib.ks_gru_forward(self._handle, _lib.current_stream(), M, _lib.ptr(x), _lib.ptr(h),
                                             _lib.ptr(fresh), _lib.ptr(out), _lib.ptr(ws)))
         return out
+
+    # ------------------------------------------------------------------ training (ksim/task/ppo.py:572-694)
+    def train_init(self) -> None:
+        """fp32 master weights, gradients and Adam moments of both projections; afterwards `proj_i` / `proj_h` expose them."""
+        _lib.check(self._lib.ks_gru_train_init(self._handle))
+        pi, ph = ctypes.c_void_p(), ctypes.c_void_p()
+        _lib.check(self._lib.ks_gru_projections(self._handle, ctypes.byref(pi), ctypes.byref(ph)))
+        H = self.hidden_size
+        self.proj_i = MLP._borrow(self._lib, pi, (self.input_size, 3 * H), self.dtype)
+        self.proj_h = MLP._borrow(self._lib, ph, (H, 3 * H), self.dtype)
+        self._bws: torch.Tensor | None = None
+
+    def train_forward(self, x, h, fresh, out, saved) -> torch.Tensor:
+        """`__call__` that also fills `saved` (M, 5H) = r | z | n | hn | h for `backward_step`."""
+        _lib.require_cuda(x, h, out, saved, dtype=torch.float32)
+        _lib.require_cuda(fresh, dtype=torch.uint8)
+        M, H = x.shape[0], self.hidden_size
+        if tuple(x.shape) != (M, self.input_size) or tuple(h.shape) != (M, H) or tuple(out.shape) != (M, H) or tuple(saved.shape) != (M, 5 * H):
+            raise _lib.KsError("expected x (M, input), h and out (M, H), saved (M, 5H)")
+        _lib.check(self._lib.ks_gru_train_forward(self._handle, _lib.current_stream(), M, _lib.ptr(x), _lib.ptr(h), _lib.ptr(fresh),
+                                                  _lib.ptr(out), _lib.ptr(saved), _lib.ptr(self.workspace(M, x.device))))
+        return out
+
+    def backward_step(self, dh_out, saved, fresh, d_gi, d_gh, dh_in) -> None:
+        """One step of the backward pass through time: dh_out (M, H) -> d_gi, d_gh (M, 3H) and dh_in (M, H)."""
+        _lib.require_cuda(dh_out, saved, d_gi, d_gh, dh_in, dtype=torch.float32)
+        _lib.require_cuda(fresh, dtype=torch.uint8)
+        M, H = dh_out.shape[0], self.hidden_size
+        if (tuple(dh_out.shape) != (M, H) or tuple(saved.shape) != (M, 5 * H) or tuple(d_gi.shape) != (M, 3 * H)
+                or tuple(d_gh.shape) != (M, 3 * H) or tuple(dh_in.shape) != (M, H)):
+            raise _lib.KsError("expected dh_out, dh_in (M, H), saved (M, 5H), d_gi, d_gh (M, 3H)")
+        need = int(self._lib.ks_gru_backward_workspace_bytes(self._handle, M))
+        if self._bws is None or self._bws.numel() < need or self._bws.device != dh_out.device:
+            self._bws = torch.empty(need, dtype=torch.uint8, device=dh_out.device)
+        _lib.check(self._lib.ks_gru_backward_step(self._handle, _lib.current_stream(), M, _lib.ptr(dh_out), _lib.ptr(saved),
+                                                  _lib.ptr(fresh), _lib.ptr(d_gi), _lib.ptr(d_gh), _lib.ptr(dh_in), _lib.ptr(self._bws)))
+
+    def grad_sqnorm(self, acc: torch.Tensor) -> None:
+        _lib.check(self._lib.ks_gru_grad_sqnorm(self._handle, _lib.current_stream(), _lib.ptr(acc)))
+
+    def adam_step(self, params, sqnorm) -> None:
+        _lib.check(self._lib.ks_gru_adam_step(self._handle, _lib.current_stream(), ctypes.byref(params), _lib.ptr(sqnorm)))
+
+    def parameters(self, gradients: bool = False) -> dict:
+        """Copies of weight_ih, weight_hh, bias (3H) and bias_n (H), or of their gradients."""
+        (wi, bi), = self.proj_i.parameters(gradients)
+        (wh, bh), = self.proj_h.parameters(gradients)
+        return dict(weight_ih=wi, weight_hh=wh, bias=bi, bias_n=bh[2 * self.hidden_size:].clone())
 
     def __del__(self):
         h = getattr(self, "_handle", None)
@@ -184,3 +232,72 @@ class RecurrentNetwork:
             else:
                 x = cell(x, carry[i], fresh, out=carry[i])
         return self.output_proj(x, out=out)
+
+    # ------------------------------------------------------------------ training: backward pass through time (GRU stacks)
+    def train_init(self) -> None:
+        if self.lstm:
+            raise _lib.KsError("the backward pass through time is built for GRU stacks")
+        self.input_proj.train_init()
+        for c in self.cells:
+            c.train_init()
+        self.output_proj.train_init()
+
+    def train_forward(self, obs: torch.Tensor, carry0: torch.Tensor, fresh: torch.Tensor) -> torch.Tensor:
+        """The network over a trajectory, obs (T, M, in), starting from carry0 (depth, M, H); envs flagged in fresh (T, M)
+        uint8 start an episode at that step (their carry is zero there).  Returns (T, M, out) and keeps what `backward`
+        needs.  This is the scan over time inside the loss of PPOTask._single_step (ksim/task/ppo.py:572-694)."""
+        T_, M = obs.shape[0], obs.shape[1]
+        H, dev = self.hidden_size, obs.device
+        _lib.require_cuda(obs, carry0, dtype=torch.float32)
+        _lib.require_cuda(fresh, dtype=torch.uint8)
+        if tuple(obs.shape) != (T_, M, self.in_dim) or tuple(carry0.shape) != (self.depth, M, H) or tuple(fresh.shape) != (T_, M):
+            raise _lib.KsError("expected obs (T, M, in), carry0 (depth, M, H), fresh (T, M)")
+        obs = obs.contiguous()
+        x = self.input_proj(obs.view(T_ * M, self.in_dim)).view(T_, M, H)
+        xs, saved = [], []
+        for i, cell in enumerate(self.cells):
+            hs = torch.empty(T_, M, H, dtype=torch.float32, device=dev)
+            sv = torch.empty(T_, M, 5 * H, dtype=torch.float32, device=dev)
+            for t in range(T_):
+                cell.train_forward(x[t], carry0[i] if t == 0 else hs[t - 1], fresh[t], hs[t], sv[t])
+            xs.append(x)
+            saved.append(sv)
+            x = hs
+        out = self.output_proj.train_forward(x.view(T_ * M, H)).view(T_, M, self.out_dim)
+        self._tape = dict(obs=obs, xs=xs, saved=saved, top=x, fresh=fresh.contiguous(), T=T_, M=M)
+        return out
+
+    def backward(self, d_out: torch.Tensor) -> None:
+        """Gradients of sum(d_out * output) with respect to every parameter, into the handles (the jax.grad through the
+        scan).  Per layer, top to bottom: a sweep over the steps, last to first, that carries the gradient of the hidden
+        state, then one pass over all (step, env) rows for the weight gradients and the gradient of the layer's inputs."""
+        tp = self._tape
+        T_, M, H = tp["T"], tp["M"], self.hidden_size
+        dev = d_out.device
+        _lib.require_cuda(d_out, dtype=torch.float32)
+        if tuple(d_out.shape) != (T_, M, self.out_dim):
+            raise _lib.KsError("d_out must have the shape of the output")
+        dH = torch.empty(T_, M, H, dtype=torch.float32, device=dev)
+        self.output_proj.backward_dx(tp["top"].view(T_ * M, H), d_out.contiguous().view(T_ * M, self.out_dim), dH.view(T_ * M, H))
+        for i in range(self.depth - 1, -1, -1):
+            cell, sv = self.cells[i], tp["saved"][i]
+            d_gi = torch.empty(T_, M, 3 * H, dtype=torch.float32, device=dev)
+            d_gh = torch.empty(T_, M, 3 * H, dtype=torch.float32, device=dev)
+            carry = torch.zeros(2, M, H, dtype=torch.float32, device=dev)
+            for t in range(T_ - 1, -1, -1):
+                dH[t] += carry[t & 1]
+                cell.backward_step(dH[t], sv[t], tp["fresh"][t], d_gi[t], d_gh[t], carry[(t + 1) & 1])
+            h_used = sv[:, :, 4 * H:].contiguous().view(T_ * M, H)
+            cell.proj_h.backward(h_used, d_gh.view(T_ * M, 3 * H))
+            dX = torch.empty(T_, M, H, dtype=torch.float32, device=dev)
+            cell.proj_i.backward_dx(tp["xs"][i].reshape(T_ * M, H), d_gi.view(T_ * M, 3 * H), dX.view(T_ * M, H))
+            dH = dX
+        self.input_proj.backward(tp["obs"].view(T_ * M, self.in_dim), dH.view(T_ * M, H))
+
+    def grad_sqnorm(self, acc: torch.Tensor) -> None:
+        for net in (self.input_proj, *self.cells, self.output_proj):
+            net.grad_sqnorm(acc)
+
+    def adam_step(self, params, sqnorm) -> None:
+        for net in (self.input_proj, *self.cells, self.output_proj):
+            net.adam_step(params, sqnorm)

@@ -68,3 +68,60 @@ def recurrent_network(obs, carry, fresh, input_proj, cells, out_weights, out_bia
             x = gru_cell(x, h, *c)
             new.append(x)
     return mlp(x, out_weights, out_biases, act), np.stack(new)
+
+
+def elu(x):
+    x = np.asarray(x, dtype=np.float64)
+    return np.where(x > 0, x, np.expm1(np.minimum(x, 0.0)))
+
+
+def recurrent_sequence(obs, carry0, fresh, input_proj, cells, out_weights, out_biases, act=elu):
+    """The GRU network over a trajectory obs (T, N, in): `recurrent_network` step after step.  Returns (T, N, out)."""
+    carry, outs = np.asarray(carry0, dtype=np.float64), []
+    for t in range(len(obs)):
+        y, carry = recurrent_network(obs[t], carry, fresh[t], input_proj, cells, out_weights, out_biases, act)
+        outs.append(y)
+    return np.stack(outs)
+
+
+def recurrent_sequence_gradients(obs, carry0, fresh, input_proj, cells, out_weights, out_biases, d_out, act="elu"):
+    """Gradients of sum(d_out * recurrent_sequence(...)) with respect to every parameter: the backward pass through time
+    that jax.grad performs through the scan over the trajectory (ksim/task/ppo.py:572-694).  The same equations as
+    `recurrent_sequence`, written with torch float64 tensors so that the library's reverse-mode differentiation yields the
+    gradients; tests pin the forward value to `recurrent_sequence` and single entries to central differences of it.
+    Returns (outputs, dict(input_proj=(dW, db), cells=[(dW_ih, dW_hh, db, db_n)], out=[(dW, db)]))."""
+    import torch
+
+    f = {"elu": torch.nn.functional.elu, "tanh": torch.tanh, "relu": torch.relu}[act]
+    t64 = lambda a: torch.tensor(np.asarray(a, dtype=np.float64), requires_grad=True)  # noqa: E731
+    wp, bp = t64(input_proj[0]), t64(input_proj[1])
+    cs = [tuple(t64(p) for p in c) for c in cells]
+    ow, ob = [t64(w) for w in out_weights], [t64(b) for b in out_biases]
+    obs_t = torch.tensor(np.asarray(obs, dtype=np.float64))
+    carry = torch.tensor(np.asarray(carry0, dtype=np.float64))
+    outs = []
+    for t in range(obs_t.shape[0]):
+        keep = torch.tensor(1.0 - np.asarray(fresh[t], dtype=np.float64))
+        carry = carry * keep[None, :, None]
+        x = obs_t[t] @ wp.T + bp
+        new = []
+        for (wi, wh, b, bn), h in zip(cs, carry):
+            H = h.shape[-1]
+            gi, gh = x @ wi.T + b, h @ wh.T
+            r = torch.sigmoid(gi[:, :H] + gh[:, :H])
+            z = torch.sigmoid(gi[:, H:2 * H] + gh[:, H:2 * H])
+            n = torch.tanh(gi[:, 2 * H:] + r * (gh[:, 2 * H:] + bn))
+            x = n + z * (h - n)
+            new.append(x)
+        carry = torch.stack(new)
+        y = x
+        for i, (w, b) in enumerate(zip(ow, ob)):
+            y = y @ w.T + b
+            if i + 1 < len(ow):
+                y = f(y)
+        outs.append(y)
+    out = torch.stack(outs)
+    (out * torch.tensor(np.asarray(d_out, dtype=np.float64))).sum().backward()
+    g = lambda p: p.grad.numpy()  # noqa: E731
+    return out.detach().numpy(), dict(input_proj=(g(wp), g(bp)), cells=[tuple(g(p) for p in c) for c in cs],
+                                      out=[(g(w), g(b)) for w, b in zip(ow, ob)])

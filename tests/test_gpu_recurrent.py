@@ -136,3 +136,68 @@ def test_lstm_cell_and_network(N, I, H):
         want, want_carry = orec.recurrent_network(obs, want_carry, fr, proj, cells, ow, ob_, act=elu)
         np.testing.assert_allclose(out.cpu().numpy(), want, rtol=2e-4, atol=2e-4)
         np.testing.assert_allclose(carry.cpu().numpy(), want_carry, rtol=2e-4, atol=2e-4)
+
+
+@pytest.mark.parametrize("dtype,tol", [("f32", 2e-4), ("bf16", 6e-2)])
+def test_backward_through_time_matches_the_oracle(dtype, tol):
+    """Gradients of a GRU actor over a trajectory (input projection, two GRU layers, ELU output network) with episode
+    starts inside it, against torch float64 reverse-mode differentiation of the oracle network; then one optimiser step.
+    Tolerances are relative to the largest entry of each gradient array: fp32 accumulation only for f32; for bf16 the
+    activations and the gradients between layers are rounded to bf16 at every one of the T steps."""
+    from ksim_amd import _lib_terms as T
+    from ksim_amd.mlp import MLP
+    from ksim_amd.recurrent import GRUCell, RecurrentNetwork
+
+    rng = np.random.default_rng(41)
+    Tn, N, I, H, O = 12, 96, 37, 64, 10
+    proj = (rng.normal(size=(H, I)) / np.sqrt(I), rng.normal(size=H) * 0.1)
+    cells = [(rng.normal(size=(3 * H, H)) / np.sqrt(H), rng.normal(size=(3 * H, H)) / np.sqrt(H), rng.normal(size=3 * H) * 0.1,
+              rng.normal(size=H) * 0.1) for _ in range(2)]
+    ow = [rng.normal(size=(H, H)) / np.sqrt(H), rng.normal(size=(O, H)) / np.sqrt(H)]
+    ob = [rng.normal(size=H) * 0.1, rng.normal(size=O) * 0.1]
+    obs, carry0 = rng.normal(size=(Tn, N, I)), rng.normal(size=(2, N, H)) * 0.5
+    fresh = rng.random((Tn, N)) < 0.08
+    d_out = rng.normal(size=(Tn, N, O))
+    if dtype == "bf16":  # both sides start from bf16-representable weights
+        rb = lambda a: torch.tensor(a, dtype=torch.float32).to(torch.bfloat16).to(torch.float64).numpy()  # noqa: E731
+        proj = (rb(proj[0]), proj[1]); ow = [rb(w) for w in ow]
+        cells = [(rb(c[0]), rb(c[1]), c[2], c[3]) for c in cells]
+    want_out, want = orec.recurrent_sequence_gradients(obs, carry0, fresh, proj, cells, ow, ob, d_out)
+
+    net = RecurrentNetwork(proj, [GRUCell(*c, dtype=dtype) for c in cells], MLP(ow, ob, activation="elu", dtype=dtype), dtype=dtype)
+    net.train_init()
+    out = net.train_forward(t32(obs), t32(carry0), torch.tensor(fresh, dtype=torch.uint8, device=DEV))
+    scale = np.abs(want_out).max()
+    assert np.abs(out.cpu().numpy() - want_out).max() <= (1e-4 if dtype == "f32" else 3e-2) * scale
+    net.backward(t32(d_out))
+    got = {"input_proj.W": net.input_proj.parameters(True)[0][0], "input_proj.b": net.input_proj.parameters(True)[0][1]}
+    ref = {"input_proj.W": want["input_proj"][0], "input_proj.b": want["input_proj"][1]}
+    for i, c in enumerate(net.cells):
+        g = c.parameters(True)
+        for k, j in (("weight_ih", 0), ("weight_hh", 1), ("bias", 2), ("bias_n", 3)):
+            got[f"cell{i}.{k}"], ref[f"cell{i}.{k}"] = g[k], want["cells"][i][j]
+    for l, (w, b) in enumerate(net.output_proj.parameters(True)):
+        got[f"out{l}.W"], ref[f"out{l}.W"], got[f"out{l}.b"], ref[f"out{l}.b"] = w, want["out"][l][0], b, want["out"][l][1]
+    for k in ref:
+        err = np.abs(got[k].cpu().numpy() - ref[k]).max() / np.abs(ref[k]).max()
+        assert err <= tol, f"{k}: {err:.2e} > {tol}"
+    # the hidden projection has no reset / update bias of its own: those entries stay out of the update
+    before = [c.parameters() for c in net.cells]
+    acc = torch.zeros(1, dtype=torch.float64, device=DEV)
+    net.grad_sqnorm(acc)
+    total = sum(float((np.asarray(v) ** 2).sum()) for v in ref.values())
+    assert acc.item() == pytest.approx(total, rel=2e-3 if dtype == "f32" else 0.15)
+    params = T.KsAdamParams(1e-3, 0.9, 0.999, 1e-8, 0.0, 0.0, 1)
+    net.adam_step(params, None)
+    for c, b0 in zip(net.cells, before):
+        p = c.parameters()
+        (_, bh), = c.proj_h.parameters()
+        assert torch.equal(bh[:2 * H], torch.zeros(2 * H, device=DEV))
+        # first Adam step: every parameter with a gradient moves by lr against the gradient's sign
+        moved = (p["bias_n"] - b0["bias_n"]).cpu().numpy()
+        gn = c.parameters(True)["bias_n"].cpu().numpy()
+        big = np.abs(gn) > 1e-4
+        np.testing.assert_allclose(moved[big], -1e-3 * np.sign(gn[big]), rtol=1e-3)
+    # the forward pass of the rollout sees the updated b_n also for envs that start an episode
+    h1 = net.cells[0](t32(rng.normal(size=(N, H))), t32(np.zeros((N, H))), torch.ones(N, dtype=torch.uint8, device=DEV))
+    assert torch.isfinite(h1).all()
