@@ -626,6 +626,19 @@ int ks_gru_backward_step(KsGru* gru, ks_stream_t stream, int64_t M, const float*
                          const uint8_t* fresh, float* d_gi, float* d_gh, float* dh_in, void* workspace);
 int ks_gru_grad_sqnorm(const KsGru* gru, ks_stream_t stream, double* acc);
 int ks_gru_adam_step(KsGru* gru, ks_stream_t stream, const KsAdamParams* params /*host*/, const double* sqnorm);
+/* The same for LSTM stacks (the recurrent actor and critic of examples/kbot/train.py:903-915): saved is (M, 7H) =
+ * i | f | g | o | tanh(c') | c | h; a step takes dh_out and dc_out and returns d_g (M, 4H), the gradient of both
+ * projections' outputs, with dh_in and dc_in. */
+int ks_lstm_train_init(KsLstm* lstm);
+int ks_lstm_projections(KsLstm* lstm, KsMlp** input_projection, KsMlp** hidden_projection);
+int ks_lstm_train_forward(const KsLstm* lstm, ks_stream_t stream, int64_t M, const float* x, const float* h_in,
+                          const float* c_in, const uint8_t* fresh, float* h_out, float* c_out, float* saved /*(M, 7H)*/,
+                          void* workspace /*ks_lstm_workspace_bytes*/);
+int64_t ks_lstm_backward_workspace_bytes(const KsLstm* lstm, int64_t M);
+int ks_lstm_backward_step(KsLstm* lstm, ks_stream_t stream, int64_t M, const float* dh_out, const float* dc_out,
+                          const float* saved, const uint8_t* fresh, float* d_g, float* dh_in, float* dc_in, void* workspace);
+int ks_lstm_grad_sqnorm(const KsLstm* lstm, ks_stream_t stream, double* acc);
+int ks_lstm_adam_step(KsLstm* lstm, ks_stream_t stream, const KsAdamParams* params /*host*/, const double* sqnorm);
 
 /* Gaussian policy head and the gradient of the PPO objective (ppo.py:149-246, total 473-486):
  *   ks_gaussian_log_prob: per action dimension log N(action; mean, exp(log_std)) and entropy

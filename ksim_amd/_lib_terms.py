@@ -212,8 +212,18 @@ def bind(lib) -> None:
                                          c_void_p]
     lib.ks_gru_grad_sqnorm.argtypes = [c_void_p, c_void_p, c_void_p]
     lib.ks_gru_adam_step.argtypes = [c_void_p, c_void_p, POINTER(KsAdamParams), c_void_p]
+    lib.ks_lstm_train_init.argtypes = [c_void_p]
+    lib.ks_lstm_projections.argtypes = [c_void_p, POINTER(c_void_p), POINTER(c_void_p)]
+    lib.ks_lstm_train_forward.argtypes = [c_void_p, c_void_p, c_int64] + [c_void_p] * 8
+    lib.ks_lstm_backward_workspace_bytes.argtypes = [c_void_p, c_int64]
+    lib.ks_lstm_backward_workspace_bytes.restype = c_int64
+    lib.ks_lstm_backward_step.argtypes = [c_void_p, c_void_p, c_int64] + [c_void_p] * 8
+    lib.ks_lstm_grad_sqnorm.argtypes = [c_void_p, c_void_p, c_void_p]
+    lib.ks_lstm_adam_step.argtypes = [c_void_p, c_void_p, POINTER(KsAdamParams), c_void_p]
     for name in ("ks_mlp_train_backward_dx", "ks_mlp_freeze_bias_prefix", "ks_gru_train_init", "ks_gru_projections",
-                 "ks_gru_train_forward", "ks_gru_backward_step", "ks_gru_grad_sqnorm", "ks_gru_adam_step"):
+                 "ks_gru_train_forward", "ks_gru_backward_step", "ks_gru_grad_sqnorm", "ks_gru_adam_step",
+                 "ks_lstm_train_init", "ks_lstm_projections", "ks_lstm_train_forward", "ks_lstm_backward_step",
+                 "ks_lstm_grad_sqnorm", "ks_lstm_adam_step"):
         getattr(lib, name).restype = c_int32
     lib.ks_mlp_grad_sqnorm.argtypes = [c_void_p, c_void_p, c_void_p]
     lib.ks_mlp_adam_step.argtypes = [c_void_p, c_void_p, POINTER(KsAdamParams), c_void_p]

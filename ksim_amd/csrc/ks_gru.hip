@@ -102,6 +102,59 @@ __global__ __launch_bounds__(256) void lstm_gate_kernel(int64_t M, int H, const 
   h_out[idx] = so * tanhf(cn);
 }
 
+// The LSTM cell for training: saved (M, 7H) = i | f | g | o | tanh(c') | c | h with the gate activations, the cell and
+// hidden state the step actually used (zero for a fresh env).
+__global__ __launch_bounds__(256) void lstm_gate_train_kernel(int64_t M, int H, const float* __restrict__ gi,
+                                                              const float* __restrict__ gh, const float* __restrict__ h_in,
+                                                              const float* __restrict__ c_in, const uint8_t* __restrict__ fresh,
+                                                              float* __restrict__ h_out, float* __restrict__ c_out,
+                                                              float* __restrict__ saved) {
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= M * H) return;
+  const int64_t m = idx / H;
+  const int j = (int)(idx - m * H);
+  const bool f = fresh && fresh[m];
+  const float* a = gi + m * 4 * H;
+  const float* b = gh + m * 4 * H;
+  float g[4];
+#pragma unroll
+  for (int k = 0; k < 4; ++k) g[k] = a[k * H + j] + (f ? 0.f : b[k * H + j]);
+  const float c = f ? 0.f : c_in[idx], h = f ? 0.f : h_in[idx];
+  const float si = 1.f / (1.f + expf(-g[0])), sf = 1.f / (1.f + expf(-g[1])), so = 1.f / (1.f + expf(-g[3]));
+  const float tg = tanhf(g[2]);
+  const float cn = sf * c + si * tg;
+  const float tc = tanhf(cn);
+  c_out[idx] = cn;
+  h_out[idx] = so * tc;
+  float* sv = saved + m * 7 * H;
+  sv[j] = si; sv[H + j] = sf; sv[2 * H + j] = tg; sv[3 * H + j] = so; sv[4 * H + j] = tc; sv[5 * H + j] = c; sv[6 * H + j] = h;
+}
+
+// Backward through the gates of one LSTM step: dh_out, dc_out are the gradients reaching h' and c'.  d_g (M, 4H) is the
+// gradient of the summed gate pre-activations, hence of both projections' outputs; dc_in = dc f is the gradient of the
+// incoming cell state and dh_in starts at zero (the hidden projection adds its share afterwards); both are zero for a fresh env.
+__global__ __launch_bounds__(256) void lstm_gate_backward_kernel(int64_t M, int H, const float* __restrict__ dh_out,
+                                                                 const float* __restrict__ dc_out, const float* __restrict__ saved,
+                                                                 const uint8_t* __restrict__ fresh, float* __restrict__ d_g,
+                                                                 float* __restrict__ dh_in, float* __restrict__ dc_in) {
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= M * H) return;
+  const int64_t m = idx / H;
+  const int j = (int)(idx - m * H);
+  const bool f = fresh && fresh[m];
+  const float* sv = saved + m * 7 * H;
+  const float si = sv[j], sf = sv[H + j], tg = sv[2 * H + j], so = sv[3 * H + j], tc = sv[4 * H + j], c = sv[5 * H + j];
+  const float dh = dh_out[idx];
+  const float dc = dc_out[idx] + dh * so * (1.f - tc * tc);
+  float* a = d_g + m * 4 * H;
+  a[j] = dc * tg * si * (1.f - si);
+  a[H + j] = dc * c * sf * (1.f - sf);
+  a[2 * H + j] = dc * si * (1.f - tg * tg);
+  a[3 * H + j] = dh * tc * so * (1.f - so);
+  dc_in[idx] = f ? 0.f : dc * sf;
+  dh_in[idx] = 0.f;
+}
+
 }  // namespace ks
 
 using namespace ks;
@@ -317,4 +370,77 @@ extern "C" int ks_lstm_forward(const KsLstm* g, ks_stream_t stream, int64_t M, c
   hipLaunchKernelGGL(lstm_gate_kernel, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, M, g->H, gi, gh, c_in, fresh,
                      h_out, c_out);
   return check_launch("ks_lstm_forward");
+}
+
+extern "C" int ks_lstm_train_init(KsLstm* g) {
+  if (!g) return fail(KS_EINVAL, "ks_lstm_train_init: null handle");
+  int rc = ks_mlp_train_init(g->proj_i);
+  if (rc == KS_OK) rc = ks_mlp_train_init(g->proj_h);
+  // the cell has one bias, carried by the input projection: the hidden projection's stays zero
+  if (rc == KS_OK) rc = ks_mlp_freeze_bias_prefix(g->proj_h, 0, 4 * g->H);
+  return rc;
+}
+
+extern "C" int ks_lstm_projections(KsLstm* g, KsMlp** input_projection, KsMlp** hidden_projection) {
+  if (!g || !input_projection || !hidden_projection) return fail(KS_EINVAL, "ks_lstm_projections: null argument");
+  *input_projection = g->proj_i;
+  *hidden_projection = g->proj_h;
+  return KS_OK;
+}
+
+extern "C" int ks_lstm_train_forward(const KsLstm* g, ks_stream_t stream, int64_t M, const float* x, const float* h_in,
+                                     const float* c_in, const uint8_t* fresh, float* h_out, float* c_out, float* saved,
+                                     void* workspace) {
+  if (!g || !x || !h_in || !c_in || !h_out || !c_out || !saved) return fail(KS_EINVAL, "ks_lstm_train_forward: null argument");
+  if (M < 0) return fail(KS_EINVAL, "ks_lstm_train_forward: negative row count");
+  if (M == 0) return KS_OK;
+  if (!workspace) return fail(KS_EINVAL, "ks_lstm_train_forward: workspace is required");
+  const int64_t gates = up256(M * 4 * g->H * 4);
+  char* w = (char*)workspace;
+  float* gi = (float*)w;
+  float* gh = (float*)(w + gates);
+  void* wi = w + 2 * gates;
+  void* wh = w + 2 * gates + up256(ks_mlp_workspace_bytes(g->proj_i, M));
+  int rc = ks_mlp_forward(g->proj_i, stream, M, x, gi, wi);
+  if (rc != KS_OK) return rc;
+  rc = ks_mlp_forward(g->proj_h, stream, M, h_in, gh, wh);
+  if (rc != KS_OK) return rc;
+  const int64_t n = M * g->H, grid = (n + 255) / 256;
+  if (grid > 0x7fffffff) return fail(KS_ELIMIT, "ks_lstm_train_forward: too many elements");
+  hipLaunchKernelGGL(lstm_gate_train_kernel, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, M, g->H, gi, gh, h_in, c_in,
+                     fresh, h_out, c_out, saved);
+  return check_launch("ks_lstm_train_forward");
+}
+
+extern "C" int64_t ks_lstm_backward_workspace_bytes(const KsLstm* g, int64_t M) {
+  if (!g || M < 0) return -1;
+  return ks_mlp_train_workspace_bytes(g->proj_h, M);
+}
+
+extern "C" int ks_lstm_backward_step(KsLstm* g, ks_stream_t stream, int64_t M, const float* dh_out, const float* dc_out,
+                                     const float* saved, const uint8_t* fresh, float* d_g, float* dh_in, float* dc_in,
+                                     void* workspace) {
+  if (!g || !dh_out || !dc_out || !saved || !d_g || !dh_in || !dc_in || !workspace) return fail(KS_EINVAL, "ks_lstm_backward_step: null argument");
+  if (M < 0) return fail(KS_EINVAL, "ks_lstm_backward_step: negative row count");
+  if (M == 0) return KS_OK;
+  const int64_t n = M * g->H, grid = (n + 255) / 256;
+  if (grid > 0x7fffffff) return fail(KS_ELIMIT, "ks_lstm_backward_step: too many elements");
+  hipLaunchKernelGGL(lstm_gate_backward_kernel, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, M, g->H, dh_out, dc_out,
+                     saved, fresh, d_g, dh_in, dc_in);
+  const int rc = check_launch("ks_lstm_backward_step");
+  if (rc != KS_OK) return rc;
+  // dh_in = d_g W_hh, except across an episode boundary
+  return ks_mlp_train_backward_dx(g->proj_h, stream, M, nullptr, d_g, dh_in, 0, 1, fresh, workspace);
+}
+
+extern "C" int ks_lstm_grad_sqnorm(const KsLstm* g, ks_stream_t stream, double* acc) {
+  if (!g || !acc) return fail(KS_EINVAL, "ks_lstm_grad_sqnorm: null argument");
+  const int rc = ks_mlp_grad_sqnorm(g->proj_i, stream, acc);
+  return rc != KS_OK ? rc : ks_mlp_grad_sqnorm(g->proj_h, stream, acc);
+}
+
+extern "C" int ks_lstm_adam_step(KsLstm* g, ks_stream_t stream, const KsAdamParams* params, const double* sqnorm) {
+  if (!g) return fail(KS_EINVAL, "ks_lstm_adam_step: null handle");
+  const int rc = ks_mlp_adam_step(g->proj_i, stream, params, sqnorm);
+  return rc != KS_OK ? rc : ks_mlp_adam_step(g->proj_h, stream, params, sqnorm);
 }

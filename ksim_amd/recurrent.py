@@ -186,6 +186,54 @@ class LSTMCell:
                                              _lib.ptr(fresh), _lib.ptr(ho), _lib.ptr(co), _lib.ptr(ws)))
         return ho, co
 
+    # ------------------------------------------------------------------ training (ksim/task/ppo.py:572-694)
+    def train_init(self) -> None:
+        _lib.check(self._lib.ks_lstm_train_init(self._handle))
+        pi, ph = ctypes.c_void_p(), ctypes.c_void_p()
+        _lib.check(self._lib.ks_lstm_projections(self._handle, ctypes.byref(pi), ctypes.byref(ph)))
+        H = self.hidden_size
+        self.proj_i = MLP._borrow(self._lib, pi, (self.input_size, 4 * H), self.dtype)
+        self.proj_h = MLP._borrow(self._lib, ph, (H, 4 * H), self.dtype)
+        self._bws: torch.Tensor | None = None
+
+    def train_forward(self, x, h, c, fresh, h_out, c_out, saved) -> None:
+        """`__call__` that also fills `saved` (M, 7H) = i | f | g | o | tanh(c') | c | h for `backward_step`."""
+        _lib.require_cuda(x, h, c, h_out, c_out, saved, dtype=torch.float32)
+        _lib.require_cuda(fresh, dtype=torch.uint8)
+        M, H = x.shape[0], self.hidden_size
+        if tuple(x.shape) != (M, self.input_size) or any(tuple(t.shape) != (M, H) for t in (h, c, h_out, c_out)) or tuple(saved.shape) != (M, 7 * H):
+            raise _lib.KsError("expected x (M, input), h, c and outputs (M, H), saved (M, 7H)")
+        _lib.check(self._lib.ks_lstm_train_forward(self._handle, _lib.current_stream(), M, _lib.ptr(x), _lib.ptr(h), _lib.ptr(c),
+                                                   _lib.ptr(fresh), _lib.ptr(h_out), _lib.ptr(c_out), _lib.ptr(saved),
+                                                   _lib.ptr(self.workspace(M, x.device))))
+
+    def backward_step(self, dh_out, dc_out, saved, fresh, d_g, dh_in, dc_in) -> None:
+        """One step of the backward pass through time: (dh_out, dc_out) -> d_g (M, 4H), dh_in, dc_in (M, H)."""
+        _lib.require_cuda(dh_out, dc_out, saved, d_g, dh_in, dc_in, dtype=torch.float32)
+        _lib.require_cuda(fresh, dtype=torch.uint8)
+        M, H = dh_out.shape[0], self.hidden_size
+        if (any(tuple(t.shape) != (M, H) for t in (dh_out, dc_out, dh_in, dc_in)) or tuple(saved.shape) != (M, 7 * H)
+                or tuple(d_g.shape) != (M, 4 * H)):
+            raise _lib.KsError("expected gradients of the states (M, H), saved (M, 7H), d_g (M, 4H)")
+        need = int(self._lib.ks_lstm_backward_workspace_bytes(self._handle, M))
+        if self._bws is None or self._bws.numel() < need or self._bws.device != dh_out.device:
+            self._bws = torch.empty(need, dtype=torch.uint8, device=dh_out.device)
+        _lib.check(self._lib.ks_lstm_backward_step(self._handle, _lib.current_stream(), M, _lib.ptr(dh_out), _lib.ptr(dc_out),
+                                                   _lib.ptr(saved), _lib.ptr(fresh), _lib.ptr(d_g), _lib.ptr(dh_in),
+                                                   _lib.ptr(dc_in), _lib.ptr(self._bws)))
+
+    def grad_sqnorm(self, acc: torch.Tensor) -> None:
+        _lib.check(self._lib.ks_lstm_grad_sqnorm(self._handle, _lib.current_stream(), _lib.ptr(acc)))
+
+    def adam_step(self, params, sqnorm) -> None:
+        _lib.check(self._lib.ks_lstm_adam_step(self._handle, _lib.current_stream(), ctypes.byref(params), _lib.ptr(sqnorm)))
+
+    def parameters(self, gradients: bool = False) -> dict:
+        """Copies of weight_ih, weight_hh and bias (4H), or of their gradients."""
+        (wi, bi), = self.proj_i.parameters(gradients)
+        (wh, _), = self.proj_h.parameters(gradients)
+        return dict(weight_ih=wi, weight_hh=wh, bias=bi)
+
     def __del__(self):
         h = getattr(self, "_handle", None)
         if h:
@@ -233,33 +281,39 @@ class RecurrentNetwork:
                 x = cell(x, carry[i], fresh, out=carry[i])
         return self.output_proj(x, out=out)
 
-    # ------------------------------------------------------------------ training: backward pass through time (GRU stacks)
+    # ------------------------------------------------------------------ training: backward pass through time
     def train_init(self) -> None:
-        if self.lstm:
-            raise _lib.KsError("the backward pass through time is built for GRU stacks")
         self.input_proj.train_init()
         for c in self.cells:
             c.train_init()
         self.output_proj.train_init()
 
     def train_forward(self, obs: torch.Tensor, carry0: torch.Tensor, fresh: torch.Tensor) -> torch.Tensor:
-        """The network over a trajectory, obs (T, M, in), starting from carry0 (depth, M, H); envs flagged in fresh (T, M)
-        uint8 start an episode at that step (their carry is zero there).  Returns (T, M, out) and keeps what `backward`
-        needs.  This is the scan over time inside the loss of PPOTask._single_step (ksim/task/ppo.py:572-694)."""
+        """The network over a trajectory, obs (T, M, in), starting from carry0 (the rollout's carry layout); envs flagged
+        in fresh (T, M) uint8 start an episode at that step (their carry is zero there).  Returns (T, M, out) and keeps
+        what `backward` needs.  This is the scan over time inside the loss of PPOTask._single_step
+        (ksim/task/ppo.py:572-694)."""
         T_, M = obs.shape[0], obs.shape[1]
         H, dev = self.hidden_size, obs.device
         _lib.require_cuda(obs, carry0, dtype=torch.float32)
         _lib.require_cuda(fresh, dtype=torch.uint8)
-        if tuple(obs.shape) != (T_, M, self.in_dim) or tuple(carry0.shape) != (self.depth, M, H) or tuple(fresh.shape) != (T_, M):
-            raise _lib.KsError("expected obs (T, M, in), carry0 (depth, M, H), fresh (T, M)")
+        want = (self.depth, 2, M, H) if self.lstm else (self.depth, M, H)
+        if tuple(obs.shape) != (T_, M, self.in_dim) or tuple(carry0.shape) != want or tuple(fresh.shape) != (T_, M):
+            raise _lib.KsError(f"expected obs (T, M, in), carry0 {want}, fresh (T, M)")
         obs = obs.contiguous()
         x = self.input_proj(obs.view(T_ * M, self.in_dim)).view(T_, M, H)
         xs, saved = [], []
         for i, cell in enumerate(self.cells):
             hs = torch.empty(T_, M, H, dtype=torch.float32, device=dev)
-            sv = torch.empty(T_, M, 5 * H, dtype=torch.float32, device=dev)
-            for t in range(T_):
-                cell.train_forward(x[t], carry0[i] if t == 0 else hs[t - 1], fresh[t], hs[t], sv[t])
+            sv = torch.empty(T_, M, (7 if self.lstm else 5) * H, dtype=torch.float32, device=dev)
+            if self.lstm:
+                cs = torch.empty(T_, M, H, dtype=torch.float32, device=dev)
+                for t in range(T_):
+                    h0, c0 = (carry0[i, 0], carry0[i, 1]) if t == 0 else (hs[t - 1], cs[t - 1])
+                    cell.train_forward(x[t], h0, c0, fresh[t], hs[t], cs[t], sv[t])
+            else:
+                for t in range(T_):
+                    cell.train_forward(x[t], carry0[i] if t == 0 else hs[t - 1], fresh[t], hs[t], sv[t])
             xs.append(x)
             saved.append(sv)
             x = hs
@@ -269,10 +323,12 @@ class RecurrentNetwork:
 
     def backward(self, d_out: torch.Tensor) -> None:
         """Gradients of sum(d_out * output) with respect to every parameter, into the handles (the jax.grad through the
-        scan).  Per layer, top to bottom: a sweep over the steps, last to first, that carries the gradient of the hidden
-        state, then one pass over all (step, env) rows for the weight gradients and the gradient of the layer's inputs."""
+        scan).  Per layer, top to bottom: a sweep over the steps, last to first, that carries the gradient of the
+        recurrent state, then one pass over all (step, env) rows for the weight gradients and the gradient of the layer's
+        inputs."""
         tp = self._tape
         T_, M, H = tp["T"], tp["M"], self.hidden_size
+        G = 4 if self.lstm else 3
         dev = d_out.device
         _lib.require_cuda(d_out, dtype=torch.float32)
         if tuple(d_out.shape) != (T_, M, self.out_dim):
@@ -281,16 +337,20 @@ class RecurrentNetwork:
         self.output_proj.backward_dx(tp["top"].view(T_ * M, H), d_out.contiguous().view(T_ * M, self.out_dim), dH.view(T_ * M, H))
         for i in range(self.depth - 1, -1, -1):
             cell, sv = self.cells[i], tp["saved"][i]
-            d_gi = torch.empty(T_, M, 3 * H, dtype=torch.float32, device=dev)
-            d_gh = torch.empty(T_, M, 3 * H, dtype=torch.float32, device=dev)
-            carry = torch.zeros(2, M, H, dtype=torch.float32, device=dev)
+            d_gi = torch.empty(T_, M, G * H, dtype=torch.float32, device=dev)
+            d_gh = d_gi if self.lstm else torch.empty(T_, M, G * H, dtype=torch.float32, device=dev)
+            carry = torch.zeros(2, M, H, dtype=torch.float32, device=dev)   # gradient of the hidden state, ping-pong
+            ccarry = torch.zeros(2, M, H, dtype=torch.float32, device=dev)  # and of the cell state (LSTM)
             for t in range(T_ - 1, -1, -1):
                 dH[t] += carry[t & 1]
-                cell.backward_step(dH[t], sv[t], tp["fresh"][t], d_gi[t], d_gh[t], carry[(t + 1) & 1])
-            h_used = sv[:, :, 4 * H:].contiguous().view(T_ * M, H)
-            cell.proj_h.backward(h_used, d_gh.view(T_ * M, 3 * H))
+                if self.lstm:
+                    cell.backward_step(dH[t], ccarry[t & 1], sv[t], tp["fresh"][t], d_gi[t], carry[(t + 1) & 1], ccarry[(t + 1) & 1])
+                else:
+                    cell.backward_step(dH[t], sv[t], tp["fresh"][t], d_gi[t], d_gh[t], carry[(t + 1) & 1])
+            h_used = sv[:, :, (6 if self.lstm else 4) * H:].contiguous().view(T_ * M, H)
+            cell.proj_h.backward(h_used, d_gh.view(T_ * M, G * H))
             dX = torch.empty(T_, M, H, dtype=torch.float32, device=dev)
-            cell.proj_i.backward_dx(tp["xs"][i].reshape(T_ * M, H), d_gi.view(T_ * M, 3 * H), dX.view(T_ * M, H))
+            cell.proj_i.backward_dx(tp["xs"][i].reshape(T_ * M, H), d_gi.view(T_ * M, G * H), dX.view(T_ * M, H))
             dH = dX
         self.input_proj.backward(tp["obs"].view(T_ * M, self.in_dim), dH.view(T_ * M, H))
 

@@ -89,7 +89,9 @@ def recurrent_sequence_gradients(obs, carry0, fresh, input_proj, cells, out_weig
     that jax.grad performs through the scan over the trajectory (ksim/task/ppo.py:572-694).  The same equations as
     `recurrent_sequence`, written with torch float64 tensors so that the library's reverse-mode differentiation yields the
     gradients; tests pin the forward value to `recurrent_sequence` and single entries to central differences of it.
-    Returns (outputs, dict(input_proj=(dW, db), cells=[(dW_ih, dW_hh, db, db_n)], out=[(dW, db)]))."""
+    GRU cells are (weight_ih, weight_hh, bias, bias_n) with carry (depth, N, H); LSTM cells (weight_ih, weight_hh, bias)
+    with carry (depth, 2, N, H).
+    Returns (outputs, dict(input_proj=(dW, db), cells=[one gradient per cell parameter], out=[(dW, db)]))."""
     import torch
 
     f = {"elu": torch.nn.functional.elu, "tanh": torch.tanh, "relu": torch.relu}[act]
@@ -99,20 +101,30 @@ def recurrent_sequence_gradients(obs, carry0, fresh, input_proj, cells, out_weig
     ow, ob = [t64(w) for w in out_weights], [t64(b) for b in out_biases]
     obs_t = torch.tensor(np.asarray(obs, dtype=np.float64))
     carry = torch.tensor(np.asarray(carry0, dtype=np.float64))
+    lstm = carry.ndim == 4
     outs = []
     for t in range(obs_t.shape[0]):
         keep = torch.tensor(1.0 - np.asarray(fresh[t], dtype=np.float64))
-        carry = carry * keep[None, :, None]
+        carry = carry * (keep[None, None, :, None] if lstm else keep[None, :, None])
         x = obs_t[t] @ wp.T + bp
         new = []
-        for (wi, wh, b, bn), h in zip(cs, carry):
-            H = h.shape[-1]
-            gi, gh = x @ wi.T + b, h @ wh.T
-            r = torch.sigmoid(gi[:, :H] + gh[:, :H])
-            z = torch.sigmoid(gi[:, H:2 * H] + gh[:, H:2 * H])
-            n = torch.tanh(gi[:, 2 * H:] + r * (gh[:, 2 * H:] + bn))
-            x = n + z * (h - n)
-            new.append(x)
+        for c, h in zip(cs, carry):
+            if lstm:  # (weight_ih, weight_hh, bias), carry entry (2, N, H)
+                wi, wh, b = c
+                H = h.shape[-1]
+                g = x @ wi.T + h[0] @ wh.T + b
+                cn = torch.sigmoid(g[:, H:2 * H]) * h[1] + torch.sigmoid(g[:, :H]) * torch.tanh(g[:, 2 * H:3 * H])
+                x = torch.sigmoid(g[:, 3 * H:]) * torch.tanh(cn)
+                new.append(torch.stack([x, cn]))
+            else:
+                wi, wh, b, bn = c
+                H = h.shape[-1]
+                gi, gh = x @ wi.T + b, h @ wh.T
+                r = torch.sigmoid(gi[:, :H] + gh[:, :H])
+                z = torch.sigmoid(gi[:, H:2 * H] + gh[:, H:2 * H])
+                n = torch.tanh(gi[:, 2 * H:] + r * (gh[:, 2 * H:] + bn))
+                x = n + z * (h - n)
+                new.append(x)
         carry = torch.stack(new)
         y = x
         for i, (w, b) in enumerate(zip(ow, ob)):

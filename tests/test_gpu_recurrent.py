@@ -201,3 +201,44 @@ def test_backward_through_time_matches_the_oracle(dtype, tol):
     # the forward pass of the rollout sees the updated b_n also for envs that start an episode
     h1 = net.cells[0](t32(rng.normal(size=(N, H))), t32(np.zeros((N, H))), torch.ones(N, dtype=torch.uint8, device=DEV))
     assert torch.isfinite(h1).all()
+
+
+@pytest.mark.parametrize("dtype,tol", [("f32", 2e-4), ("bf16", 6e-2)])
+def test_lstm_backward_through_time_matches_the_oracle(dtype, tol):
+    """The same for an LSTM stack (the K-Bot example's actor shape: projection, LSTM layers, linear output)."""
+    from ksim_amd import _lib_terms as T
+    from ksim_amd.mlp import MLP
+    from ksim_amd.recurrent import LSTMCell, RecurrentNetwork
+
+    rng = np.random.default_rng(43)
+    Tn, N, I, H, O = 10, 80, 29, 64, 12
+    proj = (rng.normal(size=(H, I)) / np.sqrt(I), rng.normal(size=H) * 0.1)
+    cells = [(rng.normal(size=(4 * H, H)) / np.sqrt(H), rng.normal(size=(4 * H, H)) / np.sqrt(H), rng.normal(size=4 * H) * 0.1)
+             for _ in range(2)]
+    ow, ob = [rng.normal(size=(O, H)) / np.sqrt(H)], [rng.normal(size=O) * 0.1]
+    obs, carry0 = rng.normal(size=(Tn, N, I)), rng.normal(size=(2, 2, N, H)) * 0.5
+    fresh = rng.random((Tn, N)) < 0.08
+    d_out = rng.normal(size=(Tn, N, O))
+    if dtype == "bf16":
+        proj = (_bf16(proj[0]), proj[1]); ow = [_bf16(w) for w in ow]
+        cells = [(_bf16(c[0]), _bf16(c[1]), c[2]) for c in cells]
+    want_out, want = orec.recurrent_sequence_gradients(obs, carry0, fresh, proj, cells, ow, ob, d_out)
+    net = RecurrentNetwork(proj, [LSTMCell(*c, dtype=dtype) for c in cells], MLP(ow, ob, activation="none", dtype=dtype), dtype=dtype)
+    net.train_init()
+    out = net.train_forward(t32(obs), t32(carry0), torch.tensor(fresh, dtype=torch.uint8, device=DEV))
+    assert np.abs(out.cpu().numpy() - want_out).max() <= (1e-4 if dtype == "f32" else 3e-2) * np.abs(want_out).max()
+    net.backward(t32(d_out))
+    got = {"input_proj.W": net.input_proj.parameters(True)[0][0], "input_proj.b": net.input_proj.parameters(True)[0][1],
+           "out.W": net.output_proj.parameters(True)[0][0], "out.b": net.output_proj.parameters(True)[0][1]}
+    ref = {"input_proj.W": want["input_proj"][0], "input_proj.b": want["input_proj"][1], "out.W": want["out"][0][0], "out.b": want["out"][0][1]}
+    for i, c in enumerate(net.cells):
+        g = c.parameters(True)
+        for k, j in (("weight_ih", 0), ("weight_hh", 1), ("bias", 2)):
+            got[f"cell{i}.{k}"], ref[f"cell{i}.{k}"] = g[k], want["cells"][i][j]
+    for k in ref:
+        err = np.abs(got[k].cpu().numpy() - ref[k]).max() / np.abs(ref[k]).max()
+        assert err <= tol, f"{k}: {err:.2e} > {tol}"
+    net.adam_step(T.KsAdamParams(1e-3, 0.9, 0.999, 1e-8, 0.0, 0.0, 1), None)
+    for c in net.cells:  # the hidden projection carries no bias of its own, before and after the update
+        (_, bh), = c.proj_h.parameters()
+        assert torch.equal(bh, torch.zeros(4 * H, device=DEV))

@@ -111,3 +111,24 @@ def test_sequence_gradients_against_central_differences():
     o1 = orec.recurrent_sequence(obs, carry0, fresh, proj, cells, ow, ob_)
     o2 = orec.recurrent_sequence(obs, c2, fresh, proj, cells, ow, ob_)
     assert np.array_equal(o2[3:, 1], o1[3:, 1]) and not np.allclose(o2[:3, 1], o1[:3, 1])
+
+
+def test_lstm_sequence_gradients_against_central_differences():
+    rng = np.random.default_rng(3)
+    T, N, I, H, O = 5, 3, 4, 6, 2
+    proj = (rng.normal(size=(H, I)) * 0.5, rng.normal(size=H) * 0.1)
+    cells = [(rng.normal(size=(4 * H, H)) * 0.5, rng.normal(size=(4 * H, H)) * 0.5, rng.normal(size=4 * H) * 0.1) for _ in range(2)]
+    ow, ob_ = [rng.normal(size=(H, H)) * 0.5, rng.normal(size=(O, H)) * 0.5], [rng.normal(size=H) * 0.1, rng.normal(size=O) * 0.1]
+    obs, carry0 = rng.normal(size=(T, N, I)), rng.normal(size=(2, 2, N, H))
+    fresh = np.zeros((T, N), bool); fresh[2, 1] = True
+    d_out = rng.normal(size=(T, N, O))
+    out, g = orec.recurrent_sequence_gradients(obs, carry0, fresh, proj, cells, ow, ob_, d_out)
+    np.testing.assert_allclose(out, orec.recurrent_sequence(obs, carry0, fresh, proj, cells, ow, ob_), rtol=1e-12, atol=1e-12)
+    eps = 1e-6
+    for layer, k, idx in [(0, 0, (3, 2)), (0, 1, (20, 4)), (1, 1, (7, 0)), (1, 2, (13,)), (0, 2, (1,)), (1, 0, (23, 5))]:
+        vals = []
+        for s in (+eps, -eps):
+            c2 = [tuple(a.copy() for a in c) for c in cells]
+            c2[layer][k][idx] += s
+            vals.append(float((orec.recurrent_sequence(obs, carry0, fresh, proj, c2, ow, ob_) * d_out).sum()))
+        assert g["cells"][layer][k][idx] == pytest.approx((vals[0] - vals[1]) / (2 * eps), rel=1e-6, abs=1e-8)
