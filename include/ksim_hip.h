@@ -656,6 +656,14 @@ int ks_ppo_loss_grad(ks_stream_t stream, int64_t M, int32_t nu, const KsPpoLossP
                      const float* values, float* d_mean /*(M,nu)*/, float* d_value /*(M)*/, float* d_log_std /*(nu)*/,
                      void* workspace);
 
+/* ks_ppo_loss_grad for a network with the mean | raw deviation head of ks_sample_action_head (examples/kbot/train.py:
+ * 915-932): raw is (M, 2 nu); d_raw (M, 2 nu) receives the gradient with respect to both halves (through the softplus,
+ * the scale and the cap of the deviation), which is what the network's backward pass takes. */
+int ks_ppo_loss_grad_head(ks_stream_t stream, int64_t M, int32_t nu, const KsPpoLossParams* params /*host*/,
+                          const KsGaussianHead* head /*host*/, const float* raw, const float* action,
+                          const float* on_log_probs /*(M,nu)*/, const float* advantages, const float* value_targets,
+                          const float* on_values, const float* values, float* d_raw /*(M, 2 nu)*/, float* d_value /*(M)*/);
+
 /* ------------------------------------------------------------------ rewards over a rollout
  * Replaces get_rewards + the stateless Reward.get_reward terms the configs name
  * (ksim/task/rl.py:189-245; ksim/rewards.py:166-188 StayAlive, 374-401 BaseHeight / BaseHeightRange,

@@ -519,6 +519,65 @@ __global__ __launch_bounds__(256) void ppo_loss_grad_kernel(int64_t M, int nu, K
   }
 }
 
+// The same objective for a network that emits its own deviations: raw (M, 2 nu) = means | raw deviations,
+// std = min((softplus(raw_std) + min_std) * var_scale, max_std).  One thread per row; d_raw receives the gradient of both halves.
+__global__ __launch_bounds__(256) void ppo_loss_grad_head_kernel(int64_t M, int nu, KsPpoLossParams p, KsGaussianHead hd,
+                                                                const float* __restrict__ raw, const float* __restrict__ action,
+                                                                const float* __restrict__ on_lp, const float* __restrict__ adv,
+                                                                const float* __restrict__ tgt, const float* __restrict__ on_v,
+                                                                const float* __restrict__ v, float* __restrict__ d_raw,
+                                                                float* __restrict__ d_value) {
+  const int64_t m = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (m >= M) return;
+  const float inv_m = 1.0f / (float)M;
+  const float* rm = raw + m * 2 * nu;
+  float logr = 0.f;
+  for (int a = 0; a < nu; ++a) {
+    const float mean = rm[a] + (hd.mean_bias ? hd.mean_bias[a] : 0.f);
+    const float r = rm[nu + a];
+    const float sp = r > 20.f ? r : log1pf(expf(r));
+    const float sd = fminf((sp + hd.min_std) * hd.var_scale, hd.max_std);
+    const float z = (action[m * nu + a] - mean) / sd;
+    logr += (-0.5f * z * z - logf(sd) - kHalfLog2Pi) - on_lp[m * nu + a];
+  }
+  const bool log_inside = logr > -p.log_clip_value && logr < p.log_clip_value;
+  const float ratio = __expf(fminf(fmaxf(logr, -p.log_clip_value), p.log_clip_value));
+  const float A = adv[m];
+  const float lo = 1.f - p.clip_param, hi = 1.f + p.clip_param;
+  const float s1 = ratio * A, s2 = fminf(fmaxf(ratio, lo), hi) * A;
+  const bool ratio_inside = ratio > lo && ratio < hi;
+  float g_logr = 0.f;
+  if (log_inside && (s1 < s2 || ratio_inside)) g_logr = -A * ratio;
+  const float g_lp = (g_logr - p.kl_coef * p.kl_scale) * inv_m;
+  const float g_ent = -p.entropy_coef * inv_m;
+  for (int a = 0; a < nu; ++a) {
+    const float mean = rm[a] + (hd.mean_bias ? hd.mean_bias[a] : 0.f);
+    const float r = rm[nu + a];
+    const float sp = r > 20.f ? r : log1pf(expf(r));
+    const float pre = (sp + hd.min_std) * hd.var_scale;
+    const bool capped = pre >= hd.max_std;
+    const float sd = capped ? hd.max_std : pre;
+    const float z = (action[m * nu + a] - mean) / sd;
+    d_raw[m * 2 * nu + a] = g_lp * z / sd;
+    // d/d log(std) of the log-density is z^2 - 1 and of the entropy 1; then through the cap, the scale and the softplus
+    const float d_ls = g_lp * (z * z - 1.f) + g_ent;
+    const float sig = r > 20.f ? 1.f : 1.f / (1.f + expf(-r));
+    d_raw[m * 2 * nu + nu + a] = capped ? 0.f : d_ls / sd * hd.var_scale * sig;
+  }
+  const float vv = v[m], vo = on_v[m], t = tgt[m];
+  float gv;
+  if (p.use_clipped_value_loss) {
+    const float dvv = vv - vo;
+    const float vc = vo + fminf(fmaxf(dvv, -p.clip_param), p.clip_param);
+    const float e = vv - t, ec = vc - t;
+    if (e * e >= ec * ec) gv = e;
+    else gv = (dvv > -p.clip_param && dvv < p.clip_param) ? ec : 0.f;
+  } else {
+    gv = vv - t;
+  }
+  d_value[m] = p.value_loss_coef * gv * inv_m;
+}
+
 __global__ void ppo_grad_finish_kernel(int nblocks, int nu, const float* __restrict__ partial, float* __restrict__ d_log_std) {
   const int a = threadIdx.x;
   if (a >= nu) return;
@@ -556,4 +615,21 @@ extern "C" int ks_ppo_loss_grad(ks_stream_t stream, int64_t M, int32_t nu, const
   hipLaunchKernelGGL(ks::ppo_grad_finish_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, blocks, nu, (const float*)workspace,
                      d_log_std);
   return ks::check_launch("ks_ppo_loss_grad");
+}
+
+extern "C" int ks_ppo_loss_grad_head(ks_stream_t stream, int64_t M, int32_t nu, const KsPpoLossParams* params,
+                                     const KsGaussianHead* head, const float* raw, const float* action, const float* on_log_probs,
+                                     const float* advantages, const float* value_targets, const float* on_values,
+                                     const float* values, float* d_raw, float* d_value) {
+  if (!params || !head) return ks::fail(KS_EINVAL, "ks_ppo_loss_grad_head: null parameters");
+  if (M < 1 || nu < 1) return ks::fail(KS_EINVAL, "ks_ppo_loss_grad_head: bad shape");
+  if (!raw || !action || !on_log_probs || !advantages || !value_targets || !on_values || !values || !d_raw || !d_value)
+    return ks::fail(KS_EINVAL, "ks_ppo_loss_grad_head: null pointer");
+  if (!(head->max_std > 0.f) || head->min_std < 0.f || !(head->var_scale > 0.f))
+    return ks::fail(KS_EINVAL, "ks_ppo_loss_grad_head: bad deviation bounds");
+  const int64_t grid = (M + 255) / 256;
+  if (grid > 0x7fffffff) return ks::fail(KS_ELIMIT, "ks_ppo_loss_grad_head: too many rows");
+  hipLaunchKernelGGL(ks::ppo_loss_grad_head_kernel, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, M, nu, *params, *head, raw,
+                     action, on_log_probs, advantages, value_targets, on_values, values, d_raw, d_value);
+  return ks::check_launch("ks_ppo_loss_grad_head");
 }

@@ -157,3 +157,57 @@ def update_model(policy: GaussianMlpPolicy, cfg: PPOUpdateConfig, actor_obs, cri
             out.append(single_step(policy, cfg, sel(actor_obs), sel(critic_obs), sel(action), sel(rewards), sel(done),
                                    sel(success), sel(on_lp), sel(on_v)))
     return out
+
+
+# --------------------------------------------------------------------------- recurrent actor / critic (GRU or LSTM stacks)
+@dataclass
+class RecurrentHeadPolicy:
+    """Recurrent actor whose output is (means | raw deviations) per action (examples/kbot/train.py:903-932) and a
+    recurrent critic; `min_std`, `max_std`, `var_scale`, `mean_bias` describe the deviation head."""
+    actor: "object"
+    critic: "object"
+    min_std: float
+    max_std: float
+    var_scale: float = 1.0
+    mean_bias: torch.Tensor | None = None
+    opt_step: int = 0
+
+    def train_init(self) -> None:
+        self.actor.train_init()
+        self.critic.train_init()
+
+
+def single_step_recurrent(policy: RecurrentHeadPolicy, cfg: PPOUpdateConfig, actor_obs, critic_obs, action, rewards, done, success,
+                          on_log_probs, on_values, actor_carry0, critic_carry0, fresh) -> dict:
+    """One minibatch step (ppo.py:495-565) for recurrent networks: both networks run over the (T, b) trajectory slice
+    from the carries the rollout started with, envs flagged in `fresh` (T, b) restart their carry, and the gradient goes
+    back through time.  GAE is recomputed from the current values and enters as a constant."""
+    lib = _lib.load()
+    Tn, b = done.shape
+    rows = Tn * b
+    nu = action.shape[-1]
+    raw = policy.actor.train_forward(actor_obs, actor_carry0, fresh)        # (T, b, 2 nu)
+    value = policy.critic.train_forward(critic_obs, critic_carry0, fresh)   # (T, b, 1)
+    inputs = ppo_mod.compute_ppo_inputs(value.view(Tn, b), rewards, done, success, cfg.gamma, cfg.lam,
+                                        normalize_advantages=cfg.normalize_advantages,
+                                        monte_carlo_returns=cfg.monte_carlo_returns, time_major=True)
+    p = _lib.KsPpoLossParams(cfg.clip_param, cfg.value_loss_coef, cfg.entropy_coef, cfg.kl_coef, cfg.log_clip_value, 1.0,
+                             int(cfg.use_clipped_value_loss))
+    head = T.KsGaussianHead(float(policy.min_std), float(policy.max_std), float(policy.var_scale), 0, _lib.ptr(policy.mean_bias).value)
+    d_raw = torch.empty(Tn, b, 2 * nu, dtype=torch.float32, device=raw.device)
+    d_value = torch.empty(Tn, b, 1, dtype=torch.float32, device=raw.device)
+    _lib.check(lib.ks_ppo_loss_grad_head(_lib.current_stream(), rows, nu, ctypes.byref(p), ctypes.byref(head), _lib.ptr(raw),
+                                         _lib.ptr(action.contiguous()), _lib.ptr(on_log_probs.contiguous()),
+                                         _lib.ptr(inputs.advantages_bt), _lib.ptr(inputs.value_targets_bt),
+                                         _lib.ptr(on_values.contiguous()), _lib.ptr(value), _lib.ptr(d_raw), _lib.ptr(d_value)))
+    policy.actor.backward(d_raw)
+    policy.critic.backward(d_value)
+    sq = torch.zeros(1, dtype=torch.float64, device=raw.device)
+    policy.actor.grad_sqnorm(sq)
+    policy.critic.grad_sqnorm(sq)
+    policy.opt_step += 1
+    ap = _adam(cfg, policy.opt_step)
+    policy.actor.adam_step(ap, sq)
+    policy.critic.adam_step(ap, sq)
+    return {"grad_norm": sq.sqrt(), "d_raw": d_raw, "d_value": d_value, "raw": raw, "values": value,
+            "advantages": inputs.advantages_bt}

@@ -37,6 +37,15 @@ def gaussian(mean, log_std, action):
     return lp, ent
 
 
+def gaussian_head(raw, action, min_std, max_std, var_scale, mean_bias=None):
+    """Log-density and entropy per action for the mean | raw deviation head (examples/kbot/train.py:915-932):
+    std = min((softplus(raw_std) + min_std) * var_scale, max_std)."""
+    nu = raw.shape[-1] // 2
+    mean = raw[..., :nu] + (0.0 if mean_bias is None else mean_bias)
+    std = torch.clamp((F.softplus(raw[..., nu:]) + min_std) * var_scale, max=max_std)
+    return gaussian(mean, torch.log(std), action)
+
+
 def ppo_loss_torch(adv, tgt, on_lp, on_v, lp, v, ent, cfg, kl_scale=1.0):
     """ppo.py:207-246 per element and 485-486 total, in torch so that autograd can differentiate it."""
     log_ratio = (lp - on_lp).sum(-1)
@@ -136,3 +145,27 @@ def update_model(params, rollout, cfg, permutations, act="elu"):
             params = unflat(new_p, params)
             losses.append(loss)
     return params, losses
+
+
+def recurrent_loss_and_grads(actor, critic, batch, cfg, head, act="none"):
+    """The minibatch loss of PPOTask for a recurrent actor with the mean | raw deviation head and a recurrent critic
+    (ppo.py:412-492 with the scan over time), and its gradients by float64 reverse-mode differentiation.
+    actor / critic: dict(input_proj, cells, out_w, out_b, carry0); batch: (T, b, ...) arrays with `fresh`; head:
+    dict(min_std, max_std, var_scale, mean_bias).  Returns (loss, actor gradients, critic gradients, aux)."""
+    from . import recurrent as orec
+
+    pa = orec.torch_parameters(actor["input_proj"], actor["cells"], actor["out_w"], actor["out_b"])
+    pc = orec.torch_parameters(critic["input_proj"], critic["cells"], critic["out_w"], critic["out_b"])
+    raw = orec.torch_sequence(batch["actor_obs"], actor["carry0"], batch["fresh"], *pa, act=act)
+    v = orec.torch_sequence(batch["critic_obs"], critic["carry0"], batch["fresh"], *pc, act=act)[..., 0]
+    # GAE from the current values, as a constant (ppo.py:450-459); the oracle works on (B, T)
+    gae = oppo.compute_ppo_inputs(v.detach().numpy().T, batch["rewards"].T, batch["done"].T, batch["success"].T, cfg["gamma"],
+                                  cfg["lam"], normalize_advantages=cfg["normalize_advantages"],
+                                  monte_carlo_returns=cfg["monte_carlo_returns"])
+    adv, tgt = torch.tensor(gae["advantages"].T.copy()), torch.tensor(gae["value_targets"].T.copy())
+    bias = None if head.get("mean_bias") is None else torch.tensor(np.asarray(head["mean_bias"], dtype=np.float64))
+    lp, ent = gaussian_head(raw, torch.tensor(np.asarray(batch["action"], dtype=np.float64)), head["min_std"], head["max_std"],
+                            head["var_scale"], bias)
+    loss, _ = ppo_loss_torch(adv, tgt, torch.tensor(batch["on_log_probs"]), torch.tensor(batch["on_values"]), lp, v, ent, cfg)
+    loss.backward()
+    return float(loss.detach()), orec.parameter_gradients(pa), orec.parameter_gradients(pc), {"raw": raw.detach().numpy(), "values": v.detach().numpy()}

@@ -84,21 +84,11 @@ def recurrent_sequence(obs, carry0, fresh, input_proj, cells, out_weights, out_b
     return np.stack(outs)
 
 
-def recurrent_sequence_gradients(obs, carry0, fresh, input_proj, cells, out_weights, out_biases, d_out, act="elu"):
-    """Gradients of sum(d_out * recurrent_sequence(...)) with respect to every parameter: the backward pass through time
-    that jax.grad performs through the scan over the trajectory (ksim/task/ppo.py:572-694).  The same equations as
-    `recurrent_sequence`, written with torch float64 tensors so that the library's reverse-mode differentiation yields the
-    gradients; tests pin the forward value to `recurrent_sequence` and single entries to central differences of it.
-    GRU cells are (weight_ih, weight_hh, bias, bias_n) with carry (depth, N, H); LSTM cells (weight_ih, weight_hh, bias)
-    with carry (depth, 2, N, H).
-    Returns (outputs, dict(input_proj=(dW, db), cells=[one gradient per cell parameter], out=[(dW, db)]))."""
+def torch_sequence(obs, carry0, fresh, wp, bp, cs, ow, ob, act="elu"):
+    """`recurrent_sequence` on torch float64 tensors (parameters may require gradients): returns the (T, N, out) tensor."""
     import torch
 
-    f = {"elu": torch.nn.functional.elu, "tanh": torch.tanh, "relu": torch.relu}[act]
-    t64 = lambda a: torch.tensor(np.asarray(a, dtype=np.float64), requires_grad=True)  # noqa: E731
-    wp, bp = t64(input_proj[0]), t64(input_proj[1])
-    cs = [tuple(t64(p) for p in c) for c in cells]
-    ow, ob = [t64(w) for w in out_weights], [t64(b) for b in out_biases]
+    f = {"elu": torch.nn.functional.elu, "tanh": torch.tanh, "relu": torch.relu, "none": lambda t: t}[act]
     obs_t = torch.tensor(np.asarray(obs, dtype=np.float64))
     carry = torch.tensor(np.asarray(carry0, dtype=np.float64))
     lstm = carry.ndim == 4
@@ -127,13 +117,39 @@ def recurrent_sequence_gradients(obs, carry0, fresh, input_proj, cells, out_weig
                 new.append(x)
         carry = torch.stack(new)
         y = x
-        for i, (w, b) in enumerate(zip(ow, ob)):
+        for k, (w, b) in enumerate(zip(ow, ob)):
             y = y @ w.T + b
-            if i + 1 < len(ow):
+            if k + 1 < len(ow):
                 y = f(y)
         outs.append(y)
-    out = torch.stack(outs)
-    (out * torch.tensor(np.asarray(d_out, dtype=np.float64))).sum().backward()
+    return torch.stack(outs)
+
+
+def torch_parameters(input_proj, cells, out_weights, out_biases):
+    import torch
+
+    t64 = lambda a: torch.tensor(np.asarray(a, dtype=np.float64), requires_grad=True)  # noqa: E731
+    return (t64(input_proj[0]), t64(input_proj[1]), [tuple(t64(p) for p in c) for c in cells],
+            [t64(w) for w in out_weights], [t64(b) for b in out_biases])
+
+
+def parameter_gradients(params):
+    wp, bp, cs, ow, ob = params
     g = lambda p: p.grad.numpy()  # noqa: E731
-    return out.detach().numpy(), dict(input_proj=(g(wp), g(bp)), cells=[tuple(g(p) for p in c) for c in cs],
-                                      out=[(g(w), g(b)) for w, b in zip(ow, ob)])
+    return dict(input_proj=(g(wp), g(bp)), cells=[tuple(g(p) for p in c) for c in cs], out=[(g(w), g(b)) for w, b in zip(ow, ob)])
+
+
+def recurrent_sequence_gradients(obs, carry0, fresh, input_proj, cells, out_weights, out_biases, d_out, act="elu"):
+    """Gradients of sum(d_out * recurrent_sequence(...)) with respect to every parameter: the backward pass through time
+    that jax.grad performs through the scan over the trajectory (ksim/task/ppo.py:572-694).  The same equations as
+    `recurrent_sequence`, written with torch float64 tensors so that the library's reverse-mode differentiation yields the
+    gradients; tests pin the forward value to `recurrent_sequence` and single entries to central differences of it.
+    GRU cells are (weight_ih, weight_hh, bias, bias_n) with carry (depth, N, H); LSTM cells (weight_ih, weight_hh, bias)
+    with carry (depth, 2, N, H).
+    Returns (outputs, dict(input_proj=(dW, db), cells=[one gradient per cell parameter], out=[(dW, db)]))."""
+    import torch
+
+    params = torch_parameters(input_proj, cells, out_weights, out_biases)
+    out = torch_sequence(obs, carry0, fresh, *params, act=act)
+    (out * torch.tensor(np.asarray(d_out, dtype=np.float64))).sum().backward()
+    return out.detach().numpy(), parameter_gradients(params)

@@ -87,6 +87,43 @@ def test_ppo_loss_gradient_kernel_matches_autograd():
     np.testing.assert_allclose(ent_k.cpu().numpy(), ent.detach().numpy(), rtol=1e-6, atol=1e-6)
 
 
+def test_ppo_loss_gradient_for_the_deviation_head_matches_autograd():
+    """d loss / d (mean | raw deviation) for a network that emits its own deviations, against float64 autograd of the
+    oracle loss; rows with a capped deviation get no deviation gradient."""
+    from ksim_amd import _lib, _lib_terms as T
+
+    lib = _lib.load()
+    rng = np.random.default_rng(13)
+    M, A = 4000, 20
+    raw = rng.normal(size=(M, 2 * A))
+    raw[:50, A:] = 6.0  # (softplus + 0.01) * 0.5 above the cap of 1.5
+    bias = rng.normal(size=A) * 0.1
+    hd = dict(min_std=0.01, max_std=1.5, var_scale=0.5)
+    tr = torch.tensor(raw, requires_grad=True)
+    with torch.no_grad():
+        sd = torch.clamp((torch.nn.functional.softplus(tr[:, A:]) + 0.01) * 0.5, max=1.5).numpy()
+    act = raw[:, :A] + bias + sd * rng.normal(size=(M, A))
+    on_lp = ou.gaussian_head(torch.tensor(raw + rng.normal(size=raw.shape) * 0.02), torch.tensor(act), mean_bias=torch.tensor(bias), **hd)[0].numpy()
+    adv, tgt, on_v = rng.normal(size=M), rng.normal(size=M), rng.normal(size=M)
+    v = on_v + rng.normal(size=M) * 0.3
+    tv = torch.tensor(v, requires_grad=True)
+    lp, ent = ou.gaussian_head(tr, torch.tensor(act), mean_bias=torch.tensor(bias), **hd)
+    loss, _ = ou.ppo_loss_torch(torch.tensor(adv), torch.tensor(tgt), torch.tensor(on_lp), torch.tensor(on_v), lp, tv, ent, CFG, 1.3)
+    loss.backward()
+    p = _lib.KsPpoLossParams(0.2, 0.5, 0.008, 1e-3, 5.0, 1.3, 1)
+    bias_d = t32(bias)
+    head = T.KsGaussianHead(0.01, 1.5, 0.5, 0, _lib.ptr(bias_d).value)
+    d_raw, d_value = torch.empty(M, 2 * A, device=DEV), torch.empty(M, device=DEV)
+    args = [t32(a) for a in (raw, act, on_lp, adv, tgt, on_v, v)]
+    _lib.check(lib.ks_ppo_loss_grad_head(_lib.current_stream(), M, A, ctypes.byref(p), ctypes.byref(head), *[_lib.ptr(a) for a in args],
+                                         _lib.ptr(d_raw), _lib.ptr(d_value)))
+    g = tr.grad.numpy()
+    assert rel(d_raw[:, :A].cpu().numpy(), g[:, :A]) < 1e-4
+    assert rel(d_raw[:, A:].cpu().numpy(), g[:, A:]) < 1e-4
+    assert rel(d_value.cpu().numpy(), tv.grad.numpy()) < 1e-5
+    assert (d_raw[:50, A:] == 0).all() and (g[:50, A:] == 0).all()
+
+
 def test_adam_chain_kernel_matches_optax_restatement():
     from ksim_amd import _lib, _lib_terms as T
 
@@ -182,3 +219,65 @@ def test_update_model_tracks_oracle():
     assert np.median(np.concatenate(errs)) < 2e-6, "typical parameter error after the update"
     moved = np.abs(pol.actor.parameters()[0][0].cpu().numpy() - params["actor_w"][0]).max()
     assert moved > 0.5 * cfg.learning_rate, "the update did not move the parameters"
+
+
+def test_recurrent_single_step_gradients_match_oracle():
+    """One minibatch step of a K-Bot-shaped policy (LSTM actor emitting means | raw deviations, LSTM critic; projection,
+    two LSTM layers, linear output) over a (T, b) slice with episode starts: gradients of every parameter against float64
+    reverse-mode differentiation of the whole loss (scan over time, head, GAE as a constant, PPO objective)."""
+    from ksim_amd import ppo_update as pu
+    from ksim_amd.mlp import MLP
+    from ksim_amd.recurrent import LSTMCell, RecurrentNetwork
+
+    rng = np.random.default_rng(51)
+    Tn, b, I, H, nu = 8, 64, 23, 64, 6
+
+    def make(out_dim):
+        proj = (rng.normal(size=(H, I)) / np.sqrt(I), rng.normal(size=H) * 0.1)
+        cells = [(rng.normal(size=(4 * H, H)) / np.sqrt(H), rng.normal(size=(4 * H, H)) / np.sqrt(H), rng.normal(size=4 * H) * 0.1)
+                 for _ in range(2)]
+        ow, ob = [rng.normal(size=(out_dim, H)) / np.sqrt(H)], [rng.normal(size=out_dim) * 0.1]
+        carry0 = rng.normal(size=(2, 2, b, H)) * 0.3
+        net = RecurrentNetwork(proj, [LSTMCell(*c, dtype="f32") for c in cells], MLP(ow, ob, activation="none", dtype="f32"), dtype="f32")
+        return dict(input_proj=proj, cells=cells, out_w=ow, out_b=ob, carry0=carry0), net
+
+    oa, actor = make(2 * nu)
+    oc, critic = make(1)
+    head = dict(min_std=0.01, max_std=1.0, var_scale=0.5, mean_bias=rng.normal(size=nu) * 0.1)
+    obs = rng.normal(size=(Tn, b, I))
+    fresh = rng.random((Tn, b)) < 0.08
+    done = np.roll(fresh, -1, axis=0); done[-1] = False   # an env restarts at the step after it finished
+    batch = dict(actor_obs=obs + rng.normal(size=obs.shape) * 0.01, critic_obs=obs, fresh=fresh, done=done,
+                 success=np.zeros((Tn, b), bool), rewards=rng.normal(size=(Tn, b)))
+    # the old policy: the same networks a little perturbed, so that ratios differ from one on both sides of the clip
+    _, _, _, aux0 = ou.recurrent_loss_and_grads(oa, oc, dict(batch, action=np.zeros((Tn, b, nu)), on_log_probs=np.zeros((Tn, b, nu)),
+                                                             on_values=np.zeros((Tn, b))), CFG, head)
+    raw0 = aux0["raw"] + rng.normal(size=aux0["raw"].shape) * 0.05
+    sd0 = np.minimum((np.logaddexp(0, raw0[..., nu:]) + 0.01) * 0.5, 1.0)
+    batch["action"] = raw0[..., :nu] + head["mean_bias"] + sd0 * rng.normal(size=sd0.shape)
+    batch["on_log_probs"] = ou.gaussian_head(torch.tensor(raw0), torch.tensor(batch["action"]), 0.01, 1.0, 0.5,
+                                             torch.tensor(head["mean_bias"]))[0].numpy()
+    batch["on_values"] = aux0["values"] + rng.normal(size=(Tn, b)) * 0.2
+    loss, ga, gc, aux = ou.recurrent_loss_and_grads(oa, oc, batch, CFG, head)
+
+    policy = pu.RecurrentHeadPolicy(actor, critic, 0.01, 1.0, 0.5, t32(head["mean_bias"]))
+    policy.train_init()
+    cfg = pu.PPOUpdateConfig(**{k: v for k, v in CFG.items() if k not in ("batch_size", "num_passes")}, batch_size=b)
+    u8 = lambda a: torch.tensor(a, dtype=torch.uint8, device=DEV)  # noqa: E731
+    m = pu.single_step_recurrent(policy, cfg, t32(batch["actor_obs"]), t32(batch["critic_obs"]), t32(batch["action"]),
+                                 t32(batch["rewards"]), u8(done), u8(batch["success"]), t32(batch["on_log_probs"]),
+                                 t32(batch["on_values"]), t32(oa["carry0"]), t32(oc["carry0"]), u8(fresh))
+    assert rel(m["raw"].cpu().numpy(), aux["raw"]) < 1e-4 and rel(m["values"].cpu().numpy()[..., 0], aux["values"]) < 1e-4
+    # gradients were taken before the optimiser step moved the parameters
+    for net, want in ((actor, ga), (critic, gc)):
+        got = {"proj.W": net.input_proj.parameters(True)[0][0], "proj.b": net.input_proj.parameters(True)[0][1],
+               "out.W": net.output_proj.parameters(True)[0][0], "out.b": net.output_proj.parameters(True)[0][1]}
+        ref = {"proj.W": want["input_proj"][0], "proj.b": want["input_proj"][1], "out.W": want["out"][0][0], "out.b": want["out"][0][1]}
+        for i, c in enumerate(net.cells):
+            g = c.parameters(True)
+            for k, j in (("weight_ih", 0), ("weight_hh", 1), ("bias", 2)):
+                got[f"cell{i}.{k}"], ref[f"cell{i}.{k}"] = g[k], want["cells"][i][j]
+        for k in ref:
+            assert rel(got[k].cpu().numpy(), ref[k]) < 2e-3, k
+    total = sum(float((np.asarray(v) ** 2).sum()) for g in (ga, gc) for v in (g["input_proj"] + tuple(x for c in g["cells"] for x in c) + tuple(x for o in g["out"] for x in o)))
+    assert m["grad_norm"].item() == pytest.approx(np.sqrt(total), rel=2e-3)
