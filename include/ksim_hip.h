@@ -507,7 +507,7 @@ int ks_sample_action_mixture(ks_stream_t stream, int64_t N, int32_t nu, const fl
  */
 #define KS_MAX_LAYERS 8
 enum { KS_ACT_NONE = 0, KS_ACT_ELU = 1, KS_ACT_RELU = 2, KS_ACT_TANH = 3,
-       KS_ACT_GELU = 4 /* tanh form, jax.nn.gelu's default (examples/walking.py:103); forward only */ };
+       KS_ACT_GELU = 4 /* tanh form, jax.nn.gelu's default (examples/walking.py:103) */ };
 enum { KS_MLP_F32 = 0, KS_MLP_BF16 = 1 };
 typedef struct KsMlpDesc {
   int32_t n_layers;

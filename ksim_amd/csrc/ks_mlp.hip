@@ -566,6 +566,26 @@ __global__ __launch_bounds__(256) void transpose_kernel(int64_t M, int C, int64_
   }
 }
 
+// y = gelu(z), tanh form, over a whole (M, ld) buffer
+template <typename T>
+__global__ __launch_bounds__(256) void gelu_forward_kernel(int64_t n, const T* __restrict__ z, T* __restrict__ y) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= n) return;
+  const float x = to_f32(z[idx]);
+  y[idx] = from_f32<T>(0.5f * x * (1.f + tanhf(0.7978845608028654f * (x + 0.044715f * x * x * x))));
+}
+
+// dZ = dY * gelu'(Z) from the stored pre-activation, written over dY
+template <typename T>
+__global__ __launch_bounds__(256) void gelu_backward_kernel(int64_t n, const T* __restrict__ z, T* __restrict__ dy) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= n) return;
+  const float x = to_f32(z[idx]);
+  const float t = tanhf(0.7978845608028654f * (x + 0.044715f * x * x * x));
+  const float d = 0.5f * (1.f + t) + 0.5f * x * (1.f - t * t) * 0.7978845608028654f * (1.f + 3.f * 0.044715f * x * x);
+  dy[idx] = from_f32<T>(to_f32(dy[idx]) * d);
+}
+
 // dZ = dY * act'(Z), written over dY; act' is expressed through the stored activation output Y.
 template <typename T, int ACT>
 __global__ __launch_bounds__(256) void act_backward_kernel(int64_t n, const T* __restrict__ y, T* __restrict__ dy) {
@@ -1040,7 +1060,6 @@ static void refresh_layers(DevMlp& m, hipStream_t s);
 
 extern "C" int ks_mlp_train_init(KsMlp* h) {
   if (!h) return fail(KS_EINVAL, "ks_mlp_train_init: null handle");
-  if (h->m.activation == KS_ACT_GELU) return fail(KS_EINVAL, "ks_mlp_train_init: the backward pass keeps activations, not pre-activations, and GELU cannot be differentiated from its output");
   DevMlp& m = h->m;
   if (m.train) return KS_OK;
   const size_t esz = m.dtype == KS_MLP_BF16 ? 2 : 4;
@@ -1094,6 +1113,7 @@ constexpr int kDwSplit = 16;  // most slices the weight-gradient reduction over 
 // workspace: hidden activations of every layer, two (M, widest) gradient buffers, two transposes (widest, Mp)
 struct TrainWs {
   char* act[KS_MAX_LAYERS];
+  char* pre[KS_MAX_LAYERS];  // pre-activations of the hidden layers, kept only for GELU (not recoverable from its output)
   char *d0, *d1, *t0, *t1, *t2;
   float* part;  // partial sums of the split reductions
   int64_t Mp;
@@ -1111,6 +1131,8 @@ static int64_t carve_train(const DevMlp& m, int64_t M, char* base, TrainWs* ws) 
   TrainWs w;
   std::memset(&w, 0, sizeof(w));
   for (int l = 0; l + 1 < m.n_layers; ++l) w.act[l] = take(M * m.npad[l] * esz);
+  if (m.activation == KS_ACT_GELU)
+    for (int l = 0; l + 1 < m.n_layers; ++l) w.pre[l] = take(M * m.npad[l] * esz);
   w.d0 = take(M * wz * esz);
   w.d1 = take(M * wz * esz);
   w.t0 = take((int64_t)wz * Mp * esz);
@@ -1136,14 +1158,21 @@ static int train_forward(DevMlp& m, hipStream_t s, int64_t M, const float* x, fl
   int64_t ldin = m.dims[0];
   for (int l = 0; l < m.n_layers; ++l) {
     const bool first = l == 0, last = l == m.n_layers - 1;
-    void* outp = last ? (void*)y : (void*)ws.act[l];
+    const bool split_act = !last && m.activation == KS_ACT_GELU;  // keep the pre-activation, then apply GELU
+    void* outp = last ? (void*)y : (split_act ? (void*)ws.pre[l] : (void*)ws.act[l]);
     const int64_t ldo = last ? m.dims[l + 1] : m.npad[l];
+    const int act_l = split_act ? KS_ACT_NONE : m.activation;
     int rc;
-    if (first && last) rc = launch_layer<T, true, true>(m.activation, s, M, m.npad[l], m.kpad[l], m.dims[l], m.dims[l + 1], in, ldin, m.W[l], m.b[l], outp, ldo);
-    else if (first) rc = launch_layer<T, true, false>(m.activation, s, M, m.npad[l], m.kpad[l], m.dims[l], m.dims[l + 1], in, ldin, m.W[l], m.b[l], outp, ldo);
-    else if (last) rc = launch_layer<T, false, true>(m.activation, s, M, m.npad[l], m.kpad[l], m.dims[l], m.dims[l + 1], in, ldin, m.W[l], m.b[l], outp, ldo);
-    else rc = launch_layer<T, false, false>(m.activation, s, M, m.npad[l], m.kpad[l], m.dims[l], m.dims[l + 1], in, ldin, m.W[l], m.b[l], outp, ldo);
+    if (first && last) rc = launch_layer<T, true, true>(act_l, s, M, m.npad[l], m.kpad[l], m.dims[l], m.dims[l + 1], in, ldin, m.W[l], m.b[l], outp, ldo);
+    else if (first) rc = launch_layer<T, true, false>(act_l, s, M, m.npad[l], m.kpad[l], m.dims[l], m.dims[l + 1], in, ldin, m.W[l], m.b[l], outp, ldo);
+    else if (last) rc = launch_layer<T, false, true>(act_l, s, M, m.npad[l], m.kpad[l], m.dims[l], m.dims[l + 1], in, ldin, m.W[l], m.b[l], outp, ldo);
+    else rc = launch_layer<T, false, false>(act_l, s, M, m.npad[l], m.kpad[l], m.dims[l], m.dims[l + 1], in, ldin, m.W[l], m.b[l], outp, ldo);
     if (rc != KS_OK) return rc;
+    if (split_act) {
+      const int64_t n = M * m.npad[l];
+      hipLaunchKernelGGL(gelu_forward_kernel<T>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, n, (const T*)ws.pre[l], (T*)ws.act[l]);
+      outp = ws.act[l];
+    }
     in = outp;
     ldin = ldo;
   }
@@ -1202,7 +1231,7 @@ static int train_backward(DevMlp& m, hipStream_t s, int64_t M, const float* x, c
       // input gradient, then through the activation of the layer below
       rc = launch_layer<T, false, false>(KS_ACT_NONE, s, M, kp, np, np, kp, dz, np, m.Wt[l], m.zero_bias, dnext, kp);
       if (rc != KS_OK) return rc;
-      const bool fused = want_w && kp % 64 == 0 && kp == kp128 && kp == m.npad[l - 1];
+      const bool fused = want_w && m.activation != KS_ACT_GELU && kp % 64 == 0 && kp == kp128 && kp == m.npad[l - 1];
       if (fused) {
 #define KS_PREP(A) hipLaunchKernelGGL((bwd_prep_kernel<T, A>), dim3((unsigned)(kp / 64), kColsumSlices), dim3(256), 0, s, M, Mp, kp, \
                                       (const T*)ws.act[l - 1], dnext, dzT_next, (T*)ws.t1, ws.part)
@@ -1222,6 +1251,9 @@ static int train_backward(DevMlp& m, hipStream_t s, int64_t M, const float* x, c
           case KS_ACT_ELU: KS_ACTB(KS_ACT_ELU); break;
           case KS_ACT_RELU: KS_ACTB(KS_ACT_RELU); break;
           case KS_ACT_TANH: KS_ACTB(KS_ACT_TANH); break;
+          case KS_ACT_GELU:
+            hipLaunchKernelGGL(gelu_backward_kernel<T>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, n, (const T*)ws.pre[l - 1], dnext);
+            break;
           default: break;
         }
 #undef KS_ACTB

@@ -18,7 +18,8 @@ import torch.nn.functional as F
 
 from . import ppo as oppo
 
-_ACT = {"elu": F.elu, "relu": F.relu, "tanh": torch.tanh, "none": lambda t: t}
+_ACT = {"elu": F.elu, "relu": F.relu, "tanh": torch.tanh, "none": lambda t: t,
+        "gelu": lambda t: F.gelu(t, approximate="tanh")}  # jax.nn.gelu's default form
 
 
 def mlp(x, ws, bs, act="elu"):

@@ -88,7 +88,8 @@ def torch_sequence(obs, carry0, fresh, wp, bp, cs, ow, ob, act="elu"):
     """`recurrent_sequence` on torch float64 tensors (parameters may require gradients): returns the (T, N, out) tensor."""
     import torch
 
-    f = {"elu": torch.nn.functional.elu, "tanh": torch.tanh, "relu": torch.relu, "none": lambda t: t}[act]
+    f = {"elu": torch.nn.functional.elu, "tanh": torch.tanh, "relu": torch.relu, "none": lambda t: t,
+         "gelu": lambda t: torch.nn.functional.gelu(t, approximate="tanh")}[act]
     obs_t = torch.tensor(np.asarray(obs, dtype=np.float64))
     carry = torch.tensor(np.asarray(carry0, dtype=np.float64))
     lstm = carry.ndim == 4

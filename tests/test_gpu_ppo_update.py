@@ -28,6 +28,8 @@ def rel(got, want):
     ((71, 256, 256, 21), "f32", "elu", 300, 2e-4),     # fp32 path: accumulation-order error only
     ((68, 512, 512, 512, 20), "bf16", "elu", 1000, 3e-2),  # bf16 operands, fp32 accumulate
     ((33, 130, 2), "f32", "tanh", 77, 2e-4), ((40, 64, 64, 1), "f32", "relu", 129, 2e-4),
+    # GELU (the walking example's output networks): the pre-activations are kept for the derivative
+    ((64, 128, 128, 36), "f32", "gelu", 257, 2e-4), ((256, 256, 256, 256, 60), "bf16", "gelu", 1000, 3e-2),
 ])
 def test_mlp_backward_matches_autograd(dims, dtype, act, M, tol):
     from ksim_amd.mlp import MLP

@@ -95,9 +95,6 @@ def test_gelu_mlp_bf16():
         assert np.abs(got - h).max() < 6e-3 * max(1.0, np.abs(h).max())
         got32 = MLP(ws, bs, activation="gelu", dtype="f32")(t32(x)).cpu().numpy()
         np.testing.assert_allclose(got32, orec.mlp(x, ws, bs, orec.gelu), rtol=2e-5, atol=2e-5)
-    m = MLP(ws, bs, activation="gelu", dtype="f32")
-    with pytest.raises(Exception, match="GELU"):
-        m.train_init()
 
 
 @pytest.mark.parametrize("N,I,H", [(40, 12, 16), (4096, 128, 128)])
@@ -138,9 +135,9 @@ def test_lstm_cell_and_network(N, I, H):
         np.testing.assert_allclose(carry.cpu().numpy(), want_carry, rtol=2e-4, atol=2e-4)
 
 
-@pytest.mark.parametrize("dtype,tol", [("f32", 2e-4), ("bf16", 6e-2)])
-def test_backward_through_time_matches_the_oracle(dtype, tol):
-    """Gradients of a GRU actor over a trajectory (input projection, two GRU layers, ELU output network) with episode
+@pytest.mark.parametrize("dtype,tol,act", [("f32", 2e-4, "elu"), ("bf16", 6e-2, "elu"), ("f32", 2e-4, "gelu")])
+def test_backward_through_time_matches_the_oracle(dtype, tol, act):
+    """Gradients of a GRU actor over a trajectory (input projection, two GRU layers, ELU or GELU output network) with episode
     starts inside it, against torch float64 reverse-mode differentiation of the oracle network; then one optimiser step.
     Tolerances are relative to the largest entry of each gradient array: fp32 accumulation only for f32; for bf16 the
     activations and the gradients between layers are rounded to bf16 at every one of the T steps."""
@@ -162,9 +159,9 @@ def test_backward_through_time_matches_the_oracle(dtype, tol):
         rb = lambda a: torch.tensor(a, dtype=torch.float32).to(torch.bfloat16).to(torch.float64).numpy()  # noqa: E731
         proj = (rb(proj[0]), proj[1]); ow = [rb(w) for w in ow]
         cells = [(rb(c[0]), rb(c[1]), c[2], c[3]) for c in cells]
-    want_out, want = orec.recurrent_sequence_gradients(obs, carry0, fresh, proj, cells, ow, ob, d_out)
+    want_out, want = orec.recurrent_sequence_gradients(obs, carry0, fresh, proj, cells, ow, ob, d_out, act=act)
 
-    net = RecurrentNetwork(proj, [GRUCell(*c, dtype=dtype) for c in cells], MLP(ow, ob, activation="elu", dtype=dtype), dtype=dtype)
+    net = RecurrentNetwork(proj, [GRUCell(*c, dtype=dtype) for c in cells], MLP(ow, ob, activation=act, dtype=dtype), dtype=dtype)
     net.train_init()
     out = net.train_forward(t32(obs), t32(carry0), torch.tensor(fresh, dtype=torch.uint8, device=DEV))
     scale = np.abs(want_out).max()
