@@ -138,9 +138,11 @@ typedef struct KsModelDesc {
    * examples/kbot/robot/kbot-headless/robot.mjcf:66-217), and dry joint friction (dof_frictionloss, robot.mjcf:5-18).
    * A violated limit is one constraint row J = +-e_j, friction one row J = e_j whose force saturates at
    * +-frictionloss; both are regularised with dof_invweight0[j], the diagonal of the inverse mass matrix at qpos0,
-   * and use the model's solref / solimp.  All zero: neither. */
+   * and use dof_solref / dof_solimp (MuJoCo's per-joint solreflimit, solimplimit, solreffriction, solimpfriction, one
+   * pair for all of them here; all zero = the contacts' solref / solimp).  Everything zero: neither limits nor friction. */
   int32_t jnt_limited[KS_MAX_BODIES];
   double jnt_range[KS_MAX_BODIES][2], dof_invweight0[KS_MAX_DOFS], dof_frictionloss[KS_MAX_DOFS];
+  double dof_solref[2], dof_solimp[5];
 } KsModelDesc;
 
 typedef struct KsModel KsModel;

@@ -228,20 +228,28 @@ struct LsPoint {
   float alpha, cost, d0, d1;
 };
 
-// constraint impedance d(|pos|) of the model's solimp
-__device__ __forceinline__ float impedance(const DevModel& m, float pos) {
-  const float ix = fabsf(pos) / m.width;
+// constraint impedance d(|pos|) of a solimp whose parameters are already clamped
+__device__ __forceinline__ float impedance_of(float pos, float dmin, float dmax, float width, float mid, float power, float imp_a,
+                                              float imp_b) {
+  const float ix = fabsf(pos) / width;
   // x^power: the default power of 2 (and 1) without the general power function
   const float ox = 1.f - ix;
-  const float px = m.power == 2.f ? ix * ix : (m.power == 1.f ? ix : powf(ix, m.power));
-  const float po = m.power == 2.f ? ox * ox : (m.power == 1.f ? ox : powf(ox, m.power));
-  const float ia = m.imp_a * px;
-  const float ib = 1.f - m.imp_b * po;
-  const float iy = ix < m.mid ? ia : ib;
-  float imp = m.dmin + iy * (m.dmax - m.dmin);
-  imp = fminf(fmaxf(imp, m.dmin), m.dmax);
-  if (ix > 1.f) imp = m.dmax;
+  const float px = power == 2.f ? ix * ix : (power == 1.f ? ix : powf(ix, power));
+  const float po = power == 2.f ? ox * ox : (power == 1.f ? ox : powf(ox, power));
+  const float ia = imp_a * px;
+  const float ib = 1.f - imp_b * po;
+  const float iy = ix < mid ? ia : ib;
+  float imp = dmin + iy * (dmax - dmin);
+  imp = fminf(fmaxf(imp, dmin), dmax);
+  if (ix > 1.f) imp = dmax;
   return imp;
+}
+// of the contact rows, and of the rows of joint limits and dry friction
+__device__ __forceinline__ float impedance(const DevModel& m, float pos) {
+  return impedance_of(pos, m.dmin, m.dmax, m.width, m.mid, m.power, m.imp_a, m.imp_b);
+}
+__device__ __forceinline__ float impedance_dof(const DevModel& m, float pos) {
+  return impedance_of(pos, m.dr_dmin, m.dr_dmax, m.dr_width, m.dr_mid, m.dr_power, m.dr_imp_a, m.dr_imp_b);
 }
 
 // The rows a dof lane carries itself: the violated limit of its hinge (J = lim_s e_j, lim_s = +-1, 0 when none) and its
@@ -781,14 +789,14 @@ void step_kernel(StepArgs a) {
           const float pos = fminf(dlo, dhi);
           if (pos < 0.f) {  // the nearer side, once violated
             dr.lim_s = dlo < dhi ? 1.f : -1.f;
-            const float imp = impedance(m, pos);
+            const float imp = impedance_dof(m, pos);
             dr.lim_D = 1.f / fmaxf(rr->d_invw * (1.f - imp) / imp, 1e-15f);
-            dr.lim_aref = -m.con_b * dr.lim_s * my_qvel - m.con_k * imp * pos;
+            dr.lim_aref = -m.dr_b * dr.lim_s * my_qvel - m.dr_k * imp * pos;
           }
         }
         dr.fr_fl = rr->d_floss;
         dr.fr_D = rr->d_frD;
-        dr.fr_aref = -m.con_b * my_qvel;
+        dr.fr_aref = -m.dr_b * my_qvel;
       }
       ndr = __popcll(__ballot(dr.lim_s != 0.f)) + m.nfriction;
     }
@@ -1189,19 +1197,30 @@ extern "C" int ks_model_create(const KsModelDesc* d, KsModel** out) {
   for (int k = 0; k < 3; ++k) m.gravity[k] = (float)d->gravity[k];
   m.tolerance = (float)d->tolerance; m.ls_tolerance = (float)d->ls_tolerance;
   m.meaninertia = (float)d->meaninertia; m.friction = (float)d->friction; m.impratio = (float)d->impratio;
-  {  // solref / solimp -> (k, b) and clamped impedance parameters
-    double timeconst = d->solref[0], dampratio = d->solref[1];
-    double dmin = d->solimp[0], dmax = d->solimp[1], width = d->solimp[2], mid = d->solimp[3], power = d->solimp[4];
-    if (timeconst < 2 * d->dt) timeconst = 2 * d->dt;
-    auto clampd = [](double x, double lo, double hi) { return x < lo ? lo : (x > hi ? hi : x); };
-    dmin = clampd(dmin, 1e-4, 0.9999); dmax = clampd(dmax, 1e-4, 0.9999);
-    width = width < 1e-15 ? 1e-15 : width; mid = clampd(mid, 1e-4, 0.9999); power = power < 1 ? 1 : power;
-    double k = 1.0 / (dmax * dmax * timeconst * timeconst * dampratio * dampratio), b = 2.0 / (dmax * timeconst);
-    if (d->solref[0] <= 0) k = -d->solref[0] / (dmax * dmax);
-    if (d->solref[1] <= 0) b = -d->solref[1] / dmax;
-    m.con_k = (float)k; m.con_b = (float)b; m.dmin = (float)dmin; m.dmax = (float)dmax; m.width = (float)width;
-    m.mid = (float)mid; m.power = (float)power;
-    m.imp_a = (float)(1.0 / std::pow(mid, power - 1.0)); m.imp_b = (float)(1.0 / std::pow(1.0 - mid, power - 1.0));
+  {  // solref / solimp -> (k, b) and clamped impedance parameters, for the contact rows and for the dof-lane rows
+    auto convert = [&](const double* solref, const double* solimp, float* out /*k b dmin dmax width mid power imp_a imp_b*/) {
+      double timeconst = solref[0], dampratio = solref[1];
+      double dmin = solimp[0], dmax = solimp[1], width = solimp[2], mid = solimp[3], power = solimp[4];
+      if (timeconst < 2 * d->dt) timeconst = 2 * d->dt;
+      auto clampd = [](double x, double lo, double hi) { return x < lo ? lo : (x > hi ? hi : x); };
+      dmin = clampd(dmin, 1e-4, 0.9999); dmax = clampd(dmax, 1e-4, 0.9999);
+      width = width < 1e-15 ? 1e-15 : width; mid = clampd(mid, 1e-4, 0.9999); power = power < 1 ? 1 : power;
+      double k = 1.0 / (dmax * dmax * timeconst * timeconst * dampratio * dampratio), b = 2.0 / (dmax * timeconst);
+      if (solref[0] <= 0) k = -solref[0] / (dmax * dmax);
+      if (solref[1] <= 0) b = -solref[1] / dmax;
+      out[0] = (float)k; out[1] = (float)b; out[2] = (float)dmin; out[3] = (float)dmax; out[4] = (float)width;
+      out[5] = (float)mid; out[6] = (float)power;
+      out[7] = (float)(1.0 / std::pow(mid, power - 1.0)); out[8] = (float)(1.0 / std::pow(1.0 - mid, power - 1.0));
+    };
+    float c[9];
+    convert(d->solref, d->solimp, c);
+    m.con_k = c[0]; m.con_b = c[1]; m.dmin = c[2]; m.dmax = c[3]; m.width = c[4]; m.mid = c[5]; m.power = c[6]; m.imp_a = c[7]; m.imp_b = c[8];
+    bool own = false;
+    for (int k = 0; k < 2; ++k) own |= d->dof_solref[k] != 0.0;
+    for (int k = 0; k < 5; ++k) own |= d->dof_solimp[k] != 0.0;
+    if (own) convert(d->dof_solref, d->dof_solimp, c);
+    m.dr_k = c[0]; m.dr_b = c[1]; m.dr_dmin = c[2]; m.dr_dmax = c[3]; m.dr_width = c[4]; m.dr_mid = c[5]; m.dr_power = c[6];
+    m.dr_imp_a = c[7]; m.dr_imp_b = c[8];
   }
   for (int b = 0; b < d->nb; ++b) {
     m.body_parent[b] = d->body_parent[b]; m.body_jtype[b] = d->body_jtype[b]; m.body_qadr[b] = d->body_qadr[b];
@@ -1302,7 +1321,7 @@ extern "C" int ks_model_create(const KsModelDesc* d, KsModel** out) {
       r.d_rlo = (float)d->jnt_range[r.d_body][0]; r.d_rhi = (float)d->jnt_range[r.d_body][1];
       r.d_invw = (float)d->dof_invweight0[dl];
       r.d_floss = (float)d->dof_frictionloss[dl];
-      const double imp0 = m.dmin;  // impedance at pos = 0
+      const double imp0 = m.dr_dmin;  // impedance at pos = 0
       r.d_frD = (float)(1.0 / std::max(d->dof_invweight0[dl] * (1.0 - imp0) / imp0, 1e-15));
     }
     const int sl = L < d->ns ? L : 0;

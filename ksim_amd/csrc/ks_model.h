@@ -26,6 +26,8 @@ struct DevModel {
   // contact impedance constants, already clamped the way the constraint builder wants them
   float con_k, con_b, dmin, dmax, width, mid, power;
   float imp_a, imp_b;  // 1 / mid^(power-1) and 1 / (1-mid)^(power-1), the constant factors of the impedance curve
+  // the same constants for the rows of joint limits and dry friction
+  float dr_k, dr_b, dr_dmin, dr_dmax, dr_width, dr_mid, dr_power, dr_imp_a, dr_imp_b;
   int body_parent[kMaxB], body_jtype[kMaxB], body_qadr[kMaxB], body_dofadr[kMaxB], body_subtree_end[kMaxB],
       body_depth[kMaxB];
   int body_chain[kMaxB][kMaxDepth];  // ancestors from the tree root down to the body itself

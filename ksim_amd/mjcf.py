@@ -1,0 +1,319 @@
+"""MJCF -> KinematicModel for the model subset the step kernel runs.
+
+The reference compiles its robot files with MuJoCo (`mujoco.MjModel.from_xml_path`, ksim/task/rl.py:717-748,
+ksim/utils/mujoco.py:388-391) and hands the result to MJX.  This loader reads the same files for robots of the K-Bot's
+kind (examples/kbot/robot/kbot-headless/robot.mjcf): a floating base, hinge joints (one per body), explicit `<inertial>`
+elements, `<motor>` actuators, and sphere or capsule collision geoms against the ground plane.  What MuJoCo's compiler does
+for such a file is restated here:
+
+* `<default>` classes nest and inherit; `childclass` on a body applies to everything below it;
+* a body without a joint is welded to its parent: its inertia, geoms and children move into the parent's frame, and the
+  parent's inertial becomes the composite (mass, centre of mass, inertia tensor by the parallel-axis theorem, principal
+  axes by an eigendecomposition);
+* a body without `<inertial>` takes its inertia from its sphere / capsule geoms at the default density of 1000;
+* a capsule touches the plane with its two end spheres, so each collision capsule becomes two contact spheres;
+* a joint with a `range` is limited (autolimits); `armature`, `damping`, `frictionloss` come from the joint or its class.
+
+Anything else (ball or slide joints, several joints on a body, meshes or boxes as collision geoms or as the only source of
+inertia, tendons, equality constraints, position actuators) raises ValueError: the file needs MuJoCo's full compiler.
+"""
+from __future__ import annotations
+
+import xml.etree.ElementTree as ET
+
+import numpy as np
+
+from .model import KinematicModel, ModelBuilder
+
+_DENSITY = 1000.0
+
+
+def _vec(text, n=None, default=None):
+    if text is None:
+        return None if default is None else np.array(default, dtype=np.float64)
+    v = np.array([float(t) for t in text.split()], dtype=np.float64)
+    if n is not None and v.size != n:
+        raise ValueError(f"expected {n} numbers, got {text!r}")
+    return v
+
+
+def quat_mul(a, b):
+    aw, ax, ay, az = a
+    bw, bx, by, bz = b
+    return np.array([aw * bw - ax * bx - ay * by - az * bz, aw * bx + ax * bw + ay * bz - az * by,
+                     aw * by - ax * bz + ay * bw + az * bx, aw * bz + ax * by - ay * bx + az * bw])
+
+
+def quat_to_mat(q):
+    w, x, y, z = q / np.linalg.norm(q)
+    return np.array([[1 - 2 * (y * y + z * z), 2 * (x * y - w * z), 2 * (x * z + w * y)],
+                     [2 * (x * y + w * z), 1 - 2 * (x * x + z * z), 2 * (y * z - w * x)],
+                     [2 * (x * z - w * y), 2 * (y * z + w * x), 1 - 2 * (x * x + y * y)]])
+
+
+def mat_to_quat(R):
+    """Unit quaternion (w, x, y, z) of a proper rotation matrix."""
+    t = np.trace(R)
+    if t > 0:
+        s = np.sqrt(t + 1.0) * 2
+        q = np.array([0.25 * s, (R[2, 1] - R[1, 2]) / s, (R[0, 2] - R[2, 0]) / s, (R[1, 0] - R[0, 1]) / s])
+    else:
+        i = int(np.argmax(np.diag(R)))
+        j, k = (i + 1) % 3, (i + 2) % 3
+        s = np.sqrt(1.0 + R[i, i] - R[j, j] - R[k, k]) * 2
+        q = np.zeros(4)
+        q[0] = (R[k, j] - R[j, k]) / s
+        q[1 + i] = 0.25 * s
+        q[1 + j] = (R[j, i] + R[i, j]) / s
+        q[1 + k] = (R[k, i] + R[i, k]) / s
+    return q / np.linalg.norm(q)
+
+
+class _Defaults:
+    """The nested `<default>` classes: attributes of an element type resolved through the class chain."""
+
+    def __init__(self, root):
+        self.classes: dict[str, dict] = {}
+        top = root.find("default")
+        self._walk(top, "main", {}) if top is not None else self.classes.setdefault("main", {})
+
+    def _walk(self, node, name, inherited):
+        own = {k: dict(v) for k, v in inherited.items()}
+        for child in node:
+            if child.tag != "default":
+                own.setdefault(child.tag, {}).update(child.attrib)
+        self.classes[name] = own
+        for child in node:
+            if child.tag == "default":
+                self._walk(child, child.get("class"), own)
+
+    def resolve(self, elem, childclass):
+        cls = elem.get("class") or childclass or "main"
+        if cls not in self.classes:
+            raise ValueError(f"unknown default class {cls!r}")
+        out = dict(self.classes[cls].get(elem.tag, {}))
+        out.update(elem.attrib)
+        return out
+
+
+def _geom_inertia(kind, size, fromto, pos, quat):
+    """(mass, com, inertia tensor about the com) of a sphere or capsule geom in the body frame, density 1000."""
+    if kind == "sphere":
+        r = size[0]
+        m = _DENSITY * 4.0 / 3.0 * np.pi * r**3
+        return m, pos, np.eye(3) * (0.4 * m * r * r)
+    if kind == "capsule":
+        r = size[0]
+        if fromto is not None:
+            a, b = fromto[:3], fromto[3:]
+            length, centre = np.linalg.norm(b - a), 0.5 * (a + b)
+            z = (b - a) / length
+        else:
+            length, centre = 2 * size[1], pos
+            z = quat_to_mat(quat)[:, 2]
+        mc = _DENSITY * np.pi * r * r * length            # cylinder
+        ms = _DENSITY * 4.0 / 3.0 * np.pi * r**3           # the two half spheres together
+        h = length
+        ixx = mc * (r * r / 4 + h * h / 12) + ms * (0.4 * r * r + h * h / 4 + 3.0 / 8.0 * h * r)
+        izz = mc * r * r / 2 + ms * 0.4 * r * r
+        x = np.cross(z, [1.0, 0, 0] if abs(z[0]) < 0.9 else [0, 1.0, 0])
+        x /= np.linalg.norm(x)
+        R = np.stack([x, np.cross(z, x), z], axis=1)
+        return mc + ms, centre, R @ np.diag([ixx, ixx, izz]) @ R.T
+    raise ValueError(f"a {kind} geom cannot give a body its inertia here (sphere and capsule only)")
+
+
+class _Body:
+    def __init__(self, name):
+        self.name = name
+        self.pos, self.quat = np.zeros(3), np.array([1.0, 0, 0, 0])
+        self.joint = None                 # dict or None
+        self.parts = []                   # (mass, com, tensor about com) in this body's frame
+        self.spheres = []                 # (pos, radius) in this body's frame
+        self.children = []
+        self.contact = None               # (friction, solref, solimp) of its collision geoms
+
+
+def load_mjcf(path: str, **options) -> KinematicModel:
+    """Reads an MJCF file into a KinematicModel.  `options` are ModelBuilder's (dt, iterations, integrator, ...): ksim sets
+    them in code (ksim/task/rl.py:717-748), not in the file; an `<option timestep>` in the file is the default for dt."""
+    root = ET.parse(path).getroot()
+    if root.tag != "mujoco":
+        raise ValueError("not an MJCF file")
+    for tag in ("tendon", "equality"):
+        if root.find(tag) is not None and len(root.find(tag)):
+            raise ValueError(f"<{tag}> is outside the model subset")
+    comp = root.find("compiler")
+    degrees = comp is None or comp.get("angle", "degree") == "degree"
+    defaults = _Defaults(root)
+    opt = root.find("option")
+    if opt is not None and "timestep" in opt.attrib:
+        options.setdefault("dt", float(opt.get("timestep")))
+
+    def angle(v):
+        return np.radians(v) if degrees else v
+
+    def frame(attrib):
+        for bad in ("euler", "axisangle", "xyaxes", "zaxis"):
+            if bad in attrib:
+                raise ValueError(f"orientation by {bad} is outside the model subset (use quat)")
+        return _vec(attrib.get("pos"), 3, (0, 0, 0)), _vec(attrib.get("quat"), 4, (1, 0, 0, 0))
+
+    contact_params = []
+
+    def read_body(elem, childclass):
+        b = _Body(elem.get("name", ""))
+        b.pos, b.quat = frame(elem.attrib)
+        b.quat = b.quat / np.linalg.norm(b.quat)
+        childclass = elem.get("childclass", childclass)
+        joints = [e for e in elem if e.tag in ("joint", "freejoint")]
+        if len(joints) > 1:
+            raise ValueError(f"body {b.name!r}: several joints on one body are outside the model subset")
+        if joints:
+            j = joints[0]
+            if j.tag == "freejoint":
+                b.joint = dict(type="free", name=j.get("name", ""))
+            else:
+                a = defaults.resolve(j, childclass)
+                jt = a.get("type", "hinge")
+                if jt == "free":
+                    b.joint = dict(type="free", name=a.get("name", ""))
+                elif jt != "hinge":
+                    raise ValueError(f"joint {a.get('name')!r}: type {jt} is outside the model subset")
+                else:
+                    if float(a.get("ref", 0.0)) != 0.0 or float(a.get("stiffness", 0.0)) != 0.0:
+                        raise ValueError(f"joint {a.get('name')!r}: ref and stiffness are outside the model subset")
+                    rng = _vec(a.get("range"), 2)
+                    limited = a.get("limited", "auto")
+                    if limited == "false" or (limited == "auto" and rng is None):
+                        rng = None
+                    elif rng is None:
+                        raise ValueError(f"joint {a.get('name')!r}: limited without a range")
+                    b.joint = dict(type="hinge", name=a.get("name", ""), axis=_vec(a.get("axis"), 3, (0, 0, 1)),
+                                   pos=_vec(a.get("pos"), 3, (0, 0, 0)), range=None if rng is None else tuple(angle(rng)),
+                                   armature=float(a.get("armature", 0.0)), damping=float(a.get("damping", 0.0)),
+                                   frictionloss=float(a.get("frictionloss", 0.0)))
+        inertial = elem.find("inertial")
+        geoms = [defaults.resolve(g, childclass) for g in elem if g.tag == "geom"]
+        if inertial is not None:
+            if "fullinertia" in inertial.attrib:
+                f = _vec(inertial.get("fullinertia"), 6)
+                tensor = np.array([[f[0], f[3], f[4]], [f[3], f[1], f[5]], [f[4], f[5], f[2]]])
+            else:
+                R = quat_to_mat(_vec(inertial.get("quat"), 4, (1, 0, 0, 0)))
+                tensor = R @ np.diag(_vec(inertial.get("diaginertia"), 3)) @ R.T
+            b.parts.append((float(inertial.get("mass")), _vec(inertial.get("pos"), 3, (0, 0, 0)), tensor))
+        else:
+            for g in geoms:
+                kind = g.get("type", "sphere")
+                if kind == "mesh" or kind == "plane":
+                    if kind == "mesh":
+                        raise ValueError(f"body {b.name!r}: inertia from a mesh is outside the model subset (give <inertial>)")
+                    continue
+                gp, gq = frame(g)
+                b.parts.append(_geom_inertia(kind, _vec(g.get("size")), _vec(g.get("fromto"), 6), gp, gq))
+        for g in geoms:
+            if int(g.get("contype", 1)) == 0 and int(g.get("conaffinity", 1)) == 0:
+                continue  # visual only
+            kind = g.get("type", "sphere")
+            size, gp = _vec(g.get("size")), frame(g)[0]
+            if kind == "sphere":
+                b.spheres.append((gp, float(size[0])))
+            elif kind == "capsule":
+                if g.get("fromto") is not None:
+                    ft = _vec(g.get("fromto"), 6)
+                    ends = (ft[:3], ft[3:])
+                else:
+                    z = quat_to_mat(frame(g)[1])[:, 2] * size[1]
+                    ends = (gp - z, gp + z)
+                b.spheres.extend((e, float(size[0])) for e in ends)
+            else:
+                raise ValueError(f"body {b.name!r}: a colliding {kind} is outside the model subset (sphere and capsule only)")
+            si = _vec(g.get("solimp"), None, (0.9, 0.95, 0.001, 0.5, 2.0))
+            si = np.concatenate([si, np.array([0.9, 0.95, 0.001, 0.5, 2.0])[si.size:]])
+            contact_params.append((float(_vec(g.get("friction"), None, (1.0, 0.005, 0.0001))[0]),
+                                   tuple(_vec(g.get("solref"), 2, (0.02, 1.0))), tuple(si)))
+        b.children = [read_body(c, childclass) for c in elem if c.tag == "body"]
+        return b
+
+    world = root.find("worldbody")
+    tops = [read_body(e, None) for e in world if e.tag == "body"]
+    if len(tops) != 1:
+        raise ValueError("exactly one robot body under <worldbody> is expected")
+
+    def weld(b):
+        """Moves every jointless child (recursively) into b's frame."""
+        kept = []
+        for c in b.children:
+            weld(c)
+            if c.joint is not None:
+                kept.append(c)
+                continue
+            R = quat_to_mat(c.quat)
+            b.parts.extend((m, c.pos + R @ com, R @ I @ R.T) for m, com, I in c.parts)
+            b.spheres.extend((c.pos + R @ p, r) for p, r in c.spheres)
+            for g in c.children:  # grandchildren keep their joints; their frame is re-expressed in b
+                g.pos, g.quat = c.pos + R @ g.pos, quat_mul(c.quat, g.quat)
+                kept.append(g)
+        b.children = kept
+
+    top = tops[0]
+    if top.joint is None:
+        raise ValueError("the robot's top body needs a joint (a fixed base is outside the model subset)")
+    weld(top)
+
+    def composite(parts):
+        if not parts:
+            raise ValueError("a moving body without mass")
+        m = sum(p[0] for p in parts)
+        com = sum(p[0] * p[1] for p in parts) / m
+        I = np.zeros((3, 3))
+        for mi, ci, Ii in parts:
+            d = ci - com
+            I += Ii + mi * (d @ d * np.eye(3) - np.outer(d, d))
+        w, V = np.linalg.eigh(0.5 * (I + I.T))
+        if np.linalg.det(V) < 0:
+            V[:, 2] = -V[:, 2]
+        return m, com, w, mat_to_quat(V)
+
+    if contact_params:
+        if len(set(contact_params)) != 1:
+            raise ValueError("the collision geoms must share friction, solref and solimp")
+        fr, sr, si = contact_params[0]
+        options.setdefault("friction", fr)
+        options.setdefault("solref", sr)
+        options.setdefault("solimp", si)
+        # the joints keep MuJoCo's defaults for their limit and friction rows
+        options.setdefault("dof_solref", (0.02, 1.0))
+        options.setdefault("dof_solimp", (0.9, 0.95, 0.001, 0.5, 2.0))
+    mb = ModelBuilder(**options)
+    joint_body: dict[str, int] = {}
+
+    def add(b, parent):
+        m, com, inertia, iquat = composite(b.parts)
+        j = b.joint
+        if j["type"] == "free":
+            idx = mb.add_body(parent, b.pos, joint="free", quat=b.quat, mass=m, ipos=com, iquat=iquat, inertia=inertia, name=b.name)
+        else:
+            idx = mb.add_body(parent, b.pos, joint="hinge", axis=j["axis"], joint_pos=j["pos"], quat=b.quat, mass=m, ipos=com,
+                              iquat=iquat, inertia=inertia, damping=j["damping"], armature=j["armature"], range=j["range"],
+                              frictionloss=j["frictionloss"], name=b.name)
+        joint_body[j["name"]] = idx
+        for p, r in b.spheres:
+            mb.add_contact_sphere(idx, p, r)
+        for c in b.children:
+            add(c, idx)
+
+    add(top, 0)
+    act = root.find("actuator")
+    for a in ([] if act is None else act):
+        if a.tag != "motor":
+            raise ValueError(f"actuator <{a.tag}> is outside the model subset (motors only; ksim's PD law runs outside MuJoCo)")
+        at = defaults.resolve(a, None)
+        if at.get("joint") not in joint_body:
+            raise ValueError(f"motor {at.get('name')!r} drives an unknown joint")
+        cr = _vec(at.get("ctrlrange"), 2)
+        limited = at.get("ctrllimited", "auto")
+        mb.add_actuator(joint_body[at["joint"]], gear=float(_vec(at.get("gear"), None, (1.0,))[0]),
+                        ctrlrange=None if (cr is None or limited == "false") else tuple(cr))
+    return mb.build()

@@ -122,6 +122,9 @@ class KinematicModel:
     jnt_limited: np.ndarray
     jnt_range: np.ndarray
     dof_frictionloss: np.ndarray
+    # solref / solimp of the limit and friction rows (MuJoCo: per joint, its defaults here unless given)
+    dof_solref: np.ndarray
+    dof_solimp: np.ndarray
     # actuators (motors: force = gear * clip(ctrl, ctrlrange))
     act_dof: np.ndarray
     act_gear: np.ndarray
@@ -160,7 +163,7 @@ class ModelBuilder:
 
     def __init__(self, dt=0.005, gravity=(0.0, 0.0, -9.81), iterations=8, ls_iterations=8, tolerance=1e-10,
                  ls_tolerance=0.01, impratio=1.0, eulerdamp=False, solref=(0.02, 1.0),
-                 solimp=(0.9, 0.95, 0.001, 0.5, 2.0), friction=1.0, integrator=None):
+                 solimp=(0.9, 0.95, 0.001, 0.5, 2.0), friction=1.0, integrator=None, dof_solref=None, dof_solimp=None):
         # integrator: "euler" (explicit joint damping unless `eulerdamp`) or "implicitfast", the one ksim sets
         # (ksim/task/rl.py:555-578).  With torque motors the only velocity-dependent smooth force is joint damping, so
         # implicitfast is the damping-implicit velocity update, (M + dt diag(damping)) a = M qacc.
@@ -171,7 +174,9 @@ class ModelBuilder:
                         ls_iterations=int(ls_iterations), tolerance=float(tolerance),
                         ls_tolerance=float(ls_tolerance), impratio=float(impratio), eulerdamp=bool(eulerdamp),
                         solref=np.array(solref, dtype=np.float64), solimp=np.array(solimp, dtype=np.float64),
-                        friction=float(friction))
+                        friction=float(friction),
+                        dof_solref=np.array(solref if dof_solref is None else dof_solref, dtype=np.float64),
+                        dof_solimp=np.array(solimp if dof_solimp is None else dof_solimp, dtype=np.float64))
         self.bodies = [dict(parent=-1, jtype=JNT_NONE, pos=np.zeros(3), quat=np.array([1.0, 0, 0, 0]), mass=0.0,
                             ipos=np.zeros(3), iquat=np.array([1.0, 0, 0, 0]), inertia=np.zeros(3),
                             axis=np.array([0.0, 0, 1]), jpos=np.zeros(3), damping=0.0, armature=0.0, qpos0=0.0,

@@ -356,26 +356,37 @@ static REAL impedance(REAL pos, REAL dmin, REAL dmax, REAL width, REAL mid, REAL
   return imp;
 }
 
+static void sol_params(const double* solref, const double* solimp, double dt, REAL* kk, REAL* bb, REAL* dmin, REAL* dmax,
+                       REAL* width, REAL* mid, REAL* power) {
+  REAL timeconst = (REAL)solref[0], dampratio = (REAL)solref[1];
+  *dmin = (REAL)solimp[0]; *dmax = (REAL)solimp[1]; *width = (REAL)solimp[2]; *mid = (REAL)solimp[3]; *power = (REAL)solimp[4];
+  if (timeconst < 2 * (REAL)dt) timeconst = 2 * (REAL)dt;
+  *dmin = *dmin < MINIMP ? MINIMP : (*dmin > MAXIMP ? MAXIMP : *dmin);
+  *dmax = *dmax < MINIMP ? MINIMP : (*dmax > MAXIMP ? MAXIMP : *dmax);
+  *width = *width < MINVAL ? MINVAL : *width;
+  *mid = *mid < MINIMP ? MINIMP : (*mid > MAXIMP ? MAXIMP : *mid);
+  *power = *power < 1 ? 1 : *power;
+  *kk = 1 / (*dmax * *dmax * timeconst * timeconst * dampratio * dampratio);
+  *bb = 2 / (*dmax * timeconst);
+  if (solref[0] <= 0) *kk = -(REAL)solref[0] / (*dmax * *dmax);
+  if (solref[1] <= 0) *bb = -(REAL)solref[1] / *dmax;
+}
+
 /* Rows in the order contacts, joint limits, dry friction (MuJoCo orders them friction, limits, contacts; the order
  * only changes the order of summation). */
 void FN(ksor_make_constraint)(const KsorModel* m, Data* d) {
   const int nv = m->nv;
   int nefc = 0;
   const REAL mu = d->friction;
-  /* solref / solimp -> stiffness k, damping b (refsafe) */
-  REAL timeconst = (REAL)m->solref[0], dampratio = (REAL)m->solref[1];
-  REAL dmin = (REAL)m->solimp[0], dmax = (REAL)m->solimp[1], width = (REAL)m->solimp[2], mid = (REAL)m->solimp[3],
-       power = (REAL)m->solimp[4];
-  if (timeconst < 2 * (REAL)m->dt) timeconst = 2 * (REAL)m->dt;
-  dmin = dmin < MINIMP ? MINIMP : (dmin > MAXIMP ? MAXIMP : dmin);
-  dmax = dmax < MINIMP ? MINIMP : (dmax > MAXIMP ? MAXIMP : dmax);
-  width = width < MINVAL ? MINVAL : width;
-  mid = mid < MINIMP ? MINIMP : (mid > MAXIMP ? MAXIMP : mid);
-  power = power < 1 ? 1 : power;
-  REAL kk = 1 / (dmax * dmax * timeconst * timeconst * dampratio * dampratio);
-  REAL bb = 2 / (dmax * timeconst);
-  if (m->solref[0] <= 0) kk = -(REAL)m->solref[0] / (dmax * dmax);
-  if (m->solref[1] <= 0) bb = -(REAL)m->solref[1] / dmax;
+  /* solref / solimp -> stiffness k, damping b (refsafe) and clamped impedance parameters: one set for the contact rows,
+   * one for the rows of joint limits and dry friction (dof_solref / dof_solimp; all zero = the contact set) */
+  REAL kk, bb, dmin, dmax, width, mid, power;
+  sol_params(m->solref, m->solimp, m->dt, &kk, &bb, &dmin, &dmax, &width, &mid, &power);
+  int own = 0;
+  for (int k = 0; k < 2; ++k) own |= m->dof_solref[k] != 0;
+  for (int k = 0; k < 5; ++k) own |= m->dof_solimp[k] != 0;
+  REAL jk = kk, jb = bb, jdmin = dmin, jdmax = dmax, jwidth = width, jmid = mid, jpower = power;
+  if (own) sol_params(m->dof_solref, m->dof_solimp, m->dt, &jk, &jb, &jdmin, &jdmax, &jwidth, &jmid, &jpower);
 
   for (int s = 0; s < m->ns; ++s) {
     const int b = m->sph_body[s];
@@ -427,11 +438,11 @@ void FN(ksor_make_constraint)(const KsorModel* m, Data* d) {
     REAL* row = d->efc_J + nefc * nv;
     for (int i = 0; i < nv; ++i) row[i] = 0;
     row[j] = side;
-    const REAL imp = impedance(pos, dmin, dmax, width, mid, power);
+    const REAL imp = impedance(pos, jdmin, jdmax, jwidth, jmid, jpower);
     REAL R = (REAL)m->dof_invweight0[j] * (1 - imp) / imp;
     if (R < MINVAL) R = MINVAL;
     d->efc_pos[nefc] = pos;
-    d->efc_aref[nefc] = -bb * side * d->qvel[j] - kk * imp * pos;
+    d->efc_aref[nefc] = -jb * side * d->qvel[j] - jk * imp * pos;
     d->efc_D[nefc] = 1 / R;
     d->efc_floss[nefc] = 0;
     ++nefc;
@@ -443,11 +454,11 @@ void FN(ksor_make_constraint)(const KsorModel* m, Data* d) {
     REAL* row = d->efc_J + nefc * nv;
     for (int i = 0; i < nv; ++i) row[i] = 0;
     row[j] = 1;
-    const REAL imp = impedance(0, dmin, dmax, width, mid, power);
+    const REAL imp = impedance(0, jdmin, jdmax, jwidth, jmid, jpower);
     REAL R = (REAL)m->dof_invweight0[j] * (1 - imp) / imp;
     if (R < MINVAL) R = MINVAL;
     d->efc_pos[nefc] = 0;
-    d->efc_aref[nefc] = -bb * d->qvel[j];
+    d->efc_aref[nefc] = -jb * d->qvel[j];
     d->efc_D[nefc] = 1 / R;
     d->efc_floss[nefc] = fl;
     ++nefc;

@@ -42,6 +42,7 @@ typedef struct KsorModel {
    * dof_invweight0 is the diagonal of the inverse mass matrix at qpos0, which scales their regularisation */
   int jnt_limited[KSOR_MAXB];
   double jnt_range[KSOR_MAXB][2], dof_invweight0[KSOR_MAXV], dof_frictionloss[KSOR_MAXV];
+  double dof_solref[2], dof_solimp[5]; /* solref / solimp of the limit and friction rows; all zero = those of the contacts */
   int act_dof[KSOR_MAXU];
   double act_gear[KSOR_MAXU], act_lo[KSOR_MAXU], act_hi[KSOR_MAXU];
   int sph_body[KSOR_MAXS];

@@ -25,7 +25,14 @@ MODELS = {"chain": km.pendulum_chain_model, "humanoid": km.humanoid_model, "kbot
           # (much deeper violations make the cost so large that its fp32 rounding hides the last Newton improvements).
           "chain-friction": lambda: km.pendulum_chain_model(integrator="implicitfast", frictionloss=0.3),
           "humanoid-limits": lambda: km.humanoid_model(joint_range=(-0.45, 0.5)),
-          "kbot-limits": lambda: km.kbot_scale_model(integrator="implicitfast", joint_range=(-0.45, 0.5), frictionloss=0.2)}
+          "kbot-limits": lambda: km.kbot_scale_model(integrator="implicitfast", joint_range=(-0.45, 0.5), frictionloss=0.2),
+          # the real K-Bot's contact parameters (robot.mjcf:24): five times stiffer rows than MuJoCo's defaults
+          "kbot-stiff-feet": lambda: km.kbot_scale_model(integrator="implicitfast", joint_range=(-0.45, 0.5), frictionloss=0.2,
+                                                         solref=(0.02, 0.8), solimp=(0.98, 0.99, 0.1, 0.5, 2.0),
+                                                         dof_solref=(0.02, 1.0), dof_solimp=(0.9, 0.95, 0.001, 0.5, 2.0))}
+# fp32 against float64 on the stiff-feet model: the constraint stiffness D = d / ((1 - d) invweight) with d = 0.98..0.99 is
+# five times the default one, and so is the amplification of rounding in H = M + J^T D J
+STIFF_TOL = 5e-4
 ONE_STEP_TOL, TEN_STEP_TOL = 1e-4, 1e-3
 
 
@@ -69,9 +76,10 @@ def test_forward_quantities_match_oracle(setup):
     for got, ref, tol in [("dbg_M", "M", 1e-5), ("dbg_bias", "qfrc_bias", 1e-5), ("xpos", "xpos", 1e-5),
                           ("xquat", "xquat", 1e-5), ("cvel", "cvel", 1e-5), ("cinert", "cinert", 1e-5),
                           # contact forces are -D (J qacc - aref) with D ~ 1e3..1e4: they amplify the rounding of qacc
-                          ("cfrc_ext", "cfrc_ext", 2e-3),
+                                                    ("cfrc_ext", "cfrc_ext", 1e-2 if name == "kbot-stiff-feet" else 2e-3),
                           ("dbg_qacc_smooth", "qacc_smooth", 1e-4),
-                          ("qacc", "qacc", ONE_STEP_TOL), ("qacc_warmstart", "qacc", ONE_STEP_TOL)]:
+                          ("qacc", "qacc", STIFF_TOL if name == "kbot-stiff-feet" else ONE_STEP_TOL),
+                          ("qacc_warmstart", "qacc", STIFF_TOL if name == "kbot-stiff-feet" else ONE_STEP_TOL)]:
         err = rel_err(g[got], want[ref]).max()
         assert err <= tol, f"{name}.{ref}: rel err {err:.2e} > {tol}"
     if m.ns:
@@ -514,3 +522,44 @@ def test_joint_limit_and_dry_friction_closed_forms():
     R = (1 / inertia) * (1 - imp) / imp
     # fp32 state: the penetration is ~1e-4 rad on an angle of 0.3, so it is resolved to about three digits
     assert (1 / R) * k * imp * abs(pos) == pytest.approx(mass * 9.81 * (L / 2) * np.sin(q), rel=5e-3)
+
+
+def test_model_loaded_from_mjcf_matches_oracle():
+    """A model read from an MJCF file (welded bodies, capsule feet, limits, dry friction, its own contact and joint
+    solref / solimp): forward quantities and ten physics steps against the oracle."""
+    import os
+    from ksim_amd import physics
+    from ksim_amd._lib_dyn import KS_ACT_TORQUE
+    from ksim_amd.mjcf import load_mjcf
+
+    m = load_mjcf(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "mini_biped.mjcf"), integrator="implicitfast")
+    dm = physics.DeviceModel(m)
+    N = 40
+    rng = np.random.default_rng(61)
+    qpos, qvel = random_states(m, N, seed=62, vel_scale=0.3)
+    # hips within and slightly beyond their ranges, knees around their lower limit
+    qpos[:, 7] = rng.uniform(-1.05, 1.55, N); qpos[:, 9] = rng.uniform(-1.55, 1.05, N)
+    qpos[:, 8] = rng.uniform(-0.05, 1.0, N); qpos[:, 10] = rng.uniform(-0.5, 0.5, N)
+    ctrl = rng.normal(size=(N, m.nu)) * 3
+    warm = np.zeros((N, m.nv))
+    want = oracle_forward(m, qpos, qvel, ctrl, None, None, warm)
+    buf = dict(qpos=t32(qpos), qvel=t32(qvel), qacc_warmstart=t32(warm), ctrl_in=t32(ctrl), qacc=zeros(N, m.nv),
+               xpos=zeros(N, m.nb * 3), nefc=zeros(N, dtype=torch.int32), contact_dist=zeros(N, m.ns))
+    physics.forward(dm, buf)
+    assert rel_err(buf["xpos"].cpu().numpy(), want["xpos"]).max() < 1e-5
+    assert np.array_equal(buf["nefc"].cpu().numpy(), want["nefc"])
+    assert (want["nefc"] > 4).sum() >= N // 3  # friction rows always, limit and contact rows in many envs
+    assert rel_err(buf["qacc"].cpu().numpy(), want["qacc"]).max() <= ONE_STEP_TOL
+    orc = Oracle(m.arrays())
+    wq, wv = [], []
+    for e in range(N):
+        d = orc.data(qpos[e], qvel[e])
+        d.ctrl = ctrl[e]
+        for _ in range(10):
+            orc.step(d)
+        wq.append(np.array(d.qpos)); wv.append(np.array(d.qvel))
+    buf = dict(qpos=t32(qpos), qvel=t32(qvel), qacc_warmstart=zeros(N, m.nv), time=zeros(N), last_ctrl=t32(ctrl), action=t32(ctrl))
+    for _ in range(10):
+        physics.control_step(dm, buf, substeps=1, actuator_type=KS_ACT_TORQUE)
+    eq, ev = rel_err(buf["qpos"].cpu().numpy(), wq).max(), rel_err(buf["qvel"].cpu().numpy(), wv).max()
+    assert eq <= TEN_STEP_TOL and ev <= TEN_STEP_TOL, f"qpos {eq:.2e} qvel {ev:.2e}"

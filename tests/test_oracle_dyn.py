@@ -423,8 +423,8 @@ def test_contact_forces_on_bodies(model):
 
 
 # --------------------------------------------------------------------------- joint limits and dry joint friction
-def _impedance(m, pos):
-    dmin, dmax, width, mid, power = m.solimp
+def _impedance(m, pos, solimp=None):
+    dmin, dmax, width, mid, power = m.solimp if solimp is None else solimp
     x = abs(pos) / width
     y = (1 / mid ** (power - 1)) * x**power if x < mid else 1 - (1 / (1 - mid) ** (power - 1)) * (1 - x) ** power
     return dmax if x > 1 else float(np.clip(dmin + y * (dmax - dmin), dmin, dmax))
@@ -487,7 +487,10 @@ def test_pendulum_rests_on_its_limit_where_the_spring_predicts():
     """One link on a horizontal hinge, range (0.3, 1.0): gravity pulls it towards 0 and it settles just below 0.3,
     where the limit force D k imp |pos| balances the gravity torque m g (L/2) sin q."""
     L, mass = 0.5, 1.0
-    m = km.pendulum_chain_model(n_links=1, length=L, mass=mass, damping=0.5, joint_range=(0.3, 1.0))
+    # the limit row has its own solref / solimp, different from the contacts'
+    m = km.pendulum_chain_model(n_links=1, length=L, mass=mass, damping=0.5, joint_range=(0.3, 1.0), dof_solref=(0.04, 1.0),
+                                dof_solimp=(0.8, 0.9, 0.01, 0.5, 2.0))
+    assert tuple(m.solref) == (0.02, 1.0) and tuple(m.dof_solref) == (0.04, 1.0)
     orc = Oracle(m.arrays())
     d = orc.data(np.array([0.6]), np.zeros(1))
     for _ in range(4000):
@@ -496,15 +499,16 @@ def test_pendulum_rests_on_its_limit_where_the_spring_predicts():
     q = float(d.qpos[0])
     pos = q - 0.3
     assert -0.01 < pos < 0
-    tc = max(m.solref[0], 2 * m.dt)
-    k = 1 / (m.solimp[1] ** 2 * tc**2 * m.solref[1] ** 2)
-    imp = _impedance(m, pos)
+    tc = max(m.dof_solref[0], 2 * m.dt)
+    k = 1 / (m.dof_solimp[1] ** 2 * tc**2 * m.dof_solref[1] ** 2)
+    imp = _impedance(m, pos, m.dof_solimp)
     inertia = float(d.M[0, 0])  # the hinge's inertia, pinned against the Jacobian sum elsewhere
     assert m.dof_invweight0[0] == pytest.approx(1 / inertia)
     R = (1 / inertia) * (1 - imp) / imp
     assert (1 / R) * k * imp * abs(pos) == pytest.approx(mass * 9.81 * (L / 2) * np.sin(q), rel=1e-6)
     # inside the range the limit does nothing
     free = km.pendulum_chain_model(n_links=1, length=L, mass=mass, damping=0.5)
+    assert tuple(free.dof_solref) == tuple(free.solref) and tuple(free.dof_solimp) == tuple(free.solimp)  # default: the contacts' pair
     a, b = orc.data(np.array([0.7]), np.array([0.1])), Oracle(free.arrays()).data(np.array([0.7]), np.array([0.1]))
     orc.forward(a); Oracle(free.arrays()).forward(b)
     assert a.nefc == 0 and a.qacc[0] == b.qacc[0]
