@@ -255,7 +255,7 @@ __device__ __forceinline__ float impedance_dof(const DevModel& m, float pos) {
 // The rows a dof lane carries itself: the violated limit of its hinge (J = lim_s e_j, lim_s = +-1, 0 when none) and its
 // dry friction (J = e_j, force clipped at +-fr_fl, 0 when none).  All zero on lanes that hold no dof.
 struct DofRows {
-  float lim_s, lim_aref, lim_D, fr_fl, fr_aref, fr_D;
+  float lim_s, lim_aref, lim_D, fr_fl, fr_aref, fr_D, fr_rf;  // fr_rf = fr_fl / fr_D, where the friction force saturates
 };
 
 // Cost of the lane's rows at acceleration qa; their force on the dof, their Hessian diagonal and which of them are in
@@ -268,7 +268,7 @@ __device__ __forceinline__ float dofrow_eval(const DofRows& r, float qa, float& 
     cost = 0.5f * r.lim_D * xl * xl; force = -r.lim_D * xl * r.lim_s; hdiag = r.lim_D; zone = 1;
   }
   if (r.fr_fl > 0.f) {
-    const float xf = qa - r.fr_aref, rf = r.fr_fl / r.fr_D;
+    const float xf = qa - r.fr_aref, rf = r.fr_rf;
     if (xf <= -rf) { cost += r.fr_fl * (-0.5f * rf - xf); force += r.fr_fl; }
     else if (xf >= rf) { cost += r.fr_fl * (-0.5f * rf + xf); force -= r.fr_fl; }
     else { cost += 0.5f * r.fr_D * xf * xf; force -= r.fr_D * xf; hdiag += r.fr_D; zone |= 2; }
@@ -285,7 +285,7 @@ __device__ __forceinline__ void dofrow_quad(const DofRows& r, float qa, float sd
     t0 = 0.5f * x0 * x0 * r.lim_D; t1 = jv * x0 * r.lim_D; t2 = 0.5f * jv * jv * r.lim_D;
   }
   if (r.fr_fl > 0.f) {
-    const float f0 = qa - r.fr_aref, rf = r.fr_fl / r.fr_D, x = f0 + alpha * sdir;
+    const float f0 = qa - r.fr_aref, rf = r.fr_rf, x = f0 + alpha * sdir;
     if (x <= -rf) { t0 += r.fr_fl * (-0.5f * rf - f0); t1 -= r.fr_fl * sdir; }
     else if (x >= rf) { t0 += r.fr_fl * (-0.5f * rf + f0); t1 += r.fr_fl * sdir; }
     else { t0 += 0.5f * f0 * f0 * r.fr_D; t1 += sdir * f0 * r.fr_D; t2 += 0.5f * sdir * sdir * r.fr_D; }
@@ -776,7 +776,7 @@ void step_kernel(StepArgs a) {
     int niter = 0;
     // ---- rows on the dof lanes (models with joint limits or dry friction only).  Their Jacobians are unit vectors, so
     // nothing of them is stored: lane j derives J a - aref of its rows from its own qacc wherever the solver needs it.
-    DofRows dr = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    DofRows dr = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     int ndr = 0;
     if (DR) {
       int lane_r = threadIdx.x;
@@ -796,6 +796,7 @@ void step_kernel(StepArgs a) {
         }
         dr.fr_fl = rr->d_floss;
         dr.fr_D = rr->d_frD;
+        dr.fr_rf = dr.fr_fl / dr.fr_D;
         dr.fr_aref = -m.dr_b * my_qvel;
       }
       ndr = __popcll(__ballot(dr.lim_s != 0.f)) + m.nfriction;
@@ -966,8 +967,9 @@ void step_kernel(StepArgs a) {
         // Rows 16..31 ride along as a second copy in the same lanes, so up to 32 rows need no more reduction steps.
         const bool packed = nefc <= 32, two = nefc > 16;
         float pk_j = 0.f, pk_jv = 0.f, pk_q = 0.f, pk_j2 = 0.f, pk_jv2 = 0.f, pk_q2 = 0.f;
+        const int grp = lane >> 4;
         if (packed) {
-          const int r = lane & 15, grp = lane >> 4;
+          const int r = lane & 15;
           pk_j = __shfl(Jaref, r);
           pk_jv = __shfl(jv, r);
           const float c0 = __shfl(q0r, r), c1 = __shfl(q1r, r), c2 = __shfl(q2r, r);
@@ -984,20 +986,30 @@ void step_kernel(StepArgs a) {
           if (packed) {
             float x = (pk_j + alpha * pk_jv < 0.f) ? pk_q : 0.f;  // rows beyond nefc carry zeros
             if (two) x += (pk_j2 + alpha * pk_jv2 < 0.f) ? pk_q2 : 0.f;
+            if (DR && ndr > 0) {
+              // The rows on the dof lanes join the same reduction.  Lane j < 32 holds the three coefficients of its own rows:
+              // the constant one belongs in group 0, the linear one in group 1, so each lane keeps the one of its own group
+              // and swaps the other with the lane 16 away; the quadratic ones go to the upper lane half (groups 2 and 3).
+              float t0, t1, t2;
+              dofrow_quad(dr, qacc, search, alpha, t0, t1, t2);
+              const float got = __shfl_xor(grp == 0 ? t1 : t0, 16);
+              const float up = __shfl(t2, lane & 31);
+              x += grp == 0 ? t0 + got : (grp == 1 ? t1 + got : up);
+            }
             x += dpp_shift<0x111, 0xf>(x);
             x += dpp_shift<0x112, 0xf>(x);
             x += dpp_shift<0x114, 0xf>(x);
             x += dpp_shift<0x118, 0xf>(x);  // lane 15 of each 16-lane group holds the group's total
             q0 = g0 + lane_bcast(x, 15);
             q1 = g1 + lane_bcast(x, 31);
-            q2 = g2 + lane_bcast(x, 47);
+            q2 = g2 + lane_bcast(x, 47) + (DR ? lane_bcast(x, 63) : 0.f);
           } else {
             const bool on = is_row && (Jaref + alpha * jv < 0.f);
             q0 = g0 + wave_sum(on ? q0r : 0.f);
             q1 = g1 + wave_sum(on ? q1r : 0.f);
             q2 = g2 + wave_sum(on ? q2r : 0.f);
           }
-          if (DR && ndr > 0) {
+          if (DR && ndr > 0 && !packed) {
             float t0, t1, t2;
             dofrow_quad(dr, qacc, search, alpha, t0, t1, t2);
             q0 += wave_sum(t0);
