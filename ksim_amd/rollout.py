@@ -18,12 +18,39 @@ from . import _lib_terms as T
 from . import ppo as ppo_mod
 from .commands import CommandSet
 from .engine import HipEngine
-from .env_terms import EnvTerms, sample_action
+from .env_terms import EnvTerms, sample_action, sample_action_head, sample_action_mixture
 from .mlp import MLP
 from .physics import DeviceModel
 from .recurrent import RecurrentNetwork
 from .rewards import Reward, get_rewards, reward_carry_size
 from .types import PhysicsState, RewardState, Trajectory
+
+
+@dataclass(frozen=True)
+class GaussianHead:
+    """The actor emits (means | raw deviations), 2 per action entry (examples/kbot/train.py:915-932)."""
+    min_std: float
+    max_std: float
+    var_scale: float = 1.0
+    mean_bias: torch.Tensor | None = None
+
+    def width(self, na: int) -> int:
+        return 2 * na
+
+
+@dataclass(frozen=True)
+class MixtureHead:
+    """The actor emits component means, raw deviations and logits, 3 K per action entry (examples/walking.py:127-144)."""
+    num_mixtures: int
+    min_std: float
+    max_std: float
+    var_scale: float = 1.0
+    mean_bias: torch.Tensor | None = None
+    clip_lo: torch.Tensor | None = None
+    clip_hi: torch.Tensor | None = None
+
+    def width(self, na: int) -> int:
+        return 3 * na * self.num_mixtures
 
 
 @dataclass
@@ -39,6 +66,7 @@ class RolloutConstants:  # the static pieces, ksim/task/rl.py:138-150
     reward_clip_min: float | None = None
     reward_clip_max: float | None = None
     commands: CommandSet | None = None  # commands advanced once per control step (rl.py:1082-1098); None: constant
+    head: GaussianHead | MixtureHead | None = None  # None: one mean per action entry and the log_std vector
 
 
 class RolloutEnvState:  # ksim/task/rl.py:110-123, batched
@@ -71,7 +99,7 @@ class Rollout:
         b = lambda *s: torch.zeros(*s, dtype=torch.uint8, device=dev)  # noqa: E731
         self.obs, self.noisy_obs = f(Tn, N, c.terms.obs_dim), f(Tn, N, c.terms.obs_dim)
         na = c.engine.actuators.action_dim(m.nu)  # 2 nu for position-velocity actuators
-        self.action, self.mean = f(Tn, N, na), f(N, na)
+        self.action, self.mean = f(Tn, N, na), f(N, na if c.head is None else c.head.width(na))
         self.qpos, self.qvel = f(Tn, N, m.nq), f(Tn, N, m.nv)
         self.xpos, self.xquat, self.ctrl = f(Tn, N, m.nb * 3), f(Tn, N, m.nb * 4), f(Tn, N, m.nu)
         self.done, self.success, self.timestep = b(Tn, N), b(Tn, N), f(Tn, N)
@@ -84,8 +112,8 @@ class Rollout:
         # Philox step counter of graph replays: kernels add it to the step baked into the captured launch
         self.step_base = torch.zeros(1, dtype=torch.int64, device=dev)
         self._graph = None
-        if c.actor.in_dim != c.terms.obs_dim or c.actor.out_dim != na:
-            raise _lib.KsError("actor must map the observation vector to one mean per action entry")
+        if c.actor.in_dim != c.terms.obs_dim or c.actor.out_dim != self.mean.shape[1]:
+            raise _lib.KsError("actor must map the observation vector to one mean per action entry (or to what its head takes)")
         if c.critic is not None and (c.critic.in_dim != c.terms.obs_dim or c.critic.out_dim != 1):
             raise _lib.KsError("critic must map the observation vector to one value")
 
@@ -121,8 +149,18 @@ class Rollout:
                 c.critic(self.obs[t], env.critic_carry, fresh=self.reset_mask, out=self.values[t])
             elif c.critic is not None:
                 c.critic(self.obs[t], out=self.values[t])
-        sample_action(self.mean, c.log_std, noise=noise.get("action_normal"), seed=env.seed, step=step,
-                      step_base=step_base, clip_max=c.action_clip_max, out=self.action[t])
+        if isinstance(c.head, GaussianHead):
+            sample_action_head(self.mean, min_std=c.head.min_std, max_std=c.head.max_std, var_scale=c.head.var_scale,
+                               mean_bias=c.head.mean_bias, noise=noise.get("action_normal"), seed=env.seed, step=step,
+                               step_base=step_base, clip_max=c.action_clip_max, out=self.action[t])
+        elif isinstance(c.head, MixtureHead):
+            sample_action_mixture(self.mean, c.head.num_mixtures, min_std=c.head.min_std, max_std=c.head.max_std,
+                                  var_scale=c.head.var_scale, mean_bias=c.head.mean_bias, clip_lo=c.head.clip_lo,
+                                  clip_hi=c.head.clip_hi, uniform=noise.get("action_uniform"), noise=noise.get("action_normal"),
+                                  seed=env.seed, step=step, step_base=step_base, clip_max=c.action_clip_max, out=self.action[t])
+        else:
+            sample_action(self.mean, c.log_std, noise=noise.get("action_normal"), seed=env.seed, step=step,
+                          step_base=step_base, clip_max=c.action_clip_max, out=self.action[t])
         # the step kernel also writes ctrl / xpos / xquat of the post-step data into the transition slot
         c.engine.step(self.action[t], c.physics_model, ps, level, env.seed + env.step, env.randomization_dict,
                       noise=noise.get("engine"), record=dict(ctrl=self.ctrl[t], xpos=self.xpos[t], xquat=self.xquat[t]),

@@ -17,7 +17,7 @@ def t32(a):
     return torch.tensor(np.asarray(a), dtype=torch.float32, device=DEV).contiguous()
 
 
-def build(N, T, seed=0, min_height=0.9, events=None, gait=False, recurrent=False):
+def build(N, T, seed=0, min_height=0.9, events=None, gait=False, recurrent=False, head=None):
     from ksim_amd import actuators, engine, model as km, observation as ob, physics, randomization as rnd, resets as rs
     from ksim_amd import rewards as rw, terminations as tm
     from ksim_amd.env_terms import EnvTerms
@@ -88,9 +88,17 @@ def build(N, T, seed=0, min_height=0.9, events=None, gait=False, recurrent=False
             n = RecurrentNetwork(proj, [GRUCell(*c_, dtype="f32") for c_ in cells], MLP(ow, ob_, activation=act, dtype="f32"), dtype="f32")
             n.params = (proj, cells, ow, ob_)
             return n
-        actor, critic = net(m.nu, "gelu"), net(1, "elu")
+        head_bias = t32(rng.normal(size=m.nu) * 0.05)
+        if head == "gaussian":   # means | raw deviations, deviations squeezed to ~0 so that the sample shows the mean
+            from ksim_amd.rollout import GaussianHead
+            head = GaussianHead(min_std=0.0, max_std=1e-6, mean_bias=head_bias)
+        elif head == "mixture":
+            from ksim_amd.rollout import MixtureHead
+            head = MixtureHead(num_mixtures=2, min_std=0.0, max_std=1e-6, mean_bias=head_bias,
+                               clip_lo=t32(np.full(m.nu, -0.3)), clip_hi=t32(np.full(m.nu, 0.3)))
+        actor, critic = net(m.nu if head is None else head.width(m.nu), "gelu"), net(1, "elu")
     consts = RolloutConstants(physics_model=dm, engine=eng, terms=terms, rewards=rewards,
-                              actor=actor, critic=critic, log_std=t32(log_std), commands=commands)
+                              actor=actor, critic=critic, log_std=t32(log_std), commands=commands, head=head)
     gen = torch.Generator(device=DEV); gen.manual_seed(seed)
     randomization = rnd.get_physics_randomizers(m, {"f": rnd.FloorFrictionRandomizer(0.4, 1.2),
                                                     "m": rnd.AllBodiesMassMultiplicationRandomizer(0.9, 1.1)}, N, gen)
@@ -392,15 +400,18 @@ def test_rollout_written_to_the_dataset_format_and_read_back(tmp_path):
         assert torch.equal(r.total, rew.total[:, e]) and torch.equal(r.components["height"], rew.components["height"][:, e])
 
 
-def test_recurrent_actor_and_critic_in_the_rollout():
+@pytest.mark.parametrize("head", [None, "gaussian", "mixture"])
+def test_recurrent_actor_and_critic_in_the_rollout(head):
     """GRU actor and critic inside the environment loop: the carries replayed by the oracle from the recorded
-    observations and done flags (a finished env continues from a zero carry), and the graph replay equal to eager."""
+    observations and done flags (a finished env continues from a zero carry), and the graph replay equal to eager.  With a
+    head, the actor's output goes through the deviation head or the mixture head; their deviations are squeezed to 1e-6
+    here, so the recorded action must be the (biased, clipped) mean, of one of the components for the mixture."""
     from oracle import recurrent as orec
 
     N, T = 24, 8
     runs = []
     for use_graph in (False, True):
-        m, c, rnd_, _, ro, EnvState = build(N, T, seed=13, min_height=0.95, recurrent=True)
+        m, c, rnd_, _, ro, EnvState = build(N, T, seed=13, min_height=0.95, recurrent=True, head=head)
         ps = c.engine.reset(c.physics_model, 1.0, 3, N, rnd_)
         env = EnvState(ps, rnd_, torch.zeros(N, 2, device=DEV), None, seed=21)
         want = {"actor": np.zeros((2, N, 32)), "critic": np.zeros((2, N, 32))}
@@ -418,8 +429,16 @@ def test_recurrent_actor_and_critic_in_the_rollout():
                 proj, cells, ow, ob_ = c.critic.params
                 v, want["critic"] = orec.recurrent_network(obs[t], want["critic"], fresh, proj, cells, ow, ob_, act=lambda x: np.where(x > 0, x, np.expm1(x)))
                 proj, cells, ow, ob_ = c.actor.params
-                _, want["actor"] = orec.recurrent_network(noisy[t], want["actor"], fresh, proj, cells, ow, ob_)
+                y, want["actor"] = orec.recurrent_network(noisy[t], want["actor"], fresh, proj, cells, ow, ob_)
                 np.testing.assert_allclose(ro.values[t].cpu().numpy(), v, rtol=2e-4, atol=2e-4)
+                if head is not None:
+                    act_t, nu = traj.action[t].cpu().numpy(), m.nu
+                    bias = c.head.mean_bias.cpu().numpy()
+                    if head == "gaussian":
+                        np.testing.assert_allclose(act_t, y[:, :nu] + bias, rtol=2e-4, atol=2e-4)
+                    else:
+                        means = np.clip(y[:, :2 * nu].reshape(N, nu, 2) + bias[None, :, None], -0.3, 0.3)
+                        assert np.abs(means - act_t[..., None]).min(-1).max() < 2e-4
                 fresh = done[t].astype(bool)
             np.testing.assert_allclose(env.actor_carry.cpu().numpy(), want["actor"], rtol=2e-4, atol=2e-4)
         runs.append(snaps)
