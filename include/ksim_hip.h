@@ -661,6 +661,9 @@ int ks_ppo_loss_grad(ks_stream_t stream, int64_t M, int32_t nu, const KsPpoLossP
 /* ks_ppo_loss_grad for a network with the mean | raw deviation head of ks_sample_action_head (examples/kbot/train.py:
  * 915-932): raw is (M, 2 nu); d_raw (M, 2 nu) receives the gradient with respect to both halves (through the softplus,
  * the scale and the cap of the deviation), which is what the network's backward pass takes. */
+int ks_gaussian_head_log_prob(ks_stream_t stream, int64_t M, int32_t nu, const KsGaussianHead* head /*host*/,
+                              const float* raw /*(M, 2 nu)*/, const float* action, float* log_prob /*(M,nu)*/,
+                              float* entropy /*(M,nu) nullable*/);
 int ks_ppo_loss_grad_head(ks_stream_t stream, int64_t M, int32_t nu, const KsPpoLossParams* params /*host*/,
                           const KsGaussianHead* head /*host*/, const float* raw, const float* action,
                           const float* on_log_probs /*(M,nu)*/, const float* advantages, const float* value_targets,

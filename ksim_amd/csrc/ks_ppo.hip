@@ -519,6 +519,23 @@ __global__ __launch_bounds__(256) void ppo_loss_grad_kernel(int64_t M, int nu, K
   }
 }
 
+// log N(action; mean, std) and the entropy per action for the mean | raw deviation head
+__global__ __launch_bounds__(256) void gaussian_head_log_prob_kernel(int64_t n, int nu, KsGaussianHead hd, const float* __restrict__ raw,
+                                                                    const float* __restrict__ action, float* __restrict__ lp,
+                                                                    float* __restrict__ ent) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= n) return;
+  const int64_t m = idx / nu;
+  const int a = (int)(idx - m * nu);
+  const float mean = raw[m * 2 * nu + a] + (hd.mean_bias ? hd.mean_bias[a] : 0.f);
+  const float r = raw[m * 2 * nu + nu + a];
+  const float sp = r > 20.f ? r : log1pf(expf(r));
+  const float sd = fminf((sp + hd.min_std) * hd.var_scale, hd.max_std);
+  const float z = (action[idx] - mean) / sd, ls = logf(sd);
+  lp[idx] = -0.5f * z * z - ls - kHalfLog2Pi;
+  if (ent) ent[idx] = 0.5f + kHalfLog2Pi + ls;
+}
+
 // The same objective for a network that emits its own deviations: raw (M, 2 nu) = means | raw deviations,
 // std = min((softplus(raw_std) + min_std) * var_scale, max_std).  One thread per row; d_raw receives the gradient of both halves.
 __global__ __launch_bounds__(256) void ppo_loss_grad_head_kernel(int64_t M, int nu, KsPpoLossParams p, KsGaussianHead hd,
@@ -632,4 +649,18 @@ extern "C" int ks_ppo_loss_grad_head(ks_stream_t stream, int64_t M, int32_t nu, 
   hipLaunchKernelGGL(ks::ppo_loss_grad_head_kernel, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, M, nu, *params, *head, raw,
                      action, on_log_probs, advantages, value_targets, on_values, values, d_raw, d_value);
   return ks::check_launch("ks_ppo_loss_grad_head");
+}
+
+extern "C" int ks_gaussian_head_log_prob(ks_stream_t stream, int64_t M, int32_t nu, const KsGaussianHead* head, const float* raw,
+                                         const float* action, float* log_prob, float* entropy) {
+  if (M < 0 || nu < 1) return ks::fail(KS_EINVAL, "ks_gaussian_head_log_prob: bad shape");
+  if (M == 0) return KS_OK;
+  if (!head || !raw || !action || !log_prob) return ks::fail(KS_EINVAL, "ks_gaussian_head_log_prob: null pointer");
+  if (!(head->max_std > 0.f) || head->min_std < 0.f || !(head->var_scale > 0.f))
+    return ks::fail(KS_EINVAL, "ks_gaussian_head_log_prob: bad deviation bounds");
+  const int64_t n = M * nu, grid = (n + 255) / 256;
+  if (grid > 0x7fffffff) return ks::fail(KS_ELIMIT, "ks_gaussian_head_log_prob: too many elements");
+  hipLaunchKernelGGL(ks::gaussian_head_log_prob_kernel, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, n, nu, *head, raw, action,
+                     log_prob, entropy);
+  return ks::check_launch("ks_gaussian_head_log_prob");
 }

@@ -211,3 +211,47 @@ def single_step_recurrent(policy: RecurrentHeadPolicy, cfg: PPOUpdateConfig, act
     policy.critic.adam_step(ap, sq)
     return {"grad_norm": sq.sqrt(), "d_raw": d_raw, "d_value": d_value, "raw": raw, "values": value,
             "advantages": inputs.advantages_bt}
+
+
+def recurrent_on_policy(policy: RecurrentHeadPolicy, actor_obs, critic_obs, action, actor_carry0, critic_carry0, fresh):
+    """Log-probabilities (T, N, nu) and values (T, N) of the recorded actions under the current parameters: the pass that
+    update_model makes once over the whole rollout before any minibatch step (ppo.py:603-607)."""
+    Tn, N, nu = action.shape
+    a_carry, c_carry = actor_carry0.clone(), critic_carry0.clone()
+    raw = torch.empty(Tn, N, 2 * nu, dtype=torch.float32, device=action.device)
+    values = torch.empty(Tn, N, 1, dtype=torch.float32, device=action.device)
+    for t in range(Tn):
+        policy.actor(actor_obs[t], a_carry, fresh=fresh[t], out=raw[t])
+        policy.critic(critic_obs[t], c_carry, fresh=fresh[t], out=values[t])
+    lp = torch.empty(Tn, N, nu, dtype=torch.float32, device=action.device)
+    head = T.KsGaussianHead(float(policy.min_std), float(policy.max_std), float(policy.var_scale), 0, _lib.ptr(policy.mean_bias).value)
+    _lib.check(_lib.load().ks_gaussian_head_log_prob(_lib.current_stream(), Tn * N, nu, ctypes.byref(head), _lib.ptr(raw),
+                                                     _lib.ptr(action.contiguous()), _lib.ptr(lp), None))
+    return lp, values[..., 0]
+
+
+def update_model_recurrent(policy: RecurrentHeadPolicy, cfg: PPOUpdateConfig, actor_obs, critic_obs, action, rewards, done, success,
+                           actor_carry0, critic_carry0, fresh, permutations: list[torch.Tensor] | None = None,
+                           seed: int = 0) -> list[dict]:
+    """num_passes x (N / batch_size) minibatch steps over a (T, N) rollout for a recurrent actor and critic
+    (ppo.py:572-694): a minibatch is a set of env columns together with their carries at the rollout's first step."""
+    Tn, N = done.shape
+    if cfg.adaptive_kl:
+        raise _lib.KsError("adaptive KL is built for the MLP policy update only")
+    on_lp, on_v = recurrent_on_policy(policy, actor_obs, critic_obs, action, actor_carry0, critic_carry0, fresh)
+    bs = min(cfg.batch_size, N)
+    if N % bs:
+        raise _lib.KsError("the env count must be a multiple of the batch size (ppo.py:647 reshapes the permutation)")
+    gen = torch.Generator(device=done.device)
+    gen.manual_seed(seed)
+    env_axis = {True: 2, False: 1}  # carries: (depth, 2, N, H) for LSTM stacks, (depth, N, H) for GRU stacks
+    out = []
+    for k in range(cfg.num_passes):
+        perm = permutations[k] if permutations is not None else torch.randperm(N, generator=gen, device=done.device)
+        for idx in perm.view(-1, bs):
+            sel = lambda t: t.index_select(1, idx).contiguous()  # noqa: E731
+            ca = actor_carry0.index_select(env_axis[actor_carry0.dim() == 4], idx).contiguous()
+            cc = critic_carry0.index_select(env_axis[critic_carry0.dim() == 4], idx).contiguous()
+            out.append(single_step_recurrent(policy, cfg, sel(actor_obs), sel(critic_obs), sel(action), sel(rewards), sel(done),
+                                             sel(success), sel(on_lp), sel(on_v), ca, cc, sel(fresh)))
+    return out

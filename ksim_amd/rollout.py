@@ -106,6 +106,11 @@ class Rollout:
         self.components = torch.zeros(Tn, max(c.terms.n_terms, 1), N, dtype=torch.int8, device=dev)
         self.values = f(Tn, N, 1) if c.critic is not None else None
         self.reset_mask = b(N)
+        # what a recurrent policy update replays the rollout from: the envs that started an episode at each step and the
+        # carries the rollout began with (the model carry of the trajectory's first step, ksim/task/rl.py:117)
+        self.fresh = b(Tn, N) if any(isinstance(n, RecurrentNetwork) for n in (c.actor, c.critic)) else None
+        self.actor_carry0 = c.actor.initial_carry(N, dev) if isinstance(c.actor, RecurrentNetwork) else None
+        self.critic_carry0 = c.critic.initial_carry(N, dev) if isinstance(c.critic, RecurrentNetwork) else None
         self.command = f(Tn, N, c.commands.command_dim) if c.commands is not None else None
         if c.commands is not None and c.commands.command_dim != c.terms.command_dim:
             raise _lib.KsError("the command set and the observation terms disagree about the width of the command vector")
@@ -137,6 +142,13 @@ class Rollout:
                         carry_uniform=noise.get("obs_carry_uniform"))
         # actor reads the noisy copy (walking.py:592-595), critic the clean one (walking.py:626-638); recurrent networks
         # advance their carries, which restart from zero for the envs the previous control step reset
+        if self.fresh is not None:
+            self.fresh[t].copy_(self.reset_mask)
+            if t == 0:
+                if self.actor_carry0 is not None:
+                    self.actor_carry0.copy_(env.actor_carry)
+                if self.critic_carry0 is not None:
+                    self.critic_carry0.copy_(env.critic_carry)
         if isinstance(c.actor, MLP) and isinstance(c.critic, MLP):
             # two plain MLPs over the same rows share one launch
             c.actor.forward_pair(self.noisy_obs[t], self.mean, c.critic, self.obs[t], self.values[t])

@@ -92,6 +92,9 @@ def build(N, T, seed=0, min_height=0.9, events=None, gait=False, recurrent=False
         if head == "gaussian":   # means | raw deviations, deviations squeezed to ~0 so that the sample shows the mean
             from ksim_amd.rollout import GaussianHead
             head = GaussianHead(min_std=0.0, max_std=1e-6, mean_bias=head_bias)
+        elif head == "gaussian-wide":   # deviations a policy update can work with
+            from ksim_amd.rollout import GaussianHead
+            head = GaussianHead(min_std=0.05, max_std=0.5, var_scale=0.5, mean_bias=head_bias)
         elif head == "mixture":
             from ksim_amd.rollout import MixtureHead
             head = MixtureHead(num_mixtures=2, min_std=0.0, max_std=1e-6, mean_bias=head_bias,
@@ -446,3 +449,34 @@ def test_recurrent_actor_and_critic_in_the_rollout(head):
     for it, (a, b) in enumerate(zip(*runs)):
         for x, y, name in zip(a, b, ("action", "values", "actor carry", "critic carry")):
             assert torch.equal(x, y), f"replay {it}: {name} differs from the eager rollout"
+
+
+def test_recurrent_policy_update_from_a_rollout():
+    """A rollout with a GRU actor (deviation head) and a GRU critic, then the recurrent policy update on its buffers: the
+    on-policy pass, replayed from the recorded first-step carries and episode starts, reproduces the values the rollout
+    computed bit for bit; the minibatch steps run through time, move every parameter and keep everything finite."""
+    from ksim_amd import ppo_update as pu
+
+    N, T = 32, 8
+    m, c, rnd_, _, ro, EnvState = build(N, T, seed=17, min_height=0.95, recurrent=True, head="gaussian-wide")
+    ps = c.engine.reset(c.physics_model, 1.0, 3, N, rnd_)
+    env = EnvState(ps, rnd_, torch.zeros(N, 2, device=DEV), None, seed=23)
+    for _ in range(3):  # the third rollout starts from carries that are not zero
+        traj, rew = ro.unroll(env)
+    assert ro.fresh.sum().item() > 0 and ro.actor_carry0.abs().max().item() > 0
+    assert torch.equal(ro.fresh[1:], traj.done[:-1])  # an env starts an episode at the step after it finished
+    policy = pu.RecurrentHeadPolicy(c.actor, c.critic, c.head.min_std, c.head.max_std, c.head.var_scale, c.head.mean_bias)
+    policy.train_init()
+    args = (traj.obs["noisy_obs"], traj.obs["obs"], traj.action, rew.total, traj.done, traj.success, ro.actor_carry0, ro.critic_carry0, ro.fresh)
+    on_lp, on_v = pu.recurrent_on_policy(policy, args[0], args[1], args[2], *args[6:])
+    assert torch.equal(on_v, ro.values[..., 0])
+    assert torch.isfinite(on_lp).all()
+    before = [p.clone() for cell in c.actor.cells for p in cell.parameters().values()]
+    cfg = pu.PPOUpdateConfig(batch_size=16, num_passes=2, learning_rate=1e-3)
+    out = pu.update_model_recurrent(policy, cfg, *args, seed=1)
+    assert len(out) == 4 and all(torch.isfinite(o["grad_norm"]).all() and o["grad_norm"].item() > 0 for o in out)
+    after = [p for cell in c.actor.cells for p in cell.parameters().values()]
+    assert all(torch.isfinite(a).all() and not torch.equal(a, b) for a, b in zip(after, before))
+    # the rollout goes on with the updated networks
+    traj2, _ = ro.unroll(env)
+    assert torch.isfinite(traj2.action).all() and torch.isfinite(ro.values).all()
