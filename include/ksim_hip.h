@@ -474,6 +474,24 @@ int ks_sample_action_head(ks_stream_t stream, int64_t N, int32_t nu, const float
                           KsRng rng, float clip_max, float* action /*(N,nu)*/, float* mean_out /*nullable*/,
                           float* std_out /*nullable*/, float* log_prob_out /*(N,nu) nullable*/);
 
+/* Action filters between the network output and the sampled action (ksim/actions.py:31-257): small per-env recursions on
+ * the target positions, whose state is part of the model carry and restarts with the episode.
+ *   KS_FILTER_LOWPASS               y = y_last + alpha (x - y_last), alpha = dt / (1 / (2 pi p0) + dt)   (actions.py:248-257)
+ *   KS_FILTER_CLIP_ACCELERATION     v = (x - pos) / dt, a = clip((v - vel) / dt, +-p0), vel += a dt, pos += vel dt (54-80)
+ *   KS_FILTER_INTEGRATE_VELOCITY    pos += x dt                                                          (108-133)
+ *   KS_FILTER_INTEGRATE_ACCELERATION vel = clip(vel + x dt, +-p0), pos += vel dt                         (162-191)
+ *   KS_FILTER_CLIP_POSITIONS        y = clip(x, lo, hi)                                                  (194-214)
+ *   KS_FILTER_TANH_POSITIONS        y = tanh(x) (hi - lo) + lo                                           (217-241)
+ * state is (N, 2 nu) = position-like part | velocity-like part (the low-pass keeps y_last in the first half); y is the
+ * filter's output (the new position-like part for the stateful kinds).  Envs flagged in fresh restart from init (N, nu),
+ * or from zero, with zero velocity, before the step is applied. */
+enum { KS_FILTER_LOWPASS = 0, KS_FILTER_CLIP_ACCELERATION = 1, KS_FILTER_INTEGRATE_VELOCITY = 2,
+       KS_FILTER_INTEGRATE_ACCELERATION = 3, KS_FILTER_CLIP_POSITIONS = 4, KS_FILTER_TANH_POSITIONS = 5 };
+int ks_action_filter(ks_stream_t stream, int64_t N, int32_t nu, int32_t kind, float ctrl_dt, float p0,
+                     const float* lo /*(nu) device, range kinds*/, const float* hi, const float* x /*(N,nu)*/,
+                     float* state /*(N, 2 nu) in-out, stateful kinds*/, const uint8_t* fresh /*(N) nullable*/,
+                     const float* init /*(N,nu) nullable*/, float* y /*(N,nu)*/);
+
 /* Mixture-of-Gaussians head of the walking example's actor (examples/walking.py:127-144): raw is (N, 3 nu K) = component
  * means (nu, K), raw deviations (nu, K), logits (nu, K) per env.  mean = clip(raw_mean + mean_bias, clip_lo, clip_hi)
  * (zero bias and ClipPositions, walking.py:138-142), std = min((softplus(raw_std) + min_std) * var_scale, max_std).  Per

@@ -184,6 +184,8 @@ def bind(lib) -> None:
     lib.ks_sample_action_head.argtypes = [c_void_p, c_int64, c_int32, c_void_p, POINTER(KsGaussianHead), c_void_p, KsRng,
                                           c_float, c_void_p, c_void_p, c_void_p, c_void_p]
     lib.ks_sample_action_head.restype = c_int32
+    lib.ks_action_filter.argtypes = [c_void_p, c_int64, c_int32, c_int32, c_float, c_float] + [c_void_p] * 7
+    lib.ks_action_filter.restype = c_int32
     lib.ks_sample_action_mixture.argtypes = [c_void_p, c_int64, c_int32, c_void_p, POINTER(KsMixtureHead), c_void_p, c_void_p,
                                              KsRng, c_float, c_void_p, c_void_p, c_void_p]
     lib.ks_sample_action_mixture.restype = c_int32

@@ -331,6 +331,41 @@ __global__ __launch_bounds__(256) void sample_action_head_kernel(int64_t n, int 
   action[idx] = a;
 }
 
+// Action filters: one lane per (env, joint); the state row of an env is position-like | velocity-like.
+__global__ __launch_bounds__(256) void action_filter_kernel(int64_t n, int nu, int kind, float dt, float p0,
+                                                            const float* __restrict__ lo, const float* __restrict__ hi,
+                                                            const float* __restrict__ x, float* __restrict__ state,
+                                                            const uint8_t* __restrict__ fresh, const float* __restrict__ init,
+                                                            float* __restrict__ y) {
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= n) return;
+  const int64_t e = idx / nu;
+  const int j = (int)(idx - e * nu);
+  const float v = x[idx];
+  if (kind == KS_FILTER_CLIP_POSITIONS) { y[idx] = fminf(fmaxf(v, lo[j]), hi[j]); return; }
+  if (kind == KS_FILTER_TANH_POSITIONS) { y[idx] = tanhf(v) * (hi[j] - lo[j]) + lo[j]; return; }
+  float* st = state + e * 2 * nu;
+  float pos = st[j], vel = st[nu + j];
+  if (fresh && fresh[e]) { pos = init ? init[idx] : 0.f; vel = 0.f; }
+  if (kind == KS_FILTER_LOWPASS) {
+    const float alpha = dt / (1.f / (6.28318530717958647692f * p0) + dt);
+    pos = pos + alpha * (v - pos);
+  } else if (kind == KS_FILTER_CLIP_ACCELERATION) {
+    const float cv = (v - pos) / dt;
+    const float ca = fminf(fmaxf((cv - vel) / dt, -p0), p0);
+    vel = vel + ca * dt;
+    pos = pos + vel * dt;
+  } else if (kind == KS_FILTER_INTEGRATE_VELOCITY) {
+    pos = pos + v * dt;
+  } else {  // KS_FILTER_INTEGRATE_ACCELERATION
+    vel = fminf(fmaxf(vel + v * dt, -p0), p0);
+    pos = pos + vel * dt;
+  }
+  st[j] = pos;
+  st[nu + j] = vel;
+  y[idx] = pos;
+}
+
 // Mixture-of-Gaussians head: one lane per (env, action dimension) walks its K components three times (softmax
 // normaliser, component pick by inverse CDF, log-density of the sample), all in registers.
 __global__ __launch_bounds__(256) void sample_action_mixture_kernel(int64_t n, int nu, const float* __restrict__ raw,
@@ -833,6 +868,26 @@ extern "C" int ks_sample_action_head(ks_stream_t stream, int64_t N, int32_t nu, 
   hipLaunchKernelGGL(sample_action_head_kernel, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, n, (int)nu, raw, *head,
                      noise_normal, rng, clip_max, action, mean_out, std_out, log_prob_out);
   return check_launch("ks_sample_action_head");
+}
+
+extern "C" int ks_action_filter(ks_stream_t stream, int64_t N, int32_t nu, int32_t kind, float ctrl_dt, float p0, const float* lo,
+                                const float* hi, const float* x, float* state, const uint8_t* fresh, const float* init, float* y) {
+  using namespace ks;
+  if (N < 0 || nu < 1) return fail(KS_EINVAL, "ks_action_filter: bad sizes");
+  if (kind < KS_FILTER_LOWPASS || kind > KS_FILTER_TANH_POSITIONS) return fail(KS_EINVAL, "ks_action_filter: unknown kind %d", kind);
+  if (N == 0) return KS_OK;
+  if (!x || !y) return fail(KS_EINVAL, "ks_action_filter: null pointer");
+  const bool ranged = kind == KS_FILTER_CLIP_POSITIONS || kind == KS_FILTER_TANH_POSITIONS;
+  if (ranged && (!lo || !hi)) return fail(KS_EINVAL, "ks_action_filter: the range kinds need lo and hi");
+  if (!ranged && !state) return fail(KS_EINVAL, "ks_action_filter: the stateful kinds need their state");
+  if (!ranged && !(ctrl_dt > 0.f)) return fail(KS_EINVAL, "ks_action_filter: ctrl_dt must be positive");
+  if ((kind == KS_FILTER_LOWPASS || kind == KS_FILTER_CLIP_ACCELERATION || kind == KS_FILTER_INTEGRATE_ACCELERATION) && !(p0 > 0.f))
+    return fail(KS_EINVAL, "ks_action_filter: the cutoff frequency / acceleration / velocity bound must be positive");
+  const int64_t n = N * nu, grid = (n + 255) / 256;
+  if (grid > 0x7fffffff) return fail(KS_ELIMIT, "ks_action_filter: too many elements");
+  hipLaunchKernelGGL(action_filter_kernel, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, n, (int)nu, (int)kind, ctrl_dt, p0, lo,
+                     hi, x, state, fresh, init, y);
+  return check_launch("ks_action_filter");
 }
 
 extern "C" int ks_sample_action_mixture(ks_stream_t stream, int64_t N, int32_t nu, const float* raw, const KsMixtureHead* head,

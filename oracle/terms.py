@@ -459,3 +459,34 @@ def mixture_head(raw, num_mixtures, *, min_std, max_std, var_scale=1.0, mean_bia
     logp = np.logaddexp.reduce(logw - 0.5 * d * d - np.log(std) - 0.5 * np.log(2 * np.pi), axis=-1)
     action = np.clip(np.where(np.isnan(action), 0.0, action), -clip_max, clip_max)
     return action, logp, comp
+
+
+# --------------------------------------------------------------------------- action filters (ksim/actions.py)
+def lowpass_one_pole(x, y_last, ctrl_dt, fc):  # actions.py:248-257
+    alpha = ctrl_dt / (1.0 / (2.0 * np.pi * fc) + ctrl_dt)
+    return np.asarray(y_last, np.float64) + alpha * (np.asarray(x, np.float64) - y_last)
+
+
+def clip_acceleration(target, position, velocity, max_acceleration, ctrl_dt):  # actions.py:54-80: (position, velocity)
+    target, position, velocity = (np.asarray(a, np.float64) for a in (target, position, velocity))
+    cur_v = (target - position) / ctrl_dt
+    acc = np.clip((cur_v - velocity) / ctrl_dt, -max_acceleration, max_acceleration)
+    nv = velocity + acc * ctrl_dt
+    return position + nv * ctrl_dt, nv
+
+
+def integrate_velocity(velocity, position, ctrl_dt):  # actions.py:108-133
+    return np.asarray(position, np.float64) + np.asarray(velocity, np.float64) * ctrl_dt
+
+
+def integrate_acceleration(acceleration, position, velocity, ctrl_dt, max_velocity=10.0):  # actions.py:162-191
+    nv = np.clip(np.asarray(velocity, np.float64) + np.asarray(acceleration, np.float64) * ctrl_dt, -max_velocity, max_velocity)
+    return np.asarray(position, np.float64) + nv * ctrl_dt, nv
+
+
+def clip_positions(x, lo, hi):  # actions.py:211-213
+    return np.clip(np.asarray(x, np.float64), lo, hi)
+
+
+def tanh_positions(x, lo, hi):  # actions.py:234-237 (the image is lo + (hi - lo) tanh x, as written there)
+    return np.tanh(np.asarray(x, np.float64)) * (np.asarray(hi) - np.asarray(lo)) + np.asarray(lo)

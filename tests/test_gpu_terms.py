@@ -6,6 +6,7 @@ import numpy as np
 import pytest
 import torch
 
+from ksim_amd import model as km
 from oracle import terms as ot
 
 pytestmark = pytest.mark.gpu
@@ -668,3 +669,59 @@ def test_mixture_of_gaussians_head():
         sample_action_mixture(t32(raw), 7, **kw)
     with pytest.raises(Exception, match="components"):
         sample_action_mixture(t32(raw[:, :54]), 9, **kw)
+
+
+def test_action_filters_against_oracle():
+    """ks_action_filter through the reference-named wrappers, a few steps each, with episode starts in between."""
+    from ksim_amd import actions as A
+
+    rng = np.random.default_rng(71)
+    N, nu, dt = 50, 20, 0.02
+    fresh = rng.random((6, N)) < 0.2
+    u8 = lambda a: torch.tensor(a, dtype=torch.uint8, device=DEV)  # noqa: E731
+    xs = rng.normal(size=(6, N, nu))
+    init = rng.normal(size=(N, nu)) * 0.1
+    # low-pass
+    p, w = A.LowPassFilterParams.initialize(N, nu), np.zeros((N, nu))
+    for t in range(6):
+        y, p = A.lowpass_one_pole(t32(xs[t]), dt, 3.0, p, fresh=u8(fresh[t]))
+        w = ot.lowpass_one_pole(xs[t], np.where(fresh[t][:, None], 0.0, w), dt, 3.0)
+        np.testing.assert_allclose(y.cpu().numpy(), w, rtol=1e-5, atol=1e-6)
+        np.testing.assert_allclose(p.y_last.cpu().numpy(), w, rtol=1e-5, atol=1e-6)
+    ys, _ = A.lowpass_one_pole_scan(t32(xs), dt, 3.0, A.LowPassFilterParams.initialize(N, nu))
+    w = np.zeros((N, nu))
+    for t in range(6):
+        w = ot.lowpass_one_pole(xs[t], w, dt, 3.0)
+        np.testing.assert_allclose(ys[t].cpu().numpy(), w, rtol=1e-5, atol=1e-6)
+    # acceleration clip, restarting from `init`
+    p = A.ClipAccelerationParams.initialize_from(t32(init))
+    wp, wv = init.copy(), np.zeros((N, nu))
+    for t in range(6):
+        p = A.clip_acceleration(t32(xs[t]), p, 40.0, dt, fresh=u8(fresh[t]), init=t32(init))
+        wp, wv = np.where(fresh[t][:, None], init, wp), np.where(fresh[t][:, None], 0.0, wv)
+        wp, wv = ot.clip_acceleration(xs[t], wp, wv, 40.0, dt)
+        np.testing.assert_allclose(p.position.cpu().numpy(), wp, rtol=1e-4, atol=1e-5)
+        np.testing.assert_allclose(p.velocity.cpu().numpy(), wv, rtol=1e-4, atol=1e-4)
+    # integrators
+    pv, wpv = A.IntegrateVelocityParams.initialize(N, nu), np.zeros((N, nu))
+    pa, wpa, wva = A.IntegrateAccelerationParams.initialize(N, nu), np.zeros((N, nu)), np.zeros((N, nu))
+    for t in range(6):
+        pv = A.integrate_velocity(t32(xs[t]), pv, dt, fresh=u8(fresh[t]))
+        wpv = ot.integrate_velocity(xs[t], np.where(fresh[t][:, None], 0.0, wpv), dt)
+        np.testing.assert_allclose(pv.position.cpu().numpy(), wpv, rtol=1e-5, atol=1e-6)
+        pa = A.integrate_acceleration(t32(xs[t] * 100), pa, dt, max_velocity=3.0, fresh=u8(fresh[t]))
+        wpa, wva = ot.integrate_acceleration(xs[t] * 100, np.where(fresh[t][:, None], 0.0, wpa), np.where(fresh[t][:, None], 0.0, wva), dt, 3.0)
+        np.testing.assert_allclose(pa.position.cpu().numpy(), wpa, rtol=1e-5, atol=1e-5)
+        assert np.abs(pa.velocity.cpu().numpy()).max() <= 3.0 and (np.abs(wva) == 3.0).any()
+    # ranges
+    ranges = [(-1.0 - 0.1 * j, 0.5 + 0.05 * j) for j in range(nu)]
+    lo, hi = np.array(ranges).T
+    np.testing.assert_allclose(A.ClipPositions(ranges).clip(t32(xs[0] * 2)).cpu().numpy(), ot.clip_positions(xs[0] * 2, lo, hi), rtol=1e-6)
+    tp = A.TanhPositions(ranges)
+    np.testing.assert_allclose(tp.clip(t32(xs[0])).cpu().numpy(), ot.tanh_positions(xs[0], lo, hi), rtol=1e-5, atol=1e-6)
+    zeros = t32(np.full((1, nu), 0.1))
+    np.testing.assert_allclose(tp.clip(tp.get_bias(zeros)).cpu().numpy(), 0.1, rtol=1e-4, atol=1e-5)
+    m = km.kbot_scale_model(joint_range=(-0.7, 0.9))
+    assert A.ClipPositions.from_physics_model(m).num_joints == m.nu and A.ClipPositions.from_physics_model(m).max_ranges[0] == 0.9
+    with pytest.raises(Exception, match="kind"):
+        A._run(9, t32(xs[0]))

@@ -344,3 +344,39 @@ def test_mixture_head_against_scipy_and_special_cases():
     _, _, cb = terms.mixture_head(big, K, uniform=rng.random((20000, nu)), normal=np.zeros((20000, nu)), **kw)
     freq = np.stack([(cb == k).mean(0) for k in range(K)], -1)
     assert np.abs(freq - w[0]).max() < 0.015
+
+
+def test_action_filters_closed_forms():
+    """Low-pass: step response x (1 - (1 - alpha)^k) and the -3 dB meaning of alpha; acceleration clip: reaches a reachable
+    target exactly in one step, ramps at the bound otherwise; the integrators against constant-rate kinematics."""
+    dt, fc = 0.02, 3.0
+    alpha = dt / (1 / (2 * np.pi * fc) + dt)
+    y = np.zeros(3)
+    for k in range(1, 30):
+        y = terms.lowpass_one_pole(np.array([1.0, -2.0, 0.5]), y, dt, fc)
+        np.testing.assert_allclose(y, np.array([1.0, -2.0, 0.5]) * (1 - (1 - alpha) ** k), rtol=1e-12)
+    assert alpha == pytest.approx(0.2737, abs=1e-4)  # dt / (RC + dt) with RC = 1 / (2 pi 3 Hz) = 53.05 ms
+    # acceleration clip: from rest, a target 1 mm away needs a = x / dt^2 = 2.5 <= 10 -> reached exactly, at velocity x / dt
+    p, v = terms.clip_acceleration(np.array([0.001]), np.zeros(1), np.zeros(1), 10.0, dt)
+    assert p[0] == pytest.approx(0.001) and v[0] == pytest.approx(0.05)
+    # a far target: constant acceleration at the bound, p_k = a dt^2 k (k + 1) / 2
+    p, v = np.zeros(1), np.zeros(1)
+    for k in range(1, 8):
+        p, v = terms.clip_acceleration(np.array([5.0]), p, v, 10.0, dt)
+        assert v[0] == pytest.approx(10.0 * dt * k) and p[0] == pytest.approx(10.0 * dt * dt * k * (k + 1) / 2)
+    # integrators
+    p = np.array([0.3])
+    for k in range(1, 6):
+        p = terms.integrate_velocity(np.array([2.0]), p, dt)
+        assert p[0] == pytest.approx(0.3 + 2.0 * dt * k)
+    p, v = np.zeros(1), np.zeros(1)
+    for k in range(1, 40):
+        p, v = terms.integrate_acceleration(np.array([20.0]), p, v, dt, max_velocity=5.0)
+        assert v[0] == pytest.approx(min(20.0 * dt * k, 5.0))
+    assert v[0] == 5.0
+    # ranges: clip, and tanh with its inverse bias
+    lo, hi = np.array([-1.0, 0.0]), np.array([2.0, 0.5])
+    np.testing.assert_allclose(terms.clip_positions(np.array([[-3.0, 0.2], [5.0, 0.7]]), lo, hi), [[-1.0, 0.2], [2.0, 0.5]])
+    zeros = np.array([0.5, 0.1])
+    bias = np.arctanh((zeros - lo) / (hi - lo))
+    np.testing.assert_allclose(terms.tanh_positions(bias, lo, hi), zeros, rtol=1e-12)
