@@ -56,10 +56,12 @@ class Trajectory:  # ksim/types.py:46-76
     termination_components: Mapping[str, torch.Tensor] = field(default_factory=dict)
     aux_outputs: Mapping[str, Any] = field(default_factory=dict)
 
-    def episode_length(self) -> torch.Tensor:  # ksim/types.py:72-76: mean over finished steps
-        done = self.done.bool()
-        t = self.timestep
-        return (t * done).sum() / done.sum().clamp(min=1)
+    def episode_length(self) -> torch.Tensor:
+        """Per env, the mean of the recorded timestep over the steps that end an episode, the rollout's last step counted
+        as one (ksim/types.py:72-76); arrays are time-major here, so the reference's last axis is axis 0."""
+        done = self.done.bool().clone()
+        done[-1] = True
+        return (self.timestep * done).sum(dim=0) / done.sum(dim=0)
 
 
 @dataclass

@@ -240,3 +240,52 @@ def test_position_velocity_actuator_widths():
     m = km.kbot_scale_model()
     d, slices, _, _, _ = compile_terms(m, {"a": ob.LastActionObservation(action_dim=2 * m.nu)}, {}, [], action_dim=2 * m.nu)
     assert d.action_dim == 2 * m.nu and d.obs_dim == 2 * m.nu
+
+
+def test_curricula_hand_computed():
+    """ksim/curriculum.py's level updates on small hand-made rollouts (time-major (T, N) arrays)."""
+    import torch
+    from ksim_amd import curriculum as cu
+    from ksim_amd.types import Trajectory
+
+    def traj(done, timestep, qpos=None):
+        return Trajectory(qpos=qpos, qvel=None, xpos=None, xquat=None, ctrl=None, obs={}, command={}, event_state={}, action=None,
+                          done=torch.tensor(done, dtype=torch.uint8), success=None, timestep=torch.tensor(timestep, dtype=torch.float32))
+
+    # episode_length: per env, mean timestep over episode ends, the last step always counted (types.py:72-76)
+    t = traj([[0, 1], [0, 0], [0, 0]], [[0.1, 0.5], [0.2, 0.02], [0.3, 0.04]])
+    assert t.episode_length().tolist() == pytest.approx([0.3, (0.5 + 0.04) / 2])
+    c = cu.ConstantCurriculum(level=0.7)
+    s = c.get_initial_state()
+    assert c(t, None, 5, s).level == 0.7
+    lin = cu.LinearCurriculum(step_size=0.1, step_every_n_epochs=2, min_level=0.05, delay_steps=3)
+    assert lin.get_initial_state().level == 0.05
+    assert [lin(t, None, n, None).level for n in (0, 3, 4, 5, 9, 40)] == pytest.approx([0.05, 0.05, 0.05, 0.1, 0.3, 1.0])
+    # episode length: EMA 0.5 * prev + 0.5 * mean length; a level step when the counter is at zero, then a pause
+    el = cu.EpisodeLengthCurriculum(num_levels=10, increase_threshold=0.2, decrease_threshold=0.1, min_level_steps=2, ema_decay=0.5)
+    s = el.get_initial_state()
+    assert s.level == 0.0 and s.state == (2, 0.0)
+    mean_len = (0.3 + 0.27) / 2
+    s = el(t, None, 0, s); assert s.state == (1, pytest.approx(0.5 * mean_len)) and s.level == 0.0          # counter 2 -> 1
+    s = el(t, None, 1, s); assert s.state[0] == 0 and s.level == 0.0                                          # 1 -> 0
+    s = el(t, None, 2, s)                                                                                      # may step: EMA 0.249 > 0.2
+    assert s.level == pytest.approx(0.1) and s.state[0] == 2 and s.state[1] == pytest.approx(mean_len * (1 - 0.5**3))
+    short = traj([[1, 1], [1, 1], [1, 1]], [[0.02, 0.02]] * 3)
+    for _ in range(6):
+        s = el(short, None, 3, s)
+    assert s.level == pytest.approx(0.0) and s.state[1] < 0.1                                                 # back down, clipped at min_level
+    # distance from origin
+    q = torch.zeros(3, 2, 7); q[2, 1, :3] = torch.tensor([3.0, 4.0, 0.0])
+    dc = cu.DistanceFromOriginCurriculum(num_levels=4, increase_threshold=2.0, decrease_threshold=1.0, min_level_steps=1, ema_decay=0.0)
+    s = dc.get_initial_state()
+    s = dc(traj([[0, 0]] * 3, [[0.0, 0.0]] * 3, q), None, 0, s)
+    assert s.state[1] == pytest.approx(5.0) and s.level == 0.25 and s.state[0] == 1
+    s = dc(traj([[0, 0]] * 3, [[0.0, 0.0]] * 3, q), None, 1, s)
+    assert s.level == 0.5
+    # deaths per env
+    sw = cu.StepWhenSaturated(num_levels=5, increase_threshold=0.6, decrease_threshold=1.5, min_level_steps=1)
+    s = sw.get_initial_state()
+    s = sw(t, None, 0, s); assert s == cu.CurriculumState(0.0, 0)              # waits one call
+    s = sw(t, None, 1, s); assert s.level == pytest.approx(0.2) and s.state == 1   # 0.5 deaths per env < 0.6
+    s = sw(short, None, 2, s); assert s.level == pytest.approx(0.2)              # waits
+    s = sw(short, None, 3, s); assert s.level == pytest.approx(0.0)              # 3 deaths per env > 1.5
