@@ -270,6 +270,16 @@ typedef struct KsStepIO {
      (ArmatureRandomizer, JointDampingRandomizer, ksim/randomization.py:108-123,226-243; the root's six dofs keep 1) */
   const float* armature_scale; /* (N, nv) */
   const float* damping_scale;  /* (N, nv) */
+  /* per-env replacements of model fields (inputs, nullable = the model's own values): dry joint friction
+     (StaticFrictionRandomizer, randomization.py:56-71), centres of mass (COMRandomizer, AllBodiesCOMRandomizer, 290-356),
+     principal inertias (AllBodiesInertiaRandomizer, 359-383, together with mass_scale), and the contact spheres
+     (CollisionBodyRandomizer, 386-487: a jittered capsule is two jittered spheres).  frictionloss selects the kernel
+     variant with dof-lane rows even for a model without dry friction of its own. */
+  const float* frictionloss;   /* (N, nv) */
+  const float* body_ipos;      /* (N, nb*3) */
+  const float* body_inertia;   /* (N, nb*3) */
+  const float* sph_pos;        /* (N, ns*3); with sph_radius */
+  const float* sph_radius;     /* (N, ns) */
   /* launch order (no counterpart in the reference: its vmapped solver runs all envs in lock step).  Envs differ a lot in
      cost (contacts, Newton iterations), and with only a few wavefronts per hardware slot the launch ends with the last heavy
      env.  `work` returns an estimate of each env's cost in this step; ks_work_order turns it into a heaviest-first

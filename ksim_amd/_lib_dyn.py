@@ -42,7 +42,8 @@ STEP_IO_POINTERS = (
     "torque_limit_scale", "action_bias", "torque_bias", "action_noise", "torque_noise", "friction", "mass_scale",
     "env_mask",
     "qacc", "ctrl_out", "xpos", "xquat", "cvel", "traj_ctrl", "traj_xpos", "traj_xquat", "solver_niter", "nefc",
-    "dbg_M", "dbg_bias", "dbg_qacc_smooth", "contact_dist", "cinert", "cfrc_ext", "armature_scale", "damping_scale", "env_order", "work",
+    "dbg_M", "dbg_bias", "dbg_qacc_smooth", "contact_dist", "cinert", "cfrc_ext", "armature_scale", "damping_scale",
+    "frictionloss", "body_ipos", "body_inertia", "sph_pos", "sph_radius", "env_order", "work",
 )
 
 

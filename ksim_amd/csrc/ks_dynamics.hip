@@ -368,8 +368,11 @@ void step_kernel(StepArgs a) {
     const int b_parent = rec.b_parent, b_jtype = rec.b_jtype, b_qadr = rec.b_qadr, b_dofadr = rec.b_dofadr,
               b_depth = rec.b_depth;
     (void)b_parent;
-    const V3 b_pos = {rec.b_pos[0], rec.b_pos[1], rec.b_pos[2]}, b_ipos = {rec.b_ipos[0], rec.b_ipos[1], rec.b_ipos[2]},
-             b_inertia = {rec.b_inertia[0], rec.b_inertia[1], rec.b_inertia[2]},
+    const V3 b_pos = {rec.b_pos[0], rec.b_pos[1], rec.b_pos[2]};
+    V3 b_ipos = {rec.b_ipos[0], rec.b_ipos[1], rec.b_ipos[2]}, b_inertia = {rec.b_inertia[0], rec.b_inertia[1], rec.b_inertia[2]};
+    if (a.body_ipos && is_body) b_ipos = ld3(a.body_ipos + (env * nb + bl) * 3);        // per-env centres of mass
+    if (a.body_inertia && is_body) b_inertia = ld3(a.body_inertia + (env * nb + bl) * 3);  // and principal inertias
+    const V3
              b_jaxis = {rec.b_jaxis[0], rec.b_jaxis[1], rec.b_jaxis[2]}, b_jpos = {rec.b_jpos[0], rec.b_jpos[1], rec.b_jpos[2]};
     const Quat b_quat = {rec.b_quat[0], rec.b_quat[1], rec.b_quat[2], rec.b_quat[3]};
     const Quat b_iquat = {rec.b_iquat[0], rec.b_iquat[1], rec.b_iquat[2], rec.b_iquat[3]};
@@ -380,8 +383,13 @@ void step_kernel(StepArgs a) {
     const float d_armature = rec.d_armature, d_gear = rec.d_gear, d_lo = rec.d_lo, d_hi = rec.d_hi;
     (void)d_armature;
     const int s_body = rec.s_body;
-    const V3 s_pos = {rec.s_pos[0], rec.s_pos[1], rec.s_pos[2]};
-    const float s_rad = rec.s_rad, s_invw = rec.s_invw;
+    V3 s_pos = {rec.s_pos[0], rec.s_pos[1], rec.s_pos[2]};
+    float s_rad = rec.s_rad;
+    const float s_invw = rec.s_invw;
+    if (a.sph_pos && lane < ns) {  // per-env contact spheres
+      s_pos = ld3(a.sph_pos + (env * ns + lane) * 3);
+      s_rad = a.sph_radius[env * ns + lane];
+    }
     const unsigned s_mask = rec.s_mask;
     int pk[kMaxPairs / 64 + 1];
 #pragma unroll
@@ -794,12 +802,12 @@ void step_kernel(StepArgs a) {
             dr.lim_aref = -m.dr_b * dr.lim_s * my_qvel - m.dr_k * imp * pos;
           }
         }
-        dr.fr_fl = rr->d_floss;
+        dr.fr_fl = a.frictionloss ? ((rr->d_jtype == kJntHinge) ? a.frictionloss[env * nv + lane] : 0.f) : rr->d_floss;
         dr.fr_D = rr->d_frD;
         dr.fr_rf = dr.fr_fl / dr.fr_D;
         dr.fr_aref = -m.dr_b * my_qvel;
       }
-      ndr = __popcll(__ballot(dr.lim_s != 0.f)) + m.nfriction;
+      ndr = __popcll(__ballot(dr.lim_s != 0.f)) + __popcll(__ballot(dr.fr_fl > 0.f));
     }
     if (nefc > 0 || (DR && ndr > 0)) {
       // ---- constraint rows: lane r builds row r of J in registers and mirrors it to LDS for column access
@@ -1269,6 +1277,9 @@ extern "C" int ks_model_create(const KsModelDesc* d, KsModel** out) {
     if (!(d->dof_invweight0[d->body_dofadr[b]] > 0.0)) { delete km; return fail(KS_EINVAL, "ks_model_create: body %d: a limited joint needs dof_invweight0 > 0", b); }
     m.dofrows = 1;
   }
+  m.invw_ok = 1;
+  for (int j = 0; j < d->nv; ++j)
+    if (d->body_jtype[d->dof_body[j]] == kJntHinge && !(d->dof_invweight0[j] > 0.0)) m.invw_ok = 0;
   for (int j = 0; j < d->nv; ++j) {
     if (d->dof_frictionloss[j] == 0.0) continue;
     if (!(d->dof_frictionloss[j] > 0.0) || d->body_jtype[d->dof_body[j]] != kJntHinge) { delete km; return fail(KS_EINVAL, "ks_model_create: dof %d: frictionloss must be positive and on a hinge", j); }
@@ -1386,6 +1397,10 @@ static int launch_step(const KsModel* km, ks_stream_t stream, const KsStepIO* io
   a.dbg_M = io->dbg_M; a.dbg_bias = io->dbg_bias; a.dbg_qacc_smooth = io->dbg_qacc_smooth;
   a.contact_dist = io->contact_dist; a.cinert = io->cinert; a.cfrc_ext = io->cfrc_ext;
   a.armature_scale = io->armature_scale; a.damping_scale = io->damping_scale;
+  a.frictionloss = io->frictionloss; a.body_ipos = io->body_ipos; a.body_inertia = io->body_inertia;
+  a.sph_pos = io->sph_pos; a.sph_radius = io->sph_radius;
+  if ((io->sph_pos == nullptr) != (io->sph_radius == nullptr)) return fail(KS_EINVAL, "ks_step: sph_pos and sph_radius come together");
+  if (io->frictionloss && !m.invw_ok) return fail(KS_EINVAL, "ks_step: per-env frictionloss needs dof_invweight0 > 0 on every hinge");
   a.env_order = forward_only ? nullptr : io->env_order; a.work = io->work;
   a.ctrl_in = io->ctrl_in;
   if (!forward_only) {
@@ -1432,7 +1447,7 @@ static int launch_step(const KsModel* km, ks_stream_t stream, const KsStepIO* io
   switch (padded_nv(m.nv)) {
 #define KS_CASE(W)                                                                                       \
   case W:                                                                                                \
-    fn = m.dofrows ? (forward_only ? step_kernel<true, W, true> : step_kernel<false, W, true>)           \
+    fn = (m.dofrows || io->frictionloss) ? (forward_only ? step_kernel<true, W, true> : step_kernel<false, W, true>)           \
                    : (forward_only ? step_kernel<true, W, false> : step_kernel<false, W, false>);        \
     break;
     KS_CASE(8) KS_CASE(16) KS_CASE(24) KS_CASE(28) KS_CASE(32)

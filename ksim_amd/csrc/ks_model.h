@@ -21,7 +21,8 @@ enum { kJntNone = 0, kJntFree = 1, kJntHinge = 2 };
 struct DevModel {
   int nb, nq, nv, nu, ns, iterations, ls_iterations, eulerdamp, npairs, nvs /* row stride of the mass matrix in LDS, a multiple of 4 */, max_depth,
       js /* row stride of the constraint Jacobian in LDS, a multiple of 4 */,
-      dofrows /* 1 when a joint is limited or has dry friction */, nfriction /* dofs with dry friction */;
+      dofrows /* 1 when a joint is limited or has dry friction */, nfriction /* dofs with dry friction */,
+      invw_ok /* 1 when every hinge dof has a positive inverse weight (what rows on the dof lanes are regularised with) */;
   float dt, gravity[3], tolerance, ls_tolerance, meaninertia, friction, impratio;
   // contact impedance constants, already clamped the way the constraint builder wants them
   float con_k, con_b, dmin, dmax, width, mid, power;

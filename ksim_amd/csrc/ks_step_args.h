@@ -24,6 +24,7 @@ struct StepArgs {
   int32_t *solver_niter, *nefc;
   float *dbg_M, *dbg_bias, *dbg_qacc_smooth, *contact_dist, *cinert, *cfrc_ext;
   const float *armature_scale, *damping_scale;
+  const float *frictionloss, *body_ipos, *body_inertia, *sph_pos, *sph_radius;
   const int32_t* env_order;
   int32_t* work;
   int n_events;

@@ -26,6 +26,9 @@ EngineType = Literal["hip"]
 MISSING = None
 
 
+# per-env replacements of model fields that randomisers may produce (ksim/randomization.py), passed to the kernels as they are
+_MODEL_FIELD_OVERRIDES = ("frictionloss", "body_ipos", "body_inertia", "sph_pos", "sph_radius")
+
 @dataclass
 class EngineConfig:  # engine.py:48-139
     action_latency_range: tuple[float, float] = (0.0, 0.0)
@@ -221,6 +224,7 @@ class HipEngine(PhysicsEngine):
         physics.forward(physics_model, dict(qpos=d.qpos, qvel=d.qvel, qacc_warmstart=d.qacc_warmstart, env_mask=mask,
                                             friction=rnd.get("friction"), mass_scale=rnd.get("mass_scale"),
                                             armature_scale=rnd.get("armature_scale"), damping_scale=rnd.get("damping_scale"),
+                                            **{k: rnd.get(k) for k in _MODEL_FIELD_OVERRIDES},
                                             xpos=d.xpos, xquat=d.xquat, cvel=d.cvel, contact_dist=d.contact_dist,
                                             cinert=d.cinert, cfrc_ext=d.cfrc_ext))
         # engine.py:217-220: qvel and qacc are zeroed after the forward pass (qvel is already zero here)
@@ -265,7 +269,7 @@ class HipEngine(PhysicsEngine):
         buf = dict(qpos=d.qpos, qvel=d.qvel, qacc_warmstart=d.qacc_warmstart, time=d.time, last_ctrl=s.last_ctrl,
                    action=action, latency=s.action_latency, zero_offset=s.zero_offset, drop=drop,
                    friction=rnd.get("friction"), mass_scale=rnd.get("mass_scale"), armature_scale=rnd.get("armature_scale"),
-                   damping_scale=rnd.get("damping_scale"), qacc=d.qacc, ctrl_out=d.ctrl,
+                   damping_scale=rnd.get("damping_scale"), **{k: rnd.get(k) for k in _MODEL_FIELD_OVERRIDES}, qacc=d.qacc, ctrl_out=d.ctrl,
                    xpos=d.xpos, xquat=d.xquat, cvel=d.cvel if want_cvel else None, contact_dist=d.contact_dist,
                    cinert=d.cinert if want_cinert else None, cfrc_ext=d.cfrc_ext if want_cfrc_ext else None,
                    action_noise=noise.get("action_noise"),

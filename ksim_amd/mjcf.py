@@ -129,7 +129,7 @@ class _Body:
         self.pos, self.quat = np.zeros(3), np.array([1.0, 0, 0, 0])
         self.joint = None                 # dict or None
         self.parts = []                   # (mass, com, tensor about com) in this body's frame
-        self.spheres = []                 # (pos, radius) in this body's frame
+        self.spheres = []                 # (pos, radius, geom name) in this body's frame
         self.children = []
         self.contact = None               # (friction, solref, solimp) of its collision geoms
 
@@ -218,7 +218,7 @@ def load_mjcf(path: str, **options) -> KinematicModel:
             kind = g.get("type", "sphere")
             size, gp = _vec(g.get("size")), frame(g)[0]
             if kind == "sphere":
-                b.spheres.append((gp, float(size[0])))
+                b.spheres.append((gp, float(size[0]), g.get("name", "")))
             elif kind == "capsule":
                 if g.get("fromto") is not None:
                     ft = _vec(g.get("fromto"), 6)
@@ -226,7 +226,7 @@ def load_mjcf(path: str, **options) -> KinematicModel:
                 else:
                     z = quat_to_mat(frame(g)[1])[:, 2] * size[1]
                     ends = (gp - z, gp + z)
-                b.spheres.extend((e, float(size[0])) for e in ends)
+                b.spheres.extend((e, float(size[0]), g.get("name", "")) for e in ends)
             else:
                 raise ValueError(f"body {b.name!r}: a colliding {kind} is outside the model subset (sphere and capsule only)")
             si = _vec(g.get("solimp"), None, (0.9, 0.95, 0.001, 0.5, 2.0))
@@ -251,7 +251,7 @@ def load_mjcf(path: str, **options) -> KinematicModel:
                 continue
             R = quat_to_mat(c.quat)
             b.parts.extend((m, c.pos + R @ com, R @ I @ R.T) for m, com, I in c.parts)
-            b.spheres.extend((c.pos + R @ p, r) for p, r in c.spheres)
+            b.spheres.extend((c.pos + R @ p, r, n) for p, r, n in c.spheres)
             for g in c.children:  # grandchildren keep their joints; their frame is re-expressed in b
                 g.pos, g.quat = c.pos + R @ g.pos, quat_mul(c.quat, g.quat)
                 kept.append(g)
@@ -299,8 +299,8 @@ def load_mjcf(path: str, **options) -> KinematicModel:
                               iquat=iquat, inertia=inertia, damping=j["damping"], armature=j["armature"], range=j["range"],
                               frictionloss=j["frictionloss"], name=b.name)
         joint_body[j["name"]] = idx
-        for p, r in b.spheres:
-            mb.add_contact_sphere(idx, p, r)
+        for p, r, n in b.spheres:
+            mb.add_contact_sphere(idx, p, r, name=n or None)
         for c in b.children:
             add(c, idx)
 

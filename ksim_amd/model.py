@@ -138,6 +138,7 @@ class KinematicModel:
     dof_invweight0: np.ndarray
     meaninertia: float
     body_names: tuple = field(default=())
+    sph_names: tuple = field(default=())  # collision geom of each contact sphere (both ends of a capsule carry its name)
 
     @property
     def has_free_root(self) -> bool:
@@ -236,8 +237,10 @@ class ModelBuilder:
         self.actuators.append(dict(body=body, gear=float(gear), lo=float(lo), hi=float(hi)))
         return len(self.actuators) - 1
 
-    def add_contact_sphere(self, body: int, pos, radius: float) -> int:
-        self.spheres.append(dict(body=body, pos=np.array(pos, dtype=np.float64), radius=float(radius)))
+    def add_contact_sphere(self, body: int, pos, radius: float, name: str | None = None) -> int:
+        """`name`: the collision geom the sphere comes from; the two end spheres of a capsule share their geom's name."""
+        self.spheres.append(dict(body=body, pos=np.array(pos, dtype=np.float64), radius=float(radius),
+                                 name=name or f"sphere{len(self.spheres)}"))
         return len(self.spheres) - 1
 
     def build(self) -> KinematicModel:
@@ -308,7 +311,7 @@ class ModelBuilder:
             sph_body=np.array([s["body"] for s in self.spheres], np.int32).reshape(ns),
             sph_pos=np.array([s["pos"] for s in self.spheres], np.float64).reshape(ns, 3),
             sph_radius=np.array([s["radius"] for s in self.spheres], np.float64).reshape(ns),
-            body_names=tuple(b["name"] for b in self.bodies),
+            body_names=tuple(b["name"] for b in self.bodies), sph_names=tuple(s["name"] for s in self.spheres),
         )
         inv_b, inv_d, mean_inertia = _compile_constants(partial)
         return KinematicModel(**partial, body_invweight0=inv_b, dof_invweight0=inv_d, meaninertia=mean_inertia)

@@ -55,7 +55,8 @@ class DeviceModel:
 _F32 = ("qpos", "qvel", "qacc_warmstart", "time", "last_ctrl", "action", "ctrl_in", "latency", "zero_offset", "kp",
         "kd", "ctrl_clip", "kp_scale", "kd_scale", "torque_limit_scale", "action_bias", "torque_bias", "action_noise",
         "torque_noise", "friction", "mass_scale", "qacc", "ctrl_out", "xpos", "xquat", "cvel", "dbg_M", "dbg_bias",
-        "dbg_qacc_smooth", "contact_dist", "cinert", "cfrc_ext", "armature_scale", "damping_scale")
+        "dbg_qacc_smooth", "contact_dist", "cinert", "cfrc_ext", "armature_scale", "damping_scale", "frictionloss", "body_ipos",
+        "body_inertia", "sph_pos", "sph_radius")
 _I32 = ("solver_niter", "nefc", "env_order", "work")
 
 
@@ -72,6 +73,7 @@ def _expected_shapes(m: KinematicModel, N: int, S: int, actuator_type: int = _li
         "traj_xpos": (N, nb * 3), "traj_xquat": (N, nb * 4), "solver_niter": (N,), "nefc": (N,),
         "dbg_M": (N, nv * nv), "dbg_bias": (N, nv), "dbg_qacc_smooth": (N, nv), "contact_dist": (N, ns),
         "cinert": (N, nb * 10), "cfrc_ext": (N, nb * 6), "armature_scale": (N, nv), "damping_scale": (N, nv), "env_order": (N,), "work": (N,),
+        "frictionloss": (N, nv), "body_ipos": (N, nb * 3), "body_inertia": (N, nb * 3), "sph_pos": (N, ns * 3), "sph_radius": (N, ns),
     }
 
 

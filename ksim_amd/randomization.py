@@ -1,8 +1,9 @@
 """Per-env physics randomisers with the reference's names (ksim/randomization.py:39-243).
 
 Each returns ``{field: (N, ...) tensor}`` sampled once per env at initialisation (ksim/task/rl.py:2231-2243);
-the step kernel reads ``friction`` (N), ``mass_scale`` (N, nb), ``armature_scale`` and ``damping_scale`` (N, nv)
-every step (rl.py:1182).
+the step kernel reads ``friction`` (N), ``mass_scale`` (N, nb), ``armature_scale``, ``damping_scale`` and
+``frictionloss`` (N, nv), ``body_ipos`` / ``body_inertia`` (N, nb*3), ``sph_pos`` (N, ns*3) and ``sph_radius`` (N, ns) every
+step (rl.py:1182).
 """
 from __future__ import annotations
 
@@ -92,6 +93,98 @@ class MassAdditionRandomizer(PhysicsRandomizer):  # randomization.py:126-163: on
         add = self.scale_lower + (self.scale_upper - self.scale_lower) * torch.rand(num_envs, generator=gen, device=gen.device)
         s[:, self.body_id] = (float(model.body_mass[self.body_id]) + add) / float(model.body_mass[self.body_id])
         return {"mass_scale": s}
+
+
+@dataclass(frozen=True)
+class StaticFrictionRandomizer(PhysicsRandomizer):  # randomization.py:56-71: dof_frictionloss[6:] *= U
+    scale_lower: float = 0.5
+    scale_upper: float = 2.0
+
+    def __call__(self, model, num_envs, gen):
+        base = torch.tensor(model.dof_frictionloss, dtype=torch.float32, device=gen.device)
+        return {"frictionloss": base[None, :] * _joint_scale(model, num_envs, gen, self.scale_lower, self.scale_upper)}
+
+
+def _ipos(model, device):
+    return torch.tensor(model.body_ipos, dtype=torch.float32, device=device)
+
+
+@dataclass(frozen=True)
+class COMRandomizer(PhysicsRandomizer):  # randomization.py:290-333: one body's centre of mass += U(-scale, scale)^3
+    body_id: int = 1
+    scale: float = 0.01
+
+    @classmethod
+    def from_body_name(cls, model, body_name: str, scale: float = 0.01):
+        if body_name not in model.body_names:
+            raise ValueError(f"Body name {body_name} not found in model")
+        return cls(body_id=list(model.body_names).index(body_name), scale=scale)
+
+    def __call__(self, model, num_envs, gen):
+        ipos = _ipos(model, gen.device)[None].repeat(num_envs, 1, 1)
+        ipos[:, self.body_id] += (2 * torch.rand(num_envs, 3, generator=gen, device=gen.device) - 1) * self.scale
+        return {"body_ipos": ipos.reshape(num_envs, -1)}
+
+
+@dataclass(frozen=True)
+class AllBodiesCOMRandomizer(PhysicsRandomizer):  # randomization.py:336-356
+    scale: float = 0.01
+
+    def __call__(self, model, num_envs, gen):
+        off = (2 * torch.rand(num_envs, model.nb, 3, generator=gen, device=gen.device) - 1) * self.scale
+        return {"body_ipos": (_ipos(model, gen.device)[None] + off).reshape(num_envs, -1)}
+
+
+@dataclass(frozen=True)
+class AllBodiesInertiaRandomizer(PhysicsRandomizer):
+    """body_mass *= s, body_inertia *= s * shape with s ~ 1 + U(-scale, scale) per body and shape ~ 1 + U(-scale, scale) per
+    principal axis (randomization.py:359-383; the inverse weights stay as they are, as there)."""
+    scale: float = 0.02
+
+    def __call__(self, model, num_envs, gen):
+        s = 1 + (2 * torch.rand(num_envs, model.nb, generator=gen, device=gen.device) - 1) * self.scale
+        shape = 1 + (2 * torch.rand(num_envs, model.nb, 3, generator=gen, device=gen.device) - 1) * self.scale
+        inertia = torch.tensor(model.body_inertia, dtype=torch.float32, device=gen.device)[None] * s[..., None] * shape
+        return {"mass_scale": s, "body_inertia": inertia.reshape(num_envs, -1)}
+
+
+@dataclass(frozen=True)
+class CollisionBodyRandomizer(PhysicsRandomizer):
+    """Jitters collision capsules (randomization.py:386-487): radius and half-length scaled by 1 + U(-s, s), the centre moved
+    by U(-j, j) per axis.  A capsule is the pair of contact spheres at its ends, `capsules` lists those pairs: the radius
+    scale applies to both spheres, the length scale moves them symmetrically about the centre."""
+    capsules: tuple = ()
+    radius_scale: float = 0.05
+    length_scale: float = 0.05
+    position_jitter_x: float = 0.001
+    position_jitter_y: float = 0.001
+    position_jitter_z: float = 0.001
+
+    @classmethod
+    def from_geom_names(cls, model, geom_names, **kw):
+        pairs = []
+        for name in geom_names:
+            idx = [i for i, n in enumerate(model.sph_names) if n == name]
+            if len(idx) != 2:
+                raise ValueError(f"Geom name '{name}' is not a collision capsule of the model. Available geoms: {sorted(set(model.sph_names))}")
+            pairs.append(tuple(idx))
+        return cls(capsules=tuple(pairs), **kw)
+
+    def __call__(self, model, num_envs, gen):
+        dev = gen.device
+        pos = torch.tensor(model.sph_pos, dtype=torch.float32, device=dev)[None].repeat(num_envs, 1, 1)
+        rad = torch.tensor(model.sph_radius, dtype=torch.float32, device=dev)[None].repeat(num_envs, 1)
+        n = len(self.capsules)
+        u = lambda *shape: 2 * torch.rand(*shape, generator=gen, device=dev) - 1  # noqa: E731
+        rs, ls = 1 + u(num_envs, n) * self.radius_scale, 1 + u(num_envs, n) * self.length_scale
+        jit = u(num_envs, n, 3) * torch.tensor([self.position_jitter_x, self.position_jitter_y, self.position_jitter_z], device=dev)
+        for k, (i, j) in enumerate(self.capsules):
+            centre, half = 0.5 * (pos[:, i] + pos[:, j]), 0.5 * (pos[:, j] - pos[:, i])
+            pos[:, i] = centre + jit[:, k] - half * ls[:, k, None]
+            pos[:, j] = centre + jit[:, k] + half * ls[:, k, None]
+            rad[:, i] *= rs[:, k]
+            rad[:, j] *= rs[:, k]
+        return {"sph_pos": pos.reshape(num_envs, -1), "sph_radius": rad}
 
 
 def get_physics_randomizers(model, randomizers: dict, num_envs: int, gen) -> dict:

@@ -52,7 +52,11 @@ def _data_struct(real):
             ("qpos", real * MAXQ), ("qvel", real * MAXV), ("ctrl", real * MAXU), ("qacc_warmstart", real * MAXV),
             ("time", real),
             ("mass_scale", real * MAXB), ("friction", real), ("armature_scale", real * MAXV),
-            ("damping_scale", real * MAXV), ("xfrc_applied", real * 6 * MAXB),
+            ("damping_scale", real * MAXV),
+            ("has_ipos", c_int), ("has_inertia", c_int), ("has_frictionloss", c_int), ("has_spheres", c_int),
+            ("body_ipos", real * 3 * MAXB), ("body_inertia", real * 3 * MAXB), ("dof_frictionloss", real * MAXV),
+            ("sph_pos", real * 3 * MAXS), ("sph_radius", real * MAXS),
+            ("xfrc_applied", real * 6 * MAXB),
             ("xpos", real * 3 * MAXB), ("xquat", real * 4 * MAXB), ("xmat", real * 9 * MAXB),
             ("xipos", real * 3 * MAXB), ("ximat", real * 9 * MAXB), ("xanchor", real * 3 * MAXB),
             ("xaxis", real * 3 * MAXB), ("com", real * 3),
@@ -162,7 +166,8 @@ class Oracle:
         f.restype = None
         return f
 
-    def data(self, qpos=None, qvel=None, friction=None, mass_scale=None, armature_scale=None, damping_scale=None) -> DataView:
+    def data(self, qpos=None, qvel=None, friction=None, mass_scale=None, armature_scale=None, damping_scale=None,
+             body_ipos=None, body_inertia=None, dof_frictionloss=None, sph_pos=None, sph_radius=None) -> DataView:
         raw = self.Data()
         d = DataView(raw, self.a)
         d.qpos = self.a["qpos0"] if qpos is None else qpos
@@ -176,6 +181,18 @@ class Oracle:
         if damping_scale is not None:
             d.damping_scale = damping_scale
         d.friction = self.a["friction"] if friction is None else friction
+        # per-env replacements of model fields (None: the model's own)
+        nb, nv, ns = self.a["nb"], self.a["nv"], self.a["ns"]
+        for flag, fields in (("has_ipos", (("body_ipos", body_ipos, nb),)), ("has_inertia", (("body_inertia", body_inertia, nb),)),
+                             ("has_frictionloss", (("dof_frictionloss", dof_frictionloss, nv),)),
+                             ("has_spheres", (("sph_pos", sph_pos, ns), ("sph_radius", sph_radius, ns)))):
+            given = [v is not None for _, v, _ in fields]
+            if any(given):
+                if not all(given):
+                    raise ValueError("sph_pos and sph_radius come together")
+                for name, v, n in fields:
+                    np.ctypeslib.as_array(getattr(raw, name))[:n] = np.asarray(v)
+                setattr(raw, flag, 1)
         return d
 
     def call(self, name, d: DataView):

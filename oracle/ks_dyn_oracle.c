@@ -27,6 +27,11 @@ typedef struct FN(KsorData) {
   /* per-env parameters */
   REAL mass_scale[KSOR_MAXB], friction;
   REAL armature_scale[KSOR_MAXV], damping_scale[KSOR_MAXV]; /* ksim/randomization.py:108-123, 226-243 */
+  /* per-env replacements of model fields, used when their flag is set (ksim/randomization.py:56-71 dof_frictionloss,
+   * 290-356 body_ipos, 359-383 body_inertia, 386-487 collision geometry, here the contact spheres) */
+  int has_ipos, has_inertia, has_frictionloss, has_spheres;
+  REAL body_ipos[KSOR_MAXB][3], body_inertia[KSOR_MAXB][3], dof_frictionloss[KSOR_MAXV], sph_pos[KSOR_MAXS][3],
+      sph_radius[KSOR_MAXS];
   /* Cartesian force (3) and torque (3) per body, world frame, acting at the body's centre of mass: MuJoCo's
    * xfrc_applied, which ForcePushEvent writes (ksim/events.py:302-307) */
   REAL xfrc_applied[KSOR_MAXB][6];
@@ -156,6 +161,7 @@ void FN(ksor_kinematics)(const KsorModel* m, Data* d) {
     for (int k = 0; k < 4; ++k) d->xquat[b][k] = quat[k];
     quat2mat(d->xmat[b], quat);
     REAL ipos[3] = {(REAL)m->body_ipos[b][0], (REAL)m->body_ipos[b][1], (REAL)m->body_ipos[b][2]};
+    if (d->has_ipos) for (int k = 0; k < 3; ++k) ipos[k] = d->body_ipos[b][k];
     REAL iquat[4] = {(REAL)m->body_iquat[b][0], (REAL)m->body_iquat[b][1], (REAL)m->body_iquat[b][2], (REAL)m->body_iquat[b][3]};
     REAL v[3], q2[4];
     mat_vec(v, d->xmat[b], ipos);
@@ -180,6 +186,7 @@ void FN(ksor_com_pos)(const KsorModel* m, Data* d) {
     const REAL mass = (REAL)m->body_mass[b] * d->mass_scale[b];
     const REAL* R = d->ximat[b];
     REAL I[3] = {(REAL)m->body_inertia[b][0], (REAL)m->body_inertia[b][1], (REAL)m->body_inertia[b][2]};
+    if (d->has_inertia) for (int k = 0; k < 3; ++k) I[k] = d->body_inertia[b][k];
     REAL dif[3];
     for (int k = 0; k < 3; ++k) dif[k] = d->xipos[b][k] - d->com[k];
     REAL* ci = d->cinert[b];
@@ -391,9 +398,10 @@ void FN(ksor_make_constraint)(const KsorModel* m, Data* d) {
   for (int s = 0; s < m->ns; ++s) {
     const int b = m->sph_body[s];
     REAL lp[3] = {(REAL)m->sph_pos[s][0], (REAL)m->sph_pos[s][1], (REAL)m->sph_pos[s][2]}, c[3];
+    if (d->has_spheres) for (int k = 0; k < 3; ++k) lp[k] = d->sph_pos[s][k];
     mat_vec(c, d->xmat[b], lp);
     for (int k = 0; k < 3; ++k) c[k] += d->xpos[b][k];
-    const REAL r = (REAL)m->sph_radius[s];
+    const REAL r = d->has_spheres ? d->sph_radius[s] : (REAL)m->sph_radius[s];
     const REAL dist = c[2] - r;
     d->con_dist[s] = dist;
     d->con_pos[s][0] = c[0]; d->con_pos[s][1] = c[1]; d->con_pos[s][2] = c[2] - r - dist * (REAL)0.5;
@@ -449,7 +457,7 @@ void FN(ksor_make_constraint)(const KsorModel* m, Data* d) {
   }
   /* dry joint friction: a row J = e_j at pos = 0 whose force saturates at +-frictionloss */
   for (int j = 0; j < nv; ++j) {
-    const REAL fl = (REAL)m->dof_frictionloss[j];
+    const REAL fl = d->has_frictionloss ? d->dof_frictionloss[j] : (REAL)m->dof_frictionloss[j];
     if (!(fl > 0)) continue;
     REAL* row = d->efc_J + nefc * nv;
     for (int i = 0; i < nv; ++i) row[i] = 0;

@@ -563,3 +563,43 @@ def test_model_loaded_from_mjcf_matches_oracle():
         physics.control_step(dm, buf, substeps=1, actuator_type=KS_ACT_TORQUE)
     eq, ev = rel_err(buf["qpos"].cpu().numpy(), wq).max(), rel_err(buf["qvel"].cpu().numpy(), wv).max()
     assert eq <= TEN_STEP_TOL and ev <= TEN_STEP_TOL, f"qpos {eq:.2e} qvel {ev:.2e}"
+
+
+def test_per_env_model_field_overrides_match_oracle():
+    """Per-env centres of mass, principal inertias, dry friction and contact spheres (the remaining physics randomisers)
+    through the step kernel, two control steps of four substeps against the oracle; dry friction given per env to a model
+    that has none of its own selects the kernel variant with dof-lane rows."""
+    from ksim_amd import physics
+    from ksim_amd._lib_dyn import KS_ACT_TORQUE
+
+    for name, m in (("with friction", km.kbot_scale_model(integrator="implicitfast", frictionloss=0.1, joint_range=(-1.0, 1.0))),
+                    ("friction per env only", km.kbot_scale_model(integrator="implicitfast"))):
+        dm = physics.DeviceModel(m)
+        N = 24
+        rng = np.random.default_rng(81)
+        qpos, qvel = random_states(m, N, seed=82, vel_scale=0.3)
+        ipos = m.body_ipos[None] + rng.uniform(-0.01, 0.01, (N,) + m.body_ipos.shape)
+        inertia = m.body_inertia[None] * rng.uniform(0.95, 1.05, (N,) + m.body_inertia.shape)
+        floss = np.concatenate([np.zeros((N, 6)), rng.uniform(0.05, 0.3, (N, m.nv - 6))], axis=1)
+        spos = m.sph_pos[None] + rng.uniform(-0.002, 0.002, (N,) + m.sph_pos.shape)
+        srad = m.sph_radius[None] * rng.uniform(0.95, 1.05, (N, m.ns))
+        ctrl = rng.normal(size=(N, m.nu)) * 3
+        orc = Oracle(m.arrays())
+        wq, wv = [], []
+        for e in range(N):
+            d = orc.data(qpos[e], qvel[e], body_ipos=ipos[e], body_inertia=inertia[e], dof_frictionloss=floss[e], sph_pos=spos[e],
+                         sph_radius=srad[e])
+            d.ctrl = ctrl[e]
+            for _ in range(8):
+                orc.step(d)
+            wq.append(np.array(d.qpos)); wv.append(np.array(d.qvel))
+        buf = dict(qpos=t32(qpos), qvel=t32(qvel), qacc_warmstart=zeros(N, m.nv), time=zeros(N), last_ctrl=t32(ctrl), action=t32(ctrl),
+                   body_ipos=t32(ipos.reshape(N, -1)), body_inertia=t32(inertia.reshape(N, -1)), frictionloss=t32(floss),
+                   sph_pos=t32(spos.reshape(N, -1)), sph_radius=t32(srad), nefc=zeros(N, dtype=torch.int32))
+        for _ in range(2):
+            physics.control_step(dm, buf, substeps=4, actuator_type=KS_ACT_TORQUE)
+        eq, ev = rel_err(buf["qpos"].cpu().numpy(), wq).max(), rel_err(buf["qvel"].cpu().numpy(), wv).max()
+        assert eq <= TEN_STEP_TOL and ev <= TEN_STEP_TOL, f"{name}: qpos {eq:.2e} qvel {ev:.2e}"
+        assert (buf["nefc"] >= m.nv - 6).all()  # a friction row per hinge in every env
+    with pytest.raises(Exception, match="come together"):
+        physics.control_step(dm, dict(buf, sph_radius=None), substeps=1, actuator_type=KS_ACT_TORQUE)

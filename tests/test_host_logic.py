@@ -289,3 +289,47 @@ def test_curricula_hand_computed():
     s = sw(t, None, 1, s); assert s.level == pytest.approx(0.2) and s.state == 1   # 0.5 deaths per env < 0.6
     s = sw(short, None, 2, s); assert s.level == pytest.approx(0.2)              # waits
     s = sw(short, None, 3, s); assert s.level == pytest.approx(0.0)              # 3 deaths per env > 1.5
+
+
+def test_remaining_randomizers_produce_the_kernel_inputs():
+    """Static friction, centre-of-mass, inertia and collision-capsule randomisers (ksim/randomization.py:56-71, 290-487):
+    shapes, ranges, which entries move, and the capsule geometry (both ends share the radius factor, the length factor
+    moves them symmetrically about the jittered centre)."""
+    import os
+    import torch
+    from ksim_amd import randomization as rnd
+    from ksim_amd.mjcf import load_mjcf
+
+    m = load_mjcf(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "mini_biped.mjcf"))
+    gen = torch.Generator(); gen.manual_seed(0)
+    N = 200
+    r = rnd.get_physics_randomizers(m, {"sf": rnd.StaticFrictionRandomizer(0.5, 2.0), "com": rnd.AllBodiesCOMRandomizer(0.01),
+                                        "inertia": rnd.AllBodiesInertiaRandomizer(0.02),
+                                        "feet": rnd.CollisionBodyRandomizer.from_geom_names(m, ["foot_l", "foot_r"], radius_scale=0.1,
+                                                                                            length_scale=0.2, position_jitter_x=0.003,
+                                                                                            position_jitter_y=0.0, position_jitter_z=0.001)}, N, gen)
+    fl = r["frictionloss"].numpy()
+    assert fl.shape == (N, m.nv) and (fl[:, :6] == 0).all()
+    ratio = fl[:, 6:] / m.dof_frictionloss[6:]
+    assert ratio.min() >= 0.5 and ratio.max() <= 2.0 and ratio.std() > 0.3
+    ip = r["body_ipos"].numpy().reshape(N, m.nb, 3) - m.body_ipos
+    assert np.abs(ip).max() <= 0.01 + 1e-7 and np.abs(ip).mean() > 0.003
+    s = r["mass_scale"].numpy()
+    inert = r["body_inertia"].numpy().reshape(N, m.nb, 3) / np.where(m.body_inertia > 0, m.body_inertia, 1.0)
+    assert np.abs(s - 1).max() <= 0.02 + 1e-6
+    shape = inert[:, 1:] / s[:, 1:, None]
+    assert np.abs(shape - 1).max() <= 0.02 + 1e-5 and shape.std() > 0.005
+    pos, rad = r["sph_pos"].numpy().reshape(N, m.ns, 3), r["sph_radius"].numpy()
+    i, j = [k for k, n in enumerate(m.sph_names) if n == "foot_l"]
+    assert np.allclose(rad[:, i], rad[:, j]) and np.abs(rad[:, i] / 0.02 - 1).max() <= 0.1 + 1e-6
+    centre, half = 0.5 * (pos[:, i] + pos[:, j]), 0.5 * (pos[:, j] - pos[:, i])
+    c0, h0 = 0.5 * (m.sph_pos[i] + m.sph_pos[j]), 0.5 * (m.sph_pos[j] - m.sph_pos[i])
+    jit = centre - c0
+    assert np.abs(jit[:, 0]).max() <= 0.003 + 1e-6 and np.abs(jit[:, 1]).max() < 1e-6 and np.abs(jit[:, 2]).max() <= 0.001 + 1e-6
+    scale = np.linalg.norm(half, axis=1) / np.linalg.norm(h0)
+    assert np.abs(scale - 1).max() <= 0.2 + 1e-5 and scale.std() > 0.05
+    assert np.allclose(np.cross(half, h0[None]), 0, atol=1e-7)  # the capsule keeps its axis
+    com1 = rnd.COMRandomizer.from_body_name(m, "knee_l", scale=0.02)(m, N, gen)["body_ipos"].numpy().reshape(N, m.nb, 3) - m.body_ipos
+    assert np.abs(com1[:, 3]).max() > 0.01 and np.abs(np.delete(com1, 3, axis=1)).max() < 1e-7
+    with pytest.raises(ValueError, match="not a collision capsule"):
+        rnd.CollisionBodyRandomizer.from_geom_names(m, ["nope"])

@@ -544,3 +544,31 @@ def test_dry_friction_closed_forms():
     # above it the joint accelerates with the excess
     d4 = orc.data(np.zeros(1), np.zeros(1)); d4.ctrl = np.array([1.0]); orc.forward(d4)
     assert d4.qacc[0] == pytest.approx((1.0 - f) / inertia, rel=1e-8)
+
+
+def test_per_env_model_field_overrides_equal_a_model_built_with_them():
+    """Per-env replacements of body_ipos, body_inertia, dof_frictionloss and the contact spheres (what the COM, inertia,
+    static-friction and collision-body randomisers produce) give exactly what a model carrying those values gives."""
+    base = km.kbot_scale_model(frictionloss=0.1, joint_range=(-1.0, 1.0))
+    rng = np.random.default_rng(20)
+    ipos = base.body_ipos + rng.uniform(-0.01, 0.01, base.body_ipos.shape)
+    inertia = base.body_inertia * rng.uniform(0.95, 1.05, base.body_inertia.shape)
+    floss = base.dof_frictionloss * rng.uniform(0.5, 2.0, base.nv)
+    spos = base.sph_pos + rng.uniform(-0.002, 0.002, base.sph_pos.shape)
+    srad = base.sph_radius * rng.uniform(0.95, 1.05, base.ns)
+    a2 = dict(base.arrays()); a2.update(body_ipos=ipos, body_inertia=inertia, dof_frictionloss=floss, sph_pos=spos, sph_radius=srad)
+    qpos, qvel = _random_state(base, rng, vel_scale=0.5)
+    qpos = _sink_to_contact(base, qpos)
+    ctrl = rng.normal(size=base.nu)
+    o1, o2 = Oracle(base.arrays()), Oracle(a2)
+    d1 = o1.data(qpos, qvel, body_ipos=ipos, body_inertia=inertia, dof_frictionloss=floss, sph_pos=spos, sph_radius=srad)
+    d2 = o2.data(qpos, qvel)
+    d0 = o1.data(qpos, qvel)
+    for d, o in ((d1, o1), (d2, o2), (d0, o1)):
+        d.ctrl = ctrl
+        for _ in range(3):
+            o.step(d)
+    assert np.array_equal(d1.qpos, d2.qpos) and np.array_equal(d1.qvel, d2.qvel) and d1.nefc == d2.nefc
+    assert not np.allclose(d1.qvel, d0.qvel, rtol=1e-6)  # and they do change the motion
+    with pytest.raises(ValueError):
+        o1.data(qpos, qvel, sph_pos=spos)
