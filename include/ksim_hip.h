@@ -328,10 +328,18 @@ enum { /* KsObsElem.kind */
                            column carry[carry + d * stride], d = 0..comp-1, oldest first; it emits slot 0 (minus
                            zero_offset when src is qpos), shifts the column down and appends src[index].  A fresh
                            episode fills the column with the current value. */
-  KS_OBS_GRAVITY_EMA = 5 /* component `comp` of the lagged, biased gravity reading (observation.py:355-442):
+  KS_OBS_GRAVITY_EMA = 5, /* component `comp` of the lagged, biased gravity reading (observation.py:355-442):
                            p = R(euler bias) (q^-1 (c0,c1,c2) q), x <- x lag + p (1 - lag), emits x.
                            carry[carry .. carry+6] = x(3), lag, bias(3); a fresh episode sets x = 0,
                            lag ~ U(q0, q1), bias ~ U(-q2, q2)^3 from four draws. */
+  KS_OBS_SITE_GYRO = 6,  /* component `comp` of a gyro at a site of body `index` (MuJoCo's gyro sensor, which
+                           SensorObservation reads from sensordata, observation.py:307-340): the body's angular velocity in
+                           the site frame, (q_body q_site)^-1 w, with q_body = xquat[index], w = cvel[index][0:3] (both of
+                           the last substep's forward pass, as sensordata is) and q_site = (e0, e1, e2, e3) */
+  KS_OBS_SITE_ACCEL = 7  /* component `comp` of an accelerometer at a site of the floating base (body `index`, the one the
+                           free joint moves): the site's acceleration minus gravity in the site frame,
+                           (q_body q_site)^-1 (qacc[0:3] + alpha x r + w x (w x r) - g), alpha = R_body qacc[3:6],
+                           r = R_body (c0, c1, c2), g = (q0, q1, q2), q_site = (e0, e1, e2, e3) */
 };
 enum { KS_NOISE_NONE = 0, KS_NOISE_ADD_GAUSSIAN = 1, KS_NOISE_ADD_UNIFORM = 2, KS_NOISE_MUL_GAUSSIAN = 3,
        KS_NOISE_MUL_UNIFORM = 4 }; /* ksim/noise.py:184-213 */
@@ -341,7 +349,8 @@ typedef struct KsObsElem {
   int32_t noise_kind;
   float noise_mean, noise_scale; /* std or mag, multiplied by the curriculum level (noise.py:86,102) */
   int32_t carry, stride;         /* stateful kinds: offset into the env's carry row, distance between delay slots */
-  float q0, q1, q2;              /* KS_OBS_GRAVITY_EMA: min_lag, max_lag, imu_bias */
+  float q0, q1, q2;              /* KS_OBS_GRAVITY_EMA: min_lag, max_lag, imu_bias; KS_OBS_SITE_ACCEL: gravity */
+  float e0, e1, e2, e3;          /* site kinds: the site's orientation in its body, wxyz */
 } KsObsElem;
 
 /* Terminations (replaces get_terminations + terms, rl.py:288-299, ksim/terminations.py:60-192). */

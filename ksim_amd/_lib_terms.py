@@ -7,7 +7,7 @@ from ctypes import POINTER, c_float, c_int8, c_int32, c_int64, c_uint8, c_uint64
 KS_MAX_OBS, KS_MAX_TERMS, KS_MAX_QPOS, KS_MAX_LAYERS = 512, 16, 40, 8
 (SRC_QPOS, SRC_QVEL, SRC_QACC, SRC_CTRL, SRC_LAST_ACTION, SRC_COMMAND, SRC_TIME, SRC_XPOS, SRC_XQUAT, SRC_CVEL,
  SRC_CONST, SRC_CONTACT_DIST, SRC_CINERT, SRC_CFRC_EXT, SRC_COUNT) = range(15)
-OBS_COPY, OBS_JOINT_POS, OBS_ROT_INV, OBS_CONTACT, OBS_DELAYED, OBS_GRAVITY_EMA = range(6)
+OBS_COPY, OBS_JOINT_POS, OBS_ROT_INV, OBS_CONTACT, OBS_DELAYED, OBS_GRAVITY_EMA, OBS_SITE_GYRO, OBS_SITE_ACCEL = range(8)
 NOISE_NONE, NOISE_ADD_GAUSSIAN, NOISE_ADD_UNIFORM, NOISE_MUL_GAUSSIAN, NOISE_MUL_UNIFORM = range(5)
 (TERM_MIN_HEIGHT, TERM_BAD_Z, TERM_NOT_UPRIGHT, TERM_BAD_VELOCITY, TERM_FAR_FROM_ORIGIN,
  TERM_EPISODE_LENGTH, TERM_ILLEGAL_CONTACT) = range(7)
@@ -19,7 +19,7 @@ class KsObsElem(ctypes.Structure):
     _fields_ = [("kind", c_int32), ("src", c_int32), ("index", c_int32), ("comp", c_int32), ("c0", c_float),
                 ("c1", c_float), ("c2", c_float), ("noise_kind", c_int32), ("noise_mean", c_float),
                 ("noise_scale", c_float), ("carry", c_int32), ("stride", c_int32), ("q0", c_float), ("q1", c_float),
-                ("q2", c_float)]
+                ("q2", c_float), ("e0", c_float), ("e1", c_float), ("e2", c_float), ("e3", c_float)]
 
 
 class KsTermDesc(ctypes.Structure):

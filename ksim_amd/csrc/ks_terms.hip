@@ -98,6 +98,27 @@ __global__ __launch_bounds__(256) void observe_kernel(ObserveArgs a) {
     x = x * lag + p[el.comp] * (1.f - lag);
     c[el.comp] = x;
     v = x;
+  } else if (el.kind == KS_OBS_SITE_GYRO || el.kind == KS_OBS_SITE_ACCEL) {
+    const float* qb = a.src[KS_SRC_XQUAT] + e * a.src_dim[KS_SRC_XQUAT] + 4 * el.index;
+    const float* w = a.src[KS_SRC_CVEL] + e * a.src_dim[KS_SRC_CVEL] + 6 * el.index;  // angular velocity, world axes
+    float vec[3] = {w[0], w[1], w[2]};
+    if (el.kind == KS_OBS_SITE_ACCEL) {
+      const float* qa = a.src[KS_SRC_QACC] + e * a.src_dim[KS_SRC_QACC];
+      float r[3], al[3];
+      const float al_l[3] = {qa[3], qa[4], qa[5]}, r_l[3] = {el.c0, el.c1, el.c2};
+      rot_fwd(qb, r_l, r);
+      rot_fwd(qb, al_l, al);
+      // w x r, then alpha x r + w x (w x r)
+      const float wr[3] = {w[1] * r[2] - w[2] * r[1], w[2] * r[0] - w[0] * r[2], w[0] * r[1] - w[1] * r[0]};
+      vec[0] = qa[0] + (al[1] * r[2] - al[2] * r[1]) + (w[1] * wr[2] - w[2] * wr[1]) - el.q0;
+      vec[1] = qa[1] + (al[2] * r[0] - al[0] * r[2]) + (w[2] * wr[0] - w[0] * wr[2]) - el.q1;
+      vec[2] = qa[2] + (al[0] * r[1] - al[1] * r[0]) + (w[0] * wr[1] - w[1] * wr[0]) - el.q2;
+    }
+    float in_body[3], out[3];
+    const float qs[4] = {el.e0, el.e1, el.e2, el.e3};
+    rot_inv(qb, vec[0], vec[1], vec[2], in_body);
+    rot_inv(qs, in_body[0], in_body[1], in_body[2], out);
+    v = out[el.comp];
   } else {
     float vec[3] = {el.c0, el.c1, el.c2}, out[3];
     if (el.src != KS_SRC_CONST) {
@@ -737,7 +758,13 @@ extern "C" int ks_terms_create(const KsTermsDesc* d, KsTerms** out) {
   for (int k = 0; k < d->obs_dim; ++k) {
     const KsObsElem& el = d->obs[k];
     if (el.src < 0 || el.src >= KS_SRC_COUNT) return fail(KS_EINVAL, "ks_terms_create: obs %d: bad source %d", k, el.src);
-    if (el.kind < KS_OBS_COPY || el.kind > KS_OBS_GRAVITY_EMA) return fail(KS_EINVAL, "ks_terms_create: obs %d: bad kind", k);
+    if (el.kind < KS_OBS_COPY || el.kind > KS_OBS_SITE_ACCEL) return fail(KS_EINVAL, "ks_terms_create: obs %d: bad kind", k);
+    if (el.kind == KS_OBS_SITE_GYRO || el.kind == KS_OBS_SITE_ACCEL) {
+      if (el.comp < 0 || el.comp > 2 || el.index < 0 || el.index >= d->nb) return fail(KS_EINVAL, "ks_terms_create: obs %d: bad site sensor (component %d, body %d)", k, el.comp, el.index);
+      if (!(el.e0 * el.e0 + el.e1 * el.e1 + el.e2 * el.e2 + el.e3 * el.e3 > 0.f)) return fail(KS_EINVAL, "ks_terms_create: obs %d: the site orientation is not a quaternion", k);
+      if (el.kind == KS_OBS_SITE_ACCEL && d->nv < 6) return fail(KS_EINVAL, "ks_terms_create: obs %d: an accelerometer needs a floating base", k);
+      continue;
+    }
     if (el.kind == KS_OBS_DELAYED) {
       if (el.comp < 1 || el.stride < 1 || el.carry < 0 || el.carry + (el.comp - 1) * el.stride >= d->carry_dim)
         return fail(KS_EINVAL, "ks_terms_create: obs %d: delay buffer outside the carry row", k);
@@ -796,6 +823,11 @@ extern "C" int ks_observe(const KsTerms* t, ks_stream_t stream, const KsObserveI
   bool needs_quat = false, needs_noise = false;
   for (int k = 0; k < d.obs_dim; ++k) {
     const KsObsElem& el = d.obs[k];
+    if (el.kind == KS_OBS_SITE_GYRO || el.kind == KS_OBS_SITE_ACCEL) {
+      if (!io->src[KS_SRC_XQUAT] || !io->src[KS_SRC_CVEL] || (el.kind == KS_OBS_SITE_ACCEL && !io->src[KS_SRC_QACC]))
+        return fail(KS_EINVAL, "ks_observe: observation %d (site sensor) needs xquat, cvel and, for an accelerometer, qacc", k);
+      continue;
+    }
     if (el.src != KS_SRC_CONST && !io->src[el.src]) return fail(KS_EINVAL, "ks_observe: observation %d reads source %d, which is NULL", k, el.src);
     needs_quat |= el.kind == KS_OBS_ROT_INV || el.kind == KS_OBS_GRAVITY_EMA;
     needs_noise |= el.noise_kind != KS_NOISE_NONE;

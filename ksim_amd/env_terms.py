@@ -54,9 +54,12 @@ def compile_terms(model: KinematicModel, observations: Mapping[str, Observation]
             e.c0, e.c1, e.c2 = el.const
             e.carry, e.stride = carry_at + el.carry, el.stride
             e.q0, e.q1, e.q2 = el.q
+            e.e0, e.e1, e.e2, e.e3 = el.e
             sources_used.add(el.src)
             if el.kind == T.OBS_GRAVITY_EMA:
                 sources_used.add(T.SRC_QPOS)
+            if el.kind in (T.OBS_SITE_GYRO, T.OBS_SITE_ACCEL):
+                sources_used.update((T.SRC_XQUAT, T.SRC_CVEL) + ((T.SRC_QACC,) if el.kind == T.OBS_SITE_ACCEL else ()))
             if noise is not None:
                 e.noise_kind, e.noise_mean, e.noise_scale = noise.kind, noise.mean, noise.scale
             bias_std.append(0.0 if obs.bias is None else float(obs.bias))

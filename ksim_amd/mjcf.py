@@ -130,6 +130,7 @@ class _Body:
         self.joint = None                 # dict or None
         self.parts = []                   # (mass, com, tensor about com) in this body's frame
         self.spheres = []                 # (pos, radius, geom name) in this body's frame
+        self.sites = []                   # (name, pos, quat) in this body's frame
         self.children = []
         self.contact = None               # (friction, solref, solimp) of its collision geoms
 
@@ -233,6 +234,10 @@ def load_mjcf(path: str, **options) -> KinematicModel:
             si = np.concatenate([si, np.array([0.9, 0.95, 0.001, 0.5, 2.0])[si.size:]])
             contact_params.append((float(_vec(g.get("friction"), None, (1.0, 0.005, 0.0001))[0]),
                                    tuple(_vec(g.get("solref"), 2, (0.02, 1.0))), tuple(si)))
+        for st in (e for e in elem if e.tag == "site"):
+            sa = defaults.resolve(st, childclass)
+            sp, sq = frame(sa)
+            b.sites.append((sa.get("name", ""), sp, sq / np.linalg.norm(sq)))
         b.children = [read_body(c, childclass) for c in elem if c.tag == "body"]
         return b
 
@@ -252,6 +257,7 @@ def load_mjcf(path: str, **options) -> KinematicModel:
             R = quat_to_mat(c.quat)
             b.parts.extend((m, c.pos + R @ com, R @ I @ R.T) for m, com, I in c.parts)
             b.spheres.extend((c.pos + R @ p, r, n) for p, r, n in c.spheres)
+            b.sites.extend((n, c.pos + R @ p, quat_mul(c.quat, q)) for n, p, q in c.sites)
             for g in c.children:  # grandchildren keep their joints; their frame is re-expressed in b
                 g.pos, g.quat = c.pos + R @ g.pos, quat_mul(c.quat, g.quat)
                 kept.append(g)
@@ -301,6 +307,8 @@ def load_mjcf(path: str, **options) -> KinematicModel:
         joint_body[j["name"]] = idx
         for p, r, n in b.spheres:
             mb.add_contact_sphere(idx, p, r, name=n or None)
+        for n, p, q in b.sites:
+            mb.add_site(n, idx, p, q)
         for c in b.children:
             add(c, idx)
 
@@ -316,4 +324,9 @@ def load_mjcf(path: str, **options) -> KinematicModel:
         limited = at.get("ctrllimited", "auto")
         mb.add_actuator(joint_body[at["joint"]], gear=float(_vec(at.get("gear"), None, (1.0,))[0]),
                         ctrlrange=None if (cr is None or limited == "false") else tuple(cr))
+    sens = root.find("sensor")
+    for se in ([] if sens is None else sens):  # sensors that refer to a site; others (joint, actuator sensors) are not read
+        site = se.get("site") or (se.get("objname") if se.get("objtype") == "site" else None)
+        if site in mb.sites and se.get("name"):
+            mb.add_sensor(se.get("name"), se.tag, site)
     return mb.build()

@@ -139,6 +139,8 @@ class KinematicModel:
     meaninertia: float
     body_names: tuple = field(default=())
     sph_names: tuple = field(default=())  # collision geom of each contact sphere (both ends of a capsule carry its name)
+    sites: dict = field(default_factory=dict)    # name -> (body, position (3), orientation wxyz (4)) in the body frame
+    sensors: dict = field(default_factory=dict)  # name -> (MuJoCo sensor type, site name)
 
     @property
     def has_free_root(self) -> bool:
@@ -184,6 +186,8 @@ class ModelBuilder:
                             range=None, frictionloss=0.0, name="world")]
         self.actuators: list[dict] = []
         self.spheres: list[dict] = []
+        self.sites: dict = {}
+        self.sensors: dict = {}
 
     def add_body(self, parent: int, pos, *, joint: str | None = "hinge", axis=(0.0, 1.0, 0.0),
                  joint_pos=(0.0, 0.0, 0.0), quat=(1.0, 0.0, 0.0, 0.0), mass: float, ipos=(0.0, 0.0, 0.0),
@@ -242,6 +246,15 @@ class ModelBuilder:
         self.spheres.append(dict(body=body, pos=np.array(pos, dtype=np.float64), radius=float(radius),
                                  name=name or f"sphere{len(self.spheres)}"))
         return len(self.spheres) - 1
+
+    def add_site(self, name: str, body: int, pos=(0.0, 0.0, 0.0), quat=(1.0, 0.0, 0.0, 0.0)) -> None:
+        q = np.array(quat, dtype=np.float64)
+        self.sites[name] = (int(body), tuple(float(v) for v in pos), tuple(q / np.linalg.norm(q)))
+
+    def add_sensor(self, name: str, kind: str, site: str) -> None:
+        if site not in self.sites:
+            raise ValueError(f"sensor {name!r} refers to the unknown site {site!r}")
+        self.sensors[name] = (kind, site)
 
     def build(self) -> KinematicModel:
         nb = len(self.bodies)
@@ -314,7 +327,8 @@ class ModelBuilder:
             body_names=tuple(b["name"] for b in self.bodies), sph_names=tuple(s["name"] for s in self.spheres),
         )
         inv_b, inv_d, mean_inertia = _compile_constants(partial)
-        return KinematicModel(**partial, body_invweight0=inv_b, dof_invweight0=inv_d, meaninertia=mean_inertia)
+        return KinematicModel(**partial, body_invweight0=inv_b, dof_invweight0=inv_d, meaninertia=mean_inertia,
+                              sites=dict(self.sites), sensors=dict(self.sensors))
 
 
 # --------------------------------------------------------------------------- host kinematics (float64, init-time only)

@@ -25,6 +25,7 @@ class ObsElem:
     carry: int = 0      # offset inside the observation's own carry block
     stride: int = 0
     q: tuple = (0.0, 0.0, 0.0)
+    e: tuple = (1.0, 0.0, 0.0, 0.0)  # site kinds: the site's orientation in its body
 
 
 @dataclass(frozen=True)
@@ -316,3 +317,37 @@ class CommandObservation(Observation):
 
     def elements(self, m, command_dim):
         return _copy(T.SRC_COMMAND, 0, command_dim)
+
+
+@dataclass(frozen=True)
+class SensorObservation(Observation):
+    """A sensor of the model by name (observation.py:307-340 reads its slice of `sensordata`).  Built sensor types:
+    `gyro` (angular velocity in the site frame), `accelerometer` (acceleration minus gravity in the site frame; the site
+    must sit on the floating base, where an IMU does) and `touch` (the normal contact force on the site's body: every
+    contact sphere of that body is taken to lie inside the site's volume, which holds for the feet of the shipped robots).
+    Like `sensordata`, they describe the state the last substep started from."""
+    sensor_name: str = ""
+
+    @classmethod
+    def create(cls, *, physics_model: KinematicModel, sensor_name: str, noise=None):
+        if sensor_name not in physics_model.sensors:
+            options = "\n".join(sorted(physics_model.sensors))
+            raise ValueError(f"{sensor_name} not found in model. Available:\n{options}")
+        kind = physics_model.sensors[sensor_name][0]
+        if kind not in ("gyro", "accelerometer", "touch"):
+            raise ValueError(f"sensor {sensor_name!r} of type {kind} is not built (gyro, accelerometer, touch are)")
+        return cls(sensor_name=sensor_name, noise=noise)
+
+    def elements(self, m, command_dim):
+        kind, site = m.sensors[self.sensor_name]
+        body, pos, quat = m.sites[site]
+        if kind == "touch":
+            return [ObsElem(T.OBS_COPY, T.SRC_CFRC_EXT, 6 * body + 5)]
+        if kind == "gyro":
+            return [ObsElem(T.OBS_SITE_GYRO, T.SRC_CVEL, body, c, e=tuple(quat)) for c in range(3)]
+        if body != 1 or not m.has_free_root:
+            raise ValueError(f"accelerometer {self.sensor_name!r}: its site must sit on the floating base")
+        return [ObsElem(T.OBS_SITE_ACCEL, T.SRC_CVEL, body, c, const=tuple(pos), q=tuple(m.gravity), e=tuple(quat)) for c in range(3)]
+
+    def get_name(self) -> str:
+        return self.sensor_name

@@ -490,3 +490,22 @@ def clip_positions(x, lo, hi):  # actions.py:211-213
 
 def tanh_positions(x, lo, hi):  # actions.py:234-237 (the image is lo + (hi - lo) tanh x, as written there)
     return np.tanh(np.asarray(x, np.float64)) * (np.asarray(hi) - np.asarray(lo)) + np.asarray(lo)
+
+
+# --------------------------------------------------------------------------- site sensors (MuJoCo gyro / accelerometer)
+def site_gyro(xquat_body, omega_world, site_quat):
+    """MuJoCo's gyro: the body's angular velocity in the site frame, (q_body q_site)^-1 w (what SensorObservation reads
+    from sensordata, ksim/observation.py:307-340)."""
+    in_body = rotate_vector_by_quat(np.asarray(omega_world, np.float64), np.asarray(xquat_body, np.float64), inverse=True)
+    return rotate_vector_by_quat(in_body, np.asarray(site_quat, np.float64), inverse=True)
+
+
+def site_accelerometer(qacc6, xquat_body, omega_world, site_pos, site_quat, gravity):
+    """MuJoCo's accelerometer for a site on the floating base: the site's acceleration minus gravity, in the site frame.
+    qacc6 = the free joint's accelerations (origin acceleration in world axes, angular acceleration in body axes)."""
+    qacc6, q = np.asarray(qacc6, np.float64), np.asarray(xquat_body, np.float64)
+    w = np.asarray(omega_world, np.float64)
+    r = rotate_vector_by_quat(np.asarray(site_pos, np.float64), q)
+    alpha = rotate_vector_by_quat(qacc6[..., 3:6], q)
+    a = qacc6[..., :3] + np.cross(alpha, r) + np.cross(w, np.cross(w, r)) - np.asarray(gravity, np.float64)
+    return rotate_vector_by_quat(rotate_vector_by_quat(a, q, inverse=True), np.asarray(site_quat, np.float64), inverse=True)

@@ -725,3 +725,50 @@ def test_action_filters_against_oracle():
     assert A.ClipPositions.from_physics_model(m).num_joints == m.nu and A.ClipPositions.from_physics_model(m).max_ranges[0] == 0.9
     with pytest.raises(Exception, match="kind"):
         A._run(9, t32(xs[0]))
+
+
+def test_sensor_observations_gyro_accelerometer_touch():
+    """SensorObservation on a model read from MJCF: one physics step through the kernel, then the sensor elements of
+    ks_observe against the oracle formulas on the step's own outputs; the gyro of a site with the base's orientation is
+    the free joint's body-frame angular velocity the substep started from; touch is the foot body's normal contact force."""
+    from ksim_amd import _lib_terms as T, observation as ob, physics
+    from ksim_amd._lib_dyn import KS_ACT_TORQUE
+    from ksim_amd.env_terms import EnvTerms
+    from ksim_amd.mjcf import load_mjcf
+    from dyn_common import random_states
+
+    m = load_mjcf(os.path.join(GOLD, "mini_biped.mjcf"), integrator="implicitfast")
+    dm = physics.DeviceModel(m)
+    N = 64
+    qpos, qvel = random_states(m, N, seed=93, vel_scale=0.8, joint_range=0.3)
+    ctrl = np.random.default_rng(94).normal(size=(N, m.nu)) * 2
+    z = lambda *s: torch.zeros(*s, device=DEV)  # noqa: E731
+    buf = dict(qpos=t32(qpos), qvel=t32(qvel), qacc_warmstart=z(N, m.nv), time=z(N), last_ctrl=t32(ctrl), action=t32(ctrl),
+               qacc=z(N, m.nv), xpos=z(N, m.nb * 3), xquat=z(N, m.nb * 4), cvel=z(N, m.nb * 6), cfrc_ext=z(N, m.nb * 6))
+    physics.control_step(dm, buf, substeps=1, actuator_type=KS_ACT_TORQUE)
+    observations = {n: ob.SensorObservation.create(physics_model=m, sensor_name=n)
+                    for n in ("imu_gyro", "imu_acc", "left_foot_touch", "right_foot_touch")}
+    terms = EnvTerms(m, observations, {}, [])
+    assert terms.obs_dim == 3 + 3 + 1 + 1 and list(terms.obs_slices) == ["imu_gyro", "imu_acc", "left_foot_touch", "right_foot_touch"]
+    src = {T.SRC_QPOS: buf["qpos"], T.SRC_QVEL: buf["qvel"], T.SRC_QACC: buf["qacc"], T.SRC_XQUAT: buf["xquat"],
+           T.SRC_CVEL: buf["cvel"], T.SRC_CFRC_EXT: buf["cfrc_ext"]}
+    obs = torch.empty(N, terms.obs_dim, device=DEV)
+    terms.observe(src, N, obs=obs)
+    got = obs.cpu().numpy()
+    xq = buf["xquat"].cpu().numpy().reshape(N, m.nb, 4).astype(np.float64)
+    cv = buf["cvel"].cpu().numpy().reshape(N, m.nb, 6).astype(np.float64)
+    qa = buf["qacc"].cpu().numpy().astype(np.float64)
+    cf = buf["cfrc_ext"].cpu().numpy().reshape(N, m.nb, 6)
+    _, spos, squat = m.sites["imu_site"]
+    np.testing.assert_allclose(got[:, 0:3], ot.site_gyro(xq[:, 1], cv[:, 1, :3], squat), rtol=1e-5, atol=1e-5)
+    np.testing.assert_allclose(got[:, 3:6], ot.site_accelerometer(qa[:, :6], xq[:, 1], cv[:, 1, :3], spos, squat, m.gravity),
+                               rtol=1e-4, atol=1e-3)
+    np.testing.assert_allclose(got[:, 6], cf[:, m.sites["left_foot"][0], 5], rtol=1e-6)
+    np.testing.assert_allclose(got[:, 7], cf[:, m.sites["right_foot"][0], 5], rtol=1e-6)
+    assert (got[:, 6:] >= 0).all() and (got[:, 6:] > 1.0).sum() > N // 4  # feet in the ground in many envs
+    # the angular velocity the forward pass of this (single) substep saw is the state's own, in body axes
+    np.testing.assert_allclose(ot.site_gyro(xq[:, 1], cv[:, 1, :3], [1, 0, 0, 0]), qvel[:, 3:6], rtol=1e-4, atol=1e-4)
+    # a body at rest on the ground would read +9.81 along the world's up axis: here check the size in free fall instead
+    air = (cf[:, :, 5].sum(1) == 0)
+    if air.any():  # no contact: the base origin accelerates with gravity plus what the joints do; the reading stays moderate
+        assert np.isfinite(got[air, 3:6]).all()

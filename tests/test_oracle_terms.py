@@ -380,3 +380,36 @@ def test_action_filters_closed_forms():
     zeros = np.array([0.5, 0.1])
     bias = np.arctanh((zeros - lo) / (hi - lo))
     np.testing.assert_allclose(terms.tanh_positions(bias, lo, hi), zeros, rtol=1e-12)
+
+
+def test_site_sensors_against_rigid_motion():
+    """Gyro and accelerometer at a site of a floating base: scipy rotations, the free joint's own body-frame angular
+    velocity, the reading at rest, and a central second difference of the site's world position along an analytic rigid
+    motion (constant linear acceleration, angular velocity w0 + alpha t in body axes)."""
+    from scipy.spatial.transform import Rotation as R
+
+    rng = np.random.default_rng(91)
+    q0 = rng.normal(size=4); q0 /= np.linalg.norm(q0)
+    qs = rng.normal(size=4); qs /= np.linalg.norm(qs)
+    Rb, Rs = R.from_quat(q0[[1, 2, 3, 0]]), R.from_quat(qs[[1, 2, 3, 0]])
+    w_l, al_l, a0 = rng.normal(size=3), rng.normal(size=3) * 2, rng.normal(size=3) * 3
+    r_s = np.array([0.05, -0.02, 0.4])
+    g = np.array([0.0, 0.0, -9.81])
+    w_world = Rb.apply(w_l)
+    # gyro: body-frame angular velocity (what the free joint's qvel[3:6] holds), turned into the site frame
+    np.testing.assert_allclose(terms.site_gyro(q0, w_world, qs), Rs.inv().apply(w_l), atol=1e-12)
+    np.testing.assert_allclose(terms.site_gyro(q0, w_world, [1, 0, 0, 0]), w_l, atol=1e-12)
+    # at rest the accelerometer reads minus gravity in its own frame
+    rest = terms.site_accelerometer(np.zeros(6), q0, np.zeros(3), r_s, qs, g)
+    np.testing.assert_allclose(rest, (Rb * Rs).inv().apply([0, 0, 9.81]), atol=1e-12)
+    # moving: second difference of p(t) = x(t) + R(t) r_s
+    def p(t):
+        rot = Rb * R.from_rotvec(w_l * t + 0.5 * al_l * t * t)   # exact to O(t^3)
+        return 0.5 * a0 * t * t + rot.apply(r_s)
+    h = 1e-4
+    acc_fd = (p(h) - 2 * p(0.0) + p(-h)) / h**2
+    want = (Rb * Rs).inv().apply(acc_fd - g)
+    got = terms.site_accelerometer(np.concatenate([a0, al_l]), q0, w_world, r_s, qs, g)
+    np.testing.assert_allclose(got, want, rtol=1e-4, atol=1e-4)
+    # dropped terms would show: centripetal and tangential parts are both far above the tolerance here
+    assert np.linalg.norm(np.cross(w_world, np.cross(w_world, Rb.apply(r_s)))) > 0.05 and np.linalg.norm(np.cross(Rb.apply(al_l), Rb.apply(r_s))) > 0.05
