@@ -231,7 +231,7 @@ def gae_bandwidth(torch, ppo, reps=8):
 
 
 def ppo_update_rate(torch, reps=6):
-    """One minibatch step of the policy update at BASELINE config 5's shape: 2048 envs x T=32 rows through actor and
+    """One minibatch step of the policy update at benchmark config 5's shape: 2048 envs x T=32 rows through actor and
     critic (3x512 bf16), GAE, loss gradient, backward GEMMs, optimiser chain."""
     from ksim_amd.mlp import random_mlp
     from ksim_amd.ppo_update import GaussianMlpPolicy, PPOUpdateConfig, get_ppo_variables, single_step

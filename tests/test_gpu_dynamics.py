@@ -1,6 +1,6 @@
 """Parity of the fused HIP control-step kernel against the CPU oracle (through the C ABI).
 
-Tolerances are BASELINE's: qacc and one-step state 1e-4 relative, 10-step trajectories 1e-3
+Tolerances are the benchmark definition's: qacc and one-step state 1e-4 relative, 10-step trajectories 1e-3
 (fp32 kernel against the float64 oracle; "relative" = max abs error of an env's vector over
 that vector's max magnitude).
 """
@@ -178,7 +178,7 @@ def test_position_controlled_steps(name, S, T, period):
 
 
 def test_cfg1_chain_200_steps():
-    """BASELINE config 1: 128 envs, 200 steps, targets resampled every step; checked at steps 1, 10, 200."""
+    """benchmark config 1: 128 envs, 200 steps, targets resampled every step; checked at steps 1, 10, 200."""
     from ksim_amd import physics
 
     m = km.pendulum_chain_model()

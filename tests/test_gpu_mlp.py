@@ -21,7 +21,7 @@ def reference(x, ws, bs, act, bf16):
 
 
 @pytest.mark.parametrize("dims,dtype,act,M", [
-    ((71, 256, 256, 256, 21), "f32", "elu", 300),      # BASELINE config 3 actor
+    ((71, 256, 256, 256, 21), "f32", "elu", 300),      # benchmark config 3 actor
     ((68, 512, 512, 512, 20), "bf16", "elu", 1000),    # config 4 actor
     ((68, 512, 512, 512, 1), "bf16", "elu", 129),      # config 4 critic, ragged tile
     ((71, 256, 256, 1), "bf16", "relu", 64),           # config 5 discriminator shape

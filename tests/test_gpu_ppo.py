@@ -8,7 +8,7 @@ from oracle import terms as oterms
 
 pytestmark = pytest.mark.gpu
 
-GAE_TOL = 1e-5  # BASELINE tolerance for GAE and returns (relative to the array's max magnitude)
+GAE_TOL = 1e-5  # benchmark tolerance for GAE and returns (relative to the array's max magnitude)
 
 
 def _inputs(seed, B, T, p_done=0.01, p_succ=0.3):

@@ -82,7 +82,7 @@ def test_term_tables_compile():
     resets = [rs.RandomJointPositionReset(scale=0.1, scale_by_curriculum=False), rs.RandomHeightReset(range=(0.0, 0.1)),
               rs.RandomHeadingReset(), rs.RandomJointVelocityReset()]
     d, slices, used, bias, tab = compile_terms(m, observations, {"h": tm.MinimumHeightTermination(0.5)}, resets, 2)
-    assert d.obs_dim == 71 and slices["g"] == slice(42, 45) and slices["c"] == slice(69, 71)  # BASELINE config 3: 71
+    assert d.obs_dim == 71 and slices["g"] == slice(42, 45) and slices["c"] == slice(69, 71)  # benchmark config 3: 71
     assert d.obs[0].kind == T.OBS_JOINT_POS and d.obs[0].index == 7 and d.obs[0].noise_kind == T.NOISE_ADD_GAUSSIAN
     assert d.obs[42].kind == T.OBS_ROT_INV and d.obs[44].comp == 2 and d.obs[44].c2 == pytest.approx(-9.81)
     assert T.SRC_CVEL not in used and T.SRC_QPOS in used
