@@ -519,7 +519,7 @@ int ks_action_filter(ks_stream_t stream, int64_t N, int32_t nu, int32_t kind, fl
  * mean_k, std_k)) of the sample before the NaN scrub and clip.  deterministic: the mean of the most probable component.
  * The distribution itself (xax.MixtureOfGaussians) is a third-party class that is not part of the reference tree; this
  * is the textbook mixture. */
-#define KS_MAX_MIXTURES 8
+#define KS_MAX_MIXTURES 16
 typedef struct KsMixtureHead {
   int32_t num_mixtures;   /* K in 1..KS_MAX_MIXTURES */
   float min_std, max_std, var_scale;

@@ -668,7 +668,17 @@ def test_mixture_of_gaussians_head():
     with pytest.raises(Exception, match="3 nu K"):
         sample_action_mixture(t32(raw), 7, **kw)
     with pytest.raises(Exception, match="components"):
-        sample_action_mixture(t32(raw[:, :54]), 9, **kw)
+        sample_action_mixture(t32(raw[:, :51]), 17, **kw)
+    # the walking example's ten components (examples/walking.py:273-276)
+    raw10 = rng.normal(size=(64, 3 * nu * 10))
+    u10, z10 = rng.random((64, nu)), rng.normal(size=(64, nu))
+    w10 = ot.mixture_head(raw10, 10, uniform=u10, normal=z10, **kw)
+    g10 = sample_action_mixture(t32(raw10), 10, uniform=t32(u10), noise=t32(z10), want_stats=True, **kw)
+    lg10 = raw10[:, 2 * nu * 10:].reshape(64, nu, 10)
+    cum10 = np.cumsum(np.exp(lg10 - np.logaddexp.reduce(lg10, -1, keepdims=True)), -1)
+    ok10 = np.abs(cum10 - u10[..., None]).min(-1) > 1e-5
+    assert np.array_equal(g10[2].cpu().numpy()[ok10], w10[2][ok10])
+    np.testing.assert_allclose(g10[1].cpu().numpy()[ok10], w10[1][ok10], rtol=2e-4, atol=2e-4)
 
 
 def test_action_filters_against_oracle():
