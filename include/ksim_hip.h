@@ -706,6 +706,16 @@ int ks_ppo_loss_grad_head(ks_stream_t stream, int64_t M, int32_t nu, const KsPpo
                           const float* on_log_probs /*(M,nu)*/, const float* advantages, const float* value_targets,
                           const float* on_values, const float* values, float* d_raw /*(M, 2 nu)*/, float* d_value /*(M)*/);
 
+/* The same for the mixture-of-Gaussians head of ks_sample_action_mixture (examples/walking.py:127-144): raw and d_raw are
+ * (M, 3 nu K).  The policy and KL terms differentiate the mixture's log-density exactly (responsibilities); the entropy
+ * term uses the upper bound sum_k pi_k H_k + H(pi) of a mixture's entropy, which has no closed form (what
+ * xax.MixtureOfGaussians.entropy computes is outside the reference tree: unpinned).  on_log_probs are the per-action
+ * log-densities that ks_sample_action_mixture returned when the actions were drawn. */
+int ks_ppo_loss_grad_mixture(ks_stream_t stream, int64_t M, int32_t nu, const KsPpoLossParams* params /*host*/,
+                             const KsMixtureHead* head /*host*/, const float* raw, const float* action,
+                             const float* on_log_probs /*(M,nu)*/, const float* advantages, const float* value_targets,
+                             const float* on_values, const float* values, float* d_raw /*(M, 3 nu K)*/, float* d_value /*(M)*/);
+
 /* ------------------------------------------------------------------ rewards over a rollout
  * Replaces get_rewards + the stateless Reward.get_reward terms the configs name
  * (ksim/task/rl.py:189-245; ksim/rewards.py:166-188 StayAlive, 374-401 BaseHeight / BaseHeightRange,

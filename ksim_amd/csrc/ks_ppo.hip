@@ -595,6 +595,105 @@ __global__ __launch_bounds__(256) void ppo_loss_grad_head_kernel(int64_t M, int 
   d_value[m] = p.value_loss_coef * gv * inv_m;
 }
 
+// The same objective for the mixture-of-Gaussians head: raw (M, 3 nu K) = component means, raw deviations and logits per
+// action.  One thread per row walks its actions twice (log ratio, then gradients).  The entropy term uses the usual
+// upper bound of a mixture's entropy, sum_k pi_k H_k + H(pi).
+__global__ __launch_bounds__(128) void ppo_loss_grad_mixture_kernel(int64_t M, int nu, KsPpoLossParams p, KsMixtureHead hd,
+                                                                   const float* __restrict__ raw, const float* __restrict__ action,
+                                                                   const float* __restrict__ on_lp, const float* __restrict__ adv,
+                                                                   const float* __restrict__ tgt, const float* __restrict__ on_v,
+                                                                   const float* __restrict__ v, float* __restrict__ d_raw,
+                                                                   float* __restrict__ d_value) {
+  const int64_t m = (int64_t)blockIdx.x * 128 + threadIdx.x;
+  if (m >= M) return;
+  const int K = hd.num_mixtures;
+  const float inv_m = 1.0f / (float)M;
+  const float* rm = raw + m * 3 * nu * K;
+  float* dm = d_raw + m * 3 * nu * K;
+  auto component = [&](int a, int k, float& mean, float& sd, bool& mean_clipped, bool& sd_capped, float& sig) {
+    const float r0 = rm[a * K + k] + (hd.mean_bias ? hd.mean_bias[a] : 0.f);
+    const float lo = hd.clip_lo ? hd.clip_lo[a] : -INFINITY, hi = hd.clip_hi ? hd.clip_hi[a] : INFINITY;
+    mean = fminf(fmaxf(r0, lo), hi);
+    mean_clipped = r0 < lo || r0 > hi;
+    const float r = rm[(nu + a) * K + k];
+    const float sp = r > 20.f ? r : log1pf(expf(r));
+    const float pre = (sp + hd.min_std) * hd.var_scale;
+    sd_capped = pre >= hd.max_std;
+    sd = sd_capped ? hd.max_std : pre;
+    sig = r > 20.f ? 1.f : 1.f / (1.f + expf(-r));
+  };
+  auto log_mix = [&](int a, float x, float& lse_logits) {  // log density of the mixture at x, and the logits' normaliser
+    float lmax = -INFINITY;
+    for (int k = 0; k < K; ++k) lmax = fmaxf(lmax, rm[(2 * nu + a) * K + k]);
+    float zs = 0.f;
+    for (int k = 0; k < K; ++k) zs += expf(rm[(2 * nu + a) * K + k] - lmax);
+    lse_logits = lmax + logf(zs);
+    float tmax = -INFINITY, t[KS_MAX_MIXTURES];
+    for (int k = 0; k < K; ++k) {
+      float mean, sd, sg; bool c1, c2;
+      component(a, k, mean, sd, c1, c2, sg);
+      const float z = (x - mean) / sd;
+      t[k] = (rm[(2 * nu + a) * K + k] - lse_logits) - 0.5f * z * z - logf(sd) - kHalfLog2Pi;
+      tmax = fmaxf(tmax, t[k]);
+    }
+    float acc = 0.f;
+    for (int k = 0; k < K; ++k) acc += expf(t[k] - tmax);
+    return tmax + logf(acc);
+  };
+  float logr = 0.f;
+  for (int a = 0; a < nu; ++a) {
+    float lse;
+    logr += log_mix(a, action[m * nu + a], lse) - on_lp[m * nu + a];
+  }
+  const bool log_inside = logr > -p.log_clip_value && logr < p.log_clip_value;
+  const float ratio = __expf(fminf(fmaxf(logr, -p.log_clip_value), p.log_clip_value));
+  const float A = adv[m];
+  const float lo_r = 1.f - p.clip_param, hi_r = 1.f + p.clip_param;
+  const float s1 = ratio * A, s2 = fminf(fmaxf(ratio, lo_r), hi_r) * A;
+  const bool ratio_inside = ratio > lo_r && ratio < hi_r;
+  float g_logr = 0.f;
+  if (log_inside && (s1 < s2 || ratio_inside)) g_logr = -A * ratio;
+  const float g_lp = (g_logr - p.kl_coef * p.kl_scale) * inv_m;
+  const float g_ent = -p.entropy_coef * inv_m;
+  for (int a = 0; a < nu; ++a) {
+    const float x = action[m * nu + a];
+    float lse;
+    const float lp = log_mix(a, x, lse);
+    // entropy bound: sum_k pi_k (h_k - log pi_k), h_k = 1/2 + log sqrt(2 pi) + log sd_k
+    float gbar = 0.f;
+    for (int k = 0; k < K; ++k) {
+      float mean, sd, sg; bool c1, c2;
+      component(a, k, mean, sd, c1, c2, sg);
+      const float lpi = rm[(2 * nu + a) * K + k] - lse;
+      gbar += expf(lpi) * (0.5f + kHalfLog2Pi + logf(sd) - lpi);
+    }
+    for (int k = 0; k < K; ++k) {
+      float mean, sd, sg; bool mean_clipped, sd_capped;
+      component(a, k, mean, sd, mean_clipped, sd_capped, sg);
+      const float lpi = rm[(2 * nu + a) * K + k] - lse, pi = expf(lpi);
+      const float z = (x - mean) / sd;
+      const float resp = expf(lpi - 0.5f * z * z - logf(sd) - kHalfLog2Pi - lp);  // responsibility of component k
+      dm[a * K + k] = mean_clipped ? 0.f : g_lp * resp * z / sd;
+      const float d_ls = g_lp * resp * (z * z - 1.f) + g_ent * pi;
+      dm[(nu + a) * K + k] = sd_capped ? 0.f : d_ls / sd * hd.var_scale * sg;
+      const float gk = 0.5f + kHalfLog2Pi + logf(sd) - lpi;
+      dm[(2 * nu + a) * K + k] = g_lp * (resp - pi) + g_ent * pi * (gk - gbar);
+    }
+  }
+  const float vv = v[m], vo = on_v[m], t = tgt[m];
+  float gv;
+  if (p.use_clipped_value_loss) {
+    const float dvv = vv - vo;
+    const float vc = vo + fminf(fmaxf(dvv, -p.clip_param), p.clip_param);
+    const float e = vv - t, ec = vc - t;
+    if (e * e >= ec * ec) gv = e;
+    else gv = (dvv > -p.clip_param && dvv < p.clip_param) ? ec : 0.f;
+  } else {
+    gv = vv - t;
+  }
+  d_value[m] = p.value_loss_coef * gv * inv_m;
+}
+
 __global__ void ppo_grad_finish_kernel(int nblocks, int nu, const float* __restrict__ partial, float* __restrict__ d_log_std) {
   const int a = threadIdx.x;
   if (a >= nu) return;
@@ -663,4 +762,24 @@ extern "C" int ks_gaussian_head_log_prob(ks_stream_t stream, int64_t M, int32_t 
   hipLaunchKernelGGL(ks::gaussian_head_log_prob_kernel, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, n, nu, *head, raw, action,
                      log_prob, entropy);
   return ks::check_launch("ks_gaussian_head_log_prob");
+}
+
+extern "C" int ks_ppo_loss_grad_mixture(ks_stream_t stream, int64_t M, int32_t nu, const KsPpoLossParams* params,
+                                        const KsMixtureHead* head, const float* raw, const float* action, const float* on_log_probs,
+                                        const float* advantages, const float* value_targets, const float* on_values,
+                                        const float* values, float* d_raw, float* d_value) {
+  if (!params || !head) return ks::fail(KS_EINVAL, "ks_ppo_loss_grad_mixture: null parameters");
+  if (M < 1 || nu < 1) return ks::fail(KS_EINVAL, "ks_ppo_loss_grad_mixture: bad shape");
+  if (head->num_mixtures < 1 || head->num_mixtures > KS_MAX_MIXTURES)
+    return ks::fail(KS_ELIMIT, "ks_ppo_loss_grad_mixture: %d components, 1..%d are built", head->num_mixtures, KS_MAX_MIXTURES);
+  if (!raw || !action || !on_log_probs || !advantages || !value_targets || !on_values || !values || !d_raw || !d_value)
+    return ks::fail(KS_EINVAL, "ks_ppo_loss_grad_mixture: null pointer");
+  if (!(head->max_std > 0.f) || head->min_std < 0.f || !(head->var_scale > 0.f))
+    return ks::fail(KS_EINVAL, "ks_ppo_loss_grad_mixture: bad deviation bounds");
+  if ((head->clip_lo == nullptr) != (head->clip_hi == nullptr)) return ks::fail(KS_EINVAL, "ks_ppo_loss_grad_mixture: clip_lo and clip_hi come together");
+  const int64_t grid = (M + 127) / 128;
+  if (grid > 0x7fffffff) return ks::fail(KS_ELIMIT, "ks_ppo_loss_grad_mixture: too many rows");
+  hipLaunchKernelGGL(ks::ppo_loss_grad_mixture_kernel, dim3((unsigned)grid), dim3(128), 0, (hipStream_t)stream, M, nu, *params, *head, raw,
+                     action, on_log_probs, advantages, value_targets, on_values, values, d_raw, d_value);
+  return ks::check_launch("ks_ppo_loss_grad_mixture");
 }

@@ -47,6 +47,25 @@ def gaussian_head(raw, action, min_std, max_std, var_scale, mean_bias=None):
     return gaussian(mean, torch.log(std), action)
 
 
+def mixture_head(raw, action, num_mixtures, min_std, max_std, var_scale, mean_bias=None, clip_lo=None, clip_hi=None):
+    """Log-density per action of the mixture-of-Gaussians head (examples/walking.py:127-144) and the upper bound
+    sum_k pi_k H_k + H(pi) of its entropy (a mixture's entropy has no closed form; xax's own choice is unpinned)."""
+    K = num_mixtures
+    nu = raw.shape[-1] // (3 * K)
+    lead = raw.shape[:-1]
+    mean = raw[..., : nu * K].reshape(*lead, nu, K)
+    if mean_bias is not None:
+        mean = mean + mean_bias[..., None]
+    if clip_lo is not None:
+        mean = torch.maximum(torch.minimum(mean, clip_hi[..., None]), clip_lo[..., None])
+    std = torch.clamp((F.softplus(raw[..., nu * K: 2 * nu * K].reshape(*lead, nu, K)) + min_std) * var_scale, max=max_std)
+    logw = torch.log_softmax(raw[..., 2 * nu * K:].reshape(*lead, nu, K), dim=-1)
+    z = (action[..., None] - mean) / std
+    lp = torch.logsumexp(logw - 0.5 * z * z - torch.log(std) - 0.5 * math.log(2 * math.pi), dim=-1)
+    ent = (torch.exp(logw) * (0.5 + 0.5 * math.log(2 * math.pi) + torch.log(std) - logw)).sum(-1)
+    return lp, ent
+
+
 def ppo_loss_torch(adv, tgt, on_lp, on_v, lp, v, ent, cfg, kl_scale=1.0):
     """ppo.py:207-246 per element and 485-486 total, in torch so that autograd can differentiate it."""
     log_ratio = (lp - on_lp).sum(-1)

@@ -283,3 +283,49 @@ def test_recurrent_single_step_gradients_match_oracle():
             assert rel(got[k].cpu().numpy(), ref[k]) < 2e-3, k
     total = sum(float((np.asarray(v) ** 2).sum()) for g in (ga, gc) for v in (g["input_proj"] + tuple(x for c in g["cells"] for x in c) + tuple(x for o in g["out"] for x in o)))
     assert m["grad_norm"].item() == pytest.approx(np.sqrt(total), rel=2e-3)
+
+
+def test_ppo_loss_gradient_for_the_mixture_head_matches_autograd():
+    """d loss / d (means | raw deviations | logits) for the mixture head against float64 autograd of the oracle loss (policy
+    and KL terms through the exact mixture log-density, entropy term through the stated upper bound); clipped means and
+    capped deviations get no gradient."""
+    from ksim_amd import _lib, _lib_terms as T
+    from oracle import terms as ot
+
+    lib = _lib.load()
+    rng = np.random.default_rng(23)
+    M, A, K = 1500, 6, 10
+    raw = rng.normal(size=(M, 3 * A * K))
+    raw[:40, A * K:2 * A * K] = 6.0          # capped deviations
+    raw[40:80, :A * K] = 3.0                 # means beyond the clip range
+    bias = rng.normal(size=A) * 0.1
+    lo, hi = -np.ones(A) * 1.5, np.ones(A) * 1.8
+    hd = dict(min_std=0.01, max_std=1.2, var_scale=0.5)
+    act, _, _ = ot.mixture_head(raw, K, uniform=rng.random((M, A)), normal=rng.normal(size=(M, A)), mean_bias=bias, clip_lo=lo,
+                                clip_hi=hi, **hd)
+    tb, tlo, thi = torch.tensor(bias), torch.tensor(lo), torch.tensor(hi)
+    on_lp = ou.mixture_head(torch.tensor(raw + rng.normal(size=raw.shape) * 0.02), torch.tensor(act), K, mean_bias=tb, clip_lo=tlo,
+                            clip_hi=thi, **hd)[0].numpy()
+    adv, tgt, on_v = rng.normal(size=M), rng.normal(size=M), rng.normal(size=M)
+    v = on_v + rng.normal(size=M) * 0.3
+    tr, tv = torch.tensor(raw, requires_grad=True), torch.tensor(v, requires_grad=True)
+    lp, ent = ou.mixture_head(tr, torch.tensor(act), K, mean_bias=tb, clip_lo=tlo, clip_hi=thi, **hd)
+    loss, _ = ou.ppo_loss_torch(torch.tensor(adv), torch.tensor(tgt), torch.tensor(on_lp), torch.tensor(on_v), lp, tv, ent, CFG, 1.3)
+    loss.backward()
+    p = _lib.KsPpoLossParams(0.2, 0.5, 0.008, 1e-3, 5.0, 1.3, 1)
+    dev = [t32(a) for a in (bias, lo, hi)]
+    head = T.KsMixtureHead(K, 0.01, 1.2, 0.5, 0, *[_lib.ptr(t).value for t in dev])
+    d_raw, d_value = torch.empty(M, 3 * A * K, device=DEV), torch.empty(M, device=DEV)
+    args = [t32(a) for a in (raw, act, on_lp, adv, tgt, on_v, v)]
+    _lib.check(lib.ks_ppo_loss_grad_mixture(_lib.current_stream(), M, A, ctypes.byref(p), ctypes.byref(head), *[_lib.ptr(a) for a in args],
+                                            _lib.ptr(d_raw), _lib.ptr(d_value)))
+    g, got = tr.grad.numpy(), d_raw.cpu().numpy()
+    for name, sl in (("means", slice(0, A * K)), ("deviations", slice(A * K, 2 * A * K)), ("logits", slice(2 * A * K, None))):
+        assert rel(got[:, sl], g[:, sl]) < 2e-4, name
+    assert rel(d_value.cpu().numpy(), tv.grad.numpy()) < 1e-5
+    assert (got[:40, A * K:2 * A * K] == 0).all() and (got[40:80, :A * K] == 0).all() and (g[40:80, :A * K] == 0).all()
+    # the kernel that drew the actions reports the log-density this gradient starts from
+    from ksim_amd.env_terms import sample_action_mixture
+    _, lp_k, _ = sample_action_mixture(args[0], K, mean_bias=dev[0], clip_lo=dev[1], clip_hi=dev[2], uniform=t32(rng.random((M, A))),
+                                       noise=t32(rng.normal(size=(M, A))), want_stats=True, **hd)
+    assert torch.isfinite(lp_k).all()

@@ -87,3 +87,26 @@ def test_optimiser_chain_known_answers():
     cfg3 = dict(cfg, adam_weight_decay=0.1, adam_b1=0.0, adam_b2=0.0)
     _, m1, _, _ = ou.optax_chain_step([np.array([10.0])], [np.array([1.0])], [np.zeros(1)], [np.zeros(1)], 1, cfg3)
     np.testing.assert_allclose(m1[0], [2.0])
+
+
+def test_mixture_head_in_torch_matches_the_numpy_oracle_and_bounds_the_entropy():
+    """The differentiable mixture head used for the gradient check: its log-density equals the numpy oracle's (pinned by
+    scipy), and its entropy term is an upper bound of the mixture's entropy (Monte-Carlo estimate on one mixture)."""
+    from oracle import terms as ot
+
+    rng = np.random.default_rng(5)
+    M, A, K = 30, 4, 3
+    raw = rng.normal(size=(M, 3 * A * K))
+    bias = rng.normal(size=A) * 0.1
+    lo, hi = -np.ones(A), np.ones(A) * 1.2
+    hd = dict(min_std=0.02, max_std=0.8, var_scale=0.5)
+    act, logp, _ = ot.mixture_head(raw, K, uniform=rng.random((M, A)), normal=rng.normal(size=(M, A)), mean_bias=bias, clip_lo=lo, clip_hi=hi, **hd)
+    lp, ent = ou.mixture_head(torch.tensor(raw), torch.tensor(act), K, mean_bias=torch.tensor(bias), clip_lo=torch.tensor(lo),
+                              clip_hi=torch.tensor(hi), **hd)
+    np.testing.assert_allclose(lp.numpy(), logp, rtol=1e-10, atol=1e-10)
+    # entropy of env 0, action 0 by sampling: -E[log p] <= sum_k pi_k H_k + H(pi)
+    one = np.tile(raw[:1], (200000, 1))
+    a, l, _ = ot.mixture_head(one, K, uniform=rng.random((200000, A)), normal=rng.normal(size=(200000, A)), mean_bias=bias, clip_lo=lo, clip_hi=hi, **hd)
+    h_mc = -l[:, 0].mean()
+    assert h_mc <= float(ent[0, 0]) + 0.01
+    assert float(ent[0, 0]) - h_mc < np.log(K) + 0.01  # and within the mixing entropy of it
