@@ -711,6 +711,8 @@ int ks_ppo_loss_grad_head(ks_stream_t stream, int64_t M, int32_t nu, const KsPpo
  * term uses the upper bound sum_k pi_k H_k + H(pi) of a mixture's entropy, which has no closed form (what
  * xax.MixtureOfGaussians.entropy computes is outside the reference tree: unpinned).  on_log_probs are the per-action
  * log-densities that ks_sample_action_mixture returned when the actions were drawn. */
+int ks_mixture_head_log_prob(ks_stream_t stream, int64_t M, int32_t nu, const KsMixtureHead* head /*host*/,
+                             const float* raw /*(M, 3 nu K)*/, const float* action /*(M,nu)*/, float* log_prob /*(M,nu)*/);
 int ks_ppo_loss_grad_mixture(ks_stream_t stream, int64_t M, int32_t nu, const KsPpoLossParams* params /*host*/,
                              const KsMixtureHead* head /*host*/, const float* raw, const float* action,
                              const float* on_log_probs /*(M,nu)*/, const float* advantages, const float* value_targets,

@@ -218,6 +218,8 @@ def bind(lib) -> None:
     lib.ks_ppo_loss_grad_head.restype = c_int32
     lib.ks_ppo_loss_grad_mixture.argtypes = [c_void_p, c_int64, c_int32, c_void_p, POINTER(KsMixtureHead)] + [c_void_p] * 9
     lib.ks_ppo_loss_grad_mixture.restype = c_int32
+    lib.ks_mixture_head_log_prob.argtypes = [c_void_p, c_int64, c_int32, POINTER(KsMixtureHead), c_void_p, c_void_p, c_void_p]
+    lib.ks_mixture_head_log_prob.restype = c_int32
     lib.ks_gaussian_head_log_prob.argtypes = [c_void_p, c_int64, c_int32, POINTER(KsGaussianHead), c_void_p, c_void_p, c_void_p, c_void_p]
     lib.ks_gaussian_head_log_prob.restype = c_int32
     lib.ks_lstm_train_init.argtypes = [c_void_p]

@@ -393,7 +393,8 @@ __global__ __launch_bounds__(256) void sample_action_mixture_kernel(int64_t n, i
                                                                     KsMixtureHead hd, const float* __restrict__ uniform,
                                                                     const float* __restrict__ noise, KsRng rng,
                                                                     float clip_max, float* __restrict__ action,
-                                                                    float* __restrict__ logp_out, int* __restrict__ comp_out) {
+                                                                    float* __restrict__ logp_out, int* __restrict__ comp_out,
+                                                                    const float* __restrict__ given) {
   const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= n) return;
   const int64_t e = idx / nu;
@@ -450,6 +451,7 @@ __global__ __launch_bounds__(256) void sample_action_mixture_kernel(int64_t n, i
   for (int k = 0; k < KS_MAX_MIXTURES; ++k)
     if (k == pick) { pm = mean[k]; ps = sd[k]; }
   float a = hd.deterministic ? pm : pm + ps * z;
+  if (given) a = given[idx];  // log-density of a recorded action instead of a fresh sample
   if (logp_out) {
     float t[KS_MAX_MIXTURES], tmax = -INFINITY;
 #pragma unroll
@@ -464,6 +466,7 @@ __global__ __launch_bounds__(256) void sample_action_mixture_kernel(int64_t n, i
     logp_out[idx] = tmax + logf(acc);
   }
   if (comp_out) comp_out[idx] = pick;
+  if (!action) return;
   if (a != a) a = 0.f;
   a = fminf(fmaxf(a, -clip_max), clip_max);
   action[idx] = a;
@@ -938,8 +941,28 @@ extern "C" int ks_sample_action_mixture(ks_stream_t stream, int64_t N, int32_t n
   const int64_t n = N * nu, grid = (n + 255) / 256;
   if (grid > 0x7fffffff) return fail(KS_ELIMIT, "ks_sample_action_mixture: too many elements");
   hipLaunchKernelGGL(sample_action_mixture_kernel, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, n, (int)nu, raw, *head,
-                     uniform, noise_normal, rng, clip_max, action, log_prob_out, component_out);
+                     uniform, noise_normal, rng, clip_max, action, log_prob_out, component_out, (const float*)nullptr);
   return check_launch("ks_sample_action_mixture");
+}
+
+extern "C" int ks_mixture_head_log_prob(ks_stream_t stream, int64_t M, int32_t nu, const KsMixtureHead* head, const float* raw,
+                                        const float* action, float* log_prob) {
+  using namespace ks;
+  if (M < 0 || nu < 1) return fail(KS_EINVAL, "ks_mixture_head_log_prob: bad sizes");
+  if (M == 0) return KS_OK;
+  if (!raw || !head || !action || !log_prob) return fail(KS_EINVAL, "ks_mixture_head_log_prob: null pointer");
+  if (head->num_mixtures < 1 || head->num_mixtures > KS_MAX_MIXTURES)
+    return fail(KS_ELIMIT, "ks_mixture_head_log_prob: %d components, 1..%d are built", head->num_mixtures, KS_MAX_MIXTURES);
+  if (!(head->max_std > 0.f) || head->min_std < 0.f || !(head->var_scale > 0.f)) return fail(KS_EINVAL, "ks_mixture_head_log_prob: bad deviation bounds");
+  if ((head->clip_lo == nullptr) != (head->clip_hi == nullptr)) return fail(KS_EINVAL, "ks_mixture_head_log_prob: clip_lo and clip_hi come together");
+  const int64_t n = M * nu, grid = (n + 255) / 256;
+  if (grid > 0x7fffffff) return fail(KS_ELIMIT, "ks_mixture_head_log_prob: too many elements");
+  KsMixtureHead hd = *head;
+  hd.deterministic = 1;  // no draws: only the density of the given action is wanted
+  KsRng none = {0, 0, nullptr};
+  hipLaunchKernelGGL(sample_action_mixture_kernel, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, n, (int)nu, raw, hd,
+                     (const float*)nullptr, (const float*)nullptr, none, 1.f, (float*)nullptr, log_prob, (int*)nullptr, action);
+  return check_launch("ks_mixture_head_log_prob");
 }
 
 extern "C" int ks_rewards(ks_stream_t stream, const KsRewardIO* io) {

@@ -171,10 +171,21 @@ class RecurrentHeadPolicy:
     var_scale: float = 1.0
     mean_bias: torch.Tensor | None = None
     opt_step: int = 0
+    # a mixture-of-Gaussians head instead (examples/walking.py:127-144): the actor emits 3 K values per action
+    num_mixtures: int = 0
+    clip_lo: torch.Tensor | None = None
+    clip_hi: torch.Tensor | None = None
 
     def train_init(self) -> None:
         self.actor.train_init()
         self.critic.train_init()
+
+    def width(self, nu: int) -> int:
+        return 3 * nu * self.num_mixtures if self.num_mixtures else 2 * nu
+
+    def _mixture(self) -> "T.KsMixtureHead":
+        return T.KsMixtureHead(int(self.num_mixtures), float(self.min_std), float(self.max_std), float(self.var_scale), 0,
+                               _lib.ptr(self.mean_bias).value, _lib.ptr(self.clip_lo).value, _lib.ptr(self.clip_hi).value)
 
 
 def single_step_recurrent(policy: RecurrentHeadPolicy, cfg: PPOUpdateConfig, actor_obs, critic_obs, action, rewards, done, success,
@@ -193,10 +204,13 @@ def single_step_recurrent(policy: RecurrentHeadPolicy, cfg: PPOUpdateConfig, act
                                         monte_carlo_returns=cfg.monte_carlo_returns, time_major=True)
     p = _lib.KsPpoLossParams(cfg.clip_param, cfg.value_loss_coef, cfg.entropy_coef, cfg.kl_coef, cfg.log_clip_value, 1.0,
                              int(cfg.use_clipped_value_loss))
-    head = T.KsGaussianHead(float(policy.min_std), float(policy.max_std), float(policy.var_scale), 0, _lib.ptr(policy.mean_bias).value)
-    d_raw = torch.empty(Tn, b, 2 * nu, dtype=torch.float32, device=raw.device)
+    mixture = policy.num_mixtures > 0
+    head = policy._mixture() if mixture else T.KsGaussianHead(float(policy.min_std), float(policy.max_std), float(policy.var_scale), 0,
+                                                              _lib.ptr(policy.mean_bias).value)
+    d_raw = torch.empty(Tn, b, policy.width(nu), dtype=torch.float32, device=raw.device)
     d_value = torch.empty(Tn, b, 1, dtype=torch.float32, device=raw.device)
-    _lib.check(lib.ks_ppo_loss_grad_head(_lib.current_stream(), rows, nu, ctypes.byref(p), ctypes.byref(head), _lib.ptr(raw),
+    grad_fn = lib.ks_ppo_loss_grad_mixture if mixture else lib.ks_ppo_loss_grad_head
+    _lib.check(grad_fn(_lib.current_stream(), rows, nu, ctypes.byref(p), ctypes.byref(head), _lib.ptr(raw),
                                          _lib.ptr(action.contiguous()), _lib.ptr(on_log_probs.contiguous()),
                                          _lib.ptr(inputs.advantages_bt), _lib.ptr(inputs.value_targets_bt),
                                          _lib.ptr(on_values.contiguous()), _lib.ptr(value), _lib.ptr(d_raw), _lib.ptr(d_value)))
@@ -218,15 +232,20 @@ def recurrent_on_policy(policy: RecurrentHeadPolicy, actor_obs, critic_obs, acti
     update_model makes once over the whole rollout before any minibatch step (ppo.py:603-607)."""
     Tn, N, nu = action.shape
     a_carry, c_carry = actor_carry0.clone(), critic_carry0.clone()
-    raw = torch.empty(Tn, N, 2 * nu, dtype=torch.float32, device=action.device)
+    raw = torch.empty(Tn, N, policy.width(nu), dtype=torch.float32, device=action.device)
     values = torch.empty(Tn, N, 1, dtype=torch.float32, device=action.device)
     for t in range(Tn):
         policy.actor(actor_obs[t], a_carry, fresh=fresh[t], out=raw[t])
         policy.critic(critic_obs[t], c_carry, fresh=fresh[t], out=values[t])
     lp = torch.empty(Tn, N, nu, dtype=torch.float32, device=action.device)
-    head = T.KsGaussianHead(float(policy.min_std), float(policy.max_std), float(policy.var_scale), 0, _lib.ptr(policy.mean_bias).value)
-    _lib.check(_lib.load().ks_gaussian_head_log_prob(_lib.current_stream(), Tn * N, nu, ctypes.byref(head), _lib.ptr(raw),
-                                                     _lib.ptr(action.contiguous()), _lib.ptr(lp), None))
+    if policy.num_mixtures:
+        head = policy._mixture()
+        _lib.check(_lib.load().ks_mixture_head_log_prob(_lib.current_stream(), Tn * N, nu, ctypes.byref(head), _lib.ptr(raw),
+                                                        _lib.ptr(action.contiguous()), _lib.ptr(lp)))
+    else:
+        head = T.KsGaussianHead(float(policy.min_std), float(policy.max_std), float(policy.var_scale), 0, _lib.ptr(policy.mean_bias).value)
+        _lib.check(_lib.load().ks_gaussian_head_log_prob(_lib.current_stream(), Tn * N, nu, ctypes.byref(head), _lib.ptr(raw),
+                                                         _lib.ptr(action.contiguous()), _lib.ptr(lp), None))
     return lp, values[..., 0]
 
 

@@ -99,6 +99,10 @@ def build(N, T, seed=0, min_height=0.9, events=None, gait=False, recurrent=False
             from ksim_amd.rollout import MixtureHead
             head = MixtureHead(num_mixtures=2, min_std=0.0, max_std=1e-6, mean_bias=head_bias,
                                clip_lo=t32(np.full(m.nu, -0.3)), clip_hi=t32(np.full(m.nu, 0.3)))
+        elif head == "mixture-wide":
+            from ksim_amd.rollout import MixtureHead
+            head = MixtureHead(num_mixtures=3, min_std=0.05, max_std=0.5, var_scale=0.5, mean_bias=head_bias,
+                               clip_lo=t32(np.full(m.nu, -0.6)), clip_hi=t32(np.full(m.nu, 0.6)))
         actor, critic = net(m.nu if head is None else head.width(m.nu), "gelu"), net(1, "elu")
     consts = RolloutConstants(physics_model=dm, engine=eng, terms=terms, rewards=rewards,
                               actor=actor, critic=critic, log_std=t32(log_std), commands=commands, head=head)
@@ -451,14 +455,15 @@ def test_recurrent_actor_and_critic_in_the_rollout(head):
             assert torch.equal(x, y), f"replay {it}: {name} differs from the eager rollout"
 
 
-def test_recurrent_policy_update_from_a_rollout():
+@pytest.mark.parametrize("head", ["gaussian-wide", "mixture-wide"])
+def test_recurrent_policy_update_from_a_rollout(head):
     """A rollout with a GRU actor (deviation head) and a GRU critic, then the recurrent policy update on its buffers: the
     on-policy pass, replayed from the recorded first-step carries and episode starts, reproduces the values the rollout
     computed bit for bit; the minibatch steps run through time, move every parameter and keep everything finite."""
     from ksim_amd import ppo_update as pu
 
     N, T = 32, 8
-    m, c, rnd_, _, ro, EnvState = build(N, T, seed=17, min_height=0.95, recurrent=True, head="gaussian-wide")
+    m, c, rnd_, _, ro, EnvState = build(N, T, seed=17, min_height=0.95, recurrent=True, head=head)
     ps = c.engine.reset(c.physics_model, 1.0, 3, N, rnd_)
     env = EnvState(ps, rnd_, torch.zeros(N, 2, device=DEV), None, seed=23)
     for _ in range(3):  # the third rollout starts from carries that are not zero
@@ -466,6 +471,8 @@ def test_recurrent_policy_update_from_a_rollout():
     assert ro.fresh.sum().item() > 0 and ro.actor_carry0.abs().max().item() > 0
     assert torch.equal(ro.fresh[1:], traj.done[:-1])  # an env starts an episode at the step after it finished
     policy = pu.RecurrentHeadPolicy(c.actor, c.critic, c.head.min_std, c.head.max_std, c.head.var_scale, c.head.mean_bias)
+    if head == "mixture-wide":
+        policy.num_mixtures, policy.clip_lo, policy.clip_hi = c.head.num_mixtures, c.head.clip_lo, c.head.clip_hi
     policy.train_init()
     args = (traj.obs["noisy_obs"], traj.obs["obs"], traj.action, rew.total, traj.done, traj.success, ro.actor_carry0, ro.critic_carry0, ro.fresh)
     on_lp, on_v = pu.recurrent_on_policy(policy, args[0], args[1], args[2], *args[6:])
