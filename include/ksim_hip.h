@@ -143,6 +143,8 @@ typedef struct KsModelDesc {
   int32_t jnt_limited[KS_MAX_BODIES];
   double jnt_range[KS_MAX_BODIES][2], dof_invweight0[KS_MAX_DOFS], dof_frictionloss[KS_MAX_DOFS];
   double dof_solref[2], dof_solimp[5];
+  double dof_stiffness[KS_MAX_DOFS]; /* joint springs of hinges about qpos0 (MuJoCo jnt_stiffness, springref = qpos0;
+                                        examples/data/scene.mjcf:43-66): passive force -stiffness (q - qpos0) */
 } KsModelDesc;
 
 typedef struct KsModel KsModel;

@@ -30,6 +30,7 @@ class KsModelDesc(ctypes.Structure):
         ("sph_body", c_int32 * MAXS), ("sph_pos", c_double * 3 * MAXS), ("sph_radius", c_double * MAXS),
         ("jnt_limited", c_int32 * MAXB), ("jnt_range", c_double * 2 * MAXB), ("dof_invweight0", c_double * MAXV),
         ("dof_frictionloss", c_double * MAXV), ("dof_solref", c_double * 2), ("dof_solimp", c_double * 5),
+        ("dof_stiffness", c_double * MAXV),
     ]
 
 
@@ -77,7 +78,7 @@ def model_desc(m) -> KsModelDesc:
               "body_subtree_end", "body_pos", "body_quat", "body_mass", "body_ipos", "body_iquat", "body_inertia",
               "jnt_axis", "jnt_pos", "qpos0", "dof_body", "dof_parent", "dof_damping", "dof_armature", "act_dof",
               "act_gear", "sph_body", "sph_pos", "sph_radius", "jnt_limited", "jnt_range", "dof_invweight0",
-              "dof_frictionloss", "dof_solref", "dof_solimp"):
+              "dof_frictionloss", "dof_solref", "dof_solimp", "dof_stiffness"):
         fill(k, getattr(m, k))
     fill("body_invweight0", m.body_invweight0[:, 0])
     fill("act_lo", m.act_ctrlrange.reshape(-1, 2)[:, 0])

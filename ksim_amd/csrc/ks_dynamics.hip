@@ -207,7 +207,7 @@ __device__ __forceinline__ float row_dot(const float* row, const float (&vv)[NP]
 struct LaneRec {
   int b_parent, b_jtype, b_qadr, b_dofadr;
   int b_depth;
-  float b_q0, b_mass, pad0;
+  float b_q0, b_mass, d_stiffness;  // d_stiffness: spring of the hinge whose dof this lane holds
   float b_pos[3], b_ipos[3], b_inertia[3], b_jaxis[3], b_jpos[3], pad1;
   float b_quat[4], b_iquat[4];
   int d_body, d_act, d_jtype, d_k;
@@ -720,6 +720,7 @@ void step_kernel(StepArgs a) {
       my_qvel = l.qvel[lane];
       const float bias = dot(my_cdof, ld6(l.fsub + 6 * d_body));
       float f = -d_damping * my_qvel - bias;
+      if (rec.d_stiffness != 0.f) f -= rec.d_stiffness * (l.qpos[rec.d_qadr] - m.qpos0[rec.d_qadr]);  // joint spring about qpos0
       if (d_act >= 0) f += d_gear * fminf(fmaxf(l.tau[d_act], d_lo), d_hi);
       qfs = f;
       if (a.dbg_bias) a.dbg_bias[env * nv + lane] = bias;
@@ -1335,12 +1336,14 @@ extern "C" int ks_model_create(const KsModelDesc* d, KsModel** out) {
     r.d_jtype = m.body_jtype[r.d_body];
     r.d_k = dl - m.body_dofadr[r.d_body];
     r.d_damping = m.dof_damping[dl]; r.d_armature = m.dof_armature[dl];
+    r.d_stiffness = 0.f;
     const int ua = r.d_act >= 0 ? r.d_act : 0;
     r.d_gear = m.act_gear[ua]; r.d_lo = m.act_lo[ua]; r.d_hi = m.act_hi[ua];
     r.d_limited = 0; r.d_qadr = 0; r.d_rlo = 0.f; r.d_rhi = 0.f; r.d_invw = 0.f; r.d_floss = 0.f; r.d_frD = 0.f;
     if (is_dof && r.d_jtype == kJntHinge) {
       r.d_limited = d->jnt_limited[r.d_body] != 0;
       r.d_qadr = m.body_qadr[r.d_body];
+      r.d_stiffness = (float)d->dof_stiffness[dl];
       r.d_rlo = (float)d->jnt_range[r.d_body][0]; r.d_rhi = (float)d->jnt_range[r.d_body][1];
       r.d_invw = (float)d->dof_invweight0[dl];
       r.d_floss = (float)d->dof_frictionloss[dl];

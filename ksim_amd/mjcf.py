@@ -2,8 +2,9 @@
 
 The reference compiles its robot files with MuJoCo (`mujoco.MjModel.from_xml_path`, ksim/task/rl.py:717-748,
 ksim/utils/mujoco.py:388-391) and hands the result to MJX.  This loader reads the same files for robots of the K-Bot's
-kind (examples/kbot/robot/kbot-headless/robot.mjcf): a floating base, hinge joints (one per body), explicit `<inertial>`
-elements, `<motor>` actuators, and sphere or capsule collision geoms against the ground plane.  What MuJoCo's compiler does
+kind (examples/kbot/robot/kbot-headless/robot.mjcf) and for the humanoid of the walking example
+(examples/data/scene.mjcf): a floating base, hinge joints, `<inertial>` elements or inertia from sphere / capsule geoms,
+`<motor>` actuators, and sphere or capsule collision geoms against the ground plane.  What MuJoCo's compiler does
 for such a file is restated here:
 
 * `<default>` classes nest and inherit; `childclass` on a body applies to everything below it;
@@ -12,10 +13,15 @@ for such a file is restated here:
   axes by an eigendecomposition);
 * a body without `<inertial>` takes its inertia from its sphere / capsule geoms at the default density of 1000;
 * a capsule touches the plane with its two end spheres, so each collision capsule becomes two contact spheres;
-* a joint with a `range` is limited (autolimits); `armature`, `damping`, `frictionloss` come from the joint or its class.
+* a joint with a `range` is limited (autolimits); `armature`, `damping`, `frictionloss`, `stiffness` (a spring about the
+  joint's reference angle) come from the joint or its class;
+* several hinges on one body act in the order they are listed: the body becomes a chain of massless bodies, one per
+  joint but the last, at the same place, and the last joint carries the body itself;
+* collisions come from `contype` / `conaffinity` or from explicit `<contact><pair>` elements against the floor plane.
 
-Anything else (ball or slide joints, several joints on a body, meshes or boxes as collision geoms or as the only source of
-inertia, tendons, equality constraints, position actuators) raises ValueError: the file needs MuJoCo's full compiler.
+Anything else (ball or slide joints, meshes or boxes as collision geoms or as the only source of inertia, tendons,
+equality constraints, position actuators, contact dimensions other than 3) raises ValueError: the file needs MuJoCo's
+full compiler.
 """
 from __future__ import annotations
 
@@ -127,7 +133,7 @@ class _Body:
     def __init__(self, name):
         self.name = name
         self.pos, self.quat = np.zeros(3), np.array([1.0, 0, 0, 0])
-        self.joint = None                 # dict or None
+        self.joints = []                  # dicts, in the order they act
         self.parts = []                   # (mass, com, tensor about com) in this body's frame
         self.spheres = []                 # (pos, radius, geom name) in this body's frame
         self.sites = []                   # (name, pos, quat) in this body's frame
@@ -154,6 +160,12 @@ def load_mjcf(path: str, **options) -> KinematicModel:
     def angle(v):
         return np.radians(v) if degrees else v
 
+    def geom_frame(attrib, kind):
+        """A geom's frame; the orientation of a sphere, or of a capsule given by its end points, does not matter."""
+        if kind == "sphere" or attrib.get("fromto") is not None:
+            return _vec(attrib.get("pos"), 3, (0, 0, 0)), np.array([1.0, 0, 0, 0])
+        return frame(attrib)
+
     def frame(attrib):
         for bad in ("euler", "axisangle", "xyaxes", "zaxis"):
             if bad in attrib:
@@ -161,39 +173,56 @@ def load_mjcf(path: str, **options) -> KinematicModel:
         return _vec(attrib.get("pos"), 3, (0, 0, 0)), _vec(attrib.get("quat"), 4, (1, 0, 0, 0))
 
     contact_params = []
+    limit_params = []
+    world = root.find("worldbody")
+    planes = {g.get("name") for g in world if g.tag == "geom" and defaults.resolve(g, None).get("type", "sphere") == "plane"}
+    pairs: dict[str, dict] = {}  # geom name -> attributes of its explicit contact pair with the floor
+    con = root.find("contact")
+    for pr in ([] if con is None else con):
+        if pr.tag != "pair":
+            continue  # <exclude> only matters between bodies, which never collide here
+        at = defaults.resolve(pr, None)
+        g1, g2 = at.get("geom1"), at.get("geom2")
+        if (g1 in planes) == (g2 in planes):
+            raise ValueError(f"contact pair {g1!r} / {g2!r}: only pairs of a robot geom with the floor plane are in the model subset")
+        if int(at.get("condim", 3)) != 3:
+            raise ValueError(f"contact pair {g1!r} / {g2!r}: condim {at.get('condim')} is outside the model subset (3 only)")
+        pairs[g2 if g1 in planes else g1] = at
 
     def read_body(elem, childclass):
         b = _Body(elem.get("name", ""))
         b.pos, b.quat = frame(elem.attrib)
         b.quat = b.quat / np.linalg.norm(b.quat)
         childclass = elem.get("childclass", childclass)
-        joints = [e for e in elem if e.tag in ("joint", "freejoint")]
-        if len(joints) > 1:
-            raise ValueError(f"body {b.name!r}: several joints on one body are outside the model subset")
-        if joints:
-            j = joints[0]
+        for j in (e for e in elem if e.tag in ("joint", "freejoint")):
             if j.tag == "freejoint":
-                b.joint = dict(type="free", name=j.get("name", ""))
-            else:
-                a = defaults.resolve(j, childclass)
-                jt = a.get("type", "hinge")
-                if jt == "free":
-                    b.joint = dict(type="free", name=a.get("name", ""))
-                elif jt != "hinge":
-                    raise ValueError(f"joint {a.get('name')!r}: type {jt} is outside the model subset")
-                else:
-                    if float(a.get("ref", 0.0)) != 0.0 or float(a.get("stiffness", 0.0)) != 0.0:
-                        raise ValueError(f"joint {a.get('name')!r}: ref and stiffness are outside the model subset")
-                    rng = _vec(a.get("range"), 2)
-                    limited = a.get("limited", "auto")
-                    if limited == "false" or (limited == "auto" and rng is None):
-                        rng = None
-                    elif rng is None:
-                        raise ValueError(f"joint {a.get('name')!r}: limited without a range")
-                    b.joint = dict(type="hinge", name=a.get("name", ""), axis=_vec(a.get("axis"), 3, (0, 0, 1)),
-                                   pos=_vec(a.get("pos"), 3, (0, 0, 0)), range=None if rng is None else tuple(angle(rng)),
-                                   armature=float(a.get("armature", 0.0)), damping=float(a.get("damping", 0.0)),
-                                   frictionloss=float(a.get("frictionloss", 0.0)))
+                b.joints.append(dict(type="free", name=j.get("name", "")))
+                continue
+            a = defaults.resolve(j, childclass)
+            jt = a.get("type", "hinge")
+            if jt == "free":
+                b.joints.append(dict(type="free", name=a.get("name", "")))
+                continue
+            if jt != "hinge":
+                raise ValueError(f"joint {a.get('name')!r}: type {jt} is outside the model subset")
+            if float(a.get("ref", 0.0)) != 0.0 or float(a.get("springref", 0.0)) != 0.0:
+                raise ValueError(f"joint {a.get('name')!r}: ref and springref are outside the model subset")
+            rng = _vec(a.get("range"), 2)
+            limited = a.get("limited", "auto")
+            if limited == "false" or (limited == "auto" and rng is None):
+                rng = None
+            elif rng is None:
+                raise ValueError(f"joint {a.get('name')!r}: limited without a range")
+            if rng is not None:
+                sl = _vec(a.get("solimplimit"), None, (0.9, 0.95, 0.001, 0.5, 2.0))
+                sl = np.concatenate([sl, np.array([0.9, 0.95, 0.001, 0.5, 2.0])[sl.size:]])
+                limit_params.append((tuple(_vec(a.get("solreflimit"), 2, (0.02, 1.0))), tuple(sl)))
+            b.joints.append(dict(type="hinge", name=a.get("name", ""), axis=_vec(a.get("axis"), 3, (0, 0, 1)),
+                                 pos=_vec(a.get("pos"), 3, (0, 0, 0)), range=None if rng is None else tuple(angle(rng)),
+                                 armature=float(a.get("armature", 0.0)), damping=float(a.get("damping", 0.0)),
+                                 frictionloss=float(a.get("frictionloss", 0.0)), stiffness=float(a.get("stiffness", 0.0))))
+        if len(b.joints) > 1 and any(j["type"] == "free" for j in b.joints):
+            raise ValueError(f"body {b.name!r}: a free joint next to other joints is outside the model subset")
         inertial = elem.find("inertial")
         geoms = [defaults.resolve(g, childclass) for g in elem if g.tag == "geom"]
         if inertial is not None:
@@ -211,13 +240,18 @@ def load_mjcf(path: str, **options) -> KinematicModel:
                     if kind == "mesh":
                         raise ValueError(f"body {b.name!r}: inertia from a mesh is outside the model subset (give <inertial>)")
                     continue
-                gp, gq = frame(g)
+                gp, gq = geom_frame(g, kind)
                 b.parts.append(_geom_inertia(kind, _vec(g.get("size")), _vec(g.get("fromto"), 6), gp, gq))
         for g in geoms:
-            if int(g.get("contype", 1)) == 0 and int(g.get("conaffinity", 1)) == 0:
+            pair = pairs.get(g.get("name"))
+            if pair is None and int(g.get("contype", 1)) == 0 and int(g.get("conaffinity", 1)) == 0:
                 continue  # visual only
             kind = g.get("type", "sphere")
-            size, gp = _vec(g.get("size")), frame(g)[0]
+            if kind == "plane":
+                continue
+            if pair is None and int(g.get("condim", 3)) != 3:
+                raise ValueError(f"geom {g.get('name')!r}: condim {g.get('condim')} is outside the model subset (3 only)")
+            size, gp = _vec(g.get("size")), geom_frame(g, kind)[0]
             if kind == "sphere":
                 b.spheres.append((gp, float(size[0]), g.get("name", "")))
             elif kind == "capsule":
@@ -230,10 +264,11 @@ def load_mjcf(path: str, **options) -> KinematicModel:
                 b.spheres.extend((e, float(size[0]), g.get("name", "")) for e in ends)
             else:
                 raise ValueError(f"body {b.name!r}: a colliding {kind} is outside the model subset (sphere and capsule only)")
-            si = _vec(g.get("solimp"), None, (0.9, 0.95, 0.001, 0.5, 2.0))
+            src = pair if pair is not None else g  # an explicit pair carries its own parameters (MuJoCo's defaults otherwise)
+            si = _vec(src.get("solimp"), None, (0.9, 0.95, 0.001, 0.5, 2.0))
             si = np.concatenate([si, np.array([0.9, 0.95, 0.001, 0.5, 2.0])[si.size:]])
-            contact_params.append((float(_vec(g.get("friction"), None, (1.0, 0.005, 0.0001))[0]),
-                                   tuple(_vec(g.get("solref"), 2, (0.02, 1.0))), tuple(si)))
+            contact_params.append((float(_vec(src.get("friction"), None, (1.0, 0.005, 0.0001))[0]),
+                                   tuple(_vec(src.get("solref"), 2, (0.02, 1.0))), tuple(si)))
         for st in (e for e in elem if e.tag == "site"):
             sa = defaults.resolve(st, childclass)
             sp, sq = frame(sa)
@@ -241,7 +276,6 @@ def load_mjcf(path: str, **options) -> KinematicModel:
         b.children = [read_body(c, childclass) for c in elem if c.tag == "body"]
         return b
 
-    world = root.find("worldbody")
     tops = [read_body(e, None) for e in world if e.tag == "body"]
     if len(tops) != 1:
         raise ValueError("exactly one robot body under <worldbody> is expected")
@@ -251,7 +285,7 @@ def load_mjcf(path: str, **options) -> KinematicModel:
         kept = []
         for c in b.children:
             weld(c)
-            if c.joint is not None:
+            if c.joints:
                 kept.append(c)
                 continue
             R = quat_to_mat(c.quat)
@@ -264,7 +298,7 @@ def load_mjcf(path: str, **options) -> KinematicModel:
         b.children = kept
 
     top = tops[0]
-    if top.joint is None:
+    if not top.joints:
         raise ValueError("the robot's top body needs a joint (a fixed base is outside the model subset)")
     weld(top)
 
@@ -289,22 +323,31 @@ def load_mjcf(path: str, **options) -> KinematicModel:
         options.setdefault("friction", fr)
         options.setdefault("solref", sr)
         options.setdefault("solimp", si)
-        # the joints keep MuJoCo's defaults for their limit and friction rows
-        options.setdefault("dof_solref", (0.02, 1.0))
-        options.setdefault("dof_solimp", (0.9, 0.95, 0.001, 0.5, 2.0))
+    # the joints' limit rows: solreflimit / solimplimit, MuJoCo's defaults when absent (friction rows use the same pair here)
+    if len(set(limit_params)) > 1:
+        raise ValueError("the limited joints must share solreflimit and solimplimit")
+    jr, ji = limit_params[0] if limit_params else ((0.02, 1.0), (0.9, 0.95, 0.001, 0.5, 2.0))
+    options.setdefault("dof_solref", jr)
+    options.setdefault("dof_solimp", ji)
     mb = ModelBuilder(**options)
     joint_body: dict[str, int] = {}
 
     def add(b, parent):
         m, com, inertia, iquat = composite(b.parts)
-        j = b.joint
-        if j["type"] == "free":
-            idx = mb.add_body(parent, b.pos, joint="free", quat=b.quat, mass=m, ipos=com, iquat=iquat, inertia=inertia, name=b.name)
-        else:
-            idx = mb.add_body(parent, b.pos, joint="hinge", axis=j["axis"], joint_pos=j["pos"], quat=b.quat, mass=m, ipos=com,
-                              iquat=iquat, inertia=inertia, damping=j["damping"], armature=j["armature"], range=j["range"],
-                              frictionloss=j["frictionloss"], name=b.name)
-        joint_body[j["name"]] = idx
+        idx = parent
+        for k, j in enumerate(b.joints):
+            last = k == len(b.joints) - 1
+            pos, quat = (b.pos, b.quat) if k == 0 else (np.zeros(3), np.array([1.0, 0, 0, 0]))
+            # all but the last joint move a massless body at the same place; the last one carries the body itself
+            mass = dict(mass=m, ipos=com, iquat=iquat, inertia=inertia) if last else dict(mass=0.0, inertia=np.zeros(3))
+            name = b.name if last else f"{b.name}#{j['name']}"
+            if j["type"] == "free":
+                idx = mb.add_body(idx, pos, joint="free", quat=quat, name=name, **mass)
+            else:
+                idx = mb.add_body(idx, pos, joint="hinge", axis=j["axis"], joint_pos=j["pos"], quat=quat, damping=j["damping"],
+                                  armature=j["armature"], range=j["range"], frictionloss=j["frictionloss"],
+                                  stiffness=j["stiffness"], name=name, **mass)
+            joint_body[j["name"]] = idx
         for p, r, n in b.spheres:
             mb.add_contact_sphere(idx, p, r, name=n or None)
         for n, p, q in b.sites:

@@ -125,6 +125,7 @@ class KinematicModel:
     # solref / solimp of the limit and friction rows (MuJoCo: per joint, its defaults here unless given)
     dof_solref: np.ndarray
     dof_solimp: np.ndarray
+    dof_stiffness: np.ndarray  # joint springs of hinges about qpos0
     # actuators (motors: force = gear * clip(ctrl, ctrlrange))
     act_dof: np.ndarray
     act_gear: np.ndarray
@@ -183,7 +184,7 @@ class ModelBuilder:
         self.bodies = [dict(parent=-1, jtype=JNT_NONE, pos=np.zeros(3), quat=np.array([1.0, 0, 0, 0]), mass=0.0,
                             ipos=np.zeros(3), iquat=np.array([1.0, 0, 0, 0]), inertia=np.zeros(3),
                             axis=np.array([0.0, 0, 1]), jpos=np.zeros(3), damping=0.0, armature=0.0, qpos0=0.0,
-                            range=None, frictionloss=0.0, name="world")]
+                            range=None, frictionloss=0.0, stiffness=0.0, name="world")]
         self.actuators: list[dict] = []
         self.spheres: list[dict] = []
         self.sites: dict = {}
@@ -192,7 +193,7 @@ class ModelBuilder:
     def add_body(self, parent: int, pos, *, joint: str | None = "hinge", axis=(0.0, 1.0, 0.0),
                  joint_pos=(0.0, 0.0, 0.0), quat=(1.0, 0.0, 0.0, 0.0), mass: float, ipos=(0.0, 0.0, 0.0),
                  iquat=(1.0, 0.0, 0.0, 0.0), inertia, damping=0.0, armature=0.0, range=None, frictionloss=0.0,
-                 name: str | None = None) -> int:
+                 stiffness=0.0, name: str | None = None) -> int:
         b = len(self.bodies)
         if not (0 <= parent < b):
             raise ValueError(f"parent {parent} does not exist")
@@ -224,7 +225,7 @@ class ModelBuilder:
                                 iquat=iq / np.linalg.norm(iq), inertia=np.array(inertia, dtype=np.float64), axis=ax,
                                 jpos=np.array(joint_pos, dtype=np.float64), damping=float(damping),
                                 armature=float(armature), qpos0=0.0, range=range, frictionloss=float(frictionloss),
-                                name=name or f"body{b}"))
+                                stiffness=float(stiffness), name=name or f"body{b}"))
         return b
 
     def add_capsule_body(self, parent: int, pos, direction, length: float, radius: float, mass: float, **kw) -> int:
@@ -275,7 +276,7 @@ class ModelBuilder:
         for b in range(nb - 1, 0, -1):
             subtree_end[parent[b]] = max(subtree_end[parent[b]], subtree_end[b])
         dof_body, dof_parent = np.zeros(nv, np.int32), np.full(nv, -1, np.int32)
-        damping, armature, frictionloss = np.zeros(nv), np.zeros(nv), np.zeros(nv)
+        damping, armature, frictionloss, stiffness = np.zeros(nv), np.zeros(nv), np.zeros(nv), np.zeros(nv)
         limited, jrange = np.zeros(nb, np.int32), np.zeros((nb, 2))
 
         def last_dof_of(body: int) -> int:
@@ -300,6 +301,7 @@ class ModelBuilder:
                 dof_parent[i] = last_dof_of(int(parent[b]))
                 damping[i], armature[i] = body["damping"], body["armature"]
                 frictionloss[i] = body["frictionloss"]
+                stiffness[i] = body["stiffness"]
                 if body["range"] is not None:
                     limited[b], jrange[b] = 1, body["range"]
         qpos0 = np.zeros(nq)
@@ -317,7 +319,7 @@ class ModelBuilder:
             body_mass=stack("mass"), body_ipos=stack("ipos"), body_iquat=stack("iquat"),
             body_inertia=stack("inertia"), jnt_axis=stack("axis"), jnt_pos=stack("jpos"), qpos0=qpos0,
             dof_body=dof_body, dof_parent=dof_parent, dof_damping=damping, dof_armature=armature,
-            jnt_limited=limited, jnt_range=jrange, dof_frictionloss=frictionloss,
+            jnt_limited=limited, jnt_range=jrange, dof_frictionloss=frictionloss, dof_stiffness=stiffness,
             act_dof=np.array([dofadr[a["body"]] for a in self.actuators], np.int32).reshape(nu),
             act_gear=np.array([a["gear"] for a in self.actuators], np.float64).reshape(nu),
             act_ctrlrange=np.array([[a["lo"], a["hi"]] for a in self.actuators], np.float64).reshape(nu, 2),
@@ -422,7 +424,7 @@ def _compile_constants(m: dict):
 # --------------------------------------------------------------------------- procedural models of the benchmark configs
 def pendulum_chain_model(n_links: int = 3, length: float = 0.5, radius: float = 0.05, mass: float = 1.0,
                          damping: float = 0.1, dt: float = 0.005, joint_range=None, frictionloss: float = 0.0,
-                         **opts) -> KinematicModel:
+                         stiffness: float = 0.0, **opts) -> KinematicModel:
     """Planar hinge chain hanging from the world origin along -z, hinge axes along y, no contacts."""
     mb = ModelBuilder(dt=dt, **opts)
     parent = 0
@@ -430,7 +432,7 @@ def pendulum_chain_model(n_links: int = 3, length: float = 0.5, radius: float = 
         pos = (0.0, 0.0, 0.0) if i == 0 else (0.0, 0.0, -length)
         parent = mb.add_capsule_body(parent, pos, (0.0, 0.0, -1.0), length, radius, mass, joint="hinge",
                                      axis=(0.0, 1.0, 0.0), damping=damping, range=joint_range,
-                                     frictionloss=frictionloss, name=f"link{i}")
+                                     frictionloss=frictionloss, stiffness=stiffness, name=f"link{i}")
         mb.add_actuator(parent)
     return mb.build()
 

@@ -40,6 +40,7 @@ class KsorModel(ctypes.Structure):
         ("dof_armature", c_double * MAXV),
         ("jnt_limited", c_int * MAXB), ("jnt_range", c_double * 2 * MAXB), ("dof_invweight0", c_double * MAXV),
         ("dof_frictionloss", c_double * MAXV), ("dof_solref", c_double * 2), ("dof_solimp", c_double * 5),
+        ("dof_stiffness", c_double * MAXV),
         ("act_dof", c_int * MAXU), ("act_gear", c_double * MAXU), ("act_lo", c_double * MAXU),
         ("act_hi", c_double * MAXU),
         ("sph_body", c_int * MAXS), ("sph_pos", c_double * 3 * MAXS), ("sph_radius", c_double * MAXS),
@@ -105,7 +106,7 @@ def make_model(a: dict) -> KsorModel:
     for k in ("body_pos", "body_quat", "body_ipos", "body_iquat", "body_inertia", "jnt_axis", "jnt_pos", "sph_pos"):
         fill(k, a[k])
     fill("body_invweight0", np.asarray(a["body_invweight0"])[:, 0])
-    for k in ("jnt_limited", "jnt_range", "dof_invweight0", "dof_frictionloss", "dof_solref", "dof_solimp"):
+    for k in ("jnt_limited", "jnt_range", "dof_invweight0", "dof_frictionloss", "dof_solref", "dof_solimp", "dof_stiffness"):
         if k in a:  # absent: no limits, no dry friction
             fill(k, a[k])
     fill("act_lo", np.asarray(a["act_ctrlrange"]).reshape(-1, 2)[:, 0])

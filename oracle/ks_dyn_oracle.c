@@ -688,6 +688,11 @@ void FN(ksor_forward)(const KsorModel* m, Data* d) {
   FN(ksor_com_vel)(m, d);
   FN(ksor_rne)(m, d);
   for (int i = 0; i < nv; ++i) { d->qfrc_passive[i] = -(REAL)m->dof_damping[i] * d->damping_scale[i] * d->qvel[i]; d->qfrc_actuator[i] = 0; }
+  for (int b = 1; b < m->nb; ++b) { /* joint springs (hinges): the spring's rest position is the joint's qpos0 */
+    if (m->body_jtype[b] != KSOR_JNT_HINGE) continue;
+    const int j = m->body_dofadr[b], qa = m->body_qadr[b];
+    d->qfrc_passive[j] -= (REAL)m->dof_stiffness[j] * (d->qpos[qa] - (REAL)m->qpos0[qa]);
+  }
   for (int u = 0; u < m->nu; ++u) {
     REAL c = d->ctrl[u];
     if (c < (REAL)m->act_lo[u]) c = (REAL)m->act_lo[u];

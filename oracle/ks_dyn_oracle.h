@@ -43,6 +43,7 @@ typedef struct KsorModel {
   int jnt_limited[KSOR_MAXB];
   double jnt_range[KSOR_MAXB][2], dof_invweight0[KSOR_MAXV], dof_frictionloss[KSOR_MAXV];
   double dof_solref[2], dof_solimp[5]; /* solref / solimp of the limit and friction rows; all zero = those of the contacts */
+  double dof_stiffness[KSOR_MAXV];     /* joint springs about qpos0: passive force -stiffness (q - qpos0) on hinges */
   int act_dof[KSOR_MAXU];
   double act_gear[KSOR_MAXU], act_lo[KSOR_MAXU], act_hi[KSOR_MAXU];
   int sph_body[KSOR_MAXS];

@@ -24,6 +24,8 @@ MODELS = {"chain": km.pendulum_chain_model, "humanoid": km.humanoid_model, "kbot
           # states draw hinge angles from U(-0.6, 0.6), so about a fifth of the joints start up to 0.15 rad beyond a limit
           # (much deeper violations make the cost so large that its fp32 rounding hides the last Newton improvements).
           "chain-friction": lambda: km.pendulum_chain_model(integrator="implicitfast", frictionloss=0.3),
+          # joint springs about the reference angles (a passive force)
+          "chain-springs": lambda: km.pendulum_chain_model(integrator="implicitfast", damping=0.2, stiffness=6.0),
           "humanoid-limits": lambda: km.humanoid_model(joint_range=(-0.45, 0.5)),
           "kbot-limits": lambda: km.kbot_scale_model(integrator="implicitfast", joint_range=(-0.45, 0.5), frictionloss=0.2),
           # the real K-Bot's contact parameters (robot.mjcf:24): five times stiffer rows than MuJoCo's defaults
@@ -555,6 +557,54 @@ def test_model_loaded_from_mjcf_matches_oracle():
     for e in range(N):
         d = orc.data(qpos[e], qvel[e])
         d.ctrl = ctrl[e]
+        for _ in range(10):
+            orc.step(d)
+        wq.append(np.array(d.qpos)); wv.append(np.array(d.qvel))
+    buf = dict(qpos=t32(qpos), qvel=t32(qvel), qacc_warmstart=zeros(N, m.nv), time=zeros(N), last_ctrl=t32(ctrl), action=t32(ctrl))
+    for _ in range(10):
+        physics.control_step(dm, buf, substeps=1, actuator_type=KS_ACT_TORQUE)
+    eq, ev = rel_err(buf["qpos"].cpu().numpy(), wq).max(), rel_err(buf["qvel"].cpu().numpy(), wv).max()
+    assert eq <= TEN_STEP_TOL and ev <= TEN_STEP_TOL, f"qpos {eq:.2e} qvel {ev:.2e}"
+
+
+def test_humanoid_file_with_several_hinges_per_body_matches_oracle():
+    """A model of the walking example's kind read from an MJCF file: bodies with three hinges (massless bodies in between),
+    joint springs, limit rows with their own solimp, feet that collide through explicit pairs; forward quantities and ten
+    physics steps against the oracle."""
+    import os
+    from ksim_amd import physics
+    from ksim_amd._lib_dyn import KS_ACT_TORQUE
+    from ksim_amd.mjcf import load_mjcf
+
+    m = load_mjcf(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "mini_humanoid.mjcf"), integrator="implicitfast")
+    dm = physics.DeviceModel(m)
+    N = 40
+    rng = np.random.default_rng(91)
+    qpos, qvel = random_states(m, N, seed=92, vel_scale=0.3, joint_range=0.3)
+    # knees from bent to slightly beyond their upper limit of 5 degrees, some hips slightly beyond theirs
+    qpos[:, 10] = rng.uniform(-1.2, 0.05, N); qpos[:, 14] = rng.uniform(-1.2, 0.05, N)
+    qpos[0::3, 10] = rng.uniform(0.09, 0.14, len(qpos[0::3])); qpos[1::3, 14] = rng.uniform(0.09, 0.12, len(qpos[1::3]))
+    qpos[2::4, 7] = rng.uniform(0.35, 0.4, len(qpos[2::4]))
+    ctrl = rng.normal(size=(N, m.nu)) * 0.5
+    warm = np.zeros((N, m.nv))
+    want = oracle_forward(m, qpos, qvel, ctrl, None, None, warm)
+    buf = dict(qpos=t32(qpos), qvel=t32(qvel), qacc_warmstart=t32(warm), ctrl_in=t32(ctrl), qacc=zeros(N, m.nv),
+               xpos=zeros(N, m.nb * 3), xquat=zeros(N, m.nb * 4), nefc=zeros(N, dtype=torch.int32), contact_dist=zeros(N, m.ns),
+               dbg_M=zeros(N, m.nv * m.nv), dbg_qacc_smooth=zeros(N, m.nv))
+    physics.forward(dm, buf)
+    assert rel_err(buf["xpos"].cpu().numpy(), want["xpos"]).max() < 1e-5
+    assert rel_err(buf["xquat"].cpu().numpy(), want["xquat"]).max() < 1e-5
+    assert rel_err(buf["dbg_M"].cpu().numpy(), want["M"]).max() < 1e-5
+    assert rel_err(buf["dbg_qacc_smooth"].cpu().numpy(), want["qacc_smooth"]).max() <= ONE_STEP_TOL  # springs included
+    assert np.array_equal(buf["nefc"].cpu().numpy(), want["nefc"])
+    assert (want["nefc"] > 0).sum() >= N // 2
+    err = rel_err(buf["qacc"].cpu().numpy(), want["qacc"]).max()
+    assert err <= ONE_STEP_TOL, f"qacc {err:.2e}"
+    orc = Oracle(m.arrays())
+    wq, wv = [], []
+    for e in range(N):
+        d = orc.data(qpos[e], qvel[e])
+        d.ctrl = ctrl[e]  # clipped to the motors' control range and geared inside the model
         for _ in range(10):
             orc.step(d)
         wq.append(np.array(d.qpos)); wv.append(np.array(d.qvel))

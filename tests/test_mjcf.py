@@ -154,3 +154,128 @@ def test_sites_and_sensors_are_read_through_the_welds():
     with pytest.raises(ValueError, match="not built"):
         SensorObservation.create(physics_model=m, sensor_name="imu_quat")
     assert SensorObservation.create(physics_model=m, sensor_name="imu_gyro").get_name() == "imu_gyro"
+
+
+HUMANOID_MINI = os.path.join(HERE, "golden", "mini_humanoid.mjcf")
+SCENE = "/root/reference/examples/data/scene.mjcf"
+
+
+def test_mini_humanoid_several_hinges_on_one_body():
+    """A body with three hinges becomes two massless bodies and the body itself; the joints act in file order, so the
+    thigh's orientation is R_x(q1) R_z(q2) R_y(q3) about the common anchor, and everything below hangs from that."""
+    m = load_mjcf(HUMANOID_MINI)
+    assert (m.nb, m.nq, m.nv, m.nu, m.ns) == (10, 15, 14, 8, 2)
+    names = list(m.body_names)
+    assert names[2:5] == ["thigh_right#hip_x_right", "thigh_right#hip_z_right", "thigh_right"]
+    assert m.body_mass[2] == 0 and m.body_mass[3] == 0 and m.body_mass[4] > 0
+    # degrees -> radians, class ranges, springs (the knee's class switches its spring off), shared limit-row parameters
+    np.testing.assert_allclose(m.jnt_range[2:6], np.deg2rad([[-30, 20], [-50, 40], [-120, 30], [-150, 5]]))
+    np.testing.assert_allclose(m.dof_stiffness[6:10], [8, 8, 8, 0])
+    np.testing.assert_allclose(m.dof_damping[6:10], [4, 4, 4, 0.3])
+    np.testing.assert_allclose(m.dof_armature[6:], 0.02)
+    assert tuple(m.dof_solref) == (0.02, 1.0) and tuple(m.dof_solimp) == (0.0, 0.99, 0.01, 0.5, 2.0)
+    # the feet collide through their explicit pairs only, with a pair's own defaults (not the geoms' class values)
+    assert list(m.sph_names) == ["foot_right", "foot_left"]
+    assert m.friction == 1.0 and tuple(m.solref) == (0.02, 1.0) and tuple(m.solimp) == (0.9, 0.95, 0.001, 0.5, 2.0)
+    # gears follow the motors to the bodies that carry their joints
+    np.testing.assert_allclose(m.arrays()["act_gear"][:8], [40, 40, 120, 80] * 2)
+    np.testing.assert_array_equal(m.arrays()["act_dof"][:8], np.arange(6, 14))
+
+    rng = np.random.default_rng(5)
+    q = m.qpos0.copy()
+    q[7:] = rng.uniform(-0.5, 0.5, 8)
+    kin = km.host_kinematics(m.arrays(), q)
+    base = np.array([0, 0, 0.83])
+    for side, sy, ax in ((0, -1.0, 1.0), (1, 1.0, -1.0)):
+        a = q[7 + 4 * side: 11 + 4 * side]
+        R = (Rotation.from_rotvec([ax * a[0], 0, 0]) * Rotation.from_rotvec([0, 0, ax * a[1]]) * Rotation.from_rotvec([0, a[2], 0]))
+        thigh = 4 + 4 * side
+        hip = base + np.array([0, 0.1 * sy, -0.04])
+        np.testing.assert_allclose(kin["xpos"][thigh], hip, atol=1e-12)
+        np.testing.assert_allclose(kin["xmat"][thigh], R.as_matrix(), atol=1e-12)
+        # the knee turns about -y through an anchor 2 cm above the shin's origin
+        Rk = R * Rotation.from_rotvec([0, -a[3], 0])
+        anchor = hip + R.apply([0, -0.01 * sy, -0.4] + np.array([0, 0, 0.02]))
+        shin = anchor - Rk.apply([0, 0, 0.02])
+        np.testing.assert_allclose(kin["xpos"][thigh + 1], shin, atol=1e-12)
+        foot = kin["xpos"][thigh + 1] + kin["xmat"][thigh + 1] @ m.sph_pos[side]
+        np.testing.assert_allclose(foot, shin + Rk.apply([0, 0, -0.35]), atol=1e-12)
+
+
+def test_mini_humanoid_inertia_from_class_geoms():
+    """Masses from the geoms' volumes at the default density (sizes and end points partly from default classes), the
+    foot's sphere welded into the shin, and the composite shin's centre of mass by hand."""
+    m = load_mjcf(HUMANOID_MINI)
+    cap = lambda r, length: 1000 * (np.pi * r * r * length + 4 / 3 * np.pi * r**3)  # noqa: E731
+    ball = 1000 * 4 / 3 * np.pi * 0.05**3
+    thigh = cap(0.05, np.hypot(0.01, 0.34))
+    shin = cap(0.04, 0.3)
+    assert m.body_mass[1] == pytest.approx(cap(0.08, 0.16), rel=1e-12)
+    assert m.body_mass[4] == pytest.approx(thigh, rel=1e-12) and m.body_mass[8] == pytest.approx(thigh, rel=1e-12)
+    assert m.body_mass[5] == pytest.approx(shin + ball, rel=1e-12)
+    np.testing.assert_allclose(m.body_ipos[5], [0, 0, (shin * -0.15 + ball * -0.35) / (shin + ball)], atol=1e-12)
+    np.testing.assert_allclose(m.body_ipos[4], [0, 0.005, -0.17], atol=1e-12)
+    # the shin's inertia about its centre of mass: capsule + sphere through the parallel-axis theorem (z is the long axis)
+    r, h = 0.04, 0.3
+    mc, mh = 1000 * np.pi * r * r * h, 1000 * 4 / 3 * np.pi * r**3
+    izz = mc * r * r / 2 + mh * 2 * r * r / 5
+    ixx = mc * (r * r / 4 + h * h / 12) + mh * (2 * r * r / 5 + h * h / 4 + 3 * h * r / 8)
+    zc = m.body_ipos[5][2]
+    ixx_tot = ixx + shin * (zc + 0.15) ** 2 + ball * 2 / 5 * 0.05**2 + ball * (zc + 0.35) ** 2
+    izz_tot = izz + ball * 2 / 5 * 0.05**2
+    np.testing.assert_allclose(sorted(m.body_inertia[5]), sorted([ixx_tot, ixx_tot, izz_tot]), rtol=1e-10)
+
+
+def test_mini_humanoid_runs_and_springs_pull_back():
+    """The loaded model steps in the oracle; with gravity off and the base held high, a displaced hip joint accelerates
+    back toward its reference angle at -k q / (effective inertia), sign checked per joint."""
+    m = load_mjcf(HUMANOID_MINI, gravity=(0, 0, 0))
+    orc = Oracle(m.arrays())
+    q = m.qpos0.copy()
+    q[2] = 3.0
+    q[7 + 2] = 0.3    # right hip_y
+    d = orc.data(qpos=q)
+    orc.forward(d)
+    assert d.nefc == 0
+    assert d.qfrc_passive[6 + 2] == pytest.approx(-8 * 0.3, rel=1e-12) and d.qacc[6 + 2] < 0
+    m = load_mjcf(HUMANOID_MINI)
+    orc = Oracle(m.arrays())
+    d = orc.data()
+    for _ in range(40):
+        orc.step(d)
+    assert np.isfinite(d.qpos).all()
+
+
+def test_mini_humanoid_outside_the_subset_raises(tmp_path):
+    text = open(HUMANOID_MINI).read()
+    for old, new, msg in [('<pair geom1="foot_left" geom2="floor" />', '<pair geom1="foot_left" geom2="foot_right" />', "floor plane"),
+                          ('<pair geom1="foot_left" geom2="floor" />', '<pair geom1="foot_left" geom2="floor" condim="1" />', "condim"),
+                          ('<joint pos="0 0 .02" axis="0 -1 0" range="-150 5" stiffness="0" />',
+                           '<joint pos="0 0 .02" axis="0 -1 0" range="-150 5" stiffness="0" solimplimit=".5 .9 .01" />', "share"),
+                          ('<joint name="hip_y_left" class="hip_y" />', '<joint name="hip_y_left" class="hip_y" springref="10" />', "springref")]:
+        assert old in text
+        p = tmp_path / "bad.mjcf"
+        p.write_text(text.replace(old, new, 1))
+        with pytest.raises(ValueError, match=msg):
+            load_mjcf(str(p))
+
+
+@pytest.mark.skipif(not os.path.exists(SCENE), reason="the reference tree is not present")
+def test_walking_example_scene_from_the_reference():
+    """examples/data/scene.mjcf, the humanoid of examples/walking.py: 17 hinges (abdomen 2+1, hips 3, shoulders 2) on a
+    floating base, 17 motors, two foot spheres that meet the floor through explicit pairs."""
+    m = load_mjcf(SCENE)
+    assert (m.nb, m.nq, m.nv, m.nu, m.ns) == (19, 24, 23, 17, 2)
+    assert list(m.sph_names) == ["foot_right", "foot_left"] and m.friction == 1.0
+    assert m.jnt_limited[2:].all() and tuple(m.dof_solimp[:3]) == (0.0, 0.99, 0.01)
+    np.testing.assert_allclose(m.dof_stiffness[6:9], [20, 10, 10])   # abdomen z (stiff class), y, x
+    assert sum(n.count("#") for n in m.body_names) == 1 + 2 * 2 + 2 * 1
+    kin = km.host_kinematics(m.arrays(), m.qpos0)
+    # at qpos0 the feet hang straight below the hips: 1.4 - .26 - .165 - .04 - .4 - .39 above the floor
+    for b, p in zip(m.sph_body, m.sph_pos):
+        assert (kin["xpos"][b] + kin["xmat"][b] @ p)[2] == pytest.approx(1.4 - 0.26 - 0.165 - 0.04 - 0.4 - 0.39, abs=1e-12)
+    orc = Oracle(m.arrays())
+    d = orc.data()
+    for _ in range(20):
+        orc.step(d)
+    assert np.isfinite(d.qpos).all()

@@ -572,3 +572,29 @@ def test_per_env_model_field_overrides_equal_a_model_built_with_them():
     assert not np.allclose(d1.qvel, d0.qvel, rtol=1e-6)  # and they do change the motion
     with pytest.raises(ValueError):
         o1.data(qpos, qvel, sph_pos=spos)
+
+
+def test_joint_spring_closed_forms():
+    """A hinge with a spring about qpos0, no gravity, no damping: the restoring acceleration is -k q / I and the motion is
+    harmonic with frequency sqrt(k / I); in gravity a link settles where the spring torque balances the weight."""
+    k = 3.0
+    m = km.pendulum_chain_model(n_links=1, damping=0.0, stiffness=k, gravity=(0.0, 0.0, 0.0), dt=0.0005)
+    orc = Oracle(m.arrays())
+    d = orc.data(np.array([0.2]), np.zeros(1))
+    orc.forward(d)
+    inertia = float(d.M[0, 0])
+    assert d.qacc[0] == pytest.approx(-k * 0.2 / inertia, rel=1e-12)
+    w = np.sqrt(k / inertia)
+    steps = int(round(0.75 * 2 * np.pi / w / m.dt))  # three quarters of a period: q ~ 0, moving up
+    for _ in range(steps):
+        orc.step(d)
+    t = steps * m.dt
+    assert d.qpos[0] == pytest.approx(0.2 * np.cos(w * t), abs=1e-3) and d.qvel[0] == pytest.approx(-0.2 * w * np.sin(w * t), rel=2e-3)  # semi-implicit Euler: phase error of order dt
+    # static balance against gravity: k q = m g (L / 2) sin q
+    mg = km.pendulum_chain_model(n_links=1, length=0.5, mass=1.0, damping=2.0, stiffness=4.0)
+    og = Oracle(mg.arrays())
+    dg = og.data(np.array([1.2]), np.zeros(1))
+    for _ in range(6000):
+        og.step(dg)
+    q = float(dg.qpos[0])
+    assert abs(dg.qvel[0]) < 1e-8 and 4.0 * q == pytest.approx(-1.0 * 9.81 * 0.25 * np.sin(q), rel=1e-6)
