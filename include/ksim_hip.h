@@ -641,6 +641,18 @@ int ks_mlp_train_backward_dx(KsMlp* mlp, ks_stream_t stream, int64_t M, const fl
                              void* workspace);
 /* The first `count` bias entries of a layer are constants: the optimiser and the gradient norm skip them. */
 int ks_mlp_freeze_bias_prefix(KsMlp* mlp, int32_t layer, int32_t count);
+
+/* ksim/task/amp.py:360-438 (get_disc_losses, _grad_penalty, _get_amp_disc_loss_and_metrics): gradient of the AMP
+ * discriminator's loss
+ *   0.5 sum (D(real) - 1)^2 + 0.5 sum (D(sim) + 1)^2 + grad_penalty_coef / 2 * mean_motions sum_frames |dD/dx (real frame)|^2
+ * with respect to every weight and bias of the discriminator, an MLP with one output applied to each frame (ELU, ReLU, tanh or
+ * no activation), into the handle's gradient buffers (then ks_mlp_grad_sqnorm / ks_mlp_adam_step as for any network).
+ * real (n_real, in) holds n_motions reference motions of n_real / n_motions frames each, sim (n_sim, in) the frames of
+ * the simulated trajectories.  losses[3] (device) receives the real, simulated and penalty terms.  Computed in fp32 on the
+ * master weights whatever the network's working precision. */
+int64_t ks_mlp_disc_workspace_bytes(const KsMlp* mlp, int64_t n_real, int64_t n_sim);
+int ks_mlp_disc_loss_grad(KsMlp* mlp, ks_stream_t stream, int64_t n_real, const float* real, int64_t n_sim, const float* sim,
+                          float grad_penalty_coef, int64_t n_motions, float* losses, void* workspace);
 int ks_grad_sqnorm(ks_stream_t stream, int64_t n, const float* g, double* acc);
 int ks_mlp_grad_sqnorm(const KsMlp* mlp, ks_stream_t stream, double* acc);
 int ks_mlp_adam_step(KsMlp* mlp, ks_stream_t stream, const KsAdamParams* params /*host*/, const double* sqnorm);

@@ -235,6 +235,10 @@ def bind(lib) -> None:
                  "ks_lstm_train_init", "ks_lstm_projections", "ks_lstm_train_forward", "ks_lstm_backward_step",
                  "ks_lstm_grad_sqnorm", "ks_lstm_adam_step"):
         getattr(lib, name).restype = c_int32
+    lib.ks_mlp_disc_workspace_bytes.argtypes = [c_void_p, c_int64, c_int64]
+    lib.ks_mlp_disc_workspace_bytes.restype = c_int64
+    lib.ks_mlp_disc_loss_grad.argtypes = [c_void_p, c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_float, c_int64, c_void_p, c_void_p]
+    lib.ks_mlp_disc_loss_grad.restype = c_int32
     lib.ks_mlp_grad_sqnorm.argtypes = [c_void_p, c_void_p, c_void_p]
     lib.ks_mlp_adam_step.argtypes = [c_void_p, c_void_p, POINTER(KsAdamParams), c_void_p]
     lib.ks_adam_step.argtypes = [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, POINTER(KsAdamParams), c_void_p]

@@ -1375,6 +1375,337 @@ extern "C" int ks_mlp_adam_step(KsMlp* h, ks_stream_t stream, const KsAdamParams
   return check_launch("ks_mlp_adam_step");
 }
 
+// ---------------------------------------------------------------- discriminator update (ksim/task/amp.py:360-438)
+// Gradient of   0.5 sum (D(real) - 1)^2 + 0.5 sum (D(sim) + 1)^2 + coef / 2 * mean_b sum_t |grad_x D(real[b, t])|^2
+// with respect to every weight and bias of an MLP D with one output, applied frame by frame.  The last term differentiates
+// the network twice.  With z_l = W_l y_{l-1} + b_l, y_l = f(z_l), the input gradient is g = W_1^T d_1 with d_L = 1,
+// d_l = f'(z_l) * (W_{l+1}^T d_{l+1}) =: f'(z_l) * a_l.  The gradient of P(g) walks that computation backwards, which is a
+// forward sweep through the layers: with v_0 = dP/dg,
+//   dP/dW_l += d_l^T v_{l-1},   u_l = v_{l-1} W_l^T,   v_l = u_l * f'(z_l),   r_l = u_l * a_l * f''(z_l),
+// and r_l, the part that reaches z_l through f', joins the ordinary backward pass of the squared-error terms as an extra
+// gradient of z_l on the real rows.  The discriminator is small next to the policy, so everything here runs in fp32 on the
+// master weights with a plain LDS-tiled product.
+namespace ks {
+
+// C(i, j) (+)= sum_k A(i, k) B(k, j): 64 x 64 tile per workgroup, 16-deep slices through LDS, 4 x 4 outputs per thread.
+// A_KC: A is stored (i, k) with k contiguous, otherwise (k, i); B_KC: B is stored (j, k) with k contiguous, otherwise (k, j).
+// gridDim.z cuts the k range into slices of kslice; with more than one slice, slice z writes its partial product (M, N)
+// densely to C + z * M * N and sum_slices_kernel adds them up in a fixed order.
+template <bool A_KC, bool B_KC>
+__global__ __launch_bounds__(256) void sgemm_kernel(int M, int N, int K, const float* __restrict__ A, int64_t lda,
+                                                    const float* __restrict__ B, int64_t ldb, float* __restrict__ C, int64_t ldc,
+                                                    int kslice, const float* __restrict__ bias, int act, int accumulate) {
+  __shared__ float As[16][68];
+  __shared__ float Bs[16][68];
+  const int t = threadIdx.x, i0 = blockIdx.y * 64, j0 = blockIdx.x * 64;
+  const int kbeg = blockIdx.z * kslice, kend = min(K, kbeg + kslice);
+  const int ti = t / 16, tj = t % 16;
+  float acc[4][4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r)
+#pragma unroll
+    for (int c = 0; c < 4; ++c) acc[r][c] = 0.f;
+  for (int k0 = kbeg; k0 < kend; k0 += 16) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int ka = A_KC ? t % 16 : t / 64 + 4 * r, ia = A_KC ? t / 16 + 16 * r : t % 64;
+      const int gi = i0 + ia, gka = k0 + ka;
+      As[ka][ia] = (gi < M && gka < kend) ? (A_KC ? A[(int64_t)gi * lda + gka] : A[(int64_t)gka * lda + gi]) : 0.f;
+      const int kb = B_KC ? t % 16 : t / 64 + 4 * r, jb = B_KC ? t / 16 + 16 * r : t % 64;
+      const int gj = j0 + jb, gkb = k0 + kb;
+      Bs[kb][jb] = (gj < N && gkb < kend) ? (B_KC ? B[(int64_t)gj * ldb + gkb] : B[(int64_t)gkb * ldb + gj]) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < 16; ++k) {
+      float a[4], b[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) { a[r] = As[k][ti * 4 + r]; b[r] = Bs[k][tj * 4 + r]; }
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+#pragma unroll
+        for (int c = 0; c < 4; ++c) acc[r][c] = fmaf(a[r], b[c], acc[r][c]);
+    }
+    __syncthreads();
+  }
+  const bool sliced = gridDim.z > 1;
+  float* out = sliced ? C + (int64_t)blockIdx.z * M * N : C;
+  const int64_t ld = sliced ? N : ldc;
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int gi = i0 + ti * 4 + r;
+    if (gi >= M) continue;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const int gj = j0 + tj * 4 + c;
+      if (gj >= N) continue;
+      float v = acc[r][c];
+      if (!sliced) {
+        if (bias) v += bias[gj];
+        if (act == KS_ACT_ELU) v = v > 0.f ? v : expm1f(v);
+        else if (act == KS_ACT_RELU) v = fmaxf(v, 0.f);
+        else if (act == KS_ACT_TANH) v = tanhf(v);
+        if (accumulate) v += out[(int64_t)gi * ld + gj];
+      }
+      out[(int64_t)gi * ld + gj] = v;
+    }
+  }
+}
+
+__global__ __launch_bounds__(256) void sum_slices_kernel(int M, int N, int nz, const float* __restrict__ part, float* __restrict__ C,
+                                                         int64_t ldc, int accumulate) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= (int64_t)M * N) return;
+  float s = 0.f;
+  for (int z = 0; z < nz; ++z) s += part[(int64_t)z * M * N + idx];
+  const int i = (int)(idx / N), j = (int)(idx - (int64_t)i * N);
+  C[(int64_t)i * ldc + j] = accumulate ? C[(int64_t)i * ldc + j] + s : s;
+}
+
+__global__ __launch_bounds__(256) void fill_kernel(int64_t n, float v, float* __restrict__ p) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx < n) p[idx] = v;
+}
+
+// first and second derivative of the activation from its output y = f(z)
+__device__ __forceinline__ void act_derivatives(int act, float y, float& d1, float& d2) {
+  d1 = 1.f; d2 = 0.f;
+  if (act == KS_ACT_ELU) { if (y <= 0.f) { d1 = y + 1.f; d2 = y + 1.f; } }  // exp(z) = elu(z) + 1 for z <= 0
+  else if (act == KS_ACT_RELU) d1 = y > 0.f ? 1.f : 0.f;
+  else if (act == KS_ACT_TANH) { d1 = 1.f - y * y; d2 = -2.f * y * d1; }
+}
+
+// dz = out - target (target +1 on the first n_real rows, -1 on the rest) and the two squared-error sums (one workgroup)
+__global__ __launch_bounds__(1024) void disc_signal_kernel(int64_t n_real, int64_t n, const float* __restrict__ out, float* __restrict__ dz,
+                                                           float* __restrict__ losses) {
+  __shared__ double sh[2][1024];
+  double a = 0.0, b = 0.0;
+  for (int64_t i = threadIdx.x; i < n; i += 1024) {
+    const float e = out[i] - (i < n_real ? 1.f : -1.f);
+    dz[i] = e;
+    if (i < n_real) a += 0.5 * (double)e * e; else b += 0.5 * (double)e * e;
+  }
+  sh[0][threadIdx.x] = a; sh[1][threadIdx.x] = b;
+  __syncthreads();
+  for (int w = 512; w > 0; w >>= 1) {
+    if ((int)threadIdx.x < w) { sh[0][threadIdx.x] += sh[0][threadIdx.x + w]; sh[1][threadIdx.x] += sh[1][threadIdx.x + w]; }
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) { losses[0] = (float)sh[0][0]; losses[1] = (float)sh[1][0]; }
+}
+
+// penalty value coef / 2 * sum g^2 / n_motions and, in place, its gradient v = coef / n_motions * g (one workgroup)
+__global__ __launch_bounds__(1024) void disc_penalty_kernel(int64_t n, float coef, float inv_motions, float* __restrict__ g,
+                                                            float* __restrict__ loss) {
+  __shared__ double sh[1024];
+  double a = 0.0;
+  for (int64_t i = threadIdx.x; i < n; i += 1024) {
+    const float v = g[i];
+    a += (double)v * v;
+    g[i] = coef * inv_motions * v;
+  }
+  sh[threadIdx.x] = a;
+  __syncthreads();
+  for (int w = 512; w > 0; w >>= 1) {
+    if ((int)threadIdx.x < w) sh[threadIdx.x] += sh[threadIdx.x + w];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) *loss = (float)(0.5 * coef * inv_motions * sh[0]);
+}
+
+// d = f'(y) * a
+__global__ __launch_bounds__(256) void disc_delta_kernel(int64_t n, int act, const float* __restrict__ y, const float* __restrict__ a,
+                                                         float* __restrict__ d) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= n) return;
+  float d1, d2;
+  act_derivatives(act, y[idx], d1, d2);
+  d[idx] = d1 * a[idx];
+}
+
+// v = u * f'(y), r = u * a * f''(y)
+__global__ __launch_bounds__(256) void disc_tangent_kernel(int64_t n, int act, const float* __restrict__ y, const float* __restrict__ a,
+                                                           const float* __restrict__ u, float* __restrict__ v, float* __restrict__ r) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= n) return;
+  float d1, d2;
+  act_derivatives(act, y[idx], d1, d2);
+  const float uu = u[idx];
+  v[idx] = uu * d1;
+  r[idx] = uu * a[idx] * d2;
+}
+
+// dz = dy * f'(y) (+ r on the first n_extra elements)
+__global__ __launch_bounds__(256) void disc_dz_kernel(int64_t n, int64_t n_extra, int act, const float* __restrict__ y,
+                                                      const float* __restrict__ r, float* __restrict__ dz) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= n) return;
+  float d1, d2;
+  act_derivatives(act, y[idx], d1, d2);
+  float v = dz[idx] * d1;
+  if (idx < n_extra) v += r[idx];
+  dz[idx] = v;
+}
+
+}  // namespace ks
+
+constexpr int kDiscMaxSlices = 64;
+
+struct DiscWs {
+  float* y[KS_MAX_LAYERS];      // hidden outputs, all rows
+  float* a[KS_MAX_LAYERS];      // real rows: W_{l+1}^T d_{l+1}
+  float* d[KS_MAX_LAYERS];      // real rows: d_l
+  float* r[KS_MAX_LAYERS];      // real rows: extra gradient of z_l
+  float *out, *dz0, *dz1, *g, *u, *v, *ones, *part;
+};
+
+static int64_t carve_disc(const DevMlp& m, int64_t R, int64_t M, char* base, DiscWs* ws) {
+  int64_t off = 0;
+  auto take = [&](int64_t floats) {
+    char* p = base ? base + off : nullptr;
+    off += (floats * 4 + 255) / 256 * 256;
+    return (float*)p;
+  };
+  DiscWs w;
+  std::memset(&w, 0, sizeof(w));
+  int wmax = 1;
+  int64_t maxw = 1;
+  for (int l = 0; l <= m.n_layers; ++l) wmax = m.dims[l] > wmax ? m.dims[l] : wmax;
+  for (int l = 0; l < m.n_layers; ++l) maxw = (int64_t)m.dims[l] * m.dims[l + 1] > maxw ? (int64_t)m.dims[l] * m.dims[l + 1] : maxw;
+  for (int l = 0; l + 1 < m.n_layers; ++l) {
+    w.y[l] = take(M * m.dims[l + 1]);
+    w.a[l] = take(R * m.dims[l + 1]);
+    w.d[l] = take(R * m.dims[l + 1]);
+    w.r[l] = take(R * m.dims[l + 1]);
+  }
+  w.out = take(M);
+  w.dz0 = take(M * wmax);
+  w.dz1 = take(M * wmax);
+  w.g = take(R * m.dims[0]);
+  w.u = take(R * wmax);
+  w.v = take(R * wmax);
+  w.ones = take(M);
+  w.part = take(kDiscMaxSlices * maxw);
+  if (ws) *ws = w;
+  return off;
+}
+
+// launches one product; cuts the k range when the output alone would leave most of the chip idle
+template <bool A_KC, bool B_KC>
+static void sgemm(hipStream_t s, int64_t M, int N, int64_t K, const float* A, int64_t lda, const float* B, int64_t ldb, float* C,
+                  int64_t ldc, const float* bias, int act, bool accumulate, float* part) {
+  if (M <= 0 || N <= 0 || K <= 0) return;  // every caller with an empty sum adds into its output
+  const int64_t tiles = ((M + 63) / 64) * ((N + 63) / 64);
+  int slices = 1;
+  if (part && tiles < 128 && K >= 2048) {
+    slices = (int)((K + 511) / 512);
+    const int64_t want = (512 + tiles - 1) / tiles;
+    if (slices > want) slices = (int)want;
+    if (slices > kDiscMaxSlices) slices = kDiscMaxSlices;
+  }
+  int kslice = (int)((K + slices - 1) / slices);
+  kslice = (kslice + 15) / 16 * 16;
+  slices = (int)((K + kslice - 1) / kslice);
+  if (slices < 1) slices = 1;
+  hipLaunchKernelGGL((sgemm_kernel<A_KC, B_KC>), dim3((unsigned)((N + 63) / 64), (unsigned)((M + 63) / 64), (unsigned)slices), dim3(256), 0, s,
+                     (int)M, N, (int)K, A, lda, B, ldb, slices > 1 ? part : C, ldc, kslice, bias, act, accumulate ? 1 : 0);
+  if (slices > 1) {
+    const int64_t n = M * N;
+    hipLaunchKernelGGL(sum_slices_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, (int)M, N, slices, part, C, ldc, accumulate ? 1 : 0);
+  }
+}
+
+extern "C" int64_t ks_mlp_disc_workspace_bytes(const KsMlp* h, int64_t n_real, int64_t n_sim) {
+  if (!h || n_real < 0 || n_sim < 0) return 0;
+  return carve_disc(h->m, n_real, n_real + n_sim, nullptr, nullptr) + 256;
+}
+
+extern "C" int ks_mlp_disc_loss_grad(KsMlp* h, ks_stream_t stream, int64_t n_real, const float* real, int64_t n_sim, const float* sim,
+                                     float grad_penalty_coef, int64_t n_motions, float* losses, void* workspace) {
+  if (!h || !h->m.train) return fail(KS_EINVAL, "ks_mlp_disc_loss_grad: call ks_mlp_train_init first");
+  DevMlp& m = h->m;
+  const int L = m.n_layers, act = m.activation;
+  const int64_t R = n_real, M = n_real + n_sim;
+  if (m.dims[L] != 1) return fail(KS_EINVAL, "ks_mlp_disc_loss_grad: the discriminator must have one output, not %d", m.dims[L]);
+  if (act == KS_ACT_GELU) return fail(KS_EINVAL, "ks_mlp_disc_loss_grad: GELU is not supported here (ELU, ReLU, tanh or none)");
+  if (n_real < 0 || n_sim < 0 || M <= 0 || (n_real > 0 && !real) || (n_sim > 0 && !sim) || !losses || !workspace)
+    return fail(KS_EINVAL, "ks_mlp_disc_loss_grad: bad argument");
+  if (M > 4000000) return fail(KS_ELIMIT, "ks_mlp_disc_loss_grad: %lld rows exceed the limit of 4000000", (long long)M);
+  const bool penalty = grad_penalty_coef != 0.f && R > 0;
+  if (penalty && (n_motions <= 0 || n_real % n_motions != 0))
+    return fail(KS_EINVAL, "ks_mlp_disc_loss_grad: %lld real frames do not divide into %lld motions", (long long)n_real, (long long)n_motions);
+  hipStream_t s = (hipStream_t)stream;
+  DiscWs ws;
+  carve_disc(m, R, M, (char*)workspace, &ws);
+  auto blocks = [](int64_t n) { return dim3((unsigned)((n + 255) / 256)); };
+  for (int l = 0; l < L; ++l) {  // everything below adds into the gradient buffers
+    const int64_t nw = (int64_t)m.npad[l] * m.kpad[l];
+    hipLaunchKernelGGL(fill_kernel, blocks(nw), dim3(256), 0, s, nw, 0.f, m.gW[l]);
+    hipLaunchKernelGGL(fill_kernel, blocks(m.npad[l]), dim3(256), 0, s, (int64_t)m.npad[l], 0.f, m.gb[l]);
+  }
+  hipLaunchKernelGGL(fill_kernel, blocks(M), dim3(256), 0, s, M, 1.f, ws.ones);
+  hipLaunchKernelGGL(fill_kernel, dim3(1), dim3(256), 0, s, (int64_t)3, 0.f, losses);
+
+  // forward over the real rows, then the simulated ones
+  for (int l = 0; l < L; ++l) {
+    const bool last = l == L - 1;
+    float* outp = last ? ws.out : ws.y[l];
+    const int n = m.dims[l + 1], k = m.dims[l];
+    const int a_l = last ? KS_ACT_NONE : act;
+    if (l == 0) {
+      sgemm<true, true>(s, R, n, k, real, k, m.mW[0], m.kpad[0], outp, n, m.mb[0], a_l, false, nullptr);
+      sgemm<true, true>(s, n_sim, n, k, sim, k, m.mW[0], m.kpad[0], outp + R * n, n, m.mb[0], a_l, false, nullptr);
+    } else {
+      sgemm<true, true>(s, M, n, k, ws.y[l - 1], k, m.mW[l], m.kpad[l], outp, n, m.mb[l], a_l, false, nullptr);
+    }
+  }
+  hipLaunchKernelGGL(disc_signal_kernel, dim3(1), dim3(1024), 0, s, R, M, ws.out, ws.dz0, losses);
+
+  if (penalty) {
+    // input gradient on the real rows: d_L = 1, down to g = d_1 W_1
+    const float* dnext = ws.ones;
+    for (int l = L - 1; l >= 1; --l) {  // hidden layer l (its output is y[l - 1])
+      const int n = m.dims[l], k = m.dims[l + 1];
+      sgemm<true, false>(s, R, n, k, dnext, k, m.mW[l], m.kpad[l], ws.a[l - 1], n, nullptr, KS_ACT_NONE, false, nullptr);
+      hipLaunchKernelGGL(disc_delta_kernel, blocks(R * n), dim3(256), 0, s, R * n, act, ws.y[l - 1], ws.a[l - 1], ws.d[l - 1]);
+      dnext = ws.d[l - 1];
+    }
+    sgemm<true, false>(s, R, m.dims[0], m.dims[1], dnext, m.dims[1], m.mW[0], m.kpad[0], ws.g, m.dims[0], nullptr, KS_ACT_NONE, false, nullptr);
+    hipLaunchKernelGGL(disc_penalty_kernel, dim3(1), dim3(1024), 0, s, R * m.dims[0], grad_penalty_coef, 1.f / (float)n_motions, ws.g,
+                       losses + 2);
+    // the sweep back through that computation, first layer to last
+    const float* prev = ws.g;
+    float *u = ws.u, *v = ws.v;
+    for (int l = 1; l <= L; ++l) {
+      const int n = m.dims[l], k = m.dims[l - 1];
+      const float* dl = l == L ? ws.ones : ws.d[l - 1];
+      sgemm<false, false>(s, n, k, R, dl, n, prev, k, m.gW[l - 1], m.kpad[l - 1], nullptr, KS_ACT_NONE, true, ws.part);
+      if (l == L) break;
+      sgemm<true, true>(s, R, n, k, prev, k, m.mW[l - 1], m.kpad[l - 1], u, n, nullptr, KS_ACT_NONE, false, nullptr);
+      hipLaunchKernelGGL(disc_tangent_kernel, blocks(R * n), dim3(256), 0, s, R * n, act, ws.y[l - 1], ws.a[l - 1], u, v, ws.r[l - 1]);
+      prev = v;  // the next layer's products read v and write u; only then does its elementwise pass overwrite v
+    }
+  }
+
+  // ordinary backward pass of the squared-error terms over all rows, with r_l added on the real rows
+  float *dz = ws.dz0, *dnx = ws.dz1;
+  for (int l = L; l >= 1; --l) {
+    const int n = m.dims[l], k = m.dims[l - 1];
+    if (l == 1) {
+      sgemm<false, false>(s, n, k, R, dz, n, real, k, m.gW[0], m.kpad[0], nullptr, KS_ACT_NONE, true, ws.part);
+      sgemm<false, false>(s, n, k, n_sim, dz + R * n, n, sim, k, m.gW[0], m.kpad[0], nullptr, KS_ACT_NONE, true, ws.part);
+    } else {
+      sgemm<false, false>(s, n, k, M, dz, n, ws.y[l - 2], k, m.gW[l - 1], m.kpad[l - 1], nullptr, KS_ACT_NONE, true, ws.part);
+    }
+    sgemm<false, false>(s, n, 1, M, dz, n, ws.ones, 1, m.gb[l - 1], 1, nullptr, KS_ACT_NONE, true, ws.part);
+    if (l == 1) break;
+    sgemm<true, false>(s, M, k, n, dz, n, m.mW[l - 1], m.kpad[l - 1], dnx, k, nullptr, KS_ACT_NONE, false, nullptr);
+    hipLaunchKernelGGL(disc_dz_kernel, blocks(M * k), dim3(256), 0, s, M * k, penalty ? R * k : (int64_t)0, act, ws.y[l - 2], ws.r[l - 2], dnx);
+    float* tmp = dz; dz = dnx; dnx = tmp;
+  }
+  return check_launch("ks_mlp_disc_loss_grad");
+}
+
 // strided copy of the meaningful (out, in) block of a padded (npad, kpad) matrix
 __global__ __launch_bounds__(256) void unpad_kernel(int rows, int cols, int ld, const float* __restrict__ src, float* __restrict__ dst) {
   const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;

@@ -149,6 +149,23 @@ class MLP:
                                                       _lib.ptr(zero_rows), _lib.ptr(self._train_ws(M, dy.device))))
         return dx
 
+    def disc_loss_grad(self, real: torch.Tensor, sim: torch.Tensor, grad_penalty_coef: float) -> torch.Tensor:
+        """Gradient of the AMP discriminator loss (ksim/task/amp.py:360-438) into the handle: real (B, T, in) reference
+        motions, sim (B2, T2, in) simulated ones; returns the (real, simulated, penalty) terms of the loss, on the device."""
+        _lib.require_cuda(real, sim, dtype=torch.float32)
+        if real.dim() != 3 or sim.dim() != 3 or real.shape[2] != self.in_dim or sim.shape[2] != self.in_dim:
+            raise _lib.KsError(f"motions must be (B, T, {self.in_dim}), got {tuple(real.shape)} and {tuple(sim.shape)}")
+        n_real, n_sim = real.shape[0] * real.shape[1], sim.shape[0] * sim.shape[1]
+        need = int(self._lib.ks_mlp_disc_workspace_bytes(self._handle, n_real, n_sim))
+        ws = getattr(self, "_dws", None)
+        if ws is None or ws.numel() < need or ws.device != real.device:
+            ws = torch.empty(need, dtype=torch.uint8, device=real.device)
+            self._dws = ws
+        losses = torch.empty(3, dtype=torch.float32, device=real.device)
+        _lib.check(self._lib.ks_mlp_disc_loss_grad(self._handle, _lib.current_stream(), n_real, _lib.ptr(real), n_sim, _lib.ptr(sim),
+                                                   float(grad_penalty_coef), max(real.shape[0], 1), _lib.ptr(losses), _lib.ptr(ws)))
+        return losses
+
     @classmethod
     def _borrow(cls, lib, handle, dims, dtype: str) -> "MLP":
         """A view of a network that another object owns (the projections inside a GRU cell): never destroyed here."""
