@@ -755,8 +755,29 @@ enum { KS_REW_STAY_ALIVE = 0, KS_REW_BASE_HEIGHT = 1, KS_REW_BASE_HEIGHT_RANGE =
                                   the signs (zero inside +-p3) agree, else -1 */
        KS_REW_OFF_AXIS = 13,   /* exp(-v^2 / (2 p0^2)) of v = qvel[2] (norm 0), qvel[4] (norm 1), qvel[5] (norm 2) */
        KS_REW_MOTIONLESS = 14, /* |qvel[6:]| while |qvel[0:2]| < p0 and qvel[5] < p1, else 0 (rewards.py:1206-1221) */
-       KS_REW_FORCE = 15       /* max over `norm` bodies of (max(|obs[index + 3 b .. +3]| - p1, 0) / p0)^2 (rewards.py:1224-1240) */ };
+       KS_REW_FORCE = 15,      /* max over `norm` bodies of (max(|obs[index + 3 b .. +3]| - p1, 0) / p0)^2 (rewards.py:1224-1240) */
+       /* The kinds below read per-term constants from the table `params` of KsRewardIO at param_offset. */
+       KS_REW_JOINT_SMOOTH = 16, /* SmallJointVelocity / Acceleration / JerkReward (rewards.py:463-508): mean over the joints
+                                    qpos[7:] of exp(-x^2 / (2 p0^2)), x the first / second / third (norm = 1 / 2 / 3) difference
+                                    along the rollout, edge-padded at its start and zeroed after a step that was done */
+       KS_REW_AVOID_LIMITS = 17, /* mean over the joints of -min(q - lo, 0) + max(q - hi, 0); params (nq - 7, 2) (rewards.py:521-533) */
+       KS_REW_TORQUE = 18,       /* mean |ctrl / params[u]| (rewards.py:556-581) */
+       KS_REW_ENERGY = 19,       /* mean |ctrl / params[u] * qvel[6 + u]| (rewards.py:584-592) */
+       KS_REW_JOINT_DEVIATION = 20, /* sum over `count` joints of norm((qpos[7 + index_k] - target_k) weight_k); params
+                                       (count, 3) = index, target, weight (rewards.py:595-639) */
+       KS_REW_FLAT_BODY = 21,    /* mean over `count` bodies of (R(xquat_b)^T p) . p; params = count body indices, then p
+                                    (rewards.py:665-682) */
+       KS_REW_POSITION_TRACKING = 22, /* exp(-e^2 / (2 p0^2)), e = sum_i norm((xpos[index2] - xpos[count])_i - command[index + i])
+                                         (rewards.py:703-719); index2 = tracked body, count = base body */
+       KS_REW_NO_ROLL_ANGVEL = 23, /* k(qvel[3]) (rewards.py:779-804) */
+       KS_REW_NO_ROLL_POSE = 24,   /* k(-atan2(z_b.y, z_b.z)), z_b the world's z axis in the base frame */
+       KS_REW_LINK_SMOOTH = 25,  /* LinkAcceleration / JerkPenalty (rewards.py:808-840): mean over the bodies 1.. of
+                                    norm(second / third (p0 = 2 / 3) difference of |xpos(t) - xpos(t - 1)|), padded and
+                                    zeroed like KS_REW_JOINT_SMOOTH; `norm` is the l1 / l2 choice */
+       KS_REW_FEET_SLIP = 26     /* sum over `norm` feet of |obs[index2 + 6 f .. + 6]| while any of the foot's `count` contact
+                                    flags obs[index + c * norm + f] > 0.5 (rewards.py:1088-1105) */ };
 enum { KS_NORM_L1 = 0, KS_NORM_L2 = 1 }; /* xax.get_norm: l1 = |x|, l2 = x^2 (reference tests/test_rewards.py:95-98) */
+#define KS_MAX_REWARD_PARAMS 320
 typedef struct KsRewardDesc {
   int32_t kind;
   int32_t norm;   /* action-difference penalties */
@@ -764,6 +785,7 @@ typedef struct KsRewardDesc {
   float p0, p1, p2; /* balance,success_reward,has_success_reward | target,kernel_scale | lo,hi,dropoff | scale,sq,abs */
   float p3;
   int32_t index;    /* offset into the command or observation vector, for the kinds that read one */
+  int32_t index2, param_offset, count; /* see the kinds that name them */
 } KsRewardDesc;
 typedef struct KsRewardIO {
   int64_t T, N;
@@ -782,7 +804,12 @@ typedef struct KsRewardIO {
   const float* stateful; /* (n_slots, T, N) output of ks_reward_scan, KS_REW_STATEFUL only */
   int32_t command_dim, obs_dim;
   const float* command;  /* (T, N, command_dim), command-tracking kinds only */
-  const float* obs;      /* (T, N, obs_dim), KS_REW_FORCE only */
+  const float* obs;      /* (T, N, obs_dim), KS_REW_FORCE and KS_REW_FEET_SLIP */
+  int32_t nb, n_params;
+  const float* ctrl;     /* (T, N, nu) applied torques, KS_REW_TORQUE / KS_REW_ENERGY */
+  const float* xpos;     /* (T, N, nb, 3) */
+  const float* xquat;    /* (T, N, nb, 4) */
+  float params[KS_MAX_REWARD_PARAMS]; /* per-term constants, n_params of them in use */
 } KsRewardIO;
 int ks_rewards(ks_stream_t stream, const KsRewardIO* io /*host*/);
 

@@ -76,7 +76,9 @@ class KsMlpDesc(ctypes.Structure):
 
 (REW_STAY_ALIVE, REW_BASE_HEIGHT, REW_BASE_HEIGHT_RANGE, REW_ACTION_VEL, REW_ACTION_ACC, REW_ACTION_JERK,
  REW_UPRIGHT_ANGVEL, REW_UPRIGHT_LINVEL, REW_UPRIGHT_POSE, REW_AMP, REW_STATEFUL, REW_LINVEL_CMD, REW_ANGVEL_CMD,
- REW_OFF_AXIS, REW_MOTIONLESS, REW_FORCE) = range(16)
+ REW_OFF_AXIS, REW_MOTIONLESS, REW_FORCE, REW_JOINT_SMOOTH, REW_AVOID_LIMITS, REW_TORQUE, REW_ENERGY, REW_JOINT_DEVIATION,
+ REW_FLAT_BODY, REW_POSITION_TRACKING, REW_NO_ROLL_ANGVEL, REW_NO_ROLL_POSE, REW_LINK_SMOOTH, REW_FEET_SLIP) = range(27)
+KS_MAX_REWARD_PARAMS = 320
 KS_MAX_REWARD_SCANS, KS_MAX_SCAN_BODIES = 4, 8
 SCAN_FEET_AIR_TIME, SCAN_SPARSE_TARGET_HEIGHT = 0, 1
 NORM_L1, NORM_L2 = 0, 1
@@ -85,7 +87,8 @@ KS_MAX_REWARD_TERMS = 32
 
 class KsRewardDesc(ctypes.Structure):
     _fields_ = [("kind", c_int32), ("norm", c_int32), ("scale", c_float), ("p0", c_float), ("p1", c_float),
-                ("p2", c_float), ("p3", c_float), ("index", c_int32)]
+                ("p2", c_float), ("p3", c_float), ("index", c_int32), ("index2", c_int32), ("param_offset", c_int32),
+                ("count", c_int32)]
 
 
 class KsRewardIO(ctypes.Structure):
@@ -94,7 +97,9 @@ class KsRewardIO(ctypes.Structure):
                 ("use_clip_max", c_int32), ("clip_min", c_float), ("clip_max", c_float), ("qpos", c_void_p),
                 ("qvel", c_void_p), ("action", c_void_p), ("done", c_void_p), ("success", c_void_p),
                 ("disc_logits", c_void_p), ("components", c_void_p), ("total", c_void_p), ("stateful", c_void_p),
-                ("command_dim", c_int32), ("obs_dim", c_int32), ("command", c_void_p), ("obs", c_void_p)]
+                ("command_dim", c_int32), ("obs_dim", c_int32), ("command", c_void_p), ("obs", c_void_p),
+                ("nb", c_int32), ("n_params", c_int32), ("ctrl", c_void_p), ("xpos", c_void_p), ("xquat", c_void_p),
+                ("params", c_float * KS_MAX_REWARD_PARAMS)]
 
 
 class KsRewardScanDesc(ctypes.Structure):

@@ -482,6 +482,25 @@ __device__ inline float kernel_with_penalty(float x, float scale, float sq, floa
   return fabsf(x) * -ab + x * x * -sq + expf(-(x * x) / (2.f * scale * scale));
 }
 
+__device__ inline float dist3(const float* a, const float* b) {
+  const float x = a[0] - b[0], y = a[1] - b[1], z = a[2] - b[2];
+  return sqrtf(x * x + y * y + z * z);
+}
+
+// first / second / third difference (order 1 / 2 / 3) of x along the rollout from x(t), x(t-1), x(t-2), x(t-3) (already clamped to
+// the rollout's first step, which is the reference's edge padding); d_k says that step t - k was done, which zeroes every
+// difference taken across it (rewards.py:469-508)
+__device__ inline float smooth_difference(int order, float x0, float x1, float x2, float x3, bool d1, bool d2, bool d3) {
+  const float v0 = d1 ? 0.f : x0 - x1;
+  if (order == 1) return v0;
+  const float v1 = d2 ? 0.f : x1 - x2;
+  const float A0 = d1 ? 0.f : v0 - v1;
+  if (order == 2) return A0;
+  const float v2 = d3 ? 0.f : x2 - x3;
+  const float A1 = d2 ? 0.f : v1 - v2;
+  return d1 ? 0.f : A0 - A1;
+}
+
 __global__ __launch_bounds__(256) void rewards_kernel(KsRewardIO io) {
   const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   const int64_t TN = io.T * io.N;
@@ -592,6 +611,100 @@ __global__ __launch_bounds__(256) void rewards_kernel(KsRewardIO io) {
           best = b == 0 ? e * e : fmaxf(best, e * e);
         }
         val = best;
+      } break;
+      case KS_REW_JOINT_SMOOTH: {
+        const int nj = io.nq - 7;
+        const int64_t s1 = t >= 1 ? io.N * io.nq : 0, s2 = s1 + (t >= 2 ? io.N * io.nq : 0), s3 = s2 + (t >= 3 ? io.N * io.nq : 0);
+        float s = 0.f;
+        for (int u = 0; u < nj; ++u) {
+          const float* a0 = q + 7 + u;
+          const float x = smooth_difference(r.norm, a0[0], a0[-s1], a0[-s2], a0[-s3], d1, d2, d3);
+          s += expf(-(x * x) / (2.f * r.p0 * r.p0));
+        }
+        val = s / (float)nj;
+      } break;
+      case KS_REW_AVOID_LIMITS: {
+        const int nj = io.nq - 7;
+        const float* lim = io.params + r.param_offset;
+        float s = 0.f;
+        for (int u = 0; u < nj; ++u) s += -fminf(q[7 + u] - lim[2 * u], 0.f) + fmaxf(q[7 + u] - lim[2 * u + 1], 0.f);
+        val = s / (float)nj;
+      } break;
+      case KS_REW_TORQUE:
+      case KS_REW_ENERGY: {
+        const float* c = io.ctrl + idx * io.nu;
+        const float* sc = io.params + r.param_offset;
+        float s = 0.f;
+        for (int u = 0; u < io.nu; ++u) s += fabsf(r.kind == KS_REW_TORQUE ? c[u] / sc[u] : c[u] / sc[u] * v[6 + u]);
+        val = s / (float)io.nu;
+      } break;
+      case KS_REW_JOINT_DEVIATION: {
+        const float* pr = io.params + r.param_offset;
+        float s = 0.f;
+        for (int k = 0; k < r.count; ++k) {
+          const float x = (q[7 + (int)pr[3 * k]] - pr[3 * k + 1]) * pr[3 * k + 2];
+          s += r.norm == KS_NORM_L1 ? fabsf(x) : x * x;
+        }
+        val = s;
+      } break;
+      case KS_REW_FLAT_BODY: {
+        const float* pr = io.params + r.param_offset;
+        const float* pl = pr + r.count;
+        float s = 0.f;
+        for (int k = 0; k < r.count; ++k) {
+          float uv[3];
+          rot_inv(io.xquat + (idx * io.nb + (int)pr[k]) * 4, pl[0], pl[1], pl[2], uv);
+          s += uv[0] * pl[0] + uv[1] * pl[1] + uv[2] * pl[2];
+        }
+        val = s / (float)r.count;
+      } break;
+      case KS_REW_POSITION_TRACKING: {
+        const float* pb = io.xpos + (idx * io.nb + r.index2) * 3;
+        const float* p0 = io.xpos + (idx * io.nb + r.count) * 3;
+        const float* cmd = io.command + idx * io.command_dim + r.index;
+        float e = 0.f;
+        for (int i = 0; i < 3; ++i) {
+          const float x = (pb[i] - p0[i]) - cmd[i];
+          e += r.norm == KS_NORM_L1 ? fabsf(x) : x * x;
+        }
+        val = expf(-(e * e) / (2.f * r.p0 * r.p0));
+      } break;
+      case KS_REW_NO_ROLL_ANGVEL: val = kernel_with_penalty(v[3], r.p0, r.p1, r.p2); break;
+      case KS_REW_NO_ROLL_POSE: {
+        float zb[3];
+        rot_inv(q + 3, 0.f, 0.f, 1.f, zb);
+        val = kernel_with_penalty(-atan2f(zb[1], zb[2]), r.p0, r.p1, r.p2);
+      } break;
+      case KS_REW_LINK_SMOOTH: {
+        const int order = (int)r.p0;
+        const int64_t st = io.N * io.nb * 3;
+        const int64_t s1 = t >= 1 ? st : 0, s2 = s1 + (t >= 2 ? st : 0), s3 = s2 + (t >= 3 ? st : 0);
+        float s = 0.f;
+        for (int b = 1; b < io.nb; ++b) {
+          const float* p = io.xpos + (idx * io.nb + b) * 3;
+          // speeds |p(t - k) - p(t - k - 1)|, zeroed after a done step, then plain differences of those
+          const float w0 = d1 ? 0.f : dist3(p, p - s1), w1 = d2 ? 0.f : dist3(p - s1, p - s2), w2 = d3 ? 0.f : dist3(p - s2, p - s3);
+          const float A0 = d1 ? 0.f : w0 - w1;
+          float x = A0;
+          if (order == 3) {
+            const float A1 = d2 ? 0.f : w1 - w2;
+            x = d1 ? 0.f : A0 - A1;
+          }
+          s += r.norm == KS_NORM_L1 ? fabsf(x) : x * x;
+        }
+        val = s / (float)(io.nb - 1);
+      } break;
+      case KS_REW_FEET_SLIP: {
+        const float* ob = io.obs + idx * io.obs_dim;
+        float s = 0.f;
+        for (int f = 0; f < r.norm; ++f) {
+          bool touching = false;
+          for (int c = 0; c < r.count; ++c) touching = touching || ob[r.index + c * r.norm + f] > 0.5f;
+          const float* w = ob + r.index2 + 6 * f;
+          const float n2 = w[0] * w[0] + w[1] * w[1] + w[2] * w[2] + w[3] * w[3] + w[4] * w[4] + w[5] * w[5];
+          s += touching ? sqrtf(n2) : 0.f;
+        }
+        val = s;
       } break;
       default: break;
     }
@@ -973,7 +1086,7 @@ extern "C" int ks_rewards(ks_stream_t stream, const KsRewardIO* io) {
   if (!io->done) return fail(KS_EINVAL, "ks_rewards: done is required");
   for (int j = 0; j < io->n_rewards; ++j) {
     const int k = io->rewards[j].kind;
-    if (k < KS_REW_STAY_ALIVE || k > KS_REW_FORCE) return fail(KS_EINVAL, "ks_rewards: term %d: bad kind", j);
+    if (k < KS_REW_STAY_ALIVE || k > KS_REW_FEET_SLIP) return fail(KS_EINVAL, "ks_rewards: term %d: bad kind", j);
     const KsRewardDesc& rd = io->rewards[j];
     if (k == KS_REW_LINVEL_CMD || k == KS_REW_ANGVEL_CMD) {
       const int span = k == KS_REW_LINVEL_CMD ? 4 : 1;
@@ -990,6 +1103,77 @@ extern "C" int ks_rewards(ks_stream_t stream, const KsRewardIO* io) {
     if (needs_q && (!io->qpos || io->nq < 7)) return fail(KS_EINVAL, "ks_rewards: term %d needs qpos of a floating base", j);
     if (needs_v && (!io->qvel || io->nv < 6)) return fail(KS_EINVAL, "ks_rewards: term %d needs qvel of a floating base", j);
     if (needs_a && (!io->action || io->nu < 1)) return fail(KS_EINVAL, "ks_rewards: term %d needs actions", j);
+    {
+      const KsRewardDesc& r = io->rewards[j];
+      const int nj = io->nq - 7;
+      int need_params = 0;
+      bool uses_params = true;
+      switch (k) {
+        case KS_REW_JOINT_SMOOTH:
+          if (!io->qpos || nj < 1 || r.norm < 1 || r.norm > 3 || !(r.p0 > 0.f))
+            return fail(KS_EINVAL, "ks_rewards: term %d: joint smoothness needs joints behind a floating base, order 1..3 and a positive scale", j);
+          uses_params = false;
+          break;
+        case KS_REW_AVOID_LIMITS:
+          if (!io->qpos || nj < 1) return fail(KS_EINVAL, "ks_rewards: term %d needs joints behind a floating base", j);
+          need_params = 2 * nj;
+          break;
+        case KS_REW_TORQUE:
+        case KS_REW_ENERGY:
+          if (!io->ctrl || io->nu < 1) return fail(KS_EINVAL, "ks_rewards: term %d needs the applied torques", j);
+          if (k == KS_REW_ENERGY && (!io->qvel || io->nv != io->nu + 6)) return fail(KS_EINVAL, "ks_rewards: term %d needs qvel with one entry per actuator behind a floating base", j);
+          need_params = io->nu;
+          break;
+        case KS_REW_JOINT_DEVIATION:
+          if (!io->qpos || nj < 1 || r.count < 1) return fail(KS_EINVAL, "ks_rewards: term %d needs joints behind a floating base", j);
+          need_params = 3 * r.count;
+          break;
+        case KS_REW_FLAT_BODY:
+          if (!io->xquat || io->nb < 1 || r.count < 1) return fail(KS_EINVAL, "ks_rewards: term %d needs body orientations", j);
+          need_params = r.count + 3;
+          break;
+        case KS_REW_POSITION_TRACKING:
+          if (!io->xpos || r.index2 < 0 || r.index2 >= io->nb || r.count < 0 || r.count >= io->nb)
+            return fail(KS_EINVAL, "ks_rewards: term %d: body outside the trajectory's positions", j);
+          if (!io->command || r.index < 0 || r.index + 3 > io->command_dim) return fail(KS_EINVAL, "ks_rewards: term %d: command block outside the command vector", j);
+          if (!(r.p0 > 0.f)) return fail(KS_EINVAL, "ks_rewards: term %d: the kernel scale must be positive", j);
+          uses_params = false;
+          break;
+        case KS_REW_NO_ROLL_ANGVEL:
+          if (!io->qvel || io->nv < 6) return fail(KS_EINVAL, "ks_rewards: term %d needs qvel of a floating base", j);
+          uses_params = false;
+          break;
+        case KS_REW_NO_ROLL_POSE:
+          if (!io->qpos || io->nq < 7) return fail(KS_EINVAL, "ks_rewards: term %d needs qpos of a floating base", j);
+          uses_params = false;
+          break;
+        case KS_REW_LINK_SMOOTH:
+          if (!io->xpos || io->nb < 2 || (r.p0 != 2.f && r.p0 != 3.f)) return fail(KS_EINVAL, "ks_rewards: term %d needs body positions and order 2 or 3", j);
+          uses_params = false;
+          break;
+        case KS_REW_FEET_SLIP:
+          if (!io->obs || r.norm < 1 || r.count < 1 || r.index < 0 || r.index + r.count * r.norm > io->obs_dim || r.index2 < 0 ||
+              r.index2 + 6 * r.norm > io->obs_dim)
+            return fail(KS_EINVAL, "ks_rewards: term %d: contact or velocity block outside the observation", j);
+          uses_params = false;
+          break;
+        default: uses_params = false; break;
+      }
+      if (uses_params) {
+        if (io->n_params < 0 || io->n_params > KS_MAX_REWARD_PARAMS || r.param_offset < 0 || r.param_offset + need_params > io->n_params)
+          return fail(KS_EINVAL, "ks_rewards: term %d: its %d constants do not fit the table of %d", j, need_params, io->n_params);
+        const float* pr = io->params + r.param_offset;
+        if (k == KS_REW_TORQUE || k == KS_REW_ENERGY)
+          for (int u = 0; u < io->nu; ++u)
+            if (!(pr[u] != 0.f)) return fail(KS_EINVAL, "ks_rewards: term %d: zero control scale for actuator %d", j, u);
+        if (k == KS_REW_JOINT_DEVIATION)
+          for (int c = 0; c < r.count; ++c)
+            if (!(pr[3 * c] >= 0.f && pr[3 * c] < (float)nj)) return fail(KS_EINVAL, "ks_rewards: term %d: joint %d outside 0..%d", j, (int)pr[3 * c], nj - 1);
+        if (k == KS_REW_FLAT_BODY)
+          for (int c = 0; c < r.count; ++c)
+            if (!(pr[c] >= 0.f && pr[c] < (float)io->nb)) return fail(KS_EINVAL, "ks_rewards: term %d: body %d outside 0..%d", j, (int)pr[c], io->nb - 1);
+      }
+    }
     if (k == KS_REW_AMP && !io->disc_logits) return fail(KS_EINVAL, "ks_rewards: term %d needs the discriminator logits", j);
     if (k == KS_REW_STAY_ALIVE && !(io->rewards[j].p0 != 0.f)) return fail(KS_EINVAL, "ks_rewards: term %d: zero balance", j);
   }

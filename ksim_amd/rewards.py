@@ -123,6 +123,188 @@ class UprightReward(Reward):  # rewards.py:746-777 — a mapping of three compon
                 ("pose", T.REW_UPRIGHT_POSE, 0, self.pose_scale, self.pose_sq_scale, self.pose_abs_scale)]
 
 
+def _extra(**kw) -> dict:
+    """The trailing entry of a descriptor for the kinds with a second index, a count or a table of constants."""
+    return kw
+
+
+@dataclass(frozen=True)
+class SmallJointVelocityReward(Reward):  # rewards.py:463-476
+    kernel_scale: float = 0.25
+    _order = 1
+
+    def descs(self):
+        return [(None, T.REW_JOINT_SMOOTH, self._order, self.kernel_scale, 0.0, 0.0)]
+
+
+@dataclass(frozen=True)
+class SmallJointAccelerationReward(SmallJointVelocityReward):  # rewards.py:479-492
+    _order = 2
+
+
+@dataclass(frozen=True)
+class SmallJointJerkReward(SmallJointVelocityReward):  # rewards.py:495-509
+    _order = 3
+
+
+@dataclass(frozen=True)
+class AvoidLimitsPenalty(Reward):  # rewards.py:521-553
+    joint_limits: tuple = ()  # ((lo, hi), ...) one pair per joint behind the floating base
+
+    def __post_init__(self):
+        arr = np.asarray(self.joint_limits, dtype=np.float32)
+        if arr.ndim != 2 or arr.shape[1] != 2:
+            raise ValueError(f"Joint range must have shape (n_joints, 2), got {arr.shape}")
+        if not np.all(arr[:, 0] <= arr[:, 1]):
+            raise ValueError(f"Joint range must be sorted, got {arr}")
+
+    def descs(self):
+        flat = [float(x) for pair in self.joint_limits for x in pair]
+        return [(None, T.REW_AVOID_LIMITS, 0, 0.0, 0.0, 0.0, 0.0, 0, _extra(params=flat))]
+
+    @classmethod
+    def create(cls, model, factor: float = 0.05, scale=1.0) -> "AvoidLimitsPenalty":
+        """Limits widened by factor x range on both sides, none where a joint is not limited (rewards.py:535-553); `model` is a
+        `KinematicModel` with a floating base."""
+        rng = np.asarray(model.jnt_range, dtype=np.float64)[2:model.nb]   # body 0 is the world, body 1 the base
+        lim = np.asarray(model.jnt_limited)[2:model.nb].astype(bool)
+        diff = (rng[:, 1] - rng[:, 0]) * factor
+        lo = np.where(lim, rng[:, 0] - diff, -np.inf)
+        hi = np.where(lim, rng[:, 1] + diff, np.inf)
+        return cls(joint_limits=tuple((float(a), float(b)) for a, b in zip(lo, hi)), scale=scale)
+
+
+@dataclass(frozen=True)
+class TorquePenalty(Reward):  # rewards.py:556-581
+    ctrl_scales: tuple = ()
+    _kind = T.REW_TORQUE
+
+    def descs(self):
+        return [(None, self._kind, 0, 0.0, 0.0, 0.0, 0.0, 0, _extra(params=[float(x) for x in self.ctrl_scales]))]
+
+    @classmethod
+    def create(cls, model, scale=1.0):
+        """Half the width of each actuator's control range (rewards.py:571-581)."""
+        cr = np.asarray(model.arrays()["act_ctrlrange"], dtype=np.float64)[:model.nu]
+        return cls(ctrl_scales=tuple(float(x) for x in (cr[:, 1] - cr[:, 0]) / 2.0), scale=scale)
+
+
+@dataclass(frozen=True)
+class EnergyPenalty(TorquePenalty):  # rewards.py:584-592
+    _kind = T.REW_ENERGY
+
+
+@dataclass(frozen=True)
+class JointDeviationPenalty(Reward):  # rewards.py:595-662
+    norm: str = "l2"
+    joint_indices: tuple = ()
+    joint_targets: tuple = ()
+    joint_weights: tuple | None = None
+
+    def descs(self):
+        if len(self.joint_indices) != len(self.joint_targets):
+            raise ValueError(f"Joint names and targets must match, got {len(self.joint_indices)} and {len(self.joint_targets)}")
+        w = self.joint_weights if self.joint_weights is not None else (1.0,) * len(self.joint_indices)
+        if len(w) != len(self.joint_indices):
+            raise ValueError(f"Joint weights and names must match, got {len(w)} and {len(self.joint_indices)}")
+        flat = [float(x) for trip in zip(self.joint_indices, self.joint_targets, w) for x in trip]
+        return [(None, T.REW_JOINT_DEVIATION, _norm(self.norm), 0.0, 0.0, 0.0, 0.0, 0, _extra(count=len(self.joint_indices), params=flat))]
+
+    @classmethod
+    def create(cls, physics_model, joint_names, joint_targets, scale=1.0, joint_weights=None):
+        """Joints are named after the body they move (a `KinematicModel` keeps body names); index = qpos address - 7."""
+        names = list(physics_model.body_names)
+        idx = tuple(int(physics_model.body_qadr[names.index(n)]) - 7 for n in joint_names)
+        return cls(joint_indices=idx, joint_targets=tuple(float(x) for x in joint_targets),
+                   joint_weights=None if joint_weights is None else tuple(float(x) for x in joint_weights), scale=scale)
+
+
+@dataclass(frozen=True)
+class FlatBodyReward(Reward):  # rewards.py:665-700
+    body_indices: tuple = ()
+    plane: tuple = (0.0, 0.0, 1.0)
+    norm: str = "l2"
+
+    def descs(self):
+        _norm(self.norm)
+        flat = [float(b) for b in self.body_indices] + [float(x) for x in self.plane]
+        return [(None, T.REW_FLAT_BODY, 0, 0.0, 0.0, 0.0, 0.0, 0, _extra(count=len(self.body_indices), params=flat))]
+
+    @classmethod
+    def create(cls, physics_model, body_names, plane=(0.0, 0.0, 1.0), norm="l2", scale=1.0):
+        names = list(physics_model.body_names)
+        return cls(body_indices=tuple(names.index(n) for n in body_names), plane=tuple(plane), norm=norm, scale=scale)
+
+
+@dataclass(frozen=True)
+class PositionTrackingReward(Reward):  # rewards.py:703-743
+    tracked_body_idx: int = 0
+    base_body_idx: int = 0
+    command_name: str = ""
+    body_name: str = ""
+    norm: str = "l1"
+    kernel_scale: float = 0.25
+
+    def descs(self):  # pragma: no cover
+        raise ValueError("PositionTrackingReward reads a named command: pass command_slices to get_rewards")
+
+    def descs_in(self, obs_slices, command_slices):
+        sl = _named(command_slices, self.command_name, "command")
+        return [(None, T.REW_POSITION_TRACKING, _norm(self.norm), self.kernel_scale, 0.0, 0.0, 0.0, sl.start,
+                 _extra(index2=self.tracked_body_idx, count=self.base_body_idx))]
+
+    @classmethod
+    def create(cls, model, command_name, tracked_body_name, base_body_name, norm="l1", kernel_scale=0.25, scale=1.0):
+        names = list(model.body_names)
+        return cls(tracked_body_idx=names.index(tracked_body_name), base_body_idx=names.index(base_body_name), norm=norm,
+                   command_name=command_name, body_name=tracked_body_name, scale=scale, kernel_scale=kernel_scale)
+
+
+@dataclass(frozen=True)
+class NoRollReward(Reward):  # rewards.py:778-804 — a mapping of two components
+    angvel_scale: float = 0.25
+    roll_scale: float = 0.25
+    angvel_sq_scale: float = 0.1
+    angvel_abs_scale: float = 0.1
+    roll_sq_scale: float = 0.1
+    roll_abs_scale: float = 0.1
+
+    def descs(self):
+        return [("angvel", T.REW_NO_ROLL_ANGVEL, 0, self.angvel_scale, self.angvel_sq_scale, self.angvel_abs_scale),
+                ("pose", T.REW_NO_ROLL_POSE, 0, self.roll_scale, self.roll_sq_scale, self.roll_abs_scale)]
+
+
+@dataclass(frozen=True)
+class LinkAccelerationPenalty(Reward):  # rewards.py:807-821
+    norm: str = "l2"
+    _order = 2
+
+    def descs(self):
+        return [(None, T.REW_LINK_SMOOTH, _norm(self.norm), float(self._order), 0.0, 0.0)]
+
+
+@dataclass(frozen=True)
+class LinkJerkPenalty(LinkAccelerationPenalty):  # rewards.py:824-840
+    _order = 3
+
+
+@dataclass(frozen=True)
+class FeetSlipPenalty(Reward):  # rewards.py:1088-1105
+    contact_obs: str = ""
+    velocity_obs: str = ""
+
+    def descs(self):  # pragma: no cover
+        raise ValueError("FeetSlipPenalty reads named observations: pass obs_slices to get_rewards")
+
+    def descs_in(self, obs_slices, command_slices):
+        c, v = _named(obs_slices, self.contact_obs, "observation"), _named(obs_slices, self.velocity_obs, "observation")
+        nv_, nc_ = v.stop - v.start, c.stop - c.start
+        if nv_ % 6 != 0 or nv_ == 0 or nc_ % (nv_ // 6) != 0:
+            raise ValueError(f"velocity observation of {nv_} entries is not (n, 6) for the {nc_} contact flags")
+        n = nv_ // 6
+        return [(None, T.REW_FEET_SLIP, n, 0.0, 0.0, 0.0, 0.0, c.start, _extra(index2=v.start, count=nc_ // n))]
+
+
 DISCRIMINATOR_OUTPUT_KEY = "_discriminator_output"  # ksim/task/amp.py:47
 
 
@@ -377,6 +559,7 @@ def get_rewards(trajectory: Trajectory, rewards: Mapping[str, Reward], clip_min:
     io = T.KsRewardIO()
     io.T, io.N = Tn, N
     names = []
+    n_params = 0
     scanned, first_slot = None, {}
     if any(isinstance(r, StatefulReward) for r in rewards.values()):
         scanned, first_slot, rewards_carry = _scan_stateful(trajectory, rewards, rewards_carry, obs_slices, command_slices,
@@ -401,6 +584,17 @@ def get_rewards(trajectory: Trajectory, rewards: Mapping[str, Reward], clip_min:
             d.kind, d.norm, d.scale, d.p0, d.p1, d.p2 = kind, norm, sign * _reward_scale(rew, level), p0, p1, p2
             if more:
                 d.p3, d.index = float(more[0]), int(more[1])
+            if len(more) >= 3:
+                ex = more[2]
+                d.index2, d.count = int(ex.get("index2", 0)), int(ex.get("count", 0))
+                pr = ex.get("params")
+                if pr is not None:
+                    if n_params + len(pr) > T.KS_MAX_REWARD_PARAMS:
+                        raise _lib.KsError(f"the rewards' constants exceed the table of {T.KS_MAX_REWARD_PARAMS} entries")
+                    d.param_offset = n_params
+                    for x in pr:
+                        io.params[n_params] = x
+                        n_params += 1
             names.append(name if suffix is None else f"{name}/{suffix}")  # rl.py:223-226
     io.n_rewards = len(names)
     if not names:
@@ -429,19 +623,40 @@ def get_rewards(trajectory: Trajectory, rewards: Mapping[str, Reward], clip_min:
                              "an AMP task, which populates the auxiliary output for you.")
         logits = tensor(trajectory.aux_outputs[DISCRIMINATOR_OUTPUT_KEY], torch.float32, None)
     kinds = {io.rewards[j].kind for j in range(len(names))}
-    if kinds & {T.REW_LINVEL_CMD, T.REW_ANGVEL_CMD}:
+    io.n_params = n_params
+    if kinds & {T.REW_TORQUE, T.REW_ENERGY}:
+        if trajectory.ctrl is None:
+            raise _lib.KsError("torque and energy penalties read trajectory.ctrl")
+        ctrl = tensor(trajectory.ctrl, torch.float32, trajectory.ctrl.shape[-1])
+        io.ctrl = ctrl.data_ptr()
+        if action is not None and ctrl.shape[-1] != action.shape[-1]:
+            raise _lib.KsError("trajectory.ctrl and trajectory.action differ in width")
+        nu_ctrl = ctrl.shape[-1]
+    else:
+        nu_ctrl = None
+    if kinds & {T.REW_FLAT_BODY, T.REW_POSITION_TRACKING, T.REW_LINK_SMOOTH}:
+        for leaf, per, name in ((trajectory.xpos, 3, "xpos"), (trajectory.xquat, 4, "xquat")):
+            if leaf is None:
+                continue
+            flat = leaf.reshape(Tn, N, -1) if leaf.dim() == 4 else leaf
+            flat = tensor(flat, torch.float32, flat.shape[-1])
+            if flat.shape[-1] % per != 0 or (io.nb and io.nb != flat.shape[-1] // per):
+                raise _lib.KsError(f"trajectory.{name} has {flat.shape[-1]} entries per step: not (nb, {per}) for the other leaf's nb")
+            io.nb = flat.shape[-1] // per
+            setattr(io, name, flat.data_ptr())
+    if kinds & {T.REW_LINVEL_CMD, T.REW_ANGVEL_CMD, T.REW_POSITION_TRACKING}:
         cmd = trajectory.command.get("_buffer") if trajectory.command else None
         if cmd is None:
             raise KeyError('command-tracking rewards read trajectory.command["_buffer"] (T, N, command_dim)')
         cmd = tensor(cmd, torch.float32, cmd.shape[-1])
         io.command, io.command_dim = cmd.data_ptr(), cmd.shape[-1]
-    if T.REW_FORCE in kinds:
+    if kinds & {T.REW_FORCE, T.REW_FEET_SLIP}:
         ob_ = trajectory.obs[obs_key]
         ob_ = tensor(ob_, torch.float32, ob_.shape[-1])
         io.obs, io.obs_dim = ob_.data_ptr(), ob_.shape[-1]
     io.nq = 0 if qpos is None else qpos.shape[-1]
     io.nv = 0 if qvel is None else qvel.shape[-1]
-    io.nu = 0 if action is None else action.shape[-1]
+    io.nu = (nu_ctrl or 0) if action is None else action.shape[-1]
     io.use_clip_min, io.clip_min = int(clip_min is not None), float(clip_min or 0.0)
     io.use_clip_max, io.clip_max = int(clip_max is not None), float(clip_max or 0.0)
     total = torch.empty((Tn, N), dtype=torch.float32, device=done.device)

@@ -92,6 +92,88 @@ def action_jerk_penalty(action_ta, done_t, norm="l2"):  # rewards.py:449-460
     return np.where(np.arange(len(pen)) >= 3, pen, 0.0)
 
 
+def _padded_differences(x, done_t, order):
+    """The differencing shared by the joint and link smoothness terms (rewards.py:469-508, 814-839): pad `order` copies of the
+    first row in front, difference `order` times, and zero each difference where the step before it was done."""
+    x = _edge_pad_front(np.asarray(x, dtype=np.float64), order)
+    done = _edge_pad_front(np.asarray(done_t).astype(bool), order)[:-1]
+    done = done.reshape(done.shape + (1,) * (x.ndim - 1))
+    return x, done
+
+
+def small_joint_reward(qpos_tq, done_t, order, kernel_scale=0.25):  # rewards.py:463-508 (order 1, 2, 3 = velocity, acceleration, jerk)
+    q, done = _padded_differences(np.asarray(qpos_tq)[:, 7:], done_t, order)
+    d = np.where(done, 0.0, q[1:] - q[:-1])
+    for k in range(1, order):
+        d = np.where(done[k:], 0.0, d[1:] - d[:-1])
+    return exp_kernel(d, kernel_scale).mean(axis=-1)
+
+
+def avoid_limits_penalty(qpos_tq, joint_limits):  # rewards.py:527-533
+    q = np.asarray(qpos_tq, dtype=np.float64)[:, 7:]
+    lim = np.asarray(joint_limits, dtype=np.float64)
+    return (-np.clip(q - lim[:, 0], None, 0.0) + np.clip(q - lim[:, 1], 0.0, None)).mean(axis=-1)
+
+
+def avoid_limits_create(jnt_range, jnt_limited, factor=0.05):  # rewards.py:535-553 (rows: every joint, the free joint first)
+    rng = np.asarray(jnt_range, dtype=np.float64)
+    diff = (rng[:, 1] - rng[:, 0]) * factor
+    lo = np.where(jnt_limited, rng[:, 0] - diff, -np.inf)
+    hi = np.where(jnt_limited, rng[:, 1] + diff, np.inf)
+    return np.stack([lo, hi], axis=-1)[1:]
+
+
+def torque_penalty(ctrl_tu, ctrl_scales):  # rewards.py:567-569
+    return np.abs(np.asarray(ctrl_tu, dtype=np.float64) / np.asarray(ctrl_scales, dtype=np.float64)).mean(axis=-1)
+
+
+def energy_penalty(ctrl_tu, qvel_tv, ctrl_scales):  # rewards.py:588-591
+    ctrl_n = np.asarray(ctrl_tu, dtype=np.float64) / np.asarray(ctrl_scales, dtype=np.float64)
+    return np.abs(ctrl_n * np.asarray(qvel_tv, dtype=np.float64)[:, 6:]).mean(axis=-1)
+
+
+def joint_deviation_penalty(qpos_tq, joint_indices, joint_targets, joint_weights=None, norm="l2"):  # rewards.py:629-639
+    diff = np.asarray(qpos_tq, dtype=np.float64)[:, np.asarray(joint_indices) + 7] - np.asarray(joint_targets, dtype=np.float64)
+    if joint_weights is not None:
+        diff = diff * np.asarray(joint_weights, dtype=np.float64)
+    return get_norm(diff, norm).sum(axis=-1)
+
+
+def flat_body_reward(xquat_tb4, body_indices, plane=(0.0, 0.0, 1.0)):  # rewards.py:678-682
+    quat = np.asarray(xquat_tb4, dtype=np.float64)[:, list(body_indices), :]
+    plane = np.asarray(plane, dtype=np.float64)
+    unit = rotate_vector_by_quat(np.broadcast_to(plane, quat.shape[:-1] + (3,)), quat, inverse=True)
+    return (unit * plane).sum(axis=-1).mean(axis=-1)
+
+
+def position_tracking_reward(xpos_tb3, cmd_t3, tracked, base, norm="l1", kernel_scale=0.25):  # rewards.py:713-719
+    x = np.asarray(xpos_tb3, dtype=np.float64)
+    err = get_norm((x[:, tracked] - x[:, base]) - np.asarray(cmd_t3, dtype=np.float64)[:, :3], norm).sum(-1)
+    return exp_kernel(err, kernel_scale)
+
+
+def no_roll_reward(qpos_tq, qvel_tv, s=0.25, sq=0.1, ab=0.1):  # rewards.py:789-804 (defaults); returns (angvel, pose)
+    q, v = np.asarray(qpos_tq, dtype=np.float64), np.asarray(qvel_tv, dtype=np.float64)
+    zb = rotate_vector_by_quat(np.broadcast_to(np.array([0.0, 0.0, 1.0]), q.shape[:-1] + (3,)), q[:, 3:7], inverse=True)
+    roll = -np.arctan2(zb[:, 1], zb[:, 2])
+    return exp_kernel_with_penalty(v[:, 3], s, sq, ab), exp_kernel_with_penalty(roll, s, sq, ab)
+
+
+def link_smoothness_penalty(xpos_tb3, done_t, order, norm="l2"):  # rewards.py:813-821 (order 2), 830-840 (order 3)
+    p, done = _padded_differences(np.asarray(xpos_tb3)[:, 1:], done_t, order)
+    done = done[..., 0]
+    d = np.where(done, 0.0, np.linalg.norm(p[1:] - p[:-1], axis=-1))
+    for k in range(1, order):
+        d = np.where(done[k:], 0.0, d[1:] - d[:-1])
+    return get_norm(d, norm).mean(axis=-1)
+
+
+def feet_slip_penalty(contact_tcn, velocity_tn6):  # rewards.py:1095-1105
+    touching = (np.asarray(contact_tcn) > 0.5).any(axis=-2)
+    speed = np.linalg.norm(np.asarray(velocity_tn6, dtype=np.float64), axis=-1)
+    return np.where(touching, speed, 0.0).sum(axis=-1)
+
+
 def stay_alive_reward(done_t, success_t, balance=100.0, success_reward=None):  # rewards.py:178-188
     alive = 1.0 / balance
     return np.where(done_t, np.where(success_t, alive if success_reward is None else success_reward, -1.0), alive)

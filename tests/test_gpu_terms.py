@@ -553,6 +553,91 @@ def test_command_tracking_rest_and_force_rewards():
         rw.get_rewards(traj, {"ang": rw.AngularVelocityReward(cmd="a")}, command_slices={"a": slice(8, 9)})
 
 
+def test_smoothness_limits_effort_and_body_frame_rewards():
+    """The remaining stateless rewards of ksim/rewards.py against the oracle: joint and link smoothness (with episode ends
+    inside the rollout and at its first steps), limit avoidance, torque and energy, joint deviation, flat bodies, position
+    tracking, roll, feet slip."""
+    from ksim_amd import model as km
+    from ksim_amd import rewards as rw
+    from ksim_amd.types import Trajectory
+
+    m = km.kbot_scale_model(joint_range=(-0.8, 0.9))
+    Tn, N, nq, nv, nu, nb = 24, 13, m.nq, m.nv, m.nu, m.nb
+    rng = np.random.default_rng(77)
+    qpos = rng.normal(size=(Tn, N, nq)) * 0.7; qpos[..., 3:7] /= np.linalg.norm(qpos[..., 3:7], axis=-1, keepdims=True)
+    qpos[..., 7:] = np.cumsum(rng.normal(size=(Tn, N, nq - 7)) * 0.1, axis=0)   # smooth enough that the kernels are not all ~0
+    qvel = rng.normal(size=(Tn, N, nv))
+    ctrl = rng.normal(size=(Tn, N, nu)) * 10
+    xpos = np.cumsum(rng.normal(size=(Tn, N, nb, 3)) * 0.05, axis=0)
+    xquat = rng.normal(size=(Tn, N, nb, 4)); xquat /= np.linalg.norm(xquat, axis=-1, keepdims=True)
+    cmd = rng.normal(size=(Tn, N, 5)) * 0.2
+    obs = rng.normal(size=(Tn, N, 20)); obs[..., 2:6] = rng.random((Tn, N, 4)) < 0.4   # contact flags (c = 2, n = 2)
+    done = rng.random((Tn, N)) < 0.12
+    done[0, :4] = True; done[1, 2:6] = True
+    targets = (0.1, -0.2, 0.3)
+    rewards = {"jv": rw.SmallJointVelocityReward(scale=0.5, kernel_scale=0.2), "ja": rw.SmallJointAccelerationReward(scale=0.6),
+               "jj": rw.SmallJointJerkReward(scale=0.7, kernel_scale=0.4),
+               "limits": rw.AvoidLimitsPenalty.create(m, factor=0.05, scale=0.3),
+               "torque": rw.TorquePenalty(ctrl_scales=tuple(float(x) for x in np.linspace(5.0, 40.0, nu)), scale=0.01),
+               "energy": rw.EnergyPenalty(ctrl_scales=tuple(float(x) for x in np.linspace(40.0, 5.0, nu)), scale=0.02),
+               "dev": rw.JointDeviationPenalty(scale=0.4, norm="l1", joint_indices=(0, 7, 19), joint_targets=targets, joint_weights=(1.0, 2.0, 0.5)),
+               "dev2": rw.JointDeviationPenalty.create(m, [m.body_names[3], m.body_names[5]], (0.0, 0.5), scale=0.2),
+               "flat": rw.FlatBodyReward(scale=0.9, body_indices=(1, 4, nb - 1), plane=(0.0, 0.6, 0.8)),
+               "track": rw.PositionTrackingReward(scale=1.1, tracked_body_idx=6, base_body_idx=1, command_name="hand", norm="l2", kernel_scale=0.5),
+               "roll": rw.NoRollReward(scale=0.8, roll_scale=0.5, angvel_abs_scale=0.2),
+               "lacc": rw.LinkAccelerationPenalty(scale=2.0, norm="l1"), "ljerk": rw.LinkJerkPenalty(scale=3.0),
+               "slip": rw.FeetSlipPenalty(scale=0.1, contact_obs="contact", velocity_obs="feet_vel")}
+    traj = Trajectory(qpos=t32(qpos), qvel=t32(qvel), xpos=t32(xpos.reshape(Tn, N, -1)), xquat=t32(xquat), ctrl=t32(ctrl),
+                      obs={"obs": t32(obs)}, command={"_buffer": t32(cmd)}, event_state={}, action=None,
+                      done=torch.from_numpy(done).to(DEV), success=None, timestep=None)
+    st = rw.get_rewards(traj, rewards, obs_slices={"contact": slice(2, 6), "feet_vel": slice(7, 19)}, command_slices={"hand": slice(1, 4)})
+    f32 = lambda a: a.astype(np.float32).astype(np.float64)  # noqa: E731
+    q, v, c, xp, xq, cm, ob = f32(qpos), f32(qvel), f32(ctrl), f32(xpos), f32(xquat), f32(cmd), f32(obs)
+    lim = ot.avoid_limits_create(m.jnt_range[1:m.nb], np.asarray(m.jnt_limited[1:m.nb]).astype(bool), 0.05)
+    t_scales, e_scales = np.linspace(5.0, 40.0, nu), np.linspace(40.0, 5.0, nu)
+    qa = [int(m.body_qadr[3]) - 7, int(m.body_qadr[5]) - 7]
+    want = {k: [] for k in ("jv", "ja", "jj", "limits", "torque", "energy", "dev", "dev2", "flat", "track", "roll/angvel", "roll/pose",
+                            "lacc", "ljerk", "slip")}
+    for e in range(N):
+        dn = done[:, e]
+        ang, pose = ot.no_roll_reward(q[:, e], v[:, e], s=0.25, sq=0.1, ab=0.2)
+        _, pose = ot.no_roll_reward(q[:, e], v[:, e], s=0.5, sq=0.1, ab=0.1)
+        vals = {"jv": 0.5 * ot.small_joint_reward(q[:, e], dn, 1, 0.2), "ja": 0.6 * ot.small_joint_reward(q[:, e], dn, 2),
+                "jj": 0.7 * ot.small_joint_reward(q[:, e], dn, 3, 0.4), "limits": -0.3 * ot.avoid_limits_penalty(q[:, e], lim),
+                "torque": -0.01 * ot.torque_penalty(c[:, e], t_scales), "energy": -0.02 * ot.energy_penalty(c[:, e], v[:, e], e_scales),
+                "dev": -0.4 * ot.joint_deviation_penalty(q[:, e], (0, 7, 19), targets, (1.0, 2.0, 0.5), "l1"),
+                "dev2": -0.2 * ot.joint_deviation_penalty(q[:, e], qa, (0.0, 0.5), None, "l2"),
+                "flat": 0.9 * ot.flat_body_reward(xq[:, e], (1, 4, nb - 1), (0.0, 0.6, 0.8)),
+                "track": 1.1 * ot.position_tracking_reward(xp[:, e], cm[:, e, 1:4], 6, 1, "l2", 0.5),
+                "roll/angvel": 0.8 * ang, "roll/pose": 0.8 * pose,
+                "lacc": -2.0 * ot.link_smoothness_penalty(xp[:, e], dn, 2, "l1"), "ljerk": -3.0 * ot.link_smoothness_penalty(xp[:, e], dn, 3, "l2"),
+                "slip": -0.1 * ot.feet_slip_penalty(ob[:, e, 2:6].reshape(Tn, 2, 2), ob[:, e, 7:19].reshape(Tn, 2, 6))}
+        for k, x in vals.items():
+            want[k].append(x)
+    assert list(st.components) == list(want)
+    assert np.isfinite(lim).all() and (ot.avoid_limits_penalty(q[:, 0], lim) > 0).any()
+    for k, w in want.items():
+        w = np.stack(w, axis=1)
+        assert np.abs(w).max() > 1e-3, k
+        np.testing.assert_allclose(st.components[k].cpu().numpy(), w, rtol=3e-5, atol=3e-5, err_msg=k)
+    total = sum(st.components[k] for k in st.components)
+    np.testing.assert_allclose(st.total.cpu().numpy(), total.cpu().numpy(), rtol=1e-5, atol=1e-5)
+    # error paths: a joint or body outside the model, a table that does not fit, missing leaves
+    with pytest.raises(Exception, match="joint"):
+        rw.get_rewards(traj, {"dev": rw.JointDeviationPenalty(joint_indices=(nq,), joint_targets=(0.0,))})
+    with pytest.raises(Exception, match="body"):
+        rw.get_rewards(traj, {"flat": rw.FlatBodyReward(body_indices=(nb,))})
+    with pytest.raises(Exception, match="constants"):
+        rw.get_rewards(traj, {"limits": rw.AvoidLimitsPenalty(joint_limits=((-1.0, 1.0),) * 3)})
+    with pytest.raises(Exception, match="zero control scale"):
+        rw.get_rewards(traj, {"t": rw.TorquePenalty(ctrl_scales=(0.0,) * nu)})
+    with pytest.raises(ValueError, match="sorted"):
+        rw.AvoidLimitsPenalty(joint_limits=((1.0, -1.0),))
+    import dataclasses
+    with pytest.raises(Exception, match="trajectory.ctrl"):
+        rw.get_rewards(dataclasses.replace(traj, ctrl=None), {"t": rewards["torque"]})
+
+
 def test_velocity_commands_against_oracle():
     """LinearVelocityCommand / AngularVelocityCommand over several control steps with explicit draws: episode starts,
     slewing, switches, zero and backward targets; the recorded copy is the incoming command."""

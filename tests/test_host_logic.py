@@ -333,3 +333,26 @@ def test_remaining_randomizers_produce_the_kernel_inputs():
     assert np.abs(com1[:, 3]).max() > 0.01 and np.abs(np.delete(com1, 3, axis=1)).max() < 1e-7
     with pytest.raises(ValueError, match="not a collision capsule"):
         rnd.CollisionBodyRandomizer.from_geom_names(m, ["nope"])
+
+
+def test_reward_constructors_from_a_model():
+    """`create` of the rewards that read the model (ksim/rewards.py:535-553, 571-581, 641-662, 684-700)."""
+    import os
+    from ksim_amd import rewards as rw
+    from ksim_amd.mjcf import load_mjcf
+
+    m = load_mjcf(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "mini_humanoid.mjcf"))
+    lim = rw.AvoidLimitsPenalty.create(m, factor=0.1)
+    lo, hi = np.deg2rad(-30), np.deg2rad(20)
+    assert len(lim.joint_limits) == m.nq - 7
+    np.testing.assert_allclose(lim.joint_limits[0], (lo - 0.1 * (hi - lo), hi + 0.1 * (hi - lo)), rtol=1e-6)
+    assert rw.TorquePenalty.create(m).ctrl_scales == (1.0,) * m.nu      # control range -1..1 on every motor
+    assert isinstance(rw.EnergyPenalty.create(m), rw.EnergyPenalty) and rw.EnergyPenalty(ctrl_scales=(1.0,)).is_penalty
+    dev = rw.JointDeviationPenalty.create(m, ["shin_right", "thigh_left"], (0.1, 0.2), joint_weights=(1.0, 3.0))
+    assert dev.joint_indices == (3, 6) and dev.joint_weights == (1.0, 3.0)
+    flat = rw.FlatBodyReward.create(m, ("pelvis", "shin_left"))
+    assert flat.body_indices == (1, 9)
+    tr = rw.PositionTrackingReward.create(m, "cmd", "shin_left", "pelvis")
+    assert (tr.tracked_body_idx, tr.base_body_idx, tr.norm) == (9, 1, "l1")
+    with pytest.raises(ValueError, match="must match"):
+        rw.JointDeviationPenalty(joint_indices=(0, 1), joint_targets=(0.0,)).descs()

@@ -7,6 +7,7 @@ import numpy as np
 import pytest
 
 from oracle import terms
+from oracle import terms as ot
 
 GOLD = os.path.join(os.path.dirname(__file__), "golden")
 REWARD_KATS = json.load(open(os.path.join(GOLD, "reward_kats.json")))
@@ -413,3 +414,90 @@ def test_site_sensors_against_rigid_motion():
     np.testing.assert_allclose(got, want, rtol=1e-4, atol=1e-4)
     # dropped terms would show: centripetal and tangential parts are both far above the tolerance here
     assert np.linalg.norm(np.cross(w_world, np.cross(w_world, Rb.apply(r_s)))) > 0.05 and np.linalg.norm(np.cross(Rb.apply(al_l), Rb.apply(r_s))) > 0.05
+
+
+def test_joint_and_link_smoothness_hand_computed():
+    """Polynomial motions have constant differences: a ramp a constant velocity, a parabola a constant acceleration, a cubic
+    a constant jerk; the edge padding makes the first `order` values build up from zero and a done step restarts that."""
+    T = 8
+    t = np.arange(T, dtype=np.float64)
+    base = np.tile([0, 0, 1, 1, 0, 0, 0.0], (T, 1))
+    done = np.zeros(T, bool)
+    k = lambda x, s=0.25: np.exp(-x * x / (2 * s * s))  # noqa: E731
+    ramp = np.concatenate([base, np.stack([0.1 * t, -0.2 * t], axis=1)], axis=1)
+    want = np.full(T, (k(0.1) + k(0.2)) / 2); want[0] = 1.0
+    np.testing.assert_allclose(ot.small_joint_reward(ramp, done, 1), want, rtol=1e-12)
+    par = np.concatenate([base, (0.05 * t * t)[:, None]], axis=1)    # second difference 0.1 from t = 2; at t = 1: v(1) - 0 = 0.05
+    want = np.full(T, k(0.1)); want[0] = 1.0; want[1] = k(0.05)
+    np.testing.assert_allclose(ot.small_joint_reward(par, done, 2), want, rtol=1e-12)
+    cub = np.concatenate([base, (0.01 * t**3)[:, None]], axis=1)    # third difference 0.06 from t = 3
+    got = ot.small_joint_reward(cub, done, 3)
+    np.testing.assert_allclose(got[3:], k(0.06), rtol=1e-9)
+    np.testing.assert_allclose(got[:3], [1.0, k(0.01), k(0.08 - 3 * 0.01)], rtol=1e-9)  # x(1); x(2) - 3 x(1)
+    # a done step at t = 3 zeroes the differences taken across it: velocity at t = 4, acceleration at t = 4 (zeroed) and at
+    # t = 5 (v(5) - 0)
+    done[3] = True
+    got = ot.small_joint_reward(ramp, done, 1)
+    assert got[4] == 1.0 and got[5] == pytest.approx((k(0.1) + k(0.2)) / 2)
+    got = ot.small_joint_reward(par, done, 2)
+    v5 = 0.05 * (25 - 16)
+    assert got[4] == 1.0 and got[5] == pytest.approx(k(v5)) and got[6] == pytest.approx(k(0.1))
+    # links: body 1 moves along a diagonal with quadratic arc length, body 0 (the world) is skipped
+    done[:] = False
+    s = 0.05 * t * t
+    xpos = np.zeros((T, 3, 3))
+    xpos[:, 1] = s[:, None] * np.array([0.6, 0.0, 0.8])
+    xpos[:, 2] = (0.3 * t)[:, None] * np.array([0.0, 1.0, 0.0])    # constant speed: no acceleration after the build-up
+    acc = ot.link_smoothness_penalty(xpos, done, 2, "l1")
+    np.testing.assert_allclose(acc[2:], (0.1 + 0.0) / 2, rtol=1e-9)
+    np.testing.assert_allclose(acc[:2], [0.0, (0.05 + 0.3) / 2], rtol=1e-9)
+    jerk = ot.link_smoothness_penalty(xpos, done, 3, "l2")
+    np.testing.assert_allclose(jerk[3:], 0.0, atol=1e-20)
+    # t = 1: jerk = acc(1) = speed(1); t = 2: acc(2) - acc(1)
+    np.testing.assert_allclose(jerk[:3], [0.0, (0.05**2 + 0.3**2) / 2, ((0.1 - 0.05) ** 2 + (0.0 - 0.3) ** 2) / 2], rtol=1e-9)
+
+
+def test_joint_space_penalties_hand_computed():
+    q = np.array([[0, 0, 1, 1, 0, 0, 0, 0.5, -1.2, 0.0], [0, 0, 1, 1, 0, 0, 0, 1.3, 0.2, -0.4]])
+    lim = np.array([[-1.0, 1.0], [-1.0, 1.0], [-np.inf, np.inf]])
+    np.testing.assert_allclose(ot.avoid_limits_penalty(q, lim), [0.2 / 3, 0.3 / 3], rtol=1e-12)
+    # create: 5 % of the range on each side, unlimited joints never penalised, the free joint's row dropped
+    made = ot.avoid_limits_create(np.array([[0, 0], [-1, 1], [0, 2], [0, 0]]), np.array([False, True, True, False]), factor=0.05)
+    np.testing.assert_allclose(made, [[-1.1, 1.1], [-0.1, 2.1], [-np.inf, np.inf]])
+    ctrl = np.array([[2.0, -1.0, 0.5], [0.0, 4.0, -3.0]])
+    np.testing.assert_allclose(ot.torque_penalty(ctrl, (2.0, 1.0, 0.5)), [1.0, (4 + 6) / 3], rtol=1e-12)
+    qvel = np.array([[0] * 6 + [1.0, -2.0, 0.0], [0] * 6 + [3.0, 0.5, -1.0]])
+    np.testing.assert_allclose(ot.energy_penalty(ctrl, qvel, (2.0, 1.0, 0.5)), [(1 + 2 + 0) / 3, (0 + 2 + 6) / 3], rtol=1e-12)
+    np.testing.assert_allclose(ot.joint_deviation_penalty(q, (2, 0), (0.1, 0.0), (2.0, 1.0), "l2"), [0.04 + 0.25, 1.0 + 1.69], rtol=1e-12)
+    np.testing.assert_allclose(ot.joint_deviation_penalty(q, (1,), (0.2,), None, "l1"), [1.4, 0.0], atol=1e-15)
+
+
+def test_body_frame_rewards_hand_computed():
+    from scipy.spatial.transform import Rotation
+
+    def wxyz(r):
+        x, y, z, w = r.as_quat()
+        return np.array([w, x, y, z])
+
+    # a body tilted by angle a about any horizontal axis sees the vertical at cos a
+    a, b = 0.4, 1.1
+    xquat = np.zeros((1, 3, 4)); xquat[0, 0] = [1, 0, 0, 0]
+    xquat[0, 1] = wxyz(Rotation.from_rotvec([a, 0, 0])); xquat[0, 2] = wxyz(Rotation.from_rotvec([0, b, 0]) * Rotation.from_rotvec([0, 0, 0.7]))
+    np.testing.assert_allclose(ot.flat_body_reward(xquat, (1, 2)), [(np.cos(a) + np.cos(b)) / 2], rtol=1e-12)
+    np.testing.assert_allclose(ot.flat_body_reward(xquat, (0,), plane=(1.0, 0, 0)), [1.0], rtol=1e-12)
+    # a base rolled by phi about its x axis: roll = -phi; the yaw before it does not matter
+    phi = 0.3
+    q = np.zeros((1, 7)); q[0, 3:7] = wxyz(Rotation.from_rotvec([0, 0, 1.0]) * Rotation.from_rotvec([phi, 0, 0]))
+    v = np.zeros((1, 6)); v[0, 3] = -0.5
+    k = lambda x: np.exp(-x * x / (2 * 0.25**2)) - 0.1 * abs(x) - 0.1 * x * x  # noqa: E731
+    ang, pose = ot.no_roll_reward(q, v)
+    np.testing.assert_allclose([ang[0], pose[0]], [k(0.5), k(phi)], rtol=1e-12)
+    # position tracking: offset (0.3, -0.1, 0.5) against a command (0.2, 0.1, 0.5): l1 error 0.3, l2 "norm" 0.01 + 0.04
+    xpos = np.zeros((1, 3, 3)); xpos[0, 1] = [1, 1, 1]; xpos[0, 2] = [1.3, 0.9, 1.5]
+    cmd = np.array([[0.2, 0.1, 0.5, 9.0]])
+    np.testing.assert_allclose(ot.position_tracking_reward(xpos, cmd, 2, 1, "l1", 0.25), [np.exp(-0.3**2 / (2 * 0.25**2))], rtol=1e-12)
+    np.testing.assert_allclose(ot.position_tracking_reward(xpos, cmd, 2, 1, "l2", 0.25), [np.exp(-0.05**2 / (2 * 0.25**2))], rtol=1e-12)
+    # feet slip: only the foot with a contact flag set counts
+    contact = np.array([[[0.0, 1.0], [0.0, 0.0]]])    # (T, c = 2, n = 2)
+    vel = np.array([[[1, 2, 2, 0, 0, 0], [3, 0, 4, 0, 0, 12.0]]])
+    np.testing.assert_allclose(ot.feet_slip_penalty(contact, vel), [13.0], rtol=1e-12)
