@@ -451,7 +451,14 @@ enum { KS_CMD_CONST = 0, KS_CMD_LINEAR_VELOCITY = 1, KS_CMD_ANGULAR_VELOCITY = 2
        /* FloatVectorCommand / IntVectorCommand (commands.py:97-170): `dim` <= KS_MAX_VECTOR_COMMAND scalars, each uniform in
           [lo, hi] (integers: lo..hi inclusive), all zero with probability zero_prob; redrawn at an episode start and with
           probability switch_prob per step, otherwise kept.  Draws: u0 switch, u1 zero, u2.. one per scalar. */
-       KS_CMD_FLOAT_VECTOR = 3, KS_CMD_INT_VECTOR = 4 };
+       KS_CMD_FLOAT_VECTOR = 3, KS_CMD_INT_VECTOR = 4,
+       /* StartPositionCommand / StartQuaternionCommand (commands.py:173-215): qpos[0:3] / qpos[3:7] of the state an episode
+          starts from, kept until the next start (dim 3 / 4). */
+       KS_CMD_START_POSITION = 5, KS_CMD_START_QUATERNION = 6,
+       /* BaseHeightCommand (commands.py:773-796): a height uniform in [lo[0], hi[0]] at an episode start; afterwards one draw
+          u0 decides both: replaced by lo + u0 (hi - lo) when u0 < switch_prob (the reference passes one key to both its
+          uniform and its Bernoulli draw, so the two are the same number). */
+       KS_CMD_BASE_HEIGHT = 7 };
 typedef struct KsCommandDesc {
   int32_t kind, index, dim;    /* offset and length inside the command vector */
   float min_vel, max_vel, max_yaw, zero_prob, backward_prob, switch_prob; /* scales already evaluated at the curriculum level */

@@ -124,7 +124,8 @@ class KsGruDesc(ctypes.Structure):
 
 KS_MAX_COMMANDS, KS_COMMAND_DRAWS = 8, 8
 KS_MAX_VECTOR_COMMAND = 6
-CMD_CONST, CMD_LINEAR_VELOCITY, CMD_ANGULAR_VELOCITY, CMD_FLOAT_VECTOR, CMD_INT_VECTOR = range(5)
+(CMD_CONST, CMD_LINEAR_VELOCITY, CMD_ANGULAR_VELOCITY, CMD_FLOAT_VECTOR, CMD_INT_VECTOR, CMD_START_POSITION,
+ CMD_START_QUATERNION, CMD_BASE_HEIGHT) = range(8)
 
 
 class KsCommandDesc(ctypes.Structure):

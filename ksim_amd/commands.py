@@ -117,6 +117,40 @@ class IntVectorCommand(FloatVectorCommand):  # commands.py:136-170: integers lo.
     _kind = T.CMD_INT_VECTOR
 
 
+@dataclass(frozen=True)
+class StartPositionCommand(Command):  # commands.py:173-192: where the episode started
+    _kind, _dim = T.CMD_START_POSITION, 3
+
+    def dim(self):
+        return self._dim
+
+    def desc(self, level):
+        d = T.KsCommandDesc()
+        d.kind, d.dim = self._kind, self._dim
+        return d
+
+
+@dataclass(frozen=True)
+class StartQuaternionCommand(StartPositionCommand):  # commands.py:195-215: the orientation the episode started with
+    _kind, _dim = T.CMD_START_QUATERNION, 4
+
+
+@dataclass(frozen=True)
+class BaseHeightCommand(Command):  # commands.py:773-796
+    min_height: float = 0.0
+    max_height: float = 1.0
+    switch_prob: float = 0.005
+
+    def dim(self):
+        return 1
+
+    def desc(self, level):
+        d = T.KsCommandDesc()
+        d.kind, d.dim, d.switch_prob = T.CMD_BASE_HEIGHT, 1, float(self.switch_prob)
+        d.lo[0], d.hi[0] = float(self.min_height), float(self.max_height)
+        return d
+
+
 class CommandSet:
     def __init__(self, commands: Mapping[str, Command]):
         if len(commands) > T.KS_MAX_COMMANDS:

@@ -830,6 +830,13 @@ __global__ __launch_bounds__(256) void command_kernel(KsCommandIO io) {
       yaw += fminf(fmaxf(ty - yaw, -c.angular_accel), c.angular_accel) * c.ctrl_dt;
     }
     cmd[0] = vel; cmd[1] = yaw; cmd[2] = vel * cosf(yaw); cmd[3] = vel * sinf(yaw); cmd[4] = tv; cmd[5] = ty;
+  } else if (c.kind == KS_CMD_START_POSITION || c.kind == KS_CMD_START_QUATERNION) {
+    if (fresh) {
+      const float* q = io.qpos + e * io.nq + (c.kind == KS_CMD_START_POSITION ? 0 : 3);
+      for (int j = 0; j < c.dim; ++j) cmd[j] = q[j];
+    }
+  } else if (c.kind == KS_CMD_BASE_HEIGHT) {
+    if (fresh || u[0] < c.switch_prob) cmd[0] = c.lo[0] + u[0] * (c.hi[0] - c.lo[0]);
   } else if (c.kind == KS_CMD_FLOAT_VECTOR || c.kind == KS_CMD_INT_VECTOR) {
     if (fresh || u[0] < c.switch_prob) {
       const bool zero = u[1] < c.zero_prob;
@@ -1220,9 +1227,16 @@ extern "C" int ks_commands(ks_stream_t stream, const KsCommandIO* io) {
   if (!io->command) return fail(KS_EINVAL, "ks_commands: the command buffer is required");
   for (int k = 0; k < io->n_commands; ++k) {
     const KsCommandDesc& c = io->commands[k];
-    const int need = c.kind == KS_CMD_LINEAR_VELOCITY ? 6 : (c.kind == KS_CMD_ANGULAR_VELOCITY ? 2 : c.dim);
-    if (c.kind < KS_CMD_CONST || c.kind > KS_CMD_INT_VECTOR) return fail(KS_EINVAL, "ks_commands: command %d: bad kind", k);
-    if (c.kind >= KS_CMD_FLOAT_VECTOR && c.dim > KS_MAX_VECTOR_COMMAND) return fail(KS_ELIMIT, "ks_commands: command %d: %d scalars (at most %d)", k, c.dim, KS_MAX_VECTOR_COMMAND);
+    int need = c.dim;
+    if (c.kind == KS_CMD_LINEAR_VELOCITY) need = 6;
+    if (c.kind == KS_CMD_ANGULAR_VELOCITY) need = 2;
+    if (c.kind == KS_CMD_START_POSITION) need = 3;
+    if (c.kind == KS_CMD_START_QUATERNION) need = 4;
+    if (c.kind == KS_CMD_BASE_HEIGHT) need = 1;
+    if (c.kind < KS_CMD_CONST || c.kind > KS_CMD_BASE_HEIGHT) return fail(KS_EINVAL, "ks_commands: command %d: bad kind", k);
+    if ((c.kind == KS_CMD_START_POSITION || c.kind == KS_CMD_START_QUATERNION) && (!io->qpos || io->nq < 7))
+      return fail(KS_EINVAL, "ks_commands: command %d reads the pose of a floating base", k);
+    if ((c.kind == KS_CMD_FLOAT_VECTOR || c.kind == KS_CMD_INT_VECTOR) && c.dim > KS_MAX_VECTOR_COMMAND) return fail(KS_ELIMIT, "ks_commands: command %d: %d scalars (at most %d)", k, c.dim, KS_MAX_VECTOR_COMMAND);
     if (c.dim != need || c.dim < 1 || c.index < 0 || c.index + c.dim > io->command_dim) return fail(KS_EINVAL, "ks_commands: command %d: [%d,%d) outside the %d-wide command vector or of the wrong length", k, c.index, c.index + c.dim, io->command_dim);
     if ((c.kind == KS_CMD_LINEAR_VELOCITY || c.kind == KS_CMD_ANGULAR_VELOCITY) && (!io->qpos || !io->qvel || io->nq < 7 || io->nv < 6))
       return fail(KS_EINVAL, "ks_commands: velocity commands read the state of a floating base");

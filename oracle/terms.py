@@ -499,6 +499,18 @@ def angular_velocity_command(prev, qvel, u, fresh, *, max_vel, min_vel=0.0, zero
     return np.array([vel, tv])
 
 
+def start_pose_command(prev, qpos, fresh, quaternion=False):  # commands.py:173-215
+    return np.array(qpos[3:7] if quaternion else qpos[:3], dtype=np.float64) if fresh else np.asarray(prev, dtype=np.float64)
+
+
+def base_height_command(prev, u, fresh, *, min_height, max_height, switch_prob=0.005):  # commands.py:773-796
+    """`u` is the single uniform draw of the step: the reference hands the same key to jax.random.uniform and to
+    jax.random.bernoulli (which compares a uniform draw of that key with p), so the new height and the decision to switch
+    come from one number."""
+    new = min_height + u * (max_height - min_height)
+    return new if (fresh or u < switch_prob) else prev
+
+
 def position_velocity_actuator_torque(action, qpos, qvel, kp, kd, ctrl_clip, pos_noise=0.0, vel_noise=0.0, torque_noise=0.0):
     """PositionVelocityActuator.get_ctrl (ksim/actuators.py:261-293): action = (position targets, velocity targets)."""
     n = len(qpos)

@@ -680,6 +680,42 @@ def test_velocity_commands_against_oracle():
         cs.update(a, t32(qpos), t32(qvel), uniform=t32(u[:, :2]))
 
 
+def test_start_pose_and_base_height_commands():
+    """StartPositionCommand / StartQuaternionCommand hold the pose an episode started from; BaseHeightCommand redraws its height
+    at a start and, with one draw deciding both, when that draw falls under switch_prob."""
+    from ksim_amd import _lib_terms as T
+    from ksim_amd.commands import BaseHeightCommand, CommandSet, StartPositionCommand, StartQuaternionCommand
+
+    N, steps = 37, 10
+    rng = np.random.default_rng(43)
+    hp = dict(min_height=0.6, max_height=1.1, switch_prob=0.3)
+    cs = CommandSet({"pos": StartPositionCommand(), "height": BaseHeightCommand(**hp), "quat": StartQuaternionCommand()})
+    assert cs.command_dim == 8 and cs.slices["quat"] == slice(4, 8)
+    cmd = cs.initial(N, DEV)
+    want = np.zeros((N, 8))
+    switched = 0
+    for k in range(steps):
+        qpos = rng.normal(size=(N, 27)).astype(np.float32)
+        qvel = rng.normal(size=(N, 26)).astype(np.float32)
+        u = rng.random((N, 3, T.KS_COMMAND_DRAWS)).astype(np.float32)
+        fresh = np.ones(N, bool) if k == 0 else rng.random(N) < 0.15
+        rec = torch.empty(N, 8, device=DEV)
+        cs.update(cmd, t32(qpos), t32(qvel), fresh=torch.from_numpy(fresh.astype(np.uint8)).to(DEV), record=rec, uniform=t32(u))
+        np.testing.assert_allclose(rec.cpu().numpy(), want, rtol=1e-6, atol=1e-7)
+        for e in range(N):
+            want[e, :3] = ot.start_pose_command(want[e, :3], qpos[e], bool(fresh[e]))
+            new = ot.base_height_command(want[e, 3], float(u[e, 1, 0]), bool(fresh[e]), **hp)
+            switched += (not fresh[e]) and new != want[e, 3]
+            want[e, 3] = new
+            want[e, 4:] = ot.start_pose_command(want[e, 4:], qpos[e], bool(fresh[e]), quaternion=True)
+        np.testing.assert_allclose(cmd.cpu().numpy(), want, rtol=1e-6, atol=1e-6)
+    assert switched > 20
+    # a switched height comes from a draw below switch_prob, so it sits in the lowest part of the range
+    assert (want[:, 3] >= 0.6).all() and (want[:, 3] <= 1.1).all()
+    with pytest.raises(Exception, match="floating base"):
+        cs.update(cmd, t32(qpos[:, :5]), t32(qvel), all_fresh=True, seed=1, step=1)
+
+
 def test_vector_commands():
     """FloatVectorCommand / IntVectorCommand: the properties the reference's own tests check (shape, bounds, a command
     that never switches stays what it was, reference tests/test_commands.py:64-96) and the draw arithmetic."""

@@ -501,3 +501,14 @@ def test_body_frame_rewards_hand_computed():
     contact = np.array([[[0.0, 1.0], [0.0, 0.0]]])    # (T, c = 2, n = 2)
     vel = np.array([[[1, 2, 2, 0, 0, 0], [3, 0, 4, 0, 0, 12.0]]])
     np.testing.assert_allclose(ot.feet_slip_penalty(contact, vel), [13.0], rtol=1e-12)
+
+
+def test_start_pose_and_base_height_commands_hand_computed():
+    q = np.array([1.0, 2.0, 3.0, 0.5, 0.5, 0.5, 0.5, 9.0])
+    np.testing.assert_array_equal(ot.start_pose_command([0, 0, 0], q, True), [1, 2, 3])
+    np.testing.assert_array_equal(ot.start_pose_command([7, 7, 7], q, False), [7, 7, 7])
+    np.testing.assert_array_equal(ot.start_pose_command([0] * 4, q, True, quaternion=True), [0.5] * 4)
+    kw = dict(min_height=0.5, max_height=1.5, switch_prob=0.1)
+    assert ot.base_height_command(0.8, 0.75, True, **kw) == 1.25          # episode start: always a new height
+    assert ot.base_height_command(0.8, 0.75, False, **kw) == 0.8          # draw above switch_prob: kept
+    assert ot.base_height_command(0.8, 0.04, False, **kw) == pytest.approx(0.54)   # the same draw picks the height
