@@ -781,8 +781,11 @@ enum { KS_REW_STAY_ALIVE = 0, KS_REW_BASE_HEIGHT = 1, KS_REW_BASE_HEIGHT_RANGE =
        KS_REW_LINK_SMOOTH = 25,  /* LinkAcceleration / JerkPenalty (rewards.py:808-840): mean over the bodies 1.. of
                                     norm(second / third (p0 = 2 / 3) difference of |xpos(t) - xpos(t - 1)|), padded and
                                     zeroed like KS_REW_JOINT_SMOOTH; `norm` is the l1 / l2 choice */
-       KS_REW_FEET_SLIP = 26     /* sum over `norm` feet of |obs[index2 + 6 f .. + 6]| while any of the foot's `count` contact
-                                    flags obs[index + c * norm + f] > 0.5 (rewards.py:1088-1105) */ };
+       KS_REW_FEET_SLIP = 26,    /* sum over `norm` feet of |obs[index2 + 6 f .. + 6]| while any of the foot's `count` contact
+                                    flags obs[index + c * norm + f] > 0.5 (rewards.py:1088-1105) */
+       KS_REW_REACHABILITY = 27, /* sum over the joints of norm(max(0, |action - qpos[7:]| - params[u])) (rewards.py:1108-1129) */
+       KS_REW_INTERSECTION = 28  /* 1 when two of the `norm` points obs[index + 3 i .. + 3] are closer than p0, else 0
+                                    (rewards.py:1417-1430) */ };
 enum { KS_NORM_L1 = 0, KS_NORM_L2 = 1 }; /* xax.get_norm: l1 = |x|, l2 = x^2 (reference tests/test_rewards.py:95-98) */
 #define KS_MAX_REWARD_PARAMS 320
 typedef struct KsRewardDesc {

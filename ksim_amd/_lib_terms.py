@@ -77,7 +77,8 @@ class KsMlpDesc(ctypes.Structure):
 (REW_STAY_ALIVE, REW_BASE_HEIGHT, REW_BASE_HEIGHT_RANGE, REW_ACTION_VEL, REW_ACTION_ACC, REW_ACTION_JERK,
  REW_UPRIGHT_ANGVEL, REW_UPRIGHT_LINVEL, REW_UPRIGHT_POSE, REW_AMP, REW_STATEFUL, REW_LINVEL_CMD, REW_ANGVEL_CMD,
  REW_OFF_AXIS, REW_MOTIONLESS, REW_FORCE, REW_JOINT_SMOOTH, REW_AVOID_LIMITS, REW_TORQUE, REW_ENERGY, REW_JOINT_DEVIATION,
- REW_FLAT_BODY, REW_POSITION_TRACKING, REW_NO_ROLL_ANGVEL, REW_NO_ROLL_POSE, REW_LINK_SMOOTH, REW_FEET_SLIP) = range(27)
+ REW_FLAT_BODY, REW_POSITION_TRACKING, REW_NO_ROLL_ANGVEL, REW_NO_ROLL_POSE, REW_LINK_SMOOTH, REW_FEET_SLIP,
+ REW_REACHABILITY, REW_INTERSECTION) = range(29)
 KS_MAX_REWARD_PARAMS = 320
 KS_MAX_REWARD_SCANS, KS_MAX_SCAN_BODIES = 4, 8
 SCAN_FEET_AIR_TIME, SCAN_SPARSE_TARGET_HEIGHT = 0, 1

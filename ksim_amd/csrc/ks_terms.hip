@@ -706,6 +706,23 @@ __global__ __launch_bounds__(256) void rewards_kernel(KsRewardIO io) {
         }
         val = s;
       } break;
+      case KS_REW_REACHABILITY: {
+        const float* dm = io.params + r.param_offset;
+        const float* a0 = io.action + idx * io.nu;
+        float s = 0.f;
+        for (int u = 0; u < io.nu; ++u) {
+          const float x = fmaxf(0.f, fabsf(a0[u] - q[7 + u]) - dm[u]);
+          s += r.norm == KS_NORM_L1 ? x : x * x;
+        }
+        val = s;
+      } break;
+      case KS_REW_INTERSECTION: {
+        const float* ob = io.obs + idx * io.obs_dim + r.index;
+        bool close = false;
+        for (int i = 1; i < r.norm; ++i)
+          for (int k = 0; k < i; ++k) close = close || dist3(ob + 3 * i, ob + 3 * k) < r.p0;
+        val = close ? 1.f : 0.f;
+      } break;
       default: break;
     }
     val *= r.scale;
@@ -1093,7 +1110,7 @@ extern "C" int ks_rewards(ks_stream_t stream, const KsRewardIO* io) {
   if (!io->done) return fail(KS_EINVAL, "ks_rewards: done is required");
   for (int j = 0; j < io->n_rewards; ++j) {
     const int k = io->rewards[j].kind;
-    if (k < KS_REW_STAY_ALIVE || k > KS_REW_FEET_SLIP) return fail(KS_EINVAL, "ks_rewards: term %d: bad kind", j);
+    if (k < KS_REW_STAY_ALIVE || k > KS_REW_INTERSECTION) return fail(KS_EINVAL, "ks_rewards: term %d: bad kind", j);
     const KsRewardDesc& rd = io->rewards[j];
     if (k == KS_REW_LINVEL_CMD || k == KS_REW_ANGVEL_CMD) {
       const int span = k == KS_REW_LINVEL_CMD ? 4 : 1;
@@ -1162,6 +1179,14 @@ extern "C" int ks_rewards(ks_stream_t stream, const KsRewardIO* io) {
           if (!io->obs || r.norm < 1 || r.count < 1 || r.index < 0 || r.index + r.count * r.norm > io->obs_dim || r.index2 < 0 ||
               r.index2 + 6 * r.norm > io->obs_dim)
             return fail(KS_EINVAL, "ks_rewards: term %d: contact or velocity block outside the observation", j);
+          uses_params = false;
+          break;
+        case KS_REW_REACHABILITY:
+          if (!io->qpos || !io->action || io->nu < 1 || io->nq != io->nu + 7) return fail(KS_EINVAL, "ks_rewards: term %d needs actions and qpos with one joint per action behind a floating base", j);
+          need_params = io->nu;
+          break;
+        case KS_REW_INTERSECTION:
+          if (!io->obs || r.norm < 2 || r.index < 0 || r.index + 3 * r.norm > io->obs_dim) return fail(KS_EINVAL, "ks_rewards: term %d: position block outside the observation", j);
           uses_params = false;
           break;
         default: uses_params = false; break;

@@ -305,6 +305,31 @@ class FeetSlipPenalty(Reward):  # rewards.py:1088-1105
         return [(None, T.REW_FEET_SLIP, n, 0.0, 0.0, 0.0, 0.0, c.start, _extra(index2=v.start, count=nc_ // n))]
 
 
+@dataclass(frozen=True)
+class ReachabilityPenalty(Reward):  # rewards.py:1108-1129
+    delta_max_j: tuple = ()
+    squared: bool = True
+
+    def descs(self):
+        return [(None, T.REW_REACHABILITY, T.NORM_L2 if self.squared else T.NORM_L1, 0.0, 0.0, 0.0, 0.0, 0,
+                 _extra(params=[float(x) for x in self.delta_max_j]))]
+
+
+@dataclass(frozen=True)
+class IntersectionPenalty(Reward):  # rewards.py:1417-1430
+    position_obs: str = ""
+    min_distance: float = 0.0
+
+    def descs(self):  # pragma: no cover
+        raise ValueError("IntersectionPenalty reads a named observation: pass obs_slices to get_rewards")
+
+    def descs_in(self, obs_slices, command_slices):
+        sl = _named(obs_slices, self.position_obs, "observation")
+        if (sl.stop - sl.start) % 3 != 0:
+            raise ValueError(f"position observation of {sl.stop - sl.start} entries is not (n, 3)")
+        return [(None, T.REW_INTERSECTION, (sl.stop - sl.start) // 3, self.min_distance, 0.0, 0.0, 0.0, sl.start)]
+
+
 DISCRIMINATOR_OUTPUT_KEY = "_discriminator_output"  # ksim/task/amp.py:47
 
 
@@ -650,7 +675,7 @@ def get_rewards(trajectory: Trajectory, rewards: Mapping[str, Reward], clip_min:
             raise KeyError('command-tracking rewards read trajectory.command["_buffer"] (T, N, command_dim)')
         cmd = tensor(cmd, torch.float32, cmd.shape[-1])
         io.command, io.command_dim = cmd.data_ptr(), cmd.shape[-1]
-    if kinds & {T.REW_FORCE, T.REW_FEET_SLIP}:
+    if kinds & {T.REW_FORCE, T.REW_FEET_SLIP, T.REW_INTERSECTION}:
         ob_ = trajectory.obs[obs_key]
         ob_ = tensor(ob_, torch.float32, ob_.shape[-1])
         io.obs, io.obs_dim = ob_.data_ptr(), ob_.shape[-1]

@@ -174,6 +174,19 @@ def feet_slip_penalty(contact_tcn, velocity_tn6):  # rewards.py:1095-1105
     return np.where(touching, speed, 0.0).sum(axis=-1)
 
 
+def reachability_penalty(action_tj, qpos_tq, delta_max_j, squared=True):  # rewards.py:1119-1129
+    excess = np.maximum(0.0, np.abs(np.asarray(action_tj, dtype=np.float64) - np.asarray(qpos_tq, dtype=np.float64)[:, 7:])
+                        - np.asarray(delta_max_j, dtype=np.float64))
+    return (excess**2 if squared else excess).sum(axis=-1)
+
+
+def intersection_penalty(position_tn3, min_distance):  # rewards.py:1424-1430
+    p = np.asarray(position_tn3, dtype=np.float64)
+    dist = np.linalg.norm(p[:, :, None, :] - p[:, None, :, :], axis=-1)
+    dist = dist + np.triu(np.ones_like(dist)) * min_distance * 2
+    return np.where((dist < min_distance).any(axis=(-2, -1)), 1.0, 0.0)
+
+
 def stay_alive_reward(done_t, success_t, balance=100.0, success_reward=None):  # rewards.py:178-188
     alive = 1.0 / balance
     return np.where(done_t, np.where(success_t, alive if success_reward is None else success_reward, -1.0), alive)

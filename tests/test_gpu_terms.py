@@ -638,6 +638,35 @@ def test_smoothness_limits_effort_and_body_frame_rewards():
         rw.get_rewards(dataclasses.replace(traj, ctrl=None), {"t": rewards["torque"]})
 
 
+def test_reachability_and_intersection_penalties():
+    from ksim_amd import rewards as rw
+    from ksim_amd.types import Trajectory
+
+    Tn, N, nu = 9, 21, 6
+    rng = np.random.default_rng(5)
+    qpos = rng.normal(size=(Tn, N, nu + 7)) * 0.3
+    action = rng.normal(size=(Tn, N, nu)) * 0.3
+    obs = rng.normal(size=(Tn, N, 11)) * 0.12
+    dm = tuple(float(x) for x in np.linspace(0.05, 0.3, nu))
+    traj = Trajectory(qpos=t32(qpos), qvel=None, xpos=None, xquat=None, ctrl=None, obs={"obs": t32(obs)}, command={}, event_state={},
+                      action=t32(action), done=torch.zeros(Tn, N, dtype=torch.bool, device=DEV), success=None, timestep=None)
+    st = rw.get_rewards(traj, {"reach": rw.ReachabilityPenalty(scale=2.0, delta_max_j=dm), "reach1": rw.ReachabilityPenalty(delta_max_j=dm, squared=False),
+                               "cross": rw.IntersectionPenalty(scale=0.5, position_obs="feet", min_distance=0.15)},
+                        obs_slices={"feet": slice(1, 10)})
+    f32 = lambda a: a.astype(np.float32).astype(np.float64)  # noqa: E731
+    q, a, o = f32(qpos), f32(action), f32(obs)
+    for e in range(N):
+        np.testing.assert_allclose(st.components["reach"][:, e].cpu().numpy(), -2.0 * ot.reachability_penalty(a[:, e], q[:, e], dm), rtol=2e-5, atol=1e-6)
+        np.testing.assert_allclose(st.components["reach1"][:, e].cpu().numpy(), -ot.reachability_penalty(a[:, e], q[:, e], dm, False), rtol=2e-5, atol=1e-6)
+        np.testing.assert_array_equal(st.components["cross"][:, e].cpu().numpy(), -0.5 * ot.intersection_penalty(o[:, e, 1:10].reshape(Tn, 3, 3), 0.15))
+    frac = float((st.components["cross"] != 0).float().mean())
+    assert 0.1 < frac < 0.9
+    short = Trajectory(qpos=t32(qpos[..., :10]), qvel=None, xpos=None, xquat=None, ctrl=None, obs={}, command={}, event_state={},
+                       action=t32(action), done=torch.zeros(Tn, N, dtype=torch.bool, device=DEV), success=None, timestep=None)
+    with pytest.raises(Exception, match="one joint per action"):
+        rw.get_rewards(short, {"reach": rw.ReachabilityPenalty(delta_max_j=dm)})
+
+
 def test_velocity_commands_against_oracle():
     """LinearVelocityCommand / AngularVelocityCommand over several control steps with explicit draws: episode starts,
     slewing, switches, zero and backward targets; the recorded copy is the incoming command."""

@@ -512,3 +512,13 @@ def test_start_pose_and_base_height_commands_hand_computed():
     assert ot.base_height_command(0.8, 0.75, True, **kw) == 1.25          # episode start: always a new height
     assert ot.base_height_command(0.8, 0.75, False, **kw) == 0.8          # draw above switch_prob: kept
     assert ot.base_height_command(0.8, 0.04, False, **kw) == pytest.approx(0.54)   # the same draw picks the height
+
+
+def test_reachability_and_intersection_hand_computed():
+    q = np.array([[0, 0, 1, 1, 0, 0, 0, 0.5, -0.2]])
+    a = np.array([[0.9, -0.25]])
+    np.testing.assert_allclose(ot.reachability_penalty(a, q, (0.1, 0.1)), [0.3**2], rtol=1e-12)
+    np.testing.assert_allclose(ot.reachability_penalty(a, q, (0.1, 0.01), squared=False), [0.3 + 0.04], rtol=1e-12)
+    pts = np.array([[[0, 0, 0], [0.3, 0, 0], [0, 0.05, 0]], [[0, 0, 0], [0.3, 0, 0], [0, 0.5, 0]]], dtype=float)
+    np.testing.assert_array_equal(ot.intersection_penalty(pts, 0.1), [1.0, 0.0])
+    np.testing.assert_array_equal(ot.intersection_penalty(pts[:, :1], 0.1), [0.0, 0.0])   # a point is never too close to itself
