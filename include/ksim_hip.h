@@ -458,7 +458,14 @@ enum { KS_CMD_CONST = 0, KS_CMD_LINEAR_VELOCITY = 1, KS_CMD_ANGULAR_VELOCITY = 2
        /* BaseHeightCommand (commands.py:773-796): a height uniform in [lo[0], hi[0]] at an episode start; afterwards one draw
           u0 decides both: replaced by lo + u0 (hi - lo) when u0 < switch_prob (the reference passes one key to both its
           uniform and its Bernoulli draw, so the two are the same number). */
-       KS_CMD_BASE_HEIGHT = 7 };
+       KS_CMD_BASE_HEIGHT = 7,
+       /* SinusoidalGaitCommand (commands.py:696-770): moving flag, phase, then one target foot height per foot (dim = 2 + feet,
+          feet <= KS_MAX_VECTOR_COMMAND).  lo[0..4] = gait_period, max_height, height_offset, stance_ratio, moving_threshold.
+          Start: flag 1, phase 0.  Step: phase <- (phase + ctrl_dt / gait_period) mod 1 while the flag is set, else 0; when
+          |qvel[0:2]| <= moving_threshold the flag and the phase drop to 0 (the flag stays down until the next start).
+          Foot f at phase p_f = (phase + f / feet) mod 1 gets height_offset + max_height sin(pi (p_f - stance) / (1 - stance))
+          in swing (p_f >= stance), height_offset in stance. */
+       KS_CMD_SINUSOIDAL_GAIT = 8 };
 typedef struct KsCommandDesc {
   int32_t kind, index, dim;    /* offset and length inside the command vector */
   float min_vel, max_vel, max_yaw, zero_prob, backward_prob, switch_prob; /* scales already evaluated at the curriculum level */
@@ -784,6 +791,8 @@ enum { KS_REW_STAY_ALIVE = 0, KS_REW_BASE_HEIGHT = 1, KS_REW_BASE_HEIGHT_RANGE =
        KS_REW_FEET_SLIP = 26,    /* sum over `norm` feet of |obs[index2 + 6 f .. + 6]| while any of the foot's `count` contact
                                     flags obs[index + c * norm + f] > 0.5 (rewards.py:1088-1105) */
        KS_REW_REACHABILITY = 27, /* sum over the joints of norm(max(0, |action - qpos[7:]| - params[u])) (rewards.py:1108-1129) */
+       KS_REW_SINUSOIDAL_GAIT = 29, /* 1 - sum over `norm` feet of |obs[index + 3 f + 2] - command[index2 + f]| / p0
+                                       (rewards.py:1320-1335); index2 = where the command's heights start */
        KS_REW_INTERSECTION = 28  /* 1 when two of the `norm` points obs[index + 3 i .. + 3] are closer than p0, else 0
                                     (rewards.py:1417-1430) */ };
 enum { KS_NORM_L1 = 0, KS_NORM_L2 = 1 }; /* xax.get_norm: l1 = |x|, l2 = x^2 (reference tests/test_rewards.py:95-98) */

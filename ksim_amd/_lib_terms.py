@@ -78,7 +78,7 @@ class KsMlpDesc(ctypes.Structure):
  REW_UPRIGHT_ANGVEL, REW_UPRIGHT_LINVEL, REW_UPRIGHT_POSE, REW_AMP, REW_STATEFUL, REW_LINVEL_CMD, REW_ANGVEL_CMD,
  REW_OFF_AXIS, REW_MOTIONLESS, REW_FORCE, REW_JOINT_SMOOTH, REW_AVOID_LIMITS, REW_TORQUE, REW_ENERGY, REW_JOINT_DEVIATION,
  REW_FLAT_BODY, REW_POSITION_TRACKING, REW_NO_ROLL_ANGVEL, REW_NO_ROLL_POSE, REW_LINK_SMOOTH, REW_FEET_SLIP,
- REW_REACHABILITY, REW_INTERSECTION) = range(29)
+ REW_REACHABILITY, REW_INTERSECTION, REW_SINUSOIDAL_GAIT) = range(30)
 KS_MAX_REWARD_PARAMS = 320
 KS_MAX_REWARD_SCANS, KS_MAX_SCAN_BODIES = 4, 8
 SCAN_FEET_AIR_TIME, SCAN_SPARSE_TARGET_HEIGHT = 0, 1
@@ -126,7 +126,7 @@ class KsGruDesc(ctypes.Structure):
 KS_MAX_COMMANDS, KS_COMMAND_DRAWS = 8, 8
 KS_MAX_VECTOR_COMMAND = 6
 (CMD_CONST, CMD_LINEAR_VELOCITY, CMD_ANGULAR_VELOCITY, CMD_FLOAT_VECTOR, CMD_INT_VECTOR, CMD_START_POSITION,
- CMD_START_QUATERNION, CMD_BASE_HEIGHT) = range(8)
+ CMD_START_QUATERNION, CMD_BASE_HEIGHT, CMD_SINUSOIDAL_GAIT) = range(9)
 
 
 class KsCommandDesc(ctypes.Structure):

@@ -151,6 +151,27 @@ class BaseHeightCommand(Command):  # commands.py:773-796
         return d
 
 
+@dataclass(frozen=True)
+class SinusoidalGaitCommand(Command):  # commands.py:696-770: layout moving_flag, phase, height per foot
+    gait_period: float = 1.0
+    ctrl_dt: float = 0.02
+    max_height: float = 0.1
+    height_offset: float = 0.0
+    num_feet: int = 2
+    stance_ratio: float = 0.6
+    moving_threshold: float = 0.05
+
+    def dim(self):
+        return 2 + self.num_feet
+
+    def desc(self, level):
+        d = T.KsCommandDesc()
+        d.kind, d.dim, d.ctrl_dt = T.CMD_SINUSOIDAL_GAIT, 2 + self.num_feet, float(self.ctrl_dt)
+        for j, x in enumerate((self.gait_period, self.max_height, self.height_offset, self.stance_ratio, self.moving_threshold)):
+            d.lo[j] = float(x)
+        return d
+
+
 class CommandSet:
     def __init__(self, commands: Mapping[str, Command]):
         if len(commands) > T.KS_MAX_COMMANDS:

@@ -716,6 +716,13 @@ __global__ __launch_bounds__(256) void rewards_kernel(KsRewardIO io) {
         }
         val = s;
       } break;
+      case KS_REW_SINUSOIDAL_GAIT: {
+        const float* ob = io.obs + idx * io.obs_dim + r.index;
+        const float* hc = io.command + idx * io.command_dim + r.index2;
+        float s = 0.f;
+        for (int f = 0; f < r.norm; ++f) s += fabsf(ob[3 * f + 2] - hc[f]);
+        val = 1.f - s / r.p0;
+      } break;
       case KS_REW_INTERSECTION: {
         const float* ob = io.obs + idx * io.obs_dim + r.index;
         bool close = false;
@@ -851,6 +858,24 @@ __global__ __launch_bounds__(256) void command_kernel(KsCommandIO io) {
     if (fresh) {
       const float* q = io.qpos + e * io.nq + (c.kind == KS_CMD_START_POSITION ? 0 : 3);
       for (int j = 0; j < c.dim; ++j) cmd[j] = q[j];
+    }
+  } else if (c.kind == KS_CMD_SINUSOIDAL_GAIT) {
+    const int feet = c.dim - 2;
+    const float period = c.lo[0], max_h = c.lo[1], offset = c.lo[2], stance = c.lo[3], threshold = c.lo[4];
+    float flag = 1.f, phase = 0.f;
+    if (!fresh) {
+      flag = cmd[0];
+      const float stepped = cmd[1] + c.ctrl_dt / period;
+      phase = flag != 0.f ? stepped - floorf(stepped) : 0.f;
+      const bool moving = sqrtf(qv[0] * qv[0] + qv[1] * qv[1]) > threshold;
+      if (!moving) { flag = 0.f; phase = 0.f; }
+    }
+    cmd[0] = flag; cmd[1] = phase;
+    for (int f = 0; f < feet; ++f) {
+      float pf = phase + (float)f / (float)feet;
+      pf -= floorf(pf);
+      const float prog = fminf(fmaxf((pf - stance) / (1.f - stance), 0.f), 1.f);
+      cmd[2 + f] = (pf >= stance ? max_h * sinf(3.14159265358979323846f * prog) : 0.f) + offset;
     }
   } else if (c.kind == KS_CMD_BASE_HEIGHT) {
     if (fresh || u[0] < c.switch_prob) cmd[0] = c.lo[0] + u[0] * (c.hi[0] - c.lo[0]);
@@ -1110,7 +1135,7 @@ extern "C" int ks_rewards(ks_stream_t stream, const KsRewardIO* io) {
   if (!io->done) return fail(KS_EINVAL, "ks_rewards: done is required");
   for (int j = 0; j < io->n_rewards; ++j) {
     const int k = io->rewards[j].kind;
-    if (k < KS_REW_STAY_ALIVE || k > KS_REW_INTERSECTION) return fail(KS_EINVAL, "ks_rewards: term %d: bad kind", j);
+    if (k < KS_REW_STAY_ALIVE || k > KS_REW_SINUSOIDAL_GAIT) return fail(KS_EINVAL, "ks_rewards: term %d: bad kind", j);
     const KsRewardDesc& rd = io->rewards[j];
     if (k == KS_REW_LINVEL_CMD || k == KS_REW_ANGVEL_CMD) {
       const int span = k == KS_REW_LINVEL_CMD ? 4 : 1;
@@ -1185,6 +1210,12 @@ extern "C" int ks_rewards(ks_stream_t stream, const KsRewardIO* io) {
           if (!io->qpos || !io->action || io->nu < 1 || io->nq != io->nu + 7) return fail(KS_EINVAL, "ks_rewards: term %d needs actions and qpos with one joint per action behind a floating base", j);
           need_params = io->nu;
           break;
+        case KS_REW_SINUSOIDAL_GAIT:
+          if (!io->obs || !io->command || r.norm < 1 || r.index < 0 || r.index + 3 * r.norm > io->obs_dim || r.index2 < 0 ||
+              r.index2 + r.norm > io->command_dim || !(r.p0 != 0.f))
+            return fail(KS_EINVAL, "ks_rewards: term %d: foot positions or target heights outside their vectors, or zero max height", j);
+          uses_params = false;
+          break;
         case KS_REW_INTERSECTION:
           if (!io->obs || r.norm < 2 || r.index < 0 || r.index + 3 * r.norm > io->obs_dim) return fail(KS_EINVAL, "ks_rewards: term %d: position block outside the observation", j);
           uses_params = false;
@@ -1258,7 +1289,11 @@ extern "C" int ks_commands(ks_stream_t stream, const KsCommandIO* io) {
     if (c.kind == KS_CMD_START_POSITION) need = 3;
     if (c.kind == KS_CMD_START_QUATERNION) need = 4;
     if (c.kind == KS_CMD_BASE_HEIGHT) need = 1;
-    if (c.kind < KS_CMD_CONST || c.kind > KS_CMD_BASE_HEIGHT) return fail(KS_EINVAL, "ks_commands: command %d: bad kind", k);
+    if (c.kind == KS_CMD_SINUSOIDAL_GAIT) {
+      if (c.dim < 3 || c.dim > 2 + KS_MAX_VECTOR_COMMAND) return fail(KS_ELIMIT, "ks_commands: command %d: 1..%d feet", k, KS_MAX_VECTOR_COMMAND);
+      if (!(c.lo[0] > 0.f) || !(c.lo[3] < 1.f) || !io->qvel || io->nv < 2) return fail(KS_EINVAL, "ks_commands: command %d: gait period, stance ratio or the base velocity missing", k);
+    }
+    if (c.kind < KS_CMD_CONST || c.kind > KS_CMD_SINUSOIDAL_GAIT) return fail(KS_EINVAL, "ks_commands: command %d: bad kind", k);
     if ((c.kind == KS_CMD_START_POSITION || c.kind == KS_CMD_START_QUATERNION) && (!io->qpos || io->nq < 7))
       return fail(KS_EINVAL, "ks_commands: command %d reads the pose of a floating base", k);
     if ((c.kind == KS_CMD_FLOAT_VECTOR || c.kind == KS_CMD_INT_VECTOR) && c.dim > KS_MAX_VECTOR_COMMAND) return fail(KS_ELIMIT, "ks_commands: command %d: %d scalars (at most %d)", k, c.dim, KS_MAX_VECTOR_COMMAND);

@@ -330,6 +330,27 @@ class IntersectionPenalty(Reward):  # rewards.py:1417-1430
         return [(None, T.REW_INTERSECTION, (sl.stop - sl.start) // 3, self.min_distance, 0.0, 0.0, 0.0, sl.start)]
 
 
+@dataclass(frozen=True)
+class SinusoidalGaitReward(Reward):  # rewards.py:1320-1335
+    ctrl_dt: float = 0.02
+    max_height: float = 0.1
+    pos_obs: str = ""
+    pos_cmd: str = ""
+    num_feet: int = 2
+
+    def descs(self):  # pragma: no cover
+        raise ValueError("SinusoidalGaitReward reads a named observation and command: pass obs_slices and command_slices to get_rewards")
+
+    def descs_in(self, obs_slices, command_slices):
+        if self.pos_cmd not in command_slices:
+            raise ValueError(f"Command {self.pos_cmd} not found! Ensure that it is in the task.")
+        ob, cm = _named(obs_slices, self.pos_obs, "observation"), command_slices[self.pos_cmd]
+        feet = cm.stop - cm.start - 2
+        if ob.stop - ob.start != 3 * feet:
+            raise ValueError(f"position observation of {ob.stop - ob.start} entries is not ({feet}, 3) for the command's {feet} feet")
+        return [(None, T.REW_SINUSOIDAL_GAIT, feet, self.max_height, 0.0, 0.0, 0.0, ob.start, _extra(index2=cm.start + 2))]
+
+
 DISCRIMINATOR_OUTPUT_KEY = "_discriminator_output"  # ksim/task/amp.py:47
 
 
@@ -669,13 +690,13 @@ def get_rewards(trajectory: Trajectory, rewards: Mapping[str, Reward], clip_min:
                 raise _lib.KsError(f"trajectory.{name} has {flat.shape[-1]} entries per step: not (nb, {per}) for the other leaf's nb")
             io.nb = flat.shape[-1] // per
             setattr(io, name, flat.data_ptr())
-    if kinds & {T.REW_LINVEL_CMD, T.REW_ANGVEL_CMD, T.REW_POSITION_TRACKING}:
+    if kinds & {T.REW_LINVEL_CMD, T.REW_ANGVEL_CMD, T.REW_POSITION_TRACKING, T.REW_SINUSOIDAL_GAIT}:
         cmd = trajectory.command.get("_buffer") if trajectory.command else None
         if cmd is None:
             raise KeyError('command-tracking rewards read trajectory.command["_buffer"] (T, N, command_dim)')
         cmd = tensor(cmd, torch.float32, cmd.shape[-1])
         io.command, io.command_dim = cmd.data_ptr(), cmd.shape[-1]
-    if kinds & {T.REW_FORCE, T.REW_FEET_SLIP, T.REW_INTERSECTION}:
+    if kinds & {T.REW_FORCE, T.REW_FEET_SLIP, T.REW_INTERSECTION, T.REW_SINUSOIDAL_GAIT}:
         ob_ = trajectory.obs[obs_key]
         ob_ = tensor(ob_, torch.float32, ob_.shape[-1])
         io.obs, io.obs_dim = ob_.data_ptr(), ob_.shape[-1]

@@ -524,6 +524,27 @@ def base_height_command(prev, u, fresh, *, min_height, max_height, switch_prob=0
     return new if (fresh or u < switch_prob) else prev
 
 
+def sinusoidal_gait_command(prev, qvel, fresh, *, gait_period, ctrl_dt, max_height, height_offset=0.0, num_feet=2, stance_ratio=0.6,
+                            moving_threshold=0.05):  # commands.py:696-770; the value is (moving_flag, phase, heights...)
+    def heights(phase):
+        per_foot = (phase + np.linspace(0.0, 1.0, num_feet, endpoint=False)) % 1.0
+        progress = np.clip((per_foot - stance_ratio) / (1.0 - stance_ratio), 0.0, 1.0)
+        return np.where(per_foot >= stance_ratio, max_height * np.sin(np.pi * progress), 0.0) + height_offset
+
+    if fresh:
+        return np.concatenate([[1.0, 0.0], heights(0.0)])
+    flag, phase = prev[0], prev[1]
+    new_phase = (phase + ctrl_dt / gait_period) % 1.0 if flag else 0.0
+    moving = np.linalg.norm(qvel[:2]) > moving_threshold
+    flag = flag if moving else 0.0
+    new_phase = new_phase if moving else 0.0
+    return np.concatenate([[flag, new_phase], heights(new_phase)])
+
+
+def sinusoidal_gait_reward(position_tn3, height_tn, max_height):  # rewards.py:1331-1335
+    return 1.0 - np.abs(np.asarray(position_tn3, dtype=np.float64)[..., 2] - np.asarray(height_tn, dtype=np.float64)).sum(axis=-1) / max_height
+
+
 def position_velocity_actuator_torque(action, qpos, qvel, kp, kd, ctrl_clip, pos_noise=0.0, vel_noise=0.0, torque_noise=0.0):
     """PositionVelocityActuator.get_ctrl (ksim/actuators.py:261-293): action = (position targets, velocity targets)."""
     n = len(qpos)

@@ -745,6 +745,43 @@ def test_start_pose_and_base_height_commands():
         cs.update(cmd, t32(qpos[:, :5]), t32(qvel), all_fresh=True, seed=1, step=1)
 
 
+def test_sinusoidal_gait_command_and_reward():
+    from ksim_amd import rewards as rw
+    from ksim_amd.commands import CommandSet, ConstantCommand, SinusoidalGaitCommand
+    from ksim_amd.types import Trajectory
+
+    N, steps = 33, 14
+    rng = np.random.default_rng(47)
+    kw = dict(gait_period=0.37, ctrl_dt=0.02 * 3, max_height=0.15, height_offset=0.02, num_feet=3, stance_ratio=0.55, moving_threshold=0.3)
+    cs = CommandSet({"pad": ConstantCommand(size=1), "gait": SinusoidalGaitCommand(**kw)})
+    assert cs.command_dim == 6 and cs.slices["gait"] == slice(1, 6)
+    cmd = cs.initial(N, DEV)
+    want = np.zeros((N, 6))
+    rec_all, pos_all = [], []
+    for k in range(steps):
+        qpos = rng.normal(size=(N, 12)).astype(np.float32)
+        qvel = (rng.normal(size=(N, 11)) * 0.5).astype(np.float32)
+        fresh = np.ones(N, bool) if k == 0 else rng.random(N) < 0.1
+        rec = torch.empty(N, 6, device=DEV)
+        cs.update(cmd, t32(qpos), t32(qvel), fresh=torch.from_numpy(fresh.astype(np.uint8)).to(DEV), record=rec, seed=1, step=k)
+        np.testing.assert_allclose(rec.cpu().numpy(), want, rtol=1e-5, atol=1e-6)
+        for e in range(N):
+            want[e, 1:] = ot.sinusoidal_gait_command(want[e, 1:], qvel[e].astype(np.float64), bool(fresh[e]), **kw)
+        np.testing.assert_allclose(cmd.cpu().numpy(), want, rtol=1e-5, atol=2e-6)
+        rec_all.append(want.copy()); pos_all.append(rng.normal(size=(N, 9)) * 0.1)
+    assert (want[:, 1] == 0).any() and (want[:, 1] == 1).any() and (want[:, 3:] > 0.05).any()
+    commands, pos = np.stack(rec_all), np.stack(pos_all)
+    traj = Trajectory(qpos=None, qvel=None, xpos=None, xquat=None, ctrl=None, obs={"obs": t32(pos)}, command={"_buffer": t32(commands)},
+                      event_state={}, action=None, done=torch.zeros(steps, N, dtype=torch.bool, device=DEV), success=None, timestep=None)
+    st = rw.get_rewards(traj, {"gait": rw.SinusoidalGaitReward(scale=0.6, max_height=0.15, pos_obs="feet", pos_cmd="gait", num_feet=3)},
+                        obs_slices={"feet": slice(0, 9)}, command_slices=cs.slices)
+    f32 = lambda a: a.astype(np.float32).astype(np.float64)  # noqa: E731
+    want_r = 0.6 * ot.sinusoidal_gait_reward(f32(pos).reshape(steps, N, 3, 3), f32(commands)[..., 3:6], 0.15)
+    np.testing.assert_allclose(st.total.cpu().numpy(), want_r, rtol=2e-5, atol=2e-5)
+    with pytest.raises(ValueError, match="not found"):
+        rw.get_rewards(traj, {"gait": rw.SinusoidalGaitReward(pos_obs="feet", pos_cmd="nope")}, obs_slices={"feet": slice(0, 9)}, command_slices=cs.slices)
+
+
 def test_vector_commands():
     """FloatVectorCommand / IntVectorCommand: the properties the reference's own tests check (shape, bounds, a command
     that never switches stays what it was, reference tests/test_commands.py:64-96) and the draw arithmetic."""

@@ -522,3 +522,25 @@ def test_reachability_and_intersection_hand_computed():
     pts = np.array([[[0, 0, 0], [0.3, 0, 0], [0, 0.05, 0]], [[0, 0, 0], [0.3, 0, 0], [0, 0.5, 0]]], dtype=float)
     np.testing.assert_array_equal(ot.intersection_penalty(pts, 0.1), [1.0, 0.0])
     np.testing.assert_array_equal(ot.intersection_penalty(pts[:, :1], 0.1), [0.0, 0.0])   # a point is never too close to itself
+
+
+def test_sinusoidal_gait_command_and_reward_hand_computed():
+    kw = dict(gait_period=0.4, ctrl_dt=0.1, max_height=0.2, height_offset=0.01, num_feet=2, stance_ratio=0.5, moving_threshold=0.05)
+    v = np.array([0.3, 0.0, 0, 0, 0, 0])
+    c = ot.sinusoidal_gait_command(None, v, True, **kw)
+    # phase 0: foot 0 in stance, foot 1 at phase 0.5 = start of its swing (sin 0 = 0)
+    np.testing.assert_allclose(c, [1, 0, 0.01, 0.01], atol=1e-15)
+    c = ot.sinusoidal_gait_command(c, v, False, **kw)
+    # phase 0.25: foot 1 at 0.75 = the middle of its swing
+    np.testing.assert_allclose(c, [1, 0.25, 0.01, 0.21], atol=1e-15)
+    c = ot.sinusoidal_gait_command(c, v, False, **kw)
+    c = ot.sinusoidal_gait_command(c, v, False, **kw)
+    np.testing.assert_allclose(c, [1, 0.75, 0.21, 0.01], atol=1e-12)      # foot 0 mid-swing, foot 1 back in stance (phase 0.25)
+    c = ot.sinusoidal_gait_command(c, v, False, **kw)
+    np.testing.assert_allclose(c[:2], [1, 0.0], atol=1e-12)               # wrapped
+    c = ot.sinusoidal_gait_command(c, np.array([0.01, 0.02, 0, 0, 0, 0]), False, **kw)
+    np.testing.assert_allclose(c, [0, 0, 0.01, 0.01], atol=1e-15)         # standing still: flag and phase drop
+    c = ot.sinusoidal_gait_command(c, v, False, **kw)
+    np.testing.assert_allclose(c[:2], [0, 0], atol=1e-15)                 # and the flag stays down while the episode lasts
+    pos = np.array([[[0, 0, 0.05], [0, 0, 0.2]]])
+    np.testing.assert_allclose(ot.sinusoidal_gait_reward(pos, np.array([[0.01, 0.21]]), 0.2), [1 - (0.04 + 0.01) / 0.2], rtol=1e-12)
