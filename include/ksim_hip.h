@@ -61,6 +61,13 @@ int ks_gae_tn(ks_stream_t stream, int64_t T, int64_t N, const float* values, con
 #define KS_REDUCE_WORKSPACE_BYTES (2 * 1024 * 8 + 64)
 int ks_normalize_advantages(ks_stream_t stream, int64_t n, const float* gae, float* advantages,
                             void* workspace);
+/* The same result with no workspace argument and no allocation of any kind.  No counterpart in the reference: it is for
+ * callers that cannot allocate device memory (code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc).  The block partials live in a device array of KS_REDUCE_WORKSPACE_BYTES bytes inside the library, one copy
+ * per GPU, held until the process ends; n above KS_NORMALIZE_STATIC_MAX_N is rejected with KS_ELIMIT.  All calls on one
+ * GPU share that array: calls that overlap on one GPU (two streams, two threads) race; calls on one stream do not. */
+#define KS_NORMALIZE_STATIC_MAX_N ((int64_t)1 << 28)
+int ks_normalize_advantages_static(ks_stream_t stream, int64_t n, const float* gae, float* advantages);
 
 /* ------------------------------------------------------------------ PPO loss
  * Replaces compute_ppo_loss + clipped_value_loss (ppo.py:124-135,149-246) and the

@@ -52,6 +52,8 @@ def load() -> ctypes.CDLL:
     lib.ks_gae_bt.argtypes = [p, c_int64, c_int64, p, p, p, p, c_float, c_float, c_int32, p, p, p]
     lib.ks_gae_tn.argtypes = lib.ks_gae_bt.argtypes
     lib.ks_normalize_advantages.argtypes = [p, c_int64, p, p, p]
+    lib.ks_normalize_advantages_static.argtypes = [p, c_int64, p, p]
+    lib.ks_normalize_advantages_static.restype = c_int32
     lib.ks_ppo_loss.argtypes = [p, c_int64, c_int32, POINTER(KsPpoLossParams)] + [p] * 13
     lib.ks_reward_total.argtypes = [p, c_int64, c_int32, p, POINTER(c_float), c_int32, c_float, c_int32, c_float, p,
                                     c_int32, p, p, p]

@@ -2,6 +2,7 @@
 // reduction for gfx950.  Streaming, HBM-bound kernels: every array is read or
 // written exactly once per launch, with 64 consecutive elements per wavefront.
 #include "ks_common.h"
+#include <mutex>
 
 namespace ks {
 
@@ -381,6 +382,54 @@ extern "C" int ks_normalize_advantages(ks_stream_t stream, int64_t n, const floa
   hipLaunchKernelGGL(normalize_kernel, dim3(grid_for(n, 256, 4096)), dim3(256), 0, (hipStream_t)stream, n, g, gae,
                      partial, advantages);
   return check_launch("ks_normalize_advantages");
+}
+
+// ---------------------------------------------------------------------------------------------
+// ks_normalize_advantages without a workspace argument: the block partials live in a file-scope device array.
+// The array's name is only a host-side handle; its device address is looked up once per device with
+// hipGetSymbolAddress (each GPU holds its own copy) and that pointer is what the kernels receive.
+// ---------------------------------------------------------------------------------------------
+namespace ks {
+static __device__ __align__(256) unsigned char scratch[KS_REDUCE_WORKSPACE_BYTES];
+constexpr int kMaxDevices = 64;
+static void* g_scratch_ptr[kMaxDevices] = {};
+static std::mutex g_scratch_mutex;
+
+// Device address of `scratch` on the current device.
+static int scratch_on_current_device(const char* who, void** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return fail(KS_ELAUNCH, "%s: hipGetDevice: %s", who, hipGetErrorString(e));
+  if (dev < 0 || dev >= kMaxDevices)
+    return fail(KS_ELIMIT, "%s: device %d beyond the %d this library keeps scratch for", who, dev, kMaxDevices);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p) return fail(KS_ELAUNCH, "%s: hipGetSymbolAddress: %s", who, hipGetErrorString(e));
+    g_scratch_ptr[dev] = p;
+  }
+  *out = g_scratch_ptr[dev];
+  return KS_OK;
+}
+}  // namespace ks
+
+extern "C" int ks_normalize_advantages_static(ks_stream_t stream, int64_t n, const float* gae, float* advantages) {
+  if (n < 0) return fail(KS_EINVAL, "ks_normalize_advantages_static: negative size");
+  if (n > KS_NORMALIZE_STATIC_MAX_N)
+    return fail(KS_ELIMIT, "ks_normalize_advantages_static: n = %lld beyond the maximum of %lld elements", (long long)n,
+                (long long)KS_NORMALIZE_STATIC_MAX_N);
+  if (n == 0) return KS_OK;
+  if (!gae || !advantages) return fail(KS_EINVAL, "ks_normalize_advantages_static: null pointer");
+  void* ptr = nullptr;
+  if (int rc = scratch_on_current_device("ks_normalize_advantages_static", &ptr)) return rc;
+  double* partial = (double*)ptr;
+  // every partial that stage 2 reads is written by stage 1 of the same call, so nothing has to be cleared
+  const int g = grid_for(n, 256 * 4, kMaxPartials);
+  hipLaunchKernelGGL(moments_kernel, dim3(g), dim3(256), 0, (hipStream_t)stream, n, gae, partial);
+  hipLaunchKernelGGL(normalize_kernel, dim3(grid_for(n, 256, 4096)), dim3(256), 0, (hipStream_t)stream, n, g, gae,
+                     partial, advantages);
+  return check_launch("ks_normalize_advantages_static");
 }
 
 extern "C" int ks_ppo_loss(ks_stream_t stream, int64_t n, int32_t A, const KsPpoLossParams* params,
