@@ -21,15 +21,18 @@ BF16_PEAK_TFLOPS = 2500.0  # dense MFMA bf16
 FP32_VALU_PEAK_TFLOPS = 157.3
 
 
-def cpu_baseline(target_seconds: float = 12.0):
-    """The oracle's C restatement of the control step (float32, OpenMP over envs) on this host's cores."""
+def cpu_baseline(integrator: str, target_seconds: float = 12.0):
+    """The oracle's C restatement of the control step (float32, OpenMP over envs) on this host's cores, on the same
+    model (same integrator) as the GPU leg."""
     import numpy as np
 
     from ksim_amd import model as km
     from ksim_amd.configs import KBOT_TORQUE_LIMITS
     from oracle.dyn import Oracle
 
-    m = km.kbot_scale_model(seed=1004, integrator="implicitfast")  # the integrator ksim selects (ksim/task/rl.py:555-578)
+    from ksim_amd.configs import integrator_name
+
+    m = km.kbot_scale_model(seed=1004, integrator=integrator)
     orc = Oracle(m.arrays(), np.float32)
     cores = min(16, os.cpu_count() or 1)
     N = 2048
@@ -61,8 +64,8 @@ def cpu_baseline(target_seconds: float = 12.0):
     k = max(2, int(target_seconds / max(t1 / 2, 1e-3)))
     t = run(k)
     return {"value": N * k / t, "unit": "env-steps/s", "cores": cores, "kind": "port",
-            "sample": f"physics control step only (PD + 4 substeps), {N} envs x {k} steps, float32 C restatement "
-                      f"of the MJX path (not MJX), OpenMP over envs"}
+            "sample": f"physics control step only (PD + 4 substeps, {integrator_name(m)}), {N} envs x {k} steps, "
+                      f"float32 C restatement of the MJX path (not MJX), OpenMP over envs"}
 
 
 def main() -> None:
@@ -72,6 +75,9 @@ def main() -> None:
     ap.add_argument("--warmup", type=int, default=40)
     ap.add_argument("--envs", type=int, default=8192)
     ap.add_argument("--rollout", type=int, default=32)
+    ap.add_argument("--integrator", choices=("euler", "implicitfast"), default="euler",
+                    help="velocity update of the headline rollout: semi-implicit Euler (what the benchmark configs name) or "
+                         "implicitfast (what ksim's RLConfig selects); the other one is reported under 'other_integrator'")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="also launch ks_copy_f32 on 64 Mi floats once: the known-size kernel for counter calibration")
@@ -83,47 +89,21 @@ def main() -> None:
     import torch
 
     from ksim_amd import _lib, ppo
-    from ksim_amd.configs import kbot_rollout, step_algorithmic_bytes
-    from ksim_amd.rewards import get_rewards
+    from ksim_amd.configs import integrator_name, step_algorithmic_bytes
 
     _lib.load()
     assert torch.cuda.is_available(), "bench.py needs a GPU"
-    N, T = args.envs, args.rollout
-    consts, env, ro, _ = kbot_rollout(num_envs=N, rollout_length=T)
+    N = args.envs
+    T = max(1, min(args.rollout, args.steps))  # the timed region holds whole rollouts, so rewards and GAE are inside it
+    head = timed_rollout(torch, args.integrator, N, T, args.steps, args.warmup)
+    consts, env, ro, elapsed, kernel_ms, ndone = (head[k] for k in ("consts", "env", "ro", "elapsed", "kernel_ms", "ndone"))
     m = consts.physics_model.model
-
-    # time the dominant kernel (the fused physics control step) with events on the launch stream
-    step_events: list = []
-    orig_step = consts.engine.step
-
-    def timed_step(*a, **kw):
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        out = orig_step(*a, **kw)
-        e1.record()
-        step_events.append((e0, e1))
-        return out
-
-    def one_step(k: int) -> None:
-        t = k % T
-        ro.step_engine(env, t)
-        if t == T - 1:
-            rew = get_rewards(ro.trajectory(), consts.rewards, want_components=False)
-            ro.ppo_inputs(rew, 0.99, 0.95, normalize_advantages=True)
-
-    for k in range(args.warmup):
-        one_step(k)
-    consts.engine.step = timed_step
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for k in range(args.warmup, args.warmup + args.steps):
-        one_step(k)
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-    consts.engine.step = orig_step
-    kernel_ms = sum(a.elapsed_time(b) for a, b in step_events) / len(step_events)
-    ndone = int(ro.done.sum().item())
-    assert torch.isfinite(env.physics_state.data.qpos).all(), "non-finite state after the benchmark"
+    other = "implicitfast" if args.integrator == "euler" else "euler"
+    alt = timed_rollout(torch, other, N, T, max(T, min(args.steps, 2 * T)), min(args.warmup, T))
+    other_entry = {"integrator": integrator_name(alt["consts"].physics_model.model),
+                   "value": N * alt["steps"] / alt["elapsed"], "unit": "env-steps/s", "steps": alt["steps"],
+                   "ms_per_step": alt["elapsed"] / alt["steps"] * 1e3, "step_kernel_ms": alt["kernel_ms"]}
+    del alt
 
     # The same rollout captured once as a HIP graph and replayed: the launches leave the host out of the loop.
     # Reported beside the headline (whose timed region keeps per-launch events for the roofline figure).
@@ -177,21 +157,67 @@ def main() -> None:
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": "cfg4: K-Bot-scale biped (free root + 20 hinges, 8 foot spheres), per-env friction/mass "
                                "randomisation, obs noise 0.01, reset on z<0.5, actor+critic 3x512 bf16 MLP, "
-                               "dt=0.005 x 4 substeps, Newton 8/8, implicitfast (damping-implicit) integration", "num_envs": N, "rollout_length": T, "substeps": 4,
+                               f"dt=0.005 x 4 substeps, Newton 8/8, {integrator_name(m)} integration; rewards + GAE after "
+                               f"every {T} control steps inside the timed region",
+                   "integrator": integrator_name(m), "num_envs": N, "rollout_length": T, "substeps": 4,
                    "obs_dim": obs_dim, "episodes_finished_in_last_rollout": ndone},
         "roofline": {"bound": "hbm", "kernel": "step_kernel (fused control step)", "achieved": achieved,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
                      "algorithmic_bytes_per_env_step": bytes_per_env, "kernel_ms": kernel_ms,
                      "valu_issue_fraction_profiled": valu.get("valu_issue_fraction"),
                      "valu_insts_per_env_step_profiled": valu.get("valu_insts_per_env_step"),
+                     "counters_source": "traffic and valu_* are read from the committed rocprofv3 --pmc summaries under "
+                                        "profiles/ (separate counter runs of this command), not re-measured in this run",
                      "note": "the fused step is bound by fp32 vector-ALU issue (~1e3 flop/byte; the profiled share of "
                              "cycles with a VALU instruction issuing is given beside); the HBM fraction is reported "
                              "against the bytes the engine contract obliges a step to move"},
+        "other_integrator": other_entry,
         "gae": gae, "policy_mlp": mlp, "ppo_update": upd, "graph_replay": graph,
     }
     if not args.no_cpu_baseline:
-        line["cpu_baseline"] = cpu_baseline()
+        line["cpu_baseline"] = cpu_baseline(args.integrator)
     print(json.dumps(line))
+
+
+def timed_rollout(torch, integrator: str, N: int, T: int, steps: int, warmup: int) -> dict:
+    """`warmup` untimed control steps, then exactly `steps` timed ones of the cfg 4 rollout built with `integrator`.
+    The rollout slot restarts at 0 where the timed region begins, so it holds steps // T reward + GAE passes."""
+    from ksim_amd.configs import kbot_rollout
+    from ksim_amd.rewards import get_rewards
+
+    consts, env, ro, _ = kbot_rollout(num_envs=N, rollout_length=T, integrator=integrator)
+    # time the dominant kernel (the fused physics control step) with events on the launch stream
+    step_events: list = []
+    orig_step = consts.engine.step
+
+    def timed_step(*a, **kw):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        out = orig_step(*a, **kw)
+        e1.record()
+        step_events.append((e0, e1))
+        return out
+
+    def one_step(t: int) -> None:
+        ro.step_engine(env, t)
+        if t == T - 1:
+            rew = get_rewards(ro.trajectory(), consts.rewards, want_components=False)
+            ro.ppo_inputs(rew, 0.99, 0.95, normalize_advantages=True)
+
+    for k in range(warmup):
+        one_step(k % T)
+    consts.engine.step = timed_step
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for k in range(steps):
+        one_step(k % T)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    consts.engine.step = orig_step
+    kernel_ms = sum(a.elapsed_time(b) for a, b in step_events) / len(step_events)
+    ndone = int(ro.done.sum().item())
+    assert torch.isfinite(env.physics_state.data.qpos).all(), "non-finite state after the benchmark"
+    return dict(consts=consts, env=env, ro=ro, elapsed=elapsed, kernel_ms=kernel_ms, ndone=ndone, steps=steps)
 
 
 def gae_bandwidth(torch, ppo, reps=8):

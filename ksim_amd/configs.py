@@ -21,12 +21,18 @@ def _net(dims, rng, last_scale=1.0, dtype="bf16"):
     return MLP(ws, bs, activation="elu", dtype=dtype)
 
 
+def integrator_name(model) -> str:
+    """What a workload description must say about the velocity update of `model` (read off the model's own flag)."""
+    return "implicitfast (damping-implicit)" if model.eulerdamp else "semi-implicit Euler"
+
+
 def kbot_rollout(num_envs: int = 8192, rollout_length: int = 32, seed: int = 1004, hidden: int = 512,
-                 dtype: str = "bf16", min_height: float = 0.5):
+                 dtype: str = "bf16", min_height: float = 0.5, integrator: str = "euler"):
     """K-Bot-scale biped rollout: free root + 20 hinges, 8 foot spheres, per-env friction ~U(0.4,1.2) and
     mass scale ~U(0.9,1.1), observation noise N(0,0.01), reset on base height < `min_height`, actor and critic
-    3 x `hidden` MLPs, dt 0.005 with 4 physics substeps per control step."""
-    m = km.kbot_scale_model(seed=seed)
+    3 x `hidden` MLPs, dt 0.005 with 4 physics substeps per control step.  `integrator`: "euler" (semi-implicit
+    Euler, what the benchmark configs name) or "implicitfast" (what ksim's RLConfig selects, ksim/task/rl.py:555-578)."""
+    m = km.kbot_scale_model(seed=seed, integrator=integrator)
     rng = np.random.default_rng(seed)
     kps = rng.uniform(20.0, 150.0, m.nu)
     kds = rng.uniform(0.5, 1.5, m.nu)

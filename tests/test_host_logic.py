@@ -1,5 +1,6 @@
 """Host-side logic that needs no GPU: config validation, table compilation, struct layouts, model builder."""
 import ctypes
+import os
 
 import numpy as np
 import pytest
@@ -356,3 +357,24 @@ def test_reward_constructors_from_a_model():
     assert (tr.tracked_body_idx, tr.base_body_idx, tr.norm) == (9, 1, "l1")
     with pytest.raises(ValueError, match="must match"):
         rw.JointDeviationPenalty(joint_indices=(0, 1), joint_targets=(0.0,)).descs()
+
+
+def test_benchmark_workload_label_follows_the_model_flag():
+    """The bench line's integrator text is derived from the model it actually builds, for both legs."""
+    import re
+
+    from ksim_amd import model as km
+    from ksim_amd.configs import integrator_name
+
+    euler = km.kbot_scale_model(seed=1004, integrator="euler")
+    fast = km.kbot_scale_model(seed=1004, integrator="implicitfast")
+    assert not euler.eulerdamp and not euler.arrays()["eulerdamp"]
+    assert fast.eulerdamp and fast.arrays()["eulerdamp"]
+    assert integrator_name(euler) == "semi-implicit Euler"
+    assert integrator_name(fast).startswith("implicitfast")
+    src = open(os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "bench.py")).read()
+    # no hard-coded integrator in the workload text, and both legs take the same argument
+    assert "integrator_name(m)" in src and not re.search(r'"[^"\n]*implicitfast \(damping', src)
+    assert "cpu_baseline(args.integrator)" in src and "timed_rollout(torch, args.integrator" in src
+    src_cfg = open(os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "ksim_amd", "configs.py")).read()
+    assert "kbot_scale_model(seed=seed, integrator=integrator)" in src_cfg
