@@ -34,7 +34,7 @@ const char* ks_last_error(void);
  * 0 KsPpoLossParams, 1 KsModelDesc, 2 KsStepIO, 3 KsTermsDesc, 4 KsObserveIO, 5 KsTerminateIO, 6 KsMlpDesc,
  * 7 KsRewardIO, 8 KsObsElem, 9 KsTermDesc, 10 KsRewardDesc, 11 KsRng, 12 KsAdamParams, 13 KsEventDesc,
  * 14 KsRewardScanIO, 15 KsRewardScanDesc, 16 KsGruDesc, 17 KsLstmDesc, 18 KsGaussianHead, 19 KsCommandIO,
- * 20 KsMixtureHead;
+ * 20 KsMixtureHead, 21 KsNoiseStage, 22 KsRandomVar;
  * -1 for anything else. */
 int64_t ks_abi_sizeof(int32_t which);
 
@@ -350,13 +350,29 @@ enum { /* KsObsElem.kind */
                            (q_body q_site)^-1 (qacc[0:3] + alpha x r + w x (w x r) - g), alpha = R_body qacc[3:6],
                            r = R_body (c0, c1, c2), g = (q0, q1, q2), q_site = (e0, e1, e2, e3) */
 };
+/* Noise and bias of an observation (ksim/noise.py:129-229, applied by Observation.add_noise, ksim/observation.py:110-142:
+ * first the noise, then the per-episode bias).  A stage draws rv = mean + level (scale z + scale2 w) with z ~ N(0,1),
+ * w ~ U(-1,1) (Gaussian kinds: scale = std; uniform kinds: scale2 = mag; the uniform-Gaussian kinds of
+ * UniformGaussianRandomVariable, noise.py:106-121, use both) and adds it to the observation or multiplies the observation
+ * by it.  ChainedNoise (noise.py:222-229) applies several stages with ONE key: all stages of an element see the same z and w.
+ * One key also ties w to z inside a stage: jax.random builds a normal draw as sqrt(2) erfinv of the uniform the same bits
+ * give, so w = erf(z / sqrt 2).  The in-kernel Philox stream draws z and derives w that way; explicit noise_normal /
+ * noise_uniform buffers are taken as they are (a caller comparing with the reference passes a consistent pair). */
 enum { KS_NOISE_NONE = 0, KS_NOISE_ADD_GAUSSIAN = 1, KS_NOISE_ADD_UNIFORM = 2, KS_NOISE_MUL_GAUSSIAN = 3,
-       KS_NOISE_MUL_UNIFORM = 4 }; /* ksim/noise.py:184-213 */
+       KS_NOISE_MUL_UNIFORM = 4, KS_NOISE_ADD_UNIFORM_GAUSSIAN = 5, KS_NOISE_MUL_UNIFORM_GAUSSIAN = 6 };
+#define KS_MAX_NOISE_CHAIN 4
+typedef struct KsNoiseStage {
+  int32_t kind;
+  float mean, scale, scale2; /* scale: std (Gaussian kinds) or mag (uniform kinds); scale2: mag of the uniform-Gaussian kinds */
+} KsNoiseStage;
 typedef struct KsObsElem {
   int32_t kind, src, index, comp;
   float c0, c1, c2;
-  int32_t noise_kind;
-  float noise_mean, noise_scale; /* std or mag, multiplied by the curriculum level (noise.py:86,102) */
+  int32_t n_noise;               /* stages in use, 0 = no noise */
+  KsNoiseStage noise[KS_MAX_NOISE_CHAIN];
+  KsNoiseStage bias;             /* per-episode bias (KS_NOISE_NONE: none): the same kinds, evaluated every step from the env's
+                                    stored standard draw (KsObserveIO.bias_draw) at the current curriculum level, which is what
+                                    re-drawing with the episode's key gives (observation.py:136-141, ksim/task/rl.py:263-271) */
   int32_t carry, stride;         /* stateful kinds: offset into the env's carry row, distance between delay slots */
   float q0, q1, q2;              /* KS_OBS_GRAVITY_EMA: min_lag, max_lag, imu_bias; KS_OBS_SITE_ACCEL: gravity */
   float e0, e1, e2, e3;          /* site kinds: the site's orientation in its body, wxyz */
@@ -401,7 +417,10 @@ typedef struct KsObserveIO {
   float level;               /* curriculum level */
   const float* src[KS_SRC_COUNT]; /* indexed by KS_SRC_*; an unused source may be NULL */
   const float* zero_offset;  /* (N, nu) nullable */
-  const float* bias;         /* (N, obs_dim) additive per-episode bias value, nullable */
+  float* bias_draw;          /* (N, obs_dim, 2) in/out: the episode's standard draws (z, w) behind each element's bias; required
+                                when an element has a bias.  Envs flagged in `fresh` get new ones first (the reference re-keys
+                                the biases of an env that was reset, ksim/task/rl.py:1110-1117) */
+  const float* bias_redraw;  /* (N, obs_dim, 2) the (z, w) that fresh envs take, nullable -> Philox */
   const float* noise_normal; /* (N, obs_dim) standard normal draws, nullable -> Philox */
   const float* noise_uniform;/* (N, obs_dim) U[0,1) draws, nullable -> Philox */
   KsRng rng;
@@ -410,10 +429,19 @@ typedef struct KsObserveIO {
   /* stateful observations (rl.py:166-176: observe_stateful with the carry of the previous control step) */
   float* carry;               /* (N, carry_dim) in/out; required when carry_dim > 0 */
   const uint8_t* fresh;       /* (N) nullable: non-zero = the env starts an episode, its carries are initialised from the
-                                 current state before observing (initial_carry, rl.py:1034-1080); NULL = none */
+                                 current state before observing (initial_carry, rl.py:1034-1080) and its bias draws are
+                                 renewed; NULL = none */
   const float* carry_uniform; /* (N, carry_dim) U[0,1) draws for the initial carries, nullable -> Philox */
 } KsObserveIO;
 int ks_observe(const KsTerms* terms, ks_stream_t stream, const KsObserveIO* io /*host*/);
+
+/* A random variable of ksim/noise.py:50-121 as parameters: value = mean + s (std z + mag w), z ~ N(0,1), w ~ U(-1,1),
+ * s = the curriculum level where the reference passes one, else 1.  same_key: both parts come from one key
+ * (UniformGaussianRandomVariable, noise.py:106-121), so w = erf(z / sqrt 2) as described at KsNoiseStage. */
+typedef struct KsRandomVar {
+  float mean, mag, std;
+  int32_t same_key;
+} KsRandomVar;
 
 /* Terminations, trajectory record and reset predication for the post-step state
  * (replaces RLTask._get_step_env_state, rl.py:1023-1136, for the physics part):
@@ -438,6 +466,23 @@ typedef struct KsTerminateIO {
   const float* event_reset_uniform; /* (N, n_events) U[0,1) draws, nullable -> Philox */
   float* event_force;               /* (n_events, N, KS_EVENT_FORCE_STATE), nullable: zeroed for the reset envs */
   const float* contact_dist;        /* (N, ns) KsStepIO.contact_dist of the step just taken; KS_TERM_ILLEGAL_CONTACT only */
+  /* Per-episode quantities of the envs that start a fresh episode, re-drawn like MjxEngine.reset does under cond(done)
+   * (ksim/engine.py:222-245, ksim/task/rl.py:1072-1080).  Every buffer is nullable = left alone. */
+  float* action_latency;            /* (N) <- U(latency_lo level, latency_hi level), in physics steps (engine.py:233-237) */
+  float latency_lo, latency_hi;
+  float* zero_offset;               /* (N, nu) <- zero_offset_rv at the curriculum level (engine.py:238-242) */
+  KsRandomVar zero_offset_rv;
+  /* ActuatorState of PositionActuators.get_initial_state (ksim/actuators.py:219-238), drawn at level 1 */
+  float* act_action_bias;           /* (N, nu) */
+  float* act_torque_bias;           /* (N, nu) */
+  float* act_kp_scale;              /* (N) */
+  float* act_kd_scale;              /* (N) */
+  float* act_torque_limit_scale;    /* (N) */
+  KsRandomVar action_bias_rv, torque_bias_rv, kp_scale_rv, kd_scale_rv, torque_limit_scale_rv;
+  /* explicit draws, (N, 3 nu + 4) each, nullable -> Philox; columns: latency, zero offset (nu), action bias (nu),
+   * torque bias (nu), kp scale, kd scale, torque limit scale */
+  const float* episode_uniform;     /* U(-1,1); the latency takes lo + (u + 1) / 2 (hi - lo) */
+  const float* episode_normal;      /* N(0,1) */
 } KsTerminateIO;
 int ks_terminate_reset(const KsTerms* terms, ks_stream_t stream, const KsTerminateIO* io /*host*/);
 

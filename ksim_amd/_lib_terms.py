@@ -8,17 +8,27 @@ KS_MAX_OBS, KS_MAX_TERMS, KS_MAX_QPOS, KS_MAX_LAYERS = 512, 16, 40, 8
 (SRC_QPOS, SRC_QVEL, SRC_QACC, SRC_CTRL, SRC_LAST_ACTION, SRC_COMMAND, SRC_TIME, SRC_XPOS, SRC_XQUAT, SRC_CVEL,
  SRC_CONST, SRC_CONTACT_DIST, SRC_CINERT, SRC_CFRC_EXT, SRC_COUNT) = range(15)
 OBS_COPY, OBS_JOINT_POS, OBS_ROT_INV, OBS_CONTACT, OBS_DELAYED, OBS_GRAVITY_EMA, OBS_SITE_GYRO, OBS_SITE_ACCEL = range(8)
-NOISE_NONE, NOISE_ADD_GAUSSIAN, NOISE_ADD_UNIFORM, NOISE_MUL_GAUSSIAN, NOISE_MUL_UNIFORM = range(5)
+(NOISE_NONE, NOISE_ADD_GAUSSIAN, NOISE_ADD_UNIFORM, NOISE_MUL_GAUSSIAN, NOISE_MUL_UNIFORM, NOISE_ADD_UNIFORM_GAUSSIAN,
+ NOISE_MUL_UNIFORM_GAUSSIAN) = range(7)
+KS_MAX_NOISE_CHAIN = 4
 (TERM_MIN_HEIGHT, TERM_BAD_Z, TERM_NOT_UPRIGHT, TERM_BAD_VELOCITY, TERM_FAR_FROM_ORIGIN,
  TERM_EPISODE_LENGTH, TERM_ILLEGAL_CONTACT) = range(7)
 ACT_NONE, ACT_ELU, ACT_RELU, ACT_TANH, ACT_GELU = range(5)
 MLP_F32, MLP_BF16 = 0, 1
 
 
+class KsNoiseStage(ctypes.Structure):
+    _fields_ = [("kind", c_int32), ("mean", c_float), ("scale", c_float), ("scale2", c_float)]
+
+
+class KsRandomVar(ctypes.Structure):
+    _fields_ = [("mean", c_float), ("mag", c_float), ("std", c_float), ("same_key", c_int32)]
+
+
 class KsObsElem(ctypes.Structure):
     _fields_ = [("kind", c_int32), ("src", c_int32), ("index", c_int32), ("comp", c_int32), ("c0", c_float),
-                ("c1", c_float), ("c2", c_float), ("noise_kind", c_int32), ("noise_mean", c_float),
-                ("noise_scale", c_float), ("carry", c_int32), ("stride", c_int32), ("q0", c_float), ("q1", c_float),
+                ("c1", c_float), ("c2", c_float), ("n_noise", c_int32), ("noise", KsNoiseStage * KS_MAX_NOISE_CHAIN),
+                ("bias", KsNoiseStage), ("carry", c_int32), ("stride", c_int32), ("q0", c_float), ("q1", c_float),
                 ("q2", c_float), ("e0", c_float), ("e1", c_float), ("e2", c_float), ("e3", c_float)]
 
 
@@ -54,7 +64,8 @@ class KsEventDesc(ctypes.Structure):
 
 class KsObserveIO(ctypes.Structure):
     _fields_ = [("N", c_int64), ("level", c_float), ("src", c_void_p * SRC_COUNT), ("zero_offset", c_void_p),
-                ("bias", c_void_p), ("noise_normal", c_void_p), ("noise_uniform", c_void_p), ("rng", KsRng),
+                ("bias_draw", c_void_p), ("bias_redraw", c_void_p), ("noise_normal", c_void_p), ("noise_uniform", c_void_p),
+                ("rng", KsRng),
                 ("obs", c_void_p), ("noisy_obs", c_void_p), ("carry", c_void_p), ("fresh", c_void_p),
                 ("carry_uniform", c_void_p)]
 
@@ -66,7 +77,13 @@ class KsTerminateIO(ctypes.Structure):
                 ("traj_time", c_void_p), ("reset_mask", c_void_p), ("episode_length", c_void_p),
                 ("reset_uniform", c_void_p), ("rng", KsRng), ("apply_reset", c_int32), ("n_events", c_int32),
                 ("event_interval", (c_float * 2) * KS_MAX_EVENTS), ("event_state", c_void_p),
-                ("event_reset_uniform", c_void_p), ("event_force", c_void_p), ("contact_dist", c_void_p)]
+                ("event_reset_uniform", c_void_p), ("event_force", c_void_p), ("contact_dist", c_void_p),
+                ("action_latency", c_void_p), ("latency_lo", c_float), ("latency_hi", c_float), ("zero_offset", c_void_p),
+                ("zero_offset_rv", KsRandomVar), ("act_action_bias", c_void_p), ("act_torque_bias", c_void_p),
+                ("act_kp_scale", c_void_p), ("act_kd_scale", c_void_p), ("act_torque_limit_scale", c_void_p),
+                ("action_bias_rv", KsRandomVar), ("torque_bias_rv", KsRandomVar), ("kp_scale_rv", KsRandomVar),
+                ("kd_scale_rv", KsRandomVar), ("torque_limit_scale_rv", KsRandomVar), ("episode_uniform", c_void_p),
+                ("episode_normal", c_void_p)]
 
 
 class KsMlpDesc(ctypes.Structure):

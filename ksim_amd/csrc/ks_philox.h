@@ -34,7 +34,7 @@ __device__ inline float normal_from(uint32_t a, uint32_t b) {
   return sqrtf(-2.0f * logf(u1)) * cosf(6.28318530717958647692f * u2);
 }
 
-enum { kRngObsNoise = 1, kRngReset = 2, kRngAction = 3, kRngEvent = 4, kRngObsCarry = 5, kRngCommand = 6 };
+enum { kRngObsNoise = 1, kRngReset = 2, kRngAction = 3, kRngEvent = 4, kRngObsCarry = 5, kRngCommand = 6, kRngObsBias = 7, kRngEpisode = 8 };
 
 // draw for (env, element) of a purpose at a step: counter = (env lo, env hi ^ purpose<<24, step lo, element)
 __device__ inline Philox4 draw(uint64_t seed, uint64_t step, int purpose, uint64_t env, uint32_t element) {

@@ -335,6 +335,8 @@ extern "C" int64_t ks_abi_sizeof(int32_t which) {
     case 18: return sizeof(KsGaussianHead);
     case 19: return sizeof(KsCommandIO);
     case 20: return sizeof(KsMixtureHead);
+    case 21: return sizeof(KsNoiseStage);
+    case 22: return sizeof(KsRandomVar);
     default: return -1;
   }
 }

@@ -30,7 +30,8 @@ struct ObserveArgs {
   float level;
   const float* src[KS_SRC_COUNT];
   int src_dim[KS_SRC_COUNT];
-  const float *zero_offset, *bias, *noise_normal, *noise_uniform;
+  const float *zero_offset, *bias_redraw, *noise_normal, *noise_uniform;
+  float* bias_draw;
   KsRng rng;
   float *obs, *noisy;
   int obs_dim, nq, nu;
@@ -47,6 +48,19 @@ __device__ inline void rot_fwd(const float* q4, const float* v, float* out) {
   out[0] = v[0] + w * tx + (y * tz - z * ty);
   out[1] = v[1] + w * ty + (z * tx - x * tz);
   out[2] = v[2] + w * tz + (x * ty - y * tx);
+}
+
+// one noise or bias stage on the value v with the standard draws z ~ N(0,1), w ~ U(-1,1) (ksim/noise.py:74-121,184-213)
+__device__ inline float apply_stage(const KsNoiseStage& st, float v, float z, float w, float level) {
+  float rv = st.mean;
+  switch (st.kind) {
+    case KS_NOISE_ADD_GAUSSIAN: case KS_NOISE_MUL_GAUSSIAN: rv += z * (st.scale * level); break;
+    case KS_NOISE_ADD_UNIFORM: case KS_NOISE_MUL_UNIFORM: rv += w * (st.scale * level); break;
+    case KS_NOISE_ADD_UNIFORM_GAUSSIAN: case KS_NOISE_MUL_UNIFORM_GAUSSIAN: rv += z * (st.scale * level) + w * (st.scale2 * level); break;
+    default: return v;
+  }
+  const bool add = st.kind == KS_NOISE_ADD_GAUSSIAN || st.kind == KS_NOISE_ADD_UNIFORM || st.kind == KS_NOISE_ADD_UNIFORM_GAUSSIAN;
+  return add ? v + rv : v * rv;
 }
 
 __global__ __launch_bounds__(256) void observe_kernel(ObserveArgs a) {
@@ -129,24 +143,35 @@ __global__ __launch_bounds__(256) void observe_kernel(ObserveArgs a) {
     v = out[el.comp];
   }
   if (a.obs) a.obs[idx] = v;
+  const uint64_t step = a.rng.step + (a.rng.step_base ? *a.rng.step_base : 0ull);
+  if (el.bias.kind != KS_NOISE_NONE && a.fresh && a.fresh[e]) {  // a new episode: new bias draws (rl.py:1110-1117)
+    float z, w;
+    if (a.bias_redraw) {
+      z = a.bias_redraw[2 * idx];
+      w = a.bias_redraw[2 * idx + 1];
+    } else {
+      const Philox4 r = draw(a.rng.seed, step, kRngObsBias, (uint64_t)e, (uint32_t)k);
+      z = normal_from(r.x, r.y);
+      w = erff(z * 0.70710678118654752440f);
+    }
+    a.bias_draw[2 * idx] = z;
+    a.bias_draw[2 * idx + 1] = w;
+  }
   if (a.noisy) {
     float nv = v;
-    if (el.noise_kind != KS_NOISE_NONE) {
-      float n01, u01v;
+    if (el.n_noise > 0) {
+      float z, w;
       if (a.noise_normal && a.noise_uniform) {
-        n01 = a.noise_normal[idx];
-        u01v = a.noise_uniform[idx];
+        z = a.noise_normal[idx];
+        w = 2.f * a.noise_uniform[idx] - 1.f;
       } else {
-        const Philox4 r = draw(a.rng.seed, a.rng.step + (a.rng.step_base ? *a.rng.step_base : 0ull), kRngObsNoise, (uint64_t)e, (uint32_t)k);
-        n01 = normal_from(r.x, r.y);
-        u01v = u01(r.z);
+        const Philox4 r = draw(a.rng.seed, step, kRngObsNoise, (uint64_t)e, (uint32_t)k);
+        z = normal_from(r.x, r.y);
+        w = erff(z * 0.70710678118654752440f);  // the uniform that the same random bits give
       }
-      const float sc = el.noise_scale * a.level;
-      const bool gauss = el.noise_kind == KS_NOISE_ADD_GAUSSIAN || el.noise_kind == KS_NOISE_MUL_GAUSSIAN;
-      const float rv = gauss ? n01 * sc + el.noise_mean : (el.noise_mean - sc) + 2.f * sc * u01v;
-      nv = (el.noise_kind == KS_NOISE_ADD_GAUSSIAN || el.noise_kind == KS_NOISE_ADD_UNIFORM) ? v + rv : v * rv;
+      for (int j = 0; j < el.n_noise; ++j) nv = apply_stage(el.noise[j], nv, z, w, a.level);
     }
-    if (a.bias) nv += a.bias[idx];
+    if (el.bias.kind != KS_NOISE_NONE) nv = apply_stage(el.bias, nv, a.bias_draw[2 * idx], a.bias_draw[2 * idx + 1], a.level);
     a.noisy[idx] = nv;
   }
 }
@@ -171,7 +196,18 @@ struct TerminateArgs {
   float* event_force;
   const float* contact_dist;
   int ns, na;
+  float *action_latency, *zero_offset, *act_action_bias, *act_torque_bias, *act_kp_scale, *act_kd_scale, *act_torque_limit_scale;
+  float latency_lo, latency_hi;
+  KsRandomVar zero_offset_rv, action_bias_rv, torque_bias_rv, kp_scale_rv, kd_scale_rv, torque_limit_scale_rv;
+  const float *episode_uniform, *episode_normal;
+  int redraw;  // any of the per-episode buffers is given
 };
+
+// value of a random variable from its standard draws (ksim/noise.py:74-121)
+__device__ inline float rv_value(const KsRandomVar& rv, float u, float z, float s) {
+  const float w = rv.same_key ? erff(z * 0.70710678118654752440f) : u;
+  return rv.mean + s * (rv.std * z + rv.mag * w);
+}
 
 // A 256-thread workgroup owns kTermEnvs consecutive envs.  The state rows of those envs are contiguous in memory,
 // so the transition copies, the finiteness check and the reset writes all walk them as flat, coalesced
@@ -282,6 +318,39 @@ __global__ __launch_bounds__(256) void terminate_kernel(TerminateArgs a) {
   if (a.last_ctrl)
     for (int idx = tid; idx < ne * a.na; idx += 256)
       if (s_reset[idx / a.na]) a.last_ctrl[e0 * a.na + idx] = 0.f;
+  // ---- per-episode quantities of the fresh episodes (engine.py:222-245, actuators.py:219-238)
+  if (a.redraw) {
+    const int ned = 3 * nu + 4;
+    for (int idx = tid; idx < ne * ned; idx += 256) {
+      const int le = idx / ned, j = idx - le * ned;
+      if (!s_reset[le]) continue;
+      const int64_t e = e0 + le;
+      float u, z;
+      if (a.episode_uniform && a.episode_normal) {
+        u = a.episode_uniform[e * ned + j];
+        z = a.episode_normal[e * ned + j];
+      } else {
+        const Philox4 r = draw(a.rng.seed, step, kRngEpisode, (uint64_t)e, (uint32_t)j);
+        u = a.episode_uniform ? a.episode_uniform[e * ned + j] : 2.f * u01(r.x) - 1.f;
+        z = a.episode_normal ? a.episode_normal[e * ned + j] : normal_from(r.y, r.z);
+      }
+      if (j == 0) {
+        if (a.action_latency) a.action_latency[e] = a.latency_lo * a.level + 0.5f * (u + 1.f) * ((a.latency_hi - a.latency_lo) * a.level);
+      } else if (j <= nu) {
+        if (a.zero_offset) a.zero_offset[e * nu + (j - 1)] = rv_value(a.zero_offset_rv, u, z, a.level);
+      } else if (j <= 2 * nu) {
+        if (a.act_action_bias) a.act_action_bias[e * nu + (j - 1 - nu)] = rv_value(a.action_bias_rv, u, z, 1.f);
+      } else if (j <= 3 * nu) {
+        if (a.act_torque_bias) a.act_torque_bias[e * nu + (j - 1 - 2 * nu)] = rv_value(a.torque_bias_rv, u, z, 1.f);
+      } else if (j == 3 * nu + 1) {
+        if (a.act_kp_scale) a.act_kp_scale[e] = rv_value(a.kp_scale_rv, u, z, 1.f);
+      } else if (j == 3 * nu + 2) {
+        if (a.act_kd_scale) a.act_kd_scale[e] = rv_value(a.kd_scale_rv, u, z, 1.f);
+      } else {
+        if (a.act_torque_limit_scale) a.act_torque_limit_scale[e] = rv_value(a.torque_limit_scale_rv, u, z, 1.f);
+      }
+    }
+  }
   if (a.random_heading && nq >= 7) {
     __syncthreads();  // the base orientation written above is read back by the env's own lane
     if (tid < ne && s_reset[tid]) {
@@ -948,7 +1017,13 @@ extern "C" int ks_terms_create(const KsTermsDesc* d, KsTerms** out) {
       return fail(KS_EINVAL, "ks_terms_create: obs %d: joint position index %d out of range", k, el.index);
     if (el.kind == KS_OBS_ROT_INV && (el.comp < 0 || el.comp > 2 || d->nq < 7))
       return fail(KS_EINVAL, "ks_terms_create: obs %d: bad rotation component", k);
-    if (el.noise_kind < KS_NOISE_NONE || el.noise_kind > KS_NOISE_MUL_UNIFORM) return fail(KS_EINVAL, "ks_terms_create: obs %d: bad noise kind", k);
+  }
+  for (int k = 0; k < d->obs_dim; ++k) {
+    const KsObsElem& el = d->obs[k];
+    if (el.n_noise < 0 || el.n_noise > KS_MAX_NOISE_CHAIN) return fail(KS_ELIMIT, "ks_terms_create: obs %d: %d noise stages (0..%d)", k, el.n_noise, KS_MAX_NOISE_CHAIN);
+    for (int j = 0; j < el.n_noise; ++j)
+      if (el.noise[j].kind <= KS_NOISE_NONE || el.noise[j].kind > KS_NOISE_MUL_UNIFORM_GAUSSIAN) return fail(KS_EINVAL, "ks_terms_create: obs %d: bad noise kind", k);
+    if (el.bias.kind < KS_NOISE_NONE || el.bias.kind > KS_NOISE_MUL_UNIFORM_GAUSSIAN) return fail(KS_EINVAL, "ks_terms_create: obs %d: bad bias kind", k);
   }
   for (int j = 0; j < d->n_terms; ++j) {
     const KsTermDesc& t = d->terms[j];
@@ -995,14 +1070,20 @@ extern "C" int ks_observe(const KsTerms* t, ks_stream_t stream, const KsObserveI
     }
     if (el.src != KS_SRC_CONST && !io->src[el.src]) return fail(KS_EINVAL, "ks_observe: observation %d reads source %d, which is NULL", k, el.src);
     needs_quat |= el.kind == KS_OBS_ROT_INV || el.kind == KS_OBS_GRAVITY_EMA;
-    needs_noise |= el.noise_kind != KS_NOISE_NONE;
   }
+  bool needs_bias = false;
+  for (int k = 0; k < d.obs_dim; ++k) {
+    const KsObsElem& el = d.obs[k];
+    needs_noise |= el.n_noise > 0;
+    needs_bias |= el.bias.kind != KS_NOISE_NONE;
+  }
+  if (needs_bias && io->noisy_obs && !io->bias_draw) return fail(KS_EINVAL, "ks_observe: observations with a bias need the bias_draw buffer");
   if (needs_quat && !io->src[KS_SRC_QPOS]) return fail(KS_EINVAL, "ks_observe: qpos is required for body-frame observations");
   if ((io->noise_normal == nullptr) != (io->noise_uniform == nullptr)) return fail(KS_EINVAL, "ks_observe: pass both explicit noise buffers or neither");
   (void)needs_noise;
   a.t = t->dev; a.N = io->N; a.level = io->level;
   for (int s = 0; s < KS_SRC_COUNT; ++s) { a.src[s] = io->src[s]; a.src_dim[s] = src_dim[s]; }
-  a.zero_offset = io->zero_offset; a.bias = io->bias; a.noise_normal = io->noise_normal; a.noise_uniform = io->noise_uniform;
+  a.zero_offset = io->zero_offset; a.bias_draw = needs_bias ? io->bias_draw : nullptr; a.bias_redraw = io->bias_redraw; a.noise_normal = io->noise_normal; a.noise_uniform = io->noise_uniform;
   a.rng = io->rng; a.obs = io->obs; a.noisy = io->noisy_obs; a.obs_dim = d.obs_dim; a.nq = d.nq; a.nu = d.nu;
   a.carry = io->carry; a.fresh = io->fresh; a.carry_uniform = io->carry_uniform; a.carry_dim = d.carry_dim;
   const int64_t n = io->N * d.obs_dim;
@@ -1034,6 +1115,17 @@ extern "C" int ks_terminate_reset(const KsTerms* t, ks_stream_t stream, const Ks
     if (d.terms[j].kind == KS_TERM_ILLEGAL_CONTACT && !io->contact_dist) return fail(KS_EINVAL, "ks_terminate_reset: termination %d reads contact_dist", j);
   a.n_events = io->n_events; a.event_state = io->event_state; a.event_reset_uniform = io->event_reset_uniform; a.event_force = io->event_force;
   for (int k = 0; k < io->n_events; ++k) { a.event_interval[k][0] = io->event_interval[k][0]; a.event_interval[k][1] = io->event_interval[k][1]; }
+  a.action_latency = io->action_latency; a.zero_offset = io->zero_offset; a.act_action_bias = io->act_action_bias;
+  a.act_torque_bias = io->act_torque_bias; a.act_kp_scale = io->act_kp_scale; a.act_kd_scale = io->act_kd_scale;
+  a.act_torque_limit_scale = io->act_torque_limit_scale;
+  a.latency_lo = io->latency_lo; a.latency_hi = io->latency_hi;
+  a.zero_offset_rv = io->zero_offset_rv; a.action_bias_rv = io->action_bias_rv; a.torque_bias_rv = io->torque_bias_rv;
+  a.kp_scale_rv = io->kp_scale_rv; a.kd_scale_rv = io->kd_scale_rv; a.torque_limit_scale_rv = io->torque_limit_scale_rv;
+  a.episode_uniform = io->episode_uniform; a.episode_normal = io->episode_normal;
+  a.redraw = (a.action_latency || a.zero_offset || a.act_action_bias || a.act_torque_bias || a.act_kp_scale || a.act_kd_scale ||
+              a.act_torque_limit_scale) ? 1 : 0;
+  if (a.action_latency && !(io->latency_lo >= 0.f && io->latency_hi >= io->latency_lo))
+    return fail(KS_EINVAL, "ks_terminate_reset: latency range must satisfy 0 <= lo <= hi");
   const int64_t grid = (io->N + kTermEnvs - 1) / kTermEnvs;
   if (grid > 0x7fffffff) return fail(KS_ELIMIT, "ks_terminate_reset: too many envs");
   hipLaunchKernelGGL(terminate_kernel, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, a);

@@ -77,7 +77,8 @@ class EngineConfig:  # engine.py:48-139
         return 1
 
     def zero_offset_random_variable(self) -> RandomVariable:  # engine.py:117-138
-        return RandomVariable(mean=0.0, std=self.zero_offset_std or 0.0, mag=self.zero_offset_mag or 0.0)
+        both = self.zero_offset_std is not None and self.zero_offset_mag is not None  # then one key draws both parts
+        return RandomVariable(mean=0.0, std=self.zero_offset_std or 0.0, mag=self.zero_offset_mag or 0.0, same_key=both)
 
 
 @dataclass(frozen=True)
@@ -161,7 +162,7 @@ class HipEngine(PhysicsEngine):
 
     # -------------------------------------------------------------------------------------- reset (engine.py:205-246)
     def reset(self, physics_model: physics.DeviceModel, curriculum_level, rng, num_envs: int,
-              randomization: Mapping[str, torch.Tensor] | None = None, reset_uniform=None) -> PhysicsState:
+              randomization: Mapping[str, torch.Tensor] | None = None, reset_uniform=None, episode_draws=None) -> PhysicsState:
         self._check(physics_model)
         m, N, dev = physics_model.model, int(num_envs), torch.device("cuda")
         gen = _generator(rng, dev)
@@ -169,17 +170,38 @@ class HipEngine(PhysicsEngine):
         data = PhysicsData(qpos=z(N, m.nq), qvel=z(N, m.nv), qacc=z(N, m.nv), qacc_warmstart=z(N, m.nv),
                            ctrl=z(N, m.nu), time=z(N), xpos=z(N, m.nb * 3), xquat=z(N, m.nb * 4), cvel=z(N, m.nb * 6),
                            contact_dist=z(N, m.ns) if m.ns else None, cinert=z(N, m.nb * 10), cfrc_ext=z(N, m.nb * 6))
-        level = float(curriculum_level)
-        lo, hi = self.data.min_action_latency_step * level, self.data.max_action_latency_step * level
+        # latency, zero offset and actuator state are filled by the reset kernel below, the same code that re-draws them
+        # for an env that is reset in the middle of a rollout (engine.py:222-245)
+        act_state = None
+        if isinstance(self.actuators, PositionActuators):
+            act_state = {"action": z(N, m.nu), "torque": z(N, m.nu), "kp_scale": z(N), "kd_scale": z(N),
+                         "torque_limit_scale": z(N)}
         state = PhysicsState(
             last_ctrl=z(N, self.actuators.action_dim(m.nu)), data=data, event_states=self._initial_event_states(N, gen, dev),
-            actuator_state=self.actuators.get_initial_state(N, gen) if isinstance(self.actuators, PositionActuators) else None,
-            action_latency=lo + (hi - lo) * torch.rand(N, generator=gen, device=dev),
-            zero_offset=self.data.zero_offset.sample((N, m.nu), gen, level),
+            actuator_state=act_state, action_latency=z(N), zero_offset=z(N, m.nu),
         )
         seed = int(torch.randint(0, 2**31 - 1, (1,), generator=gen, device=dev).item())
-        self.reset_where(physics_model, state, None, curriculum_level, seed, 0, randomization, reset_uniform)
+        self.reset_where(physics_model, state, None, curriculum_level, seed, 0, randomization, reset_uniform,
+                         episode_draws=episode_draws)
         return state
+
+    def episode_args(self, state: PhysicsState, draws: Mapping | None = None) -> dict:
+        """What `EnvTerms.terminate_reset(episode=...)` takes: the per-episode buffers of `state`, the random variables
+        behind them, and optionally explicit draws {"uniform", "normal"}, each (N, 3 nu + 4)."""
+        out = dict(action_latency=state.action_latency, zero_offset=state.zero_offset,
+                   latency_range=(self.data.min_action_latency_step, self.data.max_action_latency_step),
+                   zero_offset_rv=self.data.zero_offset)
+        act = self.actuators
+        if isinstance(act, PositionActuators) and state.actuator_state is not None:
+            ast, rv = state.actuator_state, act._rv
+            out.update(act_action_bias=ast["action"], act_torque_bias=ast["torque"], act_kp_scale=ast["kp_scale"],
+                       act_kd_scale=ast["kd_scale"], act_torque_limit_scale=ast["torque_limit_scale"],
+                       action_bias_rv=act.action_bias or RandomVariable(), torque_bias_rv=act.torque_bias or RandomVariable(),
+                       kp_scale_rv=rv(act.kp_scale) or RandomVariable(mean=1.0), kd_scale_rv=rv(act.kd_scale) or RandomVariable(mean=1.0),
+                       torque_limit_scale_rv=rv(act.torque_limit_scale) or RandomVariable(mean=1.0))
+        if draws:
+            out.update(episode_uniform=draws.get("uniform"), episode_normal=draws.get("normal"))
+        return out
 
     def _initial_event_states(self, N: int, gen, dev) -> dict:
         """One timer per event and env (engine.py:226-232); rows of one (n_events, N) buffer, which the kernels take."""
@@ -208,14 +230,15 @@ class HipEngine(PhysicsEngine):
         return descs, physics_state.event_states["_buffer"], uniform, rng, physics_state.event_states.get("_force_buffer")
 
     def reset_where(self, physics_model, state: PhysicsState, mask, curriculum_level, seed: int, step: int,
-                    randomization=None, reset_uniform=None) -> None:
-        """Fresh episodes for the envs in `mask` (all when None): resets, then mjx.forward's counterpart."""
+                    randomization=None, reset_uniform=None, episode_draws=None) -> None:
+        """With `mask` None: fresh episodes for every env (resets, per-episode draws, then mjx.forward's counterpart).
+        With a mask: only the forward pass of the masked envs, whose state `EnvTerms.terminate_reset` has already reset."""
         d = state.data
         terms = self._reset_terms(physics_model)
         st = dict(qpos=d.qpos, qvel=d.qvel, qacc_warmstart=d.qacc_warmstart, time=d.time, last_ctrl=state.last_ctrl)
         if mask is None:
             terms.terminate_reset(st, level=float(curriculum_level), seed=seed, step=step, apply_reset=2,
-                                  reset_uniform=reset_uniform)
+                                  reset_uniform=reset_uniform, episode=self.episode_args(state, episode_draws))
         self.forward(physics_model, state, mask, randomization)
 
     def forward(self, physics_model, state: PhysicsState, mask=None, randomization=None) -> None:

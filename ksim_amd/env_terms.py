@@ -32,8 +32,9 @@ def compile_terms(model: KinematicModel, observations: Mapping[str, Observation]
                   terminate_on_nonfinite: bool = True, action_dim: int | None = None):
     """Host-side compilation of the task's terms into the flat tables of KsTermsDesc (no GPU involved).
 
-    Returns (desc, obs_slices, sources_used, bias_std, reset_table); `desc.carry_dim` is the length of the per-env
-    carry row of the stateful observations, laid out in dict order."""
+    Returns (desc, obs_slices, sources_used, has_bias, reset_table); `desc.carry_dim` is the length of the per-env
+    carry row of the stateful observations, laid out in dict order; `has_bias` says whether any observation carries a
+    per-episode bias (then `observe` needs the bias-draw buffer)."""
     d = T.KsTermsDesc()
     d.nq, d.nv, d.nu, d.nb, d.command_dim = model.nq, model.nv, model.nu, model.nb, int(command_dim)
     d.ns = model.ns
@@ -41,11 +42,11 @@ def compile_terms(model: KinematicModel, observations: Mapping[str, Observation]
     carry_at = 0
     obs_slices: dict[str, slice] = {}
     sources_used: set[int] = set()
-    bias_std: list[float] = []
+    has_bias = False
     k = 0
     for name, obs in observations.items():
         elems = obs.elements(model, int(command_dim))
-        noise = obs._noise()
+        noise, bias = obs._noise(), obs._bias()
         if k + len(elems) > T.KS_MAX_OBS:
             raise _lib.KsError(f"observation vector longer than {T.KS_MAX_OBS}")
         for el in elems:
@@ -61,8 +62,13 @@ def compile_terms(model: KinematicModel, observations: Mapping[str, Observation]
             if el.kind in (T.OBS_SITE_GYRO, T.OBS_SITE_ACCEL):
                 sources_used.update((T.SRC_XQUAT, T.SRC_CVEL) + ((T.SRC_QACC,) if el.kind == T.OBS_SITE_ACCEL else ()))
             if noise is not None:
-                e.noise_kind, e.noise_mean, e.noise_scale = noise.kind, noise.mean, noise.scale
-            bias_std.append(0.0 if obs.bias is None else float(obs.bias))
+                stages = noise.stages()
+                e.n_noise = len(stages)
+                for j, st in enumerate(stages):
+                    e.noise[j].kind, e.noise[j].mean, e.noise[j].scale, e.noise[j].scale2 = st.kind, st.mean, st.scale, st.scale2
+            if bias is not None and bias.kind != T.NOISE_NONE:
+                e.bias.kind, e.bias.mean, e.bias.scale, e.bias.scale2 = bias.kind, bias.mean, bias.scale, bias.scale2
+                has_bias = True
             k += 1
         obs_slices[name] = slice(k - len(elems), k)
         carry_at += obs.carry_size(model)
@@ -81,7 +87,7 @@ def compile_terms(model: KinematicModel, observations: Mapping[str, Observation]
         d.reset_by_level[i] = int(tab["by_level"][i])
     d.random_heading = int(tab["heading"])
     d.nonfinite_terminates = int(terminate_on_nonfinite)
-    return d, obs_slices, sources_used, bias_std, tab
+    return d, obs_slices, sources_used, has_bias, tab
 
 
 class EnvTerms:
@@ -93,7 +99,7 @@ class EnvTerms:
         self.model, self._lib = model, lib
         self.observations, self.terminations, self.resets = dict(observations), dict(terminations), tuple(resets)
         self.command_dim = int(command_dim)
-        d, self.obs_slices, self.sources_used, self.bias_std, self.reset_table = compile_terms(
+        d, self.obs_slices, self.sources_used, self.has_bias, self.reset_table = compile_terms(
             model, self.observations, self.terminations, self.resets, self.command_dim, terminate_on_nonfinite, action_dim)
         self.action_dim = int(d.action_dim)
         self.obs_dim, self.n_terms, self.carry_dim = int(d.obs_dim), int(d.n_terms), int(d.carry_dim)
@@ -102,11 +108,12 @@ class EnvTerms:
 
     # ------------------------------------------------------------------ observations
     def observe(self, sources: Mapping[int, torch.Tensor | None], N: int, *, level: float = 1.0,
-                zero_offset=None, bias=None, noise_normal=None, noise_uniform=None, seed: int = 0, step: int = 0,
-                step_base=None, carry=None, fresh=None, carry_uniform=None,
+                zero_offset=None, bias_draw=None, bias_redraw=None, noise_normal=None, noise_uniform=None, seed: int = 0,
+                step: int = 0, step_base=None, carry=None, fresh=None, carry_uniform=None,
                 obs: torch.Tensor | None = None, noisy_obs: torch.Tensor | None = None):
         """`carry` (N, carry_dim) is advanced in place; `fresh` (N) uint8 marks the envs whose carries are initialised
-        from the current state first (those that were just reset)."""
+        from the current state first (those that were just reset) and whose bias draws `bias_draw` (N, obs_dim, 2) are
+        renewed (from `bias_redraw` when given, else from the Philox stream)."""
         m = self.model
         dims = {T.SRC_QPOS: m.nq, T.SRC_QVEL: m.nv, T.SRC_QACC: m.nv, T.SRC_CTRL: m.nu, T.SRC_LAST_ACTION: self.action_dim,
                 T.SRC_COMMAND: self.command_dim, T.SRC_TIME: 1, T.SRC_XPOS: m.nb * 3, T.SRC_XQUAT: m.nb * 4,
@@ -120,7 +127,8 @@ class EnvTerms:
             if t.numel() != N * dims[s]:
                 raise _lib.KsError(f"observation source {s}: expected {N}x{dims[s]} elements, got {tuple(t.shape)}")
             io.src[s] = t.data_ptr()
-        for name, t, shape in (("zero_offset", zero_offset, (N, m.nu)), ("bias", bias, (N, self.obs_dim)),
+        for name, t, shape in (("zero_offset", zero_offset, (N, m.nu)), ("bias_draw", bias_draw, (N, self.obs_dim, 2)),
+                               ("bias_redraw", bias_redraw, (N, self.obs_dim, 2)),
                                ("noise_normal", noise_normal, (N, self.obs_dim)),
                                ("noise_uniform", noise_uniform, (N, self.obs_dim)), ("obs", obs, (N, self.obs_dim)),
                                ("noisy_obs", noisy_obs, (N, self.obs_dim)), ("carry", carry, (N, self.carry_dim)),
@@ -145,7 +153,10 @@ class EnvTerms:
                         success=None, traj_qpos=None, traj_qvel=None, traj_time=None, reset_mask=None,
                         episode_length=None, reset_uniform=None, seed: int = 0, step: int = 0, step_base=None,
                         event_state=None, event_intervals=(), event_reset_uniform=None, event_force=None,
-                        contact_dist=None, apply_reset: bool = True) -> None:
+                        contact_dist=None, apply_reset: bool = True, episode: Mapping | None = None) -> None:
+        """`episode`: the per-episode quantities that the envs starting a fresh episode re-draw (engine.py:222-245), as
+        `HipEngine.episode_args` builds them: buffers `action_latency`, `zero_offset`, `act_*`, the matching random
+        variables, and optionally explicit draws `episode_uniform` / `episode_normal` (N, 3 nu + 4)."""
         m = self.model
         qpos = state["qpos"]
         N = qpos.shape[0]
@@ -191,6 +202,24 @@ class EnvTerms:
                 if tuple(event_force.shape) != (len(event_intervals), N, T.KS_EVENT_FORCE_STATE):
                     raise _lib.KsError("force-push state must be (n_events, N, KS_EVENT_FORCE_STATE)")
                 io.event_force = event_force.data_ptr()
+        if episode:
+            nu, ned = m.nu, 3 * m.nu + 4
+            shapes = dict(action_latency=(N,), zero_offset=(N, nu), act_action_bias=(N, nu), act_torque_bias=(N, nu),
+                          act_kp_scale=(N,), act_kd_scale=(N,), act_torque_limit_scale=(N,), episode_uniform=(N, ned),
+                          episode_normal=(N, ned))
+            for name, shape in shapes.items():
+                t = episode.get(name)
+                if t is None:
+                    continue
+                _lib.require_cuda(t, dtype=torch.float32)
+                if tuple(t.shape) != shape:
+                    raise _lib.KsError(f"{name}: expected {shape}, got {tuple(t.shape)}")
+                setattr(io, name, t.data_ptr())
+            io.latency_lo, io.latency_hi = (float(x) for x in episode.get("latency_range", (0.0, 0.0)))
+            for name in ("zero_offset_rv", "action_bias_rv", "torque_bias_rv", "kp_scale_rv", "kd_scale_rv", "torque_limit_scale_rv"):
+                rv = episode.get(name)
+                if rv is not None:
+                    setattr(io, name, rv.desc())
         _lib.check(self._lib.ks_terminate_reset(self._handle, _lib.current_stream(), ctypes.byref(io)))
 
     def close(self) -> None:

@@ -12,7 +12,7 @@ from dataclasses import dataclass, field
 
 from . import _lib_terms as T
 from .model import KinematicModel
-from .noise import Noise, convert_to_noise
+from .noise import Bias, Noise, convert_to_bias, convert_to_noise
 
 
 @dataclass(frozen=True)
@@ -31,7 +31,7 @@ class ObsElem:
 @dataclass(frozen=True)
 class Observation:
     noise: Noise | float | None = None
-    bias: float | None = None  # std of the per-episode additive Gaussian bias (observation.py:79-86)
+    bias: Bias | float | None = None  # per-episode bias; a float is the std of an additive Gaussian one (observation.py:79-86)
 
     def elements(self, model: KinematicModel, command_dim: int) -> list[ObsElem]:  # pragma: no cover
         raise NotImplementedError
@@ -51,6 +51,9 @@ class Observation:
 
     def _noise(self) -> Noise | None:
         return convert_to_noise(self.noise)
+
+    def _bias(self) -> Bias | None:
+        return convert_to_bias(self.bias)
 
 
 def _copy(src, start, n):

@@ -75,7 +75,7 @@ class RolloutEnvState:  # ksim/task/rl.py:110-123, batched
         self.physics_state = physics_state
         self.randomization_dict = dict(randomization)
         self.commands = commands
-        self.obs_bias = obs_bias
+        self.obs_bias = obs_bias  # (N, obs_dim, 2) standard draws (z, w) behind the per-episode observation biases, or None
         self.seed = int(seed)
         self.step = 0
         self.obs_carry = None     # (N, carry_dim) carries of the stateful observations (rl.py:118), made on first use
@@ -135,10 +135,11 @@ class Rollout:
                T.SRC_CFRC_EXT: d.cfrc_ext}
         self._prepare_env(env)
         # the reset mask still holds the envs that the previous control step reset: their carries start afresh
-        c.terms.observe(src, self.N, level=level, zero_offset=ps.zero_offset, bias=env.obs_bias,
+        c.terms.observe(src, self.N, level=level, zero_offset=ps.zero_offset, bias_draw=env.obs_bias,
+                        bias_redraw=noise.get("obs_bias_redraw"),
                         noise_normal=noise.get("obs_normal"), noise_uniform=noise.get("obs_uniform"), seed=env.seed,
                         step=step, step_base=step_base, obs=self.obs[t], noisy_obs=self.noisy_obs[t],
-                        carry=env.obs_carry, fresh=self.reset_mask if c.terms.carry_dim else None,
+                        carry=env.obs_carry, fresh=self.reset_mask if (c.terms.carry_dim or c.terms.has_bias) else None,
                         carry_uniform=noise.get("obs_carry_uniform"))
         # actor reads the noisy copy (walking.py:592-595), critic the clean one (walking.py:626-638); recurrent networks
         # advance their carries, which restart from zero for the envs the previous control step reset
@@ -188,7 +189,7 @@ class Rollout:
                                 event_intervals=[ev.interval_range for ev in c.engine.events.values()],
                                 event_reset_uniform=noise.get("event_reset_uniform"),
                                 event_force=ps.event_states.get("_force_buffer") if ps.event_states else None,
-                                contact_dist=d.contact_dist)
+                                contact_dist=d.contact_dist, episode=c.engine.episode_args(ps, noise.get("episode")))
         # refresh the derived fields and the warm start of the reset envs (engine.py:213)
         c.engine.forward(c.physics_model, ps, self.reset_mask, env.randomization_dict)
         if c.commands is not None:  # record the commands this step ran under, then advance them (rl.py:1082-1098)
@@ -239,6 +240,10 @@ class Rollout:
         if self.c.terms.carry_dim and env.obs_carry is None:
             env.obs_carry = torch.zeros(self.N, self.c.terms.carry_dim, dtype=torch.float32, device=self.done.device)
             self.reset_mask.fill_(1)  # every env starts an episode: the first observation initialises all carries
+        if self.c.terms.has_bias and env.obs_bias is None:
+            # the episode's standard draws behind the observation biases (rl.py:121,263-271 keeps keys instead)
+            env.obs_bias = torch.zeros(self.N, self.c.terms.obs_dim, 2, dtype=torch.float32, device=self.done.device)
+            self.reset_mask.fill_(1)  # every env starts an episode: the first observation draws all of them
         if self.c.commands is not None and not env.commands_drawn:  # get_initial_commands on the reset state (rl.py:319-332)
             d = env.physics_state.data
             self.c.commands.update(env.commands, d.qpos, d.qvel, all_fresh=True, seed=env.seed, step=(1 << 62) + env.step)

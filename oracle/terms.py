@@ -305,6 +305,78 @@ def latency_blend(step_num, latency, last_ctrl, action, drop):
     return np.where(drop, last_ctrl, last_ctrl * (1.0 - prct) + action * prct)
 
 
+# --------------------------------------------------------------------------- random variables, noise, bias
+def same_key_uniform(z):
+    """The U(-1, 1) draw that the random bits behind the standard normal draw z give: jax.random builds a normal as
+    sqrt(2) erfinv(u) of the uniform u in (-1, 1) those bits give, so u = erf(z / sqrt 2) = 2 Phi(z) - 1.  This is what
+    'both drawn with the same key' (ksim/noise.py:106-121, 222-229) means for explicit draws.  jax is third-party and
+    absent here: the construction is restated, parity unpinned; that the result is uniform when z is normal is a theorem
+    (probability integral transform) and is tested."""
+    from math import erf, sqrt
+
+    return np.vectorize(lambda x: erf(x / sqrt(2.0)))(np.asarray(z, dtype=np.float64))
+
+
+def random_variable(mean, mag, std, u, z, level=1.0, same_key=False):
+    """ksim/noise.py:74-121 with explicit standard draws u ~ U(-1,1), z ~ N(0,1): Uniform (std 0), Gaussian (mag 0),
+    UniformGaussian (both, same_key) and Zero (all 0) random variables."""
+    w = same_key_uniform(z) if same_key else np.asarray(u, dtype=np.float64)
+    return mean + np.asarray(z, dtype=np.float64) * (std * level) + w * (mag * level)
+
+
+def apply_noise(obs, kind, mean, scale, z, w, level, scale2=0.0):
+    """One Noise or Bias of ksim/noise.py:129-213 on an observation.  kind: 'add_gaussian', 'add_uniform', 'mul_gaussian',
+    'mul_uniform', 'add_uniform_gaussian', 'mul_uniform_gaussian' or 'none'."""
+    if kind == "none":
+        return np.asarray(obs, dtype=np.float64)
+    op, dist = kind.split("_", 1)
+    if dist == "gaussian":
+        rv = random_variable(mean, 0.0, scale, 0.0, z, level)
+    elif dist == "uniform":
+        rv = random_variable(mean, scale, 0.0, w, 0.0, level)
+    else:
+        rv = random_variable(mean, scale2, scale, w, z, level)
+    return obs + rv if op == "add" else obs * rv
+
+
+def add_noise(obs, noises, bias, z, w, bias_z, bias_w, level):
+    """Observation.add_noise (ksim/observation.py:110-142): the noise (a chain applies every member with the same key,
+    noise.py:222-229, hence the same z and w), then the per-episode bias, whose draw (bias_z, bias_w) is fixed over the
+    episode while its scale follows the current level.  noises: list of (kind, mean, scale[, scale2]); bias: one or None."""
+    out = np.asarray(obs, dtype=np.float64)
+    for st in noises:
+        out = apply_noise(out, st[0], st[1], st[2], z, w, level, *(st[3:4]))
+    if bias is not None:
+        out = apply_noise(out, bias[0], bias[1], bias[2], bias_z, bias_w, level, *(bias[3:4]))
+    return out
+
+
+def engine_reset_draws(nu, level, u, z, *, latency_range, zero_offset, action_bias=None, torque_bias=None, kp_scale=None,
+                       kd_scale=None, torque_limit_scale=None):
+    """What MjxEngine.reset draws besides the state (ksim/engine.py:222-245) with PositionActuators.get_initial_state
+    (ksim/actuators.py:219-238), from explicit standard draws u ~ U(-1,1), z ~ N(0,1) of length 3 nu + 4 laid out as
+    [latency, zero offset (nu), action bias (nu), torque bias (nu), kp scale, kd scale, torque limit scale].
+    latency_range is in physics steps; the random variables are dicts(mean, mag, std[, same_key]); None means the
+    reference's default (zero bias, unit scale).  Latency and zero offset scale with the curriculum level, the actuator
+    state does not (get_random_variable is called without a level there)."""
+    u, z = np.asarray(u, dtype=np.float64), np.asarray(z, dtype=np.float64)
+
+    def rv(spec, sl, lvl, default_mean):
+        spec = spec or dict(mean=default_mean, mag=0.0, std=0.0)
+        return random_variable(spec["mean"], spec.get("mag", 0.0), spec.get("std", 0.0), u[sl], z[sl], lvl, spec.get("same_key", False))
+
+    lo, hi = latency_range[0] * level, latency_range[1] * level
+    return {
+        "action_latency": lo + 0.5 * (u[0] + 1.0) * (hi - lo),  # uniform(minval, maxval), engine.py:233-237
+        "zero_offset": rv(zero_offset, slice(1, 1 + nu), level, 0.0),
+        "action": rv(action_bias, slice(1 + nu, 1 + 2 * nu), 1.0, 0.0),
+        "torque": rv(torque_bias, slice(1 + 2 * nu, 1 + 3 * nu), 1.0, 0.0),
+        "kp_scale": rv(kp_scale, 3 * nu + 1, 1.0, 1.0),
+        "kd_scale": rv(kd_scale, 3 * nu + 2, 1.0, 1.0),
+        "torque_limit_scale": rv(torque_limit_scale, 3 * nu + 3, 1.0, 1.0),
+    }
+
+
 def scrub_action(action, clip_max=1e3):
     """rl.py:998-1001: NaN -> 0, then clip."""
     a = np.where(np.isnan(action), 0.0, action)

@@ -17,7 +17,14 @@ def t32(a):
     return torch.tensor(np.asarray(a), dtype=torch.float32, device=DEV).contiguous()
 
 
-def build(N, T, seed=0, min_height=0.9, events=None, gait=False, recurrent=False, head=None):
+# per-episode sim2real quantities of the `sim2real` builds, as the oracle's engine_reset_draws takes them
+SIM2REAL = dict(latency_range=(1.0, 3.0), zero_offset=dict(mean=0.0, mag=0.0, std=0.01),
+                action_bias=dict(mean=0.0, mag=0.02, std=0.0), torque_bias=dict(mean=0.0, mag=0.0, std=0.3),
+                kp_scale=dict(mean=1.0, mag=0.1, std=0.0), kd_scale=dict(mean=1.0, mag=0.0, std=0.05),
+                torque_limit_scale=dict(mean=0.95, mag=0.05, std=0.0))
+
+
+def build(N, T, seed=0, min_height=0.9, events=None, gait=False, recurrent=False, head=None, sim2real=False):
     from ksim_amd import actuators, engine, model as km, observation as ob, physics, randomization as rnd, resets as rs
     from ksim_amd import rewards as rw, terminations as tm
     from ksim_amd.env_terms import EnvTerms
@@ -32,8 +39,16 @@ def build(N, T, seed=0, min_height=0.9, events=None, gait=False, recurrent=False
     act = actuators.PositionActuators(kps=tuple(kps), kds=tuple(kds), ctrl_clip=tuple(clip))
     resets = [rs.RandomJointPositionReset(scale=0.1, scale_by_curriculum=False)]
     cfg = engine.EngineConfig(dt=0.005, ctrl_dt=0.02)
+    if sim2real:  # what ksim's sim2real knobs add: every one of these is drawn afresh for each episode
+        from ksim_amd import noise as kn
+        act = actuators.PositionActuators(kps=tuple(kps), kds=tuple(kds), ctrl_clip=tuple(clip),
+                                          action_bias=kn.UniformRandomVariable(0.0, 0.02), torque_bias=kn.GaussianRandomVariable(0.0, 0.3),
+                                          kp_scale=kn.UniformRandomVariable(1.0, 0.1), kd_scale=kn.GaussianRandomVariable(1.0, 0.05),
+                                          torque_limit_scale=kn.UniformRandomVariable(0.95, 0.05))
+        cfg = engine.EngineConfig(dt=0.005, ctrl_dt=0.02, action_latency_range=(0.005, 0.015), zero_offset_std=0.01)
     eng = engine.get_physics_engine("hip", resets, events or {}, act, cfg)
-    observations = {"jp": ob.JointPositionObservation(noise=0.01), "jv": ob.JointVelocityObservation(noise=0.01),
+    observations = {"jp": ob.JointPositionObservation(noise=0.01),
+                    "jv": ob.JointVelocityObservation(noise=0.01, bias=0.02 if sim2real else None),
                     "g": ob.ProjectedGravityObservation(noise=0.01),
                     "w": ob.BaseAngularVelocityObservation(in_robot_frame=True, noise=0.01),
                     "a": ob.LastActionObservation(), "c": ob.CommandObservation()}
@@ -121,13 +136,21 @@ def _mlp64(x, ws, bs):
     return h.numpy()
 
 
-def test_rollout_matches_oracle_composition():
+@pytest.mark.parametrize("sim2real", [False, True])
+def test_rollout_matches_oracle_composition(sim2real):
+    """`sim2real`: action latency, zero offset, actuator gain / bias randomisation and an observation bias, all of which the
+    reference draws per episode (ksim/engine.py:222-245, ksim/actuators.py:219-238, ksim/task/rl.py:1110-1117): an env that
+    is reset during the rollout must continue with the oracle's re-draw, the others with what they had."""
     N, T = 12, 3
-    m, c, rnd_, (ws, bs, cws, cbs, log_std, kps, kds, clip), ro, EnvState = build(N, T, seed=5)
+    m, c, rnd_, (ws, bs, cws, cbs, log_std, kps, kds, clip), ro, EnvState = build(N, T, seed=5, sim2real=sim2real)
     rng = np.random.default_rng(6)
-    K = c.terms.obs_dim
+    K, nu, ned = c.terms.obs_dim, m.nu, 3 * m.nu + 4
     u0 = rng.uniform(-1, 1, (N, m.nq + 1))
-    ps = c.engine.reset(c.physics_model, 1.0, 0, N, rnd_, reset_uniform=t32(u0))
+    eu, ez = rng.uniform(-1, 1, (N, ned)), rng.normal(size=(N, ned))
+    ps = c.engine.reset(c.physics_model, 1.0, 0, N, rnd_, reset_uniform=t32(u0), episode_draws=dict(uniform=t32(eu), normal=t32(ez)))
+    spec = SIM2REAL if sim2real else dict(latency_range=(0.0, 0.0), zero_offset=None)
+    epi = [ot.engine_reset_draws(nu, 1.0, eu[e], ez[e], **spec) for e in range(N)]  # the oracle's per-episode quantities
+    bias_zw = np.zeros((N, K, 2))
     # a third of the envs start just below the termination height (feet touching), so they finish on the first step
     low = np.arange(N) % 3 == 0
     ps.data.qpos[torch.from_numpy(low).to(DEV), 2] = 0.87
@@ -144,16 +167,25 @@ def test_rollout_matches_oracle_composition():
         orc.forward(d)  # engine.py:213 — warm start of the fresh episode
         d.qvel = 0.0
     last = np.zeros((N, m.nu))
+    fresh = np.ones(N, bool)  # every env starts an episode at the first step
     for t in range(T):
         noise = dict(obs_normal=rng.normal(size=(N, K)), obs_uniform=rng.random((N, K)),
-                     action_normal=rng.normal(size=(N, m.nu)), reset_uniform=rng.uniform(-1, 1, (N, m.nq + 1)))
-        ro.step_engine(env, t, 1.0, {k: t32(v) for k, v in noise.items()})
-        # oracle: observation
+                     action_normal=rng.normal(size=(N, m.nu)), reset_uniform=rng.uniform(-1, 1, (N, m.nq + 1)),
+                     obs_bias_redraw=np.stack([rng.normal(size=(N, K)), rng.uniform(-1, 1, (N, K))], -1),
+                     episode=dict(uniform=rng.uniform(-1, 1, (N, ned)), normal=rng.normal(size=(N, ned))))
+        ro.step_engine(env, t, 1.0, {k: ({kk: t32(vv) for kk, vv in v.items()} if isinstance(v, dict) else t32(v))
+                                     for k, v in noise.items()})
+        # oracle: observation; the envs that start an episode take new bias draws first (rl.py:1110-1117)
+        bias_zw[fresh] = noise["obs_bias_redraw"][fresh]
+        zo = np.array([ep["zero_offset"] for ep in epi])
         q = np.array([np.array(d.qpos) for d in datas]); v = np.array([np.array(d.qvel) for d in datas])
         g = ot.rotate_vector_by_quat(np.broadcast_to([0, 0, -9.81], (N, 3)), q[:, 3:7], inverse=True)
         w = ot.rotate_vector_by_quat(v[:, 3:6], q[:, 3:7], inverse=True)
-        obs = np.concatenate([q[:, 7:], v[:, 6:], g, w, last, cmd], axis=1)
+        obs = np.concatenate([q[:, 7:] - zo, v[:, 6:], g, w, last, cmd], axis=1)
         noisy = obs.copy(); noisy[:, : 2 * m.nu + 6] += 0.01 * noise["obs_normal"][:, : 2 * m.nu + 6]
+        if sim2real:
+            noisy[:, nu:2 * nu] += 0.02 * bias_zw[:, nu:2 * nu, 0]
+            np.testing.assert_allclose(ro.noisy_obs[t].cpu().numpy(), noisy, rtol=1e-4, atol=2e-4)
         np.testing.assert_allclose(ro.obs[t].cpu().numpy(), obs, rtol=1e-4, atol=2e-4)
         mean = _mlp64(noisy, ws, bs)
         action = ot.scrub_action(mean + np.exp(log_std.astype(np.float64)) * noise["action_normal"])
@@ -163,9 +195,12 @@ def test_rollout_matches_oracle_composition():
         # oracle: physics (4 substeps, blend + PD), termination, reset
         for e, d in enumerate(datas):
             tau = np.zeros(m.nu)
+            ep = epi[e]
             for s in range(4):
-                ctl = ot.latency_blend(float(s), 0.0, last[e], action[e], np.zeros(m.nu, bool))
-                tau = ot.position_actuator_torque(ctl, np.array(d.qpos[7:]), np.array(d.qvel[6:]), kps, kds, clip)
+                ctl = ot.latency_blend(float(s), ep["action_latency"], last[e], action[e], np.zeros(m.nu, bool))
+                tau = ot.position_actuator_torque(ctl, np.array(d.qpos[7:]) - ep["zero_offset"], np.array(d.qvel[6:]), kps, kds, clip,
+                                                  action_bias=ep["action"], torque_bias=ep["torque"], kp_scale=ep["kp_scale"],
+                                                  kd_scale=ep["kd_scale"], torque_limit_scale=ep["torque_limit_scale"])
                 d.ctrl = tau
                 orc.step(d)
         last = action.copy()
@@ -186,6 +221,12 @@ def test_rollout_matches_oracle_composition():
             datas[e] = orc.data(nq, friction=fr[e], mass_scale=ms[e])
             orc.forward(datas[e])
             last[e] = 0.0
+            epi[e] = ot.engine_reset_draws(nu, 1.0, noise["episode"]["uniform"][e], noise["episode"]["normal"][e], **spec)
+        fresh = done.copy()
+        if sim2real:  # the live per-episode state: re-drawn where an episode ended, untouched elsewhere
+            got = dict(action_latency=ps.action_latency, zero_offset=ps.zero_offset, **ps.actuator_state)
+            for k, buf in got.items():
+                np.testing.assert_allclose(buf.cpu().numpy(), np.array([ep[k] for ep in epi]), rtol=2e-6, atol=2e-7, err_msg=k)
         if t == 0:
             assert done.sum() == low.sum()
         # sphere-floor distances of the last collision pass (data.contact.dist): of the last substep for the envs that go
@@ -241,22 +282,27 @@ def _push_events(force=False):
     return evs
 
 
-@pytest.mark.parametrize("with_events", [False, True])
-def test_graph_replay_equals_eager_rollout(with_events):
+@pytest.mark.parametrize("with_events,sim2real", [(False, False), (True, False), (False, True)])
+def test_graph_replay_equals_eager_rollout(with_events, sim2real):
     """A captured rollout graph, replayed several times with eager work and synchronisations in between, gives
     the same bits as the eager loop on every replay (same Philox keys: device step counter + baked step)."""
     N, T, iters = 192, 8, 10
     runs = []
     for use_graph in (False, True):
-        m, c, rnd_, _, ro, EnvState = build(N, T, seed=5, min_height=0.8, events=_push_events(force=True) if with_events else None)
+        m, c, rnd_, _, ro, EnvState = build(N, T, seed=5, min_height=0.8, events=_push_events(force=True) if with_events else None,
+                                            sim2real=sim2real)
         ps = c.engine.reset(c.physics_model, 1.0, 3, N, rnd_)
         env = EnvState(ps, rnd_, torch.zeros(N, 2, device=DEV), None, seed=123)
         snaps, pushed = [], False
+        lat0 = ps.action_latency.clone()
         for it in range(iters):
             traj, rew = ro.unroll(env, graph=use_graph)
             torch.cuda.synchronize()
             snaps.append((traj.qpos.clone(), traj.action.clone(), traj.done.clone(), rew.total.clone(),
                           ps.data.qpos.clone(), env.episode_length.clone()))
+            if sim2real:  # the per-episode draws are part of what a replay must reproduce
+                snaps[-1] += (ps.action_latency.clone(), ps.zero_offset.clone(), ps.actuator_state["kp_scale"].clone(),
+                              ps.actuator_state["torque"].clone(), env.obs_bias.clone())
             if with_events:
                 shove = ps.event_states["shove"]  # (time remaining, duration left, wrench) like the reference's tuple
                 snaps[-1] += (ps.event_states["_buffer"].clone(), shove[1].clone(), shove[2].clone())
@@ -265,11 +311,16 @@ def test_graph_replay_equals_eager_rollout(with_events):
             (junk @ junk).sum().item()
         assert env.step == iters * T
         assert pushed or not with_events, "no force push was ever drawn"
+        if sim2real:
+            changed = (ps.action_latency != lat0).float().mean().item()
+            assert 0.02 < changed < 1.0, f"latency re-drawn for {changed:.2f} of the envs: expected only those that were reset"
         runs.append(snaps)
     assert sum(int(s[2].sum().item()) for s in runs[0]) > 0, "no resets happened: the reset path was not replayed"
     for it, (a, b) in enumerate(zip(*runs)):
-        for x, y, name in zip(a, b, ("qpos", "action", "done", "reward", "state", "episode_length", "event timers",
-                                     "force duration", "held wrench")):
+        names = ("qpos", "action", "done", "reward", "state", "episode_length") + (
+            ("latency", "zero offset", "kp scale", "torque bias", "observation bias draws") if sim2real else
+            ("event timers", "force duration", "held wrench"))
+        for x, y, name in zip(a, b, names):
             assert torch.equal(x, y), f"replay {it}: {name} differs from the eager rollout"
 
 

@@ -41,22 +41,37 @@ def test_observation_assembly_and_noise():
         "base_angular_velocity": ob.BaseAngularVelocityObservation(in_robot_frame=True, noise=noise.AdditiveUniformNoise(mag=0.2, mean=0.1)),
         "last_action": ob.LastActionObservation(),
         "command": ob.CommandObservation(),
-        "base_linear_velocity": ob.BaseLinearVelocityObservation(noise=noise.MultiplicativeGaussianNoise(std=0.05)),
+        "base_linear_velocity": ob.BaseLinearVelocityObservation(noise=noise.MultiplicativeGaussianNoise(std=0.05),
+                                                                 bias=noise.MultiplicativeUniformBias(mag=0.1)),
         "timestep": ob.TimestepObservation(),
-        "actuator_force": ob.ActuatorForceObservation(bias=0.02),
+        "actuator_force": ob.ActuatorForceObservation(
+            noise=noise.ChainedNoise([noise.AdditiveGaussianNoise(std=0.3), noise.MultiplicativeUniformNoise(mag=0.2),
+                                      noise.AdditiveUniformGaussianNoise(std=0.05, mag=0.1)]), bias=0.02),
     }
     terms = EnvTerms(m, observations, {}, [], command_dim=2)
     assert terms.obs_dim == 21 + 21 + 3 + 3 + 21 + 2 + 3 + 1 + 21
     assert terms.obs_dim - 25 == 71  # the first six are the 71-wide actor input of benchmark config 3
     K = terms.obs_dim
     nn, uu = s["rng"].normal(size=(N, K)), s["rng"].random((N, K))
-    bias = s["rng"].normal(size=(N, K)) * 0.02
+    bias0 = np.stack([s["rng"].normal(size=(N, K)), s["rng"].uniform(-1, 1, size=(N, K))], axis=-1)  # an older episode's draws
+    bias1 = np.stack([s["rng"].normal(size=(N, K)), s["rng"].uniform(-1, 1, size=(N, K))], axis=-1)  # what fresh envs take
+    fresh = np.arange(N) % 4 == 1
+    bias_draw = t32(bias0)
     level = 0.7
     src = {T.SRC_QPOS: t32(s["qpos"]), T.SRC_QVEL: t32(s["qvel"]), T.SRC_QACC: t32(s["qacc"]), T.SRC_CTRL: t32(s["ctrl"]),
            T.SRC_LAST_ACTION: t32(s["last"]), T.SRC_COMMAND: t32(s["cmd"]), T.SRC_TIME: t32(s["time"])}
     obs = torch.empty(N, K, device=DEV); noisy = torch.empty(N, K, device=DEV)
-    terms.observe(src, N, level=level, zero_offset=t32(s["zero"]), bias=t32(bias), noise_normal=t32(nn),
-                  noise_uniform=t32(uu), obs=obs, noisy_obs=noisy)
+    terms.observe(src, N, level=level, zero_offset=t32(s["zero"]), bias_draw=bias_draw, bias_redraw=t32(bias1),
+                  fresh=torch.from_numpy(fresh.astype(np.uint8)).to(DEV), noise_normal=t32(nn), noise_uniform=t32(uu), obs=obs,
+                  noisy_obs=noisy)
+    # envs that start an episode took new bias draws, the others kept theirs, bit for bit
+    bias = np.where(fresh[:, None, None], bias1, bias0)
+    got_draw = bias_draw.cpu().numpy()
+    for name in ("base_linear_velocity", "actuator_force"):
+        a = terms.obs_slices[name]
+        np.testing.assert_array_equal(got_draw[:, a], bias[:, a].astype(np.float32))
+    a = terms.obs_slices["joint_position"]
+    np.testing.assert_array_equal(got_draw[:, a], bias0[:, a].astype(np.float32))  # no bias there: never touched
     q, v = s["qpos"], s["qvel"]
     g = ot.rotate_vector_by_quat(np.broadcast_to([0, 0, -9.81], (N, 3)), q[:, 3:7], inverse=True)
     w = ot.rotate_vector_by_quat(v[:, 3:6], q[:, 3:7], inverse=True)
@@ -68,15 +83,28 @@ def test_observation_assembly_and_noise():
     a = sl["joint_position"]; wn[:, a] = want[:, a] + nn[:, a] * 0.01 * level            # noise.py:102
     a = sl["joint_velocity"]; wn[:, a] = want[:, a] * ((1.0 - 0.1 * level) + 2 * 0.1 * level * uu[:, a])  # noise.py:86
     a = sl["base_angular_velocity"]; wn[:, a] = want[:, a] + (0.1 - 0.2 * level) + 2 * 0.2 * level * uu[:, a]
-    a = sl["base_linear_velocity"]; wn[:, a] = want[:, a] * (nn[:, a] * 0.05 * level + 1.0)
-    wn = wn + bias
+    ww = 2 * uu - 1
+    a = sl["base_linear_velocity"]
+    wn[:, a] = ot.add_noise(want[:, a], [("mul_gaussian", 1.0, 0.05)], ("mul_uniform", 1.0, 0.1), nn[:, a], ww[:, a],
+                            bias[:, a, 0], bias[:, a, 1], level)
+    a = sl["actuator_force"]
+    wn[:, a] = ot.add_noise(want[:, a], [("add_gaussian", 0.0, 0.3), ("mul_uniform", 1.0, 0.2), ("add_uniform_gaussian", 0.0, 0.05, 0.1)],
+                            ("add_gaussian", 0.0, 0.02), nn[:, a], ww[:, a], bias[:, a, 0], bias[:, a, 1], level)
     np.testing.assert_allclose(noisy.cpu().numpy(), wn, rtol=3e-6, atol=3e-6)
     # in-kernel Philox: deterministic for a (seed, step), different across steps, unit-variance normals
     a1 = torch.empty(N, K, device=DEV); a2 = torch.empty(N, K, device=DEV); a3 = torch.empty(N, K, device=DEV)
-    terms.observe(src, N, seed=5, step=1, zero_offset=t32(s["zero"]), noisy_obs=a1)
-    terms.observe(src, N, seed=5, step=1, zero_offset=t32(s["zero"]), noisy_obs=a2)
-    terms.observe(src, N, seed=5, step=2, zero_offset=t32(s["zero"]), noisy_obs=a3)
-    assert torch.equal(a1, a2) and not torch.equal(a1, a3)
+    all_fresh = torch.ones(N, dtype=torch.uint8, device=DEV)
+    d1, d2 = torch.zeros(N, K, 2, device=DEV), torch.zeros(N, K, 2, device=DEV)
+    terms.observe(src, N, seed=5, step=1, zero_offset=t32(s["zero"]), noisy_obs=a1, bias_draw=d1, fresh=all_fresh)
+    terms.observe(src, N, seed=5, step=1, zero_offset=t32(s["zero"]), noisy_obs=a2, bias_draw=d2, fresh=all_fresh)
+    terms.observe(src, N, seed=5, step=2, zero_offset=t32(s["zero"]), noisy_obs=a3, bias_draw=d2)
+    assert torch.equal(a1, a2) and not torch.equal(a1, a3) and torch.equal(d1, d2)  # step 2 had no fresh env: draws kept
+    # the Philox bias draws: a standard normal and the uniform the same bits give
+    zb, wb = d1[:, sl["actuator_force"], 0].flatten().cpu().numpy(), d1[:, sl["actuator_force"], 1].flatten().cpu().numpy()
+    assert abs(zb.mean()) < 0.15 and abs(zb.std() - 1.0) < 0.15
+    np.testing.assert_allclose(wb, ot.same_key_uniform(zb), atol=2e-6)
+    with pytest.raises(Exception, match="bias_draw"):
+        terms.observe(src, N, zero_offset=t32(s["zero"]), noisy_obs=a1)
     z = ((a1 - obs)[:, sl["joint_position"]] / 0.01).flatten()
     assert abs(z.mean().item()) < 0.15 and abs(z.std().item() - 1.0) < 0.15
 
@@ -182,6 +210,79 @@ def test_reset_predication():
     assert torch.equal(st2["qpos"], st3["qpos"])
     j = st2["qpos"].cpu().numpy()[dn][:, 7:]
     assert (np.abs(j) <= 0.25 + 1e-6).all() and j.std() > 0.03
+
+
+def test_reset_redraws_per_episode_quantities():
+    """An env that is reset mid-rollout gets a new action latency, zero offset and actuator state, as MjxEngine.reset draws
+    them under cond(done) (ksim/engine.py:222-245, ksim/actuators.py:219-238); a continuing env keeps its own."""
+    from ksim_amd import actuators, engine, model as km, noise, physics, resets as rs, terminations as tm
+    from ksim_amd.env_terms import EnvTerms
+
+    m = km.kbot_scale_model()
+    N, nu = 70, m.nu
+    act = actuators.PositionActuators(kps=(50.0,) * nu, kds=(1.0,) * nu, action_bias=noise.UniformRandomVariable(0.0, 0.05),
+                                      torque_bias=noise.GaussianRandomVariable(0.1, 0.5), kp_scale=noise.UniformRandomVariable(1.0, 0.2),
+                                      kd_scale=0.9, torque_limit_scale=noise.GaussianRandomVariable(1.0, 0.05))
+    cfg = engine.EngineConfig(dt=0.005, ctrl_dt=0.02, action_latency_range=(0.005, 0.015), zero_offset_std=0.01, zero_offset_mag=0.02)
+    resets = [rs.RandomJointPositionReset(scale=0.1, scale_by_curriculum=False)]
+    eng = engine.get_physics_engine("hip", resets, {}, act, cfg)
+    dm = physics.DeviceModel(m)
+    rng = np.random.default_rng(11)
+    ned = 3 * nu + 4
+    level = 0.6
+    spec = dict(latency_range=(1.0, 3.0), zero_offset=dict(mean=0.0, mag=0.02, std=0.01, same_key=True),
+                action_bias=dict(mean=0.0, mag=0.05, std=0.0), torque_bias=dict(mean=0.1, mag=0.0, std=0.5),
+                kp_scale=dict(mean=1.0, mag=0.2, std=0.0), kd_scale=dict(mean=0.9, mag=0.0, std=0.0),
+                torque_limit_scale=dict(mean=1.0, mag=0.0, std=0.05))
+
+    def check(ps, rows, u, z):
+        ast = ps.actuator_state
+        got = dict(action_latency=ps.action_latency, zero_offset=ps.zero_offset, action=ast["action"], torque=ast["torque"],
+                   kp_scale=ast["kp_scale"], kd_scale=ast["kd_scale"], torque_limit_scale=ast["torque_limit_scale"])
+        got = {k: v.cpu().numpy() for k, v in got.items()}
+        for e in rows:
+            want = ot.engine_reset_draws(nu, level, u[e], z[e], **spec)
+            for k, w in want.items():
+                np.testing.assert_allclose(got[k][e], w, rtol=2e-6, atol=2e-7, err_msg=f"{k} of env {e}")
+
+    # the first reset of every env draws them through the same kernel
+    u0, z0 = rng.uniform(-1, 1, (N, ned)), rng.normal(size=(N, ned))
+    ps = eng.reset(dm, level, 3, N, episode_draws=dict(uniform=t32(u0), normal=t32(z0)))
+    check(ps, range(N), u0, z0)
+    lat = ps.action_latency.cpu().numpy()
+    assert (lat >= 1.0 * level - 1e-6).all() and (lat <= 3.0 * level + 1e-6).all() and lat.std() > 0.1
+    # a control step later some envs have fallen: only those re-draw
+    terms = EnvTerms(m, {}, {"h": tm.MinimumHeightTermination(0.5)}, resets)
+    d = ps.data
+    fallen = np.arange(N) % 5 == 2
+    d.qpos[:, 2] = torch.from_numpy(np.where(fallen, 0.3, 0.9).astype(np.float32)).to(DEV)
+    keep_before = {k: v.clone() for k, v in dict(lat=ps.action_latency, zo=ps.zero_offset, **ps.actuator_state).items()}
+    u1, z1 = rng.uniform(-1, 1, (N, ned)), rng.normal(size=(N, ned))
+    st = dict(qpos=d.qpos, qvel=d.qvel, qacc_warmstart=d.qacc_warmstart, time=d.time, last_ctrl=ps.last_ctrl)
+    done = torch.zeros(N, dtype=torch.uint8, device=DEV)
+    terms.terminate_reset(st, level=level, done=done, episode=eng.episode_args(ps, dict(uniform=t32(u1), normal=t32(z1))))
+    assert np.array_equal(done.cpu().numpy().astype(bool), fallen)
+    check(ps, np.nonzero(fallen)[0], u1, z1)
+    after = dict(lat=ps.action_latency, zo=ps.zero_offset, **ps.actuator_state)
+    keep = torch.from_numpy(~fallen).to(DEV)
+    for k, v in after.items():
+        assert torch.equal(v[keep], keep_before[k][keep]), k           # continuing envs: bit for bit the same
+        assert not torch.equal(v[~keep], keep_before[k][~keep]) or k == "kd_scale", k  # reset envs: new values
+    # Philox draws: reproducible for a (seed, step), in range, and different between steps
+    snaps = []
+    for step in (4, 4, 5):
+        d.qpos[:, 2] = 0.3
+        terms.terminate_reset(st, level=level, seed=21, step=step, episode=eng.episode_args(ps))
+        snaps.append({k: v.clone() for k, v in dict(lat=ps.action_latency, zo=ps.zero_offset, **ps.actuator_state).items()})
+    for k in snaps[0]:
+        assert torch.equal(snaps[0][k], snaps[1][k]), k
+    assert not torch.equal(snaps[0]["lat"], snaps[2]["lat"]) and not torch.equal(snaps[0]["zo"], snaps[2]["zo"])
+    lat = snaps[0]["lat"].cpu().numpy()
+    assert (lat >= 0.6 - 1e-6).all() and (lat <= 1.8 + 1e-6).all()
+    kp = snaps[0]["kp_scale"].cpu().numpy()
+    assert (np.abs(kp - 1.0) <= 0.2 + 1e-6).all() and kp.std() > 0.05
+    zo = snaps[0]["zo"].cpu().numpy()
+    assert (np.abs(zo) <= level * (0.02 + 5 * 0.01)).all() and zo.std() > 0.003
 
 
 def test_sample_action_scrub_and_clip():

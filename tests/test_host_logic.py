@@ -17,7 +17,8 @@ def test_struct_layouts_match_the_library():
     lib.ks_abi_sizeof.argtypes = [ctypes.c_int32]
     structs = [_lib.KsPpoLossParams, _lib_dyn.KsModelDesc, _lib_dyn.KsStepIO, T.KsTermsDesc, T.KsObserveIO,
                T.KsTerminateIO, T.KsMlpDesc, T.KsRewardIO, T.KsObsElem, T.KsTermDesc, T.KsRewardDesc, T.KsRng,
-               T.KsAdamParams, T.KsEventDesc, T.KsRewardScanIO, T.KsRewardScanDesc, T.KsGruDesc, T.KsLstmDesc, T.KsGaussianHead, T.KsCommandIO, T.KsMixtureHead]
+               T.KsAdamParams, T.KsEventDesc, T.KsRewardScanIO, T.KsRewardScanDesc, T.KsGruDesc, T.KsLstmDesc, T.KsGaussianHead, T.KsCommandIO, T.KsMixtureHead,
+               T.KsNoiseStage, T.KsRandomVar]
     for i, st in enumerate(structs):
         assert lib.ks_abi_sizeof(i) == ctypes.sizeof(st), st.__name__
     assert lib.ks_abi_sizeof(99) == -1
@@ -77,14 +78,24 @@ def test_actuator_and_term_validation():
 
 def test_term_tables_compile():
     m = km.humanoid_model()
-    observations = {"jp": ob.JointPositionObservation(noise=0.01), "jv": ob.JointVelocityObservation(),
+    chain = noise.ChainedNoise([noise.AdditiveGaussianNoise(std=0.02), noise.MultiplicativeUniformNoise(mag=0.1)])
+    observations = {"jp": ob.JointPositionObservation(noise=0.01),
+                    "jv": ob.JointVelocityObservation(noise=chain, bias=noise.MultiplicativeUniformBias(mag=0.05)),
                     "g": ob.ProjectedGravityObservation(), "w": ob.BaseAngularVelocityObservation(in_robot_frame=True),
                     "a": ob.LastActionObservation(), "c": ob.CommandObservation()}
     resets = [rs.RandomJointPositionReset(scale=0.1, scale_by_curriculum=False), rs.RandomHeightReset(range=(0.0, 0.1)),
               rs.RandomHeadingReset(), rs.RandomJointVelocityReset()]
     d, slices, used, bias, tab = compile_terms(m, observations, {"h": tm.MinimumHeightTermination(0.5)}, resets, 2)
     assert d.obs_dim == 71 and slices["g"] == slice(42, 45) and slices["c"] == slice(69, 71)  # benchmark config 3: 71
-    assert d.obs[0].kind == T.OBS_JOINT_POS and d.obs[0].index == 7 and d.obs[0].noise_kind == T.NOISE_ADD_GAUSSIAN
+    assert d.obs[0].kind == T.OBS_JOINT_POS and d.obs[0].index == 7
+    assert d.obs[0].n_noise == 1 and d.obs[0].noise[0].kind == T.NOISE_ADD_GAUSSIAN and d.obs[0].bias.kind == T.NOISE_NONE
+    jv = d.obs[slices["jv"].start]
+    assert jv.n_noise == 2 and jv.noise[1].kind == T.NOISE_MUL_UNIFORM and jv.noise[1].mean == 1.0
+    assert jv.bias.kind == T.NOISE_MUL_UNIFORM and jv.bias.scale == pytest.approx(0.05) and bias is True
+    assert noise.convert_to_bias(0.1).kind == T.NOISE_ADD_GAUSSIAN and noise.convert_to_bias(None) is None
+    zo = engine.EngineConfig(dt=0.005, ctrl_dt=0.02, zero_offset_std=0.01, zero_offset_mag=0.02).zero_offset_random_variable()
+    assert zo.same_key and zo.std == 0.01 and zo.mag == 0.02  # one key draws both parts (engine.py:117-124)
+    assert not engine.EngineConfig(dt=0.005, ctrl_dt=0.02, zero_offset_std=0.01).zero_offset_random_variable().same_key
     assert d.obs[42].kind == T.OBS_ROT_INV and d.obs[44].comp == 2 and d.obs[44].c2 == pytest.approx(-9.81)
     assert T.SRC_CVEL not in used and T.SRC_QPOS in used
     assert d.n_terms == 1 and d.terms[0].kind == T.TERM_MIN_HEIGHT and d.terms[0].value == -1

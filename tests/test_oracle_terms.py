@@ -544,3 +544,68 @@ def test_sinusoidal_gait_command_and_reward_hand_computed():
     np.testing.assert_allclose(c[:2], [0, 0], atol=1e-15)                 # and the flag stays down while the episode lasts
     pos = np.array([[[0, 0, 0.05], [0, 0, 0.2]]])
     np.testing.assert_allclose(ot.sinusoidal_gait_reward(pos, np.array([[0.01, 0.21]]), 0.2), [1 - (0.04 + 0.01) / 0.2], rtol=1e-12)
+
+
+def test_random_variables_noise_and_bias_hand_computed():
+    """ksim/noise.py:74-229 and Observation.add_noise (ksim/observation.py:110-142) on hand-computed numbers."""
+    from scipy import stats
+
+    # uniform: U(mean - mag level, mean + mag level); u = +-1 are the ends, u = 0 the mean
+    assert ot.random_variable(2.0, 0.5, 0.0, 1.0, 0.0, level=0.5) == pytest.approx(2.25)
+    assert ot.random_variable(2.0, 0.5, 0.0, -1.0, 0.0, level=0.5) == pytest.approx(1.75)
+    # gaussian: z std level + mean
+    assert ot.random_variable(1.0, 0.0, 0.2, 0.7, -1.5, level=0.5) == pytest.approx(1.0 - 0.15)
+    # level 0 leaves the mean whatever the draws
+    assert ot.random_variable(3.0, 1.0, 1.0, 0.3, 0.4, level=0.0) == pytest.approx(3.0)
+    # one key for both parts: the uniform part is 2 Phi(z) - 1 (scipy's normal CDF, not the oracle's erf)
+    z = np.array([-2.0, -0.3, 0.0, 1.1])
+    np.testing.assert_allclose(ot.same_key_uniform(z), 2 * stats.norm.cdf(z) - 1, rtol=0, atol=1e-15)
+    got = ot.random_variable(0.5, 0.2, 0.1, 99.0, z, level=1.0, same_key=True)  # the explicit uniform is ignored
+    np.testing.assert_allclose(got, 0.5 + 0.1 * z + 0.2 * (2 * stats.norm.cdf(z) - 1), atol=1e-15)
+    # ... and it is uniform on (-1, 1) when z is standard normal
+    zz = np.random.default_rng(3).normal(size=20000)
+    assert stats.kstest(ot.same_key_uniform(zz), stats.uniform(-1, 2).cdf).pvalue > 1e-3
+    # additive / multiplicative noise; multiplicative means default to 1 in the reference (noise.py:201-213)
+    assert ot.apply_noise(2.0, "add_gaussian", 0.0, 0.1, 1.5, 0.0, 1.0) == pytest.approx(2.15)
+    assert ot.apply_noise(2.0, "mul_uniform", 1.0, 0.1, 0.0, -1.0, 0.5) == pytest.approx(2.0 * 0.95)
+    assert ot.apply_noise(2.0, "mul_gaussian", 1.0, 0.1, 2.0, 0.0, 1.0) == pytest.approx(2.4)
+    assert ot.apply_noise(2.0, "add_uniform", 0.1, 0.2, 0.0, 0.5, 1.0) == pytest.approx(2.2)
+    assert ot.apply_noise(2.0, "add_uniform_gaussian", 0.0, 0.1, 1.0, 0.5, 1.0, 0.4) == pytest.approx(2.0 + 0.1 + 0.2)
+    assert ot.apply_noise(2.0, "none", 0.0, 0.0, 1.0, 1.0, 1.0) == 2.0
+    # a chain applies its members in order with the same draws, then the bias with the episode's draw:
+    # ((2 + 0.1 * 1.5) * (1 + 0.1 * 0.5)) + 0.02 * (-2) = 2.15 * 1.05 - 0.04
+    got = ot.add_noise(2.0, [("add_gaussian", 0.0, 0.1), ("mul_uniform", 1.0, 0.1)], ("add_gaussian", 0.0, 0.02), 1.5, 0.5,
+                       -2.0, 0.0, 1.0)
+    assert got == pytest.approx(2.15 * 1.05 - 0.04)
+    # the order matters, which a swapped implementation would fail: (2 * 1.05) + 0.15
+    got = ot.add_noise(2.0, [("mul_uniform", 1.0, 0.1), ("add_gaussian", 0.0, 0.1)], None, 1.5, 0.5, 0.0, 0.0, 1.0)
+    assert got == pytest.approx(2.0 * 1.05 + 0.15)
+    # the bias follows the current level with a fixed draw (observation.py:139 passes curriculum_level every step)
+    b1 = ot.add_noise(1.0, [], ("mul_uniform", 1.0, 0.2), 0.0, 0.0, 0.0, 0.5, 1.0)
+    b2 = ot.add_noise(1.0, [], ("mul_uniform", 1.0, 0.2), 0.0, 0.0, 0.0, 0.5, 0.5)
+    assert b1 == pytest.approx(1.1) and b2 == pytest.approx(1.05)
+
+
+def test_engine_reset_draws_hand_computed():
+    """ksim/engine.py:222-245 and ksim/actuators.py:219-238: ranges, level scaling and layout of the per-episode draws."""
+    nu = 2
+    u = np.array([0.5, -1.0, 1.0, 0.2, -0.2, 0.0, 0.4, 1.0, -1.0, 0.0])
+    z = np.array([9.0, 1.0, -2.0, 0.5, 0.25, -1.0, 2.0, 0.3, 0.1, -0.5])
+    out = ot.engine_reset_draws(nu, 0.5, u, z, latency_range=(1.0, 3.0), zero_offset=dict(mean=0.0, mag=0.0, std=0.02),
+                                action_bias=dict(mean=0.0, mag=0.1, std=0.0), torque_bias=dict(mean=0.5, mag=0.0, std=2.0),
+                                kp_scale=dict(mean=1.0, mag=0.2, std=0.0), kd_scale=None,
+                                torque_limit_scale=dict(mean=0.9, mag=0.0, std=0.1))
+    # latency ~ U(1 * 0.5, 3 * 0.5): u = 0.5 is three quarters of the way
+    assert out["action_latency"] == pytest.approx(0.5 + 0.75 * 1.0)
+    np.testing.assert_allclose(out["zero_offset"], [1.0 * 0.02 * 0.5, -2.0 * 0.02 * 0.5])       # scaled by the level
+    np.testing.assert_allclose(out["action"], [0.2 * 0.1, -0.2 * 0.1])                          # not scaled by the level
+    np.testing.assert_allclose(out["torque"], [0.5 - 2.0, 0.5 + 4.0])
+    assert out["kp_scale"] == pytest.approx(1.0 + 0.2) and out["kd_scale"] == pytest.approx(1.0)
+    assert out["torque_limit_scale"] == pytest.approx(0.9 - 0.05)
+    # defaults: no bias, unit scales, zero latency range gives zero latency whatever the draw
+    out = ot.engine_reset_draws(nu, 1.0, u, z, latency_range=(0.0, 0.0), zero_offset=None)
+    assert out["action_latency"] == 0.0 and not out["zero_offset"].any() and not out["action"].any()
+    assert out["kp_scale"] == 1.0 and out["torque_limit_scale"] == 1.0
+    # both zero-offset parts with one key (engine.py:117-124): the uniform part is a function of the normal draw
+    out = ot.engine_reset_draws(nu, 1.0, u, z, latency_range=(0.0, 0.0), zero_offset=dict(mean=0.0, mag=0.1, std=0.01, same_key=True))
+    np.testing.assert_allclose(out["zero_offset"], 0.01 * z[1:3] + 0.1 * ot.same_key_uniform(z[1:3]))
