@@ -78,6 +78,9 @@ def main() -> None:
     ap.add_argument("--integrator", choices=("euler", "implicitfast"), default="euler",
                     help="velocity update of the headline rollout: semi-implicit Euler (what the benchmark configs name) or "
                          "implicitfast (what ksim's RLConfig selects); the other one is reported under 'other_integrator'")
+    ap.add_argument("--only", choices=("mlp", "gae", "update", "rollout"), default=None,
+                    help="run one section alone and print its JSON (the command the counter runs under profiles/ use)")
+    ap.add_argument("--mlp-rows", type=int, default=0, help="with --only mlp: a single row count instead of 8192 and 524288")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="also launch ks_copy_f32 on 64 Mi floats once: the known-size kernel for counter calibration")
@@ -93,12 +96,25 @@ def main() -> None:
 
     _lib.load()
     assert torch.cuda.is_available(), "bench.py needs a GPU"
+    if args.only == "mlp":
+        print(json.dumps({"policy_mlp": mlp_rate(torch, rows=(args.mlp_rows,) if args.mlp_rows else (8192, 524288))}))
+        return
+    if args.only == "gae":
+        print(json.dumps({"gae": gae_bandwidth(torch, ppo)}))
+        return
+    if args.only == "update":
+        print(json.dumps({"ppo_update": ppo_update_rate(torch)}))
+        return
     N = args.envs
     T = max(1, min(args.rollout, args.steps))  # the timed region holds whole rollouts, so rewards and GAE are inside it
     head = timed_rollout(torch, args.integrator, N, T, args.steps, args.warmup)
     consts, env, ro, elapsed, kernel_ms, ndone = (head[k] for k in ("consts", "env", "ro", "elapsed", "kernel_ms", "ndone"))
     m = consts.physics_model.model
     other = "implicitfast" if args.integrator == "euler" else "euler"
+    if args.only == "rollout":  # the timed rollout alone: what the kernel-trace and counter runs of the step kernel profile
+        print(json.dumps({"value": N * args.steps / elapsed, "ms_per_step": elapsed / args.steps * 1e3,
+                          "step_kernel_ms": kernel_ms, "integrator": integrator_name(m), "num_envs": N, "rollout_length": T}))
+        return
     alt = timed_rollout(torch, other, N, T, max(T, min(args.steps, 2 * T)), min(args.warmup, T))
     other_entry = {"integrator": integrator_name(alt["consts"].physics_model.model),
                    "value": N * alt["steps"] / alt["elapsed"], "unit": "env-steps/s", "steps": alt["steps"],
@@ -131,7 +147,7 @@ def main() -> None:
 
     # GAE on rotating cfg-2 sized buffers (T=128, N=4096): larger than the caches in total
     gae = gae_bandwidth(torch, ppo)
-    mlp = mlp_rate(torch, consts)
+    mlp = mlp_rate(torch)
     upd = ppo_update_rate(torch)
 
     obs_dim = consts.terms.obs_dim
@@ -293,9 +309,22 @@ def ppo_update_rate(torch, reps=6):
                     "gradient and optimiser chain on 2048 envs x 32 steps"}
 
 
-def mlp_rate(torch, consts, reps=20):
+def mlp_rate(torch, rows=(8192, 524288), reps=20):
+    """Forward pass of the cfg 4 actor (68 -> 3 x 512 -> 20, bf16 operands, fp32 accumulate) alone, at the rollout's
+    row count and at a whole cfg 5 rollout's."""
+    import numpy as np
+
+    from ksim_amd.configs import _net
+
+    actor = _net((68, 512, 512, 512, 20), np.random.default_rng(1004), last_scale=0.1)
+
+    class _C:  # keeps the loop below reading like the rollout's call
+        pass
+
+    consts = _C()
+    consts.actor = actor
     out = {}
-    for M in (8192, 524288):
+    for M in rows:
         x = torch.randn(M, consts.actor.in_dim, device="cuda")
         y = torch.empty(M, consts.actor.out_dim, device="cuda")
         consts.actor(x, out=y)
