@@ -81,6 +81,8 @@ def main() -> None:
     ap.add_argument("--only", choices=("mlp", "gae", "update", "rollout"), default=None,
                     help="run one section alone and print its JSON (the command the counter runs under profiles/ use)")
     ap.add_argument("--mlp-rows", type=int, default=0, help="with --only mlp: a single row count instead of 8192 and 524288")
+    ap.add_argument("--streams", type=int, default=2,
+                    help="groups the envs are rolled out in, each on its own HIP stream (1: a single chain of launches)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="also launch ks_copy_f32 on 64 Mi floats once: the known-size kernel for counter calibration")
@@ -107,22 +109,30 @@ def main() -> None:
         return
     N = args.envs
     T = max(1, min(args.rollout, args.steps))  # the timed region holds whole rollouts, so rewards and GAE are inside it
-    head = timed_rollout(torch, args.integrator, N, T, args.steps, args.warmup)
-    consts, env, ro, elapsed, kernel_ms, ndone = (head[k] for k in ("consts", "env", "ro", "elapsed", "kernel_ms", "ndone"))
+    head = timed_rollout(torch, args.integrator, N, T, args.steps, args.warmup, args.streams)
+    consts, elapsed, kernel_ms, ndone = (head[k] for k in ("consts", "elapsed", "kernel_ms", "ndone"))
+    envs_per_launch = head["envs_per_launch"]
     m = consts.physics_model.model
     other = "implicitfast" if args.integrator == "euler" else "euler"
     if args.only == "rollout":  # the timed rollout alone: what the kernel-trace and counter runs of the step kernel profile
         print(json.dumps({"value": N * args.steps / elapsed, "ms_per_step": elapsed / args.steps * 1e3,
-                          "step_kernel_ms": kernel_ms, "integrator": integrator_name(m), "num_envs": N, "rollout_length": T}))
+                          "step_kernel_ms": kernel_ms, "integrator": integrator_name(m), "num_envs": N, "rollout_length": T,
+                          "streams": args.streams, "envs_per_step_launch": envs_per_launch}))
         return
-    alt = timed_rollout(torch, other, N, T, max(T, min(args.steps, 2 * T)), min(args.warmup, T))
+    del head
+    alt = timed_rollout(torch, other, N, T, max(T, min(args.steps, 2 * T)), min(args.warmup, T), args.streams)
     other_entry = {"integrator": integrator_name(alt["consts"].physics_model.model),
                    "value": N * alt["steps"] / alt["elapsed"], "unit": "env-steps/s", "steps": alt["steps"],
                    "ms_per_step": alt["elapsed"] / alt["steps"] * 1e3, "step_kernel_ms": alt["kernel_ms"]}
     del alt
 
-    # The same rollout captured once as a HIP graph and replayed: the launches leave the host out of the loop.
-    # Reported beside the headline (whose timed region keeps per-launch events for the roofline figure).
+    # The same workload as ONE chain of launches on one stream (all N envs per launch), and that chain captured once as a
+    # HIP graph and replayed, which takes the host out of the loop.
+    single = timed_rollout(torch, args.integrator, N, T, max(T, min(args.steps, 2 * T)), min(args.warmup, T), 1)
+    env, ro = single["env"], single["ro"]
+    single_entry = {"value": N * single["steps"] / single["elapsed"], "unit": "env-steps/s", "steps": single["steps"],
+                    "ms_per_step": single["elapsed"] / single["steps"] * 1e3, "step_kernel_ms": single["kernel_ms"],
+                    "envs_per_step_launch": N}
     graph = None
     if not args.traffic_probe:
         reps = max(1, args.steps // T)
@@ -152,7 +162,7 @@ def main() -> None:
 
     obs_dim = consts.terms.obs_dim
     bytes_per_env = step_algorithmic_bytes(m, obs_dim, 1 + m.nb)
-    achieved = bytes_per_env * N / (kernel_ms * 1e-3) / 1e9
+    achieved = bytes_per_env * envs_per_launch / (kernel_ms * 1e-3) / 1e9  # one launch steps the envs of one group
     traffic = None
     tpath = os.path.join(ROOT, "profiles", "step_kernel_cfg4_hbm_traffic.txt")
     if os.path.exists(tpath):  # measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, see that file
@@ -174,12 +184,15 @@ def main() -> None:
         "config": {"workload": "cfg4: K-Bot-scale biped (free root + 20 hinges, 8 foot spheres), per-env friction/mass "
                                "randomisation, obs noise 0.01, reset on z<0.5, actor+critic 3x512 bf16 MLP, "
                                f"dt=0.005 x 4 substeps, Newton 8/8, {integrator_name(m)} integration; rewards + GAE after "
-                               f"every {T} control steps inside the timed region",
+                               f"every {T} control steps inside the timed region; envs in {args.streams} independent "
+                               f"group(s), one HIP stream each",
                    "integrator": integrator_name(m), "num_envs": N, "rollout_length": T, "substeps": 4,
+                   "streams": args.streams, "envs_per_step_launch": envs_per_launch,
                    "obs_dim": obs_dim, "episodes_finished_in_last_rollout": ndone},
         "roofline": {"bound": "hbm", "kernel": "step_kernel (fused control step)", "achieved": achieved,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
                      "algorithmic_bytes_per_env_step": bytes_per_env, "kernel_ms": kernel_ms,
+                     "envs_per_launch": envs_per_launch,
                      "valu_issue_fraction_profiled": valu.get("valu_issue_fraction"),
                      "valu_insts_per_env_step_profiled": valu.get("valu_insts_per_env_step"),
                      "counters_source": "traffic and valu_* are read from the committed rocprofv3 --pmc summaries under "
@@ -187,7 +200,7 @@ def main() -> None:
                      "note": "the fused step is bound by fp32 vector-ALU issue (~1e3 flop/byte; the profiled share of "
                              "cycles with a VALU instruction issuing is given beside); the HBM fraction is reported "
                              "against the bytes the engine contract obliges a step to move"},
-        "other_integrator": other_entry,
+        "other_integrator": other_entry, "single_stream": single_entry,
         "gae": gae, "policy_mlp": mlp, "ppo_update": upd, "graph_replay": graph,
     }
     if not args.no_cpu_baseline:
@@ -195,14 +208,18 @@ def main() -> None:
     print(json.dumps(line))
 
 
-def timed_rollout(torch, integrator: str, N: int, T: int, steps: int, warmup: int) -> dict:
+def timed_rollout(torch, integrator: str, N: int, T: int, steps: int, warmup: int, streams: int = 2) -> dict:
     """`warmup` untimed control steps, then exactly `steps` timed ones of the cfg 4 rollout built with `integrator`.
-    The rollout slot restarts at 0 where the timed region begins, so it holds steps // T reward + GAE passes."""
-    from ksim_amd.configs import kbot_rollout
+    The rollout slot restarts at 0 where the timed region begins, so it holds steps // T reward + GAE passes.
+    `streams`: the N envs run as that many independent groups, each on its own HIP stream (1 = one launch chain)."""
+    from ksim_amd.configs import kbot_rollout, kbot_split_rollout
     from ksim_amd.rewards import get_rewards
 
-    consts, env, ro, _ = kbot_rollout(num_envs=N, rollout_length=T, integrator=integrator)
-    # time the dominant kernel (the fused physics control step) with events on the launch stream
+    if streams > 1:
+        consts, envs, ro = kbot_split_rollout(num_envs=N, rollout_length=T, splits=streams, integrator=integrator)
+    else:
+        consts, env, ro, _ = kbot_rollout(num_envs=N, rollout_length=T, integrator=integrator)
+    # time the dominant kernel (the fused physics control step) with events on the stream of each launch
     step_events: list = []
     orig_step = consts.engine.step
 
@@ -215,11 +232,22 @@ def timed_rollout(torch, integrator: str, N: int, T: int, steps: int, warmup: in
         return out
 
     def one_step(t: int) -> None:
-        ro.step_engine(env, t)
-        if t == T - 1:
-            rew = get_rewards(ro.trajectory(), consts.rewards, want_components=False)
-            ro.ppo_inputs(rew, 0.99, 0.95, normalize_advantages=True)
+        if streams > 1:
+            ro.step_engine(envs, t)
+            if t == T - 1:
+                rews = []
+                for part, st in zip(ro.parts, ro.streams):
+                    with torch.cuda.stream(st):
+                        rews.append(get_rewards(part.trajectory(), consts.rewards, want_components=False))
+                ro.ppo_inputs(rews, 0.99, 0.95, normalize_advantages=True)  # joins the groups for the normalisation
+        else:
+            ro.step_engine(env, t)
+            if t == T - 1:
+                rew = get_rewards(ro.trajectory(), consts.rewards, want_components=False)
+                ro.ppo_inputs(rew, 0.99, 0.95, normalize_advantages=True)
 
+    if streams > 1:
+        ro.fork()
     for k in range(warmup):
         one_step(k % T)
     consts.engine.step = timed_step
@@ -231,9 +259,13 @@ def timed_rollout(torch, integrator: str, N: int, T: int, steps: int, warmup: in
     elapsed = time.perf_counter() - t0
     consts.engine.step = orig_step
     kernel_ms = sum(a.elapsed_time(b) for a, b in step_events) / len(step_events)
-    ndone = int(ro.done.sum().item())
-    assert torch.isfinite(env.physics_state.data.qpos).all(), "non-finite state after the benchmark"
-    return dict(consts=consts, env=env, ro=ro, elapsed=elapsed, kernel_ms=kernel_ms, ndone=ndone, steps=steps)
+    parts = ro.parts if streams > 1 else [ro]
+    states = envs if streams > 1 else [env]
+    ndone = sum(int(p.done.sum().item()) for p in parts)
+    for e in states:
+        assert torch.isfinite(e.physics_state.data.qpos).all(), "non-finite state after the benchmark"
+    return dict(consts=consts, env=states[0], ro=parts[0], elapsed=elapsed, kernel_ms=kernel_ms, ndone=ndone, steps=steps,
+                envs_per_launch=N // streams)
 
 
 def gae_bandwidth(torch, ppo, reps=8):

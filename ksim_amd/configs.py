@@ -8,7 +8,7 @@ from . import actuators, engine, model as km, observation as ob, physics, random
 from . import rewards as rw, terminations as tm
 from .env_terms import EnvTerms
 from .mlp import MLP
-from .rollout import Rollout, RolloutConstants, RolloutEnvState
+from .rollout import Rollout, RolloutConstants, RolloutEnvState, SplitRollout
 
 # soft torque limits by joint class (N m): legs (hip pitch/roll/yaw, knee, ankle), arms (shoulder x3, elbow, wrist)
 KBOT_TORQUE_LIMITS = np.array([60.0, 40.0, 40.0, 60.0, 17.0] * 2 + [17.0, 17.0, 14.0, 14.0, 5.0] * 2)
@@ -26,12 +26,7 @@ def integrator_name(model) -> str:
     return "implicitfast (damping-implicit)" if model.eulerdamp else "semi-implicit Euler"
 
 
-def kbot_rollout(num_envs: int = 8192, rollout_length: int = 32, seed: int = 1004, hidden: int = 512,
-                 dtype: str = "bf16", min_height: float = 0.5, integrator: str = "euler"):
-    """K-Bot-scale biped rollout: free root + 20 hinges, 8 foot spheres, per-env friction ~U(0.4,1.2) and
-    mass scale ~U(0.9,1.1), observation noise N(0,0.01), reset on base height < `min_height`, actor and critic
-    3 x `hidden` MLPs, dt 0.005 with 4 physics substeps per control step.  `integrator`: "euler" (semi-implicit
-    Euler, what the benchmark configs name) or "implicitfast" (what ksim's RLConfig selects, ksim/task/rl.py:555-578)."""
+def _kbot_constants(seed: int, hidden: int, dtype: str, min_height: float, integrator: str):
     m = km.kbot_scale_model(seed=seed, integrator=integrator)
     rng = np.random.default_rng(seed)
     kps = rng.uniform(20.0, 150.0, m.nu)
@@ -58,14 +53,38 @@ def kbot_rollout(num_envs: int = 8192, rollout_length: int = 32, seed: int = 100
                "upright": rw.UprightReward(scale=0.2), "action_velocity": rw.ActionVelocityPenalty(scale=0.01)}
     consts = RolloutConstants(physics_model=dm, engine=eng, terms=terms, rewards=rewards, actor=actor, critic=critic,
                               log_std=torch.full((m.nu,), -2.0, device=dev))
+    return m, consts, dict(kps=kps, kds=kds, clip=KBOT_TORQUE_LIMITS)
+
+
+def _kbot_env_state(m, consts, num_envs: int, seed: int) -> RolloutEnvState:
+    dev = torch.device("cuda")
     gen = torch.Generator(device=dev)
     gen.manual_seed(seed)
     randomization = rnd.get_physics_randomizers(
         m, {"floor_friction": rnd.FloorFrictionRandomizer(0.4, 1.2),
             "mass": rnd.AllBodiesMassMultiplicationRandomizer(0.9, 1.1)}, num_envs, gen)
-    ps = eng.reset(dm, 1.0, gen, num_envs, randomization)
-    env = RolloutEnvState(ps, randomization, torch.zeros(num_envs, 2, device=dev), None, seed=seed)
-    return consts, env, Rollout(consts, num_envs, rollout_length), dict(kps=kps, kds=kds, clip=KBOT_TORQUE_LIMITS)
+    ps = consts.engine.reset(consts.physics_model, 1.0, gen, num_envs, randomization)
+    return RolloutEnvState(ps, randomization, torch.zeros(num_envs, 2, device=dev), None, seed=seed)
+
+
+def kbot_rollout(num_envs: int = 8192, rollout_length: int = 32, seed: int = 1004, hidden: int = 512,
+                 dtype: str = "bf16", min_height: float = 0.5, integrator: str = "euler"):
+    """K-Bot-scale biped rollout: free root + 20 hinges, 8 foot spheres, per-env friction ~U(0.4,1.2) and
+    mass scale ~U(0.9,1.1), observation noise N(0,0.01), reset on base height < `min_height`, actor and critic
+    3 x `hidden` MLPs, dt 0.005 with 4 physics substeps per control step.  `integrator`: "euler" (semi-implicit
+    Euler, what the benchmark configs name) or "implicitfast" (what ksim's RLConfig selects, ksim/task/rl.py:555-578)."""
+    m, consts, gains = _kbot_constants(seed, hidden, dtype, min_height, integrator)
+    env = _kbot_env_state(m, consts, num_envs, seed)
+    return consts, env, Rollout(consts, num_envs, rollout_length), gains
+
+
+def kbot_split_rollout(num_envs: int = 8192, rollout_length: int = 32, splits: int = 2, seed: int = 1004, hidden: int = 512,
+                       dtype: str = "bf16", min_height: float = 0.5, integrator: str = "euler"):
+    """The same workload with the envs in `splits` groups on separate streams (`SplitRollout`): returns the constants,
+    one env state per group (seeded seed, seed + 1, ...) and the split rollout."""
+    m, consts, _ = _kbot_constants(seed, hidden, dtype, min_height, integrator)
+    envs = [_kbot_env_state(m, consts, num_envs // splits, seed + g) for g in range(splits)]
+    return consts, envs, SplitRollout(consts, num_envs, rollout_length, splits)
 
 
 def step_algorithmic_bytes(m, obs_dim: int, per_env_params: int) -> int:

@@ -47,7 +47,7 @@ class MLP:
         self._lib = lib
         self._handle = ctypes.c_void_p()
         _lib.check(lib.ks_mlp_create(ctypes.byref(d), ctypes.byref(self._handle)))
-        self._ws: torch.Tensor | None = None
+        self._ws: dict | None = None
 
     @property
     def in_dim(self) -> int:
@@ -61,10 +61,16 @@ class MLP:
         return 2 * sum(a * b for a, b in zip(self.dims[:-1], self.dims[1:]))
 
     def workspace(self, M: int, device) -> torch.Tensor:
+        """Scratch of the per-layer path, one buffer per stream: calls on different streams may overlap on the GPU."""
         need = int(self._lib.ks_mlp_workspace_bytes(self._handle, M))
-        if self._ws is None or self._ws.numel() < need or self._ws.device != torch.device(device):
-            self._ws = torch.empty(need, dtype=torch.uint8, device=device)
-        return self._ws
+        key = torch.cuda.current_stream().cuda_stream if need else 0
+        if self._ws is None:
+            self._ws = {}
+        ws = self._ws.get(key)
+        if ws is None or ws.numel() < need or ws.device != torch.device(device):
+            ws = torch.empty(need, dtype=torch.uint8, device=device)
+            self._ws[key] = ws
+        return ws
 
     def __call__(self, x: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
         _lib.require_cuda(x, dtype=torch.float32)

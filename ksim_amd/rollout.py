@@ -283,3 +283,96 @@ class Rollout:
             raise _lib.KsError("a critic is required for GAE")
         return ppo_mod.compute_ppo_inputs(self.values.view(self.T, self.N), rewards.total, self.done, self.success,
                                           gamma, lam, normalize_advantages=normalize_advantages, time_major=True)
+
+
+_STREAMS: list = []
+
+
+def _group_streams(n: int) -> list:
+    """One pool of side streams for every SplitRollout of the process: a process has few hardware queues (4 by default),
+    and streams beyond them share a queue, which serialises launches that were meant to overlap."""
+    while len(_STREAMS) < n:
+        _STREAMS.append(torch.cuda.Stream())
+    return _STREAMS[:n]
+
+
+class SplitRollout:
+    """The same rollout with the N envs cut into `splits` independent groups, each on its own HIP stream.
+
+    No counterpart in the reference, whose vmapped step runs all envs in lock step.  Here a control step is a chain of
+    launches whose longest one, the fused physics step, ends with its slowest env, and the short launches around it
+    (observation, networks, termination, reset pass) cannot fill the GPU on their own.  With two groups in flight the tail
+    of one group's physics launch and its short launches overlap the other group's physics launch.  Envs never interact
+    inside a rollout, so every env's trajectory is what the single-stream `Rollout` gives it for the same draws; only
+    advantage normalisation spans the groups (`ppo_inputs`).  Streams are created at the default priority.
+    """
+
+    def __init__(self, constants: RolloutConstants, num_envs: int, rollout_length: int, splits: int = 2):
+        if splits < 1 or num_envs % splits:
+            raise _lib.KsError("the env count must be a multiple of the number of groups")
+        if any(isinstance(n, RecurrentNetwork) for n in (constants.actor, constants.critic)):
+            raise _lib.KsError("recurrent networks keep one workspace per cell: roll them out on a single stream")
+        self.c, self.N, self.T, self.splits = constants, int(num_envs), int(rollout_length), int(splits)
+        self.parts = [Rollout(constants, num_envs // splits, rollout_length) for _ in range(splits)]
+        self.streams = _group_streams(splits)
+        dev = torch.device("cuda")
+        n = self.N // splits
+        # GAE outputs of all groups side by side, so that advantage normalisation can run over their union
+        self._gae = torch.empty(splits, self.T, n, dtype=torch.float32, device=dev)
+        self._ret = torch.empty_like(self._gae)
+        self._tgt = torch.empty_like(self._gae)
+        self._adv = torch.empty_like(self._gae)
+        self._ws = torch.empty(_lib.KS_REDUCE_WORKSPACE_BYTES, dtype=torch.uint8, device=dev)
+
+    def fork(self) -> None:
+        """The groups' streams wait for what the current stream has queued so far."""
+        cur = torch.cuda.current_stream()
+        for st in self.streams:
+            st.wait_stream(cur)
+
+    def join(self) -> None:
+        """The current stream waits for the groups."""
+        cur = torch.cuda.current_stream()
+        for st in self.streams:
+            cur.wait_stream(st)
+
+    def step_engine(self, envs: Sequence[RolloutEnvState], t: int, level: float = 1.0,
+                    noise: Sequence[Mapping | None] | None = None) -> None:
+        """One control step of every group (no synchronisation: bracket a run of steps with `fork` and `join`)."""
+        for g, (ro, env, st) in enumerate(zip(self.parts, envs, self.streams)):
+            with torch.cuda.stream(st):
+                ro.step_engine(env, t, level, noise[g] if noise is not None else None)
+
+    def unroll(self, envs: Sequence[RolloutEnvState], level: float = 1.0) -> list[tuple[Trajectory, RewardState]]:
+        """T control steps and the reward pass of every group; returns one (trajectory, rewards) per group."""
+        self.fork()
+        for t in range(self.T):
+            self.step_engine(envs, t, level)
+        out = []
+        for ro, env, st in zip(self.parts, envs, self.streams):
+            with torch.cuda.stream(st):
+                traj = ro.trajectory()
+                out.append((traj, ro._rewards(traj, env, level)))
+        self.join()
+        return out
+
+    def ppo_inputs(self, rewards: Sequence[RewardState], gamma: float, lam: float, normalize_advantages: bool = True):
+        """GAE / returns per group (ksim/task/ppo.py:54-121) with the advantages normalised over ALL envs, as one
+        rollout of N envs has them (ppo.py:116-119).  Returns one PPOInputs per group (views of shared buffers)."""
+        lib = _lib.load()
+        self.fork()
+        for g, (ro, rew, st) in enumerate(zip(self.parts, rewards, self.streams)):
+            if ro.values is None:
+                raise _lib.KsError("a critic is required for GAE")
+            with torch.cuda.stream(st):
+                _lib.check(lib.ks_gae_tn(_lib.current_stream(), ro.T, ro.N, _lib.ptr(ro.values), _lib.ptr(rew.total),
+                                         _lib.ptr(ro.done), _lib.ptr(ro.success), float(gamma), float(lam), 0,
+                                         _lib.ptr(self._gae[g]), _lib.ptr(self._ret[g]), _lib.ptr(self._tgt[g])))
+        self.join()
+        adv = self._gae
+        if normalize_advantages:
+            _lib.check(lib.ks_normalize_advantages(_lib.current_stream(), self._gae.numel(), _lib.ptr(self._gae),
+                                                   _lib.ptr(self._adv), _lib.ptr(self._ws)))
+            adv = self._adv
+        return [ppo_mod.PPOInputs(advantages_bt=adv[g], value_targets_bt=self._tgt[g], gae_bt=self._gae[g],
+                                  returns_bt=self._ret[g]) for g in range(self.splits)]

@@ -538,3 +538,66 @@ def test_recurrent_policy_update_from_a_rollout(head):
     # the rollout goes on with the updated networks
     traj2, _ = ro.unroll(env)
     assert torch.isfinite(traj2.action).all() and torch.isfinite(ro.values).all()
+
+
+def test_split_rollout_equals_single_stream_rollout():
+    """Two groups of envs on two streams give every env, bit for bit, the trajectory the single-stream rollout gives it
+    for the same draws (resets and per-episode re-draws included); advantage normalisation spans both groups."""
+    from ksim_amd.rollout import SplitRollout
+
+    N, T, G = 64, 6, 2
+    m, c, rnd_, _, ro, EnvState = build(N, T, seed=5, min_height=0.9, sim2real=True)
+    rng = np.random.default_rng(17)
+    K, nu, ned, n = c.terms.obs_dim, m.nu, 3 * m.nu + 4, N // G
+    u0 = t32(rng.uniform(-1, 1, (N, m.nq + 1)))
+    eu, ez = t32(rng.uniform(-1, 1, (N, ned))), t32(rng.normal(size=(N, ned)))
+    cmd = t32(rng.normal(size=(N, 2)))
+    sl = [slice(g * n, (g + 1) * n) for g in range(G)]
+    cut = lambda x, g: x[sl[g]].contiguous()  # noqa: E731
+
+    def start(rows, rnd_rows):
+        ps = c.engine.reset(c.physics_model, 1.0, 0, rows.stop - rows.start, rnd_rows, reset_uniform=u0[rows].contiguous(),
+                            episode_draws=dict(uniform=eu[rows].contiguous(), normal=ez[rows].contiguous()))
+        low = (torch.arange(rows.start, rows.stop, device=DEV) % 3) == 0  # these start below the termination height
+        ps.data.qpos[low, 2] = 0.87
+        return EnvState(ps, rnd_rows, cmd[rows].contiguous(), None, seed=1)
+
+    env = start(slice(0, N), rnd_)
+    envs = [start(sl[g], {k: cut(v, g) for k, v in rnd_.items()}) for g in range(G)]
+    sro = SplitRollout(c, N, T, splits=G)
+    sro.fork()
+    for t in range(T):
+        noise = dict(obs_normal=t32(rng.normal(size=(N, K))), obs_uniform=t32(rng.random((N, K))),
+                     action_normal=t32(rng.normal(size=(N, nu))), reset_uniform=t32(rng.uniform(-1, 1, (N, m.nq + 1))),
+                     obs_bias_redraw=t32(np.stack([rng.normal(size=(N, K)), rng.uniform(-1, 1, (N, K))], -1)),
+                     episode=dict(uniform=t32(rng.uniform(-1, 1, (N, ned))), normal=t32(rng.normal(size=(N, ned)))))
+        ro.step_engine(env, t, 1.0, noise)
+        parts = [{k: ({kk: cut(vv, g) for kk, vv in v.items()} if isinstance(v, dict) else cut(v, g)) for k, v in noise.items()}
+                 for g in range(G)]
+        torch.cuda.synchronize()  # the per-group copies above were made on the current stream
+        sro.step_engine(envs, t, 1.0, parts)
+    sro.join()
+    torch.cuda.synchronize()
+    assert int(ro.done.sum().item()) > 0, "no env was reset: the reset path was not compared"
+    for name in ("qpos", "qvel", "xpos", "xquat", "ctrl", "action", "obs", "noisy_obs", "done", "success", "timestep", "values"):
+        whole = getattr(ro, name)
+        joined = torch.cat([getattr(p, name) for p in sro.parts], dim=1)
+        assert torch.equal(whole, joined), name
+    for name in ("action_latency", "zero_offset"):
+        assert torch.equal(getattr(env.physics_state, name), torch.cat([getattr(e.physics_state, name) for e in envs])), name
+    assert torch.equal(env.physics_state.data.qpos, torch.cat([e.physics_state.data.qpos for e in envs]))
+    assert torch.equal(env.obs_bias, torch.cat([e.obs_bias for e in envs]))
+    # rewards and GAE per group; normalised advantages over the union of the groups
+    from ksim_amd.rewards import get_rewards
+    rew = get_rewards(ro.trajectory(), c.rewards)
+    rews = [get_rewards(p.trajectory(), c.rewards) for p in sro.parts]
+    assert torch.equal(rew.total, torch.cat([r.total for r in rews], dim=1))
+    whole = ro.ppo_inputs(rew, 0.99, 0.95, normalize_advantages=True)
+    split = sro.ppo_inputs(rews, 0.99, 0.95, normalize_advantages=True)
+    torch.cuda.synchronize()
+    assert torch.equal(whole.gae_bt, torch.cat([s.gae_bt for s in split], dim=1))
+    assert torch.equal(whole.value_targets_bt, torch.cat([s.value_targets_bt for s in split], dim=1))
+    np.testing.assert_allclose(torch.cat([s.advantages_bt for s in split], dim=1).cpu().numpy(), whole.advantages_bt.cpu().numpy(),
+                               rtol=2e-6, atol=2e-6)
+    with pytest.raises(Exception, match="multiple"):
+        SplitRollout(c, 63, T, splits=2)

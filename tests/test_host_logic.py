@@ -386,6 +386,6 @@ def test_benchmark_workload_label_follows_the_model_flag():
     src = open(os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "bench.py")).read()
     # no hard-coded integrator in the workload text, and both legs take the same argument
     assert "integrator_name(m)" in src and not re.search(r'"[^"\n]*implicitfast \(damping', src)
-    assert "cpu_baseline(args.integrator)" in src and "timed_rollout(torch, args.integrator" in src
+    assert "cpu_baseline(args.integrator)" in src and "timed_rollout(torch, args.integrator, N, T, args.steps, args.warmup, args.streams)" in src
     src_cfg = open(os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "ksim_amd", "configs.py")).read()
     assert "kbot_scale_model(seed=seed, integrator=integrator)" in src_cfg
