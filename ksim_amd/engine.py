@@ -241,15 +241,19 @@ class HipEngine(PhysicsEngine):
                                   reset_uniform=reset_uniform, episode=self.episode_args(state, episode_draws))
         self.forward(physics_model, state, mask, randomization)
 
-    def forward(self, physics_model, state: PhysicsState, mask=None, randomization=None) -> None:
+    def forward(self, physics_model, state: PhysicsState, mask=None, randomization=None, live=None) -> None:
+        """`live`: names of the derived fields of `state.data` to refresh (None = all of them); a rollout whose terms read
+        none of a field leaves it out, and the field then holds stale values."""
         d = state.data
         rnd = randomization or {}
+        keep = (lambda name, buf: buf) if live is None else (lambda name, buf: buf if name in live else None)
         physics.forward(physics_model, dict(qpos=d.qpos, qvel=d.qvel, qacc_warmstart=d.qacc_warmstart, env_mask=mask,
                                             friction=rnd.get("friction"), mass_scale=rnd.get("mass_scale"),
                                             armature_scale=rnd.get("armature_scale"), damping_scale=rnd.get("damping_scale"),
                                             **{k: rnd.get(k) for k in _MODEL_FIELD_OVERRIDES},
-                                            xpos=d.xpos, xquat=d.xquat, cvel=d.cvel, contact_dist=d.contact_dist,
-                                            cinert=d.cinert, cfrc_ext=d.cfrc_ext))
+                                            xpos=keep("xpos", d.xpos), xquat=keep("xquat", d.xquat), cvel=keep("cvel", d.cvel),
+                                            contact_dist=keep("contact_dist", d.contact_dist),
+                                            cinert=keep("cinert", d.cinert), cfrc_ext=keep("cfrc_ext", d.cfrc_ext)))
         # engine.py:217-220: qvel and qacc are zeroed after the forward pass (qvel is already zero here)
 
     def prepare_state(self, state: PhysicsState):
@@ -281,9 +285,13 @@ class HipEngine(PhysicsEngine):
              noise: Mapping[str, torch.Tensor] | None = None,
              record: Mapping[str, torch.Tensor] | None = None, want_cvel: bool = True, want_cinert: bool = False,
              want_cfrc_ext: bool = False,
-             step: int = 0, step_base=None, event_seed: int = 0) -> PhysicsState:
+             step: int = 0, step_base=None, event_seed: int = 0, live=None) -> PhysicsState:
+        """`live`: names among qacc, ctrl, xpos, xquat, contact_dist of the derived fields of `physics_state.data` that
+        the caller reads afterwards (None = all).  The rollout records ctrl / xpos / xquat into its own slot through
+        `record`, so a task whose observations read none of them need not have them written twice."""
         m, d, s = physics_model.model, physics_state.data, physics_state
         rnd, noise, record = randomization or {}, noise or {}, record or {}
+        keep = (lambda name, b: b) if live is None else (lambda name, b: b if name in live else None)
         drop = noise.get("drop")
         p_drop = self.data.drop_action_prob * float(curriculum_level)
         if drop is None and p_drop > 0:  # engine.py:277-278
@@ -292,8 +300,10 @@ class HipEngine(PhysicsEngine):
         buf = dict(qpos=d.qpos, qvel=d.qvel, qacc_warmstart=d.qacc_warmstart, time=d.time, last_ctrl=s.last_ctrl,
                    action=action, latency=s.action_latency, zero_offset=s.zero_offset, drop=drop,
                    friction=rnd.get("friction"), mass_scale=rnd.get("mass_scale"), armature_scale=rnd.get("armature_scale"),
-                   damping_scale=rnd.get("damping_scale"), **{k: rnd.get(k) for k in _MODEL_FIELD_OVERRIDES}, qacc=d.qacc, ctrl_out=d.ctrl,
-                   xpos=d.xpos, xquat=d.xquat, cvel=d.cvel if want_cvel else None, contact_dist=d.contact_dist,
+                   damping_scale=rnd.get("damping_scale"), **{k: rnd.get(k) for k in _MODEL_FIELD_OVERRIDES},
+                   qacc=keep("qacc", d.qacc), ctrl_out=keep("ctrl", d.ctrl),
+                   xpos=keep("xpos", d.xpos), xquat=keep("xquat", d.xquat), cvel=d.cvel if want_cvel else None,
+                   contact_dist=keep("contact_dist", d.contact_dist),
                    cinert=d.cinert if want_cinert else None, cfrc_ext=d.cfrc_ext if want_cfrc_ext else None,
                    action_noise=noise.get("action_noise"),
                    torque_noise=noise.get("torque_noise"), traj_ctrl=record.get("ctrl"),

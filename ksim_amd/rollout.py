@@ -117,6 +117,13 @@ class Rollout:
         # Philox step counter of graph replays: kernels add it to the step baked into the captured launch
         self.step_base = torch.zeros(1, dtype=torch.int64, device=dev)
         self._graph = None
+        # derived fields of the live physics data that the task's terms read: the others are recorded into the rollout
+        # slot only (the step kernel would otherwise write xpos / xquat / ctrl twice per control step)
+        used = c.terms.sources_used
+        need = {T.SRC_QACC: "qacc", T.SRC_CTRL: "ctrl", T.SRC_XPOS: "xpos", T.SRC_XQUAT: "xquat", T.SRC_CVEL: "cvel",
+                T.SRC_CONTACT_DIST: "contact_dist", T.SRC_CINERT: "cinert", T.SRC_CFRC_EXT: "cfrc_ext"}
+        self._live = {name for src, name in need.items() if src in used}
+        self._live.add("contact_dist")  # a few floats per env, also read by the illegal-contact termination
         if c.actor.in_dim != c.terms.obs_dim or c.actor.out_dim != self.mean.shape[1]:
             raise _lib.KsError("actor must map the observation vector to one mean per action entry (or to what its head takes)")
         if c.critic is not None and (c.critic.in_dim != c.terms.obs_dim or c.critic.out_dim != 1):
@@ -178,7 +185,8 @@ class Rollout:
         c.engine.step(self.action[t], c.physics_model, ps, level, env.seed + env.step, env.randomization_dict,
                       noise=noise.get("engine"), record=dict(ctrl=self.ctrl[t], xpos=self.xpos[t], xquat=self.xquat[t]),
                       want_cvel=T.SRC_CVEL in c.terms.sources_used, want_cinert=T.SRC_CINERT in c.terms.sources_used,
-                      want_cfrc_ext=T.SRC_CFRC_EXT in c.terms.sources_used, step=step, step_base=step_base, event_seed=env.seed)
+                      want_cfrc_ext=T.SRC_CFRC_EXT in c.terms.sources_used, step=step, step_base=step_base, event_seed=env.seed,
+                      live=self._live)
         ev_buf = ps.event_states.get("_buffer") if ps.event_states else None
         st = dict(qpos=d.qpos, qvel=d.qvel, qacc_warmstart=d.qacc_warmstart, time=d.time, last_ctrl=ps.last_ctrl)
         c.terms.terminate_reset(st, level=level, components=self.components[t][: c.terms.n_terms] if c.terms.n_terms else None,
@@ -189,9 +197,9 @@ class Rollout:
                                 event_intervals=[ev.interval_range for ev in c.engine.events.values()],
                                 event_reset_uniform=noise.get("event_reset_uniform"),
                                 event_force=ps.event_states.get("_force_buffer") if ps.event_states else None,
-                                contact_dist=d.contact_dist, episode=c.engine.episode_args(ps, noise.get("episode")))
+                                contact_dist=d.contact_dist if "contact_dist" in self._live else None, episode=c.engine.episode_args(ps, noise.get("episode")))
         # refresh the derived fields and the warm start of the reset envs (engine.py:213)
-        c.engine.forward(c.physics_model, ps, self.reset_mask, env.randomization_dict)
+        c.engine.forward(c.physics_model, ps, self.reset_mask, env.randomization_dict, live=self._live)
         if c.commands is not None:  # record the commands this step ran under, then advance them (rl.py:1082-1098)
             c.commands.update(env.commands, d.qpos, d.qvel, level=level, fresh=self.reset_mask, record=self.command[t],
                               uniform=noise.get("command_uniform"), seed=env.seed, step=step, step_base=step_base)
