@@ -87,6 +87,60 @@ def kbot_split_rollout(num_envs: int = 8192, rollout_length: int = 32, splits: i
     return consts, envs, SplitRollout(consts, num_envs, rollout_length, splits)
 
 
+def humanoid_rollout(num_envs: int = 4096, rollout_length: int = 16, seed: int = 1003, min_height: float = 0.6):
+    """Benchmark config 3: free root + 21 hinges in a 5-limb tree, 4 foot spheres, friction 1.0, 21 PD actuators, root height
+    1.3 m, joints ~U(-0.1, 0.1), dt 0.005 with 4 substeps, fp32 actor 71 -> 3 x 256 (ELU) -> 21 means."""
+    m = km.humanoid_model(seed=seed)
+    rng = np.random.default_rng(seed)
+    act = actuators.PositionActuators(kps=tuple(rng.uniform(20.0, 150.0, m.nu)), kds=tuple(rng.uniform(0.5, 1.5, m.nu)))
+    resets = [rs.RandomJointPositionReset(scale=0.1, scale_by_curriculum=False)]
+    eng = engine.get_physics_engine("hip", resets, {}, act, engine.EngineConfig(dt=0.005, ctrl_dt=0.02))
+    observations = {
+        "joint_position": ob.JointPositionObservation(), "joint_velocity": ob.JointVelocityObservation(),
+        "projected_gravity": ob.ProjectedGravityObservation(),
+        "base_angular_velocity": ob.BaseAngularVelocityObservation(in_robot_frame=True),
+        "last_action": ob.LastActionObservation(), "command": ob.CommandObservation(),
+    }
+    terms = EnvTerms(m, observations, {"minimum_height": tm.MinimumHeightTermination(min_height)}, resets, command_dim=2)
+    assert terms.obs_dim == 71
+    dm = physics.DeviceModel(m)
+    dev = torch.device("cuda")
+    actor = _net((71, 256, 256, 256, m.nu), rng, last_scale=0.1, dtype="f32")
+    critic = _net((71, 256, 256, 256, 1), rng, dtype="f32")
+    rewards = {"stay_alive": rw.StayAliveReward(scale=1.0), "upright": rw.UprightReward(scale=0.2)}
+    consts = RolloutConstants(physics_model=dm, engine=eng, terms=terms, rewards=rewards, actor=actor, critic=critic,
+                              log_std=torch.full((m.nu,), -2.0, device=dev))
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(seed)
+    ps = eng.reset(dm, 1.0, gen, num_envs, {})
+    ps.data.qpos[:, 2] = 1.3
+    eng.forward(dm, ps)
+    env = RolloutEnvState(ps, {}, torch.zeros(num_envs, 2, device=dev), None, seed=seed)
+    return consts, env, Rollout(consts, num_envs, rollout_length)
+
+
+def kbot_ppo_iteration(num_envs: int = 16384, rollout_length: int = 32, seed: int = 1005, batch_size: int = 2048,
+                       num_passes: int = 4, integrator: str = "euler"):
+    """Benchmark config 5: the K-Bot-scale rollout with T = 32, then `num_passes` epochs of minibatch steps of the bf16 actor
+    and critic, and an AMP-style discriminator 71 -> 2 x 256 -> 1 scoring the trajectory's motion frames against seeded
+    reference-motion frames ~N(0, 1).  Returns what `train_step.rl_train_loop_step` takes."""
+    from .amp import AMPConfig, DiscriminatorUpdate
+    from .ppo_update import GaussianMlpPolicy, PPOUpdateConfig
+    from .train_step import AMPSetup
+
+    m, consts, _ = _kbot_constants(seed, 512, "bf16", 0.5, integrator)
+    consts.rewards = dict(consts.rewards, amp=rw.AMPReward(scale=0.5))
+    env = _kbot_env_state(m, consts, num_envs, seed)
+    rng = np.random.default_rng(seed)
+    frame = (m.nq - 2) + m.nv + m.nu
+    disc = _net((frame, 256, 256, 1), rng, dtype="bf16")
+    real = torch.from_numpy(rng.normal(size=(64, rollout_length, frame)).astype(np.float32)).cuda()
+    setup = AMPSetup(update=DiscriminatorUpdate(disc, AMPConfig(amp_reference_batch_size=32, disc_num_passes=1)), real_motions=real)
+    policy = GaussianMlpPolicy(actor=consts.actor, critic=consts.critic, log_std=consts.log_std)
+    cfg = PPOUpdateConfig(num_passes=num_passes, batch_size=batch_size)
+    return consts, env, Rollout(consts, num_envs, rollout_length), policy, cfg, setup
+
+
 def step_algorithmic_bytes(m, obs_dim: int, per_env_params: int) -> int:
     """Bytes one fused control step is obliged to move per env: state in/out, transition record, observation."""
     return 4 * (2 * m.nq + 4 * m.nv + 3 * m.nu + 1 + 7 * m.nb + obs_dim + per_env_params) + 2

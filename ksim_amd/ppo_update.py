@@ -130,10 +130,13 @@ def single_step(policy: GaussianMlpPolicy, cfg: PPOUpdateConfig, actor_obs, crit
 
 
 def update_model(policy: GaussianMlpPolicy, cfg: PPOUpdateConfig, actor_obs, critic_obs, action, rewards, done, success,
-                 permutations: list[torch.Tensor] | None = None, seed: int = 0) -> list[dict]:
+                 permutations: list[torch.Tensor] | None = None, seed: int = 0, after_step=None) -> list[dict]:
     """num_passes x (N / batch_size) minibatch steps over a (T, N) rollout (ppo.py:572-694).
 
-    `permutations` (one index vector per pass) replaces the reference's `jax.random.permutation`."""
+    `permutations` (one index vector per pass) replaces the reference's `jax.random.permutation`.  `after_step(idx)`,
+    when given, runs after every minibatch step with the env indices of that minibatch: the hook through which the AMP
+    task's `_single_step` appends its discriminator passes (ksim/task/amp.py:455-545); what it returns is stored in the
+    step's metrics under "after_step"."""
     Tn, N = done.shape
     if policy._m1 is None:
         policy.train_init()
@@ -156,6 +159,8 @@ def update_model(policy: GaussianMlpPolicy, cfg: PPOUpdateConfig, actor_obs, cri
             sel = lambda t: t.index_select(1, idx).contiguous()  # noqa: E731
             out.append(single_step(policy, cfg, sel(actor_obs), sel(critic_obs), sel(action), sel(rewards), sel(done),
                                    sel(success), sel(on_lp), sel(on_v)))
+            if after_step is not None:
+                out[-1]["after_step"] = after_step(idx)
     return out
 
 
