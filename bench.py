@@ -78,7 +78,7 @@ def main() -> None:
     ap.add_argument("--integrator", choices=("euler", "implicitfast"), default="euler",
                     help="velocity update of the headline rollout: semi-implicit Euler (what the benchmark configs name) or "
                          "implicitfast (what ksim's RLConfig selects); the other one is reported under 'other_integrator'")
-    ap.add_argument("--only", choices=("mlp", "gae", "update", "rollout"), default=None,
+    ap.add_argument("--only", choices=("mlp", "gae", "update", "rollout", "iteration"), default=None,
                     help="run one section alone and print its JSON (the command the counter runs under profiles/ use)")
     ap.add_argument("--mlp-rows", type=int, default=0, help="with --only mlp: a single row count instead of 8192 and 524288")
     ap.add_argument("--streams", type=int, default=2,
@@ -106,6 +106,9 @@ def main() -> None:
         return
     if args.only == "update":
         print(json.dumps({"ppo_update": ppo_update_rate(torch)}))
+        return
+    if args.only == "iteration":
+        print(json.dumps({"ppo_iteration": ppo_iteration_rate(torch)}))
         return
     N = args.envs
     T = max(1, min(args.rollout, args.steps))  # the timed region holds whole rollouts, so rewards and GAE are inside it
@@ -159,6 +162,7 @@ def main() -> None:
     gae = gae_bandwidth(torch, ppo)
     mlp = mlp_rate(torch)
     upd = ppo_update_rate(torch)
+    iteration = ppo_iteration_rate(torch)
 
     obs_dim = consts.terms.obs_dim
     bytes_per_env = step_algorithmic_bytes(m, obs_dim, 1 + m.nb)
@@ -201,7 +205,7 @@ def main() -> None:
                              "cycles with a VALU instruction issuing is given beside); the HBM fraction is reported "
                              "against the bytes the engine contract obliges a step to move"},
         "other_integrator": other_entry, "single_stream": single_entry,
-        "gae": gae, "policy_mlp": mlp, "ppo_update": upd, "graph_replay": graph,
+        "gae": gae, "policy_mlp": mlp, "ppo_update": upd, "ppo_iteration": iteration, "graph_replay": graph,
     }
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(args.integrator)
@@ -339,6 +343,41 @@ def ppo_update_rate(torch, reps=6):
             "mfma_utilisation": flops / ms / 1e9 / (BF16_PEAK_TFLOPS),
             "what": "forward + backward (3x the forward flops) of actor and critic 68-3x512-{20,1} bf16, GAE, loss "
                     "gradient and optimiser chain on 2048 envs x 32 steps"}
+
+
+def ppo_iteration_rate(torch, reps=3):
+    """Whole training iterations at benchmark config 5's size: a 16384-env x 32-step rollout, discriminator scoring of the
+    trajectory's motion frames, rewards with the AMP term, GAE and the on-policy pass, then 4 passes x 8 minibatches of
+    2048 envs of actor / critic forward + backward + optimiser, with a discriminator step after each."""
+    from ksim_amd.configs import kbot_ppo_iteration
+    from ksim_amd.train_step import rl_train_loop_step
+
+    consts, env, ro, policy, cfg, setup = kbot_ppo_iteration()
+    gen = torch.Generator().manual_seed(0)
+    rl_train_loop_step(ro, env, policy, cfg, amp=setup, generator=gen)  # warm-up: workspaces, optimiser state
+    torch.cuda.synchronize()
+    parts = {"rollout": 0.0, "update": 0.0}
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        out = rl_train_loop_step(ro, env, policy, cfg, amp=setup, generator=gen)
+    torch.cuda.synchronize()
+    elapsed = (time.perf_counter() - t0) / reps
+    assert torch.isfinite(out["rewards"].total).all() and torch.isfinite(policy.log_std).all()
+    # the rollout's share, timed alone on the same state
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for t in range(ro.T):
+        ro.step_engine(env, t, 1.0, None)
+    torch.cuda.synchronize()
+    parts["rollout"] = time.perf_counter() - t0
+    parts["update"] = elapsed - parts["rollout"]
+    n = ro.N * ro.T
+    return {"num_envs": ro.N, "rollout_length": ro.T, "transitions": n, "num_passes": cfg.num_passes,
+            "minibatch_envs": cfg.batch_size, "minibatch_steps": len(out["steps"]), "discriminator": setup.disc.dims,
+            "s_per_iteration": elapsed, "transitions_per_s": n / elapsed, "iterations_per_s": 1.0 / elapsed,
+            "rollout_s": parts["rollout"], "postprocess_and_update_s": parts["update"],
+            "what": "one rl_train_loop_step: rollout, discriminator scoring, rewards + GAE, 32 actor/critic minibatch steps "
+                    "(bf16 3x512) each followed by a discriminator step (71-256-256-1); host wall-clock per iteration"}
 
 
 def mlp_rate(torch, rows=(8192, 524288), reps=20):
