@@ -1,10 +1,18 @@
 /* ksim_hip.h — C ABI of libksimhip.so: the MI355X (gfx950) rollout hot path of ksim.
  *
- * Every entry point is asynchronous on the caller's HIP stream, allocates nothing,
- * never synchronises the host, keeps no mutable global state (re-entrant) and
- * returns 0 on success or a negative KS_E* code; ks_last_error() gives the
+ * Compute entry points are asynchronous on the caller's HIP stream, allocate nothing,
+ * never synchronise the host, keep no mutable global state (re-entrant) and
+ * return 0 on success or a negative KS_E* code; ks_last_error() gives the
  * calling thread's last message.  All pointers are DEVICE pointers unless a
  * parameter says "host".  The caller owns every buffer.
+ *
+ * The set-up calls are the exception, and the only ones that allocate device memory
+ * and block the host (uploads, one stream synchronisation in ks_mlp_train_init):
+ *   ks_model_create, ks_terms_create, ks_mlp_create, ks_gru_create, ks_lstm_create   (tables and weights of a handle)
+ *   ks_mlp_train_init, ks_gru_train_init, ks_lstm_train_init   (master weights, gradients, Adam moments, transposes)
+ * Their memory belongs to the handle and is released by the matching *_destroy; a set-up call that fails releases
+ * what it had allocated.  Call them outside graph capture and outside timed loops.  Gradients and optimiser state
+ * live in the handle, so two streams must not train one handle at once.
  *
  * Each declaration cites the reference (kscalelabs/ksim 0.2.10) interface it
  * replaces as file:line.
@@ -85,6 +93,7 @@ typedef struct KsPpoLossParams {
   float log_clip_value;  /* 5.0 */
   float kl_scale;        /* adaptive-KL runtime factor, ppo.py:475; 1.0 */
   int32_t use_clipped_value_loss; /* 1 */
+  const float* kl_scale_device; /* when not NULL: a device float read in place of kl_scale (see ks_ppo_adapt_kl) */
 } KsPpoLossParams;
 int ks_ppo_loss(ks_stream_t stream, int64_t n, int32_t A, const KsPpoLossParams* params /*host*/,
                 const float* advantages, const float* value_targets, const float* on_log_probs,
@@ -720,6 +729,13 @@ int64_t ks_mlp_disc_workspace_bytes(const KsMlp* mlp, int64_t n_real, int64_t n_
 int ks_mlp_disc_loss_grad(KsMlp* mlp, ks_stream_t stream, int64_t n_real, const float* real, int64_t n_sim, const float* sim,
                           float grad_penalty_coef, int64_t n_motions, float* losses, void* workspace);
 int ks_grad_sqnorm(ks_stream_t stream, int64_t n, const float* g, double* acc);
+/* ksim/task/ppo.py:546-563 (adaptive KL in _single_step), without a trip to the host: with
+ * kl_mean = mean_rows(sum_a(on_log_probs - log_probs)) * kl_coef * *kl_scale, the coefficient kl_coef * *kl_scale is
+ * multiplied by 1.5 when kl_mean > 1.5 desired_kl, divided by 1.5 when kl_mean < desired_kl / 1.5, clipped to
+ * [1e-8, 1e2], and *kl_scale (device, in/out) becomes that coefficient / kl_coef.  The next ks_ppo_loss_grad reads it
+ * through KsPpoLossParams.kl_scale_device.  workspace: 256 floats (device).  Sums in a fixed order. */
+int ks_ppo_adapt_kl(ks_stream_t stream, int64_t rows, int32_t A, const float* on_log_probs, const float* log_probs,
+                    float kl_coef, float desired_kl, float* kl_scale, float* workspace);
 int ks_mlp_grad_sqnorm(const KsMlp* mlp, ks_stream_t stream, double* acc);
 int ks_mlp_adam_step(KsMlp* mlp, ks_stream_t stream, const KsAdamParams* params /*host*/, const double* sqnorm);
 int ks_adam_step(ks_stream_t stream, int64_t n, float* param, const float* grad, float* m1, float* m2,

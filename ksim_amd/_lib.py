@@ -26,6 +26,7 @@ class KsPpoLossParams(ctypes.Structure):
         ("log_clip_value", c_float),
         ("kl_scale", c_float),
         ("use_clipped_value_loss", c_int32),
+        ("kl_scale_device", c_void_p),
     ]
 
 
@@ -60,6 +61,8 @@ def load() -> ctypes.CDLL:
     lib.ks_copy_f32.argtypes = [p, c_int64, p, p]
     lib.ks_ppo_loss_grad.argtypes = [p, c_int64, c_int32, POINTER(KsPpoLossParams)] + [p] * 12
     lib.ks_ppo_loss_grad.restype = c_int32
+    lib.ks_ppo_adapt_kl.argtypes = [p, c_int64, c_int32, p, p, c_float, c_float, p, p]
+    lib.ks_ppo_adapt_kl.restype = c_int32
     for name in ("ks_gae_bt", "ks_gae_tn", "ks_normalize_advantages", "ks_ppo_loss", "ks_reward_total", "ks_copy_f32"):
         getattr(lib, name).restype = c_int32
     _bind_optional(lib)

@@ -512,6 +512,7 @@ struct DevMlp {
   void* Wt[KS_MAX_LAYERS];      // (kpad, npad) working-precision transpose
   int bias_frozen[KS_MAX_LAYERS];  // leading bias entries of the layer that the optimiser leaves alone
   float* zero_bias;             // zeros, as wide as the widest GEMM output
+  double* sq_part;              // kSqBlocks partial sums of squares per gradient tensor (weights and biases of every layer)
 };
 
 
@@ -692,12 +693,18 @@ __global__ __launch_bounds__(256) void sum_parts_kernel(int64_t n, int nz, const
   out[i] = s;
 }
 
-// sum of squares of a buffer, NaNs counted as zero (the optimiser zeroes them first), added to *acc in double.
-// One atomic per workgroup: the order of the additions can differ between runs in the last bit of the double.
-__global__ __launch_bounds__(256) void sqnorm_kernel(int64_t n, const float* __restrict__ g, double* __restrict__ acc) {
-  __shared__ double red[256];
+// Sum of squares of gradient buffers, NaNs counted as zero (the optimiser zeroes them first), added to *acc in double.
+// Every addition happens in a fixed order (a strided pass per lane, a tree over the lanes, then the partial sums one after
+// the other), so the clip factor, and with it a whole update, is the same bits on every run.
+constexpr int kSqBlocks = 64;
+struct SqTensors {
+  const float* g[2 * KS_MAX_LAYERS];
+  int64_t n[2 * KS_MAX_LAYERS];
+};
+
+__device__ __forceinline__ double block_sqsum(const float* __restrict__ g, int64_t n, int first, int stride, double* red) {
   double s = 0.0;
-  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
+  for (int64_t i = first; i < n; i += stride) {
     const float v = g[i];
     if (v == v) s += (double)v * (double)v;
   }
@@ -707,7 +714,35 @@ __global__ __launch_bounds__(256) void sqnorm_kernel(int64_t n, const float* __r
     if ((int)threadIdx.x < w) red[threadIdx.x] += red[threadIdx.x + w];
     __syncthreads();
   }
-  if (threadIdx.x == 0) atomicAdd(acc, red[0]);
+  return red[0];
+}
+
+// grid (kSqBlocks, tensors): part[tensor][block] = this block's share of the tensor
+__global__ __launch_bounds__(256) void sqnorm_parts_kernel(SqTensors t, double* __restrict__ part) {
+  __shared__ double red[256];
+  const double v = block_sqsum(t.g[blockIdx.y], t.n[blockIdx.y], (int)(blockIdx.x * 256 + threadIdx.x), kSqBlocks * 256, red);
+  if (threadIdx.x == 0) part[blockIdx.y * kSqBlocks + blockIdx.x] = v;
+}
+
+// one workgroup: *acc += the partial sums, in index order
+__global__ __launch_bounds__(256) void sqnorm_finish_kernel(int n, const double* __restrict__ part, double* __restrict__ acc) {
+  __shared__ double red[256];
+  double s = 0.0;
+  for (int i = threadIdx.x; i < n; i += 256) s += part[i];
+  red[threadIdx.x] = s;
+  __syncthreads();
+  for (int w = 128; w > 0; w >>= 1) {
+    if ((int)threadIdx.x < w) red[threadIdx.x] += red[threadIdx.x + w];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) *acc += red[0];
+}
+
+// one workgroup over a whole buffer (small tensors that belong to no network: log standard deviations, head parameters)
+__global__ __launch_bounds__(256) void sqnorm_kernel(int64_t n, const float* __restrict__ g, double* __restrict__ acc) {
+  __shared__ double red[256];
+  const double v = block_sqsum(g, n, (int)threadIdx.x, 256, red);
+  if (threadIdx.x == 0) *acc += v;
 }
 
 // optax.chain(zero_nans, clip_by_global_norm, add_decayed_weights, scale_by_adam, scale(lr), scale(-1)) on one tensor
@@ -901,6 +936,7 @@ extern "C" int ks_mlp_destroy(KsMlp* h) {
     if (h->m.Wt[l]) (void)hipFree(h->m.Wt[l]);
   }
   if (h->m.zero_bias) (void)hipFree(h->m.zero_bias);
+  if (h->m.sq_part) (void)hipFree(h->m.sq_part);
   delete h;
   return KS_OK;
 }
@@ -1066,6 +1102,24 @@ extern "C" int ks_mlp_train_init(KsMlp* h) {
   if (!h) return fail(KS_EINVAL, "ks_mlp_train_init: null handle");
   DevMlp& m = h->m;
   if (m.train) return KS_OK;
+  // a failure part way leaves nothing behind: what was allocated so far is released and the handle stays untrained
+  auto give_up = [&](const char* what) {
+    for (int l = 0; l < KS_MAX_LAYERS; ++l) {
+      float** t[] = {&m.mW[l], &m.mb[l], &m.gW[l], &m.gb[l], &m.m1W[l], &m.m2W[l], &m.m1b[l], &m.m2b[l]};
+      for (float** q : t) {
+        if (*q) (void)hipFree(*q);
+        *q = nullptr;
+      }
+      if (m.Wt[l]) (void)hipFree(m.Wt[l]);
+      m.Wt[l] = nullptr;
+    }
+    if (m.zero_bias) (void)hipFree(m.zero_bias);
+    if (m.sq_part) (void)hipFree(m.sq_part);
+    m.zero_bias = nullptr;
+    m.sq_part = nullptr;
+    m.train = 0;
+    return fail(KS_ELAUNCH, "ks_mlp_train_init: %s failed", what);
+  };
   const size_t esz = m.dtype == KS_MLP_BF16 ? 2 : 4;
   for (int l = 0; l < m.n_layers; ++l) {
     const size_t n = (size_t)m.npad[l] * m.kpad[l], nb = m.npad[l];
@@ -1077,25 +1131,27 @@ extern "C" int ks_mlp_train_init(KsMlp* h) {
     float** wbufs[] = {&m.mW[l], &m.gW[l], &m.m1W[l], &m.m2W[l]};
     float** bbufs[] = {&m.mb[l], &m.gb[l], &m.m1b[l], &m.m2b[l]};
     for (float** q : wbufs)
-      if (hipMalloc((void**)q, n * 4) != hipSuccess || hipMemset(*q, 0, n * 4) != hipSuccess) return fail(KS_ELAUNCH, "ks_mlp_train_init: allocation failed");
+      if (hipMalloc((void**)q, n * 4) != hipSuccess || hipMemset(*q, 0, n * 4) != hipSuccess) return give_up("allocation");
     for (float** q : bbufs)
-      if (hipMalloc((void**)q, nb * 4) != hipSuccess || hipMemset(*q, 0, nb * 4) != hipSuccess) return fail(KS_ELAUNCH, "ks_mlp_train_init: allocation failed");
+      if (hipMalloc((void**)q, nb * 4) != hipSuccess || hipMemset(*q, 0, nb * 4) != hipSuccess) return give_up("allocation");
     if (hipMemcpy(m.mW[l], w.data(), n * 4, hipMemcpyHostToDevice) != hipSuccess ||
         hipMemcpy(m.mb[l], b.data(), nb * 4, hipMemcpyHostToDevice) != hipSuccess)
-      return fail(KS_ELAUNCH, "ks_mlp_train_init: upload failed");
+      return give_up("upload");
     // the first layer's transpose is padded to whole output tiles of the input-gradient product; the padding stays zero
     const size_t nt = l == 0 ? (size_t)round_up(m.kpad[0], kBN) * m.npad[0] : n;
     if (hipMalloc(&m.Wt[l], nt * esz) != hipSuccess || hipMemset(m.Wt[l], 0, nt * esz) != hipSuccess)
-      return fail(KS_ELAUNCH, "ks_mlp_train_init: allocation failed");
+      return give_up("allocation");
   }
   const int wz = widest_pad(m);
   if (hipMalloc((void**)&m.zero_bias, (size_t)wz * 4) != hipSuccess || hipMemset(m.zero_bias, 0, (size_t)wz * 4) != hipSuccess)
-    return fail(KS_ELAUNCH, "ks_mlp_train_init: allocation failed");
+    return give_up("allocation");
+  if (hipMalloc((void**)&m.sq_part, sizeof(double) * kSqBlocks * 2 * KS_MAX_LAYERS) != hipSuccess)
+    return give_up("allocation");
   m.train = 1;
   // working copies (among them the transposes, which did not exist yet) from the master weights
   if (m.dtype == KS_MLP_BF16) refresh_layers<__bf16>(m, (hipStream_t)0);
   else refresh_layers<float>(m, (hipStream_t)0);
-  if (hipStreamSynchronize((hipStream_t)0) != hipSuccess) return fail(KS_ELAUNCH, "ks_mlp_train_init: refresh failed");
+  if (hipStreamSynchronize((hipStream_t)0) != hipSuccess) return give_up("refresh");
   return KS_OK;
 }
 
@@ -1328,18 +1384,25 @@ extern "C" int ks_mlp_freeze_bias_prefix(KsMlp* h, int32_t layer, int32_t count)
 extern "C" int ks_grad_sqnorm(ks_stream_t stream, int64_t n, const float* g, double* acc) {
   if (n < 0 || !acc || (n > 0 && !g)) return fail(KS_EINVAL, "ks_grad_sqnorm: bad argument");
   if (n == 0) return KS_OK;
-  hipLaunchKernelGGL(sqnorm_kernel, dim3((unsigned)(n >= 65536 ? 64 : 1)), dim3(256), 0, (hipStream_t)stream, n, g, acc);
+  hipLaunchKernelGGL(sqnorm_kernel, dim3(1), dim3(256), 0, (hipStream_t)stream, n, g, acc);
   return check_launch("ks_grad_sqnorm");
 }
 
 extern "C" int ks_mlp_grad_sqnorm(const KsMlp* h, ks_stream_t stream, double* acc) {
   if (!h || !h->m.train || !acc) return fail(KS_EINVAL, "ks_mlp_grad_sqnorm: bad argument");
+  SqTensors t;
+  int nt = 0;
   for (int l = 0; l < h->m.n_layers; ++l) {
-    hipLaunchKernelGGL(sqnorm_kernel, dim3(64), dim3(256), 0, (hipStream_t)stream, (int64_t)h->m.npad[l] * h->m.kpad[l], h->m.gW[l], acc);
+    t.g[nt] = h->m.gW[l];
+    t.n[nt++] = (int64_t)h->m.npad[l] * h->m.kpad[l];
     const int fz = h->m.bias_frozen[l];
-    if (h->m.npad[l] > fz)
-      hipLaunchKernelGGL(sqnorm_kernel, dim3(1), dim3(256), 0, (hipStream_t)stream, (int64_t)h->m.npad[l] - fz, h->m.gb[l] + fz, acc);
+    if (h->m.npad[l] > fz) {
+      t.g[nt] = h->m.gb[l] + fz;
+      t.n[nt++] = (int64_t)h->m.npad[l] - fz;
+    }
   }
+  hipLaunchKernelGGL(sqnorm_parts_kernel, dim3(kSqBlocks, (unsigned)nt), dim3(256), 0, (hipStream_t)stream, t, h->m.sq_part);
+  hipLaunchKernelGGL(sqnorm_finish_kernel, dim3(1), dim3(256), 0, (hipStream_t)stream, nt * kSqBlocks, h->m.sq_part, acc);
   return check_launch("ks_mlp_grad_sqnorm");
 }
 

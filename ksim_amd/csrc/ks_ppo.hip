@@ -198,6 +198,9 @@ __global__ __launch_bounds__(256) void normalize_kernel(int64_t n, int nparts, c
     out[i] = (x[i] - mean) * inv;
 }
 
+// the adaptive-KL factor: a device scalar when the caller keeps it there, otherwise the host's number
+__device__ __forceinline__ float kl_scale_of(const KsPpoLossParams& p) { return p.kl_scale_device ? *p.kl_scale_device : p.kl_scale; }
+
 // ---------------------------------------------------------------------------------------------
 // PPO loss (ppo.py:207-246).  One lane per (b, t) element; the A log-probs of an element are
 // contiguous, so a wavefront touches one contiguous 64*A*4-byte span per array.
@@ -239,7 +242,7 @@ __global__ __launch_bounds__(256) void ppo_loss_kernel(
       vobj = 0.5f * er * er;
     }
     const float value = vobj * p.value_loss_coef;
-    const float klv = kl * p.kl_coef * p.kl_scale;
+    const float klv = kl * p.kl_coef * kl_scale_of(p);
     const float entv = ent ? -es * p.entropy_coef : 0.f;
     if (o_policy) o_policy[i] = policy;
     if (o_value) o_value[i] = value;
@@ -535,7 +538,7 @@ __global__ __launch_bounds__(256) void ppo_loss_grad_kernel(int64_t M, int nu, K
       if (s1 < s2 || ratio_inside) g_logr = -A * ratio;   // the unclipped surrogate is active (or both are the same)
     }
     // kl term: (on_lp - lp) * kl_coef * kl_scale per action
-    const float g_lp = (g_logr - p.kl_coef * p.kl_scale) * inv_m;
+    const float g_lp = (g_logr - p.kl_coef * kl_scale_of(p)) * inv_m;
     const float g_ent = -p.entropy_coef * inv_m;
     for (int a = 0; a < nu; ++a) {
       const float ls = log_std[a];
@@ -616,7 +619,7 @@ __global__ __launch_bounds__(256) void ppo_loss_grad_head_kernel(int64_t M, int 
   const bool ratio_inside = ratio > lo && ratio < hi;
   float g_logr = 0.f;
   if (log_inside && (s1 < s2 || ratio_inside)) g_logr = -A * ratio;
-  const float g_lp = (g_logr - p.kl_coef * p.kl_scale) * inv_m;
+  const float g_lp = (g_logr - p.kl_coef * kl_scale_of(p)) * inv_m;
   const float g_ent = -p.entropy_coef * inv_m;
   for (int a = 0; a < nu; ++a) {
     const float mean = rm[a] + (hd.mean_bias ? hd.mean_bias[a] : 0.f);
@@ -704,7 +707,7 @@ __global__ __launch_bounds__(128) void ppo_loss_grad_mixture_kernel(int64_t M, i
   const bool ratio_inside = ratio > lo_r && ratio < hi_r;
   float g_logr = 0.f;
   if (log_inside && (s1 < s2 || ratio_inside)) g_logr = -A * ratio;
-  const float g_lp = (g_logr - p.kl_coef * p.kl_scale) * inv_m;
+  const float g_lp = (g_logr - p.kl_coef * kl_scale_of(p)) * inv_m;
   const float g_ent = -p.entropy_coef * inv_m;
   for (int a = 0; a < nu; ++a) {
     const float x = action[m * nu + a];
@@ -753,7 +756,56 @@ __global__ void ppo_grad_finish_kernel(int nblocks, int nu, const float* __restr
   d_log_std[a] = s;
 }
 
+// adaptive KL: partial[b] = sum over the block's strided share of (on_lp - lp), every element of every row
+__global__ __launch_bounds__(256) void kl_parts_kernel(int64_t n, const float* __restrict__ on_lp, const float* __restrict__ lp,
+                                                       float* __restrict__ partial) {
+  __shared__ float red[256];
+  float s = 0.f;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) s += on_lp[i] - lp[i];
+  red[threadIdx.x] = s;
+  __syncthreads();
+  for (int w = 128; w > 0; w >>= 1) {
+    if ((int)threadIdx.x < w) red[threadIdx.x] += red[threadIdx.x + w];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) partial[blockIdx.x] = red[0];
+}
+
+__global__ __launch_bounds__(256) void kl_adapt_kernel(int nblocks, float inv_rows, float kl_coef, float desired,
+                                                       const float* __restrict__ partial, float* __restrict__ kl_scale) {
+  __shared__ float red[256];
+  red[threadIdx.x] = (int)threadIdx.x < nblocks ? partial[threadIdx.x] : 0.f;
+  __syncthreads();
+  for (int w = 128; w > 0; w >>= 1) {
+    if ((int)threadIdx.x < w) red[threadIdx.x] += red[threadIdx.x + w];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) {
+    const float coef = kl_coef * *kl_scale;
+    const float kl_mean = red[0] * inv_rows * coef;
+    float c = coef;
+    if (kl_mean > desired * 1.5f) c = coef * 1.5f;
+    if (kl_mean < desired / 1.5f) c = c / 1.5f;
+    c = fminf(fmaxf(c, 1e-8f), 1e2f);
+    *kl_scale = c / kl_coef;
+  }
+}
+
 }  // namespace ks
+
+extern "C" int ks_ppo_adapt_kl(ks_stream_t stream, int64_t rows, int32_t A, const float* on_log_probs, const float* log_probs,
+                               float kl_coef, float desired_kl, float* kl_scale, float* workspace) {
+  if (rows < 1 || A < 1) return ks::fail(KS_EINVAL, "ks_ppo_adapt_kl: bad shape");
+  if (!on_log_probs || !log_probs || !kl_scale || !workspace) return ks::fail(KS_EINVAL, "ks_ppo_adapt_kl: null pointer");
+  if (!(kl_coef > 0.f) || !(desired_kl > 0.f)) return ks::fail(KS_EINVAL, "ks_ppo_adapt_kl: kl_coef and desired_kl must be positive");
+  const int64_t n = rows * A;
+  const int64_t want = (n + 1023) / 1024;
+  const int blocks = (int)(want < 256 ? want : 256);
+  hipLaunchKernelGGL(ks::kl_parts_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream, n, on_log_probs, log_probs, workspace);
+  hipLaunchKernelGGL(ks::kl_adapt_kernel, dim3(1), dim3(256), 0, (hipStream_t)stream, blocks, 1.f / (float)rows, kl_coef, desired_kl,
+                     (const float*)workspace, kl_scale);
+  return ks::check_launch("ks_ppo_adapt_kl");
+}
 
 extern "C" int ks_gaussian_log_prob(ks_stream_t stream, int64_t M, int32_t nu, const float* mean, const float* log_std,
                                     const float* action, float* log_prob, float* entropy) {

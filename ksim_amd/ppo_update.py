@@ -52,9 +52,13 @@ class GaussianMlpPolicy:
     critic: MLP
     log_std: torch.Tensor
     opt_step: int = 0
-    kl_coef: float | None = None
+    kl_scale: torch.Tensor | None = None  # adaptive KL: current coefficient / cfg.kl_coef, one device float
     _m1: torch.Tensor | None = field(default=None, repr=False)
     _m2: torch.Tensor | None = field(default=None, repr=False)
+
+    def kl_coef(self, cfg: "PPOUpdateConfig") -> float:
+        """The current KL coefficient (reads the device scalar: for logging, not for the update loop)."""
+        return cfg.kl_coef * (float(self.kl_scale.item()) if self.kl_scale is not None else 1.0)
 
     def train_init(self) -> None:
         self.actor.train_init()
@@ -91,9 +95,12 @@ def single_step(policy: GaussianMlpPolicy, cfg: PPOUpdateConfig, actor_obs, crit
     inputs = ppo_mod.compute_ppo_inputs(value.view(Tn, b), rewards, done, success, cfg.gamma, cfg.lam,
                                         normalize_advantages=cfg.normalize_advantages,
                                         monte_carlo_returns=cfg.monte_carlo_returns, time_major=True)
-    kl_coef_now = policy.kl_coef if (cfg.adaptive_kl and policy.kl_coef is not None) else cfg.kl_coef
+    # adaptive KL (ppo.py:546-563): the running factor kl_coef_now / kl_coef is a device scalar that the loss kernel reads
+    # and ks_ppo_adapt_kl updates after the step, so no value crosses to the host between minibatch steps
+    if cfg.adaptive_kl and policy.kl_scale is None:
+        policy.kl_scale = torch.ones(1, dtype=torch.float32, device=actor_obs.device)
     p = _lib.KsPpoLossParams(cfg.clip_param, cfg.value_loss_coef, cfg.entropy_coef, cfg.kl_coef, cfg.log_clip_value,
-                             kl_coef_now / cfg.kl_coef, int(cfg.use_clipped_value_loss))
+                             1.0, int(cfg.use_clipped_value_loss), _lib.ptr(policy.kl_scale) if cfg.adaptive_kl else None)
     d_mean = torch.empty_like(mean)
     d_value = torch.empty(rows, 1, dtype=torch.float32, device=mean.device)
     d_log_std = torch.empty_like(policy.log_std)
@@ -118,14 +125,9 @@ def single_step(policy: GaussianMlpPolicy, cfg: PPOUpdateConfig, actor_obs, crit
                                 _lib.ptr(policy._m1), _lib.ptr(policy._m2), ctypes.byref(ap), _lib.ptr(sq)))
     metrics = {"grad_norm": sq.sqrt(), "d_mean": d_mean, "d_value": d_value, "d_log_std": d_log_std,
                "log_probs": lp, "values": value, "advantages": inputs.advantages_bt}
-    if cfg.adaptive_kl:  # ppo.py:548-563
-        kl_mean = float((on_lp - lp).sum(-1).mean().item()) * kl_coef_now
-        new = kl_coef_now
-        if kl_mean > cfg.desired_kl * 1.5:
-            new = kl_coef_now * 1.5
-        if kl_mean < cfg.desired_kl / 1.5:
-            new = new / 1.5
-        policy.kl_coef = min(max(new, 1e-8), 1e2)
+    if cfg.adaptive_kl:
+        _lib.check(lib.ks_ppo_adapt_kl(_lib.current_stream(), rows, nu, _lib.ptr(on_lp), _lib.ptr(lp), cfg.kl_coef,
+                                       cfg.desired_kl, _lib.ptr(policy.kl_scale), _lib.ptr(ws)))
     return metrics
 
 
@@ -140,8 +142,6 @@ def update_model(policy: GaussianMlpPolicy, cfg: PPOUpdateConfig, actor_obs, cri
     Tn, N = done.shape
     if policy._m1 is None:
         policy.train_init()
-    if cfg.adaptive_kl and policy.kl_coef is None:
-        policy.kl_coef = cfg.kl_coef
     nu = action.shape[-1]
     # on-policy variables of the whole rollout with the pre-update parameters (ppo.py:603-607)
     on_lp, on_v, _, _ = get_ppo_variables(policy, actor_obs.reshape(Tn * N, -1), critic_obs.reshape(Tn * N, -1),

@@ -329,3 +329,71 @@ def test_ppo_loss_gradient_for_the_mixture_head_matches_autograd():
     _, lp_k, _ = sample_action_mixture(args[0], K, mean_bias=dev[0], clip_lo=dev[1], clip_hi=dev[2], uniform=t32(rng.random((M, A))),
                                        noise=t32(rng.normal(size=(M, A))), want_stats=True, **hd)
     assert torch.isfinite(lp_k).all()
+
+
+def test_adaptive_kl_coefficient_is_updated_on_the_device():
+    """ppo.py:546-563: the coefficient grows by 1.5 above 1.5 x desired, shrinks by 1.5 below desired / 1.5, stays inside the
+    band and is clipped to [1e-8, 1e2].  Expected values below are worked out by hand from the mean of the row sums."""
+    from ksim_amd import _lib
+
+    lib = _lib.load()
+    rows, A, kl_coef = 1000, 5, 1e-3
+    rng = np.random.default_rng(3)
+    lp = rng.normal(size=(rows, A)).astype(np.float32)
+    ws = torch.empty(256, device=DEV)
+
+    def run(diff_per_element, scale0, desired):
+        on_lp = lp + np.float32(diff_per_element)  # mean over rows of sum over actions = A * diff
+        s = torch.tensor([scale0], dtype=torch.float32, device=DEV)
+        a, b = t32(on_lp), t32(lp)
+        _lib.check(lib.ks_ppo_adapt_kl(_lib.current_stream(), rows, A, _lib.ptr(a), _lib.ptr(b), kl_coef, desired,
+                                       _lib.ptr(s), _lib.ptr(ws)))
+        return float(s.item())
+
+    # kl_mean = 5 * 0.4 * 1e-3 * 2 = 4e-3
+    assert run(0.4, 2.0, 0.002) == pytest.approx(3.0, rel=1e-5)       # 4e-3 > 3e-3: x 1.5
+    assert run(0.4, 2.0, 0.01) == pytest.approx(2.0 / 1.5, rel=1e-5)  # 4e-3 < 6.67e-3: / 1.5
+    assert run(0.4, 2.0, 0.004) == pytest.approx(2.0, rel=1e-6)       # inside the band
+    assert run(0.4, 9e4, 1e-6) == pytest.approx(1e5, rel=1e-5)        # 90 x 1.5 = 135 is clipped to 1e2 = 1e5 x kl_coef
+    assert run(-0.4, 1.2e-5, 1.0) == pytest.approx(1e-5, rel=1e-5)    # 1.2e-8 / 1.5 is clipped to 1e-8
+
+
+def test_adaptive_kl_in_single_step_follows_the_host_rule_without_a_sync():
+    from ksim_amd.ppo_update import PPOUpdateConfig, get_ppo_variables, single_step
+
+    Tn, N, od, A = 16, 8, 30, 6
+    pol, params, ro, rng = _setup(11, Tn, N, od, A, 64)
+    pol.train_init()
+    cfg = PPOUpdateConfig(**dict(CFG, learning_rate=3e-3), adaptive_kl=True, desired_kl=2e-4)
+    d = {k: (torch.tensor(v, device=DEV) if v.dtype == bool else t32(v)) for k, v in ro.items()}
+    rows = Tn * N
+    on_lp, on_v, _, _ = get_ppo_variables(pol, d["actor_obs"].reshape(rows, od), d["critic_obs"].reshape(rows, od), d["action"].reshape(rows, A))
+    on_lp, on_v = on_lp.view(Tn, N, A).clone(), on_v.view(Tn, N).clone()
+    coef, seen = cfg.kl_coef, set()
+    for _ in range(8):
+        met = single_step(pol, cfg, d["actor_obs"], d["critic_obs"], d["action"], d["rewards"], d["done"], d["success"], on_lp, on_v)
+        kl_mean = float((on_lp.reshape(rows, A).double() - met["log_probs"].double()).sum(-1).mean().item()) * coef
+        new = coef * 1.5 if kl_mean > cfg.desired_kl * 1.5 else coef
+        new = new / 1.5 if kl_mean < cfg.desired_kl / 1.5 else new
+        seen.add("up" if new > coef else "down" if new < coef else "same")
+        coef = min(max(new, 1e-8), 1e2)
+        assert pol.kl_coef(cfg) == pytest.approx(coef, rel=1e-5)
+    assert {"up", "down"} <= seen, f"the test drove the coefficient only {seen}"
+
+
+def test_gradient_norm_and_update_are_bit_reproducible():
+    """The global norm behind clip_by_global_norm is summed in a fixed order: two updates from the same state are the same bits."""
+    from ksim_amd.ppo_update import PPOUpdateConfig, update_model
+
+    outs = []
+    for _ in range(2):
+        Tn, N, od, A = 12, 64, 24, 4
+        pol, params, ro, rng = _setup(13, Tn, N, od, A, 512)
+        cfg = PPOUpdateConfig(**dict(CFG, grad_clip=0.05, batch_size=16))
+        d = {k: (torch.tensor(v, device=DEV) if v.dtype == bool else t32(v)) for k, v in ro.items()}
+        perms = [torch.tensor(np.random.default_rng(p).permutation(N), device=DEV) for p in range(cfg.num_passes)]
+        mets = update_model(pol, cfg, d["actor_obs"], d["critic_obs"], d["action"], d["rewards"], d["done"], d["success"], permutations=perms)
+        outs.append([m["grad_norm"].clone() for m in mets] + [p.clone() for pair in pol.actor.parameters() + pol.critic.parameters() for p in pair])
+    assert float(outs[0][0].item()) > 0.05, "the clip is not active"
+    for a, b in zip(*outs):
+        assert torch.equal(a, b)
