@@ -65,7 +65,38 @@ def cpu_baseline(integrator: str, target_seconds: float = 12.0):
     t = run(k)
     return {"value": N * k / t, "unit": "env-steps/s", "cores": cores, "kind": "port",
             "sample": f"physics control step only (PD + 4 substeps, {integrator_name(m)}), {N} envs x {k} steps, "
-                      f"float32 C restatement of the MJX path (not MJX), OpenMP over envs"}
+                      f"float32 C restatement of the MJX path (not MJX), OpenMP over envs",
+            "flops_per_env_step": oracle_flops_per_env_step(m, KBOT_TORQUE_LIMITS)}
+
+
+def oracle_flops_per_env_step(m, ctrl_clip, envs: int = 32, settle: int = 10, counted: int = 4) -> float:
+    """Floating-point operations of one control step (PD + 4 substeps) of one env, counted by running the oracle's C
+    source with a scalar type that counts +, -, *, / and elementary functions as one operation each (dense algebra as the
+    oracle writes it; the kernel skips structural zeros of the tree, so this is an upper bound on the useful work)."""
+    import numpy as np
+
+    from oracle.dyn import Oracle
+
+    orc = Oracle(m.arrays(), np.float64, count_flops=True)
+    rng = np.random.default_rng(1004)
+    block = orc.batch(envs)
+    for e in range(envs):
+        q = m.qpos0.copy()
+        q[7:] += rng.uniform(-0.1, 0.1, m.nu)
+        for i, v in enumerate(q):
+            block[e].qpos[i] = v
+        for b in range(m.nb):
+            block[e].mass_scale[b] = rng.uniform(0.9, 1.1)
+        block[e].friction = rng.uniform(0.4, 1.2)
+    last = np.zeros((envs, m.nu))
+    kp = np.tile(rng.uniform(20, 150, m.nu), (envs, 1))
+    kd = np.tile(rng.uniform(0.5, 1.5, m.nu), (envs, 1))
+    for k in range(settle + counted):
+        if k == settle:
+            orc.flops_reset()
+        orc.ctrl_step_batch(block, 4, 1, rng.normal(scale=0.1, size=(envs, m.nu)), last, np.zeros(envs), None, kp, kd,
+                            ctrl_clip, nthreads=1)
+    return orc.flops() / (envs * counted)
 
 
 def main() -> None:
@@ -78,7 +109,7 @@ def main() -> None:
     ap.add_argument("--integrator", choices=("euler", "implicitfast"), default="euler",
                     help="velocity update of the headline rollout: semi-implicit Euler (what the benchmark configs name) or "
                          "implicitfast (what ksim's RLConfig selects); the other one is reported under 'other_integrator'")
-    ap.add_argument("--only", choices=("mlp", "gae", "update", "rollout", "iteration"), default=None,
+    ap.add_argument("--only", choices=("mlp", "gae", "update", "rollout", "iteration", "phases"), default=None,
                     help="run one section alone and print its JSON (the command the counter runs under profiles/ use)")
     ap.add_argument("--mlp-rows", type=int, default=0, help="with --only mlp: a single row count instead of 8192 and 524288")
     ap.add_argument("--streams", type=int, default=2,
@@ -96,8 +127,23 @@ def main() -> None:
     from ksim_amd import _lib, ppo
     from ksim_amd.configs import integrator_name, step_algorithmic_bytes
 
+    if args.only == "phases":  # needs the -DKS_PROFILE build: python -m ksim_amd.csrc.build --profile
+        from ksim_amd.csrc.build import PROFILE_LIB
+
+        if not os.path.exists(PROFILE_LIB):
+            sys.exit(f"{PROFILE_LIB} is not built: run `python -m ksim_amd.csrc.build --profile` first")
+        _lib.LIB_PATH = PROFILE_LIB
     _lib.load()
     assert torch.cuda.is_available(), "bench.py needs a GPU"
+    if args.traffic_probe:  # first, so that every --only section carries the calibration launch
+        n = 64 * 1024 * 1024
+        src, dst = torch.ones(n, device="cuda"), torch.empty(n, device="cuda")
+        _lib.check(_lib.load().ks_copy_f32(_lib.current_stream(), n, _lib.ptr(src), _lib.ptr(dst)))
+        torch.cuda.synchronize()
+        del src, dst
+    if args.only == "phases":
+        print(json.dumps({"step_kernel_phases": step_kernel_phases(torch, args.integrator, args.envs)}))
+        return
     if args.only == "mlp":
         print(json.dumps({"policy_mlp": mlp_rate(torch, rows=(args.mlp_rows,) if args.mlp_rows else (8192, 524288))}))
         return
@@ -152,12 +198,6 @@ def main() -> None:
                  "ms_per_step": g_elapsed / (reps * T) * 1e3,
                  "what": "the same control steps, rewards and GAE with each T-step rollout replayed from one HIP graph"}
 
-    if args.traffic_probe:
-        n = 64 * 1024 * 1024
-        src, dst = torch.ones(n, device="cuda"), torch.empty(n, device="cuda")
-        _lib.check(_lib.load().ks_copy_f32(_lib.current_stream(), n, _lib.ptr(src), _lib.ptr(dst)))
-        torch.cuda.synchronize()
-
     # GAE on rotating cfg-2 sized buffers (T=128, N=4096): larger than the caches in total
     gae = gae_bandwidth(torch, ppo)
     mlp = mlp_rate(torch)
@@ -208,7 +248,16 @@ def main() -> None:
         "gae": gae, "policy_mlp": mlp, "ppo_update": upd, "ppo_iteration": iteration, "graph_replay": graph,
     }
     if not args.no_cpu_baseline:
-        line["cpu_baseline"] = cpu_baseline(args.integrator)
+        base = cpu_baseline(args.integrator)
+        flops = base.pop("flops_per_env_step")
+        line["cpu_baseline"] = base
+        rate = flops * envs_per_launch / (kernel_ms * 1e-3) / 1e12
+        line["roofline"]["fp32_valu"] = {
+            "achieved": rate, "peak": FP32_VALU_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": rate / FP32_VALU_PEAK_TFLOPS,
+            "flops_per_env_step": flops,
+            "what": "floating-point operations of one env's control step as the float64 oracle performs them (counted by "
+                    "a build of its C source with a counting scalar type, 32 standing envs) x envs per launch / the "
+                    "step kernel's measured duration"}
     print(json.dumps(line))
 
 
@@ -305,6 +354,36 @@ def gae_bandwidth(torch, ppo, reps=8):
         out[name] = {"layout": "(B,T) fp32, dones int8", "ms_per_call": ms, "achieved_GBps": nbytes / (ms * 1e-3) / 1e9,
                      "frac_of_hbm_peak": nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "algorithmic_bytes": nbytes,
                      "buffer_sets": sets}
+    # the rollout's own layout (T, N), with the success flags it carries: cfg 4 / cfg 5 shapes and a large one
+    for name, N, T, sets in (("rollout_T32_N8192", 8192, 32, 64), ("rollout_T32_N16384", 16384, 32, 32),
+                             ("large_T128_N65536_tn", 65536, 128, 4)):
+        g = torch.Generator(device="cuda")
+        g.manual_seed(1004)
+        bufs = [(torch.randn(T, N, device="cuda", generator=g), torch.randn(T, N, device="cuda", generator=g),
+                 (torch.rand(T, N, device="cuda", generator=g) < 0.01).view(torch.uint8),
+                 torch.zeros(T, N, dtype=torch.uint8, device="cuda")) for _ in range(sets)]
+        res = [torch.empty(T, N, device="cuda") for _ in range(3)]
+        st = _lib.current_stream()
+
+        def run_tn(v, r, d, sc):
+            _lib.check(lib.ks_gae_tn(st, T, N, _lib.ptr(v), _lib.ptr(r), _lib.ptr(d), _lib.ptr(sc), 0.99, 0.95, 0,
+                                     _lib.ptr(res[0]), _lib.ptr(res[1]), _lib.ptr(res[2])))
+
+        for b in bufs[:2]:
+            run_tn(*b)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            for b in bufs:
+                run_tn(*b)
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / (reps * sets)
+        nbytes = T * N * 22
+        out[name] = {"layout": "(T,N) fp32, dones and successes int8", "ms_per_call": ms,
+                     "achieved_GBps": nbytes / (ms * 1e-3) / 1e9, "frac_of_hbm_peak": nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                     "algorithmic_bytes": nbytes, "buffer_sets": sets}
     return out
 
 
@@ -343,6 +422,44 @@ def ppo_update_rate(torch, reps=6):
             "mfma_utilisation": flops / ms / 1e9 / (BF16_PEAK_TFLOPS),
             "what": "forward + backward (3x the forward flops) of actor and critic 68-3x512-{20,1} bf16, GAE, loss "
                     "gradient and optimiser chain on 2048 envs x 32 steps"}
+
+
+STEP_PHASES = ("actuator + reload of constants", "forward kinematics", "com / cinert / cdof", "composite inertia + M",
+               "velocities + RNE bias", "M rows / smooth force", "contacts", "Cholesky(M) + solve", "Jacobian rows",
+               "warm start + cost", "constraint update", "Hessian JtDJ", "Cholesky(H) + solve", "line search", "-",
+               "integration")
+
+
+def step_kernel_phases(torch, integrator: str, N: int, steps: int = 30) -> dict:
+    """Clock cycles (s_memtime, 100 MHz) that one env's wavefront spends in each phase of a control step (4 substeps), mean
+    over the envs of the benchmark's standing K-Bot-scale robots; read from the profiling build of the library."""
+    import numpy as np
+
+    from ksim_amd import model as km
+    from ksim_amd import physics
+
+    m = km.kbot_scale_model(seed=1004, integrator=integrator)
+    dm = physics.DeviceModel(m)
+    rng = np.random.default_rng(0)
+    t = lambda a: torch.tensor(a, dtype=torch.float32, device="cuda").contiguous()  # noqa: E731
+    z = lambda *s, **k: torch.zeros(*s, device="cuda", **k)  # noqa: E731
+    qpos = np.tile(m.qpos0, (N, 1))
+    qpos[:, 7:] += rng.uniform(-0.1, 0.1, (N, m.nu))
+    buf = dict(qpos=t(qpos), qvel=z(N, m.nv), qacc_warmstart=z(N, m.nv), time=z(N), last_ctrl=z(N, m.nu),
+               action=t(rng.uniform(-0.1, 0.1, (N, m.nu))), kp=t(rng.uniform(20, 150, m.nu)), kd=t(rng.uniform(0.5, 1.5, m.nu)),
+               ctrl_clip=t(np.full(m.nu, 80.0)), friction=t(rng.uniform(0.4, 1.2, N)), mass_scale=t(rng.uniform(0.9, 1.1, (N, m.nb))),
+               xpos=z(N, m.nb * 3), xquat=z(N, m.nb * 4), solver_niter=z(N, dtype=torch.int32), nefc=z(N, dtype=torch.int32),
+               dbg_M=z(N, m.nv * m.nv))
+    for _ in range(steps):
+        physics.control_step(dm, buf, substeps=4)
+    torch.cuda.synchronize()
+    p = buf["dbg_M"][:, :16].cpu().numpy().astype(np.float64)
+    total = float(p.sum(1).mean())
+    return {"num_envs": N, "integrator": integrator, "lds_bytes_per_env": dm.lds_bytes, "cycles_per_control_step": total,
+            "newton_iterations_mean": float(buf["solver_niter"].float().mean().item()),
+            "constraint_rows_mean": float(buf["nefc"].float().mean().item()),
+            "phases": {n: {"cycles": float(p[:, i].mean()), "share": float(p[:, i].mean()) / total}
+                       for i, n in enumerate(STEP_PHASES) if n != "-"}}
 
 
 def ppo_iteration_rate(torch, reps=3):

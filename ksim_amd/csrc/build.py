@@ -1,6 +1,10 @@
 """Builds libksimhip.so for gfx950 with hipcc (in-tree, no JIT cache).
 
-Usage: python -m ksim_amd.csrc.build [--force]
+Usage: python -m ksim_amd.csrc.build [--force] [--profile]
+
+--profile builds libksimhip_prof.so instead: the same sources with -DKS_PROFILE, whose step kernel writes the clock cycles
+it spends in each phase into the `dbg_M` debug buffer (and whose fused MLP kernel stamps its phases).  A tuning aid that
+nothing loads by default.
 """
 from __future__ import annotations
 
@@ -11,6 +15,7 @@ import sys
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB = os.path.join(os.path.dirname(HERE), "libksimhip.so")
+PROFILE_LIB = os.path.join(os.path.dirname(HERE), "libksimhip_prof.so")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "-O3", "-std=c++17", "--offload-arch=gfx950", "-fPIC", "-shared", "-fno-gpu-rdc",
@@ -35,16 +40,18 @@ def is_stale() -> bool:
     return any(os.path.getmtime(p) > t for p in sources() + headers())
 
 
-def build(force: bool = True, verbose: bool = True) -> str:
-    if not force and not is_stale():
+def build(force: bool = True, verbose: bool = True, profile: bool = False) -> str:
+    if not force and not profile and not is_stale():
         return LIB
     objs = []
     procs = []
     os.makedirs(os.path.join(HERE, "build"), exist_ok=True)
+    extra = ["-DKS_PROFILE"] if profile else []
+    target = PROFILE_LIB if profile else LIB
     for src in sources():
-        obj = os.path.join(HERE, "build", os.path.basename(src) + ".o")
+        obj = os.path.join(HERE, "build", os.path.basename(src) + (".prof.o" if profile else ".o"))
         objs.append(obj)
-        cmd = [HIPCC] + [f for f in FLAGS if f != "-shared"] + ["-c", src, "-o", obj]
+        cmd = [HIPCC] + [f for f in FLAGS if f != "-shared"] + extra + ["-c", src, "-o", obj]
         if verbose:
             print(" ".join(cmd), flush=True)
         procs.append((src, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
@@ -55,13 +62,12 @@ def build(force: bool = True, verbose: bool = True) -> str:
             raise RuntimeError(f"hipcc failed on {src}:\n{out}")
         if verbose and out:
             print(out)
-    cmd = [HIPCC, "-shared", "-fPIC", "--offload-arch=gfx950", "-fno-gpu-rdc", "-o", LIB] + objs
+    cmd = [HIPCC, "-shared", "-fPIC", "--offload-arch=gfx950", "-fno-gpu-rdc", "-o", target] + objs
     if verbose:
         print(" ".join(cmd), flush=True)
     subprocess.run(cmd, check=True)
-    return LIB
+    return target
 
 
 if __name__ == "__main__":
-    build(force="--force" in sys.argv or True)
-    print("built", LIB)
+    print("built", build(force=True, profile="--profile" in sys.argv))

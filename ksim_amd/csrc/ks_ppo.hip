@@ -104,32 +104,59 @@ __global__ __launch_bounds__(256) void gae_bt_kernel(
   }
 }
 
-// GAE, (T, N) layout: one lane per env, walking back in time; a wavefront reads 64
-// consecutive envs per step (256 B), and the loads of the next steps do not depend on the
-// recurrence so the compiler can keep several in flight.
+// GAE, (T, N) layout.  A workgroup owns 32 consecutive envs and walks back in time in chunks of 32 steps: all 256
+// threads load the chunk's (32 steps x 32 envs) tiles into LDS (128-byte rows, every load independent of the
+// recurrence), the first 32 threads run the recurrence out of LDS, one env each, and all threads write the results
+// back.  With one lane per env doing its own loads, 8192 envs would be 128 wavefronts with one dependent stream of
+// loads each; here every CU has eight times as many loads in flight and N / 32 workgroups spread over the chip.
+constexpr int kTnEnvs = 32, kTnSteps = 32;
 __global__ __launch_bounds__(256) void gae_tn_kernel(
     int64_t T, int64_t N, const float* __restrict__ values, const float* __restrict__ rewards,
     const uint8_t* __restrict__ dones, const uint8_t* __restrict__ successes, float gamma, float lam,
     int mc, float* __restrict__ gae, float* __restrict__ returns, float* __restrict__ targets) {
-  const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (e >= N) return;
+  __shared__ float sv[kTnSteps][kTnEnvs], sr[kTnSteps][kTnEnvs], oa[kTnSteps][kTnEnvs], orr[kTnSteps][kTnEnvs];
+  __shared__ uint8_t sd[kTnSteps][kTnEnvs], ss[kTnSteps][kTnEnvs];
+  const int tx = threadIdx.x & (kTnEnvs - 1), ty = threadIdx.x / kTnEnvs;
+  const int64_t e = (int64_t)blockIdx.x * kTnEnvs + tx;
+  const bool in = e < N;
   const float gl = gamma * lam, omg = 1.0f - gamma;
-  float R = 0.f, A = 0.f;
-  float v_up = values[(T - 1) * N + e];
-#pragma unroll 4
-  for (int64_t t = T - 1; t >= 0; --t) {
-    const int64_t i = t * N + e;
-    const float v = values[i], r = rewards[i];
-    const float mask = dones[i] ? 0.f : 1.f;
-    const float sc = (successes && successes[i]) ? 1.f : 0.f;
-    const float rb = omg * r + gamma * v * sc;
-    const float delta = rb + gamma * v_up * mask - v;
-    R = rb + gamma * mask * R;
-    A = delta + gl * mask * A;
-    if (gae) gae[i] = A;
-    if (returns) returns[i] = R;
-    if (targets) targets[i] = mc ? R : A + v;
-    v_up = v;
+  float R = 0.f, A = 0.f, v_up = 0.f;
+  for (int64_t t1 = T; t1 > 0; t1 -= kTnSteps) {
+    const int64_t t0 = t1 > kTnSteps ? t1 - kTnSteps : 0;
+    const int n = (int)(t1 - t0);
+    for (int k = ty; k < n; k += 256 / kTnEnvs) {
+      const int64_t i = (t0 + k) * N + e;
+      sv[k][tx] = in ? values[i] : 0.f;
+      sr[k][tx] = in ? rewards[i] : 0.f;
+      sd[k][tx] = in ? dones[i] : (uint8_t)0;
+      ss[k][tx] = (in && successes) ? successes[i] : (uint8_t)0;
+    }
+    __syncthreads();
+    if (threadIdx.x < kTnEnvs) {
+      if (t1 == T) v_up = sv[n - 1][tx];
+      for (int k = n - 1; k >= 0; --k) {
+        const float v = sv[k][tx], r = sr[k][tx];
+        const float mask = sd[k][tx] ? 0.f : 1.f;
+        const float sc = ss[k][tx] ? 1.f : 0.f;
+        const float rb = omg * r + gamma * v * sc;
+        const float delta = rb + gamma * v_up * mask - v;
+        R = rb + gamma * mask * R;
+        A = delta + gl * mask * A;
+        oa[k][tx] = A;
+        orr[k][tx] = R;
+        v_up = v;
+      }
+    }
+    __syncthreads();
+    if (in)
+      for (int k = ty; k < n; k += 256 / kTnEnvs) {
+        const int64_t i = (t0 + k) * N + e;
+        const float a = oa[k][tx], rr = orr[k][tx];
+        if (gae) gae[i] = a;
+        if (returns) returns[i] = rr;
+        if (targets) targets[i] = mc ? rr : a + sv[k][tx];
+      }
+    __syncthreads();
   }
 }
 
@@ -369,9 +396,9 @@ extern "C" int ks_gae_tn(ks_stream_t stream, int64_t T, int64_t N, const float* 
                          int monte_carlo_returns, float* gae, float* returns, float* targets) {
   if (int rc = check_gae_args(T, N, values, rewards, dones)) return rc;
   if (N == 0 || T == 0) return KS_OK;
-  const int64_t grid = (N + 63) / 64;
+  const int64_t grid = (N + kTnEnvs - 1) / kTnEnvs;
   if (grid > 0x7fffffff) return fail(KS_ELIMIT, "ks_gae_tn: N too large");
-  hipLaunchKernelGGL(gae_tn_kernel, dim3((unsigned)grid), dim3(64), 0, (hipStream_t)stream, T, N, values, rewards,
+  hipLaunchKernelGGL(gae_tn_kernel, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, T, N, values, rewards,
                      dones, successes, gamma, lam, monte_carlo_returns, gae, returns, targets);
   return check_launch("ks_gae_tn");
 }

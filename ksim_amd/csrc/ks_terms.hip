@@ -68,7 +68,9 @@ __global__ __launch_bounds__(256) void observe_kernel(ObserveArgs a) {
   if (idx >= a.N * a.obs_dim) return;
   const int64_t e = idx / a.obs_dim;
   const int k = (int)(idx - e * a.obs_dim);
-  const KsObsElem el = a.t->d.obs[k];
+  // read in place (the table sits in the caches): a private copy of the element, whose noise chain is indexed at run
+  // time, would live in scratch memory and cost a write and a read of the whole element per thread
+  const KsObsElem& el = a.t->d.obs[k];
   float v;
   if (el.kind == KS_OBS_COPY) {
     v = (el.src == KS_SRC_CONST) ? el.c0 : a.src[el.src][e * a.src_dim[el.src] + el.index];

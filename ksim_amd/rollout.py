@@ -219,27 +219,34 @@ class Rollout:
     def _unroll_graph(self, env: RolloutEnvState, level: float) -> tuple[Trajectory, RewardState]:
         if self.c.engine.data.drop_action_prob * float(level) > 0:
             raise _lib.KsError("graph replay needs drop_action_prob == 0 (the drop mask is sampled on the host side)")
-        key = (id(env), float(level))
-        if self._graph is None or self._graph[0] != key:
-            self.step_base.fill_(env.step)
-            self.c.engine.prepare(self.step_base.device)
-            self._prepare_env(env)
-            torch.cuda.synchronize()
-            g = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(g):
-                for t in range(self.T):
-                    self.step_engine(env, t, level, _relative_step=True)
-                traj = self.trajectory()
-                rewards = self._rewards(traj, env, level)
-                self.step_base += self.T
-            self._graph = (key, g, traj, rewards)
-        elif int(env.step) != self._graph_step:
+        if not self._capture(env, level) and int(env.step) != self._graph_step:
             self.step_base.fill_(env.step)  # the eager path ran in between
         _, g, traj, rewards = self._graph
         g.replay()
         env.step += self.T
         self._graph_step = int(env.step)
         return traj, rewards
+
+    def _capture(self, env: RolloutEnvState, level: float) -> bool:
+        """Captures the rollout of `env` at `level` as a HIP graph unless that is the graph already held; True when it
+        captured (which synchronises the device)."""
+        key = (id(env), float(level))
+        if self._graph is not None and self._graph[0] == key:
+            return False
+        self.step_base.fill_(env.step)
+        self.c.engine.prepare(self.step_base.device)
+        self._prepare_env(env)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            for t in range(self.T):
+                self.step_engine(env, t, level, _relative_step=True)
+            traj = self.trajectory()
+            rewards = self._rewards(traj, env, level)
+            self.step_base += self.T
+        self._graph = (key, g, traj, rewards)
+        self._graph_step = int(env.step)
+        return True
 
     def _prepare_env(self, env: RolloutEnvState) -> None:
         """Carry buffers of an env state seen for the first time (never inside a graph capture: `_unroll_graph`
@@ -351,16 +358,27 @@ class SplitRollout:
             with torch.cuda.stream(st):
                 ro.step_engine(env, t, level, noise[g] if noise is not None else None)
 
-    def unroll(self, envs: Sequence[RolloutEnvState], level: float = 1.0) -> list[tuple[Trajectory, RewardState]]:
-        """T control steps and the reward pass of every group; returns one (trajectory, rewards) per group."""
+    def unroll(self, envs: Sequence[RolloutEnvState], level: float = 1.0, graph: bool = False) -> list[tuple[Trajectory, RewardState]]:
+        """T control steps and the reward pass of every group; returns one (trajectory, rewards) per group.  With
+        `graph=True` each group's launches are captured once as a HIP graph of its own and the graphs are replayed side by
+        side on the groups' streams (`Rollout.unroll(graph=True)` per group): the same bits, without the per-launch host
+        cost, which with two chains of launches to feed is what the eager path spends most of a step on."""
+        if graph and any(ro._graph is None for ro in self.parts):
+            for ro, env in zip(self.parts, envs):  # captures synchronise the device: do them before the groups fork
+                ro._capture(env, level)
         self.fork()
-        for t in range(self.T):
-            self.step_engine(envs, t, level)
         out = []
-        for ro, env, st in zip(self.parts, envs, self.streams):
-            with torch.cuda.stream(st):
-                traj = ro.trajectory()
-                out.append((traj, ro._rewards(traj, env, level)))
+        if graph:
+            for ro, env, st in zip(self.parts, envs, self.streams):
+                with torch.cuda.stream(st):
+                    out.append(ro.unroll(env, level, graph=True))
+        else:
+            for t in range(self.T):
+                self.step_engine(envs, t, level)
+            for ro, env, st in zip(self.parts, envs, self.streams):
+                with torch.cuda.stream(st):
+                    traj = ro.trajectory()
+                    out.append((traj, ro._rewards(traj, env, level)))
         self.join()
         return out
 

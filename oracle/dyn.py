@@ -14,12 +14,13 @@ import numpy as np
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB = os.path.join(HERE, "libksoracle.so")
+FLOPS_LIB = os.path.join(HERE, "libksoracle_flops.so")
 MAXB, MAXQ, MAXV, MAXU, MAXS, MAXR = 32, 40, 32, 32, 16, 128
 
 
 def build(force: bool = False) -> str:
-    src = [os.path.join(HERE, f) for f in ("ks_dyn_oracle.c", "ks_dyn_oracle.h", "Makefile")]
-    if force or not os.path.exists(LIB) or any(os.path.getmtime(s) > os.path.getmtime(LIB) for s in src):
+    src = [os.path.join(HERE, f) for f in ("ks_dyn_oracle.c", "ks_dyn_oracle.h", "flop_count.cpp", "Makefile")]
+    if force or not os.path.exists(LIB) or not os.path.exists(FLOPS_LIB) or any(os.path.getmtime(s) > os.path.getmtime(LIB) for s in src):
         subprocess.run(["make", "-C", HERE, "-B"], check=True, capture_output=True)
     return LIB
 
@@ -151,13 +152,17 @@ class DataView:
 
 
 class Oracle:
-    def __init__(self, model_arrays: dict, dtype=np.float64):
+    def __init__(self, model_arrays: dict, dtype=np.float64, count_flops: bool = False):
+        """`count_flops`: the float64 oracle built with a scalar type that counts its floating-point operations
+        (flop_count.cpp); `flops()` reads the count, `flops_reset()` clears it.  One thread only."""
         build()
-        self.lib = ctypes.CDLL(LIB)
+        self.lib = ctypes.CDLL(FLOPS_LIB if count_flops else LIB)
         self.a = model_arrays
         self.model = make_model(model_arrays)
         self.dtype = np.dtype(dtype)
-        self.suf = "_f64" if self.dtype == np.float64 else "_f32"
+        if count_flops and self.dtype != np.float64:
+            raise ValueError("the counting oracle computes in float64")
+        self.suf = "_cnt" if count_flops else "_f64" if self.dtype == np.float64 else "_f32"
         self.Data = DataF64 if self.dtype == np.float64 else DataF32
         size = getattr(self.lib, "ksor_sizeof_data" + self.suf)()
         assert size == ctypes.sizeof(self.Data), (size, ctypes.sizeof(self.Data))
@@ -195,6 +200,14 @@ class Oracle:
                     np.ctypeslib.as_array(getattr(raw, name))[:n] = np.asarray(v)
                 setattr(raw, flag, 1)
         return d
+
+    def flops(self) -> float:
+        f = self.lib.ksor_flops
+        f.restype = c_double
+        return float(f())
+
+    def flops_reset(self) -> None:
+        self.lib.ksor_flops_reset()
 
     def call(self, name, d: DataView):
         self.fn(name)(ctypes.byref(self.model), ctypes.byref(d.raw))
