@@ -1249,6 +1249,14 @@ extern "C" int ks_model_create(const KsModelDesc* d, KsModel** out) {
     if (b > 0 && (d->body_parent[b] < 0 || d->body_parent[b] >= b)) { delete km; return fail(KS_EINVAL, "ks_model_create: body %d has parent %d (must precede it)", b, d->body_parent[b]); }
     if (d->body_subtree_end[b] <= b || d->body_subtree_end[b] > d->nb) { delete km; return fail(KS_EINVAL, "ks_model_create: bad subtree_end for body %d", b); }
     if (b > 0 && d->body_jtype[b] != kJntFree && d->body_jtype[b] != kJntHinge) { delete km; return fail(KS_EINVAL, "ks_model_create: body %d needs a free or hinge joint", b); }
+    if (b > 0) {  // the joint's coordinates and dofs must lie inside qpos / qvel: the kernel and the tables below index with them
+      const int nqj = d->body_jtype[b] == kJntFree ? 7 : 1, nvj = d->body_jtype[b] == kJntFree ? 6 : 1;
+      if (d->body_qadr[b] < 0 || d->body_qadr[b] + nqj > d->nq || d->body_dofadr[b] < 0 || d->body_dofadr[b] + nvj > d->nv) {
+        delete km;
+        return fail(KS_EINVAL, "ks_model_create: body %d has qpos address %d and dof address %d outside nq=%d / nv=%d", b,
+                    d->body_qadr[b], d->body_dofadr[b], d->nq, d->nv);
+      }
+    }
     for (int k = 0; k < 3; ++k) {
       m.body_pos[b][k] = (float)d->body_pos[b][k]; m.body_ipos[b][k] = (float)d->body_ipos[b][k];
       m.body_inertia[b][k] = (float)d->body_inertia[b][k]; m.jnt_axis[b][k] = (float)d->jnt_axis[b][k];

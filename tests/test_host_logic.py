@@ -389,3 +389,33 @@ def test_benchmark_workload_label_follows_the_model_flag():
     assert "cpu_baseline(args.integrator)" in src and "timed_rollout(torch, args.integrator, N, T, args.steps, args.warmup, args.streams)" in src
     src_cfg = open(os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "ksim_amd", "configs.py")).read()
     assert "kbot_scale_model(seed=seed, integrator=integrator)" in src_cfg
+
+
+def test_model_create_rejects_joint_addresses_outside_the_state():
+    """ks_model_create validates before it touches the GPU: a body whose qpos or dof address (plus the joint's width) leaves
+    qpos / qvel is refused, so the kernel's tables are never indexed out of range."""
+    import ctypes
+
+    from ksim_amd import _lib, _lib_dyn
+    from ksim_amd import model as km
+
+    lib = _lib.load()
+    m = km.kbot_scale_model()
+
+    def create(edit):
+        desc = _lib_dyn.model_desc(m)
+        edit(desc)
+        h = ctypes.c_void_p()
+        rc = lib.ks_model_create(ctypes.byref(desc), ctypes.byref(h))
+        return rc, lib.ks_last_error().decode()
+
+    def set_field(name, b, v):
+        def edit(desc):
+            getattr(desc, name)[b] = v
+        return edit
+
+    for name, b, v in (("body_dofadr", 5, m.nv), ("body_dofadr", 5, -1), ("body_qadr", 7, m.nq), ("body_qadr", 7, -3),
+                       ("body_dofadr", 1, m.nv - 5),   # the free joint needs six dofs
+                       ("body_qadr", 1, m.nq - 6)):    # and seven coordinates
+        rc, msg = create(set_field(name, b, v))
+        assert rc == -1 and f"body {b}" in msg and "outside" in msg, (name, b, v, rc, msg)

@@ -598,3 +598,136 @@ def test_joint_spring_closed_forms():
         og.step(dg)
     q = float(dg.qpos[0])
     assert abs(dg.qvel[0]) < 1e-8 and 4.0 * q == pytest.approx(-1.0 * 9.81 * 0.25 * np.sin(q), rel=1e-6)
+
+
+# ------------------------------------------------------------------ constraint constants, pinned by what MuJoCo documents
+# MuJoCo's "Solver parameters": in constraint space  a1 + d (b v + k r) = (1 - d) a0  with a0 the unconstrained and a1 the
+# constrained acceleration, d the impedance, and for positive solref = (timeconst, dampratio)
+#   b = 2 / (dmax timeconst),  k = d / (dmax^2 timeconst^2 dampratio^2);  timeconst is raised to 2 dt (refsafe);
+# negative solref = (-stiffness, -damping) gives  b = damping / dmax,  k = stiffness d / dmax^2.
+# A ball pushed straight into the plane with friction 1 and impratio 1 is the one-dimensional case of this: its four
+# pyramid edges (0, +-1, 1), (-+1, 0, 1) act as one normal constraint whose inverse inertia 1 / m is exact, so the
+# oracle's vertical acceleration must satisfy the identity to rounding, whatever it does inside.
+def _pressed_ball(r, v, gravity=-9.81, **opts):
+    m = _ball(radius=0.1, mass=2.0, z=0.1 + r, gravity=(0.0, 0.0, gravity), iterations=100, ls_iterations=50, **opts)
+    orc = Oracle(m.arrays())
+    d = orc.data(qvel=np.array([0, 0, v, 0, 0, 0.0]))
+    orc.forward(d)
+    return m, orc, d
+
+
+@pytest.mark.parametrize("solref,solimp,dt,b,k_over_d", [
+    # (timeconst, dampratio), constant impedance d = 0.9: b = 2 / (0.9 * 0.02), k / d = 1 / (0.81 * 0.02^2 * 1)
+    ((0.02, 1.0), (0.9, 0.9, 0.001, 0.5, 2.0), 0.005, 2 / 0.018, 1 / (0.81 * 4e-4)),
+    ((0.05, 0.7), (0.8, 0.8, 0.001, 0.5, 2.0), 0.005, 2 / 0.04, 1 / (0.64 * 25e-4 * 0.49)),
+    # timeconst below 2 dt = 0.01 is raised to 0.01 (refsafe)
+    ((0.001, 1.0), (0.9, 0.9, 0.001, 0.5, 2.0), 0.005, 2 / 0.009, 1 / (0.81 * 1e-4)),
+    # negative solref: stiffness 3000, damping 80, taken as they are
+    ((-3000.0, -80.0), (0.9, 0.9, 0.001, 0.5, 2.0), 0.005, 80 / 0.9, 3000 / 0.81),
+    # impedance saturated at dmax = 0.81 (|r| far beyond the width) while dmin = 0.5: b and k are set by dmax, not dmin
+    ((0.02, 1.0), (0.5, 0.81, 1e-6, 0.5, 2.0), 0.005, 2 / (0.81 * 0.02), 1 / (0.81**2 * 4e-4)),
+])
+def test_contact_acceleration_is_the_documented_spring_damper(solref, solimp, dt, b, k_over_d):
+    dimp = solimp[1]
+    for r, v in ((-0.01, -0.05), (-0.004, 0.02), (-0.02, 0.0)):
+        m, orc, d = _pressed_ball(r, v, solref=solref, solimp=solimp, dt=dt, friction=1.0)
+        assert d.nefc == 4 and (np.array(d.efc_force) > 0).all()
+        want = (1 - dimp) * (-9.81) - dimp * (b * v + k_over_d * dimp * r)
+        assert d.qacc[2] == pytest.approx(want, rel=1e-9), (solref, r, v)
+        assert np.abs(np.delete(np.array(d.qacc), 2)).max() < 1e-9  # nothing sideways, no spin
+
+
+def test_impedance_curve_at_its_documented_points():
+    """solimp = (dmin, dmax, width, midpoint, power): d(0) = dmin, d(>= width) = dmax, and the curve passes through
+    (midpoint, midpoint) in normalised coordinates, so d(midpoint * width) = dmin + midpoint (dmax - dmin).  The impedance is
+    read off the resting acceleration without gravity, a1 = -d k r = -d^2 r / (dmax^2 timeconst^2 dampratio^2)."""
+    dmin, dmax, width, tc = 0.3, 0.9, 0.01, 0.02
+
+    def d_at(r, mid, power):
+        m, orc, d = _pressed_ball(-r, 0.0, gravity=0.0, solref=(tc, 1.0), solimp=(dmin, dmax, width, mid, power), friction=1.0)
+        return dmax * tc * np.sqrt(d.qacc[2] / r)
+
+    for mid, power in ((0.5, 2.0), (0.3, 3.0), (0.7, 1.0), (0.5, 6.0)):
+        assert d_at(1e-9, mid, power) == pytest.approx(dmin, rel=1e-6)
+        assert d_at(width, mid, power) == pytest.approx(dmax, rel=1e-9)
+        assert d_at(3 * width, mid, power) == pytest.approx(dmax, rel=1e-9)
+        assert d_at(mid * width, mid, power) == pytest.approx(dmin + mid * (dmax - dmin), rel=1e-9)
+    # power 1 is the straight line; power 2 with midpoint 0.5 is the smoothstep-like curve with y(1/4) = 1/8, y(3/4) = 7/8
+    assert d_at(0.25 * width, 0.7, 1.0) == pytest.approx(dmin + 0.25 * (dmax - dmin), rel=1e-9)
+    assert d_at(0.25 * width, 0.5, 2.0) == pytest.approx(dmin + 0.125 * (dmax - dmin), rel=1e-9)
+    assert d_at(0.75 * width, 0.5, 2.0) == pytest.approx(dmin + 0.875 * (dmax - dmin), rel=1e-9)
+    # monotone in between
+    ds = [d_at(x * width, 0.4, 3.0) for x in np.linspace(0.01, 0.99, 25)]
+    assert all(b > a for a, b in zip(ds, ds[1:]))
+
+
+def test_contact_relaxes_like_the_documented_oscillator_until_it_would_have_to_pull():
+    """Time domain: without gravity and with constant impedance d = dmax, the penetration obeys r'' = -d b r' - d k r with
+    d b = 2 / timeconst and d k = 1 / (timeconst dampratio)^2: a mass-spring-damper with decay rate 1 / timeconst whose
+    damping ratio is dampratio, whatever the impedance.  Released from rest at depth r0 it follows the textbook solution for
+    as long as that asks the contact to push (r'' > 0); a contact cannot pull, so at the moment the solution's acceleration
+    changes sign the force reaches zero and the ball coasts.  dampratio 1 (critical): r = r0 (1 + t / tc) exp(-t / tc),
+    release at t = tc.  dampratio 2 (overdamped): roots s = (-1 +- sqrt(3) / 2) / tc, release at ln(s2 / s1) / (s1 - s2)."""
+    dimp, tc, dt, r0 = 0.81, 0.02, 1e-4, -0.01
+    for dr in (1.0, 2.0):
+        m = _ball(radius=0.1, mass=2.0, z=0.1 + r0, gravity=(0, 0, 0.0), dt=dt, solref=(tc, dr),
+                  solimp=(dimp, dimp, 0.001, 0.5, 2.0), friction=1.0, iterations=50, ls_iterations=50)
+        orc = Oracle(m.arrays())
+        d = orc.data()
+        steps = int(round(3 * tc / dt))
+        rs, pushing = [], []
+        for _ in range(steps):
+            orc.step(d)  # the force in d is the one that produced this step
+            pushing.append(d.nefc == 4 and float(np.array(d.efc_force).sum()) > 0)
+            rs.append(d.qpos[2] - 0.1)
+        rs, pushing = np.array(rs), np.array(pushing)
+        t = dt * np.arange(1, steps + 1)
+        release = int(np.argmin(pushing))  # first step without a contact force
+        assert pushing[:release].all() and not pushing[release:].any() and (rs[:release] < 0).all()
+        if dr == 1.0:
+            want, t_release = r0 * (1 + t / tc) * np.exp(-t / tc), tc
+        else:
+            w2 = 1 / (tc * dr) ** 2
+            s1, s2 = -1 / tc + np.sqrt(1 / tc**2 - w2), -1 / tc - np.sqrt(1 / tc**2 - w2)
+            want, t_release = r0 * (s2 * np.exp(s1 * t) - s1 * np.exp(s2 * t)) / (s2 - s1), np.log(s2 / s1) / (s1 - s2)
+        np.testing.assert_allclose(rs[:release], want[:release], rtol=5e-3)  # first-order integrator at dt = tc / 200
+        assert t[release] == pytest.approx(t_release, rel=0.02)
+        v_release = (rs[release] - rs[release - 1]) / dt
+        np.testing.assert_allclose(np.diff(rs[release:]) / dt, v_release, rtol=1e-9)  # coasting afterwards
+
+
+@pytest.mark.parametrize("mu", [0.3, 1.0, 2.0])
+def test_resting_pyramid_carries_the_weight_for_any_friction(mu):
+    m = _ball(z=0.1, friction=mu)
+    orc = Oracle(m.arrays())
+    d = orc.data()
+    for _ in range(3000):
+        orc.step(d)
+    assert np.abs(d.qvel).max() < 1e-7 and d.nefc == 4
+    f = np.array(d.efc_force)
+    assert f.sum() == pytest.approx(2.0 * 9.81, rel=1e-7)  # every edge has normal component 1
+    assert np.ptp(f) < 1e-9 * f.sum()                      # and by symmetry an equal share
+    np.testing.assert_allclose(np.array(d.qfrc_constraint)[:3], [0, 0, 2.0 * 9.81], atol=1e-6)
+
+
+@pytest.mark.parametrize("dof_solref,b,k_over_d", [
+    ((0.04, 1.0), 2 / (0.9 * 0.04), 1 / (0.81 * 16e-4)),
+    ((0.003, 0.5), 2 / (0.9 * 0.01), 1 / (0.81 * 1e-4 * 0.25)),  # timeconst raised to 2 dt = 0.01
+    ((-500.0, -20.0), 20 / 0.9, 500 / 0.81),
+])
+def test_joint_limit_acceleration_is_the_documented_spring_damper(dof_solref, b, k_over_d):
+    """The same identity a1 + d (b v + k r) = (1 - d) a0 for a limit row: one hinge (its inverse inertia is exact), pushed
+    past its upper limit.  The constraint coordinate is r = upper - q, so its velocity and acceleration are minus the
+    joint's; gravity acts through a0 = the unconstrained joint acceleration, read from the same state without the range."""
+    dimp = 0.9
+    kw = dict(n_links=1, length=0.5, mass=1.0, damping=0.0)
+    m = km.pendulum_chain_model(joint_range=(-1.0, 0.4), dof_solref=dof_solref, dof_solimp=(dimp, dimp, 0.01, 0.5, 2.0), **kw)
+    free = km.pendulum_chain_model(**kw)
+    ai = dict(m.arrays()); ai["iterations"] = 100; ai["ls_iterations"] = 50
+    for q, qd in ((0.43, 0.2), (0.44, -0.05), (0.47, 0.0)):  # deep enough that the limit has to push against gravity
+        d, f = Oracle(ai).data(np.array([q]), np.array([qd])), Oracle(free.arrays()).data(np.array([q]), np.array([qd]))
+        Oracle(ai).forward(d); Oracle(free.arrays()).forward(f)
+        assert d.nefc == 1 and d.efc_force[0] > 0
+        r, v, a0 = 0.4 - q, -qd, -float(f.qacc[0])
+        a1 = (1 - dimp) * a0 - dimp * (b * v + k_over_d * dimp * r)
+        assert -float(d.qacc[0]) == pytest.approx(a1, rel=1e-9), (dof_solref, q, qd)
