@@ -398,9 +398,15 @@ typedef struct KsTermDesc {
   float p0, p1, p2, p3; /* min_height | min_z,max_z,final_min_z,final_max_z | max_radians | max_vel | max_dist | max_sec,disable_level(<0: never) */
 } KsTermDesc;
 
-/* Resets (replaces the Reset list applied in MjxEngine.reset, engine.py:207-220, ksim/resets.py:122-189,
- * 308-334): qpos[i] <- clip(base[i] + u*mag[i]*(level if by_level[i]), lo[i], hi[i]) with u ~ U(-1,1);
- * optional heading: quat <- quat * yaw(U(-pi,pi)); qvel, time and last_ctrl <- 0. */
+/* Resets (replaces the Reset list applied in MjxEngine.reset, engine.py:207-220, ksim/resets.py:44-189,
+ * 284-354): qpos[i] <- clip(start[i] + u*mag[i]*(level if by_level[i]), lo[i], hi[i]) with u ~ U(-1,1) and
+ * start[i] = base[i], or for elements marked reset_from_motion the reference-motion frame drawn for the env plus base[i]
+ * (InitialMotionStateReset, resets.py:284-306; time <- frame * ctrl_dt then, otherwise 0);
+ * reset_hfield: z <- hfield[ix, iy] + base[2] with the cell looked up from the new x, y (HFieldXYPositionReset, resets.py:45-90);
+ * then the base orientation: quat <- quat * yaw(U(-pi,pi)) (RandomHeadingReset, resets.py:309-320) and
+ * quat <- quat * euler(roll, pitch, 0) with roll and pitch from ONE uniform draw mapped to their ranges, as one key
+ * gives them (RandomPitchRollReset, resets.py:338-354), in the order reset_pitch_roll says;
+ * qvel, warm start and last_ctrl <- 0. */
 #define KS_MAX_OBS 512
 #define KS_MAX_TERMS 16
 typedef struct KsTermsDesc {
@@ -416,6 +422,11 @@ typedef struct KsTermsDesc {
   KsTermDesc terms[KS_MAX_TERMS];
   float reset_base[KS_MAX_QPOS], reset_mag[KS_MAX_QPOS], reset_lo[KS_MAX_QPOS], reset_hi[KS_MAX_QPOS];
   int32_t reset_by_level[KS_MAX_QPOS];
+  int32_t reset_from_motion[KS_MAX_QPOS]; /* 1: start from the reference-motion frame (KsTerminateIO.reset_motion_qpos) */
+  int32_t reset_pitch_roll;               /* 0 none, 1 applied after the heading, 2 applied before it */
+  float reset_pitch[2], reset_roll[2];    /* (min, max) in radians */
+  int32_t reset_hfield;                   /* 1: base height from the height field (KsTerminateIO.reset_hfield) */
+  float hfield_bound[2];                  /* half extents (x, y) of the height field */
 } KsTermsDesc;
 typedef struct KsTerms KsTerms;
 int ks_terms_create(const KsTermsDesc* desc /*host*/, KsTerms** out);
@@ -466,6 +477,13 @@ typedef struct KsTerminateIO {
   uint8_t* reset_mask;       /* (N) = done, nullable */
   int32_t* episode_length;   /* (N) control steps in the current episode, in/out, nullable */
   const float* reset_uniform; /* (N, nq + 1) U(-1,1) draws (last one: heading), nullable -> Philox */
+  const float* reset_pitch_roll_uniform; /* (N) U[0,1) draws of RandomPitchRollReset, nullable -> Philox */
+  const float* reset_motion_qpos;  /* (reset_motion_frames, nq) reference motion, required when the table marks elements */
+  int32_t reset_motion_frames;
+  float reset_motion_dt;           /* ctrl_dt of the motion: time <- frame * dt */
+  const int32_t* reset_frame;      /* (N) frame per env, nullable -> floor(U[0,1) * frames) from Philox */
+  const float* reset_hfield;       /* (hfield_nx, hfield_ny) heights, required when reset_hfield is set */
+  int32_t hfield_nx, hfield_ny;
   KsRng rng;
   int32_t apply_reset;       /* 0: report terminations only; 1: reset finished envs; 2: reset every env (initial reset) */
   /* event timers of the envs that start a fresh episode: a new interval each (engine.py:226-232) */

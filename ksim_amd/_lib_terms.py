@@ -44,7 +44,9 @@ class KsTermsDesc(ctypes.Structure):
                 ("obs", KsObsElem * KS_MAX_OBS), ("terms", KsTermDesc * KS_MAX_TERMS),
                 ("reset_base", c_float * KS_MAX_QPOS), ("reset_mag", c_float * KS_MAX_QPOS),
                 ("reset_lo", c_float * KS_MAX_QPOS), ("reset_hi", c_float * KS_MAX_QPOS),
-                ("reset_by_level", c_int32 * KS_MAX_QPOS)]
+                ("reset_by_level", c_int32 * KS_MAX_QPOS), ("reset_from_motion", c_int32 * KS_MAX_QPOS),
+                ("reset_pitch_roll", c_int32), ("reset_pitch", c_float * 2), ("reset_roll", c_float * 2),
+                ("reset_hfield", c_int32), ("hfield_bound", c_float * 2)]
 
 
 class KsRng(ctypes.Structure):
@@ -75,7 +77,10 @@ class KsTerminateIO(ctypes.Structure):
                 ("qacc_warmstart", c_void_p), ("time", c_void_p), ("last_ctrl", c_void_p), ("components", c_void_p),
                 ("done", c_void_p), ("success", c_void_p), ("traj_qpos", c_void_p), ("traj_qvel", c_void_p),
                 ("traj_time", c_void_p), ("reset_mask", c_void_p), ("episode_length", c_void_p),
-                ("reset_uniform", c_void_p), ("rng", KsRng), ("apply_reset", c_int32), ("n_events", c_int32),
+                ("reset_uniform", c_void_p), ("reset_pitch_roll_uniform", c_void_p), ("reset_motion_qpos", c_void_p),
+                ("reset_motion_frames", c_int32), ("reset_motion_dt", c_float), ("reset_frame", c_void_p),
+                ("reset_hfield", c_void_p), ("hfield_nx", c_int32), ("hfield_ny", c_int32),
+                ("rng", KsRng), ("apply_reset", c_int32), ("n_events", c_int32),
                 ("event_interval", (c_float * 2) * KS_MAX_EVENTS), ("event_state", c_void_p),
                 ("event_reset_uniform", c_void_p), ("event_force", c_void_p), ("contact_dist", c_void_p),
                 ("action_latency", c_void_p), ("latency_lo", c_float), ("latency_hi", c_float), ("zero_offset", c_void_p),

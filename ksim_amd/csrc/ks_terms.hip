@@ -203,6 +203,10 @@ struct TerminateArgs {
   KsRandomVar zero_offset_rv, action_bias_rv, torque_bias_rv, kp_scale_rv, kd_scale_rv, torque_limit_scale_rv;
   const float *episode_uniform, *episode_normal;
   int redraw;  // any of the per-episode buffers is given
+  const float *reset_pitch_roll_uniform, *reset_motion_qpos, *reset_hfield;
+  const int32_t* reset_frame;
+  int reset_motion_frames, hfield_nx, hfield_ny;
+  float reset_motion_dt;
 };
 
 // value of a random variable from its standard draws (ksim/noise.py:74-121)
@@ -221,6 +225,7 @@ constexpr int kTermEnvs = 32;
 __global__ __launch_bounds__(256) void terminate_kernel(TerminateArgs a) {
   __shared__ int s_bad[kTermEnvs];    // non-finite state seen
   __shared__ int s_reset[kTermEnvs];  // env starts a fresh episode
+  __shared__ int s_frame[kTermEnvs];  // its frame of the reference motion
   const KsTermsDesc& d = a.t->d;
   const int tid = threadIdx.x;
   const int64_t e0 = (int64_t)blockIdx.x * kTermEnvs;
@@ -287,7 +292,17 @@ __global__ __launch_bounds__(256) void terminate_kernel(TerminateArgs a) {
     s_reset[tid] = do_reset ? 1 : 0;
     if (a.reset_mask) a.reset_mask[e] = do_reset ? 1 : 0;
     if (a.episode_length) a.episode_length[e] = do_reset ? 0 : a.episode_length[e] + 1;
-    if (do_reset && a.time) a.time[e] = 0.f;
+    int frame = 0;
+    if (do_reset && a.reset_motion_qpos) {  // resets.py:291: randint(0, num_frames)
+      if (a.reset_frame) frame = a.reset_frame[e];
+      else {
+        const uint64_t st = a.rng.step + (a.rng.step_base ? *a.rng.step_base : 0ull);
+        frame = (int)(u01(draw(a.rng.seed, st, kRngReset, (uint64_t)e, (uint32_t)nq + 2u).x) * (float)a.reset_motion_frames);
+      }
+      frame = frame < 0 ? 0 : (frame >= a.reset_motion_frames ? a.reset_motion_frames - 1 : frame);
+    }
+    s_frame[tid] = frame;
+    if (do_reset && a.time) a.time[e] = a.reset_motion_qpos ? (float)frame * a.reset_motion_dt : 0.f;
     if (do_reset)
       for (int k = 0; k < a.n_events; ++k) {
         float u;
@@ -309,8 +324,22 @@ __global__ __launch_bounds__(256) void terminate_kernel(TerminateArgs a) {
     if (a.reset_uniform) u = a.reset_uniform[e * (nq + 1) + i];
     else u = 2.f * u01(draw(a.rng.seed, step, kRngReset, (uint64_t)e, (uint32_t)i).x) - 1.f;
     const float mag = d.reset_mag[i] * (d.reset_by_level[i] ? a.level : 1.f);
-    const float x = d.reset_base[i] + u * mag;
+    float start = d.reset_base[i];
+    if (d.reset_from_motion[i] && a.reset_motion_qpos) start += a.reset_motion_qpos[(int64_t)s_frame[le] * nq + i];
+    const float x = start + u * mag;
     qb[idx] = fminf(fmaxf(x, d.reset_lo[i]), d.reset_hi[i]);
+  }
+  if (d.reset_hfield && a.reset_hfield && nq >= 3) {
+    __syncthreads();  // x and y written above are read back by the env's own lane
+    if (tid < ne && s_reset[tid]) {
+      float* q = qb + tid * nq;
+      const int nx = a.hfield_nx, ny = a.hfield_ny;
+      int ix = (int)(((q[0] + d.hfield_bound[0]) / (2.f * d.hfield_bound[0])) * (float)(nx - 1));  // truncation, as astype(int32)
+      int iy = (int)(((q[1] + d.hfield_bound[1]) / (2.f * d.hfield_bound[1])) * (float)(ny - 1));
+      ix = ix < 0 ? 0 : (ix > nx - 1 ? nx - 1 : ix);
+      iy = iy < 0 ? 0 : (iy > ny - 1 ? ny - 1 : iy);
+      q[2] = a.reset_hfield[(int64_t)ix * ny + iy] + d.reset_base[2];
+    }
   }
   for (int idx = tid; idx < ne * nv; idx += 256) {
     if (!s_reset[idx / nv]) continue;
@@ -353,18 +382,38 @@ __global__ __launch_bounds__(256) void terminate_kernel(TerminateArgs a) {
       }
     }
   }
-  if (a.random_heading && nq >= 7) {
+  if ((a.random_heading || d.reset_pitch_roll) && nq >= 7) {
     __syncthreads();  // the base orientation written above is read back by the env's own lane
     if (tid < ne && s_reset[tid]) {
       const int64_t e = e0 + tid;
       float* q = qb + tid * nq;
-      float u;
-      if (a.reset_uniform) u = a.reset_uniform[e * (nq + 1) + nq];
-      else u = 2.f * u01(draw(a.rng.seed, step, kRngReset, (uint64_t)e, (uint32_t)nq).x) - 1.f;
-      const float h = 0.5f * 3.14159265358979323846f * u;  // yaw/2, yaw ~ U(-pi, pi)
-      const float cw = cosf(h), sz = sinf(h);
-      const float w = q[3], x = q[4], y = q[5], z = q[6];
-      q[3] = w * cw - z * sz; q[4] = x * cw + y * sz; q[5] = y * cw - x * sz; q[6] = z * cw + w * sz;
+      auto heading = [&]() {
+        float u;
+        if (a.reset_uniform) u = a.reset_uniform[e * (nq + 1) + nq];
+        else u = 2.f * u01(draw(a.rng.seed, step, kRngReset, (uint64_t)e, (uint32_t)nq).x) - 1.f;
+        const float h = 0.5f * 3.14159265358979323846f * u;  // yaw/2, yaw ~ U(-pi, pi)
+        const float cw = cosf(h), sz = sinf(h);
+        const float w = q[3], x = q[4], y = q[5], z = q[6];
+        q[3] = w * cw - z * sz; q[4] = x * cw + y * sz; q[5] = y * cw - x * sz; q[6] = z * cw + w * sz;
+      };
+      auto pitch_roll = [&]() {
+        // one draw for both angles: the reference samples pitch and roll from the same key (resets.py:348-349)
+        float u;
+        if (a.reset_pitch_roll_uniform) u = a.reset_pitch_roll_uniform[e];
+        else u = u01(draw(a.rng.seed, step, kRngReset, (uint64_t)e, (uint32_t)nq + 1u).x);
+        const float pitch = d.reset_pitch[0] + u * (d.reset_pitch[1] - d.reset_pitch[0]);
+        const float roll = d.reset_roll[0] + u * (d.reset_roll[1] - d.reset_roll[0]);
+        const float cr = cosf(0.5f * roll), sr = sinf(0.5f * roll), cp = cosf(0.5f * pitch), sp = sinf(0.5f * pitch);
+        const float bw = cr * cp, bx = sr * cp, by = cr * sp, bz = -sr * sp;  // euler (roll, pitch, 0) as a quaternion
+        const float w = q[3], x = q[4], y = q[5], z = q[6];
+        q[3] = w * bw - x * bx - y * by - z * bz;
+        q[4] = w * bx + x * bw + y * bz - z * by;
+        q[5] = w * by - x * bz + y * bw + z * bx;
+        q[6] = w * bz + x * by - y * bx + z * bw;
+      };
+      if (d.reset_pitch_roll == 2) pitch_roll();
+      if (a.random_heading) heading();
+      if (d.reset_pitch_roll == 1) pitch_roll();
     }
   }
 }
@@ -991,6 +1040,10 @@ extern "C" int ks_terms_create(const KsTermsDesc* d, KsTerms** out) {
   if (d->nq < 0 || d->nq > KS_MAX_QPOS || d->nv < 0 || d->nu < 0 || d->nb < 1) return fail(KS_EINVAL, "ks_terms_create: bad sizes");
   const int src_dim[KS_SRC_COUNT] = {d->nq, d->nv, d->nv, d->nu, d->action_dim > 0 ? d->action_dim : d->nu, d->command_dim, 1, d->nb * 3, d->nb * 4, d->nb * 6, 0, d->ns, d->nb * 10, d->nb * 6};
   if (d->ns < 0 || d->carry_dim < 0) return fail(KS_EINVAL, "ks_terms_create: negative sphere count or carry size");
+  if (d->reset_pitch_roll < 0 || d->reset_pitch_roll > 2) return fail(KS_EINVAL, "ks_terms_create: reset_pitch_roll must be 0, 1 or 2");
+  if ((d->reset_pitch_roll || d->random_heading) && d->nq < 7) return fail(KS_EINVAL, "ks_terms_create: an orientation reset needs a floating base");
+  if (d->reset_hfield && (d->nq < 3 || !(d->hfield_bound[0] > 0.f) || !(d->hfield_bound[1] > 0.f)))
+    return fail(KS_EINVAL, "ks_terms_create: the height-field reset needs a floating base and positive half extents");
   for (int k = 0; k < d->obs_dim; ++k) {
     const KsObsElem& el = d->obs[k];
     if (el.src < 0 || el.src >= KS_SRC_COUNT) return fail(KS_EINVAL, "ks_terms_create: obs %d: bad source %d", k, el.src);
@@ -1124,6 +1177,19 @@ extern "C" int ks_terminate_reset(const KsTerms* t, ks_stream_t stream, const Ks
   a.zero_offset_rv = io->zero_offset_rv; a.action_bias_rv = io->action_bias_rv; a.torque_bias_rv = io->torque_bias_rv;
   a.kp_scale_rv = io->kp_scale_rv; a.kd_scale_rv = io->kd_scale_rv; a.torque_limit_scale_rv = io->torque_limit_scale_rv;
   a.episode_uniform = io->episode_uniform; a.episode_normal = io->episode_normal;
+  a.reset_pitch_roll_uniform = io->reset_pitch_roll_uniform; a.reset_frame = io->reset_frame;
+  bool from_motion = false;
+  for (int i = 0; i < d.nq; ++i) from_motion |= d.reset_from_motion[i] != 0;
+  if (from_motion && io->apply_reset) {
+    if (!io->reset_motion_qpos || io->reset_motion_frames < 1)
+      return fail(KS_EINVAL, "ks_terminate_reset: the reset table starts from a reference motion: reset_motion_qpos and its frame count are required");
+    a.reset_motion_qpos = io->reset_motion_qpos; a.reset_motion_frames = io->reset_motion_frames; a.reset_motion_dt = io->reset_motion_dt;
+  }
+  if (d.reset_hfield && io->apply_reset) {
+    if (!io->reset_hfield || io->hfield_nx < 1 || io->hfield_ny < 1)
+      return fail(KS_EINVAL, "ks_terminate_reset: the reset table reads a height field: reset_hfield and its shape are required");
+    a.reset_hfield = io->reset_hfield; a.hfield_nx = io->hfield_nx; a.hfield_ny = io->hfield_ny;
+  }
   a.redraw = (a.action_latency || a.zero_offset || a.act_action_bias || a.act_torque_bias || a.act_kp_scale || a.act_kd_scale ||
               a.act_torque_limit_scale) ? 1 : 0;
   if (a.action_latency && !(io->latency_lo >= 0.f && io->latency_hi >= io->latency_lo))

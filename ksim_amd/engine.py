@@ -187,7 +187,8 @@ class HipEngine(PhysicsEngine):
 
     def episode_args(self, state: PhysicsState, draws: Mapping | None = None) -> dict:
         """What `EnvTerms.terminate_reset(episode=...)` takes: the per-episode buffers of `state`, the random variables
-        behind them, and optionally explicit draws {"uniform", "normal"}, each (N, 3 nu + 4)."""
+        behind them, and optionally explicit draws {"uniform", "normal"}, each (N, 3 nu + 4), and for the resets that
+        use them {"pitch_roll_uniform"} (N) in [0, 1) and {"frame"} (N, int32)."""
         out = dict(action_latency=state.action_latency, zero_offset=state.zero_offset,
                    latency_range=(self.data.min_action_latency_step, self.data.max_action_latency_step),
                    zero_offset_rv=self.data.zero_offset)
@@ -200,7 +201,8 @@ class HipEngine(PhysicsEngine):
                        kp_scale_rv=rv(act.kp_scale) or RandomVariable(mean=1.0), kd_scale_rv=rv(act.kd_scale) or RandomVariable(mean=1.0),
                        torque_limit_scale_rv=rv(act.torque_limit_scale) or RandomVariable(mean=1.0))
         if draws:
-            out.update(episode_uniform=draws.get("uniform"), episode_normal=draws.get("normal"))
+            out.update(episode_uniform=draws.get("uniform"), episode_normal=draws.get("normal"),
+                       reset_pitch_roll_uniform=draws.get("pitch_roll_uniform"), reset_frame=draws.get("frame"))
         return out
 
     def _initial_event_states(self, N: int, gen, dev) -> dict:

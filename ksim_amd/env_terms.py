@@ -85,7 +85,14 @@ def compile_terms(model: KinematicModel, observations: Mapping[str, Observation]
         d.reset_base[i], d.reset_mag[i] = tab["base"][i], tab["mag"][i]
         d.reset_lo[i], d.reset_hi[i] = max(tab["lo"][i], -big), min(tab["hi"][i], big)
         d.reset_by_level[i] = int(tab["by_level"][i])
+        d.reset_from_motion[i] = int(tab["motion"][i])
     d.random_heading = int(tab["heading"])
+    d.reset_pitch_roll = int(tab["pitch_roll"])
+    d.reset_pitch[0], d.reset_pitch[1] = (float(x) for x in tab["pitch"])
+    d.reset_roll[0], d.reset_roll[1] = (float(x) for x in tab["roll"])
+    if tab["hfield"] is not None:
+        d.reset_hfield = 1
+        d.hfield_bound[0], d.hfield_bound[1] = (float(x) for x in tab["hfield"]["bound"])
     d.nonfinite_terminates = int(terminate_on_nonfinite)
     return d, obs_slices, sources_used, has_bias, tab
 
@@ -102,6 +109,7 @@ class EnvTerms:
         d, self.obs_slices, self.sources_used, self.has_bias, self.reset_table = compile_terms(
             model, self.observations, self.terminations, self.resets, self.command_dim, terminate_on_nonfinite, action_dim)
         self.action_dim = int(d.action_dim)
+        self._motion = self._hfield = None  # device copies of the reset tables' data, made on first use
         self.obs_dim, self.n_terms, self.carry_dim = int(d.obs_dim), int(d.n_terms), int(d.carry_dim)
         self._handle = ctypes.c_void_p()
         _lib.check(lib.ks_terms_create(ctypes.byref(d), ctypes.byref(self._handle)))
@@ -156,7 +164,8 @@ class EnvTerms:
                         contact_dist=None, apply_reset: bool = True, episode: Mapping | None = None) -> None:
         """`episode`: the per-episode quantities that the envs starting a fresh episode re-draw (engine.py:222-245), as
         `HipEngine.episode_args` builds them: buffers `action_latency`, `zero_offset`, `act_*`, the matching random
-        variables, and optionally explicit draws `episode_uniform` / `episode_normal` (N, 3 nu + 4)."""
+        variables, and optionally explicit draws `episode_uniform` / `episode_normal` (N, 3 nu + 4),
+        `reset_pitch_roll_uniform` (N) in [0, 1) and `reset_frame` (N, int32) for the resets that draw them."""
         m = self.model
         qpos = state["qpos"]
         N = qpos.shape[0]
@@ -202,6 +211,24 @@ class EnvTerms:
                 if tuple(event_force.shape) != (len(event_intervals), N, T.KS_EVENT_FORCE_STATE):
                     raise _lib.KsError("force-push state must be (n_events, N, KS_EVENT_FORCE_STATE)")
                 io.event_force = event_force.data_ptr()
+        # tables of the resets that read data: the reference motion and the height field live on the device from first use
+        tab = self.reset_table
+        if apply_reset and tab["motion"].any():
+            if self._motion is None:
+                self._motion = torch.from_numpy(tab["motion_qpos"]).to(qpos.device)
+            io.reset_motion_qpos, io.reset_motion_frames = self._motion.data_ptr(), self._motion.shape[0]
+            io.reset_motion_dt = tab["motion_dt"]
+        if apply_reset and tab["hfield"] is not None:
+            if self._hfield is None:
+                self._hfield = torch.from_numpy(tab["hfield"]["data"]).to(qpos.device)
+            io.reset_hfield, io.hfield_nx, io.hfield_ny = self._hfield.data_ptr(), self._hfield.shape[0], self._hfield.shape[1]
+        for name, dt in (("reset_pitch_roll_uniform", torch.float32), ("reset_frame", torch.int32)):
+            t = (episode or {}).get(name)
+            if t is not None:
+                _lib.require_cuda(t, dtype=dt)
+                if tuple(t.shape) != (N,):
+                    raise _lib.KsError(f"{name}: expected ({N},), got {tuple(t.shape)}")
+                setattr(io, name, t.data_ptr())
         if episode:
             nu, ned = m.nu, 3 * m.nu + 4
             shapes = dict(action_latency=(N,), zero_offset=(N, nu), act_action_bias=(N, nu), act_torque_bias=(N, nu),

@@ -709,3 +709,51 @@ def site_accelerometer(qacc6, xquat_body, omega_world, site_pos, site_quat, grav
     alpha = rotate_vector_by_quat(qacc6[..., 3:6], q)
     a = qacc6[..., :3] + np.cross(alpha, r) + np.cross(w, np.cross(w, r)) - np.asarray(gravity, np.float64)
     return rotate_vector_by_quat(rotate_vector_by_quat(a, q, inverse=True), np.asarray(site_quat, np.float64), inverse=True)
+
+
+# ------------------------------------------------------------------ resets (ksim/resets.py), one env, explicit draws
+def xy_position_reset(qpos, ux, uy, *, x_range, y_range, padded_bounds, z=None, hfield=None, hfield_bounds=None,
+                      robot_base_height=0.0):
+    """PlaneXYPositionReset (resets.py:93-120) with `z` = the plane's height, or HFieldXYPositionReset (resets.py:45-90)
+    with `hfield` (nx, ny) and `hfield_bounds` = (x_bound, y_bound, z_top).  ux, uy in [-1, 1)."""
+    lower_x, upper_x, lower_y, upper_y = padded_bounds
+    q = np.array(qpos, dtype=np.float64)
+    q[0] = np.clip(ux * x_range, lower_x, upper_x)
+    q[1] = np.clip(uy * y_range, lower_y, upper_y)
+    if hfield is None:
+        q[2] = z + robot_base_height
+        return q
+    x_bound, y_bound, z_top = hfield_bounds
+    nx, ny = hfield.shape
+    ix = int(np.clip(np.int32(((q[0] + x_bound) / (2 * x_bound)) * (nx - 1)), 0, nx - 1))
+    iy = int(np.clip(np.int32(((q[1] + y_bound) / (2 * y_bound)) * (ny - 1)), 0, ny - 1))
+    q[2] = hfield[ix, iy] + z_top + robot_base_height
+    return q
+
+
+def initial_motion_state_reset(qpos, frame, motion_qpos, ctrl_dt, freejoint):
+    """InitialMotionStateReset (resets.py:284-306): returns (qpos, time)."""
+    q = np.array(qpos, dtype=np.float64)
+    ref = np.asarray(motion_qpos, dtype=np.float64)[frame % len(motion_qpos)]
+    if freejoint:
+        q[:] = ref
+    else:
+        q[7:] = ref[7:]
+    return q, frame * ctrl_dt
+
+
+def random_heading_reset(qpos, u):
+    """RandomHeadingReset (resets.py:309-320): quat <- quat * yaw, yaw = pi u, u in [-1, 1)."""
+    q = np.array(qpos, dtype=np.float64)
+    q[3:7] = quat_mul(q[3:7], euler_to_quat(np.array([0.0, 0.0, np.pi * u])))
+    return q
+
+
+def random_pitch_roll_reset(qpos, u01, pitch_range, roll_range):
+    """RandomPitchRollReset (resets.py:338-354): both angles come from the SAME key, hence from one uniform number
+    u01 in [0, 1): pitch = min_p + u (max_p - min_p), roll = min_r + u (max_r - min_r); quat <- quat * euler(roll, pitch, 0)."""
+    q = np.array(qpos, dtype=np.float64)
+    pitch = pitch_range[0] + u01 * (pitch_range[1] - pitch_range[0])
+    roll = roll_range[0] + u01 * (roll_range[1] - roll_range[0])
+    q[3:7] = quat_mul(q[3:7], euler_to_quat(np.array([roll, pitch, 0.0])))
+    return q

@@ -212,6 +212,94 @@ def test_reset_predication():
     assert (np.abs(j) <= 0.25 + 1e-6).all() and j.std() > 0.03
 
 
+def test_motion_height_field_and_pitch_roll_resets_match_the_reference_list_order():
+    """InitialMotionStateReset, HFieldXYPositionReset / PlaneXYPositionReset and RandomPitchRollReset (resets.py:45-120,
+    284-354) through the reset kernel, in three reset lists whose order matters, against the oracle's restatement applied
+    in list order with the same draws; then with the kernel's own draws, through what the draws must satisfy."""
+    from ksim_amd import model as km, resets as rs, terminations as tm
+    from ksim_amd.env_terms import EnvTerms
+    from ksim_amd.priors import MotionReferenceData
+
+    m = km.kbot_scale_model()
+    N, F = 96, 11
+    rng = np.random.default_rng(21)
+    mq = rng.normal(size=(F, m.nq)) * 0.3
+    mq[:, 3:7] /= np.linalg.norm(mq[:, 3:7], axis=1, keepdims=True)
+    motion = MotionReferenceData(qpos=mq, qvel=np.zeros((F, m.nv)), cartesian_poses={}, ctrl_dt=0.02)
+    hf = rng.uniform(0.0, 0.4, size=(9, 7))
+    hreset = rs.HFieldXYPositionReset(bounds=(4.0, 3.0, 0.25, 0.1), padded_bounds=(-3.0, 3.0, -2.0, 2.0), x_range=5.0, y_range=2.5,
+                                      hfield_data=hf, robot_base_height=0.9)
+    preset = rs.PlaneXYPositionReset(bounds=(5.0, 5.0, 0.05), padded_bounds=(-1.0, 1.0, -4.0, 4.0), x_range=2.0, y_range=3.0,
+                                     robot_base_height=0.8)
+    pr = rs.RandomPitchRollReset(pitch_range=(-0.3, 0.5), roll_range=(0.2, -0.4))
+    cases = {
+        "motion joints, height, pitch/roll then heading": [rs.InitialMotionStateReset(reference_motion=motion), rs.RandomHeightReset(range=(0.1, 0.3)), pr, rs.RandomHeadingReset()],
+        "height field, heading then pitch/roll": [hreset, rs.RandomHeadingReset(), pr],
+        "whole motion frame, plane overrides the position": [rs.InitialMotionStateReset(reference_motion=motion, freejoint=True), preset, pr],
+    }
+    u = rng.uniform(-1, 1, size=(N, m.nq + 1))
+    upr = rng.random(N)
+    frames = rng.integers(0, F, N).astype(np.int32)
+    for name, resets in cases.items():
+        terms = EnvTerms(m, {}, {"h": tm.MinimumHeightTermination(0.5)}, resets)
+        s = _state(m, N, 5)
+        st = dict(qpos=t32(s["qpos"]), qvel=t32(s["qvel"]), qacc_warmstart=t32(s["qacc"]), time=t32(s["time"]), last_ctrl=t32(s["last"]))
+        draws = dict(reset_pitch_roll_uniform=t32(upr), reset_frame=torch.tensor(frames, device=DEV))
+        terms.terminate_reset(st, level=0.7, apply_reset=2, reset_uniform=t32(u), episode=draws)
+        got_q, got_t = st["qpos"].cpu().numpy(), st["time"].cpu().numpy()
+        assert np.abs(st["qvel"].cpu().numpy()).max() == 0
+        for e in range(N):
+            q, t = m.qpos0.astype(np.float64).copy(), 0.0
+            for r in resets:  # engine.py:209-211
+                if isinstance(r, rs.InitialMotionStateReset):
+                    q, t = ot.initial_motion_state_reset(q, int(frames[e]), mq, 0.02, r.freejoint)
+                elif isinstance(r, rs.RandomHeightReset):
+                    q[2] += r.range[0] + 0.5 * (u[e, 2] + 1) * (r.range[1] - r.range[0])
+                elif isinstance(r, rs.RandomPitchRollReset):
+                    q = ot.random_pitch_roll_reset(q, upr[e], r.pitch_range, r.roll_range)
+                elif isinstance(r, rs.RandomHeadingReset):
+                    q = ot.random_heading_reset(q, u[e, m.nq])
+                elif isinstance(r, rs.HFieldXYPositionReset):
+                    q = ot.xy_position_reset(q, u[e, 0], u[e, 1], x_range=r.x_range, y_range=r.y_range, padded_bounds=r.padded_bounds,
+                                             hfield=hf.astype(np.float32), hfield_bounds=r.bounds[:3], robot_base_height=r.robot_base_height)
+                else:
+                    q = ot.xy_position_reset(q, u[e, 0], u[e, 1], x_range=r.x_range, y_range=r.y_range, padded_bounds=r.padded_bounds,
+                                             z=r.bounds[2], robot_base_height=r.robot_base_height)
+            np.testing.assert_allclose(got_q[e], q, atol=2e-6, err_msg=f"{name}, env {e}")
+            assert got_t[e] == pytest.approx(t, abs=1e-6), name
+        terms.close()
+    # a height-field cell boundary is a discontinuity: no unclipped x above may sit near one (the clipped ones land on
+    # cells 1 and 7 exactly, in float32 as in float64)
+    x = u[:, 0] * 5.0
+    cells = ((x[np.abs(x) < 3] + 4.0) / 8.0) * 8
+    assert np.abs(cells - np.round(cells)).min() > 1e-4
+
+    # the kernel's own draws: frames cover the motion, time = frame * dt, the joints are that frame's, and the base
+    # orientation is quat0 * euler(roll, pitch, 0) with roll and pitch at the same fraction of their ranges
+    N2 = 4096
+    terms = EnvTerms(m, {}, {}, [rs.InitialMotionStateReset(reference_motion=motion), pr])
+    st = dict(qpos=torch.zeros(N2, m.nq, device=DEV), qvel=torch.zeros(N2, m.nv, device=DEV), time=torch.zeros(N2, device=DEV))
+    terms.terminate_reset(st, apply_reset=2, seed=3, step=5)
+    q, t = st["qpos"].cpu().numpy().astype(np.float64), st["time"].cpu().numpy()
+    fr = np.round(t / 0.02).astype(int)
+    assert np.abs(t - fr * 0.02).max() < 1e-6 and set(fr) == set(range(F))
+    counts = np.bincount(fr, minlength=F)
+    assert counts.min() > 0.7 * N2 / F and counts.max() < 1.3 * N2 / F
+    np.testing.assert_allclose(q[:, 7:], mq[fr][:, 7:], atol=1e-6)
+    w, x, y, z = q[:, 3], q[:, 4], q[:, 5], q[:, 6]  # base quat0 is the identity here
+    roll = np.arctan2(2 * (w * x + y * z), 1 - 2 * (x * x + y * y))
+    pitch = np.arcsin(np.clip(2 * (w * y - z * x), -1, 1))
+    fp, frl = (pitch + 0.3) / 0.8, (roll - 0.2) / -0.6
+    assert fp.min() >= -1e-5 and fp.max() <= 1 + 1e-5 and fp.std() > 0.25
+    np.testing.assert_allclose(fp, frl, atol=2e-5)
+    np.testing.assert_allclose(np.arctan2(2 * (w * z + x * y), 1 - 2 * (y * y + z * z)), 0.0, atol=1e-5)  # no yaw
+    st2 = dict(qpos=torch.zeros(N2, m.nq, device=DEV), qvel=torch.zeros(N2, m.nv, device=DEV), time=torch.zeros(N2, device=DEV))
+    terms.terminate_reset(st2, apply_reset=2, seed=3, step=5)
+    assert torch.equal(st2["qpos"], st["qpos"])  # same key, same draws
+    terms.terminate_reset(st2, apply_reset=2, seed=3, step=6)
+    assert not torch.equal(st2["time"], st["time"])
+
+
 def test_reset_redraws_per_episode_quantities():
     """An env that is reset mid-rollout gets a new action latency, zero offset and actuator state, as MjxEngine.reset draws
     them under cond(done) (ksim/engine.py:222-245, ksim/actuators.py:219-238); a continuing env keeps its own."""

@@ -609,3 +609,43 @@ def test_engine_reset_draws_hand_computed():
     # both zero-offset parts with one key (engine.py:117-124): the uniform part is a function of the normal draw
     out = ot.engine_reset_draws(nu, 1.0, u, z, latency_range=(0.0, 0.0), zero_offset=dict(mean=0.0, mag=0.1, std=0.01, same_key=True))
     np.testing.assert_allclose(out["zero_offset"], 0.01 * z[1:3] + 0.1 * ot.same_key_uniform(z[1:3]))
+
+
+def test_new_reset_restatements_hand_computed():
+    """resets.py:45-120, 284-354 by hand: the cell of a height field, the frame of a motion, and rotations whose effect
+    on a vector is known."""
+    q0 = np.zeros(10)
+    q0[3] = 1.0
+    # plane: x = clip(0.5 * 4, -1.5, 1.5) = 1.5, y = -0.25 * 2 = -0.5, z = plane 0.1 + base height 0.9
+    q = ot.xy_position_reset(q0, 0.5, -0.25, x_range=4.0, y_range=2.0, padded_bounds=(-1.5, 1.5, -3.0, 3.0), z=0.1,
+                             robot_base_height=0.9)
+    np.testing.assert_allclose(q[:3], [1.5, -0.5, 1.0])
+    # height field 5 x 3 over [-2, 2] x [-1, 1]: x = 1.0 -> (3 / 4) * 4 = 3; y = 0.4 -> (1.4 / 2) * 2 = 1.4 -> 1
+    h = np.arange(15.0).reshape(5, 3)
+    q = ot.xy_position_reset(q0, 0.25, 0.2, x_range=4.0, y_range=2.0, padded_bounds=(-2, 2, -1, 1), hfield=h,
+                             hfield_bounds=(2.0, 1.0, 0.5), robot_base_height=0.25)
+    np.testing.assert_allclose(q[:3], [1.0, 0.4, h[3, 1] + 0.75])
+    # the far corner clips to the last cell
+    q = ot.xy_position_reset(q0, 1.0, 1.0, x_range=9.0, y_range=9.0, padded_bounds=(-2, 2, -1, 1), hfield=h,
+                             hfield_bounds=(2.0, 1.0, 0.0))
+    assert q[2] == h[4, 2]
+    # motion: frame 7 of 5 wraps to 2; joints only unless the free joint is included; time = frame * dt
+    motion = np.arange(50.0).reshape(5, 10)
+    q, t = ot.initial_motion_state_reset(q0, 7, motion, 0.02, freejoint=False)
+    np.testing.assert_allclose(q[:7], q0[:7]); np.testing.assert_allclose(q[7:], motion[2, 7:]); assert t == pytest.approx(0.14)
+    q, _ = ot.initial_motion_state_reset(q0, 1, motion, 0.02, freejoint=True)
+    np.testing.assert_allclose(q, motion[1])
+    # heading u = 0.5 is a quarter turn about z: the body's x axis points along world y
+    q = ot.random_heading_reset(q0, 0.5)
+    np.testing.assert_allclose(ot.rotate_vector_by_quat(np.array([1.0, 0, 0]), q[3:7]), [0, 1, 0], atol=1e-12)
+    # pitch and roll share one draw: u = 0.75 in (-0.2, 0.2) and (0.4, 0.0) gives pitch 0.1, roll 0.1;
+    # u = 1/2 in symmetric ranges is no rotation; a pure pitch of pi / 2 turns the body's x axis to world -z
+    q = ot.random_pitch_roll_reset(q0, 0.75, (-0.2, 0.2), (0.4, 0.0))
+    np.testing.assert_allclose(q[3:7], ot.euler_to_quat([0.1, 0.1, 0.0]))
+    np.testing.assert_allclose(ot.random_pitch_roll_reset(q0, 0.5, (-0.3, 0.3), (-0.1, 0.1))[3:7], [1, 0, 0, 0], atol=1e-15)
+    q = ot.random_pitch_roll_reset(q0, 1.0, (0.0, np.pi / 2), (0.0, 0.0))
+    np.testing.assert_allclose(ot.rotate_vector_by_quat(np.array([1.0, 0, 0]), q[3:7]), [0, 0, -1], atol=1e-12)
+    # roll about x then heading: the order matters, quat <- quat * next
+    a = ot.random_heading_reset(ot.random_pitch_roll_reset(q0, 1.0, (0.0, 0.0), (0.0, 0.6)), 0.5)
+    b = ot.random_pitch_roll_reset(ot.random_heading_reset(q0, 0.5), 1.0, (0.0, 0.0), (0.0, 0.6))
+    assert np.abs(a[3:7] - b[3:7]).max() > 0.1
