@@ -747,6 +747,19 @@ int64_t ks_mlp_disc_workspace_bytes(const KsMlp* mlp, int64_t n_real, int64_t n_
 int ks_mlp_disc_loss_grad(KsMlp* mlp, ks_stream_t stream, int64_t n_real, const float* real, int64_t n_sim, const float* sim,
                           float grad_penalty_coef, int64_t n_motions, float* losses, void* workspace);
 int ks_grad_sqnorm(ks_stream_t stream, int64_t n, const float* g, double* acc);
+/* Mirror (left / right symmetry) losses of a task, examples/kbot/train.py:1458-1477, for networks applied to flat rows.
+ * A mirror map is a signed permutation: mirrored[j] = sign[j] * x[perm[j]] (mirror_joints / mirror_obs / mirror_cmd,
+ * train.py:1565-1760, each negate and reorder entries of their vector).
+ *   ks_signed_permute     out[r][j] = sign[j] * x[r][perm[j]]: the mirrored rows that the networks see
+ *   ks_mirror_loss_grad   with y (rows, n) the network's output on the rows and ym (rows, n) its output on the mirrored
+ *                         rows:  loss[r] = scale * mean_j (y[r][j] - sign[j] ym[r][perm[j]])^2  (train.py:1466-1469; for
+ *                         a critic n = 1, perm = {0}, sign = {1}: scale * (v - vm)^2, train.py:1477), and the gradient of
+ *                         mean_r loss[r] is ADDED to dy and WRITTEN to dym.  perm must be a permutation of 0..n-1.
+ * The loss joins the PPO loss as an auxiliary term (ksim/task/ppo.py:241-244, 485-486: mean over rows of the sum of terms). */
+int ks_signed_permute(ks_stream_t stream, int64_t rows, int32_t n, const float* x, const int32_t* perm, const float* sign,
+                      float* out);
+int ks_mirror_loss_grad(ks_stream_t stream, int64_t rows, int32_t n, float scale, const float* y, const float* ym,
+                        const int32_t* perm, const float* sign, float* dy, float* dym, float* loss /*(rows), nullable*/);
 /* ksim/task/ppo.py:546-563 (adaptive KL in _single_step), without a trip to the host: with
  * kl_mean = mean_rows(sum_a(on_log_probs - log_probs)) * kl_coef * *kl_scale, the coefficient kl_coef * *kl_scale is
  * multiplied by 1.5 when kl_mean > 1.5 desired_kl, divided by 1.5 when kl_mean < desired_kl / 1.5, clipped to

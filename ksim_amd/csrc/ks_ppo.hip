@@ -818,7 +818,65 @@ __global__ __launch_bounds__(256) void kl_adapt_kernel(int nblocks, float inv_ro
   }
 }
 
+// mirrored rows: out[r][j] = sign[j] * x[r][perm[j]]
+__global__ __launch_bounds__(256) void signed_permute_kernel(int64_t total, int n, const float* __restrict__ x, const int* __restrict__ perm,
+                                                             const float* __restrict__ sign, float* __restrict__ out) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= total) return;
+  const int64_t r = idx / n;
+  const int j = (int)(idx - r * n);
+  out[idx] = sign[j] * x[r * n + perm[j]];
+}
+
+// One thread per (row, j): diff = y[r][j] - sign[j] ym[r][perm[j]].  perm is a bijection, so the thread owns dym[r][perm[j]].
+// The row's loss is summed by the thread of j = 0 over the row, in index order.
+__global__ __launch_bounds__(256) void mirror_loss_grad_kernel(int64_t rows, int n, float scale, const float* __restrict__ y,
+                                                               const float* __restrict__ ym, const int* __restrict__ perm,
+                                                               const float* __restrict__ sign, float* __restrict__ dy,
+                                                               float* __restrict__ dym, float* __restrict__ loss) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= rows * n) return;
+  const int64_t r = idx / n;
+  const int j = (int)(idx - r * n);
+  const float c = 2.f * scale / ((float)n * (float)rows);
+  const int pj = perm[j];
+  const float sj = sign[j];
+  const float diff = y[idx] - sj * ym[r * n + pj];
+  dy[idx] += c * diff;
+  dym[r * n + pj] = -c * sj * diff;
+  if (loss && j == 0) {
+    float s = 0.f;
+    for (int k = 0; k < n; ++k) {
+      const float d = y[r * n + k] - sign[k] * ym[r * n + perm[k]];
+      s += d * d;
+    }
+    loss[r] = scale * s / (float)n;
+  }
+}
+
 }  // namespace ks
+
+extern "C" int ks_signed_permute(ks_stream_t stream, int64_t rows, int32_t n, const float* x, const int32_t* perm, const float* sign,
+                                 float* out) {
+  if (rows < 0 || n < 1) return ks::fail(KS_EINVAL, "ks_signed_permute: bad shape");
+  if (rows == 0) return KS_OK;
+  if (!x || !perm || !sign || !out || x == out) return ks::fail(KS_EINVAL, "ks_signed_permute: null pointer, or in place");
+  const int64_t total = rows * n, grid = (total + 255) / 256;
+  if (grid > 0x7fffffff) return ks::fail(KS_ELIMIT, "ks_signed_permute: too many elements");
+  hipLaunchKernelGGL(ks::signed_permute_kernel, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, total, n, x, perm, sign, out);
+  return ks::check_launch("ks_signed_permute");
+}
+
+extern "C" int ks_mirror_loss_grad(ks_stream_t stream, int64_t rows, int32_t n, float scale, const float* y, const float* ym,
+                                   const int32_t* perm, const float* sign, float* dy, float* dym, float* loss) {
+  if (rows < 1 || n < 1) return ks::fail(KS_EINVAL, "ks_mirror_loss_grad: bad shape");
+  if (!y || !ym || !perm || !sign || !dy || !dym) return ks::fail(KS_EINVAL, "ks_mirror_loss_grad: null pointer");
+  const int64_t total = rows * n, grid = (total + 255) / 256;
+  if (grid > 0x7fffffff) return ks::fail(KS_ELIMIT, "ks_mirror_loss_grad: too many elements");
+  hipLaunchKernelGGL(ks::mirror_loss_grad_kernel, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, rows, n, scale, y, ym, perm,
+                     sign, dy, dym, loss);
+  return ks::check_launch("ks_mirror_loss_grad");
+}
 
 extern "C" int ks_ppo_adapt_kl(ks_stream_t stream, int64_t rows, int32_t A, const float* on_log_probs, const float* log_probs,
                                float kl_coef, float desired_kl, float* kl_scale, float* workspace) {

@@ -12,6 +12,7 @@ from __future__ import annotations
 
 import ctypes
 from dataclasses import dataclass, field
+from typing import Sequence
 
 import torch
 
@@ -43,6 +44,40 @@ class PPOUpdateConfig:  # ksim/task/ppo.py:254-311 defaults, examples/walking.py
     adam_eps: float = 1e-8
     adam_weight_decay: float = 0.0
     grad_clip: float = 2.0
+    actor_mirror_loss_scale: float = 0.0   # examples/kbot/train.py:117-124
+    critic_mirror_loss_scale: float = 0.0
+
+
+@dataclass
+class MirrorSpec:
+    """Left / right mirror maps of a task as signed permutations (examples/kbot/train.py:1565-1760: mirror_joints, mirror_obs
+    and mirror_cmd reorder and negate entries): mirrored[j] = sign[j] * x[perm[j]] for the actor's observation row, the
+    critic's observation row and the action vector."""
+    actor_obs_perm: Sequence[int]
+    actor_obs_sign: Sequence[float]
+    critic_obs_perm: Sequence[int]
+    critic_obs_sign: Sequence[float]
+    action_perm: Sequence[int]
+    action_sign: Sequence[float]
+    _dev: dict = field(default_factory=dict, repr=False)
+
+    def __post_init__(self):
+        for name in ("actor_obs", "critic_obs", "action"):
+            perm, sign = list(getattr(self, name + "_perm")), list(getattr(self, name + "_sign"))
+            if sorted(perm) != list(range(len(perm))) or len(sign) != len(perm):
+                raise ValueError(f"{name}: the mirror map must be a permutation with one sign per entry")
+
+    def device(self, name: str, dev) -> tuple[torch.Tensor, torch.Tensor]:
+        if name not in self._dev:
+            self._dev[name] = (torch.tensor(list(getattr(self, name + "_perm")), dtype=torch.int32, device=dev),
+                               torch.tensor(list(getattr(self, name + "_sign")), dtype=torch.float32, device=dev))
+        return self._dev[name]
+
+
+def kbot_mirror_joints() -> tuple[list[int], list[float]]:
+    """mirror_joints of the K-Bot example (examples/kbot/train.py:1565-1573) as (perm, sign): the legs swap, the arm blocks
+    keep their places, every joint is negated."""
+    return list(range(5, 10)) + list(range(0, 5)) + list(range(10, 20)), [-1.0] * 20
 
 
 @dataclass
@@ -53,6 +88,7 @@ class GaussianMlpPolicy:
     log_std: torch.Tensor
     opt_step: int = 0
     kl_scale: torch.Tensor | None = None  # adaptive KL: current coefficient / cfg.kl_coef, one device float
+    mirror: MirrorSpec | None = None      # the task's symmetry, for the mirror losses
     _m1: torch.Tensor | None = field(default=None, repr=False)
     _m2: torch.Tensor | None = field(default=None, repr=False)
 
@@ -91,7 +127,30 @@ def single_step(policy: GaussianMlpPolicy, cfg: PPOUpdateConfig, actor_obs, crit
     rows = Tn * b
     nu = action.shape[-1]
     a_obs, c_obs, act = actor_obs.reshape(rows, -1), critic_obs.reshape(rows, -1), action.reshape(rows, nu)
-    lp, value, ent, mean = get_ppo_variables(policy, a_obs, c_obs, act, train=True)
+    # Mirror losses (examples/kbot/train.py:1458-1477): each network also runs on the mirrored rows.  Both passes share the
+    # weights, so the mirrored rows ride in the same forward and backward pass as rows [rows, 2 rows).
+    mirror_a = cfg.actor_mirror_loss_scale != 0.0
+    mirror_c = cfg.critic_mirror_loss_scale != 0.0
+    if (mirror_a or mirror_c) and policy.mirror is None:
+        raise _lib.KsError("mirror loss scales are set but the policy has no MirrorSpec")
+    st = _lib.current_stream()
+
+    def with_mirrored(x, name):
+        perm, sign = policy.mirror.device(name, x.device)
+        if perm.numel() != x.shape[1]:
+            raise _lib.KsError(f"the {name} mirror map has {perm.numel()} entries, the rows have {x.shape[1]}")
+        both = torch.empty(2 * rows, x.shape[1], dtype=torch.float32, device=x.device)
+        both[:rows].copy_(x)
+        _lib.check(lib.ks_signed_permute(st, rows, x.shape[1], _lib.ptr(both[:rows]), _lib.ptr(perm), _lib.ptr(sign), _lib.ptr(both[rows:])))
+        return both
+
+    a_in = with_mirrored(a_obs, "actor_obs") if mirror_a else a_obs
+    c_in = with_mirrored(c_obs, "critic_obs") if mirror_c else c_obs
+    mean_all = policy.actor.train_forward(a_in)
+    value_all = policy.critic.train_forward(c_in)
+    mean, value = mean_all[:rows], value_all[:rows].reshape(-1)
+    lp, ent = torch.empty_like(mean), torch.empty_like(mean)
+    _lib.check(lib.ks_gaussian_log_prob(st, rows, nu, _lib.ptr(mean), _lib.ptr(policy.log_std), _lib.ptr(act), _lib.ptr(lp), _lib.ptr(ent)))
     inputs = ppo_mod.compute_ppo_inputs(value.view(Tn, b), rewards, done, success, cfg.gamma, cfg.lam,
                                         normalize_advantages=cfg.normalize_advantages,
                                         monte_carlo_returns=cfg.monte_carlo_returns, time_major=True)
@@ -101,8 +160,9 @@ def single_step(policy: GaussianMlpPolicy, cfg: PPOUpdateConfig, actor_obs, crit
         policy.kl_scale = torch.ones(1, dtype=torch.float32, device=actor_obs.device)
     p = _lib.KsPpoLossParams(cfg.clip_param, cfg.value_loss_coef, cfg.entropy_coef, cfg.kl_coef, cfg.log_clip_value,
                              1.0, int(cfg.use_clipped_value_loss), _lib.ptr(policy.kl_scale) if cfg.adaptive_kl else None)
-    d_mean = torch.empty_like(mean)
-    d_value = torch.empty(rows, 1, dtype=torch.float32, device=mean.device)
+    d_mean_all = torch.empty_like(mean_all)
+    d_value_all = torch.empty(value_all.shape[0], 1, dtype=torch.float32, device=mean.device)
+    d_mean, d_value = d_mean_all[:rows], d_value_all[:rows]
     d_log_std = torch.empty_like(policy.log_std)
     ws = torch.empty(256 * nu, dtype=torch.float32, device=mean.device)
     on_lp, on_v = on_log_probs.reshape(rows, nu), on_values.reshape(rows)
@@ -110,8 +170,23 @@ def single_step(policy: GaussianMlpPolicy, cfg: PPOUpdateConfig, actor_obs, crit
                                     _lib.ptr(policy.log_std), _lib.ptr(act), _lib.ptr(on_lp),
                                     _lib.ptr(inputs.advantages_bt), _lib.ptr(inputs.value_targets_bt), _lib.ptr(on_v),
                                     _lib.ptr(value), _lib.ptr(d_mean), _lib.ptr(d_value), _lib.ptr(d_log_std), _lib.ptr(ws)))
-    policy.actor.backward(a_obs, d_mean)
-    policy.critic.backward(c_obs, d_value)
+    aux = {}
+    if mirror_a:
+        perm, sign = policy.mirror.device("action", mean.device)
+        aux["action_mirror_loss"] = torch.empty(rows, dtype=torch.float32, device=mean.device)
+        _lib.check(lib.ks_mirror_loss_grad(st, rows, nu, cfg.actor_mirror_loss_scale, _lib.ptr(mean), _lib.ptr(mean_all[rows:]),
+                                           _lib.ptr(perm), _lib.ptr(sign), _lib.ptr(d_mean), _lib.ptr(d_mean_all[rows:]),
+                                           _lib.ptr(aux["action_mirror_loss"])))
+    if mirror_c:
+        if "_one" not in policy.mirror._dev:
+            policy.mirror._dev["_one"] = (torch.zeros(1, dtype=torch.int32, device=mean.device), torch.ones(1, device=mean.device))
+        perm, sign = policy.mirror._dev["_one"]
+        aux["value_mirror_loss"] = torch.empty(rows, dtype=torch.float32, device=mean.device)
+        _lib.check(lib.ks_mirror_loss_grad(st, rows, 1, cfg.critic_mirror_loss_scale, _lib.ptr(value_all), _lib.ptr(value_all[rows:]),
+                                           _lib.ptr(perm), _lib.ptr(sign), _lib.ptr(d_value), _lib.ptr(d_value_all[rows:]),
+                                           _lib.ptr(aux["value_mirror_loss"])))
+    policy.actor.backward(a_in, d_mean_all)
+    policy.critic.backward(c_in, d_value_all)
     # optimiser chain over every parameter together: global norm first
     sq = torch.zeros(1, dtype=torch.float64, device=mean.device)
     policy.actor.grad_sqnorm(sq)
@@ -124,7 +199,7 @@ def single_step(policy: GaussianMlpPolicy, cfg: PPOUpdateConfig, actor_obs, crit
     _lib.check(lib.ks_adam_step(_lib.current_stream(), nu, _lib.ptr(policy.log_std), _lib.ptr(d_log_std),
                                 _lib.ptr(policy._m1), _lib.ptr(policy._m2), ctypes.byref(ap), _lib.ptr(sq)))
     metrics = {"grad_norm": sq.sqrt(), "d_mean": d_mean, "d_value": d_value, "d_log_std": d_log_std,
-               "log_probs": lp, "values": value, "advantages": inputs.advantages_bt}
+               "log_probs": lp, "values": value, "advantages": inputs.advantages_bt, **aux}
     if cfg.adaptive_kl:
         _lib.check(lib.ks_ppo_adapt_kl(_lib.current_stream(), rows, nu, _lib.ptr(on_lp), _lib.ptr(lp), cfg.kl_coef,
                                        cfg.desired_kl, _lib.ptr(policy.kl_scale), _lib.ptr(ws)))

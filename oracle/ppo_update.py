@@ -83,8 +83,27 @@ def ppo_loss_torch(adv, tgt, on_lp, on_v, lp, v, ent, cfg, kl_scale=1.0):
     return (policy + value + kl + entropy).mean(), {"policy": policy, "value": value, "kl": kl, "entropy": entropy}
 
 
-def loss_and_grads(params, batch, cfg, kl_scale=1.0, act="elu"):
+def mirror_terms(mean, v, actor_obs, critic_obs, tp, mirror, act):
+    """The K-Bot task's mirror losses per transition (examples/kbot/train.py:1458-1477): the actor's mode against the
+    mirrored-back mode on the mirrored observation, and the value against the value of the mirrored observation.
+    mirror: dict(actor_obs=(perm, sign), critic_obs=(perm, sign), action=(perm, sign), actor_scale, critic_scale) with
+    mirrored[j] = sign[j] x[perm[j]]."""
+    def m(x, key):
+        perm, sign = mirror[key]
+        return x[..., list(perm)] * torch.tensor(np.asarray(sign, dtype=np.float64))
+    out = {}
+    if mirror.get("actor_scale", 0.0):
+        mean_m = mlp(m(actor_obs, "actor_obs"), tp["actor_w"], tp["actor_b"], act)
+        out["action_mirror_loss"] = ((mean - m(mean_m, "action")) ** 2).mean(-1) * mirror["actor_scale"]
+    if mirror.get("critic_scale", 0.0):
+        v_m = mlp(m(critic_obs, "critic_obs"), tp["critic_w"], tp["critic_b"], act)[..., 0]
+        out["value_mirror_loss"] = (v - v_m) ** 2 * mirror["critic_scale"]
+    return out
+
+
+def loss_and_grads(params, batch, cfg, kl_scale=1.0, act="elu", mirror=None):
     """params: dict(actor_w, actor_b, critic_w, critic_b: lists of float64 arrays; log_std).  batch: (T, b, ...) arrays.
+    `mirror`: see mirror_terms; its terms join the loss like any auxiliary loss (ppo.py:241-244).
     Returns (loss, grads with the structure of params, aux)."""
     tp = {k: ([torch.tensor(np.asarray(a, dtype=np.float64), requires_grad=True) for a in v] if isinstance(v, list)
               else torch.tensor(np.asarray(v, dtype=np.float64), requires_grad=True)) for k, v in params.items()}
@@ -99,6 +118,11 @@ def loss_and_grads(params, batch, cfg, kl_scale=1.0, act="elu"):
                                  cfg["monte_carlo_returns"], np.float64)
     adv, tgt = t64(gi["advantages"].T), t64(gi["value_targets"].T)
     loss, terms = ppo_loss_torch(adv, tgt, t64(batch["on_log_probs"]), t64(batch["on_values"]), lp, v, ent, cfg, kl_scale)
+    if mirror:
+        extra = mirror_terms(mean, v, t64(batch["actor_obs"]), t64(batch["critic_obs"]), tp, mirror, act)
+        for name, term in extra.items():
+            loss = loss + term.mean()
+            terms[name] = term
     loss.backward()
     grads = {k: ([a.grad.numpy() for a in v] if isinstance(v, list) else v.grad.numpy()) for k, v in tp.items()}
     aux = {"mean": mean.detach().numpy(), "values": v.detach().numpy(), "log_probs": lp.detach().numpy(),

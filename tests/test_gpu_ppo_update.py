@@ -397,3 +397,65 @@ def test_gradient_norm_and_update_are_bit_reproducible():
     assert float(outs[0][0].item()) > 0.05, "the clip is not active"
     for a, b in zip(*outs):
         assert torch.equal(a, b)
+
+
+def test_mirror_losses_match_autograd_and_vanish_for_a_symmetric_policy():
+    """Mirror losses of the K-Bot task (examples/kbot/train.py:1458-1477) inside the minibatch step: per-transition loss values
+    and every parameter gradient against float64 autograd of the same terms added to the PPO loss; a policy that already
+    commutes with the mirror maps has zero mirror loss and the gradients of plain PPO."""
+    from ksim_amd.mlp import MLP
+    from ksim_amd.ppo_update import GaussianMlpPolicy, MirrorSpec, PPOUpdateConfig, get_ppo_variables, kbot_mirror_joints, single_step
+
+    Tn, N, od, A = 8, 8, 26, 20
+    pol, params, ro, rng = _setup(17, Tn, N, od, A, 64)
+    aperm, asign = kbot_mirror_joints()
+    assert aperm[:10] == [5, 6, 7, 8, 9, 0, 1, 2, 3, 4] and aperm[10:] == list(range(10, 20)) and set(asign) == {-1.0}
+    operm = list(rng.permutation(od))
+    osign = list(rng.choice([-1.0, 1.0], od))
+    cperm = list(rng.permutation(od))
+    csign = list(rng.choice([-1.0, 1.0], od))
+    pol.mirror = MirrorSpec(operm, osign, cperm, csign, aperm, asign)
+    pol.train_init()
+    cfgd = dict(CFG, batch_size=N)
+    cfg = PPOUpdateConfig(**cfgd, actor_mirror_loss_scale=0.7, critic_mirror_loss_scale=0.3)
+    d = {k: (torch.tensor(v, device=DEV) if v.dtype == bool else t32(v)) for k, v in ro.items()}
+    rows = Tn * N
+    on_lp, on_v, _, _ = get_ppo_variables(pol, d["actor_obs"].reshape(rows, od), d["critic_obs"].reshape(rows, od), d["action"].reshape(rows, A))
+    on_lp, on_v = on_lp.view(Tn, N, A).clone() - 0.03, on_v.view(Tn, N).clone() + 0.05
+    batch = dict(ro, on_log_probs=on_lp.cpu().numpy(), on_values=on_v.cpu().numpy())
+    mirror = dict(actor_obs=(operm, osign), critic_obs=(cperm, csign), action=(aperm, asign), actor_scale=0.7, critic_scale=0.3)
+    loss, grads, aux = ou.loss_and_grads(params, batch, cfgd, mirror=mirror)
+    plain = ou.loss_and_grads(params, batch, cfgd)[1]
+    assert rel(grads["actor_w"][0], plain["actor_w"][0]) > 0.05, "the mirror terms do not matter in this test"
+    met = single_step(pol, cfg, d["actor_obs"], d["critic_obs"], d["action"], d["rewards"], d["done"], d["success"], on_lp, on_v)
+    assert rel(met["action_mirror_loss"].cpu().numpy(), aux["terms"]["action_mirror_loss"].reshape(-1)) < 1e-4
+    assert rel(met["value_mirror_loss"].cpu().numpy(), aux["terms"]["value_mirror_loss"].reshape(-1)) < 1e-4
+    for net, kw, kb in ((pol.actor, "actor_w", "actor_b"), (pol.critic, "critic_w", "critic_b")):
+        for (gw, gb), w, b in zip(net.parameters(gradients=True), grads[kw], grads[kb]):
+            assert rel(gw.cpu().numpy(), w) < 5e-4 and rel(gb.cpu().numpy(), b) < 5e-4
+    assert rel(met["d_log_std"].cpu().numpy(), grads["log_std"]) < 5e-4
+
+    # a linear actor W with W = P_a W P_o^T (and a critic row w = w P_c^T) is mirror-symmetric: zero loss, PPO's gradients
+    def sym(perm_out, sign_out, perm_in, sign_in, w):
+        po = np.zeros((len(perm_out), len(perm_out)))
+        po[np.arange(len(perm_out)), perm_out] = sign_out   # mirrored[j] = sign[j] x[perm[j]]
+        pi = np.zeros((len(perm_in), len(perm_in)))
+        pi[np.arange(len(perm_in)), perm_in] = sign_in
+        return (0.5 * (w + po @ w @ np.linalg.inv(pi))).astype(np.float32)  # average over the two-element group generated by a pair of involutions
+
+    # the K-Bot joint mirror is an involution; give the observation an involution too
+    oinv = list(range(od)); oinv[0], oinv[1] = 1, 0; oinv[4], oinv[9] = 9, 4
+    osg = [1.0] * od; osg[2] = -1.0; osg[4] = osg[9] = -1.0
+    wa = sym(aperm, asign, oinv, osg, rng.normal(size=(A, od)) * 0.2)
+    wc = sym([0], [1.0], oinv, osg, rng.normal(size=(1, od)) * 0.2)
+    pol2 = GaussianMlpPolicy(actor=MLP([wa], [np.zeros(A, np.float32)], dtype="f32"), critic=MLP([wc], [np.zeros(1, np.float32)], dtype="f32"),
+                             log_std=pol.log_std.clone(), mirror=MirrorSpec(oinv, osg, oinv, osg, aperm, asign))
+    pol3 = GaussianMlpPolicy(actor=MLP([wa], [np.zeros(A, np.float32)], dtype="f32"), critic=MLP([wc], [np.zeros(1, np.float32)], dtype="f32"),
+                             log_std=pol.log_std.clone())
+    pol2.train_init(); pol3.train_init()
+    m2 = single_step(pol2, cfg, d["actor_obs"], d["critic_obs"], d["action"], d["rewards"], d["done"], d["success"], on_lp, on_v)
+    single_step(pol3, PPOUpdateConfig(**cfgd), d["actor_obs"], d["critic_obs"], d["action"], d["rewards"], d["done"], d["success"], on_lp, on_v)
+    assert float(m2["action_mirror_loss"].abs().max()) < 1e-10 and float(m2["value_mirror_loss"].abs().max()) < 1e-10
+    for a, b in zip(pol2.actor.parameters(gradients=True) + pol2.critic.parameters(gradients=True),
+                    pol3.actor.parameters(gradients=True) + pol3.critic.parameters(gradients=True)):
+        assert rel(a[0].cpu().numpy(), b[0].cpu().numpy()) < 1e-5 and rel(a[1].cpu().numpy(), b[1].cpu().numpy()) < 1e-5
