@@ -892,8 +892,14 @@ enum { KS_REW_STAY_ALIVE = 0, KS_REW_BASE_HEIGHT = 1, KS_REW_BASE_HEIGHT_RANGE =
        KS_REW_REACHABILITY = 27, /* sum over the joints of norm(max(0, |action - qpos[7:]| - params[u])) (rewards.py:1108-1129) */
        KS_REW_SINUSOIDAL_GAIT = 29, /* 1 - sum over `norm` feet of |obs[index + 3 f + 2] - command[index2 + f]| / p0
                                        (rewards.py:1320-1335); index2 = where the command's heights start */
-       KS_REW_INTERSECTION = 28  /* 1 when two of the `norm` points obs[index + 3 i .. + 3] are closer than p0, else 0
-                                    (rewards.py:1417-1430) */ };
+       KS_REW_INTERSECTION = 28, /* 1 when two of the `norm` points obs[index + 3 i .. + 3] are closer than p0, else 0
+                                    (rewards.py:1417-1430) */
+       KS_REW_JOINT_POSITION = 30, /* JointPositionReward "pos" (rewards.py:1352-1380): mean over the `count` joints params[k]
+                                      of kernel_with_penalty(current_position_k - qpos[7 + joint]; p0, p1, p2), where the
+                                      command block at `index` holds a JointPositionCommandValue (commands.py:795-818) as
+                                      [start (count), target (count), total_time, num_steps, step_id] and
+                                      current_position = start + (target - start) step_id / num_steps */
+       KS_REW_JOINT_VELOCITY_CMD = 31 /* its "vel" part: current_velocity = (target - start) / total_time against qvel[6 + joint] */ };
 enum { KS_NORM_L1 = 0, KS_NORM_L2 = 1 }; /* xax.get_norm: l1 = |x|, l2 = x^2 (reference tests/test_rewards.py:95-98) */
 #define KS_MAX_REWARD_PARAMS 320
 typedef struct KsRewardDesc {
@@ -940,9 +946,18 @@ int ks_rewards(ks_stream_t stream, const KsRewardIO* io /*host*/);
  *   KS_SCAN_SPARSE_TARGET_HEIGHT (rewards.py:1148-1192): carry = n running maximum heights, one output slot.
  * Contact flags are the (n_contact, n) block of 0/1 values at obs[contact_index...] (any over n_contact, > 0.5);
  * positions the (n, 3) block at obs[position_index...]. */
-#define KS_MAX_REWARD_SCANS 4
+#define KS_MAX_REWARD_SCANS 8
 #define KS_MAX_SCAN_BODIES 8
-enum { KS_SCAN_FEET_AIR_TIME = 0, KS_SCAN_SPARSE_TARGET_HEIGHT = 1 };
+#define KS_MAX_SCAN_JOINTS 32
+enum { KS_SCAN_FEET_AIR_TIME = 0, KS_SCAN_SPARSE_TARGET_HEIGHT = 1,
+       KS_SCAN_SYMMETRY = 2,          /* SymmetryReward (rewards.py:843-896): with x[t][j] = qpos[t][7 + joints[j]] - targets[j],
+                                         carry <- carry (1 - alpha) + mean_t x[t] alpha once per rollout, then
+                                         out[t] = -sum_j x[t][j] carry[j]; n joints, carry of n floats, one slot; a carry
+                                         that restarts begins at the targets (initial_carry) */
+       KS_SCAN_PAIRWISE_SYMMETRY = 3  /* PairwiseSymmetryReward (rewards.py:899-936): joints[0..1] = left, right,
+                                         targets[0..1] their zeros, right negated when `flipped`; slot "lr" =
+                                         kernel_with_penalty(left - right; kernel_scale, sq_scale, abs_scale), slot "self" as
+                                         KS_SCAN_SYMMETRY over the pair; carry of 2 floats restarting at the zeros */ };
 typedef struct KsRewardScanDesc {
   int32_t kind;
   int32_t n;               /* feet / bodies */
@@ -956,6 +971,10 @@ typedef struct KsRewardScanDesc {
   float bias, ground_penalty;
   float linvel_threshold, angvel_threshold;
   float height;            /* sparse target height: the reward is clipped at it */
+  int32_t joints[KS_MAX_SCAN_JOINTS]; /* symmetry kinds: joint indices (qpos address - 7) */
+  float targets[KS_MAX_SCAN_JOINTS];
+  float alpha, kernel_scale, sq_scale, abs_scale;
+  int32_t flipped;
 } KsRewardScanDesc;
 typedef struct KsRewardScanIO {
   int64_t T, N;
@@ -963,6 +982,8 @@ typedef struct KsRewardScanIO {
   KsRewardScanDesc scans[KS_MAX_REWARD_SCANS];
   const float* obs;      /* (T, N, obs_dim) */
   const float* qvel;     /* (T, N, nv) */
+  const float* qpos;     /* (T, N, nq), required by the symmetry kinds */
+  int32_t nq;
   const float* command;  /* (T, N, command_dim) nullable unless a *_cmd_index is set */
   const uint8_t* done;   /* (T, N) */
   float* carry;          /* (N, carry_dim) in/out */

@@ -100,10 +100,10 @@ class KsMlpDesc(ctypes.Structure):
  REW_UPRIGHT_ANGVEL, REW_UPRIGHT_LINVEL, REW_UPRIGHT_POSE, REW_AMP, REW_STATEFUL, REW_LINVEL_CMD, REW_ANGVEL_CMD,
  REW_OFF_AXIS, REW_MOTIONLESS, REW_FORCE, REW_JOINT_SMOOTH, REW_AVOID_LIMITS, REW_TORQUE, REW_ENERGY, REW_JOINT_DEVIATION,
  REW_FLAT_BODY, REW_POSITION_TRACKING, REW_NO_ROLL_ANGVEL, REW_NO_ROLL_POSE, REW_LINK_SMOOTH, REW_FEET_SLIP,
- REW_REACHABILITY, REW_INTERSECTION, REW_SINUSOIDAL_GAIT) = range(30)
+ REW_REACHABILITY, REW_INTERSECTION, REW_SINUSOIDAL_GAIT, REW_JOINT_POSITION, REW_JOINT_VELOCITY_CMD) = range(32)
 KS_MAX_REWARD_PARAMS = 320
-KS_MAX_REWARD_SCANS, KS_MAX_SCAN_BODIES = 4, 8
-SCAN_FEET_AIR_TIME, SCAN_SPARSE_TARGET_HEIGHT = 0, 1
+KS_MAX_REWARD_SCANS, KS_MAX_SCAN_BODIES, KS_MAX_SCAN_JOINTS = 8, 8, 32
+SCAN_FEET_AIR_TIME, SCAN_SPARSE_TARGET_HEIGHT, SCAN_SYMMETRY, SCAN_PAIRWISE_SYMMETRY = 0, 1, 2, 3
 NORM_L1, NORM_L2 = 0, 1
 KS_MAX_REWARD_TERMS = 32
 
@@ -130,14 +130,16 @@ class KsRewardScanDesc(ctypes.Structure):
                 ("position_index", c_int32), ("slot", c_int32), ("carry_index", c_int32),
                 ("linvel_cmd_index", c_int32), ("angvel_cmd_index", c_int32), ("air_steps", c_float),
                 ("gnd_steps", c_float), ("bias", c_float), ("ground_penalty", c_float), ("linvel_threshold", c_float),
-                ("angvel_threshold", c_float), ("height", c_float)]
+                ("angvel_threshold", c_float), ("height", c_float), ("joints", c_int32 * KS_MAX_SCAN_JOINTS),
+                ("targets", c_float * KS_MAX_SCAN_JOINTS), ("alpha", c_float), ("kernel_scale", c_float),
+                ("sq_scale", c_float), ("abs_scale", c_float), ("flipped", c_int32)]
 
 
 class KsRewardScanIO(ctypes.Structure):
     _fields_ = [("T", c_int64), ("N", c_int64), ("obs_dim", c_int32), ("nv", c_int32), ("command_dim", c_int32),
                 ("n_scans", c_int32), ("carry_dim", c_int32), ("n_slots", c_int32),
                 ("scans", KsRewardScanDesc * KS_MAX_REWARD_SCANS), ("obs", c_void_p), ("qvel", c_void_p),
-                ("command", c_void_p), ("done", c_void_p), ("carry", c_void_p), ("out", c_void_p)]
+                ("qpos", c_void_p), ("nq", c_int32), ("command", c_void_p), ("done", c_void_p), ("carry", c_void_p), ("out", c_void_p)]
 
 
 class KsGruDesc(ctypes.Structure):

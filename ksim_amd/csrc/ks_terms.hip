@@ -836,6 +836,21 @@ __global__ __launch_bounds__(256) void rewards_kernel(KsRewardIO io) {
         }
         val = s;
       } break;
+      case KS_REW_JOINT_POSITION:
+      case KS_REW_JOINT_VELOCITY_CMD: {
+        const float* pr = io.params + r.param_offset;
+        const float* cm = io.command + idx * io.command_dim + r.index;  // [start, target, total_time, num_steps, step_id]
+        const float total_time = cm[2 * r.count], num_steps = cm[2 * r.count + 1], step_id = cm[2 * r.count + 2];
+        float sum = 0.f;
+        for (int k = 0; k < r.count; ++k) {
+          const int jn = (int)pr[k];
+          const float start = cm[k], target = cm[r.count + k];
+          const float diff = r.kind == KS_REW_JOINT_POSITION ? start + (target - start) * step_id / num_steps - q[7 + jn]
+                                                             : (target - start) / total_time - v[6 + jn];
+          sum += kernel_with_penalty(diff, r.p0, r.p1, r.p2);
+        }
+        val = sum / (float)r.count;
+      } break;
       case KS_REW_SINUSOIDAL_GAIT: {
         const float* ob = io.obs + idx * io.obs_dim + r.index;
         const float* hc = io.command + idx * io.command_dim + r.index2;
@@ -869,8 +884,39 @@ __global__ __launch_bounds__(256) void reward_scan_kernel(KsRewardScanIO io) {
   const int64_t TN = io.T * io.N;
   const bool restart = io.done[(io.T - 1) * io.N + e] != 0;  // ksim/task/rl.py:206-214
   for (int sidx = 0; sidx < io.n_scans; ++sidx) {
-    const KsRewardScanDesc s = io.scans[sidx];
+    const KsRewardScanDesc& s = io.scans[sidx];
     float* cr = io.carry + e * io.carry_dim + s.carry_index;
+    if (s.kind == KS_SCAN_SYMMETRY || s.kind == KS_SCAN_PAIRWISE_SYMMETRY) {
+      // one update of the carry per rollout with the rollout's mean, then a second walk for the rewards; the carry row
+      // itself is the accumulator, so any number of joints needs no registers
+      const int n = s.kind == KS_SCAN_SYMMETRY ? s.n : 2;
+      const float inv_t = 1.f / (float)io.T;
+      for (int j = 0; j < n; ++j) {
+        const float sign = (s.kind == KS_SCAN_PAIRWISE_SYMMETRY && j == 1 && s.flipped) ? -1.f : 1.f;
+        float sum = 0.f;
+        for (int64_t t = 0; t < io.T; ++t) sum += sign * (io.qpos[(t * io.N + e) * io.nq + 7 + s.joints[j]] - s.targets[j]);
+        const float old = restart ? s.targets[j] : cr[j];
+        cr[j] = old * (1.0f - s.alpha) + (sum * inv_t) * s.alpha;
+      }
+      for (int64_t t = 0; t < io.T; ++t) {
+        const int64_t idx = t * io.N + e;
+        const float* q = io.qpos + idx * io.nq + 7;
+        float acc = 0.f;
+        for (int j = 0; j < n; ++j) {
+          const float sign = (s.kind == KS_SCAN_PAIRWISE_SYMMETRY && j == 1 && s.flipped) ? -1.f : 1.f;
+          acc += sign * (q[s.joints[j]] - s.targets[j]) * -cr[j];
+        }
+        if (s.kind == KS_SCAN_SYMMETRY) {
+          io.out[(int64_t)s.slot * TN + idx] = acc;
+        } else {
+          const float ql = q[s.joints[0]] - s.targets[0];
+          const float qr = (s.flipped ? -1.f : 1.f) * (q[s.joints[1]] - s.targets[1]);
+          io.out[(int64_t)s.slot * TN + idx] = kernel_with_penalty(ql - qr, s.kernel_scale, s.sq_scale, s.abs_scale);
+          io.out[(int64_t)(s.slot + 1) * TN + idx] = acc;
+        }
+      }
+      continue;
+    }
     float c[3 * KS_MAX_SCAN_BODIES];  // counter k of body f at c[k * KS_MAX_SCAN_BODIES + f]; packed as k * n + f in memory
     const int nk = s.kind == KS_SCAN_FEET_AIR_TIME ? 3 : 1;
     for (int k = 0; k < 3; ++k)
@@ -1295,7 +1341,7 @@ extern "C" int ks_rewards(ks_stream_t stream, const KsRewardIO* io) {
   if (!io->done) return fail(KS_EINVAL, "ks_rewards: done is required");
   for (int j = 0; j < io->n_rewards; ++j) {
     const int k = io->rewards[j].kind;
-    if (k < KS_REW_STAY_ALIVE || k > KS_REW_SINUSOIDAL_GAIT) return fail(KS_EINVAL, "ks_rewards: term %d: bad kind", j);
+    if (k < KS_REW_STAY_ALIVE || k > KS_REW_JOINT_VELOCITY_CMD) return fail(KS_EINVAL, "ks_rewards: term %d: bad kind", j);
     const KsRewardDesc& rd = io->rewards[j];
     if (k == KS_REW_LINVEL_CMD || k == KS_REW_ANGVEL_CMD) {
       const int span = k == KS_REW_LINVEL_CMD ? 4 : 1;
@@ -1370,6 +1416,14 @@ extern "C" int ks_rewards(ks_stream_t stream, const KsRewardIO* io) {
           if (!io->qpos || !io->action || io->nu < 1 || io->nq != io->nu + 7) return fail(KS_EINVAL, "ks_rewards: term %d needs actions and qpos with one joint per action behind a floating base", j);
           need_params = io->nu;
           break;
+        case KS_REW_JOINT_POSITION:
+        case KS_REW_JOINT_VELOCITY_CMD:
+          if (!io->qpos || !io->qvel || nj < 1 || r.count < 1) return fail(KS_EINVAL, "ks_rewards: term %d needs joints behind a floating base", j);
+          if (!io->command || r.index < 0 || r.index + 2 * r.count + 3 > io->command_dim)
+            return fail(KS_EINVAL, "ks_rewards: term %d: the joint-position command block (2 n + 3 numbers) lies outside the command vector", j);
+          if (!(r.p0 > 0.f)) return fail(KS_EINVAL, "ks_rewards: term %d: the kernel scale must be positive", j);
+          need_params = r.count;
+          break;
         case KS_REW_SINUSOIDAL_GAIT:
           if (!io->obs || !io->command || r.norm < 1 || r.index < 0 || r.index + 3 * r.norm > io->obs_dim || r.index2 < 0 ||
               r.index2 + r.norm > io->command_dim || !(r.p0 != 0.f))
@@ -1392,6 +1446,9 @@ extern "C" int ks_rewards(ks_stream_t stream, const KsRewardIO* io) {
         if (k == KS_REW_JOINT_DEVIATION)
           for (int c = 0; c < r.count; ++c)
             if (!(pr[3 * c] >= 0.f && pr[3 * c] < (float)nj)) return fail(KS_EINVAL, "ks_rewards: term %d: joint %d outside 0..%d", j, (int)pr[3 * c], nj - 1);
+        if (k == KS_REW_JOINT_POSITION || k == KS_REW_JOINT_VELOCITY_CMD)
+          for (int c = 0; c < r.count; ++c)
+            if (!(pr[c] >= 0.f && pr[c] < (float)nj)) return fail(KS_EINVAL, "ks_rewards: term %d: joint %d outside 0..%d", j, (int)pr[c], nj - 1);
         if (k == KS_REW_FLAT_BODY)
           for (int c = 0; c < r.count; ++c)
             if (!(pr[c] >= 0.f && pr[c] < (float)io->nb)) return fail(KS_EINVAL, "ks_rewards: term %d: body %d outside 0..%d", j, (int)pr[c], io->nb - 1);
@@ -1412,10 +1469,23 @@ extern "C" int ks_reward_scan(ks_stream_t stream, const KsRewardScanIO* io) {
   if (io->T < 0 || io->N < 0) return fail(KS_EINVAL, "ks_reward_scan: negative size");
   if (io->n_scans < 0 || io->n_scans > KS_MAX_REWARD_SCANS) return fail(KS_ELIMIT, "ks_reward_scan: more than %d scans", KS_MAX_REWARD_SCANS);
   if (io->T == 0 || io->N == 0 || io->n_scans == 0) return KS_OK;
-  if (!io->obs || !io->qvel || !io->done || !io->carry || !io->out) return fail(KS_EINVAL, "ks_reward_scan: obs, qvel, done, carry and out are required");
-  if (io->nv < 6) return fail(KS_EINVAL, "ks_reward_scan: the rewards read the velocity of a floating base");
+  if (!io->done || !io->carry || !io->out) return fail(KS_EINVAL, "ks_reward_scan: done, carry and out are required");
   for (int j = 0; j < io->n_scans; ++j) {
     const KsRewardScanDesc& s = io->scans[j];
+    if (s.kind == KS_SCAN_SYMMETRY || s.kind == KS_SCAN_PAIRWISE_SYMMETRY) {
+      const bool pair = s.kind == KS_SCAN_PAIRWISE_SYMMETRY;
+      const int n = pair ? 2 : s.n;
+      if (!io->qpos || io->nq < 8) return fail(KS_EINVAL, "ks_reward_scan: scan %d reads the joints behind a floating base (qpos)", j);
+      if (n < 1 || n > KS_MAX_SCAN_JOINTS) return fail(KS_ELIMIT, "ks_reward_scan: scan %d: %d joints (1..%d)", j, n, KS_MAX_SCAN_JOINTS);
+      for (int k = 0; k < n; ++k)
+        if (s.joints[k] < 0 || s.joints[k] + 7 >= io->nq) return fail(KS_EINVAL, "ks_reward_scan: scan %d: joint %d outside 0..%d", j, s.joints[k], io->nq - 8);
+      if (s.slot < 0 || s.slot + (pair ? 2 : 1) > io->n_slots) return fail(KS_EINVAL, "ks_reward_scan: scan %d: output slot outside n_slots", j);
+      if (s.carry_index < 0 || s.carry_index + n > io->carry_dim) return fail(KS_EINVAL, "ks_reward_scan: scan %d: carry outside the carry row", j);
+      if (pair && (!(s.kernel_scale > 0.f) || !(s.sq_scale > 0.f) || !(s.abs_scale > 0.f))) return fail(KS_EINVAL, "ks_reward_scan: scan %d: the kernel scales must be positive", j);
+      continue;
+    }
+    if (!io->obs || !io->qvel) return fail(KS_EINVAL, "ks_reward_scan: scan %d reads obs and qvel", j);
+    if (io->nv < 6) return fail(KS_EINVAL, "ks_reward_scan: the rewards read the velocity of a floating base");
     if (s.kind != KS_SCAN_FEET_AIR_TIME && s.kind != KS_SCAN_SPARSE_TARGET_HEIGHT) return fail(KS_EINVAL, "ks_reward_scan: scan %d: bad kind", j);
     const bool feet = s.kind == KS_SCAN_FEET_AIR_TIME;
     if (s.n < 1 || s.n > KS_MAX_SCAN_BODIES || s.n_contact < 1) return fail(KS_ELIMIT, "ks_reward_scan: scan %d: %d bodies (1..%d), %d contact rows", j, s.n, KS_MAX_SCAN_BODIES, s.n_contact);

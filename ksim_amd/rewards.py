@@ -351,6 +351,44 @@ class SinusoidalGaitReward(Reward):  # rewards.py:1320-1335
         return [(None, T.REW_SINUSOIDAL_GAIT, feet, self.max_height, 0.0, 0.0, 0.0, ob.start, _extra(index2=cm.start + 2))]
 
 
+@dataclass(frozen=True)
+class JointPositionReward(Reward):  # rewards.py:1352-1380
+    """Tracks a joint-position command: "pos" and "vel" are means over the joints of a kernel of (commanded - actual).
+    The command named `command_name` is a JointPositionCommandValue (commands.py:795-818) laid out in the command vector as
+    [start_position (n), target_position (n), total_time, num_steps, step_id]."""
+    command_name: str = ""
+    indices: tuple = ()
+    pos_scale: float = 0.25
+    vel_scale: float = 0.25
+    sq_scale: float = 0.1
+    abs_scale: float = 0.1
+
+    def descs(self):  # pragma: no cover
+        raise ValueError("JointPositionReward reads a named command: pass command_slices to get_rewards")
+
+    def descs_in(self, obs_slices, command_slices):
+        if self.command_name not in command_slices:
+            raise ValueError(f"Command {self.command_name} not found! Ensure that it is in the task.")
+        if not (self.sq_scale > 0.0 and self.abs_scale > 0.0):
+            raise ValueError("sq_scale and abs_scale must be positive")
+        cm, n = command_slices[self.command_name], len(self.indices)
+        if cm.stop - cm.start != 2 * n + 3:
+            raise ValueError(f"the command holds {cm.stop - cm.start} numbers, a joint-position command of {n} joints holds {2 * n + 3}")
+        idx = [float(i) for i in self.indices]
+        return [("pos", T.REW_JOINT_POSITION, 0, self.pos_scale, self.sq_scale, self.abs_scale, 0.0, cm.start, _extra(count=n, params=idx)),
+                ("vel", T.REW_JOINT_VELOCITY_CMD, 0, self.vel_scale, self.sq_scale, self.abs_scale, 0.0, cm.start, _extra(count=n, params=idx))]
+
+    @classmethod
+    def create(cls, physics_model, joint_names, command_name, pos_scale=0.25, vel_scale=0.25, sq_scale=0.1, abs_scale=0.1, scale=1.0):
+        names = list(physics_model.body_names)
+        for n in joint_names:
+            if n not in names:
+                raise ValueError(f"Joint {n} not found in the model! Options are: {names[1:]}")
+        idx = tuple(int(physics_model.body_qadr[names.index(n)]) - 7 for n in joint_names)
+        return cls(command_name=command_name, indices=idx, pos_scale=pos_scale, vel_scale=vel_scale, sq_scale=sq_scale,
+                   abs_scale=abs_scale, scale=scale)
+
+
 DISCRIMINATOR_OUTPUT_KEY = "_discriminator_output"  # ksim/task/amp.py:47
 
 
@@ -458,6 +496,10 @@ class StatefulReward(Reward):
     def suffixes(self) -> tuple:
         return (None,)
 
+    def initial_carry(self) -> tuple:
+        """The carry an env starts with, and restarts with when its rollout ended on a done step (rl.py:206-214)."""
+        return (0.0,) * self.carry_size()
+
     def scan_desc(self, obs_slices: Mapping[str, slice], command_slices: Mapping[str, slice], level: float) -> T.KsRewardScanDesc:
         raise NotImplementedError  # pragma: no cover
 
@@ -544,8 +586,99 @@ class SparseTargetHeightReward(StatefulReward):  # rewards.py:1148-1192
         return d
 
 
+@dataclass(frozen=True)
+class SymmetryReward(StatefulReward):  # rewards.py:843-896
+    """With x = qpos[7 + joint] - target: the carry follows the rollout's mean x with rate alpha (once per rollout), and the
+    reward is -sum_j x_j carry_j, which pushes each joint away from the side it has been leaning to."""
+    joint_indices: tuple = ()
+    joint_targets: tuple = ()
+    alpha: float = 0.1
+
+    def carry_size(self):
+        return len(self.joint_indices)
+
+    def n_slots(self):
+        return 1
+
+    def initial_carry(self):
+        return tuple(float(x) for x in self.joint_targets)  # rewards.py:865-866
+
+    def scan_desc(self, obs_slices, command_slices, level):
+        n = len(self.joint_indices)
+        if n != len(self.joint_targets):
+            raise ValueError(f"Joint names and targets must match, got {n} and {len(self.joint_targets)}")
+        if not 1 <= n <= T.KS_MAX_SCAN_JOINTS:
+            raise ValueError(f"1..{T.KS_MAX_SCAN_JOINTS} joints, got {n}")
+        d = T.KsRewardScanDesc()
+        d.kind, d.n, d.alpha = T.SCAN_SYMMETRY, n, self.alpha
+        for k, (j, t) in enumerate(zip(self.joint_indices, self.joint_targets)):
+            d.joints[k], d.targets[k] = int(j), float(t)
+        return d
+
+    @classmethod
+    def create(cls, physics_model, joint_names, joint_targets, alpha=0.1, scale=1.0):
+        names = list(physics_model.body_names)
+        idx = tuple(int(physics_model.body_qadr[names.index(n)]) - 7 for n in joint_names)
+        if len(joint_names) != len(joint_targets):
+            raise ValueError(f"Joint names and targets must match, got {len(joint_names)} and {len(joint_targets)}")
+        return cls(joint_indices=idx, joint_targets=tuple(float(x) for x in joint_targets), alpha=alpha, scale=scale)
+
+
+@dataclass(frozen=True)
+class PairwiseSymmetryReward(StatefulReward):  # rewards.py:899-936
+    """Two terms for a left / right pair of joints (each minus its zero, the right one negated when `flipped`): "lr", a
+    kernel of their difference, and "self", the SymmetryReward of the pair."""
+    left_joint_index: int = 0
+    right_joint_index: int = 0
+    left_zero: float = 0.0
+    right_zero: float = 0.0
+    flipped: bool = False
+    alpha: float = 0.1
+    kernel_scale: float = 0.25
+    sq_scale: float = 0.1
+    abs_scale: float = 0.1
+
+    def carry_size(self):
+        return 2
+
+    def n_slots(self):
+        return 2
+
+    def suffixes(self):
+        return ("lr", "self")
+
+    def initial_carry(self):
+        return (float(self.left_zero), float(self.right_zero))  # rewards.py:913-914
+
+    def scan_desc(self, obs_slices, command_slices, level):
+        if not (self.sq_scale > 0.0 and self.abs_scale > 0.0):
+            raise ValueError("sq_scale and abs_scale must be positive")
+        d = T.KsRewardScanDesc()
+        d.kind, d.n, d.alpha, d.flipped = T.SCAN_PAIRWISE_SYMMETRY, 2, self.alpha, int(self.flipped)
+        d.joints[0], d.joints[1] = int(self.left_joint_index), int(self.right_joint_index)
+        d.targets[0], d.targets[1] = float(self.left_zero), float(self.right_zero)
+        d.kernel_scale, d.sq_scale, d.abs_scale = self.kernel_scale, self.sq_scale, self.abs_scale
+        return d
+
+    @classmethod
+    def create(cls, physics_model, left_joint_name, right_joint_name, left_zero=0.0, right_zero=0.0, flipped=False, alpha=0.1,
+               kernel_scale=0.25, sq_scale=0.1, abs_scale=0.1, scale=1.0):
+        names = list(physics_model.body_names)
+        li, ri = (int(physics_model.body_qadr[names.index(n)]) - 7 for n in (left_joint_name, right_joint_name))
+        return cls(left_joint_index=li, right_joint_index=ri, left_zero=left_zero, right_zero=right_zero, flipped=flipped,
+                   alpha=alpha, kernel_scale=kernel_scale, sq_scale=sq_scale, abs_scale=abs_scale, scale=scale)
+
+
 def reward_carry_size(rewards: Mapping[str, Reward]) -> int:
     return sum(r.carry_size() for r in rewards.values() if isinstance(r, StatefulReward))
+
+
+def initial_reward_carry(rewards: Mapping[str, Reward], num_envs: int, device) -> torch.Tensor | None:
+    """(N, reward_carry_size) filled with every stateful reward's initial carry, or None without stateful rewards."""
+    row = [x for r in rewards.values() if isinstance(r, StatefulReward) for x in r.initial_carry()]
+    if not row:
+        return None
+    return torch.tensor(row, dtype=torch.float32, device=device).repeat(int(num_envs), 1).contiguous()
 
 
 def _scan_stateful(trajectory, rewards, rewards_carry, obs_slices, command_slices, obs_key, level, Tn, N):
@@ -553,14 +686,21 @@ def _scan_stateful(trajectory, rewards, rewards_carry, obs_slices, command_slice
     stateful = {n: r for n, r in rewards.items() if isinstance(r, StatefulReward)}
     if len(stateful) > T.KS_MAX_REWARD_SCANS:
         raise _lib.KsError(f"at most {T.KS_MAX_REWARD_SCANS} stateful rewards")
-    if obs_slices is None:
-        raise _lib.KsError("stateful rewards read named observations: pass obs_slices (EnvTerms.obs_slices)")
-    obs = trajectory.obs[obs_key]
-    _lib.require_cuda(obs, dtype=torch.float32)
-    if obs.dim() != 3 or tuple(obs.shape[:2]) != (Tn, N):
-        raise _lib.KsError(f"observation leaf has shape {tuple(obs.shape)}, expected ({Tn}, {N}, obs_dim)")
+    reads_obs = any(not isinstance(r, (SymmetryReward, PairwiseSymmetryReward)) for r in stateful.values())
     io = T.KsRewardScanIO()
-    io.T, io.N, io.obs_dim, io.nv = Tn, N, obs.shape[-1], trajectory.qvel.shape[-1]
+    io.T, io.N, io.nv = Tn, N, trajectory.qvel.shape[-1]
+    obs = None
+    if reads_obs:
+        if obs_slices is None:
+            raise _lib.KsError("stateful rewards read named observations: pass obs_slices (EnvTerms.obs_slices)")
+        obs = trajectory.obs[obs_key]
+        _lib.require_cuda(obs, dtype=torch.float32)
+        if obs.dim() != 3 or tuple(obs.shape[:2]) != (Tn, N):
+            raise _lib.KsError(f"observation leaf has shape {tuple(obs.shape)}, expected ({Tn}, {N}, obs_dim)")
+        io.obs_dim, io.obs = obs.shape[-1], obs.data_ptr()
+    _lib.require_cuda(trajectory.qpos, dtype=torch.float32)
+    io.qpos, io.nq = trajectory.qpos.data_ptr(), trajectory.qpos.shape[-1]
+    dev = trajectory.qpos.device
     slots, carry_at, first = 0, 0, {}
     for j, (name, r) in enumerate(stateful.items()):
         d = r.scan_desc(obs_slices, command_slices or {}, level)
@@ -571,7 +711,7 @@ def _scan_stateful(trajectory, rewards, rewards_carry, obs_slices, command_slice
         carry_at += r.carry_size()
     io.n_scans, io.n_slots, io.carry_dim = len(stateful), slots, carry_at
     if rewards_carry is None:
-        rewards_carry = torch.zeros((N, carry_at), dtype=torch.float32, device=obs.device)  # initial_carry: zeros
+        rewards_carry = initial_reward_carry(rewards, N, dev)
     _lib.require_cuda(rewards_carry, dtype=torch.float32)
     if tuple(rewards_carry.shape) != (N, carry_at):
         raise _lib.KsError(f"reward carry has shape {tuple(rewards_carry.shape)}, expected {(N, carry_at)}")
@@ -581,9 +721,9 @@ def _scan_stateful(trajectory, rewards, rewards_carry, obs_slices, command_slice
         if cmd.dim() != 3 or tuple(cmd.shape[:2]) != (Tn, N):
             raise _lib.KsError(f"command leaf has shape {tuple(cmd.shape)}, expected ({Tn}, {N}, command_dim)")
         io.command_dim, io.command = cmd.shape[-1], cmd.data_ptr()
-    out = torch.empty((slots, Tn, N), dtype=torch.float32, device=obs.device)
+    out = torch.empty((slots, Tn, N), dtype=torch.float32, device=dev)
     done = trajectory.done.view(torch.uint8) if trajectory.done.dtype == torch.bool else trajectory.done
-    io.obs, io.qvel, io.done = obs.data_ptr(), trajectory.qvel.data_ptr(), done.data_ptr()
+    io.qvel, io.done = trajectory.qvel.data_ptr(), done.data_ptr()
     io.carry, io.out = rewards_carry.data_ptr(), out.data_ptr()
     _lib.check(_lib.load().ks_reward_scan(_lib.current_stream(), ctypes.byref(io)))
     return out, first, rewards_carry
@@ -690,7 +830,8 @@ def get_rewards(trajectory: Trajectory, rewards: Mapping[str, Reward], clip_min:
                 raise _lib.KsError(f"trajectory.{name} has {flat.shape[-1]} entries per step: not (nb, {per}) for the other leaf's nb")
             io.nb = flat.shape[-1] // per
             setattr(io, name, flat.data_ptr())
-    if kinds & {T.REW_LINVEL_CMD, T.REW_ANGVEL_CMD, T.REW_POSITION_TRACKING, T.REW_SINUSOIDAL_GAIT}:
+    if kinds & {T.REW_LINVEL_CMD, T.REW_ANGVEL_CMD, T.REW_POSITION_TRACKING, T.REW_SINUSOIDAL_GAIT, T.REW_JOINT_POSITION,
+                T.REW_JOINT_VELOCITY_CMD}:
         cmd = trajectory.command.get("_buffer") if trajectory.command else None
         if cmd is None:
             raise KeyError('command-tracking rewards read trajectory.command["_buffer"] (T, N, command_dim)')

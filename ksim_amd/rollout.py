@@ -22,7 +22,7 @@ from .env_terms import EnvTerms, sample_action, sample_action_head, sample_actio
 from .mlp import MLP
 from .physics import DeviceModel
 from .recurrent import RecurrentNetwork
-from .rewards import Reward, get_rewards, reward_carry_size
+from .rewards import Reward, get_rewards, initial_reward_carry, reward_carry_size
 from .types import PhysicsState, RewardState, Trajectory
 
 
@@ -268,7 +268,7 @@ class Rollout:
                 setattr(env, name, net.initial_carry(self.N, self.done.device))
         n = reward_carry_size(self.c.rewards)
         if n and env.reward_carry is None:
-            env.reward_carry = torch.zeros(self.N, n, dtype=torch.float32, device=self.done.device)
+            env.reward_carry = initial_reward_carry(self.c.rewards, self.N, self.done.device)
 
     def _rewards(self, traj: Trajectory, env: RolloutEnvState, level: float, want_components: bool = False) -> RewardState:
         """get_rewards over the recorded rollout; the carries of stateful rewards live in the env state (rl.py:1640-1650)."""

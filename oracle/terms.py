@@ -757,3 +757,40 @@ def random_pitch_roll_reset(qpos, u01, pitch_range, roll_range):
     roll = roll_range[0] + u01 * (roll_range[1] - roll_range[0])
     q[3:7] = quat_mul(q[3:7], euler_to_quat(np.array([roll, pitch, 0.0])))
     return q
+
+
+# ------------------------------------------------------------------ symmetry and joint-position rewards
+def symmetry_reward(qpos_tq, carry, done_last, joint_indices, joint_targets, alpha=0.1):
+    """SymmetryReward.get_reward_stateful (rewards.py:868-877) with the carry restart of get_rewards (rl.py:206-214):
+    returns (reward (T,), new carry)."""
+    targets = np.asarray(joint_targets, dtype=np.float64)
+    carry = targets.copy() if done_last else np.asarray(carry, dtype=np.float64)
+    q = np.asarray(qpos_tq, dtype=np.float64)[:, np.asarray(joint_indices) + 7] - targets
+    new = carry * (1.0 - alpha) + q.mean(axis=0) * alpha
+    return (q * -new[None, :]).sum(axis=-1), new
+
+
+def pairwise_symmetry_reward(qpos_tq, carry, done_last, left, right, left_zero=0.0, right_zero=0.0, flipped=False, alpha=0.1,
+                             kernel_scale=0.25, sq_scale=0.1, abs_scale=0.1):
+    """PairwiseSymmetryReward.get_reward_stateful (rewards.py:916-936): returns ({"lr", "self"} each (T,), new carry)."""
+    carry = np.array([left_zero, right_zero], dtype=np.float64) if done_last else np.asarray(carry, dtype=np.float64)
+    q = np.asarray(qpos_tq, dtype=np.float64)
+    ql, qr = q[:, left + 7] - left_zero, q[:, right + 7] - right_zero
+    if flipped:
+        qr = -qr
+    lr = exp_kernel_with_penalty(ql - qr, kernel_scale, sq_scale, abs_scale)
+    pair = np.stack([ql, qr], axis=-1)
+    new = carry * (1.0 - alpha) + pair.mean(axis=0) * alpha
+    return {"lr": lr, "self": (pair * -new[None, :]).sum(axis=-1)}, new
+
+
+def joint_position_reward(qpos_tq, qvel_tv, start, target, total_time, num_steps, step_id, indices, pos_scale=0.25,
+                          vel_scale=0.25, sq_scale=0.1, abs_scale=0.1):
+    """JointPositionReward.get_reward (rewards.py:1366-1380) with JointPositionCommandValue.current_position / velocity
+    (commands.py:803-818).  start, target: (T, n); total_time, num_steps, step_id: (T,)."""
+    idx = np.asarray(indices)
+    cur_pos = start + (target - start) * (step_id / num_steps)[:, None]
+    cur_vel = (target - start) / total_time[:, None]
+    pos = exp_kernel_with_penalty(cur_pos - np.asarray(qpos_tq)[:, idx + 7], pos_scale, sq_scale, abs_scale)
+    vel = exp_kernel_with_penalty(cur_vel - np.asarray(qvel_tv)[:, idx + 6], vel_scale, sq_scale, abs_scale)
+    return {"pos": pos.mean(axis=-1), "vel": vel.mean(axis=-1)}

@@ -627,6 +627,67 @@ def test_stateful_rewards_scan_against_oracle():
         rw.get_rewards(traj, rewards, obs_slices={"feet_pos": slice(0, 6)}, command_slices={"lin": slice(0, 1), "ang": slice(2, 3)})
 
 
+def test_symmetry_and_joint_position_rewards_against_oracle():
+    """SymmetryReward, PairwiseSymmetryReward (stateful: the carry follows the rollout mean, restarts at the targets when
+    the rollout ended on a done step) and JointPositionReward over two consecutive rollouts, beside a stateless term."""
+    from ksim_amd import rewards as rw
+    from ksim_amd.types import Trajectory
+
+    Tn, N, nq, nv, nu = 16, 37, 27, 26, 20
+    rng = np.random.default_rng(31)
+    joints, targets = (0, 5, 3, 12, 19), (0.1, -0.2, 0.0, 0.3, -0.05)
+    cmd_idx = (2, 7, 11)
+    rewards = {
+        "alive": rw.StayAliveReward(scale=0.5),
+        "sym": rw.SymmetryReward(scale=1.5, joint_indices=joints, joint_targets=targets, alpha=0.2),
+        "hips": rw.PairwiseSymmetryReward(scale=0.7, left_joint_index=1, right_joint_index=6, left_zero=0.05, right_zero=-0.1,
+                                          flipped=True, alpha=0.3, kernel_scale=0.4, sq_scale=0.2, abs_scale=0.15),
+        "arms": rw.JointPositionReward(scale=2.0, command_name="arm_cmd", indices=cmd_idx, pos_scale=0.3, vel_scale=0.6,
+                                       sq_scale=0.05, abs_scale=0.1),
+    }
+    command_slices = {"other": slice(0, 2), "arm_cmd": slice(2, 2 + 2 * 3 + 3)}
+    carry = None
+    oc_sym = [np.array(targets) for _ in range(N)]
+    oc_pair = [np.array([0.05, -0.1]) for _ in range(N)]
+    for rollout in range(2):
+        qpos = rng.normal(size=(Tn, N, nq)).astype(np.float32) * 0.3
+        qvel = rng.normal(size=(Tn, N, nv)).astype(np.float32) * 0.5
+        cmd = rng.normal(size=(Tn, N, 11)).astype(np.float32) * 0.4
+        cmd[..., 8] = rng.uniform(0.1, 1.0, (Tn, N))                       # total_time
+        cmd[..., 9] = np.ceil(cmd[..., 8] / 0.02)                          # num_steps
+        cmd[..., 10] = np.floor(rng.random((Tn, N)) * (cmd[..., 9] + 1))   # step_id
+        done = rng.random((Tn, N)) < 0.05
+        done[-1] = rng.random(N) < 0.4
+        traj = Trajectory(qpos=t32(qpos), qvel=t32(qvel), xpos=None, xquat=None, ctrl=None, obs={}, command={"_buffer": t32(cmd)},
+                          event_state={}, action=t32(rng.normal(size=(Tn, N, nu))), done=torch.from_numpy(done).to(DEV), success=None,
+                          timestep=None)
+        st = rw.get_rewards(traj, rewards, rewards_carry=carry, command_slices=command_slices)
+        carry = st.carry["_buffer"]
+        assert list(st.components) == ["alive", "sym", "hips/lr", "hips/self", "arms/pos", "arms/vel"]
+        comp = {k: v.cpu().numpy() for k, v in st.components.items()}
+        want_total = np.zeros((Tn, N))
+        for e in range(N):
+            r, oc_sym[e] = ot.symmetry_reward(qpos[:, e], oc_sym[e], bool(done[-1, e]), joints, targets, alpha=0.2)
+            pr, oc_pair[e] = ot.pairwise_symmetry_reward(qpos[:, e], oc_pair[e], bool(done[-1, e]), 1, 6, 0.05, -0.1, flipped=True, alpha=0.3,
+                                                         kernel_scale=0.4, sq_scale=0.2, abs_scale=0.15)
+            jp = ot.joint_position_reward(qpos[:, e].astype(np.float64), qvel[:, e].astype(np.float64), cmd[:, e, 2:5].astype(np.float64),
+                                          cmd[:, e, 5:8].astype(np.float64), cmd[:, e, 8].astype(np.float64), cmd[:, e, 9].astype(np.float64),
+                                          cmd[:, e, 10].astype(np.float64), cmd_idx, pos_scale=0.3, vel_scale=0.6, sq_scale=0.05, abs_scale=0.1)
+            np.testing.assert_allclose(comp["sym"][:, e], 1.5 * r, rtol=2e-5, atol=2e-6)
+            np.testing.assert_allclose(comp["hips/lr"][:, e], 0.7 * pr["lr"], rtol=2e-5, atol=2e-6)
+            np.testing.assert_allclose(comp["hips/self"][:, e], 0.7 * pr["self"], rtol=2e-5, atol=2e-6)
+            np.testing.assert_allclose(comp["arms/pos"][:, e], 2.0 * jp["pos"], rtol=2e-5, atol=2e-6)
+            np.testing.assert_allclose(comp["arms/vel"][:, e], 2.0 * jp["vel"], rtol=2e-5, atol=2e-6)
+            want_total[:, e] = 1.5 * r + 0.7 * (pr["lr"] + pr["self"]) + 2.0 * (jp["pos"] + jp["vel"]) + comp["alive"][:, e]
+        np.testing.assert_allclose(st.total.cpu().numpy(), want_total, rtol=2e-5, atol=1e-5)
+        cr = carry.cpu().numpy()
+        np.testing.assert_allclose(cr[:, :5], np.array(oc_sym), rtol=1e-5, atol=1e-6)
+        np.testing.assert_allclose(cr[:, 5:7], np.array(oc_pair), rtol=1e-5, atol=1e-6)
+    assert rw.reward_carry_size(rewards) == 7
+    with pytest.raises(ValueError, match="not found"):
+        rw.get_rewards(traj, rewards, command_slices={"other": slice(0, 2)})
+
+
 def test_gaussian_head_with_state_dependent_deviation():
     """mean | raw deviation head (examples/kbot/train.py:915-932): softplus, floor, scale and cap of the deviation, the
     sample, its log-density against scipy, scrub and clip."""

@@ -649,3 +649,31 @@ def test_new_reset_restatements_hand_computed():
     a = ot.random_heading_reset(ot.random_pitch_roll_reset(q0, 1.0, (0.0, 0.0), (0.0, 0.6)), 0.5)
     b = ot.random_pitch_roll_reset(ot.random_heading_reset(q0, 0.5), 1.0, (0.0, 0.0), (0.0, 0.6))
     assert np.abs(a[3:7] - b[3:7]).max() > 0.1
+
+
+def test_symmetry_and_joint_position_rewards_hand_computed():
+    """rewards.py:843-936, 1352-1380 on numbers small enough to do by hand."""
+    # two joints (qpos 7 and 9), targets (0.1, -0.2), two steps: x = [[0.4, 0.2], [0.0, 0.6]], mean (0.2, 0.4)
+    q = np.zeros((2, 10))
+    q[:, 7], q[:, 9] = [0.5, 0.1], [0.0, 0.4]
+    r, c = ot.symmetry_reward(q, np.array([1.0, -1.0]), False, (0, 2), (0.1, -0.2), alpha=0.5)
+    np.testing.assert_allclose(c, [0.5 + 0.1, -0.5 + 0.2])            # 0.5 carry + 0.5 mean
+    np.testing.assert_allclose(r, [-(0.4 * 0.6 + 0.2 * -0.3), -(0.0 * 0.6 + 0.6 * -0.3)])
+    _, c2 = ot.symmetry_reward(q, np.array([1.0, -1.0]), True, (0, 2), (0.1, -0.2), alpha=0.5)
+    np.testing.assert_allclose(c2, [0.05 + 0.1, -0.1 + 0.2])          # restarts from the targets
+    # a pair, right joint flipped: ql = (0.3, 0.1), qr = -(q8 - 0.1) = (0.2, -0.1); difference (0.1, 0.2)
+    q = np.zeros((2, 10))
+    q[:, 7], q[:, 8] = [0.3, 0.1], [-0.1, 0.2]
+    out, c = ot.pairwise_symmetry_reward(q, np.zeros(2), False, 0, 1, 0.0, 0.1, flipped=True, alpha=1.0, kernel_scale=0.5,
+                                         sq_scale=0.2, abs_scale=0.3)
+    np.testing.assert_allclose(c, [0.2, 0.05])
+    np.testing.assert_allclose(out["self"], [-(0.3 * 0.2 + 0.2 * 0.05), -(0.1 * 0.2 - 0.1 * 0.05)])
+    d = np.array([0.1, 0.2])
+    np.testing.assert_allclose(out["lr"], np.exp(-d**2 / (2 * 0.25)) - 0.2 * d**2 - 0.3 * np.abs(d))
+    # joint-position command half way (step 2 of 4) from 0 to 1 over 0.5 s: position 0.5, velocity 2
+    q, v = np.zeros((1, 9)), np.zeros((1, 8))
+    q[0, 8], v[0, 7] = 0.5, 1.5
+    out = ot.joint_position_reward(q, v, np.array([[0.0]]), np.array([[1.0]]), np.array([0.5]), np.array([4.0]), np.array([2.0]), (1,),
+                                   pos_scale=0.25, vel_scale=0.5, sq_scale=0.1, abs_scale=0.2)
+    assert out["pos"][0] == pytest.approx(1.0)                        # on target: exp(0) and no penalty
+    assert out["vel"][0] == pytest.approx(np.exp(-0.25 / 0.5) - 0.1 * 0.25 - 0.2 * 0.5)
