@@ -354,11 +354,17 @@ enum { /* KsObsElem.kind */
                            SensorObservation reads from sensordata, observation.py:307-340): the body's angular velocity in
                            the site frame, (q_body q_site)^-1 w, with q_body = xquat[index], w = cvel[index][0:3] (both of
                            the last substep's forward pass, as sensordata is) and q_site = (e0, e1, e2, e3) */
-  KS_OBS_SITE_ACCEL = 7  /* component `comp` of an accelerometer at a site of the floating base (body `index`, the one the
+  KS_OBS_SITE_ACCEL = 7, /* component `comp` of an accelerometer at a site of the floating base (body `index`, the one the
                            free joint moves): the site's acceleration minus gravity in the site frame,
                            (q_body q_site)^-1 (qacc[0:3] + alpha x r + w x (w x r) - g), alpha = R_body qacc[3:6],
                            r = R_body (c0, c1, c2), g = (q0, q1, q2), q_site = (e0, e1, e2, e3) */
+  KS_OBS_SITE_ROT6D = 8, /* entry `comp` (0..5) of the 6-D rotation of a site of body `index` (SiteOrientationObservation,
+                           observation.py:645-669): the first two rows of R(q_body q_site), row-major */
+  KS_OBS_CONTACT_ANY = 9 /* 1 when any contact sphere whose bit is set in `index` touches the floor: the floor's own entry of
+                           ContactObservation (observation.py:452-478), whose geom list holds the floor and some spheres */
 };
+/* Site kinds with env_site = 1 read the site's pose per env from KsObserveIO.site_pose instead of (e0..e3) and (c0, c1, c2):
+ * the IMU mounting error of IMUAlignmentRandomizer (ksim/randomization.py:245-284) is a model field there, one per env. */
 /* Noise and bias of an observation (ksim/noise.py:129-229, applied by Observation.add_noise, ksim/observation.py:110-142:
  * first the noise, then the per-episode bias).  A stage draws rv = mean + level (scale z + scale2 w) with z ~ N(0,1),
  * w ~ U(-1,1) (Gaussian kinds: scale = std; uniform kinds: scale2 = mag; the uniform-Gaussian kinds of
@@ -385,6 +391,7 @@ typedef struct KsObsElem {
   int32_t carry, stride;         /* stateful kinds: offset into the env's carry row, distance between delay slots */
   float q0, q1, q2;              /* KS_OBS_GRAVITY_EMA: min_lag, max_lag, imu_bias; KS_OBS_SITE_ACCEL: gravity */
   float e0, e1, e2, e3;          /* site kinds: the site's orientation in its body, wxyz */
+  int32_t env_site;              /* site kinds: 1 = take the site's pose from KsObserveIO.site_pose */
 } KsObsElem;
 
 /* Terminations (replaces get_terminations + terms, rl.py:288-299, ksim/terminations.py:60-192). */
@@ -452,6 +459,8 @@ typedef struct KsObserveIO {
                                  current state before observing (initial_carry, rl.py:1034-1080) and its bias draws are
                                  renewed; NULL = none */
   const float* carry_uniform; /* (N, carry_dim) U[0,1) draws for the initial carries, nullable -> Philox */
+  const float* site_pose;     /* (N, 7) per-env orientation (wxyz) and position of the randomised site in its body; required
+                                 when an element has env_site set */
 } KsObserveIO;
 int ks_observe(const KsTerms* terms, ks_stream_t stream, const KsObserveIO* io /*host*/);
 

@@ -7,7 +7,8 @@ from ctypes import POINTER, c_float, c_int8, c_int32, c_int64, c_uint8, c_uint64
 KS_MAX_OBS, KS_MAX_TERMS, KS_MAX_QPOS, KS_MAX_LAYERS = 512, 16, 40, 8
 (SRC_QPOS, SRC_QVEL, SRC_QACC, SRC_CTRL, SRC_LAST_ACTION, SRC_COMMAND, SRC_TIME, SRC_XPOS, SRC_XQUAT, SRC_CVEL,
  SRC_CONST, SRC_CONTACT_DIST, SRC_CINERT, SRC_CFRC_EXT, SRC_COUNT) = range(15)
-OBS_COPY, OBS_JOINT_POS, OBS_ROT_INV, OBS_CONTACT, OBS_DELAYED, OBS_GRAVITY_EMA, OBS_SITE_GYRO, OBS_SITE_ACCEL = range(8)
+(OBS_COPY, OBS_JOINT_POS, OBS_ROT_INV, OBS_CONTACT, OBS_DELAYED, OBS_GRAVITY_EMA, OBS_SITE_GYRO, OBS_SITE_ACCEL,
+ OBS_SITE_ROT6D, OBS_CONTACT_ANY) = range(10)
 (NOISE_NONE, NOISE_ADD_GAUSSIAN, NOISE_ADD_UNIFORM, NOISE_MUL_GAUSSIAN, NOISE_MUL_UNIFORM, NOISE_ADD_UNIFORM_GAUSSIAN,
  NOISE_MUL_UNIFORM_GAUSSIAN) = range(7)
 KS_MAX_NOISE_CHAIN = 4
@@ -29,7 +30,7 @@ class KsObsElem(ctypes.Structure):
     _fields_ = [("kind", c_int32), ("src", c_int32), ("index", c_int32), ("comp", c_int32), ("c0", c_float),
                 ("c1", c_float), ("c2", c_float), ("n_noise", c_int32), ("noise", KsNoiseStage * KS_MAX_NOISE_CHAIN),
                 ("bias", KsNoiseStage), ("carry", c_int32), ("stride", c_int32), ("q0", c_float), ("q1", c_float),
-                ("q2", c_float), ("e0", c_float), ("e1", c_float), ("e2", c_float), ("e3", c_float)]
+                ("q2", c_float), ("e0", c_float), ("e1", c_float), ("e2", c_float), ("e3", c_float), ("env_site", c_int32)]
 
 
 class KsTermDesc(ctypes.Structure):
@@ -69,7 +70,7 @@ class KsObserveIO(ctypes.Structure):
                 ("bias_draw", c_void_p), ("bias_redraw", c_void_p), ("noise_normal", c_void_p), ("noise_uniform", c_void_p),
                 ("rng", KsRng),
                 ("obs", c_void_p), ("noisy_obs", c_void_p), ("carry", c_void_p), ("fresh", c_void_p),
-                ("carry_uniform", c_void_p)]
+                ("carry_uniform", c_void_p), ("site_pose", c_void_p)]
 
 
 class KsTerminateIO(ctypes.Structure):

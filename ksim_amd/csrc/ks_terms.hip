@@ -38,6 +38,7 @@ struct ObserveArgs {
   float* carry;
   const uint8_t* fresh;
   const float* carry_uniform;
+  const float* site_pose;
   int carry_dim;
 };
 
@@ -114,6 +115,25 @@ __global__ __launch_bounds__(256) void observe_kernel(ObserveArgs a) {
     x = x * lag + p[el.comp] * (1.f - lag);
     c[el.comp] = x;
     v = x;
+  } else if (el.kind == KS_OBS_CONTACT_ANY) {
+    bool any = false;
+    for (int sidx = 0; sidx < a.src_dim[KS_SRC_CONTACT_DIST]; ++sidx)
+      any |= ((el.index >> sidx) & 1) && a.src[KS_SRC_CONTACT_DIST][e * a.src_dim[KS_SRC_CONTACT_DIST] + sidx] < 0.f;
+    v = any ? 1.f : 0.f;
+  } else if (el.kind == KS_OBS_SITE_ROT6D) {
+    const float* qb = a.src[KS_SRC_XQUAT] + e * a.src_dim[KS_SRC_XQUAT] + 4 * el.index;
+    float qs[4] = {el.e0, el.e1, el.e2, el.e3};
+    if (el.env_site) for (int k = 0; k < 4; ++k) qs[k] = a.site_pose[e * 7 + k];
+    // world orientation of the site: q = q_body q_site; row i of R(q) is what the inverse rotation makes of axis i
+    const float q[4] = {qb[0] * qs[0] - qb[1] * qs[1] - qb[2] * qs[2] - qb[3] * qs[3],
+                        qb[0] * qs[1] + qb[1] * qs[0] + qb[2] * qs[3] - qb[3] * qs[2],
+                        qb[0] * qs[2] - qb[1] * qs[3] + qb[2] * qs[0] + qb[3] * qs[1],
+                        qb[0] * qs[3] + qb[1] * qs[2] - qb[2] * qs[1] + qb[3] * qs[0]};
+    const int row = el.comp / 3, col = el.comp - 3 * row;
+    float col_vec[3], axis[3] = {0.f, 0.f, 0.f};
+    axis[col] = 1.f;
+    rot_fwd(q, axis, col_vec);  // column `col` of R
+    v = col_vec[row];
   } else if (el.kind == KS_OBS_SITE_GYRO || el.kind == KS_OBS_SITE_ACCEL) {
     const float* qb = a.src[KS_SRC_XQUAT] + e * a.src_dim[KS_SRC_XQUAT] + 4 * el.index;
     const float* w = a.src[KS_SRC_CVEL] + e * a.src_dim[KS_SRC_CVEL] + 6 * el.index;  // angular velocity, world axes
@@ -121,7 +141,9 @@ __global__ __launch_bounds__(256) void observe_kernel(ObserveArgs a) {
     if (el.kind == KS_OBS_SITE_ACCEL) {
       const float* qa = a.src[KS_SRC_QACC] + e * a.src_dim[KS_SRC_QACC];
       float r[3], al[3];
-      const float al_l[3] = {qa[3], qa[4], qa[5]}, r_l[3] = {el.c0, el.c1, el.c2};
+      const float al_l[3] = {qa[3], qa[4], qa[5]};
+      float r_l[3] = {el.c0, el.c1, el.c2};
+      if (el.env_site) for (int k = 0; k < 3; ++k) r_l[k] = a.site_pose[e * 7 + 4 + k];
       rot_fwd(qb, r_l, r);
       rot_fwd(qb, al_l, al);
       // w x r, then alpha x r + w x (w x r)
@@ -131,7 +153,8 @@ __global__ __launch_bounds__(256) void observe_kernel(ObserveArgs a) {
       vec[2] = qa[2] + (al[0] * r[1] - al[1] * r[0]) + (w[0] * wr[1] - w[1] * wr[0]) - el.q2;
     }
     float in_body[3], out[3];
-    const float qs[4] = {el.e0, el.e1, el.e2, el.e3};
+    float qs[4] = {el.e0, el.e1, el.e2, el.e3};
+    if (el.env_site) for (int k = 0; k < 4; ++k) qs[k] = a.site_pose[e * 7 + k];
     rot_inv(qb, vec[0], vec[1], vec[2], in_body);
     rot_inv(qs, in_body[0], in_body[1], in_body[2], out);
     v = out[el.comp];
@@ -1093,7 +1116,16 @@ extern "C" int ks_terms_create(const KsTermsDesc* d, KsTerms** out) {
   for (int k = 0; k < d->obs_dim; ++k) {
     const KsObsElem& el = d->obs[k];
     if (el.src < 0 || el.src >= KS_SRC_COUNT) return fail(KS_EINVAL, "ks_terms_create: obs %d: bad source %d", k, el.src);
-    if (el.kind < KS_OBS_COPY || el.kind > KS_OBS_SITE_ACCEL) return fail(KS_EINVAL, "ks_terms_create: obs %d: bad kind", k);
+    if (el.kind < KS_OBS_COPY || el.kind > KS_OBS_CONTACT_ANY) return fail(KS_EINVAL, "ks_terms_create: obs %d: bad kind", k);
+    if (el.kind == KS_OBS_CONTACT_ANY) {
+      if (d->ns < 1 || el.index <= 0 || (d->ns < 32 && (el.index >> d->ns) != 0)) return fail(KS_EINVAL, "ks_terms_create: obs %d: sphere mask 0x%x outside the model's %d spheres", k, el.index, d->ns);
+      continue;
+    }
+    if (el.kind == KS_OBS_SITE_ROT6D) {
+      if (el.comp < 0 || el.comp > 5 || el.index < 0 || el.index >= d->nb) return fail(KS_EINVAL, "ks_terms_create: obs %d: bad site orientation entry (component %d, body %d)", k, el.comp, el.index);
+      if (!(el.e0 * el.e0 + el.e1 * el.e1 + el.e2 * el.e2 + el.e3 * el.e3 > 0.f)) return fail(KS_EINVAL, "ks_terms_create: obs %d: the site orientation is not a quaternion", k);
+      continue;
+    }
     if (el.kind == KS_OBS_SITE_GYRO || el.kind == KS_OBS_SITE_ACCEL) {
       if (el.comp < 0 || el.comp > 2 || el.index < 0 || el.index >= d->nb) return fail(KS_EINVAL, "ks_terms_create: obs %d: bad site sensor (component %d, body %d)", k, el.comp, el.index);
       if (!(el.e0 * el.e0 + el.e1 * el.e1 + el.e2 * el.e2 + el.e3 * el.e3 > 0.f)) return fail(KS_EINVAL, "ks_terms_create: obs %d: the site orientation is not a quaternion", k);
@@ -1164,9 +1196,19 @@ extern "C" int ks_observe(const KsTerms* t, ks_stream_t stream, const KsObserveI
   bool needs_quat = false, needs_noise = false;
   for (int k = 0; k < d.obs_dim; ++k) {
     const KsObsElem& el = d.obs[k];
+    const bool site_kind = el.kind == KS_OBS_SITE_GYRO || el.kind == KS_OBS_SITE_ACCEL || el.kind == KS_OBS_SITE_ROT6D;
+    if (site_kind && el.env_site && !io->site_pose) return fail(KS_EINVAL, "ks_observe: observation %d reads the per-env site pose, which is NULL", k);
     if (el.kind == KS_OBS_SITE_GYRO || el.kind == KS_OBS_SITE_ACCEL) {
       if (!io->src[KS_SRC_XQUAT] || !io->src[KS_SRC_CVEL] || (el.kind == KS_OBS_SITE_ACCEL && !io->src[KS_SRC_QACC]))
         return fail(KS_EINVAL, "ks_observe: observation %d (site sensor) needs xquat, cvel and, for an accelerometer, qacc", k);
+      continue;
+    }
+    if (el.kind == KS_OBS_SITE_ROT6D) {
+      if (!io->src[KS_SRC_XQUAT]) return fail(KS_EINVAL, "ks_observe: observation %d (site orientation) needs xquat", k);
+      continue;
+    }
+    if (el.kind == KS_OBS_CONTACT_ANY) {
+      if (!io->src[KS_SRC_CONTACT_DIST]) return fail(KS_EINVAL, "ks_observe: observation %d reads contact_dist, which is NULL", k);
       continue;
     }
     if (el.src != KS_SRC_CONST && !io->src[el.src]) return fail(KS_EINVAL, "ks_observe: observation %d reads source %d, which is NULL", k, el.src);
@@ -1187,6 +1229,7 @@ extern "C" int ks_observe(const KsTerms* t, ks_stream_t stream, const KsObserveI
   a.zero_offset = io->zero_offset; a.bias_draw = needs_bias ? io->bias_draw : nullptr; a.bias_redraw = io->bias_redraw; a.noise_normal = io->noise_normal; a.noise_uniform = io->noise_uniform;
   a.rng = io->rng; a.obs = io->obs; a.noisy = io->noisy_obs; a.obs_dim = d.obs_dim; a.nq = d.nq; a.nu = d.nu;
   a.carry = io->carry; a.fresh = io->fresh; a.carry_uniform = io->carry_uniform; a.carry_dim = d.carry_dim;
+  a.site_pose = io->site_pose;
   const int64_t n = io->N * d.obs_dim;
   const int64_t grid = (n + 255) / 256;
   if (grid > 0x7fffffff) return fail(KS_ELIMIT, "ks_observe: too many elements");

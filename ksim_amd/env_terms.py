@@ -56,9 +56,14 @@ def compile_terms(model: KinematicModel, observations: Mapping[str, Observation]
             e.carry, e.stride = carry_at + el.carry, el.stride
             e.q0, e.q1, e.q2 = el.q
             e.e0, e.e1, e.e2, e.e3 = el.e
+            e.env_site = int(el.env_site)
             sources_used.add(el.src)
             if el.kind == T.OBS_GRAVITY_EMA:
                 sources_used.add(T.SRC_QPOS)
+            if el.kind == T.OBS_CONTACT_ANY:
+                sources_used.add(T.SRC_CONTACT_DIST)
+            if el.kind == T.OBS_SITE_ROT6D:
+                sources_used.add(T.SRC_XQUAT)
             if el.kind in (T.OBS_SITE_GYRO, T.OBS_SITE_ACCEL):
                 sources_used.update((T.SRC_XQUAT, T.SRC_CVEL) + ((T.SRC_QACC,) if el.kind == T.OBS_SITE_ACCEL else ()))
             if noise is not None:
@@ -117,11 +122,12 @@ class EnvTerms:
     # ------------------------------------------------------------------ observations
     def observe(self, sources: Mapping[int, torch.Tensor | None], N: int, *, level: float = 1.0,
                 zero_offset=None, bias_draw=None, bias_redraw=None, noise_normal=None, noise_uniform=None, seed: int = 0,
-                step: int = 0, step_base=None, carry=None, fresh=None, carry_uniform=None,
+                step: int = 0, step_base=None, carry=None, fresh=None, carry_uniform=None, site_pose=None,
                 obs: torch.Tensor | None = None, noisy_obs: torch.Tensor | None = None):
         """`carry` (N, carry_dim) is advanced in place; `fresh` (N) uint8 marks the envs whose carries are initialised
         from the current state first (those that were just reset) and whose bias draws `bias_draw` (N, obs_dim, 2) are
-        renewed (from `bias_redraw` when given, else from the Philox stream)."""
+        renewed (from `bias_redraw` when given, else from the Philox stream).  `site_pose` (N, 7): per-env orientation
+        (wxyz) and position of the site that the observations built with `site_pose_per_env` read."""
         m = self.model
         dims = {T.SRC_QPOS: m.nq, T.SRC_QVEL: m.nv, T.SRC_QACC: m.nv, T.SRC_CTRL: m.nu, T.SRC_LAST_ACTION: self.action_dim,
                 T.SRC_COMMAND: self.command_dim, T.SRC_TIME: 1, T.SRC_XPOS: m.nb * 3, T.SRC_XQUAT: m.nb * 4,
@@ -140,7 +146,7 @@ class EnvTerms:
                                ("noise_normal", noise_normal, (N, self.obs_dim)),
                                ("noise_uniform", noise_uniform, (N, self.obs_dim)), ("obs", obs, (N, self.obs_dim)),
                                ("noisy_obs", noisy_obs, (N, self.obs_dim)), ("carry", carry, (N, self.carry_dim)),
-                               ("carry_uniform", carry_uniform, (N, self.carry_dim))):
+                               ("carry_uniform", carry_uniform, (N, self.carry_dim)), ("site_pose", site_pose, (N, 7))):
             if t is None:
                 continue
             _lib.require_cuda(t, dtype=torch.float32)

@@ -26,6 +26,7 @@ class ObsElem:
     stride: int = 0
     q: tuple = (0.0, 0.0, 0.0)
     e: tuple = (1.0, 0.0, 0.0, 0.0)  # site kinds: the site's orientation in its body
+    env_site: int = 0   # site kinds: 1 = the site's pose comes per env (IMUAlignmentRandomizer)
 
 
 @dataclass(frozen=True)
@@ -304,6 +305,77 @@ class FeetContactObservation(Observation):
         return out
 
 
+FLOOR_GEOM = -1  # the floor plane in a list of geoms; contact spheres go by their index
+
+
+@dataclass(frozen=True)
+class ContactObservation(Observation):  # observation.py:452-478
+    """For each listed geom, whether it touches another listed geom (geoms_colliding of the list with itself, any over the
+    partners).  The collision model here is contact spheres against the floor plane, so a sphere's entry is its own floor
+    contact when `FLOOR_GEOM` is in the list (otherwise 0: spheres do not collide with each other) and the floor's entry
+    is whether any listed sphere touches it."""
+    geom_idxs: tuple = ()
+    contact_group: str | None = None
+
+    @classmethod
+    def create(cls, *, physics_model, geom_names, contact_group=None, noise=None):
+        """Geoms by name: "floor", or a body's name for all of its contact spheres."""
+        names = [geom_names] if isinstance(geom_names, str) else list(geom_names)
+        idx = []
+        for n in names:
+            if n == "floor":
+                idx.append(FLOOR_GEOM)
+                continue
+            if n not in physics_model.body_names:
+                raise ValueError(f"Geom name {n} not found in model")
+            b = list(physics_model.body_names).index(n)
+            idx += [i for i, sb in enumerate(physics_model.sph_body) if int(sb) == b]
+        return cls(geom_idxs=tuple(idx), contact_group=contact_group, noise=noise)
+
+    def elements(self, m, command_dim):
+        spheres = [int(g) for g in self.geom_idxs if g != FLOOR_GEOM]
+        if any(g < 0 or g >= m.ns for g in spheres):
+            raise ValueError(f"contact spheres are numbered 0..{m.ns - 1}")
+        has_floor = FLOOR_GEOM in self.geom_idxs
+        mask = sum(1 << g for g in set(spheres))
+        out = []
+        for g in self.geom_idxs:
+            if g == FLOOR_GEOM:
+                out.append(ObsElem(T.OBS_CONTACT_ANY, T.SRC_CONTACT_DIST, mask) if mask else ObsElem(T.OBS_COPY, T.SRC_CONST, 0))
+            elif has_floor:
+                out.append(ObsElem(T.OBS_CONTACT, T.SRC_CONTACT_DIST, int(g)))
+            else:
+                out.append(ObsElem(T.OBS_COPY, T.SRC_CONST, 0))
+        return out
+
+
+@dataclass(frozen=True)
+class SiteOrientationObservation(Observation):  # observation.py:645-669
+    """6-D rotation of each named site in the world frame: the first two rows of its rotation matrix, row-major.  (The
+    reference calls xax.rotation_matrix_to_rotation6d, whose entry order is not stated in the reference's own files.)"""
+    site_names: tuple = ()
+    name: str = "site_orientation"
+    site_pose_per_env: bool = False  # the site's pose is randomised per env (IMUAlignmentRandomizer): read it from `site_pose`
+
+    @classmethod
+    def create(cls, *, physics_model, site_names, noise=None):
+        for n in site_names:
+            if n not in physics_model.sites:
+                raise ValueError(f"site {n!r} not found in model. Available: {sorted(physics_model.sites)}")
+        return cls(site_names=tuple(site_names), name="site_orientation_observation_" + "_".join(site_names), noise=noise)
+
+    def elements(self, m, command_dim):
+        out = []
+        for n in self.site_names:
+            body, pos, quat = m.sites[n]
+            env = int(self.site_pose_per_env)
+            out += [ObsElem(T.OBS_SITE_ROT6D, T.SRC_XQUAT, body, c, e=tuple(quat), env_site=env) for c in range(6)]
+        return out
+
+    def get_name(self) -> str:
+        return self.name
+
+
 @dataclass(frozen=True)
 class LastActionObservation(Observation):
     """The previous control step's action (PhysicsState.last_ctrl, ksim/types.py:33-43)."""
@@ -330,6 +402,7 @@ class SensorObservation(Observation):
     contact sphere of that body is taken to lie inside the site's volume, which holds for the feet of the shipped robots).
     Like `sensordata`, they describe the state the last substep started from."""
     sensor_name: str = ""
+    site_pose_per_env: bool = False  # the sensor's site is randomised per env (IMUAlignmentRandomizer, randomization.py:245-284)
 
     @classmethod
     def create(cls, *, physics_model: KinematicModel, sensor_name: str, noise=None):
@@ -346,11 +419,13 @@ class SensorObservation(Observation):
         body, pos, quat = m.sites[site]
         if kind == "touch":
             return [ObsElem(T.OBS_COPY, T.SRC_CFRC_EXT, 6 * body + 5)]
+        env = int(self.site_pose_per_env)
         if kind == "gyro":
-            return [ObsElem(T.OBS_SITE_GYRO, T.SRC_CVEL, body, c, e=tuple(quat)) for c in range(3)]
+            return [ObsElem(T.OBS_SITE_GYRO, T.SRC_CVEL, body, c, e=tuple(quat), env_site=env) for c in range(3)]
         if body != 1 or not m.has_free_root:
             raise ValueError(f"accelerometer {self.sensor_name!r}: its site must sit on the floating base")
-        return [ObsElem(T.OBS_SITE_ACCEL, T.SRC_CVEL, body, c, const=tuple(pos), q=tuple(m.gravity), e=tuple(quat)) for c in range(3)]
+        return [ObsElem(T.OBS_SITE_ACCEL, T.SRC_CVEL, body, c, const=tuple(pos), q=tuple(m.gravity), e=tuple(quat), env_site=env)
+                for c in range(3)]
 
     def get_name(self) -> str:
         return self.sensor_name

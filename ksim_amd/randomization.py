@@ -187,6 +187,46 @@ class CollisionBodyRandomizer(PhysicsRandomizer):
         return {"sph_pos": pos.reshape(num_envs, -1), "sph_radius": rad}
 
 
+@dataclass(frozen=True)
+class IMUAlignmentRandomizer(PhysicsRandomizer):  # randomization.py:245-284
+    """Mounting error of the IMU site: small roll and pitch ~ N(0, tilt_std_rad), optionally yaw and a translation.  The
+    offset is the normalised product of the small-angle quaternions [1, angle / 2] about z, y, x, applied on the left of
+    the site's orientation.  Returns `site_pose` (N, 7): orientation (wxyz) then position of the site in its body, which the
+    observations built with `site_pose_per_env=True` read."""
+    site_name: str = "imu_site"
+    tilt_std_rad: float = 0.03490658503988659
+    yaw_std_rad: float | None = None
+    translate_std_m: float | None = None
+
+    def __call__(self, model, num_envs, gen, normal=None):
+        """`normal` (N, 6): explicit standard normal draws (rx, ry, rz, dx, dy, dz) instead of the generator's."""
+        if self.site_name not in model.sites:
+            raise ValueError(f"site {self.site_name!r} not found in model. Available: {sorted(model.sites)}")
+        dev = gen.device
+        z = torch.randn(num_envs, 6, generator=gen, device=dev) if normal is None else normal.to(dev)
+        body, pos, quat = model.sites[self.site_name]
+        h = 0.5
+        rx, ry = z[:, 0] * self.tilt_std_rad, z[:, 1] * self.tilt_std_rad
+        rz = z[:, 2] * self.yaw_std_rad if self.yaw_std_rad is not None else torch.zeros(num_envs, device=dev)
+        one, zero = torch.ones(num_envs, device=dev), torch.zeros(num_envs, device=dev)
+
+        def mul(a, b):  # Hamilton product, wxyz
+            aw, ax, ay, az = a
+            bw, bx, by, bz = b
+            return (aw * bw - ax * bx - ay * by - az * bz, aw * bx + ax * bw + ay * bz - az * by,
+                    aw * by - ax * bz + ay * bw + az * bx, aw * bz + ax * by - ay * bx + az * bw)
+
+        qx, qy, qz = (one, rx * h, zero, zero), (one, zero, ry * h, zero), (one, zero, zero, rz * h)
+        off = torch.stack(mul(qz, mul(qy, qx)), dim=-1)
+        off = off / off.norm(dim=-1, keepdim=True)
+        site = tuple(torch.full((num_envs,), float(v), device=dev) for v in quat)
+        new_quat = torch.stack(mul(tuple(off[:, k] for k in range(4)), site), dim=-1)
+        new_pos = torch.tensor(pos, dtype=torch.float32, device=dev)[None].repeat(num_envs, 1)
+        if self.translate_std_m is not None and self.translate_std_m > 0.0:
+            new_pos = new_pos + z[:, 3:6] * self.translate_std_m
+        return {"site_pose": torch.cat([new_quat, new_pos], dim=-1).float()}
+
+
 def get_physics_randomizers(model, randomizers: dict, num_envs: int, gen) -> dict:
     """Merges the randomisers' fields; duplicate fields raise (ksim/task/rl.py:343-346)."""
     out: dict = {}

@@ -147,7 +147,7 @@ class Rollout:
                         noise_normal=noise.get("obs_normal"), noise_uniform=noise.get("obs_uniform"), seed=env.seed,
                         step=step, step_base=step_base, obs=self.obs[t], noisy_obs=self.noisy_obs[t],
                         carry=env.obs_carry, fresh=self.reset_mask if (c.terms.carry_dim or c.terms.has_bias) else None,
-                        carry_uniform=noise.get("obs_carry_uniform"))
+                        carry_uniform=noise.get("obs_carry_uniform"), site_pose=(env.randomization_dict or {}).get("site_pose"))
         # actor reads the noisy copy (walking.py:592-595), critic the clean one (walking.py:626-638); recurrent networks
         # advance their carries, which restart from zero for the envs the previous control step reset
         if self.fresh is not None:

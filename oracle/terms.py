@@ -794,3 +794,40 @@ def joint_position_reward(qpos_tq, qvel_tv, start, target, total_time, num_steps
     pos = exp_kernel_with_penalty(cur_pos - np.asarray(qpos_tq)[:, idx + 7], pos_scale, sq_scale, abs_scale)
     vel = exp_kernel_with_penalty(cur_vel - np.asarray(qvel_tv)[:, idx + 6], vel_scale, sq_scale, abs_scale)
     return {"pos": pos.mean(axis=-1), "vel": vel.mean(axis=-1)}
+
+
+# ------------------------------------------------------------------ IMU mounting error, site orientation, contact list
+def imu_alignment_offset(rx, ry, rz=0.0):
+    """IMUAlignmentRandomizer's rotation offset (ksim/randomization.py:262-271): small-angle quaternions [1, angle / 2]
+    about x, y, z composed as qz * (qy * qx), normalised."""
+    qx, qy, qz = np.array([1.0, 0.5 * rx, 0.0, 0.0]), np.array([1.0, 0.0, 0.5 * ry, 0.0]), np.array([1.0, 0.0, 0.0, 0.5 * rz])
+    q = quat_mul(qz, quat_mul(qy, qx))
+    return q / np.linalg.norm(q)
+
+
+def quat_to_matrix(q):
+    w, x, y, z = (float(v) for v in np.asarray(q, dtype=np.float64) / np.linalg.norm(q))
+    return np.array([[1 - 2 * (y * y + z * z), 2 * (x * y - w * z), 2 * (x * z + w * y)],
+                     [2 * (x * y + w * z), 1 - 2 * (x * x + z * z), 2 * (y * z - w * x)],
+                     [2 * (x * z - w * y), 2 * (y * z + w * x), 1 - 2 * (x * x + y * y)]])
+
+
+def site_rotation6d(xquat_body, site_quat):
+    """SiteOrientationObservation (ksim/observation.py:664-669): site_xmat = R(q_body q_site), then its 6-D form, taken
+    here as the first two rows, row-major."""
+    return quat_to_matrix(quat_mul(np.asarray(xquat_body, np.float64), np.asarray(site_quat, np.float64)))[:2].reshape(6)
+
+
+def contact_observation(contact_dist, geom_idxs, floor=-1):
+    """ContactObservation (ksim/observation.py:452-478) for sphere-against-floor collisions: entry i says whether geom i
+    touches another geom of the list.  Spheres never touch each other."""
+    dist = np.asarray(contact_dist)
+    has_floor = floor in geom_idxs
+    spheres = [g for g in geom_idxs if g != floor]
+    out = []
+    for g in geom_idxs:
+        if g == floor:
+            out.append(any(dist[s] < 0 for s in spheres))
+        else:
+            out.append(bool(has_floor and dist[g] < 0))
+    return np.array(out)

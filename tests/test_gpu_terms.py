@@ -1219,3 +1219,42 @@ def test_sensor_observations_gyro_accelerometer_touch():
     air = (cf[:, :, 5].sum(1) == 0)
     if air.any():  # no contact: the base origin accelerates with gravity plus what the joints do; the reading stays moderate
         assert np.isfinite(got[air, 3:6]).all()
+
+    # IMUAlignmentRandomizer: every env has its own site pose; the sensors and the site's 6-D rotation follow it
+    from ksim_amd import randomization as rnd
+
+    zn = np.random.default_rng(95).normal(size=(N, 6))
+    r = rnd.IMUAlignmentRandomizer(site_name="imu_site", tilt_std_rad=0.05, yaw_std_rad=0.1, translate_std_m=0.01)
+    gen = torch.Generator(device=DEV); gen.manual_seed(1)
+    pose = r(m, N, gen, normal=t32(zn))["site_pose"]
+    want_pose = np.array([np.concatenate([ot.quat_mul(ot.imu_alignment_offset(0.05 * zn[e, 0], 0.05 * zn[e, 1], 0.1 * zn[e, 2]), np.array(squat)),
+                                          np.array(spos) + 0.01 * zn[e, 3:6]]) for e in range(N)])
+    np.testing.assert_allclose(pose.cpu().numpy(), want_pose, rtol=1e-6, atol=1e-7)
+    drawn = r(m, N, gen)["site_pose"].cpu().numpy()  # the generator's own draws: unit quaternions, tilts of the right size
+    np.testing.assert_allclose(np.linalg.norm(drawn[:, :4], axis=1), 1.0, atol=1e-6)
+    assert 0.5 * 0.05 < 2 * np.abs(drawn[:, 1]).std() < 2 * 0.05
+    obs2 = {"gyro": ob.SensorObservation(sensor_name="imu_gyro", site_pose_per_env=True),
+            "acc": ob.SensorObservation(sensor_name="imu_acc", site_pose_per_env=True),
+            "rot": ob.SiteOrientationObservation.create(physics_model=m, site_names=("imu_site", "left_foot")),
+            "rot_env": ob.SiteOrientationObservation(site_names=("imu_site",), site_pose_per_env=True),
+            "contact": ob.ContactObservation(geom_idxs=(0, ob.FLOOR_GEOM, m.ns - 1)),
+            "no_floor": ob.ContactObservation(geom_idxs=(0, 1))}
+    terms2 = EnvTerms(m, obs2, {}, [])
+    dist = np.random.default_rng(96).normal(size=(N, m.ns)) * 0.02
+    src[T.SRC_CONTACT_DIST] = t32(dist)
+    o2 = torch.empty(N, terms2.obs_dim, device=DEV)
+    with pytest.raises(Exception, match="site pose"):
+        terms2.observe(src, N, obs=o2)
+    terms2.observe(src, N, obs=o2, site_pose=pose)
+    g2, sl = o2.cpu().numpy(), terms2.obs_slices
+    lf_body, _, lf_quat = m.sites["left_foot"]
+    for e in range(N):
+        np.testing.assert_allclose(g2[e, sl["gyro"]], ot.site_gyro(xq[e, 1], cv[e, 1, :3], want_pose[e, :4]), rtol=1e-5, atol=1e-5)
+        np.testing.assert_allclose(g2[e, sl["acc"]], ot.site_accelerometer(qa[e, :6], xq[e, 1], cv[e, 1, :3], want_pose[e, 4:], want_pose[e, :4], m.gravity),
+                                   rtol=1e-4, atol=1e-3)
+        np.testing.assert_allclose(g2[e, sl["rot"]], np.concatenate([ot.site_rotation6d(xq[e, 1], squat), ot.site_rotation6d(xq[e, lf_body], lf_quat)]),
+                                   rtol=1e-5, atol=1e-5)
+        np.testing.assert_allclose(g2[e, sl["rot_env"]], ot.site_rotation6d(xq[e, 1], want_pose[e, :4]), rtol=1e-5, atol=1e-5)
+        assert np.array_equal(g2[e, sl["contact"]].astype(bool), ot.contact_observation(dist[e], (0, -1, m.ns - 1)))
+        assert not g2[e, sl["no_floor"]].any()
+    assert np.abs(g2[:, sl["gyro"]] - got[:, 0:3]).max() > 1e-3, "the mounting error changes nothing in this test"

@@ -677,3 +677,27 @@ def test_symmetry_and_joint_position_rewards_hand_computed():
                                    pos_scale=0.25, vel_scale=0.5, sq_scale=0.1, abs_scale=0.2)
     assert out["pos"][0] == pytest.approx(1.0)                        # on target: exp(0) and no penalty
     assert out["vel"][0] == pytest.approx(np.exp(-0.25 / 0.5) - 0.1 * 0.25 - 0.2 * 0.5)
+
+
+def test_imu_offset_site_rotation_and_contact_list_hand_computed():
+    # a pure roll error of 0.2 rad: [1, 0.1, 0, 0] normalised; to first order a rotation by 0.2 about x
+    q = ot.imu_alignment_offset(0.2, 0.0)
+    np.testing.assert_allclose(q, np.array([1, 0.1, 0, 0]) / np.sqrt(1.01))
+    v = ot.rotate_vector_by_quat(np.array([0.0, 1.0, 0.0]), q)
+    assert v[2] == pytest.approx(np.sin(2 * np.arctan(0.1)))  # the exact angle of [1, t] is 2 atan(t)
+    # order: yaw last, i.e. qz on the left; with all three angles the product differs from the reversed order
+    a = ot.imu_alignment_offset(0.3, -0.2, 0.5)
+    qx, qy, qz = np.array([1, 0.15, 0, 0]), np.array([1, 0, -0.1, 0]), np.array([1, 0, 0, 0.25])
+    b = ot.quat_mul(qz, ot.quat_mul(qy, qx))
+    np.testing.assert_allclose(a, b / np.linalg.norm(b))
+    wrong = ot.quat_mul(qx, ot.quat_mul(qy, qz))
+    assert np.abs(a - wrong / np.linalg.norm(wrong)).max() > 1e-2
+    # site rotation: body turned a quarter about z, site a quarter about x.  R = Rz(90) Rx(90): rows (0,0,1), (1,0,0)
+    s = np.sqrt(0.5)
+    np.testing.assert_allclose(ot.site_rotation6d([s, 0, 0, s], [s, s, 0, 0]), [0, 0, 1, 1, 0, 0], atol=1e-12)
+    np.testing.assert_allclose(ot.quat_to_matrix([s, 0, 0, s]) @ [1, 0, 0], [0, 1, 0], atol=1e-12)
+    # contact list: spheres 0 and 2 with the floor; 0 touches.  Without the floor in the list nothing collides.
+    dist = np.array([-0.01, -0.5, 0.02])
+    assert ot.contact_observation(dist, (0, -1, 2)).tolist() == [True, True, False]
+    assert ot.contact_observation(dist, (0, 1)).tolist() == [False, False]
+    assert ot.contact_observation(np.array([0.1, -0.5, 0.02]), (0, -1, 2)).tolist() == [False, False, False]
