@@ -136,6 +136,9 @@ typedef struct KsModelDesc {
                                         That is MuJoCo's Euler step with EULERDAMP and also, for models whose smooth forces
                                         depend on velocity only through joint damping (torque motors), its implicitfast
                                         integrator, which ksim selects (rl.py:555-578,730-748).  0: plain semi-implicit Euler */
+  int32_t condim;                    /* contact dimension of every sphere-floor contact: 3 (0 means 3) = friction pyramid, four
+                                        rows per contact; 1 = frictionless, one normal row regularised with the body's
+                                        translational inverse weight (MuJoCo condim, as examples/data/scene.mjcf:19,72 uses) */
   double dt, gravity[3], tolerance, ls_tolerance, impratio, meaninertia, friction;
   double solref[2], solimp[5];
   int32_t body_parent[KS_MAX_BODIES], body_jtype[KS_MAX_BODIES], body_qadr[KS_MAX_BODIES],

@@ -13,7 +13,7 @@ KS_ACT_TORQUE, KS_ACT_POSITION, KS_ACT_POSITION_VELOCITY = 0, 1, 2
 class KsModelDesc(ctypes.Structure):
     _fields_ = [
         ("nb", c_int32), ("nq", c_int32), ("nv", c_int32), ("nu", c_int32), ("ns", c_int32),
-        ("iterations", c_int32), ("ls_iterations", c_int32), ("eulerdamp", c_int32),
+        ("iterations", c_int32), ("ls_iterations", c_int32), ("eulerdamp", c_int32), ("condim", c_int32),
         ("dt", c_double), ("gravity", c_double * 3), ("tolerance", c_double), ("ls_tolerance", c_double),
         ("impratio", c_double), ("meaninertia", c_double), ("friction", c_double),
         ("solref", c_double * 2), ("solimp", c_double * 5),
@@ -61,6 +61,7 @@ def model_desc(m) -> KsModelDesc:
     for k in ("nb", "nq", "nv", "nu", "ns", "iterations", "ls_iterations"):
         setattr(d, k, int(getattr(m, k)))
     d.eulerdamp = int(bool(m.eulerdamp))
+    d.condim = int(getattr(m, "condim", 3))
     for k in ("dt", "tolerance", "ls_tolerance", "impratio", "meaninertia", "friction"):
         setattr(d, k, float(getattr(m, k)))
 

@@ -746,7 +746,8 @@ void step_kernel(StepArgs a) {
     const bool touching = is_sph && (dist < 0.f);
     const unsigned long long cmask = __ballot(touching);
     const int ncon = __popcll(cmask);
-    const int nefc = 4 * ncon;
+    const bool frictionless = m.frictionless != 0;
+    const int nefc = frictionless ? ncon : 4 * ncon;
     // A launch ends with its slowest wavefront, and an env with many contacts runs several times longer than an airborne
     // one: waves with more constraint rows get a higher issue priority on their SIMD, which shortens exactly those.
     if (nefc >= 20) __builtin_amdgcn_s_setprio(3);
@@ -758,7 +759,7 @@ void step_kernel(StepArgs a) {
       l.con_body[c] = s_body;
       l.con_mask[c] = s_mask;
       st3(l.con_off + 3 * c, cpos - com);
-      const float invweight = (s_invw + mu * mu * s_invw) * 2.f * mu * mu / m.impratio;
+      const float invweight = frictionless ? s_invw : (s_invw + mu * mu * s_invw) * 2.f * mu * mu / m.impratio;
       const float imp = impedance(m, dist);
       const float Rr = fmaxf(invweight * (1.f - imp) / imp, 1e-15f);
       l.con_D[c] = 1.0f / Rr;
@@ -815,7 +816,7 @@ void step_kernel(StepArgs a) {
       const bool is_row = lane < nefc;
       float aref = 0.f, D = 0.f;
       {
-        const int c = is_row ? lane >> 2 : 0, q = lane & 3;
+        const int c = is_row ? (frictionless ? lane : lane >> 2) : 0, q = lane & 3;
         const unsigned cm = is_row ? l.con_mask[c] : 0u;
         const V3 off = ld3(l.con_off + 3 * c);
         const float smu = (q & 1) ? -mu : mu;
@@ -831,7 +832,7 @@ void step_kernel(StepArgs a) {
             const Sp cd = ld6(l.cdof + 6 * j);
             const V3 jac = cd.l + cross(cd.a, off);
             const float tang = (q < 2) ? jac.y : -jac.x;
-            val = ((cm >> j) & 1u) ? jac.z + smu * tang : 0.f;
+            val = ((cm >> j) & 1u) ? (frictionless ? jac.z : jac.z + smu * tang) : 0.f;
           }
           vel += val * vv[j];
           if (is_row) l.J[lane * js + j] = val;
@@ -1073,13 +1074,16 @@ void step_kernel(StepArgs a) {
       if (a.cfrc_ext && sub == nsub - 1) {
         const float f = (is_row && Jaref < 0.f) ? -D * Jaref : 0.f;
         const int q = lane & 3;
-        float fx = q == 3 ? mu * f : (q == 2 ? -mu * f : 0.f);
-        float fy = q == 0 ? mu * f : (q == 1 ? -mu * f : 0.f);
-        float fz = f;
-        fx += __shfl_xor(fx, 1); fy += __shfl_xor(fy, 1); fz += __shfl_xor(fz, 1);
-        fx += __shfl_xor(fx, 2); fy += __shfl_xor(fy, 2); fz += __shfl_xor(fz, 2);
+        float fx = 0.f, fy = 0.f, fz = f;
+        if (!frictionless) {
+          fx = q == 3 ? mu * f : (q == 2 ? -mu * f : 0.f);
+          fy = q == 0 ? mu * f : (q == 1 ? -mu * f : 0.f);
+          fx += __shfl_xor(fx, 1); fy += __shfl_xor(fy, 1); fz += __shfl_xor(fz, 1);
+          fx += __shfl_xor(fx, 2); fy += __shfl_xor(fy, 2); fz += __shfl_xor(fz, 2);
+        }
         KS_SYNC();  // the line search is done with drow
-        if (is_row && q == 0) { l.drow[3 * (lane >> 2)] = fx; l.drow[3 * (lane >> 2) + 1] = fy; l.drow[3 * (lane >> 2) + 2] = fz; }
+        const int cc = frictionless ? lane : lane >> 2;
+        if (is_row && (frictionless || q == 0)) { l.drow[3 * cc] = fx; l.drow[3 * cc + 1] = fy; l.drow[3 * cc + 2] = fz; }
         KS_SYNC();
         if (lane < nb) {
           Sp w = {{0.f, 0.f, 0.f}, {0.f, 0.f, 0.f}};
@@ -1206,12 +1210,14 @@ extern "C" int ks_model_create(const KsModelDesc* d, KsModel** out) {
     return fail(KS_ELIMIT, "ks_model_create: sizes nb=%d nq=%d nv=%d nu=%d ns=%d exceed %d/%d/%d/%d/%d", d->nb, d->nq,
                 d->nv, d->nu, d->ns, kMaxB, kMaxQ, kMaxV, kMaxU, kMaxS);
   if (d->nv > 64 || 4 * d->ns > 64) return fail(KS_ELIMIT, "ks_model_create: more than 64 dofs or constraint rows");
+  if (d->condim != 0 && d->condim != 1 && d->condim != 3) return fail(KS_EINVAL, "ks_model_create: condim %d (1 or 3)", d->condim);
   if (!(d->dt > 0.0)) return fail(KS_EINVAL, "ks_model_create: dt must be positive");
   KsModel* km = new KsModel();
   DevModel& m = km->host;
   std::memset(&m, 0, sizeof(m));
   m.nb = d->nb; m.nq = d->nq; m.nv = d->nv; m.nu = d->nu; m.ns = d->ns;
   m.iterations = d->iterations; m.ls_iterations = d->ls_iterations; m.eulerdamp = d->eulerdamp;
+  m.frictionless = d->condim == 1 ? 1 : 0;
   m.nvs = m_stride(d->nv);
   m.js = j_stride(d->nv);
   m.dt = (float)d->dt;

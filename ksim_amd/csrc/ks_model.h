@@ -22,7 +22,8 @@ struct DevModel {
   int nb, nq, nv, nu, ns, iterations, ls_iterations, eulerdamp, npairs, nvs /* row stride of the mass matrix in LDS, a multiple of 4 */, max_depth,
       js /* row stride of the constraint Jacobian in LDS, a multiple of 4 */,
       dofrows /* 1 when a joint is limited or has dry friction */, nfriction /* dofs with dry friction */,
-      invw_ok /* 1 when every hinge dof has a positive inverse weight (what rows on the dof lanes are regularised with) */;
+      invw_ok /* 1 when every hinge dof has a positive inverse weight (what rows on the dof lanes are regularised with) */,
+      frictionless /* 1: condim 1, one normal row per contact instead of the four pyramid edges */;
   float dt, gravity[3], tolerance, ls_tolerance, meaninertia, friction, impratio;
   // contact impedance constants, already clamped the way the constraint builder wants them
   float con_k, con_b, dmin, dmax, width, mid, power;

@@ -176,6 +176,12 @@ def load_mjcf(path: str, **options) -> KinematicModel:
     limit_params = []
     world = root.find("worldbody")
     planes = {g.get("name") for g in world if g.tag == "geom" and defaults.resolve(g, None).get("type", "sphere") == "plane"}
+    # condim of a geom-floor contact: an explicit pair's own, otherwise the larger of the two geoms' (MuJoCo's rule); every
+    # contact of the model must agree, on 1 (frictionless, what examples/data/scene.mjcf uses) or 3 (friction pyramid)
+    plane_condim = {g.get("name"): int(defaults.resolve(g, None).get("condim", 3)) for g in world
+                    if g.tag == "geom" and defaults.resolve(g, None).get("type", "sphere") == "plane"}
+    floor_condim = max(plane_condim.values()) if plane_condim else 3
+    condims: list[int] = []
     pairs: dict[str, dict] = {}  # geom name -> attributes of its explicit contact pair with the floor
     con = root.find("contact")
     for pr in ([] if con is None else con):
@@ -185,8 +191,8 @@ def load_mjcf(path: str, **options) -> KinematicModel:
         g1, g2 = at.get("geom1"), at.get("geom2")
         if (g1 in planes) == (g2 in planes):
             raise ValueError(f"contact pair {g1!r} / {g2!r}: only pairs of a robot geom with the floor plane are in the model subset")
-        if int(at.get("condim", 3)) != 3:
-            raise ValueError(f"contact pair {g1!r} / {g2!r}: condim {at.get('condim')} is outside the model subset (3 only)")
+        if int(at.get("condim", 3)) not in (1, 3):
+            raise ValueError(f"contact pair {g1!r} / {g2!r}: condim {at.get('condim')} is outside the model subset (1 or 3)")
         pairs[g2 if g1 in planes else g1] = at
 
     def read_body(elem, childclass):
@@ -249,8 +255,10 @@ def load_mjcf(path: str, **options) -> KinematicModel:
             kind = g.get("type", "sphere")
             if kind == "plane":
                 continue
-            if pair is None and int(g.get("condim", 3)) != 3:
-                raise ValueError(f"geom {g.get('name')!r}: condim {g.get('condim')} is outside the model subset (3 only)")
+            cd = int(pair.get("condim", 3)) if pair is not None else max(int(g.get("condim", 3)), floor_condim)
+            if cd not in (1, 3):
+                raise ValueError(f"geom {g.get('name')!r}: condim {cd} is outside the model subset (1 or 3)")
+            condims.append(cd)
             size, gp = _vec(g.get("size")), geom_frame(g, kind)[0]
             if kind == "sphere":
                 b.spheres.append((gp, float(size[0]), g.get("name", "")))
@@ -316,6 +324,10 @@ def load_mjcf(path: str, **options) -> KinematicModel:
             V[:, 2] = -V[:, 2]
         return m, com, w, mat_to_quat(V)
 
+    if condims:
+        if len(set(condims)) != 1:
+            raise ValueError("the contacts of the model must share one condim (all frictionless or all with friction)")
+        options.setdefault("condim", condims[0])
     if contact_params:
         if len(set(contact_params)) != 1:
             raise ValueError("the collision geoms must share friction, solref and solimp")

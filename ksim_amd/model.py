@@ -95,6 +95,7 @@ class KinematicModel:
     ls_tolerance: float
     impratio: float
     eulerdamp: bool
+    condim: int  # 3: friction pyramid; 1: frictionless contacts (MuJoCo condim of every sphere-floor pair)
     solref: np.ndarray
     solimp: np.ndarray
     friction: float
@@ -167,18 +168,21 @@ class ModelBuilder:
 
     def __init__(self, dt=0.005, gravity=(0.0, 0.0, -9.81), iterations=8, ls_iterations=8, tolerance=1e-10,
                  ls_tolerance=0.01, impratio=1.0, eulerdamp=False, solref=(0.02, 1.0),
-                 solimp=(0.9, 0.95, 0.001, 0.5, 2.0), friction=1.0, integrator=None, dof_solref=None, dof_solimp=None):
+                 solimp=(0.9, 0.95, 0.001, 0.5, 2.0), friction=1.0, integrator=None, dof_solref=None, dof_solimp=None,
+                 condim=3):
         # integrator: "euler" (explicit joint damping unless `eulerdamp`) or "implicitfast", the one ksim sets
         # (ksim/task/rl.py:555-578).  With torque motors the only velocity-dependent smooth force is joint damping, so
         # implicitfast is the damping-implicit velocity update, (M + dt diag(damping)) a = M qacc.
         if integrator not in (None, "euler", "implicitfast"):
             raise ValueError(f"unknown integrator {integrator!r}")
         eulerdamp = bool(eulerdamp) or integrator == "implicitfast"
+        if int(condim) not in (1, 3):
+            raise ValueError(f"condim {condim}: contacts are frictionless (1) or pyramidal (3)")
         self.opt = dict(dt=float(dt), gravity=np.array(gravity, dtype=np.float64), iterations=int(iterations),
                         ls_iterations=int(ls_iterations), tolerance=float(tolerance),
                         ls_tolerance=float(ls_tolerance), impratio=float(impratio), eulerdamp=bool(eulerdamp),
                         solref=np.array(solref, dtype=np.float64), solimp=np.array(solimp, dtype=np.float64),
-                        friction=float(friction),
+                        friction=float(friction), condim=int(condim),
                         dof_solref=np.array(solref if dof_solref is None else dof_solref, dtype=np.float64),
                         dof_solimp=np.array(solimp if dof_solimp is None else dof_solimp, dtype=np.float64))
         self.bodies = [dict(parent=-1, jtype=JNT_NONE, pos=np.zeros(3), quat=np.array([1.0, 0, 0, 0]), mass=0.0,

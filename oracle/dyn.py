@@ -28,7 +28,7 @@ def build(force: bool = False) -> str:
 class KsorModel(ctypes.Structure):
     _fields_ = [
         ("nb", c_int), ("nq", c_int), ("nv", c_int), ("nu", c_int), ("ns", c_int),
-        ("iterations", c_int), ("ls_iterations", c_int), ("eulerdamp", c_int),
+        ("iterations", c_int), ("ls_iterations", c_int), ("eulerdamp", c_int), ("condim", c_int),
         ("dt", c_double), ("gravity", c_double * 3), ("tolerance", c_double), ("ls_tolerance", c_double),
         ("impratio", c_double), ("meaninertia", c_double), ("solref", c_double * 2), ("solimp", c_double * 5),
         ("body_parent", c_int * MAXB), ("body_jtype", c_int * MAXB), ("body_qadr", c_int * MAXB),
@@ -86,6 +86,7 @@ def make_model(a: dict) -> KsorModel:
     for k in ("nb", "nq", "nv", "nu", "ns", "iterations", "ls_iterations"):
         setattr(m, k, int(a[k]))
     m.eulerdamp = int(bool(a["eulerdamp"]))
+    m.condim = int(a.get("condim", 3))
     for k in ("dt", "tolerance", "ls_tolerance", "impratio", "meaninertia"):
         setattr(m, k, float(a[k]))
 

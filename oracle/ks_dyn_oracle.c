@@ -413,9 +413,24 @@ void FN(ksor_make_constraint)(const KsorModel* m, Data* d) {
     const REAL* Jy = jacp + 1 * nv;
     const REAL* Jx = jacp;
     const REAL t = (REAL)m->body_invweight0[b];
-    const REAL invweight = (t + mu * mu * t) * 2 * mu * mu / (REAL)m->impratio;
     const REAL pos = dist;
     const REAL imp = impedance(pos, dmin, dmax, width, mid, power);
+    if (m->condim == 1) {
+      /* frictionless contact (MJX _instantiate_contact_frictionless): the normal row alone, regularised with the
+       * body's translational inverse weight */
+      REAL R = t * (1 - imp) / imp;
+      if (R < MINVAL) R = MINVAL;
+      REAL* row = d->efc_J + nefc * nv;
+      REAL vel = 0;
+      for (int j = 0; j < nv; ++j) { row[j] = Jn[j]; vel += row[j] * d->qvel[j]; }
+      d->efc_pos[nefc] = pos;
+      d->efc_aref[nefc] = -bb * vel - kk * imp * pos;
+      d->efc_D[nefc] = 1 / R;
+      d->efc_floss[nefc] = 0;
+      nefc += 1;
+      continue;
+    }
+    const REAL invweight = (t + mu * mu * t) * 2 * mu * mu / (REAL)m->impratio;
     REAL R = invweight * (1 - imp) / imp;
     if (R < MINVAL) R = MINVAL;
     for (int q = 0; q < 4; ++q) {
@@ -729,12 +744,17 @@ void FN(ksor_forward)(const KsorModel* m, Data* d) {
   for (int s = 0; s < m->ns; ++s) {
     if (!(d->con_dist[s] < 0)) continue;
     REAL F[3] = {0, 0, 0};
-    for (int q = 0; q < 4; ++q) {
-      const REAL f = d->efc_force[row + q], smu = (q & 1) ? -d->friction : d->friction;
-      F[2] += f;
-      if (q < 2) F[1] += smu * f; else F[0] -= smu * f;
+    if (m->condim == 1) {
+      F[2] = d->efc_force[row];
+      row += 1;
+    } else {
+      for (int q = 0; q < 4; ++q) {
+        const REAL f = d->efc_force[row + q], smu = (q & 1) ? -d->friction : d->friction;
+        F[2] += f;
+        if (q < 2) F[1] += smu * f; else F[0] -= smu * f;
+      }
+      row += 4;
     }
-    row += 4;
     REAL off[3], tq[3];
     for (int k = 0; k < 3; ++k) off[k] = d->con_pos[s][k] - d->com[k];
     cross3(tq, off, F);

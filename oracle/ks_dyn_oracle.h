@@ -28,6 +28,7 @@ enum { KSOR_JNT_NONE = 0, KSOR_JNT_FREE = 1, KSOR_JNT_HINGE = 2 };
 typedef struct KsorModel {
   int nb, nq, nv, nu, ns;
   int iterations, ls_iterations, eulerdamp;
+  int condim; /* 3 (or 0): pyramidal friction, four rows per contact; 1: frictionless, one normal row */
   double dt, gravity[3], tolerance, ls_tolerance, impratio, meaninertia;
   double solref[2], solimp[5];
   int body_parent[KSOR_MAXB], body_jtype[KSOR_MAXB], body_qadr[KSOR_MAXB], body_dofadr[KSOR_MAXB];

@@ -28,6 +28,9 @@ MODELS = {"chain": km.pendulum_chain_model, "humanoid": km.humanoid_model, "kbot
           "chain-springs": lambda: km.pendulum_chain_model(integrator="implicitfast", damping=0.2, stiffness=6.0),
           "humanoid-limits": lambda: km.humanoid_model(joint_range=(-0.45, 0.5)),
           "kbot-limits": lambda: km.kbot_scale_model(integrator="implicitfast", joint_range=(-0.45, 0.5), frictionloss=0.2),
+          # frictionless contacts (condim 1, what the reference's examples/data/scene.mjcf uses): one normal row per contact
+          "kbot-frictionless": lambda: km.kbot_scale_model(integrator="implicitfast", condim=1),
+          "humanoid-frictionless-limits": lambda: km.humanoid_model(joint_range=(-0.45, 0.5), condim=1),
           # the real K-Bot's contact parameters (robot.mjcf:24): five times stiffer rows than MuJoCo's defaults
           "kbot-stiff-feet": lambda: km.kbot_scale_model(integrator="implicitfast", joint_range=(-0.45, 0.5), frictionloss=0.2,
                                                          solref=(0.02, 0.8), solimp=(0.98, 0.99, 0.1, 0.5, 2.0),

@@ -419,3 +419,28 @@ def test_model_create_rejects_joint_addresses_outside_the_state():
                        ("body_qadr", 1, m.nq - 6)):    # and seven coordinates
         rc, msg = create(set_field(name, b, v))
         assert rc == -1 and f"body {b}" in msg and "outside" in msg, (name, b, v, rc, msg)
+
+
+def test_mjcf_contact_dimension_follows_mujocos_rule(tmp_path):
+    """condim of a geom-floor contact is the larger of the two geoms' (an explicit pair carries its own); the model takes
+    the one value all contacts share: 1 = frictionless as in the reference's examples/data/scene.mjcf, 3 = friction pyramid."""
+    from ksim_amd.mjcf import load_mjcf
+
+    def robot(floor, foot, pair=""):
+        return f"""<mujoco><worldbody>
+          <geom name="floor" type="plane" size="0 0 .05" condim="{floor}"/>
+          <body name="base" pos="0 0 0.5"><freejoint/>
+            <geom name="torso" type="sphere" size="0.1" mass="1" contype="0" conaffinity="0"/>
+            <geom name="foot" type="sphere" size="0.05" pos="0 0 -0.2" mass="0.2" condim="{foot}"/>
+          </body></worldbody>{pair}</mujoco>"""
+
+    for floor, foot, pair, want in ((1, 1, "", 1), (1, 3, "", 3), (3, 1, "", 3), (3, 3, "", 3),
+                                    (3, 3, '<contact><pair geom1="foot" geom2="floor" condim="1"/></contact>', 1)):
+        path = tmp_path / f"r{floor}{foot}{len(pair)}.xml"
+        path.write_text(robot(floor, foot, pair))
+        m = load_mjcf(str(path))
+        assert m.condim == want and m.ns == 1, (floor, foot, pair)
+    path = tmp_path / "bad.xml"
+    path.write_text(robot(4, 1))
+    with pytest.raises(ValueError, match="condim"):
+        load_mjcf(str(path))

@@ -696,6 +696,31 @@ def test_contact_relaxes_like_the_documented_oscillator_until_it_would_have_to_p
         np.testing.assert_allclose(np.diff(rs[release:]) / dt, v_release, rtol=1e-9)  # coasting afterwards
 
 
+@pytest.mark.parametrize("mu", [0.3, 1.0])
+def test_frictionless_contact_is_one_normal_row_with_the_same_spring_damper(mu):
+    """condim 1: a single row along the normal whose inverse inertia 1 / m is exact for a ball, so the documented identity
+    a1 = (1 - d) a0 - d (b v + k r) holds for any friction coefficient (which plays no part), and sideways motion and spin
+    feel nothing."""
+    dimp, b, k_over_d = 0.9, 2 / 0.018, 1 / (0.81 * 4e-4)
+    for r, v in ((-0.01, -0.05), (-0.004, 0.02)):
+        m = _ball(radius=0.1, mass=2.0, z=0.1 + r, iterations=100, ls_iterations=50, solref=(0.02, 1.0),
+                  solimp=(dimp, dimp, 0.001, 0.5, 2.0), friction=mu, condim=1)
+        orc = Oracle(m.arrays())
+        d = orc.data(qvel=np.array([0.7, -0.3, v, 0.5, 0.2, -0.1]))
+        orc.forward(d)
+        assert d.nefc == 1 and d.efc_force[0] > 0
+        np.testing.assert_allclose(d.efc_J[0], [0, 0, 1, 0, 0, 0], atol=1e-12)
+        want = (1 - dimp) * (-9.81) - dimp * (b * v + k_over_d * dimp * r)
+        assert d.qacc[2] == pytest.approx(want, rel=1e-9)
+        assert np.abs(np.delete(np.array(d.qacc), 2)).max() < 1e-9
+        np.testing.assert_allclose(np.array(d.cfrc_ext)[1], [0, 0, 0, 0, 0, d.efc_force[0]], atol=1e-9)
+    # the pyramid at the same state does brake the sideways motion
+    m3 = _ball(radius=0.1, mass=2.0, z=0.09, friction=1.0, iterations=100, ls_iterations=50)
+    d3 = Oracle(m3.arrays()).data(qvel=np.array([0.7, 0, 0, 0, 0, 0.0]))
+    Oracle(m3.arrays()).forward(d3)
+    assert d3.nefc == 4 and d3.qacc[0] < -0.5
+
+
 @pytest.mark.parametrize("mu", [0.3, 1.0, 2.0])
 def test_resting_pyramid_carries_the_weight_for_any_friction(mu):
     m = _ball(z=0.1, friction=mu)
