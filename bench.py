@@ -211,8 +211,8 @@ def main() -> None:
     tpath = os.path.join(ROOT, "profiles", "step_kernel_cfg4_hbm_traffic.txt")
     if os.path.exists(tpath):  # measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, see that file
         for ln in open(tpath):
-            if ln.startswith("hbm_bytes_per_launch="):
-                traffic = float(ln.split("=", 1)[1])
+            if ln.startswith("hbm_bytes_per_env_step="):  # counted on launches of 8192 envs; scaled to this run's launch size
+                traffic = float(ln.split("=", 1)[1]) * envs_per_launch
     valu = {}
     vpath = os.path.join(ROOT, "profiles", "step_kernel_cfg4_instruction_mix.txt")
     if os.path.exists(vpath):  # rocprofv3 --pmc SQ_* summary, see that file
@@ -252,12 +252,14 @@ def main() -> None:
         flops = base.pop("flops_per_env_step")
         line["cpu_baseline"] = base
         rate = flops * envs_per_launch / (kernel_ms * 1e-3) / 1e12
+        whole = flops * N / (elapsed / args.steps) / 1e12  # all groups together, per wall-clock control step
         line["roofline"]["fp32_valu"] = {
             "achieved": rate, "peak": FP32_VALU_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": rate / FP32_VALU_PEAK_TFLOPS,
-            "flops_per_env_step": flops,
+            "flops_per_env_step": flops, "achieved_all_groups": whole, "frac_all_groups": whole / FP32_VALU_PEAK_TFLOPS,
             "what": "floating-point operations of one env's control step as the float64 oracle performs them (counted by "
                     "a build of its C source with a counting scalar type, 32 standing envs) x envs per launch / the "
-                    "step kernel's measured duration"}
+                    "step kernel's measured duration; with several groups in flight a launch shares the chip with the "
+                    "other group's, so 'all_groups' divides the flops of all envs by the wall-clock time of a control step"}
     print(json.dumps(line))
 
 

@@ -117,7 +117,11 @@ __global__ __launch_bounds__(256) void gae_tn_kernel(
   __shared__ float sv[kTnSteps][kTnEnvs], sr[kTnSteps][kTnEnvs], oa[kTnSteps][kTnEnvs], orr[kTnSteps][kTnEnvs];
   __shared__ uint8_t sd[kTnSteps][kTnEnvs], ss[kTnSteps][kTnEnvs];
   const int tx = threadIdx.x & (kTnEnvs - 1), ty = threadIdx.x / kTnEnvs;
-  const int64_t e = (int64_t)blockIdx.x * kTnEnvs + tx;
+  // Workgroups are dealt round-robin to the 8 XCDs, each with its own L2.  Four neighbouring tiles share every 128-byte
+  // line of the byte arrays, so neighbouring tiles go to one XCD: workgroup b takes tile (b % 8) * (grid / 8) + b / 8.
+  int64_t tile = blockIdx.x;
+  if (gridDim.x % 8 == 0) tile = (int64_t)(blockIdx.x % 8) * (gridDim.x / 8) + blockIdx.x / 8;
+  const int64_t e = tile * kTnEnvs + tx;
   const bool in = e < N;
   const float gl = gamma * lam, omg = 1.0f - gamma;
   float R = 0.f, A = 0.f, v_up = 0.f;

@@ -756,3 +756,31 @@ def test_joint_limit_acceleration_is_the_documented_spring_damper(dof_solref, b,
         r, v, a0 = 0.4 - q, -qd, -float(f.qacc[0])
         a1 = (1 - dimp) * a0 - dimp * (b * v + k_over_d * dimp * r)
         assert -float(d.qacc[0]) == pytest.approx(a1, rel=1e-9), (dof_solref, q, qd)
+
+
+def test_flop_counting_build_matches_the_float64_oracle():
+    """The counting build (oracle/flop_count.cpp) computes in double with the same source: same bits as the float64 oracle,
+    a count that is reproducible, additive over steps, and larger for a state with contacts than for one in the air."""
+    m = km.kbot_scale_model()
+    rng = np.random.default_rng(8)
+    qpos, qvel = _random_state(m, rng, vel_scale=0.3)
+    ground = _sink_to_contact(m, qpos)
+    o64, ocnt = Oracle(m.arrays(), np.float64), Oracle(m.arrays(), np.float64, count_flops=True)
+    counts = {}
+    for name, q in (("air", qpos + np.concatenate([[0, 0, 1.0], np.zeros(m.nq - 3)])), ("ground", ground)):
+        a, b = o64.data(q, qvel), ocnt.data(q, qvel)
+        ocnt.flops_reset()
+        for _ in range(3):
+            o64.step(a); ocnt.step(b)
+        three = ocnt.flops()
+        assert np.array_equal(np.array(a.qpos), np.array(b.qpos)) and np.array_equal(np.array(a.qacc), np.array(b.qacc))
+        c = ocnt.data(q, qvel)
+        ocnt.flops_reset()
+        ocnt.step(c)
+        one = ocnt.flops()
+        ocnt.step(c); ocnt.step(c)
+        assert ocnt.flops() == three and 0 < one < three
+        counts[name] = three
+    assert counts["ground"] > 1.2 * counts["air"] and counts["air"] > 5e4
+    with pytest.raises(ValueError):
+        Oracle(m.arrays(), np.float32, count_flops=True)
