@@ -1,4 +1,6 @@
 """End-to-end rollout (obs -> MLP -> action -> fused physics -> termination -> reset -> record) vs the oracle."""
+import os
+
 import numpy as np
 import pytest
 import torch
@@ -601,3 +603,108 @@ def test_split_rollout_equals_single_stream_rollout():
                                rtol=2e-6, atol=2e-6)
     with pytest.raises(Exception, match="multiple"):
         SplitRollout(c, 63, T, splits=2)
+
+
+def test_split_rollout_replayed_from_per_group_graphs_equals_its_eager_run():
+    """`SplitRollout.unroll(graph=True)`: one HIP graph per group, replayed side by side on the groups' streams, gives the eager
+    split rollout's bits on every replay (Philox draws, resets on the way)."""
+    from ksim_amd.rollout import SplitRollout
+
+    N, T, G = 64, 5, 2
+    outs = []
+    for graph in (False, True):
+        m, c, rnd_, _, _, EnvState = build(N, T, seed=6, min_height=0.9, sim2real=True)
+        n = N // G
+        envs = []
+        for g in range(G):
+            rows = {k: v[g * n:(g + 1) * n].contiguous() for k, v in rnd_.items()}
+            ps = c.engine.reset(c.physics_model, 1.0, 3 + g, n, rows)
+            ps.data.qpos[::3, 2] = 0.87
+            envs.append(EnvState(ps, rows, torch.zeros(n, 2, device=DEV), None, seed=11 + g))
+        sro = SplitRollout(c, N, T, splits=G)
+        run = []
+        for k in range(4):
+            res = sro.unroll(envs, graph=graph)
+            torch.cuda.synchronize()
+            run.append([x.clone() for traj, rew in res for x in (traj.qpos, traj.action, traj.done, rew.total)])
+        assert sum(int(r[2].sum()) + int(r[6].sum()) for r in run) > 0, "no env was reset"
+        outs.append(run)
+    for a, b in zip(*outs):
+        for x, y in zip(a, b):
+            assert torch.equal(x, y)
+
+
+def test_motion_resets_symmetry_rewards_and_imu_misalignment_in_the_rollout():
+    """The pieces an AMP / sim-to-real task adds, together in one rollout on a model read from MJCF: episodes that start from
+    a frame of a reference motion with a random pitch / roll and heading, a misaligned IMU site per env read by the gyro,
+    the accelerometer and the site-orientation observation, contact flags over a geom list, symmetry rewards with their
+    rollout-mean carry.  Checked: reset envs restart on a motion frame at time frame * dt, and the HIP-graph replay gives the eager
+    rollout's bits."""
+    from ksim_amd import actuators, engine, observation as ob, physics, randomization as rnd, resets as rs
+    from ksim_amd import rewards as rw, terminations as tm
+    from ksim_amd.env_terms import EnvTerms
+    from ksim_amd.mjcf import load_mjcf
+    from ksim_amd.mlp import MLP
+    from ksim_amd.priors import MotionReferenceData
+    from ksim_amd.rollout import Rollout, RolloutConstants, RolloutEnvState
+
+    m = load_mjcf(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "mini_biped.mjcf"), integrator="implicitfast")
+    N, T, F = 64, 10, 9
+    rng = np.random.default_rng(41)
+    mq = np.tile(m.qpos0, (F, 1))
+    mq[:, 7:] += rng.uniform(-0.2, 0.2, (F, m.nq - 7))
+    motion = MotionReferenceData(qpos=mq, qvel=np.zeros((F, m.nv)), cartesian_poses={}, ctrl_dt=0.02)
+    resets = [rs.InitialMotionStateReset(reference_motion=motion), rs.RandomPitchRollReset(pitch_range=(-0.2, 0.2), roll_range=(-0.1, 0.1)),
+              rs.RandomHeadingReset()]
+    act = actuators.PositionActuators(kps=(40.0,) * m.nu, kds=(1.0,) * m.nu, ctrl_clip=(30.0,) * m.nu)
+    eng = engine.get_physics_engine("hip", resets, {}, act, engine.EngineConfig(dt=m.dt, ctrl_dt=0.02))
+    observations = {"jp": ob.JointPositionObservation(noise=0.01), "jv": ob.JointVelocityObservation(),
+                    "gyro": ob.SensorObservation(sensor_name="imu_gyro", site_pose_per_env=True, noise=0.01),
+                    "acc": ob.SensorObservation(sensor_name="imu_acc", site_pose_per_env=True),
+                    "imu_rot": ob.SiteOrientationObservation(site_names=("imu_site",), site_pose_per_env=True),
+                    "contact": ob.ContactObservation(geom_idxs=tuple(range(m.ns)) + (ob.FLOOR_GEOM,)),
+                    "a": ob.LastActionObservation()}
+    z0 = float(m.qpos0[2])
+    terms = EnvTerms(m, observations, {"h": tm.MinimumHeightTermination(z0 - 0.008)}, resets)
+    nj = m.nq - 7
+    rewards = {"alive": rw.StayAliveReward(scale=1.0),
+               "sym": rw.SymmetryReward(scale=0.5, joint_indices=tuple(range(nj)), joint_targets=(0.0,) * nj, alpha=0.3),
+               "pair": rw.PairwiseSymmetryReward(scale=0.2, left_joint_index=0, right_joint_index=nj // 2, flipped=True)}
+    dims = (terms.obs_dim, 32, m.nu)
+    ws = [rng.normal(scale=0.3 / np.sqrt(i), size=(o, i)).astype(np.float32) for i, o in zip(dims[:-1], dims[1:])]
+    cws = [rng.normal(scale=1 / np.sqrt(terms.obs_dim), size=(1, terms.obs_dim)).astype(np.float32)]
+    consts = RolloutConstants(physics_model=physics.DeviceModel(m), engine=eng, terms=terms, rewards=rewards,
+                              actor=MLP(ws, [np.zeros(o, np.float32) for o in dims[1:]], dtype="f32"),
+                              critic=MLP(cws, [np.zeros(1, np.float32)], dtype="f32"), log_std=t32(np.full(m.nu, -1.0)))
+
+    # eager, then the graph replay from an identical start
+    runs = []
+    for graph in (False, True):
+        gen = torch.Generator(device=DEV); gen.manual_seed(100)
+        rnd_ = rnd.get_physics_randomizers(m, {"imu": rnd.IMUAlignmentRandomizer(site_name="imu_site", tilt_std_rad=0.05, yaw_std_rad=0.05,
+                                                                                   translate_std_m=0.01),
+                                               "f": rnd.FloorFrictionRandomizer(0.5, 1.0)}, N, gen)
+        ps = eng.reset(consts.physics_model, 1.0, 7, N, rnd_)
+        env = RolloutEnvState(ps, rnd_, torch.zeros(N, 0, device=DEV), None, seed=5)
+        ro = Rollout(consts, N, T)
+        outs = []
+        for k in range(3):
+            traj, rew = ro.unroll(env, graph=graph)
+            outs.append((traj.qpos.clone(), traj.obs["obs"].clone() if isinstance(traj.obs, dict) and "obs" in traj.obs else ro.obs.clone(),
+                         traj.done.clone(), rew.total.clone(), env.reward_carry.clone(), traj.timestep.clone()))
+        runs.append(outs)
+    for a, b in zip(runs[0], runs[1]):
+        for x, y in zip(a, b):
+            assert torch.equal(x, y)
+    qpos, obs, done, total, carry, tstep = runs[0][-1]
+    assert torch.isfinite(total).all() and torch.isfinite(obs).all()
+    alld = torch.cat([r[2] for r in runs[0]])
+    assert int(alld.sum()) > 10, "no episode ended: the motion reset was not exercised"
+    # an env that is reset at step t shows, at step t + 1, a state that started one control step earlier on a motion frame:
+    # its recorded time is frame * dt + 0.02 for some frame, and the carry of the symmetry reward is not stuck at its start
+    tt = torch.cat([r[5] for r in runs[0]]).cpu().numpy()
+    dd = alld.cpu().numpy().astype(bool)
+    after = tt[1:][dd[:-1]]
+    frames = (after - 0.02) / 0.02
+    assert np.abs(frames - np.round(frames)).max() < 1e-4 and frames.min() > -1e-4 and frames.max() < F - 1 + 1e-4
+    assert float(carry.abs().max()) > 1e-3
