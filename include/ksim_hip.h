@@ -306,7 +306,9 @@ typedef struct KsStepIO {
      env.  `work` returns an estimate of each env's cost in this step; ks_work_order turns it into a heaviest-first
      permutation that the next step takes as `env_order`, so the heavy envs start first and the light ones fill the gaps.
      Results do not depend on the order. */
-  const int32_t* env_order;    /* (N) a permutation of 0..N-1: workgroup i steps env env_order[i]; nullable = identity */
+  const int32_t* env_order;    /* (N) a permutation of 0..N-1: workgroup i steps env env_order[i]; nullable = the natural order
+                                  dealt to the XCDs in contiguous eighths (workgroup i steps env (i % 8) (N / 8) + i / 8 when
+                                  N is a multiple of 8) */
   int32_t* work;               /* (N) nullable */
   /* events (ks_step only) */
   int32_t n_events;
@@ -318,7 +320,10 @@ typedef struct KsStepIO {
 } KsStepIO;
 
 int ks_step(const KsModel* model, ks_stream_t stream, const KsStepIO* io /*host*/);
-/* order = the envs sorted by work, heaviest first (a counting sort in one workgroup; ties in arbitrary order). */
+/* order = the envs sorted by work, heaviest first (counting sort; ties in arbitrary order).  When N is a multiple of 8 (and at
+ * least 512) the sort runs inside the eight regions [r N / 8, (r + 1) N / 8) and region r's envs go to order[r], order[r + 8],
+ * ...: workgroup b of the step launch runs on XCD b % 8, so every XCD then steps one contiguous eighth of the env arrays,
+ * heaviest first, and the 128-byte lines that neighbouring envs' rows share stay in one L2. */
 int ks_work_order(ks_stream_t stream, int64_t N, const int32_t* work, int32_t* order);
 int ks_forward(const KsModel* model, ks_stream_t stream, const KsStepIO* io /*host*/);
 

@@ -317,7 +317,11 @@ void step_kernel(StepArgs a) {
   extern __shared__ __attribute__((aligned(16))) float lds_raw[];
   const DevModel& m = *a.model;
   const int lane = threadIdx.x;
-  const int64_t env = a.env_order ? a.env_order[blockIdx.x] : blockIdx.x;  // heaviest envs first when an order is given
+  // heaviest envs first when an order is given (ks_work_order, which also keeps neighbouring envs on one XCD); without
+  // one, workgroup b takes env (b % 8) (N / 8) + b / 8 for the same reason
+  int64_t env = blockIdx.x;
+  if (a.env_order) env = a.env_order[blockIdx.x];
+  else if (a.N % 8 == 0) env = (int64_t)(blockIdx.x % 8) * (a.N / 8) + blockIdx.x / 8;
   if (a.env_mask && !a.env_mask[env]) return;  // wave-uniform
   int work = 0;  // wave-uniform cost estimate of this control step
   const int nb = m.nb, nq = m.nq, nv = m.nv, nu = m.nu, ns = m.ns, nvs = m.nvs, js = m.js;
@@ -1489,14 +1493,21 @@ extern "C" int ks_forward(const KsModel* model, ks_stream_t stream, const KsStep
 
 namespace ks {
 constexpr int kWorkBuckets = 2048;
-// Counting sort of the envs by descending work in one workgroup: histogram, suffix sums, scatter.
+constexpr int kXcds = 8;  // workgroup b of a launch runs on XCD b % 8, each XCD with an L2 of its own
+// Counting sort of envs by descending work in one workgroup: histogram, suffix sums, scatter.
+// With gridDim.x == 8 (N a multiple of 8) workgroup r sorts the envs of region r = [r N / 8, (r + 1) N / 8) and writes them
+// to order[r], order[r + 8], ...: the step kernel's workgroup b = r + 8 k then runs on XCD r and finds there only envs of
+// region r.  The state rows of neighbouring envs share 128-byte lines (an env's qpos row is 108 bytes); kept inside one XCD
+// such a line is fetched into, and written back from, one L2 instead of two.
 __global__ __launch_bounds__(1024) void work_order_kernel(int64_t N, const int32_t* __restrict__ work, int32_t* __restrict__ order) {
   __shared__ int hist[kWorkBuckets];
   __shared__ int scan[kWorkBuckets];
   const int t = threadIdx.x;
+  const int regions = gridDim.x, region = blockIdx.x;
+  const int64_t n = N / regions, first = region * n;
   for (int b = t; b < kWorkBuckets; b += 1024) hist[b] = 0;
   __syncthreads();
-  for (int64_t i = t; i < N; i += 1024) atomicAdd(&hist[min(max(work[i], 0), kWorkBuckets - 1)], 1);
+  for (int64_t i = t; i < n; i += 1024) atomicAdd(&hist[min(max(work[first + i], 0), kWorkBuckets - 1)], 1);
   __syncthreads();
   // inclusive suffix sums (heaviest bucket first) by doubling
   for (int b = t; b < kWorkBuckets; b += 1024) scan[b] = hist[b];
@@ -1514,9 +1525,9 @@ __global__ __launch_bounds__(1024) void work_order_kernel(int64_t N, const int32
   // bucket b starts after all heavier buckets: scan[b] - hist[b]
   for (int b = t; b < kWorkBuckets; b += 1024) hist[b] = scan[b] - hist[b];
   __syncthreads();
-  for (int64_t i = t; i < N; i += 1024) {
-    const int pos = atomicAdd(&hist[min(max(work[i], 0), kWorkBuckets - 1)], 1);
-    order[pos] = (int32_t)i;
+  for (int64_t i = t; i < n; i += 1024) {
+    const int pos = atomicAdd(&hist[min(max(work[first + i], 0), kWorkBuckets - 1)], 1);
+    order[(int64_t)pos * regions + region] = (int32_t)(first + i);
   }
 }
 }  // namespace ks
@@ -1526,6 +1537,7 @@ extern "C" int ks_work_order(ks_stream_t stream, int64_t N, const int32_t* work,
   if (N < 0 || N > 0x7fffffff) return fail(KS_EINVAL, "ks_work_order: bad env count");
   if (N == 0) return KS_OK;
   if (!work || !order) return fail(KS_EINVAL, "ks_work_order: null argument");
-  hipLaunchKernelGGL(work_order_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, N, work, order);
+  const int regions = (N % kXcds == 0 && N >= 64 * kXcds) ? kXcds : 1;
+  hipLaunchKernelGGL(work_order_kernel, dim3(regions), dim3(1024), 0, (hipStream_t)stream, N, work, order);
   return check_launch("ks_work_order");
 }

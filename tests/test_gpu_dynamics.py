@@ -485,6 +485,16 @@ def test_launch_order_does_not_change_results_and_sorts_heaviest_first():
         assert torch.equal(a[k], b[k]), k
     rev = torch.from_numpy(np.ascontiguousarray(o[::-1])).to(DEV)
     assert torch.equal(run(rev)["qpos"], a["qpos"])
+    # a multiple of 8 envs: sorted inside the eight contiguous regions, region r at positions r, r + 8, ...
+    N2 = 1024
+    w2 = torch.from_numpy(np.random.default_rng(73).integers(64, 900, N2).astype(np.int32)).to(DEV)
+    o2 = torch.empty(N2, dtype=torch.int32, device=DEV)
+    physics.work_order(dm, w2, o2)
+    o2, w2 = o2.cpu().numpy(), w2.cpu().numpy()
+    assert sorted(o2.tolist()) == list(range(N2))
+    for r in range(8):
+        mine = o2[r::8]
+        assert mine.min() >= r * N2 // 8 and mine.max() < (r + 1) * N2 // 8 and (np.diff(w2[mine]) <= 0).all()
 
 
 def test_joint_limit_and_dry_friction_closed_forms():
