@@ -235,6 +235,9 @@ struct FusedArgs {
   const float* x;
   float* y;
   long long* prof;  // phase time stamps of wavefront 0, written only by -DKS_PROFILE builds
+  // training forward: hidden layer l's activations also go to save[l], (M, save_ld[l]) bf16 row-major, for the backward pass
+  __bf16* save[KS_MAX_LAYERS];
+  int save_ld[KS_MAX_LAYERS];
 };
 
 #ifdef KS_PROFILE
@@ -401,6 +404,17 @@ __device__ __forceinline__ void fused_layer(const FusedArgs& a, int l, __bf16* _
   }
   __syncthreads();
   KS_MLP_STAMP2(4 + 3 * l)
+  if (!LAST && a.save[l]) {
+    // the finished tile, 16 bytes per thread and pass, rows as contiguous runs; the next layer only reads the tile until every
+    // wavefront (this copy included, which sits before its matrix work in program order) has passed the next barrier
+    const int w8 = nt * 4;  // 16-byte pieces per row (32 features = 4 pieces)
+    __bf16* dst = a.save[l];
+    const int ld = a.save_ld[l];
+    for (int idx = threadIdx.x; idx < MI * 32 * w8; idx += 64 * kFusedWaves) {
+      const int r = idx / w8, c8 = idx - r * w8;
+      if (m0 + r < a.M) *reinterpret_cast<uint4*>(dst + (m0 + r) * ld + c8 * 8) = *reinterpret_cast<const uint4*>(act + r * lda + c8 * 8);
+    }
+  }
 }
 
 template <int ACT, int BM>
@@ -677,11 +691,27 @@ __global__ __launch_bounds__(256) void colsum_kernel(int64_t M, int ld, const T*
   const int c = blockIdx.x * 64 + (threadIdx.x & 63), g = threadIdx.x >> 6;
   float s = 0.f;
   if (c < ld)
-    for (int64_t m = (int64_t)blockIdx.y * 4 + g; m < M; m += 4 * kColsumSlices) s += to_f32(a[m * ld + c]);
+    for (int64_t m = (int64_t)blockIdx.y * 4 + g; m < M; m += 4 * (int64_t)gridDim.y) s += to_f32(a[m * ld + c]);
   red[g][threadIdx.x & 63] = s;
   __syncthreads();
   if (g == 0 && c < ld)
     part[(int64_t)blockIdx.y * ld + c] = (red[0][threadIdx.x] + red[1][threadIdx.x]) + (red[2][threadIdx.x] + red[3][threadIdx.x]);
+}
+
+// out[c] = sum over z of part[z][c] for the few columns of a bias gradient: a workgroup of 64 threads per column adds its nz
+// partial sums with a fixed tree (one thread walking them one after the other pays nz dependent load latencies)
+__global__ __launch_bounds__(64) void sum_parts_tree_kernel(int64_t n, int nz, const float* __restrict__ part, float* __restrict__ out) {
+  __shared__ float red[64];
+  const int64_t c = blockIdx.x;
+  float s = 0.f;
+  for (int z = threadIdx.x; z < nz; z += 64) s += part[(int64_t)z * n + c];
+  red[threadIdx.x] = s;
+  __syncthreads();
+  for (int w = 32; w > 0; w >>= 1) {
+    if ((int)threadIdx.x < w) red[threadIdx.x] += red[threadIdx.x + w];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) out[c] = red[0];
 }
 
 // out[i] = sum over z of part[z][i], z ascending
@@ -954,8 +984,13 @@ static FusedArgs fused_args(const DevMlp& m, int64_t M, const float* x, float* y
 }
 
 template <int BM>
-static int launch_fused_tile(const DevMlp& m, hipStream_t s, int64_t M, const float* x, float* y) {
+static int launch_fused_tile(const DevMlp& m, hipStream_t s, int64_t M, const float* x, float* y, char* const* save) {
   FusedArgs a = fused_args(m, M, x, y);
+  if (save)
+    for (int l = 0; l + 1 < m.n_layers; ++l) {
+      a.save[l] = (__bf16*)save[l];
+      a.save_ld[l] = m.npad[l];
+    }
 #ifdef KS_PROFILE
   if (const char* e = getenv("KS_MLP_PROF_PTR")) a.prof = (long long*)strtoull(e, nullptr, 16);
 #endif
@@ -983,18 +1018,18 @@ static int launch_fused_tile(const DevMlp& m, hipStream_t s, int64_t M, const fl
 
 // Row tile: 128 rows amortise each weight fragment over four MFMAs; smaller batches take smaller tiles so that
 // the grid still reaches every CU.
-static int launch_fused(const DevMlp& m, hipStream_t s, int64_t M, const float* x, float* y) {
+static int launch_fused(const DevMlp& m, hipStream_t s, int64_t M, const float* x, float* y, char* const* save = nullptr) {
 #ifdef KS_PROFILE
   if (const char* e = getenv("KS_MLP_BM")) {
     const int bm = atoi(e);
-    if (bm == 128) return launch_fused_tile<128>(m, s, M, x, y);
-    if (bm == 64) return launch_fused_tile<64>(m, s, M, x, y);
-    if (bm == 32) return launch_fused_tile<32>(m, s, M, x, y);
+    if (bm == 128) return launch_fused_tile<128>(m, s, M, x, y, save);
+    if (bm == 64) return launch_fused_tile<64>(m, s, M, x, y, save);
+    if (bm == 32) return launch_fused_tile<32>(m, s, M, x, y, save);
   }
 #endif
-  if (M >= 128 * 256) return launch_fused_tile<128>(m, s, M, x, y);
-  if (M >= 64 * 256) return launch_fused_tile<64>(m, s, M, x, y);
-  return launch_fused_tile<32>(m, s, M, x, y);
+  if (M >= 128 * 256) return launch_fused_tile<128>(m, s, M, x, y, save);
+  if (M >= 64 * 256) return launch_fused_tile<64>(m, s, M, x, y, save);
+  return launch_fused_tile<32>(m, s, M, x, y, save);
 }
 
 template <int BM>
@@ -1200,7 +1235,7 @@ static int64_t carve_train(const DevMlp& m, int64_t M, char* base, TrainWs* ws) 
   w.t2 = take((int64_t)wz * Mp * esz);
   int64_t maxw = 0;
   for (int l = 0; l < m.n_layers; ++l) maxw = (int64_t)m.npad[l] * m.kpad[l] > maxw ? (int64_t)m.npad[l] * m.kpad[l] : maxw;
-  const int64_t nparts = kDwSplit * maxw > (int64_t)kColsumSlices * wz ? kDwSplit * maxw : (int64_t)kColsumSlices * wz;
+  const int64_t nparts = kDwSplit * maxw > (int64_t)4 * kColsumSlices * wz ? kDwSplit * maxw : (int64_t)4 * kColsumSlices * wz;
   w.part = (float*)take(nparts * 4);
   w.Mp = Mp;
   if (ws) *ws = w;
@@ -1214,6 +1249,11 @@ extern "C" int64_t ks_mlp_train_workspace_bytes(const KsMlp* h, int64_t M) {
 
 template <typename T>
 static int train_forward(DevMlp& m, hipStream_t s, int64_t M, const float* x, float* y, const TrainWs& ws) {
+  // bf16 networks that fit the whole-network kernel run it, with every hidden layer's activations written out for the backward
+  // pass as well; the stored rows must have the width the backward pass expects (its padding is in units of 64, the kernel's 32)
+  bool whole = m.fused && m.dtype == KS_MLP_BF16 && m.activation != KS_ACT_GELU;
+  for (int l = 0; whole && l + 1 < m.n_layers; ++l) whole = m.npad[l] == m.fn[l] * 32;
+  if (whole) return launch_fused(m, s, M, x, y, ws.act);
   const void* in = x;
   int64_t ldin = m.dims[0];
   for (int l = 0; l < m.n_layers; ++l) {
@@ -1278,8 +1318,9 @@ static int train_backward(DevMlp& m, hipStream_t s, int64_t M, const float* x, c
     }
     if (!want_w && l == 0) break;
     if (want_w && !have_bias) {
-      hipLaunchKernelGGL(colsum_kernel<T>, dim3((unsigned)((np + 63) / 64), kColsumSlices), dim3(256), 0, s, M, np, dz, ws.part);
-      hipLaunchKernelGGL(sum_parts_kernel, dim3((unsigned)((np + 255) / 256)), dim3(256), 0, s, (int64_t)np, kColsumSlices, ws.part, m.gb[l]);
+      const int nz = M >= 32768 ? 4 * kColsumSlices : kColsumSlices;  // narrow layers: more row slices fill the chip
+      hipLaunchKernelGGL(colsum_kernel<T>, dim3((unsigned)((np + 63) / 64), nz), dim3(256), 0, s, M, np, dz, ws.part);
+      hipLaunchKernelGGL(sum_parts_tree_kernel, dim3((unsigned)np), dim3(64), 0, s, (int64_t)np, nz, ws.part, m.gb[l]);
     }
     if (want_w && !have_dzT)
       hipLaunchKernelGGL((transpose_kernel<T, T>), dim3((unsigned)((Mp + 31) / 32), (unsigned)((np + 31) / 32)), dim3(256), 0, s, M, np,
@@ -1302,7 +1343,7 @@ static int train_backward(DevMlp& m, hipStream_t s, int64_t M, const float* x, c
           default: KS_PREP(KS_ACT_NONE); break;
         }
 #undef KS_PREP
-        hipLaunchKernelGGL(sum_parts_kernel, dim3((unsigned)((kp + 255) / 256)), dim3(256), 0, s, (int64_t)kp, kColsumSlices, ws.part, m.gb[l - 1]);
+        hipLaunchKernelGGL(sum_parts_tree_kernel, dim3((unsigned)kp), dim3(64), 0, s, (int64_t)kp, kColsumSlices, ws.part, m.gb[l - 1]);
         have_yT = have_dzT = have_bias = true;
       } else {
         const int64_t n = M * kp;

@@ -779,12 +779,20 @@ __global__ __launch_bounds__(128) void ppo_loss_grad_mixture_kernel(int64_t M, i
   d_value[m] = p.value_loss_coef * gv * inv_m;
 }
 
-__global__ void ppo_grad_finish_kernel(int nblocks, int nu, const float* __restrict__ partial, float* __restrict__ d_log_std) {
-  const int a = threadIdx.x;
-  if (a >= nu) return;
+// d_log_std[a] = sum over the blocks' partial sums: one workgroup per action, a fixed tree over up to 256 partials (one
+// thread walking them one after the other spends 256 dependent load latencies on it)
+__global__ __launch_bounds__(256) void ppo_grad_finish_kernel(int nblocks, int nu, const float* __restrict__ partial, float* __restrict__ d_log_std) {
+  __shared__ float red[256];
+  const int a = blockIdx.x;
   float s = 0.f;
-  for (int b = 0; b < nblocks; ++b) s += partial[(int64_t)b * nu + a];
-  d_log_std[a] = s;
+  for (int b = threadIdx.x; b < nblocks; b += 256) s += partial[(int64_t)b * nu + a];
+  red[threadIdx.x] = s;
+  __syncthreads();
+  for (int w = 128; w > 0; w >>= 1) {
+    if ((int)threadIdx.x < w) red[threadIdx.x] += red[threadIdx.x + w];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) d_log_std[a] = red[0];
 }
 
 // adaptive KL: partial[b] = sum over the block's strided share of (on_lp - lp), every element of every row
@@ -920,7 +928,7 @@ extern "C" int ks_ppo_loss_grad(ks_stream_t stream, int64_t M, int32_t nu, const
   const int blocks = (int)(want < KS_PPO_GRAD_BLOCKS ? want : KS_PPO_GRAD_BLOCKS);
   hipLaunchKernelGGL(ks::ppo_loss_grad_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream, M, nu, *params, mean, log_std, action,
                      on_log_probs, advantages, value_targets, on_values, values, d_mean, d_value, (float*)workspace);
-  hipLaunchKernelGGL(ks::ppo_grad_finish_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, blocks, nu, (const float*)workspace,
+  hipLaunchKernelGGL(ks::ppo_grad_finish_kernel, dim3(nu), dim3(256), 0, (hipStream_t)stream, blocks, nu, (const float*)workspace,
                      d_log_std);
   return ks::check_launch("ks_ppo_loss_grad");
 }
