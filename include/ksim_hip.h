@@ -320,7 +320,7 @@ typedef struct KsStepIO {
 } KsStepIO;
 
 int ks_step(const KsModel* model, ks_stream_t stream, const KsStepIO* io /*host*/);
-/* order = the envs sorted by work, heaviest first (counting sort; ties in arbitrary order).  When N is a multiple of 8 (and at
+/* order = the envs sorted by work, heaviest first (counting sort over buckets of four work units; ties in arbitrary order).  When N is a multiple of 8 (and at
  * least 512) the sort runs inside the eight regions [r N / 8, (r + 1) N / 8) and region r's envs go to order[r], order[r + 8],
  * ...: workgroup b of the step launch runs on XCD b % 8, so every XCD then steps one contiguous eighth of the env arrays,
  * heaviest first, and the 128-byte lines that neighbouring envs' rows share stay in one L2. */

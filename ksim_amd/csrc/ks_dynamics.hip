@@ -1492,41 +1492,44 @@ extern "C" int ks_forward(const KsModel* model, ks_stream_t stream, const KsStep
 }
 
 namespace ks {
-constexpr int kWorkBuckets = 2048;
+constexpr int kWorkBuckets = 512, kWorkShift = 2, kWorkThreads = 256;  // buckets of four work units
 constexpr int kXcds = 8;  // workgroup b of a launch runs on XCD b % 8, each XCD with an L2 of its own
+__device__ __forceinline__ int work_bucket(int w) { return min(max(w, 0) >> kWorkShift, kWorkBuckets - 1); }
 // Counting sort of envs by descending work in one workgroup: histogram, suffix sums, scatter.
 // With gridDim.x == 8 (N a multiple of 8) workgroup r sorts the envs of region r = [r N / 8, (r + 1) N / 8) and writes them
 // to order[r], order[r + 8], ...: the step kernel's workgroup b = r + 8 k then runs on XCD r and finds there only envs of
 // region r.  The state rows of neighbouring envs share 128-byte lines (an env's qpos row is 108 bytes); kept inside one XCD
 // such a line is fetched into, and written back from, one L2 instead of two.
-__global__ __launch_bounds__(1024) void work_order_kernel(int64_t N, const int32_t* __restrict__ work, int32_t* __restrict__ order) {
+// Four wavefronts and 4 KB of LDS: in a rollout on several streams this launch has to find room on a CU that another group's
+// physics launch fills, and a small workgroup finds it as soon as one wavefront per SIMD has left.
+__global__ __launch_bounds__(kWorkThreads) void work_order_kernel(int64_t N, const int32_t* __restrict__ work, int32_t* __restrict__ order) {
   __shared__ int hist[kWorkBuckets];
   __shared__ int scan[kWorkBuckets];
   const int t = threadIdx.x;
   const int regions = gridDim.x, region = blockIdx.x;
   const int64_t n = N / regions, first = region * n;
-  for (int b = t; b < kWorkBuckets; b += 1024) hist[b] = 0;
+  for (int b = t; b < kWorkBuckets; b += kWorkThreads) hist[b] = 0;
   __syncthreads();
-  for (int64_t i = t; i < n; i += 1024) atomicAdd(&hist[min(max(work[first + i], 0), kWorkBuckets - 1)], 1);
+  for (int64_t i = t; i < n; i += kWorkThreads) atomicAdd(&hist[work_bucket(work[first + i])], 1);
   __syncthreads();
   // inclusive suffix sums (heaviest bucket first) by doubling
-  for (int b = t; b < kWorkBuckets; b += 1024) scan[b] = hist[b];
+  for (int b = t; b < kWorkBuckets; b += kWorkThreads) scan[b] = hist[b];
   __syncthreads();
   for (int off = 1; off < kWorkBuckets; off <<= 1) {
-    int v[kWorkBuckets / 1024];
-    for (int k = 0; k < kWorkBuckets / 1024; ++k) {
-      const int b = t + 1024 * k;
+    int v[kWorkBuckets / kWorkThreads];
+    for (int k = 0; k < kWorkBuckets / kWorkThreads; ++k) {
+      const int b = t + kWorkThreads * k;
       v[k] = scan[b] + (b + off < kWorkBuckets ? scan[b + off] : 0);
     }
     __syncthreads();
-    for (int k = 0; k < kWorkBuckets / 1024; ++k) scan[t + 1024 * k] = v[k];
+    for (int k = 0; k < kWorkBuckets / kWorkThreads; ++k) scan[t + kWorkThreads * k] = v[k];
     __syncthreads();
   }
   // bucket b starts after all heavier buckets: scan[b] - hist[b]
-  for (int b = t; b < kWorkBuckets; b += 1024) hist[b] = scan[b] - hist[b];
+  for (int b = t; b < kWorkBuckets; b += kWorkThreads) hist[b] = scan[b] - hist[b];
   __syncthreads();
-  for (int64_t i = t; i < n; i += 1024) {
-    const int pos = atomicAdd(&hist[min(max(work[first + i], 0), kWorkBuckets - 1)], 1);
+  for (int64_t i = t; i < n; i += kWorkThreads) {
+    const int pos = atomicAdd(&hist[work_bucket(work[first + i])], 1);
     order[(int64_t)pos * regions + region] = (int32_t)(first + i);
   }
 }
@@ -1538,6 +1541,6 @@ extern "C" int ks_work_order(ks_stream_t stream, int64_t N, const int32_t* work,
   if (N == 0) return KS_OK;
   if (!work || !order) return fail(KS_EINVAL, "ks_work_order: null argument");
   const int regions = (N % kXcds == 0 && N >= 64 * kXcds) ? kXcds : 1;
-  hipLaunchKernelGGL(work_order_kernel, dim3(regions), dim3(1024), 0, (hipStream_t)stream, N, work, order);
+  hipLaunchKernelGGL(work_order_kernel, dim3(regions), dim3(kWorkThreads), 0, (hipStream_t)stream, N, work, order);
   return check_launch("ks_work_order");
 }

@@ -418,13 +418,13 @@ __device__ __forceinline__ void fused_layer(const FusedArgs& a, int l, __bf16* _
 }
 
 template <int ACT, int BM>
-__device__ __forceinline__ void mlp_fused_body(const FusedArgs& a) {
+__device__ __forceinline__ void mlp_fused_body(const FusedArgs& a, int64_t tile) {
   constexpr int MI = BM / 32;
   constexpr int NTHR = 64 * kFusedWaves;
   extern __shared__ __attribute__((aligned(16))) unsigned char mlp_lds[];
   __bf16* act = reinterpret_cast<__bf16*>(mlp_lds);
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int64_t m0 = (int64_t)blockIdx.x * BM;
+  const int64_t m0 = tile * BM;
   const int lda = a.lda;
   KS_MLP_STAMP(0)
   {  // network input -> bf16 tile; zero beyond the batch and in the K padding of the first layer
@@ -491,7 +491,7 @@ __device__ __forceinline__ void mlp_fused_body(const FusedArgs& a) {
 template <int ACT, int BM>
 __global__ __launch_bounds__(64 * kFusedWaves) __attribute__((amdgpu_waves_per_eu(BM <= 64 ? 4 : 2, BM <= 64 ? 4 : 2)))
 void mlp_fused_kernel(const FusedArgs a) {
-  mlp_fused_body<ACT, BM>(a);
+  mlp_fused_body<ACT, BM>(a, blockIdx.x);
 }
 
 // Two networks over the same rows in one launch (actor and critic of a control step): blockIdx.y picks the network, so
@@ -499,8 +499,18 @@ void mlp_fused_kernel(const FusedArgs a) {
 template <int ACT, int BM>
 __global__ __launch_bounds__(64 * kFusedWaves) __attribute__((amdgpu_waves_per_eu(BM <= 64 ? 4 : 2, BM <= 64 ? 4 : 2)))
 void mlp_fused_pair_kernel(const FusedArgs a, const FusedArgs b) {
-  if (blockIdx.y == 0) mlp_fused_body<ACT, BM>(a);
-  else mlp_fused_body<ACT, BM>(b);
+  // Workgroup L of the launch runs on XCD L % 8.  XCDs 0-3 take the first network and 4-7 the second, so that an XCD's L2
+  // fetches one network's weights, not both (the weights are cold at every control step: the physics launch in between
+  // sweeps the L2s).
+  const int64_t L = blockIdx.x + (int64_t)blockIdx.y * gridDim.x;
+  int net = blockIdx.y;
+  int64_t tile = blockIdx.x;
+  if (gridDim.x % 4 == 0) {
+    net = (int)(L % 8) / 4;
+    tile = (L / 8) * 4 + (L % 8) % 4;
+  }
+  if (net == 0) mlp_fused_body<ACT, BM>(a, tile);
+  else mlp_fused_body<ACT, BM>(b, tile);
 }
 
 struct DevMlp {
@@ -1203,7 +1213,7 @@ static void refresh_layers(DevMlp& m, hipStream_t s) {
   }
 }
 
-constexpr int kDwSplit = 16;  // most slices the weight-gradient reduction over the rows is cut into
+constexpr int kDwSplit = 32;  // most slices the weight-gradient reduction over the rows is cut into
 
 // workspace: hidden activations of every layer, two (M, widest) gradient buffers, two transposes (widest, Mp)
 struct TrainWs {
@@ -1374,10 +1384,16 @@ static int train_backward(DevMlp& m, hipStream_t s, int64_t M, const float* x, c
                            m.npad[l - 1], (int64_t)m.npad[l - 1], (const T*)ws.act[l - 1], kp128, Mp, (T*)ws.t1);
     }
     // the reduction runs over the rows: cut it into slices so that the grid covers the chip, then add the slices up
-    int ksplit = kDwSplit;
+    // wide layers over many rows: 128 x 128 output tiles halve the operand traffic per flop, twice the slices keep the grid
+    const bool wide = Mp >= 32768 && np % 128 == 0;
+    int ksplit = wide ? kDwSplit : kDwSplit / 2;
     while (ksplit > 1 && (Mp / 64) % ksplit != 0) ksplit >>= 1;
-    rc = launch_layer_tile<T, false, true, 64, 128, 2, 2>(KS_ACT_NONE, s, np, kp128, (int)Mp, (int)Mp, kp, dzT, Mp, ws.t1,
-                                                           m.zero_bias, ksplit > 1 ? (void*)ws.part : (void*)m.gW[l], kp, ksplit);
+    if (wide)
+      rc = launch_layer_tile<T, false, true, 128, 128, 2, 2>(KS_ACT_NONE, s, np, kp128, (int)Mp, (int)Mp, kp, dzT, Mp, ws.t1,
+                                                              m.zero_bias, ksplit > 1 ? (void*)ws.part : (void*)m.gW[l], kp, ksplit);
+    else
+      rc = launch_layer_tile<T, false, true, 64, 128, 2, 2>(KS_ACT_NONE, s, np, kp128, (int)Mp, (int)Mp, kp, dzT, Mp, ws.t1,
+                                                             m.zero_bias, ksplit > 1 ? (void*)ws.part : (void*)m.gW[l], kp, ksplit);
     if (rc != KS_OK) return rc;
     if (ksplit > 1) {
       const int64_t n = (int64_t)np * kp;
