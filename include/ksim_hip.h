@@ -541,8 +541,8 @@ int ks_terminate_reset(const KsTerms* terms, ks_stream_t stream, const KsTermina
  * values move towards the targets by at most accel * ctrl_dt.  Draws u0..: linear = target speed, target yaw, zero,
  * backward, switch; angular = target speed, flip, zero, switch. */
 #define KS_MAX_COMMANDS 8
-#define KS_COMMAND_DRAWS 8
-#define KS_MAX_VECTOR_COMMAND 6
+#define KS_COMMAND_DRAWS 20
+#define KS_MAX_VECTOR_COMMAND 16
 enum { KS_CMD_CONST = 0, KS_CMD_LINEAR_VELOCITY = 1, KS_CMD_ANGULAR_VELOCITY = 2,
        /* FloatVectorCommand / IntVectorCommand (commands.py:97-170): `dim` <= KS_MAX_VECTOR_COMMAND scalars, each uniform in
           [lo, hi] (integers: lo..hi inclusive), all zero with probability zero_prob; redrawn at an episode start and with
@@ -561,12 +561,28 @@ enum { KS_CMD_CONST = 0, KS_CMD_LINEAR_VELOCITY = 1, KS_CMD_ANGULAR_VELOCITY = 2
           |qvel[0:2]| <= moving_threshold the flag and the phase drop to 0 (the flag stays down until the next start).
           Foot f at phase p_f = (phase + f / feet) mod 1 gets height_offset + max_height sin(pi (p_f - stance) / (1 - stance))
           in swing (p_f >= stance), height_offset in stance. */
-       KS_CMD_SINUSOIDAL_GAIT = 8 };
+       KS_CMD_SINUSOIDAL_GAIT = 8,
+       /* JointPositionCommand (commands.py:821-914): n = (dim - 3) / 2 <= KS_MAX_VECTOR_COMMAND joints; the value is the
+          reference's JointPositionCommandValue flattened: start (n), target (n), total_time, num_steps, step_id.  At an
+          episode start: target_j uniform in [lo[j], hi[j]] (u_j), start_j = qpos[7 + joints[j]], total_time uniform in
+          [min_time, max_time] (u_n), num_steps = ceil(total_time / ctrl_dt), step_id = 0.  Afterwards step_id += 1, and once
+          step_id > num_steps a new value is drawn the same way from the current state. */
+       KS_CMD_JOINT_POSITION = 9,
+       /* CartesianCoordinateCommand (commands.py:537-694): current (3), target (3), speed (dim 7).  lo / hi [0..2] = the box
+          (already scaled by the curriculum level), min_vel / max_vel = the speed range, ctrl_dt = the command's dt.  At an
+          episode start target = current = a point of the box (u0..u2) and speed uniform (u3).  Afterwards, with
+          d = |target - current|: when (d < dt speed / 2 and u4 < switch_prob) or u4 < jump_prob (one draw decides both) a
+          new target and speed are drawn; then current moves towards the target by min(speed dt, d) with d the distance to
+          the OLD target (commands.py:640-653). */
+       KS_CMD_CARTESIAN_COORDINATE = 10 };
 typedef struct KsCommandDesc {
   int32_t kind, index, dim;    /* offset and length inside the command vector */
   float min_vel, max_vel, max_yaw, zero_prob, backward_prob, switch_prob; /* scales already evaluated at the curriculum level */
   float ctrl_dt, linear_accel, angular_accel;
   float lo[KS_MAX_VECTOR_COMMAND], hi[KS_MAX_VECTOR_COMMAND]; /* vector commands: the ranges */
+  int32_t joints[KS_MAX_VECTOR_COMMAND]; /* joint position command: actuated-joint indices (qpos[7 + j]) */
+  float min_time, max_time;              /* joint position command: range of the time to reach a target */
+  float jump_prob;                       /* cartesian command */
 } KsCommandDesc;
 typedef struct KsCommandIO {
   int64_t N;

@@ -148,17 +148,18 @@ class KsGruDesc(ctypes.Structure):
                 ("weight_hh", c_void_p), ("bias", c_void_p), ("bias_n", c_void_p)]
 
 
-KS_MAX_COMMANDS, KS_COMMAND_DRAWS = 8, 8
-KS_MAX_VECTOR_COMMAND = 6
+KS_MAX_COMMANDS, KS_COMMAND_DRAWS = 8, 20
+KS_MAX_VECTOR_COMMAND = 16
 (CMD_CONST, CMD_LINEAR_VELOCITY, CMD_ANGULAR_VELOCITY, CMD_FLOAT_VECTOR, CMD_INT_VECTOR, CMD_START_POSITION,
- CMD_START_QUATERNION, CMD_BASE_HEIGHT, CMD_SINUSOIDAL_GAIT) = range(9)
+ CMD_START_QUATERNION, CMD_BASE_HEIGHT, CMD_SINUSOIDAL_GAIT, CMD_JOINT_POSITION, CMD_CARTESIAN_COORDINATE) = range(11)
 
 
 class KsCommandDesc(ctypes.Structure):
     _fields_ = [("kind", c_int32), ("index", c_int32), ("dim", c_int32), ("min_vel", c_float), ("max_vel", c_float),
                 ("max_yaw", c_float), ("zero_prob", c_float), ("backward_prob", c_float), ("switch_prob", c_float),
                 ("ctrl_dt", c_float), ("linear_accel", c_float), ("angular_accel", c_float),
-                ("lo", c_float * KS_MAX_VECTOR_COMMAND), ("hi", c_float * KS_MAX_VECTOR_COMMAND)]
+                ("lo", c_float * KS_MAX_VECTOR_COMMAND), ("hi", c_float * KS_MAX_VECTOR_COMMAND),
+                ("joints", c_int32 * KS_MAX_VECTOR_COMMAND), ("min_time", c_float), ("max_time", c_float), ("jump_prob", c_float)]
 
 
 class KsCommandIO(ctypes.Structure):

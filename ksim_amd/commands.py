@@ -172,6 +172,73 @@ class SinusoidalGaitCommand(Command):  # commands.py:696-770: layout moving_flag
         return d
 
 
+@dataclass(frozen=True)
+class JointPositionCommand(Command):  # commands.py:821-914; the value is JointPositionCommandValue flattened
+    """start (n), target (n), total_time, num_steps, step_id: JointPositionReward reads this layout."""
+
+    indices: tuple = ()   # actuated-joint indices (joint order without the floating base)
+    ranges: tuple = ()    # (lo, hi) per joint
+    ctrl_dt: float = 0.02
+    min_time: float = 0.1
+    max_time: float = 1.0
+
+    def __post_init__(self):
+        if not 1 <= len(self.indices) <= T.KS_MAX_VECTOR_COMMAND or len(self.ranges) != len(self.indices):
+            raise ValueError(f"a joint position command takes 1..{T.KS_MAX_VECTOR_COMMAND} joints and one range for each")
+        if not (self.min_time > 0.0 and self.max_time > 0.0):
+            raise ValueError("min_time and max_time must be positive")
+
+    @classmethod
+    def create(cls, model, ctrl_dt: float, joint_names, min_time: float = 0.1, max_time: float = 1.0):
+        """By name, with the joints' own ranges as the target ranges (commands.py:895-914).  A hinge is named after the body
+        it moves (every body here carries at most one joint)."""
+        names = list(model.body_names)
+        idx, ranges = [], []
+        for name in joint_names:
+            if name not in names or int(model.body_qadr[names.index(name)]) < 7:
+                raise ValueError(f"Joint {name} not found in the model! Options are: {[n for n in names if int(model.body_qadr[names.index(n)]) >= 7]}")
+            b = names.index(name)
+            idx.append(int(model.body_qadr[b]) - 7)
+            ranges.append((float(model.jnt_range[b][0]), float(model.jnt_range[b][1])))
+        return cls(indices=tuple(idx), ranges=tuple(ranges), ctrl_dt=ctrl_dt, min_time=min_time, max_time=max_time)
+
+    def dim(self):
+        return 2 * len(self.indices) + 3
+
+    def desc(self, level):
+        d = T.KsCommandDesc()
+        d.kind, d.dim, d.ctrl_dt = T.CMD_JOINT_POSITION, self.dim(), float(self.ctrl_dt)
+        d.min_time, d.max_time = float(self.min_time), float(self.max_time)
+        for j, (i, (lo, hi)) in enumerate(zip(self.indices, self.ranges)):
+            d.joints[j], d.lo[j], d.hi[j] = int(i), float(lo), float(hi)
+        return d
+
+
+@dataclass(frozen=True)
+class CartesianCoordinateCommand(Command):  # commands.py:537-694; the value is current (3), target (3), speed
+    box_min: tuple = (0.0, 0.0, 0.0)
+    box_max: tuple = (0.0, 0.0, 0.0)
+    dt: float = 0.02
+    min_speed: float = 0.5
+    max_speed: float = 3.0
+    switch_prob: float = 0.0
+    jump_prob: float = 0.0
+    curriculum_scale: float = 0.1
+
+    def dim(self):
+        return 7
+
+    def desc(self, level):
+        d = T.KsCommandDesc()
+        d.kind, d.dim, d.ctrl_dt = T.CMD_CARTESIAN_COORDINATE, 7, float(self.dt)
+        d.min_vel, d.max_vel, d.switch_prob, d.jump_prob = float(self.min_speed), float(self.max_speed), float(self.switch_prob), float(self.jump_prob)
+        grow = self.curriculum_scale * float(level) + 1.0  # the box grows about its centre with the level (commands.py:561-572)
+        for j in range(3):
+            centre, half = 0.5 * (self.box_min[j] + self.box_max[j]), 0.5 * (self.box_max[j] - self.box_min[j])
+            d.lo[j], d.hi[j] = centre - half * grow, centre + half * grow
+        return d
+
+
 class CommandSet:
     def __init__(self, commands: Mapping[str, Command]):
         if len(commands) > T.KS_MAX_COMMANDS:

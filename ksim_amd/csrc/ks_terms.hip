@@ -1006,7 +1006,7 @@ __global__ __launch_bounds__(256) void command_kernel(KsCommandIO io) {
   if (idx >= io.N * io.n_commands) return;
   const int64_t e = idx / io.n_commands;
   const int k = (int)(idx - e * io.n_commands);
-  const KsCommandDesc c = io.commands[k];
+  const KsCommandDesc& c = io.commands[k];  // read in place: a copy of a runtime-indexed element would go through scratch memory
   float* cmd = io.command + e * io.command_dim + c.index;
   if (io.traj_command)
     for (int j = 0; j < c.dim; ++j) io.traj_command[e * io.command_dim + c.index + j] = cmd[j];
@@ -1016,10 +1016,10 @@ __global__ __launch_bounds__(256) void command_kernel(KsCommandIO io) {
     for (int j = 0; j < KS_COMMAND_DRAWS; ++j) u[j] = io.uniform[idx * KS_COMMAND_DRAWS + j];
   } else {
     const uint64_t step = io.rng.step + (io.rng.step_base ? *io.rng.step_base : 0ull);
-    const Philox4 a = draw(io.rng.seed, step, kRngCommand, (uint64_t)e, (uint32_t)(2 * k));
-    const Philox4 b = draw(io.rng.seed, step, kRngCommand, (uint64_t)e, (uint32_t)(2 * k + 1));
-    u[0] = u01(a.x); u[1] = u01(a.y); u[2] = u01(a.z); u[3] = u01(a.w);
-    u[4] = u01(b.x); u[5] = u01(b.y); u[6] = u01(b.z); u[7] = u01(b.w);
+    for (int j = 0; j < KS_COMMAND_DRAWS / 4; ++j) {
+      const Philox4 a = draw(io.rng.seed, step, kRngCommand, (uint64_t)e, (uint32_t)((KS_COMMAND_DRAWS / 4) * k + j));
+      u[4 * j] = u01(a.x); u[4 * j + 1] = u01(a.y); u[4 * j + 2] = u01(a.z); u[4 * j + 3] = u01(a.w);
+    }
   }
   const bool fresh = io.all_fresh || (io.fresh && io.fresh[e]);
   const float* qv = io.qvel + e * io.nv;
@@ -1065,6 +1065,46 @@ __global__ __launch_bounds__(256) void command_kernel(KsCommandIO io) {
       pf -= floorf(pf);
       const float prog = fminf(fmaxf((pf - stance) / (1.f - stance), 0.f), 1.f);
       cmd[2 + f] = (pf >= stance ? max_h * sinf(3.14159265358979323846f * prog) : 0.f) + offset;
+    }
+  } else if (c.kind == KS_CMD_JOINT_POSITION) {
+    const int n = (c.dim - 3) / 2;
+    const float step_id = cmd[2 * n + 2] + 1.f;
+    if (fresh || step_id > cmd[2 * n + 1]) {  // commands.py:852-893: a new target, from where the joints are now
+      const float* q = io.qpos + e * io.nq + 7;
+      for (int j = 0; j < KS_MAX_VECTOR_COMMAND; ++j)
+        if (j < n) {
+          cmd[j] = q[c.joints[j]];
+          cmd[n + j] = c.lo[j] + u[j] * (c.hi[j] - c.lo[j]);
+        }
+      float total = 0.f;
+      for (int j = 0; j <= KS_MAX_VECTOR_COMMAND; ++j)
+        if (j == n) total = c.min_time + u[j] * (c.max_time - c.min_time);  // the draw after the targets'
+      cmd[2 * n] = total;
+      cmd[2 * n + 1] = ceilf(total / c.ctrl_dt);
+      cmd[2 * n + 2] = 0.f;
+    } else {
+      cmd[2 * n + 2] = step_id;
+    }
+  } else if (c.kind == KS_CMD_CARTESIAN_COORDINATE) {
+    float box[3], new_speed = c.min_vel + u[3] * (c.max_vel - c.min_vel);
+    for (int j = 0; j < 3; ++j) box[j] = c.lo[j] + u[j] * (c.hi[j] - c.lo[j]);
+    if (fresh) {
+      for (int j = 0; j < 3; ++j) cmd[j] = cmd[3 + j] = box[j];
+      cmd[6] = new_speed;
+    } else {
+      float speed = cmd[6];
+      const float dx = cmd[3] - cmd[0], dy = cmd[4] - cmd[1], dz = cmd[5] - cmd[2];
+      const float dist = sqrtf(dx * dx + dy * dy + dz * dz);
+      const bool reached = dist < c.ctrl_dt * speed * 0.5f;
+      if ((reached && u[4] < c.switch_prob) || u[4] < c.jump_prob) {
+        for (int j = 0; j < 3; ++j) cmd[3 + j] = box[j];
+        speed = new_speed;
+      }
+      float dir[3] = {cmd[3] - cmd[0], cmd[4] - cmd[1], cmd[5] - cmd[2]};
+      const float norm = sqrtf(dir[0] * dir[0] + dir[1] * dir[1] + dir[2] * dir[2]);
+      const float move = fminf(speed * c.ctrl_dt, dist);  // the distance to the target held before this step
+      for (int j = 0; j < 3; ++j) cmd[j] += (norm > 0.f ? dir[j] / norm : dir[j]) * move;
+      cmd[6] = speed;
     }
   } else if (c.kind == KS_CMD_BASE_HEIGHT) {
     if (fresh || u[0] < c.switch_prob) cmd[0] = c.lo[0] + u[0] * (c.hi[0] - c.lo[0]);
@@ -1566,7 +1606,15 @@ extern "C" int ks_commands(ks_stream_t stream, const KsCommandIO* io) {
       if (c.dim < 3 || c.dim > 2 + KS_MAX_VECTOR_COMMAND) return fail(KS_ELIMIT, "ks_commands: command %d: 1..%d feet", k, KS_MAX_VECTOR_COMMAND);
       if (!(c.lo[0] > 0.f) || !(c.lo[3] < 1.f) || !io->qvel || io->nv < 2) return fail(KS_EINVAL, "ks_commands: command %d: gait period, stance ratio or the base velocity missing", k);
     }
-    if (c.kind < KS_CMD_CONST || c.kind > KS_CMD_SINUSOIDAL_GAIT) return fail(KS_EINVAL, "ks_commands: command %d: bad kind", k);
+    if (c.kind == KS_CMD_CARTESIAN_COORDINATE) need = 7;
+    if (c.kind == KS_CMD_JOINT_POSITION) {
+      const int n = (c.dim - 3) / 2;
+      if (c.dim < 5 || c.dim != 2 * n + 3 || n > KS_MAX_VECTOR_COMMAND) return fail(KS_ELIMIT, "ks_commands: command %d: a joint position command holds 2 n + 3 values, 1 <= n <= %d", k, KS_MAX_VECTOR_COMMAND);
+      if (!io->qpos || !(c.ctrl_dt > 0.f) || !(c.min_time > 0.f) || !(c.max_time >= c.min_time)) return fail(KS_EINVAL, "ks_commands: command %d: joint positions, ctrl_dt or the time range missing", k);
+      for (int j = 0; j < n; ++j)
+        if (c.joints[j] < 0 || 7 + c.joints[j] >= io->nq) return fail(KS_EINVAL, "ks_commands: command %d: joint %d outside qpos[7:%d]", k, c.joints[j], io->nq);
+    }
+    if (c.kind < KS_CMD_CONST || c.kind > KS_CMD_CARTESIAN_COORDINATE) return fail(KS_EINVAL, "ks_commands: command %d: bad kind", k);
     if ((c.kind == KS_CMD_START_POSITION || c.kind == KS_CMD_START_QUATERNION) && (!io->qpos || io->nq < 7))
       return fail(KS_EINVAL, "ks_commands: command %d reads the pose of a floating base", k);
     if ((c.kind == KS_CMD_FLOAT_VECTOR || c.kind == KS_CMD_INT_VECTOR) && c.dim > KS_MAX_VECTOR_COMMAND) return fail(KS_ELIMIT, "ks_commands: command %d: %d scalars (at most %d)", k, c.dim, KS_MAX_VECTOR_COMMAND);

@@ -613,6 +613,46 @@ def sinusoidal_gait_command(prev, qvel, fresh, *, gait_period, ctrl_dt, max_heig
     return np.concatenate([[flag, new_phase], heights(new_phase)])
 
 
+def joint_position_command(prev, qpos, u, fresh, *, indices, ranges, ctrl_dt, min_time, max_time):
+    """One control step of JointPositionCommand for one env (ksim/commands.py:852-893), in float32 like the reference.
+    prev / result = start (n), target (n), total_time, num_steps, step_id; u = draws (one per target, then the time)."""
+    f = np.float32
+    n = len(indices)
+    prev = np.asarray(prev, dtype=f)
+    step_id = prev[2 * n + 2] + f(1)
+    if fresh or step_id > prev[2 * n + 1]:
+        lo, hi = np.asarray(ranges, dtype=f).T
+        target = lo + np.asarray(u[:n], dtype=f) * (hi - lo)
+        start = np.asarray(qpos, dtype=f)[7 + np.asarray(indices)]
+        total = f(min_time) + f(u[n]) * (f(max_time) - f(min_time))
+        return np.concatenate([start, target, [total, np.ceil(total / f(ctrl_dt)), f(0)]]).astype(f)
+    out = prev.copy()
+    out[2 * n + 2] = step_id
+    return out
+
+
+def cartesian_coordinate_command(prev, u, fresh, *, box_min, box_max, dt, min_speed=0.5, max_speed=3.0, switch_prob=0.0, jump_prob=0.0,
+                                 curriculum_scale=0.1, level=1.0):
+    """One control step of CartesianCoordinateCommand for one env (ksim/commands.py:556-656).  prev / result = current (3),
+    target (3), speed; u = draws (box point x, y, z; speed; switch / jump, which share one key in the reference)."""
+    lo, hi = np.asarray(box_min, dtype=np.float64), np.asarray(box_max, dtype=np.float64)
+    centre, half = (lo + hi) / 2.0, (hi - lo) / 2.0 * (curriculum_scale * level + 1.0)
+    point = (centre - half) + np.asarray(u[:3], dtype=np.float64) * (2.0 * half)
+    new_speed = min_speed + u[3] * (max_speed - min_speed)
+    if fresh:
+        return np.concatenate([point, point, [new_speed]])
+    prev = np.asarray(prev, dtype=np.float64)
+    current, target, speed = prev[:3], prev[3:6], prev[6]
+    distance = np.linalg.norm(target - current)
+    reached = distance < dt * speed * 0.5
+    if (reached and u[4] < switch_prob) or u[4] < jump_prob:
+        target, speed = point, new_speed
+    direction = target - current
+    norm = np.linalg.norm(direction)
+    direction = direction / norm if norm > 0 else direction
+    return np.concatenate([current + direction * min(speed * dt, distance), target, [speed]])
+
+
 def sinusoidal_gait_reward(position_tn3, height_tn, max_height):  # rewards.py:1331-1335
     return 1.0 - np.abs(np.asarray(position_tn3, dtype=np.float64)[..., 2] - np.asarray(height_tn, dtype=np.float64)).sum(axis=-1) / max_height
 

@@ -1032,6 +1032,47 @@ def test_sinusoidal_gait_command_and_reward():
         rw.get_rewards(traj, {"gait": rw.SinusoidalGaitReward(pos_obs="feet", pos_cmd="nope")}, obs_slices={"feet": slice(0, 9)}, command_slices=cs.slices)
 
 
+def test_joint_position_and_cartesian_commands():
+    """JointPositionCommand (with JointPositionReward reading its value) and CartesianCoordinateCommand against the oracle on
+    the same draws, episode starts mixed in."""
+    from ksim_amd import _lib_terms as T
+    from ksim_amd.commands import CartesianCoordinateCommand, CommandSet, JointPositionCommand
+
+    N, steps = 41, 40
+    rng = np.random.default_rng(59)
+    jp = dict(indices=(3, 0, 11), ranges=((-0.5, 0.7), (0.1, 0.2), (-1.0, -0.2)), ctrl_dt=0.02, min_time=0.05, max_time=0.3)
+    cc = dict(box_min=(-0.3, 0.1, 0.5), box_max=(0.4, 0.6, 1.2), dt=0.02, min_speed=0.8, max_speed=4.0, switch_prob=0.7, jump_prob=0.05, curriculum_scale=0.25)
+    cs = CommandSet({"joints": JointPositionCommand(**jp), "hand": CartesianCoordinateCommand(**cc)})
+    assert cs.command_dim == 9 + 7 and cs.slices["hand"] == slice(9, 16)
+    cmd = cs.initial(N, DEV)
+    want = np.zeros((N, 16))
+    redrawn_j = redrawn_c = 0
+    for k in range(steps):
+        qpos = rng.normal(size=(N, 27)).astype(np.float32)
+        qvel = rng.normal(size=(N, 26)).astype(np.float32)
+        u = rng.random((N, 2, T.KS_COMMAND_DRAWS)).astype(np.float32)
+        fresh = np.ones(N, bool) if k == 0 else rng.random(N) < 0.05
+        rec = torch.empty(N, 16, device=DEV)
+        cs.update(cmd, t32(qpos), t32(qvel), level=0.6, fresh=torch.from_numpy(fresh.astype(np.uint8)).to(DEV), record=rec, uniform=t32(u))
+        np.testing.assert_allclose(rec.cpu().numpy(), want, rtol=1e-6, atol=1e-6)
+        for e in range(N):
+            new = ot.joint_position_command(want[e, :9], qpos[e], u[e, 0], bool(fresh[e]), **jp)
+            redrawn_j += (not fresh[e]) and new[8] == 0
+            want[e, :9] = new
+            new = ot.cartesian_coordinate_command(want[e, 9:], u[e, 1].astype(np.float64), bool(fresh[e]), level=0.6, **cc)
+            redrawn_c += (not fresh[e]) and not np.allclose(new[3:6], want[e, 12:15])
+            want[e, 9:] = new
+        got = cmd.cpu().numpy()
+        np.testing.assert_allclose(got[:, :7], want[:, :7], rtol=1e-6, atol=1e-7)  # float32 on both sides, up to a fused multiply-add
+        np.testing.assert_array_equal(got[:, 7:9], want[:, 7:9])                   # num_steps and step_id
+        np.testing.assert_allclose(got[:, 9:], want[:, 9:], rtol=2e-5, atol=2e-6)
+    assert redrawn_j > 50 and redrawn_c > 30
+    with pytest.raises(Exception, match="outside qpos"):
+        CommandSet({"j": JointPositionCommand(indices=(25,), ranges=((0.0, 1.0),))}).update(cs.initial(N, DEV)[:, :5].contiguous(), t32(qpos), t32(qvel), all_fresh=True)
+    with pytest.raises(ValueError):
+        JointPositionCommand(indices=(1, 2), ranges=((0.0, 1.0),))
+
+
 def test_vector_commands():
     """FloatVectorCommand / IntVectorCommand: the properties the reference's own tests check (shape, bounds, a command
     that never switches stays what it was, reference tests/test_commands.py:64-96) and the draw arithmetic."""

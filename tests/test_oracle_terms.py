@@ -701,3 +701,58 @@ def test_imu_offset_site_rotation_and_contact_list_hand_computed():
     assert ot.contact_observation(dist, (0, -1, 2)).tolist() == [True, True, False]
     assert ot.contact_observation(dist, (0, 1)).tolist() == [False, False]
     assert ot.contact_observation(np.array([0.1, -0.5, 0.02]), (0, -1, 2)).tolist() == [False, False, False]
+
+
+def test_joint_position_command_reaches_its_target_on_time():
+    """What the reference's value type fixes (ksim/commands.py:795-818, 852-893): the commanded position start + (target - start)
+    step_id / num_steps moves linearly, is the target exactly when step_id = num_steps = ceil(total_time / ctrl_dt), holds for
+    that one step, and the next value starts from where the joints are then; the commanded velocity is (target - start) /
+    total_time throughout."""
+    rng = np.random.default_rng(3)
+    kw = dict(indices=(2, 0), ranges=((-1.0, 1.0), (0.2, 0.4)), ctrl_dt=0.02, min_time=0.1, max_time=0.5)
+    qpos = rng.normal(size=12)
+    u = np.array([0.25, 0.5, 0.775] + [0.0] * 5)
+    v = ot.joint_position_command(np.zeros(7), qpos, u, True, **kw)
+    np.testing.assert_allclose(v[:2], qpos[[9, 7]], rtol=1e-6)
+    np.testing.assert_allclose(v[2:4], [-0.5, 0.3], rtol=1e-6)
+    assert v[4] == pytest.approx(0.41) and v[5] == 21 and v[6] == 0  # ceil(0.41 / 0.02) = 21
+    seen = []
+    for k in range(1, 22):
+        v = ot.joint_position_command(v, rng.normal(size=12), rng.random(8), False, **kw)
+        assert v[6] == k
+        seen.append(v[:2] + (v[2:4] - v[:2]) * v[6] / v[5])
+    np.testing.assert_allclose(np.diff(np.stack(seen), axis=0), np.tile((v[2:4] - v[:2]) / 21, (20, 1)), rtol=1e-4, atol=1e-6)
+    np.testing.assert_allclose(seen[-1], v[2:4], rtol=1e-6)
+    q2, u2 = rng.normal(size=12), rng.random(8)
+    w = ot.joint_position_command(v, q2, u2, False, **kw)  # step_id 22 > 21: a new target from the current pose
+    assert w[6] == 0
+    np.testing.assert_allclose(w[:2], q2[[9, 7]].astype(np.float32), rtol=1e-6)
+    assert -1.0 <= w[2] <= 1.0 and 0.2 <= w[3] <= 0.4 and 0.1 <= w[4] <= 0.5 and w[5] == np.ceil(np.float32(w[4]) / np.float32(0.02))
+
+
+def test_cartesian_coordinate_command_moves_at_its_speed_without_overshoot():
+    """ksim/commands.py:556-656: the current point travels straight towards the target at `speed`, lands on it exactly (the
+    last stride is cut to the remaining distance), stays there while no switch is drawn, and draws a new target inside the box
+    scaled by the curriculum level once it has arrived and the switch draw allows; a jump draw replaces the target at any time."""
+    kw = dict(box_min=(-1.0, 0.0, 0.5), box_max=(1.0, 2.0, 1.5), dt=0.05, min_speed=1.0, max_speed=2.0, curriculum_scale=0.5, level=1.0)
+    first = ot.cartesian_coordinate_command(np.zeros(7), [0.0, 1.0, 0.5, 0.5, 0.9], True, **kw)
+    # the box grows by 1.5 about its centre (0, 1, 1): x in [-1.5, 1.5], y in [-0.5, 2.5], z in [0.25, 1.75]
+    np.testing.assert_allclose(first, [-1.5, 2.5, 1.0, -1.5, 2.5, 1.0, 1.5])
+    v = first.copy()
+    v[3:6] = [-1.5 + 0.3, 2.5, 1.0 + 0.4]  # a target 0.5 away; at 1.5 * 0.05 = 0.075 a step: six full strides and one of 0.05
+    path = [v[:3].copy()]
+    for k in range(9):
+        v = ot.cartesian_coordinate_command(v, [0.1, 0.2, 0.3, 0.4, 0.99], False, switch_prob=0.5, **kw)
+        path.append(v[:3].copy())
+    strides = np.linalg.norm(np.diff(np.stack(path), axis=0), axis=1)
+    np.testing.assert_allclose(strides, [0.075] * 6 + [0.05, 0.0, 0.0], atol=1e-12)
+    np.testing.assert_allclose(v[:3], v[3:6], atol=1e-12)
+    # arrived and the draw falls under switch_prob: a new target and speed; the point does not move this step (old distance 0)
+    w = ot.cartesian_coordinate_command(v, [0.5, 0.5, 0.5, 0.0, 0.2], False, switch_prob=0.5, **kw)
+    np.testing.assert_allclose(w, np.concatenate([v[:3], [0.0, 1.0, 1.0, 1.0]]), atol=1e-12)
+    # still travelling: the same draw does not switch, a jump does, and the stride of that step is still capped by the old distance
+    v[3:6] = v[:3] + [0.0, 0.0, 0.03]
+    stay = ot.cartesian_coordinate_command(v, [0.5, 0.5, 0.5, 0.0, 0.2], False, switch_prob=0.0, jump_prob=0.1, **kw)
+    np.testing.assert_allclose(stay[3:6], v[3:6]); assert np.linalg.norm(stay[:3] - v[:3]) == pytest.approx(0.03)
+    jump = ot.cartesian_coordinate_command(v, [0.5, 0.5, 0.5, 0.0, 0.05], False, switch_prob=0.0, jump_prob=0.1, **kw)
+    np.testing.assert_allclose(jump[3:], [0.0, 1.0, 1.0, 1.0]); assert np.linalg.norm(jump[:3] - v[:3]) == pytest.approx(0.03)
