@@ -37,6 +37,11 @@ typedef __attribute__((ext_vector_type(16))) float f32x16;
 #else
 #define KS_TICK(k)
 #endif
+// A phase boundary of the step kernel.  The LDS layout is rebuilt from an offset the compiler cannot see through: the
+// two dozen array addresses are then a few scalar additions at the start of each phase instead of values that stay live
+// from the top of the kernel, where they do not fit the scalar registers and every use reads its address back out of a
+// vector register lane.
+#define KS_PHASE(k) { KS_TICK(k) int off_ = 0; asm volatile("" : "+s"(off_)); l = carve(lds_raw + off_, nb, nq, nv, nu, ns, nvs, js); }
 // Register rows (mass matrix, Hessian, Jacobian) are padded from nv to a compile-time width NP, one kernel
 // instantiation per width: the padding rows are unit rows and the padding columns zero, so the factorisation,
 // the triangular solves and the row products run without any bound checks.
@@ -73,8 +78,7 @@ __host__ __device__ inline int lds_floats(int nb, int nq, int nv, int nu, int ns
   return n + 8;
 }
 
-__device__ inline Lds carve(float* p, const DevModel& m) {
-  const int nb = m.nb, nq = m.nq, nv = m.nv, nu = m.nu, ns = m.ns, nvs = m.nvs, js = m.js;
+__device__ __forceinline__ Lds carve(float* p, int nb, int nq, int nv, int nu, int ns, int nvs, int js) {
   Lds l;
   auto take = [&](int n) {
     float* r = p;
@@ -125,6 +129,9 @@ __device__ __forceinline__ void load_row(const float* p, float (&v)[NP]) {
 //   R[j], j < i : L[i][j]              R[k], k > i : L[k][i] * L[i][i]              myinv = 1 / L[i][i]
 template <int NP>
 __device__ __forceinline__ void chol_tile(f32x16& T, float (&R)[NP], float& myinv, int lane) {
+  // The lane id is made opaque so that the per-step lane masks are compared where they are used: shared between the call
+  // sites they would be sixty-odd scalar register pairs that live across the solver and are read back from spill lanes.
+  asm volatile("" : "+v"(lane));
   const int c = lane & 31, half = lane >> 5;
   myinv = 1.f;
 #pragma unroll
@@ -172,6 +179,7 @@ __device__ __forceinline__ void load_mtile(f32x16& T, const float* __restrict__ 
 // x = (L L^T)^-1 b, lane i holding b_i and returning x_i
 template <int NP>
 __device__ __forceinline__ float solve_regs(const float (&R)[NP], float myinv, int lane, float b) {
+  asm volatile("" : "+v"(lane));  // as in chol_tile: the masks lane > j, lane < k are rebuilt here, not kept
   float r = b;
 #pragma unroll
   for (int j = 0; j < NP; ++j) {  // L y = b; lane j keeps r_j = y_j * L[j][j]
@@ -325,7 +333,7 @@ void step_kernel(StepArgs a) {
   if (a.env_mask && !a.env_mask[env]) return;  // wave-uniform
   int work = 0;  // wave-uniform cost estimate of this control step
   const int nb = m.nb, nq = m.nq, nv = m.nv, nu = m.nu, ns = m.ns, nvs = m.nvs, js = m.js;
-  const Lds l = carve(lds_raw, m);
+  Lds l = carve(lds_raw, nb, nq, nv, nu, ns, nvs, js);
   const int rq = (nb > 1 && m.body_jtype[1] == kJntFree) ? 7 : 0;
   const int rv = rq ? 6 : 0;
 
@@ -481,7 +489,7 @@ void step_kernel(StepArgs a) {
       KS_SYNC();
     }
 
-    KS_TICK(0)
+    KS_PHASE(0)
     // ---- kinematics.  Every body first writes its pose relative to its parent (joint rotation included) to
     // LDS, then composes the poses along its own chain of ancestors from the root down: max_depth short
     // steps shared by all bodies instead of one full pass per tree level.
@@ -543,7 +551,7 @@ void step_kernel(StepArgs a) {
     }
     KS_SYNC();
 
-    KS_TICK(1)
+    KS_PHASE(1)
     // ---- centre of mass of the tree (wave-uniform), com-based inertias and motion axes
     const float mt = wave_sum(b_mass);
     const float minv = mt > 1e-15f ? 1.0f / mt : 0.f;
@@ -598,7 +606,7 @@ void step_kernel(StepArgs a) {
     }
     KS_SYNC();
 
-    KS_TICK(2)
+    KS_PHASE(2)
     // ---- composite inertias (subtree = contiguous body range) and the mass matrix
     for (int idx = lane; idx < nb * 10; idx += 64) {
       const int b = idx / 10, k = idx - 10 * b;
@@ -619,7 +627,7 @@ void step_kernel(StepArgs a) {
       }
     }
 
-    KS_TICK(3)
+    KS_PHASE(3)
     // ---- body velocities and bias accelerations: the motion axes are all expressed in one frame, so every
     // body accumulates them over the dofs of its own ancestor chain, root first (no pass per tree level)
     {
@@ -716,7 +724,7 @@ void step_kernel(StepArgs a) {
     }
     KS_SYNC();
 
-    KS_TICK(4)
+    KS_PHASE(4)
     // ---- mass-matrix row into registers; smooth forces: passive - bias + actuator
     const float* Mrow = l.M + (is_dof ? lane : 0) * nvs;
     float qfs = 0.f, my_qvel = 0.f;
@@ -733,7 +741,7 @@ void step_kernel(StepArgs a) {
 #endif
     }
 
-    KS_TICK(5)
+    KS_PHASE(5)
     // ---- contacts: sphere vs plane z = 0, compacted to the penetrating ones
     float dist = 1.f;
     V3 cpos = {0.f, 0.f, 0.f};
@@ -771,7 +779,7 @@ void step_kernel(StepArgs a) {
     }
     KS_SYNC();
 
-    KS_TICK(6)
+    KS_PHASE(6)
     // ---- Cholesky of M and the unconstrained acceleration (registers only)
     float R[NP];
     float myinv;
@@ -784,7 +792,7 @@ void step_kernel(StepArgs a) {
     const float qas = is_dof ? qas_all : 0.f;  // lanes that hold no row carry meaningless numbers
     if (a.dbg_qacc_smooth && is_dof) a.dbg_qacc_smooth[env * nv + lane] = qas;
 
-    KS_TICK(7)
+    KS_PHASE(7)
     float qacc = qas;
     float Mqacc = qfs;  // M qacc = smooth + constraint force: what the implicit integration step solves against
     int niter = 0;
@@ -848,8 +856,7 @@ void step_kernel(StepArgs a) {
       }
       const float warm = is_dof ? l.warm[lane] : 0.f;
       KS_SYNC();
-      KS_TICK(8)
-
+      KS_PHASE(8)
       // cost of the warm start and of the unconstrained acceleration; start from the cheaper one
       float Ma_w = 0.f, Ma_s = 0.f, Jar_w = 0.f, Jar_s = 0.f;
       {
@@ -883,8 +890,7 @@ void step_kernel(StepArgs a) {
       float cost = use_warm ? cost_w : cost_s;
       float prev_cost = INFINITY;
       bool first = true;
-      KS_TICK(9)
-
+      KS_PHASE(9)
       unsigned long long am_factored = 0ull;  // active set that R currently factors
       unsigned long long amd_factored = 0ull; // and the quadratic zones of the dof-lane rows
       bool have_factor = false;               // none yet: R holds the factor of M
@@ -921,7 +927,7 @@ void step_kernel(StepArgs a) {
         done |= improvement < m.tolerance;
         done |= gradient < m.tolerance;
         if (done && !(m.iterations == 1 && niter == 0)) break;
-        KS_TICK(10)
+        KS_PHASE(10)
         // ---- Newton direction: H = M + J^T diag(D active) J.  The rank-nefc term runs on the matrix cores: one
         // 32x32x2 fp32 MFMA per pair of constraint rows, operands straight from the LDS copy of J (lane = column,
         // lane half = row of the pair).  The accumulator tile holds, in lane c, rows {8g + 4 (lane / 32) + e} of
@@ -948,7 +954,7 @@ void step_kernel(StepArgs a) {
 #pragma unroll
               for (int e = 0; e < 4; ++e) hc[4 * g + e] += (8 * g + 4 * half + e == col) ? hd : 0.f;
           }
-          KS_TICK(11)
+          KS_PHASE(11)
           chol_tile<NP>(hc, R, myinv, lane);
           am_factored = am;
           amd_factored = amd;
@@ -956,8 +962,7 @@ void step_kernel(StepArgs a) {
         }
         const float search_all = -solve_regs<NP>(R, myinv, lane, grad);
         const float search = is_dof ? search_all : 0.f;
-        KS_TICK(12)
-
+        KS_PHASE(12)
         // ---- exact line search along `search`
         float mv = 0.f, jv = 0.f;
         {
@@ -1070,7 +1075,7 @@ void step_kernel(StepArgs a) {
         Ma += alpha * mv;
         Jaref += alpha * jv;
         ++niter;
-        KS_TICK(13)
+        KS_PHASE(13)
       }
       Mqacc = Ma;
       // ---- Cartesian contact forces on the bodies (mjData.cfrc_ext), only when asked for: a pyramid row with force f
@@ -1113,7 +1118,7 @@ void step_kernel(StepArgs a) {
     KS_SYNC();
     if (is_dof) l.warm[lane] = qacc;
 
-    KS_TICK(14)
+    KS_PHASE(14)
     // ---- semi-implicit Euler
     if (!FWD) {
       // What this stage needs of the lane's constants is read again here (through an opaque lane id, so that the loads
@@ -1165,7 +1170,7 @@ void step_kernel(StepArgs a) {
     KS_SYNC();
   }
 
-  KS_TICK(15)
+  KS_PHASE(15)
 #ifdef KS_PROFILE
   if (a.dbg_M && lane == 0) for (int k = 0; k < 16; ++k) a.dbg_M[env * nv * nv + k] = prof[k];
 #endif
