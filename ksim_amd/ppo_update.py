@@ -255,6 +255,11 @@ class RecurrentHeadPolicy:
     num_mixtures: int = 0
     clip_lo: torch.Tensor | None = None
     clip_hi: torch.Tensor | None = None
+    kl_scale: torch.Tensor | None = None  # adaptive KL: current coefficient / cfg.kl_coef, one device float
+
+    def kl_coef(self, cfg: "PPOUpdateConfig") -> float:
+        """The KL coefficient now in force (a host read: for logging and tests)."""
+        return cfg.kl_coef * (float(self.kl_scale.item()) if self.kl_scale is not None else 1.0)
 
     def train_init(self) -> None:
         self.actor.train_init()
@@ -282,8 +287,10 @@ def single_step_recurrent(policy: RecurrentHeadPolicy, cfg: PPOUpdateConfig, act
     inputs = ppo_mod.compute_ppo_inputs(value.view(Tn, b), rewards, done, success, cfg.gamma, cfg.lam,
                                         normalize_advantages=cfg.normalize_advantages,
                                         monte_carlo_returns=cfg.monte_carlo_returns, time_major=True)
+    if cfg.adaptive_kl and policy.kl_scale is None:  # as in single_step: the factor stays on the device
+        policy.kl_scale = torch.ones(1, dtype=torch.float32, device=raw.device)
     p = _lib.KsPpoLossParams(cfg.clip_param, cfg.value_loss_coef, cfg.entropy_coef, cfg.kl_coef, cfg.log_clip_value, 1.0,
-                             int(cfg.use_clipped_value_loss))
+                             int(cfg.use_clipped_value_loss), _lib.ptr(policy.kl_scale) if cfg.adaptive_kl else None)
     mixture = policy.num_mixtures > 0
     head = policy._mixture() if mixture else T.KsGaussianHead(float(policy.min_std), float(policy.max_std), float(policy.var_scale), 0,
                                                               _lib.ptr(policy.mean_bias).value)
@@ -303,8 +310,21 @@ def single_step_recurrent(policy: RecurrentHeadPolicy, cfg: PPOUpdateConfig, act
     ap = _adam(cfg, policy.opt_step)
     policy.actor.adam_step(ap, sq)
     policy.critic.adam_step(ap, sq)
-    return {"grad_norm": sq.sqrt(), "d_raw": d_raw, "d_value": d_value, "raw": raw, "values": value,
-            "advantages": inputs.advantages_bt}
+    metrics = {"grad_norm": sq.sqrt(), "d_raw": d_raw, "d_value": d_value, "raw": raw, "values": value,
+               "advantages": inputs.advantages_bt}
+    if cfg.adaptive_kl:  # ppo.py:546-563 on the log-probabilities of this step's forward pass
+        lp = torch.empty(rows, nu, dtype=torch.float32, device=raw.device)
+        if mixture:
+            _lib.check(lib.ks_mixture_head_log_prob(_lib.current_stream(), rows, nu, ctypes.byref(head), _lib.ptr(raw),
+                                                    _lib.ptr(action.contiguous()), _lib.ptr(lp)))
+        else:
+            _lib.check(lib.ks_gaussian_head_log_prob(_lib.current_stream(), rows, nu, ctypes.byref(head), _lib.ptr(raw),
+                                                     _lib.ptr(action.contiguous()), _lib.ptr(lp), None))
+        ws = torch.empty(256 * nu, dtype=torch.float32, device=raw.device)
+        _lib.check(lib.ks_ppo_adapt_kl(_lib.current_stream(), rows, nu, _lib.ptr(on_log_probs.contiguous()), _lib.ptr(lp), cfg.kl_coef,
+                                       cfg.desired_kl, _lib.ptr(policy.kl_scale), _lib.ptr(ws)))
+        metrics["log_probs"] = lp
+    return metrics
 
 
 def recurrent_on_policy(policy: RecurrentHeadPolicy, actor_obs, critic_obs, action, actor_carry0, critic_carry0, fresh):
@@ -335,8 +355,6 @@ def update_model_recurrent(policy: RecurrentHeadPolicy, cfg: PPOUpdateConfig, ac
     """num_passes x (N / batch_size) minibatch steps over a (T, N) rollout for a recurrent actor and critic
     (ppo.py:572-694): a minibatch is a set of env columns together with their carries at the rollout's first step."""
     Tn, N = done.shape
-    if cfg.adaptive_kl:
-        raise _lib.KsError("adaptive KL is built for the MLP policy update only")
     on_lp, on_v = recurrent_on_policy(policy, actor_obs, critic_obs, action, actor_carry0, critic_carry0, fresh)
     bs = min(cfg.batch_size, N)
     if N % bs:

@@ -540,6 +540,20 @@ def test_recurrent_policy_update_from_a_rollout(head):
     # the rollout goes on with the updated networks
     traj2, _ = ro.unroll(env)
     assert torch.isfinite(traj2.action).all() and torch.isfinite(ro.values).all()
+    # adaptive KL (ppo.py:546-563): after every minibatch step the coefficient follows the host rule on that step's log-probabilities
+    cfg = pu.PPOUpdateConfig(batch_size=N, num_passes=1, learning_rate=3e-3, adaptive_kl=True, desired_kl=1e-3)
+    on_lp, _ = pu.recurrent_on_policy(policy, args[0], args[1], args[2], *args[6:])
+    coef, moved = cfg.kl_coef, 0
+    for _ in range(4):
+        met = pu.update_model_recurrent(policy, cfg, *args, seed=2)[0]
+        kl_mean = float((on_lp.reshape(-1, on_lp.shape[-1]).double() - met["log_probs"].double()).sum(-1).mean().item()) * coef
+        new = coef * 1.5 if kl_mean > cfg.desired_kl * 1.5 else coef
+        new = new / 1.5 if kl_mean < cfg.desired_kl / 1.5 else new
+        moved += new != coef
+        coef = min(max(new, 1e-8), 1e2)
+        assert policy.kl_coef(cfg) == pytest.approx(coef, rel=1e-5)
+        on_lp, _ = pu.recurrent_on_policy(policy, args[0], args[1], args[2], *args[6:])
+    assert moved > 0
 
 
 def test_split_rollout_equals_single_stream_rollout():
