@@ -1508,10 +1508,12 @@ extern "C" int ks_mlp_adam_step(KsMlp* h, ks_stream_t stream, const KsAdamParams
 //   dP/dW_l += d_l^T v_{l-1},   u_l = v_{l-1} W_l^T,   v_l = u_l * f'(z_l),   r_l = u_l * a_l * f''(z_l),
 // and r_l, the part that reaches z_l through f', joins the ordinary backward pass of the squared-error terms as an extra
 // gradient of z_l on the real rows.  The discriminator is small next to the policy, so everything here runs in fp32 on the
-// master weights with a plain LDS-tiled product.
+// master weights, the products on the fp32 matrix-core instruction.
 namespace ks {
 
-// C(i, j) (+)= sum_k A(i, k) B(k, j): 64 x 64 tile per workgroup, 16-deep slices through LDS, 4 x 4 outputs per thread.
+// C(i, j) (+)= sum_k A(i, k) B(k, j) in fp32 on the matrix cores: 64 x 64 tile per workgroup, 16-deep slices through LDS,
+// each of the four wavefronts accumulating one 32 x 32 quadrant with v_mfma_f32_32x32x2_f32 (lane c + 32 h feeds
+// A(c, 2 s + h) and B(2 s + h, c) of step s and ends up with C(8 g + 4 h + e, c) in accumulator register 4 g + e).
 // A_KC: A is stored (i, k) with k contiguous, otherwise (k, i); B_KC: B is stored (j, k) with k contiguous, otherwise (k, j).
 // gridDim.z cuts the k range into slices of kslice; with more than one slice, slice z writes its partial product (M, N)
 // densely to C + z * M * N and sum_slices_kernel adds them up in a fixed order.
@@ -1523,12 +1525,11 @@ __global__ __launch_bounds__(256) void sgemm_kernel(int M, int N, int K, const f
   __shared__ float Bs[16][68];
   const int t = threadIdx.x, i0 = blockIdx.y * 64, j0 = blockIdx.x * 64;
   const int kbeg = blockIdx.z * kslice, kend = min(K, kbeg + kslice);
-  const int ti = t / 16, tj = t % 16;
-  float acc[4][4];
+  const int wave = t >> 6, lane = t & 63, c = lane & 31, h = lane >> 5;
+  const int wi = (wave >> 1) * 32, wj = (wave & 1) * 32;
+  f32x16 acc;
 #pragma unroll
-  for (int r = 0; r < 4; ++r)
-#pragma unroll
-    for (int c = 0; c < 4; ++c) acc[r][c] = 0.f;
+  for (int r = 0; r < 16; ++r) acc[r] = 0.f;
   for (int k0 = kbeg; k0 < kend; k0 += 16) {
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
@@ -1541,31 +1542,25 @@ __global__ __launch_bounds__(256) void sgemm_kernel(int M, int N, int K, const f
     }
     __syncthreads();
 #pragma unroll
-    for (int k = 0; k < 16; ++k) {
-      float a[4], b[4];
-#pragma unroll
-      for (int r = 0; r < 4; ++r) { a[r] = As[k][ti * 4 + r]; b[r] = Bs[k][tj * 4 + r]; }
-#pragma unroll
-      for (int r = 0; r < 4; ++r)
-#pragma unroll
-        for (int c = 0; c < 4; ++c) acc[r][c] = fmaf(a[r], b[c], acc[r][c]);
-    }
+    for (int s = 0; s < 8; ++s)
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(As[2 * s + h][wi + c], Bs[2 * s + h][wj + c], acc, 0, 0, 0);
     __syncthreads();
   }
   const bool sliced = gridDim.z > 1;
   float* out = sliced ? C + (int64_t)blockIdx.z * M * N : C;
   const int64_t ld = sliced ? N : ldc;
+  const int gj = j0 + wj + c;
+  if (gj >= N) return;
+  const float bj = (!sliced && bias) ? bias[gj] : 0.f;
 #pragma unroll
-  for (int r = 0; r < 4; ++r) {
-    const int gi = i0 + ti * 4 + r;
-    if (gi >= M) continue;
+  for (int g = 0; g < 4; ++g)
 #pragma unroll
-    for (int c = 0; c < 4; ++c) {
-      const int gj = j0 + tj * 4 + c;
-      if (gj >= N) continue;
-      float v = acc[r][c];
+    for (int e = 0; e < 4; ++e) {
+      const int gi = i0 + wi + 8 * g + 4 * h + e;
+      if (gi >= M) continue;
+      float v = acc[4 * g + e];
       if (!sliced) {
-        if (bias) v += bias[gj];
+        v += bj;
         if (act == KS_ACT_ELU) v = v > 0.f ? v : expm1f(v);
         else if (act == KS_ACT_RELU) v = fmaxf(v, 0.f);
         else if (act == KS_ACT_TANH) v = tanhf(v);
@@ -1573,7 +1568,6 @@ __global__ __launch_bounds__(256) void sgemm_kernel(int M, int N, int K, const f
       }
       out[(int64_t)gi * ld + gj] = v;
     }
-  }
 }
 
 __global__ __launch_bounds__(256) void sum_slices_kernel(int M, int N, int nz, const float* __restrict__ part, float* __restrict__ C,
