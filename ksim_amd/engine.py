@@ -27,6 +27,7 @@ MISSING = None
 
 
 # per-env replacements of model fields that randomisers may produce (ksim/randomization.py), passed to the kernels as they are
+_RESIDENT_ENVS = 256 * 16  # wavefronts of the step kernel that an MI355X holds at a time: 256 CUs x 4 SIMDs x 4 waves
 _MODEL_FIELD_OVERRIDES = ("frictionloss", "body_ipos", "body_inertia", "sph_pos", "sph_radius")
 
 @dataclass
@@ -262,7 +263,9 @@ class HipEngine(PhysicsEngine):
         """The (order, work) buffers of the heaviest-first launch order, made on first use; call before capturing
         `step` into a HIP graph so that their initialisation is not part of the graph."""
         sched = getattr(state, "_schedule", None)
-        if sched is None and self.data.balance_launch_order:
+        # A launch of at most _RESIDENT_ENVS envs is resident all at once (one wavefront per env), so the order in which its
+        # workgroups start changes nothing: no order is kept, and the kernel's own XCD-aware mapping applies.
+        if sched is None and self.data.balance_launch_order and state.data.qpos.shape[0] > _RESIDENT_ENVS:
             n, dev = state.data.qpos.shape[0], state.data.qpos.device
             sched = (torch.arange(n, dtype=torch.int32, device=dev), torch.zeros(n, dtype=torch.int32, device=dev))
             state._schedule = sched
