@@ -368,8 +368,13 @@ enum { /* KsObsElem.kind */
                            r = R_body (c0, c1, c2), g = (q0, q1, q2), q_site = (e0, e1, e2, e3) */
   KS_OBS_SITE_ROT6D = 8, /* entry `comp` (0..5) of the 6-D rotation of a site of body `index` (SiteOrientationObservation,
                            observation.py:645-669): the first two rows of R(q_body q_site), row-major */
-  KS_OBS_CONTACT_ANY = 9 /* 1 when any contact sphere whose bit is set in `index` touches the floor: the floor's own entry of
+  KS_OBS_CONTACT_ANY = 9, /* 1 when any contact sphere whose bit is set in `index` touches the floor: the floor's own entry of
                            ContactObservation (observation.py:452-478), whose geom list holds the floor and some spheres */
+  /* MuJoCo's framepos / framequat / magnetometer sensors of a site of body `index` (read by SensorObservation like the
+     two above): component `comp` of xpos[index] + R_body (c0, c1, c2); component `comp` (0..3) of q_body q_site; component
+     `comp` of (q_body q_site)^-1 (q0, q1, q2), the model's magnetic field in the site frame.  (frameangvel needs no kind: it
+     is cvel[index][0:3], a KS_OBS_COPY.) */
+  KS_OBS_SITE_POS = 10, KS_OBS_SITE_QUAT = 11, KS_OBS_SITE_MAGNETOMETER = 12
 };
 /* Site kinds with env_site = 1 read the site's pose per env from KsObserveIO.site_pose instead of (e0..e3) and (c0, c1, c2):
  * the IMU mounting error of IMUAlignmentRandomizer (ksim/randomization.py:245-284) is a model field there, one per env. */
@@ -397,7 +402,7 @@ typedef struct KsObsElem {
                                     stored standard draw (KsObserveIO.bias_draw) at the current curriculum level, which is what
                                     re-drawing with the episode's key gives (observation.py:136-141, ksim/task/rl.py:263-271) */
   int32_t carry, stride;         /* stateful kinds: offset into the env's carry row, distance between delay slots */
-  float q0, q1, q2;              /* KS_OBS_GRAVITY_EMA: min_lag, max_lag, imu_bias; KS_OBS_SITE_ACCEL: gravity */
+  float q0, q1, q2;              /* KS_OBS_GRAVITY_EMA: min_lag, max_lag, imu_bias; KS_OBS_SITE_ACCEL: gravity; KS_OBS_SITE_MAGNETOMETER: field */
   float e0, e1, e2, e3;          /* site kinds: the site's orientation in its body, wxyz */
   int32_t env_site;              /* site kinds: 1 = take the site's pose from KsObserveIO.site_pose */
 } KsObsElem;

@@ -8,7 +8,7 @@ KS_MAX_OBS, KS_MAX_TERMS, KS_MAX_QPOS, KS_MAX_LAYERS = 512, 16, 40, 8
 (SRC_QPOS, SRC_QVEL, SRC_QACC, SRC_CTRL, SRC_LAST_ACTION, SRC_COMMAND, SRC_TIME, SRC_XPOS, SRC_XQUAT, SRC_CVEL,
  SRC_CONST, SRC_CONTACT_DIST, SRC_CINERT, SRC_CFRC_EXT, SRC_COUNT) = range(15)
 (OBS_COPY, OBS_JOINT_POS, OBS_ROT_INV, OBS_CONTACT, OBS_DELAYED, OBS_GRAVITY_EMA, OBS_SITE_GYRO, OBS_SITE_ACCEL,
- OBS_SITE_ROT6D, OBS_CONTACT_ANY) = range(10)
+ OBS_SITE_ROT6D, OBS_CONTACT_ANY, OBS_SITE_POS, OBS_SITE_QUAT, OBS_SITE_MAGNETOMETER) = range(13)
 (NOISE_NONE, NOISE_ADD_GAUSSIAN, NOISE_ADD_UNIFORM, NOISE_MUL_GAUSSIAN, NOISE_MUL_UNIFORM, NOISE_ADD_UNIFORM_GAUSSIAN,
  NOISE_MUL_UNIFORM_GAUSSIAN) = range(7)
 KS_MAX_NOISE_CHAIN = 4

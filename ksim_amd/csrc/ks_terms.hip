@@ -134,6 +134,29 @@ __global__ __launch_bounds__(256) void observe_kernel(ObserveArgs a) {
     axis[col] = 1.f;
     rot_fwd(q, axis, col_vec);  // column `col` of R
     v = col_vec[row];
+  } else if (el.kind == KS_OBS_SITE_POS || el.kind == KS_OBS_SITE_QUAT || el.kind == KS_OBS_SITE_MAGNETOMETER) {
+    const float* qb = a.src[KS_SRC_XQUAT] + e * a.src_dim[KS_SRC_XQUAT] + 4 * el.index;
+    float qs[4] = {el.e0, el.e1, el.e2, el.e3}, r_l[3] = {el.c0, el.c1, el.c2};
+    if (el.env_site) {
+      for (int k = 0; k < 4; ++k) qs[k] = a.site_pose[e * 7 + k];
+      for (int k = 0; k < 3; ++k) r_l[k] = a.site_pose[e * 7 + 4 + k];
+    }
+    if (el.kind == KS_OBS_SITE_POS) {
+      float r[3];
+      rot_fwd(qb, r_l, r);
+      v = a.src[KS_SRC_XPOS][e * a.src_dim[KS_SRC_XPOS] + 3 * el.index + el.comp] + r[el.comp];
+    } else if (el.kind == KS_OBS_SITE_QUAT) {
+      const float q[4] = {qb[0] * qs[0] - qb[1] * qs[1] - qb[2] * qs[2] - qb[3] * qs[3],
+                          qb[0] * qs[1] + qb[1] * qs[0] + qb[2] * qs[3] - qb[3] * qs[2],
+                          qb[0] * qs[2] - qb[1] * qs[3] + qb[2] * qs[0] + qb[3] * qs[1],
+                          qb[0] * qs[3] + qb[1] * qs[2] - qb[2] * qs[1] + qb[3] * qs[0]};
+      v = q[el.comp];
+    } else {
+      float in_body[3], out[3];
+      rot_inv(qb, el.q0, el.q1, el.q2, in_body);
+      rot_inv(qs, in_body[0], in_body[1], in_body[2], out);
+      v = out[el.comp];
+    }
   } else if (el.kind == KS_OBS_SITE_GYRO || el.kind == KS_OBS_SITE_ACCEL) {
     const float* qb = a.src[KS_SRC_XQUAT] + e * a.src_dim[KS_SRC_XQUAT] + 4 * el.index;
     const float* w = a.src[KS_SRC_CVEL] + e * a.src_dim[KS_SRC_CVEL] + 6 * el.index;  // angular velocity, world axes
@@ -1156,13 +1179,18 @@ extern "C" int ks_terms_create(const KsTermsDesc* d, KsTerms** out) {
   for (int k = 0; k < d->obs_dim; ++k) {
     const KsObsElem& el = d->obs[k];
     if (el.src < 0 || el.src >= KS_SRC_COUNT) return fail(KS_EINVAL, "ks_terms_create: obs %d: bad source %d", k, el.src);
-    if (el.kind < KS_OBS_COPY || el.kind > KS_OBS_CONTACT_ANY) return fail(KS_EINVAL, "ks_terms_create: obs %d: bad kind", k);
+    if (el.kind < KS_OBS_COPY || el.kind > KS_OBS_SITE_MAGNETOMETER) return fail(KS_EINVAL, "ks_terms_create: obs %d: bad kind", k);
     if (el.kind == KS_OBS_CONTACT_ANY) {
       if (d->ns < 1 || el.index <= 0 || (d->ns < 32 && (el.index >> d->ns) != 0)) return fail(KS_EINVAL, "ks_terms_create: obs %d: sphere mask 0x%x outside the model's %d spheres", k, el.index, d->ns);
       continue;
     }
     if (el.kind == KS_OBS_SITE_ROT6D) {
       if (el.comp < 0 || el.comp > 5 || el.index < 0 || el.index >= d->nb) return fail(KS_EINVAL, "ks_terms_create: obs %d: bad site orientation entry (component %d, body %d)", k, el.comp, el.index);
+      if (!(el.e0 * el.e0 + el.e1 * el.e1 + el.e2 * el.e2 + el.e3 * el.e3 > 0.f)) return fail(KS_EINVAL, "ks_terms_create: obs %d: the site orientation is not a quaternion", k);
+      continue;
+    }
+    if (el.kind == KS_OBS_SITE_POS || el.kind == KS_OBS_SITE_QUAT || el.kind == KS_OBS_SITE_MAGNETOMETER) {
+      if (el.comp < 0 || el.comp > (el.kind == KS_OBS_SITE_QUAT ? 3 : 2) || el.index < 0 || el.index >= d->nb) return fail(KS_EINVAL, "ks_terms_create: obs %d: bad site frame sensor (component %d, body %d)", k, el.comp, el.index);
       if (!(el.e0 * el.e0 + el.e1 * el.e1 + el.e2 * el.e2 + el.e3 * el.e3 > 0.f)) return fail(KS_EINVAL, "ks_terms_create: obs %d: the site orientation is not a quaternion", k);
       continue;
     }
@@ -1236,7 +1264,8 @@ extern "C" int ks_observe(const KsTerms* t, ks_stream_t stream, const KsObserveI
   bool needs_quat = false, needs_noise = false;
   for (int k = 0; k < d.obs_dim; ++k) {
     const KsObsElem& el = d.obs[k];
-    const bool site_kind = el.kind == KS_OBS_SITE_GYRO || el.kind == KS_OBS_SITE_ACCEL || el.kind == KS_OBS_SITE_ROT6D;
+    const bool frame_kind = el.kind == KS_OBS_SITE_POS || el.kind == KS_OBS_SITE_QUAT || el.kind == KS_OBS_SITE_MAGNETOMETER;
+    const bool site_kind = el.kind == KS_OBS_SITE_GYRO || el.kind == KS_OBS_SITE_ACCEL || el.kind == KS_OBS_SITE_ROT6D || frame_kind;
     if (site_kind && el.env_site && !io->site_pose) return fail(KS_EINVAL, "ks_observe: observation %d reads the per-env site pose, which is NULL", k);
     if (el.kind == KS_OBS_SITE_GYRO || el.kind == KS_OBS_SITE_ACCEL) {
       if (!io->src[KS_SRC_XQUAT] || !io->src[KS_SRC_CVEL] || (el.kind == KS_OBS_SITE_ACCEL && !io->src[KS_SRC_QACC]))
@@ -1245,6 +1274,11 @@ extern "C" int ks_observe(const KsTerms* t, ks_stream_t stream, const KsObserveI
     }
     if (el.kind == KS_OBS_SITE_ROT6D) {
       if (!io->src[KS_SRC_XQUAT]) return fail(KS_EINVAL, "ks_observe: observation %d (site orientation) needs xquat", k);
+      continue;
+    }
+    if (frame_kind) {
+      if (!io->src[KS_SRC_XQUAT] || (el.kind == KS_OBS_SITE_POS && !io->src[KS_SRC_XPOS]))
+        return fail(KS_EINVAL, "ks_observe: observation %d (site frame sensor) needs xquat and, for a position, xpos", k);
       continue;
     }
     if (el.kind == KS_OBS_CONTACT_ANY) {

@@ -156,6 +156,8 @@ def load_mjcf(path: str, **options) -> KinematicModel:
     opt = root.find("option")
     if opt is not None and "timestep" in opt.attrib:
         options.setdefault("dt", float(opt.get("timestep")))
+    if opt is not None and opt.get("magnetic") is not None:
+        options.setdefault("magnetic", tuple(_vec(opt.get("magnetic"), 3)))
 
     def angle(v):
         return np.radians(v) if degrees else v

@@ -143,6 +143,7 @@ class KinematicModel:
     sph_names: tuple = field(default=())  # collision geom of each contact sphere (both ends of a capsule carry its name)
     sites: dict = field(default_factory=dict)    # name -> (body, position (3), orientation wxyz (4)) in the body frame
     sensors: dict = field(default_factory=dict)  # name -> (MuJoCo sensor type, site name)
+    magnetic: tuple = (0.0, -0.5, 0.0)           # the magnetic field a magnetometer reads (MuJoCo option `magnetic`, its default)
 
     @property
     def has_free_root(self) -> bool:
@@ -169,7 +170,7 @@ class ModelBuilder:
     def __init__(self, dt=0.005, gravity=(0.0, 0.0, -9.81), iterations=8, ls_iterations=8, tolerance=1e-10,
                  ls_tolerance=0.01, impratio=1.0, eulerdamp=False, solref=(0.02, 1.0),
                  solimp=(0.9, 0.95, 0.001, 0.5, 2.0), friction=1.0, integrator=None, dof_solref=None, dof_solimp=None,
-                 condim=3):
+                 condim=3, magnetic=(0.0, -0.5, 0.0)):
         # integrator: "euler" (explicit joint damping unless `eulerdamp`) or "implicitfast", the one ksim sets
         # (ksim/task/rl.py:555-578).  With torque motors the only velocity-dependent smooth force is joint damping, so
         # implicitfast is the damping-implicit velocity update, (M + dt diag(damping)) a = M qacc.
@@ -185,6 +186,7 @@ class ModelBuilder:
                         friction=float(friction), condim=int(condim),
                         dof_solref=np.array(solref if dof_solref is None else dof_solref, dtype=np.float64),
                         dof_solimp=np.array(solimp if dof_solimp is None else dof_solimp, dtype=np.float64))
+        self.magnetic = tuple(float(x) for x in magnetic)
         self.bodies = [dict(parent=-1, jtype=JNT_NONE, pos=np.zeros(3), quat=np.array([1.0, 0, 0, 0]), mass=0.0,
                             ipos=np.zeros(3), iquat=np.array([1.0, 0, 0, 0]), inertia=np.zeros(3),
                             axis=np.array([0.0, 0, 1]), jpos=np.zeros(3), damping=0.0, armature=0.0, qpos0=0.0,
@@ -334,7 +336,7 @@ class ModelBuilder:
         )
         inv_b, inv_d, mean_inertia = _compile_constants(partial)
         return KinematicModel(**partial, body_invweight0=inv_b, dof_invweight0=inv_d, meaninertia=mean_inertia,
-                              sites=dict(self.sites), sensors=dict(self.sensors))
+                              sites=dict(self.sites), sensors=dict(self.sensors), magnetic=self.magnetic)
 
 
 # --------------------------------------------------------------------------- host kinematics (float64, init-time only)

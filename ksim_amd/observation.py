@@ -398,11 +398,13 @@ class CommandObservation(Observation):
 class SensorObservation(Observation):
     """A sensor of the model by name (observation.py:307-340 reads its slice of `sensordata`).  Built sensor types:
     `gyro` (angular velocity in the site frame), `accelerometer` (acceleration minus gravity in the site frame; the site
-    must sit on the floating base, where an IMU does) and `touch` (the normal contact force on the site's body: every
-    contact sphere of that body is taken to lie inside the site's volume, which holds for the feet of the shipped robots).
-    Like `sensordata`, they describe the state the last substep started from."""
+    must sit on the floating base, where an IMU does), `touch` (the normal contact force on the site's body: every
+    contact sphere of that body is taken to lie inside the site's volume, which holds for the feet of the shipped robots),
+    `framepos`, `framequat`, `frameangvel` of a site in world axes and `magnetometer` (the model's magnetic field in the site
+    frame).  Like `sensordata`, they describe the state the last substep started from."""
     sensor_name: str = ""
     site_pose_per_env: bool = False  # the sensor's site is randomised per env (IMUAlignmentRandomizer, randomization.py:245-284)
+    BUILT = ("gyro", "accelerometer", "touch", "framepos", "framequat", "frameangvel", "magnetometer")
 
     @classmethod
     def create(cls, *, physics_model: KinematicModel, sensor_name: str, noise=None):
@@ -410,8 +412,8 @@ class SensorObservation(Observation):
             options = "\n".join(sorted(physics_model.sensors))
             raise ValueError(f"{sensor_name} not found in model. Available:\n{options}")
         kind = physics_model.sensors[sensor_name][0]
-        if kind not in ("gyro", "accelerometer", "touch"):
-            raise ValueError(f"sensor {sensor_name!r} of type {kind} is not built (gyro, accelerometer, touch are)")
+        if kind not in cls.BUILT:
+            raise ValueError(f"sensor {sensor_name!r} of type {kind} is not built ({', '.join(cls.BUILT)} are)")
         return cls(sensor_name=sensor_name, noise=noise)
 
     def elements(self, m, command_dim):
@@ -422,6 +424,14 @@ class SensorObservation(Observation):
         env = int(self.site_pose_per_env)
         if kind == "gyro":
             return [ObsElem(T.OBS_SITE_GYRO, T.SRC_CVEL, body, c, e=tuple(quat), env_site=env) for c in range(3)]
+        if kind == "frameangvel":  # the body's angular velocity in world axes, wherever on the body the site sits
+            return [ObsElem(T.OBS_COPY, T.SRC_CVEL, 6 * body + c) for c in range(3)]
+        if kind == "framepos":
+            return [ObsElem(T.OBS_SITE_POS, T.SRC_XPOS, body, c, const=tuple(pos), e=tuple(quat), env_site=env) for c in range(3)]
+        if kind == "framequat":
+            return [ObsElem(T.OBS_SITE_QUAT, T.SRC_XQUAT, body, c, e=tuple(quat), env_site=env) for c in range(4)]
+        if kind == "magnetometer":
+            return [ObsElem(T.OBS_SITE_MAGNETOMETER, T.SRC_XQUAT, body, c, q=tuple(m.magnetic), e=tuple(quat), env_site=env) for c in range(3)]
         if body != 1 or not m.has_free_root:
             raise ValueError(f"accelerometer {self.sensor_name!r}: its site must sit on the floating base")
         return [ObsElem(T.OBS_SITE_ACCEL, T.SRC_CVEL, body, c, const=tuple(pos), q=tuple(m.gravity), e=tuple(quat), env_site=env)

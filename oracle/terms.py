@@ -751,6 +751,22 @@ def site_accelerometer(qacc6, xquat_body, omega_world, site_pos, site_quat, grav
     return rotate_vector_by_quat(rotate_vector_by_quat(a, q, inverse=True), np.asarray(site_quat, np.float64), inverse=True)
 
 
+def site_frame_position(xpos_body, xquat_body, site_pos):
+    """MuJoCo's framepos sensor of a site: the site's origin in world coordinates, x_body + R_body r."""
+    return np.asarray(xpos_body, np.float64) + rotate_vector_by_quat(np.asarray(site_pos, np.float64), np.asarray(xquat_body, np.float64))
+
+
+def site_frame_quaternion(xquat_body, site_quat):
+    """MuJoCo's framequat sensor of a site: its world orientation q_body q_site (w, x, y, z)."""
+    return quat_mul(np.asarray(xquat_body, np.float64), np.asarray(site_quat, np.float64))
+
+
+def site_magnetometer(xquat_body, site_quat, magnetic):
+    """MuJoCo's magnetometer: the model's (constant, world-frame) magnetic field seen in the site frame."""
+    in_body = rotate_vector_by_quat(np.asarray(magnetic, np.float64), np.asarray(xquat_body, np.float64), inverse=True)
+    return rotate_vector_by_quat(in_body, np.asarray(site_quat, np.float64), inverse=True)
+
+
 # ------------------------------------------------------------------ resets (ksim/resets.py), one env, explicit draws
 def xy_position_reset(qpos, ux, uy, *, x_range, y_range, padded_bounds, z=None, hfield=None, hfield_bounds=None,
                       robot_base_height=0.0):

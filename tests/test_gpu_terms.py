@@ -1261,6 +1261,25 @@ def test_sensor_observations_gyro_accelerometer_touch():
     if air.any():  # no contact: the base origin accelerates with gravity plus what the joints do; the reading stays moderate
         assert np.isfinite(got[air, 3:6]).all()
 
+    # frame sensors: the foot site's position and its body's angular velocity in world axes, the IMU site's orientation,
+    # and the model's magnetic field seen from the IMU site
+    frame = {n: ob.SensorObservation.create(physics_model=m, sensor_name=n) for n in ("left_foot_pos", "left_foot_angvel", "imu_quat", "imu_mag")}
+    terms_f = EnvTerms(m, frame, {}, [])
+    assert terms_f.obs_dim == 3 + 3 + 4 + 3
+    src_f = dict(src); src_f[T.SRC_XPOS] = buf["xpos"]
+    of = torch.empty(N, terms_f.obs_dim, device=DEV)
+    terms_f.observe(src_f, N, obs=of)
+    gf = of.cpu().numpy()
+    xp = buf["xpos"].cpu().numpy().reshape(N, m.nb, 3).astype(np.float64)
+    fb, fpos, _ = m.sites["left_foot"]
+    np.testing.assert_allclose(gf[:, 0:3], ot.site_frame_position(xp[:, fb], xq[:, fb], fpos), rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(gf[:, 3:6], cv[:, fb, :3], rtol=1e-6)
+    np.testing.assert_allclose(gf[:, 6:10], ot.site_frame_quaternion(xq[:, 1], squat), rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(gf[:, 10:13], ot.site_magnetometer(xq[:, 1], squat, m.magnetic), rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(np.linalg.norm(gf[:, 10:13], axis=1), np.linalg.norm(m.magnetic), rtol=1e-5)
+    with pytest.raises(Exception, match="xpos"):
+        terms_f.observe(src, N, obs=of)
+
     # IMUAlignmentRandomizer: every env has its own site pose; the sensors and the site's 6-D rotation follow it
     from ksim_amd import randomization as rnd
 

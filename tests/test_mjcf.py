@@ -147,12 +147,15 @@ def test_sites_and_sensors_are_read_through_the_welds():
     assert m.sites["left_foot"][0] == 3 and m.sites["right_foot"][0] == 5
     assert m.sensors == {"imu_acc": ("accelerometer", "imu_site"), "imu_gyro": ("gyro", "imu_site"),
                          "left_foot_touch": ("touch", "left_foot"), "right_foot_touch": ("touch", "right_foot"),
-                         "imu_quat": ("framequat", "imu_site")}
+                         "imu_quat": ("framequat", "imu_site"), "left_foot_pos": ("framepos", "left_foot"),
+                         "left_foot_angvel": ("frameangvel", "left_foot"), "imu_mag": ("magnetometer", "imu_site"),
+                         "imu_vel": ("velocimeter", "imu_site")}
+    assert m.magnetic == (0.1, -0.4, 0.2)
     from ksim_amd.observation import SensorObservation
     with pytest.raises(ValueError, match="not found"):
         SensorObservation.create(physics_model=m, sensor_name="nope")
     with pytest.raises(ValueError, match="not built"):
-        SensorObservation.create(physics_model=m, sensor_name="imu_quat")
+        SensorObservation.create(physics_model=m, sensor_name="imu_vel")
     assert SensorObservation.create(physics_model=m, sensor_name="imu_gyro").get_name() == "imu_gyro"
 
 

@@ -756,3 +756,20 @@ def test_cartesian_coordinate_command_moves_at_its_speed_without_overshoot():
     np.testing.assert_allclose(stay[3:6], v[3:6]); assert np.linalg.norm(stay[:3] - v[:3]) == pytest.approx(0.03)
     jump = ot.cartesian_coordinate_command(v, [0.5, 0.5, 0.5, 0.0, 0.05], False, switch_prob=0.0, jump_prob=0.1, **kw)
     np.testing.assert_allclose(jump[3:], [0.0, 1.0, 1.0, 1.0]); assert np.linalg.norm(jump[:3] - v[:3]) == pytest.approx(0.03)
+
+
+def test_site_frame_sensors_against_scipy_rotations():
+    """framepos / framequat / magnetometer of a site: composition of the body's pose with the site's, checked with scipy."""
+    from scipy.spatial.transform import Rotation
+
+    rng = np.random.default_rng(21)
+    for _ in range(5):
+        qb, qs = rng.normal(size=4), rng.normal(size=4)
+        qb, qs = qb / np.linalg.norm(qb), qs / np.linalg.norm(qs)
+        xb, r, field = rng.normal(size=3), rng.normal(size=3), rng.normal(size=3)
+        Rb, Rs = Rotation.from_quat(qb[[1, 2, 3, 0]]), Rotation.from_quat(qs[[1, 2, 3, 0]])
+        np.testing.assert_allclose(ot.site_frame_position(xb, qb, r), xb + Rb.apply(r), atol=1e-12)
+        want = (Rb * Rs).as_quat()[[3, 0, 1, 2]]
+        got = ot.site_frame_quaternion(qb, qs)
+        assert min(np.abs(got - want).max(), np.abs(got + want).max()) < 1e-12
+        np.testing.assert_allclose(ot.site_magnetometer(qb, qs, field), (Rb * Rs).inv().apply(field), atol=1e-12)
