@@ -148,7 +148,7 @@ def main() -> None:
         print(json.dumps({"policy_mlp": mlp_rate(torch, rows=(args.mlp_rows,) if args.mlp_rows else (8192, 524288))}))
         return
     if args.only == "gae":
-        print(json.dumps({"gae": gae_bandwidth(torch, ppo)}))
+        print(json.dumps({"gae": gae_bandwidth(torch, ppo), "streaming": loss_and_reward_bandwidth(torch)}))
         return
     if args.only == "update":
         print(json.dumps({"ppo_update": ppo_update_rate(torch)}))
@@ -200,6 +200,7 @@ def main() -> None:
 
     # GAE on rotating cfg-2 sized buffers (T=128, N=4096): larger than the caches in total
     gae = gae_bandwidth(torch, ppo)
+    streaming = loss_and_reward_bandwidth(torch)
     mlp = mlp_rate(torch)
     upd = ppo_update_rate(torch)
     iteration = ppo_iteration_rate(torch)
@@ -245,7 +246,7 @@ def main() -> None:
                              "cycles with a VALU instruction issuing is given beside); the HBM fraction is reported "
                              "against the bytes the engine contract obliges a step to move"},
         "other_integrator": other_entry, "single_stream": single_entry,
-        "gae": gae, "policy_mlp": mlp, "ppo_update": upd, "ppo_iteration": iteration, "graph_replay": graph,
+        "gae": gae, "streaming": streaming, "policy_mlp": mlp, "ppo_update": upd, "ppo_iteration": iteration, "graph_replay": graph,
     }
     if not args.no_cpu_baseline:
         base = cpu_baseline(args.integrator)
@@ -386,6 +387,72 @@ def gae_bandwidth(torch, ppo, reps=8):
         out[name] = {"layout": "(T,N) fp32, dones and successes int8", "ms_per_call": ms,
                      "achieved_GBps": nbytes / (ms * 1e-3) / 1e9, "frac_of_hbm_peak": nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
                      "algorithmic_bytes": nbytes, "buffer_sets": sets}
+    return out
+
+
+def loss_and_reward_bandwidth(torch, reps=8, sets=16):
+    """The other two streaming kernels of cfg 2 (T=128, N=4096) through the C ABI on rotating buffer sets: the per-element PPO
+    loss terms with their mean, and the reward sum with the done / success reduction over the termination components."""
+    import ctypes
+    from ksim_amd import _lib
+
+    lib = _lib.load()
+    n, A, K, k = 4096 * 128, 1, 8, 4
+    g = torch.Generator(device="cuda")
+    g.manual_seed(1002)
+    rn = lambda *shape: torch.randn(*shape, device="cuda", generator=g)  # noqa: E731
+    st = _lib.current_stream()
+    out = {}
+
+    def timed(run, bufs):
+        for b in bufs[:2]:
+            run(*b)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            for b in bufs:
+                run(*b)
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / (reps * len(bufs))
+
+    # PPO loss: reads advantages, targets, on / off log-probabilities and values, entropy (7 floats at A = 1); writes the
+    # policy / value / KL / entropy terms per element (the reference returns them per element, ppo.py:447-492) and their mean
+    params = _lib.KsPpoLossParams(0.2, 0.5, 0.008, 1e-3, 5.0, 1.0, 1)
+    ws = torch.empty(1 << 16, dtype=torch.uint8, device="cuda")
+    res = [torch.empty(n, device="cuda") for _ in range(4)]
+    total = torch.empty((), device="cuda")
+    bufs = []
+    for _ in range(sets):
+        on_lp = rn(n, A)
+        bufs.append((rn(n), rn(n), on_lp, rn(n), on_lp + 0.05 * rn(n, A), rn(n), rn(n, A)))
+
+    def run_loss(adv, tgt, on_lp, on_v, off_lp, off_v, ent):
+        _lib.check(lib.ks_ppo_loss(st, n, A, params, _lib.ptr(adv), _lib.ptr(tgt), _lib.ptr(on_lp), _lib.ptr(on_v), _lib.ptr(off_lp),
+                                   _lib.ptr(off_v), _lib.ptr(ent), _lib.ptr(res[0]), _lib.ptr(res[1]), _lib.ptr(res[2]), _lib.ptr(res[3]),
+                                   _lib.ptr(total), _lib.ptr(ws)))
+
+    ms = timed(run_loss, bufs)
+    nbytes = n * 4 * (4 + 3 * A + 4)
+    out["ppo_loss_cfg2"] = {"ms_per_call": ms, "achieved_GBps": nbytes / (ms * 1e-3) / 1e9, "frac_of_hbm_peak": nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                            "algorithmic_bytes": nbytes, "bytes_per_element": 4 * (4 + 3 * A + 4), "buffer_sets": sets}
+    del bufs
+
+    # reward total + done / success: K reward components (f32) and k termination components (int8) per element
+    scales = (ctypes.c_float * K)(*[0.5 + 0.1 * i for i in range(K)])
+    tot, done, succ = torch.empty(n, device="cuda"), torch.empty(n, dtype=torch.uint8, device="cuda"), torch.empty(n, dtype=torch.uint8, device="cuda")
+    bufs = [(rn(K, n), (torch.randint(-1, 2, (k, n), device="cuda", generator=g) * (torch.rand(k, n, device="cuda", generator=g) < 0.01)).to(torch.int8))
+            for _ in range(sets)]
+
+    def run_reward(comp, term):
+        _lib.check(lib.ks_reward_total(st, n, K, _lib.ptr(comp), scales, 1, -5.0, 1, 5.0, _lib.ptr(tot), k, _lib.ptr(term), _lib.ptr(done), _lib.ptr(succ)))
+
+    ms = timed(run_reward, bufs)
+    nbytes = n * (4 * K + k + 6)
+    out["reward_total_cfg2"] = {"ms_per_call": ms, "achieved_GBps": nbytes / (ms * 1e-3) / 1e9, "frac_of_hbm_peak": nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                                "algorithmic_bytes": nbytes, "bytes_per_element": 4 * K + k + 6, "reward_components": K, "termination_components": k,
+                                "buffer_sets": sets}
     return out
 
 
