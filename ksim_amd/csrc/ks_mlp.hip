@@ -828,6 +828,69 @@ __global__ __launch_bounds__(256) void refresh_kernel(int npad, int kpad, const 
   }
 }
 
+// One optimiser step of a whole network in one launch: every weight and bias element goes through the chain of adam_kernel,
+// and the thread that updates a master weight also writes its working copies (W, W^T, the fragment-ordered copy of the
+// whole-network kernel), as refresh_kernel does; the thread of a layer's element o < npad updates bias o as well.  The same
+// arithmetic per element as the per-tensor launches, which it replaces (two dozen launches and copies per network).
+struct AdamNetArgs {
+  int n_layers;
+  int npad[KS_MAX_LAYERS], kpad[KS_MAX_LAYERS], fk[KS_MAX_LAYERS], fn[KS_MAX_LAYERS], frozen[KS_MAX_LAYERS];
+  int first_block[KS_MAX_LAYERS + 1];  // workgroups [first_block[l], first_block[l + 1]) belong to layer l
+  float *mW[KS_MAX_LAYERS], *m1W[KS_MAX_LAYERS], *m2W[KS_MAX_LAYERS], *mb[KS_MAX_LAYERS], *m1b[KS_MAX_LAYERS], *m2b[KS_MAX_LAYERS];
+  const float *gW[KS_MAX_LAYERS], *gb[KS_MAX_LAYERS];
+  void *W[KS_MAX_LAYERS], *Wt[KS_MAX_LAYERS];
+  __bf16* Wp[KS_MAX_LAYERS];
+  float *b[KS_MAX_LAYERS], *bp[KS_MAX_LAYERS];
+};
+
+__device__ __forceinline__ float adam_element(float p, float g, float& m1, float& m2, const KsAdamParams& a, const double* sqnorm) {
+  float gv = g;
+  if (!(gv == gv)) gv = 0.f;                                       // zero_nans
+  if (a.max_grad_norm > 0.f && sqnorm) {                           // clip_by_global_norm
+    const float norm = (float)sqrt(*sqnorm);
+    if (norm > a.max_grad_norm) gv = gv / norm * a.max_grad_norm;
+  }
+  gv += a.weight_decay * p;                                        // add_decayed_weights
+  m1 = a.b1 * m1 + (1.f - a.b1) * gv;                              // scale_by_adam
+  m2 = a.b2 * m2 + (1.f - a.b2) * gv * gv;
+  const float mhat = m1 / (1.f - powf(a.b1, (float)a.step));
+  const float vhat = m2 / (1.f - powf(a.b2, (float)a.step));
+  return p - a.lr * mhat / (sqrtf(vhat) + a.eps);
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void adam_net_kernel(AdamNetArgs n, KsAdamParams a, const double* __restrict__ sqnorm) {
+  int l = 0;
+  while (l + 1 < n.n_layers && (int)blockIdx.x >= n.first_block[l + 1]) ++l;
+  const int npad = n.npad[l], kpad = n.kpad[l];
+  const int64_t idx = (int64_t)(blockIdx.x - n.first_block[l]) * 256 + threadIdx.x;
+  if (idx < (int64_t)npad * kpad) {
+    float m1 = n.m1W[l][idx], m2 = n.m2W[l][idx];
+    const float v = adam_element(n.mW[l][idx], n.gW[l][idx], m1, m2, a, sqnorm);
+    n.m1W[l][idx] = m1; n.m2W[l][idx] = m2; n.mW[l][idx] = v;
+    const int o = (int)(idx / kpad), i = (int)(idx - (int64_t)o * kpad);
+    reinterpret_cast<T*>(n.W[l])[idx] = from_f32<T>(v);
+    if (n.Wt[l]) reinterpret_cast<T*>(n.Wt[l])[(int64_t)i * npad + o] = from_f32<T>(v);
+    // [tile o / 32][k step i / 16][lane (o % 32) + 32 ((i % 16) / 8)][i % 8].  The fragment copy is padded to 32 outputs and 16
+    // inputs, the master to the coarser tiles of the per-layer kernel: master entries beyond the fragment copy are padding
+    // (zero weights with zero gradients) and have no place in it.
+    if (n.Wp[l] && o < n.fn[l] * 32 && i < n.fk[l] * 16) {
+      const int64_t at = ((((int64_t)(o >> 5) * n.fk[l] + (i >> 4)) * 64 + (o & 31) + 32 * ((i >> 3) & 1)) << 3) + (i & 7);
+      n.Wp[l][at] = (__bf16)v;
+    }
+  }
+  if (idx < npad) {
+    float v = n.mb[l][idx];
+    if (idx >= n.frozen[l]) {
+      float m1 = n.m1b[l][idx], m2 = n.m2b[l][idx];
+      v = adam_element(v, n.gb[l][idx], m1, m2, a, sqnorm);
+      n.m1b[l][idx] = m1; n.m2b[l][idx] = m2; n.mb[l][idx] = v;
+    }
+    n.b[l][idx] = v;
+    if (n.bp[l] && idx < n.fn[l] * 32) n.bp[l][idx] = v;
+  }
+}
+
 static inline int round_up(int x, int m) { return (x + m - 1) / m * m; }
 
 static uint16_t f32_to_bf16_rne(float f) {
@@ -1486,16 +1549,21 @@ extern "C" int ks_mlp_adam_step(KsMlp* h, ks_stream_t stream, const KsAdamParams
   if (rc != KS_OK) return rc;
   DevMlp& m = h->m;
   hipStream_t s = (hipStream_t)stream;
+  AdamNetArgs n{};
+  n.n_layers = m.n_layers;
+  int blocks = 0;
   for (int l = 0; l < m.n_layers; ++l) {
-    const int64_t n = (int64_t)m.npad[l] * m.kpad[l], nb = m.npad[l];
-    hipLaunchKernelGGL(adam_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, n, m.mW[l], m.gW[l], m.m1W[l], m.m2W[l], *p, sqnorm);
-    const int fz = m.bias_frozen[l];
-    if (nb > fz)
-      hipLaunchKernelGGL(adam_kernel, dim3((unsigned)((nb - fz + 255) / 256)), dim3(256), 0, s, nb - fz, m.mb[l] + fz, m.gb[l] + fz,
-                         m.m1b[l] + fz, m.m2b[l] + fz, *p, sqnorm);
+    n.npad[l] = m.npad[l]; n.kpad[l] = m.kpad[l]; n.fk[l] = m.fk[l]; n.fn[l] = m.fn[l]; n.frozen[l] = m.bias_frozen[l];
+    n.first_block[l] = blocks;
+    blocks += (int)(((int64_t)m.npad[l] * m.kpad[l] + 255) / 256);  // npad * kpad >= npad: the bias rides on the first threads
+    n.mW[l] = m.mW[l]; n.m1W[l] = m.m1W[l]; n.m2W[l] = m.m2W[l]; n.gW[l] = m.gW[l];
+    n.mb[l] = m.mb[l]; n.m1b[l] = m.m1b[l]; n.m2b[l] = m.m2b[l]; n.gb[l] = m.gb[l];
+    n.W[l] = m.W[l]; n.Wt[l] = m.Wt[l]; n.Wp[l] = m.fused ? (__bf16*)m.Wp[l] : nullptr;
+    n.b[l] = m.b[l]; n.bp[l] = m.fused ? m.bp[l] : nullptr;
   }
-  if (m.dtype == KS_MLP_BF16) refresh_layers<__bf16>(m, s);
-  else refresh_layers<float>(m, s);
+  n.first_block[m.n_layers] = blocks;
+  if (m.dtype == KS_MLP_BF16) hipLaunchKernelGGL(adam_net_kernel<__bf16>, dim3((unsigned)blocks), dim3(256), 0, s, n, *p, sqnorm);
+  else hipLaunchKernelGGL(adam_net_kernel<float>, dim3((unsigned)blocks), dim3(256), 0, s, n, *p, sqnorm);
   return check_launch("ks_mlp_adam_step");
 }
 

@@ -150,6 +150,34 @@ def test_adam_chain_kernel_matches_optax_restatement():
     np.testing.assert_allclose(m1.cpu().numpy(), o1[0], rtol=1e-5, atol=1e-8)
 
 
+@pytest.mark.parametrize("dims,dtype", [((68, 512, 512, 20), "bf16"), ((71, 256, 21), "f32"), ((30, 64, 1), "bf16")])
+def test_optimiser_step_refreshes_every_working_copy(dims, dtype):
+    """After an optimiser step both forward paths (the whole-network kernel with its fragment-ordered weights, the training
+    forward over the per-layer copies) and the input gradient (the transposed copies) are those of a network built afresh
+    from the updated master parameters, bit for bit; widths that are not multiples of the kernels' tiles included."""
+    from ksim_amd import _lib_terms as T
+    from ksim_amd.mlp import MLP, random_mlp
+
+    rng = np.random.default_rng(6)
+    net, _, _ = random_mlp(dims, 3, dtype=dtype)
+    net.train_init()
+    M = 300
+    x, dy = t32(rng.normal(size=(M, dims[0]))), t32(rng.normal(size=(M, dims[-1])))
+    for step in (1, 2):
+        net.train_forward(x)
+        net.backward(x, dy)
+        net.adam_step(T.KsAdamParams(1e-2, 0.9, 0.999, 1e-8, 0.01, 0.0, step), None)
+    fresh = MLP([w for w, _ in net.parameters()], [b for _, b in net.parameters()], dtype=dtype)
+    fresh.train_init()
+    assert all((b != 0).any() for _, b in net.parameters())  # the biases moved too
+    assert torch.equal(net(x), fresh(x))
+    assert torch.equal(net.train_forward(x), fresh.train_forward(x))
+    dx_a, dx_b = torch.zeros_like(x), torch.zeros_like(x)
+    net.backward_dx(x, dy, dx_a, weight_gradients=False)
+    fresh.backward_dx(x, dy, dx_b, weight_gradients=False)
+    assert torch.equal(dx_a, dx_b)
+
+
 def _setup(seed, Tn, N, od, A, hidden):
     from ksim_amd.mlp import MLP
     from ksim_amd.ppo_update import GaussianMlpPolicy
