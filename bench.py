@@ -357,6 +357,23 @@ def gae_bandwidth(torch, ppo, reps=8):
         out[name] = {"layout": "(B,T) fp32, dones int8", "ms_per_call": ms, "achieved_GBps": nbytes / (ms * 1e-3) / 1e9,
                      "frac_of_hbm_peak": nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "algorithmic_bytes": nbytes,
                      "buffer_sets": sets}
+    # yardstick for cfg 2: a plain copy kernel that moves the same 11 MB per call (half read, half written), on buffers
+    # rotated the same way; what it reaches is what a single launch of this size can reach on this machine
+    n_copy = 4096 * 128 * 21 // 8
+    cb = [(torch.randn(n_copy, device="cuda"), torch.empty(n_copy, device="cuda")) for _ in range(32)]
+    for a, b in cb[:2]:
+        _lib.check(lib.ks_copy_f32(_lib.current_stream(), n_copy, _lib.ptr(a), _lib.ptr(b)))
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        for a, b in cb:
+            _lib.check(lib.ks_copy_f32(_lib.current_stream(), n_copy, _lib.ptr(a), _lib.ptr(b)))
+    e1.record()
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / (reps * len(cb))
+    out["cfg2_T128_N4096"]["plain_copy_of_the_same_bytes"] = {"ms_per_call": ms, "achieved_GBps": n_copy * 8 / (ms * 1e-3) / 1e9}
+    del cb
     # the rollout's own layout (T, N), with the success flags it carries: cfg 4 / cfg 5 shapes and a large one
     for name, N, T, sets in (("rollout_T32_N8192", 8192, 32, 64), ("rollout_T32_N16384", 16384, 32, 32),
                              ("large_T128_N65536_tn", 65536, 128, 4)):
