@@ -169,6 +169,37 @@ def UniformGaussianRandomVariable(mean: float, std: float, mag: float) -> Random
     return RandomVariable(mean=mean, mag=mag, std=std, same_key=True)
 
 
+def _kind_of(rv: RandomVariable, additive: bool) -> tuple[int, float, float, float]:
+    """(kind, mean, scale, scale2) of `observation (+ | *) rv` for the kernels' noise stages."""
+    if rv.std and rv.mag:
+        if not rv.same_key:
+            raise ValueError("a normal and a uniform part are drawn with one key (UniformGaussianRandomVariable, noise.py:106-121)")
+        return (T.NOISE_ADD_UNIFORM_GAUSSIAN if additive else T.NOISE_MUL_UNIFORM_GAUSSIAN), rv.mean, rv.std, rv.mag
+    if rv.mag:
+        return (T.NOISE_ADD_UNIFORM if additive else T.NOISE_MUL_UNIFORM), rv.mean, rv.mag, 0.0
+    return (T.NOISE_ADD_GAUSSIAN if additive else T.NOISE_MUL_GAUSSIAN), rv.mean, rv.std, 0.0  # a zero variable: the mean alone
+
+
+class AdditiveNoise(Noise):  # noise.py:184-187: observation + random variable, over any of the random variables above
+    def __init__(self, random_variable: RandomVariable) -> None:
+        super().__init__(*_kind_of(random_variable, True))
+
+
+class MultiplicativeNoise(Noise):  # noise.py:190-193
+    def __init__(self, random_variable: RandomVariable) -> None:
+        super().__init__(*_kind_of(random_variable, False))
+
+
+class AdditiveBias(Bias):  # noise.py:135-138
+    def __init__(self, random_variable: RandomVariable) -> None:
+        super().__init__(*_kind_of(random_variable, True))
+
+
+class MultiplicativeBias(Bias):  # noise.py:141-144
+    def __init__(self, random_variable: RandomVariable) -> None:
+        super().__init__(*_kind_of(random_variable, False))
+
+
 def convert_to_noise(noise) -> Noise | None:
     """A float means additive Gaussian noise of that std (ksim/observation.py:69-76)."""
     if noise is None or isinstance(noise, Noise):

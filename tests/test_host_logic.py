@@ -444,3 +444,19 @@ def test_mjcf_contact_dimension_follows_mujocos_rule(tmp_path):
     path.write_text(robot(4, 1))
     with pytest.raises(ValueError, match="condim"):
         load_mjcf(str(path))
+
+
+def test_generic_noise_and_bias_over_random_variables():
+    """AdditiveNoise / MultiplicativeNoise / AdditiveBias / MultiplicativeBias over a random variable (ksim/noise.py:129-193)
+    are the named convenience classes' stages."""
+    from ksim_amd import noise as kn
+
+    same = lambda a, b: (a.kind, a.mean, a.scale, a.scale2) == (b.kind, b.mean, b.scale, b.scale2)  # noqa: E731
+    assert same(kn.AdditiveNoise(kn.GaussianRandomVariable(0.1, 0.3)), kn.AdditiveGaussianNoise(std=0.3, mean=0.1))
+    assert same(kn.MultiplicativeNoise(kn.UniformRandomVariable(1.0, 0.2)), kn.MultiplicativeUniformNoise(mag=0.2))
+    assert same(kn.AdditiveNoise(kn.UniformGaussianRandomVariable(0.0, 0.3, 0.4)), kn.AdditiveUniformGaussianNoise(std=0.3, mag=0.4))
+    assert same(kn.MultiplicativeBias(kn.GaussianRandomVariable(1.0, 0.05)), kn.MultiplicativeGaussianBias(std=0.05))
+    assert same(kn.AdditiveBias(kn.UniformRandomVariable(0.0, 0.5)), kn.AdditiveUniformBias(mag=0.5))
+    assert isinstance(kn.AdditiveBias(kn.ZeroRandomVariable()), kn.Bias) and kn.AdditiveNoise(kn.ZeroRandomVariable()).scale == 0.0
+    with pytest.raises(ValueError, match="one key"):
+        kn.AdditiveNoise(kn.RandomVariable(mean=0.0, mag=0.1, std=0.1, same_key=False))
