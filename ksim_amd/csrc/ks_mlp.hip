@@ -238,6 +238,12 @@ struct FusedArgs {
   // training forward: hidden layer l's activations also go to save[l], (M, save_ld[l]) bf16 row-major, for the backward pass
   __bf16* save[KS_MAX_LAYERS];
   int save_ld[KS_MAX_LAYERS];
+  // training forward for the whole-network backward kernel: hidden layer l's activations in the accumulator order of the
+  // wavefronts that produced them (keep[l]: per 128-row tile [wavefront][feature tile 0..1][row tile][g][lane] x 8 bytes, so the
+  // backward kernel's epilogue reads its own entries with one 8-byte load per lane) and transposed (keep_t[l]: (width, ldt))
+  uint2* keep[KS_MAX_LAYERS];
+  __bf16* keep_t[KS_MAX_LAYERS];
+  int64_t ldt;
 };
 
 #ifdef KS_PROFILE
@@ -323,14 +329,45 @@ __device__ __forceinline__ void fused_bias_init(f32x16& acc, const float* __rest
 // Hidden layer: activation, round to bf16, back into the tile (4 consecutive features = one 8-byte LDS store).
 template <int ACT>
 __device__ __forceinline__ void fused_store_hidden(const f32x16& acc, __bf16* __restrict__ act, int lda, int j,
-                                                   int row, int lane) {
+                                                   int row, int lane, uint2* __restrict__ keep = nullptr) {
 #pragma unroll
   for (int g = 0; g < 4; ++g) {
     const int f0 = j * 32 + 8 * g + 4 * (lane >> 5);
     const uint2 packed = {pack_bf16(activate<ACT, true>(acc[4 * g]), activate<ACT, true>(acc[4 * g + 1])),
                           pack_bf16(activate<ACT, true>(acc[4 * g + 2]), activate<ACT, true>(acc[4 * g + 3]))};
     *reinterpret_cast<uint2*>(act + row * lda + f0) = packed;
+    if (keep) keep[g * 64 + lane] = packed;  // the same four values, in accumulator order
   }
+}
+
+// Entries of one 128-row tile in an accumulator-order buffer: [wavefront][feature tile 0..1][row tile 0..3][g][lane]
+constexpr int kKeepPerTile = kFusedWaves * 2 * 4 * 4 * 64;
+__device__ __forceinline__ int64_t keep_index(int64_t tile, int wave, int t, int i) {
+  return tile * kKeepPerTile + (((wave * 2 + t) * 4 + i) * 4) * 64;
+}
+
+// The finished 128-row tile, transposed, to dst (width, ld): thread p takes the columns 2 p and 2 p + 1 of the tile (one
+// 4-byte LDS read per row), 8 rows per 16-byte store (a run of 256 bytes per column and tile), and returns the columns' sums.
+__device__ __forceinline__ f32x2 tile_transposed_out(const __bf16* __restrict__ act, int lda, int p, __bf16* __restrict__ dst, int64_t ld,
+                                                     int64_t m0) {
+  f32x2 s = {0.f, 0.f};
+  __bf16* out0 = dst + (int64_t)(2 * p) * ld + m0;
+  __bf16* out1 = out0 + ld;
+#pragma unroll 2
+  for (int r0 = 0; r0 < 128; r0 += 8) {
+    bf16x2 v[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) v[k] = *reinterpret_cast<const bf16x2*>(act + (r0 + k) * lda + 2 * p);
+    __bf16 a[8], b[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      a[k] = v[k][0]; b[k] = v[k][1];
+      s[0] += (float)a[k]; s[1] += (float)b[k];
+    }
+    *reinterpret_cast<uint4*>(out0 + r0) = *reinterpret_cast<const uint4*>(a);
+    *reinterpret_cast<uint4*>(out1 + r0) = *reinterpret_cast<const uint4*>(b);
+  }
+  return s;
 }
 
 // Output layer: fp32 rows of the caller's (M, out_dim) matrix.
@@ -354,7 +391,7 @@ __device__ __forceinline__ void fused_store_output(const f32x16& acc, float* __r
 // One layer of the whole-network kernel for one wavefront: MFMA work, barrier, epilogue, barrier.
 template <int ACT, int MI, bool LAST>
 __device__ __forceinline__ void fused_layer(const FusedArgs& a, int l, __bf16* __restrict__ act, int64_t m0, int lane,
-                                            int wave) {
+                                            int wave, int64_t tile) {
   const int nk = a.fk[l], nt = a.fn[l], lda = a.lda;
   const __bf16* arow = act + (lane & 31) * lda + (lane >> 5) * 8;
   const int row = lane & 31;
@@ -398,12 +435,15 @@ __device__ __forceinline__ void fused_layer(const FusedArgs& a, int l, __bf16* _
 #pragma unroll
         for (int i = 0; i < MI; ++i) {
           if (LAST) fused_store_output(acc[t][i], a.y, a.M, a.out_dim, j, m0 + i * 32 + row, lane);
-          else fused_store_hidden<ACT>(acc[t][i], act, lda, j, i * 32 + row, lane);
+          else fused_store_hidden<ACT>(acc[t][i], act, lda, j, i * 32 + row, lane,
+                                       (MI == 4 && a.keep[l]) ? a.keep[l] + keep_index(tile, wave, t, i) : nullptr);
         }
       }
   }
   __syncthreads();
   KS_MLP_STAMP2(4 + 3 * l)
+  if (!LAST && MI == 4 && a.keep_t[l] && (int)threadIdx.x < nt * 16)
+    (void)tile_transposed_out(act, lda, (int)threadIdx.x, a.keep_t[l], a.ldt, m0);
   if (!LAST && a.save[l]) {
     // the finished tile, 16 bytes per thread and pass, rows as contiguous runs; the next layer only reads the tile until every
     // wavefront (this copy included, which sits before its matrix work in program order) has passed the next barrier
@@ -483,9 +523,9 @@ __device__ __forceinline__ void mlp_fused_body(const FusedArgs& a, int64_t tile)
   __syncthreads();
   KS_MLP_STAMP(1)
   for (int l = 0; l + 1 < a.n_layers; ++l) {
-    fused_layer<ACT, MI, false>(a, l, act, m0, lane, wave);
+    fused_layer<ACT, MI, false>(a, l, act, m0, lane, wave, tile);
   }
-  fused_layer<ACT, MI, true>(a, a.n_layers - 1, act, m0, lane, wave);
+  fused_layer<ACT, MI, true>(a, a.n_layers - 1, act, m0, lane, wave, tile);
 }
 
 template <int ACT, int BM>
@@ -513,6 +553,97 @@ void mlp_fused_pair_kernel(const FusedArgs a, const FusedArgs b) {
   else mlp_fused_body<ACT, BM>(b, tile);
 }
 
+// ---------------------------------------------------------------- whole-network backward pass of the hidden layers
+// dZ_{l-1} = (dZ_l W_l) * f'(Y_{l-1}) for l = L-1 .. 1 in one launch, a 128-row tile per workgroup that never leaves LDS: the
+// product is the forward kernel's K loop over the fragment-ordered transposed weights, its epilogue reads the stored
+// activations in accumulator order (FusedArgs::keep), and after each layer the tile goes out transposed (the operand of the
+// weight-gradient product) together with its column sums (the bias gradient, one partial row per tile).
+struct FusedBwdArgs {
+  int64_t M;
+  int n_layers, lda, ld_last;
+  int fk[KS_MAX_LAYERS], fn[KS_MAX_LAYERS];   // the forward kernel's K steps and output tiles per layer
+  const u32x4* WtP[KS_MAX_LAYERS];            // l >= 1: W_l^T in fragment order, [input tile][step over outputs][lane] x 16 bytes
+  const __bf16* dz_last;                      // (M, ld_last): gradient of the last layer's pre-activation, zero in the padding
+  const uint2* keep[KS_MAX_LAYERS];           // hidden layer l's activations in accumulator order
+  __bf16* dzT[KS_MAX_LAYERS];                 // out, l = 0 .. L-2: dZ_l^T (width, ldt)
+  float* bias_part[KS_MAX_LAYERS];            // out, l = 0 .. L-2: (tiles, width) column sums of dZ_l per tile
+  int64_t ldt;
+};
+
+template <int ACT>
+__global__ __launch_bounds__(64 * kFusedWaves) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void mlp_fused_bwd_kernel(const FusedBwdArgs a) {
+  constexpr int MI = 4, BM = 128, NTHR = 64 * kFusedWaves;
+  extern __shared__ __attribute__((aligned(16))) unsigned char mlp_lds[];
+  __bf16* act = reinterpret_cast<__bf16*>(mlp_lds);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int64_t tile = blockIdx.x, m0 = tile * BM;
+  const int lda = a.lda, L = a.n_layers;
+  {  // the last layer's gradient tile; rows beyond the batch are zero and stay zero through every layer
+    const int w8 = a.fn[L - 1] * 4;  // 16-byte pieces per row
+    for (int idx = tid; idx < BM * w8; idx += NTHR) {
+      const int r = idx / w8, c8 = idx - r * w8;
+      uint4 v = {0u, 0u, 0u, 0u};
+      if (m0 + r < a.M) v = *reinterpret_cast<const uint4*>(a.dz_last + (m0 + r) * a.ld_last + c8 * 8);
+      *reinterpret_cast<uint4*>(act + r * lda + c8 * 8) = v;
+    }
+  }
+  __syncthreads();
+  const __bf16* arow = act + (lane & 31) * lda + (lane >> 5) * 8;
+  const int row = lane & 31;
+  for (int l = L - 1; l >= 1; --l) {
+    const int nk = a.fn[l] * 2;  // K steps over layer l's outputs
+    const int nt = a.fk[l] / 2;  // 32-wide tiles over layer l - 1's outputs
+    const int mine = wave < nt ? (wave + kFusedWaves < nt ? 2 : 1) : 0;
+    const int j0 = wave < nt ? wave : 0, j1 = wave + kFusedWaves < nt ? wave + kFusedWaves : j0;
+    f32x16 acc[2][MI];
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int i = 0; i < MI; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[t][i][r] = 0.f;
+    const u32x4* w0 = a.WtP[l] + (int64_t)j0 * nk * 64 + lane;
+    const u32x4* w1 = a.WtP[l] + (int64_t)j1 * nk * 64 + lane;
+    if (mine == 2) fused_layer_mma<2, MI, kPF>(acc, w0, w1, nk, arow, lda);
+    else if (mine == 1) fused_layer_mma<1, MI, kPF>(acc, w0, w0, nk, arow, lda);
+    __syncthreads();  // every wavefront has read dZ_l; the tile can take dZ_{l-1}
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+      if (t < mine) {
+        const int j = t == 0 ? j0 : j1;
+#pragma unroll
+        for (int i = 0; i < MI; ++i) {
+          const uint2* y = a.keep[l - 1] + keep_index(tile, wave, t, i);
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            const uint2 yy = y[g * 64 + lane];
+            const float yv[4] = {__builtin_bit_cast(float, yy.x << 16), __builtin_bit_cast(float, yy.x & 0xffff0000u),
+                                 __builtin_bit_cast(float, yy.y << 16), __builtin_bit_cast(float, yy.y & 0xffff0000u)};
+            float d[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              d[e] = 1.f;
+              if (ACT == KS_ACT_ELU) d[e] = yv[e] > 0.f ? 1.f : yv[e] + 1.f;
+              if (ACT == KS_ACT_RELU) d[e] = yv[e] > 0.f ? 1.f : 0.f;
+              if (ACT == KS_ACT_TANH) d[e] = 1.f - yv[e] * yv[e];
+              d[e] *= acc[t][i][4 * g + e];
+            }
+            const int f0 = j * 32 + 8 * g + 4 * (lane >> 5);
+            *reinterpret_cast<uint2*>(act + (i * 32 + row) * lda + f0) = uint2{pack_bf16(d[0], d[1]), pack_bf16(d[2], d[3])};
+          }
+        }
+      }
+    __syncthreads();
+    if (tid < nt * 16) {  // the next layer's K loop only reads the tile, as this does
+      const f32x2 cs = tile_transposed_out(act, lda, tid, a.dzT[l - 1], a.ldt, m0);
+      float* part = a.bias_part[l - 1] + tile * (nt * 32) + 2 * tid;
+      part[0] = cs[0];
+      part[1] = cs[1];
+    }
+  }
+}
+
 struct DevMlp {
   int n_layers, activation, dtype;
   int dims[KS_MAX_LAYERS + 1];
@@ -534,6 +665,8 @@ struct DevMlp {
   float *gW[KS_MAX_LAYERS], *gb[KS_MAX_LAYERS];
   float *m1W[KS_MAX_LAYERS], *m2W[KS_MAX_LAYERS], *m1b[KS_MAX_LAYERS], *m2b[KS_MAX_LAYERS];
   void* Wt[KS_MAX_LAYERS];      // (kpad, npad) working-precision transpose
+  void* WtP[KS_MAX_LAYERS];     // l >= 1, whole-network kernel only: W_l^T in fragment order, for the whole-network backward pass
+  int chain_saved;              // the last training forward kept the activations in the whole-network backward pass's formats
   int bias_frozen[KS_MAX_LAYERS];  // leading bias entries of the layer that the optimiser leaves alone
   float* zero_bias;             // zeros, as wide as the widest GEMM output
   double* sq_part;              // kSqBlocks partial sums of squares per gradient tensor (weights and biases of every layer)
@@ -811,7 +944,8 @@ __global__ __launch_bounds__(256) void adam_kernel(int64_t n, float* __restrict_
 // the fragment-ordered copy [tile][k step][lane][8]
 template <typename T>
 __global__ __launch_bounds__(256) void refresh_kernel(int npad, int kpad, const float* __restrict__ mW, T* __restrict__ W,
-                                                      T* __restrict__ Wt, __bf16* __restrict__ Wp, int fk, int fn) {
+                                                      T* __restrict__ Wt, __bf16* __restrict__ Wp, int fk, int fn,
+                                                      __bf16* __restrict__ WtP) {
   const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (idx < (int64_t)npad * kpad) {
     const int o = (int)(idx / kpad), i = (int)(idx - (int64_t)o * kpad);
@@ -826,6 +960,13 @@ __global__ __launch_bounds__(256) void refresh_kernel(int npad, int kpad, const 
     const int o = j * 32 + (lane & 31), i = st * 16 + (lane >> 5) * 8 + e;
     Wp[idx] = (__bf16)((o < npad && i < kpad) ? mW[(int64_t)o * kpad + i] : 0.f);
   }
+  if (WtP && idx < (int64_t)fn * fk * 64 * 8) {  // the transposed roles: tiles over the inputs, 2 fn steps over the outputs
+    const int e = (int)(idx & 7), lane = (int)((idx >> 3) & 63);
+    const int64_t js = idx >> 9;
+    const int st = (int)(js % (2 * fn)), j = (int)(js / (2 * fn));
+    const int i = j * 32 + (lane & 31), o = st * 16 + (lane >> 5) * 8 + e;
+    WtP[idx] = (__bf16)((o < npad && i < kpad) ? mW[(int64_t)o * kpad + i] : 0.f);
+  }
 }
 
 // One optimiser step of a whole network in one launch: every weight and bias element goes through the chain of adam_kernel,
@@ -839,7 +980,7 @@ struct AdamNetArgs {
   float *mW[KS_MAX_LAYERS], *m1W[KS_MAX_LAYERS], *m2W[KS_MAX_LAYERS], *mb[KS_MAX_LAYERS], *m1b[KS_MAX_LAYERS], *m2b[KS_MAX_LAYERS];
   const float *gW[KS_MAX_LAYERS], *gb[KS_MAX_LAYERS];
   void *W[KS_MAX_LAYERS], *Wt[KS_MAX_LAYERS];
-  __bf16* Wp[KS_MAX_LAYERS];
+  __bf16 *Wp[KS_MAX_LAYERS], *WtP[KS_MAX_LAYERS];
   float *b[KS_MAX_LAYERS], *bp[KS_MAX_LAYERS];
 };
 
@@ -877,6 +1018,10 @@ __global__ __launch_bounds__(256) void adam_net_kernel(AdamNetArgs n, KsAdamPara
     if (n.Wp[l] && o < n.fn[l] * 32 && i < n.fk[l] * 16) {
       const int64_t at = ((((int64_t)(o >> 5) * n.fk[l] + (i >> 4)) * 64 + (o & 31) + 32 * ((i >> 3) & 1)) << 3) + (i & 7);
       n.Wp[l][at] = (__bf16)v;
+      if (n.WtP[l]) {  // the same entry with the roles of input and output exchanged
+        const int64_t att = ((((int64_t)(i >> 5) * (2 * n.fn[l]) + (o >> 4)) * 64 + (i & 31) + 32 * ((o >> 3) & 1)) << 3) + (o & 7);
+        n.WtP[l][att] = (__bf16)v;
+      }
     }
   }
   if (idx < npad) {
@@ -1037,6 +1182,7 @@ extern "C" int ks_mlp_destroy(KsMlp* h) {
     for (float* q : t)
       if (q) (void)hipFree(q);
     if (h->m.Wt[l]) (void)hipFree(h->m.Wt[l]);
+    if (h->m.WtP[l]) (void)hipFree(h->m.WtP[l]);
   }
   if (h->m.zero_bias) (void)hipFree(h->m.zero_bias);
   if (h->m.sq_part) (void)hipFree(h->m.sq_part);
@@ -1056,14 +1202,19 @@ static FusedArgs fused_args(const DevMlp& m, int64_t M, const float* x, float* y
   return a;
 }
 
+struct TrainWs;
+static void keep_args(FusedArgs& a, const DevMlp& m, const TrainWs* ws);
+
 template <int BM>
-static int launch_fused_tile(const DevMlp& m, hipStream_t s, int64_t M, const float* x, float* y, char* const* save) {
+static int launch_fused_tile(const DevMlp& m, hipStream_t s, int64_t M, const float* x, float* y, char* const* save,
+                             const TrainWs* keep = nullptr) {
   FusedArgs a = fused_args(m, M, x, y);
   if (save)
     for (int l = 0; l + 1 < m.n_layers; ++l) {
       a.save[l] = (__bf16*)save[l];
       a.save_ld[l] = m.npad[l];
     }
+  if (keep) keep_args(a, m, keep);
 #ifdef KS_PROFILE
   if (const char* e = getenv("KS_MLP_PROF_PTR")) a.prof = (long long*)strtoull(e, nullptr, 16);
 #endif
@@ -1220,6 +1371,8 @@ extern "C" int ks_mlp_train_init(KsMlp* h) {
       }
       if (m.Wt[l]) (void)hipFree(m.Wt[l]);
       m.Wt[l] = nullptr;
+      if (m.WtP[l]) (void)hipFree(m.WtP[l]);
+      m.WtP[l] = nullptr;
     }
     if (m.zero_bias) (void)hipFree(m.zero_bias);
     if (m.sq_part) (void)hipFree(m.sq_part);
@@ -1249,6 +1402,10 @@ extern "C" int ks_mlp_train_init(KsMlp* h) {
     const size_t nt = l == 0 ? (size_t)round_up(m.kpad[0], kBN) * m.npad[0] : n;
     if (hipMalloc(&m.Wt[l], nt * esz) != hipSuccess || hipMemset(m.Wt[l], 0, nt * esz) != hipSuccess)
       return give_up("allocation");
+    if (m.fused && l >= 1) {  // as many fragments as the forward copy: (fk / 2) tiles of inputs x (2 fn) steps over outputs
+      const size_t np = (size_t)m.fn[l] * m.fk[l] * 512 * 2;
+      if (hipMalloc(&m.WtP[l], np) != hipSuccess || hipMemset(m.WtP[l], 0, np) != hipSuccess) return give_up("allocation");
+    }
   }
   const int wz = widest_pad(m);
   if (hipMalloc((void**)&m.zero_bias, (size_t)wz * 4) != hipSuccess || hipMemset(m.zero_bias, 0, (size_t)wz * 4) != hipSuccess)
@@ -1270,7 +1427,7 @@ static void refresh_layers(DevMlp& m, hipStream_t s) {
     const int64_t np = m.fused ? (int64_t)m.fn[l] * m.fk[l] * 512 : 0;
     const int64_t tot = n > np ? n : np;
     hipLaunchKernelGGL(refresh_kernel<T>, dim3((unsigned)((tot + 255) / 256)), dim3(256), 0, s, m.npad[l], m.kpad[l], m.mW[l],
-                       (T*)m.W[l], (T*)m.Wt[l], m.fused ? (__bf16*)m.Wp[l] : (__bf16*)nullptr, m.fk[l], m.fn[l]);
+                       (T*)m.W[l], (T*)m.Wt[l], m.fused ? (__bf16*)m.Wp[l] : (__bf16*)nullptr, m.fk[l], m.fn[l], (__bf16*)m.WtP[l]);
     (void)hipMemcpyAsync(m.b[l], m.mb[l], (size_t)m.npad[l] * 4, hipMemcpyDeviceToDevice, s);
     if (m.fused) (void)hipMemcpyAsync(m.bp[l], m.mb[l], (size_t)m.fn[l] * 32 * 4, hipMemcpyDeviceToDevice, s);
   }
@@ -1285,7 +1442,22 @@ struct TrainWs {
   char *d0, *d1, *t0, *t1, *t2;
   float* part;  // partial sums of the split reductions
   int64_t Mp;
+  // whole-network backward pass (chain_ok): per hidden layer the activations in accumulator order and transposed, per layer
+  // dZ^T, per hidden layer one row of bias partial sums per 128-row tile; all transposes have the row stride Mp128
+  char *yacc[KS_MAX_LAYERS], *yT[KS_MAX_LAYERS], *dzT[KS_MAX_LAYERS];
+  float* bpart[KS_MAX_LAYERS];
+  int64_t Mp128;
 };
+
+// Whether a batch of M rows goes through the whole-network backward pass: bf16 networks that run the whole-network forward
+// kernel on 128-row tiles, with hidden layers wide enough that every wavefront owns whole feature tiles of all four row tiles
+// (the accumulator-order copy of the activations is laid out for that split).
+static bool chain_ok(const DevMlp& m, int64_t M) {
+  if (!m.fused || m.dtype != KS_MLP_BF16 || m.activation == KS_ACT_GELU || m.n_layers < 2 || M < 128 * 256) return false;
+  for (int l = 0; l + 1 < m.n_layers; ++l)
+    if (m.npad[l] != m.fn[l] * 32 || m.fn[l] * 4 <= kFusedWaves || !m.WtP[l + 1]) return false;
+  return true;
+}
 static int64_t carve_train(const DevMlp& m, int64_t M, char* base, TrainWs* ws) {
   const int64_t esz = m.dtype == KS_MLP_BF16 ? 2 : 4;
   const int64_t Mp = (M + 63) / 64 * 64;
@@ -1311,8 +1483,27 @@ static int64_t carve_train(const DevMlp& m, int64_t M, char* base, TrainWs* ws) 
   const int64_t nparts = kDwSplit * maxw > (int64_t)4 * kColsumSlices * wz ? kDwSplit * maxw : (int64_t)4 * kColsumSlices * wz;
   w.part = (float*)take(nparts * 4);
   w.Mp = Mp;
+  w.Mp128 = (M + 127) / 128 * 128;
+  if (chain_ok(m, M)) {
+    const int64_t tiles = w.Mp128 / 128;
+    for (int l = 0; l + 1 < m.n_layers; ++l) {
+      w.yacc[l] = take(tiles * kKeepPerTile * 8);
+      w.yT[l] = take((int64_t)m.npad[l] * w.Mp128 * esz);
+      w.bpart[l] = (float*)take(tiles * m.npad[l] * 4);
+    }
+    for (int l = 0; l < m.n_layers; ++l) w.dzT[l] = take((int64_t)m.npad[l] * w.Mp128 * esz);
+    w.yT[m.n_layers - 1] = take((int64_t)round_up(m.kpad[0], kBN) * w.Mp128 * esz);  // the network input, transposed
+  }
   if (ws) *ws = w;
   return off;
+}
+
+static void keep_args(FusedArgs& a, const DevMlp& m, const TrainWs* ws) {
+  for (int l = 0; l + 1 < m.n_layers; ++l) {
+    a.keep[l] = (uint2*)ws->yacc[l];
+    a.keep_t[l] = (__bf16*)ws->yT[l];
+  }
+  a.ldt = ws->Mp128;
 }
 
 extern "C" int64_t ks_mlp_train_workspace_bytes(const KsMlp* h, int64_t M) {
@@ -1326,6 +1517,11 @@ static int train_forward(DevMlp& m, hipStream_t s, int64_t M, const float* x, fl
   // pass as well; the stored rows must have the width the backward pass expects (its padding is in units of 64, the kernel's 32)
   bool whole = m.fused && m.dtype == KS_MLP_BF16 && m.activation != KS_ACT_GELU;
   for (int l = 0; whole && l + 1 < m.n_layers; ++l) whole = m.npad[l] == m.fn[l] * 32;
+  m.chain_saved = 0;
+  if (whole && chain_ok(m, M)) {  // activations in the formats of the whole-network backward pass, not row-major
+    m.chain_saved = 1;
+    return launch_fused_tile<128>(m, s, M, x, y, nullptr, &ws);
+  }
   if (whole) return launch_fused(m, s, M, x, y, ws.act);
   const void* in = x;
   int64_t ldin = m.dims[0];
@@ -1363,11 +1559,96 @@ extern "C" int ks_mlp_train_forward(KsMlp* h, ks_stream_t stream, int64_t M, con
   return rc != KS_OK ? rc : check_launch("ks_mlp_train_forward");
 }
 
+// The backward pass of a network whose forward kept the whole-network formats (chain_ok): the last layer's gradient by the small
+// kernels, every hidden layer's in one launch of mlp_fused_bwd_kernel, then one weight-gradient product per layer.
+template <typename T>
+static int train_backward_chain(DevMlp& m, hipStream_t s, int64_t M, const float* x, const float* dy, const TrainWs& ws) {
+  const int L = m.n_layers;
+  const int64_t Mp = ws.Mp128, tiles = Mp / 128;
+  T* dz = (T*)ws.d0;
+  const int npl = m.npad[L - 1];
+  {
+    const int64_t n = M * npl;
+    hipLaunchKernelGGL(cast_pad_kernel<T>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, M, m.dims[L], npl, dy, dz);
+    const int nz = 4 * kColsumSlices;
+    hipLaunchKernelGGL(colsum_kernel<T>, dim3((unsigned)((npl + 63) / 64), nz), dim3(256), 0, s, M, npl, dz, ws.part);
+    hipLaunchKernelGGL(sum_parts_tree_kernel, dim3((unsigned)npl), dim3(64), 0, s, (int64_t)npl, nz, ws.part, m.gb[L - 1]);
+    hipLaunchKernelGGL((transpose_kernel<T, T>), dim3((unsigned)((Mp + 31) / 32), (unsigned)((npl + 31) / 32)), dim3(256), 0, s, M, npl,
+                       (int64_t)npl, dz, npl, Mp, (T*)ws.dzT[L - 1]);
+  }
+  {
+    FusedBwdArgs a;
+    std::memset(&a, 0, sizeof(a));
+    a.M = M; a.n_layers = L; a.lda = m.lda; a.ld_last = npl; a.ldt = Mp;
+    a.dz_last = (const __bf16*)dz;
+    for (int l = 0; l < L; ++l) {
+      a.fk[l] = m.fk[l]; a.fn[l] = m.fn[l];
+      a.WtP[l] = (const u32x4*)m.WtP[l];
+      if (l + 1 < L) {
+        a.keep[l] = (const uint2*)ws.yacc[l];
+        a.dzT[l] = (__bf16*)ws.dzT[l];
+        a.bias_part[l] = ws.bpart[l];
+      }
+    }
+    const int lds = 128 * m.lda * 2;
+#define KS_LAUNCH(A)                                                                                           \
+  {                                                                                                            \
+    auto kfn = mlp_fused_bwd_kernel<A>;                                                                        \
+    if (lds > 64 * 1024 &&                                                                                     \
+        hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)  \
+      return fail(KS_ELAUNCH, "ks_mlp_train_backward: cannot raise the LDS limit to %d bytes", lds);           \
+    hipLaunchKernelGGL(kfn, dim3((unsigned)tiles), dim3(64 * kFusedWaves), lds, s, a);                         \
+  }
+    switch (m.activation) {
+      case KS_ACT_ELU: KS_LAUNCH(KS_ACT_ELU) break;
+      case KS_ACT_RELU: KS_LAUNCH(KS_ACT_RELU) break;
+      case KS_ACT_TANH: KS_LAUNCH(KS_ACT_TANH) break;
+      default: KS_LAUNCH(KS_ACT_NONE) break;
+    }
+#undef KS_LAUNCH
+  }
+  for (int l = 0; l + 1 < L; ++l)
+    hipLaunchKernelGGL(sum_parts_tree_kernel, dim3((unsigned)m.npad[l]), dim3(64), 0, s, (int64_t)m.npad[l], (int)tiles, ws.bpart[l], m.gb[l]);
+  const int kp128_0 = round_up(m.kpad[0], kBN);
+  T* xT = (T*)ws.yT[L - 1];
+  hipLaunchKernelGGL((transpose_kernel<float, T>), dim3((unsigned)((Mp + 31) / 32), (unsigned)((kp128_0 + 31) / 32)), dim3(256), 0, s, M,
+                     m.dims[0], (int64_t)m.dims[0], x, kp128_0, Mp, xT);
+  for (int l = L - 1; l >= 0; --l) {
+    const int np = m.npad[l], kp = m.kpad[l], kp128 = round_up(kp, kBN);
+    const T* dzT = (const T*)ws.dzT[l];
+    const T* yT = l > 0 ? (const T*)ws.yT[l - 1] : xT;
+    const bool wide = np % 128 == 0;
+    int ksplit = wide ? kDwSplit : kDwSplit / 2;
+    while (ksplit > 1 && (Mp / 64) % ksplit != 0) ksplit >>= 1;
+    int rc;
+    if (wide)
+      rc = launch_layer_tile<T, false, true, 128, 128, 2, 2>(KS_ACT_NONE, s, np, kp128, (int)Mp, (int)Mp, kp, dzT, Mp, yT, m.zero_bias,
+                                                              ksplit > 1 ? (void*)ws.part : (void*)m.gW[l], kp, ksplit);
+    else
+      rc = launch_layer_tile<T, false, true, 64, 128, 2, 2>(KS_ACT_NONE, s, np, kp128, (int)Mp, (int)Mp, kp, dzT, Mp, yT, m.zero_bias,
+                                                             ksplit > 1 ? (void*)ws.part : (void*)m.gW[l], kp, ksplit);
+    if (rc != KS_OK) return rc;
+    if (ksplit > 1) {
+      const int64_t n = (int64_t)np * kp;
+      hipLaunchKernelGGL(sum_parts_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, n, ksplit, ws.part, m.gW[l]);
+    }
+  }
+  return KS_OK;
+}
+
 template <typename T>
 static int train_backward(DevMlp& m, hipStream_t s, int64_t M, const float* x, const float* dy, const TrainWs& ws,
                           float* dx = nullptr, bool want_w = true, bool accumulate_dx = false, const uint8_t* zero_rows = nullptr) {
   const int L = m.n_layers;
   const int64_t Mp = ws.Mp;
+  if (m.chain_saved && sizeof(T) == 2) {
+    if (want_w && !dx) return train_backward_chain<T>(m, s, M, x, dy, ws);
+    // the layer-by-layer pass below reads row-major activations: rebuild them from the transposed copies
+    for (int l = 0; l + 1 < L; ++l)
+      hipLaunchKernelGGL((transpose_kernel<T, T>), dim3((unsigned)((m.npad[l] + 31) / 32), (unsigned)((M + 31) / 32)), dim3(256), 0, s,
+                         (int64_t)m.npad[l], (int)M, ws.Mp128, (const T*)ws.yT[l], (int)M, (int64_t)m.npad[l], (T*)ws.act[l]);
+    m.chain_saved = 0;
+  }
   T* dz = (T*)ws.d0;
   T* dnext = (T*)ws.d1;
   {  // the output gradient in working precision, padded to the last layer's width
@@ -1558,7 +1839,7 @@ extern "C" int ks_mlp_adam_step(KsMlp* h, ks_stream_t stream, const KsAdamParams
     blocks += (int)(((int64_t)m.npad[l] * m.kpad[l] + 255) / 256);  // npad * kpad >= npad: the bias rides on the first threads
     n.mW[l] = m.mW[l]; n.m1W[l] = m.m1W[l]; n.m2W[l] = m.m2W[l]; n.gW[l] = m.gW[l];
     n.mb[l] = m.mb[l]; n.m1b[l] = m.m1b[l]; n.m2b[l] = m.m2b[l]; n.gb[l] = m.gb[l];
-    n.W[l] = m.W[l]; n.Wt[l] = m.Wt[l]; n.Wp[l] = m.fused ? (__bf16*)m.Wp[l] : nullptr;
+    n.W[l] = m.W[l]; n.Wt[l] = m.Wt[l]; n.Wp[l] = m.fused ? (__bf16*)m.Wp[l] : nullptr; n.WtP[l] = (__bf16*)m.WtP[l];
     n.b[l] = m.b[l]; n.bp[l] = m.fused ? m.bp[l] : nullptr;
   }
   n.first_block[m.n_layers] = blocks;

@@ -150,6 +150,49 @@ def test_adam_chain_kernel_matches_optax_restatement():
     np.testing.assert_allclose(m1.cpu().numpy(), o1[0], rtol=1e-5, atol=1e-8)
 
 
+@pytest.mark.parametrize("dims,act,M", [((68, 512, 512, 512, 20), "elu", 33000), ((40, 128, 256, 1), "tanh", 32768),
+                                        ((68, 512, 512, 20), "relu", 40001)])
+def test_whole_network_backward_pass_at_large_batches(dims, act, M):
+    """Batches of 32768 rows and more of a bf16 network go through the whole-network backward kernel (hidden-layer gradients in
+    one launch, activations kept in accumulator order and transposed).  Its gradients against float64 reverse-mode
+    differentiation, and against the layer-by-layer pass, which the same call takes when the input gradient is asked for
+    (it rebuilds the row-major activations from the transposed copies); batch sizes that are not multiples of the tile."""
+    from ksim_amd.mlp import MLP
+
+    rng = np.random.default_rng(sum(dims) + M)
+    ws = [rng.normal(scale=1 / np.sqrt(i), size=(o, i)).astype(np.float32) for i, o in zip(dims[:-1], dims[1:])]
+    bs = [rng.normal(scale=0.1, size=o).astype(np.float32) for o in dims[1:]]
+    x = rng.normal(size=(M, dims[0])).astype(np.float32)
+    dy = (rng.normal(size=(M, dims[-1])) / M).astype(np.float32)
+    net = MLP(ws, bs, activation=act, dtype="bf16")
+    net.train_init()
+    xd, dyd = t32(x), t32(dy)
+    y = net.train_forward(xd)
+    net.backward(xd, dyd)
+    chain = [(w.clone(), b.clone()) for w, b in net.parameters(gradients=True)]
+    tw = [torch.tensor(w, dtype=torch.float64, requires_grad=True) for w in ws]
+    tb = [torch.tensor(b, dtype=torch.float64, requires_grad=True) for b in bs]
+    yo = ou.mlp(torch.tensor(x, dtype=torch.float64), tw, tb, act)
+    (yo * torch.tensor(dy, dtype=torch.float64)).sum().backward()
+    assert rel(y.cpu().numpy(), yo.detach().numpy()) < 1e-2
+    tol = 1e-1 if act == "relu" else 3e-2  # a bf16-rounded pre-activation next to zero switches the step of a ReLU's derivative
+    for (gw, gb), w, b in zip(chain, tw, tb):
+        assert rel(gw.cpu().numpy(), w.grad.numpy()) < tol
+        assert rel(gb.cpu().numpy(), b.grad.numpy()) < tol
+    # the layer-by-layer pass on the same stored activations
+    y2 = net.train_forward(xd)
+    assert torch.equal(y, y2)
+    dx = torch.zeros_like(xd)
+    net.backward_dx(xd, dyd, dx)
+    for (gw, gb), (cw, cb) in zip(net.parameters(gradients=True), chain):
+        assert rel(gw.cpu().numpy(), cw.cpu().numpy().astype(np.float64)) < 1e-2
+        assert rel(gb.cpu().numpy(), cb.cpu().numpy().astype(np.float64)) < 1e-2
+    tx = torch.tensor(x, dtype=torch.float64, requires_grad=True)
+    (ou.mlp(tx, [w.detach() for w in tw], [b.detach() for b in tb], act) * torch.tensor(dy, dtype=torch.float64)).sum().backward()
+    if act != "relu":  # a single row's input gradient has no sum over the batch to average a switched step out
+        assert rel(dx.cpu().numpy(), tx.grad.numpy()) < tol
+
+
 @pytest.mark.parametrize("dims,dtype", [((68, 512, 512, 20), "bf16"), ((71, 256, 21), "f32"), ((30, 64, 1), "bf16")])
 def test_optimiser_step_refreshes_every_working_copy(dims, dtype):
     """After an optimiser step both forward paths (the whole-network kernel with its fragment-ordered weights, the training
