@@ -389,7 +389,7 @@ __device__ __forceinline__ void fused_store_output(const f32x16& acc, float* __r
 }
 
 // One layer of the whole-network kernel for one wavefront: MFMA work, barrier, epilogue, barrier.
-template <int ACT, int MI, bool LAST>
+template <int ACT, int MI, bool LAST, bool KEEP>
 __device__ __forceinline__ void fused_layer(const FusedArgs& a, int l, __bf16* __restrict__ act, int64_t m0, int lane,
                                             int wave, int64_t tile) {
   const int nk = a.fk[l], nt = a.fn[l], lda = a.lda;
@@ -436,13 +436,13 @@ __device__ __forceinline__ void fused_layer(const FusedArgs& a, int l, __bf16* _
         for (int i = 0; i < MI; ++i) {
           if (LAST) fused_store_output(acc[t][i], a.y, a.M, a.out_dim, j, m0 + i * 32 + row, lane);
           else fused_store_hidden<ACT>(acc[t][i], act, lda, j, i * 32 + row, lane,
-                                       (MI == 4 && a.keep[l]) ? a.keep[l] + keep_index(tile, wave, t, i) : nullptr);
+                                       (KEEP && MI == 4) ? a.keep[l] + keep_index(tile, wave, t, i) : nullptr);
         }
       }
   }
   __syncthreads();
   KS_MLP_STAMP2(4 + 3 * l)
-  if (!LAST && MI == 4 && a.keep_t[l] && (int)threadIdx.x < nt * 16)
+  if (KEEP && !LAST && MI == 4 && (int)threadIdx.x < nt * 16)
     (void)tile_transposed_out(act, lda, (int)threadIdx.x, a.keep_t[l], a.ldt, m0);
   if (!LAST && a.save[l]) {
     // the finished tile, 16 bytes per thread and pass, rows as contiguous runs; the next layer only reads the tile until every
@@ -457,7 +457,7 @@ __device__ __forceinline__ void fused_layer(const FusedArgs& a, int l, __bf16* _
   }
 }
 
-template <int ACT, int BM>
+template <int ACT, int BM, bool KEEP = false>
 __device__ __forceinline__ void mlp_fused_body(const FusedArgs& a, int64_t tile) {
   constexpr int MI = BM / 32;
   constexpr int NTHR = 64 * kFusedWaves;
@@ -523,15 +523,17 @@ __device__ __forceinline__ void mlp_fused_body(const FusedArgs& a, int64_t tile)
   __syncthreads();
   KS_MLP_STAMP(1)
   for (int l = 0; l + 1 < a.n_layers; ++l) {
-    fused_layer<ACT, MI, false>(a, l, act, m0, lane, wave, tile);
+    fused_layer<ACT, MI, false, KEEP>(a, l, act, m0, lane, wave, tile);
   }
-  fused_layer<ACT, MI, true>(a, a.n_layers - 1, act, m0, lane, wave, tile);
+  fused_layer<ACT, MI, true, KEEP>(a, a.n_layers - 1, act, m0, lane, wave, tile);
 }
 
-template <int ACT, int BM>
+// KEEP: the training forward that stores every hidden layer's activations in accumulator order and transposed (FusedArgs::keep,
+// keep_t; 128-row tiles only)
+template <int ACT, int BM, bool KEEP = false>
 __global__ __launch_bounds__(64 * kFusedWaves) __attribute__((amdgpu_waves_per_eu(BM <= 64 ? 4 : 2, BM <= 64 ? 4 : 2)))
 void mlp_fused_kernel(const FusedArgs a) {
-  mlp_fused_body<ACT, BM>(a, blockIdx.x);
+  mlp_fused_body<ACT, BM, KEEP>(a, blockIdx.x);
 }
 
 // Two networks over the same rows in one launch (actor and critic of a control step): blockIdx.y picks the network, so
@@ -1223,7 +1225,7 @@ static int launch_fused_tile(const DevMlp& m, hipStream_t s, int64_t M, const fl
   if (blocks > 0x7fffffff) return fail(KS_ELIMIT, "ks_mlp_forward: too many rows");
 #define KS_LAUNCH(A)                                                                                           \
   {                                                                                                            \
-    auto kfn = mlp_fused_kernel<A, BM>;                                                                        \
+    auto kfn = (keep && BM == 128) ? mlp_fused_kernel<A, BM, BM == 128> : mlp_fused_kernel<A, BM, false>;      \
     if (lds > 64 * 1024 &&                                                                                     \
         hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)  \
       return fail(KS_ELAUNCH, "ks_mlp_forward: cannot raise the LDS limit to %d bytes", lds);                  \
