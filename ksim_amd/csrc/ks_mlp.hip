@@ -243,6 +243,8 @@ struct FusedArgs {
   // backward kernel's epilogue reads its own entries with one 8-byte load per lane) and transposed (keep_t[l]: (width, ldt))
   uint2* keep[KS_MAX_LAYERS];
   __bf16* keep_t[KS_MAX_LAYERS];
+  __bf16* keep_t_in;  // the network input, transposed: (in_t_width, ldt), zero beyond the real inputs
+  int in_t_width;
   int64_t ldt;
 };
 
@@ -468,7 +470,8 @@ __device__ __forceinline__ void mlp_fused_body(const FusedArgs& a, int64_t tile)
   const int lda = a.lda;
   KS_MLP_STAMP(0)
   {  // network input -> bf16 tile; zero beyond the batch and in the K padding of the first layer
-    const int K0 = a.fk[0] * 16, in_dim = a.in_dim;
+    const int in_dim = a.in_dim;
+    const int K0 = (KEEP && a.in_t_width > a.fk[0] * 16) ? a.in_t_width : a.fk[0] * 16;  // the transposed copy is padded further
     const int64_t rows_left = a.M - m0;
     const int rows = rows_left < BM ? (int)rows_left : BM;
     const float* src = a.x + m0 * in_dim;
@@ -522,6 +525,8 @@ __device__ __forceinline__ void mlp_fused_body(const FusedArgs& a, int64_t tile)
   }
   __syncthreads();
   KS_MLP_STAMP(1)
+  if (KEEP && BM == 128 && a.keep_t_in && tid < a.in_t_width / 2)  // the first layer overwrites the tile only after its barrier
+    (void)tile_transposed_out(act, lda, tid, a.keep_t_in, a.ldt, m0);
   for (int l = 0; l + 1 < a.n_layers; ++l) {
     fused_layer<ACT, MI, false, KEEP>(a, l, act, m0, lane, wave, tile);
   }
@@ -565,10 +570,11 @@ struct FusedBwdArgs {
   int n_layers, lda, ld_last;
   int fk[KS_MAX_LAYERS], fn[KS_MAX_LAYERS];   // the forward kernel's K steps and output tiles per layer
   const u32x4* WtP[KS_MAX_LAYERS];            // l >= 1: W_l^T in fragment order, [input tile][step over outputs][lane] x 16 bytes
-  const __bf16* dz_last;                      // (M, ld_last): gradient of the last layer's pre-activation, zero in the padding
+  const float* dy;                            // (M, out_dim): gradient of the network output, in the caller's layout
+  int out_dim, np_last;                       // np_last: rows of dzT[L-1] (the output width padded for the weight-gradient product)
   const uint2* keep[KS_MAX_LAYERS];           // hidden layer l's activations in accumulator order
-  __bf16* dzT[KS_MAX_LAYERS];                 // out, l = 0 .. L-2: dZ_l^T (width, ldt)
-  float* bias_part[KS_MAX_LAYERS];            // out, l = 0 .. L-2: (tiles, width) column sums of dZ_l per tile
+  __bf16* dzT[KS_MAX_LAYERS];                 // out, every layer: dZ_l^T (width, ldt)
+  float* bias_part[KS_MAX_LAYERS];            // out, every layer: (tiles, width) column sums of dZ_l per tile
   int64_t ldt;
 };
 
@@ -581,16 +587,21 @@ void mlp_fused_bwd_kernel(const FusedBwdArgs a) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int64_t tile = blockIdx.x, m0 = tile * BM;
   const int lda = a.lda, L = a.n_layers;
-  {  // the last layer's gradient tile; rows beyond the batch are zero and stay zero through every layer
-    const int w8 = a.fn[L - 1] * 4;  // 16-byte pieces per row
-    for (int idx = tid; idx < BM * w8; idx += NTHR) {
-      const int r = idx / w8, c8 = idx - r * w8;
-      uint4 v = {0u, 0u, 0u, 0u};
-      if (m0 + r < a.M) v = *reinterpret_cast<const uint4*>(a.dz_last + (m0 + r) * a.ld_last + c8 * 8);
-      *reinterpret_cast<uint4*>(act + r * lda + c8 * 8) = v;
+  {  // the last layer's gradient tile from the caller's fp32 rows; zero in the padding columns and beyond the batch (such rows
+     // stay zero through every layer)
+    const int np = a.np_last, od = a.out_dim;
+    for (int idx = tid; idx < BM * np; idx += NTHR) {
+      const int r = idx / np, c = idx - r * np;
+      act[r * lda + c] = (__bf16)((c < od && m0 + r < a.M) ? a.dy[(m0 + r) * od + c] : 0.f);
     }
   }
   __syncthreads();
+  if (tid < a.np_last / 2) {  // its transpose and column sums; the first K loop below only reads the tile
+    const f32x2 cs = tile_transposed_out(act, lda, tid, a.dzT[L - 1], a.ldt, m0);
+    float* part = a.bias_part[L - 1] + tile * a.np_last + 2 * tid;
+    part[0] = cs[0];
+    part[1] = cs[1];
+  }
   const __bf16* arow = act + (lane & 31) * lda + (lane >> 5) * 8;
   const int row = lane & 31;
   for (int l = L - 1; l >= 1; --l) {
@@ -1458,6 +1469,8 @@ static bool chain_ok(const DevMlp& m, int64_t M) {
   if (!m.fused || m.dtype != KS_MLP_BF16 || m.activation == KS_ACT_GELU || m.n_layers < 2 || M < 128 * 256) return false;
   for (int l = 0; l + 1 < m.n_layers; ++l)
     if (m.npad[l] != m.fn[l] * 32 || m.fn[l] * 4 <= kFusedWaves || !m.WtP[l + 1]) return false;
+  // the transposed copies of the input and of the output gradient are cut from the LDS tile at their padded widths
+  if (round_up(m.kpad[0], kBN) + 8 > m.lda || m.npad[m.n_layers - 1] + 8 > m.lda) return false;
   return true;
 }
 static int64_t carve_train(const DevMlp& m, int64_t M, char* base, TrainWs* ws) {
@@ -1494,6 +1507,7 @@ static int64_t carve_train(const DevMlp& m, int64_t M, char* base, TrainWs* ws) 
       w.bpart[l] = (float*)take(tiles * m.npad[l] * 4);
     }
     for (int l = 0; l < m.n_layers; ++l) w.dzT[l] = take((int64_t)m.npad[l] * w.Mp128 * esz);
+    w.bpart[m.n_layers - 1] = (float*)take(tiles * m.npad[m.n_layers - 1] * 4);
     w.yT[m.n_layers - 1] = take((int64_t)round_up(m.kpad[0], kBN) * w.Mp128 * esz);  // the network input, transposed
   }
   if (ws) *ws = w;
@@ -1505,6 +1519,8 @@ static void keep_args(FusedArgs& a, const DevMlp& m, const TrainWs* ws) {
     a.keep[l] = (uint2*)ws->yacc[l];
     a.keep_t[l] = (__bf16*)ws->yT[l];
   }
+  a.keep_t_in = (__bf16*)ws->yT[m.n_layers - 1];
+  a.in_t_width = round_up(m.kpad[0], kBN);
   a.ldt = ws->Mp128;
 }
 
@@ -1567,30 +1583,18 @@ template <typename T>
 static int train_backward_chain(DevMlp& m, hipStream_t s, int64_t M, const float* x, const float* dy, const TrainWs& ws) {
   const int L = m.n_layers;
   const int64_t Mp = ws.Mp128, tiles = Mp / 128;
-  T* dz = (T*)ws.d0;
   const int npl = m.npad[L - 1];
-  {
-    const int64_t n = M * npl;
-    hipLaunchKernelGGL(cast_pad_kernel<T>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, M, m.dims[L], npl, dy, dz);
-    const int nz = 4 * kColsumSlices;
-    hipLaunchKernelGGL(colsum_kernel<T>, dim3((unsigned)((npl + 63) / 64), nz), dim3(256), 0, s, M, npl, dz, ws.part);
-    hipLaunchKernelGGL(sum_parts_tree_kernel, dim3((unsigned)npl), dim3(64), 0, s, (int64_t)npl, nz, ws.part, m.gb[L - 1]);
-    hipLaunchKernelGGL((transpose_kernel<T, T>), dim3((unsigned)((Mp + 31) / 32), (unsigned)((npl + 31) / 32)), dim3(256), 0, s, M, npl,
-                       (int64_t)npl, dz, npl, Mp, (T*)ws.dzT[L - 1]);
-  }
   {
     FusedBwdArgs a;
     std::memset(&a, 0, sizeof(a));
-    a.M = M; a.n_layers = L; a.lda = m.lda; a.ld_last = npl; a.ldt = Mp;
-    a.dz_last = (const __bf16*)dz;
+    a.M = M; a.n_layers = L; a.lda = m.lda; a.ldt = Mp;
+    a.dy = dy; a.out_dim = m.dims[L]; a.np_last = npl;
     for (int l = 0; l < L; ++l) {
       a.fk[l] = m.fk[l]; a.fn[l] = m.fn[l];
       a.WtP[l] = (const u32x4*)m.WtP[l];
-      if (l + 1 < L) {
-        a.keep[l] = (const uint2*)ws.yacc[l];
-        a.dzT[l] = (__bf16*)ws.dzT[l];
-        a.bias_part[l] = ws.bpart[l];
-      }
+      if (l + 1 < L) a.keep[l] = (const uint2*)ws.yacc[l];
+      a.dzT[l] = (__bf16*)ws.dzT[l];
+      a.bias_part[l] = ws.bpart[l];
     }
     const int lds = 128 * m.lda * 2;
 #define KS_LAUNCH(A)                                                                                           \
@@ -1609,12 +1613,10 @@ static int train_backward_chain(DevMlp& m, hipStream_t s, int64_t M, const float
     }
 #undef KS_LAUNCH
   }
-  for (int l = 0; l + 1 < L; ++l)
+  for (int l = 0; l < L; ++l)
     hipLaunchKernelGGL(sum_parts_tree_kernel, dim3((unsigned)m.npad[l]), dim3(64), 0, s, (int64_t)m.npad[l], (int)tiles, ws.bpart[l], m.gb[l]);
-  const int kp128_0 = round_up(m.kpad[0], kBN);
-  T* xT = (T*)ws.yT[L - 1];
-  hipLaunchKernelGGL((transpose_kernel<float, T>), dim3((unsigned)((Mp + 31) / 32), (unsigned)((kp128_0 + 31) / 32)), dim3(256), 0, s, M,
-                     m.dims[0], (int64_t)m.dims[0], x, kp128_0, Mp, xT);
+  (void)x;  // the training forward left its transpose behind
+  const T* xT = (const T*)ws.yT[L - 1];
   for (int l = L - 1; l >= 0; --l) {
     const int np = m.npad[l], kp = m.kpad[l], kp128 = round_up(kp, kBN);
     const T* dzT = (const T*)ws.dzT[l];
