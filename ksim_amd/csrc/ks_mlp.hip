@@ -879,6 +879,41 @@ __global__ __launch_bounds__(256) void sum_parts_kernel(int64_t n, int nz, const
   out[i] = s;
 }
 
+// Every gradient of a network from its partial sums, in one launch (the whole-network backward pass): weight gradient l =
+// the sum of its nz[l] row slices, z ascending as in sum_parts_kernel; bias gradient l = the sum over the row tiles of the
+// per-tile column sums, four columns per workgroup with one wavefront each and the fixed tree of sum_parts_tree_kernel.
+struct GradFinishArgs {
+  int n_layers, tiles;
+  int nz[KS_MAX_LAYERS], nb[KS_MAX_LAYERS];
+  int64_t nW[KS_MAX_LAYERS];
+  int first_w[KS_MAX_LAYERS + 1], first_b[KS_MAX_LAYERS + 1];  // workgroups of the weights, then of the biases, per layer
+  const float *wpart[KS_MAX_LAYERS], *bpart[KS_MAX_LAYERS];
+  float *gW[KS_MAX_LAYERS], *gb[KS_MAX_LAYERS];
+};
+__global__ __launch_bounds__(256) void grad_finish_kernel(GradFinishArgs a) {
+  const int b = blockIdx.x;
+  if (b < a.first_w[a.n_layers]) {
+    int l = 0;
+    while (l + 1 < a.n_layers && b >= a.first_w[l + 1]) ++l;
+    const int64_t i = (int64_t)(b - a.first_w[l]) * 256 + threadIdx.x, n = a.nW[l];
+    if (i >= n) return;
+    float s = 0.f;
+    for (int z = 0; z < a.nz[l]; ++z) s += a.wpart[l][(int64_t)z * n + i];
+    a.gW[l][i] = s;
+    return;
+  }
+  const int bb = b - a.first_w[a.n_layers];
+  int l = 0;
+  while (l + 1 < a.n_layers && bb >= a.first_b[l + 1]) ++l;
+  const int c = (bb - a.first_b[l]) * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63, n = a.nb[l];
+  if (c >= n) return;
+  float s = 0.f;
+  for (int z = lane; z < a.tiles; z += 64) s += a.bpart[l][(int64_t)z * n + c];
+  for (int w = 32; w > 0; w >>= 1) s += __shfl_down(s, w);  // lane k adds lane k + w: the same tree for every column
+  if (lane == 0) a.gb[l][c] = s;
+}
+
+
 // Sum of squares of gradient buffers, NaNs counted as zero (the optimiser zeroes them first), added to *acc in double.
 // Every addition happens in a fixed order (a strided pass per lane, a tree over the lanes, then the partial sums one after
 // the other), so the clip factor, and with it a whole update, is the same bits on every run.
@@ -1458,7 +1493,7 @@ struct TrainWs {
   // whole-network backward pass (chain_ok): per hidden layer the activations in accumulator order and transposed, per layer
   // dZ^T, per hidden layer one row of bias partial sums per 128-row tile; all transposes have the row stride Mp128
   char *yacc[KS_MAX_LAYERS], *yT[KS_MAX_LAYERS], *dzT[KS_MAX_LAYERS];
-  float* bpart[KS_MAX_LAYERS];
+  float *bpart[KS_MAX_LAYERS], *wpart[KS_MAX_LAYERS];  // wpart: the row slices of each layer's weight-gradient product
   int64_t Mp128;
 };
 
@@ -1508,6 +1543,7 @@ static int64_t carve_train(const DevMlp& m, int64_t M, char* base, TrainWs* ws) 
     }
     for (int l = 0; l < m.n_layers; ++l) w.dzT[l] = take((int64_t)m.npad[l] * w.Mp128 * esz);
     w.bpart[m.n_layers - 1] = (float*)take(tiles * m.npad[m.n_layers - 1] * 4);
+    for (int l = 0; l < m.n_layers; ++l) w.wpart[l] = (float*)take((int64_t)kDwSplit * m.npad[l] * m.kpad[l] * 4);
     w.yT[m.n_layers - 1] = take((int64_t)round_up(m.kpad[0], kBN) * w.Mp128 * esz);  // the network input, transposed
   }
   if (ws) *ws = w;
@@ -1613,10 +1649,12 @@ static int train_backward_chain(DevMlp& m, hipStream_t s, int64_t M, const float
     }
 #undef KS_LAUNCH
   }
-  for (int l = 0; l < L; ++l)
-    hipLaunchKernelGGL(sum_parts_tree_kernel, dim3((unsigned)m.npad[l]), dim3(64), 0, s, (int64_t)m.npad[l], (int)tiles, ws.bpart[l], m.gb[l]);
   (void)x;  // the training forward left its transpose behind
   const T* xT = (const T*)ws.yT[L - 1];
+  GradFinishArgs g;
+  std::memset(&g, 0, sizeof(g));
+  g.n_layers = L; g.tiles = (int)tiles;
+  int wblocks = 0, bblocks = 0;
   for (int l = L - 1; l >= 0; --l) {
     const int np = m.npad[l], kp = m.kpad[l], kp128 = round_up(kp, kBN);
     const T* dzT = (const T*)ws.dzT[l];
@@ -1627,16 +1665,21 @@ static int train_backward_chain(DevMlp& m, hipStream_t s, int64_t M, const float
     int rc;
     if (wide)
       rc = launch_layer_tile<T, false, true, 128, 128, 2, 2>(KS_ACT_NONE, s, np, kp128, (int)Mp, (int)Mp, kp, dzT, Mp, yT, m.zero_bias,
-                                                              ksplit > 1 ? (void*)ws.part : (void*)m.gW[l], kp, ksplit);
+                                                              (void*)ws.wpart[l], kp, ksplit);
     else
       rc = launch_layer_tile<T, false, true, 64, 128, 2, 2>(KS_ACT_NONE, s, np, kp128, (int)Mp, (int)Mp, kp, dzT, Mp, yT, m.zero_bias,
-                                                             ksplit > 1 ? (void*)ws.part : (void*)m.gW[l], kp, ksplit);
+                                                             (void*)ws.wpart[l], kp, ksplit);
     if (rc != KS_OK) return rc;
-    if (ksplit > 1) {
-      const int64_t n = (int64_t)np * kp;
-      hipLaunchKernelGGL(sum_parts_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, n, ksplit, ws.part, m.gW[l]);
-    }
+    g.nz[l] = ksplit; g.nW[l] = (int64_t)np * kp; g.nb[l] = np;
+    g.wpart[l] = ws.wpart[l]; g.bpart[l] = ws.bpart[l]; g.gW[l] = m.gW[l]; g.gb[l] = m.gb[l];
   }
+  for (int l = 0; l < L; ++l) {
+    g.first_w[l] = wblocks; g.first_b[l] = bblocks;
+    wblocks += (int)((g.nW[l] + 255) / 256);
+    bblocks += (g.nb[l] + 3) / 4;
+  }
+  g.first_w[L] = wblocks; g.first_b[L] = bblocks;
+  hipLaunchKernelGGL(grad_finish_kernel, dim3((unsigned)(wblocks + bblocks)), dim3(256), 0, s, g);
   return KS_OK;
 }
 
