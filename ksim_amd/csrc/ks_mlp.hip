@@ -329,9 +329,12 @@ __device__ __forceinline__ void fused_bias_init(f32x16& acc, const float* __rest
 }
 
 // Hidden layer: activation, round to bf16, back into the tile (4 consecutive features = one 8-byte LDS store).
+// `keep_t` (nullable) points at the transposed copy's entry (feature 0, this lane's row): across the 32 lanes of a half the
+// same register holds 32 consecutive rows of one feature, so a 2-byte store per lane writes two whole 64-byte runs.
 template <int ACT>
 __device__ __forceinline__ void fused_store_hidden(const f32x16& acc, __bf16* __restrict__ act, int lda, int j,
-                                                   int row, int lane, uint2* __restrict__ keep = nullptr) {
+                                                   int row, int lane, uint2* __restrict__ keep = nullptr,
+                                                   __bf16* __restrict__ keep_t = nullptr, int64_t ldt = 0) {
 #pragma unroll
   for (int g = 0; g < 4; ++g) {
     const int f0 = j * 32 + 8 * g + 4 * (lane >> 5);
@@ -339,6 +342,11 @@ __device__ __forceinline__ void fused_store_hidden(const f32x16& acc, __bf16* __
                           pack_bf16(activate<ACT, true>(acc[4 * g + 2]), activate<ACT, true>(acc[4 * g + 3]))};
     *reinterpret_cast<uint2*>(act + row * lda + f0) = packed;
     if (keep) keep[g * 64 + lane] = packed;  // the same four values, in accumulator order
+    if (keep_t) {
+      unsigned short* o = reinterpret_cast<unsigned short*>(keep_t) + (int64_t)f0 * ldt;
+      o[0] = (unsigned short)packed.x; o[ldt] = (unsigned short)(packed.x >> 16);
+      o[2 * ldt] = (unsigned short)packed.y; o[3 * ldt] = (unsigned short)(packed.y >> 16);
+    }
   }
 }
 
@@ -438,14 +446,13 @@ __device__ __forceinline__ void fused_layer(const FusedArgs& a, int l, __bf16* _
         for (int i = 0; i < MI; ++i) {
           if (LAST) fused_store_output(acc[t][i], a.y, a.M, a.out_dim, j, m0 + i * 32 + row, lane);
           else fused_store_hidden<ACT>(acc[t][i], act, lda, j, i * 32 + row, lane,
-                                       (KEEP && MI == 4) ? a.keep[l] + keep_index(tile, wave, t, i) : nullptr);
+                                       (KEEP && MI == 4) ? a.keep[l] + keep_index(tile, wave, t, i) : nullptr,
+                                       (KEEP && MI == 4) ? a.keep_t[l] + m0 + i * 32 + row : nullptr, a.ldt);
         }
       }
   }
   __syncthreads();
   KS_MLP_STAMP2(4 + 3 * l)
-  if (KEEP && !LAST && MI == 4 && (int)threadIdx.x < nt * 16)
-    (void)tile_transposed_out(act, lda, (int)threadIdx.x, a.keep_t[l], a.ldt, m0);
   if (!LAST && a.save[l]) {
     // the finished tile, 16 bytes per thread and pass, rows as contiguous runs; the next layer only reads the tile until every
     // wavefront (this copy included, which sits before its matrix work in program order) has passed the next barrier
@@ -643,13 +650,23 @@ void mlp_fused_bwd_kernel(const FusedBwdArgs a) {
               d[e] *= acc[t][i][4 * g + e];
             }
             const int f0 = j * 32 + 8 * g + 4 * (lane >> 5);
-            *reinterpret_cast<uint2*>(act + (i * 32 + row) * lda + f0) = uint2{pack_bf16(d[0], d[1]), pack_bf16(d[2], d[3])};
+            const uint2 packed = {pack_bf16(d[0], d[1]), pack_bf16(d[2], d[3])};
+            *reinterpret_cast<uint2*>(act + (i * 32 + row) * lda + f0) = packed;
+            // transposed, straight from the registers: 32 lanes hold 32 consecutive rows of one feature
+            unsigned short* o = reinterpret_cast<unsigned short*>(a.dzT[l - 1]) + (int64_t)f0 * a.ldt + m0 + i * 32 + row;
+            o[0] = (unsigned short)packed.x; o[a.ldt] = (unsigned short)(packed.x >> 16);
+            o[2 * a.ldt] = (unsigned short)packed.y; o[3 * a.ldt] = (unsigned short)(packed.y >> 16);
           }
         }
       }
     __syncthreads();
-    if (tid < nt * 16) {  // the next layer's K loop only reads the tile, as this does
-      const f32x2 cs = tile_transposed_out(act, lda, tid, a.dzT[l - 1], a.ldt, m0);
+    if (tid < nt * 16) {  // column sums of the new tile (the bias gradient's share); the next K loop only reads the tile, as this does
+      f32x2 cs = {0.f, 0.f};
+#pragma unroll 8
+      for (int r = 0; r < BM; ++r) {
+        const bf16x2 v = *reinterpret_cast<const bf16x2*>(act + r * lda + 2 * tid);
+        cs[0] += (float)v[0]; cs[1] += (float)v[1];
+      }
       float* part = a.bias_part[l - 1] + tile * (nt * 32) + 2 * tid;
       part[0] = cs[0];
       part[1] = cs[1];
