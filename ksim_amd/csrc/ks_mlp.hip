@@ -238,10 +238,8 @@ struct FusedArgs {
   // training forward: hidden layer l's activations also go to save[l], (M, save_ld[l]) bf16 row-major, for the backward pass
   __bf16* save[KS_MAX_LAYERS];
   int save_ld[KS_MAX_LAYERS];
-  // training forward for the whole-network backward kernel: hidden layer l's activations in the accumulator order of the
-  // wavefronts that produced them (keep[l]: per 128-row tile [wavefront][feature tile 0..1][row tile][g][lane] x 8 bytes, so the
-  // backward kernel's epilogue reads its own entries with one 8-byte load per lane) and transposed (keep_t[l]: (width, ldt))
-  uint2* keep[KS_MAX_LAYERS];
+  // training forward for the whole-network backward kernel: hidden layer l's activations transposed, keep_t[l]: (width, ldt).
+  // The weight-gradient product takes them as they are, and the backward kernel's epilogue reads its f'(Y) from them.
   __bf16* keep_t[KS_MAX_LAYERS];
   __bf16* keep_t_in;  // the network input, transposed: (in_t_width, ldt), zero beyond the real inputs
   int in_t_width;
@@ -333,27 +331,19 @@ __device__ __forceinline__ void fused_bias_init(f32x16& acc, const float* __rest
 // same register holds 32 consecutive rows of one feature, so a 2-byte store per lane writes two whole 64-byte runs.
 template <int ACT>
 __device__ __forceinline__ void fused_store_hidden(const f32x16& acc, __bf16* __restrict__ act, int lda, int j,
-                                                   int row, int lane, uint2* __restrict__ keep = nullptr,
-                                                   __bf16* __restrict__ keep_t = nullptr, int64_t ldt = 0) {
+                                                   int row, int lane, __bf16* __restrict__ keep_t = nullptr, int64_t ldt = 0) {
 #pragma unroll
   for (int g = 0; g < 4; ++g) {
     const int f0 = j * 32 + 8 * g + 4 * (lane >> 5);
     const uint2 packed = {pack_bf16(activate<ACT, true>(acc[4 * g]), activate<ACT, true>(acc[4 * g + 1])),
                           pack_bf16(activate<ACT, true>(acc[4 * g + 2]), activate<ACT, true>(acc[4 * g + 3]))};
     *reinterpret_cast<uint2*>(act + row * lda + f0) = packed;
-    if (keep) keep[g * 64 + lane] = packed;  // the same four values, in accumulator order
     if (keep_t) {
       unsigned short* o = reinterpret_cast<unsigned short*>(keep_t) + (int64_t)f0 * ldt;
       o[0] = (unsigned short)packed.x; o[ldt] = (unsigned short)(packed.x >> 16);
       o[2 * ldt] = (unsigned short)packed.y; o[3 * ldt] = (unsigned short)(packed.y >> 16);
     }
   }
-}
-
-// Entries of one 128-row tile in an accumulator-order buffer: [wavefront][feature tile 0..1][row tile 0..3][g][lane]
-constexpr int kKeepPerTile = kFusedWaves * 2 * 4 * 4 * 64;
-__device__ __forceinline__ int64_t keep_index(int64_t tile, int wave, int t, int i) {
-  return tile * kKeepPerTile + (((wave * 2 + t) * 4 + i) * 4) * 64;
 }
 
 // The finished 128-row tile, transposed, to dst (width, ld): thread p takes the columns 2 p and 2 p + 1 of the tile (one
@@ -446,7 +436,6 @@ __device__ __forceinline__ void fused_layer(const FusedArgs& a, int l, __bf16* _
         for (int i = 0; i < MI; ++i) {
           if (LAST) fused_store_output(acc[t][i], a.y, a.M, a.out_dim, j, m0 + i * 32 + row, lane);
           else fused_store_hidden<ACT>(acc[t][i], act, lda, j, i * 32 + row, lane,
-                                       (KEEP && MI == 4) ? a.keep[l] + keep_index(tile, wave, t, i) : nullptr,
                                        (KEEP && MI == 4) ? a.keep_t[l] + m0 + i * 32 + row : nullptr, a.ldt);
         }
       }
@@ -540,8 +529,8 @@ __device__ __forceinline__ void mlp_fused_body(const FusedArgs& a, int64_t tile)
   fused_layer<ACT, MI, true, KEEP>(a, a.n_layers - 1, act, m0, lane, wave, tile);
 }
 
-// KEEP: the training forward that stores every hidden layer's activations in accumulator order and transposed (FusedArgs::keep,
-// keep_t; 128-row tiles only)
+// KEEP: the training forward that also stores every hidden layer's activations and the network input transposed
+// (FusedArgs::keep_t, keep_t_in; 128-row tiles only)
 template <int ACT, int BM, bool KEEP = false>
 __global__ __launch_bounds__(64 * kFusedWaves) __attribute__((amdgpu_waves_per_eu(BM <= 64 ? 4 : 2, BM <= 64 ? 4 : 2)))
 void mlp_fused_kernel(const FusedArgs a) {
@@ -569,17 +558,19 @@ void mlp_fused_pair_kernel(const FusedArgs a, const FusedArgs b) {
 
 // ---------------------------------------------------------------- whole-network backward pass of the hidden layers
 // dZ_{l-1} = (dZ_l W_l) * f'(Y_{l-1}) for l = L-1 .. 1 in one launch, a 128-row tile per workgroup that never leaves LDS: the
-// product is the forward kernel's K loop over the fragment-ordered transposed weights, its epilogue reads the stored
-// activations in accumulator order (FusedArgs::keep), and after each layer the tile goes out transposed (the operand of the
-// weight-gradient product) together with its column sums (the bias gradient, one partial row per tile).
+// product is the forward kernel's K loop over the fragment-ordered transposed weights, its epilogue reads f'(Y) from the
+// transposed activations the training forward stored (FusedArgs::keep_t) and writes the new tile both into LDS and, transposed,
+// to memory (the operand of the weight-gradient product: in the accumulator layout the 32 lanes of a half hold 32 consecutive
+// rows of one feature, so 2-byte loads and stores per lane move whole 64-byte runs), and the tile's column sums follow (the
+// bias gradient, one partial row per tile).
 struct FusedBwdArgs {
   int64_t M;
-  int n_layers, lda, ld_last;
+  int n_layers, lda;
   int fk[KS_MAX_LAYERS], fn[KS_MAX_LAYERS];   // the forward kernel's K steps and output tiles per layer
   const u32x4* WtP[KS_MAX_LAYERS];            // l >= 1: W_l^T in fragment order, [input tile][step over outputs][lane] x 16 bytes
   const float* dy;                            // (M, out_dim): gradient of the network output, in the caller's layout
   int out_dim, np_last;                       // np_last: rows of dzT[L-1] (the output width padded for the weight-gradient product)
-  const uint2* keep[KS_MAX_LAYERS];           // hidden layer l's activations in accumulator order
+  const __bf16* yT[KS_MAX_LAYERS];            // hidden layer l's activations, transposed (width, ldt), as the training forward left them
   __bf16* dzT[KS_MAX_LAYERS];                 // out, every layer: dZ_l^T (width, ldt)
   float* bias_part[KS_MAX_LAYERS];            // out, every layer: (tiles, width) column sums of dZ_l per tile
   int64_t ldt;
@@ -634,12 +625,13 @@ void mlp_fused_bwd_kernel(const FusedBwdArgs a) {
         const int j = t == 0 ? j0 : j1;
 #pragma unroll
         for (int i = 0; i < MI; ++i) {
-          const uint2* y = a.keep[l - 1] + keep_index(tile, wave, t, i);
+          // this lane's activations Y_{l-1} from the transposed copy: per feature, 32 lanes read 32 consecutive rows
+          const unsigned short* y = reinterpret_cast<const unsigned short*>(a.yT[l - 1]) + m0 + i * 32 + row;
 #pragma unroll
           for (int g = 0; g < 4; ++g) {
-            const uint2 yy = y[g * 64 + lane];
-            const float yv[4] = {__builtin_bit_cast(float, yy.x << 16), __builtin_bit_cast(float, yy.x & 0xffff0000u),
-                                 __builtin_bit_cast(float, yy.y << 16), __builtin_bit_cast(float, yy.y & 0xffff0000u)};
+            const unsigned short* yg = y + (int64_t)(j * 32 + 8 * g + 4 * (lane >> 5)) * a.ldt;
+            const float yv[4] = {__builtin_bit_cast(float, (unsigned)yg[0] << 16), __builtin_bit_cast(float, (unsigned)yg[a.ldt] << 16),
+                                 __builtin_bit_cast(float, (unsigned)yg[2 * a.ldt] << 16), __builtin_bit_cast(float, (unsigned)yg[3 * a.ldt] << 16)};
             float d[4];
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
@@ -1507,9 +1499,9 @@ struct TrainWs {
   char *d0, *d1, *t0, *t1, *t2;
   float* part;  // partial sums of the split reductions
   int64_t Mp;
-  // whole-network backward pass (chain_ok): per hidden layer the activations in accumulator order and transposed, per layer
-  // dZ^T, per hidden layer one row of bias partial sums per 128-row tile; all transposes have the row stride Mp128
-  char *yacc[KS_MAX_LAYERS], *yT[KS_MAX_LAYERS], *dzT[KS_MAX_LAYERS];
+  // whole-network backward pass (chain_ok): per hidden layer the activations transposed, per layer dZ^T and one row of bias
+  // partial sums per 128-row tile; all transposes have the row stride Mp128
+  char *yT[KS_MAX_LAYERS], *dzT[KS_MAX_LAYERS];
   float *bpart[KS_MAX_LAYERS], *wpart[KS_MAX_LAYERS];  // wpart: the row slices of each layer's weight-gradient product
   int64_t Mp128;
 };
@@ -1554,7 +1546,6 @@ static int64_t carve_train(const DevMlp& m, int64_t M, char* base, TrainWs* ws) 
   if (chain_ok(m, M)) {
     const int64_t tiles = w.Mp128 / 128;
     for (int l = 0; l + 1 < m.n_layers; ++l) {
-      w.yacc[l] = take(tiles * kKeepPerTile * 8);
       w.yT[l] = take((int64_t)m.npad[l] * w.Mp128 * esz);
       w.bpart[l] = (float*)take(tiles * m.npad[l] * 4);
     }
@@ -1569,7 +1560,6 @@ static int64_t carve_train(const DevMlp& m, int64_t M, char* base, TrainWs* ws) 
 
 static void keep_args(FusedArgs& a, const DevMlp& m, const TrainWs* ws) {
   for (int l = 0; l + 1 < m.n_layers; ++l) {
-    a.keep[l] = (uint2*)ws->yacc[l];
     a.keep_t[l] = (__bf16*)ws->yT[l];
   }
   a.keep_t_in = (__bf16*)ws->yT[m.n_layers - 1];
@@ -1645,7 +1635,7 @@ static int train_backward_chain(DevMlp& m, hipStream_t s, int64_t M, const float
     for (int l = 0; l < L; ++l) {
       a.fk[l] = m.fk[l]; a.fn[l] = m.fn[l];
       a.WtP[l] = (const u32x4*)m.WtP[l];
-      if (l + 1 < L) a.keep[l] = (const uint2*)ws.yacc[l];
+      if (l + 1 < L) a.yT[l] = (const __bf16*)ws.yT[l];
       a.dzT[l] = (__bf16*)ws.dzT[l];
       a.bias_part[l] = ws.bpart[l];
     }
