@@ -619,38 +619,53 @@ void mlp_fused_bwd_kernel(const FusedBwdArgs a) {
     if (mine == 2) fused_layer_mma<2, MI, kPF>(acc, w0, w1, nk, arow, lda);
     else if (mine == 1) fused_layer_mma<1, MI, kPF>(acc, w0, w0, nk, arow, lda);
     __syncthreads();  // every wavefront has read dZ_l; the tile can take dZ_{l-1}
+    // Epilogue in blocks of one (feature tile, row tile) pair = 16 accumulator registers.  A block's 16 activations Y_{l-1} come
+    // from the transposed copy (per feature, 32 lanes read 32 consecutive rows); the next block's loads are issued before this
+    // block is worked on, so their latency hides behind it instead of adding up 32 times per layer.
+    auto y_block = [&](int blk, unsigned short (&yv)[16]) {
+      const int t = blk >> 2, i = blk & 3;
+      const int j = t == 0 ? j0 : j1;
+      const unsigned short* y = reinterpret_cast<const unsigned short*>(a.yT[l - 1]) + m0 + i * 32 + row;
 #pragma unroll
-    for (int t = 0; t < 2; ++t)
-      if (t < mine) {
+      for (int g = 0; g < 4; ++g) {
+        const unsigned short* yg = y + (int64_t)(j * 32 + 8 * g + 4 * (lane >> 5)) * a.ldt;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) yv[4 * g + e] = yg[e * a.ldt];
+      }
+    };
+    unsigned short ya[16], yb[16];
+    const int nblk = mine * MI;
+    if (nblk > 0) y_block(0, ya);
+#pragma unroll
+    for (int blk = 0; blk < 2 * MI; ++blk) {
+      if (blk < nblk) {
+        unsigned short (&cur)[16] = (blk & 1) ? yb : ya;
+        unsigned short (&nxt)[16] = (blk & 1) ? ya : yb;
+        if (blk + 1 < nblk) y_block(blk + 1, nxt);
+        const int t = blk >> 2, i = blk & 3;
         const int j = t == 0 ? j0 : j1;
 #pragma unroll
-        for (int i = 0; i < MI; ++i) {
-          // this lane's activations Y_{l-1} from the transposed copy: per feature, 32 lanes read 32 consecutive rows
-          const unsigned short* y = reinterpret_cast<const unsigned short*>(a.yT[l - 1]) + m0 + i * 32 + row;
+        for (int g = 0; g < 4; ++g) {
+          float d[4];
 #pragma unroll
-          for (int g = 0; g < 4; ++g) {
-            const unsigned short* yg = y + (int64_t)(j * 32 + 8 * g + 4 * (lane >> 5)) * a.ldt;
-            const float yv[4] = {__builtin_bit_cast(float, (unsigned)yg[0] << 16), __builtin_bit_cast(float, (unsigned)yg[a.ldt] << 16),
-                                 __builtin_bit_cast(float, (unsigned)yg[2 * a.ldt] << 16), __builtin_bit_cast(float, (unsigned)yg[3 * a.ldt] << 16)};
-            float d[4];
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              d[e] = 1.f;
-              if (ACT == KS_ACT_ELU) d[e] = yv[e] > 0.f ? 1.f : yv[e] + 1.f;
-              if (ACT == KS_ACT_RELU) d[e] = yv[e] > 0.f ? 1.f : 0.f;
-              if (ACT == KS_ACT_TANH) d[e] = 1.f - yv[e] * yv[e];
-              d[e] *= acc[t][i][4 * g + e];
-            }
-            const int f0 = j * 32 + 8 * g + 4 * (lane >> 5);
-            const uint2 packed = {pack_bf16(d[0], d[1]), pack_bf16(d[2], d[3])};
-            *reinterpret_cast<uint2*>(act + (i * 32 + row) * lda + f0) = packed;
-            // transposed, straight from the registers: 32 lanes hold 32 consecutive rows of one feature
-            unsigned short* o = reinterpret_cast<unsigned short*>(a.dzT[l - 1]) + (int64_t)f0 * a.ldt + m0 + i * 32 + row;
-            o[0] = (unsigned short)packed.x; o[a.ldt] = (unsigned short)(packed.x >> 16);
-            o[2 * a.ldt] = (unsigned short)packed.y; o[3 * a.ldt] = (unsigned short)(packed.y >> 16);
+          for (int e = 0; e < 4; ++e) {
+            const float yv = __builtin_bit_cast(float, (unsigned)cur[4 * g + e] << 16);
+            d[e] = 1.f;
+            if (ACT == KS_ACT_ELU) d[e] = yv > 0.f ? 1.f : yv + 1.f;
+            if (ACT == KS_ACT_RELU) d[e] = yv > 0.f ? 1.f : 0.f;
+            if (ACT == KS_ACT_TANH) d[e] = 1.f - yv * yv;
+            d[e] *= acc[t][i][4 * g + e];
           }
+          const int f0 = j * 32 + 8 * g + 4 * (lane >> 5);
+          const uint2 packed = {pack_bf16(d[0], d[1]), pack_bf16(d[2], d[3])};
+          *reinterpret_cast<uint2*>(act + (i * 32 + row) * lda + f0) = packed;
+          // transposed, straight from the registers: 32 lanes hold 32 consecutive rows of one feature
+          unsigned short* o = reinterpret_cast<unsigned short*>(a.dzT[l - 1]) + (int64_t)f0 * a.ldt + m0 + i * 32 + row;
+          o[0] = (unsigned short)packed.x; o[a.ldt] = (unsigned short)(packed.x >> 16);
+          o[2 * a.ldt] = (unsigned short)packed.y; o[3 * a.ldt] = (unsigned short)(packed.y >> 16);
         }
       }
+    }
     __syncthreads();
     if (tid < nt * 16) {  // column sums of the new tile (the bias gradient's share); the next K loop only reads the tile, as this does
       f32x2 cs = {0.f, 0.f};
