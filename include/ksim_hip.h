@@ -749,7 +749,9 @@ int ks_lstm_forward(const KsLstm* lstm, ks_stream_t stream, int64_t M, const flo
  * learning rate, -1).  ks_mlp_train_init keeps fp32 master weights, gradients and Adam moments beside
  * the working-precision copies that ks_mlp_forward reads; after ks_mlp_adam_step every copy is refreshed.
  *   ks_mlp_train_forward  y = net(x), hidden activations kept in `workspace` for the backward pass
- *   ks_mlp_train_backward gradients of sum(dy * y) w.r.t. every weight and bias, into the handle
+ *   ks_mlp_train_backward gradients of sum(dy * y) w.r.t. every weight and bias, into the handle.  It follows the
+ *                         ks_mlp_train_forward of the same rows on the same workspace, whose contents (and layout: large
+ *                         bf16 batches keep their activations transposed for a one-launch backward pass) belong to the pair
  *   ks_grad_sqnorm        adds the squared norm of n floats (NaNs skipped) to *acc (device double)
  *   ks_mlp_grad_sqnorm    the same over all gradients of a network
  *   ks_mlp_adam_step      one optimiser step with `sqnorm` = squared global gradient norm over everything
