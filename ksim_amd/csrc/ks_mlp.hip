@@ -84,14 +84,14 @@ __device__ __forceinline__ u32x4 load_first(const float* __restrict__ x, int64_t
 // BM: rows per workgroup (128, or 64 for small batches so that the grid still covers every CU twice).
 // The K loop is software-pipelined: the global loads of slice k+1 are issued into registers before the MFMAs
 // of slice k run out of LDS, so HBM/L2 latency overlaps the matrix-core work.
-template <typename T, bool FIRST, bool LAST, int ACT, int BM, int BN, int WAVES_M, int WAVES_N>
+template <typename T, bool FIRST, bool LAST, int ACT, int BM, int BN, int WAVES_M, int WAVES_N, int KMUL = 1>
 __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void mlp_layer_kernel(int64_t M, int K /*padded to BK*/, int Kreal, int Nreal,
                                                         const void* __restrict__ xin, int64_t ldx,
                                                         const T* __restrict__ W /*(Np, K)*/,
                                                         const float* __restrict__ bias /*(Np)*/,
                                                         void* __restrict__ yout, int64_t ldy) {
   constexpr bool BF = sizeof(T) == 2;
-  constexpr int BK = BF ? 64 : 32;       // elements of K per slice
+  constexpr int BK = (BF ? 64 : 32) * KMUL;  // elements of K per slice (KMUL 2: half the barriers per flop, twice the LDS)
   constexpr int PAD = BF ? 8 : 4;        // keeps 16-byte row alignment and spreads LDS banks
   constexpr int VEC = 16 / sizeof(T);    // elements per 16-byte load
   constexpr int NT = 64 * WAVES_M * WAVES_N;    // threads per workgroup
@@ -1118,16 +1118,16 @@ static uint16_t f32_to_bf16_rne(float f) {
   return (uint16_t)(u >> 16);
 }
 
-template <typename T, bool FIRST, bool LAST, int BM, int BN, int WAVES_M, int WAVES_N>
+template <typename T, bool FIRST, bool LAST, int BM, int BN, int WAVES_M, int WAVES_N, int KMUL = 1>
 static int launch_layer_tile(int act, hipStream_t s, int64_t M, int npad, int K, int Kreal, int Nreal, const void* x,
                              int64_t ldx, const void* W, const float* b, void* y, int64_t ldy, int ksplit = 1) {
-  constexpr int BK = sizeof(T) == 2 ? 64 : 32, PAD = sizeof(T) == 2 ? 8 : 4;
+  constexpr int BK = (sizeof(T) == 2 ? 64 : 32) * KMUL, PAD = sizeof(T) == 2 ? 8 : 4;
   constexpr int lds = (int)sizeof(T) * (BM + BN) * (BK + PAD);
   const dim3 grid((unsigned)((M + BM - 1) / BM), (unsigned)(npad / BN), (unsigned)ksplit);
   const dim3 block(64 * WAVES_M * WAVES_N);
 #define KS_LAUNCH(A)                                                                                           \
   {                                                                                                            \
-    auto kfn = mlp_layer_kernel<T, FIRST, LAST, A, BM, BN, WAVES_M, WAVES_N>;                                  \
+    auto kfn = mlp_layer_kernel<T, FIRST, LAST, A, BM, BN, WAVES_M, WAVES_N, KMUL>;                            \
     if (lds > 64 * 1024 &&                                                                                     \
         hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)  \
       return fail(KS_ELAUNCH, "ks_mlp_forward: cannot raise the LDS limit to %d bytes", lds);                  \
@@ -1683,11 +1683,11 @@ static int train_backward_chain(DevMlp& m, hipStream_t s, int64_t M, const float
     const T* yT = l > 0 ? (const T*)ws.yT[l - 1] : xT;
     const bool wide = np % 128 == 0;
     int ksplit = wide ? kDwSplit : kDwSplit / 2;
-    while (ksplit > 1 && (Mp / 64) % ksplit != 0) ksplit >>= 1;
+    while (ksplit > 1 && (Mp / 128) % ksplit != 0) ksplit >>= 1;  // K slices of 128 rows per pass
     int rc;
     if (wide)
-      rc = launch_layer_tile<T, false, true, 128, 128, 2, 2>(KS_ACT_NONE, s, np, kp128, (int)Mp, (int)Mp, kp, dzT, Mp, yT, m.zero_bias,
-                                                              (void*)ws.wpart[l], kp, ksplit);
+      rc = launch_layer_tile<T, false, true, 128, 128, 2, 2, 2>(KS_ACT_NONE, s, np, kp128, (int)Mp, (int)Mp, kp, dzT, Mp, yT, m.zero_bias,
+                                                                 (void*)ws.wpart[l], kp, ksplit);
     else
       rc = launch_layer_tile<T, false, true, 64, 128, 2, 2>(KS_ACT_NONE, s, np, kp128, (int)Mp, (int)Mp, kp, dzT, Mp, yT, m.zero_bias,
                                                              (void*)ws.wpart[l], kp, ksplit);
