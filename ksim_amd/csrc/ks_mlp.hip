@@ -1988,6 +1988,93 @@ __global__ __launch_bounds__(256) void sgemm_kernel(int M, int N, int K, const f
     }
 }
 
+// The same product for the weight and bias gradients of wide layers, C(i, j) (+)= sum_k A(k, i) B(k, j) with both operands
+// stored (k, .) and a long reduction over the rows: a 128 x 128 tile per workgroup (each wavefront a 64 x 64 block = 2 x 2 MFMA tiles, so a value read
+// from LDS feeds two matrix instructions), 16-byte global loads (vec_a / vec_b: the operand's rows are 16-byte aligned) whose
+// next slice is in flight while the matrix cores work on this one.  A narrow B (71 columns, or the single column of ones that
+// makes the product a column sum) wastes matrix work, not memory traffic, which is what bounds these products.  Slices and
+// partial outputs as in sgemm_kernel.
+__global__ __launch_bounds__(256) void sgemm_tn128_kernel(int M, int N, int K, const float* __restrict__ A, int64_t lda,
+                                                          const float* __restrict__ B, int64_t ldb, float* __restrict__ C, int64_t ldc,
+                                                          int kslice, int accumulate, int vec_a, int vec_b) {
+  __shared__ __attribute__((aligned(16))) float As[16][132];
+  __shared__ __attribute__((aligned(16))) float Bs[16][132];
+  const int t = threadIdx.x, i0 = blockIdx.y * 128, j0 = blockIdx.x * 128;
+  const int kbeg = blockIdx.z * kslice, kend = min(K, kbeg + kslice);
+  const int wave = t >> 6, lane = t & 63, c = lane & 31, h = lane >> 5;
+  const int wi = (wave >> 1) * 64, wj = (wave & 1) * 64;
+  f32x16 acc[2][2];
+#pragma unroll
+  for (int a = 0; a < 2; ++a)
+#pragma unroll
+    for (int b = 0; b < 2; ++b)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
+  float4 ra[2], rb[2];
+  // thread t loads rows k = t / 32 and 8 + t / 32 of the slice, four consecutive columns from 4 (t % 32)
+  const int lk = t >> 5, l4 = (t & 31) * 4;
+#define KS_TN_FETCH(K0)                                                                                           \
+  _Pragma("unroll") for (int r = 0; r < 2; ++r) {                                                                 \
+    const int k = (K0) + lk + 8 * r;                                                                              \
+    const int gi = i0 + l4, gj = j0 + l4;                                                                         \
+    ra[r] = float4{0.f, 0.f, 0.f, 0.f};                                                                           \
+    rb[r] = float4{0.f, 0.f, 0.f, 0.f};                                                                           \
+    if (k < kend) {                                                                                               \
+      if (gi + 3 < M && vec_a) ra[r] = *reinterpret_cast<const float4*>(A + (int64_t)k * lda + gi);               \
+      else if (gi < M) {                                                                                          \
+        const float* q = A + (int64_t)k * lda + gi;                                                               \
+        ra[r].x = q[0]; if (gi + 1 < M) ra[r].y = q[1]; if (gi + 2 < M) ra[r].z = q[2]; if (gi + 3 < M) ra[r].w = q[3]; \
+      }                                                                                                           \
+      if (gj + 3 < N && vec_b) rb[r] = *reinterpret_cast<const float4*>(B + (int64_t)k * ldb + gj);               \
+      else if (gj < N) {                                                                                          \
+        const float* q = B + (int64_t)k * ldb + gj;                                                               \
+        rb[r].x = q[0]; if (gj + 1 < N) rb[r].y = q[1]; if (gj + 2 < N) rb[r].z = q[2]; if (gj + 3 < N) rb[r].w = q[3]; \
+      }                                                                                                           \
+    }                                                                                                             \
+  }
+  KS_TN_FETCH(kbeg)
+  for (int k0 = kbeg; k0 < kend; k0 += 16) {
+#pragma unroll
+    for (int r = 0; r < 2; ++r) {
+      *reinterpret_cast<float4*>(&As[lk + 8 * r][l4]) = ra[r];
+      *reinterpret_cast<float4*>(&Bs[lk + 8 * r][l4]) = rb[r];
+    }
+    __syncthreads();
+    KS_TN_FETCH(k0 + 16)  // beyond the slice: zeros that are never stored
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+      const float a0 = As[2 * s + h][wi + c], a1 = As[2 * s + h][wi + 32 + c];
+      const float b0 = Bs[2 * s + h][wj + c], b1 = Bs[2 * s + h][wj + 32 + c];
+      acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b0, acc[0][0], 0, 0, 0);
+      acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b1, acc[0][1], 0, 0, 0);
+      acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b0, acc[1][0], 0, 0, 0);
+      acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b1, acc[1][1], 0, 0, 0);
+    }
+    __syncthreads();
+  }
+#undef KS_TN_FETCH
+  const bool sliced = gridDim.z > 1;
+  float* out = sliced ? C + (int64_t)blockIdx.z * M * N : C;
+  const int64_t ld = sliced ? N : ldc;
+#pragma unroll
+  for (int a = 0; a < 2; ++a)
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+      const int gj = j0 + wj + 32 * b + c;
+      if (gj >= N) continue;
+#pragma unroll
+      for (int g = 0; g < 4; ++g)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int gi = i0 + wi + 32 * a + 8 * g + 4 * h + e;
+          if (gi >= M) continue;
+          float v = acc[a][b][4 * g + e];
+          if (!sliced && accumulate) v += out[(int64_t)gi * ld + gj];
+          out[(int64_t)gi * ld + gj] = v;
+        }
+    }
+}
+
 __global__ __launch_bounds__(256) void sum_slices_kernel(int M, int N, int nz, const float* __restrict__ part, float* __restrict__ C,
                                                          int64_t ldc, int accumulate) {
   const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
@@ -2131,6 +2218,26 @@ template <bool A_KC, bool B_KC>
 static void sgemm(hipStream_t s, int64_t M, int N, int64_t K, const float* A, int64_t lda, const float* B, int64_t ldb, float* C,
                   int64_t ldc, const float* bias, int act, bool accumulate, float* part) {
   if (M <= 0 || N <= 0 || K <= 0) return;  // every caller with an empty sum adds into its output
+  if (!A_KC && !B_KC && M >= 128 && !bias && act == KS_ACT_NONE) {  // gradients of wide layers: long reductions over the rows
+    const int vec_a = lda % 4 == 0 && ((uintptr_t)A & 15) == 0, vec_b = ldb % 4 == 0 && ((uintptr_t)B & 15) == 0;
+    const int64_t tiles = ((M + 127) / 128) * ((N + 127) / 128);
+    int slices = 1;
+    if (part && K >= 2048) {
+      slices = (int)((512 + tiles - 1) / tiles);
+      if (slices > kDiscMaxSlices) slices = kDiscMaxSlices;
+      if ((int64_t)slices * 256 > K) slices = (int)(K / 256);
+    }
+    int kslice = (int)((K + slices - 1) / slices);
+    kslice = (kslice + 15) / 16 * 16;
+    slices = (int)((K + kslice - 1) / kslice);
+    hipLaunchKernelGGL(sgemm_tn128_kernel, dim3((unsigned)((N + 127) / 128), (unsigned)((M + 127) / 128), (unsigned)slices), dim3(256), 0, s,
+                       (int)M, N, (int)K, A, lda, B, ldb, slices > 1 ? part : C, ldc, kslice, accumulate ? 1 : 0, vec_a, vec_b);
+    if (slices > 1) {
+      const int64_t n = M * N;
+      hipLaunchKernelGGL(sum_slices_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, (int)M, N, slices, part, C, ldc, accumulate ? 1 : 0);
+    }
+    return;
+  }
   const int64_t tiles = ((M + 63) / 64) * ((N + 63) / 64);
   int slices = 1;
   if (part && tiles < 128 && K >= 2048) {
