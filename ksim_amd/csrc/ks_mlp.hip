@@ -2218,6 +2218,11 @@ template <bool A_KC, bool B_KC>
 static void sgemm(hipStream_t s, int64_t M, int N, int64_t K, const float* A, int64_t lda, const float* B, int64_t ldb, float* C,
                   int64_t ldc, const float* bias, int act, bool accumulate, float* part) {
   if (M <= 0 || N <= 0 || K <= 0) return;  // every caller with an empty sum adds into its output
+  if (!A_KC && !B_KC && M == 1 && N >= 128 && !bias && act == KS_ACT_NONE) {
+    // one output row: the same numbers as the (N, 1) product with the operands exchanged, which takes the wide path below
+    sgemm<false, false>(s, N, 1, K, B, ldb, A, lda, C, 1, nullptr, KS_ACT_NONE, accumulate, part);
+    return;
+  }
   if (!A_KC && !B_KC && M >= 128 && !bias && act == KS_ACT_NONE) {  // gradients of wide layers: long reductions over the rows
     const int vec_a = lda % 4 == 0 && ((uintptr_t)A & 15) == 0, vec_b = ldb % 4 == 0 && ((uintptr_t)B & 15) == 0;
     const int64_t tiles = ((M + 127) / 128) * ((N + 127) / 128);
