@@ -39,7 +39,9 @@ def make_real_batch(motions: torch.Tensor, window_t: int, batch_b: int, generato
     (amp.py:570-625; the draws come from `generator`, not from jax's key splitting)."""
     clip_idx = torch.randint(0, motions.shape[0], (batch_b,), generator=generator)
     starts = torch.randint(0, motions.shape[1], (batch_b,), generator=generator)
-    return torch.stack([loop_slice(motions[int(c)], int(s), window_t) for c, s in zip(clip_idx, starts)])
+    # every window of the batch in one gather: frame (start + t) mod T_clip of the drawn clip, as loop_slice takes them
+    frames = (starts[:, None] + torch.arange(window_t)[None, :]) % motions.shape[1]
+    return motions[clip_idx[:, None].to(motions.device), frames.to(motions.device)]
 
 
 def make_sim_batch(sim_motions: torch.Tensor, batch_b: int, generator: torch.Generator) -> torch.Tensor:

@@ -127,3 +127,10 @@ def test_discriminator_argument_errors():
         amp.make_sim_batch(torch.zeros(10, 3, 6, device=DEV), 4, torch.Generator())
     w = amp.loop_slice(torch.arange(3, device=DEV), 2, 5)
     assert w.tolist() == [2, 0, 1, 2, 0]
+    # a batch of reference windows is those slices, of the clips and starts the generator draws, gathered at once
+    motions = torch.arange(4 * 7 * 2, device=DEV, dtype=torch.float32).reshape(4, 7, 2)
+    batch = amp.make_real_batch(motions, 10, 6, torch.Generator().manual_seed(5))
+    g = torch.Generator().manual_seed(5)
+    clips, starts = torch.randint(0, 4, (6,), generator=g), torch.randint(0, 7, (6,), generator=g)
+    want = torch.stack([amp.loop_slice(motions[int(c)], int(s0), 10) for c, s0 in zip(clips, starts)])
+    assert batch.shape == (6, 10, 2) and torch.equal(batch, want)
