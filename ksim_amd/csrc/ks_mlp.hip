@@ -1992,11 +1992,13 @@ __global__ __launch_bounds__(256) void sgemm_kernel(int M, int N, int K, const f
 // stored (k, .) and a long reduction over the rows: a 128 x 128 tile per workgroup (each wavefront a 64 x 64 block = 2 x 2 MFMA tiles, so a value read
 // from LDS feeds two matrix instructions), 16-byte global loads (vec_a / vec_b: the operand's rows are 16-byte aligned) whose
 // next slice is in flight while the matrix cores work on this one.  A narrow B (71 columns, or the single column of ones that
-// makes the product a column sum) wastes matrix work, not memory traffic, which is what bounds these products.  Slices and
-// partial outputs as in sgemm_kernel.
+// makes the product a column sum) wastes matrix work, not memory traffic, which is what bounds these products.  `colsum`
+// (nullable) also receives sum_k A(k, i), the bias gradient that goes with a weight gradient, from the tiles that pass through
+// LDS anyway.  Slices and partial outputs as in sgemm_kernel.
 __global__ __launch_bounds__(256) void sgemm_tn128_kernel(int M, int N, int K, const float* __restrict__ A, int64_t lda,
                                                           const float* __restrict__ B, int64_t ldb, float* __restrict__ C, int64_t ldc,
-                                                          int kslice, int accumulate, int vec_a, int vec_b) {
+                                                          int kslice, int accumulate, int vec_a, int vec_b,
+                                                          float* __restrict__ colsum) {
   __shared__ __attribute__((aligned(16))) float As[16][132];
   __shared__ __attribute__((aligned(16))) float Bs[16][132];
   const int t = threadIdx.x, i0 = blockIdx.y * 128, j0 = blockIdx.x * 128;
@@ -2011,6 +2013,7 @@ __global__ __launch_bounds__(256) void sgemm_tn128_kernel(int M, int N, int K, c
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
   float4 ra[2], rb[2];
+  float cs = 0.f;  // colsum: this thread's column of A, summed over the slice
   // thread t loads rows k = t / 32 and 8 + t / 32 of the slice, four consecutive columns from 4 (t % 32)
   const int lk = t >> 5, l4 = (t & 31) * 4;
 #define KS_TN_FETCH(K0)                                                                                           \
@@ -2041,6 +2044,10 @@ __global__ __launch_bounds__(256) void sgemm_tn128_kernel(int M, int N, int K, c
     }
     __syncthreads();
     KS_TN_FETCH(k0 + 16)  // beyond the slice: zeros that are never stored
+    if (colsum && blockIdx.x == 0 && t < 128) {  // sum_k A(k, i) on the side: the tile is in LDS anyway
+#pragma unroll
+      for (int k = 0; k < 16; ++k) cs += As[k][t];
+    }
 #pragma unroll
     for (int s = 0; s < 8; ++s) {
       const float a0 = As[2 * s + h][wi + c], a1 = As[2 * s + h][wi + 32 + c];
@@ -2056,6 +2063,10 @@ __global__ __launch_bounds__(256) void sgemm_tn128_kernel(int M, int N, int K, c
   const bool sliced = gridDim.z > 1;
   float* out = sliced ? C + (int64_t)blockIdx.z * M * N : C;
   const int64_t ld = sliced ? N : ldc;
+  if (colsum && blockIdx.x == 0 && t < 128 && i0 + t < M) {  // sliced: partial row z of (slices, M); else the sums themselves
+    float* q = colsum + (sliced ? (int64_t)blockIdx.z * M : 0) + i0 + t;
+    *q = (!sliced && accumulate) ? *q + cs : cs;
+  }
 #pragma unroll
   for (int a = 0; a < 2; ++a)
 #pragma unroll
@@ -2179,7 +2190,7 @@ struct DiscWs {
   float* a[KS_MAX_LAYERS];      // real rows: W_{l+1}^T d_{l+1}
   float* d[KS_MAX_LAYERS];      // real rows: d_l
   float* r[KS_MAX_LAYERS];      // real rows: extra gradient of z_l
-  float *out, *dz0, *dz1, *g, *u, *v, *ones, *part;
+  float *out, *dz0, *dz1, *g, *u, *v, *ones, *part, *colpart;
 };
 
 static int64_t carve_disc(const DevMlp& m, int64_t R, int64_t M, char* base, DiscWs* ws) {
@@ -2209,14 +2220,16 @@ static int64_t carve_disc(const DevMlp& m, int64_t R, int64_t M, char* base, Dis
   w.v = take(R * wmax);
   w.ones = take(M);
   w.part = take(kDiscMaxSlices * maxw);
+  w.colpart = take((int64_t)kDiscMaxSlices * wmax);
   if (ws) *ws = w;
   return off;
 }
 
 // launches one product; cuts the k range when the output alone would leave most of the chip idle
+// colsum / colpart (wide row reductions only): colsum (M) += sum_k A(k, i) from the same pass, colpart its (slices, M) partials
 template <bool A_KC, bool B_KC>
 static void sgemm(hipStream_t s, int64_t M, int N, int64_t K, const float* A, int64_t lda, const float* B, int64_t ldb, float* C,
-                  int64_t ldc, const float* bias, int act, bool accumulate, float* part) {
+                  int64_t ldc, const float* bias, int act, bool accumulate, float* part, float* colsum = nullptr, float* colpart = nullptr) {
   if (M <= 0 || N <= 0 || K <= 0) return;  // every caller with an empty sum adds into its output
   if (!A_KC && !B_KC && M == 1 && N >= 128 && !bias && act == KS_ACT_NONE) {
     // one output row: the same numbers as the (N, 1) product with the operands exchanged, which takes the wide path below
@@ -2236,10 +2249,14 @@ static void sgemm(hipStream_t s, int64_t M, int N, int64_t K, const float* A, in
     kslice = (kslice + 15) / 16 * 16;
     slices = (int)((K + kslice - 1) / kslice);
     hipLaunchKernelGGL(sgemm_tn128_kernel, dim3((unsigned)((N + 127) / 128), (unsigned)((M + 127) / 128), (unsigned)slices), dim3(256), 0, s,
-                       (int)M, N, (int)K, A, lda, B, ldb, slices > 1 ? part : C, ldc, kslice, accumulate ? 1 : 0, vec_a, vec_b);
+                       (int)M, N, (int)K, A, lda, B, ldb, slices > 1 ? part : C, ldc, kslice, accumulate ? 1 : 0, vec_a, vec_b,
+                       colsum ? (slices > 1 ? colpart : colsum) : (float*)nullptr);
     if (slices > 1) {
       const int64_t n = M * N;
       hipLaunchKernelGGL(sum_slices_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, (int)M, N, slices, part, C, ldc, accumulate ? 1 : 0);
+      if (colsum)
+        hipLaunchKernelGGL(sum_slices_kernel, dim3((unsigned)((M + 255) / 256)), dim3(256), 0, s, (int)M, 1, slices, colpart, colsum, (int64_t)1,
+                           accumulate ? 1 : 0);
     }
     return;
   }
@@ -2339,13 +2356,16 @@ extern "C" int ks_mlp_disc_loss_grad(KsMlp* h, ks_stream_t stream, int64_t n_rea
   float *dz = ws.dz0, *dnx = ws.dz1;
   for (int l = L; l >= 1; --l) {
     const int n = m.dims[l], k = m.dims[l - 1];
+    // wide layers: the bias gradient (the column sums of dz) rides on the weight gradient's pass over dz
+    const bool with_bias = n >= 128;
+    float* gb = with_bias ? m.gb[l - 1] : nullptr;
     if (l == 1) {
-      sgemm<false, false>(s, n, k, R, dz, n, real, k, m.gW[0], m.kpad[0], nullptr, KS_ACT_NONE, true, ws.part);
-      sgemm<false, false>(s, n, k, n_sim, dz + R * n, n, sim, k, m.gW[0], m.kpad[0], nullptr, KS_ACT_NONE, true, ws.part);
+      sgemm<false, false>(s, n, k, R, dz, n, real, k, m.gW[0], m.kpad[0], nullptr, KS_ACT_NONE, true, ws.part, gb, ws.colpart);
+      sgemm<false, false>(s, n, k, n_sim, dz + R * n, n, sim, k, m.gW[0], m.kpad[0], nullptr, KS_ACT_NONE, true, ws.part, gb, ws.colpart);
     } else {
-      sgemm<false, false>(s, n, k, M, dz, n, ws.y[l - 2], k, m.gW[l - 1], m.kpad[l - 1], nullptr, KS_ACT_NONE, true, ws.part);
+      sgemm<false, false>(s, n, k, M, dz, n, ws.y[l - 2], k, m.gW[l - 1], m.kpad[l - 1], nullptr, KS_ACT_NONE, true, ws.part, gb, ws.colpart);
     }
-    sgemm<false, false>(s, n, 1, M, dz, n, ws.ones, 1, m.gb[l - 1], 1, nullptr, KS_ACT_NONE, true, ws.part);
+    if (!with_bias) sgemm<false, false>(s, n, 1, M, dz, n, ws.ones, 1, m.gb[l - 1], 1, nullptr, KS_ACT_NONE, true, ws.part);
     if (l == 1) break;
     sgemm<true, false>(s, M, k, n, dz, n, m.mW[l - 1], m.kpad[l - 1], dnx, k, nullptr, KS_ACT_NONE, false, nullptr);
     hipLaunchKernelGGL(disc_dz_kernel, blocks(M * k), dim3(256), 0, s, M * k, penalty ? R * k : (int64_t)0, act, ws.y[l - 2], ws.r[l - 2], dnx);

@@ -50,11 +50,12 @@ def test_discriminator_loss_gradient_matches_oracle(act, dims, dtype):
     assert l0[2] == 0.0
 
 
-def test_discriminator_many_rows_split_reduction():
-    """Enough frames that the weight-gradient products cut their row range into slices."""
+@pytest.mark.parametrize("dims", [[30, 64, 1], [30, 256, 130, 1]])
+def test_discriminator_many_rows_split_reduction(dims):
+    """Enough frames that the weight-gradient products cut their row range into slices; with layers of 128 units and more
+    they run on the wide tiles, the bias gradients summed in the same pass (a width that ends inside a tile included)."""
     from ksim_amd.mlp import MLP
 
-    dims = [30, 64, 1]
     ws, bs = _params(dims, seed=3)
     disc = MLP(ws, bs, activation="elu", dtype="f32")
     disc.train_init()
