@@ -212,7 +212,9 @@ def main() -> None:
     tpath = os.path.join(ROOT, "profiles", "step_kernel_cfg4_hbm_traffic.txt")
     if os.path.exists(tpath):  # measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, see that file
         for ln in open(tpath):
-            if ln.startswith("hbm_bytes_per_env_step="):  # counted on launches of 8192 envs; scaled to this run's launch size
+            # counted on launches of 8192 envs and of 4096 envs (the two-stream groups): the figure of this run's shape
+            key = "hbm_bytes_per_env_step_4096_env_launch=" if envs_per_launch <= 4096 else "hbm_bytes_per_env_step="
+            if ln.startswith(key):
                 traffic = float(ln.split("=", 1)[1]) * envs_per_launch
     valu = {}
     vpath = os.path.join(ROOT, "profiles", "step_kernel_cfg4_instruction_mix.txt")

@@ -303,7 +303,8 @@ class HipEngine(PhysicsEngine):
             gen = _generator(rng, action.device)
             drop = (torch.rand(action.shape, generator=gen, device=action.device) < p_drop).to(torch.uint8)
         buf = dict(qpos=d.qpos, qvel=d.qvel, qacc_warmstart=d.qacc_warmstart, time=d.time, last_ctrl=s.last_ctrl,
-                   action=action, latency=s.action_latency, zero_offset=s.zero_offset, drop=drop,
+                   action=action, latency=s.action_latency,
+                   zero_offset=None if _constant(self.data.zero_offset, 0.0) else s.zero_offset, drop=drop,
                    friction=rnd.get("friction"), mass_scale=rnd.get("mass_scale"), armature_scale=rnd.get("armature_scale"),
                    damping_scale=rnd.get("damping_scale"), **{k: rnd.get(k) for k in _MODEL_FIELD_OVERRIDES},
                    qacc=keep("qacc", d.qacc), ctrl_out=keep("ctrl", d.ctrl),
@@ -322,9 +323,15 @@ class HipEngine(PhysicsEngine):
         if isinstance(act, PositionActuators):
             cache = self.prepare(action.device)
             ast = s.actuator_state or {}
-            buf.update(kp=cache[1], kd=cache[2], ctrl_clip=cache[3], kp_scale=ast.get("kp_scale"),
-                       kd_scale=ast.get("kd_scale"), torque_limit_scale=ast.get("torque_limit_scale"),
-                       action_bias=ast.get("action"), torque_bias=ast.get("torque"))
+            # a per-episode quantity whose random variable is a constant 0 (offsets, biases) or 1 (scales) is the
+            # kernel's default for a null pointer: its buffer holds that constant in every row and is not streamed
+            live_ast = lambda name, rv, c: None if _constant(rv, c) else ast.get(name)  # noqa: E731
+            buf.update(kp=cache[1], kd=cache[2], ctrl_clip=cache[3],
+                       kp_scale=live_ast("kp_scale", act._rv(act.kp_scale), 1.0),
+                       kd_scale=live_ast("kd_scale", act._rv(act.kd_scale), 1.0),
+                       torque_limit_scale=live_ast("torque_limit_scale", act._rv(act.torque_limit_scale), 1.0),
+                       action_bias=live_ast("action", act.action_bias, 0.0),
+                       torque_bias=live_ast("torque", act.torque_bias, 0.0))
             physics.control_step(physics_model, buf, substeps=self.data.phys_steps_per_ctrl_steps,
                                  actuator_period=self.data.phys_steps_per_actuator_step,
                                  actuator_type=act.kind, action_scale=act.action_scale, events=ev)  # incl. position-velocity
@@ -336,6 +343,11 @@ class HipEngine(PhysicsEngine):
         if sched is not None:
             physics.work_order(physics_model, sched[1], sched[0])
         return physics_state
+
+
+def _constant(rv, value: float) -> bool:
+    """True when the random variable (None = the default of its field) only ever takes `value`."""
+    return rv is None or (rv.mean == value and rv.std == 0.0 and rv.mag == 0.0)
 
 
 def get_physics_engine(engine_type: str, resets, events, actuators: Actuators, config: EngineConfig) -> PhysicsEngine:

@@ -373,6 +373,53 @@ def test_reset_redraws_per_episode_quantities():
     assert (np.abs(zo) <= level * (0.02 + 5 * 0.01)).all() and zo.std() > 0.003
 
 
+def test_constant_per_episode_quantities_are_not_streamed(monkeypatch):
+    """A per-episode buffer whose random variable is a constant 0 (offsets, biases) or 1 (gain scales) holds that constant
+    in every row, the step kernel's default for a null pointer: the engine hands the kernel only the buffers that vary
+    (ksim/engine.py:117-138, ksim/actuators.py:90-95), and the step is bit for bit the one with all of them passed."""
+    from ksim_amd import actuators, engine, model as km, noise, physics
+
+    m = km.kbot_scale_model()
+    N, nu = 48, m.nu
+    dm = physics.DeviceModel(m)
+    seen = []
+    real_step = physics.control_step
+
+    def spy(model, buf, **kw):
+        seen.append({k: v is not None for k, v in buf.items()})
+        return real_step(model, buf, **kw)
+
+    monkeypatch.setattr(physics, "control_step", spy)
+    action = t32(np.random.default_rng(5).normal(scale=0.2, size=(N, nu)))
+    names = ("zero_offset", "action_bias", "torque_bias", "kp_scale", "kd_scale", "torque_limit_scale")
+
+    def run(act, cfg, all_buffers=False):
+        eng = engine.get_physics_engine("hip", [], {}, act, cfg)
+        ps = eng.reset(dm, 1.0, 3, N)
+        with monkeypatch.context() as mp:
+            if all_buffers:
+                mp.setattr(engine, "_constant", lambda rv, value: False)
+            for _ in range(3):
+                eng.step(action, dm, ps, 1.0, 7)
+        return ps
+
+    plain = actuators.PositionActuators(kps=(50.0,) * nu, kds=(1.0,) * nu)
+    cfg0 = engine.EngineConfig(dt=0.005, ctrl_dt=0.02)
+    a = run(plain, cfg0)
+    assert not any(seen[-1][k] for k in names)
+    b = run(plain, cfg0, all_buffers=True)
+    assert all(seen[-1][k] for k in names)
+    for k in ("qpos", "qvel", "qacc_warmstart"):
+        assert torch.equal(getattr(a.data, k), getattr(b.data, k)), k
+    assert torch.equal(a.last_ctrl, b.last_ctrl)
+    # a scale that is a constant other than 1, or anything drawn, is streamed
+    varied = actuators.PositionActuators(kps=(50.0,) * nu, kds=(1.0,) * nu, kd_scale=0.9,
+                                         torque_bias=noise.GaussianRandomVariable(0.0, 0.5))
+    run(varied, engine.EngineConfig(dt=0.005, ctrl_dt=0.02, zero_offset_std=0.01))
+    want = dict(zero_offset=True, action_bias=False, torque_bias=True, kp_scale=False, kd_scale=True, torque_limit_scale=False)
+    assert {k: seen[-1][k] for k in names} == want
+
+
 def test_sample_action_scrub_and_clip():
     from ksim_amd.env_terms import sample_action
 
