@@ -127,8 +127,12 @@ __device__ __forceinline__ void load_row(const float* p, float (&v)[NP]) {
 // left of the diagonal and the scaled column c below it, exactly what the column-oriented substitutions take,
 // once the upper lane half has handed its 16 registers to the lower one.  On return, in lane i < NP:
 //   R[j], j < i : L[i][j]              R[k], k > i : L[k][i] * L[i][i]              myinv = 1 / L[i][i]
+// `nv` (wave-uniform) is the real size: the steps of the padded columns, which would multiply zeros, are branched over
+// (only steps past the next smaller instantiation's size carry the test).
+constexpr int padded_from(int np) { return np > 28 ? 28 : (np > 24 ? 24 : (np > 16 ? 16 : (np > 8 ? 8 : 0))); }
+
 template <int NP>
-__device__ __forceinline__ void chol_tile(f32x16& T, float (&R)[NP], float& myinv, int lane) {
+__device__ __forceinline__ void chol_tile(f32x16& T, float (&R)[NP], float& myinv, int lane, int nv) {
   // The lane id is made opaque so that the per-step lane masks are compared where they are used: shared between the call
   // sites they would be sixty-odd scalar register pairs that live across the solver and are read back from spill lanes.
   asm volatile("" : "+v"(lane));
@@ -136,6 +140,7 @@ __device__ __forceinline__ void chol_tile(f32x16& T, float (&R)[NP], float& myin
   myinv = 1.f;
 #pragma unroll
   for (int j = 0; j < NP; ++j) {
+    if (j >= padded_from(NP) && j >= nv) continue;  // a padded column: unit pivot, nothing below or right of it
     const int hj = (j >> 2) & 1, rho = 4 * (j >> 3) + (j & 3);
     const float piv = fmaxf(lane_bcast(T[rho], j + 32 * hj), 1e-30f);
     const float inv = __builtin_amdgcn_rsqf(piv);
@@ -178,17 +183,19 @@ __device__ __forceinline__ void load_mtile(f32x16& T, const float* __restrict__ 
 
 // x = (L L^T)^-1 b, lane i holding b_i and returning x_i
 template <int NP>
-__device__ __forceinline__ float solve_regs(const float (&R)[NP], float myinv, int lane, float b) {
+__device__ __forceinline__ float solve_regs(const float (&R)[NP], float myinv, int lane, float b, int nv) {
   asm volatile("" : "+v"(lane));  // as in chol_tile: the masks lane > j, lane < k are rebuilt here, not kept
   float r = b;
 #pragma unroll
   for (int j = 0; j < NP; ++j) {  // L y = b; lane j keeps r_j = y_j * L[j][j]
+    if (j >= padded_from(NP) && j >= nv) continue;  // padded unknowns are zero and couple to nothing
     const float yj = lane_bcast(r * myinv, j);
     r = lane > j ? r - R[j] * yj : r;
   }
   const float myinv2 = myinv * myinv;
 #pragma unroll
   for (int k = NP - 1; k >= 0; --k) {  // L^T x = y in the scaled form  sum_{k>i} R[k] x_k + L[i][i]^2 x_i = r_i
+    if (k >= padded_from(NP) && k >= nv) continue;
     const float xk = lane_bcast(r * myinv2, k);
     r = lane < k ? r - R[k] * xk : r;
   }
@@ -786,9 +793,9 @@ void step_kernel(StepArgs a) {
     {
       f32x16 T;
       load_mtile(T, l.M, nvs, nv, NP, lane);
-      chol_tile<NP>(T, R, myinv, lane);
+      chol_tile<NP>(T, R, myinv, lane, nv);
     }
-    const float qas_all = solve_regs<NP>(R, myinv, lane, qfs);
+    const float qas_all = solve_regs<NP>(R, myinv, lane, qfs, nv);
     const float qas = is_dof ? qas_all : 0.f;  // lanes that hold no row carry meaningless numbers
     if (a.dbg_qacc_smooth && is_dof) a.dbg_qacc_smooth[env * nv + lane] = qas;
 
@@ -955,12 +962,12 @@ void step_kernel(StepArgs a) {
               for (int e = 0; e < 4; ++e) hc[4 * g + e] += (8 * g + 4 * half + e == col) ? hd : 0.f;
           }
           KS_PHASE(11)
-          chol_tile<NP>(hc, R, myinv, lane);
+          chol_tile<NP>(hc, R, myinv, lane, nv);
           am_factored = am;
           amd_factored = amd;
           have_factor = true;
         }
-        const float search_all = -solve_regs<NP>(R, myinv, lane, grad);
+        const float search_all = -solve_regs<NP>(R, myinv, lane, grad, nv);
         const float search = is_dof ? search_all : 0.f;
         KS_PHASE(12)
         // ---- exact line search along `search`
@@ -1145,8 +1152,8 @@ void step_kernel(StepArgs a) {
           for (int e = 0; e < 4; ++e) T[4 * g + e] += (8 * g + 4 * half + e == c) ? hd : 0.f;
         float R2[NP];
         float inv2;
-        chol_tile<NP>(T, R2, inv2, lane);
-        const float sol = solve_regs<NP>(R2, inv2, lane, is_dof ? Mqacc : 0.f);
+        chol_tile<NP>(T, R2, inv2, lane, nv);
+        const float sol = solve_regs<NP>(R2, inv2, lane, is_dof ? Mqacc : 0.f, nv);
         qacc_int = is_dof ? sol : 0.f;
       }
       if (is_dof) l.qvel[lane] = my_qvel + m.dt * qacc_int;
