@@ -149,7 +149,8 @@ __device__ __forceinline__ void chol_tile(f32x16& T, float (&R)[NP], float& myin
     const float t = T[rho] * inv;
     const float a = sel ? t : 0.f;
     T[rho] = sel ? t : T[rho];
-    if (j + 1 < NP) T = __builtin_amdgcn_mfma_f32_32x32x2f32(-a, a, T, 0, 0, 0);
+    // the last real column has nothing right of or below it
+    if (j + 1 < NP && !(j + 1 >= padded_from(NP) && j + 1 >= nv)) T = __builtin_amdgcn_mfma_f32_32x32x2f32(-a, a, T, 0, 0, 0);
   }
 #pragma unroll
   for (int g = 0; g < 4; ++g)
