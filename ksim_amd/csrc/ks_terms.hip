@@ -1181,7 +1181,9 @@ extern "C" int ks_terms_create(const KsTermsDesc* d, KsTerms** out) {
     if (el.src < 0 || el.src >= KS_SRC_COUNT) return fail(KS_EINVAL, "ks_terms_create: obs %d: bad source %d", k, el.src);
     if (el.kind < KS_OBS_COPY || el.kind > KS_OBS_SITE_MAGNETOMETER) return fail(KS_EINVAL, "ks_terms_create: obs %d: bad kind", k);
     if (el.kind == KS_OBS_CONTACT_ANY) {
-      if (d->ns < 1 || el.index <= 0 || (d->ns < 32 && (el.index >> d->ns) != 0)) return fail(KS_EINVAL, "ks_terms_create: obs %d: sphere mask 0x%x outside the model's %d spheres", k, el.index, d->ns);
+      // a 31-bit mask in an int field, walked with a shift per sphere: more spheres than that cannot be expressed
+      if (d->ns > 31) return fail(KS_ELIMIT, "ks_terms_create: obs %d: a contact list covers at most 31 spheres, the model has %d", k, d->ns);
+      if (d->ns < 1 || el.index <= 0 || (el.index >> d->ns) != 0) return fail(KS_EINVAL, "ks_terms_create: obs %d: sphere mask 0x%x outside the model's %d spheres", k, el.index, d->ns);
       continue;
     }
     if (el.kind == KS_OBS_SITE_ROT6D) {
@@ -1294,7 +1296,8 @@ extern "C" int ks_observe(const KsTerms* t, ks_stream_t stream, const KsObserveI
     needs_noise |= el.n_noise > 0;
     needs_bias |= el.bias.kind != KS_NOISE_NONE;
   }
-  if (needs_bias && io->noisy_obs && !io->bias_draw) return fail(KS_EINVAL, "ks_observe: observations with a bias need the bias_draw buffer");
+  // the bias is applied when noisy_obs is written and re-drawn for the envs `fresh` marks: either use touches bias_draw
+  if (needs_bias && (io->noisy_obs || io->fresh) && !io->bias_draw) return fail(KS_EINVAL, "ks_observe: observations with a bias need the bias_draw buffer");
   if (needs_quat && !io->src[KS_SRC_QPOS]) return fail(KS_EINVAL, "ks_observe: qpos is required for body-frame observations");
   if ((io->noise_normal == nullptr) != (io->noise_uniform == nullptr)) return fail(KS_EINVAL, "ks_observe: pass both explicit noise buffers or neither");
   (void)needs_noise;

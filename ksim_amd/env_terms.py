@@ -27,6 +27,23 @@ def _rng(seed: int, step: int, step_base: torch.Tensor | None = None) -> T.KsRng
     return T.KsRng(int(seed) & (2**64 - 1), int(step) & (2**64 - 1), _lib.ptr(step_base).value)
 
 
+# Sources an observation element reads besides its own `src`, per kind: the same list `ks_observe` checks for null
+# pointers before it launches.  `Rollout` keeps a derived field of the live physics data up to date only when it is in
+# the union of these sets, so a kind missing here would read the values of the last reset.
+KIND_SOURCES = {
+    T.OBS_JOINT_POS: (T.SRC_QPOS,),
+    T.OBS_ROT_INV: (T.SRC_QPOS,),
+    T.OBS_GRAVITY_EMA: (T.SRC_QPOS,),
+    T.OBS_CONTACT_ANY: (T.SRC_CONTACT_DIST,),
+    T.OBS_SITE_ROT6D: (T.SRC_XQUAT,),
+    T.OBS_SITE_GYRO: (T.SRC_XQUAT, T.SRC_CVEL),
+    T.OBS_SITE_ACCEL: (T.SRC_XQUAT, T.SRC_CVEL, T.SRC_QACC),
+    T.OBS_SITE_POS: (T.SRC_XQUAT, T.SRC_XPOS),
+    T.OBS_SITE_QUAT: (T.SRC_XQUAT,),
+    T.OBS_SITE_MAGNETOMETER: (T.SRC_XQUAT,),
+}
+
+
 def compile_terms(model: KinematicModel, observations: Mapping[str, Observation],
                   terminations: Mapping[str, Termination], resets: Sequence[Reset], command_dim: int = 0,
                   terminate_on_nonfinite: bool = True, action_dim: int | None = None):
@@ -58,14 +75,7 @@ def compile_terms(model: KinematicModel, observations: Mapping[str, Observation]
             e.e0, e.e1, e.e2, e.e3 = el.e
             e.env_site = int(el.env_site)
             sources_used.add(el.src)
-            if el.kind == T.OBS_GRAVITY_EMA:
-                sources_used.add(T.SRC_QPOS)
-            if el.kind == T.OBS_CONTACT_ANY:
-                sources_used.add(T.SRC_CONTACT_DIST)
-            if el.kind == T.OBS_SITE_ROT6D:
-                sources_used.add(T.SRC_XQUAT)
-            if el.kind in (T.OBS_SITE_GYRO, T.OBS_SITE_ACCEL):
-                sources_used.update((T.SRC_XQUAT, T.SRC_CVEL) + ((T.SRC_QACC,) if el.kind == T.OBS_SITE_ACCEL else ()))
+            sources_used.update(KIND_SOURCES.get(el.kind, ()))
             if noise is not None:
                 stages = noise.stages()
                 e.n_noise = len(stages)

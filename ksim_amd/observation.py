@@ -336,6 +336,8 @@ class ContactObservation(Observation):  # observation.py:452-478
         spheres = [int(g) for g in self.geom_idxs if g != FLOOR_GEOM]
         if any(g < 0 or g >= m.ns for g in spheres):
             raise ValueError(f"contact spheres are numbered 0..{m.ns - 1}")
+        if spheres and m.ns > 31:
+            raise ValueError(f"a contact list covers at most 31 spheres (one bit each of an int32 mask); the model has {m.ns}")
         has_floor = FLOOR_GEOM in self.geom_idxs
         mask = sum(1 << g for g in set(spheres))
         out = []

@@ -5,6 +5,8 @@ with u ~ U(-1, 1) and start[i] = base[i], or the reference-motion frame drawn fo
 `InitialMotionStateReset` governs the element.  The height-field reset looks z up from the new x, y; the heading and
 pitch / roll resets multiply the base quaternion from the right, in list order.  The resets apply in list order
 (ksim/engine.py:209-211): one that sets an element replaces what earlier ones did to it, one that adds keeps it.
+Two orderings the table cannot express raise when the list is compiled: a height draw after a height-field reset, and a
+whole-qpos motion frame after a heading or pitch / roll reset.
 Velocity resets are accepted and ignored: the engine zeroes qvel after the reset's forward pass (engine.py:217-220).
 """
 from __future__ import annotations
@@ -63,6 +65,10 @@ class RandomHeightReset(Reset):  # resets.py:322-334: qpos[2] += U(range)
 
     def apply(self, table, model):
         lo, hi = self.range
+        if table["hfield"] is not None and hi != lo:
+            # the kernel's height-field path sets z = field height + base and has no draw of its own to add
+            raise ValueError("a RandomHeightReset with a non-empty range cannot follow an HFieldXYPositionReset; list it first "
+                             "or give it a single height")
         table["base"][2] += 0.5 * (lo + hi)
         table["mag"][2] = 0.5 * (hi - lo)
         table["by_level"][2] = 0
@@ -148,6 +154,10 @@ class InitialMotionStateReset(Reset):  # resets.py:284-306
         q = np.asarray(getattr(self.reference_motion.qpos, "array", self.reference_motion.qpos), dtype=np.float32)
         if q.ndim != 2 or q.shape[1] != model.nq:
             raise ValueError(f"the reference motion has frames of {q.shape[-1]} numbers, the model's qpos has {model.nq}")
+        if self.freejoint and (table["heading"] or table["pitch_roll"]):
+            # the kernel turns the base quaternion after the table pass, so it cannot replace a turn made earlier
+            raise ValueError("an InitialMotionStateReset(freejoint=True) cannot follow a heading or pitch / roll reset: it "
+                             "would have to replace the base orientation they set; list it before them")
         sl = slice(0, model.nq) if self.freejoint else slice(7, model.nq)
         table["motion"][sl] = 1
         table["base"][sl] = 0.0

@@ -262,9 +262,13 @@ def far_from_origin_termination(qpos, max_dist, pos_termination=True):  # termin
     return np.where(np.linalg.norm(np.asarray(qpos)[..., :3], axis=-1) > max_dist, val, 0).astype(np.int32)
 
 
-def episode_length_termination(time, max_length_sec, pos_termination=True):  # terminations.py:186-192
+def episode_length_termination(time, max_length_sec, pos_termination=True, level=0.0,
+                               disable_at_curriculum_level=None):  # terminations.py:186-192
     val = 1 if pos_termination else -1
-    return np.where(np.asarray(time) > max_length_sec, val, 0).astype(np.int32)
+    long_episodes = np.where(np.asarray(time) > max_length_sec, val, 0).astype(np.int32)
+    if disable_at_curriculum_level is not None:  # terminations.py:188-190: off below that curriculum level
+        return np.where(np.asarray(level) < disable_at_curriculum_level, 0, long_episodes).astype(np.int32)
+    return long_episodes
 
 
 def illegal_contact_termination(ncon, geom1, geom2, dist, illegal_geom_idxs, contact_eps=-1e-3):  # terminations.py:90-99

@@ -722,3 +722,57 @@ def test_motion_resets_symmetry_rewards_and_imu_misalignment_in_the_rollout():
     frames = (after - 0.02) / 0.02
     assert np.abs(frames - np.round(frames)).max() < 1e-4 and frames.min() > -1e-4 and frames.max() < F - 1 + 1e-4
     assert float(carry.abs().max()) > 1e-3
+
+
+def test_site_frame_sensors_follow_the_live_state_in_a_rollout():
+    """A task whose only observations of derived fields are site frame sensors (`framepos` reads xpos and, to turn the
+    site offset, xquat; `framequat` and `magnetometer` read xquat): the rollout must keep both fields of the live state
+    up to date, so the observation of step t + 1 equals the sensor formula on what step t recorded.  With a stale
+    quaternion the foot position would stay that of the reset pose's orientation."""
+    from ksim_amd import _lib_terms as T, actuators, engine, observation as ob, physics, resets as rs, rewards as rw
+    from ksim_amd import terminations as tm
+    from ksim_amd.env_terms import EnvTerms
+    from ksim_amd.mjcf import load_mjcf
+    from ksim_amd.mlp import MLP
+    from ksim_amd.rollout import Rollout, RolloutConstants, RolloutEnvState
+
+    m = load_mjcf(os.path.join(os.path.dirname(__file__), "golden", "mini_biped.mjcf"))
+    N, Tn = 16, 6
+    rng = np.random.default_rng(41)
+    act = actuators.PositionActuators(kps=(30.0,) * m.nu, kds=(1.0,) * m.nu, ctrl_clip=(20.0,) * m.nu)
+    resets = [rs.RandomJointPositionReset(scale=0.2, scale_by_curriculum=False)]
+    eng = engine.get_physics_engine("hip", resets, {}, act, engine.EngineConfig(dt=0.005, ctrl_dt=0.02))
+    observations = {"jp": ob.JointPositionObservation(),
+                    "foot": ob.SensorObservation.create(physics_model=m, sensor_name="left_foot_pos"),
+                    "quat": ob.SensorObservation.create(physics_model=m, sensor_name="imu_quat")}
+    terms = EnvTerms(m, observations, {"h": tm.MinimumHeightTermination(0.05)}, resets)
+    assert T.SRC_XQUAT in terms.sources_used and T.SRC_XPOS in terms.sources_used
+    dims = (terms.obs_dim, 32, m.nu)
+    ws = [rng.normal(scale=1 / np.sqrt(i), size=(o, i)).astype(np.float32) for i, o in zip(dims[:-1], dims[1:])]
+    bs = [np.zeros(o, np.float32) for o in dims[1:]]
+    consts = RolloutConstants(physics_model=physics.DeviceModel(m), engine=eng, terms=terms,
+                              rewards={"alive": rw.StayAliveReward(scale=1.0)}, actor=MLP(ws, bs, dtype="f32"), critic=None,
+                              log_std=t32(np.full(m.nu, -1.0)))
+    ro = Rollout(consts, N, Tn)
+    assert {"xpos", "xquat"} <= ro._live
+    ps = eng.reset(consts.physics_model, 1.0, 0, N, {})
+    env = RolloutEnvState(ps, {}, None, None, seed=3)
+    for t in range(Tn):
+        ro.step_engine(env, t, 1.0)
+    sl = terms.obs_slices
+    obs = ro.obs.cpu().numpy().astype(np.float64)
+    xp = ro.xpos.cpu().numpy().reshape(Tn, N, m.nb, 3).astype(np.float64)
+    xq = ro.xquat.cpu().numpy().reshape(Tn, N, m.nb, 4).astype(np.float64)
+    done = ro.done.cpu().numpy().astype(bool)
+    fb, fpos, _ = m.sites["left_foot"]
+    ib, _, iquat = m.sites["imu_site"]
+    checked = 0
+    for t in range(Tn - 1):
+        keep = ~done[t]  # an env that was reset observes its new pose, which the slot of step t does not hold
+        np.testing.assert_allclose(obs[t + 1][keep][:, sl["foot"]], ot.site_frame_position(xp[t][keep][:, fb], xq[t][keep][:, fb], fpos),
+                                   rtol=1e-5, atol=2e-6)
+        np.testing.assert_allclose(obs[t + 1][keep][:, sl["quat"]], ot.site_frame_quaternion(xq[t][keep][:, ib], iquat), rtol=1e-5, atol=2e-6)
+        checked += int(keep.sum())
+    assert checked > N
+    # the poses do change over the rollout, so a stale field could not have passed
+    assert np.abs(xq[Tn - 1][:, fb] - xq[0][:, fb]).max() > 1e-3

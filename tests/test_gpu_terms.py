@@ -105,6 +105,9 @@ def test_observation_assembly_and_noise():
     np.testing.assert_allclose(wb, ot.same_key_uniform(zb), atol=2e-6)
     with pytest.raises(Exception, match="bias_draw"):
         terms.observe(src, N, zero_offset=t32(s["zero"]), noisy_obs=a1)
+    # a fresh mask alone makes the kernel re-draw the biases into bias_draw: refused on the host before any launch
+    with pytest.raises(Exception, match="bias_draw"):
+        terms.observe(src, N, zero_offset=t32(s["zero"]), obs=a1, fresh=torch.ones(N, dtype=torch.uint8, device=DEV))
     z = ((a1 - obs)[:, sl["joint_position"]] / 0.01).flatten()
     assert abs(z.mean().item()) < 0.15 and abs(z.std().item() - 1.0) < 0.15
 
@@ -145,22 +148,34 @@ def test_termination_kats_and_masks_bit_exact():
         "min_height": tm.MinimumHeightTermination(0.5), "bad_z": tm.BadZTermination(-1.0, 2.0, -0.5, 1.5),
         "not_upright": tm.NotUprightTermination(1.2), "bad_vel": tm.BadVelocityTermination(2.5),
         "far": tm.FarFromOriginTermination(3.0), "length": tm.EpisodeLengthTermination(1.5),
+        # the curriculum switch of the length term (terminations.py:188-190) on both sides of the level, and the
+        # negative variants of the two terms that default to a positive termination
+        "length_off": tm.EpisodeLengthTermination(1.5, disable_at_curriculum_level=1),
+        "length_on": tm.EpisodeLengthTermination(1.5, disable_at_curriculum_level=0.25, pos_termination=False),
+        "length_at": tm.EpisodeLengthTermination(1.5, disable_at_curriculum_level=0.4),
+        "far_neg": tm.FarFromOriginTermination(2.0, pos_termination=False),
     }
     terms = EnvTerms(m, {}, term_objs, [])
     level = 0.4
-    comps = torch.zeros(6, N, dtype=torch.int8, device=DEV)
+    comps = torch.zeros(len(term_objs), N, dtype=torch.int8, device=DEV)
     done = torch.zeros(N, dtype=torch.uint8, device=DEV); succ = torch.zeros(N, dtype=torch.uint8, device=DEV)
     q32, v32, t32_ = s["qpos"].astype(np.float32), s["qvel"].astype(np.float32), s["time"].astype(np.float32)
     terms.terminate_reset(dict(qpos=t32(q32), qvel=t32(v32), time=t32(t32_)), level=level, components=comps, done=done,
                           success=succ, apply_reset=False)
     want = [ot.minimum_height_termination(q32, np.float32(0.5)), ot.bad_z_termination(q32, -1.0, 2.0, np.float32(level), -0.5, 1.5),
             ot.not_upright_termination(q32, 1.2), ot.bad_velocity_termination(v32, 2.5),
-            ot.far_from_origin_termination(q32, 3.0), ot.episode_length_termination(t32_, 1.5)]
+            ot.far_from_origin_termination(q32, 3.0), ot.episode_length_termination(t32_, 1.5),
+            ot.episode_length_termination(t32_, 1.5, True, np.float32(level), 1),
+            ot.episode_length_termination(t32_, 1.5, False, np.float32(level), 0.25),
+            ot.episode_length_termination(t32_, 1.5, True, np.float32(level), np.float32(0.4)),
+            ot.far_from_origin_termination(q32, 2.0, pos_termination=False)]
+    assert not want[6].any() and (want[7] == -1).sum() > 20 and np.array_equal(want[8], want[5])
     got = comps.cpu().numpy()
     # exclude the measure-zero band where fp32 and float64 evaluation of a norm/acos straddle the threshold
     near = np.zeros(N, bool)
     near |= np.abs(np.linalg.norm(v32[:, :3], axis=1) - 2.5) < 1e-5
     near |= np.abs(np.linalg.norm(q32[:, :3], axis=1) - 3.0) < 1e-5
+    near |= np.abs(np.linalg.norm(q32[:, :3], axis=1) - 2.0) < 1e-5
     for j, w in enumerate(want):
         assert np.array_equal(got[j][~near], w[~near]), list(term_objs)[j]
     wd, ws = ot.combine_terminations([g for g in got])

@@ -460,3 +460,64 @@ def test_generic_noise_and_bias_over_random_variables():
     assert isinstance(kn.AdditiveBias(kn.ZeroRandomVariable()), kn.Bias) and kn.AdditiveNoise(kn.ZeroRandomVariable()).scale == 0.0
     with pytest.raises(ValueError, match="one key"):
         kn.AdditiveNoise(kn.RandomVariable(mean=0.0, mag=0.1, std=0.1, same_key=False))
+
+
+def test_observation_kinds_declare_every_source_they_read():
+    """The rollout refreshes a derived field of the live state only when an observation declares it: a site position reads
+    xpos and the body quaternion that turns the site offset, the other frame sensors the quaternion."""
+    from ksim_amd.env_terms import KIND_SOURCES
+    from ksim_amd.mjcf import load_mjcf
+
+    m = load_mjcf(os.path.join(os.path.dirname(__file__), "golden", "mini_biped.mjcf"))
+    one = lambda name: compile_terms(m, {name: ob.SensorObservation.create(physics_model=m, sensor_name=name)}, {}, [])[2]  # noqa: E731
+    assert {T.SRC_XPOS, T.SRC_XQUAT} <= one("left_foot_pos")
+    assert T.SRC_XQUAT in one("imu_quat") and T.SRC_XQUAT in one("imu_mag")
+    assert {T.SRC_XQUAT, T.SRC_CVEL} <= one("imu_gyro") and {T.SRC_XQUAT, T.SRC_CVEL, T.SRC_QACC} <= one("imu_acc")
+    site_kinds = (T.OBS_SITE_GYRO, T.OBS_SITE_ACCEL, T.OBS_SITE_ROT6D, T.OBS_SITE_POS, T.OBS_SITE_QUAT, T.OBS_SITE_MAGNETOMETER)
+    assert all(T.SRC_XQUAT in KIND_SOURCES[k] for k in site_kinds)
+
+
+def test_reset_orders_the_table_cannot_express_raise():
+    m = km.kbot_scale_model()
+    field = rs.HFieldXYPositionReset(bounds=(5.0, 5.0, 0.0, 0.0), hfield_data=np.zeros((4, 4)))
+    with pytest.raises(ValueError, match="RandomHeightReset"):
+        rs.compile_resets([field, rs.RandomHeightReset(range=(0.0, 0.2))], m)
+    tab = rs.compile_resets([rs.RandomHeightReset(range=(0.0, 0.2)), field], m)  # listed first: replaced, as in the reference
+    assert tab["mag"][2] == 0.0 and tab["base"][2] == 0.0
+    tab = rs.compile_resets([field, rs.RandomHeightReset(range=(0.3, 0.3))], m)  # a single height only shifts the base
+    assert tab["base"][2] == pytest.approx(0.3)
+
+    class Motion:
+        qpos = np.tile(m.qpos0, (5, 1)).astype(np.float32)
+        ctrl_dt = 0.02
+
+    for first in (rs.RandomHeadingReset(), rs.RandomPitchRollReset()):
+        with pytest.raises(ValueError, match="freejoint"):
+            rs.compile_resets([first, rs.InitialMotionStateReset(reference_motion=Motion, freejoint=True)], m)
+        rs.compile_resets([first, rs.InitialMotionStateReset(reference_motion=Motion, freejoint=False)], m)
+        rs.compile_resets([rs.InitialMotionStateReset(reference_motion=Motion, freejoint=True), first], m)
+    with pytest.raises(ValueError, match="31 spheres"):
+        big = type("M", (), {"ns": 40})()
+        ob.ContactObservation(geom_idxs=(ob.FLOOR_GEOM, 3)).elements(big, 0)
+
+
+def test_committed_traffic_profiles_carry_sane_calibration_factors():
+    """The HBM-traffic summaries scale FETCH_SIZE / WRITE_SIZE by what the same counter reads for a 256 MiB copy: that factor
+    is about 2 for reads and 1 for writes on this part.  A factor far from that means the calibration dispatch was mixed
+    up with other launches, and every figure of the file is wrong by the same ratio."""
+    import glob
+    import re
+
+    files = sorted(glob.glob(os.path.join(os.path.dirname(__file__), "..", "profiles", "*traffic*.txt")))
+    assert files
+    for path in files:
+        text = open(path).read()
+        factors = [float(x) for x in re.findall(r"(?:FETCH|WRITE) x ([0-9.]+?)[,\s]", text)]
+        factors += [float(x) for x in re.findall(r"factor ([0-9.]+)", text)]
+        assert factors, f"{os.path.basename(path)} states no calibration factor"
+        for f in factors:
+            assert 0.5 <= f <= 4.0, f"{os.path.basename(path)}: calibration factor {f}"
+        for ratio in re.findall(r"^[^#\n]*\|[^\n]*$", text, flags=re.M):  # data rows: the traffic / algorithmic column
+            cols = [c.strip() for c in ratio.split("|")]
+            if len(cols) >= 9 and re.fullmatch(r"[0-9.]+", cols[5]):
+                assert float(cols[5]) < 4.0, f"{os.path.basename(path)}: traffic / algorithmic {cols[5]} in {cols[0]}"

@@ -36,6 +36,92 @@ def test_termination_kats(kat):
     assert int(got) == kat["expected"]
 
 
+def _q(x=0.0, y=0.0, z=0.0):
+    q = np.zeros(9)
+    q[:3] = x, y, z
+    q[3] = 1.0
+    return q
+
+
+def test_bad_z_termination_hand_computed():
+    """terminations.py:139-146: the bounds move linearly from (min_z, max_z) at level 0 to the final pair at level 1,
+    both comparisons are strict, the value is always -1.  Expected values are written out by hand."""
+    kw = dict(min_z=-1.0, max_z=2.0, final_min_z=0.0, final_max_z=1.0)
+    # level 0: bounds (-1, 2); level 0.5: (-0.5, 1.5); level 1: (0, 1)
+    cases = [
+        (0.0, -1.25, -1), (0.0, -1.0, 0), (0.0, -0.75, 0), (0.0, 1.75, 0), (0.0, 2.0, 0), (0.0, 2.25, -1),
+        (0.5, -0.75, -1), (0.5, -0.5, 0), (0.5, -0.25, 0), (0.5, 1.25, 0), (0.5, 1.5, 0), (0.5, 1.75, -1),
+        (1.0, -0.25, -1), (1.0, 0.0, 0), (1.0, 0.25, 0), (1.0, 0.75, 0), (1.0, 1.0, 0), (1.0, 1.25, -1),
+    ]
+    for level, z, want in cases:
+        assert int(ot.bad_z_termination(_q(z=z), level=level, **kw)) == want, (level, z)
+    # a point that is healthy at level 0 and unhealthy at level 1 on either side tells the interpolation direction
+    assert int(ot.bad_z_termination(_q(z=-0.5), level=0.0, **kw)) == 0 and int(ot.bad_z_termination(_q(z=-0.5), level=1.0, **kw)) == -1
+    assert int(ot.bad_z_termination(_q(z=1.5), level=0.0, **kw)) == 0 and int(ot.bad_z_termination(_q(z=1.5), level=1.0, **kw)) == -1
+    # without final bounds the level changes nothing; only the z coordinate matters
+    for level in (0.0, 0.3, 1.0):
+        assert int(ot.bad_z_termination(_q(x=9.0, y=-9.0, z=0.5), -1.0, 2.0, level)) == 0
+        assert int(ot.bad_z_termination(_q(z=-1.5), -1.0, 2.0, level)) == -1
+        assert int(ot.bad_z_termination(_q(z=2.5), -1.0, 2.0, level)) == -1
+    # only one final bound given: the other stays where it was
+    assert int(ot.bad_z_termination(_q(z=1.75), -1.0, 2.0, 1.0, final_min_z=0.0)) == 0
+    assert int(ot.bad_z_termination(_q(z=-0.5), -1.0, 2.0, 1.0, final_min_z=0.0)) == -1
+    got = ot.bad_z_termination(np.stack([_q(z=-2.0), _q(z=0.5), _q(z=3.0)]), -1.0, 2.0)
+    assert got.dtype == np.int32 and got.tolist() == [-1, 0, -1]
+
+
+def test_bad_velocity_termination_hand_computed():
+    """terminations.py:155-157: Euclidean norm of the three linear root velocities only, strictly above the limit, -1."""
+    v = np.zeros(8)
+    v[:3] = 3.0, 4.0, 0.0  # |v| = 5 exactly
+    assert int(ot.bad_velocity_termination(v, 5.0)) == 0  # on the limit: strict
+    assert int(ot.bad_velocity_termination(v, 4.999)) == -1
+    assert int(ot.bad_velocity_termination(v, 5.001)) == 0
+    v[:3] = 0.0, -3.0, 4.0  # sign and axis do not matter
+    assert int(ot.bad_velocity_termination(v, 4.999)) == -1
+    v[:3] = 2.0, 2.0, 1.0  # |v| = 3: a norm, not a sum of magnitudes (5) nor a maximum (2)
+    assert int(ot.bad_velocity_termination(v, 2.9)) == -1 and int(ot.bad_velocity_termination(v, 3.1)) == 0
+    v[:3] = 0.1, 0.0, 0.0
+    v[3:] = 100.0  # angular and joint velocities must not count
+    assert int(ot.bad_velocity_termination(v, 1.0)) == 0
+    got = ot.bad_velocity_termination(np.array([[3.0, 4.0, 0.0, 0, 0, 0], [3.0, 4.0, 0.1, 0, 0, 0]]), 5.0)
+    assert got.dtype == np.int32 and got.tolist() == [0, -1]
+
+
+def test_far_from_origin_termination_hand_computed():
+    """terminations.py:170-172: norm of the root position (x, y, z) strictly above max_dist; +1 by default."""
+    q = _q(3.0, 0.0, 4.0)  # distance 5 exactly; z counts
+    assert int(ot.far_from_origin_termination(q, 5.0)) == 0
+    assert int(ot.far_from_origin_termination(q, 4.999)) == 1  # default is a positive termination
+    assert int(ot.far_from_origin_termination(q, 4.999, pos_termination=True)) == 1
+    assert int(ot.far_from_origin_termination(q, 4.999, pos_termination=False)) == -1
+    assert int(ot.far_from_origin_termination(q, 5.001, pos_termination=False)) == 0
+    q = _q(-1.0, -2.0, 2.0)  # distance 3; the quaternion entries (w = 1) must not count
+    assert int(ot.far_from_origin_termination(q, 2.9)) == 1 and int(ot.far_from_origin_termination(q, 3.05)) == 0
+    got = ot.far_from_origin_termination(np.stack([_q(0.1), _q(0.0, 6.0)]), 5.0, pos_termination=False)
+    assert got.dtype == np.int32 and got.tolist() == [0, -1]
+
+
+def test_episode_length_termination_hand_computed():
+    """terminations.py:186-192: time strictly above the limit; +1 by default; with disable_at_curriculum_level the term is
+    off while the level is strictly below it."""
+    assert int(ot.episode_length_termination(10.0, 10.0)) == 0  # on the limit: strict
+    assert int(ot.episode_length_termination(10.005, 10.0)) == 1
+    assert int(ot.episode_length_termination(9.995, 10.0)) == 0
+    assert int(ot.episode_length_termination(10.005, 10.0, pos_termination=False)) == -1
+    assert int(ot.episode_length_termination(9.995, 10.0, pos_termination=False)) == 0
+    # disabled below level 2, active from level 2 on (the comparison is level < disable)
+    for level, want in ((0.0, 0), (1.0, 0), (1.999, 0), (2.0, 1), (3.0, 1)):
+        assert int(ot.episode_length_termination(10.005, 10.0, True, level, 2)) == want, level
+        assert int(ot.episode_length_termination(10.005, 10.0, False, level, 2)) == -want, level
+        assert int(ot.episode_length_termination(9.0, 10.0, True, level, 2)) == 0
+    # a disable level of 0 never disables (no level is below it); None ignores the level altogether
+    assert int(ot.episode_length_termination(10.005, 10.0, True, 0.0, 0)) == 1
+    assert int(ot.episode_length_termination(10.005, 10.0, True, 0.0, None)) == 1
+    got = ot.episode_length_termination(np.array([1.0, 11.0, 11.0]), 10.0, True, np.array([5.0, 5.0, 1.0]), 2)
+    assert got.dtype == np.int32 and got.tolist() == [0, 1, 0]
+
+
 def test_done_success_truth_table():
     for k in (1, 2, 3):
         for combo in itertools.product([-1, 0, 1], repeat=k):
