@@ -796,6 +796,26 @@ int ks_grad_sqnorm(ks_stream_t stream, int64_t n, const float* g, double* acc);
  *                         a critic n = 1, perm = {0}, sign = {1}: scale * (v - vm)^2, train.py:1477), and the gradient of
  *                         mean_r loss[r] is ADDED to dy and WRITTEN to dym.  perm must be a permutation of 0..n-1.
  * The loss joins the PPO loss as an auxiliary term (ksim/task/ppo.py:241-244, 485-486: mean over rows of the sum of terms). */
+/* The low-pass filter on the actor's means inside the loss of the K-Bot task: run_actor filters the biased means with
+ * ksim.lowpass_one_pole (examples/kbot/train.py:923-929, ksim/actions.py:248-257) and the filter state `lpf_params` is part
+ * of the model carry that the scan over the trajectory threads through time and restarts with the episode
+ * (train.py:1439-1451, 1506-1515, 1529-1533).
+ *   ks_lowpass_scan           rows (t, m) of ld floats; the first nu columns are the means:
+ *                             y_t = y_{t-1} + alpha (x_t + mean_bias + add_t - y_{t-1}), alpha = dt / (1 / (2 pi cutoff) + dt),
+ *                             y_{-1} = y0[m] (NULL: zero), and y_{t-1} = 0 at the steps flagged in fresh (T, M).  `add`
+ *                             (nullable) is the command-dependent bias read from the observation rows (train.py:920-921):
+ *                             add[(t M + m) add_ld + k] joins joint add_first + k, k < add_count.  Columns nu..ld-1 are
+ *                             copied (x == y is allowed and filters in place).  y_last (M, nu), nullable, receives the carry
+ *                             after the last step.  With T = 1 this is the rollout's own filter step.
+ *   ks_lowpass_scan_backward  the reverse sweep jax.grad derives through that scan: g holds dL/dy in its first nu columns
+ *                             on entry and dL/dx on return (G_t = g_t + (1 - alpha) G_{t+1}, cut where step t + 1 is
+ *                             fresh; dx_t = alpha G_t); d_y0 (M, nu), nullable, receives the gradient of the initial carry. */
+int ks_lowpass_scan(ks_stream_t stream, int64_t T, int64_t M, int32_t nu, int32_t ld, float ctrl_dt, float cutoff,
+                    const float* x, const float* mean_bias /*(nu) nullable*/, const float* add /*nullable*/, int64_t add_ld,
+                    int32_t add_first, int32_t add_count, const float* y0 /*(M,nu) nullable*/,
+                    const uint8_t* fresh /*(T,M) nullable*/, float* y, float* y_last /*(M,nu) nullable*/);
+int ks_lowpass_scan_backward(ks_stream_t stream, int64_t T, int64_t M, int32_t nu, int32_t ld, float ctrl_dt, float cutoff,
+                             const uint8_t* fresh /*(T,M) nullable*/, float* g /*(T,M,ld) in place*/, float* d_y0 /*nullable*/);
 int ks_signed_permute(ks_stream_t stream, int64_t rows, int32_t n, const float* x, const int32_t* perm, const float* sign,
                       float* out);
 int ks_mirror_loss_grad(ks_stream_t stream, int64_t rows, int32_t n, float scale, const float* y, const float* ym,

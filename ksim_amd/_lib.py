@@ -65,6 +65,10 @@ def load() -> ctypes.CDLL:
     lib.ks_signed_permute.restype = c_int32
     lib.ks_mirror_loss_grad.argtypes = [p, c_int64, c_int32, c_float, p, p, p, p, p, p, p]
     lib.ks_mirror_loss_grad.restype = c_int32
+    lib.ks_lowpass_scan.argtypes = [p, c_int64, c_int64, c_int32, c_int32, c_float, c_float, p, p, p, c_int64, c_int32, c_int32, p, p, p, p]
+    lib.ks_lowpass_scan.restype = c_int32
+    lib.ks_lowpass_scan_backward.argtypes = [p, c_int64, c_int64, c_int32, c_int32, c_float, c_float, p, p, p]
+    lib.ks_lowpass_scan_backward.restype = c_int32
     lib.ks_ppo_adapt_kl.argtypes = [p, c_int64, c_int32, p, p, c_float, c_float, p, p]
     lib.ks_ppo_adapt_kl.restype = c_int32
     for name in ("ks_gae_bt", "ks_gae_tn", "ks_normalize_advantages", "ks_ppo_loss", "ks_reward_total", "ks_copy_f32"):

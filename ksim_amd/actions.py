@@ -41,6 +41,18 @@ def _run(kind, x, position=None, velocity=None, *, ctrl_dt=0.0, p0=0.0, lo=None,
 
 
 @dataclass(frozen=True)
+class LowPass:
+    """ksim.lowpass_one_pole on an actor's biased means (examples/kbot/train.py:917-929, ksim/actions.py:248-257), as a
+    setting of the policy head: the rollout filters the means before sampling and the policy update differentiates through
+    the filter, whose state `lpf_params` rides in the model carry.  `obs_bias` = (first observation column, first action,
+    count): that many action means also take the named observation columns as a bias before the filter (the arm commands
+    of train.py:920-921)."""
+    ctrl_dt: float
+    cutoff_frequency: float
+    obs_bias: tuple | None = None
+
+
+@dataclass(frozen=True)
 class LowPassFilterParams:  # actions.py:236-245
     y_last: torch.Tensor
 

@@ -830,6 +830,59 @@ __global__ __launch_bounds__(256) void kl_adapt_kernel(int nblocks, float inv_ro
   }
 }
 
+// One-pole low-pass along the time axis of a trajectory, one thread per (env column, joint), walking the T steps in order:
+// y_t = y_{t-1} + alpha (x_t + bias - y_{t-1}), y_{t-1} = 0 at the steps flagged fresh (the carry restarts with the
+// episode) and y0 before the first step.  Rows are (t, m) with ld floats each; the first nu columns hold the signal, the
+// others travel unchanged.  `add` is an observation-dependent part of the bias: add[(t M + m) add_ld + k] joins joint
+// add_first + k.
+__global__ __launch_bounds__(256) void lowpass_scan_kernel(int64_t T, int64_t M, int nu, int ld, float alpha,
+                                                           const float* __restrict__ x, const float* __restrict__ mean_bias,
+                                                           const float* __restrict__ add, int64_t add_ld, int add_first, int add_count,
+                                                           const float* __restrict__ y0, const uint8_t* __restrict__ fresh,
+                                                           float* __restrict__ y, float* __restrict__ y_last) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= M * (int64_t)ld) return;
+  const int64_t m = idx / ld;
+  const int j = (int)(idx - m * ld);
+  if (j >= nu) {  // the columns behind the signal (raw deviations of the head): copied when the output is another buffer
+    if (x != y)
+      for (int64_t t = 0; t < T; ++t) y[(t * M + m) * ld + j] = x[(t * M + m) * ld + j];
+    return;
+  }
+  const float b = mean_bias ? mean_bias[j] : 0.f;
+  const bool has_add = add && j >= add_first && j < add_first + add_count;
+  float last = y0 ? y0[m * nu + j] : 0.f;
+  for (int64_t t = 0; t < T; ++t) {
+    const int64_t r = t * M + m;
+    if (fresh && fresh[r]) last = 0.f;
+    float v = x[r * ld + j] + b;
+    if (has_add) v += add[r * add_ld + (j - add_first)];
+    last = last + alpha * (v - last);
+    y[r * ld + j] = last;
+  }
+  if (y_last) y_last[m * nu + j] = last;
+}
+
+// Reverse sweep of the same recursion: with g_t = dL/dy_t on entry, the gradient reaching y_t is
+// G_t = g_t + (1 - alpha) G_{t+1} unless step t + 1 is fresh (the carry was cut there), and dL/dx_t = alpha G_t, written in
+// place.  d_y0 receives (1 - alpha) G_0 unless step 0 is fresh.
+__global__ __launch_bounds__(256) void lowpass_scan_backward_kernel(int64_t T, int64_t M, int nu, int ld, float alpha,
+                                                                    const uint8_t* __restrict__ fresh, float* __restrict__ g,
+                                                                    float* __restrict__ d_y0) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= M * (int64_t)nu) return;
+  const int64_t m = idx / nu;
+  const int j = (int)(idx - m * nu);
+  float carry = 0.f;  // (1 - alpha) G_{t+1}, or 0 across an episode start
+  for (int64_t t = T - 1; t >= 0; --t) {
+    const int64_t r = t * M + m;
+    const float G = g[r * ld + j] + carry;
+    g[r * ld + j] = alpha * G;
+    carry = (fresh && fresh[r]) ? 0.f : (1.f - alpha) * G;
+  }
+  if (d_y0) d_y0[idx] = carry;
+}
+
 // mirrored rows: out[r][j] = sign[j] * x[r][perm[j]]
 __global__ __launch_bounds__(256) void signed_permute_kernel(int64_t total, int n, const float* __restrict__ x, const int* __restrict__ perm,
                                                              const float* __restrict__ sign, float* __restrict__ out) {
@@ -867,6 +920,40 @@ __global__ __launch_bounds__(256) void mirror_loss_grad_kernel(int64_t rows, int
 }
 
 }  // namespace ks
+
+static float lowpass_alpha(float ctrl_dt, float cutoff) {  // actions.py:254-255, in float like ks_action_filter
+  return ctrl_dt / (1.f / (6.28318530717958647692f * cutoff) + ctrl_dt);
+}
+
+extern "C" int ks_lowpass_scan(ks_stream_t stream, int64_t T, int64_t M, int32_t nu, int32_t ld, float ctrl_dt, float cutoff,
+                               const float* x, const float* mean_bias, const float* add, int64_t add_ld, int32_t add_first,
+                               int32_t add_count, const float* y0, const uint8_t* fresh, float* y, float* y_last) {
+  if (T < 0 || M < 0 || nu < 1 || ld < nu) return ks::fail(KS_EINVAL, "ks_lowpass_scan: bad shape (T %lld, M %lld, nu %d, ld %d)", (long long)T, (long long)M, nu, ld);
+  if (!(ctrl_dt > 0.f) || !(cutoff > 0.f)) return ks::fail(KS_EINVAL, "ks_lowpass_scan: ctrl_dt and the cutoff frequency must be positive");
+  if (T == 0 || M == 0) return KS_OK;
+  if (!x || !y) return ks::fail(KS_EINVAL, "ks_lowpass_scan: null pointer");
+  if (add && (add_first < 0 || add_count < 1 || add_first + add_count > nu || add_ld < add_count))
+    return ks::fail(KS_EINVAL, "ks_lowpass_scan: the additive bias covers joints [%d, %d) of %d with rows of %lld floats", add_first,
+                    add_first + add_count, nu, (long long)add_ld);
+  const int64_t total = M * ld, grid = (total + 255) / 256;
+  if (grid > 0x7fffffff) return ks::fail(KS_ELIMIT, "ks_lowpass_scan: too many elements");
+  hipLaunchKernelGGL(ks::lowpass_scan_kernel, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, T, M, nu, ld,
+                     lowpass_alpha(ctrl_dt, cutoff), x, mean_bias, add, add_ld, add_first, add_count, y0, fresh, y, y_last);
+  return ks::check_launch("ks_lowpass_scan");
+}
+
+extern "C" int ks_lowpass_scan_backward(ks_stream_t stream, int64_t T, int64_t M, int32_t nu, int32_t ld, float ctrl_dt, float cutoff,
+                                        const uint8_t* fresh, float* g, float* d_y0) {
+  if (T < 0 || M < 0 || nu < 1 || ld < nu) return ks::fail(KS_EINVAL, "ks_lowpass_scan_backward: bad shape");
+  if (!(ctrl_dt > 0.f) || !(cutoff > 0.f)) return ks::fail(KS_EINVAL, "ks_lowpass_scan_backward: ctrl_dt and the cutoff frequency must be positive");
+  if (T == 0 || M == 0) return KS_OK;
+  if (!g) return ks::fail(KS_EINVAL, "ks_lowpass_scan_backward: null pointer");
+  const int64_t total = M * nu, grid = (total + 255) / 256;
+  if (grid > 0x7fffffff) return ks::fail(KS_ELIMIT, "ks_lowpass_scan_backward: too many elements");
+  hipLaunchKernelGGL(ks::lowpass_scan_backward_kernel, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, T, M, nu, ld,
+                     lowpass_alpha(ctrl_dt, cutoff), fresh, g, d_y0);
+  return ks::check_launch("ks_lowpass_scan_backward");
+}
 
 extern "C" int ks_signed_permute(ks_stream_t stream, int64_t rows, int32_t n, const float* x, const int32_t* perm, const float* sign,
                                  float* out) {

@@ -19,6 +19,7 @@ import torch
 from . import _lib
 from . import _lib_terms as T
 from . import ppo as ppo_mod
+from .actions import LowPass
 from .mlp import MLP
 
 
@@ -68,10 +69,13 @@ class MirrorSpec:
                 raise ValueError(f"{name}: the mirror map must be a permutation with one sign per entry")
 
     def device(self, name: str, dev) -> tuple[torch.Tensor, torch.Tensor]:
-        if name not in self._dev:
-            self._dev[name] = (torch.tensor(list(getattr(self, name + "_perm")), dtype=torch.int32, device=dev),
-                               torch.tensor(list(getattr(self, name + "_sign")), dtype=torch.float32, device=dev))
-        return self._dev[name]
+        """(perm int32, sign float32) of one of the maps on `dev`; "value" is the critic output's own map, one entry kept
+        as it is.  Cached per (map, device)."""
+        key = (name, str(torch.device(dev)))
+        if key not in self._dev:
+            perm, sign = ([0], [1.0]) if name == "value" else (list(getattr(self, name + "_perm")), list(getattr(self, name + "_sign")))
+            self._dev[key] = (torch.tensor(perm, dtype=torch.int32, device=dev), torch.tensor(sign, dtype=torch.float32, device=dev))
+        return self._dev[key]
 
 
 def kbot_mirror_joints() -> tuple[list[int], list[float]]:
@@ -178,9 +182,7 @@ def single_step(policy: GaussianMlpPolicy, cfg: PPOUpdateConfig, actor_obs, crit
                                            _lib.ptr(perm), _lib.ptr(sign), _lib.ptr(d_mean), _lib.ptr(d_mean_all[rows:]),
                                            _lib.ptr(aux["action_mirror_loss"])))
     if mirror_c:
-        if "_one" not in policy.mirror._dev:
-            policy.mirror._dev["_one"] = (torch.zeros(1, dtype=torch.int32, device=mean.device), torch.ones(1, device=mean.device))
-        perm, sign = policy.mirror._dev["_one"]
+        perm, sign = policy.mirror.device("value", mean.device)
         aux["value_mirror_loss"] = torch.empty(rows, dtype=torch.float32, device=mean.device)
         _lib.check(lib.ks_mirror_loss_grad(st, rows, 1, cfg.critic_mirror_loss_scale, _lib.ptr(value_all), _lib.ptr(value_all[rows:]),
                                            _lib.ptr(perm), _lib.ptr(sign), _lib.ptr(d_value), _lib.ptr(d_value_all[rows:]),
@@ -241,6 +243,44 @@ def update_model(policy: GaussianMlpPolicy, cfg: PPOUpdateConfig, actor_obs, cri
 
 # --------------------------------------------------------------------------- recurrent actor / critic (GRU or LSTM stacks)
 @dataclass
+class MirrorCarries:
+    """The mirrored pass's own carries at the first step of the trajectory slice (`actor_mirror`, `critic_mirror`,
+    `lpf_params_mirror` of examples/kbot/train.py:1506-1515); None entries start from zero, which is what the task's
+    rollout leaves there (it never advances them)."""
+    actor: torch.Tensor | None = None
+    critic: torch.Tensor | None = None
+    lpf: torch.Tensor | None = None
+
+
+def _cat_env(a: torch.Tensor, b: torch.Tensor | None) -> torch.Tensor:
+    """Carries of the first and the mirrored pass side by side on the env axis ((depth, 2, N, H) or (depth, N, H))."""
+    ax = 2 if a.dim() == 4 else 1
+    return torch.cat([a, torch.zeros_like(a) if b is None else b], dim=ax).contiguous()
+
+
+def actor_locations(policy: "RecurrentHeadPolicy", raw: torch.Tensor, obs: torch.Tensor, fresh: torch.Tensor,
+                    lpf0: torch.Tensor | None, y_last: torch.Tensor | None = None) -> torch.Tensor:
+    """raw (T, M, 2 nu) -> the same rows with the distribution's location (bias added, filtered) in the first half, when
+    the policy filters its means; `obs` (T, M, in) supplies the observation-dependent part of the bias."""
+    lp = policy.lowpass
+    if lp is None:
+        return raw
+    Tn, M, W = raw.shape
+    nu = W // 2
+    add, add_ld, a0, cnt = None, 0, 0, 0
+    if lp.obs_bias is not None:
+        col0, a0, cnt = (int(v) for v in lp.obs_bias)
+        if col0 < 0 or col0 + cnt > obs.shape[-1] or not obs.is_contiguous():
+            raise _lib.KsError("the observation-dependent bias reads columns outside the observation rows")
+        add, add_ld = ctypes.c_void_p(obs.data_ptr() + 4 * col0), obs.shape[-1]
+    out = torch.empty_like(raw)
+    _lib.check(_lib.load().ks_lowpass_scan(_lib.current_stream(), Tn, M, nu, W, float(lp.ctrl_dt), float(lp.cutoff_frequency),
+                                           _lib.ptr(raw), _lib.ptr(policy.mean_bias), add, add_ld, a0, cnt, _lib.ptr(lpf0),
+                                           _lib.ptr(fresh), _lib.ptr(out), _lib.ptr(y_last)))
+    return out
+
+
+@dataclass
 class RecurrentHeadPolicy:
     """Recurrent actor whose output is (means | raw deviations) per action (examples/kbot/train.py:903-932) and a
     recurrent critic; `min_std`, `max_std`, `var_scale`, `mean_bias` describe the deviation head."""
@@ -256,6 +296,8 @@ class RecurrentHeadPolicy:
     clip_lo: torch.Tensor | None = None
     clip_hi: torch.Tensor | None = None
     kl_scale: torch.Tensor | None = None  # adaptive KL: current coefficient / cfg.kl_coef, one device float
+    lowpass: "LowPass | None" = None      # the actor's means pass a one-pole low-pass whose state rides in the model carry
+    mirror: MirrorSpec | None = None      # the task's symmetry, for the mirror losses (second pass from mirrored carries)
 
     def kl_coef(self, cfg: "PPOUpdateConfig") -> float:
         """The KL coefficient now in force (a host read: for logging and tests)."""
@@ -274,36 +316,103 @@ class RecurrentHeadPolicy:
 
 
 def single_step_recurrent(policy: RecurrentHeadPolicy, cfg: PPOUpdateConfig, actor_obs, critic_obs, action, rewards, done, success,
-                          on_log_probs, on_values, actor_carry0, critic_carry0, fresh) -> dict:
+                          on_log_probs, on_values, actor_carry0, critic_carry0, fresh, lpf0=None,
+                          mirror_carries: MirrorCarries | None = None) -> dict:
     """One minibatch step (ppo.py:495-565) for recurrent networks: both networks run over the (T, b) trajectory slice
     from the carries the rollout started with, envs flagged in `fresh` (T, b) restart their carry, and the gradient goes
-    back through time.  GAE is recomputed from the current values and enters as a constant."""
+    back through time.  GAE is recomputed from the current values and enters as a constant.
+
+    With `policy.lowpass` the actor's biased means pass the one-pole filter from the state `lpf0` (b, nu) and its gradient
+    runs back through time with the networks'.  With mirror loss scales set (`policy.mirror` names the maps) each network
+    runs a second time on the mirrored observations from `mirror_carries` (examples/kbot/train.py:1458-1496): the mirrored
+    envs ride as columns [b, 2b) of the same forward and backward pass, so both passes' gradients meet in one sweep."""
     lib = _lib.load()
     Tn, b = done.shape
     rows = Tn * b
     nu = action.shape[-1]
-    raw = policy.actor.train_forward(actor_obs, actor_carry0, fresh)        # (T, b, 2 nu)
-    value = policy.critic.train_forward(critic_obs, critic_carry0, fresh)   # (T, b, 1)
+    st = _lib.current_stream()
+    dev = actor_obs.device
+    mixture = policy.num_mixtures > 0
+    mirror_a, mirror_c = cfg.actor_mirror_loss_scale != 0.0, cfg.critic_mirror_loss_scale != 0.0
+    if (mirror_a or mirror_c) and policy.mirror is None:
+        raise _lib.KsError("mirror loss scales are set but the policy has no MirrorSpec")
+    if mixture and (policy.lowpass is not None or mirror_a):
+        raise _lib.KsError("the low-pass filter and the action mirror loss are built for the mean | deviation head")
+    mc = mirror_carries or MirrorCarries()
+
+    def both(x, name):  # (T, b, n) -> (T, 2b, n): the rows and their mirror images side by side
+        perm, sign = policy.mirror.device(name, dev)
+        if perm.numel() != x.shape[-1]:
+            raise _lib.KsError(f"the {name} mirror map has {perm.numel()} entries, the rows have {x.shape[-1]}")
+        x = x.contiguous()
+        xm = torch.empty_like(x)
+        _lib.check(lib.ks_signed_permute(st, rows, x.shape[-1], _lib.ptr(x), _lib.ptr(perm), _lib.ptr(sign), _lib.ptr(xm)))
+        return torch.cat([x, xm], dim=1).contiguous()
+
+    fresh2 = torch.cat([fresh, fresh], dim=1).contiguous() if (mirror_a or mirror_c) else None
+    a_in = both(actor_obs, "actor_obs") if mirror_a else actor_obs.contiguous()
+    c_in = both(critic_obs, "critic_obs") if mirror_c else critic_obs.contiguous()
+    a_fresh, c_fresh = (fresh2 if mirror_a else fresh), (fresh2 if mirror_c else fresh)
+    raw_all = policy.actor.train_forward(a_in, _cat_env(actor_carry0, mc.actor) if mirror_a else actor_carry0, a_fresh)
+    value_all = policy.critic.train_forward(c_in, _cat_env(critic_carry0, mc.critic) if mirror_c else critic_carry0, c_fresh)
+    y0 = None
+    if policy.lowpass is not None:
+        y0 = lpf0 if lpf0 is not None else torch.zeros(b, nu, dtype=torch.float32, device=dev)
+        if mirror_a:
+            y0 = torch.cat([y0, torch.zeros_like(y0) if mc.lpf is None else mc.lpf], dim=0).contiguous()
+    loc_all = actor_locations(policy, raw_all, a_in, a_fresh, y0)   # (T, b or 2b, 2 nu): location | raw deviation
+    raw = loc_all[:, :b].contiguous() if mirror_a else loc_all
+    value = value_all[:, :b].contiguous() if mirror_c else value_all
     inputs = ppo_mod.compute_ppo_inputs(value.view(Tn, b), rewards, done, success, cfg.gamma, cfg.lam,
                                         normalize_advantages=cfg.normalize_advantages,
                                         monte_carlo_returns=cfg.monte_carlo_returns, time_major=True)
     if cfg.adaptive_kl and policy.kl_scale is None:  # as in single_step: the factor stays on the device
-        policy.kl_scale = torch.ones(1, dtype=torch.float32, device=raw.device)
+        policy.kl_scale = torch.ones(1, dtype=torch.float32, device=dev)
     p = _lib.KsPpoLossParams(cfg.clip_param, cfg.value_loss_coef, cfg.entropy_coef, cfg.kl_coef, cfg.log_clip_value, 1.0,
                              int(cfg.use_clipped_value_loss), _lib.ptr(policy.kl_scale) if cfg.adaptive_kl else None)
-    mixture = policy.num_mixtures > 0
-    head = policy._mixture() if mixture else T.KsGaussianHead(float(policy.min_std), float(policy.max_std), float(policy.var_scale), 0,
-                                                              _lib.ptr(policy.mean_bias).value)
-    d_raw = torch.empty(Tn, b, policy.width(nu), dtype=torch.float32, device=raw.device)
-    d_value = torch.empty(Tn, b, 1, dtype=torch.float32, device=raw.device)
+    # behind the filter the bias is already inside the location
+    bias_ptr = None if policy.lowpass is not None else _lib.ptr(policy.mean_bias).value
+    head = policy._mixture() if mixture else T.KsGaussianHead(float(policy.min_std), float(policy.max_std), float(policy.var_scale), 0, bias_ptr)
+    d_raw = torch.empty(Tn, b, policy.width(nu), dtype=torch.float32, device=dev)
+    d_value = torch.empty(Tn, b, 1, dtype=torch.float32, device=dev)
     grad_fn = lib.ks_ppo_loss_grad_mixture if mixture else lib.ks_ppo_loss_grad_head
-    _lib.check(grad_fn(_lib.current_stream(), rows, nu, ctypes.byref(p), ctypes.byref(head), _lib.ptr(raw),
-                                         _lib.ptr(action.contiguous()), _lib.ptr(on_log_probs.contiguous()),
-                                         _lib.ptr(inputs.advantages_bt), _lib.ptr(inputs.value_targets_bt),
-                                         _lib.ptr(on_values.contiguous()), _lib.ptr(value), _lib.ptr(d_raw), _lib.ptr(d_value)))
-    policy.actor.backward(d_raw)
-    policy.critic.backward(d_value)
-    sq = torch.zeros(1, dtype=torch.float64, device=raw.device)
+    _lib.check(grad_fn(st, rows, nu, ctypes.byref(p), ctypes.byref(head), _lib.ptr(raw),
+                       _lib.ptr(action.contiguous()), _lib.ptr(on_log_probs.contiguous()),
+                       _lib.ptr(inputs.advantages_bt), _lib.ptr(inputs.value_targets_bt),
+                       _lib.ptr(on_values.contiguous()), _lib.ptr(value), _lib.ptr(d_raw), _lib.ptr(d_value)))
+    aux = {}
+    d_raw_all, d_value_all = d_raw, d_value
+    if mirror_a:
+        # modes of the two passes (the head's bias, where no filter has absorbed it, is part of the mode)
+        mode, mode_m = raw[..., :nu].contiguous(), loc_all[:, b:, :nu].contiguous()
+        if policy.lowpass is None and policy.mean_bias is not None:
+            mode, mode_m = mode + policy.mean_bias, mode_m + policy.mean_bias
+        d_mode, d_mode_m = d_raw[..., :nu].contiguous(), torch.empty(Tn, b, nu, dtype=torch.float32, device=dev)
+        perm, sign = policy.mirror.device("action", dev)
+        aux["action_mirror_loss"] = torch.empty(Tn, b, dtype=torch.float32, device=dev)
+        _lib.check(lib.ks_mirror_loss_grad(st, rows, nu, cfg.actor_mirror_loss_scale, _lib.ptr(mode), _lib.ptr(mode_m), _lib.ptr(perm),
+                                           _lib.ptr(sign), _lib.ptr(d_mode), _lib.ptr(d_mode_m), _lib.ptr(aux["action_mirror_loss"])))
+        d_raw_all = torch.zeros(Tn, 2 * b, 2 * nu, dtype=torch.float32, device=dev)  # the mirrored deviations enter nothing
+        d_raw_all[:, :b] = d_raw
+        d_raw_all[:, :b, :nu] = d_mode
+        d_raw_all[:, b:, :nu] = d_mode_m
+    if mirror_c:
+        v_main, v_m = value.view(rows, 1), value_all[:, b:].contiguous().view(rows, 1)
+        d_v, d_vm = d_value.view(rows, 1), torch.empty(rows, 1, dtype=torch.float32, device=dev)
+        perm, sign = policy.mirror.device("value", dev)
+        aux["value_mirror_loss"] = torch.empty(Tn, b, dtype=torch.float32, device=dev)
+        _lib.check(lib.ks_mirror_loss_grad(st, rows, 1, cfg.critic_mirror_loss_scale, _lib.ptr(v_main), _lib.ptr(v_m), _lib.ptr(perm),
+                                           _lib.ptr(sign), _lib.ptr(d_v), _lib.ptr(d_vm), _lib.ptr(aux["value_mirror_loss"])))
+        d_value_all = torch.cat([d_value, d_vm.view(Tn, b, 1)], dim=1).contiguous()
+    if policy.lowpass is not None:  # dL/d location -> dL/d raw mean, back through the filter's own recursion
+        if d_raw_all is d_raw:
+            d_raw_all = d_raw.clone()  # d_raw stays what the loss kernel wrote, for the caller's metrics
+        lp_ = policy.lowpass
+        _lib.check(lib.ks_lowpass_scan_backward(st, Tn, d_raw_all.shape[1], nu, 2 * nu, float(lp_.ctrl_dt), float(lp_.cutoff_frequency),
+                                                _lib.ptr(a_fresh), _lib.ptr(d_raw_all), None))
+    policy.actor.backward(d_raw_all)
+    policy.critic.backward(d_value_all)
+    sq = torch.zeros(1, dtype=torch.float64, device=dev)
     policy.actor.grad_sqnorm(sq)
     policy.critic.grad_sqnorm(sq)
     policy.opt_step += 1
@@ -311,25 +420,27 @@ def single_step_recurrent(policy: RecurrentHeadPolicy, cfg: PPOUpdateConfig, act
     policy.actor.adam_step(ap, sq)
     policy.critic.adam_step(ap, sq)
     metrics = {"grad_norm": sq.sqrt(), "d_raw": d_raw, "d_value": d_value, "raw": raw, "values": value,
-               "advantages": inputs.advantages_bt}
+               "advantages": inputs.advantages_bt, **aux}
     if cfg.adaptive_kl:  # ppo.py:546-563 on the log-probabilities of this step's forward pass
-        lp = torch.empty(rows, nu, dtype=torch.float32, device=raw.device)
+        lp = torch.empty(rows, nu, dtype=torch.float32, device=dev)
         if mixture:
-            _lib.check(lib.ks_mixture_head_log_prob(_lib.current_stream(), rows, nu, ctypes.byref(head), _lib.ptr(raw),
+            _lib.check(lib.ks_mixture_head_log_prob(st, rows, nu, ctypes.byref(head), _lib.ptr(raw),
                                                     _lib.ptr(action.contiguous()), _lib.ptr(lp)))
         else:
-            _lib.check(lib.ks_gaussian_head_log_prob(_lib.current_stream(), rows, nu, ctypes.byref(head), _lib.ptr(raw),
+            _lib.check(lib.ks_gaussian_head_log_prob(st, rows, nu, ctypes.byref(head), _lib.ptr(raw),
                                                      _lib.ptr(action.contiguous()), _lib.ptr(lp), None))
-        ws = torch.empty(256 * nu, dtype=torch.float32, device=raw.device)
-        _lib.check(lib.ks_ppo_adapt_kl(_lib.current_stream(), rows, nu, _lib.ptr(on_log_probs.contiguous()), _lib.ptr(lp), cfg.kl_coef,
+        ws = torch.empty(256 * nu, dtype=torch.float32, device=dev)
+        _lib.check(lib.ks_ppo_adapt_kl(st, rows, nu, _lib.ptr(on_log_probs.contiguous()), _lib.ptr(lp), cfg.kl_coef,
                                        cfg.desired_kl, _lib.ptr(policy.kl_scale), _lib.ptr(ws)))
         metrics["log_probs"] = lp
     return metrics
 
 
-def recurrent_on_policy(policy: RecurrentHeadPolicy, actor_obs, critic_obs, action, actor_carry0, critic_carry0, fresh):
+def recurrent_on_policy(policy: RecurrentHeadPolicy, actor_obs, critic_obs, action, actor_carry0, critic_carry0, fresh, lpf0=None,
+                        return_raw: bool = False):
     """Log-probabilities (T, N, nu) and values (T, N) of the recorded actions under the current parameters: the pass that
-    update_model makes once over the whole rollout before any minibatch step (ppo.py:603-607)."""
+    update_model makes once over the whole rollout before any minibatch step (ppo.py:603-607).  With `return_raw` also the
+    head's input rows (T, N, width), locations filtered where the policy filters them."""
     Tn, N, nu = action.shape
     a_carry, c_carry = actor_carry0.clone(), critic_carry0.clone()
     raw = torch.empty(Tn, N, policy.width(nu), dtype=torch.float32, device=action.device)
@@ -337,25 +448,30 @@ def recurrent_on_policy(policy: RecurrentHeadPolicy, actor_obs, critic_obs, acti
     for t in range(Tn):
         policy.actor(actor_obs[t], a_carry, fresh=fresh[t], out=raw[t])
         policy.critic(critic_obs[t], c_carry, fresh=fresh[t], out=values[t])
+    if policy.lowpass is not None:
+        raw = actor_locations(policy, raw, actor_obs.contiguous(), fresh.contiguous(), lpf0)
     lp = torch.empty(Tn, N, nu, dtype=torch.float32, device=action.device)
     if policy.num_mixtures:
         head = policy._mixture()
         _lib.check(_lib.load().ks_mixture_head_log_prob(_lib.current_stream(), Tn * N, nu, ctypes.byref(head), _lib.ptr(raw),
                                                         _lib.ptr(action.contiguous()), _lib.ptr(lp)))
     else:
-        head = T.KsGaussianHead(float(policy.min_std), float(policy.max_std), float(policy.var_scale), 0, _lib.ptr(policy.mean_bias).value)
+        head = T.KsGaussianHead(float(policy.min_std), float(policy.max_std), float(policy.var_scale), 0,
+                                None if policy.lowpass is not None else _lib.ptr(policy.mean_bias).value)
         _lib.check(_lib.load().ks_gaussian_head_log_prob(_lib.current_stream(), Tn * N, nu, ctypes.byref(head), _lib.ptr(raw),
                                                          _lib.ptr(action.contiguous()), _lib.ptr(lp), None))
-    return lp, values[..., 0]
+    return (lp, values[..., 0], raw) if return_raw else (lp, values[..., 0])
 
 
 def update_model_recurrent(policy: RecurrentHeadPolicy, cfg: PPOUpdateConfig, actor_obs, critic_obs, action, rewards, done, success,
                            actor_carry0, critic_carry0, fresh, permutations: list[torch.Tensor] | None = None,
-                           seed: int = 0) -> list[dict]:
+                           seed: int = 0, lpf0=None, mirror_carries: MirrorCarries | None = None) -> list[dict]:
     """num_passes x (N / batch_size) minibatch steps over a (T, N) rollout for a recurrent actor and critic
-    (ppo.py:572-694): a minibatch is a set of env columns together with their carries at the rollout's first step."""
+    (ppo.py:572-694): a minibatch is a set of env columns together with their carries at the rollout's first step
+    (`lpf0` (N, nu): the filter state there; `mirror_carries`: the mirrored pass's, zero when None)."""
     Tn, N = done.shape
-    on_lp, on_v = recurrent_on_policy(policy, actor_obs, critic_obs, action, actor_carry0, critic_carry0, fresh)
+    on_lp, on_v = recurrent_on_policy(policy, actor_obs, critic_obs, action, actor_carry0, critic_carry0, fresh, lpf0)
+    mc = mirror_carries or MirrorCarries()
     bs = min(cfg.batch_size, N)
     if N % bs:
         raise _lib.KsError("the env count must be a multiple of the batch size (ppo.py:647 reshapes the permutation)")
@@ -369,6 +485,9 @@ def update_model_recurrent(policy: RecurrentHeadPolicy, cfg: PPOUpdateConfig, ac
             sel = lambda t: t.index_select(1, idx).contiguous()  # noqa: E731
             ca = actor_carry0.index_select(env_axis[actor_carry0.dim() == 4], idx).contiguous()
             cc = critic_carry0.index_select(env_axis[critic_carry0.dim() == 4], idx).contiguous()
+            env_sel = lambda c: None if c is None else c.index_select(env_axis[c.dim() == 4], idx).contiguous()  # noqa: E731
+            rows_sel = lambda c: None if c is None else c.index_select(0, idx).contiguous()  # noqa: E731
             out.append(single_step_recurrent(policy, cfg, sel(actor_obs), sel(critic_obs), sel(action), sel(rewards), sel(done),
-                                             sel(success), sel(on_lp), sel(on_v), ca, cc, sel(fresh)))
+                                             sel(success), sel(on_lp), sel(on_v), ca, cc, sel(fresh), rows_sel(lpf0),
+                                             MirrorCarries(env_sel(mc.actor), env_sel(mc.critic), rows_sel(mc.lpf))))
     return out

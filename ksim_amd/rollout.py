@@ -16,6 +16,7 @@ import torch
 from . import _lib
 from . import _lib_terms as T
 from . import ppo as ppo_mod
+from .actions import LowPass
 from .commands import CommandSet
 from .engine import HipEngine
 from .env_terms import EnvTerms, sample_action, sample_action_head, sample_action_mixture
@@ -33,6 +34,7 @@ class GaussianHead:
     max_std: float
     var_scale: float = 1.0
     mean_bias: torch.Tensor | None = None
+    lowpass: LowPass | None = None  # the biased means pass a one-pole low-pass before sampling (train.py:923-929)
 
     def width(self, na: int) -> int:
         return 2 * na
@@ -83,6 +85,7 @@ class RolloutEnvState:  # ksim/task/rl.py:110-123, batched
         self.commands_drawn = False  # whether the command set has drawn this env state's initial commands
         self.actor_carry = None   # (depth, N, hidden) carries of recurrent networks (rl.py:117)
         self.critic_carry = None
+        self.lpf_state = None     # (N, nu) state of the low-pass filter on the actor's means, part of the model carry
         N = physics_state.data.qpos.shape[0]
         self.episode_length = torch.zeros(N, dtype=torch.int32, device=physics_state.data.qpos.device)
 
@@ -111,6 +114,10 @@ class Rollout:
         self.fresh = b(Tn, N) if any(isinstance(n, RecurrentNetwork) for n in (c.actor, c.critic)) else None
         self.actor_carry0 = c.actor.initial_carry(N, dev) if isinstance(c.actor, RecurrentNetwork) else None
         self.critic_carry0 = c.critic.initial_carry(N, dev) if isinstance(c.critic, RecurrentNetwork) else None
+        self._lowpass = c.head.lowpass if isinstance(c.head, GaussianHead) else None
+        self.lpf_carry0 = f(N, na) if self._lowpass is not None else None  # the filter state at the rollout's first step
+        if self._lowpass is not None and self.fresh is None:
+            self.fresh = b(Tn, N)  # the update replays the filter from the same episode starts
         self.command = f(Tn, N, c.commands.command_dim) if c.commands is not None else None
         if c.commands is not None and c.commands.command_dim != c.terms.command_dim:
             raise _lib.KsError("the command set and the observation terms disagree about the width of the command vector")
@@ -170,8 +177,23 @@ class Rollout:
             elif c.critic is not None:
                 c.critic(self.obs[t], out=self.values[t])
         if isinstance(c.head, GaussianHead):
+            head_bias = c.head.mean_bias
+            if self._lowpass is not None:
+                # the filter's state belongs to the model carry: zero for the envs the previous step reset (rl.py:1072-1080)
+                if t == 0:
+                    self.lpf_carry0.copy_(env.lpf_state)
+                lp, nu_ = self._lowpass, self.action.shape[-1]
+                add, add_ld, a0, cnt = None, 0, 0, 0
+                if lp.obs_bias is not None:
+                    col0, a0, cnt = (int(v) for v in lp.obs_bias)
+                    add, add_ld = _lib.c_void_p(self.noisy_obs[t].data_ptr() + 4 * col0), self.noisy_obs.shape[-1]
+                _lib.check(_lib.load().ks_lowpass_scan(_lib.current_stream(), 1, self.N, nu_, 2 * nu_, float(lp.ctrl_dt),
+                                                       float(lp.cutoff_frequency), _lib.ptr(self.mean), _lib.ptr(head_bias), add, add_ld,
+                                                       a0, cnt, _lib.ptr(env.lpf_state), _lib.ptr(self.reset_mask), _lib.ptr(self.mean),
+                                                       _lib.ptr(env.lpf_state)))
+                head_bias = None  # now inside the filtered location
             sample_action_head(self.mean, min_std=c.head.min_std, max_std=c.head.max_std, var_scale=c.head.var_scale,
-                               mean_bias=c.head.mean_bias, noise=noise.get("action_normal"), seed=env.seed, step=step,
+                               mean_bias=head_bias, noise=noise.get("action_normal"), seed=env.seed, step=step,
                                step_base=step_base, clip_max=c.action_clip_max, out=self.action[t])
         elif isinstance(c.head, MixtureHead):
             sample_action_mixture(self.mean, c.head.num_mixtures, min_std=c.head.min_std, max_std=c.head.max_std,
@@ -263,6 +285,8 @@ class Rollout:
             d = env.physics_state.data
             self.c.commands.update(env.commands, d.qpos, d.qvel, all_fresh=True, seed=env.seed, step=(1 << 62) + env.step)
             env.commands_drawn = True
+        if self._lowpass is not None and env.lpf_state is None:
+            env.lpf_state = torch.zeros(self.N, self.action.shape[-1], dtype=torch.float32, device=self.done.device)
         for net, name in ((self.c.actor, "actor_carry"), (self.c.critic, "critic_carry")):
             if isinstance(net, RecurrentNetwork) and getattr(env, name) is None:
                 setattr(env, name, net.initial_carry(self.N, self.done.device))

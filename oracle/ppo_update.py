@@ -191,25 +191,90 @@ def update_model(params, rollout, cfg, permutations, act="elu"):
     return params, losses
 
 
-def recurrent_loss_and_grads(actor, critic, batch, cfg, head, act="none"):
+def lowpass_torch(x, ctrl_dt, fc, y0, fresh):
+    """ksim.lowpass_one_pole (ksim/actions.py:248-257) threaded through time on torch tensors, x (T, b, n): the state is y0
+    before the first step and zero at the steps flagged fresh (the model carry was replaced by the initial one after a
+    done step, examples/kbot/train.py:1529-1533)."""
+    alpha = ctrl_dt / (1.0 / (2.0 * math.pi * fc) + ctrl_dt)
+    last = torch.tensor(np.asarray(y0, dtype=np.float64))
+    out = []
+    for t in range(x.shape[0]):
+        keep = torch.tensor(1.0 - np.asarray(fresh[t], dtype=np.float64))[:, None]
+        last = last * keep
+        last = last + alpha * (x[t] - last)
+        out.append(last)
+    return torch.stack(out)
+
+
+def recurrent_loss_and_grads(actor, critic, batch, cfg, head, act="none", lowpass=None, mirror=None):
     """The minibatch loss of PPOTask for a recurrent actor with the mean | raw deviation head and a recurrent critic
     (ppo.py:412-492 with the scan over time), and its gradients by float64 reverse-mode differentiation.
     actor / critic: dict(input_proj, cells, out_w, out_b, carry0); batch: (T, b, ...) arrays with `fresh`; head:
-    dict(min_std, max_std, var_scale, mean_bias).  Returns (loss, actor gradients, critic gradients, aux)."""
+    dict(min_std, max_std, var_scale, mean_bias).
+
+    `lowpass`: dict(ctrl_dt, cutoff, y0 (b, nu), optional obs_bias=(first obs column, first action, count)): the biased
+    means pass ksim.lowpass_one_pole before they become the distribution's location (examples/kbot/train.py:917-932; the
+    command-dependent bias of train.py:920-921 is read from the observation row), the filter state riding in the carry.
+    `mirror`: dict(actor_obs=(perm, sign), critic_obs=(perm, sign), action=(perm, sign), actor_scale, critic_scale,
+    actor_carry0, critic_carry0, y0): both networks run a second time on the mirrored observations from their own mirrored
+    carries (and the actor's mirrored filter state); the squared differences of the modes (mirrored back) and of the values
+    join the loss as auxiliary terms (train.py:1458-1496, ppo.py:241-244).
+    Returns (loss, actor gradients, critic gradients, aux)."""
     from . import recurrent as orec
 
     pa = orec.torch_parameters(actor["input_proj"], actor["cells"], actor["out_w"], actor["out_b"])
     pc = orec.torch_parameters(critic["input_proj"], critic["cells"], critic["out_w"], critic["out_b"])
-    raw = orec.torch_sequence(batch["actor_obs"], actor["carry0"], batch["fresh"], *pa, act=act)
+    bias = None if head.get("mean_bias") is None else torch.tensor(np.asarray(head["mean_bias"], dtype=np.float64))
+    nu = np.asarray(batch["action"]).shape[-1]
+
+    def run_actor(obs, carry0, y0):
+        """raw (T, b, 2 nu) with the location (biased, filtered when asked) in the first half; with a filter the head's own
+        bias is spent."""
+        raw = orec.torch_sequence(obs, carry0, batch["fresh"], *pa, act=act)
+        if lowpass is None:
+            return raw, bias
+        mean = raw[..., :nu] + (0.0 if bias is None else bias)
+        if lowpass.get("obs_bias") is not None:
+            col0, a0, cnt = lowpass["obs_bias"]
+            extra = torch.zeros_like(mean)
+            extra[..., a0:a0 + cnt] = torch.tensor(np.asarray(obs, dtype=np.float64)[..., col0:col0 + cnt])
+            mean = mean + extra
+        mean = lowpass_torch(mean, lowpass["ctrl_dt"], lowpass["cutoff"], y0, batch["fresh"])
+        return torch.cat([mean, raw[..., nu:]], dim=-1), None
+
+    raw, head_bias = run_actor(batch["actor_obs"], actor["carry0"], None if lowpass is None else lowpass["y0"])
     v = orec.torch_sequence(batch["critic_obs"], critic["carry0"], batch["fresh"], *pc, act=act)[..., 0]
     # GAE from the current values, as a constant (ppo.py:450-459); the oracle works on (B, T)
     gae = oppo.compute_ppo_inputs(v.detach().numpy().T, batch["rewards"].T, batch["done"].T, batch["success"].T, cfg["gamma"],
                                   cfg["lam"], normalize_advantages=cfg["normalize_advantages"],
                                   monte_carlo_returns=cfg["monte_carlo_returns"])
     adv, tgt = torch.tensor(gae["advantages"].T.copy()), torch.tensor(gae["value_targets"].T.copy())
-    bias = None if head.get("mean_bias") is None else torch.tensor(np.asarray(head["mean_bias"], dtype=np.float64))
     lp, ent = gaussian_head(raw, torch.tensor(np.asarray(batch["action"], dtype=np.float64)), head["min_std"], head["max_std"],
-                            head["var_scale"], bias)
+                            head["var_scale"], head_bias)
     loss, _ = ppo_loss_torch(adv, tgt, torch.tensor(batch["on_log_probs"]), torch.tensor(batch["on_values"]), lp, v, ent, cfg)
+    aux = {}
+    if mirror:
+        def m(x, key):
+            perm, sign = mirror[key]
+            return x[..., list(perm)] * np.asarray(sign, dtype=np.float64)
+
+        if mirror.get("actor_scale", 0.0):
+            raw_m, bias_m = run_actor(m(np.asarray(batch["actor_obs"], dtype=np.float64), "actor_obs"), mirror["actor_carry0"],
+                                      mirror.get("y0"))
+            mode = raw[..., :nu] + (0.0 if head_bias is None else head_bias)
+            mode_m = raw_m[..., :nu] + (0.0 if bias_m is None else bias_m)
+            perm, sign = mirror["action"]
+            back = mode_m[..., list(perm)] * torch.tensor(np.asarray(sign, dtype=np.float64))
+            term = ((mode - back) ** 2).mean(-1) * mirror["actor_scale"]  # train.py:1466-1469
+            loss = loss + term.mean()
+            aux["action_mirror_loss"] = term.detach().numpy()
+            aux["raw_mirror"] = raw_m.detach().numpy()
+        if mirror.get("critic_scale", 0.0):
+            v_m = orec.torch_sequence(m(np.asarray(batch["critic_obs"], dtype=np.float64), "critic_obs"), mirror["critic_carry0"],
+                                      batch["fresh"], *pc, act=act)[..., 0]
+            term = (v - v_m) ** 2 * mirror["critic_scale"]  # train.py:1477
+            loss = loss + term.mean()
+            aux["value_mirror_loss"] = term.detach().numpy()
     loss.backward()
-    return float(loss.detach()), orec.parameter_gradients(pa), orec.parameter_gradients(pc), {"raw": raw.detach().numpy(), "values": v.detach().numpy()}
+    aux.update({"raw": raw.detach().numpy(), "values": v.detach().numpy()})
+    return float(loss.detach()), orec.parameter_gradients(pa), orec.parameter_gradients(pc), aux

@@ -711,6 +711,38 @@ def lowpass_one_pole(x, y_last, ctrl_dt, fc):  # actions.py:248-257
     return np.asarray(y_last, np.float64) + alpha * (np.asarray(x, np.float64) - y_last)
 
 
+def lowpass_scan(x, ctrl_dt, fc, y0=None, fresh=None):
+    """The filter threaded through a trajectory as the K-Bot task's scan does (examples/kbot/train.py:1439-1451, 1506-1533):
+    x (T, ..., n); the state starts at y0 (zeros when None) and is the initial one, zero, at the steps flagged in `fresh`
+    (T, ...) (the step after a done one: the carry was replaced by the initial carry).  Returns (y (T, ..., n), last state)."""
+    x = np.asarray(x, np.float64)
+    last = np.zeros(x.shape[1:]) if y0 is None else np.array(y0, dtype=np.float64)
+    out = np.empty_like(x)
+    for t in range(x.shape[0]):
+        if fresh is not None:
+            last = np.where(np.asarray(fresh[t], bool)[..., None], 0.0, last)
+        last = lowpass_one_pole(x[t], last, ctrl_dt, fc)
+        out[t] = last
+    return out, last
+
+
+def lowpass_scan_backward(dy, ctrl_dt, fc, fresh=None):
+    """Reverse-mode derivative of `lowpass_scan`, written out: from dL/dy (T, ..., n) to (dL/dx, dL/dy0).
+    y_t = (1 - a) y_{t-1} + a x_t, so the gradient reaching y_t is G_t = dy_t + (1 - a) G_{t+1} unless step t + 1 is fresh
+    (its y_{t} input was replaced by zero), and dL/dx_t = a G_t; dL/dy0 = (1 - a) G_0 unless step 0 is fresh."""
+    dy = np.asarray(dy, np.float64)
+    a = ctrl_dt / (1.0 / (2.0 * np.pi * fc) + ctrl_dt)
+    dx = np.empty_like(dy)
+    carry = np.zeros(dy.shape[1:])
+    for t in range(dy.shape[0] - 1, -1, -1):
+        G = dy[t] + carry
+        dx[t] = a * G
+        carry = (1.0 - a) * G
+        if fresh is not None:
+            carry = np.where(np.asarray(fresh[t], bool)[..., None], 0.0, carry)
+    return dx, carry
+
+
 def clip_acceleration(target, position, velocity, max_acceleration, ctrl_dt):  # actions.py:54-80: (position, velocity)
     target, position, velocity = (np.asarray(a, np.float64) for a in (target, position, velocity))
     cur_v = (target - position) / ctrl_dt

@@ -356,6 +356,142 @@ def test_recurrent_single_step_gradients_match_oracle():
     assert m["grad_norm"].item() == pytest.approx(np.sqrt(total), rel=2e-3)
 
 
+def test_lowpass_scan_kernels_match_the_oracle():
+    """The filter threaded through a trajectory and its reverse sweep, through the C ABI, against the numpy restatement
+    (itself pinned by closed forms and central differences): rows of 2 nu floats whose second half travels unchanged, a
+    bias per joint, an observation-dependent bias on some joints, restarts inside the slice, and the T = 1 in-place form
+    the rollout uses."""
+    from ksim_amd import _lib
+    from oracle import terms as ot
+
+    lib = _lib.load()
+    rng = np.random.default_rng(77)
+    Tn, M, nu, I = 11, 37, 6, 9
+    dt, fc = 0.02, 6.0
+    raw, obs = rng.normal(size=(Tn, M, 2 * nu)), rng.normal(size=(Tn, M, I))
+    bias, y0 = rng.normal(size=nu) * 0.2, rng.normal(size=(M, nu))
+    fresh = rng.random((Tn, M)) < 0.15
+    col0, a0, cnt = 5, 3, 2
+    x = raw[..., :nu] + bias
+    x[..., a0:a0 + cnt] += obs[..., col0:col0 + cnt]
+    want, want_last = ot.lowpass_scan(x, dt, fc, y0, fresh)
+    d_raw, d_obs, d_f = t32(raw), t32(obs), torch.tensor(fresh, dtype=torch.uint8, device=DEV)
+    out, last = torch.empty_like(d_raw), torch.empty(M, nu, device=DEV)
+    d_bias, d_y0in = t32(bias), t32(y0)  # named, so that they outlive the launches that read them
+    add = ctypes.c_void_p(d_obs.data_ptr() + 4 * col0)
+    _lib.check(lib.ks_lowpass_scan(_lib.current_stream(), Tn, M, nu, 2 * nu, dt, fc, _lib.ptr(d_raw), _lib.ptr(d_bias), add, I, a0, cnt,
+                                   _lib.ptr(d_y0in), _lib.ptr(d_f), _lib.ptr(out), _lib.ptr(last)))
+    got = out.cpu().numpy()
+    np.testing.assert_allclose(got[..., :nu], want, rtol=2e-5, atol=2e-6)
+    assert np.array_equal(got[..., nu:], raw[..., nu:].astype(np.float32))
+    np.testing.assert_allclose(last.cpu().numpy(), want_last, rtol=2e-5, atol=2e-6)
+    # reverse sweep, in place on the first nu columns
+    g = rng.normal(size=(Tn, M, 2 * nu))
+    want_dx, want_dy0 = ot.lowpass_scan_backward(g[..., :nu], dt, fc, fresh)
+    d_g, d_y0 = t32(g), torch.empty(M, nu, device=DEV)
+    _lib.check(lib.ks_lowpass_scan_backward(_lib.current_stream(), Tn, M, nu, 2 * nu, dt, fc, _lib.ptr(d_f), _lib.ptr(d_g), _lib.ptr(d_y0)))
+    np.testing.assert_allclose(d_g.cpu().numpy()[..., :nu], want_dx, rtol=2e-5, atol=2e-6)
+    assert np.array_equal(d_g.cpu().numpy()[..., nu:], g[..., nu:].astype(np.float32))
+    np.testing.assert_allclose(d_y0.cpu().numpy(), want_dy0, rtol=2e-5, atol=2e-6)
+    # one step in place, the state advanced in its own buffer: bit-equal to step 0 of the scan
+    state, step0 = t32(y0), t32(raw[0])
+    f0 = d_f[0].contiguous()
+    _lib.check(lib.ks_lowpass_scan(_lib.current_stream(), 1, M, nu, 2 * nu, dt, fc, _lib.ptr(step0), _lib.ptr(d_bias), add, I, a0, cnt,
+                                   _lib.ptr(state), _lib.ptr(f0), _lib.ptr(step0), _lib.ptr(state)))
+    assert torch.equal(step0, out[0]) and torch.equal(state, out[0][:, :nu])
+    assert lib.ks_lowpass_scan(_lib.current_stream(), Tn, M, nu, nu - 1, dt, fc, _lib.ptr(d_raw), None, None, 0, 0, 0, None, None, _lib.ptr(out), None) != 0
+    assert lib.ks_lowpass_scan(_lib.current_stream(), Tn, M, nu, 2 * nu, dt, fc, _lib.ptr(d_raw), None, add, I, nu - 1, 2, None, None, _lib.ptr(out), None) != 0
+
+
+@pytest.mark.parametrize("symmetric", [False, True])
+def test_kbot_training_step_with_filter_and_mirror_carries_matches_oracle(symmetric):
+    """The K-Bot task's minibatch step as shipped (examples/kbot/train.py:903-934, 1439-1533): LSTM actor whose biased means
+    (bias vector + command columns of the observation) pass the one-pole low-pass with its state in the carry, LSTM
+    critic, and the mirrored second pass of both from their own carries with the two mirror losses.  Every parameter's
+    gradient against float64 reverse-mode differentiation of that loss.  `symmetric`: the mirror map is the identity and
+    the mirrored carries equal the first pass's, so both mirror losses must vanish and leave the gradients alone."""
+    from ksim_amd import ppo_update as pu
+    from ksim_amd.actions import LowPass
+    from ksim_amd.mlp import MLP
+    from ksim_amd.recurrent import LSTMCell, RecurrentNetwork
+
+    rng = np.random.default_rng(61)
+    Tn, b, I, H, nu = 8, 48, 26, 64, 10
+
+    def make(out_dim):
+        proj = (rng.normal(size=(H, I)) / np.sqrt(I), rng.normal(size=H) * 0.1)
+        cells = [(rng.normal(size=(4 * H, H)) / np.sqrt(H), rng.normal(size=(4 * H, H)) / np.sqrt(H), rng.normal(size=4 * H) * 0.1)
+                 for _ in range(2)]
+        ow, ob = [rng.normal(size=(out_dim, H)) / np.sqrt(H)], [rng.normal(size=out_dim) * 0.1]
+        carry0 = rng.normal(size=(2, 2, b, H)) * 0.3
+        net = RecurrentNetwork(proj, [LSTMCell(*c, dtype="f32") for c in cells], MLP(ow, ob, activation="none", dtype="f32"), dtype="f32")
+        return dict(input_proj=proj, cells=cells, out_w=ow, out_b=ob, carry0=carry0), net
+
+    oa, actor = make(2 * nu)
+    oc, critic = make(1)
+    head = dict(min_std=0.01, max_std=1.0, var_scale=0.5, mean_bias=rng.normal(size=nu) * 0.1)
+    obs = rng.normal(size=(Tn, b, I))
+    fresh = rng.random((Tn, b)) < 0.1
+    done = np.roll(fresh, -1, axis=0); done[-1] = False
+    batch = dict(actor_obs=obs + rng.normal(size=obs.shape) * 0.01, critic_obs=obs, fresh=fresh, done=done,
+                 success=np.zeros((Tn, b), bool), rewards=rng.normal(size=(Tn, b)))
+    lowpass = dict(ctrl_dt=0.02, cutoff=10.0, y0=rng.normal(size=(b, nu)) * 0.2, obs_bias=(I - 4, nu - 4, 4))
+    if symmetric:
+        operm, osign, aperm, asign = np.arange(I), np.ones(I), np.arange(nu), np.ones(nu)
+        mirror = dict(actor_carry0=oa["carry0"], critic_carry0=oc["carry0"], y0=lowpass["y0"])
+    else:  # legs and arms swap, every joint negated; the observation entries reorder and change sign likewise
+        aperm, asign = np.r_[np.arange(3, 6), np.arange(0, 3), np.arange(6, 10)], -np.ones(nu)
+        operm, osign = rng.permutation(I), rng.choice([-1.0, 1.0], I)
+        mirror = dict(actor_carry0=rng.normal(size=(2, 2, b, H)) * 0.3, critic_carry0=rng.normal(size=(2, 2, b, H)) * 0.3,
+                      y0=rng.normal(size=(b, nu)) * 0.2)
+    mirror.update(actor_obs=(operm, osign), critic_obs=(operm, osign), action=(aperm, asign), actor_scale=0.8, critic_scale=0.4)
+    # the old policy: the same networks a little perturbed, so that ratios differ from one on both sides of the clip
+    zero = dict(batch, action=np.zeros((Tn, b, nu)), on_log_probs=np.zeros((Tn, b, nu)), on_values=np.zeros((Tn, b)))
+    aux0 = ou.recurrent_loss_and_grads(oa, oc, zero, CFG, head, lowpass=lowpass)[3]
+    raw0 = aux0["raw"] + rng.normal(size=aux0["raw"].shape) * 0.05
+    sd0 = np.minimum((np.logaddexp(0, raw0[..., nu:]) + 0.01) * 0.5, 1.0)
+    batch["action"] = raw0[..., :nu] + sd0 * rng.normal(size=sd0.shape)
+    batch["on_log_probs"] = ou.gaussian_head(torch.tensor(raw0), torch.tensor(batch["action"]), 0.01, 1.0, 0.5)[0].numpy()
+    batch["on_values"] = aux0["values"] + rng.normal(size=(Tn, b)) * 0.2
+    loss, ga, gc, aux = ou.recurrent_loss_and_grads(oa, oc, batch, CFG, head, lowpass=lowpass, mirror=mirror)
+    loss_plain, ga_plain, _, _ = ou.recurrent_loss_and_grads(oa, oc, batch, CFG, head, lowpass=lowpass)
+
+    spec = pu.MirrorSpec(list(operm), list(osign), list(operm), list(osign), list(aperm), list(asign))
+    policy = pu.RecurrentHeadPolicy(actor, critic, 0.01, 1.0, 0.5, t32(head["mean_bias"]), mirror=spec,
+                                    lowpass=LowPass(0.02, 10.0, obs_bias=lowpass["obs_bias"]))
+    policy.train_init()
+    cfg = pu.PPOUpdateConfig(**{k: v for k, v in CFG.items() if k not in ("batch_size", "num_passes")}, batch_size=b,
+                             actor_mirror_loss_scale=0.8, critic_mirror_loss_scale=0.4)
+    u8 = lambda a: torch.tensor(a, dtype=torch.uint8, device=DEV)  # noqa: E731
+    m = pu.single_step_recurrent(policy, cfg, t32(batch["actor_obs"]), t32(batch["critic_obs"]), t32(batch["action"]),
+                                 t32(batch["rewards"]), u8(done), u8(batch["success"]), t32(batch["on_log_probs"]),
+                                 t32(batch["on_values"]), t32(oa["carry0"]), t32(oc["carry0"]), u8(fresh), t32(lowpass["y0"]),
+                                 pu.MirrorCarries(t32(mirror["actor_carry0"]), t32(mirror["critic_carry0"]), t32(mirror["y0"])))
+    assert rel(m["raw"].cpu().numpy(), aux["raw"]) < 1e-4 and rel(m["values"].cpu().numpy()[..., 0], aux["values"]) < 1e-4
+    if symmetric:
+        assert m["action_mirror_loss"].abs().max().item() == 0.0 and m["value_mirror_loss"].abs().max().item() == 0.0
+        # (float64 matrix products of the library differ in the last bit between the two passes: 1e-32, not 0)
+        assert np.abs(aux["action_mirror_loss"]).max() < 1e-25 and loss == pytest.approx(loss_plain, rel=1e-13)
+    else:
+        assert rel(m["action_mirror_loss"].cpu().numpy(), aux["action_mirror_loss"]) < 1e-3
+        assert rel(m["value_mirror_loss"].cpu().numpy(), aux["value_mirror_loss"]) < 1e-3
+        assert aux["action_mirror_loss"].mean() > 1e-3  # the term is there, and it changes the gradient
+        assert rel(ga["out"][0][0], ga_plain["out"][0][0]) > 1e-2
+    for net, want in ((actor, ga), (critic, gc)):
+        got = {"proj.W": net.input_proj.parameters(True)[0][0], "proj.b": net.input_proj.parameters(True)[0][1],
+               "out.W": net.output_proj.parameters(True)[0][0], "out.b": net.output_proj.parameters(True)[0][1]}
+        ref = {"proj.W": want["input_proj"][0], "proj.b": want["input_proj"][1], "out.W": want["out"][0][0], "out.b": want["out"][0][1]}
+        for i, c in enumerate(net.cells):
+            g = c.parameters(True)
+            for k, j in (("weight_ih", 0), ("weight_hh", 1), ("bias", 2)):
+                got[f"cell{i}.{k}"], ref[f"cell{i}.{k}"] = g[k], want["cells"][i][j]
+        for k in ref:
+            assert rel(got[k].cpu().numpy(), ref[k]) < 2e-3, k
+    # the deviation half of the mirrored pass enters no loss: the raw-deviation rows of the output layer see the first pass only
+    total = sum(float((np.asarray(v) ** 2).sum()) for g in (ga, gc) for v in (g["input_proj"] + tuple(x for c in g["cells"] for x in c) + tuple(x for o in g["out"] for x in o)))
+    assert m["grad_norm"].item() == pytest.approx(np.sqrt(total), rel=2e-3)
+
+
 def test_ppo_loss_gradient_for_the_mixture_head_matches_autograd():
     """d loss / d (means | raw deviations | logits) for the mixture head against float64 autograd of the oracle loss (policy
     and KL terms through the exact mixture log-density, entropy term through the stated upper bound); clipped means and

@@ -109,6 +109,14 @@ def build(N, T, seed=0, min_height=0.9, events=None, gait=False, recurrent=False
         if head == "gaussian":   # means | raw deviations, deviations squeezed to ~0 so that the sample shows the mean
             from ksim_amd.rollout import GaussianHead
             head = GaussianHead(min_std=0.0, max_std=1e-6, mean_bias=head_bias)
+        elif head in ("gaussian-lowpass", "kbot"):
+            # the K-Bot actor: the biased means (bias vector + two observation columns on the last two joints) pass a
+            # one-pole low-pass whose state rides in the model carry (examples/kbot/train.py:917-929)
+            from ksim_amd.actions import LowPass
+            from ksim_amd.rollout import GaussianHead
+            lp = LowPass(ctrl_dt=0.02, cutoff_frequency=4.0, obs_bias=(0, m.nu - 2, 2))
+            head = (GaussianHead(min_std=0.0, max_std=1e-6, mean_bias=head_bias, lowpass=lp) if head == "gaussian-lowpass"
+                    else GaussianHead(min_std=0.05, max_std=0.5, var_scale=0.5, mean_bias=head_bias, lowpass=lp))
         elif head == "gaussian-wide":   # deviations a policy update can work with
             from ksim_amd.rollout import GaussianHead
             head = GaussianHead(min_std=0.05, max_std=0.5, var_scale=0.5, mean_bias=head_bias)
@@ -460,7 +468,7 @@ def test_rollout_written_to_the_dataset_format_and_read_back(tmp_path):
         assert torch.equal(r.total, rew.total[:, e]) and torch.equal(r.components["height"], rew.components["height"][:, e])
 
 
-@pytest.mark.parametrize("head", [None, "gaussian", "mixture"])
+@pytest.mark.parametrize("head", [None, "gaussian", "mixture", "gaussian-lowpass"])
 def test_recurrent_actor_and_critic_in_the_rollout(head):
     """GRU actor and critic inside the environment loop: the carries replayed by the oracle from the recorded
     observations and done flags (a finished env continues from a zero carry), and the graph replay equal to eager.  With a
@@ -474,7 +482,7 @@ def test_recurrent_actor_and_critic_in_the_rollout(head):
         m, c, rnd_, _, ro, EnvState = build(N, T, seed=13, min_height=0.95, recurrent=True, head=head)
         ps = c.engine.reset(c.physics_model, 1.0, 3, N, rnd_)
         env = EnvState(ps, rnd_, torch.zeros(N, 2, device=DEV), None, seed=21)
-        want = {"actor": np.zeros((2, N, 32)), "critic": np.zeros((2, N, 32))}
+        want = {"actor": np.zeros((2, N, 32)), "critic": np.zeros((2, N, 32)), "lpf": np.zeros((N, m.nu))}
         fresh = np.zeros(N, bool)
         snaps, finished = [], 0
         for it in range(5):
@@ -496,11 +504,18 @@ def test_recurrent_actor_and_critic_in_the_rollout(head):
                     bias = c.head.mean_bias.cpu().numpy()
                     if head == "gaussian":
                         np.testing.assert_allclose(act_t, y[:, :nu] + bias, rtol=2e-4, atol=2e-4)
+                    elif head == "gaussian-lowpass":  # the filter state restarts with the episode, like the carries
+                        x_in = y[:, :nu] + bias
+                        x_in[:, nu - 2:] += noisy[t][:, 0:2]
+                        want["lpf"] = ot.lowpass_one_pole(x_in, np.where(fresh[:, None], 0.0, want["lpf"]), 0.02, 4.0)
+                        np.testing.assert_allclose(act_t, want["lpf"], rtol=2e-4, atol=2e-4)
                     else:
                         means = np.clip(y[:, :2 * nu].reshape(N, nu, 2) + bias[None, :, None], -0.3, 0.3)
                         assert np.abs(means - act_t[..., None]).min(-1).max() < 2e-4
                 fresh = done[t].astype(bool)
             np.testing.assert_allclose(env.actor_carry.cpu().numpy(), want["actor"], rtol=2e-4, atol=2e-4)
+            if head == "gaussian-lowpass":
+                np.testing.assert_allclose(env.lpf_state.cpu().numpy(), want["lpf"], rtol=2e-4, atol=2e-4)
         runs.append(snaps)
         assert use_graph or finished > 0, "no env finished: the carry restart was not exercised"
     for it, (a, b) in enumerate(zip(*runs)):
@@ -554,6 +569,48 @@ def test_recurrent_policy_update_from_a_rollout(head):
         assert policy.kl_coef(cfg) == pytest.approx(coef, rel=1e-5)
         on_lp, _ = pu.recurrent_on_policy(policy, args[0], args[1], args[2], *args[6:])
     assert moved > 0
+
+
+def test_kbot_policy_update_from_a_rollout_with_filter_and_mirror_losses():
+    """The K-Bot task's update on a rollout's own buffers: the actor's means are filtered in the rollout, so the on-policy
+    pass has to replay the filter from the recorded first-step state and episode starts to reproduce the rollout's
+    log-probabilities; then minibatch steps with both mirror losses (the mirrored pass starts from zero carries, which is
+    what the task's rollout leaves in `actor_mirror`, `critic_mirror` and `lpf_params_mirror`)."""
+    from ksim_amd import ppo_update as pu
+    from ksim_amd.env_terms import sample_action_head
+
+    N, T = 32, 8
+    m, c, rnd_, _, ro, EnvState = build(N, T, seed=19, min_height=0.95, recurrent=True, head="kbot")
+    ps = c.engine.reset(c.physics_model, 1.0, 3, N, rnd_)
+    env = EnvState(ps, rnd_, torch.zeros(N, 2, device=DEV), None, seed=29)
+    for _ in range(3):
+        traj, rew = ro.unroll(env)
+    assert ro.fresh.sum().item() > 0 and ro.lpf_carry0.abs().max().item() > 0
+    K = c.terms.obs_dim
+    rng = np.random.default_rng(3)
+    operm, osign = rng.permutation(K), rng.choice([-1.0, 1.0], K)
+    aperm, asign = pu.kbot_mirror_joints()
+    policy = pu.RecurrentHeadPolicy(c.actor, c.critic, c.head.min_std, c.head.max_std, c.head.var_scale, c.head.mean_bias,
+                                    lowpass=c.head.lowpass, mirror=pu.MirrorSpec(list(operm), list(osign), list(operm), list(osign), aperm, asign))
+    policy.train_init()
+    args = (traj.obs["noisy_obs"], traj.obs["obs"], traj.action, rew.total, traj.done, traj.success, ro.actor_carry0, ro.critic_carry0, ro.fresh)
+    on_lp, on_v, loc = pu.recurrent_on_policy(policy, args[0], args[1], args[2], *args[6:], lpf0=ro.lpf_carry0, return_raw=True)
+    assert torch.equal(on_v, ro.values[..., 0])
+    # the replay (networks from the recorded carries, filter from the recorded state, both restarted at the recorded
+    # episode starts) arrives at the last step with the very rows the rollout sampled its last action from
+    assert torch.equal(loc[T - 1], ro.mean) and torch.isfinite(on_lp).all()
+    without = pu.recurrent_on_policy(policy, args[0], args[1], args[2], *args[6:], lpf0=None)[0]
+    assert not torch.equal(without, on_lp)  # the recorded filter state matters
+    before = [p.clone() for cell in c.actor.cells for p in cell.parameters().values()]
+    cfg = pu.PPOUpdateConfig(batch_size=16, num_passes=2, learning_rate=1e-3, actor_mirror_loss_scale=1.0, critic_mirror_loss_scale=0.5)
+    out = pu.update_model_recurrent(policy, cfg, *args, seed=1, lpf0=ro.lpf_carry0)
+    assert len(out) == 4 and all(torch.isfinite(o["grad_norm"]).all() and o["grad_norm"].item() > 0 for o in out)
+    assert all(o["action_mirror_loss"].shape == (T, 16) and o["action_mirror_loss"].mean().item() > 0 for o in out)
+    assert all(torch.isfinite(o["value_mirror_loss"]).all() for o in out)
+    after = [p for cell in c.actor.cells for p in cell.parameters().values()]
+    assert all(torch.isfinite(a).all() and not torch.equal(a, b) for a, b in zip(after, before))
+    traj2, _ = ro.unroll(env)
+    assert torch.isfinite(traj2.action).all() and torch.isfinite(env.lpf_state).all()
 
 
 def test_split_rollout_equals_single_stream_rollout():
@@ -741,7 +798,7 @@ def test_site_frame_sensors_follow_the_live_state_in_a_rollout():
     rng = np.random.default_rng(41)
     act = actuators.PositionActuators(kps=(30.0,) * m.nu, kds=(1.0,) * m.nu, ctrl_clip=(20.0,) * m.nu)
     resets = [rs.RandomJointPositionReset(scale=0.2, scale_by_curriculum=False)]
-    eng = engine.get_physics_engine("hip", resets, {}, act, engine.EngineConfig(dt=0.005, ctrl_dt=0.02))
+    eng = engine.get_physics_engine("hip", resets, {}, act, engine.EngineConfig(dt=m.dt, ctrl_dt=4 * m.dt))
     observations = {"jp": ob.JointPositionObservation(),
                     "foot": ob.SensorObservation.create(physics_model=m, sensor_name="left_foot_pos"),
                     "quat": ob.SensorObservation.create(physics_model=m, sensor_name="imu_quat")}

@@ -153,7 +153,7 @@ def test_termination_kats_and_masks_bit_exact():
         "length_off": tm.EpisodeLengthTermination(1.5, disable_at_curriculum_level=1),
         "length_on": tm.EpisodeLengthTermination(1.5, disable_at_curriculum_level=0.25, pos_termination=False),
         "length_at": tm.EpisodeLengthTermination(1.5, disable_at_curriculum_level=0.4),
-        "far_neg": tm.FarFromOriginTermination(2.0, pos_termination=False),
+        "far_neg": tm.FarFromOriginTermination(6.0, pos_termination=False),
     }
     terms = EnvTerms(m, {}, term_objs, [])
     level = 0.4
@@ -168,14 +168,14 @@ def test_termination_kats_and_masks_bit_exact():
             ot.episode_length_termination(t32_, 1.5, True, np.float32(level), 1),
             ot.episode_length_termination(t32_, 1.5, False, np.float32(level), 0.25),
             ot.episode_length_termination(t32_, 1.5, True, np.float32(level), np.float32(0.4)),
-            ot.far_from_origin_termination(q32, 2.0, pos_termination=False)]
+            ot.far_from_origin_termination(q32, 6.0, pos_termination=False)]
     assert not want[6].any() and (want[7] == -1).sum() > 20 and np.array_equal(want[8], want[5])
     got = comps.cpu().numpy()
     # exclude the measure-zero band where fp32 and float64 evaluation of a norm/acos straddle the threshold
     near = np.zeros(N, bool)
     near |= np.abs(np.linalg.norm(v32[:, :3], axis=1) - 2.5) < 1e-5
     near |= np.abs(np.linalg.norm(q32[:, :3], axis=1) - 3.0) < 1e-5
-    near |= np.abs(np.linalg.norm(q32[:, :3], axis=1) - 2.0) < 1e-5
+    near |= np.abs(np.linalg.norm(q32[:, :3], axis=1) - 6.0) < 1e-5
     for j, w in enumerate(want):
         assert np.array_equal(got[j][~near], w[~near]), list(term_objs)[j]
     wd, ws = ot.combine_terminations([g for g in got])

@@ -2,6 +2,7 @@
 import math
 
 import numpy as np
+import pytest
 import torch
 
 from oracle import ppo as oppo
@@ -110,3 +111,112 @@ def test_mixture_head_in_torch_matches_the_numpy_oracle_and_bounds_the_entropy()
     h_mc = -l[:, 0].mean()
     assert h_mc <= float(ent[0, 0]) + 0.01
     assert float(ent[0, 0]) - h_mc < np.log(K) + 0.01  # and within the mixing entropy of it
+
+
+def _kbot_case(rng, Tn=6, b=5, I=12, H=8, nu=4):
+    """A small K-Bot-shaped problem: LSTM actor (means | raw deviations) and critic, episode starts inside the slice, the
+    last two observation columns feeding the bias of the last two action means."""
+    def make(out_dim):
+        proj = (rng.normal(size=(H, I)) / np.sqrt(I), rng.normal(size=H) * 0.1)
+        cells = [(rng.normal(size=(4 * H, H)) / np.sqrt(H), rng.normal(size=(4 * H, H)) / np.sqrt(H), rng.normal(size=4 * H) * 0.1)
+                 for _ in range(2)]
+        return dict(input_proj=proj, cells=cells, out_w=[rng.normal(size=(out_dim, H)) / np.sqrt(H)], out_b=[rng.normal(size=out_dim) * 0.1],
+                    carry0=rng.normal(size=(2, 2, b, H)) * 0.3)
+
+    oa, oc = make(2 * nu), make(1)
+    head = dict(min_std=0.01, max_std=1.0, var_scale=0.5, mean_bias=rng.normal(size=nu) * 0.1)
+    obs = rng.normal(size=(Tn, b, I))
+    fresh = rng.random((Tn, b)) < 0.25
+    fresh[2, 0] = True
+    done = np.roll(fresh, -1, axis=0); done[-1] = False
+    batch = dict(actor_obs=obs + rng.normal(size=obs.shape) * 0.01, critic_obs=obs, fresh=fresh, done=done,
+                 success=np.zeros((Tn, b), bool), rewards=rng.normal(size=(Tn, b)), action=rng.normal(size=(Tn, b, nu)) * 0.3,
+                 on_log_probs=rng.normal(size=(Tn, b, nu)) * 0.1 - 0.5, on_values=rng.normal(size=(Tn, b)) * 0.3)
+    lowpass = dict(ctrl_dt=0.02, cutoff=10.0, y0=rng.normal(size=(b, nu)) * 0.2, obs_bias=(I - 2, nu - 2, 2))
+    # a mirror map that swaps and negates entries (a signed permutation, like mirror_joints / mirror_obs of the task)
+    operm = rng.permutation(I); osign = rng.choice([-1.0, 1.0], I)
+    aperm = rng.permutation(nu); asign = rng.choice([-1.0, 1.0], nu)
+    mirror = dict(actor_obs=(operm, osign), critic_obs=(operm, osign), action=(aperm, asign), actor_scale=0.7, critic_scale=0.3,
+                  actor_carry0=rng.normal(size=(2, 2, b, H)) * 0.3, critic_carry0=rng.normal(size=(2, 2, b, H)) * 0.3,
+                  y0=rng.normal(size=(b, nu)) * 0.2)
+    return oa, oc, head, batch, lowpass, mirror
+
+
+def _bump(net, path, eps):
+    """A copy of the network dict with one parameter entry moved by eps; path = (key, ..., index tuple)."""
+    import copy
+
+    out = copy.deepcopy(net)
+    obj = out
+    for k in path[:-2]:
+        obj = obj[k]
+    arr = np.array(obj[path[-2]], dtype=np.float64)
+    arr[path[-1]] += eps
+    if isinstance(obj, tuple):
+        raise TypeError
+    obj[path[-2]] = arr
+    return out
+
+
+def test_kbot_loss_with_filter_and_mirror_carries_against_central_differences():
+    """The recurrent loss with the low-pass filter on the means (state carried through time, cut at episode starts) and the
+    mirrored second pass of both networks.  GAE enters as a constant and depends on the critic only, so central differences
+    of the whole loss in ACTOR parameters are the exact gradient; for the critic the mirror term alone is differenced."""
+    rng = np.random.default_rng(7)
+    oa, oc, head, batch, lowpass, mirror = _kbot_case(rng)
+    for n in (oa, oc):  # lists, so that single entries can be moved
+        n["cells"] = [list(c) for c in n["cells"]]
+        n["input_proj"] = list(n["input_proj"])
+    loss, ga, gc, aux = ou.recurrent_loss_and_grads(oa, oc, batch, CFG, head, lowpass=lowpass, mirror=mirror)
+    loss0, ga0, gc0, aux0 = ou.recurrent_loss_and_grads(oa, oc, batch, CFG, head, lowpass=lowpass)
+    # the auxiliary terms join the mean over (t, env) of the summed terms (ppo.py:241-244, 485-486)
+    assert loss - loss0 == pytest.approx(aux["action_mirror_loss"].mean() + aux["value_mirror_loss"].mean(), rel=1e-12)
+    assert aux["action_mirror_loss"].shape == batch["done"].shape and aux["action_mirror_loss"].min() > 0
+    np.testing.assert_allclose(aux["raw"], aux0["raw"], atol=0)  # the first pass does not see the mirrored one
+    eps = 1e-6
+    f = lambda a, c: ou.recurrent_loss_and_grads(a, c, batch, CFG, head, lowpass=lowpass, mirror=mirror)  # noqa: E731
+    for path, got in ((("input_proj", 0, (3, 5)), ga["input_proj"][0][3, 5]), (("input_proj", 1, (2,)), ga["input_proj"][1][2]),
+                      (("cells", 0, 0, (7, 1)), ga["cells"][0][0][7, 1]), (("cells", 1, 1, (20, 3)), ga["cells"][1][1][20, 3]),
+                      (("cells", 1, 2, (9,)), ga["cells"][1][2][9]), (("out_w", 0, (1, 4)), ga["out"][0][0][1, 4]),
+                      (("out_w", 0, (6, 2)), ga["out"][0][0][6, 2]), (("out_b", 0, (3,)), ga["out"][0][1][3])):
+        fd = (f(_bump(oa, path, eps), oc)[0] - f(_bump(oa, path, -eps), oc)[0]) / (2 * eps)
+        assert got == pytest.approx(fd, rel=2e-5, abs=1e-9), path
+    vm = lambda c: ou.recurrent_loss_and_grads(oa, c, batch, CFG, head, lowpass=lowpass, mirror=mirror)[3]["value_mirror_loss"].mean()  # noqa: E731
+    for path, pick in ((("input_proj", 0, (1, 2)), lambda g: g["input_proj"][0][1, 2]), (("cells", 0, 1, (5, 5)), lambda g: g["cells"][0][1][5, 5]),
+                       (("out_w", 0, (0, 3)), lambda g: g["out"][0][0][0, 3])):
+        fd = (vm(_bump(oc, path, eps)) - vm(_bump(oc, path, -eps))) / (2 * eps)
+        # the actor's mirror term does not touch the critic, so the difference of the two critic gradients is this term's
+        assert pick(gc) - pick(gc0) == pytest.approx(fd, rel=2e-5, abs=1e-9), path
+
+
+def test_kbot_filter_in_the_loss_is_the_numpy_scan_and_the_head_bias_moves_inside_it():
+    from oracle import terms as ot
+
+    rng = np.random.default_rng(8)
+    oa, oc, head, batch, lowpass, _ = _kbot_case(rng)
+    nu = batch["action"].shape[-1]
+    _, _, _, plain = ou.recurrent_loss_and_grads(oa, oc, batch, CFG, head)
+    _, _, _, filt = ou.recurrent_loss_and_grads(oa, oc, batch, CFG, head, lowpass=lowpass)
+    col0, a0, cnt = lowpass["obs_bias"]
+    x = plain["raw"][..., :nu] + head["mean_bias"]
+    x[..., a0:a0 + cnt] += batch["actor_obs"][..., col0:col0 + cnt]
+    want, _ = ot.lowpass_scan(x, lowpass["ctrl_dt"], lowpass["cutoff"], lowpass["y0"], batch["fresh"])
+    np.testing.assert_allclose(filt["raw"][..., :nu], want, rtol=1e-12, atol=1e-14)
+    np.testing.assert_allclose(filt["raw"][..., nu:], plain["raw"][..., nu:], atol=0)
+
+
+def test_mirror_terms_vanish_for_a_mirror_symmetric_recurrent_policy():
+    """A policy that commutes with the mirror map (here: the map is the identity permutation with all signs +1, mirrored
+    carries and filter state equal to the first pass's) must have zero mirror losses and contribute no gradient."""
+    rng = np.random.default_rng(9)
+    oa, oc, head, batch, lowpass, mirror = _kbot_case(rng)
+    I, nu = batch["actor_obs"].shape[-1], batch["action"].shape[-1]
+    ident = dict(mirror, actor_obs=(np.arange(I), np.ones(I)), critic_obs=(np.arange(I), np.ones(I)), action=(np.arange(nu), np.ones(nu)),
+                 actor_carry0=oa["carry0"], critic_carry0=oc["carry0"], y0=lowpass["y0"])
+    loss, ga, gc, aux = ou.recurrent_loss_and_grads(oa, oc, batch, CFG, head, lowpass=lowpass, mirror=ident)
+    loss0, ga0, gc0, _ = ou.recurrent_loss_and_grads(oa, oc, batch, CFG, head, lowpass=lowpass)
+    assert np.abs(aux["action_mirror_loss"]).max() == 0 and np.abs(aux["value_mirror_loss"]).max() == 0 and loss == loss0
+    np.testing.assert_allclose(ga["out"][0][0], ga0["out"][0][0], atol=1e-15)
+    # and with different mirrored carries the same weights no longer agree: the carries do enter
+    other = dict(ident, actor_carry0=mirror["actor_carry0"])
+    assert ou.recurrent_loss_and_grads(oa, oc, batch, CFG, head, lowpass=lowpass, mirror=other)[3]["action_mirror_loss"].max() > 1e-6

@@ -859,3 +859,51 @@ def test_site_frame_sensors_against_scipy_rotations():
         got = ot.site_frame_quaternion(qb, qs)
         assert min(np.abs(got - want).max(), np.abs(got + want).max()) < 1e-12
         np.testing.assert_allclose(ot.site_magnetometer(qb, qs, field), (Rb * Rs).inv().apply(field), atol=1e-12)
+
+
+def test_lowpass_scan_and_its_backward_sweep():
+    """The filter threaded through a trajectory: equal to stepping ksim.lowpass_one_pole (pinned above by its closed form),
+    restarted from zero at fresh steps; the written-out reverse sweep against central differences of the forward scan."""
+    rng = np.random.default_rng(31)
+    Tn, b, n = 9, 4, 3
+    dt, fc = 0.02, 7.0
+    a = dt / (1.0 / (2 * np.pi * fc) + dt)
+    x = rng.normal(size=(Tn, b, n))
+    y0 = rng.normal(size=(b, n))
+    fresh = np.zeros((Tn, b), bool)
+    fresh[4, 1] = fresh[0, 2] = fresh[8, 3] = fresh[5, 3] = True
+    y, last = ot.lowpass_scan(x, dt, fc, y0, fresh)
+    # env 0 never restarts: the closed form y_t = (1-a)^(t+1) y0 + a sum_s (1-a)^(t-s) x_s
+    for t in range(Tn):
+        want = (1 - a) ** (t + 1) * y0[0] + a * sum((1 - a) ** (t - s) * x[s, 0] for s in range(t + 1))
+        np.testing.assert_allclose(y[t, 0], want, rtol=1e-12)
+    # env 1 restarts at step 4: from there on the history before it and y0 are forgotten
+    for t in range(4, Tn):
+        want = a * sum((1 - a) ** (t - s) * x[s, 1] for s in range(4, t + 1))
+        np.testing.assert_allclose(y[t, 1], want, rtol=1e-12)
+    np.testing.assert_allclose(y[0, 2], a * x[0, 2], rtol=1e-12)  # fresh at the first step: y0 is not used
+    np.testing.assert_allclose(last, y[-1], atol=0)
+    # constant input from zero: y_k = x (1 - (1-a)^k)
+    c, _ = ot.lowpass_scan(np.full((6, 1, 1), 2.0), dt, fc)
+    np.testing.assert_allclose(c[:, 0, 0], 2.0 * (1 - (1 - a) ** np.arange(1, 7)), rtol=1e-12)
+    # backward: L = sum(w * y); the recursion is linear, so central differences are exact up to rounding
+    w = rng.normal(size=y.shape)
+    dx, dy0 = ot.lowpass_scan_backward(w, dt, fc, fresh)
+    L = lambda x_, y0_: float((w * ot.lowpass_scan(x_, dt, fc, y0_, fresh)[0]).sum())  # noqa: E731
+    eps = 1e-5
+    for idx in [(0, 0, 0), (3, 1, 2), (4, 1, 0), (8, 3, 1), (5, 3, 2), (2, 2, 1), (7, 0, 2)]:
+        xp, xm = x.copy(), x.copy()
+        xp[idx] += eps; xm[idx] -= eps
+        assert dx[idx] == pytest.approx((L(xp, y0) - L(xm, y0)) / (2 * eps), rel=1e-7, abs=1e-10), idx
+    for idx in [(0, 0), (1, 2), (2, 1), (3, 0)]:
+        yp, ym = y0.copy(), y0.copy()
+        yp[idx] += eps; ym[idx] -= eps
+        assert dy0[idx] == pytest.approx((L(x, yp) - L(x, ym)) / (2 * eps), rel=1e-7, abs=1e-10), idx
+    assert np.all(dy0[2] == 0)  # env 2 is fresh at step 0: its y0 reaches nothing
+    # the cut: inputs of env 1 before its restart at step 4 reach only the outputs before it
+    w_late = np.zeros_like(w); w_late[4:, 1] = 1.0
+    assert np.all(ot.lowpass_scan_backward(w_late, dt, fc, fresh)[0][:4, 1] == 0)
+    # without any restart dx_s = a sum_{t>=s} (1-a)^(t-s) w_t
+    dx_free, _ = ot.lowpass_scan_backward(w, dt, fc)
+    s_ = 3
+    np.testing.assert_allclose(dx_free[s_, 0], a * sum((1 - a) ** (t - s_) * w[t, 0] for t in range(s_, Tn)), rtol=1e-12)
