@@ -19,6 +19,10 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
 BF16_PEAK_TFLOPS = 2500.0  # dense MFMA bf16
 FP32_VALU_PEAK_TFLOPS = 157.3
+# Untimed control steps every rollout of this file runs before its warm-up: the robots start on both feet, and it takes a
+# few seconds of simulated time before falls, resets and airborne envs are in their steady proportions.  Independent of
+# --warmup, so that a short timed window measures the same mixture as a long one.
+PREROLL_STEPS = 240
 
 
 def cpu_baseline(integrator: str, target_seconds: float = 12.0):
@@ -161,14 +165,27 @@ def main() -> None:
     head = timed_rollout(torch, args.integrator, N, T, args.steps, args.warmup, args.streams)
     consts, elapsed, kernel_ms, ndone = (head[k] for k in ("consts", "elapsed", "kernel_ms", "ndone"))
     envs_per_launch = head["envs_per_launch"]
+    head_stats = {k: head[k] for k in ("nefc_mean", "niter_mean", "in_contact")}
     m = consts.physics_model.model
     other = "implicitfast" if args.integrator == "euler" else "euler"
     if args.only == "rollout":  # the timed rollout alone: what the kernel-trace and counter runs of the step kernel profile
         print(json.dumps({"value": N * args.steps / elapsed, "ms_per_step": elapsed / args.steps * 1e3,
                           "step_kernel_ms": kernel_ms, "integrator": integrator_name(m), "num_envs": N, "rollout_length": T,
-                          "streams": args.streams, "envs_per_step_launch": envs_per_launch}))
+                          "streams": args.streams, "envs_per_step_launch": envs_per_launch,
+                          "untimed_preroll_steps": PREROLL_STEPS, "episodes_finished_in_timed_region": ndone,
+                          "constraint_rows_mean": head["nefc_mean"], "newton_iterations_mean": head["niter_mean"],
+                          "envs_in_contact": head["in_contact"]}))
         return
     del head
+    # The same rollout over a window long enough that filling and draining the two launch chains (about one control step
+    # at each end of the bracketing synchronisations) no longer shows: the figure a training run sees.
+    long_entry = None
+    if args.steps < 200:
+        lg = timed_rollout(torch, args.integrator, N, args.rollout, 200, 0, args.streams)
+        long_entry = {"value": N * lg["steps"] / lg["elapsed"], "unit": "env-steps/s", "steps": lg["steps"],
+                      "ms_per_step": lg["elapsed"] / lg["steps"] * 1e3, "step_kernel_ms": lg["kernel_ms"],
+                      "rollout_length": args.rollout, "episodes_finished_in_timed_region": lg["ndone"]}
+        del lg
     alt = timed_rollout(torch, other, N, T, max(T, min(args.steps, 2 * T)), min(args.warmup, T), args.streams)
     other_entry = {"integrator": integrator_name(alt["consts"].physics_model.model),
                    "value": N * alt["steps"] / alt["elapsed"], "unit": "env-steps/s", "steps": alt["steps"],
@@ -235,7 +252,10 @@ def main() -> None:
                                f"group(s), one HIP stream each",
                    "integrator": integrator_name(m), "num_envs": N, "rollout_length": T, "substeps": 4,
                    "streams": args.streams, "envs_per_step_launch": envs_per_launch,
-                   "obs_dim": obs_dim, "episodes_finished_in_last_rollout": ndone},
+                   "obs_dim": obs_dim, "untimed_preroll_steps": PREROLL_STEPS,
+                   "episodes_finished_in_timed_region": ndone,
+                   "constraint_rows_mean": head_stats["nefc_mean"], "newton_iterations_mean": head_stats["niter_mean"],
+                   "envs_in_contact": head_stats["in_contact"]},
         "roofline": {"bound": "hbm", "kernel": "step_kernel (fused control step)", "achieved": achieved,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
                      "algorithmic_bytes_per_env_step": bytes_per_env, "kernel_ms": kernel_ms,
@@ -247,7 +267,7 @@ def main() -> None:
                      "note": "the fused step is bound by fp32 vector-ALU issue (~1e3 flop/byte; the profiled share of "
                              "cycles with a VALU instruction issuing is given beside); the HBM fraction is reported "
                              "against the bytes the engine contract obliges a step to move"},
-        "other_integrator": other_entry, "single_stream": single_entry,
+        "same_rollout_200_steps": long_entry, "other_integrator": other_entry, "single_stream": single_entry,
         "gae": gae, "streaming": streaming, "policy_mlp": mlp, "ppo_update": upd, "ppo_iteration": iteration, "graph_replay": graph,
     }
     if not args.no_cpu_baseline:
@@ -266,8 +286,9 @@ def main() -> None:
     print(json.dumps(line))
 
 
-def timed_rollout(torch, integrator: str, N: int, T: int, steps: int, warmup: int, streams: int = 2) -> dict:
-    """`warmup` untimed control steps, then exactly `steps` timed ones of the cfg 4 rollout built with `integrator`.
+def timed_rollout(torch, integrator: str, N: int, T: int, steps: int, warmup: int, streams: int = 2,
+                  preroll: int = PREROLL_STEPS) -> dict:
+    """`preroll` + `warmup` untimed control steps, then exactly `steps` timed ones of the cfg 4 rollout built with `integrator`.
     The rollout slot restarts at 0 where the timed region begins, so it holds steps // T reward + GAE passes.
     `streams`: the N envs run as that many independent groups, each on its own HIP stream (1 = one launch chain)."""
     from ksim_amd.configs import kbot_rollout, kbot_split_rollout
@@ -304,26 +325,53 @@ def timed_rollout(torch, integrator: str, N: int, T: int, steps: int, warmup: in
                 rew = get_rewards(ro.trajectory(), consts.rewards, want_components=False)
                 ro.ppo_inputs(rew, 0.99, 0.95, normalize_advantages=True)
 
+    parts = ro.parts if streams > 1 else [ro]
+    states = envs if streams > 1 else [env]
+    group_streams = ro.streams if streams > 1 else [torch.cuda.current_stream()]
+    # episodes that end inside the timed region: each group adds up the done flags of a rollout's slots when the rollout is
+    # complete (one small reduction per group and T steps, on the group's stream, no host synchronisation)
+    finished = [torch.zeros((), dtype=torch.int64, device="cuda") for _ in parts]
+
+    def count_finished(k: int) -> None:
+        if k % T == T - 1 or k == steps - 1:
+            for part, st, acc in zip(parts, group_streams, finished):
+                with torch.cuda.stream(st):
+                    acc += part.done[: k % T + 1].sum()
+
     if streams > 1:
         ro.fork()
-    for k in range(warmup):
+    for k in range(preroll + warmup):
         one_step(k % T)
+    count_finished(T - 1)  # the reduction's first launch loads its code object: not inside the timed region
+    for acc in finished:
+        acc.zero_()
     consts.engine.step = timed_step
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for k in range(steps):
         one_step(k % T)
+        count_finished(k)
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     consts.engine.step = orig_step
     kernel_ms = sum(a.elapsed_time(b) for a, b in step_events) / len(step_events)
-    parts = ro.parts if streams > 1 else [ro]
-    states = envs if streams > 1 else [env]
-    ndone = sum(int(p.done.sum().item()) for p in parts)
+    ndone = sum(int(f.item()) for f in finished)
+    # what the solver is working on in this state of the simulation: constraint rows and Newton iterations of the last
+    # substep of one more (untimed) control step
+    nefc, niter, contact = [], [], []
+    for part, e, st in zip(parts, states, group_streams):
+        with torch.cuda.stream(st):
+            stats = {k: torch.zeros(part.N, dtype=torch.int32, device="cuda") for k in ("nefc", "solver_niter")}
+            consts.engine.step(part.action[0], consts.physics_model, e.physics_state, 1.0, e.seed + e.step, e.randomization_dict, stats=stats)
+        torch.cuda.synchronize()
+        nefc.append(stats["nefc"].float().mean().item())
+        niter.append(stats["solver_niter"].float().mean().item())
+        contact.append((stats["nefc"] > 0).float().mean().item())
     for e in states:
         assert torch.isfinite(e.physics_state.data.qpos).all(), "non-finite state after the benchmark"
+    g = len(parts)
     return dict(consts=consts, env=states[0], ro=parts[0], elapsed=elapsed, kernel_ms=kernel_ms, ndone=ndone, steps=steps,
-                envs_per_launch=N // streams)
+                envs_per_launch=N // streams, nefc_mean=sum(nefc) / g, niter_mean=sum(niter) / g, in_contact=sum(contact) / g)
 
 
 def gae_bandwidth(torch, ppo, reps=8):

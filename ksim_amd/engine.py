@@ -290,10 +290,12 @@ class HipEngine(PhysicsEngine):
              noise: Mapping[str, torch.Tensor] | None = None,
              record: Mapping[str, torch.Tensor] | None = None, want_cvel: bool = True, want_cinert: bool = False,
              want_cfrc_ext: bool = False,
-             step: int = 0, step_base=None, event_seed: int = 0, live=None) -> PhysicsState:
+             step: int = 0, step_base=None, event_seed: int = 0, live=None, stats: Mapping[str, torch.Tensor] | None = None) -> PhysicsState:
         """`live`: names among qacc, ctrl, xpos, xquat, contact_dist of the derived fields of `physics_state.data` that
         the caller reads afterwards (None = all).  The rollout records ctrl / xpos / xquat into its own slot through
-        `record`, so a task whose observations read none of them need not have them written twice."""
+        `record`, so a task whose observations read none of them need not have them written twice.
+        `stats`: optional int32 (N,) buffers `nefc` and `solver_niter` that receive the constraint rows and Newton iterations
+        of the last substep (diagnostics; the reference exposes the same numbers as `data.nefc` / `data.solver_niter`)."""
         m, d, s = physics_model.model, physics_state.data, physics_state
         rnd, noise, record = randomization or {}, noise or {}, record or {}
         keep = (lambda name, b: b) if live is None else (lambda name, b: b if name in live else None)
@@ -314,6 +316,8 @@ class HipEngine(PhysicsEngine):
                    action_noise=noise.get("action_noise"),
                    torque_noise=noise.get("torque_noise"), traj_ctrl=record.get("ctrl"),
                    traj_xpos=record.get("xpos"), traj_xquat=record.get("xquat"))
+        if stats:
+            buf.update({k: stats[k] for k in ("nefc", "solver_niter") if k in stats})
         # heaviest-first launch order from the previous step's cost estimates (kept on the state object)
         sched = self.prepare_state(s)
         if sched is not None:
