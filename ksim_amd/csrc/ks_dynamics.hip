@@ -142,15 +142,16 @@ __device__ __forceinline__ void chol_tile(f32x16& T, float (&R)[NP], float& myin
   for (int j = 0; j < NP; ++j) {
     if (j >= padded_from(NP) && j >= nv) continue;  // a padded column: unit pivot, nothing below or right of it
     const int hj = (j >> 2) & 1, rho = 4 * (j >> 3) + (j & 3);
-    const float piv = fmaxf(lane_bcast(T[rho], j + 32 * hj), 1e-30f);
-    const float inv = __builtin_amdgcn_rsqf(piv);
+    // a pivot below 1e-30 (or not a number) counts as 1e-30: the reciprocal root is capped instead of the pivot floored,
+    // which is the same number and one instruction less on the chain
+    const float inv = fminf(__builtin_amdgcn_rsqf(lane_bcast(T[rho], j + 32 * hj)), 1e15f);
     myinv = lane == j ? inv : myinv;
     const bool sel = half == hj && c > j;
     const float t = T[rho] * inv;
-    const float a = sel ? t : 0.f;
+    const float a = sel ? t : 0.f, na = sel ? -t : 0.f;
     T[rho] = sel ? t : T[rho];
     // the last real column has nothing right of or below it
-    if (j + 1 < NP && !(j + 1 >= padded_from(NP) && j + 1 >= nv)) T = __builtin_amdgcn_mfma_f32_32x32x2f32(-a, a, T, 0, 0, 0);
+    if (j + 1 < NP && !(j + 1 >= padded_from(NP) && j + 1 >= nv)) T = __builtin_amdgcn_mfma_f32_32x32x2f32(na, a, T, 0, 0, 0);
   }
 #pragma unroll
   for (int g = 0; g < 4; ++g)
@@ -209,10 +210,12 @@ __device__ __forceinline__ float row_dot(const float* row, const float (&vv)[NP]
   const float4* q = reinterpret_cast<const float4*>(row);
   float s0 = 0.f, s1 = 0.f;
 #pragma unroll
-  for (int k = 0; k < NP / 4; ++k) {
+  for (int k = 0; k < NP / 4; ++k) {  // two chains of fused multiply-adds, one instruction per product
     const float4 t = q[k];
-    s0 += t.x * vv[4 * k] + t.z * vv[4 * k + 2];
-    s1 += t.y * vv[4 * k + 1] + t.w * vv[4 * k + 3];
+    s0 = fmaf(t.x, vv[4 * k], s0);
+    s1 = fmaf(t.y, vv[4 * k + 1], s1);
+    s0 = fmaf(t.z, vv[4 * k + 2], s0);
+    s1 = fmaf(t.w, vv[4 * k + 3], s1);
   }
   return s0 + s1;
 }
@@ -832,32 +835,36 @@ void step_kernel(StepArgs a) {
       ndr = __popcll(__ballot(dr.lim_s != 0.f)) + __popcll(__ballot(dr.fr_fl > 0.f));
     }
     if (nefc > 0 || (DR && ndr > 0)) {
-      // ---- constraint rows: lane r builds row r of J in registers and mirrors it to LDS for column access
+      // ---- constraint rows.  Lane j builds column j of J: the motion axis of dof j is one LDS read away, so a contact
+      // costs the lane one cross product and its four pyramid edges, written to LDS row-wise (consecutive lanes,
+      // consecutive addresses).  The row lanes then take their reference acceleration from a row product with qvel.
       const bool is_row = lane < nefc;
       float aref = 0.f, D = 0.f;
       {
-        const int c = is_row ? (frictionless ? lane : lane >> 2) : 0, q = lane & 3;
-        const unsigned cm = is_row ? l.con_mask[c] : 0u;
-        const V3 off = ld3(l.con_off + 3 * c);
-        const float smu = (q & 1) ? -mu : mu;
-        unsigned um = 0;  // union of the dof masks of the active contacts (wave-uniform)
-        for (int k = 0; k < ncon; ++k) um |= l.con_mask[k];
-        float vv[NP];
-        load_row<NP>(l.qvel, vv);
-        float vel = 0.f;
-#pragma unroll
-        for (int j = 0; j < NP; ++j) {
-          float val = 0.f;
-          if ((um >> j) & 1u) {
-            const Sp cd = ld6(l.cdof + 6 * j);
-            const V3 jac = cd.l + cross(cd.a, off);
-            const float tang = (q < 2) ? jac.y : -jac.x;
-            val = ((cm >> j) & 1u) ? (frictionless ? jac.z : jac.z + smu * tang) : 0.f;
+        const bool col = lane < NP;  // the padding columns are written too (zeros): the row products read NP floats
+        const Sp cd = ld6(l.cdof + 6 * (is_dof ? lane : 0));
+        float* Jc = l.J + (col ? lane : 0);
+        for (int k = 0; k < ncon; ++k) {  // wave-uniform
+          const V3 off = ld3(l.con_off + 3 * k);
+          const bool on = is_dof && ((l.con_mask[k] >> lane) & 1u);
+          const V3 jac = cd.l + cross(cd.a, off);
+          if (frictionless) {
+            if (col) Jc[k * js] = on ? jac.z : 0.f;
+          } else if (col) {  // rows of a contact: z + mu y, z - mu y, z - mu x, z + mu x
+            Jc[(4 * k) * js] = on ? jac.z + mu * jac.y : 0.f;
+            Jc[(4 * k + 1) * js] = on ? jac.z - mu * jac.y : 0.f;
+            Jc[(4 * k + 2) * js] = on ? jac.z - mu * jac.x : 0.f;
+            Jc[(4 * k + 3) * js] = on ? jac.z + mu * jac.x : 0.f;
           }
-          vel += val * vv[j];
-          if (is_row) l.J[lane * js + j] = val;
         }
+        if (frictionless && col)  // whole blocks of four rows are read back below: the tail of the last block is zero
+          for (int r = nefc; r < ((nefc + 3) & ~3); ++r) Jc[r * js] = 0.f;
+        KS_SYNC();
         if (is_row) {
+          const int c = frictionless ? lane : lane >> 2;
+          float vv[NP];
+          load_row<NP>(l.qvel, vv);
+          const float vel = row_dot<NP>(l.J + lane * js, vv);
           aref = -m.con_b * vel - l.con_kip[c];
           D = l.con_D[c];
         }
@@ -908,9 +915,27 @@ void step_kernel(StepArgs a) {
         const float force = active ? -D * Jaref : 0.f;
         unsigned long long am = __ballot(active);
         float qfc = 0.f;
-        for (unsigned long long t = am; t; t &= t - 1) {
-          const int r = __builtin_ctzll(t);
-          qfc += l.J[r * js + (lane < nv ? lane : 0)] * lane_bcast(force, r);
+        if (nefc <= 32) {
+          // J^T f with the rows split between the lane halves: the forces go through LDS (one 16-byte broadcast read per
+          // block of four rows), lane j of half h sums the blocks 2 i + h of column j, and the halves meet at the end.
+          if (lane < 32) l.vbuf[lane] = force;  // zero beyond the rows and on the inactive ones
+          KS_SYNC();
+          const int jc = (lane & 31) < nv ? (lane & 31) : 0, hh = lane >> 5;
+          const int nblk = (nefc + 3) >> 2;
+          for (int b0 = 0; b0 < nblk; b0 += 2) {
+            const bool ok = b0 + hh < nblk;
+            const int bb = ok ? b0 + hh : 0;
+            const float4 f = *reinterpret_cast<const float4*>(l.vbuf + 4 * bb);
+            const float* Jb = l.J + (4 * bb) * js + jc;
+            const float sblk = (Jb[0] * f.x + Jb[js] * f.y) + (Jb[2 * js] * f.z + Jb[3 * js] * f.w);
+            qfc += ok ? sblk : 0.f;
+          }
+          qfc += __shfl_xor(qfc, 32);
+        } else {
+          for (unsigned long long t = am; t; t &= t - 1) {
+            const int r = __builtin_ctzll(t);
+            qfc += l.J[r * js + (lane < nv ? lane : 0)] * lane_bcast(force, r);
+          }
         }
         float dr_cost = 0.f, dr_force = 0.f, dr_h = 0.f;
         unsigned long long amd = 0ull;

@@ -99,9 +99,9 @@ __device__ __forceinline__ Quat qmul(Quat a, Quat b) {
           a.w * b.y - a.x * b.z + a.y * b.w + a.z * b.x, a.w * b.z + a.x * b.y - a.y * b.x + a.z * b.w};
 }
 __device__ __forceinline__ Quat qnormalize(Quat q) {
-  const float n = sqrtf(q.w * q.w + q.x * q.x + q.y * q.y + q.z * q.z);
-  if (n < 1e-15f) return {1.f, 0.f, 0.f, 0.f};
-  const float inv = 1.0f / n;
+  const float n2 = q.w * q.w + q.x * q.x + q.y * q.y + q.z * q.z;
+  if (n2 < 1e-30f) return {1.f, 0.f, 0.f, 0.f};
+  const float inv = __builtin_amdgcn_rsqf(n2);  // one instruction, 1 ulp: the quaternions here are within rounding of unit length
   return {q.w * inv, q.x * inv, q.y * inv, q.z * inv};
 }
 struct Mat3 {

@@ -295,7 +295,8 @@ class HipEngine(PhysicsEngine):
         the caller reads afterwards (None = all).  The rollout records ctrl / xpos / xquat into its own slot through
         `record`, so a task whose observations read none of them need not have them written twice.
         `stats`: optional int32 (N,) buffers `nefc` and `solver_niter` that receive the constraint rows and Newton iterations
-        of the last substep (diagnostics; the reference exposes the same numbers as `data.nefc` / `data.solver_niter`)."""
+        of the last substep (diagnostics; the reference exposes the same numbers as `data.nefc` / `data.solver_niter`), and
+        `dbg_M` (N, nv * nv) float32, which the profiling build of the library fills with cycle counts per phase."""
         m, d, s = physics_model.model, physics_state.data, physics_state
         rnd, noise, record = randomization or {}, noise or {}, record or {}
         keep = (lambda name, b: b) if live is None else (lambda name, b: b if name in live else None)
@@ -317,7 +318,7 @@ class HipEngine(PhysicsEngine):
                    torque_noise=noise.get("torque_noise"), traj_ctrl=record.get("ctrl"),
                    traj_xpos=record.get("xpos"), traj_xquat=record.get("xquat"))
         if stats:
-            buf.update({k: stats[k] for k in ("nefc", "solver_niter") if k in stats})
+            buf.update({k: stats[k] for k in ("nefc", "solver_niter", "dbg_M") if k in stats})
         # heaviest-first launch order from the previous step's cost estimates (kept on the state object)
         sched = self.prepare_state(s)
         if sched is not None:
