@@ -113,7 +113,7 @@ def main() -> None:
     ap.add_argument("--integrator", choices=("euler", "implicitfast"), default="euler",
                     help="velocity update of the headline rollout: semi-implicit Euler (what the benchmark configs name) or "
                          "implicitfast (what ksim's RLConfig selects); the other one is reported under 'other_integrator'")
-    ap.add_argument("--only", choices=("mlp", "gae", "update", "rollout", "iteration", "phases"), default=None,
+    ap.add_argument("--only", choices=("mlp", "gae", "update", "rollout", "iteration", "phases", "mfma"), default=None,
                     help="run one section alone and print its JSON (the command the counter runs under profiles/ use)")
     ap.add_argument("--mlp-rows", type=int, default=0, help="with --only mlp: a single row count instead of 8192 and 524288")
     ap.add_argument("--streams", type=int, default=2,
@@ -147,6 +147,9 @@ def main() -> None:
         del src, dst
     if args.only == "phases":
         print(json.dumps({"step_kernel_phases": step_kernel_phases(torch, args.integrator, args.envs)}))
+        return
+    if args.only == "mfma":
+        print(json.dumps({"mfma_yardstick": mfma_yardstick(torch)}))
         return
     if args.only == "mlp":
         print(json.dumps({"policy_mlp": mlp_rate(torch, rows=(args.mlp_rows,) if args.mlp_rows else (8192, 524288))}))
@@ -219,6 +222,10 @@ def main() -> None:
     gae = gae_bandwidth(torch, ppo)
     streaming = loss_and_reward_bandwidth(torch)
     mlp = mlp_rate(torch)
+    mlp["mfma_yardstick"] = mfma_yardstick(torch)
+    top = mlp["mfma_yardstick"]["all_cus_two_waves_per_simd"]["TFLOPs"]
+    for key in ("rows_8192", "rows_524288"):
+        mlp[key]["of_mfma_yardstick"] = mlp[key]["TFLOPs"] / top
     upd = ppo_update_rate(torch)
     iteration = ppo_iteration_rate(torch)
 
@@ -631,6 +638,36 @@ def ppo_iteration_rate(torch, reps=3):
             "rollout_s": parts["rollout"], "postprocess_and_update_s": parts["update"],
             "what": "one rl_train_loop_step: rollout, discriminator scoring, rewards + GAE, 32 actor/critic minibatch steps "
                     "(bf16 3x512) each followed by a discriminator step (71-256-256-1); host wall-clock per iteration"}
+
+
+def mfma_yardstick(torch, iters=20000):
+    """What a loop of nothing but 32x32x16 bf16 MFMAs on register operands reaches on this GPU (`ks_mfma_yardstick`): the
+    ceiling of any kernel built on that instruction, at the clock the part sustains under matrix load.  One wavefront per
+    SIMD (256 workgroups of four) and two per SIMD (512), the occupancy of the whole-network MLP kernel."""
+    from ksim_amd import _lib
+
+    lib = _lib.load()
+    out = {}
+    for name, wgs in (("one_cu", 1), ("all_cus_one_wave_per_simd", 256), ("all_cus_two_waves_per_simd", 512)):
+        sums = torch.empty(wgs * 256, device="cuda")
+        stamps = torch.zeros(wgs * 2, dtype=torch.int64, device="cuda")
+        _lib.check(lib.ks_mfma_yardstick(_lib.current_stream(), wgs, 200, _lib.ptr(sums), _lib.ptr(stamps)))  # warm-up
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        _lib.check(lib.ks_mfma_yardstick(_lib.current_stream(), wgs, iters, _lib.ptr(sums), _lib.ptr(stamps)))
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1)
+        st = stamps.view(wgs, 2).double()
+        n_mfma = iters * 8
+        cyc, ticks = st[:, 0].mean().item(), st[:, 1].mean().item()
+        tf = wgs * 4 * n_mfma * 32768.0 / (ms * 1e-3) / 1e12
+        out[name] = {"workgroups": wgs, "ms": ms, "TFLOPs": tf, "of_nominal_bf16_peak": tf / BF16_PEAK_TFLOPS,
+                     "shader_cycles_per_mfma_per_wave": cyc / n_mfma, "shader_clock_MHz_under_load": cyc / (ticks * 10.0) * 1e3}
+    out["what"] = ("a loop of v_mfma_f32_32x32x16_bf16 only, 8 independent accumulator tiles per wavefront, operands in registers; "
+                   "the clock is the ratio of the shader-cycle counter to the constant 100 MHz counter over the loop")
+    return out
 
 
 def mlp_rate(torch, rows=(8192, 524288), reps=20):

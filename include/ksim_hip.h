@@ -1055,6 +1055,13 @@ int ks_reward_scan(ks_stream_t stream, const KsRewardScanIO* io /*host*/);
  * A plain f32 copy of n elements (reads 4n bytes, writes 4n bytes): the known-size kernel that hardware
  * traffic counters are calibrated against.  No counterpart in the reference. */
 int ks_copy_f32(ks_stream_t stream, int64_t n, const float* src, float* dst);
+/* The matrix cores' own yardstick: `workgroups` workgroups of four wavefronts, each wavefront issuing `iters` x 8
+ * v_mfma_f32_32x32x16_bf16 on register operands (eight independent accumulator tiles, 32768 flop per instruction) and
+ * nothing else.  out (workgroups x 256 floats) receives checksums; stamps (2 per workgroup, nullable) the shader-clock
+ * cycles of the loop and the same interval in ticks of the constant 100 MHz counter, from which the clock under matrix
+ * load follows.  What this reaches is the ceiling of any kernel built on that instruction.  No counterpart in the
+ * reference. */
+int ks_mfma_yardstick(ks_stream_t stream, int32_t workgroups, int32_t iters, float* out, int64_t* stamps);
 
 #ifdef __cplusplus
 }

@@ -59,6 +59,8 @@ def load() -> ctypes.CDLL:
     lib.ks_reward_total.argtypes = [p, c_int64, c_int32, p, POINTER(c_float), c_int32, c_float, c_int32, c_float, p,
                                     c_int32, p, p, p]
     lib.ks_copy_f32.argtypes = [p, c_int64, p, p]
+    lib.ks_mfma_yardstick.argtypes = [p, c_int32, c_int32, p, p]
+    lib.ks_mfma_yardstick.restype = c_int32
     lib.ks_ppo_loss_grad.argtypes = [p, c_int64, c_int32, POINTER(KsPpoLossParams)] + [p] * 12
     lib.ks_ppo_loss_grad.restype = c_int32
     lib.ks_signed_permute.argtypes = [p, c_int64, c_int32, p, p, p, p]

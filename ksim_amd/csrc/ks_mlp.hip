@@ -213,6 +213,43 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void mlp_layer_kernel(int64
 }
 
 
+// ---------------------------------------------------------------- matrix-core yardstick
+// Nothing but 32x32x16 bf16 MFMAs on register operands: eight independent accumulator tiles per wavefront (the fused
+// kernel's own count), no loads, no LDS, no epilogue.  What this loop reaches is the most any kernel built on that
+// instruction can reach on this part at the clock it sustains under matrix load.  Per workgroup: stamps[2 b] = shader
+// clock cycles of the loop, stamps[2 b + 1] = the same interval on the constant 100 MHz counter.
+__global__ __launch_bounds__(256) void mfma_yardstick_kernel(int iters, float* __restrict__ out, long long* __restrict__ stamps) {
+  f32x16 acc[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[i][r] = 0.f;
+  bf16x8 a, b;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    // operands that differ between lanes and are neither zero nor all equal
+    const unsigned h = (threadIdx.x * 8u + e + blockIdx.x * 977u) * 2654435761u;
+    a[e] = (__bf16)(((float)(h >> 8) / 8388608.0f) - 1.0f);
+    b[e] = (__bf16)(((float)((h * 40503u) >> 8) / 8388608.0f) - 1.0f);
+  }
+  const long long c0 = clock64(), w0 = wall_clock64();
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc[i], 0, 0, 0);
+  }
+  const long long c1 = clock64(), w1 = wall_clock64();
+  float sum = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) sum += acc[i][r];
+  out[(int64_t)blockIdx.x * 256 + threadIdx.x] = sum;
+  if (stamps && threadIdx.x == 0) {
+    stamps[2 * (int64_t)blockIdx.x] = c1 - c0;
+    stamps[2 * (int64_t)blockIdx.x + 1] = w1 - w0;
+  }
+}
+
 // ---------------------------------------------------------------- whole network in one kernel (bf16)
 // A 512-thread workgroup keeps a BM-row tile of activations in LDS as bf16 for the whole network and walks the
 // layers in place; only the network input and output touch HBM.  The product is computed transposed,
@@ -1368,6 +1405,14 @@ extern "C" int ks_mlp_forward_pair(const KsMlp* h0, const KsMlp* h1, ks_stream_t
   const int rc = ks_mlp_forward(h0, stream, M, x0, y0, workspace0);
   if (rc != KS_OK) return rc;
   return ks_mlp_forward(h1, stream, M, x1, y1, workspace1);
+}
+
+extern "C" int ks_mfma_yardstick(ks_stream_t stream, int32_t workgroups, int32_t iters, float* out, int64_t* stamps) {
+  if (workgroups < 1 || iters < 1) return fail(KS_EINVAL, "ks_mfma_yardstick: workgroups and iterations must be positive");
+  if (!out) return fail(KS_EINVAL, "ks_mfma_yardstick: null output");
+  hipLaunchKernelGGL(mfma_yardstick_kernel, dim3((unsigned)workgroups), dim3(256), 0, (hipStream_t)stream, iters, out,
+                     reinterpret_cast<long long*>(stamps));
+  return check_launch("ks_mfma_yardstick");
 }
 
 extern "C" int64_t ks_mlp_workspace_bytes(const KsMlp* h, int64_t M) {
