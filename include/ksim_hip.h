@@ -317,6 +317,12 @@ typedef struct KsStepIO {
   const float* event_uniform;  /* (substeps, N, n_events, KS_EVENT_DRAWS) U[0,1) draws, nullable -> Philox */
   KsRng event_rng;
   float* event_force;          /* (n_events, N, KS_EVENT_FORCE_STATE) in/out; required when a force push is listed */
+  /* ks_step only, nullable: envs flagged here were reset by the termination pass and still owe the forward pass of
+     MjxEngine.reset (engine.py:213: mjx.forward on the reset state, whose solution becomes the new episode's warm
+     start).  The step runs that pass for them first, inside the same launch, with zero controls and without integrating;
+     what it leaves in qacc_warmstart is what a masked ks_forward before the step would have left.  The derived outputs of
+     the reset state itself (xpos, xquat ...) are not written: a caller whose terms read those runs ks_forward instead. */
+  const uint8_t* fresh;        /* (N) */
 } KsStepIO;
 
 int ks_step(const KsModel* model, ks_stream_t stream, const KsStepIO* io /*host*/);

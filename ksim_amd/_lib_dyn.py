@@ -52,7 +52,7 @@ class KsStepIO(ctypes.Structure):
     _fields_ = [("N", c_int64), ("substeps", c_int32), ("actuator_period", c_int32), ("actuator_type", c_int32),
                 ("action_scale", c_float)] + [(name, _P) for name in STEP_IO_POINTERS] + [
                     ("n_events", c_int32), ("events", _T.KsEventDesc * _T.KS_MAX_EVENTS), ("event_state", _P),
-                    ("event_uniform", _P), ("event_rng", _T.KsRng), ("event_force", _P)]
+                    ("event_uniform", _P), ("event_rng", _T.KsRng), ("event_force", _P), ("fresh", _P)]
 
 
 def model_desc(m) -> KsModelDesc:

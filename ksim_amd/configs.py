@@ -52,7 +52,7 @@ def _kbot_constants(seed: int, hidden: int, dtype: str, min_height: float, integ
     rewards = {"stay_alive": rw.StayAliveReward(scale=1.0), "base_height": rw.BaseHeightReward(scale=0.5, height_target=0.87),
                "upright": rw.UprightReward(scale=0.2), "action_velocity": rw.ActionVelocityPenalty(scale=0.01)}
     consts = RolloutConstants(physics_model=dm, engine=eng, terms=terms, rewards=rewards, actor=actor, critic=critic,
-                              log_std=torch.full((m.nu,), -2.0, device=dev))
+                              log_std=torch.full((m.nu,), -2.0, device=dev), defer_reset_forward=True)
     return m, consts, dict(kps=kps, kds=kds, clip=KBOT_TORQUE_LIMITS)
 
 

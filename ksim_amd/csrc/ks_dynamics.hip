@@ -369,7 +369,13 @@ void step_kernel(StepArgs a) {
 #endif
 
   const int nsub = FWD ? 1 : a.substeps;
-  for (int sub = 0; sub < nsub; ++sub) {
+  // An env that the termination pass has just reset still owes the forward pass of its reset (engine.py:213: derived
+  // quantities and the warm start of the new episode, from the reset state with zero controls).  With `fresh` given the
+  // step does it itself, as a pass `sub = -1` that neither actuates nor integrates, instead of a masked launch of the
+  // forward-only kernel between the termination pass and this step.
+  const bool fresh_env = !FWD && a.fresh && a.fresh[env];  // wave-uniform
+  for (int sub = fresh_env ? -1 : 0; sub < nsub; ++sub) {
+    const bool fwd = FWD || sub < 0;
     // The lane id is re-materialised per substep so that per-lane LDS addresses are recomputed inside the loop
     // instead of being hoisted out of it into ~130 long-lived registers (which would halve the occupancy).
     int lane_v = threadIdx.x;
@@ -419,7 +425,7 @@ void step_kernel(StepArgs a) {
     for (int k = 0; k < kMaxPairs / 64 + 1; ++k) pk[k] = rec.pk[k];
 
     // ---- actuators (ksim/engine.py:287-320, ksim/actuators.py:198-217)
-    if (!FWD && (sub % a.actuator_period) == 0 && lane < nu) {
+    if (!fwd && (sub % a.actuator_period) == 0 && lane < nu) {
       const int u = lane;
       // the actuator inputs of this control step are read again at every actuator update (they stay in the caches):
       // held in registers they would be live across the solver of every substep
@@ -461,7 +467,7 @@ void step_kernel(StepArgs a) {
     }
 
     // ---- events (ksim/engine.py:322-333, ksim/events.py): impulses on the root velocity when an interval runs out
-    if (!FWD && a.n_events > 0) {
+    if (!fwd && a.n_events > 0) {
       const uint64_t ev_step = a.event_rng.step + (a.event_rng.step_base ? *a.event_rng.step_base : 0ull);
 #pragma nounroll
       for (int e = 0; e < a.n_events; ++e) {  // a rolled loop: nothing of the event records is kept across the substeps
@@ -670,7 +676,7 @@ void step_kernel(StepArgs a) {
       // ---- force pushes (ksim/events.py:240-365): a wrench held on one body enters the Newton-Euler pass as an
       // external force on that body, so the subtree sums and the projection on the motion axes below turn it into
       // the generalised force J^T f.  Lane 0 owns the state in memory; the other lanes get it by broadcast.
-      if (!FWD && a.n_force_events > 0) {
+      if (!fwd && a.n_force_events > 0) {
         const uint64_t ev_step = a.event_rng.step + (a.event_rng.step_base ? *a.event_rng.step_base : 0ull);
         Sp ext = {{0.f, 0.f, 0.f}, {0.f, 0.f, 0.f}};
 #pragma nounroll
@@ -1155,7 +1161,7 @@ void step_kernel(StepArgs a) {
 
     KS_PHASE(14)
     // ---- semi-implicit Euler
-    if (!FWD) {
+    if (!fwd) {
       // What this stage needs of the lane's constants is read again here (through an opaque lane id, so that the loads
       // are not merged with those at the top of the substep): nothing of it stays live across the solver.
       int lane_e = threadIdx.x;
@@ -1451,7 +1457,7 @@ static int launch_step(const KsModel* km, ks_stream_t stream, const KsStepIO* io
   a.model = km->dev;
   a.N = io->N;
   a.qpos = io->qpos; a.qvel = io->qvel; a.qacc_warmstart = io->qacc_warmstart; a.time = io->time;
-  a.friction = io->friction; a.mass_scale = io->mass_scale; a.env_mask = io->env_mask;
+  a.friction = io->friction; a.mass_scale = io->mass_scale; a.env_mask = io->env_mask; a.fresh = io->fresh;
   a.qacc = io->qacc; a.ctrl_out = io->ctrl_out; a.xpos = io->xpos; a.xquat = io->xquat; a.cvel = io->cvel;
   a.traj_ctrl = io->traj_ctrl; a.traj_xpos = io->traj_xpos; a.traj_xquat = io->traj_xquat;
   a.solver_niter = io->solver_niter; a.nefc = io->nefc;

@@ -20,6 +20,7 @@ struct StepArgs {
   const float *action_bias, *torque_bias, *action_noise, *torque_noise;
   const float *friction, *mass_scale;
   const uint8_t* env_mask;
+  const uint8_t* fresh;
   float *qacc, *ctrl_out, *xpos, *xquat, *cvel, *traj_ctrl, *traj_xpos, *traj_xquat;
   int32_t *solver_niter, *nefc;
   float *dbg_M, *dbg_bias, *dbg_qacc_smooth, *contact_dist, *cinert, *cfrc_ext;

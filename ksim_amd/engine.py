@@ -290,13 +290,17 @@ class HipEngine(PhysicsEngine):
              noise: Mapping[str, torch.Tensor] | None = None,
              record: Mapping[str, torch.Tensor] | None = None, want_cvel: bool = True, want_cinert: bool = False,
              want_cfrc_ext: bool = False,
-             step: int = 0, step_base=None, event_seed: int = 0, live=None, stats: Mapping[str, torch.Tensor] | None = None) -> PhysicsState:
+             step: int = 0, step_base=None, event_seed: int = 0, live=None, stats: Mapping[str, torch.Tensor] | None = None,
+             fresh: torch.Tensor | None = None) -> PhysicsState:
         """`live`: names among qacc, ctrl, xpos, xquat, contact_dist of the derived fields of `physics_state.data` that
         the caller reads afterwards (None = all).  The rollout records ctrl / xpos / xquat into its own slot through
         `record`, so a task whose observations read none of them need not have them written twice.
         `stats`: optional int32 (N,) buffers `nefc` and `solver_niter` that receive the constraint rows and Newton iterations
         of the last substep (diagnostics; the reference exposes the same numbers as `data.nefc` / `data.solver_niter`), and
-        `dbg_M` (N, nv * nv) float32, which the profiling build of the library fills with cycle counts per phase."""
+        `dbg_M` (N, nv * nv) float32, which the profiling build of the library fills with cycle counts per phase.
+        `fresh`: (N,) uint8 mask of envs that were reset since their last step and have not had the forward pass of the
+        reset (engine.py:213) yet: the step kernel runs it for them first, in the same launch, instead of a separate masked
+        `forward` (the rollout's deferred mode; their derived fields at the reset state itself are then never written)."""
         m, d, s = physics_model.model, physics_state.data, physics_state
         rnd, noise, record = randomization or {}, noise or {}, record or {}
         keep = (lambda name, b: b) if live is None else (lambda name, b: b if name in live else None)
@@ -316,7 +320,7 @@ class HipEngine(PhysicsEngine):
                    cinert=d.cinert if want_cinert else None, cfrc_ext=d.cfrc_ext if want_cfrc_ext else None,
                    action_noise=noise.get("action_noise"),
                    torque_noise=noise.get("torque_noise"), traj_ctrl=record.get("ctrl"),
-                   traj_xpos=record.get("xpos"), traj_xquat=record.get("xquat"))
+                   traj_xpos=record.get("xpos"), traj_xquat=record.get("xquat"), fresh=fresh)
         if stats:
             buf.update({k: stats[k] for k in ("nefc", "solver_niter", "dbg_M") if k in stats})
         # heaviest-first launch order from the previous step's cost estimates (kept on the state object)

@@ -68,7 +68,7 @@ def _expected_shapes(m: KinematicModel, N: int, S: int, actuator_type: int = _li
         "action": (N, na), "ctrl_in": (N, nu), "latency": (N,), "zero_offset": (N, nu), "drop": (N, na),
         "kp": (nu,), "kd": (nu,), "ctrl_clip": (nu,), "kp_scale": (N,), "kd_scale": (N,),
         "torque_limit_scale": (N,), "action_bias": (N, nu), "torque_bias": (N, nu), "action_noise": (S, N, na),
-        "torque_noise": (S, N, nu), "friction": (N,), "mass_scale": (N, nb), "env_mask": (N,), "qacc": (N, nv), "ctrl_out": (N, nu),
+        "torque_noise": (S, N, nu), "friction": (N,), "mass_scale": (N, nb), "env_mask": (N,), "fresh": (N,), "qacc": (N, nv), "ctrl_out": (N, nu),
         "xpos": (N, nb * 3), "xquat": (N, nb * 4), "cvel": (N, nb * 6), "traj_ctrl": (N, nu),
         "traj_xpos": (N, nb * 3), "traj_xquat": (N, nb * 4), "solver_niter": (N,), "nefc": (N,),
         "dbg_M": (N, nv * nv), "dbg_bias": (N, nv), "dbg_qacc_smooth": (N, nv), "contact_dist": (N, ns),
@@ -94,8 +94,8 @@ def _make_io(dm: DeviceModel, buffers: Mapping[str, torch.Tensor | None], subste
             raise _lib.KsError(f"unknown step buffer {name!r}")
         if t is None:
             continue
-        want = torch.uint8 if name in ("drop", "env_mask") else (torch.int32 if name in _I32 else torch.float32)
-        if name in ("drop", "env_mask") and t.dtype == torch.bool:
+        want = torch.uint8 if name in ("drop", "env_mask", "fresh") else (torch.int32 if name in _I32 else torch.float32)
+        if name in ("drop", "env_mask", "fresh") and t.dtype == torch.bool:
             t = t.view(torch.uint8)
         _lib.require_cuda(t, dtype=want)
         if tuple(t.shape) != shapes[name] and not (t.numel() == 0 and 0 in shapes[name]):

@@ -68,6 +68,11 @@ class RolloutConstants:  # the static pieces, ksim/task/rl.py:138-150
     reward_clip_min: float | None = None
     reward_clip_max: float | None = None
     commands: CommandSet | None = None  # commands advanced once per control step (rl.py:1082-1098); None: constant
+    # The forward pass that a reset owes (engine.py:213) runs inside the next control step's physics launch instead of as a
+    # masked launch of its own right after the termination pass: one launch less per control step, the same trajectories
+    # bit for bit.  Between two steps the warm start of a freshly reset env is then not yet that of its new episode, and
+    # the mode is only taken when no term of the task reads a derived field (xpos, xquat, cvel ...) of the live state.
+    defer_reset_forward: bool = False
     head: GaussianHead | MixtureHead | None = None  # None: one mean per action entry and the log_std vector
 
 
@@ -131,6 +136,7 @@ class Rollout:
                 T.SRC_CONTACT_DIST: "contact_dist", T.SRC_CINERT: "cinert", T.SRC_CFRC_EXT: "cfrc_ext"}
         self._live = {name for src, name in need.items() if src in used}
         self._live.add("contact_dist")  # a few floats per env, also read by the illegal-contact termination
+        self._defer = bool(c.defer_reset_forward) and self._live <= {"contact_dist"}
         if c.actor.in_dim != c.terms.obs_dim or c.actor.out_dim != self.mean.shape[1]:
             raise _lib.KsError("actor must map the observation vector to one mean per action entry (or to what its head takes)")
         if c.critic is not None and (c.critic.in_dim != c.terms.obs_dim or c.critic.out_dim != 1):
@@ -208,7 +214,7 @@ class Rollout:
                       noise=noise.get("engine"), record=dict(ctrl=self.ctrl[t], xpos=self.xpos[t], xquat=self.xquat[t]),
                       want_cvel=T.SRC_CVEL in c.terms.sources_used, want_cinert=T.SRC_CINERT in c.terms.sources_used,
                       want_cfrc_ext=T.SRC_CFRC_EXT in c.terms.sources_used, step=step, step_base=step_base, event_seed=env.seed,
-                      live=self._live)
+                      live=self._live, fresh=self.reset_mask if self._defer else None)
         ev_buf = ps.event_states.get("_buffer") if ps.event_states else None
         st = dict(qpos=d.qpos, qvel=d.qvel, qacc_warmstart=d.qacc_warmstart, time=d.time, last_ctrl=ps.last_ctrl)
         c.terms.terminate_reset(st, level=level, components=self.components[t][: c.terms.n_terms] if c.terms.n_terms else None,
@@ -220,8 +226,10 @@ class Rollout:
                                 event_reset_uniform=noise.get("event_reset_uniform"),
                                 event_force=ps.event_states.get("_force_buffer") if ps.event_states else None,
                                 contact_dist=d.contact_dist if "contact_dist" in self._live else None, episode=c.engine.episode_args(ps, noise.get("episode")))
-        # refresh the derived fields and the warm start of the reset envs (engine.py:213)
-        c.engine.forward(c.physics_model, ps, self.reset_mask, env.randomization_dict, live=self._live)
+        # refresh the derived fields and the warm start of the reset envs (engine.py:213); in the deferred mode the next
+        # step's physics launch does it for the envs still flagged in the reset mask
+        if not self._defer:
+            c.engine.forward(c.physics_model, ps, self.reset_mask, env.randomization_dict, live=self._live)
         if c.commands is not None:  # record the commands this step ran under, then advance them (rl.py:1082-1098)
             c.commands.update(env.commands, d.qpos, d.qvel, level=level, fresh=self.reset_mask, record=self.command[t],
                               uniform=noise.get("command_uniform"), seed=env.seed, step=step, step_base=step_base)

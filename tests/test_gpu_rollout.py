@@ -833,3 +833,35 @@ def test_site_frame_sensors_follow_the_live_state_in_a_rollout():
     assert checked > N
     # the poses do change over the rollout, so a stale field could not have passed
     assert np.abs(xq[Tn - 1][:, fb] - xq[0][:, fb]).max() > 1e-3
+
+
+def test_reset_forward_inside_the_next_step_gives_the_same_trajectories():
+    """The forward pass a reset owes (engine.py:213), run inside the next control step's physics launch for the envs still
+    flagged in the reset mask (`RolloutConstants.defer_reset_forward`), against the masked forward launch right after the
+    termination pass: every recorded array of a rollout with many resets bit for bit, and the states the rollouts end in
+    once the pending forward pass has been run."""
+    import dataclasses
+
+    N, T = 64, 12
+    runs = []
+    for defer in (False, True):
+        m, c, rnd_, _, _, EnvState = build(N, T, seed=9, min_height=0.86)
+        c = dataclasses.replace(c, defer_reset_forward=defer)
+        from ksim_amd.rollout import Rollout
+        ro = Rollout(c, N, T)
+        assert ro._defer == defer
+        ps = c.engine.reset(c.physics_model, 1.0, 5, N, rnd_)
+        env = EnvState(ps, rnd_, torch.zeros(N, 2, device=DEV), None, seed=31)
+        snaps = []
+        for _ in range(3):
+            traj, rew = ro.unroll(env)
+            snaps.append([x.clone() for x in (traj.qpos, traj.qvel, traj.action, traj.done, traj.obs["obs"], traj.xpos, traj.ctrl,
+                                              ro.values, rew.total)])
+        if defer:  # what the last step's resets still owe
+            c.engine.forward(c.physics_model, ps, ro.reset_mask, rnd_, live=ro._live)
+        snaps.append([ps.data.qpos.clone(), ps.data.qvel.clone(), ps.data.qacc_warmstart.clone()])
+        runs.append(snaps)
+        assert sum(int(s[3].sum().item()) for s in snaps[:3]) > N // 4, "too few resets to tell the two modes apart"
+    for a, b in zip(*runs):
+        for x, y in zip(a, b):
+            assert torch.equal(x, y)
