@@ -540,6 +540,13 @@ typedef struct KsTerminateIO {
   const float* episode_normal;      /* N(0,1) */
 } KsTerminateIO;
 int ks_terminate_reset(const KsTerms* terms, ks_stream_t stream, const KsTerminateIO* io /*host*/);
+/* ks_terminate_reset of control step t and ks_observe of step t + 1 in one launch (the tail of step_engine followed by the
+ * head of the next one, ksim/task/rl.py:1049-1080 then 1164-1176 / 153-186): a workgroup takes the decisions for its envs,
+ * resets the finished ones and observes the same envs in the state the next step starts from.  oio->fresh, when given, must
+ * be tio->reset_mask (the observation's episode starts are what this call's first half decides); the observation's random
+ * numbers are keyed by oio->rng, which the caller sets to the next step's.  Same results as the two calls in a row. */
+int ks_terminate_reset_observe(const KsTerms* terms, ks_stream_t stream, const KsTerminateIO* tio /*host*/,
+                               const KsObserveIO* oio /*host*/);
 
 /* Commands (replaces get_commands / get_initial_commands, ksim/task/rl.py:302-332, called per control step at
  * rl.py:1082-1098, for the velocity commands of the shipped tasks, ksim/commands.py:281-391,451-507).  The env's command

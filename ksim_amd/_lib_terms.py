@@ -210,6 +210,8 @@ def bind(lib) -> None:
     lib.ks_terms_destroy.argtypes = [c_void_p]
     lib.ks_observe.argtypes = [c_void_p, c_void_p, POINTER(KsObserveIO)]
     lib.ks_terminate_reset.argtypes = [c_void_p, c_void_p, POINTER(KsTerminateIO)]
+    lib.ks_terminate_reset_observe.argtypes = [c_void_p, c_void_p, POINTER(KsTerminateIO), POINTER(KsObserveIO)]
+    lib.ks_terminate_reset_observe.restype = c_int32
     lib.ks_sample_action.argtypes = [c_void_p, c_int64, c_int32, c_void_p, c_void_p, c_void_p, KsRng, c_float,
                                      c_void_p]
     lib.ks_commands.argtypes = [c_void_p, POINTER(KsCommandIO)]

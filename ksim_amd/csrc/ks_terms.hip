@@ -64,9 +64,8 @@ __device__ inline float apply_stage(const KsNoiseStage& st, float v, float z, fl
   return add ? v + rv : v * rv;
 }
 
-__global__ __launch_bounds__(256) void observe_kernel(ObserveArgs a) {
-  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (idx >= a.N * a.obs_dim) return;
+// One observation element: idx = env * obs_dim + element.
+__device__ __forceinline__ void observe_one(const ObserveArgs& a, int64_t idx) {
   const int64_t e = idx / a.obs_dim;
   const int k = (int)(idx - e * a.obs_dim);
   // read in place (the table sits in the caches): a private copy of the element, whose noise chain is indexed at run
@@ -224,6 +223,12 @@ __global__ __launch_bounds__(256) void observe_kernel(ObserveArgs a) {
   }
 }
 
+__global__ __launch_bounds__(256) void observe_kernel(ObserveArgs a) {
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= a.N * a.obs_dim) return;
+  observe_one(a, idx);
+}
+
 struct TerminateArgs {
   const DevTerms* t;
   int64_t N;
@@ -267,17 +272,19 @@ __device__ inline float rv_value(const KsRandomVar& rv, float u, float z, float 
 // Termination comparisons are strict and done in fp32 on the stored state, so the integer outputs are
 // reproducible bit for bit.
 constexpr int kTermEnvs = 32;
+// In the launch that also observes, a workgroup takes fewer envs: the observation is one thread per element, and with 32
+// envs per workgroup a launch over a few thousand envs would be too few workgroups to fill the chip.
+constexpr int kTermObsEnvs = 8;
 
-__global__ __launch_bounds__(256) void terminate_kernel(TerminateArgs a) {
-  __shared__ int s_bad[kTermEnvs];    // non-finite state seen
-  __shared__ int s_reset[kTermEnvs];  // env starts a fresh episode
-  __shared__ int s_frame[kTermEnvs];  // its frame of the reference motion
+// s_bad: non-finite state seen; s_reset: env starts a fresh episode; s_frame: its frame of the reference motion
+template <int ENVS>
+__device__ __forceinline__ void terminate_block(const TerminateArgs& a, int* s_bad, int* s_reset, int* s_frame) {
   const KsTermsDesc& d = a.t->d;
   const int tid = threadIdx.x;
-  const int64_t e0 = (int64_t)blockIdx.x * kTermEnvs;
-  const int ne = a.N - e0 < kTermEnvs ? (int)(a.N - e0) : kTermEnvs;
+  const int64_t e0 = (int64_t)blockIdx.x * ENVS;
+  const int ne = a.N - e0 < ENVS ? (int)(a.N - e0) : ENVS;
   const int nq = a.nq, nv = a.nv, nu = a.nu;
-  if (tid < kTermEnvs) s_bad[tid] = 0;
+  if (tid < ENVS) s_bad[tid] = 0;
   __syncthreads();
   // ---- flat pass 1: transition record (post-step state) and finiteness
   float* qb = a.qpos + e0 * nq;
@@ -462,6 +469,26 @@ __global__ __launch_bounds__(256) void terminate_kernel(TerminateArgs a) {
       if (d.reset_pitch_roll == 1) pitch_roll();
     }
   }
+}
+
+__global__ __launch_bounds__(256) void terminate_kernel(TerminateArgs a) {
+  __shared__ int s_bad[kTermEnvs], s_reset[kTermEnvs], s_frame[kTermEnvs];
+  terminate_block<kTermEnvs>(a, s_bad, s_reset, s_frame);
+}
+
+// The termination pass of control step t and the observation of step t + 1 in one launch: a workgroup takes the decisions
+// for its envs, resets the finished ones, and then observes those same envs in the state the next step will start from
+// (one thread per element, striding over the workgroup's envs).  What the first half wrote (state rows, the reset mask that
+// the observation takes as its `fresh` flags) is read back by other threads of the same workgroup only.
+__global__ __launch_bounds__(256) void terminate_observe_kernel(TerminateArgs a, ObserveArgs o) {
+  __shared__ int s_bad[kTermObsEnvs], s_reset[kTermObsEnvs], s_frame[kTermObsEnvs];
+  terminate_block<kTermObsEnvs>(a, s_bad, s_reset, s_frame);
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  __syncthreads();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+  const int64_t e0 = (int64_t)blockIdx.x * kTermObsEnvs;
+  const int ne = a.N - e0 < kTermObsEnvs ? (int)(a.N - e0) : kTermObsEnvs;
+  for (int i = threadIdx.x; i < ne * o.obs_dim; i += 256) observe_one(o, e0 * o.obs_dim + i);
 }
 
 __global__ __launch_bounds__(256) void sample_action_kernel(int64_t n, int nu, const float* __restrict__ mean,
@@ -1254,14 +1281,15 @@ extern "C" int ks_terms_destroy(KsTerms* t) {
   return KS_OK;
 }
 
-extern "C" int ks_observe(const KsTerms* t, ks_stream_t stream, const KsObserveIO* io) {
+// Checks a ks_observe call on the host and fills the kernel arguments; `empty` when there is nothing to launch.
+static int fill_observe(const KsTerms* t, const KsObserveIO* io, ObserveArgs& a, bool& empty) {
+  empty = false;
   if (!t || !io) return fail(KS_EINVAL, "ks_observe: null argument");
   const KsTermsDesc& d = t->host;
   if (io->N < 0) return fail(KS_EINVAL, "ks_observe: negative env count");
-  if (io->N == 0 || d.obs_dim == 0) return KS_OK;
+  if (io->N == 0 || d.obs_dim == 0) { empty = true; return KS_OK; }
   const int src_dim[KS_SRC_COUNT] = {d.nq, d.nv, d.nv, d.nu, d.action_dim > 0 ? d.action_dim : d.nu, d.command_dim, 1, d.nb * 3, d.nb * 4, d.nb * 6, 0, d.ns, d.nb * 10, d.nb * 6};
   if (d.carry_dim > 0 && !io->carry) return fail(KS_EINVAL, "ks_observe: the stateful observations need a carry buffer");
-  ObserveArgs a;
   std::memset(&a, 0, sizeof(a));
   bool needs_quat = false, needs_noise = false;
   for (int k = 0; k < d.obs_dim; ++k) {
@@ -1307,20 +1335,29 @@ extern "C" int ks_observe(const KsTerms* t, ks_stream_t stream, const KsObserveI
   a.rng = io->rng; a.obs = io->obs; a.noisy = io->noisy_obs; a.obs_dim = d.obs_dim; a.nq = d.nq; a.nu = d.nu;
   a.carry = io->carry; a.fresh = io->fresh; a.carry_uniform = io->carry_uniform; a.carry_dim = d.carry_dim;
   a.site_pose = io->site_pose;
-  const int64_t n = io->N * d.obs_dim;
+  return KS_OK;
+}
+
+extern "C" int ks_observe(const KsTerms* t, ks_stream_t stream, const KsObserveIO* io) {
+  ObserveArgs a;
+  bool empty;
+  const int rc = fill_observe(t, io, a, empty);
+  if (rc != KS_OK || empty) return rc;
+  const int64_t n = a.N * a.obs_dim;
   const int64_t grid = (n + 255) / 256;
   if (grid > 0x7fffffff) return fail(KS_ELIMIT, "ks_observe: too many elements");
   hipLaunchKernelGGL(observe_kernel, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, a);
   return check_launch("ks_observe");
 }
 
-extern "C" int ks_terminate_reset(const KsTerms* t, ks_stream_t stream, const KsTerminateIO* io) {
+
+static int fill_terminate(const KsTerms* t, const KsTerminateIO* io, TerminateArgs& a, bool& empty) {
+  empty = false;
   if (!t || !io) return fail(KS_EINVAL, "ks_terminate_reset: null argument");
   const KsTermsDesc& d = t->host;
   if (io->N < 0) return fail(KS_EINVAL, "ks_terminate_reset: negative env count");
-  if (io->N == 0) return KS_OK;
+  if (io->N == 0) { empty = true; return KS_OK; }
   if (!io->qpos || !io->qvel) return fail(KS_EINVAL, "ks_terminate_reset: qpos and qvel are required");
-  TerminateArgs a;
   std::memset(&a, 0, sizeof(a));
   a.t = t->dev; a.N = io->N; a.level = io->level;
   a.qpos = io->qpos; a.qvel = io->qvel; a.warm = io->qacc_warmstart; a.time = io->time; a.last_ctrl = io->last_ctrl;
@@ -1360,11 +1397,39 @@ extern "C" int ks_terminate_reset(const KsTerms* t, ks_stream_t stream, const Ks
               a.act_torque_limit_scale) ? 1 : 0;
   if (a.action_latency && !(io->latency_lo >= 0.f && io->latency_hi >= io->latency_lo))
     return fail(KS_EINVAL, "ks_terminate_reset: latency range must satisfy 0 <= lo <= hi");
-  const int64_t grid = (io->N + kTermEnvs - 1) / kTermEnvs;
+  return KS_OK;
+}
+
+extern "C" int ks_terminate_reset(const KsTerms* t, ks_stream_t stream, const KsTerminateIO* io) {
+  TerminateArgs a;
+  bool empty;
+  const int rc = fill_terminate(t, io, a, empty);
+  if (rc != KS_OK || empty) return rc;
+  const int64_t grid = (a.N + kTermEnvs - 1) / kTermEnvs;
   if (grid > 0x7fffffff) return fail(KS_ELIMIT, "ks_terminate_reset: too many envs");
   hipLaunchKernelGGL(terminate_kernel, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, a);
   return check_launch("ks_terminate_reset");
 }
+
+extern "C" int ks_terminate_reset_observe(const KsTerms* t, ks_stream_t stream, const KsTerminateIO* tio, const KsObserveIO* oio) {
+  TerminateArgs a;
+  ObserveArgs o;
+  bool empty_t, empty_o;
+  int rc = fill_terminate(t, tio, a, empty_t);
+  if (rc != KS_OK) return rc;
+  rc = fill_observe(t, oio, o, empty_o);
+  if (rc != KS_OK) return rc;
+  if (tio->N != oio->N) return fail(KS_EINVAL, "ks_terminate_reset_observe: the two halves disagree about the env count (%lld, %lld)", (long long)tio->N, (long long)oio->N);
+  if (empty_t) return KS_OK;
+  // the observation half takes the episode starts from the mask the termination half writes in the same launch
+  if (oio->fresh && oio->fresh != tio->reset_mask) return fail(KS_EINVAL, "ks_terminate_reset_observe: the observation's fresh flags must be the reset mask of this call");
+  if (empty_o) { o.obs_dim = 0; }
+  const int64_t grid = (a.N + kTermObsEnvs - 1) / kTermObsEnvs;
+  if (grid > 0x7fffffff) return fail(KS_ELIMIT, "ks_terminate_reset_observe: too many envs");
+  hipLaunchKernelGGL(terminate_observe_kernel, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, a, o);
+  return check_launch("ks_terminate_reset_observe");
+}
+
 
 extern "C" int ks_sample_action(ks_stream_t stream, int64_t N, int32_t nu, const float* mean, const float* log_std,
                                 const float* noise_normal, KsRng rng, float clip_max, float* action) {

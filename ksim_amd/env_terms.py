@@ -133,7 +133,7 @@ class EnvTerms:
     def observe(self, sources: Mapping[int, torch.Tensor | None], N: int, *, level: float = 1.0,
                 zero_offset=None, bias_draw=None, bias_redraw=None, noise_normal=None, noise_uniform=None, seed: int = 0,
                 step: int = 0, step_base=None, carry=None, fresh=None, carry_uniform=None, site_pose=None,
-                obs: torch.Tensor | None = None, noisy_obs: torch.Tensor | None = None):
+                obs: torch.Tensor | None = None, noisy_obs: torch.Tensor | None = None, _io_only: bool = False):
         """`carry` (N, carry_dim) is advanced in place; `fresh` (N) uint8 marks the envs whose carries are initialised
         from the current state first (those that were just reset) and whose bias draws `bias_draw` (N, obs_dim, 2) are
         renewed (from `bias_redraw` when given, else from the Philox stream).  `site_pose` (N, 7): per-env orientation
@@ -169,6 +169,8 @@ class EnvTerms:
                 raise _lib.KsError(f"fresh: expected ({N},), got {tuple(fresh.shape)}")
             io.fresh = fresh.data_ptr()
         io.rng = _rng(seed, step, step_base)
+        if _io_only:
+            return io
         _lib.check(self._lib.ks_observe(self._handle, _lib.current_stream(), ctypes.byref(io)))
         return obs, noisy_obs
 
@@ -177,7 +179,7 @@ class EnvTerms:
                         success=None, traj_qpos=None, traj_qvel=None, traj_time=None, reset_mask=None,
                         episode_length=None, reset_uniform=None, seed: int = 0, step: int = 0, step_base=None,
                         event_state=None, event_intervals=(), event_reset_uniform=None, event_force=None,
-                        contact_dist=None, apply_reset: bool = True, episode: Mapping | None = None) -> None:
+                        contact_dist=None, apply_reset: bool = True, episode: Mapping | None = None, _io_only: bool = False):
         """`episode`: the per-episode quantities that the envs starting a fresh episode re-draw (engine.py:222-245), as
         `HipEngine.episode_args` builds them: buffers `action_latency`, `zero_offset`, `act_*`, the matching random
         variables, and optionally explicit draws `episode_uniform` / `episode_normal` (N, 3 nu + 4),
@@ -263,7 +265,18 @@ class EnvTerms:
                 rv = episode.get(name)
                 if rv is not None:
                     setattr(io, name, rv.desc())
+        if _io_only:
+            return io
         _lib.check(self._lib.ks_terminate_reset(self._handle, _lib.current_stream(), ctypes.byref(io)))
+
+    def terminate_reset_observe(self, state: Mapping[str, torch.Tensor], terminate: Mapping, sources: Mapping[int, torch.Tensor | None],
+                                observe: Mapping) -> None:
+        """`terminate_reset(state, **terminate)` of one control step and `observe(sources, N, **observe)` of the next one in
+        a single launch (`ks_terminate_reset_observe`): the observation sees the state the termination pass leaves, and
+        its `fresh` flags must be that pass's `reset_mask`.  Same results as the two calls in a row."""
+        tio = self.terminate_reset(state, _io_only=True, **terminate)
+        oio = self.observe(sources, state["qpos"].shape[0], _io_only=True, **observe)
+        _lib.check(self._lib.ks_terminate_reset_observe(self._handle, _lib.current_stream(), ctypes.byref(tio), ctypes.byref(oio)))
 
     def close(self) -> None:
         if self._handle:

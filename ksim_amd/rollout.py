@@ -73,6 +73,10 @@ class RolloutConstants:  # the static pieces, ksim/task/rl.py:138-150
     # bit for bit.  Between two steps the warm start of a freshly reset env is then not yet that of its new episode, and
     # the mode is only taken when no term of the task reads a derived field (xpos, xquat, cvel ...) of the live state.
     defer_reset_forward: bool = False
+    # The observation of control step t + 1 is computed by the launch that ends step t (terminations, transition record,
+    # resets): `ks_terminate_reset_observe`, one launch instead of two, the same numbers.  Taken when the task has no
+    # command set to advance in between and its observations read no derived field of the live state.
+    fuse_next_observation: bool = False
     head: GaussianHead | MixtureHead | None = None  # None: one mean per action entry and the log_std vector
 
 
@@ -136,7 +140,10 @@ class Rollout:
                 T.SRC_CONTACT_DIST: "contact_dist", T.SRC_CINERT: "cinert", T.SRC_CFRC_EXT: "cfrc_ext"}
         self._live = {name for src, name in need.items() if src in used}
         self._live.add("contact_dist")  # a few floats per env, also read by the illegal-contact termination
-        self._defer = bool(c.defer_reset_forward) and self._live <= {"contact_dist"}
+        reads_derived = any(src in used for src in need)
+        self._defer = bool(c.defer_reset_forward) and not reads_derived
+        self._fuse_obs = bool(c.fuse_next_observation) and not reads_derived and c.commands is None
+        self._obs_done = None  # (env state, slot, step) whose observation the previous step's last launch has written
         if c.actor.in_dim != c.terms.obs_dim or c.actor.out_dim != self.mean.shape[1]:
             raise _lib.KsError("actor must map the observation vector to one mean per action entry (or to what its head takes)")
         if c.critic is not None and (c.critic.in_dim != c.terms.obs_dim or c.critic.out_dim != 1):
@@ -154,13 +161,19 @@ class Rollout:
                T.SRC_XQUAT: d.xquat, T.SRC_CVEL: d.cvel, T.SRC_CONTACT_DIST: d.contact_dist, T.SRC_CINERT: d.cinert,
                T.SRC_CFRC_EXT: d.cfrc_ext}
         self._prepare_env(env)
-        # the reset mask still holds the envs that the previous control step reset: their carries start afresh
-        c.terms.observe(src, self.N, level=level, zero_offset=ps.zero_offset, bias_draw=env.obs_bias,
-                        bias_redraw=noise.get("obs_bias_redraw"),
-                        noise_normal=noise.get("obs_normal"), noise_uniform=noise.get("obs_uniform"), seed=env.seed,
-                        step=step, step_base=step_base, obs=self.obs[t], noisy_obs=self.noisy_obs[t],
-                        carry=env.obs_carry, fresh=self.reset_mask if (c.terms.carry_dim or c.terms.has_bias) else None,
-                        carry_uniform=noise.get("obs_carry_uniform"), site_pose=(env.randomization_dict or {}).get("site_pose"))
+
+        def observe_args(slot: int, at_step: int) -> dict:
+            # the reset mask holds the envs that the previous control step reset: their carries and biases start afresh
+            return dict(level=level, zero_offset=ps.zero_offset, bias_draw=env.obs_bias, seed=env.seed, step=at_step,
+                        step_base=step_base, obs=self.obs[slot], noisy_obs=self.noisy_obs[slot], carry=env.obs_carry,
+                        fresh=self.reset_mask if (c.terms.carry_dim or c.terms.has_bias) else None,
+                        site_pose=(env.randomization_dict or {}).get("site_pose"))
+
+        if self._obs_done != (id(env), t, step, _relative_step):  # else the launch that ended the previous step wrote it
+            c.terms.observe(src, self.N, bias_redraw=noise.get("obs_bias_redraw"), noise_normal=noise.get("obs_normal"),
+                            noise_uniform=noise.get("obs_uniform"), carry_uniform=noise.get("obs_carry_uniform"),
+                            **observe_args(t, step))
+        self._obs_done = None
         # actor reads the noisy copy (walking.py:592-595), critic the clean one (walking.py:626-638); recurrent networks
         # advance their carries, which restart from zero for the envs the previous control step reset
         if self.fresh is not None:
@@ -217,15 +230,21 @@ class Rollout:
                       live=self._live, fresh=self.reset_mask if self._defer else None)
         ev_buf = ps.event_states.get("_buffer") if ps.event_states else None
         st = dict(qpos=d.qpos, qvel=d.qvel, qacc_warmstart=d.qacc_warmstart, time=d.time, last_ctrl=ps.last_ctrl)
-        c.terms.terminate_reset(st, level=level, components=self.components[t][: c.terms.n_terms] if c.terms.n_terms else None,
-                                done=self.done[t], success=self.success[t], traj_qpos=self.qpos[t],
-                                traj_qvel=self.qvel[t], traj_time=self.timestep[t], reset_mask=self.reset_mask,
-                                episode_length=env.episode_length, reset_uniform=noise.get("reset_uniform"),
-                                seed=env.seed, step=step, step_base=step_base, event_state=ev_buf,
-                                event_intervals=[ev.interval_range for ev in c.engine.events.values()],
-                                event_reset_uniform=noise.get("event_reset_uniform"),
-                                event_force=ps.event_states.get("_force_buffer") if ps.event_states else None,
-                                contact_dist=d.contact_dist if "contact_dist" in self._live else None, episode=c.engine.episode_args(ps, noise.get("episode")))
+        term_args = dict(level=level, components=self.components[t][: c.terms.n_terms] if c.terms.n_terms else None,
+                         done=self.done[t], success=self.success[t], traj_qpos=self.qpos[t],
+                         traj_qvel=self.qvel[t], traj_time=self.timestep[t], reset_mask=self.reset_mask,
+                         episode_length=env.episode_length, reset_uniform=noise.get("reset_uniform"),
+                         seed=env.seed, step=step, step_base=step_base, event_state=ev_buf,
+                         event_intervals=[ev.interval_range for ev in c.engine.events.values()],
+                         event_reset_uniform=noise.get("event_reset_uniform"),
+                         event_force=ps.event_states.get("_force_buffer") if ps.event_states else None,
+                         contact_dist=d.contact_dist if "contact_dist" in self._live else None, episode=c.engine.episode_args(ps, noise.get("episode")))
+        if self._fuse_obs and t + 1 < self.T and not noise:
+            # the next step's observation rides in this launch (its random numbers are those of step + 1)
+            c.terms.terminate_reset_observe(st, term_args, src, observe_args(t + 1, step + 1))
+            self._obs_done = (id(env), t + 1, step + 1, _relative_step)
+        else:
+            c.terms.terminate_reset(st, **term_args)
         # refresh the derived fields and the warm start of the reset envs (engine.py:213); in the deferred mode the next
         # step's physics launch does it for the envs still flagged in the reset mask
         if not self._defer:

@@ -844,24 +844,26 @@ def test_reset_forward_inside_the_next_step_gives_the_same_trajectories():
 
     N, T = 64, 12
     runs = []
-    for defer in (False, True):
+    for defer, fuse in ((False, False), (True, False), (True, True)):
         m, c, rnd_, _, _, EnvState = build(N, T, seed=9, min_height=0.86)
-        c = dataclasses.replace(c, defer_reset_forward=defer)
+        # `fuse`: the next step's observation also rides in the launch that ends a step (ks_terminate_reset_observe)
+        c = dataclasses.replace(c, defer_reset_forward=defer, fuse_next_observation=fuse)
         from ksim_amd.rollout import Rollout
         ro = Rollout(c, N, T)
-        assert ro._defer == defer
+        assert ro._defer == defer and ro._fuse_obs == fuse
         ps = c.engine.reset(c.physics_model, 1.0, 5, N, rnd_)
         env = EnvState(ps, rnd_, torch.zeros(N, 2, device=DEV), None, seed=31)
         snaps = []
         for _ in range(3):
             traj, rew = ro.unroll(env)
-            snaps.append([x.clone() for x in (traj.qpos, traj.qvel, traj.action, traj.done, traj.obs["obs"], traj.xpos, traj.ctrl,
-                                              ro.values, rew.total)])
+            snaps.append([x.clone() for x in (traj.qpos, traj.qvel, traj.action, traj.done, traj.obs["obs"], traj.obs["noisy_obs"],
+                                              traj.xpos, traj.ctrl, ro.values, rew.total)])
         if defer:  # what the last step's resets still owe
             c.engine.forward(c.physics_model, ps, ro.reset_mask, rnd_, live=ro._live)
         snaps.append([ps.data.qpos.clone(), ps.data.qvel.clone(), ps.data.qacc_warmstart.clone()])
         runs.append(snaps)
-        assert sum(int(s[3].sum().item()) for s in snaps[:3]) > N // 4, "too few resets to tell the two modes apart"
-    for a, b in zip(*runs):
-        for x, y in zip(a, b):
-            assert torch.equal(x, y)
+        assert sum(int(s[3].sum().item()) for s in snaps[:3]) > N // 4, "too few resets to tell the modes apart"
+    for other in runs[1:]:
+        for a, b in zip(runs[0], other):
+            for x, y in zip(a, b):
+                assert torch.equal(x, y)
