@@ -146,7 +146,8 @@ def main() -> None:
         torch.cuda.synchronize()
         del src, dst
     if args.only == "phases":
-        print(json.dumps({"step_kernel_phases": step_kernel_phases(torch, args.integrator, args.envs)}))
+        print(json.dumps({"step_kernel_phases": step_kernel_phases(torch, args.integrator, args.envs),
+                          "mlp_phases": mlp_phases(torch)}))
         return
     if args.only == "mfma":
         print(json.dumps({"mfma_yardstick": mfma_yardstick(torch)}))
@@ -603,6 +604,35 @@ def step_kernel_phases(torch, integrator: str, N: int, steps: int = 30) -> dict:
             "constraint_rows_mean": float(buf["nefc"].float().mean().item()),
             "phases": {n: {"cycles": float(p[:, i].mean()), "share": float(p[:, i].mean()) / total}
                        for i, n in enumerate(STEP_PHASES) if n != "-"}}
+
+
+def mlp_phases(torch, rows=524288) -> dict:
+    """Where a workgroup of the whole-network MLP kernel (128-row tile, cfg 4 actor) spends its time: wall-clock stamps
+    (100 MHz counter) of wavefront 0 between the phases of each layer, mean over the workgroups of one launch; read from
+    the profiling build of the library, which takes the stamp buffer's address from KS_MLP_PROF_PTR."""
+    import numpy as np
+
+    from ksim_amd.configs import _net
+
+    actor = _net((68, 512, 512, 512, 20), np.random.default_rng(1004), last_scale=0.1)
+    blocks = (rows + 127) // 128
+    prof = torch.zeros(blocks * 32, dtype=torch.int64, device="cuda")
+    os.environ["KS_MLP_PROF_PTR"] = hex(prof.data_ptr())
+    x, y = torch.randn(rows, actor.in_dim, device="cuda"), torch.empty(rows, actor.out_dim, device="cuda")
+    for _ in range(3):
+        actor(x, out=y)
+    torch.cuda.synchronize()
+    del os.environ["KS_MLP_PROF_PTR"]
+    p = prof.cpu().numpy().reshape(blocks, 32)[:, :14].astype(np.float64)
+    d = (p[:, 1:] - p[:, :-1]) * 10.0  # ns
+    names = ["stage_input"] + [f"layer{l}_{w}" for l in range(4) for w in ("mfma_loop", "wait", "epilogue")]
+    return {"rows": rows, "workgroups": blocks, "tile_rows": 128,
+            "us_per_workgroup": float((p[:, 13] - p[:, 0]).mean() * 0.01),
+            "launch_span_us": float((p[:, 13].max() - p[:, 0].min()) * 0.01),
+            "phases_ns": {n: float(d[:, i].mean()) for i, n in enumerate(names)},
+            "what": "mfma_loop: weight fragments from L2 + MFMAs over the layer's K; wait: the barrier before the activation "
+                    "tile in LDS may be overwritten; epilogue: bias, activation, bf16 pack, write of the tile to LDS (last "
+                    "layer: to memory)"}
 
 
 def ppo_iteration_rate(torch, reps=3):
