@@ -113,7 +113,7 @@ def main() -> None:
     ap.add_argument("--integrator", choices=("euler", "implicitfast"), default="euler",
                     help="velocity update of the headline rollout: semi-implicit Euler (what the benchmark configs name) or "
                          "implicitfast (what ksim's RLConfig selects); the other one is reported under 'other_integrator'")
-    ap.add_argument("--only", choices=("mlp", "gae", "update", "rollout", "iteration", "phases", "mfma"), default=None,
+    ap.add_argument("--only", choices=("mlp", "gae", "update", "kbot_update", "rollout", "iteration", "phases", "mfma"), default=None,
                     help="run one section alone and print its JSON (the command the counter runs under profiles/ use)")
     ap.add_argument("--mlp-rows", type=int, default=0, help="with --only mlp: a single row count instead of 8192 and 524288")
     ap.add_argument("--streams", type=int, default=2,
@@ -160,6 +160,9 @@ def main() -> None:
         return
     if args.only == "update":
         print(json.dumps({"ppo_update": ppo_update_rate(torch)}))
+        return
+    if args.only == "kbot_update":
+        print(json.dumps({"kbot_update": kbot_update_rate(torch)}))
         return
     if args.only == "iteration":
         print(json.dumps({"ppo_iteration": ppo_iteration_rate(torch)}))
@@ -228,6 +231,7 @@ def main() -> None:
     for key in ("rows_8192", "rows_524288"):
         mlp[key]["of_mfma_yardstick"] = mlp[key]["TFLOPs"] / top
     upd = ppo_update_rate(torch)
+    kbot_upd = kbot_update_rate(torch)
     iteration = ppo_iteration_rate(torch)
 
     obs_dim = consts.terms.obs_dim
@@ -276,7 +280,7 @@ def main() -> None:
                              "cycles with a VALU instruction issuing is given beside); the HBM fraction is reported "
                              "against the bytes the engine contract obliges a step to move"},
         "same_rollout_200_steps": long_entry, "other_integrator": other_entry, "single_stream": single_entry,
-        "gae": gae, "streaming": streaming, "policy_mlp": mlp, "ppo_update": upd, "ppo_iteration": iteration, "graph_replay": graph,
+        "gae": gae, "streaming": streaming, "policy_mlp": mlp, "ppo_update": upd, "kbot_update": kbot_upd, "ppo_iteration": iteration, "graph_replay": graph,
     }
     if not args.no_cpu_baseline:
         base = cpu_baseline(args.integrator)
@@ -566,6 +570,69 @@ def ppo_update_rate(torch, reps=6):
             "mfma_utilisation": flops / ms / 1e9 / (BF16_PEAK_TFLOPS),
             "what": "forward + backward (3x the forward flops) of actor and critic 68-3x512-{20,1} bf16, GAE, loss "
                     "gradient and optimiser chain on 2048 envs x 32 steps"}
+
+
+def kbot_update_rate(torch, reps=4):
+    """One minibatch step of the K-Bot task as shipped (examples/kbot/train.py:80-95, 1287-1310, 1754-1757): LSTM actor
+    65 -> 2 x 128 -> 40 (means | deviations of 20 joints) and LSTM critic 475 -> 2 x 128 -> 1 in float32, 512 envs x 100
+    control steps per minibatch, the one-pole low-pass on the biased means with its state in the carry, and the second pass
+    of both networks over the mirrored observations from their own carries with the two mirror losses."""
+    import numpy as np
+
+    from ksim_amd import ppo_update as pu
+    from ksim_amd.actions import LowPass
+    from ksim_amd.mlp import MLP
+    from ksim_amd.recurrent import LSTMCell, RecurrentNetwork
+
+    rng = np.random.default_rng(7)
+    Tn, b, Ia, Ic, H, nu = 100, 512, 65, 475, 128, 20
+
+    def make(I, out_dim):
+        proj = (rng.normal(size=(H, I)) / np.sqrt(I), rng.normal(size=H) * 0.1)
+        cells = [LSTMCell(rng.normal(size=(4 * H, H)) / np.sqrt(H), rng.normal(size=(4 * H, H)) / np.sqrt(H),
+                          rng.normal(size=4 * H) * 0.1, dtype="f32") for _ in range(2)]
+        out = MLP([rng.normal(size=(out_dim, H)) / np.sqrt(H)], [rng.normal(size=out_dim) * 0.1], activation="none", dtype="f32")
+        return RecurrentNetwork(proj, cells, out, dtype="f32")
+
+    actor, critic = make(Ia, 2 * nu), make(Ic, 1)
+    sp = lambda n: (list(rng.permutation(n)), list(rng.choice([-1.0, 1.0], n)))  # noqa: E731
+    (pa, sa), (pc, sc), (pj, sj) = sp(Ia), sp(Ic), sp(nu)
+    t32 = lambda a: torch.tensor(np.asarray(a), dtype=torch.float32, device="cuda")  # noqa: E731
+    policy = pu.RecurrentHeadPolicy(actor, critic, 0.01, 1.0, 0.5, t32(rng.normal(size=nu) * 0.1),
+                                    mirror=pu.MirrorSpec(pa, sa, pc, sc, pj, sj), lowpass=LowPass(0.02, 10.0, obs_bias=(Ia - 11, 10, 10)))
+    policy.train_init()
+    cfg = pu.PPOUpdateConfig(batch_size=b, actor_mirror_loss_scale=1.0, critic_mirror_loss_scale=0.5)
+    g = torch.Generator(device="cuda")
+    g.manual_seed(0)
+    r = lambda *s: torch.randn(*s, device="cuda", generator=g)  # noqa: E731
+    aobs, cobs, act, rew = r(Tn, b, Ia), r(Tn, b, Ic), r(Tn, b, nu) * 0.3, r(Tn, b)
+    fresh = (torch.rand(Tn, b, device="cuda", generator=g) < 0.01).to(torch.uint8)
+    done = torch.roll(fresh, -1, 0)
+    done[-1] = 0
+    succ = torch.zeros_like(done)
+    on_lp, on_v = r(Tn, b, nu) * 0.1 - 1.0, r(Tn, b) * 0.1
+    carry = lambda: r(2, 2, b, H) * 0.3  # noqa: E731
+    args = (aobs, cobs, act, rew, done, succ, on_lp, on_v, carry(), carry(), fresh, r(b, nu) * 0.1,
+            pu.MirrorCarries(carry(), carry(), r(b, nu) * 0.1))
+    out = None
+    for _ in range(2):
+        out = pu.single_step_recurrent(policy, cfg, *args)
+    assert torch.isfinite(out["grad_norm"]).all()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(reps):
+        pu.single_step_recurrent(policy, cfg, *args)
+    e1.record()
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) / reps
+    ms = e0.elapsed_time(e1) / reps
+    return {"minibatch_envs": b, "rollout_steps": Tn, "mirrored_columns": b, "ms_per_minibatch_step": ms, "host_ms_per_minibatch_step": wall * 1e3,
+            "transitions_per_s": Tn * b / (ms * 1e-3),
+            "what": "K-Bot task minibatch step: LSTM actor 65-2x128-40 and critic 475-2x128-1 (float32) through 100 steps for 512 envs "
+                    "and their 512 mirror images in one pass, low-pass filter with its gradient through time, PPO + mirror losses, "
+                    "backward through time, global-norm clip and Adam"}
 
 
 STEP_PHASES = ("actuator + reload of constants", "forward kinematics", "com / cinert / cdof", "composite inertia + M",

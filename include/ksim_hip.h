@@ -878,6 +878,23 @@ int ks_lstm_backward_step(KsLstm* lstm, ks_stream_t stream, int64_t M, const flo
                           const float* saved, const uint8_t* fresh, float* d_g, float* dh_in, float* dc_in, void* workspace);
 int ks_lstm_grad_sqnorm(const KsLstm* lstm, ks_stream_t stream, double* acc);
 int ks_lstm_adam_step(KsLstm* lstm, ks_stream_t stream, const KsAdamParams* params /*host*/, const double* sqnorm);
+/* A whole trajectory of one LSTM layer in one launch each way: the lax.scan over the T steps of the trajectory inside the loss
+ * (ksim/task/ppo.py:572-694 around the model's forward, examples/kbot/train.py:903-915) and what jax.grad derives for it, for
+ * fp32 cells of hidden size 128 (ks_lstm_sequence_supported returns 1; other cells take the step-by-step entry points above).
+ *   ks_lstm_sequence_forward   gi (T, M, 4H) = W_ih x_t + bias for every step (one product over all T M rows through the
+ *                              input projection); h0, c0 (M, H) the carry the slice starts from; fresh (T, M) nullable;
+ *                              hs, cs (T, M, H) the states after every step (cs nullable), saved (T, M, 7H) nullable, in the
+ *                              layout of ks_lstm_train_forward.  With T = 1, hs / cs may alias h0 / c0; ks_lstm_forward and
+ *                              ks_lstm_train_forward are this launch with T = 1 for such cells, so a rollout's steps and the
+ *                              replay of its trajectory agree bit for bit.
+ *   ks_lstm_sequence_backward  dH (T, M, H) the gradient reaching h_t from the layer above; d_g (T, M, 4H) out, as
+ *                              ks_lstm_backward_step returns it per step; dh0, dc0 (M, H), nullable, the gradient of the
+ *                              initial carry.  Needs ks_lstm_train_init (the transposed weights). */
+int ks_lstm_sequence_supported(const KsLstm* lstm);
+int ks_lstm_sequence_forward(const KsLstm* lstm, ks_stream_t stream, int64_t T, int64_t M, const float* gi, const float* h0,
+                             const float* c0, const uint8_t* fresh, float* hs, float* cs, float* saved);
+int ks_lstm_sequence_backward(const KsLstm* lstm, ks_stream_t stream, int64_t T, int64_t M, const float* dH, const float* saved,
+                              const uint8_t* fresh, float* d_g, float* dh0, float* dc0);
 
 /* Gaussian policy head and the gradient of the PPO objective (ppo.py:149-246, total 473-486):
  *   ks_gaussian_log_prob: per action dimension log N(action; mean, exp(log_std)) and entropy

@@ -264,6 +264,12 @@ def bind(lib) -> None:
     lib.ks_lstm_backward_workspace_bytes.restype = c_int64
     lib.ks_lstm_backward_step.argtypes = [c_void_p, c_void_p, c_int64] + [c_void_p] * 8
     lib.ks_lstm_grad_sqnorm.argtypes = [c_void_p, c_void_p, c_void_p]
+    lib.ks_lstm_sequence_supported.argtypes = [c_void_p]
+    lib.ks_lstm_sequence_supported.restype = c_int32
+    lib.ks_lstm_sequence_forward.argtypes = [c_void_p, c_void_p, c_int64, c_int64] + [c_void_p] * 7
+    lib.ks_lstm_sequence_forward.restype = c_int32
+    lib.ks_lstm_sequence_backward.argtypes = [c_void_p, c_void_p, c_int64, c_int64] + [c_void_p] * 6
+    lib.ks_lstm_sequence_backward.restype = c_int32
     lib.ks_lstm_adam_step.argtypes = [c_void_p, c_void_p, POINTER(KsAdamParams), c_void_p]
     for name in ("ks_mlp_train_backward_dx", "ks_mlp_freeze_bias_prefix", "ks_gru_train_init", "ks_gru_projections",
                  "ks_gru_train_forward", "ks_gru_backward_step", "ks_gru_grad_sqnorm", "ks_gru_adam_step",

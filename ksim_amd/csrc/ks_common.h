@@ -25,4 +25,7 @@ inline int check_launch(const char* what) {
 
 constexpr int kWave = 64;
 
+// defined beside the MLP handle: weight matrix (npad, kpad) of layer l in working precision and its transpose (after train_init)
+int mlp_peek_layer(const KsMlp* h, int l, const void** W, const void** Wt, int* npad, int* kpad, int* dtype);
+
 }  // namespace ks

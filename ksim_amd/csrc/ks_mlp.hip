@@ -1280,6 +1280,18 @@ extern "C" int ks_mlp_create(const KsMlpDesc* d, KsMlp** out) {
   return KS_OK;
 }
 
+namespace ks {
+// For the recurrent sequence kernels, which multiply by a one-layer network's weights themselves: the live working-precision
+// weight matrix of layer l, (npad, kpad) row-major, and, once ks_mlp_train_init has run, its transpose (kpad, npad).  The
+// optimiser step rewrites both in place, so the pointers stay valid for the life of the handle.
+int mlp_peek_layer(const KsMlp* h, int l, const void** W, const void** Wt, int* npad, int* kpad, int* dtype) {
+  if (!h || l < 0 || l >= h->m.n_layers) return fail(KS_EINVAL, "mlp_peek_layer: no such layer");
+  *W = h->m.W[l]; *Wt = h->m.train ? h->m.Wt[l] : nullptr;
+  *npad = h->m.npad[l]; *kpad = h->m.kpad[l]; *dtype = h->m.dtype;
+  return KS_OK;
+}
+}  // namespace ks
+
 extern "C" int ks_mlp_destroy(KsMlp* h) {
   if (!h) return KS_OK;
   for (int l = 0; l < KS_MAX_LAYERS; ++l) {

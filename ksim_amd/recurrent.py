@@ -207,6 +207,36 @@ class LSTMCell:
                                                    _lib.ptr(fresh), _lib.ptr(h_out), _lib.ptr(c_out), _lib.ptr(saved),
                                                    _lib.ptr(self.workspace(M, x.device))))
 
+    @property
+    def sequence_supported(self) -> bool:
+        """Whether this cell has the one-launch-per-trajectory kernels (`ks_lstm_sequence_forward / _backward`)."""
+        return bool(self._lib.ks_lstm_sequence_supported(self._handle))
+
+    def sequence_forward(self, x, h0, c0, fresh, hs, cs, saved) -> None:
+        """The layer over a whole trajectory: x (T, M, input) -> hs, cs (T, M, H) and `saved` (T, M, 7H), from the carry
+        (h0, c0); the input projection is one product over all T M rows, the recurrence one launch."""
+        _lib.require_cuda(x, h0, c0, hs, cs, saved, dtype=torch.float32)
+        _lib.require_cuda(fresh, dtype=torch.uint8)
+        Tn, M, H = x.shape[0], x.shape[1], self.hidden_size
+        if (tuple(x.shape) != (Tn, M, self.input_size) or any(tuple(t.shape) != (M, H) for t in (h0, c0))
+                or any(tuple(t.shape) != (Tn, M, H) for t in (hs, cs)) or tuple(saved.shape) != (Tn, M, 7 * H)
+                or tuple(fresh.shape) != (Tn, M)):
+            raise _lib.KsError("expected x (T, M, input), h0, c0 (M, H), hs, cs (T, M, H), saved (T, M, 7H), fresh (T, M)")
+        gi = self.proj_i(x.reshape(Tn * M, self.input_size))
+        _lib.check(self._lib.ks_lstm_sequence_forward(self._handle, _lib.current_stream(), Tn, M, _lib.ptr(gi), _lib.ptr(h0),
+                                                      _lib.ptr(c0), _lib.ptr(fresh), _lib.ptr(hs), _lib.ptr(cs), _lib.ptr(saved)))
+
+    def sequence_backward(self, dH, saved, fresh, d_g) -> None:
+        """The reverse sweep over the trajectory: dH (T, M, H), the gradient reaching every h_t from above, -> d_g (T, M, 4H)."""
+        _lib.require_cuda(dH, saved, d_g, dtype=torch.float32)
+        _lib.require_cuda(fresh, dtype=torch.uint8)
+        Tn, M, H = dH.shape[0], dH.shape[1], self.hidden_size
+        if (tuple(dH.shape) != (Tn, M, H) or tuple(saved.shape) != (Tn, M, 7 * H) or tuple(d_g.shape) != (Tn, M, 4 * H)
+                or tuple(fresh.shape) != (Tn, M)):
+            raise _lib.KsError("expected dH (T, M, H), saved (T, M, 7H), d_g (T, M, 4H), fresh (T, M)")
+        _lib.check(self._lib.ks_lstm_sequence_backward(self._handle, _lib.current_stream(), Tn, M, _lib.ptr(dH), _lib.ptr(saved),
+                                                       _lib.ptr(fresh), _lib.ptr(d_g), None, None))
+
     def backward_step(self, dh_out, dc_out, saved, fresh, d_g, dh_in, dc_in) -> None:
         """One step of the backward pass through time: (dh_out, dc_out) -> d_g (M, 4H), dh_in, dc_in (M, H)."""
         _lib.require_cuda(dh_out, dc_out, saved, d_g, dh_in, dc_in, dtype=torch.float32)
@@ -306,7 +336,10 @@ class RecurrentNetwork:
         for i, cell in enumerate(self.cells):
             hs = torch.empty(T_, M, H, dtype=torch.float32, device=dev)
             sv = torch.empty(T_, M, (7 if self.lstm else 5) * H, dtype=torch.float32, device=dev)
-            if self.lstm:
+            if self.lstm and getattr(cell, "proj_i", None) is not None and cell.sequence_supported:
+                cs = torch.empty(T_, M, H, dtype=torch.float32, device=dev)
+                cell.sequence_forward(x, carry0[i, 0], carry0[i, 1], fresh, hs, cs, sv)
+            elif self.lstm:
                 cs = torch.empty(T_, M, H, dtype=torch.float32, device=dev)
                 for t in range(T_):
                     h0, c0 = (carry0[i, 0], carry0[i, 1]) if t == 0 else (hs[t - 1], cs[t - 1])
@@ -341,7 +374,10 @@ class RecurrentNetwork:
             d_gh = d_gi if self.lstm else torch.empty(T_, M, G * H, dtype=torch.float32, device=dev)
             carry = torch.zeros(2, M, H, dtype=torch.float32, device=dev)   # gradient of the hidden state, ping-pong
             ccarry = torch.zeros(2, M, H, dtype=torch.float32, device=dev)  # and of the cell state (LSTM)
-            for t in range(T_ - 1, -1, -1):
+            fused = self.lstm and cell.sequence_supported
+            if fused:
+                cell.sequence_backward(dH, sv, tp["fresh"], d_gi)
+            for t in range(T_ - 1, -1, -1) if not fused else ():
                 dH[t] += carry[t & 1]
                 if self.lstm:
                     cell.backward_step(dH[t], ccarry[t & 1], sv[t], tp["fresh"][t], d_gi[t], carry[(t + 1) & 1], ccarry[(t + 1) & 1])

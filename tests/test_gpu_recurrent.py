@@ -200,15 +200,17 @@ def test_backward_through_time_matches_the_oracle(dtype, tol, act):
     assert torch.isfinite(h1).all()
 
 
-@pytest.mark.parametrize("dtype,tol", [("f32", 2e-4), ("bf16", 6e-2)])
-def test_lstm_backward_through_time_matches_the_oracle(dtype, tol):
-    """The same for an LSTM stack (the K-Bot example's actor shape: projection, LSTM layers, linear output)."""
+@pytest.mark.parametrize("dtype,tol,H,N", [("f32", 2e-4, 64, 80), ("bf16", 6e-2, 64, 80), ("f32", 2e-4, 128, 77), ("f32", 2e-4, 128, 16)])
+def test_lstm_backward_through_time_matches_the_oracle(dtype, tol, H, N):
+    """The same for an LSTM stack (the K-Bot example's actor shape: projection, LSTM layers, linear output).  Hidden size
+    128 in fp32 is the K-Bot cell itself and runs through the one-launch-per-trajectory kernels (`ks_lstm_sequence_*`),
+    with a row count that does not fill the last 16-row workgroup."""
     from ksim_amd import _lib_terms as T
     from ksim_amd.mlp import MLP
     from ksim_amd.recurrent import LSTMCell, RecurrentNetwork
 
     rng = np.random.default_rng(43)
-    Tn, N, I, H, O = 10, 80, 29, 64, 12
+    Tn, I, O = 10, 29, 12
     proj = (rng.normal(size=(H, I)) / np.sqrt(I), rng.normal(size=H) * 0.1)
     cells = [(rng.normal(size=(4 * H, H)) / np.sqrt(H), rng.normal(size=(4 * H, H)) / np.sqrt(H), rng.normal(size=4 * H) * 0.1)
              for _ in range(2)]
@@ -222,6 +224,7 @@ def test_lstm_backward_through_time_matches_the_oracle(dtype, tol):
     want_out, want = orec.recurrent_sequence_gradients(obs, carry0, fresh, proj, cells, ow, ob, d_out)
     net = RecurrentNetwork(proj, [LSTMCell(*c, dtype=dtype) for c in cells], MLP(ow, ob, activation="none", dtype=dtype), dtype=dtype)
     net.train_init()
+    assert all(c.sequence_supported == (dtype == "f32" and H == 128) for c in net.cells)
     out = net.train_forward(t32(obs), t32(carry0), torch.tensor(fresh, dtype=torch.uint8, device=DEV))
     assert np.abs(out.cpu().numpy() - want_out).max() <= (1e-4 if dtype == "f32" else 3e-2) * np.abs(want_out).max()
     net.backward(t32(d_out))
@@ -239,3 +242,49 @@ def test_lstm_backward_through_time_matches_the_oracle(dtype, tol):
     for c in net.cells:  # the hidden projection carries no bias of its own, before and after the update
         (_, bh), = c.proj_h.parameters()
         assert torch.equal(bh, torch.zeros(4 * H, device=DEV))
+
+
+def test_lstm_sequence_kernels_agree_with_the_step_by_step_entry_points():
+    """One launch over the trajectory against T calls of the per-step entry points on the same cell (which, for such a cell,
+    are that launch with T = 1): states, saved activations and gate gradients bit for bit; the carry of the hidden-state
+    gradient, which the per-step path forms with a separate product, to rounding.  In place with T = 1, as the rollout
+    advances its carry."""
+    from ksim_amd import _lib
+    from ksim_amd.recurrent import LSTMCell
+
+    rng = np.random.default_rng(47)
+    Tn, M, H = 7, 45, 128
+    cell = LSTMCell(rng.normal(size=(4 * H, H)) / np.sqrt(H), rng.normal(size=(4 * H, H)) / np.sqrt(H), rng.normal(size=4 * H) * 0.1, dtype="f32")
+    cell.train_init()
+    assert cell.sequence_supported
+    x, h0, c0 = t32(rng.normal(size=(Tn, M, H))), t32(rng.normal(size=(M, H)) * 0.5), t32(rng.normal(size=(M, H)) * 0.5)
+    fresh = torch.tensor(rng.random((Tn, M)) < 0.1, dtype=torch.uint8, device=DEV)
+    z = lambda *s: torch.zeros(*s, device=DEV)  # noqa: E731
+    hs, cs, sv = z(Tn, M, H), z(Tn, M, H), z(Tn, M, 7 * H)
+    cell.sequence_forward(x, h0, c0, fresh, hs, cs, sv)
+    hs1, cs1, sv1 = z(Tn, M, H), z(Tn, M, H), z(Tn, M, 7 * H)
+    for t in range(Tn):
+        cell.train_forward(x[t], h0 if t == 0 else hs1[t - 1], c0 if t == 0 else cs1[t - 1], fresh[t], hs1[t], cs1[t], sv1[t])
+    assert torch.equal(hs, hs1) and torch.equal(cs, cs1) and torch.equal(sv, sv1)
+    h, c = h0.clone(), c0.clone()  # the rollout's step: the carry advanced in place
+    for t in range(Tn):
+        cell(x[t], h, c, fresh[t], out=(h, c))
+    assert torch.equal(h, hs[-1]) and torch.equal(c, cs[-1])
+    dH = t32(rng.normal(size=(Tn, M, H)))
+    d_g = z(Tn, M, 4 * H)
+    cell.sequence_backward(dH, sv, fresh, d_g)
+    d_g1, carry, ccarry = z(Tn, M, 4 * H), z(2, M, H), z(2, M, H)
+    dH1 = dH.clone()
+    for t in range(Tn - 1, -1, -1):
+        dH1[t] += carry[t & 1]
+        cell.backward_step(dH1[t], ccarry[t & 1], sv[t], fresh[t], d_g1[t], carry[(t + 1) & 1], ccarry[(t + 1) & 1])
+    err = (d_g - d_g1).abs().max().item() / d_g1.abs().max().item()
+    assert err < 1e-5, err
+    assert torch.equal(d_g[-1], d_g1[-1])  # the last step has no carried gradient yet: the same arithmetic
+    lib = _lib.load()  # shapes the kernels do not cover are refused, not approximated
+    small = LSTMCell(rng.normal(size=(4 * 64, 64)), rng.normal(size=(4 * 64, 64)), None, dtype="f32")
+    assert not small.sequence_supported
+    assert lib.ks_lstm_sequence_forward(small._handle, _lib.current_stream(), 1, 4, _lib.ptr(z(4, 256)), _lib.ptr(z(4, 64)), _lib.ptr(z(4, 64)),
+                                        None, _lib.ptr(z(4, 64)), None, None) != 0
+    assert lib.ks_lstm_sequence_forward(cell._handle, _lib.current_stream(), 2, M, _lib.ptr(z(2, M, 4 * H)), _lib.ptr(h0), _lib.ptr(c0),
+                                        None, _lib.ptr(h0), None, None) != 0  # aliasing is for T = 1 only
