@@ -157,15 +157,16 @@ __global__ __launch_bounds__(256) void lstm_gate_backward_kernel(int64_t M, int 
 
 // ---------------------------------------------------------------- a whole trajectory of one LSTM layer in one launch
 // The step-by-step path costs two GEMM launches and a gate kernel per step, layer and network: a minibatch of 100 control steps
-// is thousands of launches of a few microseconds each.  Here a workgroup of eight wavefronts owns 16 rows (envs) for all T
-// steps.  Wavefront w owns hidden units [16 w, 16 w + 16): its slice of W_hh, the four gates' rows of those units, stays in
-// 128 vector registers per lane for the whole sequence, the hidden state of the 16 rows lives in LDS (double buffered),
-// the cell state in registers, and each step is 128 16x16x4 fp32 MFMAs per wavefront computing G^T = W_hh h^T (lane: row
-// l % 16, registers: units 4 (l / 16) + r, so a lane holds all four gates of its units), the gate arithmetic, and one
-// barrier.  The K dimension is permuted so that k-group q = l / 16 covers the contiguous hidden units [32 q, 32 q + 32): both
-// operands are then read with 16-byte loads.  fp32 cells of hidden size 128.
+// is thousands of launches of a few microseconds each.  Here a workgroup of eight wavefronts owns 4 rows (envs) for all T
+// steps, so that a minibatch of a thousand rows is one workgroup per CU.  The product runs on v_mfma_f32_4x4x1 (sixteen
+// independent 4x4 outer products per instruction): block b = lane / 4 of wavefront w is hidden unit 16 w + b, its four A entries
+// are that unit's input / forget / cell / output rows of W_hh and its four B entries the four rows' hidden state, so after K = 128
+// instructions lane (b, j) holds the four gate pre-activations of its unit for row j.  The wavefront's slice of W_hh stays in
+// 128 vector registers per lane for the whole sequence, the hidden state of the 4 rows lives in LDS (double buffered), the
+// cell state in a register; a step is 128 MFMAs, the gate arithmetic of one (unit, row) per lane, and one barrier.
+// fp32 cells of hidden size 128.
 typedef __attribute__((ext_vector_type(4))) float f32x4;
-constexpr int kSeqRows = 16, kSeqH = 128, kSeqWaves = 8, kSeqPadH = kSeqH + 4, kSeqPadG = 4 * kSeqH + 4;
+constexpr int kSeqRows = 4, kSeqH = 128, kSeqWaves = 8, kSeqPadH = kSeqH + 4, kSeqPadG = 4 * kSeqH + 4;
 
 __device__ __forceinline__ float sigmoid_ks(float x) { return 1.f / (1.f + expf(-x)); }
 
@@ -176,30 +177,24 @@ void lstm_seq_forward_kernel(int T, int64_t M, const float* __restrict__ gi, con
   constexpr int H = kSeqH;
   __shared__ __attribute__((aligned(16))) float sh[2][kSeqRows][kSeqPadH];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int row = lane & 15, q = lane >> 4;
+  const int j = lane & 3, unit = 16 * wave + (lane >> 2);
   const int64_t r0 = (int64_t)blockIdx.x * kSeqRows;
-  const int64_t m = r0 + row;
+  const int64_t m = r0 + j;
   const bool row_ok = m < M;
   const int64_t mc = row_ok ? m : M - 1;  // loads of the rows past the batch are clamped, their stores dropped
-  const int u0 = 16 * wave + 4 * q;       // the four hidden units whose gates this lane ends up holding
-  // A operands: W_hh[gate g, unit 16 wave + l % 16][k = 32 q + s]
-  float wa[4][32];
+  // A operand of block b, entry i = lane % 4: W_hh[gate i, unit][k]
+  float wa[H];
+  {
+    const float4* src = reinterpret_cast<const float4*>(W + (int64_t)(j * H + unit) * ldw);
 #pragma unroll
-  for (int g = 0; g < 4; ++g) {
-    const float4* src = reinterpret_cast<const float4*>(W + (int64_t)(g * H + 16 * wave + row) * ldw + 32 * q);
-#pragma unroll
-    for (int s4 = 0; s4 < 8; ++s4) {
-      const float4 v = src[s4];
-      wa[g][4 * s4] = v.x; wa[g][4 * s4 + 1] = v.y; wa[g][4 * s4 + 2] = v.z; wa[g][4 * s4 + 3] = v.w;
+    for (int k4 = 0; k4 < H / 4; ++k4) {
+      const float4 v = src[k4];
+      wa[4 * k4] = v.x; wa[4 * k4 + 1] = v.y; wa[4 * k4 + 2] = v.z; wa[4 * k4 + 3] = v.w;
     }
   }
-  float c[4];
-  {
-    const float4 v = *reinterpret_cast<const float4*>(c0 + mc * H + u0);
-    c[0] = v.x; c[1] = v.y; c[2] = v.z; c[3] = v.w;
-  }
-  for (int idx = threadIdx.x; idx < kSeqRows * H / 4; idx += 64 * kSeqWaves) {
-    const int r = idx / (H / 4), k4 = idx - r * (H / 4);
+  float c = c0[mc * H + unit];
+  if (threadIdx.x < kSeqRows * H / 4) {
+    const int r = threadIdx.x / (H / 4), k4 = threadIdx.x - r * (H / 4);
     const int64_t mr = r0 + r < M ? r0 + r : M - 1;
     *reinterpret_cast<float4*>(&sh[0][r][4 * k4]) = *reinterpret_cast<const float4*>(h0 + mr * H + 4 * k4);
   }
@@ -207,54 +202,37 @@ void lstm_seq_forward_kernel(int T, int64_t M, const float* __restrict__ gi, con
   int cur = 0;
   for (int t = 0; t < T; ++t) {
     const int64_t tm = (int64_t)t * M + mc;
-    float4 gin[4];
+    float gin[4];
 #pragma unroll
-    for (int g = 0; g < 4; ++g) gin[g] = *reinterpret_cast<const float4*>(gi + tm * 4 * H + g * H + u0);
+    for (int g = 0; g < 4; ++g) gin[g] = gi[tm * 4 * H + g * H + unit];
     const bool f = fresh && fresh[tm];
-    f32x4 acc[4];
+    f32x4 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
+    const float* hrow = &sh[cur][j][0];
 #pragma unroll
-    for (int g = 0; g < 4; ++g) acc[g] = f32x4{0.f, 0.f, 0.f, 0.f};
-    const float* hrow = &sh[cur][row][32 * q];
-#pragma unroll
-    for (int s4 = 0; s4 < 8; ++s4) {
-      const float4 hb = *reinterpret_cast<const float4*>(hrow + 4 * s4);
-      const float hv[4] = {hb.x, hb.y, hb.z, hb.w};
-#pragma unroll
-      for (int e = 0; e < 4; ++e)
-#pragma unroll
-        for (int g = 0; g < 4; ++g) acc[g] = __builtin_amdgcn_mfma_f32_16x16x4f32(wa[g][4 * s4 + e], hv[e], acc[g], 0, 0, 0);
+    for (int k4 = 0; k4 < H / 4; ++k4) {
+      const float4 hb = *reinterpret_cast<const float4*>(hrow + 4 * k4);
+      acc0 = __builtin_amdgcn_mfma_f32_4x4x1f32(wa[4 * k4], hb.x, acc0, 0, 0, 0);
+      acc1 = __builtin_amdgcn_mfma_f32_4x4x1f32(wa[4 * k4 + 1], hb.y, acc1, 0, 0, 0);
+      acc0 = __builtin_amdgcn_mfma_f32_4x4x1f32(wa[4 * k4 + 2], hb.z, acc0, 0, 0, 0);
+      acc1 = __builtin_amdgcn_mfma_f32_4x4x1f32(wa[4 * k4 + 3], hb.w, acc1, 0, 0, 0);
     }
-    const float4 hp4 = *reinterpret_cast<const float4*>(&sh[cur][row][u0]);
-    const float hp[4] = {hp4.x, hp4.y, hp4.z, hp4.w};
-    const float gI[4] = {gin[0].x, gin[0].y, gin[0].z, gin[0].w}, gF[4] = {gin[1].x, gin[1].y, gin[1].z, gin[1].w};
-    const float gG[4] = {gin[2].x, gin[2].y, gin[2].z, gin[2].w}, gO[4] = {gin[3].x, gin[3].y, gin[3].z, gin[3].w};
-    float si[4], sf[4], tg[4], so[4], tc[4], cp[4], hu[4], hn[4];
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      cp[r] = f ? 0.f : c[r];
-      hu[r] = f ? 0.f : hp[r];
-      si[r] = sigmoid_ks(gI[r] + (f ? 0.f : acc[0][r]));
-      sf[r] = sigmoid_ks(gF[r] + (f ? 0.f : acc[1][r]));
-      tg[r] = tanhf(gG[r] + (f ? 0.f : acc[2][r]));
-      so[r] = sigmoid_ks(gO[r] + (f ? 0.f : acc[3][r]));
-      c[r] = sf[r] * cp[r] + si[r] * tg[r];
-      tc[r] = tanhf(c[r]);
-      hn[r] = so[r] * tc[r];
-    }
-    *reinterpret_cast<float4*>(&sh[cur ^ 1][row][u0]) = float4{hn[0], hn[1], hn[2], hn[3]};
+    const float hprev = sh[cur][j][unit];
+    const float cp = f ? 0.f : c, hu = f ? 0.f : hprev;
+    const float si = sigmoid_ks(gin[0] + (f ? 0.f : acc0[0] + acc1[0]));
+    const float sf = sigmoid_ks(gin[1] + (f ? 0.f : acc0[1] + acc1[1]));
+    const float tg = tanhf(gin[2] + (f ? 0.f : acc0[2] + acc1[2]));
+    const float so = sigmoid_ks(gin[3] + (f ? 0.f : acc0[3] + acc1[3]));
+    c = sf * cp + si * tg;
+    const float tc = tanhf(c);
+    const float hn = so * tc;
+    sh[cur ^ 1][j][unit] = hn;
     if (row_ok) {
       const int64_t o = (int64_t)t * M + m;
-      *reinterpret_cast<float4*>(hs + o * H + u0) = float4{hn[0], hn[1], hn[2], hn[3]};
-      if (cs) *reinterpret_cast<float4*>(cs + o * H + u0) = float4{c[0], c[1], c[2], c[3]};
+      hs[o * H + unit] = hn;
+      if (cs) cs[o * H + unit] = c;
       if (saved) {
-        float* sv = saved + o * 7 * H + u0;
-        *reinterpret_cast<float4*>(sv) = float4{si[0], si[1], si[2], si[3]};
-        *reinterpret_cast<float4*>(sv + H) = float4{sf[0], sf[1], sf[2], sf[3]};
-        *reinterpret_cast<float4*>(sv + 2 * H) = float4{tg[0], tg[1], tg[2], tg[3]};
-        *reinterpret_cast<float4*>(sv + 3 * H) = float4{so[0], so[1], so[2], so[3]};
-        *reinterpret_cast<float4*>(sv + 4 * H) = float4{tc[0], tc[1], tc[2], tc[3]};
-        *reinterpret_cast<float4*>(sv + 5 * H) = float4{cp[0], cp[1], cp[2], cp[3]};
-        *reinterpret_cast<float4*>(sv + 6 * H) = float4{hu[0], hu[1], hu[2], hu[3]};
+        float* sv = saved + o * 7 * H + unit;
+        sv[0] = si; sv[H] = sf; sv[2 * H] = tg; sv[3 * H] = so; sv[4 * H] = tc; sv[5 * H] = cp; sv[6 * H] = hu;
       }
     }
     __syncthreads();  // the new hidden state is complete; the buffer just read is free for the step after next
@@ -263,9 +241,11 @@ void lstm_seq_forward_kernel(int T, int64_t M, const float* __restrict__ gi, con
 }
 
 // The reverse sweep of the same layer: dH (T, M, H) is the gradient reaching h_t from the layer above; the gradient through
-// W_hh and the cell state are carried in registers.  Per step: the gate derivatives from the saved activations (lstm_gate_backward_kernel's
-// formulas) into d_g (T, M, 4H) and LDS, then dh_{t-1} = d_g W_hh as 128 16x16x4 MFMAs per wavefront over the transposed
-// weights (units [16 w, 16 w + 16) x all 4H gate rows, 128 registers per lane again; k-group q covers gate rows [128 q, 128 q + 128)).
+// W_hh and that of the cell state are carried in registers.  Per step: the gate derivatives from the saved activations
+// (lstm_gate_backward_kernel's formulas) into d_g (T, M, 4H) and LDS, then dh_{t-1} = d_g W_hh over the transposed weights.
+// Here the sixteen blocks of an MFMA are four groups of four units (entries i) times four quarters of the 4H gate rows
+// (K split four ways): lane (b, j) accumulates, for row j, the partial sums over gate rows [128 (b / 4), 128 (b / 4) + 128) of the
+// units 16 w + 4 (b % 4) + {0..3}; two lane exchanges add the quarters, and the lane keeps the unit 16 w + 4 (b % 4) + b / 4.
 __global__ __launch_bounds__(64 * kSeqWaves) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void lstm_seq_backward_kernel(int T, int64_t M, const float* __restrict__ dH, const float* __restrict__ saved,
                               const uint8_t* __restrict__ fresh, const float* __restrict__ Wt, int ldwt,
@@ -273,75 +253,64 @@ void lstm_seq_backward_kernel(int T, int64_t M, const float* __restrict__ dH, co
   constexpr int H = kSeqH;
   __shared__ __attribute__((aligned(16))) float sg[kSeqRows][kSeqPadG];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int row = lane & 15, q = lane >> 4;
+  const int j = lane & 3, ug = (lane >> 2) & 3, kg = lane >> 4;
+  const int unit = 16 * wave + 4 * ug + kg;  // the (unit, row j) whose gate arithmetic and carried gradients this lane owns
   const int64_t r0 = (int64_t)blockIdx.x * kSeqRows;
-  const int64_t m = r0 + row;
+  const int64_t m = r0 + j;
   const bool row_ok = m < M;
   const int64_t mc = row_ok ? m : M - 1;
-  const int u0 = 16 * wave + 4 * q;
-  // A operands: Wt[unit 16 wave + l % 16][gate row 128 q + s]
+  // A operand of block b, entry i = lane % 4: Wt[unit 16 w + 4 ug + i][gate row 128 kg + s]
   float wa[128];
   {
-    const float4* src = reinterpret_cast<const float4*>(Wt + (int64_t)(16 * wave + row) * ldwt + 128 * q);
+    const float4* src = reinterpret_cast<const float4*>(Wt + (int64_t)(16 * wave + 4 * ug + j) * ldwt + 128 * kg);
 #pragma unroll
     for (int s4 = 0; s4 < 32; ++s4) {
       const float4 v = src[s4];
       wa[4 * s4] = v.x; wa[4 * s4 + 1] = v.y; wa[4 * s4 + 2] = v.z; wa[4 * s4 + 3] = v.w;
     }
   }
-  float dhc[4] = {0.f, 0.f, 0.f, 0.f}, dc[4] = {0.f, 0.f, 0.f, 0.f};
+  float dhc = 0.f, dc = 0.f;
   for (int t = T - 1; t >= 0; --t) {
     const int64_t o = (int64_t)t * M + mc;
     const bool f = fresh && fresh[o];
-    const float* sv = saved + o * 7 * H + u0;
-    const float4 si4 = *reinterpret_cast<const float4*>(sv), sf4 = *reinterpret_cast<const float4*>(sv + H),
-                 tg4 = *reinterpret_cast<const float4*>(sv + 2 * H), so4 = *reinterpret_cast<const float4*>(sv + 3 * H),
-                 tc4 = *reinterpret_cast<const float4*>(sv + 4 * H), cp4 = *reinterpret_cast<const float4*>(sv + 5 * H);
-    const float4 dh4 = *reinterpret_cast<const float4*>(dH + o * H + u0);
-    const float si[4] = {si4.x, si4.y, si4.z, si4.w}, sf[4] = {sf4.x, sf4.y, sf4.z, sf4.w}, tg[4] = {tg4.x, tg4.y, tg4.z, tg4.w};
-    const float so[4] = {so4.x, so4.y, so4.z, so4.w}, tc[4] = {tc4.x, tc4.y, tc4.z, tc4.w}, cp[4] = {cp4.x, cp4.y, cp4.z, cp4.w};
-    const float dhin[4] = {dh4.x, dh4.y, dh4.z, dh4.w};
-    float gI[4], gF[4], gG[4], gO[4];
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      const float dh = dhin[r] + dhc[r];
-      const float dct = dc[r] + dh * so[r] * (1.f - tc[r] * tc[r]);
-      gI[r] = dct * tg[r] * si[r] * (1.f - si[r]);
-      gF[r] = dct * cp[r] * sf[r] * (1.f - sf[r]);
-      gG[r] = dct * si[r] * (1.f - tg[r] * tg[r]);
-      gO[r] = dh * tc[r] * so[r] * (1.f - so[r]);
-      dc[r] = f ? 0.f : dct * sf[r];
-    }
-    *reinterpret_cast<float4*>(&sg[row][u0]) = float4{gI[0], gI[1], gI[2], gI[3]};
-    *reinterpret_cast<float4*>(&sg[row][H + u0]) = float4{gF[0], gF[1], gF[2], gF[3]};
-    *reinterpret_cast<float4*>(&sg[row][2 * H + u0]) = float4{gG[0], gG[1], gG[2], gG[3]};
-    *reinterpret_cast<float4*>(&sg[row][3 * H + u0]) = float4{gO[0], gO[1], gO[2], gO[3]};
+    const float* sv = saved + o * 7 * H + unit;
+    const float si = sv[0], sf = sv[H], tg = sv[2 * H], so = sv[3 * H], tc = sv[4 * H], cp = sv[5 * H];
+    const float dh = dH[o * H + unit] + dhc;
+    const float dct = dc + dh * so * (1.f - tc * tc);
+    const float gI = dct * tg * si * (1.f - si), gF = dct * cp * sf * (1.f - sf), gG = dct * si * (1.f - tg * tg),
+                gO = dh * tc * so * (1.f - so);
+    dc = f ? 0.f : dct * sf;
+    sg[j][unit] = gI; sg[j][H + unit] = gF; sg[j][2 * H + unit] = gG; sg[j][3 * H + unit] = gO;
     if (row_ok) {
-      float* dg = d_g + ((int64_t)t * M + m) * 4 * H + u0;
-      *reinterpret_cast<float4*>(dg) = float4{gI[0], gI[1], gI[2], gI[3]};
-      *reinterpret_cast<float4*>(dg + H) = float4{gF[0], gF[1], gF[2], gF[3]};
-      *reinterpret_cast<float4*>(dg + 2 * H) = float4{gG[0], gG[1], gG[2], gG[3]};
-      *reinterpret_cast<float4*>(dg + 3 * H) = float4{gO[0], gO[1], gO[2], gO[3]};
+      float* dg = d_g + ((int64_t)t * M + m) * 4 * H + unit;
+      dg[0] = gI; dg[H] = gF; dg[2 * H] = gG; dg[3 * H] = gO;
     }
     __syncthreads();
-    f32x4 acc[4];
-#pragma unroll
-    for (int a = 0; a < 4; ++a) acc[a] = f32x4{0.f, 0.f, 0.f, 0.f};
-    const float* grow = &sg[row][128 * q];
+    f32x4 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
+    const float* grow = &sg[j][128 * kg];
 #pragma unroll
     for (int s4 = 0; s4 < 32; ++s4) {
       const float4 gb = *reinterpret_cast<const float4*>(grow + 4 * s4);
-      const float gv[4] = {gb.x, gb.y, gb.z, gb.w};
-#pragma unroll
-      for (int e = 0; e < 4; ++e) acc[e] = __builtin_amdgcn_mfma_f32_16x16x4f32(wa[4 * s4 + e], gv[e], acc[e], 0, 0, 0);
+      acc0 = __builtin_amdgcn_mfma_f32_4x4x1f32(wa[4 * s4], gb.x, acc0, 0, 0, 0);
+      acc1 = __builtin_amdgcn_mfma_f32_4x4x1f32(wa[4 * s4 + 1], gb.y, acc1, 0, 0, 0);
+      acc0 = __builtin_amdgcn_mfma_f32_4x4x1f32(wa[4 * s4 + 2], gb.z, acc0, 0, 0, 0);
+      acc1 = __builtin_amdgcn_mfma_f32_4x4x1f32(wa[4 * s4 + 3], gb.w, acc1, 0, 0, 0);
     }
+    float part[4];
 #pragma unroll
-    for (int r = 0; r < 4; ++r) dhc[r] = f ? 0.f : (acc[0][r] + acc[1][r]) + (acc[2][r] + acc[3][r]);
+    for (int r = 0; r < 4; ++r) {
+      float v = acc0[r] + acc1[r];
+      v += __shfl_xor(v, 16);
+      v += __shfl_xor(v, 32);
+      part[r] = v;
+    }
+    const float mine = kg == 0 ? part[0] : (kg == 1 ? part[1] : (kg == 2 ? part[2] : part[3]));
+    dhc = f ? 0.f : mine;
     __syncthreads();  // every wavefront has read this step's gate gradients
   }
   if (row_ok) {
-    if (dh0) *reinterpret_cast<float4*>(dh0 + m * H + u0) = float4{dhc[0], dhc[1], dhc[2], dhc[3]};
-    if (dc0) *reinterpret_cast<float4*>(dc0 + m * H + u0) = float4{dc[0], dc[1], dc[2], dc[3]};
+    if (dh0) dh0[m * H + unit] = dhc;
+    if (dc0) dc0[m * H + unit] = dc;
   }
 }
 
