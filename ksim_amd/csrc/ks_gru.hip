@@ -200,12 +200,23 @@ void lstm_seq_forward_kernel(int T, int64_t M, const float* __restrict__ gi, con
   }
   __syncthreads();
   int cur = 0;
+  // the step's inputs from memory are fetched one step ahead: their latency would otherwise stand between the matrix work and the gates
+  float gnext[4];
+  uint8_t fnext = 0;
+#pragma unroll
+  for (int g = 0; g < 4; ++g) gnext[g] = gi[mc * 4 * H + g * H + unit];
+  if (fresh) fnext = fresh[mc];
   for (int t = 0; t < T; ++t) {
-    const int64_t tm = (int64_t)t * M + mc;
     float gin[4];
 #pragma unroll
-    for (int g = 0; g < 4; ++g) gin[g] = gi[tm * 4 * H + g * H + unit];
-    const bool f = fresh && fresh[tm];
+    for (int g = 0; g < 4; ++g) gin[g] = gnext[g];
+    const bool f = fnext != 0;
+    if (t + 1 < T) {
+      const int64_t tn = (int64_t)(t + 1) * M + mc;
+#pragma unroll
+      for (int g = 0; g < 4; ++g) gnext[g] = gi[tn * 4 * H + g * H + unit];
+      if (fresh) fnext = fresh[tn];
+    }
     f32x4 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
     const float* hrow = &sh[cur][j][0];
 #pragma unroll
@@ -270,12 +281,29 @@ void lstm_seq_backward_kernel(int T, int64_t M, const float* __restrict__ dH, co
     }
   }
   float dhc = 0.f, dc = 0.f;
-  for (int t = T - 1; t >= 0; --t) {
-    const int64_t o = (int64_t)t * M + mc;
-    const bool f = fresh && fresh[o];
+  // the step's inputs from memory are fetched one step ahead, under the matrix work of the step before
+  float nx[7];
+  uint8_t fnext = 0;
+  {
+    const int64_t o = (int64_t)(T - 1) * M + mc;
     const float* sv = saved + o * 7 * H + unit;
-    const float si = sv[0], sf = sv[H], tg = sv[2 * H], so = sv[3 * H], tc = sv[4 * H], cp = sv[5 * H];
-    const float dh = dH[o * H + unit] + dhc;
+#pragma unroll
+    for (int k = 0; k < 6; ++k) nx[k] = sv[k * H];
+    nx[6] = dH[o * H + unit];
+    if (fresh) fnext = fresh[o];
+  }
+  for (int t = T - 1; t >= 0; --t) {
+    const bool f = fnext != 0;
+    const float si = nx[0], sf = nx[1], tg = nx[2], so = nx[3], tc = nx[4], cp = nx[5];
+    const float dh = nx[6] + dhc;
+    if (t > 0) {
+      const int64_t o = (int64_t)(t - 1) * M + mc;
+      const float* sv = saved + o * 7 * H + unit;
+#pragma unroll
+      for (int k = 0; k < 6; ++k) nx[k] = sv[k * H];
+      nx[6] = dH[o * H + unit];
+      if (fresh) fnext = fresh[o];
+    }
     const float dct = dc + dh * so * (1.f - tc * tc);
     const float gI = dct * tg * si * (1.f - si), gF = dct * cp * sf * (1.f - sf), gG = dct * si * (1.f - tg * tg),
                 gO = dh * tc * so * (1.f - so);
