@@ -1777,7 +1777,11 @@ static int train_backward(DevMlp& m, hipStream_t s, int64_t M, const float* x, c
   }
   T* dz = (T*)ws.d0;
   T* dnext = (T*)ws.d1;
-  {  // the output gradient in working precision, padded to the last layer's width
+  if (L == 1 && sizeof(T) == 4 && m.dims[1] == m.npad[0]) {
+    // a single fp32 layer whose width needs no padding (the projections of the recurrent cells): the caller's gradient is
+    // already the operand, and with one layer nothing below writes into this buffer
+    dz = (T*)const_cast<float*>(dy);
+  } else {  // the output gradient in working precision, padded to the last layer's width
     const int64_t n = M * m.npad[L - 1];
     hipLaunchKernelGGL(cast_pad_kernel<T>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, M, m.dims[L], m.npad[L - 1], dy, dz);
   }
