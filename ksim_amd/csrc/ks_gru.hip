@@ -171,17 +171,13 @@ constexpr int kSeqRows = 4, kSeqH = 128, kSeqWaves = 8, kSeqPadH = kSeqH + 4, kS
 __device__ __forceinline__ float sigmoid_ks(float x) { return 1.f / (1.f + expf(-x)); }
 
 __global__ __launch_bounds__(64 * kSeqWaves) __attribute__((amdgpu_waves_per_eu(2, 2)))
-void lstm_seq_forward_kernel(int T, int64_t M, const float* __restrict__ gi, const float* __restrict__ W, int ldw,
+void lstm_seq_forward_kernel(int T, int64_t M, int groups, const float* __restrict__ gi, const float* __restrict__ W, int ldw,
                              const float* h0, const float* c0, const uint8_t* __restrict__ fresh,
                              float* hs, float* cs, float* __restrict__ saved) {  // with T = 1, hs / cs may be h0 / c0
   constexpr int H = kSeqH;
   __shared__ __attribute__((aligned(16))) float sh[2][kSeqRows][kSeqPadH];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int j = lane & 3, unit = 16 * wave + (lane >> 2);
-  const int64_t r0 = (int64_t)blockIdx.x * kSeqRows;
-  const int64_t m = r0 + j;
-  const bool row_ok = m < M;
-  const int64_t mc = row_ok ? m : M - 1;  // loads of the rows past the batch are clamped, their stores dropped
   // A operand of block b, entry i = lane % 4: W_hh[gate i, unit][k]
   float wa[H];
   {
@@ -192,6 +188,15 @@ void lstm_seq_forward_kernel(int T, int64_t M, const float* __restrict__ gi, con
       wa[4 * k4] = v.x; wa[4 * k4 + 1] = v.y; wa[4 * k4 + 2] = v.z; wa[4 * k4 + 3] = v.w;
     }
   }
+  // A workgroup takes `groups` sets of 4 rows one after the other with the same registers of weights: a single step over
+  // thousands of rows (the rollout's call) would otherwise fetch the 256 KB of W_hh once per 4 rows.
+  for (int grp = 0; grp < groups; ++grp) {
+  const int64_t r0 = ((int64_t)blockIdx.x * groups + grp) * kSeqRows;
+  if (r0 >= M) break;  // the same for every thread of the workgroup
+  const int64_t m = r0 + j;
+  const bool row_ok = m < M;
+  const int64_t mc = row_ok ? m : M - 1;  // loads of the rows past the batch are clamped, their stores dropped
+  if (grp > 0) __syncthreads();  // the previous set's last read of the state buffers is over
   float c = c0[mc * H + unit];
   if (threadIdx.x < kSeqRows * H / 4) {
     const int r = threadIdx.x / (H / 4), k4 = threadIdx.x - r * (H / 4);
@@ -248,6 +253,7 @@ void lstm_seq_forward_kernel(int T, int64_t M, const float* __restrict__ gi, con
     }
     __syncthreads();  // the new hidden state is complete; the buffer just read is free for the step after next
     cur ^= 1;
+  }
   }
 }
 
@@ -588,10 +594,15 @@ extern "C" int ks_lstm_sequence_forward(const KsLstm* g, ks_stream_t stream, int
   int ldw, ldwt;
   if (!lstm_seq_weights(g, &W, &ldw, &Wt, &ldwt)) return fail(KS_EINVAL, "ks_lstm_sequence_forward: needs an fp32 cell of hidden size %d", kSeqH);
   if (T > 1 && (hs == h0 || (cs && cs == c0))) return fail(KS_EINVAL, "ks_lstm_sequence_forward: outputs may alias the initial state only for T = 1");
-  const int64_t grid = (M + kSeqRows - 1) / kSeqRows;
+  // sets of 4 rows per workgroup: one while there is at most one set per CU (long sequences want every CU), more when a short
+  // call covers so many rows that re-reading the weights per set would dominate it
+  const int64_t sets = (M + kSeqRows - 1) / kSeqRows;
+  int groups = 1;
+  if (T * 8 <= 64) while (groups < 8 && sets > (int64_t)256 * groups) groups *= 2;
+  const int64_t grid = (sets + groups - 1) / groups;
   if (grid > 0x7fffffff || T > 0x7fffffff) return fail(KS_ELIMIT, "ks_lstm_sequence_forward: too many rows or steps");
-  hipLaunchKernelGGL(lstm_seq_forward_kernel, dim3((unsigned)grid), dim3(64 * kSeqWaves), 0, (hipStream_t)stream, (int)T, M, gi, W, ldw,
-                     h0, c0, fresh, hs, cs, saved);
+  hipLaunchKernelGGL(lstm_seq_forward_kernel, dim3((unsigned)grid), dim3(64 * kSeqWaves), 0, (hipStream_t)stream, (int)T, M, groups, gi, W,
+                     ldw, h0, c0, fresh, hs, cs, saved);
   return check_launch("ks_lstm_sequence_forward");
 }
 
