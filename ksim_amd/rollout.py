@@ -78,6 +78,12 @@ class RolloutConstants:  # the static pieces, ksim/task/rl.py:138-150
     # command set to advance in between and its observations read no derived field of the live state.
     fuse_next_observation: bool = False
     head: GaussianHead | MixtureHead | None = None  # None: one mean per action entry and the log_std vector
+    # A critic that does not share a launch with the actor (a recurrent one: a dozen short launches per control step) runs on a
+    # side stream of its own, beside the actor, the sampling and the physics launch, and is joined before the termination pass
+    # (which rewrites the reset mask the critic reads).  Nothing of a control step waits for the value, so the chain of launches
+    # that a step has to wait for loses the critic's share.  Same numbers; off by default (a split rollout already has a stream
+    # per group, and a process has four hardware queues).
+    critic_on_side_stream: bool = False
 
 
 class RolloutEnvState:  # ksim/task/rl.py:110-123, batched
@@ -144,6 +150,7 @@ class Rollout:
         self._defer = bool(c.defer_reset_forward) and not reads_derived
         self._fuse_obs = bool(c.fuse_next_observation) and not reads_derived and c.commands is None
         self._obs_done = None  # (env state, slot, step) whose observation the previous step's last launch has written
+        self._side = None      # the critic's stream and its fork / join events (critic_on_side_stream), made on first use
         if c.actor.in_dim != c.terms.obs_dim or c.actor.out_dim != self.mean.shape[1]:
             raise _lib.KsError("actor must map the observation vector to one mean per action entry (or to what its head takes)")
         if c.critic is not None and (c.critic.in_dim != c.terms.obs_dim or c.critic.out_dim != 1):
@@ -183,18 +190,34 @@ class Rollout:
                     self.actor_carry0.copy_(env.actor_carry)
                 if self.critic_carry0 is not None:
                     self.critic_carry0.copy_(env.critic_carry)
+        critic_joined = True
         if isinstance(c.actor, MLP) and isinstance(c.critic, MLP):
             # two plain MLPs over the same rows share one launch
             c.actor.forward_pair(self.noisy_obs[t], self.mean, c.critic, self.obs[t], self.values[t])
         else:
+            def run_critic() -> None:
+                if isinstance(c.critic, RecurrentNetwork):
+                    c.critic(self.obs[t], env.critic_carry, fresh=self.reset_mask, out=self.values[t])
+                elif c.critic is not None:
+                    c.critic(self.obs[t], out=self.values[t])
+
+            if c.critic is not None and c.critic_on_side_stream:
+                if self._side is None:
+                    self._side = (torch.cuda.Stream(), torch.cuda.Event(), torch.cuda.Event())
+                side, forked, done_ev = self._side
+                main = torch.cuda.current_stream()
+                forked.record(main)  # the observation of this step and the previous step's reset mask are final
+                side.wait_event(forked)
+                with torch.cuda.stream(side):
+                    run_critic()
+                    done_ev.record(side)
+                critic_joined = False
+            else:
+                run_critic()
             if isinstance(c.actor, RecurrentNetwork):
                 c.actor(self.noisy_obs[t], env.actor_carry, fresh=self.reset_mask, out=self.mean)
             else:
                 c.actor(self.noisy_obs[t], out=self.mean)
-            if isinstance(c.critic, RecurrentNetwork):
-                c.critic(self.obs[t], env.critic_carry, fresh=self.reset_mask, out=self.values[t])
-            elif c.critic is not None:
-                c.critic(self.obs[t], out=self.values[t])
         if isinstance(c.head, GaussianHead):
             head_bias = c.head.mean_bias
             if self._lowpass is not None:
@@ -228,6 +251,8 @@ class Rollout:
                       want_cvel=T.SRC_CVEL in c.terms.sources_used, want_cinert=T.SRC_CINERT in c.terms.sources_used,
                       want_cfrc_ext=T.SRC_CFRC_EXT in c.terms.sources_used, step=step, step_base=step_base, event_seed=env.seed,
                       live=self._live, fresh=self.reset_mask if self._defer else None)
+        if not critic_joined:  # the termination pass rewrites the reset mask that the critic's launches read
+            torch.cuda.current_stream().wait_event(self._side[2])
         ev_buf = ps.event_states.get("_buffer") if ps.event_states else None
         st = dict(qpos=d.qpos, qvel=d.qvel, qacc_warmstart=d.qacc_warmstart, time=d.time, last_ctrl=ps.last_ctrl)
         term_args = dict(level=level, components=self.components[t][: c.terms.n_terms] if c.terms.n_terms else None,

@@ -137,6 +137,36 @@ def build(N, T, seed=0, min_height=0.9, events=None, gait=False, recurrent=False
     return m, consts, randomization, (ws, bs, cws, cbs, log_std, kps, kds, clip), Rollout(consts, N, T), RolloutEnvState
 
 
+def test_critic_on_a_side_stream_gives_the_same_rollout():
+    """A recurrent critic on a stream of its own, beside the actor and the physics launch and joined before the termination
+    pass: actions, values, carries and flags bit for bit those of the single chain, eagerly and under graph replay, over
+    rollouts in which episodes end (so the critic reads reset masks that the next termination pass rewrites)."""
+    import dataclasses
+    from ksim_amd.rollout import Rollout
+
+    N, T = 24, 8
+    runs = {}
+    for side, use_graph in ((False, False), (True, False), (True, True)):
+        m, c, rnd_, _, ro, EnvState = build(N, T, seed=13, min_height=0.95, recurrent=True, head="kbot")
+        if side:
+            c = dataclasses.replace(c, critic_on_side_stream=True)
+            ro = Rollout(c, N, T)
+        ps = c.engine.reset(c.physics_model, 1.0, 3, N, rnd_)
+        env = EnvState(ps, rnd_, torch.zeros(N, 2, device=DEV), None, seed=21)
+        snaps, finished = [], 0
+        for it in range(4):
+            traj, rew = ro.unroll(env, graph=use_graph)
+            torch.cuda.synchronize()
+            finished += int(traj.done.sum().item())
+            snaps.append((traj.action.clone(), ro.values.clone(), env.actor_carry.clone(), env.critic_carry.clone(), traj.done.clone(),
+                          rew.total.clone()))
+        assert finished > 0
+        runs[(side, use_graph)] = snaps
+    for key in ((True, False), (True, True)):
+        for a, b in zip(runs[(False, False)], runs[key]):
+            assert all(torch.equal(x, y) for x, y in zip(a, b)), key
+
+
 def _mlp64(x, ws, bs):
     h = torch.from_numpy(np.asarray(x, dtype=np.float64))
     for i, (w, b) in enumerate(zip(ws, bs)):
