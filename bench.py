@@ -162,7 +162,7 @@ def main() -> None:
         print(json.dumps({"ppo_update": ppo_update_rate(torch)}))
         return
     if args.only == "kbot_update":
-        print(json.dumps({"kbot_update": kbot_update_rate(torch)}))
+        print(json.dumps({"kbot_update": kbot_update_rate(torch), "kbot_rollout": kbot_rollout_rate(torch)}))
         return
     if args.only == "iteration":
         print(json.dumps({"ppo_iteration": ppo_iteration_rate(torch)}))
@@ -232,6 +232,7 @@ def main() -> None:
         mlp[key]["of_mfma_yardstick"] = mlp[key]["TFLOPs"] / top
     upd = ppo_update_rate(torch)
     kbot_upd = kbot_update_rate(torch)
+    kbot_ro = kbot_rollout_rate(torch)
     iteration = ppo_iteration_rate(torch)
 
     obs_dim = consts.terms.obs_dim
@@ -280,7 +281,7 @@ def main() -> None:
                              "cycles with a VALU instruction issuing is given beside); the HBM fraction is reported "
                              "against the bytes the engine contract obliges a step to move"},
         "same_rollout_200_steps": long_entry, "other_integrator": other_entry, "single_stream": single_entry,
-        "gae": gae, "streaming": streaming, "policy_mlp": mlp, "ppo_update": upd, "kbot_update": kbot_upd, "ppo_iteration": iteration, "graph_replay": graph,
+        "gae": gae, "streaming": streaming, "policy_mlp": mlp, "ppo_update": upd, "kbot_update": kbot_upd, "kbot_rollout": kbot_ro, "ppo_iteration": iteration, "graph_replay": graph,
     }
     if not args.no_cpu_baseline:
         base = cpu_baseline(args.integrator)
@@ -570,6 +571,27 @@ def ppo_update_rate(torch, reps=6):
             "mfma_utilisation": flops / ms / 1e9 / (BF16_PEAK_TFLOPS),
             "what": "forward + backward (3x the forward flops) of actor and critic 68-3x512-{20,1} bf16, GAE, loss "
                     "gradient and optimiser chain on 2048 envs x 32 steps"}
+
+
+def kbot_rollout_rate(torch, preroll=200, steps=200):
+    """Rollout rate of the K-Bot-scale env with the K-Bot example's recurrent policy (`configs.kbot_lstm_rollout`: LSTM actor
+    and critic 2 x 128 in fp32, filtered mean | deviation head, 4096 envs), after `preroll` untimed control steps."""
+    from ksim_amd.configs import kbot_lstm_rollout
+
+    consts, env, ro, _ = kbot_lstm_rollout()
+    for k in range(preroll):
+        ro.step_engine(env, k % ro.T)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for k in range(steps):
+        ro.step_engine(env, k % ro.T)
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / steps
+    assert torch.isfinite(ro.values).all() and torch.isfinite(env.actor_carry).all()
+    return {"num_envs": ro.N, "untimed_preroll_steps": preroll, "steps": steps, "ms_per_step": dt * 1e3, "value": ro.N / dt,
+            "unit": "env-steps/s",
+            "what": "control steps of 4096 envs with the K-Bot example's LSTM actor and critic (2 x 128, fp32) in the loop, "
+                    "one chain of launches with the critic on a side stream"}
 
 
 def kbot_update_rate(torch, reps=4):

@@ -90,6 +90,36 @@ def kbot_split_rollout(num_envs: int = 8192, rollout_length: int = 32, splits: i
     return consts, envs, SplitRollout(consts, num_envs, rollout_length, splits)
 
 
+def kbot_lstm_rollout(num_envs: int = 4096, rollout_length: int = 100, seed: int = 1006, integrator: str = "euler"):
+    """The K-Bot-scale rollout with the K-Bot example's policy instead of the benchmark's MLPs (examples/kbot/train.py:80-95,
+    837-995, 1754-1757): LSTM actor and critic, projection -> 2 x 128 -> linear head in fp32, the actor's head means |
+    deviations with a mean bias and the one-pole low-pass (10 Hz) whose state rides in the model carry; 4096 envs, 2 s of
+    control steps per rollout.  The critic runs on a side stream (RolloutConstants.critic_on_side_stream)."""
+    import dataclasses
+
+    from .actions import LowPass
+    from .recurrent import LSTMCell, RecurrentNetwork
+    from .rollout import GaussianHead
+
+    m, consts, gains = _kbot_constants(seed, 512, "bf16", 0.5, integrator)
+    rng = np.random.default_rng(seed)
+    H, I, nu = 128, consts.terms.obs_dim, m.nu
+
+    def net(out_dim: int, last_scale: float) -> RecurrentNetwork:
+        proj = (rng.normal(size=(H, I)) / np.sqrt(I), np.zeros(H))
+        cells = [LSTMCell(rng.normal(size=(4 * H, H)) / np.sqrt(H), rng.normal(size=(4 * H, H)) / np.sqrt(H), np.zeros(4 * H), dtype="f32")
+                 for _ in range(2)]
+        out = MLP([last_scale * rng.normal(size=(out_dim, H)) / np.sqrt(H)], [np.zeros(out_dim)], activation="none", dtype="f32")
+        return RecurrentNetwork(proj, cells, out, dtype="f32")
+
+    head = GaussianHead(min_std=0.01, max_std=1.0, var_scale=0.5, mean_bias=torch.zeros(nu, device="cuda"),
+                        lowpass=LowPass(ctrl_dt=0.02, cutoff_frequency=10.0))
+    consts = dataclasses.replace(consts, actor=net(2 * nu, 0.1), critic=net(1, 1.0), log_std=None, head=head,
+                                 critic_on_side_stream=True)
+    env = _kbot_env_state(m, consts, num_envs, seed)
+    return consts, env, Rollout(consts, num_envs, rollout_length), gains
+
+
 def humanoid_rollout(num_envs: int = 4096, rollout_length: int = 16, seed: int = 1003, min_height: float = 0.6):
     """Benchmark config 3: free root + 21 hinges in a 5-limb tree, 4 foot spheres, friction 1.0, 21 PD actuators, root height
     1.3 m, joints ~U(-0.1, 0.1), dt 0.005 with 4 substeps, fp32 actor 71 -> 3 x 256 (ELU) -> 21 means."""
