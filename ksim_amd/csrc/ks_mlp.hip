@@ -1563,6 +1563,7 @@ static void refresh_layers(DevMlp& m, hipStream_t s) {
 }
 
 constexpr int kDwSplit = 32;  // most slices the weight-gradient reduction over the rows is cut into
+constexpr int kDiscMaxSlices = 64;  // most slices a long row reduction of the fp32 products (sgemm below) is cut into
 
 // workspace: hidden activations of every layer, two (M, widest) gradient buffers, two transposes (widest, Mp)
 struct TrainWs {
@@ -1611,7 +1612,9 @@ static int64_t carve_train(const DevMlp& m, int64_t M, char* base, TrainWs* ws) 
   w.t2 = take((int64_t)wz * Mp * esz);
   int64_t maxw = 0;
   for (int l = 0; l < m.n_layers; ++l) maxw = (int64_t)m.npad[l] * m.kpad[l] > maxw ? (int64_t)m.npad[l] * m.kpad[l] : maxw;
-  const int64_t nparts = kDwSplit * maxw > (int64_t)4 * kColsumSlices * wz ? kDwSplit * maxw : (int64_t)4 * kColsumSlices * wz;
+  int64_t nparts = kDwSplit * maxw > (int64_t)4 * kColsumSlices * wz ? kDwSplit * maxw : (int64_t)4 * kColsumSlices * wz;
+  if (m.n_layers == 1 && esz == 4)  // the one-pass weight and bias gradient of a single fp32 layer: slices of both
+    nparts = nparts > (int64_t)kDiscMaxSlices * (maxw + wz) ? nparts : (int64_t)kDiscMaxSlices * (maxw + wz);
   w.part = (float*)take(nparts * 4);
   w.Mp = Mp;
   w.Mp128 = (M + 127) / 128 * 128;
@@ -1762,6 +1765,10 @@ static int train_backward_chain(DevMlp& m, hipStream_t s, int64_t M, const float
   return KS_OK;
 }
 
+template <bool A_KC, bool B_KC>
+static void sgemm(hipStream_t s, int64_t M, int N, int64_t K, const float* A, int64_t lda, const float* B, int64_t ldb, float* C,
+                  int64_t ldc, const float* bias, int act, bool accumulate, float* part, float* colsum = nullptr, float* colpart = nullptr);
+
 template <typename T>
 static int train_backward(DevMlp& m, hipStream_t s, int64_t M, const float* x, const float* dy, const TrainWs& ws,
                           float* dx = nullptr, bool want_w = true, bool accumulate_dx = false, const uint8_t* zero_rows = nullptr) {
@@ -1801,6 +1808,15 @@ static int train_backward(DevMlp& m, hipStream_t s, int64_t M, const float* x, c
                          accumulate_dx ? 1 : 0, zero_rows);
     }
     if (!want_w && l == 0) break;
+    if (L == 1 && sizeof(T) == 4 && np >= 128) {
+      // A single fp32 layer (the projections of the recurrent cells, over all the (step, env) rows of a trajectory slice): the
+      // weight gradient dZ^T X and the bias gradient, the column sums of dZ, in one pass over the row-major operands as they
+      // are, on the 128 x 128 tiles of the long-reduction product; no transposed copies.
+      float* colpart = ws.part + (int64_t)kDiscMaxSlices * np * kp;
+      sgemm<false, false>(s, np, m.dims[0], M, (const float*)dz, np, x, m.dims[0], m.gW[0], kp, nullptr, KS_ACT_NONE, false, ws.part,
+                          m.gb[0], colpart);
+      break;
+    }
     if (want_w && !have_bias) {
       const int nz = M >= 32768 ? 4 * kColsumSlices : kColsumSlices;  // narrow layers: more row slices fill the chip
       hipLaunchKernelGGL(colsum_kernel<T>, dim3((unsigned)((np + 63) / 64), nz), dim3(256), 0, s, M, np, dz, ws.part);
@@ -2244,7 +2260,7 @@ __global__ __launch_bounds__(256) void disc_dz_kernel(int64_t n, int64_t n_extra
 
 }  // namespace ks
 
-constexpr int kDiscMaxSlices = 64;
+// kDiscMaxSlices is defined beside kDwSplit: the training backward pass of single fp32 layers shares these products
 
 struct DiscWs {
   float* y[KS_MAX_LAYERS];      // hidden outputs, all rows
@@ -2290,7 +2306,7 @@ static int64_t carve_disc(const DevMlp& m, int64_t R, int64_t M, char* base, Dis
 // colsum / colpart (wide row reductions only): colsum (M) += sum_k A(k, i) from the same pass, colpart its (slices, M) partials
 template <bool A_KC, bool B_KC>
 static void sgemm(hipStream_t s, int64_t M, int N, int64_t K, const float* A, int64_t lda, const float* B, int64_t ldb, float* C,
-                  int64_t ldc, const float* bias, int act, bool accumulate, float* part, float* colsum = nullptr, float* colpart = nullptr) {
+                  int64_t ldc, const float* bias, int act, bool accumulate, float* part, float* colsum, float* colpart) {
   if (M <= 0 || N <= 0 || K <= 0) return;  // every caller with an empty sum adds into its output
   if (!A_KC && !B_KC && M == 1 && N >= 128 && !bias && act == KS_ACT_NONE) {
     // one output row: the same numbers as the (N, 1) product with the operands exchanged, which takes the wide path below
