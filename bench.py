@@ -113,7 +113,7 @@ def main() -> None:
     ap.add_argument("--integrator", choices=("euler", "implicitfast"), default="euler",
                     help="velocity update of the headline rollout: semi-implicit Euler (what the benchmark configs name) or "
                          "implicitfast (what ksim's RLConfig selects); the other one is reported under 'other_integrator'")
-    ap.add_argument("--only", choices=("mlp", "gae", "update", "kbot_update", "rollout", "iteration", "phases", "mfma"), default=None,
+    ap.add_argument("--only", choices=("mlp", "gae", "update", "kbot_update", "kbot_rollout", "rollout", "iteration", "phases", "mfma"), default=None,
                     help="run one section alone and print its JSON (the command the counter runs under profiles/ use)")
     ap.add_argument("--mlp-rows", type=int, default=0, help="with --only mlp: a single row count instead of 8192 and 524288")
     ap.add_argument("--streams", type=int, default=2,
@@ -162,7 +162,10 @@ def main() -> None:
         print(json.dumps({"ppo_update": ppo_update_rate(torch)}))
         return
     if args.only == "kbot_update":
-        print(json.dumps({"kbot_update": kbot_update_rate(torch), "kbot_rollout": kbot_rollout_rate(torch)}))
+        print(json.dumps({"kbot_update": kbot_update_rate(torch)}))
+        return
+    if args.only == "kbot_rollout":
+        print(json.dumps({"kbot_rollout": kbot_rollout_rate(torch)}))
         return
     if args.only == "iteration":
         print(json.dumps({"ppo_iteration": ppo_iteration_rate(torch)}))
