@@ -844,21 +844,40 @@ __global__ __launch_bounds__(256) void lowpass_scan_kernel(int64_t T, int64_t M,
   if (idx >= M * (int64_t)ld) return;
   const int64_t m = idx / ld;
   const int j = (int)(idx - m * ld);
+  constexpr int kAhead = 8;  // steps whose loads are in flight together: the recursion itself is a few instructions per step
   if (j >= nu) {  // the columns behind the signal (raw deviations of the head): copied when the output is another buffer
     if (x != y)
-      for (int64_t t = 0; t < T; ++t) y[(t * M + m) * ld + j] = x[(t * M + m) * ld + j];
+      for (int64_t t0 = 0; t0 < T; t0 += kAhead) {
+        float v[kAhead];
+#pragma unroll
+        for (int k = 0; k < kAhead; ++k) v[k] = t0 + k < T ? x[((t0 + k) * M + m) * ld + j] : 0.f;
+#pragma unroll
+        for (int k = 0; k < kAhead; ++k)
+          if (t0 + k < T) y[((t0 + k) * M + m) * ld + j] = v[k];
+      }
     return;
   }
   const float b = mean_bias ? mean_bias[j] : 0.f;
   const bool has_add = add && j >= add_first && j < add_first + add_count;
   float last = y0 ? y0[m * nu + j] : 0.f;
-  for (int64_t t = 0; t < T; ++t) {
-    const int64_t r = t * M + m;
-    if (fresh && fresh[r]) last = 0.f;
-    float v = x[r * ld + j] + b;
-    if (has_add) v += add[r * add_ld + (j - add_first)];
-    last = last + alpha * (v - last);
-    y[r * ld + j] = last;
+  for (int64_t t0 = 0; t0 < T; t0 += kAhead) {
+    float v[kAhead];
+    bool f[kAhead];
+#pragma unroll
+    for (int k = 0; k < kAhead; ++k) {
+      const bool in = t0 + k < T;
+      const int64_t r = in ? (t0 + k) * M + m : m;
+      v[k] = x[r * ld + j] + b;
+      if (has_add) v[k] += add[r * add_ld + (j - add_first)];
+      f[k] = fresh && fresh[r];
+    }
+#pragma unroll
+    for (int k = 0; k < kAhead; ++k)
+      if (t0 + k < T) {
+        if (f[k]) last = 0.f;
+        last = last + alpha * (v[k] - last);
+        y[((t0 + k) * M + m) * ld + j] = last;
+      }
   }
   if (y_last) y_last[m * nu + j] = last;
 }
@@ -874,11 +893,23 @@ __global__ __launch_bounds__(256) void lowpass_scan_backward_kernel(int64_t T, i
   const int64_t m = idx / nu;
   const int j = (int)(idx - m * nu);
   float carry = 0.f;  // (1 - alpha) G_{t+1}, or 0 across an episode start
-  for (int64_t t = T - 1; t >= 0; --t) {
-    const int64_t r = t * M + m;
-    const float G = g[r * ld + j] + carry;
-    g[r * ld + j] = alpha * G;
-    carry = (fresh && fresh[r]) ? 0.f : (1.f - alpha) * G;
+  constexpr int kAhead = 8;  // steps whose loads are in flight together
+  for (int64_t t0 = T - 1; t0 >= 0; t0 -= kAhead) {
+    float v[kAhead];
+    bool f[kAhead];
+#pragma unroll
+    for (int k = 0; k < kAhead; ++k) {
+      const int64_t r = (t0 - k >= 0 ? t0 - k : 0) * M + m;
+      v[k] = g[r * ld + j];
+      f[k] = fresh && fresh[r];
+    }
+#pragma unroll
+    for (int k = 0; k < kAhead; ++k)
+      if (t0 - k >= 0) {
+        const float G = v[k] + carry;
+        g[((t0 - k) * M + m) * ld + j] = alpha * G;
+        carry = f[k] ? 0.f : (1.f - alpha) * G;
+      }
   }
   if (d_y0) d_y0[idx] = carry;
 }
