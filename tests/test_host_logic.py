@@ -521,3 +521,38 @@ def test_committed_traffic_profiles_carry_sane_calibration_factors():
             cols = [c.strip() for c in ratio.split("|")]
             if len(cols) >= 9 and re.fullmatch(r"[0-9.]+", cols[5]):
                 assert float(cols[5]) < 4.0, f"{os.path.basename(path)}: traffic / algorithmic {cols[5]} in {cols[0]}"
+
+
+def test_every_public_oracle_function_is_named_in_a_cpu_test():
+    """The oracle is only as good as its pins: every public function of `oracle/*.py` must be called by name in a test that
+    runs without a GPU, or be listed here as plumbing (conversions between containers, no arithmetic of the reference)."""
+    import ast
+    import glob
+    import re
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    plumbing = {
+        "dyn.make_model": "copies a model dictionary into the C struct of the compiled oracle",
+        "recurrent.torch_sequence": "recurrent_sequence on torch tensors; recurrent_sequence_gradients, which calls it, is held "
+                                    "against the numpy network and central differences",
+        "recurrent.torch_parameters": "wraps arrays as tensors that record gradients",
+        "recurrent.parameter_gradients": "reads .grad back into the parameter structure",
+        "ppo_update.update_model": "the minibatch loop around loss_and_grads and optax_chain_step, both pinned; compared with the "
+                                   "kernel path in the GPU suite",
+    }
+    text = ""
+    for f in glob.glob(os.path.join(root, "tests", "test_*.py")):
+        src = open(f).read()
+        if "pytestmark = pytest.mark.gpu" in src or os.path.basename(f).startswith("test_gpu") or os.path.basename(f).startswith("test_zz"):
+            continue
+        text += src
+    missing = []
+    for f in sorted(glob.glob(os.path.join(root, "oracle", "*.py"))):
+        mod = os.path.basename(f)[:-3]
+        if mod.startswith("_"):
+            continue
+        for node in ast.parse(open(f).read()).body:
+            if isinstance(node, ast.FunctionDef) and not node.name.startswith("_"):
+                if f"{mod}.{node.name}" not in plumbing and not re.search(r"\b" + re.escape(node.name) + r"\b", text):
+                    missing.append(f"{mod}.{node.name}")
+    assert not missing, f"oracle functions that no CPU test names: {missing}"

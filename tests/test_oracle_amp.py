@@ -84,3 +84,16 @@ def test_relu_has_no_second_derivative_term():
     _, g1 = oamp.disc_loss_and_grads(ws, bs, real, sim, 2.0, act="relu")
     np.testing.assert_allclose(g0[0][1], g1[0][1], rtol=1e-12)
     assert np.abs(g0[0][0] - g1[0][0]).max() > 1e-3
+
+
+def test_disc_loss_terms_on_a_constant_discriminator():
+    """`disc_loss` itself: a discriminator with zero weights answers its bias b everywhere, so the real term is
+    B T (b - 1)^2 / 2, the simulated term B2 T2 (b + 1)^2 / 2, and the gradient penalty zero."""
+    import torch
+
+    ws = [torch.zeros(1, 5, dtype=torch.float64)]
+    bs = [torch.tensor([0.25], dtype=torch.float64)]
+    real, sim = torch.randn(3, 4, 5, dtype=torch.float64), torch.randn(2, 6, 5, dtype=torch.float64)
+    total, lr, ls, gp = (t.detach() for t in oamp.disc_loss(ws, bs, real, sim, 0.7, act="elu"))
+    assert float(lr) == 12 * 0.75 ** 2 / 2 and float(ls) == 12 * 1.25 ** 2 / 2 and float(gp) == 0.0
+    assert float(total) == float(lr) + float(ls)

@@ -220,3 +220,57 @@ def test_mirror_terms_vanish_for_a_mirror_symmetric_recurrent_policy():
     # and with different mirrored carries the same weights no longer agree: the carries do enter
     other = dict(ident, actor_carry0=mirror["actor_carry0"])
     assert ou.recurrent_loss_and_grads(oa, oc, batch, CFG, head, lowpass=lowpass, mirror=other)[3]["action_mirror_loss"].max() > 1e-6
+
+
+def test_deviation_head_clipped_value_loss_and_filter_helpers_hand_computed():
+    """The small restatements that the larger oracle functions are built from, each against numbers worked out by hand or a
+    library routine."""
+    from scipy.stats import norm
+
+    # mean | raw deviation head: std = min((softplus(raw) + min_std) * var_scale, max_std), with the bias on the mean
+    raw = np.array([[0.3, -0.2, 0.0, 5.0]])  # means 0.3, -0.2; raw deviations 0, 5
+    a = np.array([[0.5, 0.1]])
+    bias = np.array([0.1, -0.1])
+    lp, ent = ou.gaussian_head(torch.tensor(raw), torch.tensor(a), 0.01, 1.0, 0.5, torch.tensor(bias))
+    std = np.array([(math.log(2.0) + 0.01) * 0.5, 1.0])  # softplus(0) = ln 2; (softplus(5) + 0.01) / 2 = 2.5 capped at 1
+    np.testing.assert_allclose(lp.numpy()[0], norm.logpdf(a[0], [0.4, -0.3], std), rtol=1e-12)
+    np.testing.assert_allclose(ent.numpy()[0], norm.entropy(0, std), rtol=1e-12)
+    # clipped value loss (ppo.py:124-135): the clip holds the new value within 0.2 of the old one before the error is taken
+    got = oppo.clipped_value_loss(np.array([1.0, 1.0, 1.0]), np.array([1.5, 1.1, 0.0]), np.array([2.0, 2.0, 1.0]), 0.2)
+    np.testing.assert_allclose(got, [max(0.5**2, 0.8**2), max(0.9**2, 0.9**2), max(1.0**2, 0.2**2)], rtol=1e-15)
+    # the torch filter equals the closed form of a step response and restarts where flagged
+    al = 0.02 / (1.0 / (2 * math.pi * 4.0) + 0.02)
+    x = torch.ones(5, 1, 1, dtype=torch.float64)
+    fresh = np.zeros((5, 1), bool); fresh[3] = True
+    y = ou.lowpass_torch(x, 0.02, 4.0, np.zeros((1, 1)), fresh)
+    y = (y[0] if isinstance(y, tuple) else y).numpy()[:, 0, 0]
+    np.testing.assert_allclose(y, [1 - (1 - al) ** 1, 1 - (1 - al) ** 2, 1 - (1 - al) ** 3, al, 1 - (1 - al) ** 2], rtol=1e-13)
+    # parameter lists survive the flat / unflat round trip in the optimiser's order
+    p = dict(actor_w=[np.ones((2, 3))], actor_b=[np.zeros(2)], critic_w=[np.ones((1, 3)) * 2], critic_b=[np.ones(1)], log_std=np.zeros(2))
+    q = ou.unflat(ou.flat(p), p)
+    assert all(np.array_equal(x_, y_) for k in ("actor_w", "actor_b", "critic_w", "critic_b") for x_, y_ in zip(p[k], q[k]))
+    assert np.array_equal(q["log_std"], p["log_std"])
+
+
+def test_mirror_terms_of_the_mlp_policy_hand_computed():
+    """A linear actor and critic on a two-entry observation that the mirror map swaps and negates: the mirrored mode and value
+    follow by hand, and the terms vanish when the weights respect the symmetry."""
+    obs = torch.tensor([[[1.0, 3.0]]])                       # (T = 1, b = 1, 2)
+    mirror = dict(actor_obs=([1, 0], [-1.0, -1.0]), critic_obs=([1, 0], [-1.0, -1.0]), action=([1, 0], [-1.0, -1.0]),
+                  actor_scale=2.0, critic_scale=0.5)
+    tp = dict(actor_w=[torch.tensor([[1.0, 0.0], [0.0, 2.0]])], actor_b=[torch.zeros(2, dtype=torch.float64)],
+              critic_w=[torch.tensor([[1.0, 1.0]])], critic_b=[torch.zeros(1, dtype=torch.float64)])
+    tp = {k: [a.double() for a in v] for k, v in tp.items()}
+    obs = obs.double()
+    mean = obs @ tp["actor_w"][0].T                          # (1, 6)
+    v = (obs @ tp["critic_w"][0].T)[..., 0]                  # 4
+    out = ou.mirror_terms(mean, v, obs, obs, tp, mirror, "none")
+    # mirrored obs (-3, -1) -> mode (-3, -2) -> mirrored back (2, 3); value of the mirrored obs -4
+    np.testing.assert_allclose(out["action_mirror_loss"].numpy(), [[2.0 * ((1 - 2) ** 2 + (6 - 3) ** 2) / 2]], rtol=1e-15)
+    np.testing.assert_allclose(out["value_mirror_loss"].numpy(), [[0.5 * (4 - (-4)) ** 2]], rtol=1e-15)
+    tp["actor_w"] = [torch.tensor([[1.0, 0.5], [0.5, 1.0]], dtype=torch.float64)]   # commutes with the swap
+    tp["critic_w"] = [torch.tensor([[1.0, -1.0]], dtype=torch.float64)]             # unchanged by swapping and negating the entries
+    mean = obs @ tp["actor_w"][0].T
+    v = (obs @ tp["critic_w"][0].T)[..., 0]
+    out = ou.mirror_terms(mean, v, obs, obs, tp, mirror, "none")
+    assert float(out["action_mirror_loss"].abs().max()) < 1e-28 and float(out["value_mirror_loss"].abs().max()) < 1e-28

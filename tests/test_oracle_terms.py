@@ -907,3 +907,18 @@ def test_lowpass_scan_and_its_backward_sweep():
     dx_free, _ = ot.lowpass_scan_backward(w, dt, fc)
     s_ = 3
     np.testing.assert_allclose(dx_free[s_, 0], a * sum((1 - a) ** (t - s_) * w[t, 0] for t in range(s_, Tn)), rtol=1e-12)
+
+
+def test_norm_and_kernel_helpers_hand_computed():
+    """`get_norm`, `exp_kernel`, `exp_kernel_with_penalty` (rewards.py:72-88): the values the reference's formulas give at a
+    few points worked out by hand."""
+    x = np.array([-2.0, 0.0, 0.5])
+    np.testing.assert_array_equal(ot.get_norm(x, "l1"), [2.0, 0.0, 0.5])
+    np.testing.assert_array_equal(ot.get_norm(x, "l2"), [4.0, 0.0, 0.25])
+    with pytest.raises(ValueError):
+        ot.get_norm(x, "linf")
+    # exp(-x^2 / (2 s^2)): 1 at 0, e^-1/2 one scale away, e^-2 two scales away
+    np.testing.assert_allclose(ot.exp_kernel(np.array([0.0, 0.3, -0.6]), 0.3), [1.0, np.exp(-0.5), np.exp(-2.0)], rtol=1e-15)
+    # the penalised kernel subtracts |x| abs_scale + x^2 sq_scale from it
+    np.testing.assert_allclose(ot.exp_kernel_with_penalty(np.array([0.0, -0.6]), 0.3, 0.5, 0.25),
+                               [1.0, np.exp(-2.0) - 0.6 * 0.25 - 0.36 * 0.5], rtol=1e-15)
