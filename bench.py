@@ -113,7 +113,7 @@ def main() -> None:
     ap.add_argument("--integrator", choices=("euler", "implicitfast"), default="euler",
                     help="velocity update of the headline rollout: semi-implicit Euler (what the benchmark configs name) or "
                          "implicitfast (what ksim's RLConfig selects); the other one is reported under 'other_integrator'")
-    ap.add_argument("--only", choices=("mlp", "gae", "update", "kbot_update", "kbot_rollout", "rollout", "iteration", "phases", "mfma"), default=None,
+    ap.add_argument("--only", choices=("mlp", "gae", "update", "kbot_update", "kbot_rollout", "kbot_iteration", "rollout", "iteration", "phases", "mfma"), default=None,
                     help="run one section alone and print its JSON (the command the counter runs under profiles/ use)")
     ap.add_argument("--mlp-rows", type=int, default=0, help="with --only mlp: a single row count instead of 8192 and 524288")
     ap.add_argument("--streams", type=int, default=2,
@@ -166,6 +166,9 @@ def main() -> None:
         return
     if args.only == "kbot_rollout":
         print(json.dumps({"kbot_rollout": kbot_rollout_rate(torch)}))
+        return
+    if args.only == "kbot_iteration":
+        print(json.dumps({"kbot_iteration": kbot_iteration_rate(torch)}))
         return
     if args.only == "iteration":
         print(json.dumps({"ppo_iteration": ppo_iteration_rate(torch)}))
@@ -236,6 +239,7 @@ def main() -> None:
     upd = ppo_update_rate(torch)
     kbot_upd = kbot_update_rate(torch)
     kbot_ro = kbot_rollout_rate(torch)
+    kbot_it = kbot_iteration_rate(torch)
     iteration = ppo_iteration_rate(torch)
 
     obs_dim = consts.terms.obs_dim
@@ -284,7 +288,7 @@ def main() -> None:
                              "cycles with a VALU instruction issuing is given beside); the HBM fraction is reported "
                              "against the bytes the engine contract obliges a step to move"},
         "same_rollout_200_steps": long_entry, "other_integrator": other_entry, "single_stream": single_entry,
-        "gae": gae, "streaming": streaming, "policy_mlp": mlp, "ppo_update": upd, "kbot_update": kbot_upd, "kbot_rollout": kbot_ro, "ppo_iteration": iteration, "graph_replay": graph,
+        "gae": gae, "streaming": streaming, "policy_mlp": mlp, "ppo_update": upd, "kbot_update": kbot_upd, "kbot_rollout": kbot_ro, "kbot_iteration": kbot_it, "ppo_iteration": iteration, "graph_replay": graph,
     }
     if not args.no_cpu_baseline:
         base = cpu_baseline(args.integrator)
@@ -595,6 +599,55 @@ def kbot_rollout_rate(torch, preroll=200, steps=200):
             "unit": "env-steps/s",
             "what": "control steps of 4096 envs with the K-Bot example's LSTM actor and critic (2 x 128, fp32) in the loop, "
                     "one chain of launches with the critic on a side stream"}
+
+
+def kbot_iteration_rate(torch, reps=2):
+    """Whole iterations of the K-Bot example's task shape (examples/kbot/train.py:1754-1757): a rollout of 4096 envs x 100
+    control steps with the LSTM actor and critic in the loop, rewards, then the update: the on-policy pass replayed from the
+    recorded carries, 3 passes x 8 minibatches of 512 envs through both networks with the filter and the mirrored pass."""
+    import numpy as np
+
+    from ksim_amd import ppo_update as pu
+    from ksim_amd.configs import kbot_lstm_rollout
+
+    consts, env, ro, _ = kbot_lstm_rollout()
+    rng = np.random.default_rng(11)
+    K = consts.terms.obs_dim
+    operm, osign = list(rng.permutation(K)), list(rng.choice([-1.0, 1.0], K))
+    aperm, asign = pu.kbot_mirror_joints()
+    h = consts.head
+    policy = pu.RecurrentHeadPolicy(consts.actor, consts.critic, h.min_std, h.max_std, h.var_scale, h.mean_bias, lowpass=h.lowpass,
+                                    mirror=pu.MirrorSpec(operm, osign, operm, osign, aperm, asign))
+    policy.train_init()
+    cfg = pu.PPOUpdateConfig(batch_size=512, num_passes=3, learning_rate=3e-4, actor_mirror_loss_scale=1.0, critic_mirror_loss_scale=0.5)
+
+    def iteration(seed: int):
+        traj, rew = ro.unroll(env)
+        torch.cuda.synchronize()
+        t_roll = time.perf_counter()
+        out = pu.update_model_recurrent(policy, cfg, traj.obs["noisy_obs"], traj.obs["obs"], traj.action, rew.total, traj.done,
+                                        traj.success, ro.actor_carry0, ro.critic_carry0, ro.fresh, seed=seed, lpf0=ro.lpf_carry0)
+        return t_roll, out
+
+    for k in range(2):  # the first two rollouts also take the robots from their initial stance to falls and resets
+        iteration(k)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    roll = 0.0
+    for k in range(reps):
+        torch.cuda.synchronize()  # so that the rollout's share does not include the tail of the previous update
+        ts = time.perf_counter()
+        t_roll, out = iteration(2 + k)
+        roll += t_roll - ts
+    torch.cuda.synchronize()
+    elapsed = (time.perf_counter() - t0) / reps
+    assert all(torch.isfinite(o["grad_norm"]).all() for o in out) and torch.isfinite(env.actor_carry).all()
+    n = ro.N * ro.T
+    return {"num_envs": ro.N, "rollout_length": ro.T, "transitions": n, "minibatch_envs": cfg.batch_size, "num_passes": cfg.num_passes,
+            "minibatch_steps": len(out), "s_per_iteration": elapsed, "transitions_per_s": n / elapsed, "rollout_s": roll / reps,
+            "update_s": elapsed - roll / reps,
+            "what": "rollout of 4096 envs x 100 steps with the K-Bot example's LSTM policy, rewards, on-policy replay and 24 minibatch "
+                    "steps with filter gradient and mirror losses; host wall-clock per iteration"}
 
 
 def kbot_update_rate(torch, reps=4):
