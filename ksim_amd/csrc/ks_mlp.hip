@@ -1801,11 +1801,16 @@ static int train_backward(DevMlp& m, hipStream_t s, int64_t M, const float* x, c
   for (int l = L - 1; l >= 0; --l) {
     const int np = m.npad[l], kp = m.kpad[l], kp128 = round_up(kp, kBN);
     if (l == 0 && dx) {  // gradient with respect to the network input
-      const int rc0 = launch_layer<T, false, false>(KS_ACT_NONE, s, M, kp128, np, np, kp128, dz, np, m.Wt[0], m.zero_bias, dnext, kp128);
+      // an fp32 network whose input width needs no padding: the product writes the caller's buffer itself
+      const bool direct = sizeof(T) == 4 && m.dims[0] == kp128 && !accumulate_dx && !zero_rows;
+      const int rc0 = launch_layer<T, false, false>(KS_ACT_NONE, s, M, kp128, np, np, kp128, dz, np, m.Wt[0], m.zero_bias,
+                                                    direct ? (T*)dx : dnext, kp128);
       if (rc0 != KS_OK) return rc0;
-      const int64_t n = M * m.dims[0];
-      hipLaunchKernelGGL(unpad_cast_kernel<T>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, M, m.dims[0], kp128, (const T*)dnext, dx,
-                         accumulate_dx ? 1 : 0, zero_rows);
+      if (!direct) {
+        const int64_t n = M * m.dims[0];
+        hipLaunchKernelGGL(unpad_cast_kernel<T>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, M, m.dims[0], kp128, (const T*)dnext, dx,
+                           accumulate_dx ? 1 : 0, zero_rows);
+      }
     }
     if (!want_w && l == 0) break;
     if (L == 1 && sizeof(T) == 4 && np >= 128) {
