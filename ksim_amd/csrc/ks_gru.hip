@@ -159,16 +159,48 @@ __global__ __launch_bounds__(256) void lstm_gate_backward_kernel(int64_t M, int 
 // The step-by-step path costs two GEMM launches and a gate kernel per step, layer and network: a minibatch of 100 control steps
 // is thousands of launches of a few microseconds each.  Here a workgroup of eight wavefronts owns 4 rows (envs) for all T
 // steps, so that a minibatch of a thousand rows is one workgroup per CU.  The product runs on v_mfma_f32_4x4x1 (sixteen
-// independent 4x4 outer products per instruction): block b = lane / 4 of wavefront w is hidden unit 16 w + b, its four A entries
-// are that unit's input / forget / cell / output rows of W_hh and its four B entries the four rows' hidden state, so after K = 128
-// instructions lane (b, j) holds the four gate pre-activations of its unit for row j.  The wavefront's slice of W_hh stays in
+// independent 4x4 outer products per instruction): block b = lane / 4 of wavefront w is hidden unit 16 w + b, its four B entries
+// are that unit's input / forget / cell / output rows of W_hh and the four A entries, the same for every block and therefore
+// broadcast from one block, the four rows' hidden state; after K = 128 instructions and a 4 x 4 transpose inside each group of
+// four lanes, lane (b, j) holds the four gate pre-activations of its unit for row j.  The wavefront's slice of W_hh stays in
 // 128 vector registers per lane for the whole sequence, the hidden state of the 4 rows lives in LDS (double buffered), the
-// cell state in a register; a step is 128 MFMAs, the gate arithmetic of one (unit, row) per lane, and one barrier.
-// fp32 cells of hidden size 128.
+// cell state in a register; a step is 128 MFMAs (the fp32 matrix rate: 4 rows x 512 x 128 multiply-adds per CU), the gate
+// arithmetic of one (unit, row) per lane, and one barrier.  fp32 cells of hidden size 128.
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 constexpr int kSeqRows = 4, kSeqH = 128, kSeqWaves = 8, kSeqPadH = kSeqH + 4, kSeqPadG = 4 * kSeqH + 4;
 
 __device__ __forceinline__ float sigmoid_ks(float x) { return 1.f / (1.f + expf(-x)); }
+
+// 1 / (1 + e^-x) and tanh x = 1 - 2 / (e^2x + 1) on v_exp_f32 and v_rcp_f32; both saturate correctly (e^y = inf gives 0 and -1 + 2 = 1)
+__device__ __forceinline__ float seq_sigmoid(float x) { return __builtin_amdgcn_rcpf(1.f + __expf(-x)); }
+__device__ __forceinline__ float seq_tanh(float x) { return 1.f - 2.f * __builtin_amdgcn_rcpf(__expf(2.f * x) + 1.f); }
+
+// Barrier for data that the wavefronts of a workgroup hand each other through LDS only: it waits for this wavefront's LDS
+// traffic, not for its global loads and stores.  __syncthreads() would also drain the step's stores (and the loads fetched
+// ahead for the next step) before every barrier, a memory round trip per step of the sequence.
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+// where hidden unit u of a row sits in the LDS copy of the state: unit u = 16 q + b is register q of block b (see the forward
+// kernel), and a lane reads its block's 8 registers as 8 consecutive floats
+__device__ __forceinline__ int seq_slot(int u) { return 8 * (u & 15) + (u >> 4); }
+
+// Transpose of a 4 x 4 block held by four neighbouring lanes (lane j of the group holds a0..a3): out[g] = a_j of lane g.
+// Three lane exchanges within the group (DPP quad permutes): for d = 1, 2, 3 lane s sends its entry s ^ d to lane s ^ d.
+__device__ __forceinline__ float pick4(float a0, float a1, float a2, float a3, int i) {
+  return i == 0 ? a0 : (i == 1 ? a1 : (i == 2 ? a2 : a3));
+}
+__device__ __forceinline__ void quad_transpose(float a0, float a1, float a2, float a3, int j, float (&out)[4]) {
+  const float own = pick4(a0, a1, a2, a3, j);
+  const float s1 = pick4(a0, a1, a2, a3, j ^ 1), s2 = pick4(a0, a1, a2, a3, j ^ 2), s3 = pick4(a0, a1, a2, a3, j ^ 3);
+  const float r1 = __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, s1), 0xB1, 0xf, 0xf, true));  // quad_perm [1,0,3,2]
+  const float r2 = __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, s2), 0x4E, 0xf, 0xf, true));  // quad_perm [2,3,0,1]
+  const float r3 = __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, s3), 0x1B, 0xf, 0xf, true));  // quad_perm [3,2,1,0]
+#pragma unroll
+  for (int g = 0; g < 4; ++g) {
+    const int d = g ^ j;
+    out[g] = d == 0 ? own : (d == 1 ? r1 : (d == 2 ? r2 : r3));
+  }
+}
 
 __global__ __launch_bounds__(64 * kSeqWaves) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void lstm_seq_forward_kernel(int T, int64_t M, int groups, const float* __restrict__ gi, const float* __restrict__ W, int ldw,
@@ -178,7 +210,11 @@ void lstm_seq_forward_kernel(int T, int64_t M, int groups, const float* __restri
   __shared__ __attribute__((aligned(16))) float sh[2][kSeqRows][kSeqPadH];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int j = lane & 3, unit = 16 * wave + (lane >> 2);
-  // A operand of block b, entry i = lane % 4: W_hh[gate i, unit][k]
+  // The weights are the B operand: block b, entry lane % 4: W_hh[gate lane % 4, unit][k].  The hidden state is the A operand and
+  // is the same for all sixteen blocks, so it is broadcast from one block per instruction (CBSZ = 4, ABID = k % 16): the four
+  // lanes of block k % 16 hold h[row 0..3][k] in register k / 16, i.e. the 512 values of the state sit once in 8 registers of the
+  // wavefront instead of once per block.  In LDS the state is stored in that order (row, block, register), two 16-byte reads per
+  // lane and step.
   float wa[H];
   {
     const float4* src = reinterpret_cast<const float4*>(W + (int64_t)(j * H + unit) * ldw);
@@ -198,11 +234,8 @@ void lstm_seq_forward_kernel(int T, int64_t M, int groups, const float* __restri
   const int64_t mc = row_ok ? m : M - 1;  // loads of the rows past the batch are clamped, their stores dropped
   if (grp > 0) __syncthreads();  // the previous set's last read of the state buffers is over
   float c = c0[mc * H + unit];
-  if (threadIdx.x < kSeqRows * H / 4) {
-    const int r = threadIdx.x / (H / 4), k4 = threadIdx.x - r * (H / 4);
-    const int64_t mr = r0 + r < M ? r0 + r : M - 1;
-    *reinterpret_cast<float4*>(&sh[0][r][4 * k4]) = *reinterpret_cast<const float4*>(h0 + mr * H + 4 * k4);
-  }
+  float hprev = h0[mc * H + unit];  // the state this lane's (unit, row) enters the step with
+  sh[0][j][seq_slot(unit)] = hprev;
   __syncthreads();
   int cur = 0;
   // the step's inputs from memory are fetched one step ahead: their latency would otherwise stand between the matrix work and the gates
@@ -223,25 +256,38 @@ void lstm_seq_forward_kernel(int T, int64_t M, int groups, const float* __restri
       if (fresh) fnext = fresh[tn];
     }
     f32x4 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
-    const float* hrow = &sh[cur][j][0];
-#pragma unroll
-    for (int k4 = 0; k4 < H / 4; ++k4) {
-      const float4 hb = *reinterpret_cast<const float4*>(hrow + 4 * k4);
-      acc0 = __builtin_amdgcn_mfma_f32_4x4x1f32(wa[4 * k4], hb.x, acc0, 0, 0, 0);
-      acc1 = __builtin_amdgcn_mfma_f32_4x4x1f32(wa[4 * k4 + 1], hb.y, acc1, 0, 0, 0);
-      acc0 = __builtin_amdgcn_mfma_f32_4x4x1f32(wa[4 * k4 + 2], hb.z, acc0, 0, 0, 0);
-      acc1 = __builtin_amdgcn_mfma_f32_4x4x1f32(wa[4 * k4 + 3], hb.w, acc1, 0, 0, 0);
+    float ha[8];
+    {
+      const float4 a0 = *reinterpret_cast<const float4*>(&sh[cur][j][8 * (lane >> 2)]);
+      const float4 a1 = *reinterpret_cast<const float4*>(&sh[cur][j][8 * (lane >> 2) + 4]);
+      ha[0] = a0.x; ha[1] = a0.y; ha[2] = a0.z; ha[3] = a0.w; ha[4] = a1.x; ha[5] = a1.y; ha[6] = a1.z; ha[7] = a1.w;
     }
-    const float hprev = sh[cur][j][unit];
+    // k runs 0..127 in order, even k into one accumulator and odd k into the other
+#define KS_SEQ_MFMA(K0)                                                                                            \
+    acc0 = __builtin_amdgcn_mfma_f32_4x4x1f32(ha[(K0) >> 4], wa[(K0)], acc0, 4, (K0) & 15, 0);                       \
+    acc1 = __builtin_amdgcn_mfma_f32_4x4x1f32(ha[((K0) + 1) >> 4], wa[(K0) + 1], acc1, 4, ((K0) + 1) & 15, 0);
+#define KS_SEQ_MFMA8(K0) KS_SEQ_MFMA(K0) KS_SEQ_MFMA((K0) + 2) KS_SEQ_MFMA((K0) + 4) KS_SEQ_MFMA((K0) + 6)
+#define KS_SEQ_MFMA32(K0) KS_SEQ_MFMA8(K0) KS_SEQ_MFMA8((K0) + 8) KS_SEQ_MFMA8((K0) + 16) KS_SEQ_MFMA8((K0) + 24)
+    KS_SEQ_MFMA32(0) KS_SEQ_MFMA32(32) KS_SEQ_MFMA32(64) KS_SEQ_MFMA32(96)
+#undef KS_SEQ_MFMA32
+#undef KS_SEQ_MFMA8
+#undef KS_SEQ_MFMA
+    // lane (unit, gate lane % 4) now holds that gate for the four rows in its four registers; the gates want the transpose
+    // within each group of four lanes: lane (unit, row j) with the four gates
+    float pre[4];
+    quad_transpose(acc0[0] + acc1[0], acc0[1] + acc1[1], acc0[2] + acc1[2], acc0[3] + acc1[3], j, pre);
     const float cp = f ? 0.f : c, hu = f ? 0.f : hprev;
-    const float si = sigmoid_ks(gin[0] + (f ? 0.f : acc0[0] + acc1[0]));
-    const float sf = sigmoid_ks(gin[1] + (f ? 0.f : acc0[1] + acc1[1]));
-    const float tg = tanhf(gin[2] + (f ? 0.f : acc0[2] + acc1[2]));
-    const float so = sigmoid_ks(gin[3] + (f ? 0.f : acc0[3] + acc1[3]));
+    // the hardware exponential and reciprocal (about 1 ulp each) instead of the library's expf, tanhf and IEEE division: a
+    // fifth of the instructions, and the gates are as many instructions per step as the matrix work is cycles
+    const float si = seq_sigmoid(gin[0] + (f ? 0.f : pre[0]));
+    const float sf = seq_sigmoid(gin[1] + (f ? 0.f : pre[1]));
+    const float tg = seq_tanh(gin[2] + (f ? 0.f : pre[2]));
+    const float so = seq_sigmoid(gin[3] + (f ? 0.f : pre[3]));
     c = sf * cp + si * tg;
-    const float tc = tanhf(c);
+    const float tc = seq_tanh(c);
     const float hn = so * tc;
-    sh[cur ^ 1][j][unit] = hn;
+    hprev = hn;
+    sh[cur ^ 1][j][seq_slot(unit)] = hn;
     if (row_ok) {
       const int64_t o = (int64_t)t * M + m;
       hs[o * H + unit] = hn;
@@ -251,7 +297,7 @@ void lstm_seq_forward_kernel(int T, int64_t M, int groups, const float* __restri
         sv[0] = si; sv[H] = sf; sv[2 * H] = tg; sv[3 * H] = so; sv[4 * H] = tc; sv[5 * H] = cp; sv[6 * H] = hu;
       }
     }
-    __syncthreads();  // the new hidden state is complete; the buffer just read is free for the step after next
+    lds_barrier();  // the new hidden state is complete; the buffer just read is free for the step after next
     cur ^= 1;
   }
   }
@@ -319,7 +365,7 @@ void lstm_seq_backward_kernel(int T, int64_t M, const float* __restrict__ dH, co
       float* dg = d_g + ((int64_t)t * M + m) * 4 * H + unit;
       dg[0] = gI; dg[H] = gF; dg[2 * H] = gG; dg[3 * H] = gO;
     }
-    __syncthreads();
+    lds_barrier();
     f32x4 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
     const float* grow = &sg[j][128 * kg];
 #pragma unroll
@@ -340,7 +386,7 @@ void lstm_seq_backward_kernel(int T, int64_t M, const float* __restrict__ dH, co
     }
     const float mine = kg == 0 ? part[0] : (kg == 1 ? part[1] : (kg == 2 ? part[2] : part[3]));
     dhc = f ? 0.f : mine;
-    __syncthreads();  // every wavefront has read this step's gate gradients
+    lds_barrier();  // every wavefront has read this step's gate gradients
   }
   if (row_ok) {
     if (dh0) dh0[m * H + unit] = dhc;
