@@ -936,7 +936,14 @@ __global__ __launch_bounds__(256) void sum_parts_kernel(int64_t n, int nz, const
   const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (i >= n) return;
   float s = 0.f;
-  for (int z = 0; z < nz; ++z) s += part[(int64_t)z * n + i];
+  for (int z0 = 0; z0 < nz; z0 += 8) {  // eight slices' loads in flight, added in slice order
+    float v[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) v[k] = z0 + k < nz ? part[(int64_t)(z0 + k) * n + i] : 0.f;
+#pragma unroll
+    for (int k = 0; k < 8; ++k)
+      if (z0 + k < nz) s += v[k];
+  }
   out[i] = s;
 }
 
@@ -959,7 +966,16 @@ __global__ __launch_bounds__(256) void grad_finish_kernel(GradFinishArgs a) {
     const int64_t i = (int64_t)(b - a.first_w[l]) * 256 + threadIdx.x, n = a.nW[l];
     if (i >= n) return;
     float s = 0.f;
-    for (int z = 0; z < a.nz[l]; ++z) s += a.wpart[l][(int64_t)z * n + i];
+    const float* part = a.wpart[l];
+    const int nz = a.nz[l];
+    for (int z0 = 0; z0 < nz; z0 += 8) {  // eight slices' loads in flight, added in slice order
+      float v[8];
+#pragma unroll
+      for (int k = 0; k < 8; ++k) v[k] = z0 + k < nz ? part[(int64_t)(z0 + k) * n + i] : 0.f;
+#pragma unroll
+      for (int k = 0; k < 8; ++k)
+        if (z0 + k < nz) s += v[k];
+    }
     a.gW[l][i] = s;
     return;
   }
