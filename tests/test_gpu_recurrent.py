@@ -288,3 +288,33 @@ def test_lstm_sequence_kernels_agree_with_the_step_by_step_entry_points():
                                         None, _lib.ptr(z(4, 64)), None, None) != 0
     assert lib.ks_lstm_sequence_forward(cell._handle, _lib.current_stream(), 2, M, _lib.ptr(z(2, M, 4 * H)), _lib.ptr(h0), _lib.ptr(c0),
                                         None, _lib.ptr(h0), None, None) != 0  # aliasing is for T = 1 only
+
+
+def test_lstm_sequence_forward_over_many_rows_equals_the_same_rows_in_small_calls():
+    """A short call over thousands of rows lets each workgroup take several 4-row sets in turn (the rollout's single step over all
+    envs): the rows must come out exactly as when they are given in calls small enough for one set per workgroup, including a
+    last set that is not full, in place as the rollout calls it, and with the episode starts honoured."""
+    from ksim_amd.recurrent import LSTMCell
+
+    rng = np.random.default_rng(53)
+    M, H = 2102, 128
+    cell = LSTMCell(rng.normal(size=(4 * H, H)) / np.sqrt(H), rng.normal(size=(4 * H, H)) / np.sqrt(H), rng.normal(size=4 * H) * 0.1, dtype="f32")
+    cell.train_init()
+    z = lambda *s: torch.zeros(*s, device=DEV)  # noqa: E731
+    for Tn in (1, 3):
+        x, h0, c0 = t32(rng.normal(size=(Tn, M, H))), t32(rng.normal(size=(M, H)) * 0.5), t32(rng.normal(size=(M, H)) * 0.5)
+        fresh = torch.tensor(rng.random((Tn, M)) < 0.1, dtype=torch.uint8, device=DEV)
+        hs, cs, sv = z(Tn, M, H), z(Tn, M, H), z(Tn, M, 7 * H)
+        cell.sequence_forward(x, h0, c0, fresh, hs, cs, sv)
+        for lo in range(0, M, 700):
+            hi = min(M, lo + 700)
+            n = hi - lo
+            hs1, cs1, sv1 = z(Tn, n, H), z(Tn, n, H), z(Tn, n, 7 * H)
+            cell.sequence_forward(x[:, lo:hi].contiguous(), h0[lo:hi].contiguous(), c0[lo:hi].contiguous(), fresh[:, lo:hi].contiguous(),
+                                  hs1, cs1, sv1)
+            assert torch.equal(hs[:, lo:hi], hs1) and torch.equal(cs[:, lo:hi], cs1) and torch.equal(sv[:, lo:hi], sv1), (Tn, lo)
+    h, c = h0.clone(), c0.clone()  # one step in place over all rows, as the rollout advances its carry
+    cell(x[0], h, c, fresh[0], out=(h, c))
+    hs1, cs1, sv1 = z(1, M, H), z(1, M, H), z(1, M, 7 * H)
+    cell.sequence_forward(x[:1].contiguous(), h0, c0, fresh[:1].contiguous(), hs1, cs1, sv1)
+    assert torch.equal(h, hs1[0]) and torch.equal(c, cs1[0])
