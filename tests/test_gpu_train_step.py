@@ -251,3 +251,32 @@ def test_config5_full_ppo_iteration_16384_envs():
         outs.append([out["rewards"].total.clone(), policy.log_std.clone()] + [p.clone() for p in params])
     for a, b in zip(*outs):
         assert torch.equal(a, b), "the iteration is not reproducible bit for bit"
+
+
+def test_kbot_lstm_rollout_config_runs_and_feeds_the_recurrent_update():
+    """`configs.kbot_lstm_rollout` (the cfg 4 env with the K-Bot example's LSTM actor and critic, filtered head, critic on a
+    side stream) at a reduced env count: two runs give the same bits, everything stays finite, and the rollout's buffers are
+    what `update_model_recurrent` takes (on-policy replay equal to the recorded values bit for bit, finite parameter steps)."""
+    from ksim_amd import ppo_update as pu
+    from ksim_amd.configs import kbot_lstm_rollout
+
+    N, T = 256, 12
+    runs = []
+    for _ in range(2):
+        c, env, ro, _ = kbot_lstm_rollout(num_envs=N, rollout_length=T)
+        assert c.critic_on_side_stream and c.actor.lstm and c.actor.hidden_size == 128 and all(cell.dtype == "f32" for cell in c.actor.cells)
+        for _ in range(3):
+            traj, rew = ro.unroll(env)
+        torch.cuda.synchronize()
+        runs.append((traj.action.clone(), ro.values.clone(), env.actor_carry.clone(), env.lpf_state.clone(), traj.done.clone(), rew.total.clone()))
+    for a, b in zip(*runs):
+        assert torch.equal(a, b)
+    assert all(torch.isfinite(x.float()).all() for x in runs[1])
+    h = c.head
+    policy = pu.RecurrentHeadPolicy(c.actor, c.critic, h.min_std, h.max_std, h.var_scale, h.mean_bias, lowpass=h.lowpass)
+    policy.train_init()
+    args = (traj.obs["noisy_obs"], traj.obs["obs"], traj.action, rew.total, traj.done, traj.success, ro.actor_carry0, ro.critic_carry0, ro.fresh)
+    on_lp, on_v = pu.recurrent_on_policy(policy, args[0], args[1], args[2], *args[6:], lpf0=ro.lpf_carry0)[:2]
+    assert torch.equal(on_v, ro.values[..., 0]) and torch.isfinite(on_lp).all()
+    out = pu.update_model_recurrent(policy, pu.PPOUpdateConfig(batch_size=64, num_passes=1, learning_rate=3e-4), *args, seed=3, lpf0=ro.lpf_carry0)
+    assert len(out) == 4 and all(torch.isfinite(o["grad_norm"]).all() and o["grad_norm"].item() > 0 for o in out)
