@@ -886,7 +886,9 @@ int ks_lstm_adam_step(KsLstm* lstm, ks_stream_t stream, const KsAdamParams* para
  *                              hs, cs (T, M, H) the states after every step (cs nullable), saved (T, M, 7H) nullable, in the
  *                              layout of ks_lstm_train_forward.  With T = 1, hs / cs may alias h0 / c0; ks_lstm_forward and
  *                              ks_lstm_train_forward are this launch with T = 1 for such cells, so a rollout's steps and the
- *                              replay of its trajectory agree bit for bit.
+ *                              replay of its trajectory agree bit for bit.  The gates are evaluated with the hardware
+ *                              exponential and reciprocal (about 1 ulp each; 3e-7 from the library's expf / tanhf on unit-scale
+ *                              states).
  *   ks_lstm_sequence_backward  dH (T, M, H) the gradient reaching h_t from the layer above; d_g (T, M, 4H) out, as
  *                              ks_lstm_backward_step returns it per step; dh0, dc0 (M, H), nullable, the gradient of the
  *                              initial carry.  Needs ks_lstm_train_init (the transposed weights). */
